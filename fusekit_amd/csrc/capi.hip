@@ -1,0 +1,204 @@
+// extern "C" surface of libfusekit_hip.so: error state, device memory and the
+// operator launches.  Declarations and reference citations live in
+// include/fusekit_hip.h.
+#include <mutex>
+
+#include "fk_host.hpp"
+
+namespace fk {
+
+static thread_local std::string t_last_error;
+
+fk_status set_error(fk_status code, const std::string& msg) {
+    t_last_error = msg;
+    return code;
+}
+
+fk_status hip_error(hipError_t e, const char* what) {
+    return set_error(FK_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+fk_status device_facts(const DeviceFacts** out) {
+    static DeviceFacts facts;
+    static fk_status status = FK_OK;
+    static std::string message;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        int n = 0;
+        hipError_t e = hipGetDeviceCount(&n);
+        if (e != hipSuccess || n == 0) {
+            status = FK_ERR_HIP;
+            message = "no HIP device available (this library has no CPU path)";
+            return;
+        }
+        e = hipGetDeviceProperties(&facts.prop, 0);
+        if (e != hipSuccess) {
+            status = FK_ERR_HIP;
+            message = std::string("hipGetDeviceProperties: ") + hipGetErrorString(e);
+            return;
+        }
+        facts.cus = facts.prop.multiProcessorCount;
+        facts.max_dyn_lds = (int)facts.prop.sharedMemPerBlock;
+        int optin = 0;
+        if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, 0) == hipSuccess &&
+            optin > facts.max_dyn_lds)
+            facts.max_dyn_lds = optin;
+    });
+    if (status != FK_OK) return set_error(status, message);
+    *out = &facts;
+    return FK_OK;
+}
+
+fk_status run_launch(const Launch& l, hipStream_t s) {
+    void* params[1] = {const_cast<unsigned char*>(l.args)};
+    FK_HIP(hipLaunchKernel(l.func, l.grid, l.block, params, l.shmem, s));
+    return FK_OK;
+}
+
+}  // namespace fk
+
+using namespace fk;
+
+extern "C" {
+
+const char* fk_last_error(void) { return t_last_error.c_str(); }
+const char* fk_version(void) { return "fusekit-hip 0.1.0 (gfx950)"; }
+
+fk_status fk_device_props_get(fk_device_props* out) {
+    if (!out) return set_error(FK_ERR_INVALID, "null out");
+    const DeviceFacts* d;
+    FK_TRY(device_facts(&d));
+    memset(out, 0, sizeof(*out));
+    strncpy(out->name, d->prop.name, sizeof(out->name) - 1);
+    strncpy(out->arch, d->prop.gcnArchName, sizeof(out->arch) - 1);
+    out->compute_units = d->cus;
+    out->wavefront = d->prop.warpSize;
+    out->lds_bytes_per_block = d->max_dyn_lds;
+    out->l2_bytes = d->prop.l2CacheSize;
+    out->hbm_bytes = d->prop.totalGlobalMem;
+    out->clock_khz = d->prop.clockRate;
+    return FK_OK;
+}
+
+fk_status fk_alloc(size_t nbytes, void** dptr) {
+    if (!dptr || nbytes == 0) return set_error(FK_ERR_INVALID, "fk_alloc: null out pointer or zero size");
+    const DeviceFacts* d;
+    FK_TRY(device_facts(&d));
+    FK_HIP(hipMalloc(dptr, nbytes));
+    return FK_OK;
+}
+
+fk_status fk_free(void* dptr) {
+    if (!dptr) return FK_OK;
+    FK_HIP(hipFree(dptr));
+    return FK_OK;
+}
+
+fk_status fk_upload(void* dptr, const void* host, size_t nbytes) {
+    if (!dptr || !host) return set_error(FK_ERR_INVALID, "fk_upload: null pointer");
+    FK_HIP(hipMemcpy(dptr, host, nbytes, hipMemcpyHostToDevice));
+    return FK_OK;
+}
+
+fk_status fk_download(void* host, const void* dptr, size_t nbytes) {
+    if (!dptr || !host) return set_error(FK_ERR_INVALID, "fk_download: null pointer");
+    FK_HIP(hipMemcpy(host, dptr, nbytes, hipMemcpyDeviceToHost));
+    return FK_OK;
+}
+
+fk_status fk_stream_create(fk_stream* out) {
+    if (!out) return set_error(FK_ERR_INVALID, "null out");
+    const DeviceFacts* d;
+    FK_TRY(device_facts(&d));
+    hipStream_t s;
+    FK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = s;
+    return FK_OK;
+}
+fk_status fk_stream_destroy(fk_stream s) {
+    if (s) FK_HIP(hipStreamDestroy((hipStream_t)s));
+    return FK_OK;
+}
+fk_status fk_stream_sync(fk_stream s) {
+    FK_HIP(hipStreamSynchronize((hipStream_t)s));
+    return FK_OK;
+}
+
+fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks) {
+    g_gemv_policy.rows_per_tile = rows_per_tile;
+    g_gemv_policy.grid_blocks = grid_blocks;
+    return FK_OK;
+}
+
+fk_status fk_qgemv(const fk_weight* W, const uint16_t* x, const uint16_t* bias, uint16_t* y, fk_stream s) {
+    GemvRequest rq;
+    rq.mats[0] = W;
+    rq.bias[0] = bias;
+    rq.y[0] = y;
+    rq.x = x;
+    Launch l;
+    FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_linear_residual(const fk_weight* W, const uint16_t* x, const uint16_t* res, const uint16_t* res2,
+                             uint16_t* y, fk_stream s) {
+    if (!res) return set_error(FK_ERR_INVALID, "fk_linear_residual: null residual");
+    GemvRequest rq;
+    rq.mats[0] = W;
+    rq.y[0] = y;
+    rq.x = x;
+    rq.res = res;
+    rq.res2 = res2;
+    Launch l;
+    FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_rmsnorm_qkv(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* Wq,
+                         const fk_weight* Wk, const fk_weight* Wv, const uint16_t* bq, const uint16_t* bk,
+                         const uint16_t* bv, uint16_t* q, uint16_t* k, uint16_t* v, fk_stream s) {
+    GemvRequest rq;
+    rq.n_mats = 3;
+    rq.mats[0] = Wq; rq.mats[1] = Wk; rq.mats[2] = Wv;
+    rq.bias[0] = bq; rq.bias[1] = bk; rq.bias[2] = bv;
+    rq.y[0] = q; rq.y[1] = k; rq.y[2] = v;
+    rq.x = x;
+    rq.norm_w = norm_w;
+    rq.eps = eps;
+    Launch l;
+    FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_gateup_swiglu(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* Wg,
+                           const fk_weight* Wu, int variant, uint16_t* out, fk_stream s) {
+    if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, "fk_gateup_swiglu: variant must be 0, 1 or 2");
+    GemvRequest rq;
+    rq.swiglu = true;
+    rq.swiglu_variant = variant;
+    rq.mats[0] = Wg; rq.mats[1] = Wu;
+    rq.y[0] = out;
+    rq.x = x;
+    rq.norm_w = norm_w;
+    rq.eps = eps;
+    Launch l;
+    FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_final_rmsnorm_lm_head(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* W,
+                                   uint16_t* logits, fk_stream s) {
+    if (!norm_w) return set_error(FK_ERR_INVALID, "fk_final_rmsnorm_lm_head: null norm weight");
+    GemvRequest rq;
+    rq.mats[0] = W;
+    rq.y[0] = logits;
+    rq.x = x;
+    rq.norm_w = norm_w;
+    rq.eps = eps;
+    Launch l;
+    FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+}  // extern "C"

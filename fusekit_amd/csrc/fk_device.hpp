@@ -1,0 +1,93 @@
+// Device-side helpers shared by the gfx950 kernels: bf16 bit handling, wave64
+// reductions and block reductions with a fixed (deterministic) order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fk {
+
+constexpr int kWave = 64;
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+
+// fp32 -> bf16, round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+// T(v) as a float again: the rounding boundary the reference places on every
+// value it casts to the activation type.
+__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(f32_to_bf16_bits(f) << 16); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// acc + a.lo*b.lo + a.hi*b.hi with bf16 inputs, fp32 accumulate (v_dot2c_f32_bf16).
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
+                                           false);
+}
+
+// Butterfly reductions over `width` adjacent lanes (width a power of two <= 64).
+__device__ __forceinline__ float group_sum(float v, int width) {
+    for (int o = width >> 1; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// Block-wide sum; every thread returns the same value.  `scratch` holds one
+// float per wave plus one.  Waves are added in index order, so the result does
+// not depend on scheduling.
+template <int BLOCK>
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    constexpr int NW = BLOCK / kWave;
+    v = wave_sum(v);
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) t += scratch[i];
+        scratch[NW] = t;
+    }
+    __syncthreads();
+    float r = scratch[NW];
+    __syncthreads();
+    return r;
+}
+
+template <int BLOCK>
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    constexpr int NW = BLOCK / kWave;
+    v = wave_max(v);
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = scratch[0];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) t = fmaxf(t, scratch[i]);
+        scratch[NW] = t;
+    }
+    __syncthreads();
+    float r = scratch[NW];
+    __syncthreads();
+    return r;
+}
+
+}  // namespace fk

@@ -1,0 +1,357 @@
+// Flat-stream weight-streaming GEMV for gfx950 (batch-1 decode).
+//
+// The weight matrix is read as one flat sequence of 16-byte chunks, so every
+// wave load is 1 KiB of contiguous HBM whatever K is.  A chunk holds 32 int4,
+// 16 int8 or 8 bf16 weights of one row and always lies inside one quantization
+// group.  Activations are staged once per (persistent) block into LDS in a
+// chunk-interleaved layout -- piece j of chunk c at uint4 index j*cpr + c -- so
+// that lanes walking consecutive chunks read consecutive 16-byte LDS words.
+// Each lane turns its chunk into one fp32 partial, partials of a tile of R rows
+// go through LDS, and a second phase adds each row's partials in a fixed order
+// and applies the epilogue.  No atomics touch the value path.
+//
+// int4 dequantisation: (w >> 4j) & 0x000F000F picks nibbles j and j+4; OR-ing
+// 0x43004300 makes the two bf16 values 128+q exactly, which v_dot2c_f32_bf16
+// multiplies with the matching activation pair.  The 128 offset and the affine
+// bias fold into one per-chunk correction: s*(D - 128*Sx) + b*Sx, Sx being the
+// chunk's activation sum (computed once per block).
+#pragma once
+#include "fk_device.hpp"
+
+namespace fk {
+
+enum WKind : int { W_Q4 = 0, W_Q8 = 1, W_BF16 = 2 };
+
+constexpr int kGemvBlock = 256;
+constexpr int kGemvUnroll = 4;  // 16-byte loads in flight per lane and batch
+constexpr int kMaxMats = 3;
+
+struct GemvArgs {
+    const uint4* w[kMaxMats];
+    const uint16_t* sc[kMaxMats];
+    const uint16_t* bi[kMaxMats];
+    const uint16_t* bias[kMaxMats];  // optional bf16 projection bias per matrix
+    uint16_t* y[kMaxMats];
+    uint32_t n[kMaxMats];           // rows per matrix
+    uint32_t tile_start[kMaxMats + 1];  // first tile of each matrix (fan-out mode)
+    uint32_t n_mats;
+    uint32_t K;
+    uint32_t cpr;      // 16-byte chunks per row
+    uint32_t gshift;   // chunk index >> gshift = quantization group index
+    uint32_t R;        // rows per tile (per segment)
+    uint32_t n_tiles;
+    uint32_t lr;       // lanes per row in the row-sum phase (power of two)
+    float inv_cpr;
+    const uint16_t* x;       // bf16 activations [K]
+    const uint16_t* norm_w;  // fused RMSNorm weight or null
+    float eps;
+    const uint16_t* res;   // optional residual (matrix 0)
+    const uint16_t* res2;  // optional second residual
+    int swiglu_variant;
+};
+
+template <WKind KIND>
+struct ChunkTraits;
+template <>
+struct ChunkTraits<W_Q4> {
+    static constexpr int kValues = 32, kPieces = 4;
+};
+template <>
+struct ChunkTraits<W_Q8> {
+    static constexpr int kValues = 16, kPieces = 4;
+};
+template <>
+struct ChunkTraits<W_BF16> {
+    static constexpr int kValues = 8, kPieces = 1;
+};
+
+// LDS bytes the kernel needs: staged activations + per-chunk sums + partials + scratch.
+template <WKind KIND>
+__host__ __device__ inline uint32_t gemv_lds_bytes(uint32_t cpr, uint32_t tile_chunks) {
+    return ChunkTraits<KIND>::kPieces * cpr * 16u + cpr * 4u + tile_chunks * 4u + 64u;
+}
+
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t o) { return (a & m) | o; }
+
+__device__ __forceinline__ float q4_word_dot(uint32_t w, uint4 xp, float d) {
+    constexpr uint32_t M = 0x000F000Fu, B = 0x43004300u;
+    d = dot2_bf16(and_or(w, M, B), xp.x, d);
+    d = dot2_bf16(and_or(w >> 4, M, B), xp.y, d);
+    d = dot2_bf16(and_or(w >> 8, M, B), xp.z, d);
+    d = dot2_bf16(and_or(w >> 12, M, B), xp.w, d);
+    return d;
+}
+
+__device__ __forceinline__ float q8_word_dot(uint32_t w, uint4 xf, float d) {
+    d = fmaf((float)(w & 0xffu), __uint_as_float(xf.x), d);
+    d = fmaf((float)((w >> 8) & 0xffu), __uint_as_float(xf.y), d);
+    d = fmaf((float)((w >> 16) & 0xffu), __uint_as_float(xf.z), d);
+    d = fmaf((float)(w >> 24), __uint_as_float(xf.w), d);
+    return d;
+}
+
+// One chunk -> one fp32 partial.
+template <WKind KIND>
+__device__ __forceinline__ float chunk_partial(uint4 wv, uint32_t s_bits, uint32_t b_bits, const uint4* xs,
+                                               const float* sx, uint32_t c, uint32_t cpr) {
+    if constexpr (KIND == W_Q4) {
+        float d = 0.f;
+        d = q4_word_dot(wv.x, xs[c], d);
+        d = q4_word_dot(wv.y, xs[cpr + c], d);
+        d = q4_word_dot(wv.z, xs[2 * cpr + c], d);
+        d = q4_word_dot(wv.w, xs[3 * cpr + c], d);
+        const float s = bf16_bits_to_f32(s_bits), b = bf16_bits_to_f32(b_bits), sum_x = sx[c];
+        return fmaf(s, fmaf(-128.f, sum_x, d), b * sum_x);
+    } else if constexpr (KIND == W_Q8) {
+        float d = 0.f;
+        d = q8_word_dot(wv.x, xs[c], d);
+        d = q8_word_dot(wv.y, xs[cpr + c], d);
+        d = q8_word_dot(wv.z, xs[2 * cpr + c], d);
+        d = q8_word_dot(wv.w, xs[3 * cpr + c], d);
+        const float s = bf16_bits_to_f32(s_bits), b = bf16_bits_to_f32(b_bits);
+        return fmaf(s, d, b * sx[c]);
+    } else {
+        const uint4 xp = xs[c];
+        float d = 0.f;
+        d = dot2_bf16(wv.x, xp.x, d);
+        d = dot2_bf16(wv.y, xp.y, d);
+        d = dot2_bf16(wv.z, xp.z, d);
+        d = dot2_bf16(wv.w, xp.w, d);
+        return d;
+    }
+}
+
+// SwiGLU epilogue on the two fp32 accumulators; the three rounding variants the
+// reference emits (rmsnorm_gateup_swiglu.rs:236-257, msl.rs:1286-1294, msl.rs:2441-2449).
+__device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int variant) {
+    const float g = round_bf16(acc_g), u = round_bf16(acc_u);
+    if (variant == 0) {
+        const float e = round_bf16(expf(fabsf(g)));
+        const float den = round_bf16(1.0f + e);
+        const float sig_y = round_bf16(1.0f / den);
+        const float sig = (g < 0.0f) ? sig_y : round_bf16(1.0f - sig_y);
+        const float silu = round_bf16(g * sig);
+        return f32_to_bf16_bits(silu * u);
+    } else if (variant == 1) {
+        const float sig = 1.0f / (1.0f + expf(-g));
+        return f32_to_bf16_bits((sig * g) * u);
+    } else {
+        const float sig = round_bf16(1.0f / (1.0f + expf(-g)));
+        const float gated = round_bf16(sig * g);
+        return f32_to_bf16_bits(gated * u);
+    }
+}
+
+// Stage x (optionally RMS-normalised: T(w * T(x * r))) into the chunk-interleaved
+// LDS layout and compute the per-chunk sums.  Every thread handles 8 consecutive
+// elements per step.  K must be a multiple of 64.
+template <WKind KIND, bool NORM>
+__device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, float* sx, float* scratch) {
+    const uint32_t K = a.K, cpr = a.cpr, n8 = K >> 3;
+    const uint4* x8 = reinterpret_cast<const uint4*>(a.x);
+    float r = 1.0f;
+    if constexpr (NORM) {
+        float ss = 0.f;
+        for (uint32_t t = threadIdx.x; t < n8; t += kGemvBlock) {
+            const uint4 v = x8[t];
+            const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float lo = bf16_lo(p[i]), hi = bf16_hi(p[i]);
+                ss = fmaf(lo, lo, ss);
+                ss = fmaf(hi, hi, ss);
+            }
+        }
+        ss = block_sum<kGemvBlock>(ss, scratch);
+        r = 1.0f / sqrtf(ss / (float)K + a.eps);
+    }
+    const uint4* w8 = reinterpret_cast<const uint4*>(a.norm_w);
+    for (uint32_t t = threadIdx.x; t < n8; t += kGemvBlock) {
+        const uint4 v = x8[t];
+        const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = bf16_lo(p[i]);
+            f[2 * i + 1] = bf16_hi(p[i]);
+        }
+        if constexpr (NORM) {
+            const uint4 wv = w8[t];
+            const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f[2 * i] = round_bf16(bf16_lo(q[i]) * round_bf16(f[2 * i] * r));
+                f[2 * i + 1] = round_bf16(bf16_hi(q[i]) * round_bf16(f[2 * i + 1] * r));
+            }
+        }
+        if constexpr (KIND == W_Q4) {
+            // word j of chunk c; nibble pairs (0,4) (1,5) (2,6) (3,7)
+            const uint32_t c = t >> 2, j = t & 3u;
+            xs[j * cpr + c] = make_uint4(pack_bf16(f[0], f[4]), pack_bf16(f[1], f[5]), pack_bf16(f[2], f[6]),
+                                         pack_bf16(f[3], f[7]));
+        } else if constexpr (KIND == W_Q8) {
+            const uint32_t c = t >> 1, j = (t & 1u) * 2u;
+            xs[j * cpr + c] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                                         __float_as_uint(f[3]));
+            xs[(j + 1) * cpr + c] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]),
+                                               __float_as_uint(f[6]), __float_as_uint(f[7]));
+        } else {
+            xs[t] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]),
+                               pack_bf16(f[6], f[7]));
+        }
+    }
+    __syncthreads();
+    if constexpr (KIND != W_BF16) {
+        for (uint32_t c = threadIdx.x; c < cpr; c += kGemvBlock) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint4 v = xs[j * cpr + c];
+                if constexpr (KIND == W_Q4) {
+                    s += (bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y)) +
+                         (bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w));
+                } else {
+                    s += (__uint_as_float(v.x) + __uint_as_float(v.y)) +
+                         (__uint_as_float(v.z) + __uint_as_float(v.w));
+                }
+            }
+            sx[c] = s;
+        }
+    }
+    __syncthreads();
+}
+
+// NSEG = 1: fan-out over up to three matrices sharing x (plain GEMV, QKV,
+//           residual projections, LM head); each tile lies inside one matrix.
+// NSEG = 2: gate/up pair; a tile holds R gate rows and the same R up rows and
+//           the epilogue is SwiGLU.
+template <WKind KIND, int NSEG, bool NORM>
+__global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    constexpr int PIECES = ChunkTraits<KIND>::kPieces;
+    constexpr uint32_t BATCH = kGemvBlock * kGemvUnroll;
+    const uint32_t cpr = a.cpr, R = a.R;
+    const uint32_t seg_chunks = R * cpr;          // chunks of one segment of a full tile
+    const uint32_t tile_chunks = NSEG * seg_chunks;
+
+    uint4* xs = lds_raw;
+    float* sx = reinterpret_cast<float*>(xs + PIECES * cpr);
+    float* part = sx + cpr;
+    float* scratch = part + tile_chunks;
+
+    // Resolves a tile to (matrix, first row, valid rows).
+    auto tile_rows = [&](uint32_t tile, uint32_t& m, uint32_t& row0, uint32_t& valid) {
+        if constexpr (NSEG == 2) {
+            m = 0;
+            row0 = tile * R;
+        } else {
+            m = (a.n_mats > 1 && tile >= a.tile_start[1]) ? ((a.n_mats > 2 && tile >= a.tile_start[2]) ? 2u : 1u)
+                                                          : 0u;
+            row0 = (tile - a.tile_start[m]) * R;
+        }
+        const uint32_t left = a.n[m] - row0;
+        valid = left < R ? left : R;
+    };
+
+    // Issues the 16-byte weight loads (and scale/bias) of one batch into registers.
+    auto load_batch = [&](uint4(&wv)[kGemvUnroll], uint32_t(&sb)[kGemvUnroll], uint32_t tile, uint32_t b0) {
+        uint32_t m, row0, valid;
+        tile_rows(tile, m, row0, valid);
+        const uint32_t valid_chunks = valid * cpr;
+#pragma unroll
+        for (int j = 0; j < kGemvUnroll; ++j) {
+            const uint32_t u = b0 + j * kGemvBlock + threadIdx.x;
+            uint32_t mm = m, uu = u;
+            if constexpr (NSEG == 2) {
+                if (u >= seg_chunks) {
+                    mm = 1;
+                    uu = u - seg_chunks;
+                }
+            }
+            wv[j] = make_uint4(0, 0, 0, 0);
+            sb[j] = 0;
+            if (u < tile_chunks && uu < valid_chunks) {
+                const size_t flat = (size_t)row0 * cpr + uu;
+                wv[j] = a.w[mm][flat];
+                if constexpr (KIND != W_BF16) {
+                    const size_t g = flat >> a.gshift;
+                    sb[j] = (uint32_t)a.sc[mm][g] | ((uint32_t)a.bi[mm][g] << 16);
+                }
+            }
+        }
+    };
+
+    uint32_t tile = blockIdx.x, b0 = 0;
+
+    // Consumes the batch held in (cur, curs) while the following batch streams
+    // into (nxt, nxts).  Returns false once this block has no tile left.
+    auto step = [&](uint4(&cur)[kGemvUnroll], uint32_t(&curs)[kGemvUnroll], uint4(&nxt)[kGemvUnroll],
+                    uint32_t(&nxts)[kGemvUnroll]) -> bool {
+        uint32_t ntile = tile, nb0 = b0 + BATCH;
+        if (nb0 >= tile_chunks) {
+            ntile = tile + gridDim.x;
+            nb0 = 0;
+        }
+        if (ntile < a.n_tiles) load_batch(nxt, nxts, ntile, nb0);
+
+#pragma unroll
+        for (int j = 0; j < kGemvUnroll; ++j) {
+            const uint32_t u = b0 + j * kGemvBlock + threadIdx.x;
+            if (u < tile_chunks) {
+                uint32_t uu = u;
+                if constexpr (NSEG == 2) uu = (u >= seg_chunks) ? u - seg_chunks : u;
+                const uint32_t row = (uint32_t)(((float)uu + 0.5f) * a.inv_cpr);
+                const uint32_t c = uu - row * cpr;
+                part[u] = chunk_partial<KIND>(cur[j], curs[j] & 0xffffu, curs[j] >> 16, xs, sx, c, cpr);
+            }
+        }
+
+        if (ntile != tile) {
+            // tile complete: add each row's partials in a fixed order, then the epilogue
+            __syncthreads();
+            uint32_t m, row0, valid;
+            tile_rows(tile, m, row0, valid);
+            const uint32_t lr = a.lr, lane = threadIdx.x & (lr - 1);
+            for (uint32_t rr = threadIdx.x / lr; rr < R; rr += kGemvBlock / lr) {
+                float s0 = 0.f, s1 = 0.f;
+                for (uint32_t i = lane; i < cpr; i += lr) {
+                    s0 += part[rr * cpr + i];
+                    if constexpr (NSEG == 2) s1 += part[seg_chunks + rr * cpr + i];
+                }
+                s0 = group_sum(s0, lr);
+                if constexpr (NSEG == 2) s1 = group_sum(s1, lr);
+                if (lane == 0 && rr < valid) {
+                    const uint32_t n = row0 + rr;
+                    if constexpr (NSEG == 2) {
+                        a.y[0][n] = (uint16_t)swiglu_bits(s0, s1, a.swiglu_variant);
+                    } else {
+                        float v = s0;
+                        if (a.bias[m]) v += bf16_bits_to_f32(a.bias[m][n]);
+                        if (m == 0 && a.res) v += bf16_bits_to_f32(a.res[n]);
+                        uint32_t o = f32_to_bf16_bits(v);
+                        if (m == 0 && a.res2)
+                            o = f32_to_bf16_bits(bf16_bits_to_f32(o) + bf16_bits_to_f32(a.res2[n]));
+                        a.y[m][n] = (uint16_t)o;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        tile = ntile;
+        b0 = nb0;
+        return tile < a.n_tiles;
+    };
+
+    uint4 wa[kGemvUnroll], wb[kGemvUnroll];
+    uint32_t sa[kGemvUnroll], sbb[kGemvUnroll];
+    const bool has_work = tile < a.n_tiles;
+    if (has_work) load_batch(wa, sa, tile, 0);  // weights start streaming before x is staged
+    stage_activations<KIND, NORM>(a, xs, sx, scratch);
+    if (!has_work) return;
+    while (true) {
+        if (!step(wa, sa, wb, sbb)) break;
+        if (!step(wb, sbb, wa, sa)) break;
+    }
+}
+
+}  // namespace fk

@@ -1,0 +1,187 @@
+"""ctypes binding of libfusekit_hip.so (the C ABI in include/fusekit_hip.h).
+
+Mirrors how the reference's Python runtime talks to `_fusekit_runtime_native`
+(reference python/fusekit_runtime/dispatch.py -> python_runtime/src/lib.rs):
+Python owns no arithmetic, only pointers and sizes.  bf16 tensors travel as
+numpy uint16 bit patterns.  Loading fails loudly when the library is missing;
+there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfusekit_hip.so")
+
+FK_OK, FK_ERR_INVALID, FK_ERR_IO, FK_ERR_NOT_FOUND, FK_ERR_HIP, FK_ERR_UNSUPPORTED = range(6)
+
+
+class FusekitError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"[fk_status {status}] {message}")
+        self.status = status
+
+
+class InvalidArgument(FusekitError, ValueError):
+    """FK_ERR_INVALID: what the reference raises as PyValueError."""
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(hipcc, gfx950). fusekit_amd has no CPU fallback."
+        )
+    return C.CDLL(LIB_PATH)
+
+
+lib = _load()
+lib.fk_last_error.restype = C.c_char_p
+lib.fk_version.restype = C.c_char_p
+
+
+def check(status: int) -> None:
+    if status != FK_OK:
+        msg = lib.fk_last_error().decode("utf-8", "replace")
+        if status == FK_ERR_INVALID:
+            raise InvalidArgument(status, msg)
+        raise FusekitError(status, msg)
+
+
+def version() -> str:
+    return lib.fk_version().decode()
+
+
+class DeviceProps(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 128), ("arch", C.c_char * 32), ("compute_units", C.c_int), ("wavefront", C.c_int),
+        ("lds_bytes_per_block", C.c_int), ("l2_bytes", C.c_int), ("hbm_bytes", C.c_uint64), ("clock_khz", C.c_int),
+    ]
+
+
+def device_props() -> DeviceProps:
+    p = DeviceProps()
+    check(lib.fk_device_props_get(C.byref(p)))
+    return p
+
+
+def has_device() -> bool:
+    p = DeviceProps()
+    return lib.fk_device_props_get(C.byref(p)) == FK_OK
+
+
+class Weight(C.Structure):
+    """`fk_weight`."""
+
+    _fields_ = [
+        ("w", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p),
+        ("n", C.c_uint32), ("k", C.c_uint32), ("bits", C.c_uint32), ("group", C.c_uint32),
+    ]
+
+
+class DeviceBuffer:
+    """One device allocation owned through fk_alloc / fk_free."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        check(lib.fk_alloc(C.c_size_t(max(self.nbytes, 1)), C.byref(p)))
+        self.ptr = p.value
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        if a.nbytes:
+            check(lib.fk_upload(C.c_void_p(b.ptr), a.ctypes.data_as(C.c_void_p), C.c_size_t(a.nbytes)))
+        return b
+
+    def upload(self, a: np.ndarray, offset: int = 0) -> None:
+        a = np.ascontiguousarray(a)
+        assert offset + a.nbytes <= self.nbytes
+        check(lib.fk_upload(C.c_void_p(self.ptr + offset), a.ctypes.data_as(C.c_void_p), C.c_size_t(a.nbytes)))
+
+    def to_numpy(self, dtype, shape=None, offset: int = 0) -> np.ndarray:
+        dtype = np.dtype(dtype)
+        if shape is None:
+            shape = ((self.nbytes - offset) // dtype.itemsize,)
+        out = np.empty(shape, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(lib.fk_download(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr + offset),
+                                  C.c_size_t(out.nbytes)))
+        return out
+
+    def free(self) -> None:
+        if getattr(self, "ptr", None):
+            lib.fk_free(C.c_void_p(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class DeviceWeight:
+    """A weight matrix resident in HBM (packed + scales + biases, or dense bf16)."""
+
+    def __init__(self, w: np.ndarray, scales, biases, n: int, k: int, bits: int, group: int = 64):
+        self.n, self.k, self.bits, self.group = int(n), int(k), int(bits), int(group)
+        self.w = DeviceBuffer.from_numpy(w)
+        self.scales = None if scales is None else DeviceBuffer.from_numpy(np.asarray(scales, dtype=np.uint16))
+        self.biases = None if biases is None else DeviceBuffer.from_numpy(np.asarray(biases, dtype=np.uint16))
+
+    @property
+    def c(self) -> Weight:
+        return Weight(self.w.ptr, self.scales.ptr if self.scales else None,
+                      self.biases.ptr if self.biases else None, self.n, self.k, self.bits, self.group)
+
+    @property
+    def nbytes(self) -> int:
+        return self.w.nbytes + (self.scales.nbytes + self.biases.nbytes if self.scales else 0)
+
+
+def _ptr(b) -> C.c_void_p:
+    if b is None:
+        return C.c_void_p(None)
+    if isinstance(b, DeviceBuffer):
+        return C.c_void_p(b.ptr)
+    return C.c_void_p(int(b))
+
+
+# ---------------------------------------------------------------- operators
+
+def qgemv(W: DeviceWeight, x, bias, y, stream=None) -> None:
+    check(lib.fk_qgemv(C.byref(W.c), _ptr(x), _ptr(bias), _ptr(y), _ptr(stream)))
+
+
+def linear_residual(W: DeviceWeight, x, res, res2, y, stream=None) -> None:
+    check(lib.fk_linear_residual(C.byref(W.c), _ptr(x), _ptr(res), _ptr(res2), _ptr(y), _ptr(stream)))
+
+
+def rmsnorm_qkv(x, norm_w, eps, Wq, Wk, Wv, bq, bk, bv, q, k, v, stream=None) -> None:
+    check(lib.fk_rmsnorm_qkv(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(Wq.c), C.byref(Wk.c), C.byref(Wv.c),
+                             _ptr(bq), _ptr(bk), _ptr(bv), _ptr(q), _ptr(k), _ptr(v), _ptr(stream)))
+
+
+def gateup_swiglu(x, norm_w, eps, Wg, Wu, variant, out, stream=None) -> None:
+    check(lib.fk_gateup_swiglu(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(Wg.c), C.byref(Wu.c),
+                               C.c_int(variant), _ptr(out), _ptr(stream)))
+
+
+def final_rmsnorm_lm_head(x, norm_w, eps, W, logits, stream=None) -> None:
+    check(lib.fk_final_rmsnorm_lm_head(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(W.c), _ptr(logits),
+                                       _ptr(stream)))
+
+
+def set_gemv_policy(rows_per_tile: int = 0, grid_blocks: int = 0) -> None:
+    check(lib.fk_set_gemv_policy(C.c_uint32(rows_per_tile), C.c_uint32(grid_blocks)))
+
+
+def sync(stream=None) -> None:
+    check(lib.fk_stream_sync(_ptr(stream)))

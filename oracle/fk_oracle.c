@@ -1,0 +1,598 @@
+/*
+ * fk_oracle.c -- CPU restatement of the decode hot path of Pribess/FuseKit.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only tests/, the smoke check
+ * and the benchmark's cpu_baseline leg may load it, and only as the checker or
+ * the reported CPU baseline.  The shipped library never links or calls it.
+ *
+ * The arithmetic that FuseKit's emitted Metal kernels perform ultimately
+ * mirrors MLX (Apple, v0.31.2 per reference BENCHMARKS.md:16): mx.quantize,
+ * mx.quantized_matmul, mx.fast.rms_norm, mx.fast.rope and
+ * mx.fast.scaled_dot_product_attention.  MLX is not vendored in the reference
+ * and is not installed here; the reference holds no golden vectors for this
+ * path.  Each function below therefore follows the reference's own statement
+ * of the arithmetic (file:line cited per function, paths relative to the
+ * reference root) and is pinned by tests/test_oracle_*.py through closed
+ * forms, invariants, brute force and an independent numpy formulation.
+ *
+ * Pin status per function (see tests/test_oracle_pins.py):
+ *   quantize/pack/unpack ........ pinned (exhaustive nibble/lane, invariants)
+ *   qgemv / linear .............. pinned (numpy float64 matmul on dequant W)
+ *   rms_norm .................... pinned (closed forms + numpy restatement)
+ *   rope ........................ pinned (norm preservation, pos 0, composition)
+ *   swiglu A/B/C ................ pinned (numpy restatement per variant; A vs B
+ *                                 vs C agree within bf16 noise)
+ *   sdpa_decode ................. pinned (float64 softmax attention; kv_len=1;
+ *                                 chunk-merge invariance)
+ *   argmax ...................... pinned (brute force, tie rule)
+ *   MLX-internal accumulation order, Metal fast::cos/sin/exp bit patterns:
+ *                                 parity unpinned (cannot be observed here;
+ *                                 irrelevant under the rel-L2 <= 1e-2 bar).
+ *
+ * Conventions: activations "T" are bfloat16 held as uint16_t bit patterns;
+ * every T(...) in the reference is a round-to-nearest-even fp32->bf16 here.
+ * Dot products accumulate in double and are narrowed to float once, so the
+ * oracle is the closest fp32 value any summation order may aim for.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define FKO_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ bf16 */
+
+static inline float bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline uint16_t f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+static inline float rbf(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+FKO_API void fko_f32_to_bf16(const float *in, uint16_t *out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = f32_to_bf16(in[i]);
+}
+FKO_API void fko_bf16_to_f32(const uint16_t *in, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = bf16_to_f32(in[i]);
+}
+
+FKO_API int fko_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+FKO_API void fko_set_num_threads(int n) {
+#ifdef _OPENMP
+    omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
+/* ------------------------------------------------------- Q0: quantizer */
+/*
+ * MLX-affine quantizer, restated from the reference's own restatement at
+ * src/codegen/kernels/rope_kv_cache_store_decode_quant.rs:208-221 (same block
+ * in src/codegen/kernels/rmsnorm_qkv.rs:565-580); layout per
+ * src/fusion/ir.rs:236-242 and scripts/poc_int4_gemv.py:19-24:
+ *   packed u32 [N, K*bits/32], value j of a word at bits (j*bits), LSB first;
+ *   scales/biases T [N, K/group].
+ * The scale/bias are rounded to T *after* the integer codes are chosen from
+ * the fp32 scale/bias, as in the reference (codes from fp32, meta stored T).
+ */
+FKO_API void fko_quantize_affine(const float *w, int64_t n, int64_t k, int bits, int group,
+                                 uint32_t *packed, uint16_t *scales, uint16_t *biases) {
+    const int per_word = 32 / bits;
+    const int mask = (1 << bits) - 1;
+    const int64_t words = k / per_word, groups = k / group;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < n; ++r) {
+        const float *row = w + r * k;
+        uint32_t *prow = packed + r * words;
+        memset(prow, 0, (size_t)words * 4);
+        for (int64_t g = 0; g < groups; ++g) {
+            const float *x = row + g * group;
+            float vmin = x[0], vmax = x[0];
+            for (int i = 1; i < group; ++i) {
+                vmin = x[i] < vmin ? x[i] : vmin;
+                vmax = x[i] > vmax ? x[i] : vmax;
+            }
+            float scale_abs = fmaxf((vmax - vmin) / (float)mask, 1.0e-7f);
+            int lo_anchor = fabsf(vmin) > fabsf(vmax);
+            float scale = lo_anchor ? scale_abs : -scale_abs;
+            float edge = lo_anchor ? vmin : vmax;
+            float q0 = roundf(edge / scale);
+            int at_zero = (q0 == 0.0f);
+            scale = at_zero ? scale : (edge / q0);
+            float bias = at_zero ? 0.0f : edge;
+            float inv_scale = (scale != 0.0f) ? (1.0f / scale) : 0.0f;
+            for (int i = 0; i < group; ++i) {
+                int qi = (int)roundf((x[i] - bias) * inv_scale);
+                qi = qi < 0 ? 0 : (qi > mask ? mask : qi);
+                int64_t col = g * group + i;
+                prow[col / per_word] |= ((uint32_t)qi & (uint32_t)mask) << ((col % per_word) * bits);
+            }
+            scales[r * groups + g] = f32_to_bf16(scale);
+            biases[r * groups + g] = f32_to_bf16(bias);
+        }
+    }
+}
+
+/* w[i,j] = q(packed[i, j/per_word], j%per_word) * scales[i, j/g] + biases[i, j/g]
+ * (src/fusion/ir.rs:236-242).  Integer codes out for the bit-exact tests. */
+FKO_API void fko_unpack_codes(const uint32_t *packed, int64_t n, int64_t k, int bits, uint8_t *codes) {
+    const int per_word = 32 / bits;
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int64_t r = 0; r < n; ++r)
+        for (int64_t j = 0; j < k; ++j)
+            codes[r * k + j] =
+                (uint8_t)((packed[r * (k / per_word) + j / per_word] >> ((j % per_word) * bits)) & mask);
+}
+
+FKO_API void fko_dequantize(const uint32_t *packed, const uint16_t *scales, const uint16_t *biases,
+                            int64_t n, int64_t k, int bits, int group, float *out) {
+    const int per_word = 32 / bits;
+    const uint32_t mask = (1u << bits) - 1u;
+    const int64_t words = k / per_word, groups = k / group;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < n; ++r)
+        for (int64_t j = 0; j < k; ++j) {
+            uint32_t q = (packed[r * words + j / per_word] >> ((j % per_word) * bits)) & mask;
+            float s = bf16_to_f32(scales[r * groups + j / group]);
+            float b = bf16_to_f32(biases[r * groups + j / group]);
+            out[r * k + j] = (float)q * s + b;
+        }
+}
+
+/* --------------------------------------------------------- K1: linear */
+/*
+ * One weight matrix [n, k] in one of three storage kinds:
+ *   bits 4 / 8 : MLX-affine (packed, scales, biases, group)
+ *   bits 16    : dense bf16 (packed points at uint16 data, scales/biases NULL)
+ */
+typedef struct {
+    const void *w;
+    const uint16_t *scales;
+    const uint16_t *biases;
+    int64_t n, k;
+    int bits, group;
+} fko_weight;
+
+/* acc[i] = sum_k x[k] * (q*s + b), the per-element form of
+ * src/codegen/kernels/mod.rs:2850-2908 (q4) and :3053-3104 (q8); dense rows
+ * as src/codegen/kernels/linear_residual.rs:342-346.  x is fp32 holding values
+ * the caller already rounded to T where the reference does. */
+static void linear_acc(const fko_weight *W, const float *x, float *acc) {
+    const int64_t n = W->n, k = W->k;
+    if (W->bits == 16) {
+        const uint16_t *d = (const uint16_t *)W->w;
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < n; ++r) {
+            double a = 0.0;
+            const uint16_t *row = d + r * k;
+            for (int64_t j = 0; j < k; ++j) a += (double)x[j] * (double)bf16_to_f32(row[j]);
+            acc[r] = (float)a;
+        }
+        return;
+    }
+    const int bits = W->bits, per_word = 32 / bits, group = W->group;
+    const uint32_t mask = (1u << bits) - 1u;
+    const int64_t words = k / per_word, groups = k / group;
+    const uint32_t *p = (const uint32_t *)W->w;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < n; ++r) {
+        double a = 0.0;
+        const uint32_t *prow = p + r * words;
+        for (int64_t g = 0; g < groups; ++g) {
+            const float s = bf16_to_f32(W->scales[r * groups + g]);
+            const float b = bf16_to_f32(W->biases[r * groups + g]);
+            for (int i = 0; i < group; ++i) {
+                int64_t j = g * group + i;
+                uint32_t q = (prow[j / per_word] >> ((j % per_word) * bits)) & mask;
+                float wv = (float)q * s + b; /* fp32 dequant as in the reference */
+                a += (double)x[j] * (double)wv;
+            }
+        }
+        acc[r] = (float)a;
+    }
+}
+
+FKO_API void fko_linear_acc(const fko_weight *W, const uint16_t *x_bf16, float *acc) {
+    float *x = (float *)malloc(sizeof(float) * (size_t)W->k);
+    for (int64_t j = 0; j < W->k; ++j) x[j] = bf16_to_f32(x_bf16[j]);
+    linear_acc(W, x, acc);
+    free(x);
+}
+
+/* y = T(acc (+bias)) : quantized GEMV with one final round
+ * (src/codegen/msl.rs:434-438); bias added in fp32 before the round
+ * (src/codegen/kernels/rmsnorm_qkv.rs:417-422). */
+FKO_API void fko_qgemv(const fko_weight *W, const uint16_t *x, const uint16_t *bias, uint16_t *y) {
+    float *acc = (float *)malloc(sizeof(float) * (size_t)W->n);
+    fko_linear_acc(W, x, acc);
+    for (int64_t i = 0; i < W->n; ++i) {
+        float a = acc[i];
+        if (bias) a += bf16_to_f32(bias[i]);
+        y[i] = f32_to_bf16(a);
+    }
+    free(acc);
+}
+
+/* K1r: y = T(acc + float(res)); optional second residual rounds twice
+ * (src/codegen/kernels/linear_residual.rs:374-381). */
+FKO_API void fko_linear_residual(const fko_weight *W, const uint16_t *x, const uint16_t *res,
+                                 const uint16_t *res2, uint16_t *y) {
+    float *acc = (float *)malloc(sizeof(float) * (size_t)W->n);
+    fko_linear_acc(W, x, acc);
+    for (int64_t i = 0; i < W->n; ++i) {
+        uint16_t y0 = f32_to_bf16(acc[i] + (res ? bf16_to_f32(res[i]) : 0.0f));
+        if (res2) y0 = f32_to_bf16(bf16_to_f32(y0) + bf16_to_f32(res2[i]));
+        y[i] = y0;
+    }
+    free(acc);
+}
+
+/* ------------------------------------------------------------ N: norm */
+/* r = rsqrt(sum(x^2)/H + eps) (precise rsqrt, src/codegen/kernels/rmsnorm_qkv.rs:325);
+ * norm_y[i] = float(T(w[i] * T(x[i] * r))) (src/codegen/kernels/mod.rs:4464-4472). */
+static void rmsnorm_f(const uint16_t *x, const uint16_t *w, int64_t h, float eps, float *out) {
+    double ss = 0.0;
+    for (int64_t i = 0; i < h; ++i) {
+        double v = bf16_to_f32(x[i]);
+        ss += v * v;
+    }
+    float r = 1.0f / sqrtf((float)ss / (float)h + eps);
+    for (int64_t i = 0; i < h; ++i) {
+        float t = rbf(bf16_to_f32(x[i]) * r);
+        out[i] = rbf(bf16_to_f32(w[i]) * t);
+    }
+}
+
+FKO_API void fko_rmsnorm(const uint16_t *x, const uint16_t *w, int64_t h, float eps, uint16_t *y) {
+    float *o = (float *)malloc(sizeof(float) * (size_t)h);
+    rmsnorm_f(x, w, h, eps, o);
+    for (int64_t i = 0; i < h; ++i) y[i] = f32_to_bf16(o[i]);
+    free(o);
+}
+
+/* ------------------------------------------------------------ K2: QKV */
+/* Non-sink variant of src/codegen/kernels/rmsnorm_qkv.rs:53-736: norm into
+ * fp32 scratch, three projections, bf16 bias added before the round. */
+FKO_API void fko_rmsnorm_qkv(const uint16_t *x, const uint16_t *norm_w, float eps, const fko_weight *Wq,
+                             const fko_weight *Wk, const fko_weight *Wv, const uint16_t *bq,
+                             const uint16_t *bk, const uint16_t *bv, uint16_t *q, uint16_t *k,
+                             uint16_t *v) {
+    const int64_t h = Wq->k;
+    float *ny = (float *)malloc(sizeof(float) * (size_t)h);
+    rmsnorm_f(x, norm_w, h, eps, ny);
+    const fko_weight *Ws[3] = {Wq, Wk, Wv};
+    const uint16_t *bs[3] = {bq, bk, bv};
+    uint16_t *outs[3] = {q, k, v};
+    for (int m = 0; m < 3; ++m) {
+        float *acc = (float *)malloc(sizeof(float) * (size_t)Ws[m]->n);
+        linear_acc(Ws[m], ny, acc);
+        for (int64_t i = 0; i < Ws[m]->n; ++i) {
+            float a = acc[i];
+            if (bs[m]) a += bf16_to_f32(bs[m][i]);
+            outs[m][i] = f32_to_bf16(a);
+        }
+        free(acc);
+    }
+    free(ny);
+}
+
+/* ---------------------------------------------------------- K3a: SwiGLU */
+/* variant 0 ("A"): every op in T -- src/codegen/kernels/rmsnorm_gateup_swiglu.rs:236-257
+ * variant 1 ("B"): fp32 sigmoid, one round -- src/codegen/msl.rs:1286-1294
+ * variant 2 ("C"): rounds sig and gated -- src/codegen/msl.rs:2441-2449      */
+static uint16_t swiglu_apply(float acc_g, float acc_u, int variant) {
+    float g = rbf(acc_g), u = rbf(acc_u);
+    if (variant == 0) {
+        float e = rbf(expf(fabsf(g)));
+        float den = rbf(1.0f + e);
+        float sig_y = rbf(1.0f / den);
+        float sig = (g < 0.0f) ? sig_y : rbf(1.0f - sig_y);
+        float silu = rbf(g * sig);
+        return f32_to_bf16(silu * u);
+    } else if (variant == 1) {
+        float sig = 1.0f / (1.0f + expf(-g));
+        return f32_to_bf16((sig * g) * u);
+    } else {
+        float sig = rbf(1.0f / (1.0f + expf(-g)));
+        float gated = rbf(sig * g);
+        return f32_to_bf16(gated * u);
+    }
+}
+
+FKO_API uint16_t fko_swiglu_scalar(float acc_g, float acc_u, int variant) {
+    return swiglu_apply(acc_g, acc_u, variant);
+}
+
+/* norm_w == NULL: x is consumed as is (QmvSwiglu, src/codegen/kernels/qmv_swiglu.rs:20-246);
+ * otherwise RmsNormGateUpSwiglu (src/codegen/kernels/rmsnorm_gateup_swiglu.rs:27-267). */
+FKO_API void fko_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps, const fko_weight *Wg,
+                               const fko_weight *Wu, int variant, uint16_t *out) {
+    const int64_t h = Wg->k, n = Wg->n;
+    float *ny = (float *)malloc(sizeof(float) * (size_t)h);
+    if (norm_w)
+        rmsnorm_f(x, norm_w, h, eps, ny);
+    else
+        for (int64_t i = 0; i < h; ++i) ny[i] = bf16_to_f32(x[i]);
+    float *ag = (float *)malloc(sizeof(float) * (size_t)n);
+    float *au = (float *)malloc(sizeof(float) * (size_t)n);
+    linear_acc(Wg, ny, ag);
+    linear_acc(Wu, ny, au);
+    for (int64_t i = 0; i < n; ++i) out[i] = swiglu_apply(ag[i], au[i], variant);
+    free(ny);
+    free(ag);
+    free(au);
+}
+
+/* ------------------------------------------------------------- R: RoPE */
+/* Half-split RoPE, pair (d, d+half): inv = exp2(-(d/half) * log2(theta)) with
+ * log2(theta) computed in double then narrowed to float; angle = pos * inv in
+ * fp32 (src/codegen/kernels/rope_q_decode.rs:93-114).  The reference uses
+ * Metal fast::cos/sin; libm cosf/sinf stand in (bit patterns unpinned). */
+static inline void rope_pair(float lo, float hi, int64_t d, int64_t half, uint32_t pos, float base_log2,
+                             float *olo, float *ohi) {
+    float d_norm = (float)d / (float)half;
+    float inv_freq = exp2f(-d_norm * base_log2);
+    float angle = (float)pos * inv_freq;
+    float c = cosf(angle), s = sinf(angle);
+    *olo = lo * c - hi * s;
+    *ohi = hi * c + lo * s;
+}
+
+/* In-place on q [n_heads, head_dim]; rotates the first rope_dims of each head. */
+FKO_API void fko_rope_q(uint16_t *q, int64_t n_heads, int64_t head_dim, int64_t rope_dims, float theta,
+                        uint32_t pos) {
+    const float base_log2 = (float)log2((double)theta);
+    const int64_t half = rope_dims / 2;
+    for (int64_t h = 0; h < n_heads; ++h)
+        for (int64_t d = 0; d < half; ++d) {
+            uint16_t *p = q + h * head_dim;
+            float lo, hi;
+            rope_pair(bf16_to_f32(p[d]), bf16_to_f32(p[d + half]), d, half, pos, base_log2, &lo, &hi);
+            p[d] = f32_to_bf16(lo);
+            p[d + half] = f32_to_bf16(hi);
+        }
+}
+
+/* RoPE(K) then store K,V at cache row (write_offset % capacity); cache layout
+ * [n_kv, capacity, head_dim] (src/codegen/kernels/rope_kv_cache_store_decode.rs:87-137). */
+FKO_API void fko_rope_kv_store(const uint16_t *k, const uint16_t *v, int64_t n_kv, int64_t head_dim,
+                               int64_t rope_dims, float theta, uint32_t pos, uint32_t write_offset,
+                               uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v) {
+    const float base_log2 = (float)log2((double)theta);
+    const int64_t half = rope_dims / 2;
+    const int64_t row = write_offset % capacity;
+    for (int64_t h = 0; h < n_kv; ++h) {
+        uint16_t *ck = cache_k + (h * (int64_t)capacity + row) * head_dim;
+        uint16_t *cv = cache_v + (h * (int64_t)capacity + row) * head_dim;
+        const uint16_t *kh = k + h * head_dim;
+        for (int64_t d = 0; d < head_dim; ++d) ck[d] = kh[d];
+        for (int64_t d = 0; d < half; ++d) {
+            float lo, hi;
+            rope_pair(bf16_to_f32(kh[d]), bf16_to_f32(kh[d + half]), d, half, pos, base_log2, &lo, &hi);
+            ck[d] = f32_to_bf16(lo);
+            ck[d + half] = f32_to_bf16(hi);
+        }
+        for (int64_t d = 0; d < head_dim; ++d) cv[d] = v[h * head_dim + d];
+    }
+}
+
+/* Per-head RMSNorm T(w*T(x*r)) followed by RoPE on the normed T values
+ * (src/codegen/kernels/rmsnorm_rope_kv_cache_store_decode.rs:101-152; the q
+ * side follows src/codegen/kernels/rmsnorm_rope_qgate_decode.rs:84-136 without
+ * the gate half).  In place on [n_heads, head_dim]. */
+FKO_API void fko_headnorm_rope(uint16_t *x, const uint16_t *w, int64_t n_heads, int64_t head_dim,
+                               int64_t rope_dims, float eps, float theta, uint32_t pos) {
+    const float base_log2 = (float)log2((double)theta);
+    const int64_t half = rope_dims / 2;
+    float *ny = (float *)malloc(sizeof(float) * (size_t)head_dim);
+    for (int64_t h = 0; h < n_heads; ++h) {
+        uint16_t *p = x + h * head_dim;
+        rmsnorm_f(p, w, head_dim, eps, ny);
+        for (int64_t d = 0; d < head_dim; ++d) p[d] = f32_to_bf16(ny[d]);
+        for (int64_t d = 0; d < half; ++d) {
+            float lo, hi;
+            rope_pair(ny[d], ny[d + half], d, half, pos, base_log2, &lo, &hi);
+            p[d] = f32_to_bf16(lo);
+            p[d + half] = f32_to_bf16(hi);
+        }
+    }
+    free(ny);
+}
+
+/* Plain store of prepared K/V rows (no rope, no norm). */
+FKO_API void fko_kv_store(const uint16_t *k, const uint16_t *v, int64_t n_kv, int64_t k_dim, int64_t v_dim,
+                          uint32_t write_offset, uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v) {
+    const int64_t row = write_offset % capacity;
+    for (int64_t h = 0; h < n_kv; ++h) {
+        memcpy(cache_k + (h * (int64_t)capacity + row) * k_dim, k + h * k_dim, (size_t)k_dim * 2);
+        memcpy(cache_v + (h * (int64_t)capacity + row) * v_dim, v + h * v_dim, (size_t)v_dim * 2);
+    }
+}
+
+/* ------------------------------------------------------------ K4: SDPA */
+/* s_j = (q . k_j) * scale in fp32; softmax in fp32 (probabilities never
+ * rounded to T); o = sum p_j v_j / l; one final round
+ * (src/codegen/kernels/sdpa_decode.rs:1064-1211); GQA kv_head = head /
+ * (n_heads / n_kv) (:393); caches [n_kv, capacity, dim] (:799,868). */
+FKO_API void fko_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v,
+                             int64_t n_heads, int64_t n_kv, int64_t qk_dim, int64_t v_dim,
+                             uint32_t kv_len, uint32_t capacity, float scale, uint16_t *out) {
+    const int64_t per_kv = n_heads / n_kv;
+#pragma omp parallel for schedule(static)
+    for (int64_t h = 0; h < n_heads; ++h) {
+        const int64_t kvh = h / per_kv;
+        float *s = (float *)malloc(sizeof(float) * (size_t)kv_len);
+        float m = -INFINITY;
+        for (uint32_t j = 0; j < kv_len; ++j) {
+            const uint16_t *kr = cache_k + (kvh * (int64_t)capacity + j) * qk_dim;
+            double dot = 0.0;
+            for (int64_t d = 0; d < qk_dim; ++d)
+                dot += (double)bf16_to_f32(q[h * qk_dim + d]) * (double)bf16_to_f32(kr[d]);
+            s[j] = (float)dot * scale;
+            m = s[j] > m ? s[j] : m;
+        }
+        double l = 0.0;
+        for (uint32_t j = 0; j < kv_len; ++j) {
+            s[j] = expf(s[j] - m);
+            l += s[j];
+        }
+        for (int64_t d = 0; d < v_dim; ++d) {
+            double o = 0.0;
+            for (uint32_t j = 0; j < kv_len; ++j)
+                o += (double)s[j] * (double)bf16_to_f32(cache_v[(kvh * (int64_t)capacity + j) * v_dim + d]);
+            out[h * v_dim + d] = f32_to_bf16((float)(o / l));
+        }
+        free(s);
+    }
+}
+
+/* -------------------------------------------------------- E / H / A / U */
+/* x = T(embed[token] * scale) (src/codegen/kernels/embed_lookup_decode.rs:74-99). */
+FKO_API void fko_embed_lookup(const fko_weight *E, uint32_t token, float out_scale, uint16_t *x) {
+    const int64_t k = E->k;
+    if (E->bits == 16) {
+        const uint16_t *row = (const uint16_t *)E->w + (int64_t)token * k;
+        for (int64_t d = 0; d < k; ++d) x[d] = f32_to_bf16(bf16_to_f32(row[d]) * out_scale);
+        return;
+    }
+    const int bits = E->bits, per_word = 32 / bits;
+    const uint32_t mask = (1u << bits) - 1u;
+    const int64_t words = k / per_word, groups = k / E->group;
+    const uint32_t *p = (const uint32_t *)E->w + (int64_t)token * words;
+    for (int64_t d = 0; d < k; ++d) {
+        uint32_t qv = (p[d / per_word] >> ((d % per_word) * bits)) & mask;
+        float s = bf16_to_f32(E->scales[(int64_t)token * groups + d / E->group]);
+        float b = bf16_to_f32(E->biases[(int64_t)token * groups + d / E->group]);
+        x[d] = f32_to_bf16(((float)qv * s + b) * out_scale);
+    }
+}
+
+/* Final RMSNorm + vocabulary GEMV, logits rounded to T
+ * (src/codegen/kernels/final_rmsnorm_lm_head.rs:225-330). */
+FKO_API void fko_final_rmsnorm_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps,
+                                       const fko_weight *W, uint16_t *logits) {
+    float *ny = (float *)malloc(sizeof(float) * (size_t)W->k);
+    float *acc = (float *)malloc(sizeof(float) * (size_t)W->n);
+    rmsnorm_f(x, norm_w, W->k, eps, ny);
+    linear_acc(W, ny, acc);
+    for (int64_t i = 0; i < W->n; ++i) logits[i] = f32_to_bf16(acc[i]);
+    free(ny);
+    free(acc);
+}
+
+/* Greedy argmax, lowest index wins ties; a NaN never wins (v > max is false)
+ * (src/codegen/kernels/argmax_logits_decode.rs:63-95). */
+FKO_API uint32_t fko_argmax(const uint16_t *logits, int64_t n) {
+    float best = -INFINITY;
+    uint32_t idx = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        float v = bf16_to_f32(logits[i]);
+        if (v > best) {
+            best = v;
+            idx = (uint32_t)i;
+        }
+    }
+    return idx;
+}
+
+/* top-1 minus top-2 logit (0 on an exact tie): the margin the token-identity
+ * test logs per step. */
+FKO_API float fko_top2_margin(const uint16_t *logits, int64_t n) {
+    float a = -INFINITY, b = -INFINITY;
+    for (int64_t i = 0; i < n; ++i) {
+        float v = bf16_to_f32(logits[i]);
+        if (v > a) {
+            b = a;
+            a = v;
+        } else if (v > b) {
+            b = v;
+        }
+    }
+    return a - b;
+}
+
+/* --------------------------------------------------- dense decoder step */
+/*
+ * One decode step of the dense decoder in the reference's decode_pipeline
+ * order (src/codegen/task_graph_json.rs:54-65; per-token protocol
+ * python_runtime/src/lib.rs:1181-1226):
+ *   embed -> L x [ rmsnorm_qkv | (head-norm +) rope_q | (head-norm +) rope_k +
+ *   kv store | sdpa | o_proj + residual | rmsnorm gate/up swiglu | down +
+ *   residual ] -> final norm + lm head -> argmax.
+ */
+typedef struct {
+    const uint16_t *input_norm, *post_norm; /* [hidden] */
+    fko_weight wq, wk, wv, wo, wgate, wup, wdown;
+    const uint16_t *bq, *bk, *bv;       /* optional projection biases */
+    const uint16_t *q_norm, *k_norm;    /* optional per-head norms [head_dim] */
+    uint16_t *cache_k, *cache_v;        /* [n_kv, capacity, head_dim] */
+} fko_layer;
+
+typedef struct {
+    int64_t n_layers, hidden, n_heads, n_kv, head_dim, inter, vocab;
+    float eps, theta, attn_scale, embed_scale;
+    int swiglu_variant;
+    uint32_t capacity;
+    fko_weight embed;   /* [vocab, hidden] */
+    fko_weight lm_head; /* [vocab, hidden]; may alias embed (tied) */
+    const uint16_t *final_norm;
+    const fko_layer *layers;
+} fko_model;
+
+FKO_API uint32_t fko_decoder_step(const fko_model *M, uint32_t token, uint32_t offset,
+                                  uint16_t *logits_out /* [vocab] or NULL */, float *margin_out) {
+    const int64_t H = M->hidden, NQ = M->n_heads * M->head_dim, NKV = M->n_kv * M->head_dim;
+    uint16_t *x = (uint16_t *)malloc(2 * (size_t)H), *x2 = (uint16_t *)malloc(2 * (size_t)H);
+    uint16_t *q = (uint16_t *)malloc(2 * (size_t)NQ), *k = (uint16_t *)malloc(2 * (size_t)NKV);
+    uint16_t *v = (uint16_t *)malloc(2 * (size_t)NKV), *att = (uint16_t *)malloc(2 * (size_t)NQ);
+    uint16_t *mid = (uint16_t *)malloc(2 * (size_t)M->inter);
+    fko_embed_lookup(&M->embed, token, M->embed_scale, x);
+    for (int64_t l = 0; l < M->n_layers; ++l) {
+        const fko_layer *L = &M->layers[l];
+        fko_rmsnorm_qkv(x, L->input_norm, M->eps, &L->wq, &L->wk, &L->wv, L->bq, L->bk, L->bv, q, k, v);
+        if (L->q_norm) {
+            fko_headnorm_rope(q, L->q_norm, M->n_heads, M->head_dim, M->head_dim, M->eps, M->theta, offset);
+            fko_headnorm_rope(k, L->k_norm, M->n_kv, M->head_dim, M->head_dim, M->eps, M->theta, offset);
+            fko_kv_store(k, v, M->n_kv, M->head_dim, M->head_dim, offset, M->capacity, L->cache_k, L->cache_v);
+        } else {
+            fko_rope_q(q, M->n_heads, M->head_dim, M->head_dim, M->theta, offset);
+            fko_rope_kv_store(k, v, M->n_kv, M->head_dim, M->head_dim, M->theta, offset, offset, M->capacity,
+                              L->cache_k, L->cache_v);
+        }
+        fko_sdpa_decode(q, L->cache_k, L->cache_v, M->n_heads, M->n_kv, M->head_dim, M->head_dim, offset + 1,
+                        M->capacity, M->attn_scale, att);
+        fko_linear_residual(&L->wo, att, x, NULL, x2);
+        fko_gateup_swiglu(x2, L->post_norm, M->eps, &L->wgate, &L->wup, M->swiglu_variant, mid);
+        fko_linear_residual(&L->wdown, mid, x2, NULL, x);
+    }
+    uint16_t *logits = logits_out ? logits_out : (uint16_t *)malloc(2 * (size_t)M->vocab);
+    fko_final_rmsnorm_lm_head(x, M->final_norm, M->eps, &M->lm_head, logits);
+    uint32_t next = fko_argmax(logits, M->vocab);
+    if (margin_out) *margin_out = fko_top2_margin(logits, M->vocab);
+    if (!logits_out) free(logits);
+    free(x); free(x2); free(q); free(k); free(v); free(att); free(mid);
+    return next;
+}
