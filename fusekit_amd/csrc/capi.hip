@@ -1,6 +1,8 @@
 // extern "C" surface of libfusekit_hip.so: error state, device memory and the
 // operator launches.  Declarations and reference citations live in
 // include/fusekit_hip.h.
+#include <math.h>
+
 #include <mutex>
 
 #include "fk_host.hpp"
@@ -124,6 +126,31 @@ fk_status fk_stream_sync(fk_stream s) {
     return FK_OK;
 }
 
+fk_status fk_event_create(fk_event* out) {
+    if (!out) return set_error(FK_ERR_INVALID, "null out");
+    const DeviceFacts* d;
+    FK_TRY(device_facts(&d));
+    hipEvent_t e;
+    FK_HIP(hipEventCreate(&e));
+    *out = e;
+    return FK_OK;
+}
+fk_status fk_event_destroy(fk_event e) {
+    if (e) FK_HIP(hipEventDestroy((hipEvent_t)e));
+    return FK_OK;
+}
+fk_status fk_event_record(fk_event e, fk_stream s) {
+    if (!e) return set_error(FK_ERR_INVALID, "null event");
+    FK_HIP(hipEventRecord((hipEvent_t)e, (hipStream_t)s));
+    return FK_OK;
+}
+fk_status fk_event_elapsed_ms(fk_event start, fk_event stop, float* ms) {
+    if (!start || !stop || !ms) return set_error(FK_ERR_INVALID, "null event or out pointer");
+    FK_HIP(hipEventSynchronize((hipEvent_t)stop));
+    FK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return FK_OK;
+}
+
 fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks) {
     g_gemv_policy.rows_per_tile = rows_per_tile;
     g_gemv_policy.grid_blocks = grid_blocks;
@@ -198,6 +225,108 @@ fk_status fk_final_rmsnorm_lm_head(const uint16_t* x, const uint16_t* norm_w, fl
     rq.eps = eps;
     Launch l;
     FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+static float theta_log2(float theta) { return (float)log2((double)theta); }
+
+fk_status fk_rope_q_decode(uint16_t* q, const uint16_t* q_norm, uint32_t n_heads, uint32_t head_dim,
+                           uint32_t rope_dims, float theta, float eps, const uint32_t* d_offset, uint32_t offset,
+                           fk_stream s) {
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.q_norm = q_norm;
+    a.n_q = n_heads; a.head_dim = head_dim; a.rope_dims = rope_dims;
+    a.offset_ptr = d_offset; a.offset_imm = offset;
+    a.eps = eps; a.base_log2 = theta_log2(theta);
+    a.rope_on = rope_dims ? 1u : 0u;
+    a.capacity = 1;
+    Launch l;
+    FK_TRY(plan_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_rope_kv_cache_store_decode(const uint16_t* k, const uint16_t* v, const uint16_t* k_norm, uint32_t n_kv,
+                                        uint32_t k_dim, uint32_t v_dim, uint32_t rope_dims, float theta, float eps,
+                                        const uint32_t* d_offset, uint32_t offset, const uint32_t* d_write_offset,
+                                        uint32_t write_offset, uint32_t capacity, uint16_t* cache_k,
+                                        uint16_t* cache_v, fk_stream s) {
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.k = k; a.v = v; a.k_norm = k_norm;
+    a.n_kv = n_kv; a.k_dim = k_dim; a.v_dim = v_dim; a.rope_dims = rope_dims;
+    a.offset_ptr = d_offset; a.offset_imm = offset;
+    a.write_offset_ptr = d_write_offset; a.write_offset_imm = write_offset; a.use_write_imm = 1;
+    a.capacity = capacity;
+    a.cache_k = cache_k; a.cache_v = cache_v;
+    a.eps = eps; a.base_log2 = theta_log2(theta);
+    a.rope_on = rope_dims ? 1u : 0u;
+    Launch l;
+    FK_TRY(plan_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_qkv_rope_store_decode(uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_norm,
+                                   const uint16_t* k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                   uint32_t rope_dims, float theta, float eps, const uint32_t* d_offset,
+                                   uint32_t offset, uint32_t capacity, uint16_t* cache_k, uint16_t* cache_v,
+                                   fk_stream s) {
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.k = k; a.v = v; a.q_norm = q_norm; a.k_norm = k_norm;
+    a.n_q = n_heads; a.n_kv = n_kv; a.head_dim = head_dim; a.k_dim = head_dim; a.v_dim = head_dim;
+    a.rope_dims = rope_dims;
+    a.offset_ptr = d_offset; a.offset_imm = offset;
+    a.capacity = capacity;
+    a.cache_k = cache_k; a.cache_v = cache_v;
+    a.eps = eps; a.base_log2 = theta_log2(theta);
+    a.rope_on = rope_dims ? 1u : 0u;
+    Launch l;
+    FK_TRY(plan_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t v_dim, uint32_t max_len,
+                                  size_t* partial_bytes, size_t* counter_bytes) {
+    if (!partial_bytes || !counter_bytes || max_len == 0) return set_error(FK_ERR_INVALID, "sdpa workspace: bad argument");
+    return sdpa_workspace_bytes(n_heads, n_kv, v_dim, max_len, partial_bytes, counter_bytes);
+}
+
+fk_status fk_sdpa_decode(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,
+                         const uint32_t* d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
+                         uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
+                         float* partials, uint32_t* counters, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_kv, qk_dim, v_dim,
+                            capacity, scale, partials, counters, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_embed_lookup_decode(const fk_weight* E, const uint32_t* d_token, uint32_t token, float out_scale,
+                                 uint16_t* x, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_embed(E, d_token, token, out_scale, x, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+static_assert(FK_ARGMAX_WORKSPACE_BYTES == kArgmaxWorkspaceBytes, "header and kernel disagree");
+
+fk_status fk_argmax_logits_decode(const uint16_t* logits, uint32_t n, uint32_t* next_token, uint32_t* history,
+                                  uint32_t* hist_counter, uint32_t hist_capacity, void* workspace, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_argmax(logits, n, next_token, history, hist_counter, hist_capacity, workspace, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_step_init(step_counter, offset, kv_len, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_fill_u32(void* dptr, uint32_t value, size_t count, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_fill_u32(dptr, value, count, &l));
     return run_launch(l, (hipStream_t)s);
 }
 

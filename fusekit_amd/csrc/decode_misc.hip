@@ -1,0 +1,303 @@
+// Small decode kernels around the four streaming kernels: RoPE / per-head
+// RMSNorm / KV-cache store, embedding lookup, greedy argmax, the per-token step
+// counter and a fill kernel.  All are launch-latency sized (a few KB of data);
+// what matters is that each is one launch and keeps the reference's rounding
+// boundaries.
+#include "fk_host.hpp"
+#include "fk_device.hpp"
+
+namespace fk {
+
+// ---------------------------------------------------------------- RoPE + store
+//
+// One wave per head.  Blocks [0, n_q) rotate a q head in place, blocks
+// [n_q, n_q + n_kv) rotate a k head into the cache row, blocks beyond copy a v
+// head into the cache row.  With a norm weight the head is first RMS-normalised
+// with the reference's two roundings, T(w * T(x * r)), and the rotation acts on
+// those T values.
+__device__ __forceinline__ void rope_rotate(float lo, float hi, uint32_t d, uint32_t half, uint32_t pos,
+                                            float base_log2, float& olo, float& ohi) {
+    // inv = exp2(-(d/half) * log2(theta)); angle = pos * inv (reference rope_q_decode.rs:93-114)
+    const float d_norm = (float)d / (float)half;
+    // The fp32 exponent is rounded like the reference's; 2^t itself goes through
+    // double so that the fp32 frequency is the correctly rounded one on every
+    // platform (an ulp of inv_freq is 2.5e-3 rad at position 32767).
+    const float inv_freq = (float)exp2((double)(-d_norm * base_log2));
+    const float angle = (float)pos * inv_freq;
+    float sn, cs;
+    sincosf(angle, &sn, &cs);
+    olo = lo * cs - hi * sn;
+    ohi = hi * cs + lo * sn;
+}
+
+__global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
+    const uint32_t b = blockIdx.x, lane = threadIdx.x;
+    const uint32_t pos = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
+    const uint32_t wpos = a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos);
+    const uint32_t row = wpos % a.capacity;
+
+    if (b >= a.n_q + a.n_kv) {  // V head: straight copy into the cache row
+        const uint32_t h = b - a.n_q - a.n_kv;
+        const uint16_t* src = a.v + (size_t)h * a.v_dim;
+        uint16_t* dst = a.cache_v + ((size_t)h * a.capacity + row) * a.v_dim;
+        for (uint32_t d = lane; d < a.v_dim; d += kWave) dst[d] = src[d];
+        return;
+    }
+    const bool is_q = b < a.n_q;
+    const uint32_t h = is_q ? b : b - a.n_q;
+    const uint32_t dim = is_q ? a.head_dim : a.k_dim;
+    const uint16_t* src = is_q ? a.q + (size_t)h * dim : a.k + (size_t)h * dim;
+    uint16_t* dst = is_q ? a.q + (size_t)h * dim : a.cache_k + ((size_t)h * a.capacity + row) * dim;
+    const uint16_t* nw = is_q ? a.q_norm : a.k_norm;
+
+    float r = 1.f;
+    if (nw) {
+        float ss = 0.f;
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            const float x = bf16_bits_to_f32(src[d]);
+            ss = fmaf(x, x, ss);
+        }
+        ss = wave_sum(ss);
+        r = 1.0f / sqrtf(ss / (float)dim + a.eps);
+    }
+    auto value = [&](uint32_t d) {
+        const float x = bf16_bits_to_f32(src[d]);
+        return nw ? round_bf16(bf16_bits_to_f32(nw[d]) * round_bf16(x * r)) : x;
+    };
+    const uint32_t half = a.rope_on ? a.rope_dims / 2 : 0;
+    // rotated pairs (d, d + half); all reads of a pair happen in the lane that writes it
+    for (uint32_t d = lane; d < half; d += kWave) {
+        float lo, hi;
+        rope_rotate(value(d), value(d + half), d, half, pos, a.base_log2, lo, hi);
+        dst[d] = (uint16_t)f32_to_bf16_bits(lo);
+        dst[d + half] = (uint16_t)f32_to_bf16_bits(hi);
+    }
+    // pass-through tail (dims beyond rope_dims, or everything when rotation is off)
+    if (nw || !is_q) {
+        for (uint32_t d = 2 * half + lane; d < dim; d += kWave) dst[d] = (uint16_t)f32_to_bf16_bits(value(d));
+    }
+}
+
+fk_status plan_rope_store(const RopeArgs& in, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    RopeArgs a = in;
+    if (a.n_q && !a.q) return set_error(FK_ERR_INVALID, "rope: null q");
+    if (a.n_kv && (!a.cache_k || !a.cache_v || !a.k || !a.v)) return set_error(FK_ERR_INVALID, "rope: null k/v/cache");
+    if (a.n_q + a.n_kv == 0) return set_error(FK_ERR_INVALID, "rope: nothing to do");
+    if (a.n_kv && a.capacity == 0) return set_error(FK_ERR_INVALID, "rope: zero cache capacity");
+    if (a.rope_on && (a.rope_dims == 0 || a.rope_dims % 2 || (a.n_q && a.rope_dims > a.head_dim) ||
+                      (a.n_kv && a.rope_dims > a.k_dim)))
+        return set_error(FK_ERR_INVALID, "rope: rope_dims must be even and within the head");
+    if (!a.capacity) a.capacity = 1;
+    out->func = reinterpret_cast<const void*>(&rope_store_kernel);
+    out->grid = dim3(a.n_q + 2 * a.n_kv, 1, 1);
+    out->block = dim3(kWave, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+// ---------------------------------------------------------------- embedding
+struct EmbedArgs {
+    const void* w;
+    const uint16_t* scales;
+    const uint16_t* biases;
+    const uint32_t* token_ptr;
+    uint32_t token_imm;
+    uint32_t vocab, hidden, bits, group;
+    float out_scale;
+    uint16_t* x;
+};
+
+// x = T(embed[token] * scale); quantised rows unpack (word >> ((d % lanes) * bits)) & mask
+// (reference embed_lookup_decode.rs:74-99).
+__global__ __launch_bounds__(256) void embed_lookup_kernel(const EmbedArgs a) {
+    const uint32_t d = blockIdx.x * 256 + threadIdx.x;
+    if (d >= a.hidden) return;
+    uint32_t token = a.token_ptr ? *a.token_ptr : a.token_imm;
+    if (token >= a.vocab) token = a.vocab - 1;  // never read outside the table
+    float val;
+    if (a.bits == 16) {
+        val = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(a.w)[(size_t)token * a.hidden + d]);
+    } else {
+        const uint32_t per = 32 / a.bits, mask = (1u << a.bits) - 1u;
+        const uint32_t word = reinterpret_cast<const uint32_t*>(a.w)[(size_t)token * (a.hidden / per) + d / per];
+        const uint32_t qv = (word >> ((d % per) * a.bits)) & mask;
+        const size_t g = (size_t)token * (a.hidden / a.group) + d / a.group;
+        val = (float)qv * bf16_bits_to_f32(a.scales[g]) + bf16_bits_to_f32(a.biases[g]);
+    }
+    a.x[d] = (uint16_t)f32_to_bf16_bits(val * a.out_scale);
+}
+
+fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
+                     uint16_t* x, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!E || !E->w || !x) return set_error(FK_ERR_INVALID, "embed: null pointer");
+    if (E->bits != 4 && E->bits != 8 && E->bits != 16) return set_error(FK_ERR_UNSUPPORTED, "embed: bits 4, 8 or 16");
+    if (E->bits != 16 && (!E->scales || !E->biases || E->group == 0 || E->k % E->group))
+        return set_error(FK_ERR_INVALID, "embed: bad quantisation metadata");
+    if (!token_ptr && token_imm >= E->n) return set_error(FK_ERR_INVALID, "embed: token id outside the vocabulary");
+    EmbedArgs a;
+    memset(&a, 0, sizeof(a));
+    a.w = E->w; a.scales = E->scales; a.biases = E->biases;
+    a.token_ptr = token_ptr; a.token_imm = token_imm;
+    a.vocab = E->n; a.hidden = E->k; a.bits = E->bits; a.group = E->group;
+    a.out_scale = out_scale;
+    a.x = x;
+    out->func = reinterpret_cast<const void*>(&embed_lookup_kernel);
+    out->grid = dim3((E->k + 255) / 256, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+// ---------------------------------------------------------------- argmax
+struct ArgmaxArgs {
+    const uint16_t* logits;
+    uint32_t n;
+    uint32_t* next_token;
+    uint32_t* history;        // optional: history[(*hist_counter)++] = token
+    uint32_t* hist_counter;
+    uint32_t hist_capacity;
+    uint64_t* partial;        // [grid] packed (order-preserving key << 32) | ~index
+    uint32_t* counter;        // zero before the first launch
+};
+
+// Order-preserving key of a bf16-as-float value; NaN maps below everything so it
+// never wins (the reference's `v > max` comparison, argmax_logits_decode.rs:63-95).
+__device__ __forceinline__ uint32_t order_key(float v) {
+    if (v != v) return 0u;
+    const uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Two stages in one launch: every block reduces a slice to one packed 64-bit
+// candidate (value key in the high word, inverted index in the low word, so the
+// maximum of the packed value is the largest logit with the LOWEST index); the
+// last block to finish reduces the candidates.
+__global__ __launch_bounds__(256) void argmax_kernel(const ArgmaxArgs a) {
+    __shared__ uint64_t sm[256 / kWave];
+    __shared__ uint32_t is_last;
+    uint64_t best = 0;
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < a.n; i += gridDim.x * 256) {
+        const uint64_t cand = ((uint64_t)order_key(bf16_bits_to_f32(a.logits[i])) << 32) | (uint32_t)(~i);
+        best = cand > best ? cand : best;
+    }
+    auto block_best = [&](uint64_t v) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const uint64_t other = __shfl_xor(v, o, kWave);
+            v = other > v ? other : v;
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) sm[threadIdx.x / kWave] = v;
+        __syncthreads();
+        uint64_t r = sm[0];
+#pragma unroll
+        for (int w = 1; w < 256 / kWave; ++w) r = sm[w] > r ? sm[w] : r;
+        __syncthreads();
+        return r;
+    };
+    best = block_best(best);
+    if (threadIdx.x == 0) a.partial[blockIdx.x] = best;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = (atomicAdd(a.counter, 1u) == gridDim.x - 1) ? 1u : 0u;
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    uint64_t fin = 0;
+    for (uint32_t i = threadIdx.x; i < gridDim.x; i += 256) fin = a.partial[i] > fin ? a.partial[i] : fin;
+    fin = block_best(fin);
+    if (threadIdx.x == 0) {
+        // all-NaN / empty rows fall back to index 0 like the reference's initial local_idx
+        const uint32_t tok = (fin >> 32) ? ~(uint32_t)fin : 0u;
+        *a.next_token = tok;
+        if (a.history && a.hist_counter) {
+            const uint32_t slot = *a.hist_counter;
+            if (slot < a.hist_capacity) a.history[slot] = tok;
+            *a.hist_counter = slot + 1;
+        }
+        *a.counter = 0u;
+    }
+}
+
+fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, uint32_t* history,
+                      uint32_t* hist_counter, uint32_t hist_capacity, void* workspace, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!logits || !next_token || !workspace) return set_error(FK_ERR_INVALID, "argmax: null pointer");
+    if (n == 0) return set_error(FK_ERR_INVALID, "argmax: empty logits");
+    uint32_t grid = (n + 2047) / 2048;
+    if (grid > 160) grid = 160;
+    ArgmaxArgs a;
+    memset(&a, 0, sizeof(a));
+    a.logits = logits; a.n = n; a.next_token = next_token;
+    a.history = history; a.hist_counter = hist_counter; a.hist_capacity = hist_capacity;
+    a.counter = reinterpret_cast<uint32_t*>(workspace);
+    a.partial = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(workspace) + 8);
+    out->func = reinterpret_cast<const void*>(&argmax_kernel);
+    out->grid = dim3(grid, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+// ---------------------------------------------------------------- step counter
+// offset = step_counter++ ; kv_len = offset + 1 (reference kernels/mod.rs:544-563).
+struct StepArgs {
+    uint32_t* step_counter;
+    uint32_t* offset;
+    uint32_t* kv_len;
+};
+__global__ void step_init_kernel(const StepArgs a) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const uint32_t o = *a.step_counter;
+        *a.step_counter = o + 1;
+        *a.offset = o;
+        *a.kv_len = o + 1;
+    }
+}
+
+fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!step_counter || !offset || !kv_len) return set_error(FK_ERR_INVALID, "step_init: null pointer");
+    StepArgs a{step_counter, offset, kv_len};
+    out->func = reinterpret_cast<const void*>(&step_init_kernel);
+    out->grid = dim3(1, 1, 1);
+    out->block = dim3(kWave, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+// ---------------------------------------------------------------- fill
+struct FillArgs {
+    uint32_t* p;
+    uint32_t value;
+    size_t count;
+};
+__global__ __launch_bounds__(256) void fill_u32_kernel(const FillArgs a) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < a.count; i += (size_t)gridDim.x * 256) a.p[i] = a.value;
+}
+
+fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!p || count == 0) return set_error(FK_ERR_INVALID, "fill: null pointer or zero count");
+    FillArgs a{reinterpret_cast<uint32_t*>(p), value, count};
+    size_t blocks = (count + 255) / 256;
+    if (blocks > (size_t)dev->cus * 8) blocks = (size_t)dev->cus * 8;
+    out->func = reinterpret_cast<const void*>(&fill_u32_kernel);
+    out->grid = dim3((uint32_t)blocks, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+}  // namespace fk

@@ -73,4 +73,39 @@ struct GemvRequest {
 };
 fk_status plan_gemv(const GemvRequest& rq, Launch* out);
 
+// RoPE / per-head RMSNorm / KV-cache store (one wave per head).
+struct RopeArgs {
+    uint16_t* q;             // [n_q, head_dim] in place, or null
+    const uint16_t* k;       // [n_kv, k_dim] or null
+    const uint16_t* v;       // [n_kv, v_dim] or null
+    const uint16_t* q_norm;  // [head_dim] or null
+    const uint16_t* k_norm;  // [k_dim] or null
+    uint16_t* cache_k;       // [n_kv, capacity, k_dim]
+    uint16_t* cache_v;       // [n_kv, capacity, v_dim]
+    const uint32_t* offset_ptr;        // rotary position (device) or null -> offset_imm
+    const uint32_t* write_offset_ptr;  // cache row before the modulo, or null
+    uint32_t offset_imm, write_offset_imm;
+    uint32_t use_write_imm;  // with a null write_offset_ptr: 1 = write_offset_imm, 0 = same as offset
+    uint32_t n_q, n_kv, head_dim, k_dim, v_dim, rope_dims, capacity;
+    float eps, base_log2;
+    uint32_t rope_on;  // 0: plain store of K (no rotation)
+};
+fk_status plan_rope_store(const RopeArgs& in, Launch* out);
+
+uint32_t sdpa_chunk_len(uint32_t max_len);
+fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t v_dim, uint32_t max_len,
+                               size_t* partial_bytes, size_t* counter_bytes);
+fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,
+                           const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
+                           uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
+                           float* partials, uint32_t* counters, Launch* out_launch);
+fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
+                     uint16_t* x, Launch* out);
+// workspace: 8 bytes (counter, zeroed once) + 8 bytes per block (<= 160 blocks)
+constexpr size_t kArgmaxWorkspaceBytes = 8 + 8 * 160;
+fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, uint32_t* history,
+                      uint32_t* hist_counter, uint32_t hist_capacity, void* workspace, Launch* out);
+fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out);
+fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out);
+
 }  // namespace fk

@@ -92,7 +92,6 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     const uint32_t R = best_r;
     const uint64_t tiles = tiles_for(R);
     if (tiles > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "gemv: too many tiles");
-    const uint32_t tile_chunks = nseg * R * cpr;
 
     GemvArgs a;
     memset(&a, 0, sizeof(a));
@@ -128,9 +127,9 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
 
     uint32_t lds = 0;
     switch (kind) {
-        case W_Q4: lds = gemv_lds_bytes<W_Q4>(cpr, tile_chunks); break;
-        case W_Q8: lds = gemv_lds_bytes<W_Q8>(cpr, tile_chunks); break;
-        default: lds = gemv_lds_bytes<W_BF16>(cpr, tile_chunks); break;
+        case W_Q4: lds = gemv_lds_bytes<W_Q4>(cpr, R * cpr, nseg); break;
+        case W_Q8: lds = gemv_lds_bytes<W_Q8>(cpr, R * cpr, nseg); break;
+        default: lds = gemv_lds_bytes<W_BF16>(cpr, R * cpr, nseg); break;
     }
     if ((int)lds > dev->max_dyn_lds) return set_error(FK_ERR_UNSUPPORTED, "gemv: K too large for LDS staging");
 

@@ -67,14 +67,22 @@ struct ChunkTraits<W_BF16> {
 
 // LDS bytes the kernel needs: staged activations + per-chunk sums + partials + scratch.
 template <WKind KIND>
-__host__ __device__ inline uint32_t gemv_lds_bytes(uint32_t cpr, uint32_t tile_chunks) {
-    return ChunkTraits<KIND>::kPieces * cpr * 16u + cpr * 4u + tile_chunks * 4u + 64u;
+__host__ __device__ inline uint32_t gemv_lds_bytes(uint32_t cpr, uint32_t seg_chunks, uint32_t nseg) {
+    const uint32_t pos = kGemvBlock * (kGemvUnroll / nseg);
+    const uint32_t seg_pad = (seg_chunks + pos - 1) / pos * pos;
+    return ChunkTraits<KIND>::kPieces * cpr * 16u + cpr * 4u + nseg * seg_pad * 4u + 64u;
 }
 
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t o) { return (a & m) | o; }
+// (a & m) | o in one VALU op; the compiler splits it when both constants sit in
+// SGPRs, so the instruction is named with the OR term held in a VGPR.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t o) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(m), "v"(o));
+    return d;
+}
 
 __device__ __forceinline__ float q4_word_dot(uint32_t w, uint4 xp, float d) {
-    constexpr uint32_t M = 0x000F000Fu, B = 0x43004300u;
+    const uint32_t M = 0x000F000Fu, B = 0x43004300u;
     d = dot2_bf16(and_or(w, M, B), xp.x, d);
     d = dot2_bf16(and_or(w >> 4, M, B), xp.y, d);
     d = dot2_bf16(and_or(w >> 8, M, B), xp.z, d);
@@ -95,21 +103,21 @@ template <WKind KIND>
 __device__ __forceinline__ float chunk_partial(uint4 wv, uint32_t s_bits, uint32_t b_bits, const uint4* xs,
                                                const float* sx, uint32_t c, uint32_t cpr) {
     if constexpr (KIND == W_Q4) {
-        float d = 0.f;
-        d = q4_word_dot(wv.x, xs[c], d);
-        d = q4_word_dot(wv.y, xs[cpr + c], d);
-        d = q4_word_dot(wv.z, xs[2 * cpr + c], d);
-        d = q4_word_dot(wv.w, xs[3 * cpr + c], d);
+        float d0 = 0.f, d1 = 0.f;  // two chains keep the dot unit busy
+        d0 = q4_word_dot(wv.x, xs[c], d0);
+        d1 = q4_word_dot(wv.y, xs[cpr + c], d1);
+        d0 = q4_word_dot(wv.z, xs[2 * cpr + c], d0);
+        d1 = q4_word_dot(wv.w, xs[3 * cpr + c], d1);
         const float s = bf16_bits_to_f32(s_bits), b = bf16_bits_to_f32(b_bits), sum_x = sx[c];
-        return fmaf(s, fmaf(-128.f, sum_x, d), b * sum_x);
+        return fmaf(s, fmaf(-128.f, sum_x, d0 + d1), b * sum_x);
     } else if constexpr (KIND == W_Q8) {
-        float d = 0.f;
-        d = q8_word_dot(wv.x, xs[c], d);
-        d = q8_word_dot(wv.y, xs[cpr + c], d);
-        d = q8_word_dot(wv.z, xs[2 * cpr + c], d);
-        d = q8_word_dot(wv.w, xs[3 * cpr + c], d);
+        float d0 = 0.f, d1 = 0.f;
+        d0 = q8_word_dot(wv.x, xs[c], d0);
+        d1 = q8_word_dot(wv.y, xs[cpr + c], d1);
+        d0 = q8_word_dot(wv.z, xs[2 * cpr + c], d0);
+        d1 = q8_word_dot(wv.w, xs[3 * cpr + c], d1);
         const float s = bf16_bits_to_f32(s_bits), b = bf16_bits_to_f32(b_bits);
-        return fmaf(s, d, b * sx[c]);
+        return fmaf(s, d0 + d1, b * sx[c]);
     } else {
         const uint4 xp = xs[c];
         float d = 0.f;
@@ -229,99 +237,125 @@ template <WKind KIND, int NSEG, bool NORM>
 __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs a) {
     extern __shared__ uint4 lds_raw[];
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
-    constexpr uint32_t BATCH = kGemvBlock * kGemvUnroll;
+    constexpr int SLOTS = kGemvUnroll / NSEG;                // register slots per segment and batch
+    constexpr uint32_t POS = kGemvBlock * SLOTS;             // chunk positions of a segment per batch
     const uint32_t cpr = a.cpr, R = a.R;
-    const uint32_t seg_chunks = R * cpr;          // chunks of one segment of a full tile
-    const uint32_t tile_chunks = NSEG * seg_chunks;
+    const uint32_t seg_chunks = R * cpr;                     // chunks of one segment of a full tile
+    const uint32_t seg_pad = (seg_chunks + POS - 1) / POS * POS;
 
     uint4* xs = lds_raw;
     float* sx = reinterpret_cast<float*>(xs + PIECES * cpr);
-    float* part = sx + cpr;
-    float* scratch = part + tile_chunks;
+    float* part = sx + cpr;                                  // [NSEG][seg_pad]
+    float* scratch = part + NSEG * seg_pad;
 
-    // Resolves a tile to (matrix, first row, valid rows).
-    auto tile_rows = [&](uint32_t tile, uint32_t& m, uint32_t& row0, uint32_t& valid) {
+    // Per-tile facts, uniform over the block (scalar registers).
+    struct TileInfo {
+        const char* w[NSEG];
+        const char* sc[NSEG];
+        const char* bi[NSEG];
+        uint32_t m, row0, valid;
+    };
+    auto tile_info = [&](uint32_t tile) {
+        TileInfo t;
         if constexpr (NSEG == 2) {
-            m = 0;
-            row0 = tile * R;
+            t.m = 0;
+            t.row0 = tile * R;
         } else {
-            m = (a.n_mats > 1 && tile >= a.tile_start[1]) ? ((a.n_mats > 2 && tile >= a.tile_start[2]) ? 2u : 1u)
-                                                          : 0u;
-            row0 = (tile - a.tile_start[m]) * R;
+            t.m = (a.n_mats > 1 && tile >= a.tile_start[1]) ? ((a.n_mats > 2 && tile >= a.tile_start[2]) ? 2u : 1u)
+                                                            : 0u;
+            t.row0 = (tile - a.tile_start[t.m]) * R;
         }
-        const uint32_t left = a.n[m] - row0;
-        valid = left < R ? left : R;
+        const uint32_t left = a.n[t.m] - t.row0;
+        t.valid = left < R ? left : R;
+        const size_t base = (size_t)t.row0 * cpr;
+#pragma unroll
+        for (int sg = 0; sg < NSEG; ++sg) {
+            const uint32_t mm = (NSEG == 2) ? (uint32_t)sg : t.m;
+            t.w[sg] = reinterpret_cast<const char*>(a.w[mm] + base);
+            if constexpr (KIND != W_BF16) {
+                t.sc[sg] = reinterpret_cast<const char*>(a.sc[mm] + (base >> a.gshift));
+                t.bi[sg] = reinterpret_cast<const char*>(a.bi[mm] + (base >> a.gshift));
+            }
+        }
+        return t;
     };
 
     // Issues the 16-byte weight loads (and scale/bias) of one batch into registers.
-    auto load_batch = [&](uint4(&wv)[kGemvUnroll], uint32_t(&sb)[kGemvUnroll], uint32_t tile, uint32_t b0) {
-        uint32_t m, row0, valid;
-        tile_rows(tile, m, row0, valid);
-        const uint32_t valid_chunks = valid * cpr;
+    // Slot j belongs to segment j / SLOTS, so every slot's base pointer is uniform
+    // and the per-lane part of the address is a 32-bit byte offset.  Straight-line:
+    // positions outside the tile's valid rows read chunk 0 of the tile instead
+    // (always in bounds); their partials are never consumed.
+    auto load_batch = [&](uint4(&wv)[kGemvUnroll], uint32_t(&sc)[kGemvUnroll], uint32_t(&bi)[kGemvUnroll],
+                          uint32_t tile, uint32_t b0) {
+        const TileInfo t = tile_info(tile);
+        const uint32_t valid_chunks = t.valid * cpr;
 #pragma unroll
         for (int j = 0; j < kGemvUnroll; ++j) {
-            const uint32_t u = b0 + j * kGemvBlock + threadIdx.x;
-            uint32_t mm = m, uu = u;
-            if constexpr (NSEG == 2) {
-                if (u >= seg_chunks) {
-                    mm = 1;
-                    uu = u - seg_chunks;
-                }
-            }
-            wv[j] = make_uint4(0, 0, 0, 0);
-            sb[j] = 0;
-            if (u < tile_chunks && uu < valid_chunks) {
-                const size_t flat = (size_t)row0 * cpr + uu;
-                wv[j] = a.w[mm][flat];
-                if constexpr (KIND != W_BF16) {
-                    const size_t g = flat >> a.gshift;
-                    sb[j] = (uint32_t)a.sc[mm][g] | ((uint32_t)a.bi[mm][g] << 16);
-                }
+            const int sg = j / SLOTS;
+            const uint32_t pos = b0 + (j % SLOTS) * kGemvBlock + threadIdx.x;
+            const uint32_t idx = pos < valid_chunks ? pos : 0u;
+            wv[j] = *reinterpret_cast<const uint4*>(t.w[sg] + (idx << 4));
+            if constexpr (KIND != W_BF16) {
+                const uint32_t goff = (idx >> a.gshift) << 1;
+                sc[j] = *reinterpret_cast<const uint16_t*>(t.sc[sg] + goff);
+                bi[j] = *reinterpret_cast<const uint16_t*>(t.bi[sg] + goff);
             }
         }
     };
 
+    // Column (chunk within its row) of each slot's position; advanced per batch
+    // instead of dividing by cpr for every chunk.
+    uint32_t col0[SLOTS], col[SLOTS];
+#pragma unroll
+    for (int jj = 0; jj < SLOTS; ++jj) {
+        const uint32_t pos = jj * kGemvBlock + threadIdx.x;
+        const uint32_t row = (uint32_t)(((float)pos + 0.5f) * a.inv_cpr);
+        col0[jj] = col[jj] = pos - row * cpr;
+    }
+    const uint32_t col_step = POS % cpr;
+
     uint32_t tile = blockIdx.x, b0 = 0;
 
-    // Consumes the batch held in (cur, curs) while the following batch streams
-    // into (nxt, nxts).  Returns false once this block has no tile left.
-    auto step = [&](uint4(&cur)[kGemvUnroll], uint32_t(&curs)[kGemvUnroll], uint4(&nxt)[kGemvUnroll],
-                    uint32_t(&nxts)[kGemvUnroll]) -> bool {
-        uint32_t ntile = tile, nb0 = b0 + BATCH;
-        if (nb0 >= tile_chunks) {
+    // Consumes the batch held in cur* while the following batch streams into nxt*.
+    // Returns false once this block has no tile left.
+    auto step = [&](uint4(&cur)[kGemvUnroll], uint32_t(&csc)[kGemvUnroll], uint32_t(&cbi)[kGemvUnroll],
+                    uint4(&nxt)[kGemvUnroll], uint32_t(&nsc)[kGemvUnroll], uint32_t(&nbi)[kGemvUnroll]) -> bool {
+        uint32_t ntile = tile, nb0 = b0 + POS;
+        if (nb0 >= seg_chunks) {
             ntile = tile + gridDim.x;
             nb0 = 0;
         }
-        if (ntile < a.n_tiles) load_batch(nxt, nxts, ntile, nb0);
+        if (ntile < a.n_tiles) load_batch(nxt, nsc, nbi, ntile, nb0);
 
+        float p[kGemvUnroll];
 #pragma unroll
         for (int j = 0; j < kGemvUnroll; ++j) {
-            const uint32_t u = b0 + j * kGemvBlock + threadIdx.x;
-            if (u < tile_chunks) {
-                uint32_t uu = u;
-                if constexpr (NSEG == 2) uu = (u >= seg_chunks) ? u - seg_chunks : u;
-                const uint32_t row = (uint32_t)(((float)uu + 0.5f) * a.inv_cpr);
-                const uint32_t c = uu - row * cpr;
-                part[u] = chunk_partial<KIND>(cur[j], curs[j] & 0xffffu, curs[j] >> 16, xs, sx, c, cpr);
-            }
+            p[j] = chunk_partial<KIND>(cur[j], csc[j], cbi[j], xs, sx, col[j % SLOTS], cpr);
+            // Keep the scheduler from hoisting every chunk's LDS reads to the top
+            // (that costs ~200 VGPRs); other waves hide the LDS latency instead.
+            __builtin_amdgcn_sched_barrier(0);
         }
+        // `part` is padded to whole batches, so the store needs no guard (a guard
+        // would let the compiler sink all the arithmetic into the branch).
+#pragma unroll
+        for (int j = 0; j < kGemvUnroll; ++j)
+            part[(j / SLOTS) * seg_pad + b0 + (j % SLOTS) * kGemvBlock + threadIdx.x] = p[j];
 
         if (ntile != tile) {
             // tile complete: add each row's partials in a fixed order, then the epilogue
             __syncthreads();
-            uint32_t m, row0, valid;
-            tile_rows(tile, m, row0, valid);
+            const TileInfo t = tile_info(tile);
             const uint32_t lr = a.lr, lane = threadIdx.x & (lr - 1);
             for (uint32_t rr = threadIdx.x / lr; rr < R; rr += kGemvBlock / lr) {
                 float s0 = 0.f, s1 = 0.f;
                 for (uint32_t i = lane; i < cpr; i += lr) {
                     s0 += part[rr * cpr + i];
-                    if constexpr (NSEG == 2) s1 += part[seg_chunks + rr * cpr + i];
+                    if constexpr (NSEG == 2) s1 += part[seg_pad + rr * cpr + i];
                 }
                 s0 = group_sum(s0, lr);
                 if constexpr (NSEG == 2) s1 = group_sum(s1, lr);
-                if (lane == 0 && rr < valid) {
-                    const uint32_t n = row0 + rr;
+                if (lane == 0 && rr < t.valid) {
+                    const uint32_t n = t.row0 + rr, m = t.m;
                     if constexpr (NSEG == 2) {
                         a.y[0][n] = (uint16_t)swiglu_bits(s0, s1, a.swiglu_variant);
                     } else {
@@ -336,6 +370,14 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
                 }
             }
             __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < SLOTS; ++jj) col[jj] = col0[jj];
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < SLOTS; ++jj) {
+                const uint32_t c = col[jj] + col_step;
+                col[jj] = c >= cpr ? c - cpr : c;
+            }
         }
         tile = ntile;
         b0 = nb0;
@@ -343,14 +385,14 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
     };
 
     uint4 wa[kGemvUnroll], wb[kGemvUnroll];
-    uint32_t sa[kGemvUnroll], sbb[kGemvUnroll];
+    uint32_t sa[kGemvUnroll], sb[kGemvUnroll], ba[kGemvUnroll], bb[kGemvUnroll];
     const bool has_work = tile < a.n_tiles;
-    if (has_work) load_batch(wa, sa, tile, 0);  // weights start streaming before x is staged
+    if (has_work) load_batch(wa, sa, ba, tile, 0);  // weights start streaming before x is staged
     stage_activations<KIND, NORM>(a, xs, sx, scratch);
     if (!has_work) return;
     while (true) {
-        if (!step(wa, sa, wb, sbb)) break;
-        if (!step(wb, sbb, wa, sa)) break;
+        if (!step(wa, sa, ba, wb, sb, bb)) break;
+        if (!step(wb, sb, bb, wa, sa, ba)) break;
     }
 }
 

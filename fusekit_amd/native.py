@@ -179,9 +179,97 @@ def final_rmsnorm_lm_head(x, norm_w, eps, W, logits, stream=None) -> None:
                                        _ptr(stream)))
 
 
+def rope_q_decode(q, q_norm, n_heads, head_dim, rope_dims, theta, eps=0.0, d_offset=None, offset=0, stream=None):
+    check(lib.fk_rope_q_decode(_ptr(q), _ptr(q_norm), C.c_uint32(n_heads), C.c_uint32(head_dim),
+                               C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), _ptr(d_offset),
+                               C.c_uint32(offset), _ptr(stream)))
+
+
+def rope_kv_cache_store_decode(k, v, k_norm, n_kv, k_dim, v_dim, rope_dims, theta, eps, d_offset, offset,
+                               d_write_offset, write_offset, capacity, cache_k, cache_v, stream=None):
+    check(lib.fk_rope_kv_cache_store_decode(
+        _ptr(k), _ptr(v), _ptr(k_norm), C.c_uint32(n_kv), C.c_uint32(k_dim), C.c_uint32(v_dim),
+        C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), _ptr(d_offset), C.c_uint32(offset),
+        _ptr(d_write_offset), C.c_uint32(write_offset), C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v),
+        _ptr(stream)))
+
+
+def qkv_rope_store_decode(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope_dims, theta, eps, d_offset,
+                          offset, capacity, cache_k, cache_v, stream=None):
+    check(lib.fk_qkv_rope_store_decode(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), C.c_uint32(n_heads), C.c_uint32(n_kv),
+        C.c_uint32(head_dim), C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), _ptr(d_offset),
+        C.c_uint32(offset), C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v), _ptr(stream)))
+
+
+def sdpa_workspace_bytes(n_heads, n_kv, v_dim, max_len):
+    pb, cb = C.c_size_t(), C.c_size_t()
+    check(lib.fk_sdpa_workspace_bytes(C.c_uint32(n_heads), C.c_uint32(n_kv), C.c_uint32(v_dim),
+                                      C.c_uint32(max_len), C.byref(pb), C.byref(cb)))
+    return int(pb.value), int(cb.value)
+
+
+def sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_kv, qk_dim, v_dim, capacity,
+                scale, partials, counters, stream=None):
+    check(lib.fk_sdpa_decode(_ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(out), _ptr(d_kv_len),
+                             C.c_uint32(kv_len), C.c_uint32(max_len), C.c_uint32(n_heads), C.c_uint32(n_kv),
+                             C.c_uint32(qk_dim), C.c_uint32(v_dim), C.c_uint32(capacity), C.c_float(scale),
+                             _ptr(partials), _ptr(counters), _ptr(stream)))
+
+
+def embed_lookup_decode(E, d_token, token, out_scale, x, stream=None):
+    check(lib.fk_embed_lookup_decode(C.byref(E.c), _ptr(d_token), C.c_uint32(token), C.c_float(out_scale),
+                                     _ptr(x), _ptr(stream)))
+
+
+ARGMAX_WORKSPACE_BYTES = 1288
+
+
+def argmax_logits_decode(logits, n, next_token, history, hist_counter, hist_capacity, workspace, stream=None):
+    check(lib.fk_argmax_logits_decode(_ptr(logits), C.c_uint32(n), _ptr(next_token), _ptr(history),
+                                      _ptr(hist_counter), C.c_uint32(hist_capacity), _ptr(workspace),
+                                      _ptr(stream)))
+
+
+def step_init(step_counter, offset, kv_len, stream=None):
+    check(lib.fk_step_init(_ptr(step_counter), _ptr(offset), _ptr(kv_len), _ptr(stream)))
+
+
+def fill_u32(buf, value, count, stream=None):
+    check(lib.fk_fill_u32(_ptr(buf), C.c_uint32(value), C.c_size_t(count), _ptr(stream)))
+
+
+def zeros(nbytes: int) -> DeviceBuffer:
+    b = DeviceBuffer(nbytes)
+    b.upload(np.zeros(nbytes, dtype=np.uint8))
+    return b
+
+
 def set_gemv_policy(rows_per_tile: int = 0, grid_blocks: int = 0) -> None:
     check(lib.fk_set_gemv_policy(C.c_uint32(rows_per_tile), C.c_uint32(grid_blocks)))
 
 
 def sync(stream=None) -> None:
     check(lib.fk_stream_sync(_ptr(stream)))
+
+
+class Event:
+    def __init__(self):
+        p = C.c_void_p()
+        check(lib.fk_event_create(C.byref(p)))
+        self.ptr = p.value
+
+    def record(self, stream=None) -> None:
+        check(lib.fk_event_record(C.c_void_p(self.ptr), _ptr(stream)))
+
+    def elapsed_ms_until(self, stop: "Event") -> float:
+        ms = C.c_float()
+        check(lib.fk_event_elapsed_ms(C.c_void_p(self.ptr), C.c_void_p(stop.ptr), C.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib.fk_event_destroy(C.c_void_p(self.ptr))
+        except Exception:
+            pass

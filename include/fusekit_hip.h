@@ -81,6 +81,15 @@ fk_status fk_stream_create(fk_stream *out);
 fk_status fk_stream_destroy(fk_stream s);
 fk_status fk_stream_sync(fk_stream s);
 
+/* GPU timing on the stream the work was launched on (hipEvent pairs); the
+ * reference reports GPU seconds from command-buffer timestamps
+ * (python_runtime/src/lib.rs:745-760). */
+typedef void *fk_event;
+fk_status fk_event_create(fk_event *out);
+fk_status fk_event_destroy(fk_event e);
+fk_status fk_event_record(fk_event e, fk_stream s);
+fk_status fk_event_elapsed_ms(fk_event start, fk_event stop, float *ms); /* waits for `stop` */
+
 /* ---- operator launches ------------------------------------------------ */
 
 /* K1  y = T(x @ dequant(W)^T (+ bias)).  Replaces the qGEMV inner loop
@@ -113,6 +122,72 @@ fk_status fk_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps,
  *     src/codegen/kernels/final_rmsnorm_lm_head.rs:144-629. */
 fk_status fk_final_rmsnorm_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *W,
                                    uint16_t *logits, fk_stream s);
+
+/* Per-token scalars (rotary position, cache row, KV length) come either from a
+ * device scalar `d_*` (so a captured hipGraph can be replayed while a step
+ * kernel advances them, as the reference binds `layer_offset` / `layer_kv_len`
+ * uniform buffers, src/codegen/kernels/mod.rs:5531-5577) or, when that pointer
+ * is NULL, from the immediate value next to it. */
+
+/* R   half-split RoPE on q [n_heads, head_dim] in place; pair (d, d+rope_dims/2),
+ *     inv = exp2(-(d/half)*log2(theta)), angle = pos*inv.  Replaces
+ *     src/codegen/kernels/rope_q_decode.rs:24-125.  q_norm != NULL first applies
+ *     the per-head RMSNorm T(w*T(x*r)) (q side of
+ *     src/codegen/kernels/rmsnorm_rope_qgate_decode.rs:84-136, without the gate). */
+fk_status fk_rope_q_decode(uint16_t *q, const uint16_t *q_norm, uint32_t n_heads, uint32_t head_dim,
+                           uint32_t rope_dims, float theta, float eps, const uint32_t *d_offset,
+                           uint32_t offset, fk_stream s);
+
+/* R   RoPE(K) -> cache_k[kh, write_offset % capacity, :], V copied likewise;
+ *     caches [n_kv, capacity, dim].  Replaces
+ *     src/codegen/kernels/rope_kv_cache_store_decode.rs:21-143; with k_norm the
+ *     per-head RMSNorm variant src/codegen/kernels/rmsnorm_rope_kv_cache_store_decode.rs:11-176;
+ *     rope_dims == 0 stores K unrotated (src/codegen/kernels/kv_cache_store_decode.rs,
+ *     k_dim may differ from v_dim). */
+fk_status fk_rope_kv_cache_store_decode(const uint16_t *k, const uint16_t *v, const uint16_t *k_norm,
+                                        uint32_t n_kv, uint32_t k_dim, uint32_t v_dim, uint32_t rope_dims,
+                                        float theta, float eps, const uint32_t *d_offset, uint32_t offset,
+                                        const uint32_t *d_write_offset, uint32_t write_offset,
+                                        uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
+
+/* R   the two above in ONE launch (MI355X addition: halves the launch count of
+ *     the rope/store stage; same arithmetic). */
+fk_status fk_qkv_rope_store_decode(uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *q_norm,
+                                   const uint16_t *k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                   uint32_t rope_dims, float theta, float eps, const uint32_t *d_offset,
+                                   uint32_t offset, uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v,
+                                   fk_stream s);
+
+/* K4  GQA SDPA for one query token over the bf16 cache, fp32 softmax, split-K
+ *     with an in-kernel ordered merge.  Replaces
+ *     src/codegen/kernels/sdpa_decode.rs:133-408 (online body :1064-1211,
+ *     partial/combine :717-1046).  `max_len` bounds kv_len for this launch (it
+ *     sizes the split; use the cache capacity when replaying a graph).
+ *     Workspace sizes from fk_sdpa_workspace_bytes; `counters` must be zero
+ *     before the first launch (the kernel leaves them zero). */
+fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t v_dim, uint32_t max_len,
+                                  size_t *partial_bytes, size_t *counter_bytes);
+fk_status fk_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v, uint16_t *out,
+                         const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
+                         uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
+                         float *partials, uint32_t *counters, fk_stream s);
+
+/* E   x = T(embed[token] * out_scale), dense bf16 or MLX-affine table.  Replaces
+ *     src/codegen/kernels/embed_lookup_decode.rs:17-108. */
+fk_status fk_embed_lookup_decode(const fk_weight *E, const uint32_t *d_token, uint32_t token, float out_scale,
+                                 uint16_t *x, fk_stream s);
+
+/* A   greedy argmax over bf16 logits, lowest index wins ties, NaN never wins;
+ *     optionally appends the token to history[(*hist_counter)++].  Replaces
+ *     src/codegen/kernels/argmax_logits_{decode,scan,finalize}.rs.  Workspace:
+ *     FK_ARGMAX_WORKSPACE_BYTES, zeroed once. */
+#define FK_ARGMAX_WORKSPACE_BYTES 1288
+fk_status fk_argmax_logits_decode(const uint16_t *logits, uint32_t n, uint32_t *next_token, uint32_t *history,
+                                  uint32_t *hist_counter, uint32_t hist_capacity, void *workspace, fk_stream s);
+
+/* U   offset = step_counter++ ; kv_len = offset + 1.  Replaces fusekit_step_init
+ *     (src/codegen/kernels/mod.rs:542-563). */
+fk_status fk_step_init(uint32_t *step_counter, uint32_t *offset, uint32_t *kv_len, fk_stream s);
 
 /* Launch-geometry overrides for experiments (0 = library policy): rows per
  * tile and grid blocks of the streaming GEMV.  Process-wide. */

@@ -161,6 +161,14 @@ def dequantize(W: QWeight) -> np.ndarray:
     return out
 
 
+def dequantize_rows(W: QWeight, r0: int, r1: int) -> np.ndarray:
+    """Rows [r0, r1) of dequantize(W) without materialising the whole matrix."""
+    if W.bits == 16:
+        return bf16_to_f32(W.w[r0:r1])
+    sub = QWeight(W.w[r0:r1], W.scales[r0:r1], W.biases[r0:r1], r1 - r0, W.k, W.bits, W.group)
+    return dequantize(sub)
+
+
 # ------------------------------------------------------------------ operators
 
 def linear_acc(W: QWeight, x: np.ndarray) -> np.ndarray:
