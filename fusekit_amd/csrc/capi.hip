@@ -330,4 +330,18 @@ fk_status fk_fill_u32(void* dptr, uint32_t value, size_t count, fk_stream s) {
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_quantize_affine(const float* d_w, size_t n, size_t k, uint32_t bits, uint32_t group,
+                             uint32_t* d_packed, uint16_t* d_scales, uint16_t* d_biases, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_quantize(d_w, n, k, bits, group, d_packed, d_scales, d_biases, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_synth_fill(void* dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind, uint32_t bound,
+                        fk_stream s) {
+    Launch l;
+    FK_TRY(plan_synth(dptr, count, seed, mean, std, kind, bound, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 }  // extern "C"

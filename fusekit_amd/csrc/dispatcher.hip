@@ -1,0 +1,939 @@
+// Dispatcher: named dispatch, hipGraph build / update / replay and the native
+// per-token decode loop.  It replaces the Metal indirect-command-buffer runtime
+// of the reference (python_runtime/src/lib.rs): build_icb -> fk_build_graph,
+// update_icb_bindings -> fk_update_graph_bindings, execute_icb ->
+// fk_execute_graph, decode_chunk_gpu_chain -> fk_decode_chunk.
+//
+// A dispatch names a kernel family by prefix ("fusekit_rmsnorm_qkv_f12" selects
+// "fusekit_rmsnorm_qkv"), lists its buffers as (pointer, bytes) in the
+// reference emitters' slot order and carries a small key/value parameter block
+// (dims, eps, theta, bits ...) in place of the constants the reference bakes
+// into kernel text.  Each family has a planner that validates the shapes and
+// produces a Launch, and a read/write slot table from which hipGraph edges are
+// derived (RAW, WAW and WAR on overlapping byte ranges), the equivalent of the
+// reference's host-side barrier mask (python/fusekit_runtime/dispatch.py:36-100).
+#include <math.h>
+
+#include <algorithm>
+#include <fstream>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "fk_host.hpp"
+#include "fk_json.hpp"
+
+namespace fk {
+namespace {
+
+struct Dispatch {
+    std::string kernel;
+    std::vector<fk_arg> args;
+    std::vector<std::pair<std::string, double>> params;
+
+    double param(const char* key, double dflt) const {
+        for (const auto& kv : params)
+            if (kv.first == key) return kv.second;
+        return dflt;
+    }
+    bool has(const char* key) const {
+        for (const auto& kv : params)
+            if (kv.first == key) return true;
+        return false;
+    }
+    uint32_t u(const char* key, uint32_t dflt = 0) const { return (uint32_t)param(key, (double)dflt); }
+};
+
+struct SlotRW {
+    std::vector<uint32_t> reads, writes;
+};
+
+template <typename T>
+T* arg_ptr(const Dispatch& d, size_t slot) {
+    return reinterpret_cast<T*>(d.args[slot].ptr);
+}
+
+fk_status need_args(const Dispatch& d, size_t n) {
+    if (d.args.size() != n)
+        return set_error(FK_ERR_INVALID, d.kernel + ": expected " + std::to_string(n) + " buffers, got " +
+                                             std::to_string(d.args.size()));
+    for (size_t i = 0; i < n; ++i)
+        if (!d.args[i].ptr || d.args[i].nbytes == 0)
+            return set_error(FK_ERR_INVALID, d.kernel + ": buffer slot " + std::to_string(i) + " is null or empty");
+    return FK_OK;
+}
+
+fk_status need_bytes(const Dispatch& d, size_t slot, size_t bytes) {
+    if (d.args[slot].nbytes < bytes)
+        return set_error(FK_ERR_INVALID, d.kernel + ": buffer slot " + std::to_string(slot) + " holds " +
+                                             std::to_string(d.args[slot].nbytes) + " bytes, kernel needs " +
+                                             std::to_string(bytes));
+    return FK_OK;
+}
+
+size_t weight_bytes(uint32_t n, uint32_t k, uint32_t bits) { return (size_t)n * k * bits / 8; }
+size_t meta_bytes(uint32_t n, uint32_t k, uint32_t group) { return (size_t)n * (k / group) * 2; }
+
+void all_but_last(size_t n, size_t last, SlotRW* rw) {
+    for (uint32_t i = 0; i < n; ++i) (i + last < n ? rw->reads : rw->writes).push_back(i);
+}
+
+// Fills an fk_weight from consecutive slots: dense -> [W]; quantised -> W at
+// `w_slot`, scales at `s_slot`, biases at `b_slot`.
+fk_status bind_weight(const Dispatch& d, uint32_t bits, uint32_t group, uint32_t n, uint32_t k, size_t w_slot,
+                      size_t s_slot, size_t b_slot, fk_weight* w) {
+    if (bits != 4 && bits != 8 && bits != 16) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4, 8 or 16");
+    w->w = d.args[w_slot].ptr;
+    w->n = n;
+    w->k = k;
+    w->bits = bits;
+    w->group = group;
+    w->scales = w->biases = nullptr;
+    FK_TRY(need_bytes(d, w_slot, weight_bytes(n, k, bits)));
+    if (bits != 16) {
+        if (group == 0 || k % group) return set_error(FK_ERR_INVALID, d.kernel + ": bad group size");
+        w->scales = arg_ptr<const uint16_t>(d, s_slot);
+        w->biases = arg_ptr<const uint16_t>(d, b_slot);
+        FK_TRY(need_bytes(d, s_slot, meta_bytes(n, k, group)));
+        FK_TRY(need_bytes(d, b_slot, meta_bytes(n, k, group)));
+    }
+    return FK_OK;
+}
+
+// ------------------------------------------------------------------ families
+
+fk_status plan_step(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 3));
+    for (int i = 0; i < 3; ++i) FK_TRY(need_bytes(d, i, 4));
+    rw->reads = {0};
+    rw->writes = {0, 1, 2};
+    return plan_step_init(arg_ptr<uint32_t>(d, 0), arg_ptr<uint32_t>(d, 1), arg_ptr<uint32_t>(d, 2), l);
+}
+
+// dense: token, table, x ; quantised: token, packed, scales, biases, x
+fk_status plan_embed_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 16), hidden = d.u("hidden"), vocab = d.u("vocab"), group = d.u("group", 64);
+    const size_t n = bits == 16 ? 3 : 5;
+    FK_TRY(need_args(d, n));
+    fk_weight E;
+    FK_TRY(bind_weight(d, bits, group, vocab, hidden, 1, 2, 3, &E));
+    FK_TRY(need_bytes(d, 0, 4));
+    FK_TRY(need_bytes(d, n - 1, (size_t)hidden * 2));
+    all_but_last(n, 1, rw);
+    return plan_embed(&E, arg_ptr<const uint32_t>(d, 0), 0, (float)d.param("output_scale", 1.0),
+                      arg_ptr<uint16_t>(d, n - 1), l);
+}
+
+// x, [norm_w], W_q, W_k, W_v, [s_q, s_k, s_v, b_q, b_k, b_v], [bias_q, bias_k, bias_v], q, k, v
+// (slot order of the reference emitter, src/codegen/kernels/rmsnorm_qkv.rs:159-204)
+fk_status plan_qkv(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), hidden = d.u("hidden");
+    const uint32_t n_q = d.u("n_q"), n_kv = d.u("n_kv");
+    const bool has_norm = d.u("has_norm", 1) != 0, has_bias = d.u("has_bias", 0) != 0;
+    size_t s = 1;
+    const size_t norm_slot = has_norm ? s++ : 0;
+    const size_t w_slot = s;
+    s += 3;
+    const size_t meta_slot = s;
+    if (bits != 16) s += 6;
+    const size_t bias_slot = s;
+    if (has_bias) s += 3;
+    const size_t out_slot = s;
+    s += 3;
+    FK_TRY(need_args(d, s));
+    GemvRequest rq;
+    fk_weight W[3];
+    const uint32_t ns[3] = {n_q, n_kv, n_kv};
+    for (int m = 0; m < 3; ++m) {
+        FK_TRY(bind_weight(d, bits, group, ns[m], hidden, w_slot + m, meta_slot + m, meta_slot + 3 + m, &W[m]));
+        rq.mats[m] = &W[m];
+        if (has_bias) {
+            FK_TRY(need_bytes(d, bias_slot + m, (size_t)ns[m] * 2));
+            rq.bias[m] = arg_ptr<const uint16_t>(d, bias_slot + m);
+        }
+        FK_TRY(need_bytes(d, out_slot + m, (size_t)ns[m] * 2));
+        rq.y[m] = arg_ptr<uint16_t>(d, out_slot + m);
+    }
+    rq.n_mats = 3;
+    FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
+    rq.x = arg_ptr<const uint16_t>(d, 0);
+    if (has_norm) {
+        FK_TRY(need_bytes(d, norm_slot, (size_t)hidden * 2));
+        rq.norm_w = arg_ptr<const uint16_t>(d, norm_slot);
+    }
+    rq.eps = (float)d.param("eps", 1e-6);
+    all_but_last(s, 3, rw);
+    return plan_gemv(rq, l);
+}
+
+// x, [norm_w], W_gate, W_up, [s_g, s_u, b_g, b_u], out
+fk_status plan_gateup(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), hidden = d.u("hidden"), inter = d.u("inter");
+    const bool has_norm = d.u("has_norm", 1) != 0;
+    size_t s = 1;
+    const size_t norm_slot = has_norm ? s++ : 0;
+    const size_t w_slot = s;
+    s += 2;
+    const size_t meta_slot = s;
+    if (bits != 16) s += 4;
+    const size_t out_slot = s++;
+    FK_TRY(need_args(d, s));
+    GemvRequest rq;
+    fk_weight W[2];
+    for (int m = 0; m < 2; ++m) {
+        FK_TRY(bind_weight(d, bits, group, inter, hidden, w_slot + m, meta_slot + m, meta_slot + 2 + m, &W[m]));
+        rq.mats[m] = &W[m];
+    }
+    rq.swiglu = true;
+    const int variant = (int)d.param("variant", 0);
+    if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, d.kernel + ": swiglu variant must be 0, 1 or 2");
+    rq.swiglu_variant = variant;
+    FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)inter * 2));
+    rq.x = arg_ptr<const uint16_t>(d, 0);
+    rq.y[0] = arg_ptr<uint16_t>(d, out_slot);
+    if (has_norm) {
+        FK_TRY(need_bytes(d, norm_slot, (size_t)hidden * 2));
+        rq.norm_w = arg_ptr<const uint16_t>(d, norm_slot);
+    }
+    rq.eps = (float)d.param("eps", 1e-6);
+    all_but_last(s, 1, rw);
+    return plan_gemv(rq, l);
+}
+
+// x, W, [scales, biases], residual, [residual_extra], y   (K = "m", N = "n")
+fk_status plan_linres(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("m"), N = d.u("n");
+    const bool extra = d.u("has_extra", 0) != 0;
+    size_t s = 2;
+    if (bits != 16) s += 2;
+    const size_t res_slot = s++;
+    const size_t extra_slot = extra ? s++ : 0;
+    const size_t out_slot = s++;
+    FK_TRY(need_args(d, s));
+    GemvRequest rq;
+    fk_weight W;
+    FK_TRY(bind_weight(d, bits, group, N, K, 1, 2, 3, &W));
+    rq.mats[0] = &W;
+    FK_TRY(need_bytes(d, 0, (size_t)K * 2));
+    FK_TRY(need_bytes(d, res_slot, (size_t)N * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)N * 2));
+    rq.x = arg_ptr<const uint16_t>(d, 0);
+    rq.res = arg_ptr<const uint16_t>(d, res_slot);
+    if (extra) {
+        FK_TRY(need_bytes(d, extra_slot, (size_t)N * 2));
+        rq.res2 = arg_ptr<const uint16_t>(d, extra_slot);
+    }
+    rq.y[0] = arg_ptr<uint16_t>(d, out_slot);
+    all_but_last(s, 1, rw);
+    return plan_gemv(rq, l);
+}
+
+// x, W, [scales, biases], [bias], y
+fk_status plan_qgemv_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("m"), N = d.u("n");
+    const bool has_bias = d.u("has_bias", 0) != 0;
+    size_t s = 2;
+    if (bits != 16) s += 2;
+    const size_t bias_slot = has_bias ? s++ : 0;
+    const size_t out_slot = s++;
+    FK_TRY(need_args(d, s));
+    GemvRequest rq;
+    fk_weight W;
+    FK_TRY(bind_weight(d, bits, group, N, K, 1, 2, 3, &W));
+    rq.mats[0] = &W;
+    FK_TRY(need_bytes(d, 0, (size_t)K * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)N * 2));
+    rq.x = arg_ptr<const uint16_t>(d, 0);
+    if (has_bias) {
+        FK_TRY(need_bytes(d, bias_slot, (size_t)N * 2));
+        rq.bias[0] = arg_ptr<const uint16_t>(d, bias_slot);
+    }
+    rq.y[0] = arg_ptr<uint16_t>(d, out_slot);
+    all_but_last(s, 1, rw);
+    return plan_gemv(rq, l);
+}
+
+// x, norm_w, W, [scales, biases], logits
+fk_status plan_lm_head(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 16), group = d.u("group", 64), hidden = d.u("hidden"), vocab = d.u("vocab");
+    size_t s = 3;
+    if (bits != 16) s += 2;
+    const size_t out_slot = s++;
+    FK_TRY(need_args(d, s));
+    GemvRequest rq;
+    fk_weight W;
+    FK_TRY(bind_weight(d, bits, group, vocab, hidden, 2, 3, 4, &W));
+    rq.mats[0] = &W;
+    FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)vocab * 2));
+    rq.x = arg_ptr<const uint16_t>(d, 0);
+    rq.norm_w = arg_ptr<const uint16_t>(d, 1);
+    rq.eps = (float)d.param("eps", 1e-6);
+    rq.y[0] = arg_ptr<uint16_t>(d, out_slot);
+    all_but_last(s, 1, rw);
+    return plan_gemv(rq, l);
+}
+
+float base_log2_of(const Dispatch& d) { return (float)log2(d.param("theta", 10000.0)); }
+
+// Q, [q_weight], offset
+fk_status plan_rope_q(const Dispatch& d, Launch* l, SlotRW* rw, bool norm) {
+    const size_t n = norm ? 3 : 2;
+    FK_TRY(need_args(d, n));
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.n_q = d.u("n_heads");
+    a.head_dim = d.u("head_dim");
+    a.rope_dims = d.u("rope_dims", a.head_dim);
+    a.rope_on = a.rope_dims ? 1u : 0u;
+    FK_TRY(need_bytes(d, 0, (size_t)a.n_q * a.head_dim * 2));
+    a.q = arg_ptr<uint16_t>(d, 0);
+    if (norm) {
+        FK_TRY(need_bytes(d, 1, (size_t)a.head_dim * 2));
+        a.q_norm = arg_ptr<const uint16_t>(d, 1);
+    }
+    FK_TRY(need_bytes(d, n - 1, 4));
+    a.offset_ptr = arg_ptr<const uint32_t>(d, n - 1);
+    a.eps = (float)d.param("eps", 1e-6);
+    a.base_log2 = base_log2_of(d);
+    a.capacity = 1;
+    for (uint32_t i = 0; i < n; ++i) rw->reads.push_back(i);
+    rw->writes = {0};
+    return plan_rope_store(a, l);
+}
+
+// K, V, [k_weight], cache_k, cache_v, offset, write_offset
+fk_status plan_rope_kv(const Dispatch& d, Launch* l, SlotRW* rw, bool norm, bool rope) {
+    const size_t n = norm ? 7 : 6;
+    FK_TRY(need_args(d, n));
+    const size_t ck = norm ? 3 : 2;
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.n_kv = d.u("n_kv");
+    a.k_dim = d.u("head_dim");
+    a.v_dim = d.u("v_dim", a.k_dim);
+    a.rope_dims = rope ? d.u("rope_dims", a.k_dim) : 0;
+    a.rope_on = a.rope_dims ? 1u : 0u;
+    a.capacity = d.u("capacity");
+    if (a.capacity == 0) return set_error(FK_ERR_INVALID, d.kernel + ": capacity parameter missing");
+    FK_TRY(need_bytes(d, 0, (size_t)a.n_kv * a.k_dim * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)a.n_kv * a.v_dim * 2));
+    FK_TRY(need_bytes(d, ck, (size_t)a.n_kv * a.capacity * a.k_dim * 2));
+    FK_TRY(need_bytes(d, ck + 1, (size_t)a.n_kv * a.capacity * a.v_dim * 2));
+    FK_TRY(need_bytes(d, ck + 2, 4));
+    FK_TRY(need_bytes(d, ck + 3, 4));
+    a.k = arg_ptr<const uint16_t>(d, 0);
+    a.v = arg_ptr<const uint16_t>(d, 1);
+    if (norm) {
+        FK_TRY(need_bytes(d, 2, (size_t)a.k_dim * 2));
+        a.k_norm = arg_ptr<const uint16_t>(d, 2);
+    }
+    a.cache_k = arg_ptr<uint16_t>(d, ck);
+    a.cache_v = arg_ptr<uint16_t>(d, ck + 1);
+    a.offset_ptr = arg_ptr<const uint32_t>(d, ck + 2);
+    a.write_offset_ptr = arg_ptr<const uint32_t>(d, ck + 3);
+    a.eps = (float)d.param("eps", 1e-6);
+    a.base_log2 = base_log2_of(d);
+    for (uint32_t i = 0; i < n; ++i)
+        if (i != ck && i != ck + 1) rw->reads.push_back(i);
+    rw->writes = {(uint32_t)ck, (uint32_t)ck + 1};
+    return plan_rope_store(a, l);
+}
+
+// Q, K, V, [q_weight, k_weight], cache_k, cache_v, offset   (one launch for the whole rope/store stage)
+fk_status plan_qkv_rope_store(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const bool norm = d.u("has_norm", 0) != 0;
+    const size_t n = norm ? 8 : 6;
+    FK_TRY(need_args(d, n));
+    const size_t ck = norm ? 5 : 3;
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.n_q = d.u("n_heads");
+    a.n_kv = d.u("n_kv");
+    a.head_dim = a.k_dim = a.v_dim = d.u("head_dim");
+    a.rope_dims = d.u("rope_dims", a.head_dim);
+    a.rope_on = a.rope_dims ? 1u : 0u;
+    a.capacity = d.u("capacity");
+    if (a.capacity == 0) return set_error(FK_ERR_INVALID, d.kernel + ": capacity parameter missing");
+    FK_TRY(need_bytes(d, 0, (size_t)a.n_q * a.head_dim * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)a.n_kv * a.head_dim * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)a.n_kv * a.head_dim * 2));
+    FK_TRY(need_bytes(d, ck, (size_t)a.n_kv * a.capacity * a.head_dim * 2));
+    FK_TRY(need_bytes(d, ck + 1, (size_t)a.n_kv * a.capacity * a.head_dim * 2));
+    FK_TRY(need_bytes(d, ck + 2, 4));
+    a.q = arg_ptr<uint16_t>(d, 0);
+    a.k = arg_ptr<const uint16_t>(d, 1);
+    a.v = arg_ptr<const uint16_t>(d, 2);
+    if (norm) {
+        FK_TRY(need_bytes(d, 3, (size_t)a.head_dim * 2));
+        FK_TRY(need_bytes(d, 4, (size_t)a.head_dim * 2));
+        a.q_norm = arg_ptr<const uint16_t>(d, 3);
+        a.k_norm = arg_ptr<const uint16_t>(d, 4);
+    }
+    a.cache_k = arg_ptr<uint16_t>(d, ck);
+    a.cache_v = arg_ptr<uint16_t>(d, ck + 1);
+    a.offset_ptr = arg_ptr<const uint32_t>(d, ck + 2);
+    a.eps = (float)d.param("eps", 1e-6);
+    a.base_log2 = base_log2_of(d);
+    for (uint32_t i = 0; i < n; ++i)
+        if (i != ck && i != ck + 1) rw->reads.push_back(i);
+    rw->writes = {0, (uint32_t)ck, (uint32_t)ck + 1};
+    return plan_rope_store(a, l);
+}
+
+// Q, K, V, kv_len, out, partials, counters
+fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 7));
+    const uint32_t n_heads = d.u("n_heads"), n_kv = d.u("n_kv"), qk = d.u("qk_dim", d.u("head_dim"));
+    const uint32_t vd = d.u("v_dim", qk), capacity = d.u("capacity"), max_len = d.u("max_len", capacity);
+    if (n_heads == 0 || n_kv == 0 || qk == 0 || capacity == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / head_dim / capacity parameters missing");
+    const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)qk);  // sdpa_decode.rs:248-252
+    FK_TRY(need_bytes(d, 0, (size_t)n_heads * qk * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)n_kv * capacity * qk * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)n_kv * capacity * vd * 2));
+    FK_TRY(need_bytes(d, 3, 4));
+    FK_TRY(need_bytes(d, 4, (size_t)n_heads * vd * 2));
+    size_t pb = 0, cb = 0;
+    FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, vd, max_len, &pb, &cb));
+    FK_TRY(need_bytes(d, 5, pb));
+    FK_TRY(need_bytes(d, 6, cb));
+    rw->reads = {0, 1, 2, 3, 5, 6};
+    rw->writes = {4, 5, 6};
+    return plan_sdpa_decode(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<const uint16_t>(d, 2),
+                            arg_ptr<uint16_t>(d, 4), arg_ptr<const uint32_t>(d, 3), 0, max_len, n_heads, n_kv, qk, vd,
+                            capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l);
+}
+
+// logits, next_tok, workspace, [history, hist_counter]
+fk_status plan_argmax_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const bool hist = d.args.size() == 5;
+    FK_TRY(need_args(d, hist ? 5 : 3));
+    const uint32_t vocab = d.u("vocab");
+    FK_TRY(need_bytes(d, 0, (size_t)vocab * 2));
+    FK_TRY(need_bytes(d, 1, 4));
+    FK_TRY(need_bytes(d, 2, kArgmaxWorkspaceBytes));
+    uint32_t cap = 0;
+    if (hist) {
+        cap = (uint32_t)(d.args[3].nbytes / 4);
+        FK_TRY(need_bytes(d, 4, 4));
+        rw->reads = {0, 2, 4};
+        rw->writes = {1, 2, 3, 4};
+    } else {
+        rw->reads = {0, 2};
+        rw->writes = {1, 2};
+    }
+    return plan_argmax(arg_ptr<const uint16_t>(d, 0), vocab, arg_ptr<uint32_t>(d, 1),
+                       hist ? arg_ptr<uint32_t>(d, 3) : nullptr, hist ? arg_ptr<uint32_t>(d, 4) : nullptr, cap,
+                       d.args[2].ptr, l);
+}
+
+struct Family {
+    const char* prefix;
+    fk_status (*plan)(const Dispatch&, Launch*, SlotRW*);
+};
+
+// Longest prefix first where one family name begins another.
+const Family kFamilies[] = {
+    {"fusekit_step_init", plan_step},
+    {"fusekit_embed_lookup_decode", plan_embed_d},
+    {"fusekit_rmsnorm_qkv", plan_qkv},
+    {"fusekit_qmv_fanout", plan_qkv},
+    {"fusekit_rmsnorm_gateup_swiglu", plan_gateup},
+    {"fusekit_qmv_swiglu", plan_gateup},
+    {"fusekit_linear_residual", plan_linres},
+    {"fusekit_final_rmsnorm_lm_head", plan_lm_head},
+    {"fusekit_qgemv", plan_qgemv_d},
+    {"fusekit_rmsnorm_rope_q_decode",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_q(d, l, rw, true); }},
+    {"fusekit_rmsnorm_rope_kv_cache_store_decode",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, true, true); }},
+    {"fusekit_rope_q_decode", [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_q(d, l, rw, false); }},
+    {"fusekit_rope_kv_cache_store_decode",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, true); }},
+    {"fusekit_kv_cache_store_decode",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, false); }},
+    {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
+    {"fusekit_sdpa_decode", plan_sdpa_d},
+    {"fusekit_argmax_logits_decode", plan_argmax_d},
+};
+
+const Family* find_family(const std::string& kernel) {
+    const Family* best = nullptr;
+    size_t best_len = 0;
+    for (const Family& f : kFamilies) {
+        const size_t n = strlen(f.prefix);
+        if (kernel.compare(0, n, f.prefix) == 0 && (kernel.size() == n || kernel[n] == '_') && n > best_len) {
+            best = &f;
+            best_len = n;
+        }
+    }
+    return best;
+}
+
+fk_status plan_dispatch(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const Family* f = find_family(d.kernel);
+    if (!f) return set_error(FK_ERR_INVALID, "kernel '" + d.kernel + "' is not in this library");  // lib.rs:412-415
+    rw->reads.clear();
+    rw->writes.clear();
+    return f->plan(d, l, rw);
+}
+
+fk_status copy_dispatch(const fk_dispatch& in, Dispatch* out) {
+    if (!in.kernel) return set_error(FK_ERR_INVALID, "dispatch without a kernel name");
+    if ((in.n_args && !in.args) || (in.n_params && !in.params)) return set_error(FK_ERR_INVALID, "null args / params");
+    out->kernel = in.kernel;
+    out->args.assign(in.args, in.args + in.n_args);
+    out->params.clear();
+    for (uint32_t i = 0; i < in.n_params; ++i) {
+        if (!in.params[i].key) return set_error(FK_ERR_INVALID, "parameter without a key");
+        out->params.emplace_back(in.params[i].key, in.params[i].value);
+    }
+    return FK_OK;
+}
+
+bool overlap(const fk_arg& a, const fk_arg& b) {
+    const char* a0 = (const char*)a.ptr;
+    const char* b0 = (const char*)b.ptr;
+    return a0 < b0 + b.nbytes && b0 < a0 + a.nbytes;
+}
+
+struct Node {
+    Dispatch d;
+    Launch launch;
+    SlotRW rw;
+    hipGraphNode_t node = nullptr;
+    std::vector<uint32_t> deps;
+};
+
+struct Graph {
+    std::vector<Node> nodes;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct DispatcherState {
+    std::mutex mu;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::vector<std::unique_ptr<Graph>> graphs;
+    std::vector<std::string> kernel_names;
+    std::vector<const char*> kernel_name_ptrs;
+    std::string task_graph_path;
+    bool pending = false;
+};
+
+std::mutex g_mu;
+std::vector<std::unique_ptr<DispatcherState>> g_dispatchers;  // append-only, like lib.rs:112
+
+fk_status get_dispatcher(fk_handle h, DispatcherState** out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (h == 0 || h > g_dispatchers.size()) return set_error(FK_ERR_INVALID, "invalid dispatcher handle");  // lib.rs:198
+    *out = g_dispatchers[h - 1].get();
+    return FK_OK;
+}
+
+fk_status get_graph(DispatcherState* ds, uint32_t id, Graph** out) {
+    if (id >= ds->graphs.size()) return set_error(FK_ERR_INVALID, "invalid graph id");  // lib.rs:592
+    *out = ds->graphs[id].get();
+    return FK_OK;
+}
+
+hipKernelNodeParams node_params(Node& n, void** slot) {
+    hipKernelNodeParams p;
+    memset(&p, 0, sizeof(p));
+    p.func = const_cast<void*>(n.launch.func);
+    p.gridDim = n.launch.grid;
+    p.blockDim = n.launch.block;
+    p.sharedMemBytes = n.launch.shmem;
+    *slot = n.launch.args;
+    p.kernelParams = slot;
+    p.extra = nullptr;
+    return p;
+}
+
+// RAW / WAW / WAR edges on overlapping byte ranges, transitively reduced.
+void derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
+    const size_t n = nodes.size();
+    const size_t words = (n + 63) / 64;
+    std::vector<std::vector<uint64_t>> anc(n, std::vector<uint64_t>(words, 0));
+    for (size_t i = 0; i < n; ++i) {
+        std::vector<uint32_t> cand;
+        for (size_t j = 0; j < i; ++j) {
+            bool dep = barriers && barriers[i];
+            const Node &a = nodes[j], &b = nodes[i];
+            for (uint32_t ws : a.rw.writes) {
+                if (dep) break;
+                for (uint32_t s : b.rw.reads)
+                    if (overlap(a.d.args[ws], b.d.args[s])) { dep = true; break; }
+                if (dep) break;
+                for (uint32_t s : b.rw.writes)
+                    if (overlap(a.d.args[ws], b.d.args[s])) { dep = true; break; }
+            }
+            for (uint32_t rs : a.rw.reads) {
+                if (dep) break;
+                for (uint32_t s : b.rw.writes)
+                    if (overlap(a.d.args[rs], b.d.args[s])) { dep = true; break; }
+            }
+            if (dep) cand.push_back((uint32_t)j);
+        }
+        // keep a candidate only if no later candidate already descends from it
+        nodes[i].deps.clear();
+        for (size_t c = cand.size(); c-- > 0;) {
+            const uint32_t j = cand[c];
+            if (anc[i][j / 64] >> (j % 64) & 1) continue;  // implied through a kept dependency
+            nodes[i].deps.push_back(j);
+            anc[i][j / 64] |= 1ull << (j % 64);
+            for (size_t w = 0; w < words; ++w) anc[i][w] |= anc[j][w];
+        }
+        std::sort(nodes[i].deps.begin(), nodes[i].deps.end());
+    }
+}
+
+fk_status timed(DispatcherState* ds, double* gpu_seconds, const std::function<fk_status()>& body) {
+    FK_HIP(hipEventRecord(ds->ev0, ds->stream));
+    FK_TRY(body());
+    FK_HIP(hipEventRecord(ds->ev1, ds->stream));
+    FK_HIP(hipEventSynchronize(ds->ev1));
+    float ms = 0.f;
+    FK_HIP(hipEventElapsedTime(&ms, ds->ev0, ds->ev1));
+    if (gpu_seconds) *gpu_seconds = ms * 1e-3;
+    return FK_OK;
+}
+
+}  // namespace
+}  // namespace fk
+
+using namespace fk;
+
+extern "C" {
+
+fk_status fk_load_dispatcher(const char* code_object_path, const char* task_graph_path, fk_handle* out) {
+    if (!out) return set_error(FK_ERR_INVALID, "null out");
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    auto ds = std::make_unique<DispatcherState>();
+    // The kernels are compiled into this library; a code-object path is accepted
+    // for artifact compatibility and only checked for existence.
+    if (code_object_path && *code_object_path && strcmp(code_object_path, "builtin") != 0) {
+        std::ifstream f(code_object_path, std::ios::binary);
+        if (!f) return set_error(FK_ERR_NOT_FOUND, std::string("code object not found: ") + code_object_path);
+    }
+    if (task_graph_path && *task_graph_path) {
+        std::ifstream f(task_graph_path, std::ios::binary);
+        if (!f) return set_error(FK_ERR_NOT_FOUND, std::string("task graph not found: ") + task_graph_path);
+        std::stringstream ss;
+        ss << f.rdbuf();
+        json::Value root;
+        std::string err;
+        const std::string text = ss.str();
+        if (!json::Parser(text).parse(&root, &err)) return set_error(FK_ERR_IO, "task_graph.json: " + err);
+        const json::Value* ver = root.get("version");
+        if (!ver || !ver->is_number() || (int)ver->num != 2)
+            return set_error(FK_ERR_INVALID, "task_graph.json: unsupported version (need 2)");  // plan.rs:175-180
+        const json::Value* tasks = root.get("tasks");
+        if (!tasks || !tasks->is_array()) return set_error(FK_ERR_INVALID, "task_graph.json: missing tasks[]");
+        for (const json::Value& t : tasks->arr) {
+            const json::Value* k = t.get("kernel");
+            if (!k || !k->is_string()) return set_error(FK_ERR_INVALID, "task_graph.json: task without kernel name");
+            if (!find_family(k->str))
+                return set_error(FK_ERR_INVALID, "kernel '" + k->str + "' is not in this library");
+            if (std::find(ds->kernel_names.begin(), ds->kernel_names.end(), k->str) == ds->kernel_names.end())
+                ds->kernel_names.push_back(k->str);
+        }
+        ds->task_graph_path = task_graph_path;
+    } else {
+        for (const Family& f : kFamilies) ds->kernel_names.push_back(f.prefix);
+    }
+    for (const std::string& s : ds->kernel_names) ds->kernel_name_ptrs.push_back(s.c_str());
+    FK_HIP(hipStreamCreateWithFlags(&ds->stream, hipStreamNonBlocking));
+    FK_HIP(hipEventCreate(&ds->ev0));
+    FK_HIP(hipEventCreate(&ds->ev1));
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_dispatchers.push_back(std::move(ds));
+    *out = (fk_handle)g_dispatchers.size();
+    return FK_OK;
+}
+
+fk_status fk_kernel_names(fk_handle h, const char* const** names, size_t* n) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!names || !n) return set_error(FK_ERR_INVALID, "null out");
+    *names = ds->kernel_name_ptrs.data();
+    *n = ds->kernel_name_ptrs.size();
+    return FK_OK;
+}
+
+fk_status fk_dispatcher_stream(fk_handle h, fk_stream* out) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!out) return set_error(FK_ERR_INVALID, "null out");
+    *out = ds->stream;
+    return FK_OK;
+}
+
+fk_status fk_dispatch_batch(fk_handle h, const fk_dispatch* list, size_t n, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!list && n) return set_error(FK_ERR_INVALID, "null dispatch list");
+    std::lock_guard<std::mutex> lk(ds->mu);
+    std::vector<Launch> launches(n);
+    for (size_t i = 0; i < n; ++i) {  // validate everything before launching anything
+        Dispatch d;
+        SlotRW rw;
+        FK_TRY(copy_dispatch(list[i], &d));
+        FK_TRY(plan_dispatch(d, &launches[i], &rw));
+    }
+    return timed(ds, gpu_seconds, [&]() -> fk_status {
+        for (size_t i = 0; i < n; ++i) FK_TRY(run_launch(launches[i], ds->stream));  // stream order = barrier between each
+        return FK_OK;
+    });
+}
+
+fk_status fk_dispatch_kernel(fk_handle h, const fk_dispatch* d, double* gpu_seconds) {
+    if (!d) return set_error(FK_ERR_INVALID, "null dispatch");
+    return fk_dispatch_batch(h, d, 1, gpu_seconds);
+}
+
+fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const uint8_t* barriers, uint32_t* graph_id) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!list || n == 0 || !graph_id) return set_error(FK_ERR_INVALID, "empty dispatch list or null out");
+    std::lock_guard<std::mutex> lk(ds->mu);
+    auto g = std::make_unique<Graph>();
+    g->nodes.resize(n);
+    for (size_t i = 0; i < n; ++i) {
+        FK_TRY(copy_dispatch(list[i], &g->nodes[i].d));
+        FK_TRY(plan_dispatch(g->nodes[i].d, &g->nodes[i].launch, &g->nodes[i].rw));
+    }
+    derive_edges(g->nodes, barriers);
+    FK_HIP(hipGraphCreate(&g->graph, 0));
+    for (size_t i = 0; i < n; ++i) {
+        Node& nd = g->nodes[i];
+        std::vector<hipGraphNode_t> deps;
+        for (uint32_t j : nd.deps) deps.push_back(g->nodes[j].node);
+        void* slot = nullptr;
+        hipKernelNodeParams p = node_params(nd, &slot);
+        FK_HIP(hipGraphAddKernelNode(&nd.node, g->graph, deps.data(), deps.size(), &p));
+    }
+    FK_HIP(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    ds->graphs.push_back(std::move(g));
+    *graph_id = (uint32_t)ds->graphs.size() - 1;
+    return FK_OK;
+}
+
+fk_status fk_graph_info(fk_handle h, uint32_t graph_id, uint32_t* n_nodes, uint32_t* n_edges) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    uint32_t e = 0;
+    for (const Node& nd : g->nodes) e += (uint32_t)nd.deps.size();
+    if (n_nodes) *n_nodes = (uint32_t)g->nodes.size();
+    if (n_edges) *n_edges = e;
+    return FK_OK;
+}
+
+fk_status fk_graph_node_deps(fk_handle h, uint32_t graph_id, uint32_t node, uint32_t* deps, uint32_t cap, uint32_t* n) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (node >= g->nodes.size() || !n) return set_error(FK_ERR_INVALID, "node index out of range");
+    const auto& d = g->nodes[node].deps;
+    *n = (uint32_t)d.size();
+    for (uint32_t i = 0; i < d.size() && i < cap && deps; ++i) deps[i] = d[i];
+    return FK_OK;
+}
+
+fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_binding_update* ups, size_t n) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!ups && n) return set_error(FK_ERR_INVALID, "null updates");
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    // validate all, then apply (a failed update leaves the graph untouched)
+    std::vector<Dispatch> patched;
+    std::vector<uint32_t> touched;
+    for (size_t i = 0; i < n; ++i) {
+        const fk_binding_update& u = ups[i];
+        if (u.cmd_idx >= g->nodes.size()) return set_error(FK_ERR_INVALID, "binding update: command index out of range");
+        if (u.slot >= g->nodes[u.cmd_idx].d.args.size())
+            return set_error(FK_ERR_INVALID, "binding update: slot out of range");
+        if (!u.ptr || u.nbytes == 0) return set_error(FK_ERR_INVALID, "binding update: null or empty buffer");  // lib.rs:602-606
+        auto it = std::find(touched.begin(), touched.end(), u.cmd_idx);
+        size_t k;
+        if (it == touched.end()) {
+            touched.push_back(u.cmd_idx);
+            patched.push_back(g->nodes[u.cmd_idx].d);
+            k = patched.size() - 1;
+        } else {
+            k = (size_t)(it - touched.begin());
+        }
+        patched[k].args[u.slot] = fk_arg{u.ptr, u.nbytes};
+    }
+    std::vector<Launch> launches(touched.size());
+    for (size_t k = 0; k < touched.size(); ++k) {
+        SlotRW rw;
+        FK_TRY(plan_dispatch(patched[k], &launches[k], &rw));
+    }
+    for (size_t k = 0; k < touched.size(); ++k) {
+        Node& nd = g->nodes[touched[k]];
+        nd.d = patched[k];
+        nd.launch = launches[k];
+        void* slot = nullptr;
+        hipKernelNodeParams p = node_params(nd, &slot);
+        FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.node, &p));
+    }
+    return FK_OK;
+}
+
+fk_status fk_execute_graph(fk_handle h, uint32_t graph_id, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is pending; call fk_wait_pending first");
+    return timed(ds, gpu_seconds, [&]() -> fk_status {
+        FK_HIP(hipGraphLaunch(g->exec, ds->stream));
+        return FK_OK;
+    });
+}
+
+fk_status fk_execute_graph_repeat(fk_handle h, uint32_t graph_id, uint32_t count, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is pending; call fk_wait_pending first");
+    return timed(ds, gpu_seconds, [&]() -> fk_status {
+        for (uint32_t i = 0; i < count; ++i) FK_HIP(hipGraphLaunch(g->exec, ds->stream));
+        return FK_OK;
+    });
+}
+
+fk_status fk_execute_graph_range(fk_handle h, uint32_t graph_id, uint32_t start, uint32_t end, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (start > end || end > g->nodes.size()) return set_error(FK_ERR_INVALID, "graph range out of bounds");  // lib.rs:781-786
+    return timed(ds, gpu_seconds, [&]() -> fk_status {
+        for (uint32_t i = start; i < end; ++i) FK_TRY(run_launch(g->nodes[i].launch, ds->stream));
+        return FK_OK;
+    });
+}
+
+fk_status fk_profile_graph_nodes(fk_handle h, uint32_t graph_id, double* per_node_seconds, size_t n) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (!per_node_seconds || n < g->nodes.size()) return set_error(FK_ERR_INVALID, "profile buffer too small");
+    for (size_t i = 0; i < g->nodes.size(); ++i) {
+        FK_TRY(timed(ds, &per_node_seconds[i], [&]() -> fk_status { return run_launch(g->nodes[i].launch, ds->stream); }));
+    }
+    return FK_OK;
+}
+
+fk_status fk_submit_graph_async(fk_handle h, uint32_t graph_id) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is already pending");  // one in flight, lib.rs:57,695
+    FK_HIP(hipEventRecord(ds->ev0, ds->stream));
+    FK_HIP(hipGraphLaunch(g->exec, ds->stream));
+    FK_HIP(hipEventRecord(ds->ev1, ds->stream));
+    ds->pending = true;
+    return FK_OK;
+}
+
+fk_status fk_wait_pending(fk_handle h, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    if (!ds->pending) {
+        if (gpu_seconds) *gpu_seconds = 0.0;
+        return FK_OK;
+    }
+    FK_HIP(hipEventSynchronize(ds->ev1));
+    float ms = 0.f;
+    FK_HIP(hipEventElapsedTime(&ms, ds->ev0, ds->ev1));
+    if (gpu_seconds) *gpu_seconds = ms * 1e-3;
+    ds->pending = false;
+    return FK_OK;
+}
+
+fk_status fk_decode_chunk(fk_handle h, uint32_t graph_id, const fk_decode_uniforms* u, uint32_t start_offset,
+                          uint32_t seed_token, uint32_t count, uint32_t* out_tokens, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!u || !u->token || !u->step_counter || !u->hist_counter || !u->history)
+        return set_error(FK_ERR_INVALID, "decode uniforms: null pointer");
+    if (count == 0 || count > u->hist_capacity) return set_error(FK_ERR_INVALID, "decode chunk: count outside (0, history capacity]");
+    if (!out_tokens) return set_error(FK_ERR_INVALID, "null out_tokens");
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is pending; call fk_wait_pending first");
+    // host seeds the counters and the first token (lib.rs:1299-1303) ...
+    const uint32_t zero = 0;
+    FK_HIP(hipMemcpyAsync(u->step_counter, &start_offset, 4, hipMemcpyHostToDevice, ds->stream));
+    FK_HIP(hipMemcpyAsync(u->hist_counter, &zero, 4, hipMemcpyHostToDevice, ds->stream));
+    FK_HIP(hipMemcpyAsync(u->token, &seed_token, 4, hipMemcpyHostToDevice, ds->stream));
+    FK_HIP(hipStreamSynchronize(ds->stream));
+    // ... then replays the graph back to back and waits only for the last (lib.rs:1351-1392)
+    FK_TRY(timed(ds, gpu_seconds, [&]() -> fk_status {
+        for (uint32_t i = 0; i < count; ++i) FK_HIP(hipGraphLaunch(g->exec, ds->stream));
+        return FK_OK;
+    }));
+    FK_HIP(hipMemcpy(out_tokens, u->history, (size_t)count * 4, hipMemcpyDeviceToHost));
+    return FK_OK;
+}
+
+fk_status fk_decode_chunk_host_loop(fk_handle h, uint32_t graph_id, const fk_decode_uniforms* u,
+                                    uint32_t start_offset, const uint32_t* tokens_in, uint32_t count,
+                                    uint32_t* out_next, double* gpu_seconds) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!u || !u->token || !u->step_counter || !u->hist_counter)
+        return set_error(FK_ERR_INVALID, "decode uniforms: null pointer");
+    if (!tokens_in || !out_next || count == 0) return set_error(FK_ERR_INVALID, "host loop: null tokens or zero count");
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is pending; call fk_wait_pending first");
+    double total = 0.0;
+    for (uint32_t i = 0; i < count; ++i) {
+        const uint32_t off = start_offset + i, hist = 0;
+        FK_HIP(hipMemcpyAsync(u->token, &tokens_in[i], 4, hipMemcpyHostToDevice, ds->stream));
+        FK_HIP(hipMemcpyAsync(u->step_counter, &off, 4, hipMemcpyHostToDevice, ds->stream));
+        FK_HIP(hipMemcpyAsync(u->hist_counter, &hist, 4, hipMemcpyHostToDevice, ds->stream));
+        FK_HIP(hipStreamSynchronize(ds->stream));
+        double t = 0.0;
+        FK_TRY(timed(ds, &t, [&]() -> fk_status {
+            FK_HIP(hipGraphLaunch(g->exec, ds->stream));
+            return FK_OK;
+        }));
+        total += t;
+        FK_HIP(hipMemcpy(&out_next[i], u->token, 4, hipMemcpyDeviceToHost));
+    }
+    if (gpu_seconds) *gpu_seconds = total;
+    return FK_OK;
+}
+
+}  // extern "C"

@@ -10,11 +10,10 @@
 // go through LDS, and a second phase adds each row's partials in a fixed order
 // and applies the epilogue.  No atomics touch the value path.
 //
-// int4 dequantisation: (w >> 4j) & 0x000F000F picks nibbles j and j+4; OR-ing
-// 0x43004300 makes the two bf16 values 128+q exactly, which v_dot2c_f32_bf16
-// multiplies with the matching activation pair.  The 128 offset and the affine
-// bias fold into one per-chunk correction: s*(D - 128*Sx) + b*Sx, Sx being the
-// chunk's activation sum (computed once per block).
+// int4 dequantisation costs 7 VALU ops per packed word (two masks, one shift,
+// four fp8->bf16 pair converts, see q4_word_dot) plus four v_dot2c_f32_bf16; the
+// affine bias folds into one per-chunk term b * Sx, Sx being the chunk's
+// activation sum (computed once per block).
 #pragma once
 #include "fk_device.hpp"
 
@@ -73,20 +72,22 @@ __host__ __device__ inline uint32_t gemv_lds_bytes(uint32_t cpr, uint32_t seg_ch
     return ChunkTraits<KIND>::kPieces * cpr * 16u + cpr * 4u + nseg * seg_pad * 4u + 64u;
 }
 
-// (a & m) | o in one VALU op; the compiler splits it when both constants sit in
-// SGPRs, so the instruction is named with the OR term held in a VGPR.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t o) {
-    uint32_t d;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(m), "v"(o));
-    return d;
-}
-
+// Eight int4 codes of one packed word against eight activations.  A byte
+// 0000nnnn read as fp8 e4m3 is exactly n * 2^-9 (subnormal for n < 8, (8+m)*2^-9
+// above), so v_cvt_scalef32_pk_bf16_fp8 with scale 512 turns two such bytes into
+// the bf16 pair (n_a, n_b) in one instruction.  w & 0x0F0F0F0F holds nibbles
+// 0,2,4,6 in its bytes and (w >> 4) & 0x0F0F0F0F nibbles 1,3,5,7, which fixes the
+// activation pairing: xp = {(x0,x2), (x4,x6), (x1,x3), (x5,x7)}.
 __device__ __forceinline__ float q4_word_dot(uint32_t w, uint4 xp, float d) {
-    const uint32_t M = 0x000F000Fu, B = 0x43004300u;
-    d = dot2_bf16(and_or(w, M, B), xp.x, d);
-    d = dot2_bf16(and_or(w >> 4, M, B), xp.y, d);
-    d = dot2_bf16(and_or(w >> 8, M, B), xp.z, d);
-    d = dot2_bf16(and_or(w >> 12, M, B), xp.w, d);
+    const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+    const bf16x2_t e0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false);
+    const bf16x2_t e1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, true);
+    const bf16x2_t o0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, false);
+    const bf16x2_t o1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, true);
+    d = __builtin_amdgcn_fdot2_f32_bf16(e0, __builtin_bit_cast(bf16x2_t, xp.x), d, false);
+    d = __builtin_amdgcn_fdot2_f32_bf16(e1, __builtin_bit_cast(bf16x2_t, xp.y), d, false);
+    d = __builtin_amdgcn_fdot2_f32_bf16(o0, __builtin_bit_cast(bf16x2_t, xp.z), d, false);
+    d = __builtin_amdgcn_fdot2_f32_bf16(o1, __builtin_bit_cast(bf16x2_t, xp.w), d, false);
     return d;
 }
 
@@ -109,7 +110,7 @@ __device__ __forceinline__ float chunk_partial(uint4 wv, uint32_t s_bits, uint32
         d0 = q4_word_dot(wv.z, xs[2 * cpr + c], d0);
         d1 = q4_word_dot(wv.w, xs[3 * cpr + c], d1);
         const float s = bf16_bits_to_f32(s_bits), b = bf16_bits_to_f32(b_bits), sum_x = sx[c];
-        return fmaf(s, fmaf(-128.f, sum_x, d0 + d1), b * sum_x);
+        return fmaf(s, d0 + d1, b * sum_x);
     } else if constexpr (KIND == W_Q8) {
         float d0 = 0.f, d1 = 0.f;
         d0 = q8_word_dot(wv.x, xs[c], d0);
@@ -193,10 +194,10 @@ __device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, 
             }
         }
         if constexpr (KIND == W_Q4) {
-            // word j of chunk c; nibble pairs (0,4) (1,5) (2,6) (3,7)
+            // word j of chunk c; activation pairs (0,2) (4,6) (1,3) (5,7) as q4_word_dot wants
             const uint32_t c = t >> 2, j = t & 3u;
-            xs[j * cpr + c] = make_uint4(pack_bf16(f[0], f[4]), pack_bf16(f[1], f[5]), pack_bf16(f[2], f[6]),
-                                         pack_bf16(f[3], f[7]));
+            xs[j * cpr + c] = make_uint4(pack_bf16(f[0], f[2]), pack_bf16(f[4], f[6]), pack_bf16(f[1], f[3]),
+                                         pack_bf16(f[5], f[7]));
         } else if constexpr (KIND == W_Q8) {
             const uint32_t c = t >> 1, j = (t & 1u) * 2u;
             xs[j * cpr + c] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),

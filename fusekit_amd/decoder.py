@@ -1,0 +1,288 @@
+"""Dense decoder on the MI355X backend: random-init weights in HBM, the per-token task
+list in the reference's decode_pipeline order and the generation loop.
+
+Task order follows the reference's decode pipeline (src/codegen/task_graph_json.rs:54-65):
+  step_init -> embed_lookup -> L x [ rmsnorm_qkv | rope(+head-norm) + KV store | sdpa |
+  linear_residual(o_proj) | rmsnorm_gateup_swiglu | linear_residual(down_proj) ]
+  -> final_rmsnorm_lm_head -> argmax (+ history).
+The generation loop mirrors `_fast_generate_step`
+(python/fusekit_runtime/__init__.py:4782-5141): prompt through the graph with forced
+tokens, greedy first token, then native chunks of FK_CHUNK tokens with the argmax fed
+back on the GPU.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from . import native
+from .native import DeviceBuffer, DeviceWeight, check, lib
+from .runtime import FK_CHUNK, Dispatch, Dispatcher, arg, make_uniforms
+
+
+@dataclass
+class DecoderConfig:
+    n_layers: int
+    hidden: int
+    n_heads: int
+    n_kv: int
+    head_dim: int
+    inter: int
+    vocab: int
+    eps: float = 1e-6
+    theta: float = 1e6
+    bits: int = 4            # 4 / 8: MLX-affine projections; 16: dense bf16
+    group: int = 64
+    qk_norm: bool = False    # per-head q/k RMSNorm
+    qkv_bias: bool = False
+    swiglu_variant: int = 0
+    capacity: int = 1024     # KV-cache rows per layer
+    fuse_rope_store: bool = True   # one launch for rope_q + rope_kv_store (False: the reference's two)
+
+    @property
+    def n_q(self) -> int:
+        return self.n_heads * self.head_dim
+
+    @property
+    def n_kvd(self) -> int:
+        return self.n_kv * self.head_dim
+
+    def layer_param_bytes(self) -> int:
+        """Algorithmic weight bytes one token streams per layer (packed + scales + biases)."""
+        per = self.bits / 8 + (0 if self.bits == 16 else 4 / self.group)
+        params = self.hidden * (self.n_q + 2 * self.n_kvd) + self.n_q * self.hidden + 3 * self.inter * self.hidden
+        return int(params * per)
+
+    def token_bytes(self, ctx: int) -> int:
+        """Algorithmic HBM bytes per decoded token at context `ctx`: layer weights + tied bf16
+        LM head + K/V rows read by attention."""
+        kv = self.n_layers * 2 * self.n_kv * self.head_dim * 2 * ctx
+        return self.n_layers * self.layer_param_bytes() + self.vocab * self.hidden * 2 + kv
+
+
+QWEN25_05B_LIKE = dict(n_layers=24, hidden=896, n_heads=14, n_kv=2, head_dim=64, inter=4864, vocab=151936,
+                       qkv_bias=True)
+DENSE_4B = dict(n_layers=36, hidden=2560, n_heads=32, n_kv=8, head_dim=128, inter=9728, vocab=151936, qk_norm=True)
+
+
+def _synth(buf: DeviceBuffer, count: int, seed: int, mean: float, std: float, kind: int, bound: int = 0) -> None:
+    check(lib.fk_synth_fill(C.c_void_p(buf.ptr), C.c_size_t(count), C.c_uint64(seed), C.c_float(mean),
+                            C.c_float(std), C.c_uint32(kind), C.c_uint32(bound), None))
+
+
+def quantize_on_device(w_f32: DeviceBuffer, n: int, k: int, bits: int, group: int) -> DeviceWeight:
+    """fp32 [n, k] in HBM -> MLX-affine DeviceWeight (fk_quantize_affine)."""
+    W = DeviceWeight.__new__(DeviceWeight)
+    W.n, W.k, W.bits, W.group = n, k, bits, group
+    W.w = DeviceBuffer(n * k * bits // 8)
+    W.scales = DeviceBuffer(n * (k // group) * 2)
+    W.biases = DeviceBuffer(n * (k // group) * 2)
+    check(lib.fk_quantize_affine(C.c_void_p(w_f32.ptr), C.c_size_t(n), C.c_size_t(k), C.c_uint32(bits),
+                                 C.c_uint32(group), C.c_void_p(W.w.ptr), C.c_void_p(W.scales.ptr),
+                                 C.c_void_p(W.biases.ptr), None))
+    return W
+
+
+class DecoderWeights:
+    """Weights of one model resident in HBM, keyed by the reference's parameter paths
+    (`layers.<l>.self_attn.q_proj` ..., src/codegen/kernels/mod.rs:4907-4939)."""
+
+    def __init__(self, cfg: DecoderConfig):
+        self.cfg = cfg
+        self.mats: Dict[str, DeviceWeight] = {}
+        self.vecs: Dict[str, DeviceBuffer] = {}
+
+    @classmethod
+    def random_init(cls, cfg: DecoderConfig, seed: int = 0, std: float = 0.02) -> "DecoderWeights":
+        """Projections ~ N(0, std^2) quantised on the device; norm weights ~ 1 + N(0, 0.1^2);
+        tied bf16 embedding ~ N(0, std^2); biases ~ N(0, 0.5^2)."""
+        self = cls(cfg)
+        biggest = max(cfg.inter * cfg.hidden, cfg.n_q * cfg.hidden)
+        tmp = DeviceBuffer(biggest * 4) if cfg.bits != 16 else None
+        counter = [seed * 100003 + 1]
+
+        def next_seed() -> int:
+            counter[0] += 1
+            return counter[0]
+
+        def matrix(name: str, n: int, k: int) -> None:
+            if cfg.bits == 16:
+                W = DeviceWeight.__new__(DeviceWeight)
+                W.n, W.k, W.bits, W.group = n, k, 16, 0
+                W.w, W.scales, W.biases = DeviceBuffer(n * k * 2), None, None
+                _synth(W.w, n * k, next_seed(), 0.0, std, 1)
+            else:
+                _synth(tmp, n * k, next_seed(), 0.0, std, 0)
+                W = quantize_on_device(tmp, n, k, cfg.bits, cfg.group)
+            self.mats[name] = W
+
+        def vector(name: str, n: int, mean: float, sd: float) -> None:
+            b = DeviceBuffer(n * 2)
+            _synth(b, n, next_seed(), mean, sd, 1)
+            self.vecs[name] = b
+
+        emb = DeviceWeight.__new__(DeviceWeight)
+        emb.n, emb.k, emb.bits, emb.group = cfg.vocab, cfg.hidden, 16, 0
+        emb.w, emb.scales, emb.biases = DeviceBuffer(cfg.vocab * cfg.hidden * 2), None, None
+        _synth(emb.w, cfg.vocab * cfg.hidden, next_seed(), 0.0, std, 1)
+        self.mats["embed_tokens"] = emb
+        vector("final_norm", cfg.hidden, 1.0, 0.1)
+        for l in range(cfg.n_layers):
+            p = f"layers.{l}."
+            matrix(p + "self_attn.q_proj", cfg.n_q, cfg.hidden)
+            matrix(p + "self_attn.k_proj", cfg.n_kvd, cfg.hidden)
+            matrix(p + "self_attn.v_proj", cfg.n_kvd, cfg.hidden)
+            matrix(p + "self_attn.o_proj", cfg.hidden, cfg.n_q)
+            matrix(p + "mlp.gate_proj", cfg.inter, cfg.hidden)
+            matrix(p + "mlp.up_proj", cfg.inter, cfg.hidden)
+            matrix(p + "mlp.down_proj", cfg.hidden, cfg.inter)
+            vector(p + "input_layernorm", cfg.hidden, 1.0, 0.1)
+            vector(p + "post_attention_layernorm", cfg.hidden, 1.0, 0.1)
+            if cfg.qk_norm:
+                vector(p + "self_attn.q_norm", cfg.head_dim, 1.0, 0.1)
+                vector(p + "self_attn.k_norm", cfg.head_dim, 1.0, 0.1)
+            if cfg.qkv_bias:
+                vector(p + "self_attn.q_proj.bias", cfg.n_q, 0.0, 0.5)
+                vector(p + "self_attn.k_proj.bias", cfg.n_kvd, 0.0, 0.5)
+                vector(p + "self_attn.v_proj.bias", cfg.n_kvd, 0.0, 0.5)
+        native.sync()
+        return self
+
+    def nbytes(self) -> int:
+        return sum(m.nbytes for m in self.mats.values()) + sum(v.nbytes for v in self.vecs.values())
+
+
+class DecoderRuntime:
+    """Scratch arena, KV caches, uniforms and the captured decode graph of one model."""
+
+    def __init__(self, cfg: DecoderConfig, weights: DecoderWeights, dispatcher: Optional[Dispatcher] = None,
+                 hist_capacity: int = 4096):
+        self.cfg, self.w = cfg, weights
+        self.d = dispatcher or Dispatcher()
+        z = native.zeros
+        self.token, self.step_counter = z(4), z(4)
+        self.offset, self.kv_len, self.hist_counter = z(4), z(4), z(4)
+        self.history = z(4 * hist_capacity)
+        self.x = [DeviceBuffer(cfg.hidden * 2), DeviceBuffer(cfg.hidden * 2)]
+        self.q, self.k, self.v = DeviceBuffer(cfg.n_q * 2), DeviceBuffer(cfg.n_kvd * 2), DeviceBuffer(cfg.n_kvd * 2)
+        self.att, self.mid = DeviceBuffer(cfg.n_q * 2), DeviceBuffer(cfg.inter * 2)
+        self.logits = DeviceBuffer(cfg.vocab * 2)
+        cache_bytes = cfg.n_kv * cfg.capacity * cfg.head_dim * 2
+        self.cache_k = [z(cache_bytes) for _ in range(cfg.n_layers)]
+        self.cache_v = [z(cache_bytes) for _ in range(cfg.n_layers)]
+        pb, cb = native.sdpa_workspace_bytes(cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.capacity)
+        self.sdpa_partials, self.sdpa_counters = DeviceBuffer(max(pb, 4)), z(max(cb, 4))
+        self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
+        self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
+        self.tasks = self.build_tasks()
+        self.graph = self.d.build_graph(self.tasks)
+
+    # -- task list -------------------------------------------------------------------
+    def _wargs(self, W: DeviceWeight):
+        return [arg(W.w)] if W.bits == 16 else [arg(W.w), arg(W.scales), arg(W.biases)]
+
+    def build_tasks(self) -> List[Dispatch]:
+        c, w = self.cfg, self.w
+        q = dict(bits=c.bits, group=c.group)
+        t: List[Dispatch] = []
+        fid = [0]
+
+        def name(kind: str) -> str:
+            fid[0] += 1
+            return f"fusekit_{kind}_f{fid[0]}"
+
+        t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
+        emb = w.mats["embed_tokens"]
+        t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token), arg(emb.w), arg(self.x[0])],
+                          dict(bits=16, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            Wq, Wk, Wv = (w.mats[p + f"self_attn.{n}_proj"] for n in "qkv")
+            qkv_args = [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(Wq.w), arg(Wk.w), arg(Wv.w)]
+            if c.bits != 16:
+                qkv_args += [arg(m.scales) for m in (Wq, Wk, Wv)] + [arg(m.biases) for m in (Wq, Wk, Wv)]
+            if c.qkv_bias:
+                qkv_args += [arg(w.vecs[p + f"self_attn.{n}_proj.bias"]) for n in "qkv"]
+            qkv_args += [arg(self.q), arg(self.k), arg(self.v)]
+            t.append(Dispatch(name("rmsnorm_qkv"), qkv_args,
+                              dict(q, hidden=c.hidden, n_q=c.n_q, n_kv=c.n_kvd, eps=c.eps, has_norm=1,
+                                   has_bias=int(c.qkv_bias))))
+            rope = dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, rope_dims=c.head_dim, theta=c.theta,
+                        capacity=c.capacity, eps=c.eps)
+            if c.fuse_rope_store:
+                a = [arg(self.q), arg(self.k), arg(self.v)]
+                if c.qk_norm:
+                    a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
+                a += [arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.offset)]
+                t.append(Dispatch(name("qkv_rope_store_decode"), a, dict(rope, has_norm=int(c.qk_norm))))
+            elif c.qk_norm:
+                t.append(Dispatch(name("rmsnorm_rope_q_decode"),
+                                  [arg(self.q), arg(w.vecs[p + "self_attn.q_norm"]), arg(self.offset)], rope))
+                t.append(Dispatch(name("rmsnorm_rope_kv_cache_store_decode"),
+                                  [arg(self.k), arg(self.v), arg(w.vecs[p + "self_attn.k_norm"]),
+                                   arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.offset), arg(self.offset)],
+                                  rope))
+            else:
+                t.append(Dispatch(name("rope_q_decode"), [arg(self.q), arg(self.offset)], rope))
+                t.append(Dispatch(name("rope_kv_cache_store_decode"),
+                                  [arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]),
+                                   arg(self.offset), arg(self.offset)], rope))
+            t.append(Dispatch(name("sdpa_decode"),
+                              [arg(self.q), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+                               arg(self.att), arg(self.sdpa_partials), arg(self.sdpa_counters)],
+                              dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, capacity=c.capacity,
+                                   max_len=c.capacity)))
+            Wo = w.mats[p + "self_attn.o_proj"]
+            t.append(Dispatch(name("linear_residual"),
+                              [arg(self.att)] + self._wargs(Wo) + [arg(self.x[0]), arg(self.x[1])],
+                              dict(q, m=c.n_q, n=c.hidden)))
+            Wg, Wu = w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"]
+            ga = [arg(self.x[1]), arg(w.vecs[p + "post_attention_layernorm"]), arg(Wg.w), arg(Wu.w)]
+            if c.bits != 16:
+                ga += [arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases)]
+            ga += [arg(self.mid)]
+            t.append(Dispatch(name("rmsnorm_gateup_swiglu"), ga,
+                              dict(q, hidden=c.hidden, inter=c.inter, eps=c.eps, variant=c.swiglu_variant,
+                                   has_norm=1)))
+            Wd = w.mats[p + "mlp.down_proj"]
+            t.append(Dispatch(name("linear_residual"),
+                              [arg(self.mid)] + self._wargs(Wd) + [arg(self.x[1]), arg(self.x[0])],
+                              dict(q, m=c.inter, n=c.hidden)))
+        t.append(Dispatch(name("final_rmsnorm_lm_head"),
+                          [arg(self.x[0]), arg(w.vecs["final_norm"]), arg(emb.w), arg(self.logits)],
+                          dict(bits=16, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
+        t.append(Dispatch(name("argmax_logits_decode"),
+                          [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history),
+                           arg(self.hist_counter)], dict(vocab=c.vocab)))
+        return t
+
+    # -- generation ------------------------------------------------------------------
+    def reset(self) -> None:
+        for b in (self.step_counter, self.offset, self.kv_len, self.hist_counter):
+            b.upload(np.zeros(1, np.uint32))
+
+    def prefill(self, prompt: Sequence[int], start_offset: int = 0) -> int:
+        """Feeds the prompt through the decode graph with forced tokens; returns the greedy
+        first token (the argmax after the last prompt token)."""
+        nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
+        return nxt[-1]
+
+    def generate(self, prompt: Sequence[int], max_tokens: int):
+        """Greedy decode.  Returns (tokens, gpu_seconds of the decode chunks, decode steps timed)."""
+        if len(prompt) + max_tokens > self.cfg.capacity:
+            raise ValueError("prompt + max_tokens exceeds the KV-cache capacity")  # __init__.py:5017-5037
+        first = self.prefill(prompt)
+        out = [first]
+        offset = len(prompt)
+        gpu_s, steps = 0.0, 0
+        while len(out) < max_tokens:
+            n = min(FK_CHUNK, max_tokens - len(out), self.uniforms.hist_capacity)
+            toks, sec = self.d.decode_chunk(self.graph, self.uniforms, offset, out[-1], n)
+            out += toks
+            offset += n
+            gpu_s += sec
+            steps += n
+        return out, gpu_s, steps

@@ -123,6 +123,20 @@ fk_status fk_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps,
 fk_status fk_final_rmsnorm_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *W,
                                    uint16_t *logits, fk_stream s);
 
+/* Q0  MLX-affine quantiser on the device: w fp32 [n, k] -> packed uint32
+ *     [n, k*bits/32], scales / biases bf16 [n, k/group].  Arithmetic of the
+ *     reference's restatement of mx.quantize,
+ *     src/codegen/kernels/rope_kv_cache_store_decode_quant.rs:208-221; integer
+ *     codes are bit-exact against the CPU statement of the same formula. */
+fk_status fk_quantize_affine(const float *d_w, size_t n, size_t k, uint32_t bits, uint32_t group,
+                             uint32_t *d_packed, uint16_t *d_scales, uint16_t *d_biases, fk_stream s);
+
+/* Seeded synthetic data written straight into HBM (random-init models for
+ * `fusekit bench` without a checkpoint): element i depends only on (seed, i).
+ * kind 0: fp32 N(mean, std^2); 1: bf16 N(mean, std^2); 2: uint32 uniform in [0, bound). */
+fk_status fk_synth_fill(void *dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind,
+                        uint32_t bound, fk_stream s);
+
 /* Per-token scalars (rotary position, cache row, KV length) come either from a
  * device scalar `d_*` (so a captured hipGraph can be replayed while a step
  * kernel advances them, as the reference binds `layer_offset` / `layer_kv_len`
@@ -188,6 +202,107 @@ fk_status fk_argmax_logits_decode(const uint16_t *logits, uint32_t n, uint32_t *
 /* U   offset = step_counter++ ; kv_len = offset + 1.  Replaces fusekit_step_init
  *     (src/codegen/kernels/mod.rs:542-563). */
 fk_status fk_step_init(uint32_t *step_counter, uint32_t *offset, uint32_t *kv_len, fk_stream s);
+
+/* ---- dispatcher: replaces `_fusekit_runtime_native` ------------------------
+ *
+ * A dispatch names a kernel family by prefix ("fusekit_rmsnorm_qkv_f12" ->
+ * family "fusekit_rmsnorm_qkv"; names follow kernel_function_name,
+ * src/codegen/kernels/mod.rs:5578-5583), lists its buffers as (pointer, bytes)
+ * in slot order and carries key/value parameters (dims, eps, theta, bits ...)
+ * in place of the constants the reference bakes into kernel text.  Slot order
+ * per family ([..] optional; quantised weights add their scales then biases):
+ *   fusekit_step_init                 step_counter, offset, kv_len
+ *   fusekit_embed_lookup_decode       token, table [, scales, biases], x
+ *       {bits=16, hidden, vocab, group=64, output_scale=1}
+ *   fusekit_rmsnorm_qkv | fusekit_qmv_fanout(has_norm=0)
+ *       x, [norm_w], W_q, W_k, W_v, [s_q, s_k, s_v, b_q, b_k, b_v], [bias_q, bias_k, bias_v], q, k, v
+ *       {bits=4, group=64, hidden, n_q, n_kv, eps, has_norm=1, has_bias=0}
+ *   fusekit_rope_q_decode             Q, offset            {n_heads, head_dim, rope_dims, theta}
+ *   fusekit_rmsnorm_rope_q_decode     Q, q_weight, offset  {+ eps}
+ *   fusekit_rope_kv_cache_store_decode | fusekit_kv_cache_store_decode (no rotation)
+ *       K, V, cache_k, cache_v, offset, write_offset   {n_kv, head_dim, v_dim, rope_dims, theta, capacity}
+ *   fusekit_rmsnorm_rope_kv_cache_store_decode
+ *       K, V, k_weight, cache_k, cache_v, offset, write_offset   {+ eps}
+ *   fusekit_qkv_rope_store_decode     Q, K, V, [q_weight, k_weight], cache_k, cache_v, offset
+ *       {n_heads, n_kv, head_dim, rope_dims, theta, capacity, eps, has_norm=0}
+ *   fusekit_sdpa_decode               Q, K, V, kv_len, out, partials, counters
+ *       {n_heads, n_kv, head_dim | qk_dim, v_dim, capacity, max_len=capacity, scale=1/sqrt(qk_dim)}
+ *   fusekit_linear_residual           x, W [, scales, biases], residual, [residual_extra], y
+ *       {bits=4, group=64, m (= K), n, has_extra=0}
+ *   fusekit_rmsnorm_gateup_swiglu | fusekit_qmv_swiglu(has_norm=0)
+ *       x, [norm_w], W_gate, W_up, [s_g, s_u, b_g, b_u], out   {bits, group, hidden, inter, eps, variant=0, has_norm=1}
+ *   fusekit_final_rmsnorm_lm_head     x, norm_w, W [, scales, biases], logits   {bits=16, group, hidden, vocab, eps}
+ *   fusekit_qgemv                     x, W [, scales, biases], [bias], y        {bits, group, m, n, has_bias=0}
+ *   fusekit_argmax_logits_decode      logits, next_tok, workspace [, history, hist_counter]   {vocab}
+ * Read/write slots per family follow the reference's table
+ * (python/fusekit_runtime/dispatch.py:100-190); graph edges are derived from
+ * them on overlapping byte ranges (RAW, WAW, WAR). */
+typedef uint64_t fk_handle;
+typedef struct fk_arg { void *ptr; size_t nbytes; } fk_arg;
+typedef struct fk_param { const char *key; double value; } fk_param;
+typedef struct fk_dispatch {
+    const char *kernel;
+    const fk_arg *args;
+    uint32_t n_args;
+    const fk_param *params;
+    uint32_t n_params;
+} fk_dispatch;
+typedef struct fk_binding_update { uint32_t cmd_idx, slot; void *ptr; size_t nbytes; } fk_binding_update;
+
+/* Device scalars of the per-token protocol (python_runtime/src/lib.rs:1299-1303,
+ * src/codegen/kernels/mod.rs:544-577): `token` is read by the embedding lookup
+ * and written by the argmax (token_id_in aliases next_token_out). */
+typedef struct fk_decode_uniforms {
+    uint32_t *token;
+    uint32_t *step_counter;
+    uint32_t *hist_counter;
+    uint32_t *history;
+    uint32_t hist_capacity;
+} fk_decode_uniforms;
+
+/* load_dispatcher (lib.rs:116-169).  The kernels are compiled into the library:
+ * `code_object_path` may be NULL or "builtin"; a path is only checked to exist.
+ * `task_graph_path` (may be NULL) is parsed: version must be 2
+ * (src/runtime/plan.rs:175-180) and every task's kernel must name a family of
+ * this library (lib.rs:412-415), else FK_ERR_INVALID. */
+fk_status fk_load_dispatcher(const char *code_object_path, const char *task_graph_path, fk_handle *out);
+/* kernel_names (lib.rs:223) */
+fk_status fk_kernel_names(fk_handle h, const char *const **names, size_t *n);
+fk_status fk_dispatcher_stream(fk_handle h, fk_stream *out);
+/* dispatch_kernel (lib.rs:398) / dispatch_batch (lib.rs:1723): launch and wait, GPU seconds out */
+fk_status fk_dispatch_kernel(fk_handle h, const fk_dispatch *d, double *gpu_seconds);
+fk_status fk_dispatch_batch(fk_handle h, const fk_dispatch *list, size_t n, double *gpu_seconds);
+/* build_icb (lib.rs:461): pre-encode the list as one hipGraph.  `barriers`
+ * NULL = edges from the read/write tables; barriers[i] != 0 additionally makes
+ * command i wait for every earlier command. */
+fk_status fk_build_graph(fk_handle h, const fk_dispatch *list, size_t n, const uint8_t *barriers,
+                         uint32_t *graph_id);
+fk_status fk_graph_info(fk_handle h, uint32_t graph_id, uint32_t *n_nodes, uint32_t *n_edges);
+fk_status fk_graph_node_deps(fk_handle h, uint32_t graph_id, uint32_t node, uint32_t *deps, uint32_t cap,
+                             uint32_t *n);
+/* update_icb_bindings (lib.rs:575): patch buffers (KV-cache growth) without a rebuild */
+fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_binding_update *ups, size_t n);
+/* execute_icb (lib.rs:719), execute_icb_range (lib.rs:770), profile_icb_commands (lib.rs:823) */
+fk_status fk_execute_graph(fk_handle h, uint32_t graph_id, double *gpu_seconds);
+fk_status fk_execute_graph_repeat(fk_handle h, uint32_t graph_id, uint32_t count, double *gpu_seconds);
+fk_status fk_execute_graph_range(fk_handle h, uint32_t graph_id, uint32_t start, uint32_t end,
+                                 double *gpu_seconds);
+fk_status fk_profile_graph_nodes(fk_handle h, uint32_t graph_id, double *per_node_seconds, size_t n);
+/* submit_icb_async (lib.rs:660) + wait_pending_icb (lib.rs:702): one launch in flight */
+fk_status fk_submit_graph_async(fk_handle h, uint32_t graph_id);
+fk_status fk_wait_pending(fk_handle h, double *gpu_seconds);
+/* decode_chunk_gpu_chain (lib.rs:1277-1420): seed step_counter = start_offset,
+ * hist_counter = 0, token = seed_token; replay the graph `count` times back to
+ * back; wait for the last; copy history[0..count) out. */
+fk_status fk_decode_chunk(fk_handle h, uint32_t graph_id, const fk_decode_uniforms *u, uint32_t start_offset,
+                          uint32_t seed_token, uint32_t count, uint32_t *out_tokens, double *gpu_seconds);
+/* decode_chunk_host_loop (lib.rs:1131-1257): per step the host writes
+ * token = tokens_in[i] and step_counter = start_offset + i, replays the graph,
+ * waits and reads the next token back into out_next[i].  Used to feed a prompt
+ * (forced tokens) through the decode graph. */
+fk_status fk_decode_chunk_host_loop(fk_handle h, uint32_t graph_id, const fk_decode_uniforms *u,
+                                    uint32_t start_offset, const uint32_t *tokens_in, uint32_t count,
+                                    uint32_t *out_next, double *gpu_seconds);
 
 /* Launch-geometry overrides for experiments (0 = library policy): rows per
  * tile and grid blocks of the streaming GEMV.  Process-wide. */

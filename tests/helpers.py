@@ -43,3 +43,75 @@ def bf16_mismatch(a: np.ndarray, b: np.ndarray):
 
 def to_device(fk, W: oracle.QWeight):
     return fk.DeviceWeight(W.w, W.scales, W.biases, W.n, W.k, W.bits, W.group)
+
+
+# ---------------------------------------------------------------- whole-model oracle
+def host_weight(dw) -> oracle.QWeight:
+    """Download a fusekit_amd DeviceWeight into an oracle QWeight."""
+    if dw.bits == 16:
+        return oracle.dense(dw.w.to_numpy(np.uint16, (dw.n, dw.k)))
+    per = 32 // dw.bits
+    return oracle.QWeight(dw.w.to_numpy(np.uint32, (dw.n, dw.k // per)),
+                          dw.scales.to_numpy(np.uint16, (dw.n, dw.k // dw.group)),
+                          dw.biases.to_numpy(np.uint16, (dw.n, dw.k // dw.group)), dw.n, dw.k, dw.bits, dw.group)
+
+
+class OracleDecoder:
+    """CPU oracle of a dense decoder fed with the very bytes the GPU model holds."""
+
+    def __init__(self, cfg, weights):
+        import ctypes as C
+        self.cfg = cfg
+        self.keep = []
+        u16p = C.POINTER(C.c_uint16)
+
+        def vec(name):
+            a = weights.vecs[name].to_numpy(np.uint16)
+            self.keep.append(a)
+            return a.ctypes.data_as(u16p)
+
+        def mat(name):
+            W = host_weight(weights.mats[name])
+            self.keep.append(W)
+            return W.c
+
+        null = C.cast(None, u16p)
+        self.layers = (oracle.Layer * cfg.n_layers)()
+        cache_elems = cfg.n_kv * cfg.capacity * cfg.head_dim
+        for l in range(cfg.n_layers):
+            p = f"layers.{l}."
+            L = self.layers[l]
+            L.input_norm, L.post_norm = vec(p + "input_layernorm"), vec(p + "post_attention_layernorm")
+            L.wq, L.wk, L.wv = (mat(p + f"self_attn.{n}_proj") for n in "qkv")
+            L.wo = mat(p + "self_attn.o_proj")
+            L.wgate, L.wup, L.wdown = (mat(p + f"mlp.{n}_proj") for n in ("gate", "up", "down"))
+            L.bq, L.bk, L.bv = ((vec(p + f"self_attn.{n}_proj.bias") for n in "qkv") if cfg.qkv_bias
+                                else (null, null, null))
+            L.q_norm, L.k_norm = ((vec(p + "self_attn.q_norm"), vec(p + "self_attn.k_norm")) if cfg.qk_norm
+                                  else (null, null))
+            ck, cv = np.zeros(cache_elems, np.uint16), np.zeros(cache_elems, np.uint16)
+            self.keep += [ck, cv]
+            L.cache_k, L.cache_v = ck.ctypes.data_as(u16p), cv.ctypes.data_as(u16p)
+        emb = mat("embed_tokens")
+        self.model = oracle.Model(cfg.n_layers, cfg.hidden, cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab,
+                                  cfg.eps, cfg.theta, 1.0 / np.sqrt(cfg.head_dim), 1.0, cfg.swiglu_variant,
+                                  cfg.capacity, emb, emb, vec("final_norm"), self.layers)
+
+    def step(self, token: int, offset: int, want_logits: bool = False):
+        logits = np.empty(self.cfg.vocab, np.uint16) if want_logits else None
+        nxt, margin = oracle.decoder_step(self.model, token, offset, logits)
+        return nxt, margin, logits
+
+    def generate(self, prompt, max_tokens):
+        """Returns (tokens, margins): greedy tokens and the top-1/top-2 logit margin at each step."""
+        toks, margins = [], []
+        nxt = None
+        for i, t in enumerate(prompt):
+            nxt, m, _ = self.step(int(t), i)
+        toks.append(nxt); margins.append(m)
+        off = len(prompt)
+        while len(toks) < max_tokens:
+            nxt, m, _ = self.step(toks[-1], off)
+            toks.append(nxt); margins.append(m)
+            off += 1
+        return toks, margins
