@@ -286,10 +286,11 @@ fk_status fk_qkv_rope_store_decode(uint16_t* q, const uint16_t* k, const uint16_
     return run_launch(l, (hipStream_t)s);
 }
 
-fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t v_dim, uint32_t max_len,
+fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                   size_t* partial_bytes, size_t* counter_bytes) {
-    if (!partial_bytes || !counter_bytes || max_len == 0) return set_error(FK_ERR_INVALID, "sdpa workspace: bad argument");
-    return sdpa_workspace_bytes(n_heads, n_kv, v_dim, max_len, partial_bytes, counter_bytes);
+    if (!partial_bytes || !counter_bytes || max_len == 0 || qk_dim < 8 || v_dim < 8)
+        return set_error(FK_ERR_INVALID, "sdpa workspace: bad argument");
+    return sdpa_workspace_bytes(n_heads, n_kv, qk_dim, v_dim, max_len, partial_bytes, counter_bytes);
 }
 
 fk_status fk_sdpa_decode(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,

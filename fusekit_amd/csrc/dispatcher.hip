@@ -400,7 +400,7 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_bytes(d, 3, 4));
     FK_TRY(need_bytes(d, 4, (size_t)n_heads * vd * 2));
     size_t pb = 0, cb = 0;
-    FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, vd, max_len, &pb, &cb));
+    FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, qk, vd, max_len, &pb, &cb));
     FK_TRY(need_bytes(d, 5, pb));
     FK_TRY(need_bytes(d, 6, cb));
     rw->reads = {0, 1, 2, 3, 5, 6};

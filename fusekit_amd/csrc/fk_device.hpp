@@ -35,16 +35,27 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
                                            false);
 }
 
-// Butterfly reductions over `width` adjacent lanes (width a power of two <= 64).
+// v + (v of the lane selected by a DPP control): cross-lane adds inside a row of
+// 16 lanes without going through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true);
+    return v + __int_as_float(moved);
+}
+
+// Sum over `width` adjacent lanes (a power of two <= 64, groups aligned to width);
+// every lane of the group ends with the total.  Widths up to 16 use DPP only:
+// quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror.
 __device__ __forceinline__ float group_sum(float v, int width) {
-    for (int o = width >> 1; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    if (width >= 2) v = dpp_add<0xB1>(v);
+    if (width >= 4) v = dpp_add<0x4E>(v);
+    if (width >= 8) v = dpp_add<0x141>(v);
+    if (width >= 16) v = dpp_add<0x140>(v);
+    if (width >= 32) v += __shfl_xor(v, 16, kWave);
+    if (width >= 64) v += __shfl_xor(v, 32, kWave);
     return v;
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-    return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return group_sum(v, 64); }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));

@@ -1,4 +1,7 @@
 // Launch planner and template instances of the flat-stream GEMV.
+#include <map>
+#include <mutex>
+
 #include "fk_host.hpp"
 #include "gemv_kernel.hpp"
 
@@ -63,32 +66,76 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     const uint32_t values = bits == 4 ? 32u : (bits == 8 ? 16u : 8u);
     const uint32_t cpr = K / values;
     const uint32_t nseg = rq.swiglu ? 2u : 1u;
-    constexpr uint32_t kBatch = kGemvBlock * kGemvUnroll;
 
-    // Rows per tile: keep a tile near one batch of 16-byte loads per lane, then
-    // pick the R whose tile count spreads most evenly over the compute units
-    // (cost = tiles-per-CU x (tile chunks + a fixed per-tile overhead)).
-    uint32_t r_max = kBatch / (nseg * cpr);
-    if (r_max < 1) r_max = 1;
-    if (r_max > kGemvBlock) r_max = kGemvBlock;
-    uint32_t best_r = 1;
-    uint64_t best_cost = ~0ull;
+    const void* func = select_gemv(kind, rq.swiglu, rq.norm_w != nullptr);
     auto tiles_for = [&](uint32_t r) {
         uint64_t t = 0;
         if (rq.swiglu) return (uint64_t)((rq.mats[0]->n + r - 1) / r);
         for (int m = 0; m < nm; ++m) t += (rq.mats[m]->n + r - 1) / r;
         return t;
     };
+    auto lds_for = [&](uint32_t r) {
+        switch (kind) {
+            case W_Q4: return gemv_lds_bytes<W_Q4>(cpr, r * cpr, nseg);
+            case W_Q8: return gemv_lds_bytes<W_Q8>(cpr, r * cpr, nseg);
+            default: return gemv_lds_bytes<W_BF16>(cpr, r * cpr, nseg);
+        }
+    };
+    // Blocks that can be resident at once (registers and LDS decide): the grid never
+    // exceeds it, so no block waits for a slot and then pays the whole start-up chain
+    // (stage x, first loads) a second time; surplus tiles go to the persistent loop,
+    // whose next batch is already in flight while the current one is consumed.
+    auto resident_for = [&](uint32_t lds_bytes) -> uint32_t {
+        static std::mutex mu;
+        static std::map<std::pair<const void*, uint32_t>, int> cache;
+        std::lock_guard<std::mutex> lk(mu);
+        auto key = std::make_pair(func, lds_bytes);
+        auto it = cache.find(key);
+        if (it == cache.end()) {
+            if (lds_bytes > 48 * 1024)
+                (void)hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            int per_cu = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, func, kGemvBlock, lds_bytes) != hipSuccess ||
+                per_cu < 1)
+                per_cu = 1;
+            it = cache.emplace(key, per_cu).first;
+        }
+        return (uint32_t)it->second * (uint32_t)dev->cus;
+    };
+
+    // Rows per tile.  Candidates keep a tile within one batch of 16-byte loads per
+    // lane where K allows.  Cost = batches the busiest block runs; ties go to the
+    // choice that wastes the fewest lane slots.
+    const uint32_t pos = kGemvBlock * (kGemvUnroll / nseg);
+    uint32_t r_max = pos / cpr;
+    if (r_max < 1) r_max = 1;
+    if (r_max > kGemvBlock) r_max = kGemvBlock;
+    uint32_t best_r = 1, best_blocks = 1;
+    uint64_t best_cost = ~0ull, best_waste = ~0ull;
     for (uint32_t r = 1; r <= r_max; ++r) {
+        const uint32_t lds_r = lds_for(r);
+        if ((int)lds_r > dev->max_dyn_lds) continue;
         const uint64_t tiles = tiles_for(r);
-        const uint64_t per_cu = (tiles + dev->cus - 1) / dev->cus;
-        const uint64_t cost = per_cu * ((uint64_t)r * cpr * nseg + kGemvBlock);
-        if (cost <= best_cost) {
+        uint64_t cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : resident_for(lds_r);
+        const uint64_t blocks = tiles < cap ? tiles : cap;
+        const uint64_t per_block = (tiles + blocks - 1) / blocks;
+        const uint64_t batches = ((uint64_t)r * cpr + pos - 1) / pos;
+        const uint64_t cost = per_block * batches;
+        const uint64_t waste = tiles * batches * pos - (uint64_t)r * cpr * tiles;
+        if (cost < best_cost || (cost == best_cost && waste < best_waste)) {
             best_cost = cost;
+            best_waste = waste;
             best_r = r;
+            best_blocks = (uint32_t)blocks;
         }
     }
-    if (g_gemv_policy.rows_per_tile) best_r = g_gemv_policy.rows_per_tile;
+    if (best_cost == ~0ull) return set_error(FK_ERR_UNSUPPORTED, "gemv: K too large for LDS staging");
+    if (g_gemv_policy.rows_per_tile) {
+        best_r = g_gemv_policy.rows_per_tile;
+        const uint64_t tiles = tiles_for(best_r);
+        const uint64_t cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : resident_for(lds_for(best_r));
+        best_blocks = (uint32_t)(tiles < cap ? tiles : cap);
+    }
     const uint32_t R = best_r;
     const uint64_t tiles = tiles_for(R);
     if (tiles > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "gemv: too many tiles");
@@ -125,17 +172,10 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     a.res2 = rq.res2;
     a.swiglu_variant = rq.swiglu_variant;
 
-    uint32_t lds = 0;
-    switch (kind) {
-        case W_Q4: lds = gemv_lds_bytes<W_Q4>(cpr, R * cpr, nseg); break;
-        case W_Q8: lds = gemv_lds_bytes<W_Q8>(cpr, R * cpr, nseg); break;
-        default: lds = gemv_lds_bytes<W_BF16>(cpr, R * cpr, nseg); break;
-    }
+    const uint32_t lds = lds_for(R);
     if ((int)lds > dev->max_dyn_lds) return set_error(FK_ERR_UNSUPPORTED, "gemv: K too large for LDS staging");
-
-    uint32_t grid_cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : (uint32_t)dev->cus * 8u;
-    out->func = select_gemv(kind, rq.swiglu, rq.norm_w != nullptr);
-    out->grid = dim3((uint32_t)(tiles < grid_cap ? tiles : grid_cap), 1, 1);
+    out->func = func;
+    out->grid = dim3(best_blocks, 1, 1);
     out->block = dim3(kGemvBlock, 1, 1);
     out->shmem = lds;
     out->set_args(a);

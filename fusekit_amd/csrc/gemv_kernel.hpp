@@ -153,16 +153,32 @@ __device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int va
 
 // Stage x (optionally RMS-normalised: T(w * T(x * r))) into the chunk-interleaved
 // LDS layout and compute the per-chunk sums.  Every thread handles 8 consecutive
-// elements per step.  K must be a multiple of 64.
+// elements per step; the first kStageRegs steps stay in registers between the
+// sum-of-squares pass and the write pass, so x and the norm weight are fetched
+// once.  The threads that hold the pieces of one chunk are adjacent lanes, so the
+// chunk sum is a 2- or 4-lane butterfly.  K must be a multiple of 64.
+constexpr int kStageRegs = 4;
+
 template <WKind KIND, bool NORM>
 __device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, float* sx, float* scratch) {
     const uint32_t K = a.K, cpr = a.cpr, n8 = K >> 3;
     const uint4* x8 = reinterpret_cast<const uint4*>(a.x);
+    const uint4* w8 = reinterpret_cast<const uint4*>(a.norm_w);
+    uint4 xr[kStageRegs], wr[kStageRegs];
+#pragma unroll
+    for (int i = 0; i < kStageRegs; ++i) {
+        const uint32_t t = threadIdx.x + i * kGemvBlock;
+        xr[i] = make_uint4(0, 0, 0, 0);
+        wr[i] = make_uint4(0, 0, 0, 0);
+        if (t < n8) {
+            xr[i] = x8[t];
+            if constexpr (NORM) wr[i] = w8[t];
+        }
+    }
     float r = 1.0f;
     if constexpr (NORM) {
         float ss = 0.f;
-        for (uint32_t t = threadIdx.x; t < n8; t += kGemvBlock) {
-            const uint4 v = x8[t];
+        auto add_sq = [&](uint4 v) {
             const uint32_t p[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -170,13 +186,14 @@ __device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, 
                 ss = fmaf(lo, lo, ss);
                 ss = fmaf(hi, hi, ss);
             }
-        }
+        };
+#pragma unroll
+        for (int i = 0; i < kStageRegs; ++i) add_sq(xr[i]);  // zeros beyond n8 add nothing
+        for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8; t += kGemvBlock) add_sq(x8[t]);
         ss = block_sum<kGemvBlock>(ss, scratch);
         r = 1.0f / sqrtf(ss / (float)K + a.eps);
     }
-    const uint4* w8 = reinterpret_cast<const uint4*>(a.norm_w);
-    for (uint32_t t = threadIdx.x; t < n8; t += kGemvBlock) {
-        const uint4 v = x8[t];
+    auto emit = [&](uint32_t t, uint4 v, uint4 wv) {
         const uint32_t p[4] = {v.x, v.y, v.z, v.w};
         float f[8];
 #pragma unroll
@@ -185,7 +202,6 @@ __device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, 
             f[2 * i + 1] = bf16_hi(p[i]);
         }
         if constexpr (NORM) {
-            const uint4 wv = w8[t];
             const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -193,39 +209,45 @@ __device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, 
                 f[2 * i + 1] = round_bf16(bf16_hi(q[i]) * round_bf16(f[2 * i + 1] * r));
             }
         }
+        float s8 = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+        const bool live = t < n8;
         if constexpr (KIND == W_Q4) {
             // word j of chunk c; activation pairs (0,2) (4,6) (1,3) (5,7) as q4_word_dot wants
             const uint32_t c = t >> 2, j = t & 3u;
-            xs[j * cpr + c] = make_uint4(pack_bf16(f[0], f[2]), pack_bf16(f[4], f[6]), pack_bf16(f[1], f[3]),
-                                         pack_bf16(f[5], f[7]));
+            if (live)
+                xs[j * cpr + c] = make_uint4(pack_bf16(f[0], f[2]), pack_bf16(f[4], f[6]), pack_bf16(f[1], f[3]),
+                                             pack_bf16(f[5], f[7]));
+            s8 += __shfl_xor(s8, 1, kWave);
+            s8 += __shfl_xor(s8, 2, kWave);
+            if (live && j == 0) sx[c] = s8;
         } else if constexpr (KIND == W_Q8) {
             const uint32_t c = t >> 1, j = (t & 1u) * 2u;
-            xs[j * cpr + c] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
-                                         __float_as_uint(f[3]));
-            xs[(j + 1) * cpr + c] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]),
-                                               __float_as_uint(f[6]), __float_as_uint(f[7]));
-        } else {
-            xs[t] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]),
-                               pack_bf16(f[6], f[7]));
-        }
-    }
-    __syncthreads();
-    if constexpr (KIND != W_BF16) {
-        for (uint32_t c = threadIdx.x; c < cpr; c += kGemvBlock) {
-            float s = 0.f;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint4 v = xs[j * cpr + c];
-                if constexpr (KIND == W_Q4) {
-                    s += (bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y)) +
-                         (bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w));
-                } else {
-                    s += (__uint_as_float(v.x) + __uint_as_float(v.y)) +
-                         (__uint_as_float(v.z) + __uint_as_float(v.w));
-                }
+            if (live) {
+                xs[j * cpr + c] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                                             __float_as_uint(f[3]));
+                xs[(j + 1) * cpr + c] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]),
+                                                   __float_as_uint(f[6]), __float_as_uint(f[7]));
             }
-            sx[c] = s;
+            s8 += __shfl_xor(s8, 1, kWave);
+            if (live && j == 0) sx[c] = s8;
+        } else {
+            if (live)
+                xs[t] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]),
+                                   pack_bf16(f[6], f[7]));
         }
+    };
+#pragma unroll
+    for (int i = 0; i < kStageRegs; ++i) emit(threadIdx.x + i * kGemvBlock, xr[i], wr[i]);
+    // long rows: the rest is fetched again (whole waves stay in the loop so the
+    // butterflies above see all their lanes)
+    const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
+    for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8_up; t += kGemvBlock) {
+        uint4 v = make_uint4(0, 0, 0, 0), wv = make_uint4(0, 0, 0, 0);
+        if (t < n8) {
+            v = x8[t];
+            if constexpr (NORM) wv = w8[t];
+        }
+        emit(t, v, wv);
     }
     __syncthreads();
 }

@@ -23,6 +23,15 @@ namespace fk {
 
 constexpr int kSdpaBlock = 256;
 constexpr int kSdpaWaves = kSdpaBlock / kWave;
+constexpr int kSteps = 8;  // K rows (and at most as many V rows) each lane owns per range
+
+namespace {
+uint32_t pow2_ceil(uint32_t v) {
+    uint32_t p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+}  // namespace
 
 struct SdpaArgs {
     const uint16_t* q;
@@ -58,41 +67,52 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     float* red = s + GT * a.chunk_len;            // [waves][GT][v_dim]
     float* stat = red + kSdpaWaves * GT * a.v_dim;  // m[GT], l[GT], misc
 
+    // All K and V loads of the range are issued up front (the range is sized so that
+    // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
+    const uint32_t lpk = a.lpk, cpk = a.qk_dim >> 3;
+    const uint32_t lpv = a.lpv, cpv = a.v_dim >> 3;
+    const uint32_t ck = tid & (lpk - 1), kslot = tid / lpk, kslots = kSdpaBlock / lpk;
+    const uint32_t cv = tid & (lpv - 1), vslot = tid / lpv, vslots = kSdpaBlock / lpv;
+    const bool kcol_ok = ck < cpk, vcol_ok = cv < cpv;
+    uint4 kc[kSteps], vc[kSteps];
+    {
+        const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * ck;
+        const uint16_t* vbase = a.v + ((size_t)kvh * a.capacity + key0) * a.v_dim + 8 * cv;
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = kslot + u * kslots;
+            kc[u] = make_uint4(0, 0, 0, 0);
+            if (kcol_ok && j < nkeys) kc[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * a.qk_dim);
+        }
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = vslot + u * vslots;
+            vc[u] = make_uint4(0, 0, 0, 0);
+            if (vcol_ok && j < nkeys) vc[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)j * a.v_dim);
+        }
+    }
+
     // ---------------- phase A: scores ----------------
     {
-        const uint32_t lpk = a.lpk, cpk = a.qk_dim >> 3;
-        const uint32_t c = tid & (lpk - 1), slot = tid / lpk, slots = kSdpaBlock / lpk;
-        const bool col_ok = c < cpk;
         uint4 qf[GT];
 #pragma unroll
         for (int h = 0; h < GT; ++h) {
             qf[h] = make_uint4(0, 0, 0, 0);
-            if (col_ok && (uint32_t)h < gcount)
-                qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * c);
+            if (kcol_ok && (uint32_t)h < gcount)
+                qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
         }
-        const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * c;
-        constexpr int U = 4;
-        for (uint32_t j0 = slot; j0 < nkeys; j0 += slots * U) {
-            uint4 kc[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t j = j0 + u * slots;
-                kc[u] = make_uint4(0, 0, 0, 0);
-                if (col_ok && j < nkeys) kc[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * a.qk_dim);
-            }
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = kslot + u * kslots;
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t j = j0 + u * slots;
-#pragma unroll
-                for (int h = 0; h < GT; ++h) {
-                    float d = 0.f;
-                    d = dot2_bf16(kc[u].x, qf[h].x, d);
-                    d = dot2_bf16(kc[u].y, qf[h].y, d);
-                    d = dot2_bf16(kc[u].z, qf[h].z, d);
-                    d = dot2_bf16(kc[u].w, qf[h].w, d);
-                    d = group_sum(d, (int)lpk);
-                    if (c == 0 && j < nkeys) s[h * a.chunk_len + j] = d * a.scale;
-                }
+            for (int h = 0; h < GT; ++h) {
+                float d = 0.f;
+                d = dot2_bf16(kc[u].x, qf[h].x, d);
+                d = dot2_bf16(kc[u].y, qf[h].y, d);
+                d = dot2_bf16(kc[u].z, qf[h].z, d);
+                d = dot2_bf16(kc[u].w, qf[h].w, d);
+                d = group_sum(d, (int)lpk);
+                if (ck == 0 && j < nkeys) s[h * a.chunk_len + j] = d * a.scale;
             }
         }
     }
@@ -119,38 +139,24 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     __syncthreads();
 
     // ---------------- phase B: o = sum_j p_j v_j ----------------
-    const uint32_t lpv = a.lpv, cpv = a.v_dim >> 3;
     {
-        const uint32_t c = tid & (lpv - 1), slot = tid / lpv, slots = kSdpaBlock / lpv;
-        const bool col_ok = c < cpv;
         float acc[GT][8];
 #pragma unroll
         for (int h = 0; h < GT; ++h)
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
-        const uint16_t* vbase = a.v + ((size_t)kvh * a.capacity + key0) * a.v_dim + 8 * c;
-        constexpr int U = 4;
-        for (uint32_t j0 = slot; j0 < nkeys; j0 += slots * U) {
-            uint4 vc[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t j = j0 + u * slots;
-                vc[u] = make_uint4(0, 0, 0, 0);
-                if (col_ok && j < nkeys) vc[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)j * a.v_dim);
-            }
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = vslot + u * vslots;
+            const uint32_t jj = j < nkeys ? j : 0u;
+            const float live = j < nkeys ? 1.f : 0.f;
+            const float f[8] = {bf16_lo(vc[u].x), bf16_hi(vc[u].x), bf16_lo(vc[u].y), bf16_hi(vc[u].y),
+                                bf16_lo(vc[u].z), bf16_hi(vc[u].z), bf16_lo(vc[u].w), bf16_hi(vc[u].w)};
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t j = j0 + u * slots;
-                const uint32_t jj = j < nkeys ? j : 0u;
-                const float live = j < nkeys ? 1.f : 0.f;
-                const float f[8] = {bf16_lo(vc[u].x), bf16_hi(vc[u].x), bf16_lo(vc[u].y), bf16_hi(vc[u].y),
-                                    bf16_lo(vc[u].z), bf16_hi(vc[u].z), bf16_lo(vc[u].w), bf16_hi(vc[u].w)};
+            for (int h = 0; h < GT; ++h) {
+                const float p = s[h * a.chunk_len + jj] * live;
 #pragma unroll
-                for (int h = 0; h < GT; ++h) {
-                    const float p = s[h * a.chunk_len + jj] * live;
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
-                }
+                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
             }
         }
         // add the key slots that share this lane's column: first inside the wave ...
@@ -163,11 +169,11 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
                 acc[h][i] = v;
             }
         // ... then across waves through LDS
-        if (lane < lpv && col_ok) {
+        if (lane < lpv && vcol_ok) {
 #pragma unroll
             for (int h = 0; h < GT; ++h)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) red[(wave * GT + h) * a.v_dim + 8 * c + i] = acc[h][i];
+                for (int i = 0; i < 8; ++i) red[(wave * GT + h) * a.v_dim + 8 * cv + i] = acc[h][i];
         }
     }
     __syncthreads();
@@ -231,25 +237,18 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     }
 }
 
-namespace {
-uint32_t pow2_ceil(uint32_t v) {
-    uint32_t p = 1;
-    while (p < v) p <<= 1;
-    return p;
-}
-}  // namespace
-
-uint32_t sdpa_chunk_len(uint32_t max_len) {
-    // enough ranges to cover the chip at long contexts, no tiny ranges at short ones
-    uint32_t c = pow2_ceil((max_len + 127) / 128);
-    if (c < 32) c = 32;
-    if (c > 256) c = 256;
-    return c;
+// Positions per range: every lane owns exactly kSteps key rows, i.e.
+// kSteps * (block threads / lanes per key row).  128 positions for head_dim 128
+// (64 KiB of K+V per block); a 32k context then spreads over 256 ranges x kv heads.
+uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim) {
+    const uint32_t lpk = pow2_ceil(qk_dim / 8), lpv = pow2_ceil(v_dim / 8);
+    const uint32_t wide = lpk > lpv ? lpk : lpv;
+    return kSteps * (kSdpaBlock / wide);
 }
 
-fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t v_dim, uint32_t max_len,
+fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                size_t* partial_bytes, size_t* counter_bytes) {
-    const uint32_t chunk = sdpa_chunk_len(max_len);
+    const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim);
     const uint32_t n_splits = (max_len + chunk - 1) / chunk;
     *partial_bytes = (size_t)n_heads * n_splits * (v_dim + 2) * sizeof(float);
     *counter_bytes = (size_t)n_heads * sizeof(uint32_t);  // >= n_kv * head tiles
@@ -271,7 +270,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     if (max_len == 0 || max_len > capacity) return set_error(FK_ERR_INVALID, "sdpa: kv length outside (0, capacity]");
     if (!kv_len_ptr && (kv_len_imm == 0 || kv_len_imm > max_len))
         return set_error(FK_ERR_INVALID, "sdpa: kv_len outside (0, max_len]");
-    const uint32_t chunk = sdpa_chunk_len(max_len);
+    const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim);
     const uint32_t n_splits = (max_len + chunk - 1) / chunk;
     if (n_splits > 1 && (!partials || !counters))
         return set_error(FK_ERR_INVALID, "sdpa: workspace required when the context spans several ranges");

@@ -173,7 +173,7 @@ class DecoderRuntime:
         cache_bytes = cfg.n_kv * cfg.capacity * cfg.head_dim * 2
         self.cache_k = [z(cache_bytes) for _ in range(cfg.n_layers)]
         self.cache_v = [z(cache_bytes) for _ in range(cfg.n_layers)]
-        pb, cb = native.sdpa_workspace_bytes(cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.capacity)
+        pb, cb = native.sdpa_workspace_bytes(cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.head_dim, cfg.capacity)
         self.sdpa_partials, self.sdpa_counters = DeviceBuffer(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)

@@ -202,9 +202,9 @@ def qkv_rope_store_decode(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope
         C.c_uint32(offset), C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v), _ptr(stream)))
 
 
-def sdpa_workspace_bytes(n_heads, n_kv, v_dim, max_len):
+def sdpa_workspace_bytes(n_heads, n_kv, qk_dim, v_dim, max_len):
     pb, cb = C.c_size_t(), C.c_size_t()
-    check(lib.fk_sdpa_workspace_bytes(C.c_uint32(n_heads), C.c_uint32(n_kv), C.c_uint32(v_dim),
+    check(lib.fk_sdpa_workspace_bytes(C.c_uint32(n_heads), C.c_uint32(n_kv), C.c_uint32(qk_dim), C.c_uint32(v_dim),
                                       C.c_uint32(max_len), C.byref(pb), C.byref(cb)))
     return int(pb.value), int(cb.value)
 

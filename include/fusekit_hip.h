@@ -179,8 +179,8 @@ fk_status fk_qkv_rope_store_decode(uint16_t *q, const uint16_t *k, const uint16_
  *     sizes the split; use the cache capacity when replaying a graph).
  *     Workspace sizes from fk_sdpa_workspace_bytes; `counters` must be zero
  *     before the first launch (the kernel leaves them zero). */
-fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t v_dim, uint32_t max_len,
-                                  size_t *partial_bytes, size_t *counter_bytes);
+fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim,
+                                  uint32_t max_len, size_t *partial_bytes, size_t *counter_bytes);
 fk_status fk_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v, uint16_t *out,
                          const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
                          uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,

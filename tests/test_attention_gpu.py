@@ -90,7 +90,7 @@ def _sdpa_case(fk, n_heads, n_kv, qk, vd, kv_len, cap, seed=0, max_len=None):
     ck, cv = normal_bf16(seed + 1, n_kv * cap * qk), normal_bf16(seed + 2, n_kv * cap * vd)
     scale = 1.0 / np.sqrt(qk)
     max_len = max_len or kv_len
-    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, vd, max_len)
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, qk, vd, max_len)
     part, cnt = fk.DeviceBuffer(max(pb, 4)), fk.zeros(max(cb, 4))
     out = fk.DeviceBuffer(2 * n_heads * vd)
     dq, dck, dcv = (fk.DeviceBuffer.from_numpy(t) for t in (q, ck, cv))
@@ -98,8 +98,12 @@ def _sdpa_case(fk, n_heads, n_kv, qk, vd, kv_len, cap, seed=0, max_len=None):
     got = out.to_numpy(np.uint16)
     ref = oracle.sdpa_decode(q, ck, cv, n_heads, n_kv, qk, vd, kv_len, cap, scale)
     assert rel_l2(got, oracle.bf16_to_f32(ref)) <= REL_L2_BAR
-    frac, ulps = bf16_mismatch(got, ref)
-    assert ulps <= 2.0 and frac <= 0.05, (frac, ulps)
+    # element-wise: 2 bf16 ulps, or -- where an output is a near-total cancellation of
+    # sum p_j v_j -- the fp32 reordering bound taken relative to the typical output size
+    g, r = oracle.bf16_to_f32(got).astype(np.float64), oracle.bf16_to_f32(ref).astype(np.float64)
+    tol = 2 * 2.0 ** -8 * np.abs(r) + 1e-4 * np.sqrt(np.mean(r * r))
+    assert np.all(np.abs(g - r) <= tol), float(np.max(np.abs(g - r) - tol))
+    assert np.mean(got != ref) <= 0.05
     assert not cnt.to_numpy(np.uint32).any()  # counters are left zero for the next launch
     # a second launch on the same workspace gives the same bits (ordered merge, reset counters)
     fk.sdpa_decode(dq, dck, dcv, out, None, kv_len, max_len, n_heads, n_kv, qk, vd, cap, scale, part, cnt)
