@@ -615,8 +615,6 @@ extern "C" {
 
 fk_status fk_load_dispatcher(const char* code_object_path, const char* task_graph_path, fk_handle* out) {
     if (!out) return set_error(FK_ERR_INVALID, "null out");
-    const DeviceFacts* dev;
-    FK_TRY(device_facts(&dev));
     auto ds = std::make_unique<DispatcherState>();
     // The kernels are compiled into this library; a code-object path is accepted
     // for artifact compatibility and only checked for existence.
@@ -651,6 +649,10 @@ fk_status fk_load_dispatcher(const char* code_object_path, const char* task_grap
         for (const Family& f : kFamilies) ds->kernel_names.push_back(f.prefix);
     }
     for (const std::string& s : ds->kernel_names) ds->kernel_name_ptrs.push_back(s.c_str());
+    // the artifact is validated before the device is touched, so a bad artifact is
+    // reported as such even on a machine without a GPU
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
     FK_HIP(hipStreamCreateWithFlags(&ds->stream, hipStreamNonBlocking));
     FK_HIP(hipEventCreate(&ds->ev0));
     FK_HIP(hipEventCreate(&ds->ev1));

@@ -1,0 +1,78 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every symbol the
+header declares, compute calls fail loudly without a device (no CPU fallback), the product
+package never touches the oracle, and artifact validation reports bad task graphs."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "fusekit_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import fusekit_amd.native as fk
+    names = _declared()
+    assert len(names) >= 40
+    missing = [n for n in names if not hasattr(fk.lib, n)]
+    assert not missing, missing
+    assert "gfx950" in fk.version()
+
+
+def test_compute_fails_loudly_without_a_device():
+    import fusekit_amd.native as fk
+    if fk.has_device():
+        pytest.skip("a HIP device is present")
+    with pytest.raises(fk.FusekitError) as e:
+        fk.DeviceBuffer(16)
+    assert e.value.status == fk.FK_ERR_HIP and "no CPU path" in str(e.value)
+    w = fk.Weight(1, 1, 1, 8, 64, 4, 64)
+    assert fk.lib.fk_qgemv(C.byref(w), C.c_void_p(1), None, C.c_void_p(1), None) == fk.FK_ERR_HIP
+    h = C.c_uint64()
+    assert fk.lib.fk_load_dispatcher(None, None, C.byref(h)) == fk.FK_ERR_HIP
+
+
+def test_artifact_validation_precedes_device_use(tmp_path):
+    """A bad task graph is reported as such on any machine (version gate, unknown kernel)."""
+    import fusekit_amd.native as fk
+    h = C.c_uint64()
+    missing = str(tmp_path / "missing.json").encode()
+    assert fk.lib.fk_load_dispatcher(None, missing, C.byref(h)) == fk.FK_ERR_NOT_FOUND
+    p = tmp_path / "task_graph.json"
+    p.write_text('{"version": 1, "tasks": []}')
+    assert fk.lib.fk_load_dispatcher(None, str(p).encode(), C.byref(h)) == fk.FK_ERR_INVALID
+    assert b"version" in fk.lib.fk_last_error()
+    p.write_text('{"version": 2, "tasks": [{"id": 0, "kernel": "fusekit_not_a_kernel_f3"}]}')
+    assert fk.lib.fk_load_dispatcher(None, str(p).encode(), C.byref(h)) == fk.FK_ERR_INVALID
+    assert b"fusekit_not_a_kernel_f3" in fk.lib.fk_last_error()
+    p.write_text('{"version": 2, "tasks": [')
+    assert fk.lib.fk_load_dispatcher(None, str(p).encode(), C.byref(h)) == fk.FK_ERR_IO
+    assert fk.lib.fk_load_dispatcher(str(tmp_path / "kernel.hsaco").encode(), None, C.byref(h)) == fk.FK_ERR_NOT_FOUND
+
+
+def test_product_never_imports_or_links_the_oracle():
+    pkg = os.path.join(ROOT, "fusekit_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f), errors="replace").read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+                assert "_work/" not in text and "_work\"" not in text, os.path.join(dirpath, f)
+
+
+def test_decoder_config_byte_accounting():
+    from fusekit_amd.decoder import DENSE_4B, DecoderConfig
+    cfg = DecoderConfig(**DENSE_4B)
+    per_layer = 2560 * (4096 + 1024 + 1024) + 4096 * 2560 + 3 * 9728 * 2560
+    assert per_layer == 100925440
+    assert cfg.layer_param_bytes() == int(per_layer * 0.5625)
+    assert cfg.n_layers * cfg.layer_param_bytes() == 2043740160          # 4-bit g64 layer weights per token
+    assert cfg.token_bytes(512) == 2043740160 + 777912320 + 75497472     # + tied bf16 LM head + KV at ctx 512
+    assert DecoderConfig(**DENSE_4B, bits=8).n_layers * DecoderConfig(**DENSE_4B, bits=8).layer_param_bytes() == 3860398080
+    assert DecoderConfig(**DENSE_4B, bits=16).n_layers * DecoderConfig(**DENSE_4B, bits=16).layer_param_bytes() == 7266631680
