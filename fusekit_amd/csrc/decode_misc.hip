@@ -5,6 +5,7 @@
 // boundaries.
 #include "fk_host.hpp"
 #include "fk_device.hpp"
+#include "rope_device.hpp"
 
 namespace fk {
 
@@ -15,21 +16,6 @@ namespace fk {
 // head into the cache row.  With a norm weight the head is first RMS-normalised
 // with the reference's two roundings, T(w * T(x * r)), and the rotation acts on
 // those T values.
-__device__ __forceinline__ void rope_rotate(float lo, float hi, uint32_t d, uint32_t half, uint32_t pos,
-                                            float base_log2, float& olo, float& ohi) {
-    // inv = exp2(-(d/half) * log2(theta)); angle = pos * inv (reference rope_q_decode.rs:93-114)
-    const float d_norm = (float)d / (float)half;
-    // The fp32 exponent is rounded like the reference's; 2^t itself goes through
-    // double so that the fp32 frequency is the correctly rounded one on every
-    // platform (an ulp of inv_freq is 2.5e-3 rad at position 32767).
-    const float inv_freq = (float)exp2((double)(-d_norm * base_log2));
-    const float angle = (float)pos * inv_freq;
-    float sn, cs;
-    sincosf(angle, &sn, &cs);
-    olo = lo * cs - hi * sn;
-    ohi = hi * cs + lo * sn;
-}
-
 __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
     const uint32_t b = blockIdx.x, lane = threadIdx.x;
     const uint32_t pos = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
@@ -50,32 +36,8 @@ __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
     uint16_t* dst = is_q ? a.q + (size_t)h * dim : a.cache_k + ((size_t)h * a.capacity + row) * dim;
     const uint16_t* nw = is_q ? a.q_norm : a.k_norm;
 
-    float r = 1.f;
-    if (nw) {
-        float ss = 0.f;
-        for (uint32_t d = lane; d < dim; d += kWave) {
-            const float x = bf16_bits_to_f32(src[d]);
-            ss = fmaf(x, x, ss);
-        }
-        ss = wave_sum(ss);
-        r = 1.0f / sqrtf(ss / (float)dim + a.eps);
-    }
-    auto value = [&](uint32_t d) {
-        const float x = bf16_bits_to_f32(src[d]);
-        return nw ? round_bf16(bf16_bits_to_f32(nw[d]) * round_bf16(x * r)) : x;
-    };
-    const uint32_t half = a.rope_on ? a.rope_dims / 2 : 0;
-    // rotated pairs (d, d + half); all reads of a pair happen in the lane that writes it
-    for (uint32_t d = lane; d < half; d += kWave) {
-        float lo, hi;
-        rope_rotate(value(d), value(d + half), d, half, pos, a.base_log2, lo, hi);
-        dst[d] = (uint16_t)f32_to_bf16_bits(lo);
-        dst[d + half] = (uint16_t)f32_to_bf16_bits(hi);
-    }
-    // pass-through tail (dims beyond rope_dims, or everything when rotation is off)
-    if (nw || !is_q) {
-        for (uint32_t d = 2 * half + lane; d < dim; d += kWave) dst[d] = (uint16_t)f32_to_bf16_bits(value(d));
-    }
+    head_transform(src, dst, nw, dim, a.rope_on ? a.rope_dims : 0u, pos, a.base_log2, a.eps, nw != nullptr || !is_q,
+                   lane);
 }
 
 fk_status plan_rope_store(const RopeArgs& in, Launch* out) {

@@ -23,6 +23,7 @@
 #include <string>
 #include <vector>
 
+#include "decode_token.hpp"
 #include "fk_host.hpp"
 #include "fk_json.hpp"
 
@@ -515,6 +516,11 @@ struct Graph {
     std::vector<Node> nodes;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    // persistent whole-token mode: one kernel node; device-side tables it reads
+    bool persistent = false;
+    Launch token_launch;
+    void* d_tables = nullptr;
+    uint32_t* d_abort = nullptr;
 };
 
 struct DispatcherState {
@@ -603,6 +609,204 @@ fk_status timed(DispatcherState* ds, double* gpu_seconds, const std::function<fk
     float ms = 0.f;
     FK_HIP(hipEventElapsedTime(&ms, ds->ev0, ds->ev1));
     if (gpu_seconds) *gpu_seconds = ms * 1e-3;
+    return FK_OK;
+}
+
+// ---- persistent whole-token kernel: match the canonical decode pipeline ----
+//   step_init, embed_lookup_decode, L x [rmsnorm_qkv, rope/store (one fused task or the
+//   q + kv pair, plain or head-norm), sdpa_decode, linear_residual, rmsnorm_gateup_swiglu,
+//   linear_residual], final_rmsnorm_lm_head, argmax_logits_decode (with history)
+// and turn it into the argument tables of decode_token_kernel.
+bool is_family(const Node& n, const char* prefix) {
+    const Family* f = find_family(n.d.kernel);
+    return f && strcmp(f->prefix, prefix) == 0;
+}
+
+template <typename T>
+const T& blob(const Node& n) {
+    return *reinterpret_cast<const T*>(n.launch.args);
+}
+
+fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Graph* g) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    auto bad = [](const std::string& why) {
+        return set_error(FK_ERR_UNSUPPORTED, "persistent decode: task list is not the canonical dense pipeline (" + why + ")");
+    };
+    const size_t n = nodes.size();
+    if (n < 10) return bad("too few tasks");
+    if (!is_family(nodes[0], "fusekit_step_init")) return bad("task 0 is not step_init");
+    if (!is_family(nodes[1], "fusekit_embed_lookup_decode")) return bad("task 1 is not embed_lookup_decode");
+    if (nodes[1].d.u("bits", 16) != 16) return bad("quantised embedding table");
+    if (!is_family(nodes[n - 2], "fusekit_final_rmsnorm_lm_head") || nodes[n - 2].d.u("bits", 16) != 16)
+        return bad("no dense bf16 final_rmsnorm_lm_head before the argmax");
+    if (!is_family(nodes[n - 1], "fusekit_argmax_logits_decode") || nodes[n - 1].d.args.size() != 5)
+        return bad("last task is not argmax_logits_decode with history");
+
+    TokenArgs t;
+    memset(&t, 0, sizeof(t));
+    t.step_counter = arg_ptr<uint32_t>(nodes[0].d, 0);
+    t.offset = arg_ptr<uint32_t>(nodes[0].d, 1);
+    t.kv_len = arg_ptr<uint32_t>(nodes[0].d, 2);
+    t.token = arg_ptr<uint32_t>(nodes[1].d, 0);
+    t.embed = arg_ptr<const uint16_t>(nodes[1].d, 1);
+    t.x0 = arg_ptr<uint16_t>(nodes[1].d, 2);
+    t.hidden = nodes[1].d.u("hidden");
+    t.vocab = nodes[1].d.u("vocab");
+    t.embed_scale = (float)nodes[1].d.param("output_scale", 1.0);
+    const Node& am = nodes[n - 1];
+    t.logits = arg_ptr<const uint16_t>(am.d, 0);
+    if (arg_ptr<uint32_t>(am.d, 1) != t.token) return bad("argmax does not feed the embedding's token buffer");
+    t.history = arg_ptr<uint32_t>(am.d, 3);
+    t.hist_counter = arg_ptr<uint32_t>(am.d, 4);
+    t.hist_capacity = (uint32_t)(am.d.args[3].nbytes / 4);
+    if (am.d.u("vocab") != t.vocab) return bad("argmax and embedding disagree on the vocabulary");
+
+    // walk the layers
+    struct LayerIdx { size_t qkv, rope0, rope1, sdpa, o, gateup, down; };
+    std::vector<LayerIdx> layers;
+    size_t i = 2;
+    while (i < n - 2) {
+        LayerIdx L{};
+        if (!is_family(nodes[i], "fusekit_rmsnorm_qkv")) return bad("expected rmsnorm_qkv at task " + std::to_string(i));
+        L.qkv = i++;
+        if (is_family(nodes[i], "fusekit_qkv_rope_store_decode")) {
+            L.rope0 = L.rope1 = i++;
+        } else if ((is_family(nodes[i], "fusekit_rope_q_decode") && is_family(nodes[i + 1], "fusekit_rope_kv_cache_store_decode")) ||
+                   (is_family(nodes[i], "fusekit_rmsnorm_rope_q_decode") &&
+                    is_family(nodes[i + 1], "fusekit_rmsnorm_rope_kv_cache_store_decode"))) {
+            L.rope0 = i;
+            L.rope1 = i + 1;
+            i += 2;
+        } else {
+            return bad("expected a rope / KV-store task at " + std::to_string(i));
+        }
+        if (i + 4 > n - 2) return bad("truncated layer");
+        if (!is_family(nodes[i], "fusekit_sdpa_decode")) return bad("expected sdpa_decode at task " + std::to_string(i));
+        L.sdpa = i++;
+        if (!is_family(nodes[i], "fusekit_linear_residual")) return bad("expected linear_residual at task " + std::to_string(i));
+        L.o = i++;
+        if (!is_family(nodes[i], "fusekit_rmsnorm_gateup_swiglu")) return bad("expected rmsnorm_gateup_swiglu at task " + std::to_string(i));
+        L.gateup = i++;
+        if (!is_family(nodes[i], "fusekit_linear_residual")) return bad("expected linear_residual at task " + std::to_string(i));
+        L.down = i++;
+        layers.push_back(L);
+    }
+    if (layers.empty()) return bad("no layers");
+    const uint32_t bits = nodes[layers[0].qkv].d.u("bits", 4);
+    const int kind = bits == 4 ? W_Q4 : (bits == 8 ? W_Q8 : W_BF16);
+    const SdpaArgs& s0 = blob<SdpaArgs>(nodes[layers[0].sdpa]);
+    const uint32_t G = s0.n_heads / s0.n_kv;
+    const int gt = G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1));
+    if (gt == 1) return bad("one query head per kv head");
+
+    std::vector<GemvArgs> gemv(4 * layers.size() + 1);
+    std::vector<SdpaArgs> sdpa(layers.size());
+    uint32_t grid = (uint32_t)dev->cus * 4, lds_max = 0;
+    for (int pass = 0; pass < 3; ++pass) {
+        t_gemv_grid_override = grid;
+        lds_max = 0;
+        fk_status st = FK_OK;
+        auto replan = [&](size_t node, GemvArgs* out) -> fk_status {
+            Launch l;
+            SlotRW rw;
+            fk_status r = plan_dispatch(nodes[node].d, &l, &rw);
+            if (r != FK_OK) return r;
+            *out = *reinterpret_cast<const GemvArgs*>(l.args);
+            lds_max = std::max(lds_max, l.shmem);
+            return FK_OK;
+        };
+        for (size_t li = 0; li < layers.size() && st == FK_OK; ++li) {
+            const LayerIdx& L = layers[li];
+            for (size_t node : {L.qkv, L.o, L.gateup, L.down})
+                if (nodes[node].d.u("bits", 4) != bits) st = bad("layers mix weight formats");
+            if (st != FK_OK) break;
+            if ((st = replan(L.qkv, &gemv[4 * li])) != FK_OK) break;
+            if ((st = replan(L.o, &gemv[4 * li + 1])) != FK_OK) break;
+            if ((st = replan(L.gateup, &gemv[4 * li + 2])) != FK_OK) break;
+            if ((st = replan(L.down, &gemv[4 * li + 3])) != FK_OK) break;
+        }
+        if (st == FK_OK) st = replan(n - 2, &gemv[4 * layers.size()]);
+        t_gemv_grid_override = 0;
+        FK_TRY(st);
+        lds_max = std::max(lds_max, (uint32_t)(sdpa_lds_floats(gt, s0.chunk_len, s0.qk_dim, s0.v_dim, true) * sizeof(float)));
+        lds_max = std::max(lds_max, (uint32_t)(kGemvBlock / kWave * sizeof(unsigned long long)));
+        uint32_t max_grid = 0;
+        FK_TRY(token_kernel_max_grid(kind, gt, lds_max, &max_grid));
+        if (max_grid == grid) break;
+        grid = max_grid;
+    }
+    {   // the final grid is what fits with the final LDS need
+        uint32_t max_grid = 0;
+        FK_TRY(token_kernel_max_grid(kind, gt, lds_max, &max_grid));
+        if (grid > max_grid) grid = max_grid;
+    }
+    if ((uint64_t)grid * kGemvBlock < t.hidden) return bad("hidden size exceeds one thread per element");
+
+    for (size_t li = 0; li < layers.size(); ++li) {
+        const LayerIdx& L = layers[li];
+        SdpaArgs s = blob<SdpaArgs>(nodes[L.sdpa]);
+        if (s.kv_len_ptr != t.kv_len) return bad("sdpa does not read the step counter's kv_len");
+        if (s.n_heads / s.n_kv != G || s.qk_dim != s0.qk_dim || s.v_dim != s0.v_dim) return bad("layers differ in head layout");
+        if (s.qk_dim != s.v_dim) return bad("qk_dim != v_dim");
+        const RopeArgs& r0 = blob<RopeArgs>(nodes[L.rope0]);
+        const RopeArgs& r1 = blob<RopeArgs>(nodes[L.rope1]);
+        if (r0.offset_ptr != t.offset || r1.offset_ptr != t.offset) return bad("rope does not read the step counter's offset");
+        if (r1.write_offset_ptr && r1.write_offset_ptr != t.offset) return bad("cache row is not the rope position");
+        if (r0.q != s.q) return bad("sdpa does not read the rope task's q");
+        if (r1.cache_k != s.k || r1.cache_v != s.v) return bad("sdpa does not read the caches the store task writes");
+        if (r1.capacity != s.capacity || r1.k_dim != s.qk_dim || r1.v_dim != s.v_dim || r0.head_dim != s.qk_dim)
+            return bad("rope and sdpa disagree on dims or capacity");
+        if (!r0.rope_on || !r1.rope_on || r0.rope_dims != r1.rope_dims) return bad("rotation must be on for q and k alike");
+        if ((r0.q_norm == nullptr) != (r1.k_norm == nullptr)) return bad("q and k head norms must come together");
+        s.k_new = r1.k;
+        s.v_new = r1.v;
+        s.q_norm = r0.q_norm;
+        s.k_norm = r1.k_norm;
+        s.cache_k_w = r1.cache_k;
+        s.cache_v_w = r1.cache_v;
+        s.rope_dims = r0.rope_dims;
+        s.eps = r0.eps;
+        s.base_log2 = r0.base_log2;
+        sdpa[li] = s;
+    }
+
+    // device tables: [gemv][sdpa][argmax partials][barrier counter, base][abort]
+    const size_t gemv_bytes = gemv.size() * sizeof(GemvArgs), sdpa_bytes = sdpa.size() * sizeof(SdpaArgs);
+    const size_t part_off = (gemv_bytes + sdpa_bytes + 255) / 256 * 256, part_bytes = (size_t)grid * 8;
+    const size_t bar_off = (part_off + part_bytes + 255) / 256 * 256;
+    const size_t total = bar_off + 256;
+    std::vector<unsigned char> host(total, 0);
+    memcpy(host.data(), gemv.data(), gemv_bytes);
+    memcpy(host.data() + gemv_bytes, sdpa.data(), sdpa_bytes);
+    FK_HIP(hipMalloc(&g->d_tables, total));
+    FK_HIP(hipMemcpy(g->d_tables, host.data(), total, hipMemcpyHostToDevice));
+    char* base = reinterpret_cast<char*>(g->d_tables);
+    t.gemv = reinterpret_cast<const GemvArgs*>(base);
+    t.sdpa = reinterpret_cast<const SdpaArgs*>(base + gemv_bytes);
+    t.n_layers = (uint32_t)layers.size();
+    t.argmax_partial = reinterpret_cast<unsigned long long*>(base + part_off);
+    t.bar_counter = reinterpret_cast<unsigned long long*>(base + bar_off);
+    t.bar_base = reinterpret_cast<unsigned long long*>(base + bar_off + 8);
+    t.abort_flag = reinterpret_cast<uint32_t*>(base + bar_off + 16);
+    t.spin_limit = spin_limit;
+    g->d_abort = t.abort_flag;
+
+    TokenKernelSpec spec;
+    spec.kind = kind;
+    spec.gt = gt;
+    spec.lds_bytes = lds_max;
+    spec.args = t;
+    FK_TRY(plan_token_kernel(spec, grid, &g->token_launch));
+    g->persistent = true;
+    return FK_OK;
+}
+
+fk_status check_abort(Graph* g) {
+    if (!g->persistent) return FK_OK;
+    uint32_t flag = 0;
+    FK_HIP(hipMemcpy(&flag, g->d_abort, 4, hipMemcpyDeviceToHost));
+    if (flag) return set_error(FK_ERR_HIP, "persistent decode kernel: a grid barrier wait exceeded its spin limit; results are invalid");
     return FK_OK;
 }
 
@@ -729,6 +933,51 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
     return FK_OK;
 }
 
+fk_status fk_build_decode_graph(fk_handle h, const fk_dispatch* list, size_t n, int persistent, uint32_t spin_limit,
+                                uint32_t* graph_id) {
+    if (!persistent) return fk_build_graph(h, list, n, nullptr, graph_id);
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!list || n == 0 || !graph_id) return set_error(FK_ERR_INVALID, "empty dispatch list or null out");
+    std::lock_guard<std::mutex> lk(ds->mu);
+    auto g = std::make_unique<Graph>();
+    g->nodes.resize(n);
+    for (size_t i = 0; i < n; ++i) {
+        FK_TRY(copy_dispatch(list[i], &g->nodes[i].d));
+        FK_TRY(plan_dispatch(g->nodes[i].d, &g->nodes[i].launch, &g->nodes[i].rw));
+    }
+    FK_TRY(build_token_kernel(g->nodes, spin_limit ? spin_limit : 4000000u, g.get()));
+    FK_HIP(hipGraphCreate(&g->graph, 0));
+    {
+        hipKernelNodeParams p;
+        memset(&p, 0, sizeof(p));
+        void* slot = g->token_launch.args;
+        p.func = const_cast<void*>(g->token_launch.func);
+        p.gridDim = g->token_launch.grid;
+        p.blockDim = g->token_launch.block;
+        p.sharedMemBytes = g->token_launch.shmem;
+        p.kernelParams = &slot;
+        hipGraphNode_t node;
+        FK_HIP(hipGraphAddKernelNode(&node, g->graph, nullptr, 0, &p));
+    }
+    FK_HIP(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    ds->graphs.push_back(std::move(g));
+    *graph_id = (uint32_t)ds->graphs.size() - 1;
+    return FK_OK;
+}
+
+fk_status fk_graph_launch_shape(fk_handle h, uint32_t graph_id, uint32_t* persistent, uint32_t* grid, uint32_t* lds_bytes) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (persistent) *persistent = g->persistent ? 1u : 0u;
+    if (grid) *grid = g->persistent ? g->token_launch.grid.x : 0u;
+    if (lds_bytes) *lds_bytes = g->persistent ? g->token_launch.shmem : 0u;
+    return FK_OK;
+}
+
 fk_status fk_graph_info(fk_handle h, uint32_t graph_id, uint32_t* n_nodes, uint32_t* n_edges) {
     DispatcherState* ds;
     FK_TRY(get_dispatcher(h, &ds));
@@ -762,6 +1011,7 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
     std::lock_guard<std::mutex> lk(ds->mu);
     Graph* g;
     FK_TRY(get_graph(ds, graph_id, &g));
+    if (g->persistent) return set_error(FK_ERR_UNSUPPORTED, "a persistent decode graph holds its bindings in device tables; rebuild it instead");
     // validate all, then apply (a failed update leaves the graph untouched)
     std::vector<Dispatch> patched;
     std::vector<uint32_t> touched;
@@ -805,10 +1055,11 @@ fk_status fk_execute_graph(fk_handle h, uint32_t graph_id, double* gpu_seconds) 
     Graph* g;
     FK_TRY(get_graph(ds, graph_id, &g));
     if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is pending; call fk_wait_pending first");
-    return timed(ds, gpu_seconds, [&]() -> fk_status {
+    FK_TRY(timed(ds, gpu_seconds, [&]() -> fk_status {
         FK_HIP(hipGraphLaunch(g->exec, ds->stream));
         return FK_OK;
-    });
+    }));
+    return check_abort(g);
 }
 
 fk_status fk_execute_graph_repeat(fk_handle h, uint32_t graph_id, uint32_t count, double* gpu_seconds) {
@@ -818,10 +1069,11 @@ fk_status fk_execute_graph_repeat(fk_handle h, uint32_t graph_id, uint32_t count
     Graph* g;
     FK_TRY(get_graph(ds, graph_id, &g));
     if (ds->pending) return set_error(FK_ERR_INVALID, "an async graph launch is pending; call fk_wait_pending first");
-    return timed(ds, gpu_seconds, [&]() -> fk_status {
+    FK_TRY(timed(ds, gpu_seconds, [&]() -> fk_status {
         for (uint32_t i = 0; i < count; ++i) FK_HIP(hipGraphLaunch(g->exec, ds->stream));
         return FK_OK;
-    });
+    }));
+    return check_abort(g);
 }
 
 fk_status fk_execute_graph_range(fk_handle h, uint32_t graph_id, uint32_t start, uint32_t end, double* gpu_seconds) {
@@ -903,6 +1155,7 @@ fk_status fk_decode_chunk(fk_handle h, uint32_t graph_id, const fk_decode_unifor
         for (uint32_t i = 0; i < count; ++i) FK_HIP(hipGraphLaunch(g->exec, ds->stream));
         return FK_OK;
     }));
+    FK_TRY(check_abort(g));
     FK_HIP(hipMemcpy(out_tokens, u->history, (size_t)count * 4, hipMemcpyDeviceToHost));
     return FK_OK;
 }
@@ -932,6 +1185,7 @@ fk_status fk_decode_chunk_host_loop(fk_handle h, uint32_t graph_id, const fk_dec
             return FK_OK;
         }));
         total += t;
+        FK_TRY(check_abort(g));
         FK_HIP(hipMemcpy(&out_next[i], u->token, 4, hipMemcpyDeviceToHost));
     }
     if (gpu_seconds) *gpu_seconds = total;

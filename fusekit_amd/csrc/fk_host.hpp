@@ -57,6 +57,9 @@ struct GemvPolicy {
     uint32_t rows_per_tile = 0, grid_blocks = 0;
 };
 extern GemvPolicy g_gemv_policy;
+// When non-zero, plan_gemv on this thread sizes its tiles for exactly this many
+// blocks (the persistent whole-token kernel plans every phase for its own grid).
+extern thread_local uint32_t t_gemv_grid_override;
 
 struct GemvRequest {
     const fk_weight* mats[3] = {nullptr, nullptr, nullptr};

@@ -8,6 +8,7 @@
 namespace fk {
 
 GemvPolicy g_gemv_policy;
+thread_local uint32_t t_gemv_grid_override = 0;
 
 namespace {
 
@@ -116,7 +117,8 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
         const uint32_t lds_r = lds_for(r);
         if ((int)lds_r > dev->max_dyn_lds) continue;
         const uint64_t tiles = tiles_for(r);
-        uint64_t cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : resident_for(lds_r);
+        uint64_t cap = t_gemv_grid_override ? t_gemv_grid_override
+                       : (g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : resident_for(lds_r));
         const uint64_t blocks = tiles < cap ? tiles : cap;
         const uint64_t per_block = (tiles + blocks - 1) / blocks;
         const uint64_t batches = ((uint64_t)r * cpr + pos - 1) / pos;
@@ -133,7 +135,8 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     if (g_gemv_policy.rows_per_tile) {
         best_r = g_gemv_policy.rows_per_tile;
         const uint64_t tiles = tiles_for(best_r);
-        const uint64_t cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : resident_for(lds_for(best_r));
+        const uint64_t cap = t_gemv_grid_override ? t_gemv_grid_override
+                             : (g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : resident_for(lds_for(best_r)));
         best_blocks = (uint32_t)(tiles < cap ? tiles : cap);
     }
     const uint32_t R = best_r;

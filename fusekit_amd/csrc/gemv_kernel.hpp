@@ -159,8 +159,8 @@ __device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int va
 // chunk sum is a 2- or 4-lane butterfly.  K must be a multiple of 64.
 constexpr int kStageRegs = 4;
 
-template <WKind KIND, bool NORM>
-__device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, float* sx, float* scratch) {
+template <WKind KIND, bool NORM, typename ARGS>
+__device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, float* sx, float* scratch) {
     const uint32_t K = a.K, cpr = a.cpr, n8 = K >> 3;
     const uint4* x8 = reinterpret_cast<const uint4*>(a.x);
     const uint4* w8 = reinterpret_cast<const uint4*>(a.norm_w);
@@ -252,13 +252,88 @@ __device__ __forceinline__ void stage_activations(const GemvArgs& a, uint4* xs, 
     __syncthreads();
 }
 
+// Per-tile facts, uniform over the block (scalar registers).
+template <int NSEG>
+struct GemvTile {
+    const char* w[NSEG];
+    const char* sc[NSEG];
+    const char* bi[NSEG];
+    uint32_t m, row0, valid;
+};
+
+// ARGS is GemvArgs (kernel argument) or a constant-address-space view of one that
+// lives in device memory; either way the fields are read through scalar loads.
+template <WKind KIND, int NSEG, typename ARGS>
+__device__ __forceinline__ GemvTile<NSEG> gemv_tile(const ARGS& a, uint32_t tile) {
+    GemvTile<NSEG> t;
+    const uint32_t R = a.R, cpr = a.cpr;
+    if constexpr (NSEG == 2) {
+        t.m = 0;
+        t.row0 = tile * R;
+    } else {
+        t.m = (a.n_mats > 1 && tile >= a.tile_start[1]) ? ((a.n_mats > 2 && tile >= a.tile_start[2]) ? 2u : 1u) : 0u;
+        t.row0 = (tile - a.tile_start[t.m]) * R;
+    }
+    const uint32_t left = a.n[t.m] - t.row0;
+    t.valid = left < R ? left : R;
+    const size_t base = (size_t)t.row0 * cpr;
+#pragma unroll
+    for (int sg = 0; sg < NSEG; ++sg) {
+        const uint32_t mm = (NSEG == 2) ? (uint32_t)sg : t.m;
+        t.w[sg] = reinterpret_cast<const char*>(a.w[mm] + base);
+        if constexpr (KIND != W_BF16) {
+            t.sc[sg] = reinterpret_cast<const char*>(a.sc[mm] + (base >> a.gshift));
+            t.bi[sg] = reinterpret_cast<const char*>(a.bi[mm] + (base >> a.gshift));
+        }
+    }
+    return t;
+}
+
+// Issues the 16-byte weight loads (and scale/bias) of one batch into registers.
+// Slot j belongs to segment j / SLOTS, so every slot's base pointer is uniform
+// and the per-lane part of the address is a 32-bit byte offset.  Straight-line:
+// positions outside the tile's valid rows read chunk 0 of the tile instead
+// (always in bounds); their partials are never consumed.
+template <WKind KIND, int NSEG, typename ARGS>
+__device__ __forceinline__ void gemv_load_batch(const ARGS& a, uint4 (&wv)[kGemvUnroll],
+                                                uint32_t (&sc)[kGemvUnroll], uint32_t (&bi)[kGemvUnroll],
+                                                uint32_t tile, uint32_t b0) {
+    constexpr int SLOTS = kGemvUnroll / NSEG;
+    const GemvTile<NSEG> t = gemv_tile<KIND, NSEG, ARGS>(a, tile);
+    const uint32_t valid_chunks = t.valid * a.cpr;
+#pragma unroll
+    for (int j = 0; j < kGemvUnroll; ++j) {
+        const int sg = j / SLOTS;
+        const uint32_t pos = b0 + (j % SLOTS) * kGemvBlock + threadIdx.x;
+        const uint32_t idx = pos < valid_chunks ? pos : 0u;
+        wv[j] = *reinterpret_cast<const uint4*>(t.w[sg] + (idx << 4));
+        if constexpr (KIND != W_BF16) {
+            const uint32_t goff = (idx >> a.gshift) << 1;
+            sc[j] = *reinterpret_cast<const uint16_t*>(t.sc[sg] + goff);
+            bi[j] = *reinterpret_cast<const uint16_t*>(t.bi[sg] + goff);
+        }
+    }
+}
+
+// First batch of this block's first tile: pure weight traffic, independent of the
+// activations, so a caller may issue it before x exists (before a grid barrier).
+template <WKind KIND, int NSEG, typename ARGS>
+__device__ __forceinline__ void gemv_prefetch(const ARGS& a, uint32_t block_id, uint4 (&wv)[kGemvUnroll],
+                                              uint32_t (&sc)[kGemvUnroll], uint32_t (&bi)[kGemvUnroll]) {
+    if (block_id < a.n_tiles) gemv_load_batch<KIND, NSEG, ARGS>(a, wv, sc, bi, block_id, 0);
+}
+
+// The block's share of one GEMV: tiles block_id, block_id + n_blocks, ...
+// (wa, sa, ba) must hold the batch gemv_prefetch loaded for the same arguments.
+//
 // NSEG = 1: fan-out over up to three matrices sharing x (plain GEMV, QKV,
 //           residual projections, LM head); each tile lies inside one matrix.
 // NSEG = 2: gate/up pair; a tile holds R gate rows and the same R up rows and
 //           the epilogue is SwiGLU.
-template <WKind KIND, int NSEG, bool NORM>
-__global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs a) {
-    extern __shared__ uint4 lds_raw[];
+template <WKind KIND, int NSEG, bool NORM, typename ARGS>
+__device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint32_t n_blocks, uint4* lds_raw,
+                                         uint4 (&wa)[kGemvUnroll], uint32_t (&sa)[kGemvUnroll],
+                                         uint32_t (&ba)[kGemvUnroll]) {
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     constexpr int SLOTS = kGemvUnroll / NSEG;                // register slots per segment and batch
     constexpr uint32_t POS = kGemvBlock * SLOTS;             // chunk positions of a segment per batch
@@ -271,61 +346,6 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
     float* part = sx + cpr;                                  // [NSEG][seg_pad]
     float* scratch = part + NSEG * seg_pad;
 
-    // Per-tile facts, uniform over the block (scalar registers).
-    struct TileInfo {
-        const char* w[NSEG];
-        const char* sc[NSEG];
-        const char* bi[NSEG];
-        uint32_t m, row0, valid;
-    };
-    auto tile_info = [&](uint32_t tile) {
-        TileInfo t;
-        if constexpr (NSEG == 2) {
-            t.m = 0;
-            t.row0 = tile * R;
-        } else {
-            t.m = (a.n_mats > 1 && tile >= a.tile_start[1]) ? ((a.n_mats > 2 && tile >= a.tile_start[2]) ? 2u : 1u)
-                                                            : 0u;
-            t.row0 = (tile - a.tile_start[t.m]) * R;
-        }
-        const uint32_t left = a.n[t.m] - t.row0;
-        t.valid = left < R ? left : R;
-        const size_t base = (size_t)t.row0 * cpr;
-#pragma unroll
-        for (int sg = 0; sg < NSEG; ++sg) {
-            const uint32_t mm = (NSEG == 2) ? (uint32_t)sg : t.m;
-            t.w[sg] = reinterpret_cast<const char*>(a.w[mm] + base);
-            if constexpr (KIND != W_BF16) {
-                t.sc[sg] = reinterpret_cast<const char*>(a.sc[mm] + (base >> a.gshift));
-                t.bi[sg] = reinterpret_cast<const char*>(a.bi[mm] + (base >> a.gshift));
-            }
-        }
-        return t;
-    };
-
-    // Issues the 16-byte weight loads (and scale/bias) of one batch into registers.
-    // Slot j belongs to segment j / SLOTS, so every slot's base pointer is uniform
-    // and the per-lane part of the address is a 32-bit byte offset.  Straight-line:
-    // positions outside the tile's valid rows read chunk 0 of the tile instead
-    // (always in bounds); their partials are never consumed.
-    auto load_batch = [&](uint4(&wv)[kGemvUnroll], uint32_t(&sc)[kGemvUnroll], uint32_t(&bi)[kGemvUnroll],
-                          uint32_t tile, uint32_t b0) {
-        const TileInfo t = tile_info(tile);
-        const uint32_t valid_chunks = t.valid * cpr;
-#pragma unroll
-        for (int j = 0; j < kGemvUnroll; ++j) {
-            const int sg = j / SLOTS;
-            const uint32_t pos = b0 + (j % SLOTS) * kGemvBlock + threadIdx.x;
-            const uint32_t idx = pos < valid_chunks ? pos : 0u;
-            wv[j] = *reinterpret_cast<const uint4*>(t.w[sg] + (idx << 4));
-            if constexpr (KIND != W_BF16) {
-                const uint32_t goff = (idx >> a.gshift) << 1;
-                sc[j] = *reinterpret_cast<const uint16_t*>(t.sc[sg] + goff);
-                bi[j] = *reinterpret_cast<const uint16_t*>(t.bi[sg] + goff);
-            }
-        }
-    };
-
     // Column (chunk within its row) of each slot's position; advanced per batch
     // instead of dividing by cpr for every chunk.
     uint32_t col0[SLOTS], col[SLOTS];
@@ -337,7 +357,7 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
     }
     const uint32_t col_step = POS % cpr;
 
-    uint32_t tile = blockIdx.x, b0 = 0;
+    uint32_t tile = block_id, b0 = 0;
 
     // Consumes the batch held in cur* while the following batch streams into nxt*.
     // Returns false once this block has no tile left.
@@ -345,10 +365,10 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
                     uint4(&nxt)[kGemvUnroll], uint32_t(&nsc)[kGemvUnroll], uint32_t(&nbi)[kGemvUnroll]) -> bool {
         uint32_t ntile = tile, nb0 = b0 + POS;
         if (nb0 >= seg_chunks) {
-            ntile = tile + gridDim.x;
+            ntile = tile + n_blocks;
             nb0 = 0;
         }
-        if (ntile < a.n_tiles) load_batch(nxt, nsc, nbi, ntile, nb0);
+        if (ntile < a.n_tiles) gemv_load_batch<KIND, NSEG, ARGS>(a, nxt, nsc, nbi, ntile, nb0);
 
         float p[kGemvUnroll];
 #pragma unroll
@@ -367,7 +387,7 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
         if (ntile != tile) {
             // tile complete: add each row's partials in a fixed order, then the epilogue
             __syncthreads();
-            const TileInfo t = tile_info(tile);
+            const GemvTile<NSEG> t = gemv_tile<KIND, NSEG, ARGS>(a, tile);
             const uint32_t lr = a.lr, lane = threadIdx.x & (lr - 1);
             for (uint32_t rr = threadIdx.x / lr; rr < R; rr += kGemvBlock / lr) {
                 float s0 = 0.f, s1 = 0.f;
@@ -407,16 +427,23 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
         return tile < a.n_tiles;
     };
 
-    uint4 wa[kGemvUnroll], wb[kGemvUnroll];
-    uint32_t sa[kGemvUnroll], sb[kGemvUnroll], ba[kGemvUnroll], bb[kGemvUnroll];
-    const bool has_work = tile < a.n_tiles;
-    if (has_work) load_batch(wa, sa, ba, tile, 0);  // weights start streaming before x is staged
-    stage_activations<KIND, NORM>(a, xs, sx, scratch);
-    if (!has_work) return;
+    uint4 wb[kGemvUnroll];
+    uint32_t sb[kGemvUnroll], bb[kGemvUnroll];
+    stage_activations<KIND, NORM, ARGS>(a, xs, sx, scratch);
+    if (block_id >= a.n_tiles) return;
     while (true) {
         if (!step(wa, sa, ba, wb, sb, bb)) break;
         if (!step(wb, sb, bb, wa, sa, ba)) break;
     }
+}
+
+template <WKind KIND, int NSEG, bool NORM>
+__global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    uint4 wa[kGemvUnroll];
+    uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
+    gemv_prefetch<KIND, NSEG>(a, blockIdx.x, wa, sa, ba);  // weights start streaming before x is staged
+    gemv_run<KIND, NSEG, NORM>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba);
 }
 
 }  // namespace fk

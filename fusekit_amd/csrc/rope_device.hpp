@@ -1,0 +1,55 @@
+// Per-head transform shared by the rope/store kernel and the fused attention
+// phase: optional RMSNorm with the reference's two roundings, T(w * T(x * r)),
+// then half-split RoPE on the first rope_dims of the head.  One wave per head.
+#pragma once
+#include "fk_device.hpp"
+
+namespace fk {
+
+__device__ __forceinline__ void rope_rotate(float lo, float hi, uint32_t d, uint32_t half, uint32_t pos,
+                                            float base_log2, float& olo, float& ohi) {
+    // inv = exp2(-(d/half) * log2(theta)); angle = pos * inv (reference rope_q_decode.rs:93-114)
+    const float d_norm = (float)d / (float)half;
+    // The fp32 exponent is rounded like the reference's; 2^t itself goes through
+    // double so that the fp32 frequency is the correctly rounded one on every
+    // platform (an ulp of inv_freq is 2.5e-3 rad at position 32767).
+    const float inv_freq = (float)exp2((double)(-d_norm * base_log2));
+    const float angle = (float)pos * inv_freq;
+    float sn, cs;
+    sincosf(angle, &sn, &cs);
+    olo = lo * cs - hi * sn;
+    ohi = hi * cs + lo * sn;
+}
+
+// src -> dst (may alias: every pair is read and written by one lane).  `copy_tail`
+// writes the dims outside the rotation too (needed when dst != src or when the
+// norm changed them).
+__device__ __forceinline__ void head_transform(const uint16_t* src, uint16_t* dst, const uint16_t* nw, uint32_t dim,
+                                               uint32_t rope_dims, uint32_t pos, float base_log2, float eps,
+                                               bool copy_tail, uint32_t lane) {
+    float r = 1.f;
+    if (nw) {
+        float ss = 0.f;
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            const float x = bf16_bits_to_f32(src[d]);
+            ss = fmaf(x, x, ss);
+        }
+        ss = wave_sum(ss);
+        r = 1.0f / sqrtf(ss / (float)dim + eps);
+    }
+    auto value = [&](uint32_t d) {
+        const float x = bf16_bits_to_f32(src[d]);
+        return nw ? round_bf16(bf16_bits_to_f32(nw[d]) * round_bf16(x * r)) : x;
+    };
+    const uint32_t half = rope_dims / 2;
+    for (uint32_t d = lane; d < half; d += kWave) {
+        float lo, hi;
+        rope_rotate(value(d), value(d + half), d, half, pos, base_log2, lo, hi);
+        dst[d] = (uint16_t)f32_to_bf16_bits(lo);
+        dst[d + half] = (uint16_t)f32_to_bf16_bits(hi);
+    }
+    if (copy_tail)
+        for (uint32_t d = 2 * half + lane; d < dim; d += kWave) dst[d] = (uint16_t)f32_to_bf16_bits(value(d));
+}
+
+}  // namespace fk

@@ -1,0 +1,289 @@
+// Device side of the split-K attention decode: SdpaArgs, the per-work-item
+// function sdpa_block and the stand-alone kernel.  See sdpa.hip for the scheme.
+#pragma once
+#include "fk_device.hpp"
+#include "rope_device.hpp"
+
+namespace fk {
+
+constexpr int kSdpaBlock = 256;
+constexpr int kSdpaWaves = kSdpaBlock / kWave;
+constexpr int kSteps = 8;  // K rows (and at most as many V rows) each lane owns per range
+
+struct SdpaArgs {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    uint16_t* out;
+    const uint32_t* kv_len_ptr;  // device scalar, or null -> kv_len_imm
+    uint32_t kv_len_imm;
+    uint32_t n_heads, n_kv, qk_dim, v_dim, capacity;
+    uint32_t chunk_len, n_splits;
+    uint32_t lpk, lpv;  // lanes per key row / value row (powers of two)
+    float scale;
+    float* partials;     // [n_heads][n_splits][v_dim + 2]
+    uint32_t* counters;  // [n_kv * head tiles], zero before the first launch
+    // Fused mode (the whole-token kernel): q, k_new, v_new are the raw projection
+    // outputs of this token at position kv_len - 1.  Every block transforms its q
+    // heads itself (head norm + RoPE); the block whose range holds the new position
+    // transforms k_new, uses it and v_new in place of the cache row and writes both
+    // into the cache.
+    const uint16_t* k_new;
+    const uint16_t* v_new;
+    const uint16_t* q_norm;
+    const uint16_t* k_norm;
+    uint16_t* cache_k_w;
+    uint16_t* cache_v_w;
+    uint32_t rope_dims;
+    float eps, base_log2;
+};
+
+// m[GT] and l[GT] (GT <= 8), the last-block flag and block-reduction scratch.
+constexpr uint32_t kSdpaStatFloats = 32;
+
+// LDS floats one block needs.
+__host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk, uint32_t qk_dim, uint32_t v_dim,
+                                                     bool fused) {
+    return gt * chunk + kSdpaWaves * gt * v_dim + kSdpaStatFloats + (fused ? (gt + 1) * qk_dim / 2 + 8 : 0);
+}
+
+// One (range, kv head, head tile) work item.  Uniform per block; `kv_len` already read.
+template <int GT, bool FUSED, typename ARGS>
+__device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
+                                           uint32_t gz, uint32_t gz_count, float* lds) {
+    const uint32_t n_active = (kv_len + a.chunk_len - 1) / a.chunk_len;
+    if (split >= n_active) return;  // uniform: whole block leaves before any barrier
+
+    const uint32_t G = a.n_heads / a.n_kv;
+    const uint32_t h0 = kvh * G + gz * GT;
+    const uint32_t gcount = (G - gz * GT) < (uint32_t)GT ? (G - gz * GT) : (uint32_t)GT;
+    const uint32_t key0 = split * a.chunk_len;
+    const uint32_t nkeys = (kv_len - key0) < a.chunk_len ? (kv_len - key0) : a.chunk_len;
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+
+    float* s = lds;                               // [GT][chunk_len]
+    float* red = s + GT * a.chunk_len;            // [waves][GT][v_dim]
+    float* stat = red + kSdpaWaves * GT * a.v_dim;  // m[GT], l[GT], misc
+    uint16_t* qn = reinterpret_cast<uint16_t*>(stat + kSdpaStatFloats);  // fused: [GT][qk_dim] + k row
+    uint16_t* kn = qn + GT * a.qk_dim;
+    const uint32_t pos = kv_len - 1;  // fused: position of the new token
+    const bool owner = FUSED && pos >= key0 && pos < key0 + nkeys;
+    const uint32_t jpos = pos - key0;
+
+    if constexpr (FUSED) {
+        // head norm + RoPE of this block's q heads (one wave per head), and of the new
+        // k row in the block that owns its position; results in LDS as bf16.  Done
+        // before the K/V loads are issued: the trigonometry needs ~60 registers that
+        // the 64 registers of in-flight rows would otherwise have to share
+        for (uint32_t h = wave; h < gcount + (owner ? 1u : 0u); h += kSdpaWaves) {
+            if (h < gcount) {
+                head_transform(a.q + (size_t)(h0 + h) * a.qk_dim, qn + h * a.qk_dim, a.q_norm, a.qk_dim, a.rope_dims,
+                               pos, a.base_log2, a.eps, true, lane);
+            } else {
+                head_transform(a.k_new + (size_t)kvh * a.qk_dim, kn, a.k_norm, a.qk_dim, a.rope_dims, pos, a.base_log2,
+                               a.eps, true, lane);
+            }
+        }
+        __syncthreads();
+        if (owner && gz == 0) {  // one block per kv head appends the new rows to the cache
+            const size_t row = (size_t)kvh * a.capacity + (pos % a.capacity);
+            for (uint32_t d = tid; d < a.qk_dim; d += kSdpaBlock) a.cache_k_w[row * a.qk_dim + d] = kn[d];
+            for (uint32_t d = tid; d < a.v_dim; d += kSdpaBlock)
+                a.cache_v_w[row * a.v_dim + d] = a.v_new[(size_t)kvh * a.v_dim + d];
+        }
+    }
+
+    // All K and V loads of the range are issued up front (the range is sized so that
+    // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
+    const uint32_t lpk = a.lpk, cpk = a.qk_dim >> 3;
+    const uint32_t lpv = a.lpv, cpv = a.v_dim >> 3;
+    const uint32_t ck = tid & (lpk - 1), kslot = tid / lpk, kslots = kSdpaBlock / lpk;
+    const uint32_t cv = tid & (lpv - 1), vslot = tid / lpv, vslots = kSdpaBlock / lpv;
+    const bool kcol_ok = ck < cpk, vcol_ok = cv < cpv;
+    uint4 kc[kSteps], vc[kSteps];
+    {
+        const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * ck;
+        const uint16_t* vbase = a.v + ((size_t)kvh * a.capacity + key0) * a.v_dim + 8 * cv;
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = kslot + u * kslots;
+            kc[u] = make_uint4(0, 0, 0, 0);
+            if (kcol_ok && j < nkeys && !(owner && j == jpos))
+                kc[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * a.qk_dim);
+        }
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = vslot + u * vslots;
+            vc[u] = make_uint4(0, 0, 0, 0);
+            if (vcol_ok && j < nkeys) {
+                const uint16_t* src = vbase + (size_t)j * a.v_dim;
+                if (owner && j == jpos) src = a.v_new + (size_t)kvh * a.v_dim + 8 * cv;  // the new row, not yet cached
+                vc[u] = *reinterpret_cast<const uint4*>(src);
+            }
+        }
+    }
+
+    // ---------------- phase A: scores ----------------
+    {
+        uint4 qf[GT];
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            qf[h] = make_uint4(0, 0, 0, 0);
+            if (kcol_ok && (uint32_t)h < gcount) {
+                if constexpr (FUSED)
+                    qf[h] = *reinterpret_cast<const uint4*>(qn + h * a.qk_dim + 8 * ck);
+                else
+                    qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
+            }
+        }
+        if constexpr (FUSED) {
+            if (owner && kcol_ok) {
+#pragma unroll
+                for (int u = 0; u < kSteps; ++u)
+                    if (kslot + u * kslots == jpos) kc[u] = *reinterpret_cast<const uint4*>(kn + 8 * ck);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = kslot + u * kslots;
+#pragma unroll
+            for (int h = 0; h < GT; ++h) {
+                float d = 0.f;
+                d = dot2_bf16(kc[u].x, qf[h].x, d);
+                d = dot2_bf16(kc[u].y, qf[h].y, d);
+                d = dot2_bf16(kc[u].z, qf[h].z, d);
+                d = dot2_bf16(kc[u].w, qf[h].w, d);
+                d = group_sum(d, (int)lpk);
+                if (ck == 0 && j < nkeys) s[h * a.chunk_len + j] = d * a.scale;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---------------- softmax over this range, one wave per head ----------------
+    for (uint32_t h = wave; h < gcount; h += kSdpaWaves) {
+        float* sh = s + h * a.chunk_len;
+        float m = -INFINITY;
+        for (uint32_t j = lane; j < nkeys; j += kWave) m = fmaxf(m, sh[j]);
+        m = wave_max(m);
+        float l = 0.f;
+        for (uint32_t j = lane; j < nkeys; j += kWave) {
+            const float p = expf(sh[j] - m);
+            sh[j] = p;
+            l += p;
+        }
+        l = wave_sum(l);
+        if (lane == 0) {
+            stat[h] = m;
+            stat[GT + h] = l;
+        }
+    }
+    __syncthreads();
+
+    // ---------------- phase B: o = sum_j p_j v_j ----------------
+    {
+        float acc[GT][8];
+#pragma unroll
+        for (int h = 0; h < GT; ++h)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = vslot + u * vslots;
+            const uint32_t jj = j < nkeys ? j : 0u;
+            const float live = j < nkeys ? 1.f : 0.f;
+            const float f[8] = {bf16_lo(vc[u].x), bf16_hi(vc[u].x), bf16_lo(vc[u].y), bf16_hi(vc[u].y),
+                                bf16_lo(vc[u].z), bf16_hi(vc[u].z), bf16_lo(vc[u].w), bf16_hi(vc[u].w)};
+#pragma unroll
+            for (int h = 0; h < GT; ++h) {
+                const float p = s[h * a.chunk_len + jj] * live;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
+            }
+        }
+        // add the key slots that share this lane's column: first inside the wave ...
+#pragma unroll
+        for (int h = 0; h < GT; ++h)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float v = acc[h][i];
+                for (uint32_t o = lpv; o < (uint32_t)kWave; o <<= 1) v += __shfl_xor(v, (int)o, kWave);
+                acc[h][i] = v;
+            }
+        // ... then across waves through LDS
+        if (lane < lpv && vcol_ok) {
+#pragma unroll
+            for (int h = 0; h < GT; ++h)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) red[(wave * GT + h) * a.v_dim + 8 * cv + i] = acc[h][i];
+        }
+    }
+    __syncthreads();
+
+    const uint32_t n_out = gcount * a.v_dim;
+    const bool direct = (n_active == 1);
+    for (uint32_t e = tid; e < n_out; e += kSdpaBlock) {
+        const uint32_t h = e / a.v_dim, d = e - h * a.v_dim;
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < kSdpaWaves; ++w) o += red[(w * GT + h) * a.v_dim + d];
+        if (direct) {
+            a.out[(size_t)(h0 + h) * a.v_dim + d] = (uint16_t)f32_to_bf16_bits(o / stat[GT + h]);
+        } else {
+            float* p = a.partials + ((size_t)(h0 + h) * a.n_splits + split) * (a.v_dim + 2);
+            p[2 + d] = o;
+            if (d == 0) {
+                p[0] = stat[h];
+                p[1] = stat[GT + h];
+            }
+        }
+    }
+    if (direct) return;
+
+    // ---------------- last block merges the partials ----------------
+    __threadfence();
+    __syncthreads();
+    uint32_t* flag = reinterpret_cast<uint32_t*>(stat + 16);
+    if (tid == 0) {
+        const uint32_t prev = atomicAdd(&a.counters[kvh * gz_count + gz], 1u);
+        *flag = (prev == n_active - 1) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (*flag == 0u) return;
+    __threadfence();
+    if (tid == 0) a.counters[kvh * gz_count + gz] = 0u;  // ready for the next launch
+
+    // weights w_s = exp(m_s - M) / L per head, held in LDS (reuses the score area
+    // when the range count fits, else loops in pieces of chunk_len)
+    for (uint32_t h = 0; h < gcount; ++h) {
+        const float* ph = a.partials + (size_t)(h0 + h) * a.n_splits * (a.v_dim + 2);
+        float m = -INFINITY;
+        for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) m = fmaxf(m, ph[(size_t)sp * (a.v_dim + 2)]);
+        m = block_max<kSdpaBlock>(m, stat + 20);
+        float l = 0.f;
+        for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) {
+            const float* p = ph + (size_t)sp * (a.v_dim + 2);
+            l += p[1] * expf(p[0] - m);
+        }
+        l = block_sum<kSdpaBlock>(l, stat + 20);
+        const float inv_l = 1.0f / l;
+        // each thread owns output dims; ranges are added in index order
+        for (uint32_t d = tid; d < a.v_dim; d += kSdpaBlock) {
+            float o = 0.f;
+            for (uint32_t sp = 0; sp < n_active; ++sp) {
+                const float* p = ph + (size_t)sp * (a.v_dim + 2);
+                o = fmaf(p[2 + d], expf(p[0] - m), o);
+            }
+            a.out[(size_t)(h0 + h) * a.v_dim + d] = (uint16_t)f32_to_bf16_bits(o * inv_l);
+        }
+    }
+}
+
+template <int GT>
+__global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs a) {
+    extern __shared__ float lds[];
+    const uint32_t kv_len = a.kv_len_ptr ? *a.kv_len_ptr : a.kv_len_imm;
+    sdpa_block<GT, false, SdpaArgs>(a, kv_len, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
+}
+
+}  // namespace fk

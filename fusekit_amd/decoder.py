@@ -159,7 +159,7 @@ class DecoderRuntime:
     """Scratch arena, KV caches, uniforms and the captured decode graph of one model."""
 
     def __init__(self, cfg: DecoderConfig, weights: DecoderWeights, dispatcher: Optional[Dispatcher] = None,
-                 hist_capacity: int = 4096):
+                 hist_capacity: int = 4096, persistent: bool = False, spin_limit: int = 0):
         self.cfg, self.w = cfg, weights
         self.d = dispatcher or Dispatcher()
         z = native.zeros
@@ -178,7 +178,10 @@ class DecoderRuntime:
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
         self.tasks = self.build_tasks()
-        self.graph = self.d.build_graph(self.tasks)
+        self.persistent = persistent
+        # persistent: the same task list, run by one whole-token kernel per replay
+        self.graph = (self.d.build_decode_graph(self.tasks, True, spin_limit) if persistent
+                      else self.d.build_graph(self.tasks))
 
     # -- task list -------------------------------------------------------------------
     def _wargs(self, W: DeviceWeight):

@@ -98,6 +98,19 @@ class Dispatcher:
         check(lib.fk_build_graph(self.handle, arr, C.c_size_t(len(ds)), b, C.byref(gid)))
         return gid.value
 
+    def build_decode_graph(self, ds: Sequence[Dispatch], persistent: bool = True, spin_limit: int = 0) -> int:
+        """The decode pipeline as one graph; persistent=True runs it as ONE whole-token kernel."""
+        arr, keep = _marshal(ds)
+        gid = C.c_uint32()
+        check(lib.fk_build_decode_graph(self.handle, arr, C.c_size_t(len(ds)), C.c_int(1 if persistent else 0),
+                                        C.c_uint32(spin_limit), C.byref(gid)))
+        return gid.value
+
+    def graph_launch_shape(self, gid: int) -> Tuple[bool, int, int]:
+        p, g, l = C.c_uint32(), C.c_uint32(), C.c_uint32()
+        check(lib.fk_graph_launch_shape(self.handle, C.c_uint32(gid), C.byref(p), C.byref(g), C.byref(l)))
+        return bool(p.value), g.value, l.value
+
     def graph_info(self, gid: int) -> Tuple[int, int]:
         n, e = C.c_uint32(), C.c_uint32()
         check(lib.fk_graph_info(self.handle, C.c_uint32(gid), C.byref(n), C.byref(e)))

@@ -277,6 +277,22 @@ fk_status fk_dispatch_batch(fk_handle h, const fk_dispatch *list, size_t n, doub
  * command i wait for every earlier command. */
 fk_status fk_build_graph(fk_handle h, const fk_dispatch *list, size_t n, const uint8_t *barriers,
                          uint32_t *graph_id);
+/* Decode pipeline as a graph.  persistent = 0: same as fk_build_graph (one node
+ * per task).  persistent = 1: the task list must be the canonical dense decode
+ * pipeline (step_init, embed_lookup_decode, L x [rmsnorm_qkv, rope / KV-store
+ * task(s), sdpa_decode, linear_residual, rmsnorm_gateup_swiglu, linear_residual],
+ * final_rmsnorm_lm_head, argmax_logits_decode with history); it is run by ONE
+ * persistent kernel per token whose phases are separated by grid barriers and
+ * which prefetches the next phase's weights across them -- the working form of
+ * what the reference sketches as emit_megakernel (src/codegen/persistent.rs:57-75)
+ * and the LayerBlock experiment (src/fusion/layer_block.rs).  Same arithmetic.
+ * Otherwise FK_ERR_UNSUPPORTED.  spin_limit bounds every barrier wait in polls
+ * (0 = default); a wait that exceeds it sets an abort flag, all waves still
+ * drain, and the launching call returns FK_ERR_HIP. */
+fk_status fk_build_decode_graph(fk_handle h, const fk_dispatch *list, size_t n, int persistent,
+                                uint32_t spin_limit, uint32_t *graph_id);
+fk_status fk_graph_launch_shape(fk_handle h, uint32_t graph_id, uint32_t *persistent, uint32_t *grid,
+                                uint32_t *lds_bytes);
 fk_status fk_graph_info(fk_handle h, uint32_t graph_id, uint32_t *n_nodes, uint32_t *n_edges);
 fk_status fk_graph_node_deps(fk_handle h, uint32_t graph_id, uint32_t node, uint32_t *deps, uint32_t cap,
                              uint32_t *n);

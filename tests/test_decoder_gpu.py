@@ -17,10 +17,10 @@ def _small_cfg(**kw):
     return DecoderConfig(**base)
 
 
-def _run_pair(fk, cfg, seed, n_prompt=8, n_decode=24):
+def _run_pair(fk, cfg, seed, n_prompt=8, n_decode=24, persistent=False):
     from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
     W = DecoderWeights.random_init(cfg, seed=seed)
-    rt = DecoderRuntime(cfg, W)
+    rt = DecoderRuntime(cfg, W, persistent=persistent)
     prompt = rng(seed).integers(0, cfg.vocab, n_prompt).tolist()
     got, gpu_s, steps = rt.generate(prompt, n_decode)
     ref, margins = OracleDecoder(cfg, W).generate(prompt, n_decode)
@@ -177,3 +177,65 @@ def test_update_graph_bindings_repoints_kv_cache(fk):
         rt.d.update_graph_bindings(rt.graph, [(9999, 0, new_k.ptr, 16)])
     with pytest.raises(fk.InvalidArgument):
         rt.d.update_graph_bindings(rt.graph, [(0, 0, 0, 16)])
+
+
+# ---------------------------------------------------------------- persistent whole-token kernel
+@pytest.mark.parametrize("bits", [4, 8, 16])
+@pytest.mark.parametrize("qk_norm,bias,fuse,heads", [(True, False, True, (4, 2)), (False, True, False, (8, 2)),
+                                                      (True, False, False, (16, 2))])
+def test_persistent_kernel_tokens_match_oracle(fk, bits, qk_norm, bias, fuse, heads):
+    """One kernel per token (grid barriers between phases, weights prefetched across them) must
+    decode the same greedy tokens as the oracle -- and hence as the task-per-kernel graph."""
+    cfg = _small_cfg(bits=bits, qk_norm=qk_norm, qkv_bias=bias, fuse_rope_store=fuse, n_heads=heads[0], n_kv=heads[1],
+                     hidden=heads[0] * 64)
+    got, ref, margins, rt = _run_pair(fk, cfg, seed=4, persistent=True)
+    is_p, grid, lds = rt.d.graph_launch_shape(rt.graph)
+    assert is_p and grid >= 256 and rt.d.graph_info(rt.graph)[0] == len(rt.tasks)
+    for i, (g, r) in enumerate(zip(got, ref)):
+        assert g == r, f"step {i}: gpu {g} oracle {r} (oracle margin {margins[i]})"
+
+
+def test_persistent_kernel_matches_task_graph_state(fk):
+    """Same tokens, same KV-cache contents and same logits as the one-node-per-task graph."""
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    cfg = _small_cfg(bits=4, qk_norm=True, n_layers=4)
+    W = DecoderWeights.random_init(cfg, seed=9)
+    a, b = DecoderRuntime(cfg, W), DecoderRuntime(cfg, W, persistent=True)
+    prompt = [11, 22, 33, 44, 55]
+    ta, _, _ = a.generate(prompt, 40)
+    tb, _, _ = b.generate(prompt, 40)
+    assert ta == tb
+    for l in range(cfg.n_layers):
+        # rows written so far: prompt + 39 decode steps fed back
+        rows = len(prompt) + 39
+        ka = a.cache_k[l].to_numpy(np.uint16).reshape(cfg.n_kv, cfg.capacity, cfg.head_dim)[:, :rows]
+        kb = b.cache_k[l].to_numpy(np.uint16).reshape(cfg.n_kv, cfg.capacity, cfg.head_dim)[:, :rows]
+        frac, ulps = bf16_mismatch(ka, kb)
+        assert ulps <= 1.0 and frac < 0.01
+    frac, ulps = bf16_mismatch(a.logits.to_numpy(np.uint16), b.logits.to_numpy(np.uint16))
+    assert ulps <= 2.0 and frac < 0.05
+    assert int(b.step_counter.to_numpy(np.uint32)[0]) == len(prompt) + 39
+
+
+def test_persistent_kernel_rejects_other_task_lists(fk):
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    cfg = _small_cfg(bits=4, n_layers=1)
+    rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=1))
+    with pytest.raises(fk.FusekitError):
+        rt.d.build_decode_graph(rt.tasks[:-1], True)          # no argmax
+    with pytest.raises(fk.FusekitError):
+        rt.d.build_decode_graph(rt.tasks[:3] + rt.tasks[4:], True)   # a layer task missing
+    gid = rt.d.build_decode_graph(rt.tasks, True)
+    with pytest.raises(fk.FusekitError):
+        rt.d.update_graph_bindings(gid, [(2, 0, rt.x[0].ptr, 16)])
+
+
+def test_persistent_kernel_barrier_timeout_drains_and_reports(fk):
+    """A wait that exceeds its spin limit (forced from the host: limit of one poll) must not hang:
+    every wave drains, and the call reports the failure."""
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    cfg = _small_cfg(bits=4, n_layers=2)
+    rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=1), persistent=True, spin_limit=1)
+    with pytest.raises(fk.FusekitError) as e:
+        rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, [5])
+    assert "spin limit" in str(e.value)
