@@ -36,6 +36,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=2)
     ap.add_argument("--per-kernel", action="store_true", help="print per-family GPU time of one token to stderr")
+    ap.add_argument("--layers", type=int, default=0, help="experiment only: override the layer count (not the headline config)")
+    ap.add_argument("--mode", choices=["persistent", "graph"], default="graph",
+                    help="persistent: one whole-token kernel per replay; graph: one kernel node per task")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the decode path has no multi-GPU mode (--gpus must be 1)",
@@ -52,9 +55,12 @@ def main() -> int:
     total = args.prompt + args.warmup + args.steps
     capacity = max(1024, 1 << (total - 1).bit_length())
     cfg = DecoderConfig(**DENSE_4B, bits=args.bits, capacity=capacity)
+    if args.layers:
+        cfg.n_layers = args.layers
     t0 = time.time()
     W = DecoderWeights.random_init(cfg, seed=0)
-    rt = DecoderRuntime(cfg, W, hist_capacity=max(4096, args.steps + args.warmup))
+    rt = DecoderRuntime(cfg, W, hist_capacity=max(4096, args.steps + args.warmup),
+                        persistent=(args.mode == "persistent"))
     setup_s = time.time() - t0
 
     rng = np.random.Generator(np.random.PCG64(0))
@@ -96,7 +102,14 @@ def main() -> int:
     achieved = gateup_bytes / (gateup_us * 1e-6) / 1e9
 
     per_kernel = {}
-    if args.per_kernel:
+    if args.per_kernel and args.mode == "persistent":
+        tr = rt.d.graph_phase_trace(rt.graph)
+        names = ["embed"] + ["qkv", "attention", "o_proj", "gateup", "down"] * cfg.n_layers + ["lm_head", "argmax_scan", "argmax_final"]
+        for nm, s_ in zip(names, tr):
+            per_kernel[nm] = per_kernel.get(nm, 0.0) + s_
+        print("[bench:per-phase] " + " ".join(f"{k}={v * 1e3:.3f}ms" for k, v in per_kernel.items())
+              + f" | layer0: " + " ".join(f"{n}={t * 1e6:.1f}us" for n, t in zip(names[1:6], tr[1:6])), file=sys.stderr)
+    elif args.per_kernel:
         times = rt.d.profile_graph_nodes(rt.graph)
         for t, s in zip(rt.tasks, times):
             fam = t.kernel.rsplit("_f", 1)[0]

@@ -5,8 +5,7 @@
 // rmsnorm+gate/up+SwiGLU | down+residual], final norm + LM head, argmax -- with
 // the same device functions as the one-kernel-per-task path (gemv_run,
 // sdpa_block), so the arithmetic is identical.  The grid is exactly what is
-// resident at once; phases are separated by a grid barrier (release fence, one
-// arrival atomic, bounded polling, acquire fence).  What a kernel boundary cannot
+// resident at once; phases are separated by a grid barrier (see grid_barrier).  What a kernel boundary cannot
 // do and this can: before arriving at a barrier every block issues the 16-byte
 // weight loads of its first batch of the NEXT phase, which do not depend on the
 // activations, so HBM keeps streaming across the dependency.
@@ -29,29 +28,55 @@ __device__ __forceinline__ const ConstSdpaArgs& sdpa_args(const SdpaArgs* base, 
     return *(const ConstSdpaArgs*)(base + i);
 }
 
+// Grid barrier without device-wide fences.  A device-scope fence writes back and
+// invalidates a whole L2 and costs ~30 ns per block per barrier on this part
+// (30 us for 1024 blocks); instead every byte that crosses blocks inside this
+// kernel moves through agent-scope accesses (ld_u16 / st_u16 and friends), so a
+// barrier only has to (1) wait until this block's stores have completed
+// (workgroup-scope release), (2) count arrivals on two levels of counters -- one
+// per group of kBarFan blocks, then one for the groups, so no address sees more
+// than kBarFan atomics -- and (3) let the last arriver publish the epoch in a flag
+// the others poll.  All counters are monotonic across launches.
+constexpr uint32_t kBarFan = 32;
+
 struct BarrierState {
-    unsigned long long target;
-    unsigned long long step;  // arrivals per barrier = grid size
+    unsigned long long epoch;   // the barrier this block is about to pass
+    unsigned long long first_epoch;
+    uint32_t gsize, ngrp;
+    unsigned long long* c1;     // this block's group counter
 };
 
 __device__ __forceinline__ void grid_barrier(const TokenArgs& t, BarrierState& b) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0) {
-        __threadfence();  // release this block's writes device-wide
-        atomicAdd(t.bar_counter, 1ull);
+        bool released = false;
+        const unsigned long long prev = atomicAdd(b.c1, 1ull);
+        if (prev + 1 == b.epoch * b.gsize) {
+            const unsigned long long p2 = atomicAdd(t.bar_counter, 1ull);
+            if (p2 + 1 == b.epoch * b.ngrp) {
+                __hip_atomic_store(t.bar_flag, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                released = true;
+            }
+        }
         uint32_t spins = 0;
-        while (__hip_atomic_load(t.bar_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < b.target) {
-            if (__hip_atomic_load(t.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
-            if (++spins > t.spin_limit) {
+        while (!released && __hip_atomic_load(t.bar_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < b.epoch) {
+            ++spins;
+            if ((spins & 63u) == 0u && __hip_atomic_load(t.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
+                break;
+            if (spins > t.spin_limit) {
                 __hip_atomic_store(t.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 break;
             }
             __builtin_amdgcn_s_sleep(1);
         }
-        __threadfence();  // acquire the other blocks' writes
     }
     __syncthreads();
-    b.target += b.step;
+    b.epoch += 1;
+    if (t.trace && blockIdx.x == 0 && threadIdx.x == 0) {
+        const uint32_t i = (uint32_t)(b.epoch - b.first_epoch);
+        if (i < t.trace_capacity) t.trace[i] = wall_clock64();
+    }
 }
 
 __device__ __forceinline__ uint32_t order_key(float v) {
@@ -78,9 +103,15 @@ __device__ __forceinline__ unsigned long long block_best(unsigned long long v, u
 // The attention phase as a function of its own: its register needs (in-flight K/V
 // rows, per-head accumulators, trigonometry) then do not merge with the streaming
 // phases' allocation.
+// Only blocks that own a work item call it (the caller tests bid < items): its
+// prologue saves ~150 registers per lane, which 1000 idle blocks must not pay.
 template <int GT>
 __device__ __noinline__ void attention_phase(const SdpaArgs* sdpa, uint32_t l, uint32_t kv_len, uint32_t bid,
-                                             uint32_t nb, float* lds) {
+                                             uint32_t nb) {
+    // named here, not passed in: a pointer parameter would be a generic pointer and
+    // every LDS access in the phase would become a FLAT instruction
+    extern __shared__ uint4 lds_raw[];
+    float* lds = reinterpret_cast<float*>(lds_raw);
     const ConstSdpaArgs& s = sdpa_args(sdpa, l);
     const uint32_t G = s.n_heads / s.n_kv, gz_count = (G + GT - 1) / GT;
     const uint32_t n_active = (kv_len + s.chunk_len - 1) / s.chunk_len;
@@ -100,8 +131,14 @@ __global__ __launch_bounds__(kGemvBlock) __attribute__((amdgpu_waves_per_eu(4, 8
     const uint32_t bid = blockIdx.x, nb = gridDim.x, tid = threadIdx.x;
 
     BarrierState bar;
-    bar.step = nb;
-    bar.target = *t.bar_base + nb;
+    {
+        const uint32_t grp = bid / kBarFan, g0 = grp * kBarFan;
+        bar.ngrp = (nb + kBarFan - 1) / kBarFan;
+        bar.gsize = (nb - g0) < kBarFan ? (nb - g0) : kBarFan;
+        bar.c1 = t.bar_groups + grp * 16;  // one counter per 128-byte line
+        bar.epoch = bar.first_epoch = *t.bar_base + 1;
+        if (t.trace && bid == 0 && tid == 0) t.trace[0] = wall_clock64();
+    }
     // every block reads the step counter before the first barrier; block 0 advances it after
     const uint32_t pos = *t.step_counter;
     const uint32_t kv_len = pos + 1;
@@ -115,9 +152,15 @@ __global__ __launch_bounds__(kGemvBlock) __attribute__((amdgpu_waves_per_eu(4, 8
         const ConstGemvArgs& g0 = gemv_args(t.gemv, 0);
         gemv_prefetch<KIND, 1>(g0, bid, wa, sa, ba);
         const uint32_t tok = token_in < t.vocab ? token_in : t.vocab - 1;
+        if (bid == nb - 1 && tid < t.rope_dims / 2) {  // this token's rotary table, once for all layers
+            float cs, sn;
+            rope_cos_sin(tid, t.rope_dims / 2, pos, t.rope_base_log2, cs, sn);
+            st_f32<true>(t.rope_tab + 2 * tid, cs);
+            st_f32<true>(t.rope_tab + 2 * tid + 1, sn);
+        }
         const uint32_t d = bid * kGemvBlock + tid;
         if (d < t.hidden)
-            t.x0[d] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(t.embed[(size_t)tok * t.hidden + d]) * t.embed_scale);
+            st_u16<true>(t.x0 + d, f32_to_bf16_bits(bf16_bits_to_f32(t.embed[(size_t)tok * t.hidden + d]) * t.embed_scale));
     }
     grid_barrier(t, bar);
     if (bid == 0 && tid == 0) {
@@ -128,52 +171,36 @@ __global__ __launch_bounds__(kGemvBlock) __attribute__((amdgpu_waves_per_eu(4, 8
 
     for (uint32_t l = 0; l < t.n_layers; ++l) {
         // ---- rmsnorm + q/k/v projections ----
-        {
-            const ConstGemvArgs& g = gemv_args(t.gemv, 4 * l);
-            gemv_run<KIND, 1, true>(g, bid, nb, lds_raw, wa, sa, ba);
-        }
+        gemv_run<KIND, 1, true>(gemv_args(t.gemv, 4 * l), bid, nb, lds_raw, wa, sa, ba);
         grid_barrier(t, bar);
         // ---- head norm / rope / KV append / attention ----
         {
-            attention_phase<GT>(t.sdpa, l, kv_len, bid, nb, reinterpret_cast<float*>(lds_raw));
-            const ConstGemvArgs& g = gemv_args(t.gemv, 4 * l + 1);
-            gemv_prefetch<KIND, 1>(g, bid, wa, sa, ba);
+            const ConstSdpaArgs& s = sdpa_args(t.sdpa, l);
+            const uint32_t G = s.n_heads / s.n_kv, gz_count = (G + GT - 1) / GT;
+            const uint32_t n_active = (kv_len + s.chunk_len - 1) / s.chunk_len;
+            if (bid < n_active * s.n_kv * gz_count) attention_phase<GT>(t.sdpa, l, kv_len, bid, nb);
+            gemv_prefetch<KIND, 1>(gemv_args(t.gemv, 4 * l + 1), bid, wa, sa, ba);
         }
         grid_barrier(t, bar);
         // ---- o_proj + residual ----
-        {
-            const ConstGemvArgs& g = gemv_args(t.gemv, 4 * l + 1);
-            gemv_run<KIND, 1, false>(g, bid, nb, lds_raw, wa, sa, ba);
-            const ConstGemvArgs& gn = gemv_args(t.gemv, 4 * l + 2);
-            gemv_prefetch<KIND, 2>(gn, bid, wa, sa, ba);
-        }
+        gemv_run<KIND, 1, true>(gemv_args(t.gemv, 4 * l + 1), bid, nb, lds_raw, wa, sa, ba);
+        gemv_prefetch<KIND, 2>(gemv_args(t.gemv, 4 * l + 2), bid, wa, sa, ba);
         grid_barrier(t, bar);
         // ---- rmsnorm + gate/up + SwiGLU ----
-        {
-            const ConstGemvArgs& g = gemv_args(t.gemv, 4 * l + 2);
-            gemv_run<KIND, 2, true>(g, bid, nb, lds_raw, wa, sa, ba);
-            const ConstGemvArgs& gn = gemv_args(t.gemv, 4 * l + 3);
-            gemv_prefetch<KIND, 1>(gn, bid, wa, sa, ba);
-        }
+        gemv_run<KIND, 2, true>(gemv_args(t.gemv, 4 * l + 2), bid, nb, lds_raw, wa, sa, ba);
+        gemv_prefetch<KIND, 1>(gemv_args(t.gemv, 4 * l + 3), bid, wa, sa, ba);
         grid_barrier(t, bar);
         // ---- down_proj + residual ----
-        {
-            const ConstGemvArgs& g = gemv_args(t.gemv, 4 * l + 3);
-            gemv_run<KIND, 1, false>(g, bid, nb, lds_raw, wa, sa, ba);
-            const ConstGemvArgs& gn = gemv_args(t.gemv, 4 * l + 4);
-            if (l + 1 < t.n_layers)
-                gemv_prefetch<KIND, 1>(gn, bid, wa, sa, ba);
-            else
-                gemv_prefetch<W_BF16, 1>(gn, bid, wa, sa, ba);
-        }
+        gemv_run<KIND, 1, true>(gemv_args(t.gemv, 4 * l + 3), bid, nb, lds_raw, wa, sa, ba);
+        if (l + 1 < t.n_layers)
+            gemv_prefetch<KIND, 1>(gemv_args(t.gemv, 4 * l + 4), bid, wa, sa, ba);
+        else
+            gemv_prefetch<W_BF16, 1>(gemv_args(t.gemv, 4 * l + 4), bid, wa, sa, ba);
         grid_barrier(t, bar);
     }
 
     // ---- final norm + LM head (dense bf16) ----
-    {
-        const ConstGemvArgs& g = gemv_args(t.gemv, 4 * t.n_layers);
-        gemv_run<W_BF16, 1, true>(g, bid, nb, lds_raw, wa, sa, ba);
-    }
+    gemv_run<W_BF16, 1, true>(gemv_args(t.gemv, 4 * t.n_layers), bid, nb, lds_raw, wa, sa, ba);
     grid_barrier(t, bar);
 
     // ---- greedy argmax, lowest index wins ties (argmax_logits_decode.rs:63-95) ----
@@ -186,12 +213,15 @@ __global__ __launch_bounds__(kGemvBlock) __attribute__((amdgpu_waves_per_eu(4, 8
             best = cand > best ? cand : best;
         }
         best = block_best(best, sm);
-        if (tid == 0) t.argmax_partial[bid] = best;
+        if (tid == 0) __hip_atomic_store(&t.argmax_partial[bid], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     grid_barrier(t, bar);
     if (bid == 0) {
         unsigned long long fin = 0;
-        for (uint32_t i = tid; i < nb; i += kGemvBlock) fin = t.argmax_partial[i] > fin ? t.argmax_partial[i] : fin;
+        for (uint32_t i = tid; i < nb; i += kGemvBlock) {
+            const unsigned long long c = __hip_atomic_load(&t.argmax_partial[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            fin = c > fin ? c : fin;
+        }
         fin = block_best(fin, sm);
         if (tid == 0) {
             const uint32_t tok = (fin >> 32) ? ~(uint32_t)fin : 0u;
@@ -199,7 +229,7 @@ __global__ __launch_bounds__(kGemvBlock) __attribute__((amdgpu_waves_per_eu(4, 8
             const uint32_t slot = *t.hist_counter;
             if (slot < t.hist_capacity) t.history[slot] = tok;
             *t.hist_counter = slot + 1;
-            *t.bar_base = bar.target - nb;  // arrivals so far; the next launch counts on from here
+            *t.bar_base = bar.epoch - 1;  // barriers passed so far; the next launch counts on from here
         }
     }
 }

@@ -17,6 +17,10 @@ struct TokenArgs {
     uint16_t* x0;
     uint32_t hidden, vocab;
     float embed_scale;
+    // rotary table of this token, filled in the first phase: (cos, sin) per pair
+    float* rope_tab;
+    uint32_t rope_dims;
+    float rope_base_log2;
     // per-token protocol (python_runtime/src/lib.rs:1299-1303, kernels/mod.rs:544-577)
     uint32_t* token;         // in: token to embed; out: greedy next token
     uint32_t* step_counter;  // offset = step_counter++ ; kv_len = offset + 1
@@ -28,13 +32,19 @@ struct TokenArgs {
     // argmax over the logits the LM head phase wrote
     const uint16_t* logits;
     unsigned long long* argmax_partial;  // [grid]
-    // grid barrier: a monotonic arrival counter, the count at launch start and an
-    // abort flag (set when a wait exceeds spin_limit polls; every later wait then
-    // returns at once, so all waves always drain)
-    unsigned long long* bar_counter;
-    unsigned long long* bar_base;
+    // grid barrier: monotonic two-level arrival counters, the released-epoch flag,
+    // the epoch at launch start and an abort flag (set when a wait exceeds
+    // spin_limit polls; every later wait then returns at once, so all waves drain)
+    unsigned long long* bar_groups;   // one arrival counter per group of blocks, 128 bytes apart
+    unsigned long long* bar_counter;  // arrivals of whole groups
+    unsigned long long* bar_flag;     // last barrier every block may pass
+    unsigned long long* bar_base;     // barriers passed when the launch starts
     uint32_t* abort_flag;
     uint32_t spin_limit;
+    // optional: block 0 stamps the constant-rate clock (100 MHz) after every barrier,
+    // trace[0] at entry; the per-phase profile of the last launch (null = off)
+    unsigned long long* trace;
+    uint32_t trace_capacity;
 };
 
 struct TokenKernelSpec {

@@ -521,6 +521,8 @@ struct Graph {
     Launch token_launch;
     void* d_tables = nullptr;
     uint32_t* d_abort = nullptr;
+    unsigned long long* d_trace = nullptr;
+    uint32_t trace_len = 0;
 };
 
 struct DispatcherState {
@@ -729,7 +731,8 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
         if (st == FK_OK) st = replan(n - 2, &gemv[4 * layers.size()]);
         t_gemv_grid_override = 0;
         FK_TRY(st);
-        lds_max = std::max(lds_max, (uint32_t)(sdpa_lds_floats(gt, s0.chunk_len, s0.qk_dim, s0.v_dim, true) * sizeof(float)));
+        lds_max = std::max(lds_max, (uint32_t)(sdpa_lds_floats(gt, sdpa_chunk_len(s0.qk_dim, s0.v_dim, true), s0.qk_dim,
+                                                                 s0.v_dim, true) * sizeof(float)));
         lds_max = std::max(lds_max, (uint32_t)(kGemvBlock / kWave * sizeof(unsigned long long)));
         uint32_t max_grid = 0;
         FK_TRY(token_kernel_max_grid(kind, gt, lds_max, &max_grid));
@@ -759,6 +762,10 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
             return bad("rope and sdpa disagree on dims or capacity");
         if (!r0.rope_on || !r1.rope_on || r0.rope_dims != r1.rope_dims) return bad("rotation must be on for q and k alike");
         if ((r0.q_norm == nullptr) != (r1.k_norm == nullptr)) return bad("q and k head norms must come together");
+        // ranges of the in-kernel attention are shorter than the stand-alone kernel's; its
+        // partials and counters live in the private arena, sized for that
+        s.chunk_len = sdpa_chunk_len(s.qk_dim, s.v_dim, true);
+        s.n_splits = (s.capacity + s.chunk_len - 1) / s.chunk_len;
         s.k_new = r1.k;
         s.v_new = r1.v;
         s.q_norm = r0.q_norm;
@@ -771,26 +778,101 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
         sdpa[li] = s;
     }
 
-    // device tables: [gemv][sdpa][argmax partials][barrier counter, base][abort]
+    // Private activation arena: every layer gets its own x / q / k / v / att / mid
+    // buffers (128-byte aligned), so inside one launch no address is read before the
+    // barrier that follows its only write -- plain cached loads can never be stale.
+    const uint32_t hidden = t.hidden, n_q = s0.n_heads * s0.qk_dim, n_kvd = s0.n_kv * s0.qk_dim;
+    const uint32_t inter = gemv[2].n[0];
+    auto al = [](size_t v) { return (v + 127) / 128 * 128; };
+    const size_t sz_x = al((size_t)hidden * 2), sz_q = al((size_t)n_q * 2), sz_kv = al((size_t)n_kvd * 2),
+                 sz_mid = al((size_t)inter * 2);
+    const size_t per_layer = 2 * sz_x + 2 * sz_q + 2 * sz_kv + sz_mid;
+    const size_t sz_part = al((size_t)s0.n_heads * sdpa[0].n_splits * (s0.v_dim + 2) * sizeof(float));
+    const size_t sz_cnt = al((size_t)s0.n_heads * sizeof(uint32_t));
+    if (s0.qk_dim > 2 * kGemvBlock) return bad("head too wide for the rotary table");
+    const size_t sz_tab = al((size_t)s0.qk_dim * sizeof(float));
+    const size_t arena_bytes = per_layer * layers.size() + sz_x + sz_part + sz_cnt + sz_tab;
+    // device tables: [gemv][sdpa][argmax partials][barrier counters][flags][arena]
     const size_t gemv_bytes = gemv.size() * sizeof(GemvArgs), sdpa_bytes = sdpa.size() * sizeof(SdpaArgs);
     const size_t part_off = (gemv_bytes + sdpa_bytes + 255) / 256 * 256, part_bytes = (size_t)grid * 8;
     const size_t bar_off = (part_off + part_bytes + 255) / 256 * 256;
-    const size_t total = bar_off + 256;
-    std::vector<unsigned char> host(total, 0);
+    const size_t n_groups = ((size_t)grid + 31) / 32;
+    const size_t top_off = bar_off + n_groups * 128;
+    const size_t trace_cap = 5 * layers.size() + 8;
+    const size_t trace_off = top_off + 4 * 128;
+    const size_t arena_off = (trace_off + trace_cap * 8 + 127) / 128 * 128;
+    const size_t total = arena_off + arena_bytes;
+    FK_HIP(hipMalloc(&g->d_tables, total));
+    char* base = reinterpret_cast<char*>(g->d_tables);
+    {
+        // layer l: X0_l (input) | X1_l | q | att | k | v | mid ; X0_L after the last layer
+        auto buf = [&](size_t l, size_t off) { return reinterpret_cast<uint16_t*>(base + arena_off + l * per_layer + off); };
+        const size_t o_x0 = 0, o_x1 = sz_x, o_q = 2 * sz_x, o_att = o_q + sz_q, o_k = o_att + sz_q, o_v = o_k + sz_kv,
+                     o_mid = o_v + sz_kv;
+        t.x0 = buf(0, o_x0);
+        for (size_t l = 0; l < layers.size(); ++l) {
+            GemvArgs& qkv = gemv[4 * l];
+            GemvArgs& op = gemv[4 * l + 1];
+            GemvArgs& gu = gemv[4 * l + 2];
+            GemvArgs& dn = gemv[4 * l + 3];
+            if (qkv.n_mats != 3 || qkv.n[0] != n_q || qkv.n[1] != n_kvd || qkv.n[2] != n_kvd || qkv.K != hidden ||
+                op.K != n_q || op.n[0] != hidden || gu.K != hidden || gu.n[0] != inter || dn.K != inter ||
+                dn.n[0] != hidden || !op.res || !dn.res || op.res2 || dn.res2)
+                return bad("layer shapes do not chain");
+            qkv.x = buf(l, o_x0);
+            qkv.y[0] = buf(l, o_q);
+            qkv.y[1] = buf(l, o_k);
+            qkv.y[2] = buf(l, o_v);
+            sdpa[l].q = buf(l, o_q);
+            sdpa[l].k_new = buf(l, o_k);
+            sdpa[l].v_new = buf(l, o_v);
+            sdpa[l].out = buf(l, o_att);
+            op.x = buf(l, o_att);
+            op.res = buf(l, o_x0);
+            op.y[0] = buf(l, o_x1);
+            gu.x = buf(l, o_x1);
+            gu.y[0] = buf(l, o_mid);
+            dn.x = buf(l, o_mid);
+            dn.res = buf(l, o_x1);
+            dn.y[0] = buf(l + 1, o_x0);  // the next layer's input (or the LM head's)
+        }
+        GemvArgs& head = gemv[4 * layers.size()];
+        if (head.K != hidden) return bad("LM head width");
+        head.x = buf(layers.size(), o_x0);
+        char* tail = base + arena_off + per_layer * layers.size() + sz_x;
+        for (size_t l = 0; l < layers.size(); ++l) {
+            sdpa[l].partials = reinterpret_cast<float*>(tail);
+            sdpa[l].counters = reinterpret_cast<uint32_t*>(tail + sz_part);
+        }
+        FK_HIP(hipMemset(tail + sz_part, 0, sz_cnt));
+        t.rope_tab = reinterpret_cast<float*>(tail + sz_part + sz_cnt);
+        t.rope_dims = sdpa[0].rope_dims;
+        t.rope_base_log2 = sdpa[0].base_log2;
+        for (size_t l = 0; l < layers.size(); ++l) {
+            if (sdpa[l].rope_dims != t.rope_dims || sdpa[l].base_log2 != t.rope_base_log2)
+                return bad("layers differ in rotary parameters");
+            sdpa[l].rope_tab = t.rope_tab;
+        }
+    }
+    std::vector<unsigned char> host(arena_off, 0);
     memcpy(host.data(), gemv.data(), gemv_bytes);
     memcpy(host.data() + gemv_bytes, sdpa.data(), sdpa_bytes);
-    FK_HIP(hipMalloc(&g->d_tables, total));
-    FK_HIP(hipMemcpy(g->d_tables, host.data(), total, hipMemcpyHostToDevice));
-    char* base = reinterpret_cast<char*>(g->d_tables);
+    FK_HIP(hipMemcpy(g->d_tables, host.data(), arena_off, hipMemcpyHostToDevice));
     t.gemv = reinterpret_cast<const GemvArgs*>(base);
     t.sdpa = reinterpret_cast<const SdpaArgs*>(base + gemv_bytes);
     t.n_layers = (uint32_t)layers.size();
     t.argmax_partial = reinterpret_cast<unsigned long long*>(base + part_off);
-    t.bar_counter = reinterpret_cast<unsigned long long*>(base + bar_off);
-    t.bar_base = reinterpret_cast<unsigned long long*>(base + bar_off + 8);
-    t.abort_flag = reinterpret_cast<uint32_t*>(base + bar_off + 16);
+    t.bar_groups = reinterpret_cast<unsigned long long*>(base + bar_off);
+    t.bar_counter = reinterpret_cast<unsigned long long*>(base + top_off);
+    t.bar_flag = reinterpret_cast<unsigned long long*>(base + top_off + 128);
+    t.bar_base = reinterpret_cast<unsigned long long*>(base + top_off + 256);
+    t.abort_flag = reinterpret_cast<uint32_t*>(base + top_off + 384);
     t.spin_limit = spin_limit;
+    t.trace = reinterpret_cast<unsigned long long*>(base + trace_off);
+    t.trace_capacity = (uint32_t)trace_cap;
     g->d_abort = t.abort_flag;
+    g->d_trace = t.trace;
+    g->trace_len = (uint32_t)(5 * layers.size() + 4);
 
     TokenKernelSpec spec;
     spec.kind = kind;
@@ -975,6 +1057,21 @@ fk_status fk_graph_launch_shape(fk_handle h, uint32_t graph_id, uint32_t* persis
     if (persistent) *persistent = g->persistent ? 1u : 0u;
     if (grid) *grid = g->persistent ? g->token_launch.grid.x : 0u;
     if (lds_bytes) *lds_bytes = g->persistent ? g->token_launch.shmem : 0u;
+    return FK_OK;
+}
+
+fk_status fk_graph_phase_trace(fk_handle h, uint32_t graph_id, double* seconds, uint32_t cap, uint32_t* n) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    std::lock_guard<std::mutex> lk(ds->mu);
+    Graph* g;
+    FK_TRY(get_graph(ds, graph_id, &g));
+    if (!g->persistent || !n) return set_error(FK_ERR_INVALID, "phase trace: not a persistent decode graph");
+    std::vector<unsigned long long> ticks(g->trace_len);
+    FK_HIP(hipMemcpy(ticks.data(), g->d_trace, ticks.size() * 8, hipMemcpyDeviceToHost));
+    *n = g->trace_len - 1;
+    for (uint32_t i = 0; i + 1 < g->trace_len && i < cap && seconds; ++i)
+        seconds[i] = (double)(ticks[i + 1] - ticks[i]) * 1e-8;  // constant-rate clock, 100 MHz
     return FK_OK;
 }
 

@@ -35,6 +35,48 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
                                            false);
 }
 
+// Activation traffic between blocks of ONE running kernel (the persistent
+// whole-token kernel).  Each XCD has its own L2 and the per-CU caches are not
+// coherent, so data another block wrote during the same launch must be stored
+// write-through (agent scope) and may be read with ordinary loads only from
+// addresses nobody has read earlier in the launch; buffers that ARE reused inside
+// a launch (attention partials, counters) are read with agent-scope loads, which
+// bypass the caches.  COH = false compiles to ordinary loads and stores.
+template <bool COH>
+__device__ __forceinline__ uint32_t ld_u16(const uint16_t* p) {
+    if constexpr (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
+template <bool COH>
+__device__ __forceinline__ void st_u16(uint16_t* p, uint32_t v) {
+    if constexpr (COH)
+        __hip_atomic_store(p, (uint16_t)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *p = (uint16_t)v;
+}
+template <bool COH>
+__device__ __forceinline__ uint4 ld_u128(const uint4* p) {
+    if constexpr (COH) {
+        const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+        const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return make_uint4((uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32));
+    }
+    return *p;
+}
+template <bool COH>
+__device__ __forceinline__ float ld_f32(const float* p) {
+    if constexpr (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
+template <bool COH>
+__device__ __forceinline__ void st_f32(float* p, float v) {
+    if constexpr (COH)
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *p = v;
+}
+
 // v + (v of the lane selected by a DPP control): cross-lane adds inside a row of
 // 16 lanes without going through the LDS crossbar.
 template <int CTRL>

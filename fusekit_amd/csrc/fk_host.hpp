@@ -95,7 +95,7 @@ struct RopeArgs {
 };
 fk_status plan_rope_store(const RopeArgs& in, Launch* out);
 
-uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim);
+uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim, bool fused);
 fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                size_t* partial_bytes, size_t* counter_bytes);
 fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,

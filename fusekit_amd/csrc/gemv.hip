@@ -12,21 +12,17 @@ thread_local uint32_t t_gemv_grid_override = 0;
 
 namespace {
 
-template <WKind KIND, int NSEG, bool NORM>
+template <WKind KIND, int NSEG>
 const void* gemv_func() {
-    return reinterpret_cast<const void*>(&gemv_stream_kernel<KIND, NSEG, NORM>);
+    return reinterpret_cast<const void*>(&gemv_stream_kernel<KIND, NSEG>);
 }
 
-const void* select_gemv(WKind kind, bool swiglu, bool norm) {
-#define FK_PICK(KIND)                                                                    \
-    return swiglu ? (norm ? gemv_func<KIND, 2, true>() : gemv_func<KIND, 2, false>())    \
-                  : (norm ? gemv_func<KIND, 1, true>() : gemv_func<KIND, 1, false>())
+const void* select_gemv(WKind kind, bool swiglu) {
     switch (kind) {
-        case W_Q4: FK_PICK(W_Q4);
-        case W_Q8: FK_PICK(W_Q8);
-        default: FK_PICK(W_BF16);
+        case W_Q4: return swiglu ? gemv_func<W_Q4, 2>() : gemv_func<W_Q4, 1>();
+        case W_Q8: return swiglu ? gemv_func<W_Q8, 2>() : gemv_func<W_Q8, 1>();
+        default: return swiglu ? gemv_func<W_BF16, 2>() : gemv_func<W_BF16, 1>();
     }
-#undef FK_PICK
 }
 
 uint32_t ilog2(uint32_t v) {
@@ -68,7 +64,7 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     const uint32_t cpr = K / values;
     const uint32_t nseg = rq.swiglu ? 2u : 1u;
 
-    const void* func = select_gemv(kind, rq.swiglu, rq.norm_w != nullptr);
+    const void* func = select_gemv(kind, rq.swiglu);
     auto tiles_for = [&](uint32_t r) {
         uint64_t t = 0;
         if (rq.swiglu) return (uint64_t)((rq.mats[0]->n + r - 1) / r);

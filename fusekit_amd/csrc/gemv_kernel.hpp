@@ -159,8 +159,9 @@ __device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int va
 // chunk sum is a 2- or 4-lane butterfly.  K must be a multiple of 64.
 constexpr int kStageRegs = 4;
 
-template <WKind KIND, bool NORM, typename ARGS>
+template <WKind KIND, typename ARGS>
 __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, float* sx, float* scratch) {
+    const bool NORM = a.norm_w != nullptr;  // uniform; one code path serves both
     const uint32_t K = a.K, cpr = a.cpr, n8 = K >> 3;
     const uint4* x8 = reinterpret_cast<const uint4*>(a.x);
     const uint4* w8 = reinterpret_cast<const uint4*>(a.norm_w);
@@ -172,11 +173,11 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
         wr[i] = make_uint4(0, 0, 0, 0);
         if (t < n8) {
             xr[i] = x8[t];
-            if constexpr (NORM) wr[i] = w8[t];
+            if (NORM) wr[i] = w8[t];
         }
     }
     float r = 1.0f;
-    if constexpr (NORM) {
+    if (NORM) {
         float ss = 0.f;
         auto add_sq = [&](uint4 v) {
             const uint32_t p[4] = {v.x, v.y, v.z, v.w};
@@ -201,7 +202,7 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
             f[2 * i] = bf16_lo(p[i]);
             f[2 * i + 1] = bf16_hi(p[i]);
         }
-        if constexpr (NORM) {
+        if (NORM) {
             const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -245,7 +246,7 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
         uint4 v = make_uint4(0, 0, 0, 0), wv = make_uint4(0, 0, 0, 0);
         if (t < n8) {
             v = x8[t];
-            if constexpr (NORM) wv = w8[t];
+            if (NORM) wv = w8[t];
         }
         emit(t, v, wv);
     }
@@ -330,7 +331,11 @@ __device__ __forceinline__ void gemv_prefetch(const ARGS& a, uint32_t block_id, 
 //           residual projections, LM head); each tile lies inside one matrix.
 // NSEG = 2: gate/up pair; a tile holds R gate rows and the same R up rows and
 //           the epilogue is SwiGLU.
-template <WKind KIND, int NSEG, bool NORM, typename ARGS>
+// COH: the outputs will be read by other blocks of the same launch, so they are
+// stored write-through (see st_u16).  The inputs need nothing special as long as
+// the caller guarantees that no block has read their addresses earlier in this
+// launch (the whole-token kernel gives every layer its own activation buffers).
+template <WKind KIND, int NSEG, bool COH, typename ARGS>
 __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint32_t n_blocks, uint4* lds_raw,
                                          uint4 (&wa)[kGemvUnroll], uint32_t (&sa)[kGemvUnroll],
                                          uint32_t (&ba)[kGemvUnroll]) {
@@ -360,7 +365,8 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
     uint32_t tile = block_id, b0 = 0;
 
     // Consumes the batch held in cur* while the following batch streams into nxt*.
-    // Returns false once this block has no tile left.
+    // Returns false once this block has no tile left.  (Two copies of this body,
+    // one per register set, cost code size but no register moves and no spills.)
     auto step = [&](uint4(&cur)[kGemvUnroll], uint32_t(&csc)[kGemvUnroll], uint32_t(&cbi)[kGemvUnroll],
                     uint4(&nxt)[kGemvUnroll], uint32_t(&nsc)[kGemvUnroll], uint32_t(&nbi)[kGemvUnroll]) -> bool {
         uint32_t ntile = tile, nb0 = b0 + POS;
@@ -400,7 +406,7 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
                 if (lane == 0 && rr < t.valid) {
                     const uint32_t n = t.row0 + rr, m = t.m;
                     if constexpr (NSEG == 2) {
-                        a.y[0][n] = (uint16_t)swiglu_bits(s0, s1, a.swiglu_variant);
+                        st_u16<COH>(a.y[0] + n, swiglu_bits(s0, s1, a.swiglu_variant));
                     } else {
                         float v = s0;
                         if (a.bias[m]) v += bf16_bits_to_f32(a.bias[m][n]);
@@ -408,7 +414,7 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
                         uint32_t o = f32_to_bf16_bits(v);
                         if (m == 0 && a.res2)
                             o = f32_to_bf16_bits(bf16_bits_to_f32(o) + bf16_bits_to_f32(a.res2[n]));
-                        a.y[m][n] = (uint16_t)o;
+                        st_u16<COH>(a.y[m] + n, o);
                     }
                 }
             }
@@ -429,7 +435,7 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
 
     uint4 wb[kGemvUnroll];
     uint32_t sb[kGemvUnroll], bb[kGemvUnroll];
-    stage_activations<KIND, NORM, ARGS>(a, xs, sx, scratch);
+    stage_activations<KIND, ARGS>(a, xs, sx, scratch);
     if (block_id >= a.n_tiles) return;
     while (true) {
         if (!step(wa, sa, ba, wb, sb, bb)) break;
@@ -437,13 +443,13 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
     }
 }
 
-template <WKind KIND, int NSEG, bool NORM>
+template <WKind KIND, int NSEG>
 __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs a) {
     extern __shared__ uint4 lds_raw[];
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
     gemv_prefetch<KIND, NSEG>(a, blockIdx.x, wa, sa, ba);  // weights start streaming before x is staged
-    gemv_run<KIND, NSEG, NORM>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba);
+    gemv_run<KIND, NSEG, false>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba);
 }
 
 }  // namespace fk

@@ -24,9 +24,19 @@ __device__ __forceinline__ void rope_rotate(float lo, float hi, uint32_t d, uint
 // src -> dst (may alias: every pair is read and written by one lane).  `copy_tail`
 // writes the dims outside the rotation too (needed when dst != src or when the
 // norm changed them).
+// (cos, sin) of pair d at this position: the value rope_rotate would compute, so a
+// table filled once per token gives bit-identical rotations in every layer.
+__device__ __forceinline__ void rope_cos_sin(uint32_t d, uint32_t half, uint32_t pos, float base_log2, float& cs,
+                                             float& sn) {
+    const float d_norm = (float)d / (float)half;
+    const float inv_freq = (float)exp2((double)(-d_norm * base_log2));
+    sincosf((float)pos * inv_freq, &sn, &cs);
+}
+
+// `tab` (optional): interleaved (cos, sin) per pair, as rope_cos_sin fills it.
 __device__ __forceinline__ void head_transform(const uint16_t* src, uint16_t* dst, const uint16_t* nw, uint32_t dim,
                                                uint32_t rope_dims, uint32_t pos, float base_log2, float eps,
-                                               bool copy_tail, uint32_t lane) {
+                                               bool copy_tail, uint32_t lane, const float* tab = nullptr) {
     float r = 1.f;
     if (nw) {
         float ss = 0.f;
@@ -44,7 +54,13 @@ __device__ __forceinline__ void head_transform(const uint16_t* src, uint16_t* ds
     const uint32_t half = rope_dims / 2;
     for (uint32_t d = lane; d < half; d += kWave) {
         float lo, hi;
-        rope_rotate(value(d), value(d + half), d, half, pos, base_log2, lo, hi);
+        if (tab) {
+            const float vlo = value(d), vhi = value(d + half), cs = tab[2 * d], sn = tab[2 * d + 1];
+            lo = vlo * cs - vhi * sn;
+            hi = vhi * cs + vlo * sn;
+        } else {
+            rope_rotate(value(d), value(d + half), d, half, pos, base_log2, lo, hi);
+        }
         dst[d] = (uint16_t)f32_to_bf16_bits(lo);
         dst[d + half] = (uint16_t)f32_to_bf16_bits(hi);
     }

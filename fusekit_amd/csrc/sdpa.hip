@@ -32,15 +32,15 @@ uint32_t pow2_ceil(uint32_t v) {
 // Positions per range: every lane owns exactly kSteps key rows, i.e.
 // kSteps * (block threads / lanes per key row).  128 positions for head_dim 128
 // (64 KiB of K+V per block); a 32k context then spreads over 256 ranges x kv heads.
-uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim) {
+uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim, bool fused) {
     const uint32_t lpk = pow2_ceil(qk_dim / 8), lpv = pow2_ceil(v_dim / 8);
     const uint32_t wide = lpk > lpv ? lpk : lpv;
-    return kSteps * (kSdpaBlock / wide);
+    return (fused ? kSdpaStepsFused : kSdpaSteps) * (kSdpaBlock / wide);
 }
 
 fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                size_t* partial_bytes, size_t* counter_bytes) {
-    const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim);
+    const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim, false);
     const uint32_t n_splits = (max_len + chunk - 1) / chunk;
     *partial_bytes = (size_t)n_heads * n_splits * (v_dim + 2) * sizeof(float);
     *counter_bytes = (size_t)n_heads * sizeof(uint32_t);  // >= n_kv * head tiles
@@ -62,7 +62,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     if (max_len == 0 || max_len > capacity) return set_error(FK_ERR_INVALID, "sdpa: kv length outside (0, capacity]");
     if (!kv_len_ptr && (kv_len_imm == 0 || kv_len_imm > max_len))
         return set_error(FK_ERR_INVALID, "sdpa: kv_len outside (0, max_len]");
-    const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim);
+    const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim, false);
     const uint32_t n_splits = (max_len + chunk - 1) / chunk;
     if (n_splits > 1 && (!partials || !counters))
         return set_error(FK_ERR_INVALID, "sdpa: workspace required when the context spans several ranges");

@@ -8,7 +8,8 @@ namespace fk {
 
 constexpr int kSdpaBlock = 256;
 constexpr int kSdpaWaves = kSdpaBlock / kWave;
-constexpr int kSteps = 8;  // K rows (and at most as many V rows) each lane owns per range
+constexpr int kSdpaSteps = 8;       // K rows (and at most as many V rows) each lane owns per range
+constexpr int kSdpaStepsFused = 4;  // inside the whole-token kernel: half the registers, twice the ranges
 
 struct SdpaArgs {
     const uint16_t* q;
@@ -36,6 +37,7 @@ struct SdpaArgs {
     uint16_t* cache_v_w;
     uint32_t rope_dims;
     float eps, base_log2;
+    const float* rope_tab;  // (cos, sin) per pair at this token's position, or null
 };
 
 // m[GT] and l[GT] (GT <= 8), the last-block flag and block-reduction scratch.
@@ -51,6 +53,7 @@ __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk,
 template <int GT, bool FUSED, typename ARGS>
 __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
                                            uint32_t gz, uint32_t gz_count, float* lds) {
+    constexpr int kSteps = FUSED ? kSdpaStepsFused : kSdpaSteps;
     const uint32_t n_active = (kv_len + a.chunk_len - 1) / a.chunk_len;
     if (split >= n_active) return;  // uniform: whole block leaves before any barrier
 
@@ -78,10 +81,10 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         for (uint32_t h = wave; h < gcount + (owner ? 1u : 0u); h += kSdpaWaves) {
             if (h < gcount) {
                 head_transform(a.q + (size_t)(h0 + h) * a.qk_dim, qn + h * a.qk_dim, a.q_norm, a.qk_dim, a.rope_dims,
-                               pos, a.base_log2, a.eps, true, lane);
+                               pos, a.base_log2, a.eps, true, lane, a.rope_tab);
             } else {
                 head_transform(a.k_new + (size_t)kvh * a.qk_dim, kn, a.k_norm, a.qk_dim, a.rope_dims, pos, a.base_log2,
-                               a.eps, true, lane);
+                               a.eps, true, lane, a.rope_tab);
             }
         }
         __syncthreads();
@@ -117,8 +120,11 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             vc[u] = make_uint4(0, 0, 0, 0);
             if (vcol_ok && j < nkeys) {
                 const uint16_t* src = vbase + (size_t)j * a.v_dim;
-                if (owner && j == jpos) src = a.v_new + (size_t)kvh * a.v_dim + 8 * cv;  // the new row, not yet cached
-                vc[u] = *reinterpret_cast<const uint4*>(src);
+                if (owner && j == jpos) {  // the new row, not yet cached
+                    vc[u] = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_dim + 8 * cv);
+                } else {
+                    vc[u] = *reinterpret_cast<const uint4*>(src);
+                }
             }
         }
     }
@@ -228,20 +234,25 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 #pragma unroll
         for (int w = 0; w < kSdpaWaves; ++w) o += red[(w * GT + h) * a.v_dim + d];
         if (direct) {
-            a.out[(size_t)(h0 + h) * a.v_dim + d] = (uint16_t)f32_to_bf16_bits(o / stat[GT + h]);
+            st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o / stat[GT + h]));
         } else {
             float* p = a.partials + ((size_t)(h0 + h) * a.n_splits + split) * (a.v_dim + 2);
-            p[2 + d] = o;
+            st_f32<FUSED>(p + 2 + d, o);
             if (d == 0) {
-                p[0] = stat[h];
-                p[1] = stat[GT + h];
+                st_f32<FUSED>(p, stat[h]);
+                st_f32<FUSED>(p + 1, stat[GT + h]);
             }
         }
     }
     if (direct) return;
 
     // ---------------- last block merges the partials ----------------
-    __threadfence();
+    // (inside the persistent kernel the partials travel through agent-scope accesses,
+    // so waiting for the stores to complete replaces the device-wide fences)
+    if constexpr (FUSED)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    else
+        __threadfence();
     __syncthreads();
     uint32_t* flag = reinterpret_cast<uint32_t*>(stat + 16);
     if (tid == 0) {
@@ -250,20 +261,21 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }
     __syncthreads();
     if (*flag == 0u) return;
-    __threadfence();
-    if (tid == 0) a.counters[kvh * gz_count + gz] = 0u;  // ready for the next launch
+    if constexpr (!FUSED) __threadfence();
+    if (tid == 0)  // ready for the next launch (or the next layer of this one)
+        __hip_atomic_store(&a.counters[kvh * gz_count + gz], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // weights w_s = exp(m_s - M) / L per head, held in LDS (reuses the score area
     // when the range count fits, else loops in pieces of chunk_len)
     for (uint32_t h = 0; h < gcount; ++h) {
         const float* ph = a.partials + (size_t)(h0 + h) * a.n_splits * (a.v_dim + 2);
         float m = -INFINITY;
-        for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) m = fmaxf(m, ph[(size_t)sp * (a.v_dim + 2)]);
+        for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) m = fmaxf(m, ld_f32<FUSED>(ph + (size_t)sp * (a.v_dim + 2)));
         m = block_max<kSdpaBlock>(m, stat + 20);
         float l = 0.f;
         for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) {
             const float* p = ph + (size_t)sp * (a.v_dim + 2);
-            l += p[1] * expf(p[0] - m);
+            l += ld_f32<FUSED>(p + 1) * expf(ld_f32<FUSED>(p) - m);
         }
         l = block_sum<kSdpaBlock>(l, stat + 20);
         const float inv_l = 1.0f / l;
@@ -272,9 +284,9 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             float o = 0.f;
             for (uint32_t sp = 0; sp < n_active; ++sp) {
                 const float* p = ph + (size_t)sp * (a.v_dim + 2);
-                o = fmaf(p[2 + d], expf(p[0] - m), o);
+                o = fmaf(ld_f32<FUSED>(p + 2 + d), expf(ld_f32<FUSED>(p) - m), o);
             }
-            a.out[(size_t)(h0 + h) * a.v_dim + d] = (uint16_t)f32_to_bf16_bits(o * inv_l);
+            st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o * inv_l));
         }
     }
 }

@@ -111,6 +111,13 @@ class Dispatcher:
         check(lib.fk_graph_launch_shape(self.handle, C.c_uint32(gid), C.byref(p), C.byref(g), C.byref(l)))
         return bool(p.value), g.value, l.value
 
+    def graph_phase_trace(self, gid: int) -> List[float]:
+        """Seconds per phase of the last launch of a persistent decode graph."""
+        n = C.c_uint32()
+        buf = (C.c_double * 4096)()
+        check(lib.fk_graph_phase_trace(self.handle, C.c_uint32(gid), buf, 4096, C.byref(n)))
+        return [buf[i] for i in range(min(n.value, 4096))]
+
     def graph_info(self, gid: int) -> Tuple[int, int]:
         n, e = C.c_uint32(), C.c_uint32()
         check(lib.fk_graph_info(self.handle, C.c_uint32(gid), C.byref(n), C.byref(e)))

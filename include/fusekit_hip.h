@@ -293,6 +293,11 @@ fk_status fk_build_decode_graph(fk_handle h, const fk_dispatch *list, size_t n, 
                                 uint32_t spin_limit, uint32_t *graph_id);
 fk_status fk_graph_launch_shape(fk_handle h, uint32_t graph_id, uint32_t *persistent, uint32_t *grid,
                                 uint32_t *lds_bytes);
+/* Persistent graphs only: duration of every phase of the LAST launch, seconds
+ * (embed, then per layer qkv / attention / o_proj / gate-up / down, LM head,
+ * argmax scan, argmax final) -- the per-kernel profile of the one-kernel form,
+ * what profile_icb_commands (lib.rs:823) gives for the task-per-kernel form. */
+fk_status fk_graph_phase_trace(fk_handle h, uint32_t graph_id, double *seconds, uint32_t cap, uint32_t *n);
 fk_status fk_graph_info(fk_handle h, uint32_t graph_id, uint32_t *n_nodes, uint32_t *n_edges);
 fk_status fk_graph_node_deps(fk_handle h, uint32_t graph_id, uint32_t node, uint32_t *deps, uint32_t cap,
                              uint32_t *n);
