@@ -76,6 +76,14 @@ struct GemvRequest {
 };
 fk_status plan_gemv(const GemvRequest& rq, Launch* out);
 
+// Mixture-of-experts routed projections (w_b non-null: gate/up pair with SwiGLU).
+fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
+                           uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
+                           const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out);
+fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight, const uint16_t* residual,
+                            uint16_t* out_ptr, uint32_t n_tokens, uint32_t top_k, uint32_t O, bool has_shared,
+                            Launch* out);
+
 // RoPE / per-head RMSNorm / KV-cache store (one wave per head).
 struct RopeArgs {
     uint16_t* q;             // [n_q, head_dim] in place, or null

@@ -170,6 +170,7 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     a.res = rq.res;
     a.res2 = rq.res2;
     a.swiglu_variant = rq.swiglu_variant;
+    a.y_scale = 1.0f;
 
     const uint32_t lds = lds_for(R);
     if ((int)lds > dev->max_dyn_lds) return set_error(FK_ERR_UNSUPPORTED, "gemv: K too large for LDS staging");

@@ -47,6 +47,7 @@ struct GemvArgs {
     const uint16_t* res;   // optional residual (matrix 0)
     const uint16_t* res2;  // optional second residual
     int swiglu_variant;
+    float y_scale;  // SwiGLU variant 1 only: multiplies the fp32 product before the final round
 };
 
 template <WKind KIND>
@@ -132,7 +133,7 @@ __device__ __forceinline__ float chunk_partial(uint4 wv, uint32_t s_bits, uint32
 
 // SwiGLU epilogue on the two fp32 accumulators; the three rounding variants the
 // reference emits (rmsnorm_gateup_swiglu.rs:236-257, msl.rs:1286-1294, msl.rs:2441-2449).
-__device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int variant) {
+__device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int variant, float y_scale) {
     const float g = round_bf16(acc_g), u = round_bf16(acc_u);
     if (variant == 0) {
         const float e = round_bf16(expf(fabsf(g)));
@@ -143,7 +144,7 @@ __device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int va
         return f32_to_bf16_bits(silu * u);
     } else if (variant == 1) {
         const float sig = 1.0f / (1.0f + expf(-g));
-        return f32_to_bf16_bits((sig * g) * u);
+        return f32_to_bf16_bits(((sig * g) * u) * y_scale);  // routed_qmv_swiglu.rs:420-446 (1.0 elsewhere)
     } else {
         const float sig = round_bf16(1.0f / (1.0f + expf(-g)));
         const float gated = round_bf16(sig * g);
@@ -406,7 +407,7 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
                 if (lane == 0 && rr < t.valid) {
                     const uint32_t n = t.row0 + rr, m = t.m;
                     if constexpr (NSEG == 2) {
-                        st_u16<COH>(a.y[0] + n, swiglu_bits(s0, s1, a.swiglu_variant));
+                        st_u16<COH>(a.y[0] + n, swiglu_bits(s0, s1, a.swiglu_variant, a.y_scale));
                     } else {
                         float v = s0;
                         if (a.bias[m]) v += bf16_bits_to_f32(a.bias[m][n]);

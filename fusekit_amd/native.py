@@ -174,6 +174,30 @@ def gateup_swiglu(x, norm_w, eps, Wg, Wu, variant, out, stream=None) -> None:
                                C.c_int(variant), _ptr(out), _ptr(stream)))
 
 
+def routed_qmv_swiglu(x, n_x_rows, Wg, Wu, n_experts, row_idx, expert_idx, route_weight, n_routes, out0,
+                      stream=None) -> None:
+    """Wg / Wu: DeviceWeight whose arrays are stacked [E, n, ...] and whose n, k describe one expert."""
+    check(lib.fk_routed_qmv_swiglu(_ptr(x), C.c_uint32(n_x_rows), C.byref(Wg.c), C.byref(Wu.c),
+                                   C.c_uint32(n_experts), _ptr(row_idx), _ptr(expert_idx), _ptr(route_weight),
+                                   C.c_uint32(n_routes), _ptr(out0), _ptr(stream)))
+
+
+lib.fk_routed_reduce_workspace_bytes.restype = C.c_size_t
+
+
+def routed_reduce_workspace_bytes(n_tokens, top_k, out_dim) -> int:
+    return int(lib.fk_routed_reduce_workspace_bytes(C.c_uint32(n_tokens), C.c_uint32(top_k), C.c_uint32(out_dim)))
+
+
+def routed_qmv_reduce(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_weight, shared_x, W_shared,
+                      residual_extra, n_tokens, top_k, out, workspace, stream=None) -> None:
+    check(lib.fk_routed_qmv_reduce(_ptr(h), C.c_uint32(n_h_rows), C.byref(Wd.c), C.c_uint32(n_experts),
+                                   _ptr(row_idx), _ptr(expert_idx), _ptr(route_weight), _ptr(shared_x),
+                                   C.byref(W_shared.c) if W_shared is not None else None, _ptr(residual_extra),
+                                   C.c_uint32(n_tokens), C.c_uint32(top_k), _ptr(out), _ptr(workspace),
+                                   _ptr(stream)))
+
+
 def final_rmsnorm_lm_head(x, norm_w, eps, W, logits, stream=None) -> None:
     check(lib.fk_final_rmsnorm_lm_head(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(W.c), _ptr(logits),
                                        _ptr(stream)))

@@ -118,6 +118,32 @@ fk_status fk_rmsnorm_qkv(const uint16_t *x, const uint16_t *norm_w, float eps, c
 fk_status fk_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *Wg,
                            const fk_weight *Wu, int variant, uint16_t *out, fk_stream s);
 
+/* M1  routed gate/up + SwiGLU over expert-stacked weights.  Replaces
+ *     src/codegen/kernels/routed_qmv_swiglu.rs:20-450 (slots x, gate w/s/b, up w/s/b,
+ *     row_idx, expert_idx, [route_weight], out0).  Wg / Wu describe ONE expert's
+ *     matrix [n, k]; their pointers are the bases of tensors stacked [E, n, ...].
+ *     Route r reads activation row min(row_idx[r], n_x_rows-1) (row_idx NULL: row r)
+ *     and expert min(expert_idx[r], n_experts-1);
+ *     out0[r, o] = T(((sigmoid(g) * g) * u) * route_weight[r]) with g, u = T(acc)
+ *     (route_weight NULL: factor 1). */
+fk_status fk_routed_qmv_swiglu(const uint16_t *x, uint32_t n_x_rows, const fk_weight *Wg, const fk_weight *Wu,
+                               uint32_t n_experts, const uint32_t *row_idx, const uint32_t *expert_idx,
+                               const uint16_t *route_weight, uint32_t n_routes, uint16_t *out0, fk_stream s);
+
+/* M2  routed down projection + weighted reduction (+ shared expert + residual).
+ *     Replaces src/codegen/kernels/routed_qmv_reduce.rs:14-460.  h is [n_h_rows, k]
+ *     (M1's out0); route r = tok * top_k + slot reads row min(row_idx[r], n_h_rows-1)
+ *     (row_idx NULL: row r).  out[tok, o] = T(sum_slot rw * T(dot) [+ T(shared dot)]
+ *     [+ residual_extra[tok, o]]) in slot order, fp32; route_weight NULL means the
+ *     input was pre-weighted (rw = 1).  W_shared / shared_x (both or neither; then
+ *     n_tokens must be 1, as routed_qmv_reduce.rs:80) add the shared expert's down
+ *     projection of shared_x.  workspace: fk_routed_reduce_workspace_bytes() bytes. */
+size_t fk_routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim);
+fk_status fk_routed_qmv_reduce(const uint16_t *h, uint32_t n_h_rows, const fk_weight *Wd, uint32_t n_experts,
+                               const uint32_t *row_idx, const uint32_t *expert_idx, const uint16_t *route_weight,
+                               const uint16_t *shared_x, const fk_weight *W_shared, const uint16_t *residual_extra,
+                               uint32_t n_tokens, uint32_t top_k, uint16_t *out, void *workspace, fk_stream s);
+
 /* H   final RMSNorm + vocabulary GEMV, logits in T.  Replaces
  *     src/codegen/kernels/final_rmsnorm_lm_head.rs:144-629. */
 fk_status fk_final_rmsnorm_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *W,

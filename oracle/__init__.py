@@ -283,3 +283,49 @@ def decoder_step(model: Model, token: int, offset: int, logits: np.ndarray | Non
     nxt = _lib.fko_decoder_step(C.byref(model), C.c_uint32(token), C.c_uint32(offset), _p(logits, _u16p),
                                 C.byref(margin))
     return int(nxt), float(margin.value)
+
+
+# ------------------------------------------------------------------ MoE / multi-row
+
+class StackedWeight(QWeight):
+    """Expert-stacked MLX-affine weights: w [E, O, K*bits/32], scales / biases [E, O, K/group]."""
+
+    def __init__(self, experts):
+        first = experts[0]
+        dense_kind = first.scales is None
+        super().__init__(np.stack([e.w for e in experts]),
+                         None if dense_kind else np.stack([e.scales for e in experts]),
+                         None if dense_kind else np.stack([e.biases for e in experts]),
+                         first.n, first.k, first.bits, first.group)
+        self.n_experts = len(experts)
+
+    def expert(self, e: int) -> QWeight:
+        if self.scales is None:
+            return QWeight(self.w[e], None, None, self.n, self.k, self.bits, self.group)
+        return QWeight(self.w[e], self.scales[e], self.biases[e], self.n, self.k, self.bits, self.group)
+
+
+def routed_qmv_swiglu(x, Wg: StackedWeight, Wu: StackedWeight, row_idx, expert_idx, route_weight=None) -> np.ndarray:
+    n_routes = int(expert_idx.size)
+    out = np.empty((n_routes, Wg.n), dtype=np.uint16)
+    _lib.fko_routed_qmv_swiglu(_p(x, _u16p), C.byref(Wg.c), C.byref(Wu.c), C.c_int64(Wg.n_experts),
+                               _p(row_idx, _u32p), _p(expert_idx, _u32p), _p(route_weight, _u16p),
+                               C.c_int64(n_routes), _p(out, _u16p))
+    return out
+
+
+def routed_qmv_reduce(h, Wd: StackedWeight, expert_idx, route_weight, residual_extra, n_tokens, top_k,
+                      row_idx=None, shared_x=None, Wshared: QWeight = None) -> np.ndarray:
+    out = np.empty((n_tokens, Wd.n), dtype=np.uint16)
+    _lib.fko_routed_qmv_reduce(_p(h, _u16p), C.byref(Wd.c), C.c_int64(Wd.n_experts), _p(row_idx, _u32p),
+                               _p(expert_idx, _u32p), _p(route_weight, _u16p), _p(shared_x, _u16p),
+                               C.byref(Wshared.c) if Wshared is not None else None, _p(residual_extra, _u16p),
+                               C.c_int64(n_tokens), C.c_int64(top_k), _p(out, _u16p))
+    return out
+
+
+def qgemm(W: QWeight, x: np.ndarray, bias=None) -> np.ndarray:
+    m = x.shape[0]
+    y = np.empty((m, W.n), dtype=np.uint16)
+    _lib.fko_qgemm(C.byref(W.c), _p(x, _u16p), C.c_int64(m), _p(bias, _u16p), _p(y, _u16p))
+    return y

@@ -534,6 +534,101 @@ FKO_API float fko_top2_margin(const uint16_t *logits, int64_t n) {
     return a - b;
 }
 
+/* ------------------------------------------------------- M1 / M2: MoE */
+/*
+ * Stacked expert weights: packed u32 [E, O, K*bits/32], scales / biases T [E, O, K/group]
+ * (src/codegen/kernels/routed_qmv_swiglu.rs:44-61).  Route r = tok * top_k + slot reads
+ * activation row row_idx[r] and expert expert_idx[r] (clamped to E-1, :128-139).
+ *
+ * M1 (routed_qmv_swiglu.rs:420-446): g = T(acc_gate), u = T(acc_up),
+ *    sig = 1 / (1 + exp(-g)) in fp32, out0[r, o] = T(((sig * g) * u) * rw_r)
+ *    with rw_r = route_weight[r] when pre-scaling, else 1.
+ */
+static fko_weight expert_slice(const fko_weight *W, int64_t e) {
+    fko_weight s = *W;
+    const int64_t per_word = 32 / W->bits;
+    s.w = (const uint32_t *)W->w + e * W->n * (W->k / per_word);
+    if (W->scales) {
+        s.scales = W->scales + e * W->n * (W->k / W->group);
+        s.biases = W->biases + e * W->n * (W->k / W->group);
+    }
+    return s;
+}
+
+FKO_API void fko_routed_qmv_swiglu(const uint16_t *x, const fko_weight *Wg, const fko_weight *Wu,
+                                   int64_t n_experts, const uint32_t *row_idx, const uint32_t *expert_idx,
+                                   const uint16_t *route_weight /* or NULL */, int64_t n_routes, uint16_t *out0) {
+    const int64_t K = Wg->k, O = Wg->n;
+    float *xf = (float *)malloc(sizeof(float) * (size_t)K);
+    float *ag = (float *)malloc(sizeof(float) * (size_t)O), *au = (float *)malloc(sizeof(float) * (size_t)O);
+    for (int64_t r = 0; r < n_routes; ++r) {
+        int64_t e = expert_idx[r];
+        if (e > n_experts - 1) e = n_experts - 1;
+        const fko_weight g = expert_slice(Wg, e), u = expert_slice(Wu, e);
+        for (int64_t j = 0; j < K; ++j) xf[j] = bf16_to_f32(x[(int64_t)row_idx[r] * K + j]);
+        linear_acc(&g, xf, ag);
+        linear_acc(&u, xf, au);
+        const float rw = route_weight ? bf16_to_f32(route_weight[r]) : 1.0f;
+        for (int64_t o = 0; o < O; ++o) {
+            const float gv = rbf(ag[o]), uv = rbf(au[o]);
+            const float sig = 1.0f / (1.0f + expf(-gv));
+            out0[r * O + o] = f32_to_bf16(((sig * gv) * uv) * rw);
+        }
+    }
+    free(xf); free(ag); free(au);
+}
+
+/* M2 (routed_qmv_reduce.rs:240, 315-322, 422-434): per token, slots in order,
+ *    acc += rw_r * float(T(dot_r))   (rw_r = 1 when the input was pre-weighted),
+ *    acc += residual_extra[tok, o] when present; out[tok, o] = T(acc).
+ *    dot_r = W_down[expert_r] . h[r, :]  with h = M1's out0. */
+FKO_API void fko_routed_qmv_reduce(const uint16_t *h, const fko_weight *Wd, int64_t n_experts,
+                                   const uint32_t *row_idx /* or NULL */, const uint32_t *expert_idx,
+                                   const uint16_t *route_weight /* or NULL */, const uint16_t *shared_x /* or NULL */,
+                                   const fko_weight *Wshared /* or NULL */,
+                                   const uint16_t *residual_extra /* or NULL */, int64_t n_tokens, int64_t top_k,
+                                   uint16_t *out) {
+    const int64_t K = Wd->k, O = Wd->n;
+    const int64_t xk = (Wshared && Wshared->k > K) ? Wshared->k : K;
+    float *xf = (float *)malloc(sizeof(float) * (size_t)xk);
+    float *dot = (float *)malloc(sizeof(float) * (size_t)O);
+    float *acc = (float *)malloc(sizeof(float) * (size_t)O);
+    for (int64_t t = 0; t < n_tokens; ++t) {
+        for (int64_t o = 0; o < O; ++o) acc[o] = 0.0f;
+        for (int64_t sl = 0; sl < top_k; ++sl) {
+            const int64_t r = t * top_k + sl;
+            int64_t e = expert_idx[r];
+            if (e > n_experts - 1) e = n_experts - 1;
+            const fko_weight d = expert_slice(Wd, e);
+            const int64_t row = row_idx ? (int64_t)row_idx[r] : r;
+            for (int64_t j = 0; j < K; ++j) xf[j] = bf16_to_f32(h[row * K + j]);
+            linear_acc(&d, xf, dot);
+            const float rw = route_weight ? bf16_to_f32(route_weight[r]) : 1.0f;
+            for (int64_t o = 0; o < O; ++o) {
+                const float partial = rw * rbf(dot[o]);
+                acc[o] += partial;
+            }
+        }
+        if (Wshared) { /* routed_qmv_reduce.rs:250-307: one more partial, T(dot) of the shared expert */
+            for (int64_t j = 0; j < Wshared->k; ++j) xf[j] = bf16_to_f32(shared_x[t * Wshared->k + j]);
+            linear_acc(Wshared, xf, dot);
+            for (int64_t o = 0; o < O; ++o) acc[o] += rbf(dot[o]);
+        }
+        for (int64_t o = 0; o < O; ++o) {
+            float a = acc[o];
+            if (residual_extra) a += bf16_to_f32(residual_extra[t * O + o]);
+            out[t * O + o] = f32_to_bf16(a);
+        }
+    }
+    free(xf); free(dot); free(acc);
+}
+
+/* G: multi-row quantised matmul y[M, N] = T(x[M, K] @ dequant(W)^T (+ bias)), the row-wise
+ *    repetition of K1 (qMM-T semantics, src/codegen/msl.rs:2318-2440: fp32 accumulate, one round). */
+FKO_API void fko_qgemm(const fko_weight *W, const uint16_t *x, int64_t m, const uint16_t *bias, uint16_t *y) {
+    for (int64_t r = 0; r < m; ++r) fko_qgemv(W, x + r * W->k, bias, y + r * W->n);
+}
+
 /* --------------------------------------------------- dense decoder step */
 /*
  * One decode step of the dense decoder in the reference's decode_pipeline

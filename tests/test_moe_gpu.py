@@ -1,0 +1,166 @@
+"""GPU parity of the mixture-of-experts routed projections (M1 gate/up + SwiGLU, M2 down +
+weighted reduction) against the CPU oracle, through the C ABI.
+
+Same bars as the dense GEMV family: rel-L2 <= 1e-2 against an fp32 reference, and
+element-wise equality with the oracle except for bf16 rounding-edge flips.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
+from test_gemv_gpu import FLIP_FRACTION_BAR, REL_L2_BAR, _check_swiglu
+
+pytestmark = pytest.mark.gpu
+
+
+def _stack(seed, n_experts, n, k, bits):
+    return oracle.StackedWeight([make_qweight(seed + e, n, k, bits) for e in range(n_experts)])
+
+
+def _dev(fk, a):
+    return None if a is None else fk.DeviceBuffer.from_numpy(np.ascontiguousarray(a))
+
+
+def _swiglu_fp32(x_row, Wg, Wu, rw):
+    g, u = oracle.linear_acc(Wg, x_row).astype(np.float64), oracle.linear_acc(Wu, x_row).astype(np.float64)
+    return g / (1 + np.exp(-g)) * u * rw
+
+
+def _run_m1(fk, x, Wg, Wu, row_idx, expert_idx, route_weight):
+    n_routes = expert_idx.size
+    out = fk.DeviceBuffer(2 * n_routes * Wg.n)
+    fk.routed_qmv_swiglu(_dev(fk, x), x.shape[0], to_device(fk, Wg), to_device(fk, Wu), Wg.n_experts,
+                         _dev(fk, row_idx), _dev(fk, expert_idx), _dev(fk, route_weight), n_routes, out)
+    return out.to_numpy(np.uint16, (n_routes, Wg.n))
+
+
+@pytest.mark.parametrize("bits", [4, 8, 16])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_routed_swiglu_one_token(fk, bits, weighted):
+    E, O, K, top_k = 8, 352, 512, 6          # O not a multiple of the tile rows
+    Wg, Wu = _stack(100, E, O, K, bits), _stack(200, E, O, K, bits)
+    x = normal_bf16(3, (1, K))
+    expert_idx = np.array([5, 0, 7, 2, 2, 6], np.uint32)   # an expert may be picked twice
+    row_idx = np.zeros(top_k, np.uint32)
+    rw = normal_bf16(4, top_k, 0.1, 0.3) if weighted else None
+    got = _run_m1(fk, x, Wg, Wu, row_idx, expert_idx, rw)
+    ref = oracle.routed_qmv_swiglu(x, Wg, Wu, row_idx, expert_idx, rw)
+    for r in range(top_k):
+        e = int(expert_idx[r])
+        scale = float(oracle.bf16_to_f32(rw[r:r + 1])[0]) if weighted else 1.0
+        assert rel_l2(got[r], _swiglu_fp32(x[0], Wg.expert(e), Wu.expert(e), scale)) <= REL_L2_BAR
+        if weighted:
+            frac, ulps = bf16_mismatch(got[r], ref[r])
+            assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (r, frac, ulps)
+        else:
+            _check_swiglu(got[r], ref[r], x[0], Wg.expert(e), Wu.expert(e), 1)
+
+
+def test_routed_swiglu_rows_and_clamp(fk):
+    """Several tokens with their own activation rows; expert and row indices beyond the range clamp."""
+    E, O, K, tokens, top_k = 4, 128, 256, 5, 2
+    Wg, Wu = _stack(300, E, O, K, 4), _stack(400, E, O, K, 4)
+    x = normal_bf16(5, (tokens, K))
+    expert_idx = rng(6).integers(0, E, tokens * top_k).astype(np.uint32)
+    expert_idx[3] = 1000                     # clamps to E - 1 (routed_qmv_swiglu.rs:138)
+    row_idx = np.repeat(np.arange(tokens, dtype=np.uint32), top_k)
+    got = _run_m1(fk, x, Wg, Wu, row_idx, expert_idx, None)
+    ref = oracle.routed_qmv_swiglu(x, Wg, Wu, row_idx, expert_idx, None)
+    for r in range(tokens * top_k):
+        e = min(int(expert_idx[r]), E - 1)
+        _check_swiglu(got[r], ref[r], x[row_idx[r]], Wg.expert(e), Wu.expert(e), 1)
+    # a row index past the end reads the last row instead of faulting
+    far = row_idx.copy()
+    far[-1] = 77
+    got2 = _run_m1(fk, x, Wg, Wu, far, expert_idx, None)
+    assert np.array_equal(got2[:-1], got[:-1])
+    assert np.array_equal(got2[-1], got[-1])  # the last route already read the last row
+
+
+def _run_m2(fk, h, Wd, row_idx, expert_idx, rw, shared_x, Ws, res, tokens, top_k):
+    out = fk.DeviceBuffer(2 * tokens * Wd.n)
+    ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, Wd.n))
+    fk.routed_qmv_reduce(_dev(fk, h), h.shape[0], to_device(fk, Wd), Wd.n_experts, _dev(fk, row_idx),
+                         _dev(fk, expert_idx), _dev(fk, rw), _dev(fk, shared_x),
+                         None if Ws is None else to_device(fk, Ws), _dev(fk, res), tokens, top_k, out, ws)
+    return out.to_numpy(np.uint16, (tokens, Wd.n))
+
+
+def _m2_fp32(h, Wd, expert_idx, rw, shared_x, Ws, res, tokens, top_k):
+    ref = np.zeros((tokens, Wd.n))
+    for t in range(tokens):
+        for s in range(top_k):
+            r = t * top_k + s
+            w = float(oracle.bf16_to_f32(rw[r:r + 1])[0]) if rw is not None else 1.0
+            ref[t] += w * oracle.linear_acc(Wd.expert(int(expert_idx[r])), h[r]).astype(np.float64)
+        if Ws is not None:
+            ref[t] += oracle.linear_acc(Ws, shared_x[t]).astype(np.float64)
+        if res is not None:
+            ref[t] += oracle.bf16_to_f32(res[t]).astype(np.float64)
+    return ref
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("preweighted", [False, True])
+@pytest.mark.parametrize("shared,residual", [(False, False), (False, True), (True, True)])
+def test_routed_reduce_one_token(fk, bits, preweighted, shared, residual):
+    E, O, K, top_k = 8, 320, 448, 6
+    Wd = _stack(500, E, O, K, bits)
+    h = normal_bf16(7, (top_k, K), 0.0, 0.5)
+    expert_idx = np.array([1, 4, 4, 0, 7, 3], np.uint32)
+    rw = None if preweighted else normal_bf16(8, top_k, 0.15, 0.2)
+    Ws = make_qweight(600, O, 256, bits) if shared else None
+    sx = normal_bf16(9, (1, 256)) if shared else None
+    res = normal_bf16(10, (1, O)) if residual else None
+    got = _run_m2(fk, h, Wd, None, expert_idx, rw, sx, Ws, res, 1, top_k)
+    ref = oracle.routed_qmv_reduce(h, Wd, expert_idx, rw, res, 1, top_k, shared_x=sx, Wshared=Ws)
+    assert rel_l2(got, _m2_fp32(h, Wd, expert_idx, rw, sx, Ws, res, 1, top_k)) <= REL_L2_BAR
+    frac, ulps = bf16_mismatch(got, ref)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+
+
+def test_routed_reduce_tokens_and_row_idx(fk):
+    E, O, K, tokens, top_k = 4, 192, 256, 3, 2
+    Wd = _stack(700, E, O, K, 4)
+    h = normal_bf16(11, (tokens * top_k, K), 0.0, 0.5)
+    expert_idx = rng(12).integers(0, E, tokens * top_k).astype(np.uint32)
+    row_idx = rng(13).permutation(tokens * top_k).astype(np.uint32)
+    rw = normal_bf16(14, tokens * top_k, 0.3, 0.2)
+    res = normal_bf16(15, (tokens, O))
+    got = _run_m2(fk, h, Wd, row_idx, expert_idx, rw, None, None, res, tokens, top_k)
+    ref = oracle.routed_qmv_reduce(h, Wd, expert_idx, rw, res, tokens, top_k, row_idx=row_idx)
+    frac, ulps = bf16_mismatch(got, ref)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+
+
+def test_moe_block_full_size(fk):
+    """Config-5 shapes (hidden 2048, expert width 1408, 6 of 16 experts, int4): M1 feeds M2."""
+    E, hidden, inter, top_k = 16, 2048, 1408, 6
+    Wg, Wu, Wd = _stack(800, E, inter, hidden, 4), _stack(900, E, inter, hidden, 4), _stack(1000, E, hidden, inter, 4)
+    x = normal_bf16(16, (1, hidden))
+    expert_idx = rng(17).permutation(E)[:top_k].astype(np.uint32)
+    row_idx = np.zeros(top_k, np.uint32)
+    rw = oracle.f32_to_bf16(np.full(top_k, 1.0 / top_k, np.float32))
+    res = normal_bf16(18, (1, hidden))
+    h = _run_m1(fk, x, Wg, Wu, row_idx, expert_idx, None)
+    h_ref = oracle.routed_qmv_swiglu(x, Wg, Wu, row_idx, expert_idx, None)
+    frac, ulps = bf16_mismatch(h, h_ref)
+    assert frac <= FLIP_FRACTION_BAR, frac
+    got = _run_m2(fk, h, Wd, None, expert_idx, rw, None, None, res, 1, top_k)   # on the GPU's own h
+    ref = oracle.routed_qmv_reduce(h, Wd, expert_idx, rw, res, 1, top_k)
+    frac, ulps = bf16_mismatch(got, ref)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+
+
+def test_routed_rejects_bad_arguments(fk):
+    Wg, Wu = _stack(1100, 2, 64, 128, 4), _stack(1200, 2, 64, 128, 4)
+    x = _dev(fk, normal_bf16(1, (1, 128)))
+    idx = _dev(fk, np.zeros(2, np.uint32))
+    out = fk.DeviceBuffer(2 * 2 * 64)
+    with pytest.raises(fk.InvalidArgument):
+        fk.routed_qmv_swiglu(x, 1, to_device(fk, Wg), to_device(fk, Wu), 2, idx, None, None, 2, out)
+    with pytest.raises(fk.InvalidArgument):
+        fk.routed_qmv_swiglu(x, 1, to_device(fk, Wg), to_device(fk, Wu), 0, idx, idx, None, 2, out)
+    with pytest.raises(fk.InvalidArgument):
+        fk.routed_qmv_reduce(x, 1, to_device(fk, Wg), 2, None, idx, None, x, None, None, 1, 2, out, out)
