@@ -256,6 +256,28 @@ fk_status fk_routed_qmv_reduce(const uint16_t* h, uint32_t n_h_rows, const fk_we
     return run_launch(reduce, (hipStream_t)s);
 }
 
+fk_status fk_qgemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, uint32_t group, size_t* bytes) {
+    if (!bytes) return set_error(FK_ERR_INVALID, "fk_qgemm_workspace_bytes: null output");
+    return qgemm_workspace_bytes(m, n, k, group, bytes);
+}
+
+fk_status fk_qgemm(const fk_weight* W, const uint16_t* x, uint32_t m, const uint16_t* bias, const uint16_t* residual,
+                   uint16_t* y, void* workspace, fk_stream s) {
+    Launch main, reduce;
+    FK_TRY(plan_qgemm(W, x, m, bias, residual, y, workspace, &main, &reduce));
+    FK_TRY(run_launch(main, (hipStream_t)s));
+    return run_launch(reduce, (hipStream_t)s);
+}
+
+fk_status fk_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16_t* x, uint32_t m, int variant,
+                          uint16_t* out, void* workspace, fk_stream s) {
+    Launch gate, up, reduce;
+    FK_TRY(plan_qgemm_swiglu(Wg, Wu, x, m, variant, out, workspace, &gate, &up, &reduce));
+    FK_TRY(run_launch(gate, (hipStream_t)s));
+    FK_TRY(run_launch(up, (hipStream_t)s));
+    return run_launch(reduce, (hipStream_t)s);
+}
+
 fk_status fk_final_rmsnorm_lm_head(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* W,
                                    uint16_t* logits, fk_stream s) {
     if (!norm_w) return set_error(FK_ERR_INVALID, "fk_final_rmsnorm_lm_head: null norm weight");

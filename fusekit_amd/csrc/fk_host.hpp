@@ -84,6 +84,13 @@ fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight,
                             uint16_t* out_ptr, uint32_t n_tokens, uint32_t top_k, uint32_t O, bool has_shared,
                             Launch* out);
 
+// Multi-row quantised matmul on the matrix cores (main kernel(s) + split-k reduction).
+fk_status qgemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group, size_t* bytes);
+fk_status plan_qgemm(const fk_weight* W, const uint16_t* x, uint32_t M, const uint16_t* bias, const uint16_t* res,
+                     uint16_t* y, void* workspace, Launch* main, Launch* reduce);
+fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16_t* x, uint32_t M, int variant,
+                            uint16_t* out, void* workspace, Launch* gate, Launch* up, Launch* reduce);
+
 // RoPE / per-head RMSNorm / KV-cache store (one wave per head).
 struct RopeArgs {
     uint16_t* q;             // [n_q, head_dim] in place, or null

@@ -198,6 +198,22 @@ def routed_qmv_reduce(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_wei
                                    _ptr(stream)))
 
 
+def qgemm_workspace_bytes(m, n, k, group=64) -> int:
+    out = C.c_size_t(0)
+    check(lib.fk_qgemm_workspace_bytes(C.c_uint32(m), C.c_uint32(n), C.c_uint32(k), C.c_uint32(group), C.byref(out)))
+    return int(out.value)
+
+
+def qgemm(W, x, m, bias, residual, y, workspace, stream=None) -> None:
+    check(lib.fk_qgemm(C.byref(W.c), _ptr(x), C.c_uint32(m), _ptr(bias), _ptr(residual), _ptr(y), _ptr(workspace),
+                       _ptr(stream)))
+
+
+def qgemm_swiglu(Wg, Wu, x, m, variant, out, workspace, stream=None) -> None:
+    check(lib.fk_qgemm_swiglu(C.byref(Wg.c), C.byref(Wu.c), _ptr(x), C.c_uint32(m), C.c_int(variant), _ptr(out),
+                              _ptr(workspace), _ptr(stream)))
+
+
 def final_rmsnorm_lm_head(x, norm_w, eps, W, logits, stream=None) -> None:
     check(lib.fk_final_rmsnorm_lm_head(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(W.c), _ptr(logits),
                                        _ptr(stream)))

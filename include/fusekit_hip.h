@@ -144,6 +144,22 @@ fk_status fk_routed_qmv_reduce(const uint16_t *h, uint32_t n_h_rows, const fk_we
                                const uint16_t *shared_x, const fk_weight *W_shared, const uint16_t *residual_extra,
                                uint32_t n_tokens, uint32_t top_k, uint16_t *out, void *workspace, fk_stream s);
 
+/* G   multi-row quantised matmul on the matrix cores: y[m, N] = T(x[m, K] @ dequant(W)^T
+ *     (+ bias[N]) (+ residual[m, N])), fp32 accumulate, one round.  Replaces the
+ *     reference's qMM-T / NAX tile path (src/codegen/msl.rs:2318-2440, 3821-4330;
+ *     admission src/codegen/kernels/mod.rs:1442-1475) and its small-M shared-stream
+ *     GEMVs (fusekit_qmv_wide_impl, src/codegen/msl.rs:461-546).  Any m >= 1; bits 4
+ *     or 8, group 64 or 128.  workspace: fk_qgemm_workspace_bytes() bytes of device
+ *     memory (fp32 split-k partial sums); the SwiGLU pair needs twice that.
+ *     fk_qgemm_swiglu: out[m, N] = SwiGLU(x @ Wg^T, x @ Wu^T) with the rounding variant
+ *     as in fk_gateup_swiglu (the reference's qMM epilogue is variant 2,
+ *     src/codegen/msl.rs:2441-2449). */
+fk_status fk_qgemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, uint32_t group, size_t *bytes);
+fk_status fk_qgemm(const fk_weight *W, const uint16_t *x, uint32_t m, const uint16_t *bias,
+                   const uint16_t *residual, uint16_t *y, void *workspace, fk_stream s);
+fk_status fk_qgemm_swiglu(const fk_weight *Wg, const fk_weight *Wu, const uint16_t *x, uint32_t m, int variant,
+                          uint16_t *out, void *workspace, fk_stream s);
+
 /* H   final RMSNorm + vocabulary GEMV, logits in T.  Replaces
  *     src/codegen/kernels/final_rmsnorm_lm_head.rs:144-629. */
 fk_status fk_final_rmsnorm_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *W,
