@@ -54,6 +54,7 @@ fk_status device_facts(const DeviceFacts** out) {
 fk_status run_launch(const Launch& l, hipStream_t s) {
     void* params[1] = {const_cast<unsigned char*>(l.args)};
     FK_HIP(hipLaunchKernel(l.func, l.grid, l.block, params, l.shmem, s));
+    for (const Launch& f : l.then) FK_TRY(run_launch(f, s));
     return FK_OK;
 }
 

@@ -163,15 +163,21 @@ __global__ __launch_bounds__(256) void argmax_kernel(const ArgmaxArgs a) {
         return r;
     };
     best = block_best(best);
-    if (threadIdx.x == 0) a.partial[blockIdx.x] = best;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) is_last = (atomicAdd(a.counter, 1u) == gridDim.x - 1) ? 1u : 0u;
+    // The candidate is stored write-through (agent scope) and its arrival awaited
+    // before the block counts itself in; the last block reads the candidates past
+    // the caches.  No device-wide fence (which would write back a whole L2).
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&a.partial[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        wait_memory_ops_done();
+        is_last = (atomicAdd(a.counter, 1u) == gridDim.x - 1) ? 1u : 0u;
+    }
     __syncthreads();
     if (!is_last) return;
-    __threadfence();
     uint64_t fin = 0;
-    for (uint32_t i = threadIdx.x; i < gridDim.x; i += 256) fin = a.partial[i] > fin ? a.partial[i] : fin;
+    for (uint32_t i = threadIdx.x; i < gridDim.x; i += 256) {
+        const uint64_t c = __hip_atomic_load(&a.partial[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        fin = c > fin ? c : fin;
+    }
     fin = block_best(fin);
     if (threadIdx.x == 0) {
         // all-NaN / empty rows fall back to index 0 like the reference's initial local_idx
@@ -182,7 +188,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(const ArgmaxArgs a) {
             if (slot < a.hist_capacity) a.history[slot] = tok;
             *a.hist_counter = slot + 1;
         }
-        *a.counter = 0u;
+        __hip_atomic_store(a.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 

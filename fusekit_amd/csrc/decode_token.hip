@@ -33,7 +33,7 @@ __device__ __forceinline__ const ConstSdpaArgs& sdpa_args(const SdpaArgs* base, 
 // (30 us for 1024 blocks); instead every byte that crosses blocks inside this
 // kernel moves through agent-scope accesses (ld_u16 / st_u16 and friends), so a
 // barrier only has to (1) wait until this block's stores have completed
-// (workgroup-scope release), (2) count arrivals on two levels of counters -- one
+// (every wave waits for its own memory counter, then the block barrier), (2) count arrivals on two levels of counters -- one
 // per group of kBarFan blocks, then one for the groups, so no address sees more
 // than kBarFan atomics -- and (3) let the last arriver publish the epoch in a flag
 // the others poll.  All counters are monotonic across launches.
@@ -47,7 +47,7 @@ struct BarrierState {
 };
 
 __device__ __forceinline__ void grid_barrier(const TokenArgs& t, BarrierState& b) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    wait_memory_ops_done();  // this wave's write-through stores have landed
     __syncthreads();
     if (threadIdx.x == 0) {
         bool released = false;

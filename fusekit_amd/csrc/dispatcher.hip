@@ -411,6 +411,146 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
                             capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l);
 }
 
+// x, gate_w, gate_s, gate_b, up_w, up_s, up_b, row_idx, expert_idx, [route_weight], out0
+// (routed_qmv_swiglu.rs:99-112).  Parameters: k, o, experts, routes, x_rows, pre_scale.
+fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("k"), O = d.u("o");
+    const uint32_t experts = d.u("experts"), routes = d.u("routes"), x_rows = d.u("x_rows", 1);
+    const bool pre_scale = d.u("pre_scale", 0) != 0;
+    const size_t n_slots = pre_scale ? 11 : 10;
+    FK_TRY(need_args(d, n_slots));
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
+    if (experts == 0 || routes == 0 || K == 0 || O == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": k / o / experts / routes parameters missing");
+    fk_weight Wg, Wu;
+    FK_TRY(bind_weight(d, bits, group, O * experts, K, 1, 2, 3, &Wg));
+    FK_TRY(bind_weight(d, bits, group, O * experts, K, 4, 5, 6, &Wu));
+    Wg.n = Wu.n = O;
+    FK_TRY(need_bytes(d, 0, (size_t)x_rows * K * 2));
+    FK_TRY(need_bytes(d, 7, (size_t)routes * 4));
+    FK_TRY(need_bytes(d, 8, (size_t)routes * 4));
+    if (pre_scale) FK_TRY(need_bytes(d, 9, (size_t)routes * 2));
+    FK_TRY(need_bytes(d, n_slots - 1, (size_t)routes * O * 2));
+    all_but_last(n_slots, 1, rw);
+    return plan_routed_gemv(arg_ptr<const uint16_t>(d, 0), x_rows, &Wg, &Wu, experts, arg_ptr<const uint32_t>(d, 7),
+                            arg_ptr<const uint32_t>(d, 8), pre_scale ? arg_ptr<const uint16_t>(d, 9) : nullptr, routes,
+                            arg_ptr<uint16_t>(d, n_slots - 1), l);
+}
+
+// x, wq, scales, biases, row_idx, expert_idx, [route_weight], [shared_x, shared_w, shared_s, shared_b],
+// [residual_extra], out0, workspace   (routed_qmv_reduce.rs:110-145; the workspace slot is this
+// library's: per-route results before the ordered sum).  Parameters: k, o, experts, tokens, top_k,
+// x_rows, input_preweighted, has_shared, shared_k, has_extra.
+fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("k"), O = d.u("o");
+    const uint32_t experts = d.u("experts"), tokens = d.u("tokens", 1), top_k = d.u("top_k");
+    const bool preweighted = d.u("input_preweighted", 0) != 0, has_shared = d.u("has_shared", 0) != 0;
+    const bool has_extra = d.u("has_extra", 0) != 0;
+    const uint32_t shared_k = d.u("shared_k", K), routes = tokens * top_k, x_rows = d.u("x_rows", routes);
+    size_t s = 6;
+    const size_t rw_slot = preweighted ? 0 : s++;
+    const size_t shared_slot = s;
+    if (has_shared) s += 4;
+    const size_t extra_slot = has_extra ? s++ : 0;
+    const size_t out_slot = s++, ws_slot = s++;
+    FK_TRY(need_args(d, s));
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
+    if (experts == 0 || routes == 0 || K == 0 || O == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": k / o / experts / top_k parameters missing");
+    if (has_shared && tokens != 1) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": shared expert needs one token");
+    fk_weight Wd, Ws;
+    FK_TRY(bind_weight(d, bits, group, O * experts, K, 1, 2, 3, &Wd));
+    Wd.n = O;
+    FK_TRY(need_bytes(d, 0, (size_t)x_rows * K * 2));
+    FK_TRY(need_bytes(d, 4, (size_t)routes * 4));
+    FK_TRY(need_bytes(d, 5, (size_t)routes * 4));
+    if (!preweighted) FK_TRY(need_bytes(d, rw_slot, (size_t)routes * 2));
+    if (has_shared) {
+        FK_TRY(bind_weight(d, bits, group, O, shared_k, shared_slot + 1, shared_slot + 2, shared_slot + 3, &Ws));
+        FK_TRY(need_bytes(d, shared_slot, (size_t)shared_k * 2));
+    }
+    if (has_extra) FK_TRY(need_bytes(d, extra_slot, (size_t)tokens * O * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)tokens * O * 2));
+    FK_TRY(need_bytes(d, ws_slot, ((size_t)routes + tokens) * O * 2));
+    for (uint32_t i = 0; i < out_slot; ++i) rw->reads.push_back(i);
+    rw->reads.push_back((uint32_t)ws_slot);
+    rw->writes = {(uint32_t)out_slot, (uint32_t)ws_slot};
+
+    uint16_t* parts = arg_ptr<uint16_t>(d, ws_slot);
+    FK_TRY(plan_routed_gemv(arg_ptr<const uint16_t>(d, 0), x_rows, &Wd, nullptr, experts, arg_ptr<const uint32_t>(d, 4),
+                            arg_ptr<const uint32_t>(d, 5), nullptr, routes, parts, l));
+    if (has_shared) {
+        GemvRequest rq;
+        rq.mats[0] = &Ws;
+        rq.y[0] = parts + (size_t)routes * O;
+        rq.x = arg_ptr<const uint16_t>(d, shared_slot);
+        Launch shared;
+        FK_TRY(plan_gemv(rq, &shared));
+        l->then.push_back(shared);
+    }
+    Launch reduce;
+    FK_TRY(plan_route_reduce(parts, preweighted ? nullptr : arg_ptr<const uint16_t>(d, rw_slot),
+                             has_extra ? arg_ptr<const uint16_t>(d, extra_slot) : nullptr, arg_ptr<uint16_t>(d, out_slot),
+                             tokens, top_k, O, has_shared, &reduce));
+    l->then.push_back(reduce);
+    return FK_OK;
+}
+
+// x, W, scales, biases, [bias], [residual], y, workspace.  Parameters: m (= K), n, rows, has_bias, has_residual.
+fk_status plan_qgemm_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("m"), N = d.u("n"), rows = d.u("rows");
+    const bool has_bias = d.u("has_bias", 0) != 0, has_res = d.u("has_residual", 0) != 0;
+    size_t s = 4;
+    const size_t bias_slot = has_bias ? s++ : 0, res_slot = has_res ? s++ : 0;
+    const size_t out_slot = s++, ws_slot = s++;
+    FK_TRY(need_args(d, s));
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
+    if (rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows parameter missing");
+    fk_weight W;
+    FK_TRY(bind_weight(d, bits, group, N, K, 1, 2, 3, &W));
+    FK_TRY(need_bytes(d, 0, (size_t)rows * K * 2));
+    if (has_bias) FK_TRY(need_bytes(d, bias_slot, (size_t)N * 2));
+    if (has_res) FK_TRY(need_bytes(d, res_slot, (size_t)rows * N * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)rows * N * 2));
+    size_t ws = 0;
+    FK_TRY(qgemm_workspace_bytes(rows, N, K, group, &ws));
+    FK_TRY(need_bytes(d, ws_slot, ws));
+    for (uint32_t i = 0; i < out_slot; ++i) rw->reads.push_back(i);
+    rw->reads.push_back((uint32_t)ws_slot);
+    rw->writes = {(uint32_t)out_slot, (uint32_t)ws_slot};
+    Launch reduce;
+    FK_TRY(plan_qgemm(&W, arg_ptr<const uint16_t>(d, 0), rows, has_bias ? arg_ptr<const uint16_t>(d, bias_slot) : nullptr,
+                      has_res ? arg_ptr<const uint16_t>(d, res_slot) : nullptr, arg_ptr<uint16_t>(d, out_slot),
+                      d.args[ws_slot].ptr, l, &reduce));
+    l->then.push_back(reduce);
+    return FK_OK;
+}
+
+// x, W_gate, W_up, s_g, s_u, b_g, b_u, out, workspace.  Parameters: hidden, inter, rows, variant.
+fk_status plan_qgemm_swiglu_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), hidden = d.u("hidden"), inter = d.u("inter");
+    const uint32_t rows = d.u("rows");
+    FK_TRY(need_args(d, 9));
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
+    if (rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows parameter missing");
+    fk_weight Wg, Wu;
+    FK_TRY(bind_weight(d, bits, group, inter, hidden, 1, 3, 5, &Wg));
+    FK_TRY(bind_weight(d, bits, group, inter, hidden, 2, 4, 6, &Wu));
+    FK_TRY(need_bytes(d, 0, (size_t)rows * hidden * 2));
+    FK_TRY(need_bytes(d, 7, (size_t)rows * inter * 2));
+    size_t ws = 0;
+    FK_TRY(qgemm_workspace_bytes(rows, inter, hidden, group, &ws));
+    FK_TRY(need_bytes(d, 8, 2 * ws));
+    rw->reads = {0, 1, 2, 3, 4, 5, 6, 8};
+    rw->writes = {7, 8};
+    Launch up, reduce;
+    FK_TRY(plan_qgemm_swiglu(&Wg, &Wu, arg_ptr<const uint16_t>(d, 0), rows, (int)d.param("variant", 2),
+                             arg_ptr<uint16_t>(d, 7), d.args[8].ptr, l, &up, &reduce));
+    l->then.push_back(up);
+    l->then.push_back(reduce);
+    return FK_OK;
+}
+
 // logits, next_tok, workspace, [history, hist_counter]
 fk_status plan_argmax_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const bool hist = d.args.size() == 5;
@@ -450,6 +590,10 @@ const Family kFamilies[] = {
     {"fusekit_linear_residual", plan_linres},
     {"fusekit_final_rmsnorm_lm_head", plan_lm_head},
     {"fusekit_qgemv", plan_qgemv_d},
+    {"fusekit_qgemm", plan_qgemm_d},
+    {"fusekit_qgemm_swiglu", plan_qgemm_swiglu_d},
+    {"fusekit_routed_qmv_swiglu", plan_routed_swiglu},
+    {"fusekit_routed_qmv_reduce", plan_routed_reduce},
     {"fusekit_rmsnorm_rope_q_decode",
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_q(d, l, rw, true); }},
     {"fusekit_rmsnorm_rope_kv_cache_store_decode",
@@ -482,6 +626,7 @@ fk_status plan_dispatch(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (!f) return set_error(FK_ERR_INVALID, "kernel '" + d.kernel + "' is not in this library");  // lib.rs:412-415
     rw->reads.clear();
     rw->writes.clear();
+    l->then.clear();
     return f->plan(d, l, rw);
 }
 
@@ -509,7 +654,9 @@ struct Node {
     Launch launch;
     SlotRW rw;
     hipGraphNode_t node = nullptr;
+    std::vector<hipGraphNode_t> tail;  // nodes of launch.then, chained behind `node`
     std::vector<uint32_t> deps;
+    hipGraphNode_t last() const { return tail.empty() ? node : tail.back(); }
 };
 
 struct Graph {
@@ -552,18 +699,19 @@ fk_status get_graph(DispatcherState* ds, uint32_t id, Graph** out) {
     return FK_OK;
 }
 
-hipKernelNodeParams node_params(Node& n, void** slot) {
+hipKernelNodeParams launch_params(Launch& l, void** slot) {
     hipKernelNodeParams p;
     memset(&p, 0, sizeof(p));
-    p.func = const_cast<void*>(n.launch.func);
-    p.gridDim = n.launch.grid;
-    p.blockDim = n.launch.block;
-    p.sharedMemBytes = n.launch.shmem;
-    *slot = n.launch.args;
+    p.func = const_cast<void*>(l.func);
+    p.gridDim = l.grid;
+    p.blockDim = l.block;
+    p.sharedMemBytes = l.shmem;
+    *slot = l.args;
     p.kernelParams = slot;
     p.extra = nullptr;
     return p;
 }
+hipKernelNodeParams node_params(Node& n, void** slot) { return launch_params(n.launch, slot); }
 
 // RAW / WAW / WAR edges on overlapping byte ranges, transitively reduced.
 void derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
@@ -766,6 +914,7 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
         // partials and counters live in the private arena, sized for that
         s.chunk_len = sdpa_chunk_len(s.qk_dim, s.v_dim, true);
         s.n_splits = (s.capacity + s.chunk_len - 1) / s.chunk_len;
+        s.chunks_per_block = 1;
         s.k_new = r1.k;
         s.v_new = r1.v;
         s.q_norm = r0.q_norm;
@@ -1004,10 +1153,16 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
     for (size_t i = 0; i < n; ++i) {
         Node& nd = g->nodes[i];
         std::vector<hipGraphNode_t> deps;
-        for (uint32_t j : nd.deps) deps.push_back(g->nodes[j].node);
+        for (uint32_t j : nd.deps) deps.push_back(g->nodes[j].last());
         void* slot = nullptr;
         hipKernelNodeParams p = node_params(nd, &slot);
         FK_HIP(hipGraphAddKernelNode(&nd.node, g->graph, deps.data(), deps.size(), &p));
+        nd.tail.resize(nd.launch.then.size());
+        for (size_t f = 0; f < nd.launch.then.size(); ++f) {
+            hipGraphNode_t prev = f ? nd.tail[f - 1] : nd.node;
+            hipKernelNodeParams fp = launch_params(nd.launch.then[f], &slot);
+            FK_HIP(hipGraphAddKernelNode(&nd.tail[f], g->graph, &prev, 1, &fp));
+        }
     }
     FK_HIP(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
     ds->graphs.push_back(std::move(g));
@@ -1136,11 +1291,17 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
     }
     for (size_t k = 0; k < touched.size(); ++k) {
         Node& nd = g->nodes[touched[k]];
+        if (launches[k].then.size() != nd.tail.size())
+            return set_error(FK_ERR_UNSUPPORTED, "binding update changes the number of kernels of a task");
         nd.d = patched[k];
         nd.launch = launches[k];
         void* slot = nullptr;
         hipKernelNodeParams p = node_params(nd, &slot);
         FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.node, &p));
+        for (size_t f = 0; f < nd.tail.size(); ++f) {
+            hipKernelNodeParams fp = launch_params(nd.launch.then[f], &slot);
+            FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.tail[f], &fp));
+        }
     }
     return FK_OK;
 }

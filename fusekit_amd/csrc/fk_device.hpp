@@ -77,6 +77,13 @@ __device__ __forceinline__ void st_f32(float* p, float v) {
         *p = v;
 }
 
+// Blocks until every global store and load this wave has issued is complete
+// (s_waitcnt vmcnt(0) lgkmcnt(0)).  With write-through (agent-scope) stores this is
+// the whole "release" a block needs before it signals other blocks through an
+// atomic counter: a workgroup-scope fence compiles to no wait at all on this part,
+// and an agent-scope fence adds a write-back of the whole L2.
+__device__ __forceinline__ void wait_memory_ops_done() { __builtin_amdgcn_s_waitcnt(0x0070); }
+
 // v + (v of the lane selected by a DPP control): cross-lane adds inside a row of
 // 16 lanes without going through the LDS crossbar.
 template <int CTRL>

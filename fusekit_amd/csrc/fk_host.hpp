@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <string>
+#include <vector>
 
 #include "../../include/fusekit_hip.h"
 
@@ -18,6 +19,10 @@ struct Launch {
     uint32_t shmem = 0;
     size_t args_size = 0;
     alignas(16) unsigned char args[640];
+    // Kernels that complete the same operation and must run after this one, in
+    // order (a split-k reduction, a routed reduction).  run_launch and the graph
+    // builder treat the chain as one unit.
+    std::vector<Launch> then;
 
     template <typename T>
     void set_args(const T& a) {

@@ -63,11 +63,19 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     if (!kv_len_ptr && (kv_len_imm == 0 || kv_len_imm > max_len))
         return set_error(FK_ERR_INVALID, "sdpa: kv_len outside (0, max_len]");
     const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim, false);
-    const uint32_t n_splits = (max_len + chunk - 1) / chunk;
-    if (n_splits > 1 && (!partials || !counters))
-        return set_error(FK_ERR_INVALID, "sdpa: workspace required when the context spans several ranges");
+    const uint32_t n_chunks = (max_len + chunk - 1) / chunk;
     const uint32_t G = n_heads / n_kv;
     const int gt = G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1));
+    // Long contexts: a block walks several consecutive ranges (online softmax), so
+    // that about two blocks per CU exist and the final merge adds at most 256 partials.
+    const uint32_t tiles = n_kv * ((G + gt - 1) / gt);
+    uint32_t want = 2u * (uint32_t)dev->cus / tiles;
+    if (want < 1) want = 1;
+    if (want > 256) want = 256;
+    const uint32_t cpb = (n_chunks + want - 1) / want;
+    const uint32_t n_splits = (n_chunks + cpb - 1) / cpb;
+    if (n_splits > 1 && (!partials || !counters))
+        return set_error(FK_ERR_INVALID, "sdpa: workspace required when the context spans several ranges");
 
     SdpaArgs a;
     memset(&a, 0, sizeof(a));
@@ -77,6 +85,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     a.n_heads = n_heads; a.n_kv = n_kv; a.qk_dim = qk_dim; a.v_dim = v_dim; a.capacity = capacity;
     a.chunk_len = chunk;
     a.n_splits = n_splits;
+    a.chunks_per_block = cpb;
     a.lpk = pow2_ceil(qk_dim / 8);
     a.lpv = pow2_ceil(v_dim / 8);
     a.scale = scale;

@@ -20,6 +20,7 @@ struct SdpaArgs {
     uint32_t kv_len_imm;
     uint32_t n_heads, n_kv, qk_dim, v_dim, capacity;
     uint32_t chunk_len, n_splits;
+    uint32_t chunks_per_block;  // consecutive ranges one block walks (online softmax across them)
     uint32_t lpk, lpv;  // lanes per key row / value row (powers of two)
     float scale;
     float* partials;     // [n_heads][n_splits][v_dim + 2]
@@ -40,7 +41,7 @@ struct SdpaArgs {
     const float* rope_tab;  // (cos, sin) per pair at this token's position, or null
 };
 
-// m[GT] and l[GT] (GT <= 8), the last-block flag and block-reduction scratch.
+// m[GT] at 0, l[GT] at 8 (GT <= 8), the last-block flag at 16, the per-range rescale factors at 24.
 constexpr uint32_t kSdpaStatFloats = 32;
 
 // LDS floats one block needs.
@@ -54,14 +55,16 @@ template <int GT, bool FUSED, typename ARGS>
 __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
                                            uint32_t gz, uint32_t gz_count, float* lds) {
     constexpr int kSteps = FUSED ? kSdpaStepsFused : kSdpaSteps;
-    const uint32_t n_active = (kv_len + a.chunk_len - 1) / a.chunk_len;
+    const uint32_t span = a.chunk_len * a.chunks_per_block;  // cache positions per block
+    const uint32_t n_active = (kv_len + span - 1) / span;
     if (split >= n_active) return;  // uniform: whole block leaves before any barrier
 
     const uint32_t G = a.n_heads / a.n_kv;
     const uint32_t h0 = kvh * G + gz * GT;
     const uint32_t gcount = (G - gz * GT) < (uint32_t)GT ? (G - gz * GT) : (uint32_t)GT;
-    const uint32_t key0 = split * a.chunk_len;
-    const uint32_t nkeys = (kv_len - key0) < a.chunk_len ? (kv_len - key0) : a.chunk_len;
+    const uint32_t blk0 = split * span;
+    const uint32_t blk_keys = (kv_len - blk0) < span ? (kv_len - blk0) : span;
+    const uint32_t n_chunks = (blk_keys + a.chunk_len - 1) / a.chunk_len;
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
 
     float* s = lds;                               // [GT][chunk_len]
@@ -70,15 +73,14 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     uint16_t* qn = reinterpret_cast<uint16_t*>(stat + kSdpaStatFloats);  // fused: [GT][qk_dim] + k row
     uint16_t* kn = qn + GT * a.qk_dim;
     const uint32_t pos = kv_len - 1;  // fused: position of the new token
-    const bool owner = FUSED && pos >= key0 && pos < key0 + nkeys;
-    const uint32_t jpos = pos - key0;
+    const bool blk_owner = FUSED && pos >= blk0 && pos < blk0 + blk_keys;
 
     if constexpr (FUSED) {
         // head norm + RoPE of this block's q heads (one wave per head), and of the new
         // k row in the block that owns its position; results in LDS as bf16.  Done
         // before the K/V loads are issued: the trigonometry needs ~60 registers that
         // the 64 registers of in-flight rows would otherwise have to share
-        for (uint32_t h = wave; h < gcount + (owner ? 1u : 0u); h += kSdpaWaves) {
+        for (uint32_t h = wave; h < gcount + (blk_owner ? 1u : 0u); h += kSdpaWaves) {
             if (h < gcount) {
                 head_transform(a.q + (size_t)(h0 + h) * a.qk_dim, qn + h * a.qk_dim, a.q_norm, a.qk_dim, a.rope_dims,
                                pos, a.base_log2, a.eps, true, lane, a.rope_tab);
@@ -88,7 +90,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
         }
         __syncthreads();
-        if (owner && gz == 0) {  // one block per kv head appends the new rows to the cache
+        if (blk_owner && gz == 0) {  // one block per kv head appends the new rows to the cache
             const size_t row = (size_t)kvh * a.capacity + (pos % a.capacity);
             for (uint32_t d = tid; d < a.qk_dim; d += kSdpaBlock) a.cache_k_w[row * a.qk_dim + d] = kn[d];
             for (uint32_t d = tid; d < a.v_dim; d += kSdpaBlock)
@@ -96,13 +98,31 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
     }
 
-    // All K and V loads of the range are issued up front (the range is sized so that
-    // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
     const uint32_t lpk = a.lpk, cpk = a.qk_dim >> 3;
     const uint32_t lpv = a.lpv, cpv = a.v_dim >> 3;
     const uint32_t ck = tid & (lpk - 1), kslot = tid / lpk, kslots = kSdpaBlock / lpk;
     const uint32_t cv = tid & (lpv - 1), vslot = tid / lpv, vslots = kSdpaBlock / lpv;
     const bool kcol_ok = ck < cpk, vcol_ok = cv < cpv;
+
+    // Running softmax state per head (m, l) in LDS; the value accumulators stay in
+    // registers across ranges: a lane owns the same 8 output dims in every range.
+    if (tid < (uint32_t)GT) {
+        stat[tid] = -INFINITY;
+        stat[8 + tid] = 0.f;
+    }
+    float acc[GT][8];
+#pragma unroll
+    for (int h = 0; h < GT; ++h)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+
+    for (uint32_t c = 0; c < n_chunks; ++c) {
+    const uint32_t key0 = blk0 + c * a.chunk_len;
+    const uint32_t nkeys = (kv_len - key0) < a.chunk_len ? (kv_len - key0) : a.chunk_len;
+    const bool owner = FUSED && pos >= key0 && pos < key0 + nkeys;
+    const uint32_t jpos = pos - key0;
+    // All K and V loads of the range are issued up front (the range is sized so that
+    // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
     uint4 kc[kSteps], vc[kSteps];
     {
         const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * ck;
@@ -167,9 +187,12 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     __syncthreads();
 
     // ---------------- softmax over this range, one wave per head ----------------
+    // Online form: the running maximum may rise, in which case what was summed so
+    // far is rescaled by alpha = exp(m_old - m_new) (0 for the first range).
     for (uint32_t h = wave; h < gcount; h += kSdpaWaves) {
         float* sh = s + h * a.chunk_len;
-        float m = -INFINITY;
+        const float m_old = stat[h], l_old = stat[8 + h];
+        float m = m_old;
         for (uint32_t j = lane; j < nkeys; j += kWave) m = fmaxf(m, sh[j]);
         m = wave_max(m);
         float l = 0.f;
@@ -180,33 +203,41 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
         l = wave_sum(l);
         if (lane == 0) {
+            const float alpha = c ? expf(m_old - m) : 0.f;
             stat[h] = m;
-            stat[GT + h] = l;
+            stat[8 + h] = c ? fmaf(l_old, alpha, l) : l;
+            stat[24 + h] = alpha;
         }
     }
     __syncthreads();
 
     // ---------------- phase B: o = sum_j p_j v_j ----------------
-    {
-        float acc[GT][8];
+    if (c) {
 #pragma unroll
-        for (int h = 0; h < GT; ++h)
+        for (int h = 0; h < GT; ++h) {
+            const float alpha = stat[24 + h];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
-#pragma unroll
-        for (int u = 0; u < kSteps; ++u) {
-            const uint32_t j = vslot + u * vslots;
-            const uint32_t jj = j < nkeys ? j : 0u;
-            const float live = j < nkeys ? 1.f : 0.f;
-            const float f[8] = {bf16_lo(vc[u].x), bf16_hi(vc[u].x), bf16_lo(vc[u].y), bf16_hi(vc[u].y),
-                                bf16_lo(vc[u].z), bf16_hi(vc[u].z), bf16_lo(vc[u].w), bf16_hi(vc[u].w)};
-#pragma unroll
-            for (int h = 0; h < GT; ++h) {
-                const float p = s[h * a.chunk_len + jj] * live;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
-            }
+            for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
         }
+    }
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+        const uint32_t j = vslot + u * vslots;
+        const uint32_t jj = j < nkeys ? j : 0u;
+        const float live = j < nkeys ? 1.f : 0.f;
+        const float f[8] = {bf16_lo(vc[u].x), bf16_hi(vc[u].x), bf16_lo(vc[u].y), bf16_hi(vc[u].y),
+                            bf16_lo(vc[u].z), bf16_hi(vc[u].z), bf16_lo(vc[u].w), bf16_hi(vc[u].w)};
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            const float p = s[h * a.chunk_len + jj] * live;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
+        }
+    }
+    if (c + 1 < n_chunks) __syncthreads();  // the scores are overwritten by the next range
+    }  // ranges of this block
+
+    {
         // add the key slots that share this lane's column: first inside the wave ...
 #pragma unroll
         for (int h = 0; h < GT; ++h)
@@ -234,25 +265,24 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 #pragma unroll
         for (int w = 0; w < kSdpaWaves; ++w) o += red[(w * GT + h) * a.v_dim + d];
         if (direct) {
-            st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o / stat[GT + h]));
+            st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o / stat[8 + h]));
         } else {
             float* p = a.partials + ((size_t)(h0 + h) * a.n_splits + split) * (a.v_dim + 2);
-            st_f32<FUSED>(p + 2 + d, o);
+            st_f32<true>(p + 2 + d, o);
             if (d == 0) {
-                st_f32<FUSED>(p, stat[h]);
-                st_f32<FUSED>(p + 1, stat[GT + h]);
+                st_f32<true>(p, stat[h]);
+                st_f32<true>(p + 1, stat[8 + h]);
             }
         }
     }
     if (direct) return;
 
     // ---------------- last block merges the partials ----------------
-    // (inside the persistent kernel the partials travel through agent-scope accesses,
-    // so waiting for the stores to complete replaces the device-wide fences)
-    if constexpr (FUSED)
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    else
-        __threadfence();
+    // Partials and the arrival counter move through agent-scope (write-through /
+    // cache-bypassing) accesses, so no device-wide fence is needed: every wave waits
+    // until its own stores have landed, the block barrier collects the waves, then one
+    // thread counts the block in.
+    wait_memory_ops_done();
     __syncthreads();
     uint32_t* flag = reinterpret_cast<uint32_t*>(stat + 16);
     if (tid == 0) {
@@ -261,32 +291,56 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }
     __syncthreads();
     if (*flag == 0u) return;
-    if constexpr (!FUSED) __threadfence();
     if (tid == 0)  // ready for the next launch (or the next layer of this one)
         __hip_atomic_store(&a.counters[kvh * gz_count + gz], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-    // weights w_s = exp(m_s - M) / L per head, held in LDS (reuses the score area
-    // when the range count fits, else loops in pieces of chunk_len)
-    for (uint32_t h = 0; h < gcount; ++h) {
-        const float* ph = a.partials + (size_t)(h0 + h) * a.n_splits * (a.v_dim + 2);
+    // One wave per head, no block barriers: M = max m_s, w_s = exp(m_s - M) (kept in
+    // registers, lane s % 64 slot s / 64, for up to 256 ranges), L = sum l_s w_s, then
+    // each lane adds its output dims over the ranges in index order.
+    constexpr uint32_t kWSlots = 4;
+    const uint32_t row = a.v_dim + 2;
+    for (uint32_t h = wave; h < gcount; h += kSdpaWaves) {
+        const float* ph = a.partials + (size_t)(h0 + h) * a.n_splits * row;
         float m = -INFINITY;
-        for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) m = fmaxf(m, ld_f32<FUSED>(ph + (size_t)sp * (a.v_dim + 2)));
-        m = block_max<kSdpaBlock>(m, stat + 20);
+        for (uint32_t sp = lane; sp < n_active; sp += kWave) m = fmaxf(m, ld_f32<true>(ph + (size_t)sp * row));
+        m = wave_max(m);
+        float wreg[kWSlots];
         float l = 0.f;
-        for (uint32_t sp = tid; sp < n_active; sp += kSdpaBlock) {
-            const float* p = ph + (size_t)sp * (a.v_dim + 2);
-            l += ld_f32<FUSED>(p + 1) * expf(ld_f32<FUSED>(p) - m);
-        }
-        l = block_sum<kSdpaBlock>(l, stat + 20);
-        const float inv_l = 1.0f / l;
-        // each thread owns output dims; ranges are added in index order
-        for (uint32_t d = tid; d < a.v_dim; d += kSdpaBlock) {
-            float o = 0.f;
-            for (uint32_t sp = 0; sp < n_active; ++sp) {
-                const float* p = ph + (size_t)sp * (a.v_dim + 2);
-                o = fmaf(ld_f32<FUSED>(p + 2 + d), expf(ld_f32<FUSED>(p) - m), o);
+#pragma unroll
+        for (uint32_t i = 0; i < kWSlots; ++i) {
+            const uint32_t sp = lane + i * kWave;
+            wreg[i] = 0.f;
+            if (sp < n_active) {
+                wreg[i] = expf(ld_f32<true>(ph + (size_t)sp * row) - m);
+                l = fmaf(ld_f32<true>(ph + (size_t)sp * row + 1), wreg[i], l);
             }
-            st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o * inv_l));
+        }
+        for (uint32_t sp = lane + kWSlots * kWave; sp < n_active; sp += kWave)
+            l = fmaf(ld_f32<true>(ph + (size_t)sp * row + 1), expf(ld_f32<true>(ph + (size_t)sp * row) - m), l);
+        l = wave_sum(l);
+        const float inv_l = 1.0f / l;
+        for (uint32_t d2 = lane; d2 < (a.v_dim >> 1); d2 += kWave) {
+            const float* pd = ph + 2 + 2 * d2;
+            float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+            for (uint32_t i = 0; i < kWSlots; ++i) {
+                const uint32_t lim = n_active > i * kWave ? (n_active - i * kWave < (uint32_t)kWave ? n_active - i * kWave : (uint32_t)kWave) : 0u;
+#pragma unroll 8
+                for (uint32_t lo = 0; lo < lim; ++lo) {
+                    const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wreg[i]), (int)lo));
+                    const float* p = pd + (size_t)(i * kWave + lo) * row;
+                    o0 = fmaf(ld_f32<true>(p), w, o0);
+                    o1 = fmaf(ld_f32<true>(p + 1), w, o1);
+                }
+            }
+            for (uint32_t sp = kWSlots * kWave; sp < n_active; ++sp) {
+                const float w = expf(ld_f32<true>(ph + (size_t)sp * row) - m);
+                o0 = fmaf(ld_f32<true>(pd + (size_t)sp * row), w, o0);
+                o1 = fmaf(ld_f32<true>(pd + (size_t)sp * row + 1), w, o1);
+            }
+            uint16_t* dst = a.out + (size_t)(h0 + h) * a.v_dim + 2 * d2;
+            st_u16<FUSED>(dst, f32_to_bf16_bits(o0 * inv_l));
+            st_u16<FUSED>(dst + 1, f32_to_bf16_bits(o1 * inv_l));
         }
     }
 }

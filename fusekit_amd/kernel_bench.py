@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Per-kernel measurements of the decode hot path on one MI355X.
+
+    python -m fusekit_amd.kernel_bench [--case NAME ...] [--reps N]
+
+Every case builds one hipGraph whose nodes run the same kernel over a pool of DISTINCT
+operands larger than the 256 MB last-level cache, so each launch streams its bytes from HBM
+("cold"); a second graph re-runs one operand set ("warm", cache resident where it fits).
+Nodes are serialised (a barrier between each) so that the figure is the kernel's own
+duration plus the ~1.6 us a dependent graph node costs; `parallel` lets the graph overlap
+independent nodes instead.  GPU time comes from HIP events around whole graph launches on the
+dispatcher's stream.  One JSON line per case; bytes are the ALGORITHMIC bytes of the call
+(weights + scales + biases + activations in and out, KV rows read), peak is 8 TB/s.
+
+Weights are random bits / random bf16 scales written straight into HBM: timing does not
+depend on the values.
+"""
+import argparse
+import json
+import sys
+
+from . import native as fk
+from .decoder import _synth
+from .runtime import Dispatch, Dispatcher, arg
+
+HBM_PEAK = 8.0e12
+MFMA_BF16_PEAK = 2.5e15
+
+
+def _rand_weight(n, k, bits, seed, group=64, experts=1):
+    """Random-valued weight of the right byte sizes (timing only)."""
+    W = fk.DeviceWeight.__new__(fk.DeviceWeight)
+    W.n, W.k, W.bits, W.group = n, k, bits, group
+    words = experts * n * k * bits // 32
+    W.w = fk.DeviceBuffer(words * 4)
+    _synth(W.w, words, seed, 0.0, 0.0, 2, 0xFFFFFFFF)
+    if bits == 16:
+        W.scales = W.biases = None
+        # random words may hold NaN/Inf bf16 patterns; fill with small normals instead
+        _synth(W.w, words * 2, seed, 0.0, 0.02, 1)
+    else:
+        meta = experts * n * (k // group)
+        W.scales, W.biases = fk.DeviceBuffer(meta * 2), fk.DeviceBuffer(meta * 2)
+        _synth(W.scales, meta, seed + 1, 0.002, 0.0005, 1)
+        _synth(W.biases, meta, seed + 2, -0.015, 0.004, 1)
+    return W
+
+
+def _bf16(count, seed, std=1.0):
+    b = fk.DeviceBuffer(count * 2)
+    _synth(b, count, seed, 0.0, std, 1)
+    return b
+
+
+def _wargs(W):
+    return [arg(W.w)] + ([] if W.bits == 16 else [arg(W.scales), arg(W.biases)])
+
+
+def _time_graph(d, tasks, reps, serial=True):
+    g = d.build_graph(tasks, barriers=[serial] * len(tasks))
+    d.execute_graph(g)                      # warm-up (first launch uploads the graph)
+    sec = d.execute_graph(g, repeat=reps)
+    return sec / (reps * len(tasks))
+
+
+def _emit(case, per_call_s, nbytes, flops=None, **extra):
+    out = {"case": case, "us_per_call": round(per_call_s * 1e6, 3), "bytes_per_call": int(nbytes),
+           "GBps": round(nbytes / per_call_s / 1e9, 1), "frac_of_hbm_peak": round(nbytes / per_call_s / HBM_PEAK, 4)}
+    if flops is not None:
+        out["TFLOPs"] = round(flops / per_call_s / 1e12, 2)
+        out["frac_of_mfma_bf16_peak"] = round(flops / per_call_s / MFMA_BF16_PEAK, 4)
+    out.update(extra)
+    print(json.dumps(out), flush=True)
+
+
+def case_qgemv(d, reps, n, k, bits, pool, tag):
+    per = bits / 8 + (0 if bits == 16 else 4 / 64)
+    nbytes = n * k * per + k * 2 + n * 2
+    Ws = [_rand_weight(n, k, bits, 100 + 3 * i) for i in range(pool)]
+    x, ys = _bf16(k, 7), [fk.DeviceBuffer(n * 2) for _ in range(pool)]
+    mk = lambda W, y: Dispatch("fusekit_qgemv_f0", [arg(x)] + _wargs(W) + [arg(y)], {"bits": bits, "group": 64, "m": k, "n": n})
+    cold = [mk(W, y) for W, y in zip(Ws, ys)]
+    warm = [mk(Ws[0], ys[i]) for i in range(min(pool, 64))]
+    _emit(f"qgemv_{tag}_q{bits}_cold_serial", _time_graph(d, cold, reps), nbytes, n=n, k=k, pool=pool)
+    _emit(f"qgemv_{tag}_q{bits}_cold_parallel", _time_graph(d, cold, reps, serial=False), nbytes, n=n, k=k, pool=pool)
+    _emit(f"qgemv_{tag}_q{bits}_warm_serial", _time_graph(d, warm, reps), nbytes, n=n, k=k, pool=1)
+
+
+def case_sdpa(d, reps, length):
+    n_heads, n_kv, dim = 32, 8, 128
+    kv_bytes = 2 * n_kv * length * dim * 2
+    pool = max(2, min(256, int(600e6 // kv_bytes) + 1))
+    q, out = _bf16(n_heads * dim, 3), fk.DeviceBuffer(n_heads * dim * 2)
+    import numpy as np
+    kv_len = fk.DeviceBuffer.from_numpy(np.array([length], np.uint32))
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, dim, dim, length)
+    partials, counters = fk.DeviceBuffer(max(pb, 16)), fk.zeros(max(cb, 16))
+    tasks = []
+    keep = []
+    for i in range(pool):
+        ck, cv = _bf16(n_kv * length * dim, 10 + 2 * i), _bf16(n_kv * length * dim, 11 + 2 * i)
+        keep.append((ck, cv))
+        tasks.append(Dispatch("fusekit_sdpa_decode_f0", [arg(q), arg(ck), arg(cv), arg(kv_len), arg(out), arg(partials),
+                                                         arg(counters)],
+                              {"n_heads": n_heads, "n_kv": n_kv, "head_dim": dim, "capacity": length, "max_len": length}))
+    nbytes = kv_bytes + 2 * n_heads * dim * 2
+    _emit(f"sdpa_decode_L{length}_cold_serial", _time_graph(d, tasks, reps), nbytes, flops=4 * n_heads * length * dim,
+          pool=pool)
+    _emit(f"sdpa_decode_L{length}_warm_serial", _time_graph(d, [tasks[0]] * 16, reps), nbytes,
+          flops=4 * n_heads * length * dim, pool=1)
+
+
+def case_moe(d, reps, bits=4):
+    import numpy as np
+    E, hidden, inter, top_k, layers = 64, 2048, 1408, 6, 2
+    per = bits / 8 + 4 / 64
+    rng = np.random.Generator(np.random.PCG64(5))
+    x, res = _bf16(hidden, 1), _bf16(hidden, 2)
+    row_idx = fk.DeviceBuffer.from_numpy(np.zeros(top_k, np.uint32))       # every route reads the one token
+    h_rows = fk.DeviceBuffer.from_numpy(np.arange(top_k, dtype=np.uint32))  # route r reads row r of the SwiGLU output
+    m1, m2, keep = [], [], []
+    for L in range(layers):
+        Wg, Wu = _rand_weight(inter, hidden, bits, 300 + 10 * L, experts=E), _rand_weight(inter, hidden, bits, 303 + 10 * L, experts=E)
+        Wd = _rand_weight(hidden, inter, bits, 306 + 10 * L, experts=E)
+        keep.append((Wg, Wu, Wd))
+    for i in range(16):
+        Wg, Wu, Wd = keep[i % layers]
+        eidx = fk.DeviceBuffer.from_numpy(rng.permutation(E)[:top_k].astype(np.uint32))
+        rwt = _bf16(top_k, 50 + i, 0.2)
+        h, out = fk.DeviceBuffer(top_k * inter * 2), fk.DeviceBuffer(hidden * 2)
+        ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(1, top_k, hidden))
+        keep.append((eidx, rwt, h, out, ws))
+        m1.append(Dispatch("fusekit_routed_qmv_swiglu_f0",
+                           [arg(x), arg(Wg.w), arg(Wg.scales), arg(Wg.biases), arg(Wu.w), arg(Wu.scales), arg(Wu.biases),
+                            arg(row_idx), arg(eidx), arg(h)],
+                           {"bits": bits, "k": hidden, "o": inter, "experts": E, "routes": top_k, "x_rows": 1}))
+        m2.append(Dispatch("fusekit_routed_qmv_reduce_f0",
+                           [arg(h), arg(Wd.w), arg(Wd.scales), arg(Wd.biases), arg(h_rows), arg(eidx), arg(rwt),
+                            arg(res), arg(out), arg(ws)],
+                           {"bits": bits, "k": inter, "o": hidden, "experts": E, "tokens": 1, "top_k": top_k,
+                            "x_rows": top_k, "has_extra": 1}))
+    b1 = top_k * 2 * inter * hidden * per + hidden * 2 + top_k * inter * 2
+    b2 = top_k * hidden * inter * per + top_k * inter * 2 + 2 * hidden * 2
+    _emit(f"routed_qmv_swiglu_cfg5_q{bits}", _time_graph(d, m1, reps), b1, routes=top_k, experts=E)
+    _emit(f"routed_qmv_reduce_cfg5_q{bits}", _time_graph(d, m2, reps), b2, routes=top_k, experts=E,
+          note="three kernels: routed GEMV, ordered reduction")
+
+
+def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
+    per = bits / 8 + 4 / 64
+    pool = max(2, int(600e6 // (n * k * per)) + 1)
+    x = _bf16(rows * k, 1)
+    ws_bytes = fk.qgemm_workspace_bytes(rows, n, k, 64)
+    tasks, keep = [], []
+    for i in range(pool):
+        W, y, ws = _rand_weight(n, k, bits, 500 + 3 * i), fk.DeviceBuffer(rows * n * 2), fk.DeviceBuffer(ws_bytes)
+        keep.append((W, y, ws))
+        tasks.append(Dispatch("fusekit_qgemm_f0", [arg(x)] + _wargs(W) + [arg(y), arg(ws)],
+                              {"bits": bits, "group": 64, "m": k, "n": n, "rows": rows}))
+    nbytes = n * k * per + rows * k * 2 + rows * n * 2
+    _emit(f"qgemm_rows{rows}_{n}x{k}_q{bits}", _time_graph(d, tasks, reps), nbytes, flops=2.0 * rows * n * k, pool=pool,
+          note="two kernels: MFMA main + split-k reduction")
+
+
+CASES = {
+    "qgemv_cfg1": lambda d, r: case_qgemv(d, r, 4864, 896, 4, 512, "cfg1_4864x896"),
+    "qgemv_big_q4": lambda d, r: case_qgemv(d, r, 9728, 2560, 4, 48, "9728x2560"),
+    "qgemv_big_q8": lambda d, r: case_qgemv(d, r, 9728, 2560, 8, 28, "9728x2560"),
+    "qgemv_big_bf16": lambda d, r: case_qgemv(d, r, 9728, 2560, 16, 14, "9728x2560"),
+    "sdpa_512": lambda d, r: case_sdpa(d, r, 512),
+    "sdpa_4096": lambda d, r: case_sdpa(d, r, 4096),
+    "sdpa_32768": lambda d, r: case_sdpa(d, r, 32768),
+    "moe_cfg5": lambda d, r: case_moe(d, r),
+    "qgemm_8": lambda d, r: case_qgemm(d, r, 8),
+    "qgemm_32": lambda d, r: case_qgemm(d, r, 32),
+    "qgemm_128": lambda d, r: case_qgemm(d, r, 128),
+    "qgemm_512": lambda d, r: case_qgemm(d, r, 512),
+}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--case", action="append", choices=sorted(CASES), help="default: all")
+    ap.add_argument("--reps", type=int, default=20)
+    args = ap.parse_args()
+    d = Dispatcher()
+    for name in (args.case or list(CASES)):
+        print(f"[kernel_bench] {name}", file=sys.stderr, flush=True)
+        CASES[name](d, args.reps)
+        fk.sync()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -14,7 +14,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libfusekit_hip.so")
+LIB_PATH = os.environ.get("FUSEKIT_HIP_LIB") or os.path.join(_HERE, "libfusekit_hip.so")
 
 FK_OK, FK_ERR_INVALID, FK_ERR_IO, FK_ERR_NOT_FOUND, FK_ERR_HIP, FK_ERR_UNSUPPORTED = range(6)
 

@@ -164,3 +164,41 @@ def test_routed_rejects_bad_arguments(fk):
         fk.routed_qmv_swiglu(x, 1, to_device(fk, Wg), to_device(fk, Wu), 0, idx, idx, None, 2, out)
     with pytest.raises(fk.InvalidArgument):
         fk.routed_qmv_reduce(x, 1, to_device(fk, Wg), 2, None, idx, None, x, None, None, 1, 2, out, out)
+
+
+def test_routed_families_in_a_graph(fk):
+    """The dispatcher families (reference buffer order) give the direct calls' bytes, replay after replay."""
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    E, hidden, inter, top_k = 8, 256, 192, 4
+    Wg, Wu, Wd = _stack(1300, E, inter, hidden, 4), _stack(1400, E, inter, hidden, 4), _stack(1500, E, hidden, inter, 4)
+    Ws = make_qweight(1600, hidden, 128, 4)
+    x, sx, res = normal_bf16(20, (1, hidden)), normal_bf16(21, (1, 128)), normal_bf16(22, (1, hidden))
+    eidx, rw = np.array([3, 0, 7, 5], np.uint32), normal_bf16(23, top_k, 0.25, 0.1)
+    h_direct = _run_m1(fk, x, Wg, Wu, np.zeros(top_k, np.uint32), eidx, None)
+    out_direct = _run_m2(fk, h_direct, Wd, None, eidx, rw, sx, Ws, res, 1, top_k)
+
+    dWg, dWu, dWd, dWs = (to_device(fk, w) for w in (Wg, Wu, Wd, Ws))
+    bx, bsx, bres, beidx, brw = (_dev(fk, a) for a in (x, sx, res, eidx, rw))
+    rows0, rows = _dev(fk, np.zeros(top_k, np.uint32)), _dev(fk, np.arange(top_k, dtype=np.uint32))
+    h, out = fk.DeviceBuffer(2 * top_k * inter), fk.DeviceBuffer(2 * hidden)
+    ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(1, top_k, hidden))
+    common = {"bits": 4, "group": 64, "experts": E}
+    tasks = [
+        Dispatch("fusekit_routed_qmv_swiglu_f1",
+                 [arg(bx), arg(dWg.w), arg(dWg.scales), arg(dWg.biases), arg(dWu.w), arg(dWu.scales), arg(dWu.biases),
+                  arg(rows0), arg(beidx), arg(h)], dict(common, k=hidden, o=inter, routes=top_k, x_rows=1)),
+        Dispatch("fusekit_routed_qmv_reduce_f2",
+                 [arg(h), arg(dWd.w), arg(dWd.scales), arg(dWd.biases), arg(rows), arg(beidx), arg(brw),
+                  arg(bsx), arg(dWs.w), arg(dWs.scales), arg(dWs.biases), arg(bres), arg(out), arg(ws)],
+                 dict(common, k=inter, o=hidden, tokens=1, top_k=top_k, x_rows=top_k, has_shared=1, shared_k=128,
+                      has_extra=1)),
+    ]
+    d = Dispatcher()
+    g = d.build_graph(tasks)
+    assert d.node_deps(g, 1) == [0]
+    for _ in range(3):
+        fk.fill_u32(out, 0, hidden // 2)
+        fk.sync()
+        d.execute_graph(g)
+        assert np.array_equal(h.to_numpy(np.uint16, (top_k, inter)), h_direct)
+        assert np.array_equal(out.to_numpy(np.uint16, (1, hidden)), out_direct)

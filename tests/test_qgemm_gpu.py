@@ -111,3 +111,23 @@ def test_qgemm_rejects(fk):
         fk.qgemm(to_device(fk, make_qweight(1, 64, 128, 4)), x, 0, None, None, y, ws)
     with pytest.raises(fk.InvalidArgument):
         fk.qgemm(to_device(fk, make_qweight(1, 64, 128, 4)), x, 2, None, None, y, None)
+
+
+def test_qgemm_family_in_a_graph_with_binding_update(fk):
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    m, n, k = 8, 512, 1024
+    W = make_qweight(71, n, k, 4)
+    xa, xb = normal_bf16(72, (m, k)), normal_bf16(73, (m, k))
+    res = normal_bf16(74, (m, n))
+    dW, bxa, bxb, bres = to_device(fk, W), _dev(fk, xa), _dev(fk, xb), _dev(fk, res)
+    y, ws = fk.DeviceBuffer(2 * m * n), fk.DeviceBuffer(fk.qgemm_workspace_bytes(m, n, k))
+    d = Dispatcher()
+    g = d.build_graph([Dispatch("fusekit_qgemm_f0", [arg(bxa), arg(dW.w), arg(dW.scales), arg(dW.biases), arg(bres),
+                                                      arg(y), arg(ws)],
+                                {"bits": 4, "group": 64, "m": k, "n": n, "rows": m, "has_residual": 1})])
+    d.execute_graph(g)
+    assert np.array_equal(y.to_numpy(np.uint16, (m, n)), _run(fk, W, xa, res=res))
+    d.update_graph_bindings(g, [(0, 0, bxb.ptr, bxb.nbytes)])
+    for _ in range(2):
+        d.execute_graph(g)
+        assert np.array_equal(y.to_numpy(np.uint16, (m, n)), _run(fk, W, xb, res=res))
