@@ -4,6 +4,12 @@
 #include "fk_device.hpp"
 #include "rope_device.hpp"
 
+// Hook for timing probes: a build may define FK_SDPA_STAMP(i) to record a clock at
+// phase boundary i; the library build leaves it empty.
+#ifndef FK_SDPA_STAMP
+#define FK_SDPA_STAMP(i)
+#endif
+
 namespace fk {
 
 constexpr int kSdpaBlock = 256;
@@ -47,7 +53,10 @@ constexpr uint32_t kSdpaStatFloats = 32;
 // LDS floats one block needs.
 __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk, uint32_t qk_dim, uint32_t v_dim,
                                                      bool fused) {
-    return gt * chunk + kSdpaWaves * gt * v_dim + kSdpaStatFloats + (fused ? (gt + 1) * qk_dim / 2 + 8 : 0);
+    uint32_t lpv = 1;
+    while (lpv < v_dim / 8) lpv <<= 1;
+    const uint32_t slots = kSdpaBlock / lpv;  // key rows handled side by side in the value phase
+    return gt * chunk + slots * gt * v_dim + kSdpaStatFloats + (fused ? (gt + 1) * qk_dim / 2 + 8 : 0);
 }
 
 // One (range, kv head, head tile) work item.  Uniform per block; `kv_len` already read.
@@ -66,10 +75,11 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     const uint32_t blk_keys = (kv_len - blk0) < span ? (kv_len - blk0) : span;
     const uint32_t n_chunks = (blk_keys + a.chunk_len - 1) / a.chunk_len;
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    FK_SDPA_STAMP(0);
 
     float* s = lds;                               // [GT][chunk_len]
-    float* red = s + GT * a.chunk_len;            // [waves][GT][v_dim]
-    float* stat = red + kSdpaWaves * GT * a.v_dim;  // m[GT], l[GT], misc
+    float* red = s + GT * a.chunk_len;            // [value slots][GT][v_dim]
+    float* stat = red + (kSdpaBlock / a.lpv) * GT * a.v_dim;  // m[GT], l[GT], misc
     uint16_t* qn = reinterpret_cast<uint16_t*>(stat + kSdpaStatFloats);  // fused: [GT][qk_dim] + k row
     uint16_t* kn = qn + GT * a.qk_dim;
     const uint32_t pos = kv_len - 1;  // fused: position of the new token
@@ -116,6 +126,20 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
 
+    // This lane's 8 dims of each query head; fetched before the K/V rows so that the
+    // scores can start as soon as the first keys arrive (loads return in order).
+    uint4 qf[GT];
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+        qf[h] = make_uint4(0, 0, 0, 0);
+        if (kcol_ok && (uint32_t)h < gcount) {
+            if constexpr (FUSED)
+                qf[h] = *reinterpret_cast<const uint4*>(qn + h * a.qk_dim + 8 * ck);
+            else
+                qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
+        }
+    }
+
     for (uint32_t c = 0; c < n_chunks; ++c) {
     const uint32_t key0 = blk0 + c * a.chunk_len;
     const uint32_t nkeys = (kv_len - key0) < a.chunk_len ? (kv_len - key0) : a.chunk_len;
@@ -149,19 +173,9 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
     }
 
+    FK_SDPA_STAMP(1);
     // ---------------- phase A: scores ----------------
     {
-        uint4 qf[GT];
-#pragma unroll
-        for (int h = 0; h < GT; ++h) {
-            qf[h] = make_uint4(0, 0, 0, 0);
-            if (kcol_ok && (uint32_t)h < gcount) {
-                if constexpr (FUSED)
-                    qf[h] = *reinterpret_cast<const uint4*>(qn + h * a.qk_dim + 8 * ck);
-                else
-                    qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
-            }
-        }
         if constexpr (FUSED) {
             if (owner && kcol_ok) {
 #pragma unroll
@@ -184,7 +198,9 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
         }
     }
+    FK_SDPA_STAMP(2);
     __syncthreads();
+    FK_SDPA_STAMP(3);
 
     // ---------------- softmax over this range, one wave per head ----------------
     // Online form: the running maximum may rise, in which case what was summed so
@@ -211,6 +227,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }
     __syncthreads();
 
+    FK_SDPA_STAMP(4);
     // ---------------- phase B: o = sum_j p_j v_j ----------------
     if (c) {
 #pragma unroll
@@ -236,34 +253,27 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }
     if (c + 1 < n_chunks) __syncthreads();  // the scores are overwritten by the next range
     }  // ranges of this block
+    FK_SDPA_STAMP(5);
 
-    {
-        // add the key slots that share this lane's column: first inside the wave ...
+    // Every lane parks its sums in LDS, [value slot][head][dim]; the output loop below
+    // adds the slots in index order (no cross-lane shuffles, fixed order).
+    if (vcol_ok) {
 #pragma unroll
-        for (int h = 0; h < GT; ++h)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float v = acc[h][i];
-                for (uint32_t o = lpv; o < (uint32_t)kWave; o <<= 1) v += __shfl_xor(v, (int)o, kWave);
-                acc[h][i] = v;
-            }
-        // ... then across waves through LDS
-        if (lane < lpv && vcol_ok) {
-#pragma unroll
-            for (int h = 0; h < GT; ++h)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) red[(wave * GT + h) * a.v_dim + 8 * cv + i] = acc[h][i];
+        for (int h = 0; h < GT; ++h) {
+            float4* dst = reinterpret_cast<float4*>(red + ((size_t)vslot * GT + h) * a.v_dim + 8 * cv);
+            dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+            dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
         }
     }
     __syncthreads();
 
+    FK_SDPA_STAMP(6);
     const uint32_t n_out = gcount * a.v_dim;
     const bool direct = (n_active == 1);
     for (uint32_t e = tid; e < n_out; e += kSdpaBlock) {
         const uint32_t h = e / a.v_dim, d = e - h * a.v_dim;
         float o = 0.f;
-#pragma unroll
-        for (int w = 0; w < kSdpaWaves; ++w) o += red[(w * GT + h) * a.v_dim + d];
+        for (uint32_t sl = 0; sl < vslots; ++sl) o += red[(sl * GT + h) * a.v_dim + d];
         if (direct) {
             st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o / stat[8 + h]));
         } else {
@@ -275,6 +285,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
         }
     }
+    FK_SDPA_STAMP(7);
     if (direct) return;
 
     // ---------------- last block merges the partials ----------------
@@ -290,6 +301,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         *flag = (prev == n_active - 1) ? 1u : 0u;
     }
     __syncthreads();
+    FK_SDPA_STAMP(8);
     if (*flag == 0u) return;
     if (tid == 0)  // ready for the next launch (or the next layer of this one)
         __hip_atomic_store(&a.counters[kvh * gz_count + gz], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -343,11 +355,12 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             st_u16<FUSED>(dst + 1, f32_to_bf16_bits(o1 * inv_l));
         }
     }
+    FK_SDPA_STAMP(9);
 }
 
 template <int GT>
 __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs a) {
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     const uint32_t kv_len = a.kv_len_ptr ? *a.kv_len_ptr : a.kv_len_imm;
     sdpa_block<GT, false, SdpaArgs>(a, kv_len, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
 }
