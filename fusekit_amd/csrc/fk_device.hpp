@@ -14,20 +14,17 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as
 __device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
 
-// fp32 -> bf16, round to nearest even, NaN kept quiet.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+// fp32 -> bf16, round to nearest even, NaN kept quiet: one v_cvt_pk_bf16_f32.  The
+// instruction agrees bit for bit, on all 2^32 inputs (NaN payloads included), with
+// the integer formulation  u += 0x7fff + ((u >> 16) & 1); u >>= 16  (NaN: (u >> 16) | 0x40).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const bf16x2_t p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16(f, 0.0f) & 0xffffu; }
 // T(v) as a float again: the rounding boundary the reference places on every
 // value it casts to the activation type.
-__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(f32_to_bf16_bits(f) << 16); }
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
-}
+__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(pack_bf16(0.0f, f) & 0xffff0000u); }
 
 // acc + a.lo*b.lo + a.hi*b.hi with bf16 inputs, fp32 accumulate (v_dot2c_f32_bf16).
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {

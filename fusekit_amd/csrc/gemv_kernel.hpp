@@ -17,6 +17,12 @@
 #pragma once
 #include "fk_device.hpp"
 
+// Hook for timing probes: a build may define FK_GEMV_STAMP(i) to record a clock at
+// phase boundary i; the library build leaves it empty.
+#ifndef FK_GEMV_STAMP
+#define FK_GEMV_STAMP(i)
+#endif
+
 namespace fk {
 
 enum WKind : int { W_Q4 = 0, W_Q8 = 1, W_BF16 = 2 };
@@ -160,23 +166,34 @@ __device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int va
 // chunk sum is a 2- or 4-lane butterfly.  K must be a multiple of 64.
 constexpr int kStageRegs = 4;
 
+// Issues the loads of the register-resident part of x (and the norm weight).  A
+// stand-alone kernel calls this BEFORE the weight prefetch: loads return in issue
+// order, so x queued behind a batch of weight rows would wait for HBM although it
+// sits in cache.
+template <typename ARGS>
+__device__ __forceinline__ void stage_fetch(const ARGS& a, uint4 (&xr)[kStageRegs], uint4 (&wr)[kStageRegs]) {
+    // Straight-line on purpose (clamped index, the norm weight replaced by x itself
+    // when there is none): with branches around the loads the compiler falls back to
+    // waiting for every outstanding load, weight prefetch included.
+    const uint32_t n8 = a.K >> 3;
+    const uint4* x8 = reinterpret_cast<const uint4*>(a.x);
+    const uint4* w8 = a.norm_w ? reinterpret_cast<const uint4*>(a.norm_w) : x8;
+#pragma unroll
+    for (int i = 0; i < kStageRegs; ++i) {
+        const uint32_t t = threadIdx.x + i * kGemvBlock;
+        const uint32_t tc = t < n8 ? t : 0u;
+        xr[i] = x8[tc];
+        wr[i] = w8[tc];
+    }
+}
+
 template <WKind KIND, typename ARGS>
-__device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, float* sx, float* scratch) {
+__device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, float* sx, float* scratch,
+                                                  uint4 (&xr)[kStageRegs], uint4 (&wr)[kStageRegs]) {
     const bool NORM = a.norm_w != nullptr;  // uniform; one code path serves both
     const uint32_t K = a.K, cpr = a.cpr, n8 = K >> 3;
     const uint4* x8 = reinterpret_cast<const uint4*>(a.x);
     const uint4* w8 = reinterpret_cast<const uint4*>(a.norm_w);
-    uint4 xr[kStageRegs], wr[kStageRegs];
-#pragma unroll
-    for (int i = 0; i < kStageRegs; ++i) {
-        const uint32_t t = threadIdx.x + i * kGemvBlock;
-        xr[i] = make_uint4(0, 0, 0, 0);
-        wr[i] = make_uint4(0, 0, 0, 0);
-        if (t < n8) {
-            xr[i] = x8[t];
-            if (NORM) wr[i] = w8[t];
-        }
-    }
     float r = 1.0f;
     if (NORM) {
         float ss = 0.f;
@@ -190,7 +207,8 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
             }
         };
 #pragma unroll
-        for (int i = 0; i < kStageRegs; ++i) add_sq(xr[i]);  // zeros beyond n8 add nothing
+        for (int i = 0; i < kStageRegs; ++i)
+            if (threadIdx.x + i * kGemvBlock < n8) add_sq(xr[i]);
         for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8; t += kGemvBlock) add_sq(x8[t]);
         ss = block_sum<kGemvBlock>(ss, scratch);
         r = 1.0f / sqrtf(ss / (float)K + a.eps);
@@ -238,8 +256,10 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
                                    pack_bf16(f[6], f[7]));
         }
     };
+    // whole waves past the end skip the step (the chunk-sum butterflies need whole waves)
 #pragma unroll
-    for (int i = 0; i < kStageRegs; ++i) emit(threadIdx.x + i * kGemvBlock, xr[i], wr[i]);
+    for (int i = 0; i < kStageRegs; ++i)
+        if ((threadIdx.x & ~(uint32_t)(kWave - 1)) + i * kGemvBlock < n8) emit(threadIdx.x + i * kGemvBlock, xr[i], wr[i]);
     // long rows: the rest is fetched again (whole waves stay in the loop so the
     // butterflies above see all their lanes)
     const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
@@ -339,7 +359,8 @@ __device__ __forceinline__ void gemv_prefetch(const ARGS& a, uint32_t block_id, 
 template <WKind KIND, int NSEG, bool COH, typename ARGS>
 __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint32_t n_blocks, uint4* lds_raw,
                                          uint4 (&wa)[kGemvUnroll], uint32_t (&sa)[kGemvUnroll],
-                                         uint32_t (&ba)[kGemvUnroll]) {
+                                         uint32_t (&ba)[kGemvUnroll], uint4 (&xr)[kStageRegs],
+                                         uint4 (&wr)[kStageRegs]) {
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     constexpr int SLOTS = kGemvUnroll / NSEG;                // register slots per segment and batch
     constexpr uint32_t POS = kGemvBlock * SLOTS;             // chunk positions of a segment per batch
@@ -364,6 +385,7 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
     const uint32_t col_step = POS % cpr;
 
     uint32_t tile = block_id, b0 = 0;
+    bool first_batch = true;  // probe builds only: marks the first batch for FK_GEMV_STAMP
 
     // Consumes the batch held in cur* while the following batch streams into nxt*.
     // Returns false once this block has no tile left.  (Two copies of this body,
@@ -385,6 +407,8 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
             // (that costs ~200 VGPRs); other waves hide the LDS latency instead.
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (first_batch) FK_GEMV_STAMP(3);
+        first_batch = false;
         // `part` is padded to whole batches, so the store needs no guard (a guard
         // would let the compiler sink all the arithmetic into the branch).
 #pragma unroll
@@ -436,12 +460,26 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
 
     uint4 wb[kGemvUnroll];
     uint32_t sb[kGemvUnroll], bb[kGemvUnroll];
-    stage_activations<KIND, ARGS>(a, xs, sx, scratch);
+    FK_GEMV_STAMP(1);
+    stage_activations<KIND, ARGS>(a, xs, sx, scratch, xr, wr);
+    FK_GEMV_STAMP(2);
     if (block_id >= a.n_tiles) return;
     while (true) {
         if (!step(wa, sa, ba, wb, sb, bb)) break;
         if (!step(wb, sb, bb, wa, sa, ba)) break;
     }
+    FK_GEMV_STAMP(4);
+}
+
+// Form for callers whose activations do not exist yet when the weights are
+// prefetched (the whole-token kernel prefetches across a grid barrier).
+template <WKind KIND, int NSEG, bool COH, typename ARGS>
+__device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint32_t n_blocks, uint4* lds_raw,
+                                         uint4 (&wa)[kGemvUnroll], uint32_t (&sa)[kGemvUnroll],
+                                         uint32_t (&ba)[kGemvUnroll]) {
+    uint4 xr[kStageRegs], wr[kStageRegs];
+    stage_fetch(a, xr, wr);
+    gemv_run<KIND, NSEG, COH, ARGS>(a, block_id, n_blocks, lds_raw, wa, sa, ba, xr, wr);
 }
 
 template <WKind KIND, int NSEG>
@@ -449,8 +487,11 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs 
     extern __shared__ uint4 lds_raw[];
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
-    gemv_prefetch<KIND, NSEG>(a, blockIdx.x, wa, sa, ba);  // weights start streaming before x is staged
-    gemv_run<KIND, NSEG, false>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba);
+    uint4 xr[kStageRegs], wr[kStageRegs];
+    FK_GEMV_STAMP(0);
+    stage_fetch(a, xr, wr);                                // activations first: they return first
+    gemv_prefetch<KIND, NSEG>(a, blockIdx.x, wa, sa, ba);  // weights stream while x is staged
+    gemv_run<KIND, NSEG, false>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba, xr, wr);
 }
 
 }  // namespace fk

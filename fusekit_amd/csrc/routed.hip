@@ -86,8 +86,10 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
 
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
+    uint4 xr[kStageRegs], wr[kStageRegs];
+    stage_fetch(v, xr, wr);
     gemv_prefetch<KIND, NSEG>(v, sub, wa, sa, ba);
-    gemv_run<KIND, NSEG, false>(v, sub, a.blocks_per_route, lds_raw, wa, sa, ba);
+    gemv_run<KIND, NSEG, false>(v, sub, a.blocks_per_route, lds_raw, wa, sa, ba, xr, wr);
 }
 
 struct RouteReduceArgs {
