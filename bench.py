@@ -24,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E published peak
+# HBM bytes per launch of the int4 gate/up kernel of the 4B-class model, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE (two counter runs of this script, each scaled by what the same counter reads for the plain
+# 256 MiB copies of --calibrate-copy: 1.99981 and 1.0).  Counters cannot be read from inside this process.
+GATEUP_Q4_4B_TRAFFIC_BYTES = 29013600
 
 
 def main() -> int:
@@ -37,6 +41,9 @@ def main() -> int:
     ap.add_argument("--cpu-tokens", type=int, default=2)
     ap.add_argument("--per-kernel", action="store_true", help="print per-family GPU time of one token to stderr")
     ap.add_argument("--layers", type=int, default=0, help="experiment only: override the layer count (not the headline config)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 4 plain 256 MiB device copies (outside the timed region): the known-traffic "
+                         "kernel that rocprofv3 byte counters of the same run are scaled by")
     ap.add_argument("--mode", choices=["persistent", "graph"], default="graph",
                     help="persistent: one whole-token kernel per replay; graph: one kernel node per task")
     args = ap.parse_args()
@@ -62,6 +69,14 @@ def main() -> int:
     rt = DecoderRuntime(cfg, W, hist_capacity=max(4096, args.steps + args.warmup),
                         persistent=(args.mode == "persistent"))
     setup_s = time.time() - t0
+
+    if args.calibrate_copy:
+        src, dst = fk.DeviceBuffer(256 << 20), fk.DeviceBuffer(256 << 20)
+        fk.fill_u32(src, 0x3f803f80, (256 << 20) // 4)
+        for _ in range(4):
+            fk.copy(dst, src, 256 << 20)
+        fk.sync()
+        del src, dst
 
     rng = np.random.Generator(np.random.PCG64(0))
     prompt = rng.integers(0, cfg.vocab, args.prompt).tolist()
@@ -150,7 +165,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": GATEUP_Q4_4B_TRAFFIC_BYTES if (cfg.bits == 4 and not args.layers) else None,
             "bytes_per_launch": gateup_bytes,
             "avg_launch_us": round(gateup_us, 3),
             "launches_timed": reps * len(gateup),

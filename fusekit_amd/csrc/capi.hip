@@ -390,6 +390,12 @@ fk_status fk_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_le
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_copy(void* dst, const void* src, size_t nbytes, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_copy(dst, src, nbytes, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_fill_u32(void* dptr, uint32_t value, size_t count, fk_stream s) {
     Launch l;
     FK_TRY(plan_fill_u32(dptr, value, count, &l));

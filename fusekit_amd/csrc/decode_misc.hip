@@ -268,4 +268,33 @@ fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out) {
     return FK_OK;
 }
 
+
+// Plain device-to-device copy in 16-byte pieces.  Besides moving buffers it is the
+// known-traffic kernel hardware byte counters are calibrated against.
+struct CopyArgs {
+    uint4* dst;
+    const uint4* src;
+    size_t count;  // 16-byte pieces
+};
+__global__ __launch_bounds__(256) void copy_u128_kernel(const CopyArgs a) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < a.count; i += (size_t)gridDim.x * 256) a.dst[i] = a.src[i];
+}
+
+fk_status plan_copy(void* dst, const void* src, size_t nbytes, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!dst || !src || nbytes == 0) return set_error(FK_ERR_INVALID, "copy: null pointer or zero size");
+    if (nbytes % 16 || (reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16)
+        return set_error(FK_ERR_INVALID, "copy: pointers and size must be multiples of 16 bytes");
+    CopyArgs a{reinterpret_cast<uint4*>(dst), reinterpret_cast<const uint4*>(src), nbytes / 16};
+    size_t blocks = (a.count + 255) / 256;
+    if (blocks > (size_t)dev->cus * 8) blocks = (size_t)dev->cus * 8;
+    out->func = reinterpret_cast<const void*>(&copy_u128_kernel);
+    out->grid = dim3((uint32_t)blocks, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
 }  // namespace fk

@@ -130,6 +130,7 @@ fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, 
                       uint32_t* hist_counter, uint32_t hist_capacity, void* workspace, Launch* out);
 fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out);
 fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out);
+fk_status plan_copy(void* dst, const void* src, size_t nbytes, Launch* out);
 fk_status plan_quantize(const float* w, size_t n, size_t k, uint32_t bits, uint32_t group, uint32_t* packed,
                         uint16_t* scales, uint16_t* biases, Launch* out);
 fk_status plan_synth(void* out_ptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind, uint32_t bound,

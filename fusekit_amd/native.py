@@ -275,6 +275,10 @@ def step_init(step_counter, offset, kv_len, stream=None):
     check(lib.fk_step_init(_ptr(step_counter), _ptr(offset), _ptr(kv_len), _ptr(stream)))
 
 
+def copy(dst, src, nbytes, stream=None):
+    check(lib.fk_copy(_ptr(dst), _ptr(src), C.c_size_t(nbytes), _ptr(stream)))
+
+
 def fill_u32(buf, value, count, stream=None):
     check(lib.fk_fill_u32(_ptr(buf), C.c_uint32(value), C.c_size_t(count), _ptr(stream)))
 

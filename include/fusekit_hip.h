@@ -77,6 +77,10 @@ fk_status fk_free(void *dptr);
 fk_status fk_upload(void *dptr, const void *host, size_t nbytes);
 fk_status fk_download(void *host, const void *dptr, size_t nbytes);
 fk_status fk_fill_u32(void *dptr, uint32_t value, size_t count, fk_stream s);
+/* Device-to-device copy by a plain kernel (pointers and size multiples of 16 bytes):
+ * moves buffers inside a stream / graph and is the known-traffic kernel against
+ * which hardware byte counters are calibrated. */
+fk_status fk_copy(void *dst, const void *src, size_t nbytes, fk_stream s);
 fk_status fk_stream_create(fk_stream *out);
 fk_status fk_stream_destroy(fk_stream s);
 fk_status fk_stream_sync(fk_stream s);
