@@ -239,3 +239,60 @@ def test_persistent_kernel_barrier_timeout_drains_and_reports(fk):
     with pytest.raises(fk.FusekitError) as e:
         rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, [5])
     assert "spin limit" in str(e.value)
+
+
+def test_4b_class_greedy_32_tokens_match_oracle(fk):
+    """The headline model at full size (36 layers, hidden 2560, vocab 151936, int4 g64), 32 greedy
+    steps against the oracle on the same weight bytes.
+
+    Logits are bf16 and the weights are random, so among 151936 candidates the two largest logits
+    are often equal or one bf16 ulp apart (margins are printed).  Free-running equality is required
+    as long as the oracle's margin is clear; at a near-tie the GPU token must be one of the oracle's
+    candidates within two ulps of its maximum (either logit may sit on a rounding edge and move by
+    one ulp with the fp32 summation order), and the run continues teacher-forced on the oracle's
+    tokens so that every one of the 32 steps is checked.
+
+    The per-kernel bar (rel-L2 <= 1e-2) does not carry over to 36 stacked layers: at K = 2560..9728
+    fp32 accumulation (any order) and the oracle's double accumulation round ~1-2 % of a GEMV's
+    outputs to neighbouring bf16 values, which measures 1.7e-3 on the logits after one layer and
+    grows to ~3e-2 after 36 (the same stack at hidden 256 agrees bit for bit).  The last step's
+    logits are held to 5e-2."""
+    from fusekit_amd.decoder import DENSE_4B, DecoderConfig, DecoderRuntime, DecoderWeights
+    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=128)
+    W = DecoderWeights.random_init(cfg, seed=0)
+    rt = DecoderRuntime(cfg, W)
+    od = OracleDecoder(cfg, W)
+    prompt = rng(0).integers(0, cfg.vocab, 4).tolist()
+    n = 32
+    got_free, _, _ = rt.generate(prompt, n)
+
+    ref, margins, cands = [], [], []
+    seq = list(prompt)
+    for i in range(len(prompt) + n - 1):
+        nxt, m, logits = od.step(seq[i], i, want_logits=True)
+        if i >= len(prompt) - 1:
+            f = oracle.bf16_to_f32(logits)
+            top = float(f.max())
+            ulp = 2.0 ** (np.floor(np.log2(abs(top))) - 7)
+            ref.append(nxt); margins.append(m); cands.append(set(np.nonzero(f >= top - 2 * ulp)[0].tolist()))
+            seq.append(nxt)
+    print("oracle margins:", ["%.3g" % m for m in margins])
+    print("candidates per step:", [len(c) for c in cands])
+
+    preds, _ = rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, seq[:-1])
+    preds = preds[len(prompt) - 1:]
+    exact = sum(int(g == r) for g, r in zip(preds, ref))
+    print(f"teacher-forced: {exact}/{n} steps pick the oracle's token")
+    for i, (g, r) in enumerate(zip(preds, ref)):
+        assert g in cands[i], f"step {i}: gpu {g} is not among the oracle's near-maximal tokens {sorted(cands[i])} (oracle {r})"
+        if len(cands[i]) == 1:
+            assert g == r
+    # free-running: identical up to the first step that has more than one candidate
+    first_tie = next((i for i, c in enumerate(cands) if len(c) > 1), n)
+    assert got_free[:first_tie] == ref[:first_tie]
+    assert exact >= n - 6
+    f_got = oracle.bf16_to_f32(rt.logits.to_numpy(np.uint16)).astype(np.float64)
+    f_ref = oracle.bf16_to_f32(logits).astype(np.float64)
+    rel = np.linalg.norm(f_got - f_ref) / np.linalg.norm(f_ref)
+    print(f"last-step logits rel-L2 {rel:.3e}")
+    assert rel <= 5e-2
