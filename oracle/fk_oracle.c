@@ -25,6 +25,14 @@
  *   sdpa_decode ................. pinned (float64 softmax attention; kv_len=1;
  *                                 chunk-merge invariance)
  *   argmax ...................... pinned (brute force, tie rule)
+ *   routed gate/up, routed reduce pinned (reduce to the pinned dense pair / qGEMV on the
+ *                                 selected expert's slice; slot-order fp32 sum restated
+ *                                 in numpy; clamp, row_idx, shared expert, residual)
+ *   qgemm ....................... pinned as the row-wise repetition of qGEMV; the
+ *                                 reference's multi-row path rounds every dequantised
+ *                                 weight to bf16 first (MLX QuantizedBlockLoader, not
+ *                                 vendored): that rounding is parity unpinned
+ *   hand-derived known answers .. tests/golden/known_answers.json
  *   MLX-internal accumulation order, Metal fast::cos/sin/exp bit patterns:
  *                                 parity unpinned (cannot be observed here;
  *                                 irrelevant under the rel-L2 <= 1e-2 bar).

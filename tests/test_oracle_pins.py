@@ -315,3 +315,70 @@ def test_decoder_step_is_the_composition_of_its_parts():
         assert np.array_equal(logits, ref) and tok == oracle.argmax(ref)
         assert np.array_equal(ck, ck2) and np.array_equal(cv, cv2)
         assert margin == pytest.approx(oracle.top2_margin(ref))
+
+
+def test_routed_swiglu_is_the_dense_pair_on_the_selected_expert():
+    """M1: route r must equal the pinned dense gate/up SwiGLU (variant B) run on expert
+    min(expert_idx[r], E-1)'s slice and activation row row_idx[r]; the route weight scales the fp32
+    product before the single round (powers of two make that exact)."""
+    E, O, K = 5, 48, 128
+    experts_g = [make_qweight(100 + e, O, K, 4) for e in range(E)]
+    experts_u = [make_qweight(200 + e, O, K, 4) for e in range(E)]
+    Wg, Wu = oracle.StackedWeight(experts_g), oracle.StackedWeight(experts_u)
+    x = normal_bf16(1, (3, K))
+    row_idx = np.array([2, 0, 1, 1], np.uint32)
+    expert_idx = np.array([4, 0, 99, 3], np.uint32)           # 99 clamps to E-1 (routed_qmv_swiglu.rs:138)
+    out = oracle.routed_qmv_swiglu(x, Wg, Wu, row_idx, expert_idx)
+    for r in range(4):
+        e = min(int(expert_idx[r]), E - 1)
+        assert np.array_equal(out[r], oracle.gateup_swiglu(x[row_idx[r]], None, 0.0, experts_g[e], experts_u[e], 1))
+    rw = oracle.f32_to_bf16(np.array([0.5, 2.0, 0.25, 1.0], np.float32))
+    scaled = oracle.routed_qmv_swiglu(x, Wg, Wu, row_idx, expert_idx, rw)
+    want = oracle.bf16_to_f32(out) * oracle.bf16_to_f32(rw)[:, None]
+    assert np.array_equal(oracle.bf16_to_f32(scaled), want)
+    # the stacked layout itself: expert e starts e * O rows into the [E * O, K/8] matrix
+    flat = oracle.QWeight(Wg.w.reshape(E * O, -1), Wg.scales.reshape(E * O, -1), Wg.biases.reshape(E * O, -1), E * O, K, 4, 64)
+    assert np.array_equal(oracle.dequantize(flat)[3 * O:4 * O], oracle.dequantize(experts_g[3]))
+
+
+def test_routed_reduce_closed_forms():
+    """M2: one route with weight 1 is the pinned qGEMV; the sum runs in slot order in fp32 over the
+    ROUNDED per-route results times the route weight; the shared expert adds its rounded result last;
+    the residual is added before the single final round."""
+    E, O, K, top_k = 4, 40, 192, 3
+    experts = [make_qweight(300 + e, O, K, 4) for e in range(E)]
+    Wd = oracle.StackedWeight(experts)
+    h = normal_bf16(2, (top_k, K), 0.0, 0.5)
+    eidx = np.array([1, 3, 1], np.uint32)
+    one = oracle.routed_qmv_reduce(h[:1], Wd, eidx[:1], None, None, 1, 1)
+    assert np.array_equal(one[0], oracle.qgemv(experts[1], h[0]))
+    rw = normal_bf16(3, top_k, 0.3, 0.2)
+    res = normal_bf16(4, (1, O))
+    shared_w, shared_x = make_qweight(400, O, 64, 4), normal_bf16(5, (1, 64))
+    got = oracle.routed_qmv_reduce(h, Wd, eidx, rw, res, 1, top_k, shared_x=shared_x, Wshared=shared_w)
+    acc = np.zeros(O, np.float32)
+    for s in range(top_k):
+        part = oracle.bf16_to_f32(oracle.qgemv(experts[int(eidx[s])], h[s]))          # T(dot), pinned
+        acc = (acc + (oracle.bf16_to_f32(rw[s:s + 1])[0] * part).astype(np.float32)).astype(np.float32)
+    acc = (acc + oracle.bf16_to_f32(oracle.qgemv(shared_w, shared_x[0]))).astype(np.float32)
+    acc = (acc + oracle.bf16_to_f32(res[0])).astype(np.float32)
+    assert np.array_equal(got[0], oracle.f32_to_bf16(acc))
+    # pre-weighted input (route_weight absent) is weight 1; row_idx permutes the rows of h
+    perm = np.array([2, 0, 1], np.uint32)
+    a = oracle.routed_qmv_reduce(h, Wd, eidx, None, None, 1, top_k, row_idx=perm)
+    b = oracle.routed_qmv_reduce(h[perm], Wd, eidx, None, None, 1, top_k)
+    assert np.array_equal(a, b)
+    # two tokens are two independent reductions
+    h2 = normal_bf16(6, (2 * top_k, K), 0.0, 0.5)
+    e2 = np.array([0, 1, 2, 3, 2, 1], np.uint32)
+    both = oracle.routed_qmv_reduce(h2, Wd, e2, None, None, 2, top_k)
+    assert np.array_equal(both[1], oracle.routed_qmv_reduce(h2[top_k:], Wd, e2[top_k:], None, None, 1, top_k)[0])
+
+
+def test_qgemm_rows_are_qgemv():
+    W = make_qweight(500, 72, 256, 8)
+    x = normal_bf16(7, (4, 256))
+    bias = normal_bf16(8, 72)
+    y = oracle.qgemm(W, x, bias)
+    for r in range(4):
+        assert np.array_equal(y[r], oracle.qgemv(W, x[r], bias))
