@@ -1,0 +1,183 @@
+"""The per-model artifact of the decode path: `task_graph.json` (schema version 2) and `manifest.json`.
+
+The reference's compiler writes these next to `kernel.metallib` (src/codegen/task_graph_json.rs:31-227,
+src/manifest.rs:26-100) and its Python runtime resolves every task's buffer slots from them
+(python/fusekit_runtime/dispatch.py).  For the HIP target the kernels live in the library, so the
+artifact is the task list only.  `write_artifact` serialises a DecoderRuntime's task list in that
+schema -- kernel name, grid_threads / threadgroup as the launch planners decide them, every slot as
+an `external` (model parameter, by `source_path`) or `scratch` binding, `depends_on` from the graph's
+hazard edges, `layer_groups`, `decode_pipeline` -- plus the per-task `params` object the HIP kernels
+take instead of constants baked into generated source.  `load_artifact` is the consumer: it
+allocates what the file describes, binds the parameters of a DecoderWeights by path and returns a
+runtime whose graph replays the same decode.
+"""
+from __future__ import annotations
+
+import json
+import os
+import re
+import time
+from typing import Dict, List, Optional
+
+import numpy as np
+
+from . import native
+from .decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+from .native import DeviceBuffer
+from .runtime import Dispatch, Dispatcher, make_uniforms
+
+SCHEMA_VERSION = 2
+BACKEND_VERSION = "fusekit_amd-0.1"
+
+
+def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
+    """Device pointer -> how the slot is described in the artifact."""
+    sym: Dict[int, dict] = {}
+
+    def scratch(name: str, buf: DeviceBuffer, dtype: str, zero: bool = False):
+        sym[buf.ptr] = dict(role="scratch", role_name=name, dtype=dtype, size_bytes=buf.nbytes, zero=zero)
+
+    for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws"):
+        scratch(name, getattr(rt, name), "uint32", zero=True)
+    scratch("x.0", rt.x[0], "bfloat16")
+    scratch("x.1", rt.x[1], "bfloat16")
+    for name in ("q", "k", "v", "att", "mid", "logits"):
+        scratch(name, getattr(rt, name), "bfloat16")
+    scratch("sdpa_partials", rt.sdpa_partials, "float32")
+    for l in range(rt.cfg.n_layers):
+        scratch(f"cache_k.{l}", rt.cache_k[l], "bfloat16", zero=True)
+        scratch(f"cache_v.{l}", rt.cache_v[l], "bfloat16", zero=True)
+    for path, W in rt.w.mats.items():
+        sym[W.w.ptr] = dict(role="external", source_path=path + ".weight", dtype="uint32" if W.bits != 16 else "bfloat16",
+                            shape=[W.n, W.k * W.bits // 32] if W.bits != 16 else [W.n, W.k])
+        if W.bits != 16:
+            sym[W.scales.ptr] = dict(role="external", source_path=path + ".scales", dtype="bfloat16", shape=[W.n, W.k // W.group])
+            sym[W.biases.ptr] = dict(role="external", source_path=path + ".biases", dtype="bfloat16", shape=[W.n, W.k // W.group])
+    for path, v in rt.w.vecs.items():
+        sym[v.ptr] = dict(role="external", source_path=path, dtype="bfloat16", shape=[v.nbytes // 2])
+    return sym
+
+
+def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "synthetic") -> None:
+    if rt.persistent:
+        raise ValueError("write the artifact from a task-graph runtime (persistent=False)")
+    os.makedirs(out_dir, exist_ok=True)
+    sym = _symbols(rt)
+    scratch_ids: Dict[str, int] = {}
+    scratch_buffers: List[dict] = []
+    tasks: List[dict] = []
+    groups: Dict[str, List[int]] = {}
+    for tid, d in enumerate(rt.tasks):
+        geo = rt.d.plan_geometry(d)
+        bindings = []
+        for slot, (ptr, nbytes) in enumerate(d.args):
+            s = sym.get(ptr)
+            if s is None:
+                raise ValueError(f"task {tid} ({d.kernel}) slot {slot}: buffer is not a known parameter or scratch")
+            access = geo.slot_access[slot]
+            b = dict(slot=slot, role=s["role"], access=("rw" if access == 3 else "w" if access == 2 else "r"),
+                     nbytes=nbytes, dtype=s["dtype"])
+            if s["role"] == "external":
+                b.update(source_path=s["source_path"], shape=s["shape"], role_name=s["source_path"].rsplit(".", 1)[-1])
+            else:
+                name = s["role_name"]
+                if name not in scratch_ids:
+                    scratch_ids[name] = len(scratch_buffers)
+                    scratch_buffers.append(dict(id=scratch_ids[name], role_name=name, dtype=s["dtype"],
+                                                shape=[s["size_bytes"] // (4 if s["dtype"] != "bfloat16" else 2)],
+                                                size_bytes=s["size_bytes"], zero_init=s["zero"]))
+                b.update(scratch_id=scratch_ids[name], role_name=name)
+            bindings.append(b)
+        m = re.search(r"cache_k\.(\d+)", " ".join(b.get("role_name", "") for b in bindings))
+        lm = [re.match(r"layers\.(\d+)\.", b.get("source_path", "")) for b in bindings]
+        layer = next((int(x.group(1)) for x in lm if x), int(m.group(1)) if m else None)
+        kernels = [dict(grid=list(geo.grid[i]), threadgroup=list(geo.threadgroup[i]), lds_bytes=geo.lds_bytes[i])
+                   for i in range(geo.n_kernels)]
+        task = dict(id=tid, fusion_id=tid, kernel=d.kernel,
+                    grid_threads=[kernels[0]["grid"][a] * kernels[0]["threadgroup"][a] for a in range(3)],
+                    threadgroup=kernels[0]["threadgroup"],
+                    inputs=[b for b in bindings if b["access"] == "r"],
+                    outputs=[b for b in bindings if b["access"] != "r"],
+                    params={k: float(v) for k, v in d.params.items()},
+                    kernels=kernels, depends_on=rt.d.node_deps(rt.graph, tid), trigger_event=tid)
+        if layer is not None:
+            task["layer_idx"] = layer
+        tasks.append(task)
+        region = "embed" if layer is None and tid < 2 else (f"layer.{layer}" if layer is not None else "post")
+        groups.setdefault(region, []).append(tid)
+    c = rt.cfg
+    graph = dict(
+        version=SCHEMA_VERSION, active_m=1, backend="hip-gfx950", tasks=tasks,
+        events=[dict(id=t["id"], num_triggers=1, fires=[u["id"] for u in tasks if t["id"] in u["depends_on"]]) for t in tasks],
+        scratch_buffers=scratch_buffers, initial_tasks=[t["id"] for t in tasks if not t["depends_on"]],
+        model_params=[dict(path=s["source_path"], shape=s["shape"], dtype=s["dtype"]) for s in sym.values() if s["role"] == "external"],
+        layer_groups=[dict(region=r, task_ids=ids) for r, ids in groups.items()],
+        decode_pipeline=[t["id"] for t in tasks],
+        decode_capabilities=dict(dispatchable=True, reasons=[]),
+        uniforms=dict(token="token", step_counter="step_counter", hist_counter="hist_counter", history="history"),
+        model_config={k: getattr(c, k) for k in ("n_layers", "hidden", "n_heads", "n_kv", "head_dim", "inter", "vocab",
+                                                  "capacity", "bits", "group", "eps", "theta", "qk_norm", "qkv_bias",
+                                                  "fuse_rope_store", "swiglu_variant")})
+    with open(os.path.join(out_dir, "task_graph.json"), "w") as f:
+        json.dump(graph, f, indent=1)
+    manifest = dict(
+        schema_version=SCHEMA_VERSION, fusekit_version=BACKEND_VERSION,
+        compiled_at=time.strftime("%Y-%m-%dT%H:%M:%SZ", time.gmtime()),
+        model=dict(name=model_name, model_type="dense-decoder", hidden_size=c.hidden, num_hidden_layers=c.n_layers,
+                   num_kv_shared_layers=0, num_attention_heads=c.n_heads, num_key_value_heads=c.n_kv,
+                   head_dim=c.head_dim, vocab_size=c.vocab),
+        stats=dict(ops=len(tasks), fusions=len(tasks), tasks=len(tasks),
+                   unique_kernels=len({re.sub(r"_f\d+$", "", t["kernel"]) for t in tasks})),
+        variants=[])
+    with open(os.path.join(out_dir, "manifest.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+
+
+class ArtifactRuntime:
+    """A decode loop built from an artifact directory alone (plus the parameters it names)."""
+
+    def __init__(self, art_dir: str, weights: DecoderWeights, dispatcher: Optional[Dispatcher] = None):
+        manifest = json.load(open(os.path.join(art_dir, "manifest.json")))
+        if manifest.get("schema_version") != SCHEMA_VERSION:
+            raise ValueError(f"manifest schema {manifest.get('schema_version')} is not {SCHEMA_VERSION}")  # manifest.rs:108-112
+        path = os.path.join(art_dir, "task_graph.json")
+        graph = json.load(open(path))
+        # the native loader validates version and kernel names before the device is used
+        self.d = dispatcher or Dispatcher(None, path)
+        self.scratch: Dict[str, DeviceBuffer] = {}
+        for s in graph["scratch_buffers"]:
+            self.scratch[s["role_name"]] = native.zeros(s["size_bytes"]) if s["zero_init"] else DeviceBuffer(s["size_bytes"])
+        params: Dict[str, DeviceBuffer] = {}
+        for p, W in weights.mats.items():
+            params[p + ".weight"] = W.w
+            if W.bits != 16:
+                params[p + ".scales"], params[p + ".biases"] = W.scales, W.biases
+        params.update(weights.vecs)
+        self.tasks: List[Dispatch] = []
+        for tid in graph["decode_pipeline"]:
+            t = graph["tasks"][tid]
+            slots = sorted(t["inputs"] + t["outputs"], key=lambda b: b["slot"])
+            args = []
+            for b in slots:
+                buf = params[b["source_path"]] if b["role"] == "external" else self.scratch[b["role_name"]]
+                if b["nbytes"] > buf.nbytes:
+                    raise ValueError(f"task {tid} slot {b['slot']}: binding wants {b['nbytes']} bytes, buffer has {buf.nbytes}")
+                args.append((buf.ptr, b["nbytes"]))
+            self.tasks.append(Dispatch(t["kernel"], args, dict(t["params"])))
+        u = graph["uniforms"]
+        self.uniforms = make_uniforms(self.scratch[u["token"]], self.scratch[u["step_counter"]],
+                                      self.scratch[u["hist_counter"]], self.scratch[u["history"]])
+        self.graph = self.d.build_graph(self.tasks)
+        self.model_config = graph["model_config"]
+        self._weights = weights  # keeps the parameter buffers alive
+
+    def generate(self, prompt, max_tokens: int) -> List[int]:
+        nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, 0, list(prompt))
+        out = [nxt[-1]]
+        offset = len(prompt)
+        while len(out) < max_tokens:
+            n = min(64, max_tokens - len(out), self.uniforms.hist_capacity)
+            toks, _ = self.d.decode_chunk(self.graph, self.uniforms, offset, out[-1], n)
+            out += toks
+            offset += n
+        return out

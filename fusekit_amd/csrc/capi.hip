@@ -83,6 +83,37 @@ fk_status fk_device_props_get(fk_device_props* out) {
     return FK_OK;
 }
 
+fk_status fk_target_describe(fk_target* out) {
+    if (!out) return set_error(FK_ERR_INVALID, "null out");
+    memset(out, 0, sizeof(*out));
+    // published MI355X (gfx950, CDNA4) figures
+    strncpy(out->arch, "gfx950", sizeof(out->arch) - 1);
+    out->compute_units = 256;
+    out->xcds = 8;
+    out->wave_size = 64;
+    out->simds_per_cu = 4;
+    out->vgprs_per_lane = 512;
+    out->lds_bytes_per_cu = 160 * 1024;
+    out->workgroup_threads = 256;
+    out->gemm_min_rows = 2;
+    out->gemm_rows_per_pass = 32;
+    out->hbm_bytes = 288ull << 30;
+    out->hbm_peak_bytes_per_s = 8.0e12;
+    out->mfma_bf16_peak_flops = 2.5e15;
+    const DeviceFacts* d;
+    if (device_facts(&d) == FK_OK) {
+        out->from_device = 1;
+        strncpy(out->arch, d->prop.gcnArchName, sizeof(out->arch) - 1);
+        out->compute_units = (uint32_t)d->cus;
+        out->wave_size = (uint32_t)d->prop.warpSize;
+        out->lds_bytes_per_cu = (uint32_t)d->prop.maxSharedMemoryPerMultiProcessor;
+        out->hbm_bytes = d->prop.totalGlobalMem;
+    } else {
+        set_error(FK_OK, "");
+    }
+    return FK_OK;
+}
+
 fk_status fk_alloc(size_t nbytes, void** dptr) {
     if (!dptr || nbytes == 0) return set_error(FK_ERR_INVALID, "fk_alloc: null out pointer or zero size");
     const DeviceFacts* d;

@@ -1137,6 +1137,32 @@ fk_status fk_dispatch_kernel(fk_handle h, const fk_dispatch* d, double* gpu_seco
     return fk_dispatch_batch(h, d, 1, gpu_seconds);
 }
 
+fk_status fk_plan_geometry(fk_handle h, const fk_dispatch* d, fk_launch_geometry* out) {
+    DispatcherState* ds;
+    FK_TRY(get_dispatcher(h, &ds));
+    if (!d || !out) return set_error(FK_ERR_INVALID, "null dispatch or out");
+    Dispatch disp;
+    Launch l;
+    SlotRW rw;
+    FK_TRY(copy_dispatch(*d, &disp));
+    FK_TRY(plan_dispatch(disp, &l, &rw));
+    memset(out, 0, sizeof(*out));
+    if (1 + l.then.size() > FK_MAX_TASK_KERNELS || disp.args.size() > FK_MAX_TASK_SLOTS)
+        return set_error(FK_ERR_UNSUPPORTED, "dispatch exceeds the geometry record");
+    auto put = [&](const Launch& k) {
+        const uint32_t i = out->n_kernels++;
+        out->grid[i][0] = k.grid.x; out->grid[i][1] = k.grid.y; out->grid[i][2] = k.grid.z;
+        out->threadgroup[i][0] = k.block.x; out->threadgroup[i][1] = k.block.y; out->threadgroup[i][2] = k.block.z;
+        out->lds_bytes[i] = k.shmem;
+    };
+    put(l);
+    for (const Launch& k : l.then) put(k);
+    out->n_slots = (uint32_t)disp.args.size();
+    for (uint32_t s : rw.reads) out->slot_access[s] |= 1;
+    for (uint32_t s : rw.writes) out->slot_access[s] |= 2;
+    return FK_OK;
+}
+
 fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const uint8_t* barriers, uint32_t* graph_id) {
     DispatcherState* ds;
     FK_TRY(get_dispatcher(h, &ds));

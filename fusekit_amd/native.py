@@ -62,6 +62,21 @@ class DeviceProps(C.Structure):
     ]
 
 
+class Target(C.Structure):
+    """fk_target: the gfx950 entry of the reference's ChipModel / Budgets table."""
+    _fields_ = [("arch", C.c_char * 32), ("from_device", C.c_uint32), ("compute_units", C.c_uint32),
+                ("xcds", C.c_uint32), ("wave_size", C.c_uint32), ("simds_per_cu", C.c_uint32),
+                ("vgprs_per_lane", C.c_uint32), ("lds_bytes_per_cu", C.c_uint32), ("workgroup_threads", C.c_uint32),
+                ("gemm_min_rows", C.c_uint32), ("gemm_rows_per_pass", C.c_uint32), ("hbm_bytes", C.c_uint64),
+                ("hbm_peak_bytes_per_s", C.c_double), ("mfma_bf16_peak_flops", C.c_double)]
+
+
+def target_describe() -> Target:
+    t = Target()
+    check(lib.fk_target_describe(C.byref(t)))
+    return t
+
+
 def device_props() -> DeviceProps:
     p = DeviceProps()
     check(lib.fk_device_props_get(C.byref(p)))

@@ -37,6 +37,12 @@ class _BindingUpdate(C.Structure):
     _fields_ = [("cmd_idx", C.c_uint32), ("slot", C.c_uint32), ("ptr", C.c_void_p), ("nbytes", C.c_size_t)]
 
 
+class LaunchGeometry(C.Structure):
+    """fk_launch_geometry: kernels, grid / threadgroup / LDS of each, read-write bits per slot."""
+    _fields_ = [("n_kernels", C.c_uint32), ("grid", (C.c_uint32 * 3) * 4), ("threadgroup", (C.c_uint32 * 3) * 4),
+                ("lds_bytes", C.c_uint32 * 4), ("n_slots", C.c_uint32), ("slot_access", C.c_uint8 * 32)]
+
+
 class _Uniforms(C.Structure):
     _fields_ = [("token", C.c_void_p), ("step_counter", C.c_void_p), ("hist_counter", C.c_void_p),
                 ("history", C.c_void_p), ("hist_capacity", C.c_uint32)]
@@ -79,6 +85,12 @@ class Dispatcher:
         n = C.c_size_t()
         check(lib.fk_kernel_names(self.handle, C.byref(names), C.byref(n)))
         return [names[i].decode() for i in range(n.value)]
+
+    def plan_geometry(self, d: Dispatch) -> LaunchGeometry:
+        arr, keep = _marshal([d])
+        g = LaunchGeometry()
+        check(lib.fk_plan_geometry(self.handle, C.byref(arr[0]), C.byref(g)))
+        return g
 
     def dispatch_kernel(self, d: Dispatch) -> float:
         return self.dispatch_batch([d])

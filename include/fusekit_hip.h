@@ -94,6 +94,32 @@ fk_status fk_event_destroy(fk_event e);
 fk_status fk_event_record(fk_event e, fk_stream s);
 fk_status fk_event_elapsed_ms(fk_event start, fk_event stop, float *ms); /* waits for `stop` */
 
+/* ---- target description and launch geometry ---------------------------
+ * T1  The gfx950 entry of the reference's ChipModel / Budgets table
+ *     (src/target/mod.rs:17-200): what a code generator needs to know about the
+ *     machine, plus the policy thresholds this library applies itself.  Without a
+ *     visible GPU the published MI355X figures are returned and from_device is 0. */
+typedef struct fk_target {
+    char arch[32];                  /* "gfx950..." */
+    uint32_t from_device;           /* 1: read from the running GPU, 0: published MI355X figures */
+    uint32_t compute_units;         /* 256 */
+    uint32_t xcds;                  /* 8 accelerator dies, one L2 each */
+    uint32_t wave_size;             /* 64 (the reference's simd_width) */
+    uint32_t simds_per_cu;          /* 4 */
+    uint32_t vgprs_per_lane;        /* 512 per SIMD lane, shared by the resident waves (regs_per_thread budget) */
+    uint32_t lds_bytes_per_cu;      /* 163840 (smem_per_threadgroup ceiling) */
+    uint32_t workgroup_threads;     /* 256: threadgroup size every kernel here uses (4 waves) */
+    uint32_t gemm_min_rows;         /* active rows from which the matrix-core path is taken (the reference: 8,
+                                       src/target/mod.rs:162-171; here 2 -- one weight pass serves 32 rows) */
+    uint32_t gemm_rows_per_pass;    /* 32 */
+    uint64_t hbm_bytes;
+    double hbm_peak_bytes_per_s;    /* 8.0e12, published */
+    double mfma_bf16_peak_flops;    /* 2.5e15 dense, published */
+} fk_target;
+fk_status fk_target_describe(fk_target *out);
+
+/* (T2 fk_plan_geometry is declared with the dispatcher below.) */
+
 /* ---- operator launches ------------------------------------------------ */
 
 /* K1  y = T(x @ dequant(W)^T (+ bias)).  Replaces the qGEMV inner loop
@@ -318,6 +344,25 @@ fk_status fk_dispatcher_stream(fk_handle h, fk_stream *out);
 /* dispatch_kernel (lib.rs:398) / dispatch_batch (lib.rs:1723): launch and wait, GPU seconds out */
 fk_status fk_dispatch_kernel(fk_handle h, const fk_dispatch *d, double *gpu_seconds);
 fk_status fk_dispatch_batch(fk_handle h, const fk_dispatch *list, size_t n, double *gpu_seconds);
+/* T2  Launch geometry and slot access of one dispatch, as the planners decide it: what the
+ *     reference computes in kernel_threadgroup_for / kernel_grid_threads_impl and records per
+ *     task in task_graph.json (src/codegen/kernels/mod.rs:5694, 6218; task_graph_json.rs
+ *     grid_threads / threadgroup).  A dispatch may expand to up to FK_MAX_TASK_KERNELS kernels
+ *     that run back to back (a split-k or routed reduction).  slot_access[i]: bit 0 = the
+ *     kernels read slot i, bit 1 = they write it (the hazard mask of
+ *     python/fusekit_runtime/dispatch.py:36-100 is derived from these). */
+#define FK_MAX_TASK_KERNELS 4
+#define FK_MAX_TASK_SLOTS 32
+typedef struct fk_launch_geometry {
+    uint32_t n_kernels;
+    uint32_t grid[FK_MAX_TASK_KERNELS][3];        /* workgroups per axis */
+    uint32_t threadgroup[FK_MAX_TASK_KERNELS][3]; /* threads per workgroup */
+    uint32_t lds_bytes[FK_MAX_TASK_KERNELS];
+    uint32_t n_slots;
+    uint8_t slot_access[FK_MAX_TASK_SLOTS];
+} fk_launch_geometry;
+fk_status fk_plan_geometry(fk_handle h, const fk_dispatch *d, fk_launch_geometry *out);
+
 /* build_icb (lib.rs:461): pre-encode the list as one hipGraph.  `barriers`
  * NULL = edges from the read/write tables; barriers[i] != 0 additionally makes
  * command i wait for every earlier command. */

@@ -76,3 +76,23 @@ def test_decoder_config_byte_accounting():
     assert cfg.token_bytes(512) == 2043740160 + 777912320 + 75497472     # + tied bf16 LM head + KV at ctx 512
     assert DecoderConfig(**DENSE_4B, bits=8).n_layers * DecoderConfig(**DENSE_4B, bits=8).layer_param_bytes() == 3860398080
     assert DecoderConfig(**DENSE_4B, bits=16).n_layers * DecoderConfig(**DENSE_4B, bits=16).layer_param_bytes() == 7266631680
+
+
+def test_target_description_without_a_gpu():
+    """T1: fk_target_describe answers with the published MI355X figures when no device is visible."""
+    import ctypes as C
+    import os
+    lib = C.CDLL(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "fusekit_amd", "libfusekit_hip.so"))
+
+    class Target(C.Structure):
+        _fields_ = [("arch", C.c_char * 32), ("from_device", C.c_uint32), ("compute_units", C.c_uint32),
+                    ("xcds", C.c_uint32), ("wave_size", C.c_uint32), ("simds_per_cu", C.c_uint32),
+                    ("vgprs_per_lane", C.c_uint32), ("lds_bytes_per_cu", C.c_uint32), ("workgroup_threads", C.c_uint32),
+                    ("gemm_min_rows", C.c_uint32), ("gemm_rows_per_pass", C.c_uint32), ("hbm_bytes", C.c_uint64),
+                    ("hbm_peak_bytes_per_s", C.c_double), ("mfma_bf16_peak_flops", C.c_double)]
+    t = Target()
+    assert lib.fk_target_describe(C.byref(t)) == 0
+    assert t.arch.startswith(b"gfx950") and t.wave_size == 64 and t.workgroup_threads == 256
+    if not t.from_device:
+        assert (t.compute_units, t.xcds, t.lds_bytes_per_cu) == (256, 8, 160 * 1024)
+        assert t.hbm_peak_bytes_per_s == 8.0e12 and t.hbm_bytes == 288 << 30

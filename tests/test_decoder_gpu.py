@@ -296,3 +296,33 @@ def test_4b_class_greedy_32_tokens_match_oracle(fk):
     rel = np.linalg.norm(f_got - f_ref) / np.linalg.norm(f_ref)
     print(f"last-step logits rel-L2 {rel:.3e}")
     assert rel <= 5e-2
+
+
+def test_artifact_round_trip_and_launch_geometry(fk, tmp_path):
+    """task_graph.json / manifest.json written from a runtime, read back by a consumer that knows
+    only the files and the parameter tree: same tokens.  Also the geometry query behind the file."""
+    from fusekit_amd.artifact import ArtifactRuntime, write_artifact
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    import json
+    cfg = _small_cfg(bits=4, qk_norm=True, qkv_bias=True)
+    W = DecoderWeights.random_init(cfg, seed=21)
+    rt = DecoderRuntime(cfg, W)
+    prompt = [3, 1999, 42]
+    want, _, _ = rt.generate(prompt, 12)
+    write_artifact(rt, str(tmp_path), "tiny")
+    tg = json.load(open(tmp_path / "task_graph.json"))
+    assert tg["version"] == 2 and tg["active_m"] == 1 and len(tg["tasks"]) == len(rt.tasks)
+    assert json.load(open(tmp_path / "manifest.json"))["stats"]["tasks"] == len(rt.tasks)
+    qkv = next(t for t in tg["tasks"] if t["kernel"].startswith("fusekit_rmsnorm_qkv"))
+    assert qkv["threadgroup"] == [256, 1, 1] and qkv["grid_threads"][0] % 256 == 0 and qkv["layer_idx"] == 0
+    assert [b["role_name"] for b in qkv["outputs"]] == ["q", "k", "v"]
+    assert any(b.get("source_path") == "layers.0.self_attn.q_proj.weight" for b in qkv["inputs"])
+    art = ArtifactRuntime(str(tmp_path), W)
+    assert art.generate(prompt, 12) == want
+    # a damaged artifact is refused with the reference's error classes
+    tg["version"] = 3
+    json.dump(tg, open(tmp_path / "task_graph.json", "w"))
+    with pytest.raises(fk.InvalidArgument):
+        ArtifactRuntime(str(tmp_path), W)
+    t = fk.target_describe()
+    assert t.from_device == 1 and t.wave_size == 64 and t.compute_units >= 64 and t.arch.startswith(b"gfx950")
