@@ -1,6 +1,8 @@
 // Device side of the split-K attention decode: SdpaArgs, the per-work-item
 // function sdpa_block and the stand-alone kernel.  See sdpa.hip for the scheme.
 #pragma once
+#include <stddef.h>
+
 #include "fk_device.hpp"
 #include "rope_device.hpp"
 
@@ -14,7 +16,7 @@ namespace fk {
 
 constexpr int kSdpaBlock = 256;
 constexpr int kSdpaWaves = kSdpaBlock / kWave;
-constexpr int kSdpaSteps = 8;       // K rows (and at most as many V rows) each lane owns per range
+constexpr int kSdpaSteps = 4;       // K rows (and at most as many V rows) each lane owns per range
 constexpr int kSdpaStepsFused = 4;  // inside the whole-token kernel: half the registers, twice the ranges
 
 struct SdpaArgs {
@@ -65,15 +67,25 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
                                            uint32_t gz, uint32_t gz_count, float* lds) {
     constexpr int kSteps = FUSED ? kSdpaStepsFused : kSdpaSteps;
     const uint32_t span = a.chunk_len * a.chunks_per_block;  // cache positions per block
-    const uint32_t n_active = (kv_len + span - 1) / span;
-    if (split >= n_active) return;  // uniform: whole block leaves before any barrier
-
+    const uint32_t blk0 = split * span;
     const uint32_t G = a.n_heads / a.n_kv;
     const uint32_t h0 = kvh * G + gz * GT;
     const uint32_t gcount = (G - gz * GT) < (uint32_t)GT ? (G - gz * GT) : (uint32_t)GT;
-    const uint32_t blk0 = split * span;
-    const uint32_t blk_keys = (kv_len - blk0) < span ? (kv_len - blk0) : span;
-    const uint32_t n_chunks = (blk_keys + a.chunk_len - 1) / a.chunk_len;
+    // Stand-alone kernel: kv_len is still on its way from memory (a scalar load the
+    // caller issued); nothing below touches it until the first K/V rows have been
+    // requested, so that round trip overlaps the cache reads.
+    uint32_t n_active = 0, blk_keys = 0, n_chunks = 0;
+    auto settle = [&]() {
+        n_active = (kv_len + span - 1) / span;
+        if (split < n_active) {
+            blk_keys = (kv_len - blk0) < span ? (kv_len - blk0) : span;
+            n_chunks = (blk_keys + a.chunk_len - 1) / a.chunk_len;
+        }
+    };
+    if constexpr (FUSED) {
+        settle();
+        if (split >= n_active) return;  // uniform: whole block leaves before any barrier
+    }
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     FK_SDPA_STAMP(0);
 
@@ -82,7 +94,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     float* stat = red + (kSdpaBlock / a.lpv) * GT * a.v_dim;  // m[GT], l[GT], misc
     uint16_t* qn = reinterpret_cast<uint16_t*>(stat + kSdpaStatFloats);  // fused: [GT][qk_dim] + k row
     uint16_t* kn = qn + GT * a.qk_dim;
-    const uint32_t pos = kv_len - 1;  // fused: position of the new token
+    const uint32_t pos = FUSED ? kv_len - 1 : 0u;  // fused: position of the new token
     const bool blk_owner = FUSED && pos >= blk0 && pos < blk0 + blk_keys;
 
     if constexpr (FUSED) {
@@ -140,37 +152,71 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
     }
 
+    // All K and V loads of a range are issued up front (the range is sized so that
+    // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
+    // Stand-alone: every row that exists in the cache allocation is requested, whether
+    // or not it is below kv_len (rows past kv_len are masked where they are used).
+    uint4 kc[kSteps], vc[kSteps];
+    uint4 kn_[kSteps], vn_[kSteps];  // stand-alone: the next range, in flight while this one is consumed
+    auto request_rows = [&](uint4(&kd)[kSteps], uint4(&vd)[kSteps], uint32_t key0, uint32_t nkeys, bool owner,
+                            uint32_t jpos) {
+        const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * ck;
+        const uint16_t* vbase = a.v + ((size_t)kvh * a.capacity + key0) * a.v_dim + 8 * cv;
+        if constexpr (!FUSED) {
+            // Straight-line, clamped (row to the last row of the allocation, a lane beyond
+            // the head width to column 0): no branch separates the loads, so the compiler
+            // can wait for exactly the rows it needs while later requests stay in flight.
+            const uint16_t* khead = a.k + (size_t)kvh * a.capacity * a.qk_dim + (kcol_ok ? 8 * ck : 0u);
+            const uint16_t* vhead = a.v + (size_t)kvh * a.capacity * a.v_dim + (vcol_ok ? 8 * cv : 0u);
+            const uint32_t last = a.capacity - 1;
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                const uint32_t r = key0 + kslot + u * kslots;
+                kd[u] = *reinterpret_cast<const uint4*>(khead + (size_t)(r < last ? r : last) * a.qk_dim);
+            }
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                const uint32_t r = key0 + vslot + u * vslots;
+                vd[u] = *reinterpret_cast<const uint4*>(vhead + (size_t)(r < last ? r : last) * a.v_dim);
+            }
+            return;
+        }
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = kslot + u * kslots;
+            kd[u] = make_uint4(0, 0, 0, 0);
+            if (kcol_ok && j < nkeys && !(owner && j == jpos))
+                kd[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * a.qk_dim);
+        }
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const uint32_t j = vslot + u * vslots;
+            vd[u] = make_uint4(0, 0, 0, 0);
+            if (vcol_ok && j < nkeys) {
+                const uint16_t* src = vbase + (size_t)j * a.v_dim;
+                if (owner && j == jpos) {  // the new row, not yet cached
+                    vd[u] = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_dim + 8 * cv);
+                } else {
+                    vd[u] = *reinterpret_cast<const uint4*>(src);
+                }
+            }
+        }
+    };
+    if constexpr (!FUSED) {
+        request_rows(kc, vc, blk0, 0, false, 0);
+        settle();
+        if (split >= n_active) return;  // uniform: whole block leaves before any barrier
+    }
+
     for (uint32_t c = 0; c < n_chunks; ++c) {
     const uint32_t key0 = blk0 + c * a.chunk_len;
     const uint32_t nkeys = (kv_len - key0) < a.chunk_len ? (kv_len - key0) : a.chunk_len;
     const bool owner = FUSED && pos >= key0 && pos < key0 + nkeys;
     const uint32_t jpos = pos - key0;
-    // All K and V loads of the range are issued up front (the range is sized so that
-    // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
-    uint4 kc[kSteps], vc[kSteps];
-    {
-        const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * ck;
-        const uint16_t* vbase = a.v + ((size_t)kvh * a.capacity + key0) * a.v_dim + 8 * cv;
-#pragma unroll
-        for (int u = 0; u < kSteps; ++u) {
-            const uint32_t j = kslot + u * kslots;
-            kc[u] = make_uint4(0, 0, 0, 0);
-            if (kcol_ok && j < nkeys && !(owner && j == jpos))
-                kc[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * a.qk_dim);
-        }
-#pragma unroll
-        for (int u = 0; u < kSteps; ++u) {
-            const uint32_t j = vslot + u * vslots;
-            vc[u] = make_uint4(0, 0, 0, 0);
-            if (vcol_ok && j < nkeys) {
-                const uint16_t* src = vbase + (size_t)j * a.v_dim;
-                if (owner && j == jpos) {  // the new row, not yet cached
-                    vc[u] = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_dim + 8 * cv);
-                } else {
-                    vc[u] = *reinterpret_cast<const uint4*>(src);
-                }
-            }
-        }
+    if constexpr (FUSED) {
+        request_rows(kc, vc, key0, nkeys, owner, jpos);
+    } else {
+        if (c + 1 < n_chunks) request_rows(kn_, vn_, key0 + a.chunk_len, 0, false, 0);
     }
 
     FK_SDPA_STAMP(1);
@@ -242,8 +288,10 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         const uint32_t j = vslot + u * vslots;
         const uint32_t jj = j < nkeys ? j : 0u;
         const float live = j < nkeys ? 1.f : 0.f;
-        const float f[8] = {bf16_lo(vc[u].x), bf16_hi(vc[u].x), bf16_lo(vc[u].y), bf16_hi(vc[u].y),
-                            bf16_lo(vc[u].z), bf16_hi(vc[u].z), bf16_lo(vc[u].w), bf16_hi(vc[u].w)};
+        // rows past kv_len were requested speculatively: their bits may be anything
+        const uint4 vv = (FUSED || (j < nkeys && vcol_ok)) ? vc[u] : make_uint4(0, 0, 0, 0);
+        const float f[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
+                            bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
 #pragma unroll
         for (int h = 0; h < GT; ++h) {
             const float p = s[h * a.chunk_len + jj] * live;
@@ -251,7 +299,16 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
         }
     }
-    if (c + 1 < n_chunks) __syncthreads();  // the scores are overwritten by the next range
+    if (c + 1 < n_chunks) {
+        __syncthreads();  // the scores are overwritten by the next range
+        if constexpr (!FUSED) {
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                kc[u] = kn_[u];
+                vc[u] = vn_[u];
+            }
+        }
+    }
     }  // ranges of this block
     FK_SDPA_STAMP(5);
 
@@ -306,53 +363,50 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     if (tid == 0)  // ready for the next launch (or the next layer of this one)
         __hip_atomic_store(&a.counters[kvh * gz_count + gz], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-    // One wave per head, no block barriers: M = max m_s, w_s = exp(m_s - M) (kept in
-    // registers, lane s % 64 slot s / 64, for up to 256 ranges), L = sum l_s w_s, then
-    // each lane adds its output dims over the ranges in index order.
-    constexpr uint32_t kWSlots = 4;
+    // One wave per head, no block barriers.  The ranges are taken 16 at a time: (m, l) of
+    // each and this lane's two output dims of each are requested together (one memory
+    // round trip per 16 ranges) and folded into a running (M, L, o) with the usual
+    // rescaling, in range order, so the result does not depend on arrival order.
+    constexpr uint32_t kBatch = 16;
     const uint32_t row = a.v_dim + 2;
     for (uint32_t h = wave; h < gcount; h += kSdpaWaves) {
         const float* ph = a.partials + (size_t)(h0 + h) * a.n_splits * row;
-        float m = -INFINITY;
-        for (uint32_t sp = lane; sp < n_active; sp += kWave) m = fmaxf(m, ld_f32<true>(ph + (size_t)sp * row));
-        m = wave_max(m);
-        float wreg[kWSlots];
-        float l = 0.f;
+        for (uint32_t d2 = lane; d2 < ((a.v_dim >> 1) + kWave - 1) / kWave * kWave; d2 += kWave) {
+            const bool live = d2 < (a.v_dim >> 1);
+            const float* pd = ph + 2 + 2 * (live ? d2 : 0u);
+            float M = -INFINITY, L = 0.f, o0 = 0.f, o1 = 0.f;
+            for (uint32_t base = 0; base < n_active; base += kBatch) {
+                float pm[kBatch], pl[kBatch], p0[kBatch], p1[kBatch];
 #pragma unroll
-        for (uint32_t i = 0; i < kWSlots; ++i) {
-            const uint32_t sp = lane + i * kWave;
-            wreg[i] = 0.f;
-            if (sp < n_active) {
-                wreg[i] = expf(ld_f32<true>(ph + (size_t)sp * row) - m);
-                l = fmaf(ld_f32<true>(ph + (size_t)sp * row + 1), wreg[i], l);
-            }
-        }
-        for (uint32_t sp = lane + kWSlots * kWave; sp < n_active; sp += kWave)
-            l = fmaf(ld_f32<true>(ph + (size_t)sp * row + 1), expf(ld_f32<true>(ph + (size_t)sp * row) - m), l);
-        l = wave_sum(l);
-        const float inv_l = 1.0f / l;
-        for (uint32_t d2 = lane; d2 < (a.v_dim >> 1); d2 += kWave) {
-            const float* pd = ph + 2 + 2 * d2;
-            float o0 = 0.f, o1 = 0.f;
-#pragma unroll
-            for (uint32_t i = 0; i < kWSlots; ++i) {
-                const uint32_t lim = n_active > i * kWave ? (n_active - i * kWave < (uint32_t)kWave ? n_active - i * kWave : (uint32_t)kWave) : 0u;
-#pragma unroll 8
-                for (uint32_t lo = 0; lo < lim; ++lo) {
-                    const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wreg[i]), (int)lo));
-                    const float* p = pd + (size_t)(i * kWave + lo) * row;
-                    o0 = fmaf(ld_f32<true>(p), w, o0);
-                    o1 = fmaf(ld_f32<true>(p + 1), w, o1);
+                for (uint32_t i = 0; i < kBatch; ++i) {
+                    const size_t o = (size_t)(base + i < n_active ? base + i : base) * row;
+                    pm[i] = ld_f32<true>(ph + o);
+                    pl[i] = ld_f32<true>(ph + o + 1);
+                    p0[i] = ld_f32<true>(pd + o);
+                    p1[i] = ld_f32<true>(pd + o + 1);
                 }
+                float mn = fmaxf(M, pm[0]);
+#pragma unroll
+                for (uint32_t i = 1; i < kBatch; ++i) mn = base + i < n_active ? fmaxf(mn, pm[i]) : mn;
+                const float alpha = base ? expf(M - mn) : 0.f;
+                L *= alpha;
+                o0 *= alpha;
+                o1 *= alpha;
+#pragma unroll
+                for (uint32_t i = 0; i < kBatch; ++i) {
+                    const float w = base + i < n_active ? expf(pm[i] - mn) : 0.f;
+                    L = fmaf(pl[i], w, L);
+                    o0 = fmaf(p0[i], w, o0);
+                    o1 = fmaf(p1[i], w, o1);
+                }
+                M = mn;
             }
-            for (uint32_t sp = kWSlots * kWave; sp < n_active; ++sp) {
-                const float w = expf(ld_f32<true>(ph + (size_t)sp * row) - m);
-                o0 = fmaf(ld_f32<true>(pd + (size_t)sp * row), w, o0);
-                o1 = fmaf(ld_f32<true>(pd + (size_t)sp * row + 1), w, o1);
+            const float inv_l = 1.0f / L;
+            if (live) {
+                uint16_t* dst = a.out + (size_t)(h0 + h) * a.v_dim + 2 * d2;
+                st_u16<FUSED>(dst, f32_to_bf16_bits(o0 * inv_l));
+                st_u16<FUSED>(dst + 1, f32_to_bf16_bits(o1 * inv_l));
             }
-            uint16_t* dst = a.out + (size_t)(h0 + h) * a.v_dim + 2 * d2;
-            st_u16<FUSED>(dst, f32_to_bf16_bits(o0 * inv_l));
-            st_u16<FUSED>(dst + 1, f32_to_bf16_bits(o1 * inv_l));
         }
     }
     FK_SDPA_STAMP(9);
@@ -361,7 +415,16 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 template <int GT>
 __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs a) {
     extern __shared__ __align__(16) float lds[];
-    const uint32_t kv_len = a.kv_len_ptr ? *a.kv_len_ptr : a.kv_len_imm;
+    // One unconditional load (the immediate is read from the kernel-argument segment
+    // when there is no device scalar): a load under a branch would be waited for at
+    // the join, ahead of the cache reads it is meant to overlap.
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t* imm = (const uint32_t*)((const char*)__builtin_amdgcn_kernarg_segment_ptr() +
+                                            offsetof(SdpaArgs, kv_len_imm));
+#else
+    const uint32_t* imm = &a.kv_len_imm;
+#endif
+    const uint32_t kv_len = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
     sdpa_block<GT, false, SdpaArgs>(a, kv_len, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
 }
 
