@@ -12,7 +12,7 @@ Prints ONE JSON line: value = generated tokens/s (wall clock around the K timed 
                   its average launch duration, measured here with HIP events on the launch stream
                   over the 36 layers' distinct weights (985 MB, larger than any cache),
   cpu_baseline -- the CPU oracle (C restatement of the reference semantics) decoding the same
-                  model on the host cores, bounded to a couple of tokens.
+                  model on the host cores, bounded to --cpu-tokens decode steps (about 10 s of CPU work).
 """
 import argparse
 import json
@@ -38,7 +38,8 @@ def main() -> int:
     ap.add_argument("--bits", type=int, default=4, choices=[4, 8, 16])
     ap.add_argument("--prompt", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-tokens", type=int, default=2)
+    ap.add_argument("--cpu-tokens", type=int, default=24,
+                    help="decode steps the CPU oracle runs for cpu_baseline (about 10 s on 16 cores)")
     ap.add_argument("--per-kernel", action="store_true", help="print per-family GPU time of one token to stderr")
     ap.add_argument("--layers", type=int, default=0, help="experiment only: override the layer count (not the headline config)")
     ap.add_argument("--calibrate-copy", action="store_true",
