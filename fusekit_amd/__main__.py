@@ -1,0 +1,62 @@
+"""python -m fusekit_amd <command>
+
+  info                                   the device as the backend sees it (fk_target_describe)
+  generate --model DIR --ids 1,2,3 [--max-tokens N] [--capacity C]
+                                         greedy decode of an mlx-lm format checkpoint (token ids in,
+                                         token ids out; no tokenizer is bundled)
+  export-random --out DIR [--bits 4] [--layers 2] ...
+                                         write a small random-init model in the mlx-lm file layout
+"""
+import argparse
+import json
+import sys
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(prog="python -m fusekit_amd")
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    sub.add_parser("info")
+    g = sub.add_parser("generate")
+    g.add_argument("--model", required=True)
+    g.add_argument("--ids", required=True, help="comma-separated prompt token ids")
+    g.add_argument("--max-tokens", type=int, default=32)
+    g.add_argument("--capacity", type=int, default=1024)
+    e = sub.add_parser("export-random")
+    e.add_argument("--out", required=True)
+    e.add_argument("--bits", type=int, default=4, choices=[4, 8, 16])
+    e.add_argument("--layers", type=int, default=2)
+    e.add_argument("--hidden", type=int, default=256)
+    e.add_argument("--heads", type=int, default=4)
+    e.add_argument("--kv-heads", type=int, default=2)
+    e.add_argument("--head-dim", type=int, default=64)
+    e.add_argument("--inter", type=int, default=512)
+    e.add_argument("--vocab", type=int, default=2000)
+    e.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+
+    from . import native as fk
+    if args.cmd == "info":
+        t = fk.target_describe()
+        print(json.dumps({f: (getattr(t, f).decode() if isinstance(getattr(t, f), bytes) else getattr(t, f))
+                          for f, _ in t._fields_}, indent=1))
+        return 0
+    from .decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    if args.cmd == "export-random":
+        from .checkpoint import save_mlx_checkpoint
+        cfg = DecoderConfig(n_layers=args.layers, hidden=args.hidden, n_heads=args.heads, n_kv=args.kv_heads,
+                            head_dim=args.head_dim, inter=args.inter, vocab=args.vocab, bits=args.bits, qk_norm=True,
+                            swiglu_variant=1)
+        save_mlx_checkpoint(args.out, cfg, DecoderWeights.random_init(cfg, seed=args.seed))
+        print(f"wrote {args.out}/config.json and model.safetensors")
+        return 0
+    from .checkpoint import load_mlx_checkpoint
+    cfg, w = load_mlx_checkpoint(args.model, capacity=args.capacity)
+    rt = DecoderRuntime(cfg, w)
+    prompt = [int(t) for t in args.ids.split(",") if t.strip()]
+    toks, gpu_s, steps = rt.generate(prompt, args.max_tokens)
+    print(json.dumps({"tokens": toks, "decode_tok_per_s": round(steps / gpu_s, 1) if gpu_s else None}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -198,9 +198,10 @@ class DecoderRuntime:
             return f"fusekit_{kind}_f{fid[0]}"
 
         t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
-        emb = w.mats["embed_tokens"]
-        t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token), arg(emb.w), arg(self.x[0])],
-                          dict(bits=16, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
+        emb = w.mats["embed_tokens"]       # dense bf16 or MLX-affine (4-bit checkpoints quantise it too)
+        head = w.mats.get("lm_head", emb)  # untied output projection when the checkpoint has one
+        t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token)] + self._wargs(emb) + [arg(self.x[0])],
+                          dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
         for l in range(c.n_layers):
             p = f"layers.{l}."
             Wq, Wk, Wv = (w.mats[p + f"self_attn.{n}_proj"] for n in "qkv")
@@ -255,8 +256,8 @@ class DecoderRuntime:
                               [arg(self.mid)] + self._wargs(Wd) + [arg(self.x[1]), arg(self.x[0])],
                               dict(q, m=c.inter, n=c.hidden)))
         t.append(Dispatch(name("final_rmsnorm_lm_head"),
-                          [arg(self.x[0]), arg(w.vecs["final_norm"]), arg(emb.w), arg(self.logits)],
-                          dict(bits=16, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
+                          [arg(self.x[0]), arg(w.vecs["final_norm"])] + self._wargs(head) + [arg(self.logits)],
+                          dict(bits=head.bits, group=head.group or 64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
         t.append(Dispatch(name("argmax_logits_decode"),
                           [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history),
                            arg(self.hist_counter)], dict(vocab=c.vocab)))

@@ -93,9 +93,10 @@ class OracleDecoder:
             self.keep += [ck, cv]
             L.cache_k, L.cache_v = ck.ctypes.data_as(u16p), cv.ctypes.data_as(u16p)
         emb = mat("embed_tokens")
+        head = mat("lm_head") if "lm_head" in weights.mats else emb
         self.model = oracle.Model(cfg.n_layers, cfg.hidden, cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab,
                                   cfg.eps, cfg.theta, 1.0 / np.sqrt(cfg.head_dim), 1.0, cfg.swiglu_variant,
-                                  cfg.capacity, emb, emb, vec("final_norm"), self.layers)
+                                  cfg.capacity, emb, head, vec("final_norm"), self.layers)
 
     def step(self, token: int, offset: int, want_logits: bool = False):
         logits = np.empty(self.cfg.vocab, np.uint16) if want_logits else None

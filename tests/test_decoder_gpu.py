@@ -326,3 +326,29 @@ def test_artifact_round_trip_and_launch_geometry(fk, tmp_path):
         ArtifactRuntime(str(tmp_path), W)
     t = fk.target_describe()
     assert t.from_device == 1 and t.wave_size == 64 and t.compute_units >= 64 and t.arch.startswith(b"gfx950")
+
+
+@pytest.mark.parametrize("bits,untied", [(4, False), (8, True), (16, False)])
+def test_mlx_checkpoint_round_trip(fk, tmp_path, bits, untied):
+    """A model saved in the mlx-lm file layout and loaded back decodes the same tokens; with a
+    quantised embedding / untied head the GPU still agrees with the oracle."""
+    from fusekit_amd.checkpoint import load_mlx_checkpoint, save_mlx_checkpoint
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights, quantize_on_device, _synth
+    cfg = _small_cfg(bits=bits, qk_norm=True, qkv_bias=(bits == 8), swiglu_variant=1)
+    W = DecoderWeights.random_init(cfg, seed=31)
+    if bits != 16:   # mlx 4/8-bit checkpoints quantise the embedding as well
+        tmp = fk.DeviceBuffer(cfg.vocab * cfg.hidden * 4)
+        _synth(tmp, cfg.vocab * cfg.hidden, 777, 0.0, 0.02, 0)
+        W.mats["embed_tokens"] = quantize_on_device(tmp, cfg.vocab, cfg.hidden, bits, cfg.group)
+        if untied:
+            _synth(tmp, cfg.vocab * cfg.hidden, 778, 0.0, 0.02, 0)
+            W.mats["lm_head"] = quantize_on_device(tmp, cfg.vocab, cfg.hidden, bits, cfg.group)
+    prompt = [9, 1500, 77]
+    want, _, _ = DecoderRuntime(cfg, W).generate(prompt, 10)
+    ref, margins = OracleDecoder(cfg, W).generate(prompt, 10)
+    assert want == ref, margins
+    save_mlx_checkpoint(str(tmp_path), cfg, W)
+    cfg2, W2 = load_mlx_checkpoint(str(tmp_path), capacity=cfg.capacity)
+    assert (cfg2.bits, cfg2.qk_norm, cfg2.qkv_bias, "lm_head" in W2.mats) == (bits, True, bits == 8, untied and bits != 16)
+    got, _, _ = DecoderRuntime(cfg2, W2).generate(prompt, 10)
+    assert got == want
