@@ -382,6 +382,53 @@ fk_status fk_qkv_rope_store_decode(uint16_t* q, const uint16_t* k, const uint16_
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,
+                          fk_stream s) {
+    Launch l;
+    FK_TRY(plan_rmsnorm_rows(x, w, eps, rows, hidden, y, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_embed_lookup_rows(const fk_weight* E, const uint32_t* d_tokens, uint32_t rows, float out_scale, uint16_t* x,
+                               fk_stream s) {
+    if (!d_tokens) return set_error(FK_ERR_INVALID, "fk_embed_lookup_rows: null token array");
+    Launch l;
+    FK_TRY(plan_embed(E, d_tokens, 0, out_scale, x, &l, rows));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_qkv_rope_store_rows(uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_norm,
+                                 const uint16_t* k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                 uint32_t rope_dims, float theta, float eps, uint32_t rows, uint32_t offset,
+                                 uint32_t capacity, uint16_t* cache_k, uint16_t* cache_v, fk_stream s) {
+    if (rows == 0) return set_error(FK_ERR_INVALID, "fk_qkv_rope_store_rows: zero rows");
+    RopeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.k = k; a.v = v; a.q_norm = q_norm; a.k_norm = k_norm;
+    a.n_q = n_heads; a.n_kv = n_kv; a.head_dim = head_dim; a.k_dim = head_dim; a.v_dim = head_dim;
+    a.rope_dims = rope_dims;
+    a.offset_imm = offset;
+    a.capacity = capacity;
+    a.cache_k = cache_k; a.cache_v = cache_v;
+    a.eps = eps; a.base_log2 = theta_log2(theta);
+    a.rope_on = rope_dims ? 1u : 0u;
+    a.rows = rows;
+    Launch l;
+    FK_TRY(plan_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_sdpa_decode_rows(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,
+                              uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim,
+                              uint32_t v_dim, uint32_t capacity, float scale, float* partials, uint32_t* counters,
+                              fk_stream s) {
+    if (rows == 0 || kv_len == 0) return set_error(FK_ERR_INVALID, "fk_sdpa_decode_rows: zero rows or kv length");
+    Launch l;
+    FK_TRY(plan_sdpa_decode(q, cache_k, cache_v, out, nullptr, kv_len, kv_len + rows - 1, n_heads, n_kv, qk_dim, v_dim,
+                            capacity, scale, partials, counters, &l, rows));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                   size_t* partial_bytes, size_t* counter_bytes) {
     if (!partial_bytes || !counter_bytes || max_len == 0 || qk_dim < 8 || v_dim < 8)

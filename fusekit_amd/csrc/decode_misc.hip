@@ -17,14 +17,15 @@ namespace fk {
 // with the reference's two roundings, T(w * T(x * r)), and the rotation acts on
 // those T values.
 __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
-    const uint32_t b = blockIdx.x, lane = threadIdx.x;
-    const uint32_t pos = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
-    const uint32_t wpos = a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos);
+    const uint32_t b = blockIdx.x, lane = threadIdx.x, tr = blockIdx.y;  // tr: active token row
+    const uint32_t pos0 = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
+    const uint32_t pos = pos0 + tr;
+    const uint32_t wpos = (a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos0)) + tr;
     const uint32_t row = wpos % a.capacity;
 
     if (b >= a.n_q + a.n_kv) {  // V head: straight copy into the cache row
         const uint32_t h = b - a.n_q - a.n_kv;
-        const uint16_t* src = a.v + (size_t)h * a.v_dim;
+        const uint16_t* src = a.v + ((size_t)tr * a.n_kv + h) * a.v_dim;
         uint16_t* dst = a.cache_v + ((size_t)h * a.capacity + row) * a.v_dim;
         for (uint32_t d = lane; d < a.v_dim; d += kWave) dst[d] = src[d];
         return;
@@ -32,8 +33,8 @@ __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
     const bool is_q = b < a.n_q;
     const uint32_t h = is_q ? b : b - a.n_q;
     const uint32_t dim = is_q ? a.head_dim : a.k_dim;
-    const uint16_t* src = is_q ? a.q + (size_t)h * dim : a.k + (size_t)h * dim;
-    uint16_t* dst = is_q ? a.q + (size_t)h * dim : a.cache_k + ((size_t)h * a.capacity + row) * dim;
+    const uint16_t* src = is_q ? a.q + ((size_t)tr * a.n_q + h) * dim : a.k + ((size_t)tr * a.n_kv + h) * dim;
+    uint16_t* dst = is_q ? a.q + ((size_t)tr * a.n_q + h) * dim : a.cache_k + ((size_t)h * a.capacity + row) * dim;
     const uint16_t* nw = is_q ? a.q_norm : a.k_norm;
 
     head_transform(src, dst, nw, dim, a.rope_on ? a.rope_dims : 0u, pos, a.base_log2, a.eps, nw != nullptr || !is_q,
@@ -52,8 +53,11 @@ fk_status plan_rope_store(const RopeArgs& in, Launch* out) {
                       (a.n_kv && a.rope_dims > a.k_dim)))
         return set_error(FK_ERR_INVALID, "rope: rope_dims must be even and within the head");
     if (!a.capacity) a.capacity = 1;
+    if (!a.rows) a.rows = 1;
+    if (a.rows > 65535) return set_error(FK_ERR_UNSUPPORTED, "rope: too many rows");
+    if (a.n_kv && a.rows > a.capacity) return set_error(FK_ERR_INVALID, "rope: more rows than the cache holds");
     out->func = reinterpret_cast<const void*>(&rope_store_kernel);
-    out->grid = dim3(a.n_q + 2 * a.n_kv, 1, 1);
+    out->grid = dim3(a.n_q + 2 * a.n_kv, a.rows, 1);
     out->block = dim3(kWave, 1, 1);
     out->shmem = 0;
     out->set_args(a);
@@ -75,9 +79,9 @@ struct EmbedArgs {
 // x = T(embed[token] * scale); quantised rows unpack (word >> ((d % lanes) * bits)) & mask
 // (reference embed_lookup_decode.rs:74-99).
 __global__ __launch_bounds__(256) void embed_lookup_kernel(const EmbedArgs a) {
-    const uint32_t d = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t d = blockIdx.x * 256 + threadIdx.x, tr = blockIdx.y;
     if (d >= a.hidden) return;
-    uint32_t token = a.token_ptr ? *a.token_ptr : a.token_imm;
+    uint32_t token = a.token_ptr ? a.token_ptr[tr] : a.token_imm;
     if (token >= a.vocab) token = a.vocab - 1;  // never read outside the table
     float val;
     if (a.bits == 16) {
@@ -89,11 +93,11 @@ __global__ __launch_bounds__(256) void embed_lookup_kernel(const EmbedArgs a) {
         const size_t g = (size_t)token * (a.hidden / a.group) + d / a.group;
         val = (float)qv * bf16_bits_to_f32(a.scales[g]) + bf16_bits_to_f32(a.biases[g]);
     }
-    a.x[d] = (uint16_t)f32_to_bf16_bits(val * a.out_scale);
+    a.x[(size_t)tr * a.hidden + d] = (uint16_t)f32_to_bf16_bits(val * a.out_scale);
 }
 
 fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
-                     uint16_t* x, Launch* out) {
+                     uint16_t* x, Launch* out, uint32_t rows) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!E || !E->w || !x) return set_error(FK_ERR_INVALID, "embed: null pointer");
@@ -108,8 +112,10 @@ fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t tok
     a.vocab = E->n; a.hidden = E->k; a.bits = E->bits; a.group = E->group;
     a.out_scale = out_scale;
     a.x = x;
+    if (rows == 0 || rows > 65535 || (rows > 1 && !token_ptr))
+        return set_error(FK_ERR_INVALID, "embed: rows need a device token array");
     out->func = reinterpret_cast<const void*>(&embed_lookup_kernel);
-    out->grid = dim3((E->k + 255) / 256, 1, 1);
+    out->grid = dim3((E->k + 255) / 256, rows, 1);
     out->block = dim3(256, 1, 1);
     out->shmem = 0;
     out->set_args(a);
@@ -268,6 +274,46 @@ fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out) {
     return FK_OK;
 }
 
+
+// RMSNorm of `rows` activation rows, y = T(w * T(x * r)) with r = 1/sqrt(mean(x^2) + eps)
+// per row (the arithmetic the GEMV fuses for one row, kernels/mod.rs:4424-4516), for the
+// multi-row path whose matrix-core matmul takes already normalised rows.  One block per row.
+struct NormRowsArgs {
+    const uint16_t* x;
+    const uint16_t* w;
+    uint16_t* y;
+    uint32_t hidden;
+    float eps;
+};
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const NormRowsArgs a) {
+    __shared__ float scratch[8];
+    const uint16_t* x = a.x + (size_t)blockIdx.x * a.hidden;
+    uint16_t* y = a.y + (size_t)blockIdx.x * a.hidden;
+    float ss = 0.f;
+    for (uint32_t i = threadIdx.x; i < a.hidden; i += 256) {
+        const float v = bf16_bits_to_f32(x[i]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float r = 1.0f / sqrtf(ss / (float)a.hidden + a.eps);
+    for (uint32_t i = threadIdx.x; i < a.hidden; i += 256)
+        y[i] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(a.w[i]) * round_bf16(bf16_bits_to_f32(x[i]) * r));
+}
+
+fk_status plan_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,
+                            Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!x || !w || !y) return set_error(FK_ERR_INVALID, "rmsnorm rows: null pointer");
+    if (rows == 0 || hidden == 0) return set_error(FK_ERR_INVALID, "rmsnorm rows: empty shape");
+    NormRowsArgs a{x, w, y, hidden, eps};
+    out->func = reinterpret_cast<const void*>(&rmsnorm_rows_kernel);
+    out->grid = dim3(rows, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
 
 // Plain device-to-device copy in 16-byte pieces.  Besides moving buffers it is the
 // known-traffic kernel hardware byte counters are calibrated against.

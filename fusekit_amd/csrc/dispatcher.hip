@@ -915,6 +915,7 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
         s.chunk_len = sdpa_chunk_len(s.qk_dim, s.v_dim, true);
         s.n_splits = (s.capacity + s.chunk_len - 1) / s.chunk_len;
         s.chunks_per_block = 1;
+        s.rows = 1;
         s.k_new = r1.k;
         s.v_new = r1.v;
         s.q_norm = r0.q_norm;

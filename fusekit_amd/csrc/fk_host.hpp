@@ -112,6 +112,7 @@ struct RopeArgs {
     uint32_t n_q, n_kv, head_dim, k_dim, v_dim, rope_dims, capacity;
     float eps, base_log2;
     uint32_t rope_on;  // 0: plain store of K (no rotation)
+    uint32_t rows;     // active token rows (0 = 1): row r is position offset + r and reads q/k/v row r
 };
 fk_status plan_rope_store(const RopeArgs& in, Launch* out);
 
@@ -121,9 +122,11 @@ fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim,
 fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,
                            const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
                            uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
-                           float* partials, uint32_t* counters, Launch* out_launch);
+                           float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows = 1);
 fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
-                     uint16_t* x, Launch* out);
+                     uint16_t* x, Launch* out, uint32_t rows = 1);
+fk_status plan_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,
+                            Launch* out);
 // workspace: 8 bytes (counter, zeroed once) + 8 bytes per block (<= 160 blocks)
 constexpr size_t kArgmaxWorkspaceBytes = 8 + 8 * 160;
 fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, uint32_t* history,

@@ -51,7 +51,7 @@ fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim,
 fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,
                            const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
                            uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
-                           float* partials, uint32_t* counters, Launch* out_launch) {
+                           float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!q || !k || !v || !out) return set_error(FK_ERR_INVALID, "sdpa: null tensor");
@@ -60,6 +60,9 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     if (qk_dim == 0 || v_dim == 0 || qk_dim % 8 || v_dim % 8 || qk_dim > 512 || v_dim > 512)
         return set_error(FK_ERR_UNSUPPORTED, "sdpa: head dims must be multiples of 8, at most 512");
     if (max_len == 0 || max_len > capacity) return set_error(FK_ERR_INVALID, "sdpa: kv length outside (0, capacity]");
+    if (rows == 0 || rows > 1024) return set_error(FK_ERR_INVALID, "sdpa: 1..1024 active rows");
+    if (!kv_len_ptr && rows > 1 && kv_len_imm + rows - 1 > max_len)
+        return set_error(FK_ERR_INVALID, "sdpa: the last row's kv length exceeds max_len");
     if (!kv_len_ptr && (kv_len_imm == 0 || kv_len_imm > max_len))
         return set_error(FK_ERR_INVALID, "sdpa: kv_len outside (0, max_len]");
     const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim, false);
@@ -89,6 +92,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     a.chunk_len = chunk;
     a.n_splits = n_splits;
     a.chunks_per_block = cpb;
+    a.rows = rows;
     a.lpk = pow2_ceil(qk_dim / 8);
     a.lpv = pow2_ceil(v_dim / 8);
     a.scale = scale;
@@ -103,7 +107,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         default: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<8>); break;
     }
     out_launch->func = func;
-    out_launch->grid = dim3(n_splits, n_kv, (G + gt - 1) / gt);
+    out_launch->grid = dim3(n_splits, n_kv, ((G + gt - 1) / gt) * rows);
     out_launch->block = dim3(kSdpaBlock, 1, 1);
     out_launch->shmem = (uint32_t)(sdpa_lds_floats(gt, chunk, qk_dim, v_dim, false) * sizeof(float));
     out_launch->set_args(a);

@@ -29,6 +29,7 @@ struct SdpaArgs {
     uint32_t n_heads, n_kv, qk_dim, v_dim, capacity;
     uint32_t chunk_len, n_splits;
     uint32_t chunks_per_block;  // consecutive ranges one block walks (online softmax across them)
+    uint32_t rows;              // active token rows (stand-alone kernel): row r attends to kv_len + r positions
     uint32_t lpk, lpv;  // lanes per key row / value row (powers of two)
     float scale;
     float* partials;     // [n_heads][n_splits][v_dim + 2]
@@ -424,8 +425,22 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
 #else
     const uint32_t* imm = &a.kv_len_imm;
 #endif
-    const uint32_t kv_len = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
-    sdpa_block<GT, false, SdpaArgs>(a, kv_len, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
+    const uint32_t kv_len0 = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
+    if (a.rows <= 1) {
+        sdpa_block<GT, false, SdpaArgs>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
+        return;
+    }
+    // Several active rows (multi-token verification, chunked prefill): grid.z carries
+    // (row, head tile).  Row r is the token at position kv_len0 - 1 + r: it attends to
+    // kv_len0 + r cache rows (causal inside the group), with its own q, out and workspace.
+    const uint32_t gz_count = gridDim.z / a.rows;
+    const uint32_t tr = blockIdx.z / gz_count, gz = blockIdx.z - tr * gz_count;
+    SdpaArgs r = a;
+    r.q = a.q + (size_t)tr * a.n_heads * a.qk_dim;
+    r.out = a.out + (size_t)tr * a.n_heads * a.v_dim;
+    r.partials = a.partials + (size_t)tr * a.n_heads * a.n_splits * (a.v_dim + 2);
+    r.counters = a.counters + (size_t)tr * a.n_kv * gz_count;
+    sdpa_block<GT, false, SdpaArgs>(r, kv_len0 + tr, blockIdx.x, blockIdx.y, gz, gz_count, lds);
 }
 
 }  // namespace fk

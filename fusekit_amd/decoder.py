@@ -274,6 +274,67 @@ class DecoderRuntime:
         nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
         return nxt[-1]
 
+    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 32) -> int:
+        """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
+        active_m > 1 variants): the projections of up to 32 tokens share ONE pass over each weight
+        matrix on the matrix cores (fk_qgemm), attention is causal inside the group.  Leaves the KV
+        caches, step counter and history as token-by-token `prefill` would, and returns the greedy
+        first token.  Quantised projections only (the dense bf16 multi-row matmul is a library GEMM)."""
+        c, w = self.cfg, self.w
+        if c.bits == 16:
+            return self.prefill(prompt, start_offset)
+        prompt = list(prompt)
+        if start_offset + len(prompt) > c.capacity:
+            raise ValueError("prompt exceeds the KV-cache capacity")
+        R = max(1, min(rows_per_pass, 32))
+        if not hasattr(self, "_rows"):
+            ws = max(native.qgemm_workspace_bytes(R, n, k, c.group) for n, k in
+                     ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
+            pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.capacity)
+            self._rows = dict(
+                tok=DeviceBuffer(4 * R), x=DeviceBuffer(R * c.hidden * 2), x2=DeviceBuffer(R * c.hidden * 2),
+                xn=DeviceBuffer(R * c.hidden * 2), q=DeviceBuffer(R * c.n_q * 2), k=DeviceBuffer(R * c.n_kvd * 2),
+                v=DeviceBuffer(R * c.n_kvd * 2), att=DeviceBuffer(R * c.n_q * 2), mid=DeviceBuffer(R * c.inter * 2),
+                ws=DeviceBuffer(2 * ws), part=DeviceBuffer(max(pb, 4) * R), cnt=native.zeros(max(cb, 4) * R))
+        b = self._rows
+        emb = w.mats["embed_tokens"]
+        head = w.mats.get("lm_head", emb)
+        pos = start_offset
+        scale = 1.0 / float(np.sqrt(c.head_dim))
+        while pos < start_offset + len(prompt):
+            chunk = prompt[pos - start_offset: pos - start_offset + R]
+            m = len(chunk)
+            b["tok"].upload(np.asarray(chunk, np.uint32))
+            native.embed_lookup_rows(emb, b["tok"], m, 1.0, b["x"])
+            for l in range(c.n_layers):
+                p = f"layers.{l}."
+                native.rmsnorm_rows(b["x"], w.vecs[p + "input_layernorm"], c.eps, m, c.hidden, b["xn"])
+                for nm, dst in (("q", b["q"]), ("k", b["k"]), ("v", b["v"])):
+                    bias = w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None
+                    native.qgemm(w.mats[p + f"self_attn.{nm}_proj"], b["xn"], m, bias, None, dst, b["ws"])
+                native.qkv_rope_store_rows(b["q"], b["k"], b["v"],
+                                           w.vecs.get(p + "self_attn.q_norm") if c.qk_norm else None,
+                                           w.vecs.get(p + "self_attn.k_norm") if c.qk_norm else None,
+                                           c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.theta, c.eps, m, pos, c.capacity,
+                                           self.cache_k[l], self.cache_v[l])
+                native.sdpa_decode_rows(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + 1, c.n_heads, c.n_kv,
+                                        c.head_dim, c.head_dim, c.capacity, scale, b["part"], b["cnt"])
+                native.qgemm(w.mats[p + "self_attn.o_proj"], b["att"], m, None, b["x"], b["x2"], b["ws"])
+                native.rmsnorm_rows(b["x2"], w.vecs[p + "post_attention_layernorm"], c.eps, m, c.hidden, b["xn"])
+                native.qgemm_swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], b["xn"], m, c.swiglu_variant,
+                                    b["mid"], b["ws"])
+                native.qgemm(w.mats[p + "mlp.down_proj"], b["mid"], m, None, b["x2"], b["x"], b["ws"])
+            pos += m
+        # the last row's hidden state -> logits -> greedy token, and the decode loop's uniforms
+        last = DeviceBuffer(c.hidden * 2)
+        native.copy(last, b["x"].ptr + (m - 1) * c.hidden * 2, c.hidden * 2)
+        native.final_rmsnorm_lm_head(last, w.vecs["final_norm"], c.eps, head, self.logits)
+        native.argmax_logits_decode(self.logits, c.vocab, self.token, None, None, 0, self.argmax_ws)
+        native.sync()
+        total = start_offset + len(prompt)
+        self.step_counter.upload(np.array([total], np.uint32))
+        return int(self.token.to_numpy(np.uint32)[0])
+
     def generate(self, prompt: Sequence[int], max_tokens: int):
         """Greedy decode.  Returns (tokens, gpu_seconds of the decode chunks, decode steps timed)."""
         if len(prompt) + max_tokens > self.cfg.capacity:

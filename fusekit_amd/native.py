@@ -272,6 +272,30 @@ def sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_
                              _ptr(partials), _ptr(counters), _ptr(stream)))
 
 
+def rmsnorm_rows(x, w, eps, rows, hidden, y, stream=None):
+    check(lib.fk_rmsnorm_rows(_ptr(x), _ptr(w), C.c_float(eps), C.c_uint32(rows), C.c_uint32(hidden), _ptr(y), _ptr(stream)))
+
+
+def embed_lookup_rows(E, d_tokens, rows, out_scale, x, stream=None):
+    check(lib.fk_embed_lookup_rows(C.byref(E.c), _ptr(d_tokens), C.c_uint32(rows), C.c_float(out_scale), _ptr(x),
+                                   _ptr(stream)))
+
+
+def qkv_rope_store_rows(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope_dims, theta, eps, rows, offset,
+                        capacity, cache_k, cache_v, stream=None):
+    check(lib.fk_qkv_rope_store_rows(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), C.c_uint32(n_heads), C.c_uint32(n_kv),
+        C.c_uint32(head_dim), C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), C.c_uint32(rows),
+        C.c_uint32(offset), C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v), _ptr(stream)))
+
+
+def sdpa_decode_rows(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, qk_dim, v_dim, capacity, scale, partials,
+                     counters, stream=None):
+    check(lib.fk_sdpa_decode_rows(_ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(out), C.c_uint32(rows), C.c_uint32(kv_len),
+                                  C.c_uint32(n_heads), C.c_uint32(n_kv), C.c_uint32(qk_dim), C.c_uint32(v_dim),
+                                  C.c_uint32(capacity), C.c_float(scale), _ptr(partials), _ptr(counters), _ptr(stream)))
+
+
 def embed_lookup_decode(E, d_token, token, out_scale, x, stream=None):
     check(lib.fk_embed_lookup_decode(C.byref(E.c), _ptr(d_token), C.c_uint32(token), C.c_float(out_scale),
                                      _ptr(x), _ptr(stream)))

@@ -258,6 +258,29 @@ fk_status fk_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint1
                          uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
                          float *partials, uint32_t *counters, fk_stream s);
 
+/* ---- several active token rows (multi-token verification, chunked prefill) ----
+ * The reference compiles such variants with active_m > 1 (src/target/mod.rs:170-200,
+ * variants `prefill_mN`, src/patch.rs:103-150; causal attention
+ * src/codegen/kernels/sdpa_prefill.rs:1-30).  Row r of a group is the token at position
+ * offset + r.  The projections of a group run through fk_qgemm / fk_qgemm_swiglu on rows that
+ * fk_rmsnorm_rows normalised; the functions below are the row forms of E, R and K4. */
+fk_status fk_rmsnorm_rows(const uint16_t *x, const uint16_t *w, float eps, uint32_t rows, uint32_t hidden,
+                          uint16_t *y, fk_stream s);
+fk_status fk_embed_lookup_rows(const fk_weight *E, const uint32_t *d_tokens, uint32_t rows, float out_scale,
+                               uint16_t *x, fk_stream s);
+/* q [rows, n_heads, head_dim] in place; k, v [rows, n_kv, head_dim] -> cache rows (offset + r) % capacity */
+fk_status fk_qkv_rope_store_rows(uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *q_norm,
+                                 const uint16_t *k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                 uint32_t rope_dims, float theta, float eps, uint32_t rows, uint32_t offset,
+                                 uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
+/* Row r attends to the first kv_len + r cache positions (causal inside the group); q and out are
+ * [rows, n_heads, dim].  Workspace: rows times the sizes of fk_sdpa_workspace_bytes(max_len =
+ * kv_len + rows - 1); counters zero before the first launch. */
+fk_status fk_sdpa_decode_rows(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v, uint16_t *out,
+                              uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim,
+                              uint32_t v_dim, uint32_t capacity, float scale, float *partials, uint32_t *counters,
+                              fk_stream s);
+
 /* E   x = T(embed[token] * out_scale), dense bf16 or MLX-affine table.  Replaces
  *     src/codegen/kernels/embed_lookup_decode.rs:17-108. */
 fk_status fk_embed_lookup_decode(const fk_weight *E, const uint32_t *d_token, uint32_t token, float out_scale,

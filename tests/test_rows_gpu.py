@@ -1,0 +1,111 @@
+"""Several active token rows per launch (multi-token verification / chunked prefill): the row forms
+of RMSNorm, embedding, RoPE + KV store and causal attention against the oracle applied row by row,
+and the batched prompt path of the decoder against its token-by-token path."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import OracleDecoder, bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(fk, a):
+    return None if a is None else fk.DeviceBuffer.from_numpy(np.ascontiguousarray(a))
+
+
+def _close(got, want, frac_bar=0.02, ulp_bar=1.0):
+    frac, ulps = bf16_mismatch(got, want)
+    assert frac <= frac_bar and ulps <= ulp_bar, (frac, ulps)
+
+
+def test_rmsnorm_and_embed_rows(fk):
+    rows, hidden = 7, 896
+    x, w = normal_bf16(1, (rows, hidden)), normal_bf16(2, hidden, 0.1, 1.0)
+    y = fk.DeviceBuffer(rows * hidden * 2)
+    fk.rmsnorm_rows(_dev(fk, x), _dev(fk, w), 1e-6, rows, hidden, y)
+    got = y.to_numpy(np.uint16, (rows, hidden))
+    for r in range(rows):
+        _close(got[r], oracle.rmsnorm(x[r], w, 1e-6))
+    for bits in (16, 4):
+        E = make_qweight(3, 500, 256, bits)
+        toks = np.array([0, 499, 17, 17, 250], np.uint32)
+        out = fk.DeviceBuffer(toks.size * 256 * 2)
+        fk.embed_lookup_rows(to_device(fk, E), _dev(fk, toks), toks.size, 1.0, out)
+        got = out.to_numpy(np.uint16, (toks.size, 256))
+        for r, t in enumerate(toks):
+            assert np.array_equal(got[r], oracle.embed_lookup(E, int(t)))
+
+
+@pytest.mark.parametrize("norm", [False, True])
+def test_rope_store_rows(fk, norm):
+    rows, n_heads, n_kv, dim, cap, off = 6, 8, 2, 64, 32, 29     # rows 29..34 wrap around the cache
+    q, k, v = normal_bf16(4, (rows, n_heads * dim)), normal_bf16(5, (rows, n_kv * dim)), normal_bf16(6, (rows, n_kv * dim))
+    qn, kn = (normal_bf16(7, dim, 0.1, 1.0), normal_bf16(8, dim, 0.1, 1.0)) if norm else (None, None)
+    dq, ck, cv = _dev(fk, q), fk.zeros(n_kv * cap * dim * 2), fk.zeros(n_kv * cap * dim * 2)
+    fk.qkv_rope_store_rows(dq, _dev(fk, k), _dev(fk, v), _dev(fk, qn), _dev(fk, kn), n_heads, n_kv, dim, dim, 1e4, 1e-6,
+                           rows, off, cap, ck, cv)
+    got_q = dq.to_numpy(np.uint16, (rows, n_heads * dim))
+    rk, rv = np.zeros(n_kv * cap * dim, np.uint16), np.zeros(n_kv * cap * dim, np.uint16)
+    for r in range(rows):
+        pos = off + r
+        want_q = oracle.headnorm_rope(q[r], qn, n_heads, dim, dim, 1e-6, 1e4, pos) if norm else oracle.rope_q(q[r], n_heads, dim, dim, 1e4, pos)
+        _close(got_q[r], want_q, ulp_bar=2.0)
+        kr = oracle.headnorm_rope(k[r], kn, n_kv, dim, 0, 1e-6, 1e4, pos) if norm else k[r]   # norm only, rotation below
+        oracle.rope_kv_store(kr, v[r], n_kv, dim, dim, 1e4, pos, pos, cap, rk, rv)
+    assert np.array_equal(cv.to_numpy(np.uint16), rv)
+    gk = ck.to_numpy(np.uint16)
+    assert np.array_equal(gk == 0, rk == 0)
+    _close(gk, rk, ulp_bar=2.0)
+
+
+@pytest.mark.parametrize("kv_len,rows", [(1, 5), (60, 8), (500, 32)])
+def test_sdpa_rows_are_causal_single_row_calls(fk, kv_len, rows):
+    n_heads, n_kv, dim, cap = 32, 8, 128, 1024
+    q = normal_bf16(9, (rows, n_heads * dim))
+    ck, cv = normal_bf16(10, n_kv * cap * dim), normal_bf16(11, n_kv * cap * dim)
+    dck, dcv = _dev(fk, ck), _dev(fk, cv)
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, dim, dim, kv_len + rows - 1)
+    out = fk.DeviceBuffer(rows * n_heads * dim * 2)
+    scale = 1.0 / np.sqrt(dim)
+    fk.sdpa_decode_rows(_dev(fk, q), dck, dcv, out, rows, kv_len, n_heads, n_kv, dim, dim, cap, scale,
+                        fk.DeviceBuffer(max(pb, 16) * rows), fk.zeros(max(cb, 16) * rows))
+    got = out.to_numpy(np.uint16, (rows, n_heads * dim))
+    one = fk.DeviceBuffer(n_heads * dim * 2)
+    part, cnt = fk.DeviceBuffer(max(pb, 16)), fk.zeros(max(cb, 16))
+    for r in range(rows):
+        fk.sdpa_decode(_dev(fk, q[r]), dck, dcv, one, None, kv_len + r, kv_len + rows - 1, n_heads, n_kv, dim, dim, cap,
+                       scale, part, cnt)
+        assert np.array_equal(got[r], one.to_numpy(np.uint16)), r          # same kernel, same split: same bits
+        ref = oracle.sdpa_decode(q[r], ck, cv, n_heads, n_kv, dim, dim, kv_len + r, cap, scale)
+        assert rel_l2(got[r], oracle.bf16_to_f32(ref)) <= 1e-2
+
+
+@pytest.mark.parametrize("bits,prompt_len", [(4, 45), (8, 7)])
+def test_batched_prefill_matches_token_by_token(fk, bits, prompt_len):
+    """prefill_rows (32 tokens per weight pass on the matrix cores) leaves the caches of the
+    token-by-token path and continues with the same tokens.  The two paths sum in different
+    orders, so the caches agree to rounding flips and the greedy continuation is compared with
+    the oracle's margins in view."""
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    cfg = DecoderConfig(n_layers=3, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=2000, capacity=128,
+                        bits=bits, qk_norm=True, qkv_bias=(bits == 8), swiglu_variant=2)
+    W = DecoderWeights.random_init(cfg, seed=41)
+    prompt = rng(42).integers(0, cfg.vocab, prompt_len).tolist()
+    a, b = DecoderRuntime(cfg, W), DecoderRuntime(cfg, W)
+    first_a = a.prefill(prompt)
+    first_b = b.prefill_rows(prompt)
+    for l in range(cfg.n_layers):
+        for ca, cb_ in ((a.cache_k[l], b.cache_k[l]), (a.cache_v[l], b.cache_v[l])):
+            ga, gb = ca.to_numpy(np.uint16), cb_.to_numpy(np.uint16)
+            assert np.array_equal(ga == 0, gb == 0)
+            assert rel_l2(gb, oracle.bf16_to_f32(ga)) <= 1e-2, l
+    ref, margins = OracleDecoder(cfg, W).generate(prompt, 9)
+    assert first_a == ref[0]
+    if margins[0] > 0.05:
+        assert first_b == ref[0]
+    if first_b == first_a:
+        ta, _ = a.d.decode_chunk(a.graph, a.uniforms, prompt_len, first_a, 8)
+        tb, _ = b.d.decode_chunk(b.graph, b.uniforms, prompt_len, first_b, 8)
+        clear = next((i for i, m in enumerate(margins[1:]) if m <= 0.05), 8)
+        assert ta[:clear] == tb[:clear] == ref[1:1 + clear]
