@@ -45,8 +45,14 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
         scratch(name, getattr(rt, name), "bfloat16")
     scratch("sdpa_partials", rt.sdpa_partials, "float32")
     for l in range(rt.cfg.n_layers):
-        scratch(f"cache_k.{l}", rt.cache_k[l], "bfloat16", zero=True)
-        scratch(f"cache_v.{l}", rt.cache_v[l], "bfloat16", zero=True)
+        if rt.cfg.kv_bits:
+            for nm, c in (("cache_k", rt.cache_k[l]), ("cache_v", rt.cache_v[l])):
+                scratch(f"{nm}.{l}.packed", c.packed, "uint32", zero=True)
+                scratch(f"{nm}.{l}.scales", c.scales, "bfloat16", zero=True)
+                scratch(f"{nm}.{l}.biases", c.biases, "bfloat16", zero=True)
+        else:
+            scratch(f"cache_k.{l}", rt.cache_k[l], "bfloat16", zero=True)
+            scratch(f"cache_v.{l}", rt.cache_v[l], "bfloat16", zero=True)
     for path, W in rt.w.mats.items():
         sym[W.w.ptr] = dict(role="external", source_path=path + ".weight", dtype="uint32" if W.bits != 16 else "bfloat16",
                             shape=[W.n, W.k * W.bits // 32] if W.bits != 16 else [W.n, W.k])
@@ -117,7 +123,7 @@ def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "syntheti
         uniforms=dict(token="token", step_counter="step_counter", hist_counter="hist_counter", history="history"),
         model_config={k: getattr(c, k) for k in ("n_layers", "hidden", "n_heads", "n_kv", "head_dim", "inter", "vocab",
                                                   "capacity", "bits", "group", "eps", "theta", "qk_norm", "qkv_bias",
-                                                  "fuse_rope_store", "swiglu_variant")})
+                                                  "fuse_rope_store", "swiglu_variant", "kv_bits", "kv_group")})
     with open(os.path.join(out_dir, "task_graph.json"), "w") as f:
         json.dump(graph, f, indent=1)
     manifest = dict(

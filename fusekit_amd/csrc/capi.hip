@@ -382,6 +382,44 @@ fk_status fk_qkv_rope_store_decode(uint16_t* q, const uint16_t* k, const uint16_
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_kv_cache_store_quant(const uint16_t* k, const uint16_t* v, const uint16_t* k_norm, uint32_t n_kv,
+                                  uint32_t head_dim, uint32_t rope_dims, float theta, float eps, const uint32_t* d_offset,
+                                  uint32_t offset, uint32_t rows, uint32_t capacity, uint32_t bits, uint32_t group,
+                                  const fk_kv_quant_cache* cache_k, const fk_kv_quant_cache* cache_v, fk_stream s) {
+    if (!cache_k || !cache_v) return set_error(FK_ERR_INVALID, "fk_kv_cache_store_quant: null cache");
+    KvQuantStore a;
+    memset(&a, 0, sizeof(a));
+    a.k = k; a.v = v; a.k_norm = k_norm;
+    a.ck_packed = cache_k->packed; a.ck_scales = cache_k->scales; a.ck_biases = cache_k->biases;
+    a.cv_packed = cache_v->packed; a.cv_scales = cache_v->scales; a.cv_biases = cache_v->biases;
+    a.offset_ptr = d_offset; a.offset_imm = offset;
+    a.n_kv = n_kv; a.dim = head_dim; a.rope_dims = rope_dims; a.capacity = capacity; a.bits = bits; a.group = group;
+    a.rows = rows;
+    a.eps = eps; a.base_log2 = theta_log2(theta);
+    Launch l;
+    FK_TRY(plan_kv_store_quant(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_sdpa_decode_quant(const uint16_t* q, const fk_kv_quant_cache* cache_k, const fk_kv_quant_cache* cache_v,
+                               uint16_t* out, const uint32_t* d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t rows,
+                               uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity,
+                               uint32_t bits, uint32_t group, float scale, float* partials, uint32_t* counters,
+                               fk_stream s) {
+    if (!cache_k || !cache_v || !cache_k->packed || !cache_v->packed)
+        return set_error(FK_ERR_INVALID, "fk_sdpa_decode_quant: null cache");
+    KvQuant qz;
+    qz.k_scales = cache_k->scales; qz.k_biases = cache_k->biases;
+    qz.v_scales = cache_v->scales; qz.v_biases = cache_v->biases;
+    qz.bits = bits; qz.group = group;
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, "fk_sdpa_decode_quant: bits must be 4 or 8");
+    Launch l;
+    FK_TRY(plan_sdpa_decode(q, reinterpret_cast<const uint16_t*>(cache_k->packed),
+                            reinterpret_cast<const uint16_t*>(cache_v->packed), out, d_kv_len, kv_len, max_len, n_heads,
+                            n_kv, qk_dim, v_dim, capacity, scale, partials, counters, &l, rows ? rows : 1, &qz));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,
                           fk_stream s) {
     Launch l;

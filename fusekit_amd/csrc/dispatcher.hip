@@ -411,6 +411,94 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
                             capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l);
 }
 
+// K, V, [k_weight], keys_packed, keys_scales, keys_biases, values_packed, values_scales, values_biases, offset,
+// write_offset (rope_kv_cache_store_decode_quant.rs:77-98; the capacity is a parameter here)
+fk_status plan_rope_kv_quant(const Dispatch& d, Launch* l, SlotRW* rw, uint32_t bits) {
+    const bool norm = d.u("has_norm", 0) != 0;
+    const size_t n = norm ? 11 : 10, c0 = norm ? 3 : 2;
+    FK_TRY(need_args(d, n));
+    KvQuantStore a;
+    memset(&a, 0, sizeof(a));
+    a.n_kv = d.u("n_kv");
+    a.dim = d.u("head_dim");
+    a.rope_dims = d.u("rope_dims", a.dim);
+    a.capacity = d.u("capacity");
+    a.bits = bits;
+    a.group = d.u("group", 64);
+    a.rows = 1;
+    if (a.capacity == 0 || a.n_kv == 0 || a.dim == 0 || a.group == 0 || a.dim % a.group)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_kv / head_dim / capacity / group parameters missing or inconsistent");
+    const size_t rows = (size_t)a.n_kv * a.capacity;
+    FK_TRY(need_bytes(d, 0, (size_t)a.n_kv * a.dim * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)a.n_kv * a.dim * 2));
+    for (size_t c = 0; c < 2; ++c) {
+        FK_TRY(need_bytes(d, c0 + 3 * c, rows * a.dim * bits / 8));
+        FK_TRY(need_bytes(d, c0 + 3 * c + 1, rows * (a.dim / a.group) * 2));
+        FK_TRY(need_bytes(d, c0 + 3 * c + 2, rows * (a.dim / a.group) * 2));
+    }
+    FK_TRY(need_bytes(d, c0 + 6, 4));
+    FK_TRY(need_bytes(d, c0 + 7, 4));
+    a.k = arg_ptr<const uint16_t>(d, 0);
+    a.v = arg_ptr<const uint16_t>(d, 1);
+    if (norm) {
+        FK_TRY(need_bytes(d, 2, (size_t)a.dim * 2));
+        a.k_norm = arg_ptr<const uint16_t>(d, 2);
+    }
+    a.ck_packed = arg_ptr<uint32_t>(d, c0);
+    a.ck_scales = arg_ptr<uint16_t>(d, c0 + 1);
+    a.ck_biases = arg_ptr<uint16_t>(d, c0 + 2);
+    a.cv_packed = arg_ptr<uint32_t>(d, c0 + 3);
+    a.cv_scales = arg_ptr<uint16_t>(d, c0 + 4);
+    a.cv_biases = arg_ptr<uint16_t>(d, c0 + 5);
+    a.offset_ptr = arg_ptr<const uint32_t>(d, c0 + 6);
+    a.write_offset_ptr = arg_ptr<const uint32_t>(d, c0 + 7);
+    a.eps = (float)d.param("eps", 1e-6);
+    a.base_log2 = base_log2_of(d);
+    for (uint32_t i = 0; i < n; ++i) {
+        if (i >= c0 && i < c0 + 6) rw->writes.push_back(i);
+        else rw->reads.push_back(i);
+    }
+    return plan_kv_store_quant(a, l);
+}
+
+// Q, K_packed, K_scales, K_biases, V_packed, V_scales, V_biases, kv_len, out, partials, counters
+// (sdpa_decode_quant.rs:184-196; the capacity is a parameter here)
+fk_status plan_sdpa_quant_d(const Dispatch& d, Launch* l, SlotRW* rw, uint32_t bits) {
+    FK_TRY(need_args(d, 11));
+    const uint32_t n_heads = d.u("n_heads"), n_kv = d.u("n_kv"), qk = d.u("qk_dim", d.u("head_dim"));
+    const uint32_t vd = d.u("v_dim", qk), capacity = d.u("capacity"), max_len = d.u("max_len", capacity);
+    const uint32_t group = d.u("group", 64);
+    if (n_heads == 0 || n_kv == 0 || qk == 0 || capacity == 0 || group == 0 || qk % group || vd % group)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / head_dim / capacity / group parameters missing or inconsistent");
+    const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)qk);
+    const size_t rows = (size_t)n_kv * capacity;
+    FK_TRY(need_bytes(d, 0, (size_t)n_heads * qk * 2));
+    FK_TRY(need_bytes(d, 1, rows * qk * bits / 8));
+    FK_TRY(need_bytes(d, 2, rows * (qk / group) * 2));
+    FK_TRY(need_bytes(d, 3, rows * (qk / group) * 2));
+    FK_TRY(need_bytes(d, 4, rows * vd * bits / 8));
+    FK_TRY(need_bytes(d, 5, rows * (vd / group) * 2));
+    FK_TRY(need_bytes(d, 6, rows * (vd / group) * 2));
+    FK_TRY(need_bytes(d, 7, 4));
+    FK_TRY(need_bytes(d, 8, (size_t)n_heads * vd * 2));
+    size_t pb = 0, cb = 0;
+    FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, qk, vd, max_len, &pb, &cb));
+    FK_TRY(need_bytes(d, 9, pb));
+    FK_TRY(need_bytes(d, 10, cb));
+    rw->reads = {0, 1, 2, 3, 4, 5, 6, 7, 9, 10};
+    rw->writes = {8, 9, 10};
+    KvQuant qz;
+    qz.k_scales = arg_ptr<const uint16_t>(d, 2);
+    qz.k_biases = arg_ptr<const uint16_t>(d, 3);
+    qz.v_scales = arg_ptr<const uint16_t>(d, 5);
+    qz.v_biases = arg_ptr<const uint16_t>(d, 6);
+    qz.bits = bits;
+    qz.group = group;
+    return plan_sdpa_decode(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<const uint16_t>(d, 4),
+                            arg_ptr<uint16_t>(d, 8), arg_ptr<const uint32_t>(d, 7), 0, max_len, n_heads, n_kv, qk, vd,
+                            capacity, scale, arg_ptr<float>(d, 9), arg_ptr<uint32_t>(d, 10), l, 1, &qz);
+}
+
 // x, gate_w, gate_s, gate_b, up_w, up_s, up_b, row_idx, expert_idx, [route_weight], out0
 // (routed_qmv_swiglu.rs:99-112).  Parameters: k, o, experts, routes, x_rows, pre_scale.
 fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
@@ -605,6 +693,12 @@ const Family kFamilies[] = {
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, false); }},
     {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
     {"fusekit_sdpa_decode", plan_sdpa_d},
+    {"fusekit_rope_kv_cache_store_decode_q4",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv_quant(d, l, rw, 4); }},
+    {"fusekit_rope_kv_cache_store_decode_q8",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv_quant(d, l, rw, 8); }},
+    {"fusekit_sdpa_decode_q4", [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_sdpa_quant_d(d, l, rw, 4); }},
+    {"fusekit_sdpa_decode_q8", [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_sdpa_quant_d(d, l, rw, 8); }},
     {"fusekit_argmax_logits_decode", plan_argmax_d},
 };
 

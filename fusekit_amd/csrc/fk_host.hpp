@@ -116,13 +116,36 @@ struct RopeArgs {
 };
 fk_status plan_rope_store(const RopeArgs& in, Launch* out);
 
+// Quantised KV cache (mlx-lm QuantizedKVCache layout): packed uint32 [n_kv, capacity, dim*bits/32],
+// scales / biases bf16 [n_kv, capacity, dim/group].
+struct KvQuant {
+    const uint16_t* k_scales = nullptr;
+    const uint16_t* k_biases = nullptr;
+    const uint16_t* v_scales = nullptr;
+    const uint16_t* v_biases = nullptr;
+    uint32_t bits = 0, group = 64;  // bits 0: plain bf16 cache
+};
+struct KvQuantStore {
+    const uint16_t* k;       // [rows, n_kv, dim] raw projection output
+    const uint16_t* v;
+    const uint16_t* k_norm;  // [dim] or null
+    uint32_t* ck_packed; uint16_t* ck_scales; uint16_t* ck_biases;
+    uint32_t* cv_packed; uint16_t* cv_scales; uint16_t* cv_biases;
+    const uint32_t* offset_ptr;        // position of row 0 (device) or null -> offset_imm
+    const uint32_t* write_offset_ptr;  // cache row of row 0 before the modulo, or null -> the position
+    uint32_t offset_imm;
+    uint32_t n_kv, dim, rope_dims, capacity, bits, group, rows;
+    float eps, base_log2;
+};
+fk_status plan_kv_store_quant(const KvQuantStore& in, Launch* out);
 uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim, bool fused);
 fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                size_t* partial_bytes, size_t* counter_bytes);
 fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,
                            const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
                            uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
-                           float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows = 1);
+                           float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows = 1,
+                           const KvQuant* quant = nullptr);
 fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
                      uint16_t* x, Launch* out, uint32_t rows = 1);
 fk_status plan_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,

@@ -79,25 +79,6 @@ __host__ __device__ inline uint32_t gemv_lds_bytes(uint32_t cpr, uint32_t seg_ch
     return ChunkTraits<KIND>::kPieces * cpr * 16u + cpr * 4u + nseg * seg_pad * 4u + 64u;
 }
 
-// Eight int4 codes of one packed word against eight activations.  A byte
-// 0000nnnn read as fp8 e4m3 is exactly n * 2^-9 (subnormal for n < 8, (8+m)*2^-9
-// above), so v_cvt_scalef32_pk_bf16_fp8 with scale 512 turns two such bytes into
-// the bf16 pair (n_a, n_b) in one instruction.  w & 0x0F0F0F0F holds nibbles
-// 0,2,4,6 in its bytes and (w >> 4) & 0x0F0F0F0F nibbles 1,3,5,7, which fixes the
-// activation pairing: xp = {(x0,x2), (x4,x6), (x1,x3), (x5,x7)}.
-__device__ __forceinline__ float q4_word_dot(uint32_t w, uint4 xp, float d) {
-    const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
-    const bf16x2_t e0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false);
-    const bf16x2_t e1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, true);
-    const bf16x2_t o0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, false);
-    const bf16x2_t o1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, true);
-    d = __builtin_amdgcn_fdot2_f32_bf16(e0, __builtin_bit_cast(bf16x2_t, xp.x), d, false);
-    d = __builtin_amdgcn_fdot2_f32_bf16(e1, __builtin_bit_cast(bf16x2_t, xp.y), d, false);
-    d = __builtin_amdgcn_fdot2_f32_bf16(o0, __builtin_bit_cast(bf16x2_t, xp.z), d, false);
-    d = __builtin_amdgcn_fdot2_f32_bf16(o1, __builtin_bit_cast(bf16x2_t, xp.w), d, false);
-    return d;
-}
-
 __device__ __forceinline__ float q8_word_dot(uint32_t w, uint4 xf, float d) {
     d = fmaf((float)(w & 0xffu), __uint_as_float(xf.x), d);
     d = fmaf((float)((w >> 8) & 0xffu), __uint_as_float(xf.y), d);

@@ -51,7 +51,8 @@ fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim,
 fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,
                            const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
                            uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
-                           float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows) {
+                           float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows,
+                           const KvQuant* quant) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!q || !k || !v || !out) return set_error(FK_ERR_INVALID, "sdpa: null tensor");
@@ -61,6 +62,15 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         return set_error(FK_ERR_UNSUPPORTED, "sdpa: head dims must be multiples of 8, at most 512");
     if (max_len == 0 || max_len > capacity) return set_error(FK_ERR_INVALID, "sdpa: kv length outside (0, capacity]");
     if (rows == 0 || rows > 1024) return set_error(FK_ERR_INVALID, "sdpa: 1..1024 active rows");
+    const uint32_t kvq = quant ? quant->bits : 0u;
+    if (kvq) {
+        if (kvq != 4 && kvq != 8) return set_error(FK_ERR_UNSUPPORTED, "sdpa: quantised cache bits must be 4 or 8");
+        if (!quant->k_scales || !quant->k_biases || !quant->v_scales || !quant->v_biases)
+            return set_error(FK_ERR_INVALID, "sdpa: null cache scales / biases");
+        const uint32_t g = quant->group;
+        if ((g != 32 && g != 64 && g != 128) || qk_dim % g || v_dim % g)
+            return set_error(FK_ERR_UNSUPPORTED, "sdpa: cache group size must be 32, 64 or 128 and divide the head dims");
+    }
     if (!kv_len_ptr && rows > 1 && kv_len_imm + rows - 1 > max_len)
         return set_error(FK_ERR_INVALID, "sdpa: the last row's kv length exceeds max_len");
     if (!kv_len_ptr && (kv_len_imm == 0 || kv_len_imm > max_len))
@@ -93,6 +103,11 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     a.n_splits = n_splits;
     a.chunks_per_block = cpb;
     a.rows = rows;
+    if (kvq) {
+        a.k_scales = quant->k_scales; a.k_biases = quant->k_biases;
+        a.v_scales = quant->v_scales; a.v_biases = quant->v_biases;
+        a.kv_group = quant->group;
+    }
     a.lpk = pow2_ceil(qk_dim / 8);
     a.lpv = pow2_ceil(v_dim / 8);
     a.scale = scale;
@@ -100,12 +115,21 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     a.counters = counters;
 
     const void* func = nullptr;
-    switch (gt) {
-        case 1: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<1>); break;
-        case 2: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<2>); break;
-        case 4: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<4>); break;
-        default: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<8>); break;
+#define FK_SDPA_PICK(Q)                                                                         \
+    switch (gt) {                                                                               \
+        case 1: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<1, Q>); break;         \
+        case 2: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<2, Q>); break;         \
+        case 4: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<4, Q>); break;         \
+        default: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<8, Q>); break;        \
     }
+    if (kvq == 4) {
+        FK_SDPA_PICK(4)
+    } else if (kvq == 8) {
+        FK_SDPA_PICK(8)
+    } else {
+        FK_SDPA_PICK(0)
+    }
+#undef FK_SDPA_PICK
     out_launch->func = func;
     out_launch->grid = dim3(n_splits, n_kv, ((G + gt - 1) / gt) * rows);
     out_launch->block = dim3(kSdpaBlock, 1, 1);

@@ -30,6 +30,13 @@ struct SdpaArgs {
     uint32_t chunk_len, n_splits;
     uint32_t chunks_per_block;  // consecutive ranges one block walks (online softmax across them)
     uint32_t rows;              // active token rows (stand-alone kernel): row r attends to kv_len + r positions
+    // Quantised cache (stand-alone kernel, KVQ = 4 or 8): k / v point at packed uint32
+    // [n_kv, capacity, dim * bits / 32]; scales / biases are bf16 [n_kv, capacity, dim / kv_group].
+    const uint16_t* k_scales;
+    const uint16_t* k_biases;
+    const uint16_t* v_scales;
+    const uint16_t* v_biases;
+    uint32_t kv_group;
     uint32_t lpk, lpv;  // lanes per key row / value row (powers of two)
     float scale;
     float* partials;     // [n_heads][n_splits][v_dim + 2]
@@ -63,10 +70,11 @@ __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk,
 }
 
 // One (range, kv head, head tile) work item.  Uniform per block; `kv_len` already read.
-template <int GT, bool FUSED, typename ARGS>
+template <int GT, bool FUSED, typename ARGS, int KVQ = 0>
 __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
                                            uint32_t gz, uint32_t gz_count, float* lds) {
     constexpr int kSteps = FUSED ? kSdpaStepsFused : kSdpaSteps;
+    static_assert(!(FUSED && KVQ != 0), "the fused form reads a bf16 cache");
     const uint32_t span = a.chunk_len * a.chunks_per_block;  // cache positions per block
     const uint32_t blk0 = split * span;
     const uint32_t G = a.n_heads / a.n_kv;
@@ -134,10 +142,13 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         stat[8 + tid] = 0.f;
     }
     float acc[GT][8];
+    float accb[GT];  // quantised V: sum_j p_j * bias_j of this lane's group, added to its 8 dims at the end
 #pragma unroll
-    for (int h = 0; h < GT; ++h)
+    for (int h = 0; h < GT; ++h) {
+        accb[h] = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+    }
 
     // This lane's 8 dims of each query head; fetched before the K/V rows so that the
     // scores can start as soon as the first keys arrive (loads return in order).
@@ -153,6 +164,19 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
     }
 
+    float sq[GT];  // quantised K: sum of this lane's 8 query dims (the affine bias term b * sum q)
+    if constexpr (KVQ != 0) {
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            const uint4 v = qf[h];
+            sq[h] = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+                    ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
+            if constexpr (KVQ == 4)  // nibble pairing of q4_word_dot: (x0,x2) (x4,x6) (x1,x3) (x5,x7)
+                qf[h] = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
+                                   (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
+        }
+    }
+
     // All K and V loads of a range are issued up front (the range is sized so that
     // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
     // Stand-alone: every row that exists in the cache allocation is requested, whether
@@ -163,6 +187,36 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
                             uint32_t jpos) {
         const uint16_t* kbase = a.k + ((size_t)kvh * a.capacity + key0) * a.qk_dim + 8 * ck;
         const uint16_t* vbase = a.v + ((size_t)kvh * a.capacity + key0) * a.v_dim + 8 * cv;
+        if constexpr (KVQ != 0) {
+            // 8 dims per lane as in the bf16 layout: one packed word (int4) or two (int8) in
+            // .x / .y, the group's scale and bias bits in .z; rows clamped as below.
+            constexpr uint32_t WPL = KVQ == 4 ? 1u : 2u;
+            const uint32_t kw = a.qk_dim * KVQ / 32u, vw = a.v_dim * KVQ / 32u;
+            const uint32_t kg = a.qk_dim / a.kv_group, vg = a.v_dim / a.kv_group;
+            const uint32_t kcol = kcol_ok ? ck : 0u, vcol = vcol_ok ? cv : 0u;
+            const uint32_t* kp = reinterpret_cast<const uint32_t*>(a.k) + (size_t)kvh * a.capacity * kw + kcol * WPL;
+            const uint32_t* vp = reinterpret_cast<const uint32_t*>(a.v) + (size_t)kvh * a.capacity * vw + vcol * WPL;
+            const size_t kmeta = (size_t)kvh * a.capacity * kg + (8u * kcol) / a.kv_group;
+            const size_t vmeta = (size_t)kvh * a.capacity * vg + (8u * vcol) / a.kv_group;
+            const uint32_t last = a.capacity - 1;
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                const uint32_t r0 = key0 + kslot + u * kslots, r = r0 < last ? r0 : last;
+                kd[u].x = kp[(size_t)r * kw];
+                kd[u].y = WPL == 2 ? kp[(size_t)r * kw + 1] : 0u;
+                kd[u].z = (uint32_t)a.k_scales[kmeta + (size_t)r * kg] | ((uint32_t)a.k_biases[kmeta + (size_t)r * kg] << 16);
+                kd[u].w = 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                const uint32_t r0 = key0 + vslot + u * vslots, r = r0 < last ? r0 : last;
+                vd[u].x = vp[(size_t)r * vw];
+                vd[u].y = WPL == 2 ? vp[(size_t)r * vw + 1] : 0u;
+                vd[u].z = (uint32_t)a.v_scales[vmeta + (size_t)r * vg] | ((uint32_t)a.v_biases[vmeta + (size_t)r * vg] << 16);
+                vd[u].w = 0u;
+            }
+            return;
+        }
         if constexpr (!FUSED) {
             // Straight-line, clamped (row to the last row of the allocation, a lane beyond
             // the head width to column 0): no branch separates the loads, so the compiler
@@ -236,10 +290,22 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 #pragma unroll
             for (int h = 0; h < GT; ++h) {
                 float d = 0.f;
-                d = dot2_bf16(kc[u].x, qf[h].x, d);
-                d = dot2_bf16(kc[u].y, qf[h].y, d);
-                d = dot2_bf16(kc[u].z, qf[h].z, d);
-                d = dot2_bf16(kc[u].w, qf[h].w, d);
+                if constexpr (KVQ == 4) {
+                    d = q4_word_dot(kc[u].x, qf[h], 0.f);
+                    d = fmaf(bf16_lo(kc[u].z), d, bf16_hi(kc[u].z) * sq[h]);  // s * sum(q * code) + b * sum(q)
+                } else if constexpr (KVQ == 8) {
+                    const uint32_t w0 = kc[u].x, w1 = kc[u].y;
+                    d = dot2_bf16(pack_bf16((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu)), qf[h].x, d);
+                    d = dot2_bf16(pack_bf16((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24)), qf[h].y, d);
+                    d = dot2_bf16(pack_bf16((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu)), qf[h].z, d);
+                    d = dot2_bf16(pack_bf16((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24)), qf[h].w, d);
+                    d = fmaf(bf16_lo(kc[u].z), d, bf16_hi(kc[u].z) * sq[h]);
+                } else {
+                    d = dot2_bf16(kc[u].x, qf[h].x, d);
+                    d = dot2_bf16(kc[u].y, qf[h].y, d);
+                    d = dot2_bf16(kc[u].z, qf[h].z, d);
+                    d = dot2_bf16(kc[u].w, qf[h].w, d);
+                }
                 d = group_sum(d, (int)lpk);
                 if (ck == 0 && j < nkeys) s[h * a.chunk_len + j] = d * a.scale;
             }
@@ -282,6 +348,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             const float alpha = stat[24 + h];
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
+            accb[h] *= alpha;
         }
     }
 #pragma unroll
@@ -289,6 +356,34 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         const uint32_t j = vslot + u * vslots;
         const uint32_t jj = j < nkeys ? j : 0u;
         const float live = j < nkeys ? 1.f : 0.f;
+        if constexpr (KVQ != 0) {
+            // codes are integers (always finite); rows past kv_len were requested
+            // speculatively, so their scale / bias bits may be anything: zeroed here
+            const bool ok = j < nkeys && vcol_ok;
+            const float sc = ok ? bf16_lo(vc[u].z) : 0.f, bi = ok ? bf16_hi(vc[u].z) : 0.f;
+            float f[8];
+            if constexpr (KVQ == 4) {
+                const uint32_t even = vc[u].x & 0x0F0F0F0Fu, odd = (vc[u].x >> 4) & 0x0F0F0F0Fu;
+                f[0] = (float)(even & 0xffu); f[2] = (float)((even >> 8) & 0xffu);
+                f[4] = (float)((even >> 16) & 0xffu); f[6] = (float)(even >> 24);
+                f[1] = (float)(odd & 0xffu); f[3] = (float)((odd >> 8) & 0xffu);
+                f[5] = (float)((odd >> 16) & 0xffu); f[7] = (float)(odd >> 24);
+            } else {
+                const uint32_t w0 = vc[u].x, w1 = vc[u].y;
+                f[0] = (float)(w0 & 0xffu); f[1] = (float)((w0 >> 8) & 0xffu);
+                f[2] = (float)((w0 >> 16) & 0xffu); f[3] = (float)(w0 >> 24);
+                f[4] = (float)(w1 & 0xffu); f[5] = (float)((w1 >> 8) & 0xffu);
+                f[6] = (float)((w1 >> 16) & 0xffu); f[7] = (float)(w1 >> 24);
+            }
+#pragma unroll
+            for (int h = 0; h < GT; ++h) {
+                const float p = s[h * a.chunk_len + jj] * live;
+                const float ps = p * sc;
+                accb[h] = fmaf(p, bi, accb[h]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(ps, f[i], acc[h][i]);
+            }
+        } else {
         // rows past kv_len were requested speculatively: their bits may be anything
         const uint4 vv = (FUSED || (j < nkeys && vcol_ok)) ? vc[u] : make_uint4(0, 0, 0, 0);
         const float f[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
@@ -298,6 +393,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             const float p = s[h * a.chunk_len + jj] * live;
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
+        }
         }
     }
     if (c + 1 < n_chunks) {
@@ -315,6 +411,12 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 
     // Every lane parks its sums in LDS, [value slot][head][dim]; the output loop below
     // adds the slots in index order (no cross-lane shuffles, fixed order).
+    if constexpr (KVQ != 0) {
+#pragma unroll
+        for (int h = 0; h < GT; ++h)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][i] += accb[h];
+    }
     if (vcol_ok) {
 #pragma unroll
         for (int h = 0; h < GT; ++h) {
@@ -413,7 +515,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     FK_SDPA_STAMP(9);
 }
 
-template <int GT>
+template <int GT, int KVQ = 0>
 __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs a) {
     extern __shared__ __align__(16) float lds[];
     // One unconditional load (the immediate is read from the kernel-argument segment
@@ -427,7 +529,7 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
 #endif
     const uint32_t kv_len0 = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
     if (a.rows <= 1) {
-        sdpa_block<GT, false, SdpaArgs>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
+        sdpa_block<GT, false, SdpaArgs, KVQ>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
         return;
     }
     // Several active rows (multi-token verification, chunked prefill): grid.z carries
@@ -440,7 +542,7 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     r.out = a.out + (size_t)tr * a.n_heads * a.v_dim;
     r.partials = a.partials + (size_t)tr * a.n_heads * a.n_splits * (a.v_dim + 2);
     r.counters = a.counters + (size_t)tr * a.n_kv * gz_count;
-    sdpa_block<GT, false, SdpaArgs>(r, kv_len0 + tr, blockIdx.x, blockIdx.y, gz, gz_count, lds);
+    sdpa_block<GT, false, SdpaArgs, KVQ>(r, kv_len0 + tr, blockIdx.x, blockIdx.y, gz, gz_count, lds);
 }
 
 }  // namespace fk

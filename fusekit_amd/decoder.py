@@ -41,6 +41,8 @@ class DecoderConfig:
     swiglu_variant: int = 0
     capacity: int = 1024     # KV-cache rows per layer
     fuse_rope_store: bool = True   # one launch for rope_q + rope_kv_store (False: the reference's two)
+    kv_bits: int = 0         # 0: bf16 KV cache; 4 / 8: quantised cache (mlx-lm QuantizedKVCache layout)
+    kv_group: int = 64
 
     @property
     def n_q(self) -> int:
@@ -59,7 +61,8 @@ class DecoderConfig:
     def token_bytes(self, ctx: int) -> int:
         """Algorithmic HBM bytes per decoded token at context `ctx`: layer weights + tied bf16
         LM head + K/V rows read by attention."""
-        kv = self.n_layers * 2 * self.n_kv * self.head_dim * 2 * ctx
+        per_elem = 2.0 if not self.kv_bits else self.kv_bits / 8 + 4 / self.kv_group
+        kv = int(self.n_layers * 2 * self.n_kv * self.head_dim * per_elem * ctx)
         return self.n_layers * self.layer_param_bytes() + self.vocab * self.hidden * 2 + kv
 
 
@@ -170,9 +173,16 @@ class DecoderRuntime:
         self.q, self.k, self.v = DeviceBuffer(cfg.n_q * 2), DeviceBuffer(cfg.n_kvd * 2), DeviceBuffer(cfg.n_kvd * 2)
         self.att, self.mid = DeviceBuffer(cfg.n_q * 2), DeviceBuffer(cfg.inter * 2)
         self.logits = DeviceBuffer(cfg.vocab * 2)
-        cache_bytes = cfg.n_kv * cfg.capacity * cfg.head_dim * 2
-        self.cache_k = [z(cache_bytes) for _ in range(cfg.n_layers)]
-        self.cache_v = [z(cache_bytes) for _ in range(cfg.n_layers)]
+        if cfg.kv_bits:
+            if persistent:
+                raise ValueError("the whole-token kernel reads a bf16 KV cache; use the graph mode with kv_bits")
+            mk = lambda: native.QuantKvCache(cfg.n_kv, cfg.capacity, cfg.head_dim, cfg.kv_bits, cfg.kv_group)
+            self.cache_k = [mk() for _ in range(cfg.n_layers)]
+            self.cache_v = [mk() for _ in range(cfg.n_layers)]
+        else:
+            cache_bytes = cfg.n_kv * cfg.capacity * cfg.head_dim * 2
+            self.cache_k = [z(cache_bytes) for _ in range(cfg.n_layers)]
+            self.cache_v = [z(cache_bytes) for _ in range(cfg.n_layers)]
         pb, cb = native.sdpa_workspace_bytes(cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.head_dim, cfg.capacity)
         self.sdpa_partials, self.sdpa_counters = DeviceBuffer(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
@@ -216,7 +226,17 @@ class DecoderRuntime:
                                    has_bias=int(c.qkv_bias))))
             rope = dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, rope_dims=c.head_dim, theta=c.theta,
                         capacity=c.capacity, eps=c.eps)
-            if c.fuse_rope_store:
+            if c.kv_bits:
+                # quantised cache: rotate q in place, then quantise the rotated K row and the V row
+                qa = [arg(self.q)] + ([arg(w.vecs[p + "self_attn.q_norm"])] if c.qk_norm else []) + [arg(self.offset)]
+                t.append(Dispatch(name("rmsnorm_rope_q_decode" if c.qk_norm else "rope_q_decode"), qa, rope))
+                K, V = self.cache_k[l], self.cache_v[l]
+                ka = [arg(self.k), arg(self.v)] + ([arg(w.vecs[p + "self_attn.k_norm"])] if c.qk_norm else [])
+                ka += [arg(b) for b in (K.packed, K.scales, K.biases, V.packed, V.scales, V.biases)]
+                ka += [arg(self.offset), arg(self.offset)]
+                t.append(Dispatch(name(f"rope_kv_cache_store_decode_q{c.kv_bits}"), ka,
+                                  dict(rope, has_norm=int(c.qk_norm), group=c.kv_group)))
+            elif c.fuse_rope_store:
                 a = [arg(self.q), arg(self.k), arg(self.v)]
                 if c.qk_norm:
                     a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
@@ -234,11 +254,19 @@ class DecoderRuntime:
                 t.append(Dispatch(name("rope_kv_cache_store_decode"),
                                   [arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]),
                                    arg(self.offset), arg(self.offset)], rope))
-            t.append(Dispatch(name("sdpa_decode"),
-                              [arg(self.q), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
-                               arg(self.att), arg(self.sdpa_partials), arg(self.sdpa_counters)],
-                              dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, capacity=c.capacity,
-                                   max_len=c.capacity)))
+            if c.kv_bits:
+                K, V = self.cache_k[l], self.cache_v[l]
+                t.append(Dispatch(name(f"sdpa_decode_q{c.kv_bits}"),
+                                  [arg(self.q)] + [arg(b) for b in (K.packed, K.scales, K.biases, V.packed, V.scales, V.biases)]
+                                  + [arg(self.kv_len), arg(self.att), arg(self.sdpa_partials), arg(self.sdpa_counters)],
+                                  dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, capacity=c.capacity,
+                                       max_len=c.capacity, group=c.kv_group)))
+            else:
+                t.append(Dispatch(name("sdpa_decode"),
+                                  [arg(self.q), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+                                   arg(self.att), arg(self.sdpa_partials), arg(self.sdpa_counters)],
+                                  dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, capacity=c.capacity,
+                                       max_len=c.capacity)))
             Wo = w.mats[p + "self_attn.o_proj"]
             t.append(Dispatch(name("linear_residual"),
                               [arg(self.att)] + self._wargs(Wo) + [arg(self.x[0]), arg(self.x[1])],
@@ -312,13 +340,20 @@ class DecoderRuntime:
                 for nm, dst in (("q", b["q"]), ("k", b["k"]), ("v", b["v"])):
                     bias = w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None
                     native.qgemm(w.mats[p + f"self_attn.{nm}_proj"], b["xn"], m, bias, None, dst, b["ws"])
-                native.qkv_rope_store_rows(b["q"], b["k"], b["v"],
-                                           w.vecs.get(p + "self_attn.q_norm") if c.qk_norm else None,
-                                           w.vecs.get(p + "self_attn.k_norm") if c.qk_norm else None,
-                                           c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.theta, c.eps, m, pos, c.capacity,
-                                           self.cache_k[l], self.cache_v[l])
-                native.sdpa_decode_rows(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + 1, c.n_heads, c.n_kv,
-                                        c.head_dim, c.head_dim, c.capacity, scale, b["part"], b["cnt"])
+                qn = w.vecs.get(p + "self_attn.q_norm") if c.qk_norm else None
+                kn = w.vecs.get(p + "self_attn.k_norm") if c.qk_norm else None
+                if c.kv_bits:
+                    native.qkv_rope_store_rows(b["q"], None, None, qn, None, c.n_heads, 0, c.head_dim, c.head_dim,
+                                               c.theta, c.eps, m, pos, c.capacity, None, None)
+                    native.kv_cache_store_quant(b["k"], b["v"], kn, c.n_kv, c.head_dim, c.head_dim, c.theta, c.eps,
+                                                None, pos, m, self.cache_k[l], self.cache_v[l])
+                    native.sdpa_decode_quant(b["q"], self.cache_k[l], self.cache_v[l], b["att"], None, pos + 1,
+                                             pos + m, m, c.n_heads, scale, b["part"], b["cnt"])
+                else:
+                    native.qkv_rope_store_rows(b["q"], b["k"], b["v"], qn, kn, c.n_heads, c.n_kv, c.head_dim, c.head_dim,
+                                               c.theta, c.eps, m, pos, c.capacity, self.cache_k[l], self.cache_v[l])
+                    native.sdpa_decode_rows(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + 1, c.n_heads,
+                                            c.n_kv, c.head_dim, c.head_dim, c.capacity, scale, b["part"], b["cnt"])
                 native.qgemm(w.mats[p + "self_attn.o_proj"], b["att"], m, None, b["x"], b["x2"], b["ws"])
                 native.rmsnorm_rows(b["x2"], w.vecs[p + "post_attention_layernorm"], c.eps, m, c.hidden, b["xn"])
                 native.qgemm_swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], b["xn"], m, c.swiglu_variant,

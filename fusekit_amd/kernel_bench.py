@@ -86,6 +86,37 @@ def case_qgemv(d, reps, n, k, bits, pool, tag):
     _emit(f"qgemv_{tag}_q{bits}_warm_serial", _time_graph(d, warm, reps), nbytes, n=n, k=k, pool=1)
 
 
+def case_sdpa_quant(d, reps, length, bits):
+    """Attention over a quantised KV cache (group 64): algorithmic bytes = packed codes + scales + biases."""
+    import numpy as np
+    n_heads, n_kv, dim, group = 32, 8, 128, 64
+    rows = n_kv * length
+    kv_bytes = 2 * rows * (dim * bits // 8 + (dim // group) * 4)
+    pool = max(2, min(256, int(600e6 // kv_bytes) + 1))
+    q, out = _bf16(n_heads * dim, 3), fk.DeviceBuffer(n_heads * dim * 2)
+    kv_len = fk.DeviceBuffer.from_numpy(np.array([length], np.uint32))
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, dim, dim, length)
+    partials, counters = fk.DeviceBuffer(max(pb, 16)), fk.zeros(max(cb, 16))
+    tasks, keep = [], []
+    for i in range(pool):
+        c = []
+        for j in range(2):
+            packed = fk.DeviceBuffer(rows * dim * bits // 8)
+            _synth(packed, rows * dim * bits // 32, 100 + 2 * i + j, 0.0, 0.0, 2, 0xFFFFFFFF)
+            sc, bi = fk.DeviceBuffer(rows * (dim // group) * 2), fk.DeviceBuffer(rows * (dim // group) * 2)
+            _synth(sc, rows * (dim // group), 300 + 2 * i + j, 0.1 if bits == 4 else 0.008, 0.01, 1)
+            _synth(bi, rows * (dim // group), 500 + 2 * i + j, -0.7, 0.2, 1)
+            c += [packed, sc, bi]
+        keep.append(c)
+        tasks.append(Dispatch(f"fusekit_sdpa_decode_q{bits}_f0", [arg(q)] + [arg(b) for b in c] +
+                              [arg(kv_len), arg(out), arg(partials), arg(counters)],
+                              {"n_heads": n_heads, "n_kv": n_kv, "head_dim": dim, "capacity": length, "max_len": length,
+                               "group": group}))
+    nbytes = kv_bytes + 2 * n_heads * dim * 2
+    _emit(f"sdpa_decode_q{bits}_L{length}_cold_serial", _time_graph(d, tasks, reps), nbytes,
+          flops=4 * n_heads * length * dim, pool=pool)
+
+
 def case_sdpa(d, reps, length):
     n_heads, n_kv, dim = 32, 8, 128
     kv_bytes = 2 * n_kv * length * dim * 2
@@ -193,6 +224,10 @@ CASES = {
     "sdpa_512": lambda d, r: case_sdpa(d, r, 512),
     "sdpa_4096": lambda d, r: case_sdpa(d, r, 4096),
     "sdpa_32768": lambda d, r: case_sdpa(d, r, 32768),
+    "sdpa_q4_4096": lambda d, r: case_sdpa_quant(d, r, 4096, 4),
+    "sdpa_q8_4096": lambda d, r: case_sdpa_quant(d, r, 4096, 8),
+    "sdpa_q4_32768": lambda d, r: case_sdpa_quant(d, r, 32768, 4),
+    "sdpa_q8_32768": lambda d, r: case_sdpa_quant(d, r, 32768, 8),
     "moe_cfg5": lambda d, r: case_moe(d, r),
     "qgemm_8": lambda d, r: case_qgemm(d, r, 8),
     "qgemm_32": lambda d, r: case_qgemm(d, r, 32),

@@ -272,6 +272,45 @@ def sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_
                              _ptr(partials), _ptr(counters), _ptr(stream)))
 
 
+class _KvQuantCache(C.Structure):
+    _fields_ = [("packed", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
+
+
+class QuantKvCache:
+    """One K or V cache in the quantised layout, resident in HBM."""
+
+    def __init__(self, n_kv: int, capacity: int, dim: int, bits: int, group: int = 64, zero: bool = True):
+        self.n_kv, self.capacity, self.dim, self.bits, self.group = n_kv, capacity, dim, bits, group
+        alloc = zeros if zero else DeviceBuffer
+        self.packed = alloc(n_kv * capacity * dim * bits // 8)
+        self.scales = alloc(n_kv * capacity * (dim // group) * 2)
+        self.biases = alloc(n_kv * capacity * (dim // group) * 2)
+
+    @property
+    def c(self) -> _KvQuantCache:
+        return _KvQuantCache(self.packed.ptr, self.scales.ptr, self.biases.ptr)
+
+    @property
+    def nbytes(self) -> int:
+        return self.packed.nbytes + self.scales.nbytes + self.biases.nbytes
+
+
+def kv_cache_store_quant(k, v, k_norm, n_kv, head_dim, rope_dims, theta, eps, d_offset, offset, rows, K: QuantKvCache,
+                         V: QuantKvCache, stream=None):
+    check(lib.fk_kv_cache_store_quant(_ptr(k), _ptr(v), _ptr(k_norm), C.c_uint32(n_kv), C.c_uint32(head_dim),
+                                      C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), _ptr(d_offset),
+                                      C.c_uint32(offset), C.c_uint32(rows), C.c_uint32(K.capacity), C.c_uint32(K.bits),
+                                      C.c_uint32(K.group), C.byref(K.c), C.byref(V.c), _ptr(stream)))
+
+
+def sdpa_decode_quant(q, K: QuantKvCache, V: QuantKvCache, out, d_kv_len, kv_len, max_len, rows, n_heads, scale,
+                      partials, counters, stream=None):
+    check(lib.fk_sdpa_decode_quant(_ptr(q), C.byref(K.c), C.byref(V.c), _ptr(out), _ptr(d_kv_len), C.c_uint32(kv_len),
+                                   C.c_uint32(max_len), C.c_uint32(rows), C.c_uint32(n_heads), C.c_uint32(K.n_kv),
+                                   C.c_uint32(K.dim), C.c_uint32(V.dim), C.c_uint32(K.capacity), C.c_uint32(K.bits),
+                                   C.c_uint32(K.group), C.c_float(scale), _ptr(partials), _ptr(counters), _ptr(stream)))
+
+
 def rmsnorm_rows(x, w, eps, rows, hidden, y, stream=None):
     check(lib.fk_rmsnorm_rows(_ptr(x), _ptr(w), C.c_float(eps), C.c_uint32(rows), C.c_uint32(hidden), _ptr(y), _ptr(stream)))
 

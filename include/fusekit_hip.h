@@ -258,6 +258,30 @@ fk_status fk_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint1
                          uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
                          float *partials, uint32_t *counters, fk_stream s);
 
+/* ---- quantised KV cache (mlx-lm QuantizedKVCache: kv_bits = 4 | 8) ----------------
+ * Layout: packed uint32 [n_kv, capacity, dim*bits/32], scales / biases bf16
+ * [n_kv, capacity, dim/group] (src/codegen/kernels/sdpa_decode_quant.rs:10-17).
+ * fk_kv_cache_store_quant replaces src/codegen/kernels/rope_kv_cache_store_decode_quant.rs:
+ * rows of new K (RoPE, optional head norm, kept in fp32) and V are quantised per group and
+ * written at cache rows (offset + r) % capacity.  fk_sdpa_decode_quant replaces
+ * sdpa_decode_quant.rs: attention with k = code * scale + bias evaluated in fp32; split,
+ * workspace and counters exactly as fk_sdpa_decode; `rows` > 1 as fk_sdpa_decode_rows. */
+typedef struct fk_kv_quant_cache {
+    uint32_t *packed;
+    uint16_t *scales;
+    uint16_t *biases;
+} fk_kv_quant_cache;
+fk_status fk_kv_cache_store_quant(const uint16_t *k, const uint16_t *v, const uint16_t *k_norm, uint32_t n_kv,
+                                  uint32_t head_dim, uint32_t rope_dims, float theta, float eps,
+                                  const uint32_t *d_offset, uint32_t offset, uint32_t rows, uint32_t capacity,
+                                  uint32_t bits, uint32_t group, const fk_kv_quant_cache *cache_k,
+                                  const fk_kv_quant_cache *cache_v, fk_stream s);
+fk_status fk_sdpa_decode_quant(const uint16_t *q, const fk_kv_quant_cache *cache_k, const fk_kv_quant_cache *cache_v,
+                               uint16_t *out, const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len,
+                               uint32_t rows, uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim,
+                               uint32_t capacity, uint32_t bits, uint32_t group, float scale, float *partials,
+                               uint32_t *counters, fk_stream s);
+
 /* ---- several active token rows (multi-token verification, chunked prefill) ----
  * The reference compiles such variants with active_m > 1 (src/target/mod.rs:170-200,
  * variants `prefill_mN`, src/patch.rs:103-150; causal attention

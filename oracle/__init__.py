@@ -59,6 +59,8 @@ class Layer(C.Structure):
         ("bq", _u16p), ("bk", _u16p), ("bv", _u16p),
         ("q_norm", _u16p), ("k_norm", _u16p),
         ("cache_k", _u16p), ("cache_v", _u16p),
+        ("ck_packed", _u32p), ("ck_scales", _u16p), ("ck_biases", _u16p),
+        ("cv_packed", _u32p), ("cv_scales", _u16p), ("cv_biases", _u16p),
     ]
 
 
@@ -73,6 +75,7 @@ class Model(C.Structure):
         ("lm_head", Weight),
         ("final_norm", _u16p),
         ("layers", C.POINTER(Layer)),
+        ("kv_bits", C.c_int), ("kv_group", C.c_int),
     ]
 
 
@@ -329,3 +332,38 @@ def qgemm(W: QWeight, x: np.ndarray, bias=None) -> np.ndarray:
     y = np.empty((m, W.n), dtype=np.uint16)
     _lib.fko_qgemm(C.byref(W.c), _p(x, _u16p), C.c_int64(m), _p(bias, _u16p), _p(y, _u16p))
     return y
+
+
+# ------------------------------------------------------------------ quantised KV cache
+
+class QuantCache:
+    """K or V cache in the mlx-lm QuantizedKVCache layout: packed [n_kv, capacity, D*bits/32],
+    scales / biases [n_kv, capacity, D/group]."""
+
+    def __init__(self, n_kv: int, capacity: int, dim: int, bits: int, group: int = 64):
+        self.n_kv, self.capacity, self.dim, self.bits, self.group = n_kv, capacity, dim, bits, group
+        self.packed = np.zeros((n_kv, capacity, dim * bits // 32), np.uint32)
+        self.scales = np.zeros((n_kv, capacity, dim // group), np.uint16)
+        self.biases = np.zeros((n_kv, capacity, dim // group), np.uint16)
+
+    def dequantize(self) -> np.ndarray:
+        flat = QWeight(self.packed.reshape(-1, self.packed.shape[-1]), self.scales.reshape(-1, self.scales.shape[-1]),
+                       self.biases.reshape(-1, self.biases.shape[-1]), self.n_kv * self.capacity, self.dim, self.bits, self.group)
+        return dequantize(flat).reshape(self.n_kv, self.capacity, self.dim)
+
+
+def rope_kv_store_quant(k, v, k_norm, n_kv, head_dim, rope_dims, theta, eps, pos, write_offset, K: QuantCache, V: QuantCache):
+    _lib.fko_rope_kv_store_quant(_p(k, _u16p), _p(v, _u16p), _p(k_norm, _u16p), C.c_int64(n_kv), C.c_int64(head_dim),
+                                 C.c_int64(rope_dims), C.c_float(theta), C.c_float(eps), C.c_uint32(pos),
+                                 C.c_uint32(write_offset), C.c_uint32(K.capacity), C.c_int(K.bits), C.c_int(K.group),
+                                 _p(K.packed, _u32p), _p(K.scales, _u16p), _p(K.biases, _u16p),
+                                 _p(V.packed, _u32p), _p(V.scales, _u16p), _p(V.biases, _u16p))
+
+
+def sdpa_decode_quant(q, K: QuantCache, V: QuantCache, n_heads, kv_len, scale) -> np.ndarray:
+    out = np.empty(n_heads * V.dim, dtype=np.uint16)
+    _lib.fko_sdpa_decode_quant(_p(q, _u16p), _p(K.packed, _u32p), _p(K.scales, _u16p), _p(K.biases, _u16p),
+                               _p(V.packed, _u32p), _p(V.scales, _u16p), _p(V.biases, _u16p), C.c_int64(n_heads),
+                               C.c_int64(K.n_kv), C.c_int64(K.dim), C.c_int64(V.dim), C.c_uint32(kv_len),
+                               C.c_uint32(K.capacity), C.c_int(K.bits), C.c_int(K.group), C.c_float(scale), _p(out, _u16p))
+    return out

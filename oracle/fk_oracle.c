@@ -440,6 +440,95 @@ FKO_API void fko_kv_store(const uint16_t *k, const uint16_t *v, int64_t n_kv, in
     }
 }
 
+/* ------------------------------------------------- quantised KV cache */
+/*
+ * Store (src/codegen/kernels/rope_kv_cache_store_decode_quant.rs:100-260): the K row after
+ * half-split RoPE stays in fp32 (it is NOT rounded to T before quantisation), the V row is
+ * taken as is; every group of `group` dims along the head is quantised with the Q0 formula.
+ * Layout (src/codegen/kernels/sdpa_decode_quant.rs:10-17): packed u32 [n_kv, capacity,
+ * D*bits/32], scales / biases T [n_kv, capacity, D/group].  With a norm weight the head is
+ * first normalised as in fko_headnorm_rope (T(w*T(x*r))) and rotated from those T values.
+ */
+FKO_API void fko_rope_kv_store_quant(const uint16_t *k, const uint16_t *v, const uint16_t *k_norm, int64_t n_kv,
+                                     int64_t head_dim, int64_t rope_dims, float theta, float eps, uint32_t pos,
+                                     uint32_t write_offset, uint32_t capacity, int bits, int group,
+                                     uint32_t *ck_packed, uint16_t *ck_scales, uint16_t *ck_biases,
+                                     uint32_t *cv_packed, uint16_t *cv_scales, uint16_t *cv_biases) {
+    const float base_log2 = (float)log2((double)theta);
+    const int64_t half = rope_dims / 2, words = head_dim * bits / 32, groups = head_dim / group;
+    const int64_t row = write_offset % capacity;
+    float *kr = (float *)malloc(sizeof(float) * (size_t)head_dim), *vr = (float *)malloc(sizeof(float) * (size_t)head_dim);
+    for (int64_t h = 0; h < n_kv; ++h) {
+        const uint16_t *kh = k + h * head_dim;
+        float r = 1.0f;
+        if (k_norm) {
+            double ss = 0.0;
+            for (int64_t d = 0; d < head_dim; ++d) ss += (double)bf16_to_f32(kh[d]) * (double)bf16_to_f32(kh[d]);
+            r = 1.0f / sqrtf((float)(ss / (double)head_dim) + eps);
+        }
+        for (int64_t d = 0; d < head_dim; ++d) {
+            const float x = bf16_to_f32(kh[d]);
+            kr[d] = k_norm ? rbf(bf16_to_f32(k_norm[d]) * rbf(x * r)) : x;
+            vr[d] = bf16_to_f32(v[h * head_dim + d]);
+        }
+        for (int64_t d = 0; d < half; ++d) {
+            float lo, hi;
+            rope_pair(kr[d], kr[d + half], d, half, pos, base_log2, &lo, &hi);
+            kr[d] = lo;
+            kr[d + half] = hi;
+        }
+        const int64_t o = h * (int64_t)capacity + row;
+        fko_quantize_affine(kr, 1, head_dim, bits, group, ck_packed + o * words, ck_scales + o * groups, ck_biases + o * groups);
+        fko_quantize_affine(vr, 1, head_dim, bits, group, cv_packed + o * words, cv_scales + o * groups, cv_biases + o * groups);
+    }
+    free(kr); free(vr);
+}
+
+/* Attention over the quantised cache (sdpa_decode_quant.rs): k_jd = code * scale + bias in fp32,
+ * everything else as fko_sdpa_decode. */
+FKO_API void fko_sdpa_decode_quant(const uint16_t *q, const uint32_t *ck_packed, const uint16_t *ck_scales,
+                                   const uint16_t *ck_biases, const uint32_t *cv_packed, const uint16_t *cv_scales,
+                                   const uint16_t *cv_biases, int64_t n_heads, int64_t n_kv, int64_t qk_dim,
+                                   int64_t v_dim, uint32_t kv_len, uint32_t capacity, int bits, int group, float scale,
+                                   uint16_t *out) {
+    const int64_t per_kv = n_heads / n_kv;
+    const int per_word = 32 / bits;
+    const uint32_t mask = (1u << bits) - 1u;
+#pragma omp parallel for schedule(static)
+    for (int64_t h = 0; h < n_heads; ++h) {
+        const int64_t kvh = h / per_kv;
+        float *s = (float *)malloc(sizeof(float) * (size_t)kv_len);
+        double *acc = (double *)calloc((size_t)v_dim, sizeof(double));
+        float m = -INFINITY;
+        for (uint32_t j = 0; j < kv_len; ++j) {
+            const int64_t o = kvh * (int64_t)capacity + j;
+            double dot = 0.0;
+            for (int64_t d = 0; d < qk_dim; ++d) {
+                const uint32_t code = (ck_packed[o * (qk_dim / per_word) + d / per_word] >> ((d % per_word) * bits)) & mask;
+                const float kd = (float)code * bf16_to_f32(ck_scales[o * (qk_dim / group) + d / group]) +
+                                 bf16_to_f32(ck_biases[o * (qk_dim / group) + d / group]);
+                dot += (double)bf16_to_f32(q[h * qk_dim + d]) * (double)kd;
+            }
+            s[j] = (float)dot * scale;
+            m = s[j] > m ? s[j] : m;
+        }
+        double l = 0.0;
+        for (uint32_t j = 0; j < kv_len; ++j) {
+            const float p = expf(s[j] - m);
+            l += (double)p;
+            const int64_t o = kvh * (int64_t)capacity + j;
+            for (int64_t d = 0; d < v_dim; ++d) {
+                const uint32_t code = (cv_packed[o * (v_dim / per_word) + d / per_word] >> ((d % per_word) * bits)) & mask;
+                const float vd = (float)code * bf16_to_f32(cv_scales[o * (v_dim / group) + d / group]) +
+                                 bf16_to_f32(cv_biases[o * (v_dim / group) + d / group]);
+                acc[d] += (double)p * (double)vd;
+            }
+        }
+        for (int64_t d = 0; d < v_dim; ++d) out[h * v_dim + d] = f32_to_bf16((float)(acc[d] / l));
+        free(s); free(acc);
+    }
+}
+
 /* ------------------------------------------------------------ K4: SDPA */
 /* s_j = (q . k_j) * scale in fp32; softmax in fp32 (probabilities never
  * rounded to T); o = sum p_j v_j / l; one final round
@@ -652,6 +741,10 @@ typedef struct {
     const uint16_t *bq, *bk, *bv;       /* optional projection biases */
     const uint16_t *q_norm, *k_norm;    /* optional per-head norms [head_dim] */
     uint16_t *cache_k, *cache_v;        /* [n_kv, capacity, head_dim] */
+    /* quantised cache (model kv_bits != 0): packed [n_kv, capacity, head_dim*bits/32], scales / biases
+     * [n_kv, capacity, head_dim/group] */
+    uint32_t *ck_packed; uint16_t *ck_scales, *ck_biases;
+    uint32_t *cv_packed; uint16_t *cv_scales, *cv_biases;
 } fko_layer;
 
 typedef struct {
@@ -663,6 +756,7 @@ typedef struct {
     fko_weight lm_head; /* [vocab, hidden]; may alias embed (tied) */
     const uint16_t *final_norm;
     const fko_layer *layers;
+    int kv_bits, kv_group; /* 0: bf16 cache */
 } fko_model;
 
 FKO_API uint32_t fko_decoder_step(const fko_model *M, uint32_t token, uint32_t offset,
@@ -676,7 +770,13 @@ FKO_API uint32_t fko_decoder_step(const fko_model *M, uint32_t token, uint32_t o
     for (int64_t l = 0; l < M->n_layers; ++l) {
         const fko_layer *L = &M->layers[l];
         fko_rmsnorm_qkv(x, L->input_norm, M->eps, &L->wq, &L->wk, &L->wv, L->bq, L->bk, L->bv, q, k, v);
-        if (L->q_norm) {
+        if (M->kv_bits) {
+            if (L->q_norm) fko_headnorm_rope(q, L->q_norm, M->n_heads, M->head_dim, M->head_dim, M->eps, M->theta, offset);
+            else fko_rope_q(q, M->n_heads, M->head_dim, M->head_dim, M->theta, offset);
+            fko_rope_kv_store_quant(k, v, L->k_norm, M->n_kv, M->head_dim, M->head_dim, M->theta, M->eps, offset, offset,
+                                    M->capacity, M->kv_bits, M->kv_group, L->ck_packed, L->ck_scales, L->ck_biases,
+                                    L->cv_packed, L->cv_scales, L->cv_biases);
+        } else if (L->q_norm) {
             fko_headnorm_rope(q, L->q_norm, M->n_heads, M->head_dim, M->head_dim, M->eps, M->theta, offset);
             fko_headnorm_rope(k, L->k_norm, M->n_kv, M->head_dim, M->head_dim, M->eps, M->theta, offset);
             fko_kv_store(k, v, M->n_kv, M->head_dim, M->head_dim, offset, M->capacity, L->cache_k, L->cache_v);
@@ -685,8 +785,13 @@ FKO_API uint32_t fko_decoder_step(const fko_model *M, uint32_t token, uint32_t o
             fko_rope_kv_store(k, v, M->n_kv, M->head_dim, M->head_dim, M->theta, offset, offset, M->capacity,
                               L->cache_k, L->cache_v);
         }
-        fko_sdpa_decode(q, L->cache_k, L->cache_v, M->n_heads, M->n_kv, M->head_dim, M->head_dim, offset + 1,
-                        M->capacity, M->attn_scale, att);
+        if (M->kv_bits)
+            fko_sdpa_decode_quant(q, L->ck_packed, L->ck_scales, L->ck_biases, L->cv_packed, L->cv_scales, L->cv_biases,
+                                  M->n_heads, M->n_kv, M->head_dim, M->head_dim, offset + 1, M->capacity, M->kv_bits,
+                                  M->kv_group, M->attn_scale, att);
+        else
+            fko_sdpa_decode(q, L->cache_k, L->cache_v, M->n_heads, M->n_kv, M->head_dim, M->head_dim, offset + 1,
+                            M->capacity, M->attn_scale, att);
         fko_linear_residual(&L->wo, att, x, NULL, x2);
         fko_gateup_swiglu(x2, L->post_norm, M->eps, &L->wgate, &L->wup, M->swiglu_variant, mid);
         fko_linear_residual(&L->wdown, mid, x2, NULL, x);

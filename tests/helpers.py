@@ -89,14 +89,25 @@ class OracleDecoder:
                                 else (null, null, null))
             L.q_norm, L.k_norm = ((vec(p + "self_attn.q_norm"), vec(p + "self_attn.k_norm")) if cfg.qk_norm
                                   else (null, null))
-            ck, cv = np.zeros(cache_elems, np.uint16), np.zeros(cache_elems, np.uint16)
-            self.keep += [ck, cv]
-            L.cache_k, L.cache_v = ck.ctypes.data_as(u16p), cv.ctypes.data_as(u16p)
+            if getattr(cfg, "kv_bits", 0):
+                u32p = C.POINTER(C.c_uint32)
+                K = oracle.QuantCache(cfg.n_kv, cfg.capacity, cfg.head_dim, cfg.kv_bits, cfg.kv_group)
+                V = oracle.QuantCache(cfg.n_kv, cfg.capacity, cfg.head_dim, cfg.kv_bits, cfg.kv_group)
+                self.keep += [K, V]
+                L.ck_packed, L.ck_scales, L.ck_biases = (K.packed.ctypes.data_as(u32p), K.scales.ctypes.data_as(u16p),
+                                                         K.biases.ctypes.data_as(u16p))
+                L.cv_packed, L.cv_scales, L.cv_biases = (V.packed.ctypes.data_as(u32p), V.scales.ctypes.data_as(u16p),
+                                                         V.biases.ctypes.data_as(u16p))
+            else:
+                ck, cv = np.zeros(cache_elems, np.uint16), np.zeros(cache_elems, np.uint16)
+                self.keep += [ck, cv]
+                L.cache_k, L.cache_v = ck.ctypes.data_as(u16p), cv.ctypes.data_as(u16p)
         emb = mat("embed_tokens")
         head = mat("lm_head") if "lm_head" in weights.mats else emb
         self.model = oracle.Model(cfg.n_layers, cfg.hidden, cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab,
                                   cfg.eps, cfg.theta, 1.0 / np.sqrt(cfg.head_dim), 1.0, cfg.swiglu_variant,
-                                  cfg.capacity, emb, head, vec("final_norm"), self.layers)
+                                  cfg.capacity, emb, head, vec("final_norm"), self.layers,
+                                  getattr(cfg, "kv_bits", 0), getattr(cfg, "kv_group", 64))
 
     def step(self, token: int, offset: int, want_logits: bool = False):
         logits = np.empty(self.cfg.vocab, np.uint16) if want_logits else None

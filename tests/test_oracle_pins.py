@@ -382,3 +382,53 @@ def test_qgemm_rows_are_qgemv():
     y = oracle.qgemm(W, x, bias)
     for r in range(4):
         assert np.array_equal(y[r], oracle.qgemv(W, x[r], bias))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_quantised_kv_store_and_attention(bits):
+    """Quantised KV cache.  Store: V codes are the pinned quantiser applied to the V row; K without
+    rotation likewise; with rotation the dequantised row stays within half a quantisation step of the
+    fp32 rotation (which agrees with the pinned bf16 RoPE to one bf16 rounding); only the addressed
+    row is written.  Attention: float64 softmax attention over the dequantised cache."""
+    n_kv, dim, cap, group = 2, 128, 16, 64
+    k, v = normal_bf16(1, n_kv * dim), normal_bf16(2, n_kv * dim)
+    K, V = oracle.QuantCache(n_kv, cap, dim, bits, group), oracle.QuantCache(n_kv, cap, dim, bits, group)
+    oracle.rope_kv_store_quant(k, v, None, n_kv, dim, 0, 1e4, 0.0, 21, 21, K, V)        # rope_dims 0: plain
+    row = 21 % cap
+    for h in range(n_kv):
+        for src, cache in ((k, K), (v, V)):
+            Q = oracle.quantize(oracle.bf16_to_f32(src[h * dim:(h + 1) * dim]).reshape(1, dim), bits, group)
+            assert np.array_equal(cache.packed[h, row], Q.w[0]) and np.array_equal(cache.scales[h, row], Q.scales[0])
+            assert np.array_equal(cache.biases[h, row], Q.biases[0])
+    untouched = np.ones(cap, bool)
+    untouched[row] = False
+    assert not K.packed[:, untouched].any() and not V.scales[:, untouched].any()
+    K2, V2 = oracle.QuantCache(n_kv, cap, dim, bits, group), oracle.QuantCache(n_kv, cap, dim, bits, group)
+    oracle.rope_kv_store_quant(k, v, None, n_kv, dim, dim, 1e4, 0.0, 7, 3, K2, V2)      # rotate at pos 7, row 3
+    ck, cv = np.zeros(n_kv * cap * dim, np.uint16), np.zeros(n_kv * cap * dim, np.uint16)
+    oracle.rope_kv_store(k, v, n_kv, dim, dim, 1e4, 7, 3, cap, ck, cv)
+    want = oracle.bf16_to_f32(ck).reshape(n_kv, cap, dim)[:, 3]
+    got = K2.dequantize()[:, 3]
+    step = np.abs(oracle.bf16_to_f32(K2.scales[:, 3])).repeat(group, axis=-1)
+    # half a step inside the range; the edge opposite the anchor may fall short by up to ~1.6 steps
+    # because the scale is re-derived from the anchor (same bound as the weight quantiser's pin)
+    err = np.abs(got - want)
+    assert np.all(err <= 1.6 * step + 2.0 ** -8 * np.abs(want) + 1e-6)
+    assert np.mean(err / (step + 2.0 ** -7 * np.abs(want))) <= 0.3   # `want` itself carries one bf16 rounding
+    # attention over a filled cache
+    rs = rng(3)
+    for c in (K, V):
+        c.packed[:] = rs.integers(0, 2 ** 32, c.packed.shape, dtype=np.uint32)
+        c.scales[:] = oracle.f32_to_bf16((rs.standard_normal(c.scales.shape) * 0.02 + 0.1).astype(np.float32))
+        c.biases[:] = oracle.f32_to_bf16((rs.standard_normal(c.biases.shape) * 0.3).astype(np.float32))
+    n_heads, kv_len, scale = 4, 11, 0.09
+    q = normal_bf16(4, n_heads * dim)
+    out = oracle.bf16_to_f32(oracle.sdpa_decode_quant(q, K, V, n_heads, kv_len, scale)).reshape(n_heads, dim)
+    kd, vd = K.dequantize().astype(np.float64), V.dequantize().astype(np.float64)
+    qf = oracle.bf16_to_f32(q).astype(np.float64).reshape(n_heads, dim)
+    for h in range(n_heads):
+        kvh = h // (n_heads // n_kv)
+        sc = (kd[kvh, :kv_len] @ qf[h]) * scale
+        p = np.exp(sc - sc.max())
+        ref = (p / p.sum()) @ vd[kvh, :kv_len]
+        assert np.all(np.abs(out[h] - ref) <= 2.0 ** -8 * np.abs(ref) + 1e-6)
