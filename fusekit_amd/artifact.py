@@ -44,6 +44,8 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
     for name in ("q", "k", "v", "att", "mid", "logits"):
         scratch(name, getattr(rt, name), "bfloat16")
     scratch("sdpa_partials", rt.sdpa_partials, "float32")
+    if rt.rope_tab is not None:
+        scratch("rope_tab", rt.rope_tab, "float32")
     for l in range(rt.cfg.n_layers):
         if rt.cfg.kv_bits:
             for nm, c in (("cache_k", rt.cache_k[l]), ("cache_v", rt.cache_v[l])):
@@ -123,7 +125,7 @@ def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "syntheti
         uniforms=dict(token="token", step_counter="step_counter", hist_counter="hist_counter", history="history"),
         model_config={k: getattr(c, k) for k in ("n_layers", "hidden", "n_heads", "n_kv", "head_dim", "inter", "vocab",
                                                   "capacity", "bits", "group", "eps", "theta", "qk_norm", "qkv_bias",
-                                                  "fuse_rope_store", "swiglu_variant", "kv_bits", "kv_group")})
+                                                  "fuse_rope_store", "swiglu_variant", "kv_bits", "kv_group", "fuse_attention")})
     with open(os.path.join(out_dir, "task_graph.json"), "w") as f:
         json.dump(graph, f, indent=1)
     manifest = dict(

@@ -506,6 +506,29 @@ fk_status fk_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_le
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_step_init_rope(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, float* rope_tab,
+                            uint32_t rope_dims, float theta, fk_stream s) {
+    if (!rope_tab) return set_error(FK_ERR_INVALID, "fk_step_init_rope: null table");
+    Launch l;
+    FK_TRY(plan_step_init(step_counter, offset, kv_len, &l, rope_tab, rope_dims, theta_log2(theta)));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_rope_store_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_norm,
+                                    const uint16_t* k_norm, uint16_t* cache_k, uint16_t* cache_v, uint16_t* out,
+                                    const uint32_t* d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
+                                    uint32_t n_kv, uint32_t head_dim, uint32_t rope_dims, float theta, float eps,
+                                    uint32_t capacity, float scale, const float* rope_tab, float* partials,
+                                    uint32_t* counters, fk_stream s) {
+    SdpaFusion f;
+    f.k_new = k; f.v_new = v; f.q_norm = q_norm; f.k_norm = k_norm;
+    f.rope_dims = rope_dims; f.eps = eps; f.base_log2 = theta_log2(theta); f.rope_tab = rope_tab;
+    Launch l;
+    FK_TRY(plan_sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_kv, head_dim, head_dim,
+                            capacity, scale, partials, counters, &l, 1, nullptr, &f));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_copy(void* dst, const void* src, size_t nbytes, fk_stream s) {
     Launch l;
     FK_TRY(plan_copy(dst, src, nbytes, &l));

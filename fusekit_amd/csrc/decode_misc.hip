@@ -226,24 +226,37 @@ struct StepArgs {
     uint32_t* step_counter;
     uint32_t* offset;
     uint32_t* kv_len;
+    float* rope_tab;  // optional: (cos, sin) of every rotary pair at this position, for all layers
+    uint32_t half;
+    float base_log2;
 };
 __global__ void step_init_kernel(const StepArgs a) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        const uint32_t o = *a.step_counter;
+    const uint32_t o = *a.step_counter;
+    __syncthreads();  // every thread has read the counter before thread 0 advances it
+    if (threadIdx.x == 0) {
         *a.step_counter = o + 1;
         *a.offset = o;
         *a.kv_len = o + 1;
     }
+    if (a.rope_tab && threadIdx.x < a.half) {
+        float cs, sn;
+        rope_cos_sin(threadIdx.x, a.half, o, a.base_log2, cs, sn);
+        a.rope_tab[2 * threadIdx.x] = cs;
+        a.rope_tab[2 * threadIdx.x + 1] = sn;
+    }
 }
 
-fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out) {
+fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out, float* rope_tab,
+                         uint32_t rope_dims, float base_log2) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!step_counter || !offset || !kv_len) return set_error(FK_ERR_INVALID, "step_init: null pointer");
-    StepArgs a{step_counter, offset, kv_len};
+    if (rope_tab && (rope_dims == 0 || rope_dims % 2 || rope_dims > 512))
+        return set_error(FK_ERR_INVALID, "step_init: rope_dims must be even, at most 512");
+    StepArgs a{step_counter, offset, kv_len, rope_tab, rope_tab ? rope_dims / 2 : 0u, base_log2};
     out->func = reinterpret_cast<const void*>(&step_init_kernel);
     out->grid = dim3(1, 1, 1);
-    out->block = dim3(kWave, 1, 1);
+    out->block = dim3(rope_tab && rope_dims / 2 > kWave ? ((rope_dims / 2 + kWave - 1) / kWave) * kWave : kWave, 1, 1);
     out->shmem = 0;
     out->set_args(a);
     return FK_OK;

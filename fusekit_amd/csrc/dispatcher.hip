@@ -106,11 +106,20 @@ fk_status bind_weight(const Dispatch& d, uint32_t bits, uint32_t group, uint32_t
 
 // ------------------------------------------------------------------ families
 
+// step_counter, offset, kv_len, [rope_tab]  (the table: parameters rope_dims, theta)
 fk_status plan_step(const Dispatch& d, Launch* l, SlotRW* rw) {
-    FK_TRY(need_args(d, 3));
+    FK_TRY(need_args(d, d.args.size() == 4 ? 4 : 3));
     for (int i = 0; i < 3; ++i) FK_TRY(need_bytes(d, i, 4));
     rw->reads = {0};
     rw->writes = {0, 1, 2};
+    if (d.args.size() == 4) {
+        const uint32_t rope_dims = d.u("rope_dims");
+        if (rope_dims == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rope_dims parameter missing");
+        FK_TRY(need_bytes(d, 3, (size_t)rope_dims * 4));
+        rw->writes.push_back(3);
+        return plan_step_init(arg_ptr<uint32_t>(d, 0), arg_ptr<uint32_t>(d, 1), arg_ptr<uint32_t>(d, 2), l,
+                              arg_ptr<float>(d, 3), rope_dims, (float)log2(d.param("theta", 10000.0)));
+    }
     return plan_step_init(arg_ptr<uint32_t>(d, 0), arg_ptr<uint32_t>(d, 1), arg_ptr<uint32_t>(d, 2), l);
 }
 
@@ -411,6 +420,53 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
                             capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l);
 }
 
+// Q, K, V, [q_weight, k_weight], cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]
+// (one launch for the rope/store stage and the attention of a layer)
+fk_status plan_rope_store_sdpa(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const bool norm = d.u("has_norm", 0) != 0, table = d.u("has_table", 0) != 0;
+    const size_t c0 = norm ? 5 : 3, n = c0 + 6 + (table ? 1 : 0);
+    FK_TRY(need_args(d, n));
+    const uint32_t n_heads = d.u("n_heads"), n_kv = d.u("n_kv"), dim = d.u("head_dim");
+    const uint32_t capacity = d.u("capacity"), max_len = d.u("max_len", capacity);
+    if (n_heads == 0 || n_kv == 0 || dim == 0 || capacity == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / head_dim / capacity parameters missing");
+    const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)dim);
+    SdpaFusion f;
+    f.rope_dims = d.u("rope_dims", dim);
+    f.eps = (float)d.param("eps", 1e-6);
+    f.base_log2 = base_log2_of(d);
+    FK_TRY(need_bytes(d, 0, (size_t)n_heads * dim * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)n_kv * dim * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)n_kv * dim * 2));
+    f.k_new = arg_ptr<const uint16_t>(d, 1);
+    f.v_new = arg_ptr<const uint16_t>(d, 2);
+    if (norm) {
+        FK_TRY(need_bytes(d, 3, (size_t)dim * 2));
+        FK_TRY(need_bytes(d, 4, (size_t)dim * 2));
+        f.q_norm = arg_ptr<const uint16_t>(d, 3);
+        f.k_norm = arg_ptr<const uint16_t>(d, 4);
+    }
+    FK_TRY(need_bytes(d, c0, (size_t)n_kv * capacity * dim * 2));
+    FK_TRY(need_bytes(d, c0 + 1, (size_t)n_kv * capacity * dim * 2));
+    FK_TRY(need_bytes(d, c0 + 2, 4));
+    FK_TRY(need_bytes(d, c0 + 3, (size_t)n_heads * dim * 2));
+    size_t pb = 0, cb = 0;
+    FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, dim, dim, max_len, &pb, &cb));
+    FK_TRY(need_bytes(d, c0 + 4, pb));
+    FK_TRY(need_bytes(d, c0 + 5, cb));
+    if (table) {
+        FK_TRY(need_bytes(d, c0 + 6, (size_t)f.rope_dims * 4));
+        f.rope_tab = arg_ptr<const float>(d, c0 + 6);
+    }
+    for (uint32_t i = 0; i < n; ++i)
+        if (i != c0 + 3) rw->reads.push_back(i);
+    rw->writes = {(uint32_t)c0, (uint32_t)c0 + 1, (uint32_t)c0 + 3, (uint32_t)c0 + 4, (uint32_t)c0 + 5};
+    return plan_sdpa_decode(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, c0),
+                            arg_ptr<const uint16_t>(d, c0 + 1), arg_ptr<uint16_t>(d, c0 + 3),
+                            arg_ptr<const uint32_t>(d, c0 + 2), 0, max_len, n_heads, n_kv, dim, dim, capacity, scale,
+                            arg_ptr<float>(d, c0 + 4), arg_ptr<uint32_t>(d, c0 + 5), l, 1, nullptr, &f);
+}
+
 // K, V, [k_weight], keys_packed, keys_scales, keys_biases, values_packed, values_scales, values_biases, offset,
 // write_offset (rope_kv_cache_store_decode_quant.rs:77-98; the capacity is a parameter here)
 fk_status plan_rope_kv_quant(const Dispatch& d, Launch* l, SlotRW* rw, uint32_t bits) {
@@ -693,6 +749,7 @@ const Family kFamilies[] = {
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, false); }},
     {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
     {"fusekit_sdpa_decode", plan_sdpa_d},
+    {"fusekit_rope_store_sdpa_decode", plan_rope_store_sdpa},
     {"fusekit_rope_kv_cache_store_decode_q4",
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv_quant(d, l, rw, 4); }},
     {"fusekit_rope_kv_cache_store_decode_q8",

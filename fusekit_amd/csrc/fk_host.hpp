@@ -138,6 +138,18 @@ struct KvQuantStore {
     float eps, base_log2;
 };
 fk_status plan_kv_store_quant(const KvQuantStore& in, Launch* out);
+// RoPE (+ head norm) of q and the new k row, the cache append and the attention in one launch:
+// q / k_new / v_new are the raw projection outputs; the cache pointers of plan_sdpa_decode are
+// the cache the rows are appended to.
+struct SdpaFusion {
+    const uint16_t* k_new = nullptr;
+    const uint16_t* v_new = nullptr;
+    const uint16_t* q_norm = nullptr;  // [qk_dim] or null
+    const uint16_t* k_norm = nullptr;
+    uint32_t rope_dims = 0;
+    float eps = 1e-6f, base_log2 = 0.f;
+    const float* rope_tab = nullptr;   // (cos, sin) per pair at this token's position, or null
+};
 uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim, bool fused);
 fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                size_t* partial_bytes, size_t* counter_bytes);
@@ -145,7 +157,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
                            const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
                            uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
                            float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows = 1,
-                           const KvQuant* quant = nullptr);
+                           const KvQuant* quant = nullptr, const SdpaFusion* fusion = nullptr);
 fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
                      uint16_t* x, Launch* out, uint32_t rows = 1);
 fk_status plan_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,
@@ -154,7 +166,8 @@ fk_status plan_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uin
 constexpr size_t kArgmaxWorkspaceBytes = 8 + 8 * 160;
 fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, uint32_t* history,
                       uint32_t* hist_counter, uint32_t hist_capacity, void* workspace, Launch* out);
-fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out);
+fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_len, Launch* out,
+                         float* rope_tab = nullptr, uint32_t rope_dims = 0, float base_log2 = 0.f);
 fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out);
 fk_status plan_copy(void* dst, const void* src, size_t nbytes, Launch* out);
 fk_status plan_quantize(const float* w, size_t n, size_t k, uint32_t bits, uint32_t group, uint32_t* packed,

@@ -68,4 +68,44 @@ __device__ __forceinline__ void head_transform(const uint16_t* src, uint16_t* ds
         for (uint32_t d = 2 * half + lane; d < dim; d += kWave) dst[d] = (uint16_t)f32_to_bf16_bits(value(d));
 }
 
+// The same transform for a head that is rotated over its whole width of at most 128 dims, split
+// in two so that a caller can put other memory requests between the loads and their use: lane
+// d < half owns the pair (d, d + half); head_pair_fetch issues every load (raw values, norm weights,
+// table entry), head_pair_apply does the arithmetic of head_transform on them.
+struct HeadPair {
+    float xlo, xhi, wlo, whi, cs, sn;
+};
+
+__device__ __forceinline__ HeadPair head_pair_fetch(const uint16_t* src, const uint16_t* nw, const float* tab,
+                                                    uint32_t half, uint32_t lane) {
+    const uint32_t d = lane < half ? lane : 0u;
+    const uint16_t* w = nw ? nw : src;  // no norm: a harmless load instead of a branch around one
+    HeadPair p;
+    p.xlo = bf16_bits_to_f32(src[d]);
+    p.xhi = bf16_bits_to_f32(src[d + half]);
+    p.wlo = bf16_bits_to_f32(w[d]);
+    p.whi = bf16_bits_to_f32(w[d + half]);
+    p.cs = tab[2 * d];
+    p.sn = tab[2 * d + 1];
+    return p;
+}
+
+__device__ __forceinline__ void head_pair_apply(const HeadPair& p, uint16_t* dst, bool has_norm, uint32_t half,
+                                                float eps, uint32_t lane, bool write) {
+    float vlo = p.xlo, vhi = p.xhi;
+    if (has_norm) {
+        float ss = lane < half ? fmaf(p.xhi, p.xhi, fmaf(p.xlo, p.xlo, 0.f)) : 0.f;
+        ss = wave_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)(2 * half) + eps);
+        vlo = round_bf16(p.wlo * round_bf16(p.xlo * r));
+        vhi = round_bf16(p.whi * round_bf16(p.xhi * r));
+    }
+    const float lo = vlo * p.cs - vhi * p.sn;
+    const float hi = vhi * p.cs + vlo * p.sn;
+    if (write && lane < half) {
+        dst[lane] = (uint16_t)f32_to_bf16_bits(lo);
+        dst[lane + half] = (uint16_t)f32_to_bf16_bits(hi);
+    }
+}
+
 }  // namespace fk

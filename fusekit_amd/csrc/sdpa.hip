@@ -52,7 +52,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
                            const uint32_t* kv_len_ptr, uint32_t kv_len_imm, uint32_t max_len, uint32_t n_heads,
                            uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
                            float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows,
-                           const KvQuant* quant) {
+                           const KvQuant* quant, const SdpaFusion* fusion) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!q || !k || !v || !out) return set_error(FK_ERR_INVALID, "sdpa: null tensor");
@@ -70,6 +70,14 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         const uint32_t g = quant->group;
         if ((g != 32 && g != 64 && g != 128) || qk_dim % g || v_dim % g)
             return set_error(FK_ERR_UNSUPPORTED, "sdpa: cache group size must be 32, 64 or 128 and divide the head dims");
+    }
+    if (fusion) {
+        if (kvq || rows != 1) return set_error(FK_ERR_UNSUPPORTED, "sdpa: the fused rope/store form takes one row and a bf16 cache");
+        if (!fusion->k_new || !fusion->v_new) return set_error(FK_ERR_INVALID, "sdpa: null new k / v row");
+        if (fusion->rope_dims % 2 || fusion->rope_dims > qk_dim)
+            return set_error(FK_ERR_INVALID, "sdpa: rope_dims must be even and within the head");
+        if ((fusion->q_norm == nullptr) != (fusion->k_norm == nullptr))
+            return set_error(FK_ERR_INVALID, "sdpa: q and k head norms come together");
     }
     if (!kv_len_ptr && rows > 1 && kv_len_imm + rows - 1 > max_len)
         return set_error(FK_ERR_INVALID, "sdpa: the last row's kv length exceeds max_len");
@@ -108,6 +116,15 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         a.v_scales = quant->v_scales; a.v_biases = quant->v_biases;
         a.kv_group = quant->group;
     }
+    if (fusion) {
+        a.k_new = fusion->k_new; a.v_new = fusion->v_new;
+        a.q_norm = fusion->q_norm; a.k_norm = fusion->k_norm;
+        a.cache_k_w = const_cast<uint16_t*>(k);
+        a.cache_v_w = const_cast<uint16_t*>(v);
+        a.rope_dims = fusion->rope_dims;
+        a.eps = fusion->eps; a.base_log2 = fusion->base_log2;
+        a.rope_tab = fusion->rope_tab;
+    }
     a.lpk = pow2_ceil(qk_dim / 8);
     a.lpv = pow2_ceil(v_dim / 8);
     a.scale = scale;
@@ -122,7 +139,23 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         case 4: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<4, Q>); break;         \
         default: func = reinterpret_cast<const void*>(&sdpa_decode_kernel<8, Q>); break;        \
     }
-    if (kvq == 4) {
+    if (fusion) {
+        // whole-width rotation of at most 128 dims with a table: the form whose loads run ahead
+        const bool fast = fusion->rope_tab && fusion->rope_dims == qk_dim && qk_dim <= 128;
+#define FK_SDPA_FUSED(F)                                                                           \
+    switch (gt) {                                                                                  \
+        case 1: func = reinterpret_cast<const void*>(&sdpa_rope_store_kernel<1, F>); break;        \
+        case 2: func = reinterpret_cast<const void*>(&sdpa_rope_store_kernel<2, F>); break;        \
+        case 4: func = reinterpret_cast<const void*>(&sdpa_rope_store_kernel<4, F>); break;        \
+        default: func = reinterpret_cast<const void*>(&sdpa_rope_store_kernel<8, F>); break;       \
+    }
+        if (fast) {
+            FK_SDPA_FUSED(true)
+        } else {
+            FK_SDPA_FUSED(false)
+        }
+#undef FK_SDPA_FUSED
+    } else if (kvq == 4) {
         FK_SDPA_PICK(4)
     } else if (kvq == 8) {
         FK_SDPA_PICK(8)
@@ -133,7 +166,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     out_launch->func = func;
     out_launch->grid = dim3(n_splits, n_kv, ((G + gt - 1) / gt) * rows);
     out_launch->block = dim3(kSdpaBlock, 1, 1);
-    out_launch->shmem = (uint32_t)(sdpa_lds_floats(gt, chunk, qk_dim, v_dim, false) * sizeof(float));
+    out_launch->shmem = (uint32_t)(sdpa_lds_floats(gt, chunk, qk_dim, v_dim, fusion != nullptr) * sizeof(float));
     out_launch->set_args(a);
     return FK_OK;
 }

@@ -70,11 +70,20 @@ __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk,
 }
 
 // One (range, kv head, head tile) work item.  Uniform per block; `kv_len` already read.
-template <int GT, bool FUSED, typename ARGS, int KVQ = 0>
+// MODE 0: q is already rotated and the new K/V rows are in the cache.  MODE 1: a phase of the
+// whole-token kernel (kv_len known on entry, coherent stores); MODE 2: a kernel of its own.  In
+// modes 1 and 2 the block applies head norm + RoPE to its q heads itself, and the block whose
+// range holds the new position does the same for the new k row, uses it and v_new in place of
+// the cache row and appends both to the cache.
+// FASTHEAD (mode 2): heads rotated over their whole width of at most 128 dims with a rotary table;
+// the transforms' loads are issued ahead of the cache rows and used after them.
+template <int GT, int MODE, typename ARGS, int KVQ = 0, bool FASTHEAD = false>
 __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
                                            uint32_t gz, uint32_t gz_count, float* lds) {
+    constexpr bool FUSED = MODE == 1;   // inside the whole-token kernel
+    constexpr bool XFORM = MODE != 0;   // q / new-row transforms happen here
     constexpr int kSteps = FUSED ? kSdpaStepsFused : kSdpaSteps;
-    static_assert(!(FUSED && KVQ != 0), "the fused form reads a bf16 cache");
+    static_assert(!(XFORM && KVQ != 0), "the fused forms read a bf16 cache");
     const uint32_t span = a.chunk_len * a.chunks_per_block;  // cache positions per block
     const uint32_t blk0 = split * span;
     const uint32_t G = a.n_heads / a.n_kv;
@@ -103,17 +112,18 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     float* stat = red + (kSdpaBlock / a.lpv) * GT * a.v_dim;  // m[GT], l[GT], misc
     uint16_t* qn = reinterpret_cast<uint16_t*>(stat + kSdpaStatFloats);  // fused: [GT][qk_dim] + k row
     uint16_t* kn = qn + GT * a.qk_dim;
-    const uint32_t pos = FUSED ? kv_len - 1 : 0u;  // fused: position of the new token
-    const bool blk_owner = FUSED && pos >= blk0 && pos < blk0 + blk_keys;
+    const uint32_t pos = XFORM ? kv_len - 1 : 0u;  // fused: position of the new token
+    bool blk_owner = false;
 
-    if constexpr (FUSED) {
-        // head norm + RoPE of this block's q heads (one wave per head), and of the new
-        // k row in the block that owns its position; results in LDS as bf16.  Done
-        // before the K/V loads are issued: the trigonometry needs ~60 registers that
-        // the 64 registers of in-flight rows would otherwise have to share
-        for (uint32_t h = wave; h < gcount + (blk_owner ? 1u : 0u); h += kSdpaWaves) {
+    // Head norm + RoPE of this block's q heads (one wave per head), and of the new k row
+    // in the block that owns its position; results in LDS as bf16.  Then one block per kv
+    // head appends the new rows to the cache.
+    auto head_dst = [&](uint32_t h) { return h < gcount ? qn + h * a.qk_dim : kn; };
+    auto transform_heads = [&](uint32_t h_first) {
+        blk_owner = pos >= blk0 && pos < blk0 + blk_keys;
+        for (uint32_t h = h_first + wave; h < gcount + (blk_owner ? 1u : 0u); h += kSdpaWaves) {
             if (h < gcount) {
-                head_transform(a.q + (size_t)(h0 + h) * a.qk_dim, qn + h * a.qk_dim, a.q_norm, a.qk_dim, a.rope_dims,
+                head_transform(a.q + (size_t)(h0 + h) * a.qk_dim, head_dst(h), a.q_norm, a.qk_dim, a.rope_dims,
                                pos, a.base_log2, a.eps, true, lane, a.rope_tab);
             } else {
                 head_transform(a.k_new + (size_t)kvh * a.qk_dim, kn, a.k_norm, a.qk_dim, a.rope_dims, pos, a.base_log2,
@@ -121,13 +131,16 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
         }
         __syncthreads();
-        if (blk_owner && gz == 0) {  // one block per kv head appends the new rows to the cache
+        if (blk_owner && gz == 0) {
             const size_t row = (size_t)kvh * a.capacity + (pos % a.capacity);
             for (uint32_t d = tid; d < a.qk_dim; d += kSdpaBlock) a.cache_k_w[row * a.qk_dim + d] = kn[d];
             for (uint32_t d = tid; d < a.v_dim; d += kSdpaBlock)
                 a.cache_v_w[row * a.v_dim + d] = a.v_new[(size_t)kvh * a.v_dim + d];
         }
-    }
+    };
+    // Whole-token kernel: done before the K/V loads are issued: the trigonometry needs
+    // ~60 registers that the 64 registers of in-flight rows would otherwise have to share.
+    if constexpr (MODE == 1) transform_heads(0);
 
     const uint32_t lpk = a.lpk, cpk = a.qk_dim >> 3;
     const uint32_t lpv = a.lpv, cpv = a.v_dim >> 3;
@@ -153,16 +166,19 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     // This lane's 8 dims of each query head; fetched before the K/V rows so that the
     // scores can start as soon as the first keys arrive (loads return in order).
     uint4 qf[GT];
+    auto load_q = [&]() {
 #pragma unroll
-    for (int h = 0; h < GT; ++h) {
-        qf[h] = make_uint4(0, 0, 0, 0);
-        if (kcol_ok && (uint32_t)h < gcount) {
-            if constexpr (FUSED)
-                qf[h] = *reinterpret_cast<const uint4*>(qn + h * a.qk_dim + 8 * ck);
-            else
-                qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
+        for (int h = 0; h < GT; ++h) {
+            qf[h] = make_uint4(0, 0, 0, 0);
+            if (kcol_ok && (uint32_t)h < gcount) {
+                if constexpr (XFORM)
+                    qf[h] = *reinterpret_cast<const uint4*>(qn + h * a.qk_dim + 8 * ck);
+                else
+                    qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
+            }
         }
-    }
+    };
+    if constexpr (MODE != 2) load_q();
 
     float sq[GT];  // quantised K: sum of this lane's 8 query dims (the affine bias term b * sum q)
     if constexpr (KVQ != 0) {
@@ -217,7 +233,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
             return;
         }
-        if constexpr (!FUSED) {
+        if constexpr (MODE != 1) {
             // Straight-line, clamped (row to the last row of the allocation, a lane beyond
             // the head width to column 0): no branch separates the loads, so the compiler
             // can wait for exactly the rows it needs while later requests stay in flight.
@@ -257,16 +273,46 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
         }
     };
-    if constexpr (!FUSED) {
+    uint4 vnew = make_uint4(0, 0, 0, 0);  // mode 2: this lane's 8 dims of the new V row
+    if constexpr (MODE != 1) {
+        // Mode 2, fast heads: every wave requests the inputs of two heads (its own index and
+        // that plus the wave count; index gcount is the new k row) before the cache rows, so
+        // they arrive first and the transforms run while the rows are still in flight.
+        HeadPair ha, hb;
+        const uint32_t half = a.qk_dim >> 1, hi_a = wave, hi_b = wave + kSdpaWaves;
+        if constexpr (MODE == 2 && FASTHEAD) {
+            auto src = [&](uint32_t h) {
+                return h < gcount ? a.q + (size_t)(h0 + h) * a.qk_dim : a.k_new + (size_t)kvh * a.qk_dim;
+            };
+            ha = head_pair_fetch(src(hi_a), hi_a < gcount ? a.q_norm : a.k_norm, a.rope_tab, half, lane);
+            hb = head_pair_fetch(src(hi_b), hi_b < gcount ? a.q_norm : a.k_norm, a.rope_tab, half, lane);
+        }
         request_rows(kc, vc, blk0, 0, false, 0);
+        if constexpr (MODE == 2)
+            vnew = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_dim + (vcol_ok ? 8 * cv : 0u));
         settle();
         if (split >= n_active) return;  // uniform: whole block leaves before any barrier
+        if constexpr (MODE == 2) {
+            if constexpr (FASTHEAD) {
+                const bool own = pos >= blk0 && pos < blk0 + blk_keys;
+                head_pair_apply(ha, head_dst(hi_a), a.q_norm != nullptr, half, a.eps, lane,
+                                hi_a < gcount || (hi_a == gcount && own));
+                head_pair_apply(hb, head_dst(hi_b), a.q_norm != nullptr, half, a.eps, lane,
+                                hi_b < gcount || (hi_b == gcount && own));
+                transform_heads(2 * kSdpaWaves);  // a ninth head (tile of 8 plus the k row), barrier, cache append
+            } else {
+                // the transforms' own loads queue behind the cache rows requested above; q comes
+                // back from LDS rotated
+                transform_heads(0);
+            }
+            load_q();
+        }
     }
 
     for (uint32_t c = 0; c < n_chunks; ++c) {
     const uint32_t key0 = blk0 + c * a.chunk_len;
     const uint32_t nkeys = (kv_len - key0) < a.chunk_len ? (kv_len - key0) : a.chunk_len;
-    const bool owner = FUSED && pos >= key0 && pos < key0 + nkeys;
+    const bool owner = XFORM && pos >= key0 && pos < key0 + nkeys;
     const uint32_t jpos = pos - key0;
     if constexpr (FUSED) {
         request_rows(kc, vc, key0, nkeys, owner, jpos);
@@ -277,7 +323,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     FK_SDPA_STAMP(1);
     // ---------------- phase A: scores ----------------
     {
-        if constexpr (FUSED) {
+        if constexpr (XFORM) {
             if (owner && kcol_ok) {
 #pragma unroll
                 for (int u = 0; u < kSteps; ++u)
@@ -385,7 +431,10 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             }
         } else {
         // rows past kv_len were requested speculatively: their bits may be anything
-        const uint4 vv = (FUSED || (j < nkeys && vcol_ok)) ? vc[u] : make_uint4(0, 0, 0, 0);
+        uint4 vv = (FUSED || (j < nkeys && vcol_ok)) ? vc[u] : make_uint4(0, 0, 0, 0);
+        if constexpr (MODE == 2) {
+            if (owner && j == jpos && vcol_ok) vv = vnew;  // the new row, not yet cached
+        }
         const float f[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
                             bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
 #pragma unroll
@@ -398,7 +447,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }
     if (c + 1 < n_chunks) {
         __syncthreads();  // the scores are overwritten by the next range
-        if constexpr (!FUSED) {
+        if constexpr (MODE != 1) {
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
                 kc[u] = kn_[u];
@@ -543,6 +592,22 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     r.partials = a.partials + (size_t)tr * a.n_heads * a.n_splits * (a.v_dim + 2);
     r.counters = a.counters + (size_t)tr * a.n_kv * gz_count;
     sdpa_block<GT, false, SdpaArgs, KVQ>(r, kv_len0 + tr, blockIdx.x, blockIdx.y, gz, gz_count, lds);
+}
+
+// RoPE (+ head norm) of q and of the new k row, the cache append and the attention in one
+// launch: a.q / a.k_new / a.v_new are the raw projection outputs of the token at position
+// kv_len - 1, a.k / a.v the cache it is appended to.
+template <int GT, bool FASTHEAD>
+__global__ __launch_bounds__(kSdpaBlock) void sdpa_rope_store_kernel(const SdpaArgs a) {
+    extern __shared__ __align__(16) float lds[];
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t* imm = (const uint32_t*)((const char*)__builtin_amdgcn_kernarg_segment_ptr() +
+                                            offsetof(SdpaArgs, kv_len_imm));
+#else
+    const uint32_t* imm = &a.kv_len_imm;
+#endif
+    const uint32_t kv_len0 = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
+    sdpa_block<GT, 2, SdpaArgs, 0, FASTHEAD>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
 }
 
 }  // namespace fk

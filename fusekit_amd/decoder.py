@@ -41,6 +41,7 @@ class DecoderConfig:
     swiglu_variant: int = 0
     capacity: int = 1024     # KV-cache rows per layer
     fuse_rope_store: bool = True   # one launch for rope_q + rope_kv_store (False: the reference's two)
+    fuse_attention: bool = True    # graph mode, bf16 cache: rope/store + attention of a layer in one launch
     kv_bits: int = 0         # 0: bf16 KV cache; 4 / 8: quantised cache (mlx-lm QuantizedKVCache layout)
     kv_group: int = 64
 
@@ -187,8 +188,12 @@ class DecoderRuntime:
         self.sdpa_partials, self.sdpa_counters = DeviceBuffer(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
-        self.tasks = self.build_tasks()
         self.persistent = persistent
+        # one launch per layer for rope/store + attention: the task graph only (the whole-token kernel
+        # fuses them itself and is built from the plain task list)
+        self.fused_attention = bool(cfg.fuse_attention and not persistent and not cfg.kv_bits)
+        self.rope_tab = DeviceBuffer(cfg.head_dim * 4) if self.fused_attention else None
+        self.tasks = self.build_tasks()
         # persistent: the same task list, run by one whole-token kernel per replay
         self.graph = (self.d.build_decode_graph(self.tasks, True, spin_limit) if persistent
                       else self.d.build_graph(self.tasks))
@@ -207,7 +212,11 @@ class DecoderRuntime:
             fid[0] += 1
             return f"fusekit_{kind}_f{fid[0]}"
 
-        t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
+        if self.fused_attention:   # step_init also fills this token's (cos, sin) table, shared by all layers
+            t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len),
+                                                    arg(self.rope_tab)], dict(rope_dims=c.head_dim, theta=c.theta)))
+        else:
+            t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
         emb = w.mats["embed_tokens"]       # dense bf16 or MLX-affine (4-bit checkpoints quantise it too)
         head = w.mats.get("lm_head", emb)  # untied output projection when the checkpoint has one
         t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token)] + self._wargs(emb) + [arg(self.x[0])],
@@ -226,7 +235,15 @@ class DecoderRuntime:
                                    has_bias=int(c.qkv_bias))))
             rope = dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, rope_dims=c.head_dim, theta=c.theta,
                         capacity=c.capacity, eps=c.eps)
-            if c.kv_bits:
+            if self.fused_attention:
+                a = [arg(self.q), arg(self.k), arg(self.v)]
+                if c.qk_norm:
+                    a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
+                a += [arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len), arg(self.att),
+                      arg(self.sdpa_partials), arg(self.sdpa_counters), arg(self.rope_tab)]
+                t.append(Dispatch(name("rope_store_sdpa_decode"), a,
+                                  dict(rope, has_norm=int(c.qk_norm), has_table=1, max_len=c.capacity)))
+            elif c.kv_bits:
                 # quantised cache: rotate q in place, then quantise the rotated K row and the V row
                 qa = [arg(self.q)] + ([arg(w.vecs[p + "self_attn.q_norm"])] if c.qk_norm else []) + [arg(self.offset)]
                 t.append(Dispatch(name("rmsnorm_rope_q_decode" if c.qk_norm else "rope_q_decode"), qa, rope))
@@ -254,7 +271,9 @@ class DecoderRuntime:
                 t.append(Dispatch(name("rope_kv_cache_store_decode"),
                                   [arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]),
                                    arg(self.offset), arg(self.offset)], rope))
-            if c.kv_bits:
+            if self.fused_attention:
+                pass
+            elif c.kv_bits:
                 K, V = self.cache_k[l], self.cache_v[l]
                 t.append(Dispatch(name(f"sdpa_decode_q{c.kv_bits}"),
                                   [arg(self.q)] + [arg(b) for b in (K.packed, K.scales, K.biases, V.packed, V.scales, V.biases)]

@@ -353,6 +353,20 @@ def step_init(step_counter, offset, kv_len, stream=None):
     check(lib.fk_step_init(_ptr(step_counter), _ptr(offset), _ptr(kv_len), _ptr(stream)))
 
 
+def step_init_rope(step_counter, offset, kv_len, rope_tab, rope_dims, theta, stream=None):
+    check(lib.fk_step_init_rope(_ptr(step_counter), _ptr(offset), _ptr(kv_len), _ptr(rope_tab), C.c_uint32(rope_dims),
+                                C.c_float(theta), _ptr(stream)))
+
+
+def rope_store_sdpa_decode(q, k, v, q_norm, k_norm, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_kv,
+                           head_dim, rope_dims, theta, eps, capacity, scale, rope_tab, partials, counters, stream=None):
+    check(lib.fk_rope_store_sdpa_decode(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(cache_k), _ptr(cache_v), _ptr(out), _ptr(d_kv_len),
+        C.c_uint32(kv_len), C.c_uint32(max_len), C.c_uint32(n_heads), C.c_uint32(n_kv), C.c_uint32(head_dim),
+        C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), C.c_uint32(capacity), C.c_float(scale), _ptr(rope_tab),
+        _ptr(partials), _ptr(counters), _ptr(stream)))
+
+
 def copy(dst, src, nbytes, stream=None):
     check(lib.fk_copy(_ptr(dst), _ptr(src), C.c_size_t(nbytes), _ptr(stream)))
 

@@ -321,6 +321,24 @@ fk_status fk_argmax_logits_decode(const uint16_t *logits, uint32_t n, uint32_t *
 /* U   offset = step_counter++ ; kv_len = offset + 1.  Replaces fusekit_step_init
  *     (src/codegen/kernels/mod.rs:542-563). */
 fk_status fk_step_init(uint32_t *step_counter, uint32_t *offset, uint32_t *kv_len, fk_stream s);
+/*     The same, and fills `rope_tab` (2 * (rope_dims / 2) floats: cos, sin of every rotary pair at
+ *     position `offset`, the values rope_q_decode.rs:93-114 computes per head) once for all layers of
+ *     the token; fk_rope_store_sdpa_decode reads it. */
+fk_status fk_step_init_rope(uint32_t *step_counter, uint32_t *offset, uint32_t *kv_len, float *rope_tab,
+                            uint32_t rope_dims, float theta, fk_stream s);
+
+/* R+H+A in one launch: head norm + RoPE of q and of the new k row, the append of the new k / v rows
+ *     to the cache at row kv_len - 1, and the attention of fk_sdpa_decode over kv_len rows.  Same
+ *     arithmetic and rounding points as fk_qkv_rope_store_decode followed by fk_sdpa_decode (the
+ *     rotated q is used from on-chip memory and not written back); replaces the dispatch pair
+ *     rope_q_decode.rs / rope_kv_cache_store_decode.rs + sdpa_decode.rs of one layer.  q_norm and
+ *     k_norm come together or not at all; rope_tab from fk_step_init_rope or NULL (computed in place). */
+fk_status fk_rope_store_sdpa_decode(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *q_norm,
+                                    const uint16_t *k_norm, uint16_t *cache_k, uint16_t *cache_v, uint16_t *out,
+                                    const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
+                                    uint32_t n_kv, uint32_t head_dim, uint32_t rope_dims, float theta, float eps,
+                                    uint32_t capacity, float scale, const float *rope_tab, float *partials,
+                                    uint32_t *counters, fk_stream s);
 
 /* ---- dispatcher: replaces `_fusekit_runtime_native` ------------------------
  *

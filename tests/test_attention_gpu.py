@@ -184,3 +184,66 @@ def test_step_init(fk):
         fk.step_init(sc, off, kvl)
     assert int(sc.to_numpy(np.uint32)[0]) == 44
     assert int(off.to_numpy(np.uint32)[0]) == 43 and int(kvl.to_numpy(np.uint32)[0]) == 44
+
+
+@pytest.mark.parametrize("norm,table", [(False, False), (True, True), (True, False)])
+@pytest.mark.parametrize("n_heads,n_kv,dim,rope_dims,cap,kv_len", [
+    (32, 8, 128, 128, 1024, 1),       # first token: the only row is the new one
+    (32, 8, 128, 128, 1024, 100),     # one range
+    (32, 8, 128, 128, 1024, 577),     # several ranges, the new row in the last one
+    (14, 2, 64, 64, 4096, 2049),      # group of 7 heads (tile of 8), the new row opens a range
+    (16, 16, 192, 64, 256, 256),      # partial rotation, cache exactly full
+    (4, 1, 128, 128, 16384, 9000),    # blocks that walk several ranges
+])
+def test_rope_store_sdpa_in_one_launch(fk, norm, table, n_heads, n_kv, dim, rope_dims, cap, kv_len):
+    """fk_rope_store_sdpa_decode against the launch pair it replaces (fk_qkv_rope_store_decode, then
+    fk_sdpa_decode): the same arithmetic in the same order, so the attention output and both caches
+    are identical bit for bit; and the attention output against the oracle."""
+    theta, eps, scale, pos = 1e6, 1e-6, dim ** -0.5, kv_len - 1
+    q, k, v = normal_bf16(1, n_heads * dim), normal_bf16(2, n_kv * dim), normal_bf16(3, n_kv * dim)
+    qw, kw = (normal_bf16(4, dim, 0.1, 1.0), normal_bf16(5, dim, 0.1, 1.0)) if norm else (None, None)
+    ck, cv = normal_bf16(6, n_kv * cap * dim), normal_bf16(7, n_kv * cap * dim)
+    dev = lambda a: None if a is None else fk.DeviceBuffer.from_numpy(a)
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, dim, dim, cap)
+    part, cnt = fk.DeviceBuffer(max(pb, 16)), fk.zeros(max(cb, 16))
+    # the pair
+    dq, ck1, cv1, out1 = dev(q), dev(ck), dev(cv), fk.DeviceBuffer(n_heads * dim * 2)
+    fk.qkv_rope_store_decode(dq, dev(k), dev(v), dev(qw), dev(kw), n_heads, n_kv, dim, rope_dims, theta, eps,
+                             _u32(fk, pos), 0, cap, ck1, cv1)
+    fk.sdpa_decode(dq, ck1, cv1, out1, _u32(fk, kv_len), 0, cap, n_heads, n_kv, dim, dim, cap, scale, part, cnt)
+    # one launch
+    ck2, cv2, out2 = dev(ck), dev(cv), fk.DeviceBuffer(n_heads * dim * 2)
+    tab = None
+    if table:
+        tab = fk.DeviceBuffer(rope_dims * 4)
+        ctr, off, kvl = _u32(fk, pos), fk.zeros(4), fk.zeros(4)
+        fk.step_init_rope(ctr, off, kvl, tab, rope_dims, theta)
+        assert (ctr.to_numpy(np.uint32)[0], off.to_numpy(np.uint32)[0], kvl.to_numpy(np.uint32)[0]) == (pos + 1, pos, pos + 1)
+    fk.rope_store_sdpa_decode(dev(q), dev(k), dev(v), dev(qw), dev(kw), ck2, cv2, out2, _u32(fk, kv_len), 0, cap, n_heads,
+                              n_kv, dim, rope_dims, theta, eps, cap, scale, tab, part, cnt)
+    assert np.array_equal(ck2.to_numpy(np.uint16), ck1.to_numpy(np.uint16))
+    assert np.array_equal(cv2.to_numpy(np.uint16), cv1.to_numpy(np.uint16))
+    assert np.array_equal(out2.to_numpy(np.uint16), out1.to_numpy(np.uint16))
+    assert not np.array_equal(ck2.to_numpy(np.uint16), ck)          # the row was appended
+    ref = oracle.sdpa_decode(dq.to_numpy(np.uint16), ck1.to_numpy(np.uint16), cv1.to_numpy(np.uint16), n_heads, n_kv,
+                             dim, dim, kv_len, cap, scale)
+    assert rel_l2(out2.to_numpy(np.uint16), oracle.bf16_to_f32(ref)) <= REL_L2_BAR
+    # immediate kv_len gives the same result
+    ck3, cv3, out3 = dev(ck), dev(cv), fk.DeviceBuffer(n_heads * dim * 2)
+    fk.rope_store_sdpa_decode(dev(q), dev(k), dev(v), dev(qw), dev(kw), ck3, cv3, out3, None, kv_len, cap, n_heads,
+                              n_kv, dim, rope_dims, theta, eps, cap, scale, tab, part, cnt)
+    assert np.array_equal(out3.to_numpy(np.uint16), out1.to_numpy(np.uint16))
+    assert np.array_equal(ck3.to_numpy(np.uint16), ck1.to_numpy(np.uint16))
+
+
+def test_rope_store_sdpa_rejects_bad_arguments(fk):
+    b = fk.DeviceBuffer(1 << 16)
+    args = dict(n_heads=8, n_kv=2, dim=64)
+    with pytest.raises(fk.FusekitError):      # q norm without k norm
+        fk.rope_store_sdpa_decode(b, b, b, b, None, b, b, b, None, 4, 16, 8, 2, 64, 64, 1e4, 1e-6, 16, 0.1, None, b, b)
+    with pytest.raises(fk.FusekitError):      # odd rope_dims
+        fk.rope_store_sdpa_decode(b, b, b, None, None, b, b, b, None, 4, 16, 8, 2, 64, 33, 1e4, 1e-6, 16, 0.1, None, b, b)
+    with pytest.raises(fk.FusekitError):      # kv_len beyond max_len
+        fk.rope_store_sdpa_decode(b, b, b, None, None, b, b, b, None, 17, 16, 8, 2, 64, 64, 1e4, 1e-6, 16, 0.1, None, b, b)
+    with pytest.raises(fk.FusekitError):      # table requested with rope_dims 0
+        fk.step_init_rope(b, b, b, b, 0, 1e4)

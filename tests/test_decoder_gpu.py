@@ -29,9 +29,13 @@ def _run_pair(fk, cfg, seed, n_prompt=8, n_decode=24, persistent=False):
 
 @pytest.mark.parametrize("bits", [4, 8, 16])
 @pytest.mark.parametrize("qk_norm,bias,fuse", [(False, True, True), (True, False, True), (True, False, False),
-                                                 (False, True, False)])
+                                                 (False, True, False), (True, False, "attention"),
+                                                 (False, True, "attention")])
 def test_greedy_tokens_match_oracle(fk, bits, qk_norm, bias, fuse):
-    cfg = _small_cfg(bits=bits, qk_norm=qk_norm, qkv_bias=bias, fuse_rope_store=fuse)
+    """fuse: "attention" = rope/store + attention in one launch per layer (the default task list);
+    True = one rope/store launch, then attention; False = the reference's rope_q, rope_kv_store, sdpa."""
+    cfg = _small_cfg(bits=bits, qk_norm=qk_norm, qkv_bias=bias, fuse_rope_store=fuse is True,
+                     fuse_attention=fuse == "attention")
     got, ref, margins, _ = _run_pair(fk, cfg, seed=3)
     print("margins:", ["%.3g" % m for m in margins])
     for i, (g, r) in enumerate(zip(got, ref)):
@@ -106,7 +110,7 @@ def test_graph_edges_follow_hazards(fk):
     """RAW/WAW/WAR edges only: rope_q and rope_kv_store are siblings (no edge between them),
     both depend on the QKV projection, SDPA depends on both."""
     from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
-    cfg = _small_cfg(bits=4, n_layers=1, fuse_rope_store=False)
+    cfg = _small_cfg(bits=4, n_layers=1, fuse_rope_store=False, fuse_attention=False)
     rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=1))
     names = [t.kernel for t in rt.tasks]
     idx = {n.rsplit("_f", 1)[0]: i for i, n in enumerate(names)}
@@ -149,10 +153,11 @@ def test_dispatcher_error_paths(fk, tmp_path):
     assert Dispatcher(None, str(bad)).kernel_names() == ["fusekit_sdpa_decode_f40"]
 
 
-def test_update_graph_bindings_repoints_kv_cache(fk):
+@pytest.mark.parametrize("fuse_attention", [True, False])
+def test_update_graph_bindings_repoints_kv_cache(fk, fuse_attention):
     """Growing the KV cache re-patches bindings without a rebuild (update_icb_bindings)."""
     from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
-    cfg = _small_cfg(bits=4, n_layers=1)
+    cfg = _small_cfg(bits=4, n_layers=1, fuse_attention=fuse_attention)
     W = DecoderWeights.random_init(cfg, seed=2)
     rt = DecoderRuntime(cfg, W)
     prompt = [1, 2, 3, 4, 5]
@@ -166,7 +171,7 @@ def test_update_graph_bindings_repoints_kv_cache(fk):
                 ups.append((i, s, new_k.ptr, n))
             if p == rt.cache_v[0].ptr:
                 ups.append((i, s, new_v.ptr, n))
-    assert len(ups) == 4
+    assert len(ups) == (2 if fuse_attention else 4)   # one task binds both caches, or the store and the attention
     rt.d.update_graph_bindings(rt.graph, ups)
     old_k = rt.cache_k[0].to_numpy(np.uint16).copy()
     got, _, _ = rt.generate(prompt, 12)
@@ -219,7 +224,7 @@ def test_persistent_kernel_matches_task_graph_state(fk):
 
 def test_persistent_kernel_rejects_other_task_lists(fk):
     from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
-    cfg = _small_cfg(bits=4, n_layers=1)
+    cfg = _small_cfg(bits=4, n_layers=1, fuse_attention=False)
     rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=1))
     with pytest.raises(fk.FusekitError):
         rt.d.build_decode_graph(rt.tasks[:-1], True)          # no argmax
