@@ -116,15 +116,35 @@ __device__ __forceinline__ float group_sum(float v, int width) {
     if (width >= 4) v = dpp_add<0x4E>(v);
     if (width >= 8) v = dpp_add<0x141>(v);
     if (width >= 16) v = dpp_add<0x140>(v);
-    if (width >= 32) v += __shfl_xor(v, 16, kWave);
-    if (width >= 64) v += __shfl_xor(v, 32, kWave);
+    if (width == 32) v += __shfl_xor(v, 16, kWave);
+    if (width >= 64) {
+        // every lane of row i holds that row's total: (r0 + r1) + (r2 + r3) through scalar
+        // registers, the value the two butterfly steps over 16 and 32 lanes give
+        const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+        const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+        const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+        const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+        v = (r0 + r1) + (r2 + r3);
+    }
     return v;
 }
+// All 64 lanes must be active (the cross-row step reads lanes 0, 16, 32, 48 directly).
 __device__ __forceinline__ float wave_sum(float v) { return group_sum(v, 64); }
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false);
+    return fmaxf(v, __int_as_float(moved));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-    return v;
+    v = dpp_max<0xB1>(v);
+    v = dpp_max<0x4E>(v);
+    v = dpp_max<0x141>(v);
+    v = dpp_max<0x140>(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
 // Block-wide sum; every thread returns the same value.  `scratch` holds one
@@ -136,16 +156,12 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     v = wave_sum(v);
     if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float t = 0.f;
+    // every thread adds the wave totals itself (LDS broadcast reads): one barrier.  The
+    // caller must not rewrite `scratch` before its next barrier.
+    float t = 0.f;
 #pragma unroll
-        for (int i = 0; i < NW; ++i) t += scratch[i];
-        scratch[NW] = t;
-    }
-    __syncthreads();
-    float r = scratch[NW];
-    __syncthreads();
-    return r;
+    for (int i = 0; i < NW; ++i) t += scratch[i];
+    return t;
 }
 
 template <int BLOCK>

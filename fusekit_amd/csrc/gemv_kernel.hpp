@@ -191,24 +191,28 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
         for (int i = 0; i < kStageRegs; ++i)
             if (threadIdx.x + i * kGemvBlock < n8) add_sq(xr[i]);
         for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8; t += kGemvBlock) add_sq(x8[t]);
+        FK_GEMV_STAMP(5);
         ss = block_sum<kGemvBlock>(ss, scratch);
         r = 1.0f / sqrtf(ss / (float)K + a.eps);
+        FK_GEMV_STAMP(6);
     }
     auto emit = [&](uint32_t t, uint4 v, uint4 wv) {
-        const uint32_t p[4] = {v.x, v.y, v.z, v.w};
-        float f[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            f[2 * i] = bf16_lo(p[i]);
-            f[2 * i + 1] = bf16_hi(p[i]);
-        }
+        // nb: the staged values as bf16 pairs in element order (0,1) (2,3) (4,5) (6,7).  With the
+        // norm each pair takes two packed conversions: T(x * r), then T(w * that).
+        uint32_t nb[4] = {v.x, v.y, v.z, v.w};
         if (NORM) {
             const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                f[2 * i] = round_bf16(bf16_lo(q[i]) * round_bf16(f[2 * i] * r));
-                f[2 * i + 1] = round_bf16(bf16_hi(q[i]) * round_bf16(f[2 * i + 1] * r));
+                const uint32_t xr_ = pack_bf16(bf16_lo(nb[i]) * r, bf16_hi(nb[i]) * r);
+                nb[i] = pack_bf16(bf16_lo(q[i]) * bf16_lo(xr_), bf16_hi(q[i]) * bf16_hi(xr_));
             }
+        }
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = bf16_lo(nb[i]);
+            f[2 * i + 1] = bf16_hi(nb[i]);
         }
         float s8 = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
         const bool live = t < n8;
@@ -216,10 +220,11 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
             // word j of chunk c; activation pairs (0,2) (4,6) (1,3) (5,7) as q4_word_dot wants
             const uint32_t c = t >> 2, j = t & 3u;
             if (live)
-                xs[j * cpr + c] = make_uint4(pack_bf16(f[0], f[2]), pack_bf16(f[4], f[6]), pack_bf16(f[1], f[3]),
-                                             pack_bf16(f[5], f[7]));
-            s8 += __shfl_xor(s8, 1, kWave);
-            s8 += __shfl_xor(s8, 2, kWave);
+                xs[j * cpr + c] = make_uint4(__builtin_amdgcn_perm(nb[1], nb[0], 0x05040100u),
+                                             __builtin_amdgcn_perm(nb[3], nb[2], 0x05040100u),
+                                             __builtin_amdgcn_perm(nb[1], nb[0], 0x07060302u),
+                                             __builtin_amdgcn_perm(nb[3], nb[2], 0x07060302u));
+            s8 = group_sum(s8, 4);  // the four lanes that hold the words of one chunk
             if (live && j == 0) sx[c] = s8;
         } else if constexpr (KIND == W_Q8) {
             const uint32_t c = t >> 1, j = (t & 1u) * 2u;
@@ -229,12 +234,10 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
                 xs[(j + 1) * cpr + c] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]),
                                                    __float_as_uint(f[6]), __float_as_uint(f[7]));
             }
-            s8 += __shfl_xor(s8, 1, kWave);
+            s8 = group_sum(s8, 2);
             if (live && j == 0) sx[c] = s8;
         } else {
-            if (live)
-                xs[t] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]),
-                                   pack_bf16(f[6], f[7]));
+            if (live) xs[t] = make_uint4(nb[0], nb[1], nb[2], nb[3]);
         }
     };
     // whole waves past the end skip the step (the chunk-sum butterflies need whole waves)
@@ -252,6 +255,7 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
         }
         emit(t, v, wv);
     }
+    FK_GEMV_STAMP(7);
     __syncthreads();
 }
 
