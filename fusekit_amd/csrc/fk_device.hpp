@@ -66,6 +66,16 @@ __device__ __forceinline__ float ld_f32(const float* p) {
     if constexpr (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return *p;
 }
+// Two adjacent floats (8-byte aligned) in one load.
+template <bool COH>
+__device__ __forceinline__ float2 ld_f32x2(const float* p) {
+    if constexpr (COH) {
+        const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+        return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
+    }
+    return *reinterpret_cast<const float2*>(p);
+}
 template <bool COH>
 __device__ __forceinline__ void st_f32(float* p, float v) {
     if constexpr (COH)

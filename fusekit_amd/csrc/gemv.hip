@@ -143,7 +143,7 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
         // fewer than two blocks (eight waves) on a CU cannot hide the load latency:
         // such a choice is priced as if it ran two
         uint64_t per_cu = (blocks + dev->cus - 1) / dev->cus;
-        if (per_cu < 2) per_cu = 2;
+        if (per_cu < 512 / kGemvBlock) per_cu = 512 / kGemvBlock;
         const uint64_t cost = per_cu * per_block * batches;
         const uint64_t waste = tiles * batches + blocks;
         if (cost < best_cost || (cost == best_cost && waste < best_waste)) {

@@ -515,10 +515,12 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     if (tid == 0)  // ready for the next launch (or the next layer of this one)
         __hip_atomic_store(&a.counters[kvh * gz_count + gz], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-    // One wave per head, no block barriers.  The ranges are taken 16 at a time: (m, l) of
-    // each and this lane's two output dims of each are requested together (one memory
-    // round trip per 16 ranges) and folded into a running (M, L, o) with the usual
-    // rescaling, in range order, so the result does not depend on arrival order.
+    // One wave per head, no block barriers.  The ranges are taken 16 at a time and folded
+    // into a running (M, L, o) with the usual rescaling, in range order, so the result does
+    // not depend on arrival order.  Per batch a lane issues 17 eight-byte loads: (m, l) of
+    // range base + (lane % 16), handed to the other lanes through scalar registers, and its
+    // own two output dims of each of the 16 ranges; the next batch's loads are in flight
+    // while the current one is folded in.
     constexpr uint32_t kBatch = 16;
     const uint32_t row = a.v_dim + 2;
     for (uint32_t h = wave; h < gcount; h += kSdpaWaves) {
@@ -527,15 +529,19 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             const bool live = d2 < (a.v_dim >> 1);
             const float* pd = ph + 2 + 2 * (live ? d2 : 0u);
             float M = -INFINITY, L = 0.f, o0 = 0.f, o1 = 0.f;
-            for (uint32_t base = 0; base < n_active; base += kBatch) {
-                float pm[kBatch], pl[kBatch], p0[kBatch], p1[kBatch];
+            auto fetch = [&](uint32_t base, float2& ml, float2(&po)[kBatch]) {
+                const uint32_t mine = base + (lane & (kBatch - 1));
+                ml = ld_f32x2<true>(ph + (size_t)(mine < n_active ? mine : base) * row);
+#pragma unroll
+                for (uint32_t i = 0; i < kBatch; ++i)
+                    po[i] = ld_f32x2<true>(pd + (size_t)(base + i < n_active ? base + i : base) * row);
+            };
+            auto fold = [&](uint32_t base, const float2& ml, const float2(&po)[kBatch]) {
+                float pm[kBatch], pl[kBatch];
 #pragma unroll
                 for (uint32_t i = 0; i < kBatch; ++i) {
-                    const size_t o = (size_t)(base + i < n_active ? base + i : base) * row;
-                    pm[i] = ld_f32<true>(ph + o);
-                    pl[i] = ld_f32<true>(ph + o + 1);
-                    p0[i] = ld_f32<true>(pd + o);
-                    p1[i] = ld_f32<true>(pd + o + 1);
+                    pm[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ml.x), i));
+                    pl[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ml.y), i));
                 }
                 float mn = fmaxf(M, pm[0]);
 #pragma unroll
@@ -548,11 +554,23 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
                 for (uint32_t i = 0; i < kBatch; ++i) {
                     const float w = base + i < n_active ? expf(pm[i] - mn) : 0.f;
                     L = fmaf(pl[i], w, L);
-                    o0 = fmaf(p0[i], w, o0);
-                    o1 = fmaf(p1[i], w, o1);
+                    o0 = fmaf(po[i].x, w, o0);
+                    o1 = fmaf(po[i].y, w, o1);
                 }
                 M = mn;
+            };
+            float2 ml_a, ml_b, po_a[kBatch], po_b[kBatch];
+            uint32_t base = 0;
+            fetch(0, ml_a, po_a);
+            while (base + kBatch < n_active) {  // straight-line body: request the next batch, fold this one
+                fetch(base + kBatch, ml_b, po_b);
+                fold(base, ml_a, po_a);
+                ml_a = ml_b;
+#pragma unroll
+                for (uint32_t i = 0; i < kBatch; ++i) po_a[i] = po_b[i];
+                base += kBatch;
             }
+            fold(base, ml_a, po_a);
             const float inv_l = 1.0f / L;
             if (live) {
                 uint16_t* dst = a.out + (size_t)(h0 + h) * a.v_dim + 2 * d2;
