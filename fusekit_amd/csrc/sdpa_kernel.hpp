@@ -287,6 +287,14 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             ha = head_pair_fetch(src(hi_a), hi_a < gcount ? a.q_norm : a.k_norm, a.rope_tab, half, lane);
             hb = head_pair_fetch(src(hi_b), hi_b < gcount ? a.q_norm : a.k_norm, a.rope_tab, half, lane);
         }
+        // The first range always exists and is requested before kv_len has arrived.  Later
+        // ranges wait for it (it was the kernel's first request and is long back by now):
+        // a fixed grid sized for the whole cache would otherwise read every range's rows
+        // each launch, megabytes of traffic for a context of a few hundred tokens.
+        if (split != 0) {
+            settle();
+            if (split >= n_active) return;
+        }
         request_rows(kc, vc, blk0, 0, false, 0);
         if constexpr (MODE == 2)
             vnew = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_dim + (vcol_ok ? 8 * cv : 0u));
