@@ -3,8 +3,8 @@
 4-bit g64 MLX-affine weights, 512 generated tokens, on one MI355X.
 
 One "step" = one decoded token = one replay of the captured decode graph (step_init, embed,
-36 x [rmsnorm_qkv, rope+kv-store, sdpa, o_proj+residual, rmsnorm_gateup_swiglu,
-down_proj+residual], final norm + LM head, argmax).  Weights are random-init (seeded, generated
+36 x [rmsnorm_qkv, rope + kv-store + sdpa (one launch), o_proj+residual,
+rmsnorm_gateup_swiglu, down_proj+residual], final norm + LM head, argmax).  Weights are random-init (seeded, generated
 and quantised in HBM); inputs are resident before the timed region.
 
 Prints ONE JSON line: value = generated tokens/s (wall clock around the K timed steps), plus
@@ -26,8 +26,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E published peak
 # HBM bytes per launch of the int4 gate/up kernel of the 4B-class model, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE (two counter runs of this script, each scaled by what the same counter reads for the plain
-# 256 MiB copies of --calibrate-copy: 1.99981 and 1.0).  Counters cannot be read from inside this process.
-GATEUP_Q4_4B_TRAFFIC_BYTES = 29013600
+# 256 MiB copies of --calibrate-copy: 1.99987 and 1.0).  Counters cannot be read from inside this process.
+GATEUP_Q4_4B_TRAFFIC_BYTES = 28563359
 
 
 def main() -> int:
