@@ -32,6 +32,11 @@
  *                                 reference's multi-row path rounds every dequantised
  *                                 weight to bf16 first (MLX QuantizedBlockLoader, not
  *                                 vendored): that rounding is parity unpinned
+ *   quantised KV store / attention pinned (V rows and unrotated K rows = the pinned quantiser
+ *                                 bit for bit; rotated K rows dequantise to within the
+ *                                 quantiser's step of the pinned bf16 RoPE; only the
+ *                                 addressed row written; attention = float64 softmax
+ *                                 attention over the dequantised cache)
  *   hand-derived known answers .. tests/golden/known_answers.json
  *   MLX-internal accumulation order, Metal fast::cos/sin/exp bit patterns:
  *                                 parity unpinned (cannot be observed here;
