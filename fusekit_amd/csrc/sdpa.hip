@@ -86,7 +86,10 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     const uint32_t chunk = sdpa_chunk_len(qk_dim, v_dim, false);
     const uint32_t n_chunks = (max_len + chunk - 1) / chunk;
     const uint32_t G = n_heads / n_kv;
-    const int gt = G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1));
+    // Tiles of 1, 2 or 4 heads run the wave-local form, which needs a key row and its value row on
+    // the same lanes (equal lanes per row); other shapes take the tile of 8, which goes through LDS.
+    const bool same_lanes = pow2_ceil(qk_dim / 8) == pow2_ceil(v_dim / 8);
+    const int gt = !same_lanes ? 8 : (G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1)));
     // Long contexts: a block walks several consecutive ranges (online softmax, the next
     // range's rows in flight), so that the grid stays near one to two blocks per CU and
     // the final merge, which costs one memory round trip per 16 partials, stays short.

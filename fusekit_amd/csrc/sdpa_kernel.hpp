@@ -3,6 +3,8 @@
 #pragma once
 #include <stddef.h>
 
+#include <type_traits>
+
 #include "fk_device.hpp"
 #include "rope_device.hpp"
 
@@ -57,8 +59,9 @@ struct SdpaArgs {
     const float* rope_tab;  // (cos, sin) per pair at this token's position, or null
 };
 
-// m[GT] at 0, l[GT] at 8 (GT <= 8), the last-block flag at 16, the per-range rescale factors at 24.
-constexpr uint32_t kSdpaStatFloats = 32;
+// m[GT] at 0, l[GT] at 8 (GT <= 8), the last-block flag at 16, the per-range rescale factors at 24;
+// wave-local form: per-wave maxima [wave][8] at 32 and per-wave sums [wave][8] at 64.
+constexpr uint32_t kSdpaStatFloats = 96;
 
 // LDS floats one block needs.
 __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk, uint32_t qk_dim, uint32_t v_dim,
@@ -82,6 +85,11 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
                                            uint32_t gz, uint32_t gz_count, float* lds) {
     constexpr bool FUSED = MODE == 1;   // inside the whole-token kernel
     constexpr bool XFORM = MODE != 0;   // q / new-row transforms happen here
+    // Tiles of up to 4 heads outside the whole-token kernel: every wave runs the online softmax
+    // over its own 16 keys of a range in registers (scores never leave the lanes that computed
+    // them, a key row and its value row share their lanes: the planner guarantees lpk == lpv), so
+    // the ranges of a block need no barrier; the waves meet once, after the last range.
+    constexpr bool WAVES = MODE != 1 && GT <= 4;
     constexpr int kSteps = FUSED ? kSdpaStepsFused : kSdpaSteps;
     static_assert(!(XFORM && KVQ != 0), "the fused forms read a bf16 cache");
     const uint32_t span = a.chunk_len * a.chunks_per_block;  // cache positions per block
@@ -153,6 +161,12 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     if (tid < (uint32_t)GT) {
         stat[tid] = -INFINITY;
         stat[8 + tid] = 0.f;
+    }
+    float m_run[GT], l_run[GT];  // wave-local form: running maximum (uniform) and this lane row's share of the sum
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+        m_run[h] = -INFINITY;
+        l_run[h] = 0.f;
     }
     float acc[GT][8];
     float accb[GT];  // quantised V: sum_j p_j * bias_j of this lane's group, added to its 8 dims at the end
@@ -329,40 +343,141 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }
 
     FK_SDPA_STAMP(1);
-    // ---------------- phase A: scores ----------------
-    {
-        if constexpr (XFORM) {
-            if (owner && kcol_ok) {
+    if constexpr (XFORM) {
+        if (owner && kcol_ok) {
 #pragma unroll
-                for (int u = 0; u < kSteps; ++u)
-                    if (kslot + u * kslots == jpos) kc[u] = *reinterpret_cast<const uint4*>(kn + 8 * ck);
+            for (int u = 0; u < kSteps; ++u)
+                if (kslot + u * kslots == jpos) kc[u] = *reinterpret_cast<const uint4*>(kn + 8 * ck);
+        }
+    }
+    // q . k of key row u and head h, complete in every lane of the row
+    auto score = [&](int u, int h) {
+        float d = 0.f;
+        if constexpr (KVQ == 4) {
+            d = q4_word_dot(kc[u].x, qf[h], 0.f);
+            d = fmaf(bf16_lo(kc[u].z), d, bf16_hi(kc[u].z) * sq[h]);  // s * sum(q * code) + b * sum(q)
+        } else if constexpr (KVQ == 8) {
+            const uint32_t w0 = kc[u].x, w1 = kc[u].y;
+            d = dot2_bf16(pack_bf16((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu)), qf[h].x, d);
+            d = dot2_bf16(pack_bf16((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24)), qf[h].y, d);
+            d = dot2_bf16(pack_bf16((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu)), qf[h].z, d);
+            d = dot2_bf16(pack_bf16((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24)), qf[h].w, d);
+            d = fmaf(bf16_lo(kc[u].z), d, bf16_hi(kc[u].z) * sq[h]);
+        } else {
+            d = dot2_bf16(kc[u].x, qf[h].x, d);
+            d = dot2_bf16(kc[u].y, qf[h].y, d);
+            d = dot2_bf16(kc[u].z, qf[h].z, d);
+            d = dot2_bf16(kc[u].w, qf[h].w, d);
+        }
+        return d;  // this lane's 8 dims only: scores_of() finishes the dot over the row's lanes
+    };
+    // All scores of the range: the per-lane dots first, then ONE uniform choice of the row width
+    // around the cross-lane sums (a width test inside every sum costs six scalar branches each).
+    auto scores_of = [&](float(&d)[kSteps][GT]) {
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u)
+#pragma unroll
+            for (int h = 0; h < GT; ++h) d[u][h] = score(u, h);
+        auto reduce = [&](auto width) {
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u)
+#pragma unroll
+                for (int h = 0; h < GT; ++h) d[u][h] = group_sum(d[u][h], decltype(width)::value);
+        };
+        if (lpk == 16) reduce(std::integral_constant<int, 16>{});
+        else if (lpk == 8) reduce(std::integral_constant<int, 8>{});
+        else if (lpk == 32) reduce(std::integral_constant<int, 32>{});
+        else if (lpk == 64) reduce(std::integral_constant<int, 64>{});
+        else if (lpk == 4) reduce(std::integral_constant<int, 4>{});
+        else if (lpk == 2) reduce(std::integral_constant<int, 2>{});
+    };
+    // This lane's 8 dims of value row u as floats (quantised: the codes; `vs`, `vb` the group's
+    // scale and bias).  Rows past kv_len were requested speculatively: their bits may be
+    // anything, so they are zeroed.
+    auto value = [&](int u, uint32_t j, float(&f)[8], float& vs, float& vb) {
+        const bool ok = j < nkeys && vcol_ok;
+        if constexpr (KVQ != 0) {
+            vs = ok ? bf16_lo(vc[u].z) : 0.f;
+            vb = ok ? bf16_hi(vc[u].z) : 0.f;
+            if constexpr (KVQ == 4) {
+                const uint32_t even = vc[u].x & 0x0F0F0F0Fu, odd = (vc[u].x >> 4) & 0x0F0F0F0Fu;
+                f[0] = (float)(even & 0xffu); f[2] = (float)((even >> 8) & 0xffu);
+                f[4] = (float)((even >> 16) & 0xffu); f[6] = (float)(even >> 24);
+                f[1] = (float)(odd & 0xffu); f[3] = (float)((odd >> 8) & 0xffu);
+                f[5] = (float)((odd >> 16) & 0xffu); f[7] = (float)(odd >> 24);
+            } else {
+                const uint32_t w0 = vc[u].x, w1 = vc[u].y;
+                f[0] = (float)(w0 & 0xffu); f[1] = (float)((w0 >> 8) & 0xffu);
+                f[2] = (float)((w0 >> 16) & 0xffu); f[3] = (float)(w0 >> 24);
+                f[4] = (float)(w1 & 0xffu); f[5] = (float)((w1 >> 8) & 0xffu);
+                f[6] = (float)((w1 >> 16) & 0xffu); f[7] = (float)(w1 >> 24);
+            }
+        } else {
+            vs = 1.f;
+            vb = 0.f;
+            uint4 vv = (FUSED || ok) ? vc[u] : make_uint4(0, 0, 0, 0);
+            if constexpr (MODE == 2) {
+                if (owner && j == jpos && vcol_ok) vv = vnew;  // the new row, not yet cached
+            }
+            f[0] = bf16_lo(vv.x); f[1] = bf16_hi(vv.x); f[2] = bf16_lo(vv.y); f[3] = bf16_hi(vv.y);
+            f[4] = bf16_lo(vv.z); f[5] = bf16_hi(vv.z); f[6] = bf16_lo(vv.w); f[7] = bf16_hi(vv.w);
+        }
+    };
+
+    if constexpr (WAVES) {
+        // ---------------- wave-local: scores, online softmax and value sums in registers ----------------
+        float pr[kSteps][GT];
+        scores_of(pr);
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const bool live = kslot + u * kslots < nkeys;
+#pragma unroll
+            for (int h = 0; h < GT; ++h) pr[u][h] = live ? pr[u][h] * a.scale : -INFINITY;
+        }
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            float mx = pr[0][h];
+#pragma unroll
+            for (int u = 1; u < kSteps; ++u) mx = fmaxf(mx, pr[u][h]);
+            const float m_new = fmaxf(m_run[h], wave_max(mx));
+            const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // no live key yet: every term below is exp(-inf) = 0
+            const float alpha = __expf(m_run[h] - m_ref);
+            float psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                pr[u][h] = __expf(pr[u][h] - m_ref);
+                psum += pr[u][h];
+            }
+            l_run[h] = fmaf(l_run[h], alpha, psum);
+            m_run[h] = m_new;
+            accb[h] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
+        }
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            float f[8], vs, vb;
+            value(u, vslot + u * vslots, f, vs, vb);
+#pragma unroll
+            for (int h = 0; h < GT; ++h) {
+                const float p = pr[u][h];
+                const float ps = KVQ != 0 ? p * vs : p;
+                if constexpr (KVQ != 0) accb[h] = fmaf(p, vb, accb[h]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(ps, f[i], acc[h][i]);
             }
         }
+    } else {
+    // ---------------- phase A: scores ----------------
+    {
+        float d[kSteps][GT];
+        scores_of(d);
 #pragma unroll
         for (int u = 0; u < kSteps; ++u) {
             const uint32_t j = kslot + u * kslots;
 #pragma unroll
-            for (int h = 0; h < GT; ++h) {
-                float d = 0.f;
-                if constexpr (KVQ == 4) {
-                    d = q4_word_dot(kc[u].x, qf[h], 0.f);
-                    d = fmaf(bf16_lo(kc[u].z), d, bf16_hi(kc[u].z) * sq[h]);  // s * sum(q * code) + b * sum(q)
-                } else if constexpr (KVQ == 8) {
-                    const uint32_t w0 = kc[u].x, w1 = kc[u].y;
-                    d = dot2_bf16(pack_bf16((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu)), qf[h].x, d);
-                    d = dot2_bf16(pack_bf16((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24)), qf[h].y, d);
-                    d = dot2_bf16(pack_bf16((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu)), qf[h].z, d);
-                    d = dot2_bf16(pack_bf16((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24)), qf[h].w, d);
-                    d = fmaf(bf16_lo(kc[u].z), d, bf16_hi(kc[u].z) * sq[h]);
-                } else {
-                    d = dot2_bf16(kc[u].x, qf[h].x, d);
-                    d = dot2_bf16(kc[u].y, qf[h].y, d);
-                    d = dot2_bf16(kc[u].z, qf[h].z, d);
-                    d = dot2_bf16(kc[u].w, qf[h].w, d);
-                }
-                d = group_sum(d, (int)lpk);
-                if (ck == 0 && j < nkeys) s[h * a.chunk_len + j] = d * a.scale;
-            }
+            for (int h = 0; h < GT; ++h)
+                if (ck == 0 && j < nkeys) s[h * a.chunk_len + j] = d[u][h] * a.scale;
         }
     }
     FK_SDPA_STAMP(2);
@@ -410,51 +525,20 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         const uint32_t j = vslot + u * vslots;
         const uint32_t jj = j < nkeys ? j : 0u;
         const float live = j < nkeys ? 1.f : 0.f;
-        if constexpr (KVQ != 0) {
-            // codes are integers (always finite); rows past kv_len were requested
-            // speculatively, so their scale / bias bits may be anything: zeroed here
-            const bool ok = j < nkeys && vcol_ok;
-            const float sc = ok ? bf16_lo(vc[u].z) : 0.f, bi = ok ? bf16_hi(vc[u].z) : 0.f;
-            float f[8];
-            if constexpr (KVQ == 4) {
-                const uint32_t even = vc[u].x & 0x0F0F0F0Fu, odd = (vc[u].x >> 4) & 0x0F0F0F0Fu;
-                f[0] = (float)(even & 0xffu); f[2] = (float)((even >> 8) & 0xffu);
-                f[4] = (float)((even >> 16) & 0xffu); f[6] = (float)(even >> 24);
-                f[1] = (float)(odd & 0xffu); f[3] = (float)((odd >> 8) & 0xffu);
-                f[5] = (float)((odd >> 16) & 0xffu); f[7] = (float)(odd >> 24);
-            } else {
-                const uint32_t w0 = vc[u].x, w1 = vc[u].y;
-                f[0] = (float)(w0 & 0xffu); f[1] = (float)((w0 >> 8) & 0xffu);
-                f[2] = (float)((w0 >> 16) & 0xffu); f[3] = (float)(w0 >> 24);
-                f[4] = (float)(w1 & 0xffu); f[5] = (float)((w1 >> 8) & 0xffu);
-                f[6] = (float)((w1 >> 16) & 0xffu); f[7] = (float)(w1 >> 24);
-            }
-#pragma unroll
-            for (int h = 0; h < GT; ++h) {
-                const float p = s[h * a.chunk_len + jj] * live;
-                const float ps = p * sc;
-                accb[h] = fmaf(p, bi, accb[h]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(ps, f[i], acc[h][i]);
-            }
-        } else {
-        // rows past kv_len were requested speculatively: their bits may be anything
-        uint4 vv = (FUSED || (j < nkeys && vcol_ok)) ? vc[u] : make_uint4(0, 0, 0, 0);
-        if constexpr (MODE == 2) {
-            if (owner && j == jpos && vcol_ok) vv = vnew;  // the new row, not yet cached
-        }
-        const float f[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
-                            bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
+        float f[8], vs, vb;
+        value(u, j, f, vs, vb);
 #pragma unroll
         for (int h = 0; h < GT; ++h) {
             const float p = s[h * a.chunk_len + jj] * live;
+            const float ps = KVQ != 0 ? p * vs : p;
+            if constexpr (KVQ != 0) accb[h] = fmaf(p, vb, accb[h]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, f[i], acc[h][i]);
-        }
+            for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(ps, f[i], acc[h][i]);
         }
     }
+    }
     if (c + 1 < n_chunks) {
-        __syncthreads();  // the scores are overwritten by the next range
+        if constexpr (!WAVES) __syncthreads();  // the scores are overwritten by the next range
         if constexpr (MODE != 1) {
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
@@ -466,6 +550,31 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     }  // ranges of this block
     FK_SDPA_STAMP(5);
 
+    if constexpr (WAVES) {
+        // The waves meet: maxima through LDS, every wave rescales its sums to the block's
+        // maximum (exp(-inf) = 0 for a wave that saw no live key) and publishes its share of l.
+        float* wm = stat + 32;
+        float* wl = stat + 64;
+        if (lane == 0) {
+#pragma unroll
+            for (int h = 0; h < GT; ++h) wm[wave * 8 + h] = m_run[h];
+        }
+        __syncthreads();
+        const float inv_lanes = 1.0f / (float)lpk;  // a row's sum is held by each of its lpk lanes (power of two: exact)
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            float M = wm[h];
+#pragma unroll
+            for (int w = 1; w < kSdpaWaves; ++w) M = fmaxf(M, wm[w * 8 + h]);
+            const float f = __expf(m_run[h] - M);
+            accb[h] *= f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][i] *= f;
+            const float lw = wave_sum(l_run[h]) * inv_lanes * f;
+            if (lane == 0) wl[wave * 8 + h] = lw;
+            if (tid == 0) stat[h] = M;
+        }
+    }
     // Every lane parks its sums in LDS, [value slot][head][dim]; the output loop below
     // adds the slots in index order (no cross-lane shuffles, fixed order).
     if constexpr (KVQ != 0) {
@@ -483,6 +592,16 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
     }
     __syncthreads();
+    if constexpr (WAVES) {
+        if (tid < (uint32_t)GT) {
+            const float* wl = stat + 64;
+            float l = wl[tid];
+#pragma unroll
+            for (int w = 1; w < kSdpaWaves; ++w) l += wl[w * 8 + tid];
+            stat[8 + tid] = l;
+        }
+        __syncthreads();
+    }
 
     FK_SDPA_STAMP(6);
     const uint32_t n_out = gcount * a.v_dim;
