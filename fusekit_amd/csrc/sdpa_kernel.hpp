@@ -426,33 +426,56 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 
     if constexpr (WAVES) {
         // ---------------- wave-local: scores, online softmax and value sums in registers ----------------
+        // Scores and running maxima are kept in base-2 units (scale * log2(e) folded into one
+        // multiply), so a probability is one v_exp_f32.
         float pr[kSteps][GT];
         scores_of(pr);
+        const float scale2 = a.scale * 1.44269504088896341f;
 #pragma unroll
         for (int u = 0; u < kSteps; ++u) {
             const bool live = kslot + u * kslots < nkeys;
 #pragma unroll
-            for (int h = 0; h < GT; ++h) pr[u][h] = live ? pr[u][h] * a.scale : -INFINITY;
+            for (int h = 0; h < GT; ++h) pr[u][h] = live ? pr[u][h] * scale2 : -INFINITY;
+        }
+        float mx[GT];
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            mx[h] = pr[0][h];
+#pragma unroll
+            for (int u = 1; u < kSteps; ++u) mx[h] = fmaxf(mx[h], pr[u][h]);
+        }
+        if (lpk < 16) {  // two or more key rows share a 16-lane row: finish the maximum inside it
+#pragma unroll
+            for (int h = 0; h < GT; ++h) {
+                mx[h] = dpp_max<0xB1>(mx[h]);
+                mx[h] = dpp_max<0x4E>(mx[h]);
+                mx[h] = dpp_max<0x141>(mx[h]);
+                mx[h] = dpp_max<0x140>(mx[h]);
+            }
         }
 #pragma unroll
         for (int h = 0; h < GT; ++h) {
-            float mx = pr[0][h];
-#pragma unroll
-            for (int u = 1; u < kSteps; ++u) mx = fmaxf(mx, pr[u][h]);
-            const float m_new = fmaxf(m_run[h], wave_max(mx));
-            const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // no live key yet: every term below is exp(-inf) = 0
-            const float alpha = __expf(m_run[h] - m_ref);
+            // every 16-lane row is uniform now: the wave's maximum is that of lanes 0, 16, 32, 48
+            const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx[h]), 0));
+            const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx[h]), 16));
+            const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx[h]), 32));
+            const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx[h]), 48));
+            const float m_new = fmaxf(fmaxf(m_run[h], fmaxf(r0, r1)), fmaxf(r2, r3));
+            const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // no live key yet: every term below is 2^-inf = 0
+            const float alpha = __builtin_amdgcn_exp2f(m_run[h] - m_ref);
             float psum = 0.f;
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
-                pr[u][h] = __expf(pr[u][h] - m_ref);
+                pr[u][h] = __builtin_amdgcn_exp2f(pr[u][h] - m_ref);
                 psum += pr[u][h];
             }
             l_run[h] = fmaf(l_run[h], alpha, psum);
             m_run[h] = m_new;
-            accb[h] *= alpha;
+            if (alpha != 1.f) {  // the maximum rose (rare after the first ranges)
+                accb[h] *= alpha;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
+                for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
+            }
         }
 #pragma unroll
         for (int u = 0; u < kSteps; ++u) {
@@ -566,13 +589,13 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             float M = wm[h];
 #pragma unroll
             for (int w = 1; w < kSdpaWaves; ++w) M = fmaxf(M, wm[w * 8 + h]);
-            const float f = __expf(m_run[h] - M);
+            const float f = __builtin_amdgcn_exp2f(m_run[h] - M);
             accb[h] *= f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[h][i] *= f;
             const float lw = wave_sum(l_run[h]) * inv_lanes * f;
             if (lane == 0) wl[wave * 8 + h] = lw;
-            if (tid == 0) stat[h] = M;
+            if (tid == 0) stat[h] = M * 0.693147180559945309f;  // back to natural units for the (m, l, o) partials
         }
     }
     // Every lane parks its sums in LDS, [value slot][head][dim]; the output loop below
