@@ -145,7 +145,7 @@ __device__ __forceinline__ uint32_t swiglu_bits(float acc_g, float acc_u, int va
 // sum-of-squares pass and the write pass, so x and the norm weight are fetched
 // once.  The threads that hold the pieces of one chunk are adjacent lanes, so the
 // chunk sum is a 2- or 4-lane butterfly.  K must be a multiple of 64.
-constexpr int kStageRegs = 4;
+constexpr int kStageRegs = 5;
 
 // Issues the loads of the register-resident part of x (and the norm weight).  A
 // stand-alone kernel calls this BEFORE the weight prefetch: loads return in issue
