@@ -96,7 +96,7 @@ fk_status fk_target_describe(fk_target* out) {
     out->lds_bytes_per_cu = 160 * 1024;
     out->workgroup_threads = 256;
     out->gemm_min_rows = 2;
-    out->gemm_rows_per_pass = 32;
+    out->gemm_rows_per_pass = 128;
     out->hbm_bytes = 288ull << 30;
     out->hbm_peak_bytes_per_s = 8.0e12;
     out->mfma_bf16_peak_flops = 2.5e15;

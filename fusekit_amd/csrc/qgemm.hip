@@ -18,12 +18,24 @@
 // 64 or 128).  MFMA step j takes word j (words 2j, 2j+1) of every lane: its 16 k
 // values are 8 from each half, matched by the activation fragment read from LDS.
 //
-// A block is 4 waves = 128 weight rows over one k range and one tile of 32
-// activation rows; x is staged per 512-k slab into LDS in the lane order the MFMA
-// wants (and, for int4, in the nibble pairing of the unpack).  The k dimension is
+// From 65 activation rows up (MT = 4) the affine map is applied BEFORE the matrix
+// instruction instead: w = T(s * q + b), one bf16 rounding per weight element, as the
+// reference's multi-row path does (it dequantises into bf16 tiles, msl.rs:2318-2440), and the
+// products accumulate straight into the fp32 result.  The fold per group (32 VALU
+// instructions per tile of 32 rows and group of 64) is what bounds the exact form; the
+// dequantised form spends 22 VALU instructions per fragment, shared by four tiles, and is
+// bound by the matrix cores.
+//
+// A block is 4 waves = 128 weight rows over one k range and MT tiles of 32
+// activation rows (MT = 1, 2 or 4 by the row count): a fragment of unpacked weights
+// feeds MT matrix instructions, so the unpack work, which bounds this kernel, is
+// shared by up to 128 rows.  x is staged per k slab (512, or 256 for MT = 4) into LDS
+// in the lane order the MFMA wants (and, for int4, in the nibble pairing of the unpack).  The k dimension is
 // split over blocks until the grid fills the chip; partial sums go to an fp32
 // workspace and a second kernel adds them in split order and applies the epilogue,
 // so the result does not depend on block scheduling.
+#include <mutex>
+
 #include "fk_host.hpp"
 #include "gemv_kernel.hpp"
 
@@ -35,8 +47,11 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 constexpr int kQgemmBlock = 256;
 constexpr uint32_t kQgemmRows = 128;   // weight rows per block
 constexpr uint32_t kQgemmMTile = 32;   // activation rows per block
-constexpr uint32_t kQgemmSlabK = 512;  // k staged per LDS slab
-constexpr uint32_t kQgemmXStride = kQgemmSlabK / 8 + 1;  // uint4 per staged row (+1: bank spread)
+constexpr uint32_t qgemm_slab_k(int mt) { return mt == 4 ? 256u : 512u; }                // k staged per LDS slab
+constexpr uint32_t qgemm_x_stride(int mt) { return qgemm_slab_k(mt) / 8 + 1; }            // uint4 per staged row (+1: bank spread)
+constexpr uint32_t qgemm_lds_bytes(int mt) {
+    return (uint32_t)mt * kQgemmMTile * qgemm_x_stride(mt) * 16u + (qgemm_slab_k(mt) / 64u) * (uint32_t)mt * kQgemmMTile * 4u;
+}
 
 struct QgemmArgs {
     const uint4* w;
@@ -52,20 +67,24 @@ struct QgemmArgs {
     uint32_t n_blocks;     // blocks along N
 };
 
-constexpr uint32_t kQgemmLdsBytes = kQgemmMTile * kQgemmXStride * 16u + (kQgemmSlabK / 64u) * kQgemmMTile * 4u;
-
-template <WKind KIND>
+template <WKind KIND, int MT>
 __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
     constexpr uint32_t VPL = KIND == W_Q4 ? 32u : 16u;  // codes per 16-byte lane load
     constexpr int MF = VPL / 8;                         // MFMA steps per load
+    constexpr uint32_t SLAB = qgemm_slab_k(MT), XS = qgemm_x_stride(MT), ROWS = MT * kQgemmMTile;
+    constexpr bool DEQ = MT == 4;  // weights dequantised to bf16 before the multiply (see the head of this file)
+    constexpr int LOADS = SLAB / (2u * VPL);            // 16-byte weight loads per lane and slab
+    constexpr int UNITS = SLAB / 64u;                   // 64-k units per slab (one scale / bias pair each)
+    constexpr uint32_t S8 = SLAB / 8u;                  // 16-byte pieces of x per row and slab
+    constexpr int XPT = ROWS * S8 / kQgemmBlock;        // pieces of x per thread and slab
     extern __shared__ uint4 lds_raw[];
-    uint4* xs = lds_raw;                                                      // [32][kQgemmXStride]
-    float* sxs = reinterpret_cast<float*>(xs + kQgemmMTile * kQgemmXStride);  // [groups in slab][32]
+    uint4* xs = lds_raw;                                       // [ROWS][XS]
+    float* sxs = reinterpret_cast<float*>(xs + ROWS * XS);     // [groups in slab][ROWS]
 
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, kb = lane >> 5, nl = lane & 31u;
     const uint32_t nb = blockIdx.x % a.n_blocks, ks = blockIdx.x / a.n_blocks;
-    const uint32_t m0 = blockIdx.y * kQgemmMTile;
-    const uint32_t mt = a.M - m0 < kQgemmMTile ? a.M - m0 : kQgemmMTile;
+    const uint32_t m0 = blockIdx.y * ROWS;
+    const uint32_t mt = a.M - m0 < ROWS ? a.M - m0 : ROWS;  // live activation rows of this block
     const uint32_t n = nb * kQgemmRows + wave * 32u + nl;
     const uint32_t nc = n < a.N ? n : a.N - 1;  // rows past the end read the last row; never stored
     const uint32_t k0 = ks * a.k_per_split;
@@ -76,106 +95,169 @@ __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
     const uint16_t* brow = a.bi + (size_t)nc * a.gpr;
     const uint32_t lpg_mask = a.group / (2u * VPL) - 1u;  // loads per group - 1 (power of two)
     const uint32_t g8 = a.group >> 3;
+    const uint32_t gshift = a.group == 128 ? 7u : 6u;
 
-    f32x16_t acc;
+    f32x16_t acc[MT];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
-    for (uint32_t ks0 = k0; ks0 < k1; ks0 += kQgemmSlabK) {
-        const uint32_t slab_k = k1 - ks0 < kQgemmSlabK ? k1 - ks0 : kQgemmSlabK;
-        const uint32_t s8 = slab_k >> 3;
+    // Everything a slab needs from memory is requested one slab ahead, while the previous one
+    // is multiplied: the weight pieces and scale / bias pairs of this lane's row, and this
+    // thread's share of the activations (parked in registers until the LDS tile is free).
+    // With one request in flight per lane the kernel ran at the latency of its loads.
+    uint4 wq[LOADS], xq[XPT];
+    uint32_t sbq[UNITS];
+    auto fetch = [&](uint32_t ks0) {
+        const uint32_t slab_k = k1 - ks0 < SLAB ? k1 - ks0 : SLAB;
+        const uint32_t loads = slab_k / (2u * VPL), units = slab_k >> 6, s8 = slab_k >> 3;
+        const uint4* wp = wrow + ks0 / VPL + kb;
+#pragma unroll
+        for (int t = 0; t < LOADS; ++t) wq[t] = wp[2u * ((uint32_t)t < loads ? (uint32_t)t : 0u)];
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u) {
+            const uint32_t g = (ks0 + ((uint32_t)u < units ? (uint32_t)u : 0u) * 64u) >> gshift;
+            sbq[u] = (uint32_t)srow[g] | ((uint32_t)brow[g] << 16);
+        }
+        // requests only: nothing here may use a loaded value (that would wait for it before the
+        // remaining requests are made); rows and slab tails that do not exist are zeroed when
+        // the piece is written to LDS
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) {
+            const uint32_t idx = threadIdx.x + (uint32_t)i * kQgemmBlock, m = idx / S8, k8 = idx % S8;
+            const bool live = m < mt && k8 < s8;
+            xq[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(m0 + (live ? m : 0u)) * a.K + ks0 + (live ? k8 : 0u) * 8u);
+        }
+    };
+    fetch(k0);
+
+    for (uint32_t ks0 = k0; ks0 < k1; ks0 += SLAB) {
+        const uint32_t slab_k = k1 - ks0 < SLAB ? k1 - ks0 : SLAB;
         __syncthreads();  // the previous slab has been consumed
-        for (uint32_t idx = threadIdx.x; idx < mt * s8; idx += kQgemmBlock) {
-            const uint32_t m = idx / s8, k8 = idx - m * s8;
-            uint4 v = *reinterpret_cast<const uint4*>(a.x + (size_t)(m0 + m) * a.K + ks0 + k8 * 8u);
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) {
+            const uint32_t idx = threadIdx.x + (uint32_t)i * kQgemmBlock, m = idx / S8, k8 = idx % S8;
+            uint4 v = (m < mt && k8 < (slab_k >> 3)) ? xq[i] : make_uint4(0, 0, 0, 0);
             if constexpr (KIND == W_Q4) {
                 // nibble pairing of q4_word_dot: (x0,x2) (x4,x6) (x1,x3) (x5,x7)
                 v = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
                                (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
             }
-            xs[m * kQgemmXStride + k8] = v;
+            xs[m * XS + k8] = v;
         }
+        uint4 wcur[LOADS];
+        uint32_t sbcur[UNITS];
+#pragma unroll
+        for (int t = 0; t < LOADS; ++t) wcur[t] = wq[t];
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u) sbcur[u] = sbq[u];
+        if (ks0 + SLAB < k1) fetch(ks0 + SLAB);
         __syncthreads();
-        const uint32_t ng = slab_k / a.group;
-        for (uint32_t idx = threadIdx.x; idx < ng * kQgemmMTile; idx += kQgemmBlock) {
-            const uint32_t g = idx >> 5, m = idx & 31u;
-            float s = 0.f;
-            if (m < mt) {
+        if constexpr (!DEQ) {
+            const uint32_t ng = slab_k / a.group;
+            for (uint32_t idx = threadIdx.x; idx < ng * ROWS; idx += kQgemmBlock) {
+                const uint32_t g = idx / ROWS, m = idx - g * ROWS;
+                float s = 0.f;
                 for (uint32_t i = 0; i < g8; ++i) {
-                    const uint4 v = xs[m * kQgemmXStride + g * g8 + i];
+                    const uint4 v = xs[m * XS + g * g8 + i];
                     s += ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
                          ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
                 }
+                sxs[idx] = s;
             }
-            sxs[idx] = s;
+            __syncthreads();
         }
-        __syncthreads();
 
         const uint32_t loads = slab_k / (2u * VPL);
-        const uint4* wp = wrow + ks0 / VPL + kb;
-        const uint32_t gbase = ks0 / a.group;
-        uint4 cur = wp[0];
-        f32x16_t c;
+        f32x16_t c[MT];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) c[r] = 0.f;
-        for (uint32_t t = 0; t < loads; ++t) {
-            const uint32_t tn = t + 1 < loads ? t + 1 : t;
-            const uint4 nxt = wp[2u * tn];
-            const uint32_t gl = (t * 2u * VPL) / a.group;  // group of this load inside the slab
-            const uint32_t s_bits = srow[gbase + gl], b_bits = brow[gbase + gl];
-            const uint32_t wd[4] = {cur.x, cur.y, cur.z, cur.w};
-            const uint4* xa = xs + nl * kQgemmXStride + ((t * 2u + kb) * VPL >> 3);
+        for (int i = 0; i < MT; ++i)
 #pragma unroll
-            for (int j = 0; j < MF; ++j) {
-                uint4 bw;
-                if constexpr (KIND == W_Q4) {
-                    const uint32_t even = wd[j] & 0x0F0F0F0Fu, odd = (wd[j] >> 4) & 0x0F0F0F0Fu;
-                    bw.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false));
-                    bw.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, true));
-                    bw.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, false));
-                    bw.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, true));
-                } else {
-                    const uint32_t w0 = wd[2 * j], w1 = wd[2 * j + 1];
-                    auto pair = [](float lo, float hi) {
-                        const bf16x2_t p = {(__bf16)lo, (__bf16)hi};  // integers <= 255 are exact in bf16
-                        return __builtin_bit_cast(uint32_t, p);
-                    };
-                    bw.x = pair((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu));
-                    bw.y = pair((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24));
-                    bw.z = pair((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu));
-                    bw.w = pair((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24));
+            for (int r = 0; r < 16; ++r) c[i][r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < LOADS; ++t) {
+            if ((uint32_t)t < loads) {
+                const uint32_t sb = sbcur[(t * 2 * (int)VPL) / 64];
+                const float sf = bf16_bits_to_f32(sb & 0xffffu), bf = bf16_bits_to_f32(sb >> 16);
+                const uint32_t wd[4] = {wcur[t].x, wcur[t].y, wcur[t].z, wcur[t].w};
+                const uint4* xa = xs + nl * XS + (((uint32_t)t * 2u + kb) * VPL >> 3);
+#pragma unroll
+                for (int j = 0; j < MF; ++j) {
+                    uint4 bw;
+                    if constexpr (DEQ) {
+                        // eight codes of this lane in the order the staged activations expect:
+                        // int4 (n0, n2) (n4, n6) (n1, n3) (n5, n7), int8 in element order
+                        const uint32_t lo = KIND == W_Q4 ? (wd[j] & 0x0F0F0F0Fu) : wd[(2 * j) & 3];
+                        const uint32_t hi = KIND == W_Q4 ? ((wd[j] >> 4) & 0x0F0F0F0Fu) : wd[(2 * j + 1) & 3];
+                        auto dq = [&](uint32_t byte) { return fmaf((float)byte, sf, bf); };
+                        bw.x = pack_bf16(dq(lo & 0xffu), dq((lo >> 8) & 0xffu));
+                        bw.y = pack_bf16(dq((lo >> 16) & 0xffu), dq(lo >> 24));
+                        bw.z = pack_bf16(dq(hi & 0xffu), dq((hi >> 8) & 0xffu));
+                        bw.w = pack_bf16(dq((hi >> 16) & 0xffu), dq(hi >> 24));
+                    } else if constexpr (KIND == W_Q4) {
+                        const uint32_t even = wd[j] & 0x0F0F0F0Fu, odd = (wd[j] >> 4) & 0x0F0F0F0Fu;
+                        bw.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false));
+                        bw.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, true));
+                        bw.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, false));
+                        bw.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, true));
+                    } else {
+                        const uint32_t w0 = wd[(2 * j) & 3], w1 = wd[(2 * j + 1) & 3];
+                        auto pair = [](float lo, float hi) {
+                            const bf16x2_t p = {(__bf16)lo, (__bf16)hi};  // integers <= 255 are exact in bf16
+                            return __builtin_bit_cast(uint32_t, p);
+                        };
+                        bw.x = pair((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu));
+                        bw.y = pair((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24));
+                        bw.z = pair((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu));
+                        bw.w = pair((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24));
+                    }
+                    // the unpacked fragment serves every tile of activation rows
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        const uint4 av = xa[i * kQgemmMTile * XS + j];
+                        if constexpr (DEQ)
+                            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                             __builtin_bit_cast(bf16x8_t, bw), acc[i], 0, 0, 0);
+                        else
+                            c[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                           __builtin_bit_cast(bf16x8_t, bw), c[i], 0, 0, 0);
+                    }
                 }
-                const uint4 av = xa[j];
-                c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                            __builtin_bit_cast(bf16x8_t, bw), c, 0, 0, 0);
-            }
-            if ((t & lpg_mask) == lpg_mask) {
-                // group complete: fold the integer dot into the accumulators.  Register r
-                // of this lane is activation row (r % 4) + 8 * (r / 4) + 4 * kb.
-                const float s = bf16_bits_to_f32(s_bits), b = bf16_bits_to_f32(b_bits);
-                const float* sxg = sxs + gl * kQgemmMTile + 4u * kb;
+                if constexpr (!DEQ) {
+                    if (((uint32_t)t & lpg_mask) == lpg_mask) {
+                        // group complete: fold the integer dot into the accumulators.  Register r
+                        // of this lane is activation row (r % 4) + 8 * (r / 4) + 4 * kb of its tile.
+                        const uint32_t gl = ((uint32_t)t * 2u * VPL) >> gshift;  // group inside the slab
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 sx4 = *reinterpret_cast<const float4*>(sxg + 8 * q);
-                    acc[4 * q + 0] += fmaf(s, c[4 * q + 0], b * sx4.x);
-                    acc[4 * q + 1] += fmaf(s, c[4 * q + 1], b * sx4.y);
-                    acc[4 * q + 2] += fmaf(s, c[4 * q + 2], b * sx4.z);
-                    acc[4 * q + 3] += fmaf(s, c[4 * q + 3], b * sx4.w);
+                        for (int i = 0; i < MT; ++i) {
+                            const float* sxg = sxs + gl * ROWS + i * kQgemmMTile + 4u * kb;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                const float4 sx4 = *reinterpret_cast<const float4*>(sxg + 8 * q);
+                                acc[i][4 * q + 0] += fmaf(sf, c[i][4 * q + 0], bf * sx4.x);
+                                acc[i][4 * q + 1] += fmaf(sf, c[i][4 * q + 1], bf * sx4.y);
+                                acc[i][4 * q + 2] += fmaf(sf, c[i][4 * q + 2], bf * sx4.z);
+                                acc[i][4 * q + 3] += fmaf(sf, c[i][4 * q + 3], bf * sx4.w);
+                            }
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) c[i][r] = 0.f;
+                        }
+                    }
                 }
-#pragma unroll
-                for (int r = 0; r < 16; ++r) c[r] = 0.f;
             }
-            cur = nxt;
         }
     }
 
     if (n < a.N) {
         float* dst = a.partial + ((size_t)ks * a.M + m0) * a.N + n;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t m = (uint32_t)(r % 4 + 8 * (r / 4)) + 4u * kb;
-            if (m < mt) dst[(size_t)m * a.N] = acc[r];
-        }
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t m = (uint32_t)(i * (int)kQgemmMTile + r % 4 + 8 * (r / 4)) + 4u * kb;
+                if (m < mt) dst[(size_t)m * a.N] = acc[i][r];
+            }
     }
 }
 
@@ -210,18 +292,51 @@ namespace {
 
 struct QgemmShape {
     uint32_t n_blocks, m_tiles, ksplit, k_per_split;
+    int mt;  // tiles of 32 activation rows per block
 };
 
-fk_status qgemm_shape(const DeviceFacts* dev, uint32_t M, uint32_t N, uint32_t K, uint32_t group, QgemmShape* out) {
+const void* qgemm_func(uint32_t bits, int mt) {
+    const bool q4 = bits == 4;
+    switch (mt) {
+        case 1: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 1>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 1>);
+        case 2: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 2>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 2>);
+        default: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 4>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 4>);
+    }
+}
+
+// Blocks of this kernel form that are resident at once (registers and LDS decide).
+uint32_t qgemm_resident(const DeviceFacts* dev, uint32_t bits, int mt) {
+    static std::mutex mu;
+    static int cache[2][5] = {{0, 0, 0, 0, 0}, {0, 0, 0, 0, 0}};
+    std::lock_guard<std::mutex> lk(mu);
+    int& slot = cache[bits == 4 ? 0 : 1][mt];
+    if (slot == 0) {
+        const void* f = qgemm_func(bits, mt);
+        const uint32_t lds = qgemm_lds_bytes(mt);
+        if (lds > 48 * 1024) (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, f, kQgemmBlock, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+        slot = per_cu > 2 ? 2 : per_cu;  // more than two blocks per CU gain nothing here
+    }
+    return (uint32_t)slot * (uint32_t)dev->cus;
+}
+
+fk_status qgemm_shape(const DeviceFacts* dev, uint32_t M, uint32_t N, uint32_t K, uint32_t group, uint32_t bits,
+                      QgemmShape* out) {
     if (M == 0 || N == 0 || K == 0) return set_error(FK_ERR_INVALID, "qgemm: empty shape");
     if (group != 64 && group != 128) return set_error(FK_ERR_UNSUPPORTED, "qgemm: group size must be 64 or 128");
     if (K % group) return set_error(FK_ERR_UNSUPPORTED, "qgemm: K must be a multiple of the group size");
     if ((uint64_t)M * N > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "qgemm: output too large");
     QgemmShape s;
     s.n_blocks = (N + kQgemmRows - 1) / kQgemmRows;
-    s.m_tiles = (M + kQgemmMTile - 1) / kQgemmMTile;
-    // Split k until about two blocks per CU exist, but keep at least 256 k per block.
-    const uint32_t want = (2u * (uint32_t)dev->cus + s.n_blocks * s.m_tiles - 1) / (s.n_blocks * s.m_tiles);
+    s.mt = M > 64 ? 4 : (M > 32 ? 2 : 1);
+    s.m_tiles = (M + kQgemmMTile * s.mt - 1) / (kQgemmMTile * s.mt);
+    // Split k until the grid fills what is resident at once, never beyond (a block that waits
+    // for a slot doubles the run time), and keep at least 256 k per block.  Every split writes
+    // and re-reads an fp32 copy of the output.
+    const uint32_t blocks = s.n_blocks * s.m_tiles;
+    const uint32_t target = qgemm_resident(dev, bits, s.mt);
+    const uint32_t want = target / blocks;
     uint32_t max_split = K / 256u;
     if (max_split < 1) max_split = 1;
     uint32_t split = want < 1 ? 1 : (want > max_split ? max_split : want);
@@ -242,7 +357,7 @@ fk_status check_weight(const fk_weight* W, const char* who) {
 
 fk_status plan_qgemm_main(const DeviceFacts* dev, const fk_weight* W, const uint16_t* x, uint32_t M, float* partial,
                           QgemmShape* shape, Launch* out) {
-    FK_TRY(qgemm_shape(dev, M, W->n, W->k, W->group, shape));
+    FK_TRY(qgemm_shape(dev, M, W->n, W->k, W->group, W->bits, shape));
     QgemmArgs a;
     memset(&a, 0, sizeof(a));
     a.w = reinterpret_cast<const uint4*>(W->w);
@@ -258,12 +373,13 @@ fk_status plan_qgemm_main(const DeviceFacts* dev, const fk_weight* W, const uint
     a.group = W->group;
     a.k_per_split = shape->k_per_split;
     a.n_blocks = shape->n_blocks;
-    out->func = W->bits == 4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4>)
-                             : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8>);
+    out->func = qgemm_func(W->bits, shape->mt);
     out->grid = dim3(shape->n_blocks * shape->ksplit, shape->m_tiles, 1);
     out->block = dim3(kQgemmBlock, 1, 1);
-    out->shmem = kQgemmLdsBytes;
+    out->shmem = qgemm_lds_bytes(shape->mt);
     out->set_args(a);
+    if (out->shmem > 48 * 1024)
+        FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)out->shmem));
     return FK_OK;
 }
 
@@ -284,9 +400,11 @@ void plan_reduce(const float* p0, const float* p1, const uint16_t* bias, const u
 fk_status qgemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group, size_t* bytes) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
-    QgemmShape s;
-    FK_TRY(qgemm_shape(dev, M, N, K, group, &s));
-    *bytes = (size_t)s.ksplit * M * N * sizeof(float);
+    // the split depends on the kernel form (4- or 8-bit codes): size for the larger of the two
+    QgemmShape s4, s8;
+    FK_TRY(qgemm_shape(dev, M, N, K, group, 4, &s4));
+    FK_TRY(qgemm_shape(dev, M, N, K, group, 8, &s8));
+    *bytes = (size_t)(s4.ksplit > s8.ksplit ? s4.ksplit : s8.ksplit) * M * N * sizeof(float);
     return FK_OK;
 }
 

@@ -321,10 +321,11 @@ class DecoderRuntime:
         nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
         return nxt[-1]
 
-    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 32) -> int:
+    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 128) -> int:
         """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
-        active_m > 1 variants): the projections of up to 32 tokens share ONE pass over each weight
-        matrix on the matrix cores (fk_qgemm), attention is causal inside the group.  Leaves the KV
+        active_m > 1 variants): the projections of up to 128 tokens share ONE pass over each weight
+        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form), attention is
+        causal inside the group.  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy
         first token.  Quantised projections only (the dense bf16 multi-row matmul is a library GEMM)."""
         c, w = self.cfg, self.w
@@ -333,10 +334,13 @@ class DecoderRuntime:
         prompt = list(prompt)
         if start_offset + len(prompt) > c.capacity:
             raise ValueError("prompt exceeds the KV-cache capacity")
-        R = max(1, min(rows_per_pass, 32))
-        if not hasattr(self, "_rows"):
-            ws = max(native.qgemm_workspace_bytes(R, n, k, c.group) for n, k in
-                     ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
+        R = max(1, min(rows_per_pass, 128))
+        if getattr(self, "_rows_R", 0) != R:
+            self._rows_R = R
+            # the split of k differs between the kernel forms for <= 32, <= 64 and more rows
+            ws = max(native.qgemm_workspace_bytes(m, n, k, c.group)
+                     for m in {R, min(R, 64), min(R, 32)}
+                     for n, k in ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
             pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.capacity)
             self._rows = dict(
                 tok=DeviceBuffer(4 * R), x=DeviceBuffer(R * c.hidden * 2), x2=DeviceBuffer(R * c.hidden * 2),

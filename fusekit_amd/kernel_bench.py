@@ -193,8 +193,8 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
           note="two kernels: MFMA main + split-k reduction")
 
 
-def case_prefill(d, reps, prompt_len=512):
-    """Chunked prefill of the 4B-class model: 32 prompt tokens per pass over the weights."""
+def case_prefill(d, reps, prompt_len=512, rows_per_pass=128):
+    """Chunked prefill of the 4B-class model: `rows_per_pass` prompt tokens per pass over the weights."""
     import time
     import numpy as np
     from .decoder import DENSE_4B, DecoderConfig, DecoderRuntime, DecoderWeights
@@ -202,15 +202,15 @@ def case_prefill(d, reps, prompt_len=512):
     W = DecoderWeights.random_init(cfg, seed=0)
     rt = DecoderRuntime(cfg, W, dispatcher=d)
     prompt = np.random.Generator(np.random.PCG64(0)).integers(0, cfg.vocab, prompt_len).tolist()
-    rt.prefill_rows(prompt[:64])
+    rt.prefill_rows(prompt, rows_per_pass=rows_per_pass)
     t0 = time.perf_counter()
-    rt.prefill_rows(prompt)
+    rt.prefill_rows(prompt, rows_per_pass=rows_per_pass)
     rows_s = time.perf_counter() - t0
     t0 = time.perf_counter()
     rt.prefill(prompt[:64])
     single_s = (time.perf_counter() - t0) / 64 * prompt_len
     flops = 2.0 * prompt_len * (cfg.n_layers * (cfg.hidden * (cfg.n_q + 2 * cfg.n_kvd) + cfg.n_q * cfg.hidden + 3 * cfg.inter * cfg.hidden))
-    print(json.dumps({"case": f"prefill_4b_q4_{prompt_len}_tokens", "rows_per_pass": 32,
+    print(json.dumps({"case": f"prefill_4b_q4_{prompt_len}_tokens", "rows_per_pass": rows_per_pass,
                       "prompt_tok_per_s": round(prompt_len / rows_s, 1), "ms": round(rows_s * 1e3, 2),
                       "token_by_token_tok_per_s": round(prompt_len / single_s, 1),
                       "TFLOPs": round(flops / rows_s / 1e12, 2)}), flush=True)
@@ -233,6 +233,7 @@ CASES = {
     "qgemm_32": lambda d, r: case_qgemm(d, r, 32),
     "qgemm_128": lambda d, r: case_qgemm(d, r, 128),
     "qgemm_512": lambda d, r: case_qgemm(d, r, 512),
+    "prefill_4b_32": lambda d, r: case_prefill(d, r, 512, 32),
     "prefill_4b": lambda d, r: case_prefill(d, r),
 }
 

@@ -111,7 +111,7 @@ typedef struct fk_target {
     uint32_t workgroup_threads;     /* 256: threadgroup size every kernel here uses (4 waves) */
     uint32_t gemm_min_rows;         /* active rows from which the matrix-core path is taken (the reference: 8,
                                        src/target/mod.rs:162-171; here 2 -- one weight pass serves 32 rows) */
-    uint32_t gemm_rows_per_pass;    /* 32 */
+    uint32_t gemm_rows_per_pass;    /* 128: activation rows one block of the multi-row matmul serves */
     uint64_t hbm_bytes;
     double hbm_peak_bytes_per_s;    /* 8.0e12, published */
     double mfma_bf16_peak_flops;    /* 2.5e15 dense, published */

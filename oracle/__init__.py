@@ -334,6 +334,16 @@ def qgemm(W: QWeight, x: np.ndarray, bias=None) -> np.ndarray:
     return y
 
 
+def qgemm_bf16w(W: QWeight, x: np.ndarray, bias=None, want_acc: bool = False):
+    """Multi-row matmul with every dequantised weight rounded to bf16 first (the reference's
+    large-M form).  Returns y, or (y, unrounded fp32 sums) with want_acc."""
+    m = x.shape[0]
+    y = np.empty((m, W.n), dtype=np.uint16)
+    acc = np.empty((m, W.n), dtype=np.float32) if want_acc else None
+    _lib.fko_qgemm_bf16w(C.byref(W.c), _p(x, _u16p), C.c_int64(m), _p(bias, _u16p), _p(y, _u16p), _p(acc, _f32p))
+    return (y, acc) if want_acc else y
+
+
 # ------------------------------------------------------------------ quantised KV cache
 
 class QuantCache:

@@ -32,6 +32,10 @@
  *                                 reference's multi-row path rounds every dequantised
  *                                 weight to bf16 first (MLX QuantizedBlockLoader, not
  *                                 vendored): that rounding is parity unpinned
+ *   qgemm, weights rounded to bf16 pinned as arithmetic (numpy: dequantise, round to bf16,
+ *                                 float64 matmul; one-hot rows return T(s*q+b) exactly); that
+ *                                 MLX rounds exactly there is read from the reference's
+ *                                 emitter, MLX itself is not vendored: parity unpinned
  *   quantised KV store / attention pinned (V rows and unrotated K rows = the pinned quantiser
  *                                 bit for bit; rotated K rows dequantise to within the
  *                                 quantiser's step of the pinned bf16 RoPE; only the
@@ -729,6 +733,37 @@ FKO_API void fko_routed_qmv_reduce(const uint16_t *h, const fko_weight *Wd, int6
  *    repetition of K1 (qMM-T semantics, src/codegen/msl.rs:2318-2440: fp32 accumulate, one round). */
 FKO_API void fko_qgemm(const fko_weight *W, const uint16_t *x, int64_t m, const uint16_t *bias, uint16_t *y) {
     for (int64_t r = 0; r < m; ++r) fko_qgemv(W, x + r * W->k, bias, y + r * W->n);
+}
+
+/* G, large-M form: the reference's multi-row kernels dequantise a tile of weights into the
+ *    activation type before the multiply (msl.rs:2318-2440: QuantizedBlockLoader of MLX fills a
+ *    threadgroup tile of T), i.e. w = T(s * q + b), one bf16 rounding per weight element, then
+ *    y[M, N] = T(x @ w^T (+ bias)) with fp32 accumulation.  `acc_out` (optional) receives the
+ *    unrounded sums. */
+FKO_API void fko_qgemm_bf16w(const fko_weight *W, const uint16_t *x, int64_t m, const uint16_t *bias, uint16_t *y,
+                             float *acc_out) {
+    const int64_t N = W->n, K = W->k;
+    const int per_word = 32 / W->bits;
+    const uint32_t mask = (1u << W->bits) - 1u;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        float *w = (float *)malloc(sizeof(float) * (size_t)K);
+        for (int64_t k = 0; k < K; ++k) {
+            const uint32_t q = (((const uint32_t *)W->w)[n * (K / per_word) + k / per_word] >> ((k % per_word) * W->bits)) & mask;
+            const float s = bf16_to_f32(W->scales[n * (K / W->group) + k / W->group]);
+            const float b = bf16_to_f32(W->biases[n * (K / W->group) + k / W->group]);
+            w[k] = rbf(fmaf((float)q, s, b));
+        }
+        for (int64_t r = 0; r < m; ++r) {
+            double acc = 0.0;
+            for (int64_t k = 0; k < K; ++k) acc += (double)bf16_to_f32(x[r * K + k]) * (double)w[k];
+            float a = (float)acc;
+            if (acc_out) acc_out[r * N + n] = a;
+            if (bias) a += bf16_to_f32(bias[n]);
+            y[r * N + n] = f32_to_bf16(a);
+        }
+        free(w);
+    }
 }
 
 /* --------------------------------------------------- dense decoder step */

@@ -432,3 +432,28 @@ def test_quantised_kv_store_and_attention(bits):
         p = np.exp(sc - sc.max())
         ref = (p / p.sum()) @ vd[kvh, :kv_len]
         assert np.all(np.abs(out[h] - ref) <= 2.0 ** -8 * np.abs(ref) + 1e-6)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_qgemm_with_weights_rounded_to_bf16(bits):
+    """Large-M form: w = T(s * q + b) per element, then a float64 matmul on those bf16 weights; a
+    one-hot activation row returns the rounded weights themselves; the rounding is visible (the
+    result differs from the exact-weight form on some outputs) and small (rel-L2 << 1e-2)."""
+    n, k, m = 48, 256, 5
+    W = make_qweight(90 + bits, n, k, bits)
+    x = normal_bf16(91, (m, k))
+    x[0] = 0
+    x[0, 17] = 0x3F80                                    # one-hot row: 1.0 at k = 17
+    y, acc = oracle.qgemm_bf16w(W, x, want_acc=True)
+    wq = oracle.bf16_to_f32(oracle.f32_to_bf16(oracle.dequantize(W)))   # dequantise, then one bf16 rounding
+    ref = oracle.bf16_to_f32(x).astype(np.float64) @ wq.astype(np.float64).T
+    assert np.allclose(acc, ref, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(y, oracle.f32_to_bf16(acc))
+    assert np.array_equal(y[0], oracle.f32_to_bf16(wq[:, 17].copy()))
+    exact = oracle.qgemm(W, x)
+    assert not np.array_equal(y, exact)
+    fe = oracle.bf16_to_f32(exact).astype(np.float64)
+    assert np.linalg.norm(oracle.bf16_to_f32(y) - fe) / np.linalg.norm(fe) < 5e-3
+    bias = normal_bf16(92, n)
+    yb = oracle.qgemm_bf16w(W, x, bias)
+    assert np.array_equal(yb, oracle.f32_to_bf16(acc + oracle.bf16_to_f32(bias)))

@@ -1,10 +1,11 @@
 """GPU parity of the multi-row quantised matmul on the matrix cores (G) against the CPU oracle.
 
-The oracle applies the single-row GEMV arithmetic row by row (exact affine dequantisation,
-fp32 accumulation, one round).  The reference's own multi-row path rounds every dequantised
-weight to bf16 before the multiply (MLX QuantizedBlockLoader, not vendored in the reference):
-that intermediate rounding is parity unpinned; both agree with the fp32 result far inside the
-rel-L2 <= 1e-2 bar.
+Up to 64 activation rows the kernel keeps the single-row GEMV arithmetic (exact affine
+dequantisation folded per group, fp32 accumulation, one round) and is compared with the oracle's
+row-by-row form.  From 65 rows up it dequantises every weight to bf16 before the multiply, as the
+reference's own multi-row path does (MLX QuantizedBlockLoader, not vendored in the reference), and
+is compared with the oracle's restatement of that form.  Both agree with the fp32 result far inside
+the rel-L2 <= 1e-2 bar.
 """
 import numpy as np
 import pytest
@@ -34,9 +35,23 @@ SHAPES = [
     (32, 1152, 896),
     (33, 256, 512),     # one row into the second activation tile
     (5, 2560, 9728),    # long K: split over many blocks
-    (70, 128, 128),     # three activation tiles, one weight block
+    (70, 128, 128),     # three activation tiles, one weight block (weights rounded to bf16 from here up)
     (1, 64, 64),
+    (64, 256, 320),     # last row count of the exact form; K not a multiple of the slab
+    (65, 256, 320),     # first row count of the bf16-weight form
+    (130, 512, 1024),   # two blocks of 128 rows, the second with two live rows
+    (200, 333, 2560),   # ragged N, several slabs
+    (512, 256, 512),
 ]
+
+
+def _reference(W, x, bias=None):
+    """(bits, unrounded sums) of the form the kernel uses for this row count."""
+    if x.shape[0] > 64:
+        return oracle.qgemm_bf16w(W, x, bias, want_acc=True)
+    ref = oracle.qgemm(W, x, bias)
+    acc = np.stack([oracle.linear_acc(W, x[r]) for r in range(x.shape[0])])
+    return ref, acc
 
 
 @pytest.mark.parametrize("bits", [4, 8])
@@ -45,18 +60,20 @@ def test_qgemm_matches_oracle(fk, m, n, k, bits):
     W = make_qweight(50 + bits, n, k, bits)
     x = normal_bf16(51, (m, k))
     got = _run(fk, W, x)
-    ref = oracle.qgemm(W, x)
+    ref, acc = _reference(W, x)
     for r in range(m):
-        _check(got[r], ref[r], oracle.linear_acc(W, x[r]), W, x[r])
+        _check(got[r], ref[r], acc[r], W, x[r])
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-def test_qgemm_group_128(fk, bits):
+@pytest.mark.parametrize("m", [9, 100])
+def test_qgemm_group_128(fk, bits, m):
     W = make_qweight(60, 384, 1024, bits, group=128)
-    x = normal_bf16(61, (9, 1024))
-    got, ref = _run(fk, W, x), oracle.qgemm(W, x)
-    for r in range(9):
-        _check(got[r], ref[r], oracle.linear_acc(W, x[r]), W, x[r])
+    x = normal_bf16(61, (m, 1024))
+    got = _run(fk, W, x)
+    ref, acc = _reference(W, x)
+    for r in range(m):
+        _check(got[r], ref[r], acc[r], W, x[r])
 
 
 def test_qgemm_bias_and_residual(fk):
