@@ -372,23 +372,18 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
     uint32_t tile = block_id, b0 = 0;
     bool first_batch = true;  // probe builds only: marks the first batch for FK_GEMV_STAMP
 
-    // Position of the batch after (tile, b0): the next batch of the tile or the first of the
-    // block's next tile.
-    uint32_t ntile = tile, nb0 = 0;
-    auto look_ahead = [&]() {
-        ntile = tile;
-        nb0 = b0 + POS;
+    // Consumes the batch held in cur* while the following batch streams into nxt*.
+    // Returns false once this block has no tile left.  (Two copies of this body,
+    // one per register set, cost code size but no register moves and no spills.)
+    auto step = [&](uint4(&cur)[kGemvUnroll], uint32_t(&csc)[kGemvUnroll], uint32_t(&cbi)[kGemvUnroll],
+                    uint4(&nxt)[kGemvUnroll], uint32_t(&nsc)[kGemvUnroll], uint32_t(&nbi)[kGemvUnroll]) -> bool {
+        uint32_t ntile = tile, nb0 = b0 + POS;
         if (nb0 >= seg_chunks) {
             ntile = tile + n_blocks;
             nb0 = 0;
         }
-        return ntile < a.n_tiles;
-    };
-    // Consumes the batch held in cur* (the batch at (tile, b0)); the caller has already
-    // requested the following one, if there is one, with no branch between the request and
-    // this code: the compiler can then count exactly how many younger loads are outstanding
-    // when it waits for cur*, and two batches stay in flight.
-    auto consume = [&](uint4(&cur)[kGemvUnroll], uint32_t(&csc)[kGemvUnroll], uint32_t(&cbi)[kGemvUnroll]) {
+        if (ntile < a.n_tiles) gemv_load_batch<KIND, NSEG, ARGS>(a, nxt, nsc, nbi, ntile, nb0);
+
         float p[kGemvUnroll];
 #pragma unroll
         for (int j = 0; j < kGemvUnroll; ++j) {
@@ -445,6 +440,7 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
         }
         tile = ntile;
         b0 = nb0;
+        return tile < a.n_tiles;
     };
 
     uint4 wb[kGemvUnroll];
@@ -453,20 +449,9 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
     stage_activations<KIND, ARGS>(a, xs, sx, scratch, xr, wr);
     FK_GEMV_STAMP(2);
     if (block_id >= a.n_tiles) return;
-    // Two register sets take turns (four copies of the body: no register moves, no spills).
     while (true) {
-        if (!look_ahead()) {
-            consume(wa, sa, ba);
-            break;
-        }
-        gemv_load_batch<KIND, NSEG, ARGS>(a, wb, sb, bb, ntile, nb0);
-        consume(wa, sa, ba);
-        if (!look_ahead()) {
-            consume(wb, sb, bb);
-            break;
-        }
-        gemv_load_batch<KIND, NSEG, ARGS>(a, wa, sa, ba, ntile, nb0);
-        consume(wb, sb, bb);
+        if (!step(wa, sa, ba, wb, sb, bb)) break;
+        if (!step(wb, sb, bb, wa, sa, ba)) break;
     }
     FK_GEMV_STAMP(4);
 }
