@@ -26,8 +26,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E published peak
 # HBM bytes per launch of the int4 gate/up kernel of the 4B-class model, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE (two counter runs of this script, each scaled by what the same counter reads for the plain
-# 256 MiB copies of --calibrate-copy: 1.99987 and 1.0).  Counters cannot be read from inside this process.
-GATEUP_Q4_4B_TRAFFIC_BYTES = 28563359
+# 256 MiB copies of --calibrate-copy: 1.99989 and 1.0).  Counters cannot be read from inside this process.
+GATEUP_Q4_4B_TRAFFIC_BYTES = 28590500
 
 
 def main() -> int:
