@@ -467,6 +467,14 @@ fk_status fk_sdpa_decode_rows(const uint16_t* q, const uint16_t* cache_k, const 
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_sdpa_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,
+                          uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                          uint32_t capacity, float scale, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_sdpa_prefill(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, head_dim, capacity, scale, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,
                                   size_t* partial_bytes, size_t* counter_bytes) {
     if (!partial_bytes || !counter_bytes || max_len == 0 || qk_dim < 8 || v_dim < 8)

@@ -420,6 +420,26 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
                             capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l);
 }
 
+// Q, K, V, out: causal attention of `rows` token rows (sdpa_prefill.rs:11-21).  The reference binds
+// kv_len, L and capacity as uniforms; here they are the parameters kv_len, rows and capacity,
+// because the grid depends on them.
+fk_status plan_sdpa_prefill_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 4));
+    const uint32_t n_heads = d.u("n_heads"), n_kv = d.u("n_kv"), dim = d.u("head_dim"), capacity = d.u("capacity");
+    const uint32_t rows = d.u("rows"), kv_len = d.u("kv_len");
+    if (n_heads == 0 || n_kv == 0 || dim == 0 || capacity == 0 || rows == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / head_dim / capacity / rows parameters missing");
+    const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)dim);  // sdpa_prefill.rs:52
+    FK_TRY(need_bytes(d, 0, (size_t)rows * n_heads * dim * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)n_kv * capacity * dim * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)n_kv * capacity * dim * 2));
+    FK_TRY(need_bytes(d, 3, (size_t)rows * n_heads * dim * 2));
+    rw->reads = {0, 1, 2};
+    rw->writes = {3};
+    return plan_sdpa_prefill(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<const uint16_t>(d, 2),
+                             arg_ptr<uint16_t>(d, 3), rows, kv_len, n_heads, n_kv, dim, capacity, scale, l);
+}
+
 // Q, K, V, [q_weight, k_weight], cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]
 // (one launch for the rope/store stage and the attention of a layer)
 fk_status plan_rope_store_sdpa(const Dispatch& d, Launch* l, SlotRW* rw) {
@@ -749,6 +769,7 @@ const Family kFamilies[] = {
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, false); }},
     {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
     {"fusekit_sdpa_decode", plan_sdpa_d},
+    {"fusekit_sdpa_prefill", plan_sdpa_prefill_d},
     {"fusekit_rope_store_sdpa_decode", plan_rope_store_sdpa},
     {"fusekit_rope_kv_cache_store_decode_q4",
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv_quant(d, l, rw, 4); }},

@@ -1,0 +1,295 @@
+// Causal attention for a group of token rows (chunked prompt prefill, multi-token
+// verification) on the gfx950 matrix cores.  Semantics of the reference's prefill kernel
+// (src/codegen/kernels/sdpa_prefill.rs:1-205): row l_q of the group sits at position
+// q_kv = (kv_len - L) + l_q and sees cache positions 0 .. q_kv; scores and softmax in
+// fp32, one rounding of the output.  The reference runs one threadgroup per (row, head)
+// with all scores in threadgroup memory (kv_len <= 4096); here the scores never leave
+// registers and kv_len is bounded by the cache only.
+//
+// One block = one query head x 32 consecutive rows; its four waves take the 64-position
+// steps of the visible range round-robin (wave w: steps w, w + 4, ...), each with its own
+// running (max, sum, output), and the four are merged once at the end in wave order.
+//
+// Per step a wave computes, with v_mfma_f32_32x32x16_bf16,
+//     S^T[kv, q] = K[kv, :] . Q[q, :]        A = K rows (read from the cache as they lie),
+//                                            B = Q rows (in registers for the whole kernel)
+// so that a lane owns ONE query (column q = lane % 32) and 32 of the 64 scores of it: the
+// softmax statistics are lane-local plus one exchange between the two half-waves, and the
+// rescale of the output accumulators is lane-local too, because the second product is
+//     O^T[d, q] += V^T[d, kv] . P^T[kv, q]   A = V^T, B = P^T = the score registers as they lie.
+// Only V needs a transposition: the step's V rows are written through LDS as [d][kv] (two
+// bytes at a time), in the order of kv that makes a lane's eight values of one matrix
+// instruction contiguous.  Both products run over an index (d for the first, kv for the
+// second) whose order inside the instruction is free as long as A and B agree, which is what
+// lets every global read be a contiguous run per lane.
+#include "fk_device.hpp"
+#include "fk_host.hpp"
+
+namespace fk {
+
+typedef __bf16 pf_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float pf_f32x16_t __attribute__((ext_vector_type(16)));
+typedef unsigned int pf_u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kPrefillBlock = 256;
+constexpr uint32_t kPrefillWaves = 4;
+constexpr uint32_t kPrefillRows = 32;    // query rows per block
+constexpr uint32_t kPrefillStep = 64;    // cache positions per wave step
+constexpr uint32_t kPrefillVtStride = kPrefillStep + 8;  // bf16 per row of the transposed V tile (rows stay 16-byte aligned)
+
+constexpr uint32_t prefill_lds_bytes(uint32_t d) {
+    const uint32_t vt = kPrefillWaves * d * kPrefillVtStride * 2u;
+    const uint32_t merge = 1024u + kPrefillWaves * kPrefillRows * (d + 4u) * 4u;
+    return vt > merge ? vt : merge;
+}
+
+struct SdpaPrefillArgs {
+    const uint16_t* q;    // [rows, n_heads, D]
+    const uint16_t* k;    // [n_kv, capacity, D]
+    const uint16_t* v;
+    uint16_t* out;        // [rows, n_heads, D]
+    uint32_t rows, kv_len, n_heads, heads_per_kv, capacity, row_tiles;
+    float scale2;         // softmax scale times log2(e)
+};
+
+__device__ __forceinline__ float other_half_max(float v) {
+    const pf_u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float both_halves_sum(float v) {
+    const pf_u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// LDS traffic of ONE wave with itself: the hardware runs a wave's LDS instructions in order,
+// the fence keeps the compiler from reordering them.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int D>
+__global__ __launch_bounds__(kPrefillBlock) void sdpa_prefill_kernel(const SdpaPrefillArgs a) {
+    constexpr int KB = D / 16;  // matrix steps over the head dimension (first product)
+    constexpr int DT = D / 32;  // 32-wide tiles of the output dimension (second product)
+    constexpr int VP = D / 8;   // 16-byte pieces of one V row
+    constexpr uint32_t VS = kPrefillVtStride;
+    extern __shared__ uint4 lds_raw[];
+
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, kb = lane >> 5, nl = lane & 31u;
+    const uint32_t head = blockIdx.x % a.n_heads;
+    const uint32_t tile = a.row_tiles - 1u - blockIdx.x / a.n_heads;  // the longest rows start first
+    const uint32_t kvh = head / a.heads_per_kv;
+    const uint32_t r0 = tile * kPrefillRows;
+    const uint32_t live = a.rows - r0 < kPrefillRows ? a.rows - r0 : kPrefillRows;
+    const uint32_t prior = a.kv_len - a.rows;      // positions in the cache before this group
+    const uint32_t kv_end = prior + r0 + live;     // positions the last live row sees
+    const uint32_t first_limit = prior + r0 + 1u;  // positions the first row sees
+    const uint32_t n_steps = (kv_end + kPrefillStep - 1u) / kPrefillStep;
+
+    uint16_t* vt = reinterpret_cast<uint16_t*>(lds_raw) + wave * ((uint32_t)D * VS);
+
+    // B operand of the first product: lane (q = nl, kb) holds d = kb * D/2 + 8 j + (0..7) for step j
+    const uint32_t rq = r0 + (nl < live ? nl : live - 1u);  // rows past the group repeat the last one; never stored
+    const uint32_t q_limit = prior + rq + 1u;               // positions this lane's query sees
+    uint4 qreg[KB];
+    {
+        const uint4* qp = reinterpret_cast<const uint4*>(a.q + ((size_t)rq * a.n_heads + head) * D + kb * (D / 2));
+#pragma unroll
+        for (int j = 0; j < KB; ++j) qreg[j] = qp[j];
+    }
+
+    const uint16_t* kbase = a.k + (size_t)kvh * a.capacity * D;
+    const uint16_t* vbase = a.v + (size_t)kvh * a.capacity * D;
+    uint4 kreg[2][KB], vreg[VP];
+    // Requests only (nothing here uses a loaded value).  Positions past the visible range read
+    // the last visible row instead: their scores are masked, and their V rows meet a zero
+    // probability, so they only need to be finite.
+    auto fetch_k = [&](uint32_t kv0) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            uint32_t kv = kv0 + (uint32_t)t * 32u + nl;
+            kv = kv < kv_end ? kv : kv_end - 1u;
+            const uint4* p = reinterpret_cast<const uint4*>(kbase + (size_t)kv * D + kb * (D / 2));
+#pragma unroll
+            for (int j = 0; j < KB; ++j) kreg[t][j] = p[j];
+        }
+    };
+    auto fetch_v = [&](uint32_t kv0) {
+        uint32_t kv = kv0 + lane;
+        kv = kv < kv_end ? kv : kv_end - 1u;
+        const uint4* p = reinterpret_cast<const uint4*>(vbase + (size_t)kv * D);
+#pragma unroll
+        for (int i = 0; i < VP; ++i) vreg[i] = p[i];
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's share (its half-wave's scores)
+    pf_f32x16_t oacc[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+
+    // Position of cache row `lane` inside a row of the transposed tile: bits 2 and 3 swapped, so
+    // that the rows a lane's score registers 8t .. 8t+7 stand for (8 u + 4 kb + e, u = 0..1,
+    // e = 0..3, inside a block of 16) are the eight contiguous entries 8 kb + 4 u + e.
+    const uint32_t vpos = (lane & ~12u) | ((lane & 4u) << 1) | ((lane & 8u) >> 1);
+
+    uint32_t step = wave;
+    if (step < n_steps) {
+        fetch_k(step * kPrefillStep);
+        fetch_v(step * kPrefillStep);
+    }
+    for (; step < n_steps; step += kPrefillWaves) {
+        const uint32_t kv0 = step * kPrefillStep;
+        const uint32_t kv_next = kv0 + kPrefillWaves * kPrefillStep;  // past the range on the last pass: clamped
+
+        pf_f32x16_t s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+#pragma unroll
+            for (int j = 0; j < KB; ++j)
+                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8_t, kreg[t][j]),
+                                                               __builtin_bit_cast(pf_bf16x8_t, qreg[j]), s[t], 0, 0, 0);
+        }
+        fetch_k(kv_next);
+
+        // V rows of this step -> LDS, transposed
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const uint32_t w4[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                vt[(uint32_t)(i * 8 + e) * VS + vpos] = (uint16_t)(e & 1 ? w4[e >> 1] >> 16 : w4[e >> 1] & 0xffffu);
+        }
+        fetch_v(kv_next);
+
+        // scores in base 2; register r of tile t is cache position kv0 + 32 t + r % 4 + 8 (r / 4) + 4 kb
+        float sv[32];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sv[t * 16 + r] = s[t][r] * a.scale2;
+        if (kv0 + kPrefillStep > first_limit) {  // some position of this step is in some row's future
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t kv = kv0 + (uint32_t)(t * 32 + r % 4 + 8 * (r / 4)) + 4u * kb;
+                    if (kv >= q_limit) sv[t * 16 + r] = -INFINITY;
+                }
+        }
+        float mt = sv[0];
+#pragma unroll
+        for (int i = 1; i < 32; ++i) mt = fmaxf(mt, sv[i]);
+        mt = other_half_max(mt);
+        const float m_new = fmaxf(m_run, mt);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen nothing yet
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+        uint32_t pk[16];
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float p0 = __builtin_amdgcn_exp2f(sv[2 * i] - m_ref), p1 = __builtin_amdgcn_exp2f(sv[2 * i + 1] - m_ref);
+            psum += p0 + p1;
+            pk[i] = pack_bf16(p0, p1);
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+            for (int i = 0; i < DT; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        }
+
+        wave_lds_fence();  // the transposed tile is complete
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint4 pb = make_uint4(pk[c * 4 + 0], pk[c * 4 + 1], pk[c * 4 + 2], pk[c * 4 + 3]);
+#pragma unroll
+            for (int i = 0; i < DT; ++i) {
+                const uint4 va = *reinterpret_cast<const uint4*>(vt + (uint32_t)(i * 32 + (int)nl) * VS + c * 16 + kb * 8);
+                oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8_t, va),
+                                                                  __builtin_bit_cast(pf_bf16x8_t, pb), oacc[i], 0, 0, 0);
+            }
+        }
+        wave_lds_fence();  // the tile has been read before the next pass overwrites it
+    }
+
+    // ---- merge of the four waves, in wave order --------------------------------------------
+    l_run = both_halves_sum(l_run);
+    __syncthreads();  // every wave has left its loop: the tiles' LDS is free
+    float* ml = reinterpret_cast<float*>(lds_raw);  // [wave][m x 32 | l x 32]
+    float* ob = ml + 256;                           // [wave][row][D + 4]
+    constexpr uint32_t OS = D + 4;
+    if (kb == 0) {
+        ml[wave * 64u + nl] = m_run;
+        ml[wave * 64u + 32u + nl] = l_run;
+    }
+    __syncthreads();
+    float mx = ml[nl];  // wave 0 always holds position 0, which every row sees: finite
+#pragma unroll
+    for (uint32_t w = 1; w < kPrefillWaves; ++w) mx = fmaxf(mx, ml[w * 64u + nl]);
+    float lsum = 0.f;
+#pragma unroll
+    for (uint32_t w = 0; w < kPrefillWaves; ++w) lsum += __builtin_amdgcn_exp2f(ml[w * 64u + nl] - mx) * ml[w * 64u + 32u + nl];
+    const float f = __builtin_amdgcn_exp2f(m_run - mx) / lsum;
+    // register r of tile i is output dimension 32 i + r % 4 + 8 (r / 4) + 4 kb of query nl
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<float4*>(ob + (wave * kPrefillRows + nl) * OS + (uint32_t)(i * 32 + 8 * g) + 4u * kb) =
+                make_float4(oacc[i][4 * g + 0] * f, oacc[i][4 * g + 1] * f, oacc[i][4 * g + 2] * f, oacc[i][4 * g + 3] * f);
+    __syncthreads();
+    for (uint32_t idx = threadIdx.x; idx < kPrefillRows * (uint32_t)VP; idx += kPrefillBlock) {
+        const uint32_t row = idx / (uint32_t)VP, piece = idx % (uint32_t)VP;
+        if (row >= live) continue;
+        float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t w = 0; w < kPrefillWaves; ++w) {
+            const float4 lo = *reinterpret_cast<const float4*>(ob + (w * kPrefillRows + row) * OS + piece * 8u);
+            const float4 hi = *reinterpret_cast<const float4*>(ob + (w * kPrefillRows + row) * OS + piece * 8u + 4u);
+            o[0] += lo.x; o[1] += lo.y; o[2] += lo.z; o[3] += lo.w;
+            o[4] += hi.x; o[5] += hi.y; o[6] += hi.z; o[7] += hi.w;
+        }
+        *reinterpret_cast<uint4*>(a.out + ((size_t)(r0 + row) * a.n_heads + head) * D + piece * 8u) =
+            make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+    }
+}
+
+fk_status plan_sdpa_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,
+                            uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                            uint32_t capacity, float scale, Launch* l) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!q || !cache_k || !cache_v || !out) return set_error(FK_ERR_INVALID, "sdpa_prefill: null pointer");
+    if (rows == 0 || kv_len < rows) return set_error(FK_ERR_INVALID, "sdpa_prefill: kv_len counts the rows of the group, so 1 <= rows <= kv_len");
+    if (kv_len > capacity) return set_error(FK_ERR_INVALID, "sdpa_prefill: kv_len exceeds the cache capacity");
+    if (n_heads == 0 || n_kv == 0 || n_heads % n_kv) return set_error(FK_ERR_INVALID, "sdpa_prefill: n_heads must be a multiple of n_kv");
+    if (head_dim != 64 && head_dim != 128)
+        return set_error(FK_ERR_UNSUPPORTED, "sdpa_prefill: head dimension 64 or 128 (use fk_sdpa_decode_rows for other shapes)");
+    if (((uintptr_t)q | (uintptr_t)cache_k | (uintptr_t)cache_v | (uintptr_t)out) & 15u)
+        return set_error(FK_ERR_INVALID, "sdpa_prefill: pointers must be 16-byte aligned");
+    SdpaPrefillArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.k = cache_k; a.v = cache_v; a.out = out;
+    a.rows = rows; a.kv_len = kv_len; a.n_heads = n_heads; a.heads_per_kv = n_heads / n_kv; a.capacity = capacity;
+    a.row_tiles = (rows + kPrefillRows - 1u) / kPrefillRows;
+    a.scale2 = scale * 1.4426950408889634f;
+    if ((uint64_t)a.row_tiles * n_heads > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "sdpa_prefill: too many rows");
+    l->func = head_dim == 64 ? reinterpret_cast<const void*>(&sdpa_prefill_kernel<64>) : reinterpret_cast<const void*>(&sdpa_prefill_kernel<128>);
+    l->grid = dim3(a.row_tiles * n_heads, 1, 1);
+    l->block = dim3(kPrefillBlock, 1, 1);
+    l->shmem = prefill_lds_bytes(head_dim);
+    if ((int)l->shmem > dev->max_dyn_lds) return set_error(FK_ERR_UNSUPPORTED, "sdpa_prefill: LDS tile does not fit");
+    if (l->shmem > 48 * 1024) FK_HIP(hipFuncSetAttribute(l->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l->shmem));
+    l->set_args(a);
+    return FK_OK;
+}
+
+}  // namespace fk

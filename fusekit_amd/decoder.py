@@ -325,7 +325,8 @@ class DecoderRuntime:
         """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
         active_m > 1 variants): the projections of up to 128 tokens share ONE pass over each weight
         matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form), attention is
-        causal inside the group.  Leaves the KV
+        causal inside the group (fk_sdpa_prefill for the bf16 cache with head dimension 64 or 128,
+        else the single-row kernel once per row).  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy
         first token.  Quantised projections only (the dense bf16 multi-row matmul is a library GEMM)."""
         c, w = self.cfg, self.w
@@ -375,8 +376,12 @@ class DecoderRuntime:
                 else:
                     native.qkv_rope_store_rows(b["q"], b["k"], b["v"], qn, kn, c.n_heads, c.n_kv, c.head_dim, c.head_dim,
                                                c.theta, c.eps, m, pos, c.capacity, self.cache_k[l], self.cache_v[l])
-                    native.sdpa_decode_rows(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + 1, c.n_heads,
-                                            c.n_kv, c.head_dim, c.head_dim, c.capacity, scale, b["part"], b["cnt"])
+                    if c.head_dim in (64, 128):  # causal attention of the whole group on the matrix cores
+                        native.sdpa_prefill(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + m, c.n_heads,
+                                            c.n_kv, c.head_dim, c.capacity, scale)
+                    else:
+                        native.sdpa_decode_rows(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + 1, c.n_heads,
+                                                c.n_kv, c.head_dim, c.head_dim, c.capacity, scale, b["part"], b["cnt"])
                 native.qgemm(w.mats[p + "self_attn.o_proj"], b["att"], m, None, b["x"], b["x2"], b["ws"])
                 native.rmsnorm_rows(b["x2"], w.vecs[p + "post_attention_layernorm"], c.eps, m, c.hidden, b["xn"])
                 native.qgemm_swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], b["xn"], m, c.swiglu_variant,

@@ -141,6 +141,26 @@ def case_sdpa(d, reps, length):
           flops=4 * n_heads * length * dim, pool=1)
 
 
+def case_sdpa_prefill(d, reps, rows, kv_len):
+    """Causal attention of `rows` rows whose last one sits at position kv_len - 1 (one layer's worth)."""
+    n_heads, n_kv, dim = 32, 8, 128
+    kv_bytes = 2 * n_kv * kv_len * dim * 2
+    pool = max(2, min(64, int(600e6 // kv_bytes) + 1))
+    q, out = _bf16(rows * n_heads * dim, 3), fk.DeviceBuffer(rows * n_heads * dim * 2)
+    tasks, keep = [], []
+    for i in range(pool):
+        ck, cv = _bf16(n_kv * kv_len * dim, 10 + 2 * i), _bf16(n_kv * kv_len * dim, 11 + 2 * i)
+        keep.append((ck, cv))
+        tasks.append(Dispatch("fusekit_sdpa_prefill_f0", [arg(q), arg(ck), arg(cv), arg(out)],
+                              {"n_heads": n_heads, "n_kv": n_kv, "head_dim": dim, "capacity": kv_len, "rows": rows,
+                               "kv_len": kv_len}))
+    nbytes = kv_bytes + 2 * rows * n_heads * dim * 2
+    # row r sees kv_len - rows + r + 1 positions: 4 flops per (head, position, dimension)
+    seen = rows * (kv_len - rows) + rows * (rows + 1) // 2
+    _emit(f"sdpa_prefill_rows{rows}_L{kv_len}", _time_graph(d, tasks, reps), nbytes, flops=4.0 * n_heads * seen * dim,
+          pool=pool)
+
+
 def case_moe(d, reps, bits=4):
     import numpy as np
     E, hidden, inter, top_k, layers = 64, 2048, 1408, 6, 2
@@ -228,6 +248,10 @@ CASES = {
     "sdpa_q8_4096": lambda d, r: case_sdpa_quant(d, r, 4096, 8),
     "sdpa_q4_32768": lambda d, r: case_sdpa_quant(d, r, 32768, 4),
     "sdpa_q8_32768": lambda d, r: case_sdpa_quant(d, r, 32768, 8),
+    "sdpa_prefill_128": lambda d, r: case_sdpa_prefill(d, r, 128, 128),
+    "sdpa_prefill_512": lambda d, r: case_sdpa_prefill(d, r, 128, 512),
+    "sdpa_prefill_4096": lambda d, r: case_sdpa_prefill(d, r, 128, 4096),
+    "sdpa_prefill_32768": lambda d, r: case_sdpa_prefill(d, r, 128, 32768),
     "moe_cfg5": lambda d, r: case_moe(d, r),
     "qgemm_8": lambda d, r: case_qgemm(d, r, 8),
     "qgemm_32": lambda d, r: case_qgemm(d, r, 32),

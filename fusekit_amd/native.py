@@ -335,6 +335,13 @@ def sdpa_decode_rows(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, qk_d
                                   C.c_uint32(capacity), C.c_float(scale), _ptr(partials), _ptr(counters), _ptr(stream)))
 
 
+def sdpa_prefill(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, head_dim, capacity, scale, stream=None):
+    """Causal attention of a group of rows on the matrix cores; kv_len counts the group's rows."""
+    check(lib.fk_sdpa_prefill(_ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(out), C.c_uint32(rows), C.c_uint32(kv_len),
+                              C.c_uint32(n_heads), C.c_uint32(n_kv), C.c_uint32(head_dim), C.c_uint32(capacity),
+                              C.c_float(scale), _ptr(stream)))
+
+
 def embed_lookup_decode(E, d_token, token, out_scale, x, stream=None):
     check(lib.fk_embed_lookup_decode(C.byref(E.c), _ptr(d_token), C.c_uint32(token), C.c_float(out_scale),
                                      _ptr(x), _ptr(stream)))

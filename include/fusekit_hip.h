@@ -304,6 +304,17 @@ fk_status fk_sdpa_decode_rows(const uint16_t *q, const uint16_t *cache_k, const 
                               uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim,
                               uint32_t v_dim, uint32_t capacity, float scale, float *partials, uint32_t *counters,
                               fk_stream s);
+/* Causal attention of a group of rows on the matrix cores.  Replaces
+ * src/codegen/kernels/sdpa_prefill.rs:1-205 with its buffer contract (:11-21): q and out
+ * [rows, n_heads, head_dim]; caches [n_kv, capacity, head_dim]; `kv_len` = positions in the cache
+ * INCLUDING the rows of this group (prior + rows); row r sits at position (kv_len - rows) + r and
+ * sees positions 0 .. that one.  fp32 scores and softmax (probabilities enter the second product
+ * as bf16), one rounding of the output.  No workspace; kv_len is bounded by the capacity only (the
+ * reference: 4096).  head_dim 64 or 128, bf16 cache; other shapes and the quantised cache go
+ * through fk_sdpa_decode_rows / fk_sdpa_decode_quant. */
+fk_status fk_sdpa_prefill(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v, uint16_t *out,
+                          uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                          uint32_t capacity, float scale, fk_stream s);
 
 /* E   x = T(embed[token] * out_scale), dense bf16 or MLX-affine table.  Replaces
  *     src/codegen/kernels/embed_lookup_decode.rs:17-108. */

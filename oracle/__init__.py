@@ -255,6 +255,15 @@ def sdpa_decode(q, cache_k, cache_v, n_heads, n_kv, qk_dim, v_dim, kv_len, capac
     return out
 
 
+def sdpa_prefill(q, cache_k, cache_v, rows, n_heads, n_kv, dim, kv_len, capacity, scale) -> np.ndarray:
+    """Causal attention of `rows` rows; kv_len counts them (row r sees kv_len - rows + r + 1 positions)."""
+    out = np.empty(rows * n_heads * dim, dtype=np.uint16)
+    _lib.fko_sdpa_prefill(_p(q, _u16p), _p(cache_k, _u16p), _p(cache_v, _u16p), C.c_int64(rows), C.c_int64(n_heads),
+                          C.c_int64(n_kv), C.c_int64(dim), C.c_uint32(kv_len), C.c_uint32(capacity), C.c_float(scale),
+                          _p(out, _u16p))
+    return out
+
+
 def embed_lookup(E: QWeight, token: int, out_scale: float = 1.0) -> np.ndarray:
     x = np.empty(E.k, dtype=np.uint16)
     _lib.fko_embed_lookup(C.byref(E.c), C.c_uint32(token), C.c_float(out_scale), _p(x, _u16p))

@@ -41,6 +41,11 @@
  *                                 quantiser's step of the pinned bf16 RoPE; only the
  *                                 addressed row written; attention = float64 softmax
  *                                 attention over the dequantised cache)
+ *   sdpa_prefill ................ pinned (every row = the pinned sdpa_decode over the positions
+ *                                 it sees, to one bf16 step: the reference normalises the
+ *                                 scores before the product with V here and after it there;
+ *                                 float64 causal softmax attention in numpy; row 0 of a fresh
+ *                                 group returns V[0]; later cache rows never influence a row)
  *   hand-derived known answers .. tests/golden/known_answers.json
  *   MLX-internal accumulation order, Metal fast::cos/sin/exp bit patterns:
  *                                 parity unpinned (cannot be observed here;
@@ -570,6 +575,45 @@ FKO_API void fko_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const u
             for (uint32_t j = 0; j < kv_len; ++j)
                 o += (double)s[j] * (double)bf16_to_f32(cache_v[(kvh * (int64_t)capacity + j) * v_dim + d]);
             out[h * v_dim + d] = f32_to_bf16((float)(o / l));
+        }
+        free(s);
+    }
+}
+
+/* Causal attention of a group of L rows (src/codegen/kernels/sdpa_prefill.rs): row l_q sits at
+ * q_kv = (kv_len - L) + l_q and positions kv > q_kv are masked (:95, :109); scores dot * SCALE
+ * (:104-124); max, exp, sum, then the scores are normalised BEFORE the product with V
+ * (:128-181); out = T(sum_kv score * v) (:183-199).  q, out [L, n_heads, dim]. */
+FKO_API void fko_sdpa_prefill(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v, int64_t rows,
+                              int64_t n_heads, int64_t n_kv, int64_t dim, uint32_t kv_len, uint32_t capacity,
+                              float scale, uint16_t *out) {
+    const int64_t per_kv = n_heads / n_kv;
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t it = 0; it < rows * n_heads; ++it) {
+        const int64_t l_q = it / n_heads, h = it % n_heads, kvh = h / per_kv;
+        const uint32_t q_kv = (kv_len - (uint32_t)rows) + (uint32_t)l_q;
+        const uint16_t *qr = q + (l_q * n_heads + h) * dim;
+        float *s = (float *)malloc(sizeof(float) * (size_t)(q_kv + 1));
+        float m = -INFINITY;
+        for (uint32_t j = 0; j <= q_kv; ++j) { /* kv > q_kv: exp(-inf) = 0, contributes nothing */
+            const uint16_t *kr = cache_k + (kvh * (int64_t)capacity + j) * dim;
+            double dot = 0.0;
+            for (int64_t d = 0; d < dim; ++d) dot += (double)bf16_to_f32(qr[d]) * (double)bf16_to_f32(kr[d]);
+            s[j] = (float)dot * scale;
+            m = s[j] > m ? s[j] : m;
+        }
+        double l = 0.0;
+        for (uint32_t j = 0; j <= q_kv; ++j) {
+            s[j] = expf(s[j] - m);
+            l += s[j];
+        }
+        const float inv = 1.0f / (float)l;
+        for (uint32_t j = 0; j <= q_kv; ++j) s[j] *= inv;
+        for (int64_t d = 0; d < dim; ++d) {
+            double o = 0.0;
+            for (uint32_t j = 0; j <= q_kv; ++j)
+                o += (double)s[j] * (double)bf16_to_f32(cache_v[(kvh * (int64_t)capacity + j) * dim + d]);
+            out[(l_q * n_heads + h) * dim + d] = f32_to_bf16((float)o);
         }
         free(s);
     }

@@ -251,6 +251,48 @@ def test_sdpa_against_float64_attention_and_gqa_mapping():
                           oracle.f32_to_bf16(out))
 
 
+def test_sdpa_prefill_rows_are_causal_decode_attention():
+    n_heads, n_kv, D, cap = 6, 2, 64, 96
+    f = lambda a: oracle.bf16_to_f32(a).astype(np.float64)
+    for rows, kv_len in ((1, 1), (5, 5), (7, 40), (33, 70)):
+        q = normal_bf16(10 + rows, rows * n_heads * D)
+        ck, cv = normal_bf16(2, n_kv * cap * D), normal_bf16(3, n_kv * cap * D)
+        got = oracle.sdpa_prefill(q, ck, cv, rows, n_heads, n_kv, D, kv_len, cap, D ** -0.5).reshape(rows, n_heads, D)
+        K, V, Q = f(ck).reshape(n_kv, cap, D), f(cv).reshape(n_kv, cap, D), f(q).reshape(rows, n_heads, D)
+        for r in range(rows):
+            sees = kv_len - rows + r + 1                          # sdpa_prefill.rs:95: q_kv = (kv_len - L) + l_q, kv <= q_kv
+            # the pinned single-row attention over exactly those positions; the two differ only in where
+            # the division by the sum of exponentials happens -> at most one bf16 step apart
+            dec = oracle.sdpa_decode(q.reshape(rows, -1)[r], ck, cv, n_heads, n_kv, D, D, sees, cap, D ** -0.5).reshape(n_heads, D)
+            a, b = oracle.bf16_to_f32(got[r]), oracle.bf16_to_f32(dec)
+            assert np.mean(got[r] != dec) < 0.02 and np.allclose(a, b, rtol=2 ** -7, atol=1e-6)
+            for h in range(n_heads):                              # and an independent float64 statement
+                kvh = h // (n_heads // n_kv)
+                s = K[kvh, :sees] @ Q[r, h] * D ** -0.5
+                p = np.exp(s - s.max()); p /= p.sum()
+                assert np.allclose(a[h], p @ V[kvh, :sees], rtol=2 ** -7, atol=2e-3)
+        if kv_len == rows:                                        # a fresh group: row 0 sees one position -> v_0 bit for bit
+            assert np.array_equal(got[0], np.repeat(cv.reshape(n_kv, cap, D)[:, 0], n_heads // n_kv, axis=0))
+        # positions after a row's own never reach it: poison everything row r must not see
+        r = rows // 2
+        sees = kv_len - rows + r + 1
+        ck2, cv2 = ck.copy().reshape(n_kv, cap, D), cv.copy().reshape(n_kv, cap, D)
+        ck2[:, sees:] = 0x7FC0; cv2[:, sees:] = 0x7FC0
+        poisoned = oracle.sdpa_prefill(q, ck2.ravel(), cv2.ravel(), rows, n_heads, n_kv, D, kv_len, cap, D ** -0.5)
+        assert np.array_equal(poisoned.reshape(rows, n_heads, D)[: r + 1], got[: r + 1])
+    # identical keys: uniform probabilities, the output is the mean of the visible V rows
+    rows, kv_len = 4, 9
+    q = normal_bf16(5, rows * n_heads * D)
+    ck = np.tile(normal_bf16(6, D), n_kv * cap)
+    cv = normal_bf16(7, n_kv * cap * D)
+    got = oracle.bf16_to_f32(oracle.sdpa_prefill(q, ck, cv, rows, n_heads, n_kv, D, kv_len, cap, D ** -0.5)).reshape(rows, n_heads, D)
+    V = f(cv).reshape(n_kv, cap, D)
+    for r in range(rows):
+        sees = kv_len - rows + r + 1
+        for h in range(n_heads):
+            assert np.allclose(got[r, h], V[h // (n_heads // n_kv), :sees].mean(axis=0), rtol=2 ** -7, atol=2e-3)
+
+
 # ---------------------------------------------------------------- embed / lm head / argmax
 def test_embed_lm_head_argmax():
     E = make_qweight(1, 50, 128, 4)
