@@ -213,12 +213,12 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
           note="two kernels: MFMA main + split-k reduction")
 
 
-def case_prefill(d, reps, prompt_len=512, rows_per_pass=128):
+def case_prefill(d, reps, prompt_len=512, rows_per_pass=512, capacity=1024):
     """Chunked prefill of the 4B-class model: `rows_per_pass` prompt tokens per pass over the weights."""
     import time
     import numpy as np
     from .decoder import DENSE_4B, DecoderConfig, DecoderRuntime, DecoderWeights
-    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=1024, swiglu_variant=1)
+    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=capacity, swiglu_variant=1)
     W = DecoderWeights.random_init(cfg, seed=0)
     rt = DecoderRuntime(cfg, W, dispatcher=d)
     prompt = np.random.Generator(np.random.PCG64(0)).integers(0, cfg.vocab, prompt_len).tolist()
@@ -252,6 +252,9 @@ CASES = {
     "sdpa_prefill_512": lambda d, r: case_sdpa_prefill(d, r, 128, 512),
     "sdpa_prefill_4096": lambda d, r: case_sdpa_prefill(d, r, 128, 4096),
     "sdpa_prefill_32768": lambda d, r: case_sdpa_prefill(d, r, 128, 32768),
+    "sdpa_prefill_r32_4096": lambda d, r: case_sdpa_prefill(d, r, 32, 4096),
+    "sdpa_prefill_r512_512": lambda d, r: case_sdpa_prefill(d, r, 512, 512),
+    "sdpa_prefill_r512_4096": lambda d, r: case_sdpa_prefill(d, r, 512, 4096),
     "moe_cfg5": lambda d, r: case_moe(d, r),
     "qgemm_8": lambda d, r: case_qgemm(d, r, 8),
     "qgemm_32": lambda d, r: case_qgemm(d, r, 32),
@@ -259,6 +262,10 @@ CASES = {
     "qgemm_512": lambda d, r: case_qgemm(d, r, 512),
     "prefill_4b_32": lambda d, r: case_prefill(d, r, 512, 32),
     "prefill_4b": lambda d, r: case_prefill(d, r),
+    "prefill_4b_128": lambda d, r: case_prefill(d, r, 512, 128),
+    "prefill_4b_256": lambda d, r: case_prefill(d, r, 512, 256),
+    "prefill_4b_4096_tokens": lambda d, r: case_prefill(d, r, 4096, 512, 4608),
+    "prefill_4b_4096_tokens_1024": lambda d, r: case_prefill(d, r, 4096, 1024, 4608),
 }
 
 

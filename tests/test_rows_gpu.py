@@ -81,20 +81,20 @@ def test_sdpa_rows_are_causal_single_row_calls(fk, kv_len, rows):
         assert rel_l2(got[r], oracle.bf16_to_f32(ref)) <= 1e-2
 
 
-@pytest.mark.parametrize("bits,prompt_len", [(4, 45), (8, 7)])
-def test_batched_prefill_matches_token_by_token(fk, bits, prompt_len):
+@pytest.mark.parametrize("bits,prompt_len,rows_per_pass", [(4, 45, 128), (8, 7, 128), (4, 300, 256), (4, 333, 100)])
+def test_batched_prefill_matches_token_by_token(fk, bits, prompt_len, rows_per_pass):
     """prefill_rows (32 tokens per weight pass on the matrix cores) leaves the caches of the
     token-by-token path and continues with the same tokens.  The two paths sum in different
     orders, so the caches agree to rounding flips and the greedy continuation is compared with
     the oracle's margins in view."""
     from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
-    cfg = DecoderConfig(n_layers=3, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=2000, capacity=128,
+    cfg = DecoderConfig(n_layers=3, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=2000, capacity=512,
                         bits=bits, qk_norm=True, qkv_bias=(bits == 8), swiglu_variant=2)
     W = DecoderWeights.random_init(cfg, seed=41)
     prompt = rng(42).integers(0, cfg.vocab, prompt_len).tolist()
     a, b = DecoderRuntime(cfg, W), DecoderRuntime(cfg, W)
     first_a = a.prefill(prompt)
-    first_b = b.prefill_rows(prompt)
+    first_b = b.prefill_rows(prompt, rows_per_pass=rows_per_pass)
     for l in range(cfg.n_layers):
         for ca, cb_ in ((a.cache_k[l], b.cache_k[l]), (a.cache_v[l], b.cache_v[l])):
             ga, gb = ca.to_numpy(np.uint16), cb_.to_numpy(np.uint16)

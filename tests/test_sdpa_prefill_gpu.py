@@ -54,6 +54,21 @@ def test_head_layouts(fk, n_heads, n_kv, D):
     _case(fk, 45, 333, n_heads, n_kv, D, 512, seed=7)
 
 
+@pytest.mark.parametrize("rows,kv_len", [(65, 65), (129, 129), (200, 200), (256, 256), (300, 900), (512, 512), (512, 1536), (1000, 1000)])
+@pytest.mark.parametrize("n_heads,n_kv,D", [(8, 2, 128), (6, 3, 64)])
+def test_large_groups_few_heads(fk, rows, kv_len, n_heads, n_kv, D):
+    """Many rows, few heads: still the form whose waves split the positions (one block per 32 rows)."""
+    _case(fk, rows, kv_len, n_heads, n_kv, D, 1600, seed=13)
+
+
+@pytest.mark.parametrize("rows,kv_len", [(129, 129), (200, 200), (300, 900), (512, 512), (512, 1536), (640, 700)])
+@pytest.mark.parametrize("n_heads,n_kv,D", [(64, 8, 128), (48, 12, 64)])
+def test_large_groups_many_heads(fk, rows, kv_len, n_heads, n_kv, D):
+    """Enough (head, 32-row) tiles that the first form would need several rounds over the CUs: the
+    library takes the form with one block per 128 rows, whose waves share K and V through LDS."""
+    _case(fk, rows, kv_len, n_heads, n_kv, D, 1600, seed=17)
+
+
 def test_first_row_of_fresh_group_is_v0(fk):
     q, ck, cv, got = _case(fk, 40, 40, 32, 8, 128, 64, seed=11)
     v0 = cv.reshape(8, 64, 128)[:, 0]  # softmax over the one visible position is 1
