@@ -183,6 +183,11 @@ fk_status fk_event_elapsed_ms(fk_event start, fk_event stop, float* ms) {
     return FK_OK;
 }
 
+fk_status fk_set_gemm_library_rows(uint32_t rows) {
+    set_gemm_library_rows(rows);
+    return FK_OK;
+}
+
 fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks) {
     g_gemv_policy.rows_per_tile = rows_per_tile;
     g_gemv_policy.grid_blocks = grid_blocks;
@@ -296,7 +301,8 @@ fk_status fk_qgemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, uint32_t 
 fk_status fk_qgemm(const fk_weight* W, const uint16_t* x, uint32_t m, const uint16_t* bias, const uint16_t* residual,
                    uint16_t* y, void* workspace, fk_stream s) {
     Launch main, reduce;
-    FK_TRY(plan_qgemm(W, x, m, bias, residual, y, workspace, &main, &reduce));
+    FK_TRY(plan_qgemm(W, x, m, bias, residual, y, workspace, &main, &reduce));  // validates the arguments for both routes
+    if (qgemm_takes_library(m)) return run_qgemm_library(W, nullptr, x, m, bias, residual, 0, y, workspace, (hipStream_t)s);
     FK_TRY(run_launch(main, (hipStream_t)s));
     return run_launch(reduce, (hipStream_t)s);
 }
@@ -305,6 +311,7 @@ fk_status fk_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16
                           uint16_t* out, void* workspace, fk_stream s) {
     Launch gate, up, reduce;
     FK_TRY(plan_qgemm_swiglu(Wg, Wu, x, m, variant, out, workspace, &gate, &up, &reduce));
+    if (qgemm_takes_library(m)) return run_qgemm_library(Wg, Wu, x, m, nullptr, nullptr, variant, out, workspace, (hipStream_t)s);
     FK_TRY(run_launch(gate, (hipStream_t)s));
     FK_TRY(run_launch(up, (hipStream_t)s));
     return run_launch(reduce, (hipStream_t)s);

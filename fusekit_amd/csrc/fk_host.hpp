@@ -96,6 +96,15 @@ fk_status plan_qgemm(const fk_weight* W, const uint16_t* x, uint32_t M, const ui
 fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16_t* x, uint32_t M, int variant,
                             uint16_t* out, void* workspace, Launch* gate, Launch* up, Launch* reduce);
 
+// Large row counts, direct calls only: dequantise to bf16 once, library GEMM, the same epilogue.
+void set_gemm_library_rows(uint32_t rows);  // 0: never
+bool qgemm_takes_library(uint32_t m);
+size_t qgemm_library_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+void plan_qgemm_epilogue(const float* p0, const float* p1, const uint16_t* bias, const uint16_t* res, uint16_t* y,
+                         uint32_t M, uint32_t N, uint32_t ksplit, int variant, Launch* out);
+fk_status run_qgemm_library(const fk_weight* W0, const fk_weight* W1, const uint16_t* x, uint32_t m, const uint16_t* bias,
+                            const uint16_t* res, int variant, uint16_t* y, void* workspace, hipStream_t s);
+
 // RoPE / per-head RMSNorm / KV-cache store (one wave per head).
 struct RopeArgs {
     uint16_t* q;             // [n_q, head_dim] in place, or null

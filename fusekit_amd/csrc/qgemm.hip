@@ -139,8 +139,9 @@ __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
         for (int i = 0; i < XPT; ++i) {
             const uint32_t idx = threadIdx.x + (uint32_t)i * kQgemmBlock, m = idx / S8, k8 = idx % S8;
             uint4 v = (m < mt && k8 < (slab_k >> 3)) ? xq[i] : make_uint4(0, 0, 0, 0);
-            if constexpr (KIND == W_Q4) {
-                // nibble pairing of q4_word_dot: (x0,x2) (x4,x6) (x1,x3) (x5,x7)
+            if constexpr (KIND == W_Q4 && !DEQ) {
+                // nibble pairing of q4_word_dot: (x0,x2) (x4,x6) (x1,x3) (x5,x7); the dequantising
+                // form pairs its codes in element order instead and takes x as it lies
                 v = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
                                (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
             }
@@ -186,15 +187,22 @@ __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
                 for (int j = 0; j < MF; ++j) {
                     uint4 bw;
                     if constexpr (DEQ) {
-                        // eight codes of this lane in the order the staged activations expect:
-                        // int4 (n0, n2) (n4, n6) (n1, n3) (n5, n7), int8 in element order
+                        // eight codes of this lane in element order: int4 word j holds them as nibbles
+                        // (even ones in the bytes of `lo`, odd ones in those of `hi`), int8 as bytes
                         const uint32_t lo = KIND == W_Q4 ? (wd[j] & 0x0F0F0F0Fu) : wd[(2 * j) & 3];
                         const uint32_t hi = KIND == W_Q4 ? ((wd[j] >> 4) & 0x0F0F0F0Fu) : wd[(2 * j + 1) & 3];
                         auto dq = [&](uint32_t byte) { return fmaf((float)byte, sf, bf); };
-                        bw.x = pack_bf16(dq(lo & 0xffu), dq((lo >> 8) & 0xffu));
-                        bw.y = pack_bf16(dq((lo >> 16) & 0xffu), dq(lo >> 24));
-                        bw.z = pack_bf16(dq(hi & 0xffu), dq((hi >> 8) & 0xffu));
-                        bw.w = pack_bf16(dq((hi >> 16) & 0xffu), dq(hi >> 24));
+                        if constexpr (KIND == W_Q4) {
+                            bw.x = pack_bf16(dq(lo & 0xffu), dq(hi & 0xffu));
+                            bw.y = pack_bf16(dq((lo >> 8) & 0xffu), dq((hi >> 8) & 0xffu));
+                            bw.z = pack_bf16(dq((lo >> 16) & 0xffu), dq((hi >> 16) & 0xffu));
+                            bw.w = pack_bf16(dq(lo >> 24), dq(hi >> 24));
+                        } else {
+                            bw.x = pack_bf16(dq(lo & 0xffu), dq((lo >> 8) & 0xffu));
+                            bw.y = pack_bf16(dq((lo >> 16) & 0xffu), dq(lo >> 24));
+                            bw.z = pack_bf16(dq(hi & 0xffu), dq((hi >> 8) & 0xffu));
+                            bw.w = pack_bf16(dq((hi >> 16) & 0xffu), dq(hi >> 24));
+                        }
                     } else if constexpr (KIND == W_Q4) {
                         const uint32_t even = wd[j] & 0x0F0F0F0Fu, odd = (wd[j] >> 4) & 0x0F0F0F0Fu;
                         bw.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false));
@@ -397,6 +405,12 @@ void plan_reduce(const float* p0, const float* p1, const uint16_t* bias, const u
 
 }  // namespace
 
+// the epilogue of a product whose fp32 sums are complete (the library route)
+void plan_qgemm_epilogue(const float* p0, const float* p1, const uint16_t* bias, const uint16_t* res, uint16_t* y,
+                         uint32_t M, uint32_t N, uint32_t ksplit, int variant, Launch* out) {
+    plan_reduce(p0, p1, bias, res, y, M, N, ksplit, variant, out);
+}
+
 fk_status qgemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group, size_t* bytes) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
@@ -405,6 +419,11 @@ fk_status qgemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t gro
     FK_TRY(qgemm_shape(dev, M, N, K, group, 4, &s4));
     FK_TRY(qgemm_shape(dev, M, N, K, group, 8, &s8));
     *bytes = (size_t)(s4.ksplit > s8.ksplit ? s4.ksplit : s8.ksplit) * M * N * sizeof(float);
+    // direct calls with many rows may take the library route, which also parks the dequantised matrix here
+    if (qgemm_takes_library(M)) {
+        const size_t lib = qgemm_library_workspace_bytes(M, N, K);
+        if (lib > *bytes) *bytes = lib;
+    }
     return FK_OK;
 }
 

@@ -321,10 +321,11 @@ class DecoderRuntime:
         nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
         return nxt[-1]
 
-    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 512) -> int:
+    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 4096) -> int:
         """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
-        active_m > 1 variants): the projections of up to `rows_per_pass` (<= 1024) tokens share ONE pass over each weight
-        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form), attention is
+        active_m > 1 variants): the projections of up to `rows_per_pass` (<= 4096) tokens share ONE pass over each weight
+        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form, from 256 rows
+        up as a dequantisation to bf16 followed by a library GEMM), attention is
         causal inside the group (fk_sdpa_prefill for the bf16 cache with head dimension 64 or 128,
         else the single-row kernel once per row).  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy
@@ -335,13 +336,14 @@ class DecoderRuntime:
         prompt = list(prompt)
         if start_offset + len(prompt) > c.capacity:
             raise ValueError("prompt exceeds the KV-cache capacity")
-        R = max(1, min(rows_per_pass, 1024))
+        # buffers follow the prompt (next power of two), so a short prompt does not allocate for 4096 rows
+        R = max(1, min(rows_per_pass, 4096, 1 << max(5, (len(prompt) - 1).bit_length())))
         if getattr(self, "_rows_R", 0) != R:
             self._rows_R = R
             # the split of k differs between the kernel forms (<= 32, <= 64, more rows) and with the
             # number of 128-row tiles; the last pass of a prompt may have any row count up to R
             ws = max(native.qgemm_workspace_bytes(m, n, k, c.group)
-                     for m in {R} | {v for v in (896, 768, 640, 512, 384, 256, 128, 64, 32) if v < R}
+                     for m in {R} | {v for v in (*range(512, 4096, 128), 384, 256, 128, 64, 32) if v < R}
                      for n, k in ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
             # only the single-row attention kernel (quantised cache, other head dimensions) needs a workspace
             pb, cb = (native.sdpa_workspace_bytes(c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.capacity)

@@ -213,7 +213,7 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
           note="two kernels: MFMA main + split-k reduction")
 
 
-def case_prefill(d, reps, prompt_len=512, rows_per_pass=512, capacity=1024):
+def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024):
     """Chunked prefill of the 4B-class model: `rows_per_pass` prompt tokens per pass over the weights."""
     import time
     import numpy as np
@@ -266,6 +266,7 @@ CASES = {
     "prefill_4b_256": lambda d, r: case_prefill(d, r, 512, 256),
     "prefill_4b_4096_tokens": lambda d, r: case_prefill(d, r, 4096, 512, 4608),
     "prefill_4b_4096_tokens_1024": lambda d, r: case_prefill(d, r, 4096, 1024, 4608),
+    "prefill_4b_4096_tokens_4096": lambda d, r: case_prefill(d, r, 4096, 4096, 4608),
 }
 
 

@@ -342,6 +342,11 @@ def sdpa_prefill(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, head_dim
                               C.c_float(scale), _ptr(stream)))
 
 
+def set_gemm_library_rows(rows: int):
+    """Row count from which qgemm / qgemm_swiglu take the dequantise + library-GEMM route (0: never)."""
+    check(lib.fk_set_gemm_library_rows(C.c_uint32(rows)))
+
+
 def embed_lookup_decode(E, d_token, token, out_scale, x, stream=None):
     check(lib.fk_embed_lookup_decode(C.byref(E.c), _ptr(d_token), C.c_uint32(token), C.c_float(out_scale),
                                      _ptr(x), _ptr(stream)))

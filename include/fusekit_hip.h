@@ -180,7 +180,8 @@ fk_status fk_routed_qmv_reduce(const uint16_t *h, uint32_t n_h_rows, const fk_we
  *     admission src/codegen/kernels/mod.rs:1442-1475) and its small-M shared-stream
  *     GEMVs (fusekit_qmv_wide_impl, src/codegen/msl.rs:461-546).  Any m >= 1; bits 4
  *     or 8, group 64 or 128.  workspace: fk_qgemm_workspace_bytes() bytes of device
- *     memory (fp32 split-k partial sums); the SwiGLU pair needs twice that.
+ *     memory (fp32 split-k partial sums; from fk_set_gemm_library_rows() rows up the fp32
+ *     sums and the matrix dequantised to bf16, N*K*2 bytes); the SwiGLU pair needs twice that.
  *     fk_qgemm_swiglu: out[m, N] = SwiGLU(x @ Wg^T, x @ Wu^T) with the rounding variant
  *     as in fk_gateup_swiglu (the reference's qMM epilogue is variant 2,
  *     src/codegen/msl.rs:2441-2449). */
@@ -495,6 +496,10 @@ fk_status fk_decode_chunk_host_loop(fk_handle h, uint32_t graph_id, const fk_dec
 /* Launch-geometry overrides for experiments (0 = library policy): rows per
  * tile and grid blocks of the streaming GEMV.  Process-wide. */
 fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks);
+/* Row count from which fk_qgemm / fk_qgemm_swiglu dequantise the matrix to bf16 once and hand the
+ * product to rocBLAS (opened on first use; absent: the fused kernel is kept).  Default 256; 0 = never.
+ * Set it BEFORE sizing workspaces: fk_qgemm_workspace_bytes covers the route that will be taken. */
+fk_status fk_set_gemm_library_rows(uint32_t rows);
 
 #pragma GCC visibility pop
 #ifdef __cplusplus

@@ -103,6 +103,54 @@ def test_qgemm_swiglu(fk, variant):
         _check_swiglu(got[r], oracle.gateup_swiglu(x[r], None, 0.0, Wg, Wu, variant), x[r], Wg, Wu, variant)
 
 
+@pytest.mark.parametrize("route", ["kernel", "library"])
+@pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 128)])
+@pytest.mark.parametrize("m,n,k", [(512, 333, 2560), (700, 1152, 896), (300, 512, 4864)])
+def test_qgemm_many_rows_both_routes(fk, m, n, k, bits, group, route):
+    """From 256 rows direct calls dequantise the matrix to bf16 once and take the library GEMM; the
+    fused kernel stays reachable (and is what a graph node runs).  Same arithmetic, same oracle form,
+    with bias and residual in the epilogue."""
+    fk.set_gemm_library_rows(0 if route == "kernel" else 256)
+    try:
+        W = make_qweight(70 + bits, n, k, bits, group=group)
+        x = normal_bf16(71, (m, k))
+        bias, res = normal_bf16(72, n), normal_bf16(73, (m, n))
+        got = _run(fk, W, x)
+        ref, acc = _reference(W, x)
+        for r in range(0, m, 7):
+            _check(got[r], ref[r], acc[r], W, x[r])
+        got = _run(fk, W, x, bias=bias, res=res)
+        full = acc + oracle.bf16_to_f32(bias)[None, :] + oracle.bf16_to_f32(res)
+        want = oracle.f32_to_bf16(full.astype(np.float32))
+        for r in range(0, m, 7):
+            _check(got[r], want[r], full[r], W, x[r])
+    finally:
+        fk.set_gemm_library_rows(256)
+
+
+@pytest.mark.parametrize("route", ["kernel", "library"])
+def test_qgemm_swiglu_many_rows_both_routes(fk, route):
+    m, hidden, inter, variant = 512, 896, 1216, 2
+    fk.set_gemm_library_rows(0 if route == "kernel" else 256)
+    try:
+        Wg, Wu = make_qweight(76, inter, hidden, 4), make_qweight(77, inter, hidden, 4)
+        x = normal_bf16(78, (m, hidden))
+        out = fk.DeviceBuffer(2 * m * inter)
+        ws = fk.DeviceBuffer(2 * fk.qgemm_workspace_bytes(m, inter, hidden, 64))
+        fk.qgemm_swiglu(to_device(fk, Wg), to_device(fk, Wu), _dev(fk, x), m, variant, out, ws)
+        got = out.to_numpy(np.uint16, (m, inter))
+        _, g = oracle.qgemm_bf16w(Wg, x, None, want_acc=True)
+        _, u = oracle.qgemm_bf16w(Wu, x, None, want_acc=True)
+        want = np.array([[oracle.swiglu_scalar(float(a), float(b), variant) for a, b in zip(g[r], u[r])] for r in range(0, m, 37)],
+                        dtype=np.uint16)
+        sel = got[::37]
+        gf, wf = oracle.bf16_to_f32(sel).astype(np.float64), oracle.bf16_to_f32(want).astype(np.float64)
+        assert np.linalg.norm(gf - wf) / np.linalg.norm(wf) <= 1e-2
+        assert np.mean(sel != want) <= 0.05          # fp32 summation order may cross a bf16 rounding edge
+    finally:
+        fk.set_gemm_library_rows(256)
+
+
 def test_qgemm_rows_agree_with_gemv(fk):
     """Every row of the multi-row result lies within one rounding flip of the single-row kernel."""
     W = make_qweight(69, 1024, 2048, 4)
