@@ -300,6 +300,11 @@ fk_status fk_qgemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, uint32_t 
 
 fk_status fk_qgemm(const fk_weight* W, const uint16_t* x, uint32_t m, const uint16_t* bias, const uint16_t* residual,
                    uint16_t* y, void* workspace, fk_stream s) {
+    if (W && W->bits == 16) {  // dense bf16 weights: the plain library GEMM with this library's epilogue
+        if (!x || !y || !workspace) return set_error(FK_ERR_INVALID, "fk_qgemm: null activation, output or workspace");
+        if (!gemm_library_available()) return set_error(FK_ERR_UNSUPPORTED, "fk_qgemm: bf16 weights need rocBLAS (librocblas.so.5 not found)");
+        return run_qgemm_library(W, nullptr, x, m, bias, residual, 0, y, workspace, (hipStream_t)s);
+    }
     Launch main, reduce;
     FK_TRY(plan_qgemm(W, x, m, bias, residual, y, workspace, &main, &reduce));  // validates the arguments for both routes
     if (qgemm_takes_library(m)) return run_qgemm_library(W, nullptr, x, m, bias, residual, 0, y, workspace, (hipStream_t)s);
@@ -309,6 +314,13 @@ fk_status fk_qgemm(const fk_weight* W, const uint16_t* x, uint32_t m, const uint
 
 fk_status fk_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16_t* x, uint32_t m, int variant,
                           uint16_t* out, void* workspace, fk_stream s) {
+    if (Wg && Wu && Wg->bits == 16 && Wu->bits == 16) {
+        if (!x || !out || !workspace) return set_error(FK_ERR_INVALID, "fk_qgemm_swiglu: null activation, output or workspace");
+        if (Wg->n != Wu->n || Wg->k != Wu->k) return set_error(FK_ERR_INVALID, "fk_qgemm_swiglu: gate and up need the same shape");
+        if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, "fk_qgemm_swiglu: variant must be 0, 1 or 2");
+        if (!gemm_library_available()) return set_error(FK_ERR_UNSUPPORTED, "fk_qgemm_swiglu: bf16 weights need rocBLAS (librocblas.so.5 not found)");
+        return run_qgemm_library(Wg, Wu, x, m, nullptr, nullptr, variant, out, workspace, (hipStream_t)s);
+    }
     Launch gate, up, reduce;
     FK_TRY(plan_qgemm_swiglu(Wg, Wu, x, m, variant, out, workspace, &gate, &up, &reduce));
     if (qgemm_takes_library(m)) return run_qgemm_library(Wg, Wu, x, m, nullptr, nullptr, variant, out, workspace, (hipStream_t)s);
@@ -445,7 +457,8 @@ fk_status fk_embed_lookup_rows(const fk_weight* E, const uint32_t* d_tokens, uin
 fk_status fk_qkv_rope_store_rows(uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_norm,
                                  const uint16_t* k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                  uint32_t rope_dims, float theta, float eps, uint32_t rows, uint32_t offset,
-                                 uint32_t capacity, uint16_t* cache_k, uint16_t* cache_v, fk_stream s) {
+                                 uint32_t capacity, uint16_t* cache_k, uint16_t* cache_v, const float* rope_tab,
+                                 fk_stream s) {
     if (rows == 0) return set_error(FK_ERR_INVALID, "fk_qkv_rope_store_rows: zero rows");
     RopeArgs a;
     memset(&a, 0, sizeof(a));
@@ -458,8 +471,15 @@ fk_status fk_qkv_rope_store_rows(uint16_t* q, const uint16_t* k, const uint16_t*
     a.eps = eps; a.base_log2 = theta_log2(theta);
     a.rope_on = rope_dims ? 1u : 0u;
     a.rows = rows;
+    a.rope_tab = rope_dims ? rope_tab : nullptr;
     Launch l;
     FK_TRY(plan_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_rope_table_rows(float* tab, uint32_t rope_dims, float theta, uint32_t offset, uint32_t rows, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_rope_table(tab, rope_dims, theta_log2(theta), offset, rows, &l));
     return run_launch(l, (hipStream_t)s);
 }
 

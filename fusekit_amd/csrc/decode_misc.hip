@@ -27,7 +27,13 @@ __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
         const uint32_t h = b - a.n_q - a.n_kv;
         const uint16_t* src = a.v + ((size_t)tr * a.n_kv + h) * a.v_dim;
         uint16_t* dst = a.cache_v + ((size_t)h * a.capacity + row) * a.v_dim;
-        for (uint32_t d = lane; d < a.v_dim; d += kWave) dst[d] = src[d];
+        if ((a.v_dim & 1u) == 0) {  // rows are then 4-byte aligned
+            const uint32_t* s2 = reinterpret_cast<const uint32_t*>(src);
+            uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+            for (uint32_t d = lane; d < a.v_dim / 2u; d += kWave) d2[d] = s2[d];
+        } else {
+            for (uint32_t d = lane; d < a.v_dim; d += kWave) dst[d] = src[d];
+        }
         return;
     }
     const bool is_q = b < a.n_q;
@@ -37,8 +43,43 @@ __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
     uint16_t* dst = is_q ? a.q + ((size_t)tr * a.n_q + h) * dim : a.cache_k + ((size_t)h * a.capacity + row) * dim;
     const uint16_t* nw = is_q ? a.q_norm : a.k_norm;
 
+    const float* tab = a.rope_tab ? a.rope_tab + (size_t)tr * a.rope_dims : nullptr;
     head_transform(src, dst, nw, dim, a.rope_on ? a.rope_dims : 0u, pos, a.base_log2, a.eps, nw != nullptr || !is_q,
-                   lane);
+                   lane, tab);
+}
+
+// The rotary table of a prompt pass: without it every (head, row) wave evaluates exp2 in double and
+// sincosf per pair; the table is filled once per pass and serves every layer.  (The kernel's time at
+// 4096 rows, 92 us, is that of its short dependent chains of 2-byte accesses, one wave per head and
+// row; four heads per block or a loop over heads inside a wave were slower, 103 and 109 us.)
+struct RopeTabArgs {
+    float* tab;
+    uint32_t half, offset, rows;
+    float base_log2;
+};
+__global__ __launch_bounds__(256) void rope_table_kernel(const RopeTabArgs a) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= a.rows * a.half) return;
+    const uint32_t r = i / a.half, d = i - r * a.half;
+    float cs, sn;
+    rope_cos_sin(d, a.half, a.offset + r, a.base_log2, cs, sn);
+    a.tab[2 * (size_t)i] = cs;
+    a.tab[2 * (size_t)i + 1] = sn;
+}
+
+fk_status plan_rope_table(float* tab, uint32_t rope_dims, float base_log2, uint32_t offset, uint32_t rows, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!tab || rows == 0) return set_error(FK_ERR_INVALID, "rope table: null table or zero rows");
+    if (rope_dims == 0 || rope_dims % 2) return set_error(FK_ERR_INVALID, "rope table: rope_dims must be even and non-zero");
+    if ((uint64_t)rows * (rope_dims / 2) > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "rope table: too large");
+    RopeTabArgs a{tab, rope_dims / 2, offset, rows, base_log2};
+    out->func = reinterpret_cast<const void*>(&rope_table_kernel);
+    out->grid = dim3((rows * (rope_dims / 2) + 255u) / 256u, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
 }
 
 fk_status plan_rope_store(const RopeArgs& in, Launch* out) {

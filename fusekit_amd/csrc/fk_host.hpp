@@ -99,6 +99,8 @@ fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint
 // Large row counts, direct calls only: dequantise to bf16 once, library GEMM, the same epilogue.
 void set_gemm_library_rows(uint32_t rows);  // 0: never
 bool qgemm_takes_library(uint32_t m);
+bool gemm_library_available();
+size_t qgemm_library_sums_bytes(uint32_t m, uint32_t n, uint32_t k);
 size_t qgemm_library_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
 void plan_qgemm_epilogue(const float* p0, const float* p1, const uint16_t* bias, const uint16_t* res, uint16_t* y,
                          uint32_t M, uint32_t N, uint32_t ksplit, int variant, Launch* out);
@@ -122,8 +124,12 @@ struct RopeArgs {
     float eps, base_log2;
     uint32_t rope_on;  // 0: plain store of K (no rotation)
     uint32_t rows;     // active token rows (0 = 1): row r is position offset + r and reads q/k/v row r
+    const float* rope_tab;  // optional [rows][rope_dims/2] (cos, sin) as plan_rope_table fills it, for position offset + r
 };
 fk_status plan_rope_store(const RopeArgs& in, Launch* out);
+// (cos, sin) of every rotary pair at positions offset .. offset + rows - 1: the values the
+// rope/store kernel would compute itself, filled once per prompt pass for all layers and heads.
+fk_status plan_rope_table(float* tab, uint32_t rope_dims, float base_log2, uint32_t offset, uint32_t rows, Launch* out);
 
 // Quantised KV cache (mlx-lm QuantizedKVCache layout): packed uint32 [n_kv, capacity, dim*bits/32],
 // scales / biases bf16 [n_kv, capacity, dim/group].

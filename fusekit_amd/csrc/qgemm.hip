@@ -279,6 +279,37 @@ struct QgemmReduceArgs {
     int variant;
 };
 
+// Four consecutive outputs per thread (N a multiple of 4: 16-byte loads of the sums, one 8-byte
+// store); same order of additions per element as the scalar form below.
+__global__ __launch_bounds__(256) void qgemm_reduce4_kernel(const QgemmReduceArgs a) {
+    const uint32_t total = a.M * a.N, i = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (i >= total) return;
+    float s0[4] = {0.f, 0.f, 0.f, 0.f}, s1[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t ks = 0; ks < a.ksplit; ++ks) {
+        const float4 v = *reinterpret_cast<const float4*>(a.p0 + (size_t)ks * total + i);
+        s0[0] += v.x; s0[1] += v.y; s0[2] += v.z; s0[3] += v.w;
+        if (a.p1) {
+            const float4 u = *reinterpret_cast<const float4*>(a.p1 + (size_t)ks * total + i);
+            s1[0] += u.x; s1[1] += u.y; s1[2] += u.z; s1[3] += u.w;
+        }
+    }
+    uint32_t o[4];
+    if (a.p1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = swiglu_bits(s0[e], s1[e], a.variant, 1.0f);
+    } else {
+        const uint32_t n = i % a.N;  // i and N are multiples of 4: the four share a row
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float v = s0[e];
+            if (a.bias) v += bf16_bits_to_f32(a.bias[n + e]);
+            if (a.res) v += bf16_bits_to_f32(a.res[i + e]);
+            o[e] = f32_to_bf16_bits(v);
+        }
+    }
+    *reinterpret_cast<uint2*>(a.y + i) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+}
+
 __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const QgemmReduceArgs a) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x, total = a.M * a.N;
     if (i >= total) return;
@@ -396,8 +427,10 @@ void plan_reduce(const float* p0, const float* p1, const uint16_t* bias, const u
     QgemmReduceArgs r;
     r.p0 = p0; r.p1 = p1; r.bias = bias; r.res = res; r.y = y;
     r.M = M; r.N = N; r.ksplit = ksplit; r.variant = variant;
-    out->func = reinterpret_cast<const void*>(&qgemm_reduce_kernel);
-    out->grid = dim3((M * N + 255u) / 256u, 1, 1);
+    const bool by4 = N % 4u == 0 && ((reinterpret_cast<uintptr_t>(p0) | reinterpret_cast<uintptr_t>(p1)) & 15u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(y) & 7u) == 0;
+    out->func = by4 ? reinterpret_cast<const void*>(&qgemm_reduce4_kernel) : reinterpret_cast<const void*>(&qgemm_reduce_kernel);
+    out->grid = dim3(by4 ? (M * N / 4u + 255u) / 256u : (M * N + 255u) / 256u, 1, 1);
     out->block = dim3(256, 1, 1);
     out->shmem = 0;
     out->set_args(r);
@@ -414,16 +447,20 @@ void plan_qgemm_epilogue(const float* p0, const float* p1, const uint16_t* bias,
 fk_status qgemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group, size_t* bytes) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
+    if (group == 0) {  // dense bf16 weights: the library route's fp32 sums only
+        if (M == 0 || N == 0 || K == 0) return set_error(FK_ERR_INVALID, "qgemm: empty shape");
+        *bytes = qgemm_library_sums_bytes(M, N, K);
+        return FK_OK;
+    }
     // the split depends on the kernel form (4- or 8-bit codes): size for the larger of the two
     QgemmShape s4, s8;
     FK_TRY(qgemm_shape(dev, M, N, K, group, 4, &s4));
     FK_TRY(qgemm_shape(dev, M, N, K, group, 8, &s8));
     *bytes = (size_t)(s4.ksplit > s8.ksplit ? s4.ksplit : s8.ksplit) * M * N * sizeof(float);
-    // direct calls with many rows may take the library route, which also parks the dequantised matrix here
-    if (qgemm_takes_library(M)) {
-        const size_t lib = qgemm_library_workspace_bytes(M, N, K);
-        if (lib > *bytes) *bytes = lib;
-    }
+    // direct calls with many rows may take the library route, which also parks the dequantised matrix
+    // here; dense bf16 weights always take it and need the fp32 sums only
+    const size_t lib = qgemm_takes_library(M) ? qgemm_library_workspace_bytes(M, N, K) : qgemm_library_sums_bytes(M, N, K);
+    if (lib > *bytes) *bytes = lib;
     return FK_OK;
 }
 

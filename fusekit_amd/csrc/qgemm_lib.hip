@@ -170,9 +170,12 @@ fk_status library_product_split(const uint16_t* wb, const uint16_t* x, uint32_t 
 }
 
 bool shape_ok(const fk_weight* W, uint32_t m) {
+    if (!W || !W->w || m == 0 || W->n == 0 || W->k == 0) return false;
+    if ((uint64_t)m * W->n > 0x7fffffffull || W->n > 0x7fffffffu || W->k > 0x7fffffffu) return false;
+    if (W->bits == 16) return W->k % 8u == 0;  // dense bf16 rows, 16-byte aligned
     const uint32_t vpl = W->bits == 4 ? 32u : 16u;
-    return (W->bits == 4 || W->bits == 8) && (W->group == 64 || W->group == 128) && W->k % W->group == 0 && W->k % vpl == 0 &&
-           (uint64_t)m * W->n <= 0x7fffffffull && W->n <= 0x7fffffffu && W->k <= 0x7fffffffu;
+    return (W->bits == 4 || W->bits == 8) && W->scales && W->biases && (W->group == 64 || W->group == 128) &&
+           W->k % W->group == 0 && W->k % vpl == 0;
 }
 
 }  // namespace
@@ -185,9 +188,17 @@ bool qgemm_takes_library(uint32_t m) {
     return rocblas_ready();
 }
 
+bool gemm_library_available() {
+    std::lock_guard<std::mutex> lk(g_rb.mu);
+    return rocblas_ready();
+}
+
+size_t qgemm_library_sums_bytes(uint32_t m, uint32_t n, uint32_t k) {
+    return (size_t)library_split(m, n, k) * m * n * sizeof(float);  // one fp32 buffer per k slice
+}
+
 size_t qgemm_library_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
-    // fp32 sums (one buffer per k slice), then the dequantised matrix
-    return (size_t)library_split(m, n, k) * m * n * sizeof(float) + (size_t)n * k * 2u;
+    return qgemm_library_sums_bytes(m, n, k) + (size_t)n * k * 2u;  // the sums, then the dequantised matrix
 }
 
 // workspace: [(m x N) fp32 sums per matrix or k slice][N x K bf16 dequantised matrix, reused by the second matrix in stream order]
@@ -200,10 +211,21 @@ fk_status run_qgemm_library(const fk_weight* W0, const fk_weight* W1, const uint
     const uint32_t split = W1 ? 1u : library_split(m, W0->n, W0->k);
     float* p0 = static_cast<float*>(workspace);
     float* p1 = W1 ? p0 + sums : nullptr;
-    uint16_t* wb = reinterpret_cast<uint16_t*>(p0 + (W1 ? 2u : split) * sums);
+    uint16_t* scratch = reinterpret_cast<uint16_t*>(p0 + (W1 ? 2u : split) * sums);
     Launch l;
-    FK_TRY(plan_dequant(dev, W0, wb, &l));
-    FK_TRY(run_launch(l, s));
+    // a dense bf16 matrix is used where it lies; a quantised one is dequantised into the workspace
+    auto bf16_rows = [&](const fk_weight* W, const uint16_t** out) -> fk_status {
+        if (W->bits == 16) {
+            *out = static_cast<const uint16_t*>(W->w);
+            return FK_OK;
+        }
+        FK_TRY(plan_dequant(dev, W, scratch, &l));
+        FK_TRY(run_launch(l, s));
+        *out = scratch;
+        return FK_OK;
+    };
+    const uint16_t* wb = nullptr;
+    FK_TRY(bf16_rows(W0, &wb));
     if (split > 1) {
         FK_TRY(library_product_split(wb, x, m, W0->n, W0->k, split, p0, s));
         Launch reduce;
@@ -214,8 +236,7 @@ fk_status run_qgemm_library(const fk_weight* W0, const fk_weight* W1, const uint
         return library_product(wb, x, m, W0->n, W0->k, nullptr, y, res, s);
     FK_TRY(library_product(wb, x, m, W0->n, W0->k, p0, nullptr, nullptr, s));
     if (W1) {
-        FK_TRY(plan_dequant(dev, W1, wb, &l));
-        FK_TRY(run_launch(l, s));
+        FK_TRY(bf16_rows(W1, &wb));  // reuses the scratch: the first product is ahead of it in stream order
         FK_TRY(library_product(wb, x, m, W1->n, W1->k, p1, nullptr, nullptr, s));
     }
     Launch reduce;

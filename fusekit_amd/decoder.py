@@ -329,10 +329,8 @@ class DecoderRuntime:
         causal inside the group (fk_sdpa_prefill for the bf16 cache with head dimension 64 or 128,
         else the single-row kernel once per row).  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy
-        first token.  Quantised projections only (the dense bf16 multi-row matmul is a library GEMM)."""
+        first token.  Dense bf16 weights take the library GEMM for every row count."""
         c, w = self.cfg, self.w
-        if c.bits == 16:
-            return self.prefill(prompt, start_offset)
         prompt = list(prompt)
         if start_offset + len(prompt) > c.capacity:
             raise ValueError("prompt exceeds the KV-cache capacity")
@@ -342,7 +340,7 @@ class DecoderRuntime:
             self._rows_R = R
             # the split of k differs between the kernel forms (<= 32, <= 64, more rows) and with the
             # number of 128-row tiles; the last pass of a prompt may have any row count up to R
-            ws = max(native.qgemm_workspace_bytes(m, n, k, c.group)
+            ws = max(native.qgemm_workspace_bytes(m, n, k, 0 if c.bits == 16 else c.group)
                      for m in {R} | {v for v in (*range(512, 4096, 128), 384, 256, 128, 64, 32) if v < R}
                      for n, k in ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
             # only the single-row attention kernel (quantised cache, other head dimensions) needs a workspace
@@ -352,7 +350,8 @@ class DecoderRuntime:
                 tok=DeviceBuffer(4 * R), x=DeviceBuffer(R * c.hidden * 2), x2=DeviceBuffer(R * c.hidden * 2),
                 xn=DeviceBuffer(R * c.hidden * 2), q=DeviceBuffer(R * c.n_q * 2), k=DeviceBuffer(R * c.n_kvd * 2),
                 v=DeviceBuffer(R * c.n_kvd * 2), att=DeviceBuffer(R * c.n_q * 2), mid=DeviceBuffer(R * c.inter * 2),
-                ws=DeviceBuffer(2 * ws), part=DeviceBuffer(max(pb, 4) * R), cnt=native.zeros(max(cb, 4) * R))
+                ws=DeviceBuffer(2 * ws), part=DeviceBuffer(max(pb, 4) * R), cnt=native.zeros(max(cb, 4) * R),
+                rope=DeviceBuffer(R * c.head_dim * 4))
         b = self._rows
         emb = w.mats["embed_tokens"]
         head = w.mats.get("lm_head", emb)
@@ -363,6 +362,7 @@ class DecoderRuntime:
             m = len(chunk)
             b["tok"].upload(np.asarray(chunk, np.uint32))
             native.embed_lookup_rows(emb, b["tok"], m, 1.0, b["x"])
+            native.rope_table_rows(b["rope"], c.head_dim, c.theta, pos, m)  # once per pass, for every layer and head
             for l in range(c.n_layers):
                 p = f"layers.{l}."
                 native.rmsnorm_rows(b["x"], w.vecs[p + "input_layernorm"], c.eps, m, c.hidden, b["xn"])
@@ -373,14 +373,15 @@ class DecoderRuntime:
                 kn = w.vecs.get(p + "self_attn.k_norm") if c.qk_norm else None
                 if c.kv_bits:
                     native.qkv_rope_store_rows(b["q"], None, None, qn, None, c.n_heads, 0, c.head_dim, c.head_dim,
-                                               c.theta, c.eps, m, pos, c.capacity, None, None)
+                                               c.theta, c.eps, m, pos, c.capacity, None, None, rope_tab=b["rope"])
                     native.kv_cache_store_quant(b["k"], b["v"], kn, c.n_kv, c.head_dim, c.head_dim, c.theta, c.eps,
                                                 None, pos, m, self.cache_k[l], self.cache_v[l])
                     native.sdpa_decode_quant(b["q"], self.cache_k[l], self.cache_v[l], b["att"], None, pos + 1,
                                              pos + m, m, c.n_heads, scale, b["part"], b["cnt"])
                 else:
                     native.qkv_rope_store_rows(b["q"], b["k"], b["v"], qn, kn, c.n_heads, c.n_kv, c.head_dim, c.head_dim,
-                                               c.theta, c.eps, m, pos, c.capacity, self.cache_k[l], self.cache_v[l])
+                                               c.theta, c.eps, m, pos, c.capacity, self.cache_k[l], self.cache_v[l],
+                                               rope_tab=b["rope"])
                     if c.head_dim in (64, 128):  # causal attention of the whole group on the matrix cores
                         native.sdpa_prefill(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + m, c.n_heads,
                                             c.n_kv, c.head_dim, c.capacity, scale)

@@ -321,11 +321,17 @@ def embed_lookup_rows(E, d_tokens, rows, out_scale, x, stream=None):
 
 
 def qkv_rope_store_rows(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope_dims, theta, eps, rows, offset,
-                        capacity, cache_k, cache_v, stream=None):
+                        capacity, cache_k, cache_v, stream=None, rope_tab=None):
     check(lib.fk_qkv_rope_store_rows(
         _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), C.c_uint32(n_heads), C.c_uint32(n_kv),
         C.c_uint32(head_dim), C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), C.c_uint32(rows),
-        C.c_uint32(offset), C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v), _ptr(stream)))
+        C.c_uint32(offset), C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v), _ptr(rope_tab), _ptr(stream)))
+
+
+def rope_table_rows(tab, rope_dims, theta, offset, rows, stream=None):
+    """(cos, sin) of every rotary pair at positions offset .. offset + rows - 1, [rows][rope_dims/2][2] fp32."""
+    check(lib.fk_rope_table_rows(_ptr(tab), C.c_uint32(rope_dims), C.c_float(theta), C.c_uint32(offset), C.c_uint32(rows),
+                                 _ptr(stream)))
 
 
 def sdpa_decode_rows(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, qk_dim, v_dim, capacity, scale, partials,

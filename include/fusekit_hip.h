@@ -179,9 +179,11 @@ fk_status fk_routed_qmv_reduce(const uint16_t *h, uint32_t n_h_rows, const fk_we
  *     reference's qMM-T / NAX tile path (src/codegen/msl.rs:2318-2440, 3821-4330;
  *     admission src/codegen/kernels/mod.rs:1442-1475) and its small-M shared-stream
  *     GEMVs (fusekit_qmv_wide_impl, src/codegen/msl.rs:461-546).  Any m >= 1; bits 4
- *     or 8, group 64 or 128.  workspace: fk_qgemm_workspace_bytes() bytes of device
+ *     or 8, group 64 or 128; bits 16 (dense bf16 rows, k a multiple of 8): the plain
+ *     library GEMM (rocBLAS) with the same epilogue, direct calls only.  workspace: fk_qgemm_workspace_bytes() bytes of device
  *     memory (fp32 split-k partial sums; from fk_set_gemm_library_rows() rows up the fp32
- *     sums and the matrix dequantised to bf16, N*K*2 bytes); the SwiGLU pair needs twice that.
+ *     sums and the matrix dequantised to bf16, N*K*2 bytes; group 0 = dense bf16 weights: the
+ *     fp32 sums only); the SwiGLU pair needs twice that.
  *     fk_qgemm_swiglu: out[m, N] = SwiGLU(x @ Wg^T, x @ Wu^T) with the rounding variant
  *     as in fk_gateup_swiglu (the reference's qMM epilogue is variant 2,
  *     src/codegen/msl.rs:2441-2449). */
@@ -293,11 +295,16 @@ fk_status fk_rmsnorm_rows(const uint16_t *x, const uint16_t *w, float eps, uint3
                           uint16_t *y, fk_stream s);
 fk_status fk_embed_lookup_rows(const fk_weight *E, const uint32_t *d_tokens, uint32_t rows, float out_scale,
                                uint16_t *x, fk_stream s);
-/* q [rows, n_heads, head_dim] in place; k, v [rows, n_kv, head_dim] -> cache rows (offset + r) % capacity */
+/* q [rows, n_heads, head_dim] in place; k, v [rows, n_kv, head_dim] -> cache rows (offset + r) % capacity.
+ * rope_tab (may be NULL): [rows][rope_dims/2] (cos, sin) pairs for positions offset .. offset + rows - 1 as
+ * fk_rope_table_rows fills them -- the very values the kernel computes without it, so the results are
+ * bit-identical; a prompt pass fills the table once and every layer reuses it. */
+fk_status fk_rope_table_rows(float *tab, uint32_t rope_dims, float theta, uint32_t offset, uint32_t rows, fk_stream s);
 fk_status fk_qkv_rope_store_rows(uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *q_norm,
                                  const uint16_t *k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                  uint32_t rope_dims, float theta, float eps, uint32_t rows, uint32_t offset,
-                                 uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
+                                 uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v, const float *rope_tab,
+                                 fk_stream s);
 /* Row r attends to the first kv_len + r cache positions (causal inside the group); q and out are
  * [rows, n_heads, dim].  Workspace: rows times the sizes of fk_sdpa_workspace_bytes(max_len =
  * kv_len + rows - 1); counters zero before the first launch. */

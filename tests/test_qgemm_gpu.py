@@ -151,6 +151,21 @@ def test_qgemm_swiglu_many_rows_both_routes(fk, route):
         fk.set_gemm_library_rows(256)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 333, 256), (100, 1152, 896), (512, 256, 4864)])
+def test_qgemm_dense_bf16_weights(fk, m, n, k):
+    """bits = 16: the plain library GEMM (fp32 accumulate) with this library's epilogue."""
+    W = make_qweight(80, n, k, 16)
+    x = normal_bf16(81, (m, k))
+    bias, res = normal_bf16(82, n), normal_bf16(83, (m, n))
+    got = _run(fk, W, x)
+    for r in range(0, m, 5):
+        _check(got[r], oracle.qgemv(W, x[r]), oracle.linear_acc(W, x[r]), W, x[r])
+    got = _run(fk, W, x, bias=bias, res=res)
+    for r in range(0, m, 5):
+        full = oracle.linear_acc(W, x[r]) + oracle.bf16_to_f32(bias) + oracle.bf16_to_f32(res[r])
+        _check(got[r], oracle.f32_to_bf16(full.astype(np.float32)), full, W, x[r])
+
+
 def test_qgemm_rows_agree_with_gemv(fk):
     """Every row of the multi-row result lies within one rounding flip of the single-row kernel."""
     W = make_qweight(69, 1024, 2048, 4)
@@ -169,7 +184,9 @@ def test_qgemm_rejects(fk):
     y = fk.DeviceBuffer(2 * 2 * 64)
     ws = fk.DeviceBuffer(1 << 16)
     with pytest.raises(fk.FusekitError):
-        fk.qgemm(to_device(fk, make_qweight(1, 64, 128, 16)), x, 2, None, None, y, ws)       # dense weights
+        fk.qgemm(to_device(fk, make_qweight(1, 64, 132, 16)), _dev(fk, normal_bf16(1, (2, 132))), 2, None, None, y, ws)  # dense rows not 16-byte aligned
+    with pytest.raises(fk.InvalidArgument):
+        fk.qgemm(to_device(fk, make_qweight(1, 64, 128, 16)), x, 2, None, None, y, None)     # dense weights need the workspace too
     with pytest.raises(fk.FusekitError):
         fk.qgemm(to_device(fk, make_qweight(1, 64, 128, 4, group=32)), x, 2, None, None, y, ws)
     with pytest.raises(fk.InvalidArgument):

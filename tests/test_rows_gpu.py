@@ -57,6 +57,17 @@ def test_rope_store_rows(fk, norm):
     gk = ck.to_numpy(np.uint16)
     assert np.array_equal(gk == 0, rk == 0)
     _close(gk, rk, ulp_bar=2.0)
+    # with the rotary table of the pass (filled once, reused by every layer): the same bits
+    tab = fk.DeviceBuffer(rows * dim * 4)
+    fk.rope_table_rows(tab, dim, 1e4, off, rows)
+    dq2, ck2, cv2 = _dev(fk, q), fk.zeros(n_kv * cap * dim * 2), fk.zeros(n_kv * cap * dim * 2)
+    fk.qkv_rope_store_rows(dq2, _dev(fk, k), _dev(fk, v), _dev(fk, qn), _dev(fk, kn), n_heads, n_kv, dim, dim, 1e4, 1e-6,
+                           rows, off, cap, ck2, cv2, rope_tab=tab)
+    assert np.array_equal(dq2.to_numpy(np.uint16, (rows, n_heads * dim)), got_q)
+    assert np.array_equal(ck2.to_numpy(np.uint16), gk) and np.array_equal(cv2.to_numpy(np.uint16), rv)
+    t = tab.to_numpy(np.float32, (rows, dim // 2, 2)).astype(np.float64)
+    ang = (off + np.arange(rows))[:, None] * (1e4 ** (-np.arange(dim // 2) / (dim // 2)))[None, :]
+    assert np.allclose(t[..., 0], np.cos(ang), atol=2e-6) and np.allclose(t[..., 1], np.sin(ang), atol=2e-6)
 
 
 @pytest.mark.parametrize("kv_len,rows", [(1, 5), (60, 8), (500, 32)])
@@ -81,7 +92,8 @@ def test_sdpa_rows_are_causal_single_row_calls(fk, kv_len, rows):
         assert rel_l2(got[r], oracle.bf16_to_f32(ref)) <= 1e-2
 
 
-@pytest.mark.parametrize("bits,prompt_len,rows_per_pass", [(4, 45, 128), (8, 7, 128), (4, 300, 256), (4, 333, 100)])
+@pytest.mark.parametrize("bits,prompt_len,rows_per_pass", [(4, 45, 128), (8, 7, 128), (4, 300, 256), (4, 333, 100), (16, 45, 128),
+                                                          (16, 300, 4096)])
 def test_batched_prefill_matches_token_by_token(fk, bits, prompt_len, rows_per_pass):
     """prefill_rows (32 tokens per weight pass on the matrix cores) leaves the caches of the
     token-by-token path and continues with the same tokens.  The two paths sum in different
