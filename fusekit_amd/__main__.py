@@ -6,6 +6,10 @@
                                          token ids out; no tokenizer is bundled)
   export-random --out DIR [--bits 4] [--layers 2] ...
                                          write a small random-init model in the mlx-lm file layout
+  patch --model DIR [--out DIR/.fusekit] [--prefill-m 32,128] [--capacity C]
+                                         the reference's `fusekit patch`: write task_graph.json, manifest.json and
+                                         variants/prefill_mN/task_graph.json for a checkpoint
+  generate --model DIR --artifact DIR ... decode from the artifact's task graphs instead of a fresh runtime
 """
 import argparse
 import json
@@ -21,6 +25,12 @@ def main() -> int:
     g.add_argument("--ids", required=True, help="comma-separated prompt token ids")
     g.add_argument("--max-tokens", type=int, default=32)
     g.add_argument("--capacity", type=int, default=1024)
+    g.add_argument("--artifact", default=None, help="directory written by `patch`")
+    pa = sub.add_parser("patch")
+    pa.add_argument("--model", required=True)
+    pa.add_argument("--out", default=None)
+    pa.add_argument("--prefill-m", default="", help="comma-separated active row counts of the prefill variants")
+    pa.add_argument("--capacity", type=int, default=1024)
     e = sub.add_parser("export-random")
     e.add_argument("--out", required=True)
     e.add_argument("--bits", type=int, default=4, choices=[4, 8, 16])
@@ -51,8 +61,23 @@ def main() -> int:
         return 0
     from .checkpoint import load_mlx_checkpoint
     cfg, w = load_mlx_checkpoint(args.model, capacity=args.capacity)
-    rt = DecoderRuntime(cfg, w)
+    if args.cmd == "patch":
+        import os
+        from .artifact import write_artifact
+        from .prefill_variant import PrefillVariant
+        rt = DecoderRuntime(cfg, w)
+        out = args.out or os.path.join(args.model, ".fusekit")
+        ms = [int(v) for v in args.prefill_m.split(",") if v.strip()]
+        write_artifact(rt, out, os.path.basename(os.path.normpath(args.model)), prefill_variants=[PrefillVariant(rt, m) for m in ms])
+        print(json.dumps({"artifact": out, "tasks": len(rt.tasks), "variants": [f"prefill_m{m}" for m in ms]}))
+        return 0
     prompt = [int(t) for t in args.ids.split(",") if t.strip()]
+    if args.artifact:
+        from .artifact import ArtifactRuntime
+        art = ArtifactRuntime(args.artifact, w)
+        print(json.dumps({"tokens": art.generate(prompt, args.max_tokens), "variants": sorted(art.variants)}))
+        return 0
+    rt = DecoderRuntime(cfg, w)
     toks, gpu_s, steps = rt.generate(prompt, args.max_tokens)
     print(json.dumps({"tokens": toks, "decode_tok_per_s": round(steps / gpu_s, 1) if gpu_s else None}))
     return 0

@@ -66,25 +66,35 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
     return sym
 
 
-def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "synthetic") -> None:
-    if rt.persistent:
-        raise ValueError("write the artifact from a task-graph runtime (persistent=False)")
-    os.makedirs(out_dir, exist_ok=True)
-    sym = _symbols(rt)
+def _resolve(sym: Dict[int, dict], ptr: int):
+    """The symbol a slot points into, and the byte offset inside it (a slot may be a slice of a buffer)."""
+    s = sym.get(ptr)
+    if s is not None:
+        return s, 0
+    for base, cand in sym.items():
+        if cand["role"] == "scratch" and base < ptr < base + cand["size_bytes"]:
+            return cand, ptr - base
+    return None, 0
+
+
+def _graph_dict(rt: DecoderRuntime, task_list: List[Dispatch], graph_id: int, sym: Dict[int, dict], active_m: int,
+                uniforms: Dict[str, str]) -> dict:
     scratch_ids: Dict[str, int] = {}
     scratch_buffers: List[dict] = []
     tasks: List[dict] = []
     groups: Dict[str, List[int]] = {}
-    for tid, d in enumerate(rt.tasks):
+    for tid, d in enumerate(task_list):
         geo = rt.d.plan_geometry(d)
         bindings = []
         for slot, (ptr, nbytes) in enumerate(d.args):
-            s = sym.get(ptr)
+            s, off = _resolve(sym, ptr)
             if s is None:
                 raise ValueError(f"task {tid} ({d.kernel}) slot {slot}: buffer is not a known parameter or scratch")
             access = geo.slot_access[slot]
             b = dict(slot=slot, role=s["role"], access=("rw" if access == 3 else "w" if access == 2 else "r"),
                      nbytes=nbytes, dtype=s["dtype"])
+            if off:
+                b["offset_bytes"] = off
             if s["role"] == "external":
                 b.update(source_path=s["source_path"], shape=s["shape"], role_name=s["source_path"].rsplit(".", 1)[-1])
             else:
@@ -107,27 +117,55 @@ def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "syntheti
                     inputs=[b for b in bindings if b["access"] == "r"],
                     outputs=[b for b in bindings if b["access"] != "r"],
                     params={k: float(v) for k, v in d.params.items()},
-                    kernels=kernels, depends_on=rt.d.node_deps(rt.graph, tid), trigger_event=tid)
+                    kernels=kernels, depends_on=rt.d.node_deps(graph_id, tid), trigger_event=tid)
         if layer is not None:
             task["layer_idx"] = layer
         tasks.append(task)
         region = "embed" if layer is None and tid < 2 else (f"layer.{layer}" if layer is not None else "post")
         groups.setdefault(region, []).append(tid)
     c = rt.cfg
-    graph = dict(
-        version=SCHEMA_VERSION, active_m=1, backend="hip-gfx950", tasks=tasks,
+    return dict(
+        version=SCHEMA_VERSION, active_m=active_m, backend="hip-gfx950", tasks=tasks,
         events=[dict(id=t["id"], num_triggers=1, fires=[u["id"] for u in tasks if t["id"] in u["depends_on"]]) for t in tasks],
         scratch_buffers=scratch_buffers, initial_tasks=[t["id"] for t in tasks if not t["depends_on"]],
         model_params=[dict(path=s["source_path"], shape=s["shape"], dtype=s["dtype"]) for s in sym.values() if s["role"] == "external"],
         layer_groups=[dict(region=r, task_ids=ids) for r, ids in groups.items()],
         decode_pipeline=[t["id"] for t in tasks],
         decode_capabilities=dict(dispatchable=True, reasons=[]),
-        uniforms=dict(token="token", step_counter="step_counter", hist_counter="hist_counter", history="history"),
+        uniforms=uniforms,
         model_config={k: getattr(c, k) for k in ("n_layers", "hidden", "n_heads", "n_kv", "head_dim", "inter", "vocab",
                                                   "capacity", "bits", "group", "eps", "theta", "qk_norm", "qkv_bias",
                                                   "fuse_rope_store", "swiglu_variant", "kv_bits", "kv_group", "fuse_attention")})
+
+
+def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "synthetic", prefill_variants=()) -> None:
+    """`prefill_variants`: PrefillVariant objects of this runtime; each is written as
+    `variants/prefill_mN/task_graph.json` and listed in the manifest (src/commands/patch.rs:112-150)."""
+    if rt.persistent:
+        raise ValueError("write the artifact from a task-graph runtime (persistent=False)")
+    os.makedirs(out_dir, exist_ok=True)
+    sym = _symbols(rt)
+    graph = _graph_dict(rt, rt.tasks, rt.graph, sym, 1,
+                        dict(token="token", step_counter="step_counter", hist_counter="hist_counter", history="history"))
     with open(os.path.join(out_dir, "task_graph.json"), "w") as f:
         json.dump(graph, f, indent=1)
+    tasks = graph["tasks"]
+    variants = []
+    for v in prefill_variants:
+        vsym = dict(sym)
+        for name, buf in v.scratch().items():
+            u32 = name.rsplit(".", 1)[-1] in ("tokens", "offset", "kv_len")
+            vsym[buf.ptr] = dict(role="scratch", role_name=name, dtype="uint32" if u32 else ("float32" if name.endswith(".ws") else "bfloat16"),
+                                 size_bytes=buf.nbytes, zero=u32)
+        vg = _graph_dict(rt, v.tasks, v.graph, vsym, v.m,
+                         dict(token="token", tokens=v.name + ".tokens", offset=v.name + ".offset", kv_len=v.name + ".kv_len",
+                              hist_counter="hist_counter", history="history"))
+        vdir = os.path.join(out_dir, "variants", v.name)
+        os.makedirs(vdir, exist_ok=True)
+        with open(os.path.join(vdir, "task_graph.json"), "w") as f:
+            json.dump(vg, f, indent=1)
+        variants.append(dict(name=v.name, path="variants/" + v.name, active_m=v.m, tasks=len(vg["tasks"])))
+    c = rt.cfg
     manifest = dict(
         schema_version=SCHEMA_VERSION, fusekit_version=BACKEND_VERSION,
         compiled_at=time.strftime("%Y-%m-%dT%H:%M:%SZ", time.gmtime()),
@@ -136,7 +174,7 @@ def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "syntheti
                    head_dim=c.head_dim, vocab_size=c.vocab),
         stats=dict(ops=len(tasks), fusions=len(tasks), tasks=len(tasks),
                    unique_kernels=len({re.sub(r"_f\d+$", "", t["kernel"]) for t in tasks})),
-        variants=[])
+        variants=variants)
     with open(os.path.join(out_dir, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1)
 
@@ -161,27 +199,70 @@ class ArtifactRuntime:
             if W.bits != 16:
                 params[p + ".scales"], params[p + ".biases"] = W.scales, W.biases
         params.update(weights.vecs)
-        self.tasks: List[Dispatch] = []
-        for tid in graph["decode_pipeline"]:
-            t = graph["tasks"][tid]
-            slots = sorted(t["inputs"] + t["outputs"], key=lambda b: b["slot"])
-            args = []
-            for b in slots:
-                buf = params[b["source_path"]] if b["role"] == "external" else self.scratch[b["role_name"]]
-                if b["nbytes"] > buf.nbytes:
-                    raise ValueError(f"task {tid} slot {b['slot']}: binding wants {b['nbytes']} bytes, buffer has {buf.nbytes}")
-                args.append((buf.ptr, b["nbytes"]))
-            self.tasks.append(Dispatch(t["kernel"], args, dict(t["params"])))
+        self._params = params
+        self.tasks = self._tasks_of(graph)
         u = graph["uniforms"]
         self.uniforms = make_uniforms(self.scratch[u["token"]], self.scratch[u["step_counter"]],
                                       self.scratch[u["hist_counter"]], self.scratch[u["history"]])
         self.graph = self.d.build_graph(self.tasks)
         self.model_config = graph["model_config"]
         self._weights = weights  # keeps the parameter buffers alive
+        # prefill_mN variants (manifest `variants`, one task graph each): scratch buffers are shared by role
+        # name with the decode graph (KV caches, token, history, logits), the rest is the variant's own
+        self.variants: Dict[int, dict] = {}
+        for v in manifest.get("variants", []):
+            if not str(v.get("name", "")).startswith("prefill_m"):
+                continue
+            vg = json.load(open(os.path.join(art_dir, v["path"], "task_graph.json")))
+            if vg.get("version") != SCHEMA_VERSION or int(vg.get("active_m", 0)) != int(v["active_m"]):
+                raise ValueError(f"variant {v['name']}: task graph does not match the manifest entry")
+            for sb in vg["scratch_buffers"]:
+                have = self.scratch.get(sb["role_name"])
+                if have is None:
+                    self.scratch[sb["role_name"]] = native.zeros(sb["size_bytes"]) if sb["zero_init"] else DeviceBuffer(sb["size_bytes"])
+                elif have.nbytes < sb["size_bytes"]:
+                    raise ValueError(f"variant {v['name']}: scratch {sb['role_name']} is larger than in the decode graph")
+            vu = vg["uniforms"]
+            self.variants[int(v["active_m"])] = dict(
+                graph=self.d.build_graph(self._tasks_of(vg)), tokens=self.scratch[vu["tokens"]],
+                offset=self.scratch[vu["offset"]], kv_len=self.scratch[vu["kv_len"]], token=self.scratch[vu["token"]])
+
+    def _tasks_of(self, graph: dict) -> List[Dispatch]:
+        out: List[Dispatch] = []
+        for tid in graph["decode_pipeline"]:
+            t = graph["tasks"][tid]
+            slots = sorted(t["inputs"] + t["outputs"], key=lambda b: b["slot"])
+            args = []
+            for b in slots:
+                buf = self._params[b["source_path"]] if b["role"] == "external" else self.scratch[b["role_name"]]
+                off = int(b.get("offset_bytes", 0))
+                if off + b["nbytes"] > buf.nbytes:
+                    raise ValueError(f"task {tid} slot {b['slot']}: binding wants {off + b['nbytes']} bytes, buffer has {buf.nbytes}")
+                args.append((buf.ptr + off, b["nbytes"]))
+            out.append(Dispatch(t["kernel"], args, dict(t["params"])))
+        return out
+
+    def prefill(self, prompt) -> int:
+        """Prompt processing: whole blocks of N tokens through the largest `prefill_mN` variant that fits
+        what is left (the reference takes a variant when exactly N tokens are to be processed,
+        python/fusekit_runtime/__init__.py:4866), the rest token by token through the decode graph."""
+        from .prefill_variant import run_variant
+        prompt = list(prompt)
+        pos, nxt = 0, None
+        cap = int(self.model_config["capacity"])
+        while pos < len(prompt):
+            fit = [m for m in self.variants if m <= len(prompt) - pos]
+            if not fit:
+                toks, _ = self.d.decode_host_loop(self.graph, self.uniforms, pos, prompt[pos:])
+                return toks[-1]
+            m = max(fit)
+            v = self.variants[m]
+            nxt = run_variant(self.d, v["graph"], m, v["tokens"], v["offset"], v["kv_len"], v["token"], prompt[pos:pos + m], pos, cap)
+            pos += m
+        return nxt
 
     def generate(self, prompt, max_tokens: int) -> List[int]:
-        nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, 0, list(prompt))
-        out = [nxt[-1]]
+        out = [self.prefill(prompt)]
         offset = len(prompt)
         while len(out) < max_tokens:
             n = min(64, max_tokens - len(out), self.uniforms.hist_capacity)

@@ -130,11 +130,13 @@ fk_status plan_embed_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_args(d, n));
     fk_weight E;
     FK_TRY(bind_weight(d, bits, group, vocab, hidden, 1, 2, 3, &E));
-    FK_TRY(need_bytes(d, 0, 4));
-    FK_TRY(need_bytes(d, n - 1, (size_t)hidden * 2));
+    const uint32_t rows = d.u("rows", 1);  // active_m > 1: one token id and one output row per active row
+    if (rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows must be at least 1");
+    FK_TRY(need_bytes(d, 0, (size_t)rows * 4));
+    FK_TRY(need_bytes(d, n - 1, (size_t)rows * hidden * 2));
     all_but_last(n, 1, rw);
     return plan_embed(&E, arg_ptr<const uint32_t>(d, 0), 0, (float)d.param("output_scale", 1.0),
-                      arg_ptr<uint16_t>(d, n - 1), l);
+                      arg_ptr<uint16_t>(d, n - 1), l, rows);
 }
 
 // x, [norm_w], W_q, W_k, W_v, [s_q, s_k, s_v, b_q, b_k, b_v], [bias_q, bias_k, bias_v], q, k, v
@@ -370,9 +372,11 @@ fk_status plan_qkv_rope_store(const Dispatch& d, Launch* l, SlotRW* rw) {
     a.rope_on = a.rope_dims ? 1u : 0u;
     a.capacity = d.u("capacity");
     if (a.capacity == 0) return set_error(FK_ERR_INVALID, d.kernel + ": capacity parameter missing");
-    FK_TRY(need_bytes(d, 0, (size_t)a.n_q * a.head_dim * 2));
-    FK_TRY(need_bytes(d, 1, (size_t)a.n_kv * a.head_dim * 2));
-    FK_TRY(need_bytes(d, 2, (size_t)a.n_kv * a.head_dim * 2));
+    a.rows = d.u("rows", 1);  // active_m > 1: row r is the token at position offset + r
+    if (a.rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows must be at least 1");
+    FK_TRY(need_bytes(d, 0, (size_t)a.rows * a.n_q * a.head_dim * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)a.rows * a.n_kv * a.head_dim * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)a.rows * a.n_kv * a.head_dim * 2));
     FK_TRY(need_bytes(d, ck, (size_t)a.n_kv * a.capacity * a.head_dim * 2));
     FK_TRY(need_bytes(d, ck + 1, (size_t)a.n_kv * a.capacity * a.head_dim * 2));
     FK_TRY(need_bytes(d, ck + 2, 4));
@@ -424,20 +428,41 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
 // kv_len, L and capacity as uniforms; here they are the parameters kv_len, rows and capacity,
 // because the grid depends on them.
 fk_status plan_sdpa_prefill_d(const Dispatch& d, Launch* l, SlotRW* rw) {
-    FK_TRY(need_args(d, 4));
+    // five slots: Q, K, V, kv_len (device uint32, read at run time: the graph is replayed for any offset), out
+    const bool dev_len = d.args.size() == 5;
+    FK_TRY(need_args(d, dev_len ? 5 : 4));
+    const size_t out_slot = dev_len ? 4 : 3;
     const uint32_t n_heads = d.u("n_heads"), n_kv = d.u("n_kv"), dim = d.u("head_dim"), capacity = d.u("capacity");
-    const uint32_t rows = d.u("rows"), kv_len = d.u("kv_len");
+    const uint32_t rows = d.u("rows"), kv_len = dev_len ? rows : d.u("kv_len");
+    if (dev_len) FK_TRY(need_bytes(d, 3, 4));
     if (n_heads == 0 || n_kv == 0 || dim == 0 || capacity == 0 || rows == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / head_dim / capacity / rows parameters missing");
     const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)dim);  // sdpa_prefill.rs:52
     FK_TRY(need_bytes(d, 0, (size_t)rows * n_heads * dim * 2));
     FK_TRY(need_bytes(d, 1, (size_t)n_kv * capacity * dim * 2));
     FK_TRY(need_bytes(d, 2, (size_t)n_kv * capacity * dim * 2));
-    FK_TRY(need_bytes(d, 3, (size_t)rows * n_heads * dim * 2));
+    FK_TRY(need_bytes(d, out_slot, (size_t)rows * n_heads * dim * 2));
     rw->reads = {0, 1, 2};
-    rw->writes = {3};
+    if (dev_len) rw->reads.push_back(3);
+    rw->writes = {(uint32_t)out_slot};
     return plan_sdpa_prefill(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<const uint16_t>(d, 2),
-                             arg_ptr<uint16_t>(d, 3), rows, kv_len, n_heads, n_kv, dim, capacity, scale, l);
+                             arg_ptr<uint16_t>(d, out_slot), rows, kv_len, n_heads, n_kv, dim, capacity, scale, l,
+                             dev_len ? arg_ptr<const uint32_t>(d, 3) : nullptr);
+}
+
+// x, weight, out: RMSNorm of `rows` rows, T(w * T(x * r)) (the norm stage of the reference's multi-row
+// variants, which fuse it into their matmul prologue)
+fk_status plan_rmsnorm_rows_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 3));
+    const uint32_t rows = d.u("rows"), hidden = d.u("hidden");
+    if (rows == 0 || hidden == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows / hidden parameters missing");
+    FK_TRY(need_bytes(d, 0, (size_t)rows * hidden * 2));
+    FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)rows * hidden * 2));
+    rw->reads = {0, 1};
+    rw->writes = {2};
+    return plan_rmsnorm_rows(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), (float)d.param("eps", 1e-6), rows, hidden,
+                             arg_ptr<uint16_t>(d, 2), l);
 }
 
 // Q, K, V, [q_weight, k_weight], cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]
@@ -770,6 +795,7 @@ const Family kFamilies[] = {
     {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
     {"fusekit_sdpa_decode", plan_sdpa_d},
     {"fusekit_sdpa_prefill", plan_sdpa_prefill_d},
+    {"fusekit_rmsnorm_rows", plan_rmsnorm_rows_d},
     {"fusekit_rope_store_sdpa_decode", plan_rope_store_sdpa},
     {"fusekit_rope_kv_cache_store_decode_q4",
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv_quant(d, l, rw, 4); }},

@@ -174,10 +174,11 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
                            float* partials, uint32_t* counters, Launch* out_launch, uint32_t rows = 1,
                            const KvQuant* quant = nullptr, const SdpaFusion* fusion = nullptr);
 // Causal attention of a group of rows on the matrix cores (head dimension 64 or 128, bf16 cache):
-// kv_len counts the rows of the group, row r sees the first kv_len - rows + r + 1 positions.
+// kv_len counts the rows of the group, row r sees the first kv_len - rows + r + 1 positions.  With
+// kv_len_ptr the count is read on the device at run time (clamped to rows .. capacity).
 fk_status plan_sdpa_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,
                             uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
-                            uint32_t capacity, float scale, Launch* out_launch);
+                            uint32_t capacity, float scale, Launch* out_launch, const uint32_t* kv_len_ptr = nullptr);
 fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t token_imm, float out_scale,
                      uint16_t* x, Launch* out, uint32_t rows = 1);
 fk_status plan_rmsnorm_rows(const uint16_t* x, const uint16_t* w, float eps, uint32_t rows, uint32_t hidden, uint16_t* y,

@@ -57,7 +57,16 @@ struct SdpaPrefillArgs {
     uint16_t* out;        // [rows, n_heads, D]
     uint32_t rows, kv_len, n_heads, heads_per_kv, capacity, row_tiles;
     float scale2;         // softmax scale times log2(e)
+    const uint32_t* kv_len_ptr;  // optional: the count on the device (a replayed graph), instead of kv_len
 };
+
+// Positions in the cache including the group's rows.  A device value is clamped to what the
+// host validated for an immediate one (rows <= kv_len <= capacity), so no address leaves the cache.
+__device__ __forceinline__ uint32_t prefill_kv_len(const SdpaPrefillArgs& a) {
+    uint32_t n = a.kv_len_ptr ? *a.kv_len_ptr : a.kv_len;
+    n = n < a.rows ? a.rows : n;
+    return n > a.capacity ? a.capacity : n;
+}
 
 __device__ __forceinline__ float other_half_max(float v) {
     const pf_u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -154,7 +163,7 @@ __global__ __launch_bounds__(kPrefillBlock) void sdpa_prefill_kernel(const SdpaP
     const uint32_t kvh = head / a.heads_per_kv;
     const uint32_t r0 = tile * kPrefillRows;
     const uint32_t live = a.rows - r0 < kPrefillRows ? a.rows - r0 : kPrefillRows;
-    const uint32_t prior = a.kv_len - a.rows;      // positions in the cache before this group
+    const uint32_t prior = prefill_kv_len(a) - a.rows;      // positions in the cache before this group
     const uint32_t kv_end = prior + r0 + live;     // positions the last live row sees
     const uint32_t first_limit = prior + r0 + 1u;  // positions the first row sees
     const uint32_t n_steps = (kv_end + kPrefillStep - 1u) / kPrefillStep;
@@ -357,7 +366,7 @@ __global__ __launch_bounds__(kPrefillBlock) void sdpa_prefill_tile_kernel(const 
     const uint32_t kvh = head / a.heads_per_kv;
     const uint32_t r0 = (grp * kPrefillWaves + wave) * kPrefillRows;
     const uint32_t live = r0 < a.rows ? (a.rows - r0 < kPrefillRows ? a.rows - r0 : kPrefillRows) : 0u;
-    const uint32_t prior = a.kv_len - a.rows;
+    const uint32_t prior = prefill_kv_len(a) - a.rows;
     const uint32_t grp_end = (grp + 1u) * kPrefillWaves * kPrefillRows;
     const uint32_t kv_end_blk = prior + (grp_end < a.rows ? grp_end : a.rows);  // positions the block's last row sees
     const uint32_t first_limit = prior + r0 + 1u;
@@ -515,7 +524,7 @@ __global__ __launch_bounds__(kPrefillBlock) void sdpa_prefill_tile_kernel(const 
 
 fk_status plan_sdpa_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out,
                             uint32_t rows, uint32_t kv_len, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
-                            uint32_t capacity, float scale, Launch* l) {
+                            uint32_t capacity, float scale, Launch* l, const uint32_t* kv_len_ptr) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!q || !cache_k || !cache_v || !out) return set_error(FK_ERR_INVALID, "sdpa_prefill: null pointer");
@@ -529,6 +538,8 @@ fk_status plan_sdpa_prefill(const uint16_t* q, const uint16_t* cache_k, const ui
     SdpaPrefillArgs a;
     memset(&a, 0, sizeof(a));
     a.q = q; a.k = cache_k; a.v = cache_v; a.out = out;
+    a.kv_len_ptr = kv_len_ptr;
+    if (rows > capacity) return set_error(FK_ERR_INVALID, "sdpa_prefill: more rows than the cache holds");
     a.rows = rows; a.kv_len = kv_len; a.n_heads = n_heads; a.heads_per_kv = n_heads / n_kv; a.capacity = capacity;
     a.scale2 = scale * 1.4426950408889634f;
     // Two forms: a block per 32 rows whose waves split the positions, or a block per 128 rows whose

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import OracleDecoder, bf16_mismatch, host_weight, rng
+from helpers import OracleDecoder, bf16_mismatch, host_weight, rel_l2, rng
 
 pytestmark = pytest.mark.gpu
 
@@ -331,6 +331,56 @@ def test_artifact_round_trip_and_launch_geometry(fk, tmp_path):
         ArtifactRuntime(str(tmp_path), W)
     t = fk.target_describe()
     assert t.from_device == 1 and t.wave_size == 64 and t.compute_units >= 64 and t.arch.startswith(b"gfx950")
+
+
+@pytest.mark.parametrize("bits,qk_norm,qkv_bias", [(4, True, False), (8, False, True)])
+def test_prefill_variants_as_graphs_and_in_the_artifact(fk, tmp_path, bits, qk_norm, qkv_bias):
+    """`prefill_mN` variants (the reference: variants/prefill_mN, active_m = N): the whole model for N
+    rows as one replayable graph whose position comes from device words.  A block of the prompt through
+    the variant leaves the caches of the token-by-token path and the same greedy continuation; the
+    artifact lists the variants and a consumer that knows only the files uses them."""
+    import json
+    from fusekit_amd.artifact import ArtifactRuntime, write_artifact
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    from fusekit_amd.prefill_variant import PrefillVariant
+    cfg = _small_cfg(bits=bits, qk_norm=qk_norm, qkv_bias=qkv_bias, swiglu_variant=2)
+    W = DecoderWeights.random_init(cfg, seed=51)
+    prompt = rng(52).integers(0, cfg.vocab, 45).tolist()
+    a, b = DecoderRuntime(cfg, W), DecoderRuntime(cfg, W)
+    first_a = a.prefill(prompt)
+    v32, v8 = PrefillVariant(b, 32), PrefillVariant(b, 8)
+    v32.run(prompt[:32], 0)                       # positions 0..31
+    first8 = v8.run(prompt[32:40], 32)            # the same graph form at another position
+    nxt, _ = b.d.decode_host_loop(b.graph, b.uniforms, 40, prompt[40:])
+    for l in range(cfg.n_layers):
+        for ca, cb_ in ((a.cache_k[l], b.cache_k[l]), (a.cache_v[l], b.cache_v[l])):
+            ga, gb = ca.to_numpy(np.uint16), cb_.to_numpy(np.uint16)
+            assert np.array_equal(ga == 0, gb == 0)
+            assert rel_l2(gb, oracle.bf16_to_f32(ga)) <= 1e-2, l
+    ref, margins = OracleDecoder(cfg, W).generate(prompt, 8)
+    if margins[0] > 0.05:
+        assert nxt[-1] == first_a == ref[0]
+    ref40, m40 = OracleDecoder(cfg, W).generate(prompt[:40], 1)
+    if m40[0] > 0.05:
+        assert first8 == ref40[0]                 # the variant's own LM head + argmax on its last row
+    with pytest.raises(ValueError):
+        v8.run(prompt[:7], 0)                     # a variant processes exactly N tokens
+    # the artifact: manifest entry + variants/prefill_mN/task_graph.json, consumed without the runtime
+    write_artifact(b, str(tmp_path), "tiny", prefill_variants=[v32, v8])
+    man = json.load(open(tmp_path / "manifest.json"))
+    assert [(v["name"], v["active_m"]) for v in man["variants"]] == [("prefill_m32", 32), ("prefill_m8", 8)]
+    vg = json.load(open(tmp_path / "variants" / "prefill_m32" / "task_graph.json"))
+    assert vg["active_m"] == 32 and vg["uniforms"]["kv_len"] == "prefill_m32.kv_len"
+    att = next(t for t in vg["tasks"] if t["kernel"].startswith("fusekit_sdpa_prefill"))
+    assert [x["role_name"] for x in att["inputs"]][-1] == "prefill_m32.kv_len" and att["params"]["rows"] == 32.0
+    head = next(t for t in vg["tasks"] if t["kernel"].startswith("fusekit_final_rmsnorm_lm_head"))
+    assert head["inputs"][0]["offset_bytes"] == 31 * cfg.hidden * 2     # the last row of the block
+    art = ArtifactRuntime(str(tmp_path), W)
+    assert sorted(art.variants) == [8, 32]
+    got = art.generate(prompt, 8)                 # 32 + 8 through the variants, 5 token by token
+    want, _, _ = a.generate(prompt, 8)
+    clear = next((i for i, m in enumerate(margins) if m <= 0.05), 8)
+    assert got[:clear] == want[:clear] == ref[:clear]
 
 
 @pytest.mark.parametrize("bits,untied", [(4, False), (8, True), (16, False)])
