@@ -49,9 +49,7 @@ __global__ __launch_bounds__(kWave) void rope_store_kernel(const RopeArgs a) {
 }
 
 // The rotary table of a prompt pass: without it every (head, row) wave evaluates exp2 in double and
-// sincosf per pair; the table is filled once per pass and serves every layer.  (The kernel's time at
-// 4096 rows, 92 us, is that of its short dependent chains of 2-byte accesses, one wave per head and
-// row; four heads per block or a loop over heads inside a wave were slower, 103 and 109 us.)
+// sincosf per pair; the table is filled once per pass and serves every layer.
 struct RopeTabArgs {
     float* tab;
     uint32_t half, offset, rows;
@@ -82,6 +80,91 @@ fk_status plan_rope_table(float* tab, uint32_t rope_dims, float base_log2, uint3
     return FK_OK;
 }
 
+// Row form for prompt passes (rotation over the whole head of 64 or 128 dims, rotary table given):
+// a head row is spread over HL = dim / 8 adjacent lanes with 16 bytes each, so a wave moves 8 (4)
+// head rows with one 16-byte load and one store per lane and ONE dependent round trip to memory; the
+// pair (d, d + dim/2) sits HL/2 lanes apart and is exchanged as packed bf16, the norm's sum of squares
+// is a butterfly over the HL lanes.  One wave per (head, row) with 2-byte accesses took 92 us for
+// 4096 rows of the 4B-class model; the kernel is bound by its short chains, not by bytes.
+template <int HL>
+__global__ __launch_bounds__(256) void rope_rows_fast_kernel(const RopeArgs a) {
+    constexpr uint32_t DIM = HL * 8u, HPW = kWave / HL;
+    const uint32_t lane = threadIdx.x & (kWave - 1u);
+    const uint32_t heads = a.n_q + 2u * a.n_kv, groups = (heads + HPW - 1u) / HPW;
+    const uint32_t wg = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint32_t tr = wg / groups, g = wg - tr * groups;
+    if (tr >= a.rows) return;  // whole waves
+    const uint32_t b_raw = g * HPW + lane / HL, p = lane % HL;
+    const bool live = b_raw < heads;
+    const uint32_t b = live ? b_raw : heads - 1u;  // lanes past the last head repeat it and store nothing
+    const uint32_t pos0 = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
+    const uint32_t wpos = (a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos0)) + tr;
+    const uint32_t row = wpos % a.capacity;
+    const uint16_t* src;
+    uint16_t* dst;
+    const uint16_t* nw = nullptr;
+    bool rotate = true;
+    if (b < a.n_q) {
+        src = dst = a.q + ((size_t)tr * a.n_q + b) * DIM;
+        nw = a.q_norm;
+    } else if (b < a.n_q + a.n_kv) {
+        const uint32_t h = b - a.n_q;
+        src = a.k + ((size_t)tr * a.n_kv + h) * DIM;
+        dst = a.cache_k + ((size_t)h * a.capacity + row) * DIM;
+        nw = a.k_norm;
+    } else {
+        const uint32_t h = b - a.n_q - a.n_kv;
+        src = a.v + ((size_t)tr * a.n_kv + h) * DIM;
+        dst = a.cache_v + ((size_t)h * a.capacity + row) * DIM;
+        rotate = false;
+    }
+    // every load is issued before anything is used; lanes without a norm weight read their own row instead
+    const uint4 xv = *reinterpret_cast<const uint4*>(src + p * 8u);
+    const uint4 wv = *reinterpret_cast<const uint4*>((nw ? nw : src) + p * 8u);
+    const float4* tp = reinterpret_cast<const float4*>(a.rope_tab + (size_t)tr * DIM + 2u * ((p % (HL / 2u)) * 8u));
+    const float4 t0 = tp[0], t1 = tp[1], t2 = tp[2], t3 = tp[3];  // (cos, sin) of this lane's eight pairs
+    const float cs[8] = {t0.x, t0.z, t1.x, t1.z, t2.x, t2.z, t3.x, t3.z};
+    const float sn[8] = {t0.y, t0.w, t1.y, t1.w, t2.y, t2.w, t3.y, t3.w};
+
+    uint32_t pv[4] = {xv.x, xv.y, xv.z, xv.w};
+    const uint32_t wq[4] = {wv.x, wv.y, wv.z, wv.w};
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = bf16_lo(pv[i]), hi = bf16_hi(pv[i]);
+        ss = fmaf(lo, lo, ss);
+        ss = fmaf(hi, hi, ss);
+    }
+    ss = group_sum(ss, HL);  // all lanes take part; used only where there is a norm weight
+    if (nw) {
+        const float r = 1.0f / sqrtf(ss / (float)DIM + a.eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t xr = pack_bf16(bf16_lo(pv[i]) * r, bf16_hi(pv[i]) * r);   // T(x * r)
+            pv[i] = pack_bf16(bf16_lo(wq[i]) * bf16_lo(xr), bf16_hi(wq[i]) * bf16_hi(xr));  // T(w * that)
+        }
+    }
+    uint32_t ov[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ov[i] = (uint32_t)__shfl_xor((int)pv[i], (int)(HL / 2u), kWave);
+    uint4 res = make_uint4(pv[0], pv[1], pv[2], pv[3]);
+    if (rotate) {
+        const bool second = p >= HL / 2u;  // this lane holds the d + dim/2 side of its pairs
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float a0 = bf16_lo(pv[i]), a1 = bf16_hi(pv[i]), b0 = bf16_lo(ov[i]), b1 = bf16_hi(ov[i]);
+            const float r0 = second ? a0 * cs[2 * i] + b0 * sn[2 * i] : a0 * cs[2 * i] - b0 * sn[2 * i];
+            const float r1 = second ? a1 * cs[2 * i + 1] + b1 * sn[2 * i + 1] : a1 * cs[2 * i + 1] - b1 * sn[2 * i + 1];
+            o[i] = pack_bf16(r0, r1);
+        }
+        res = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        res = xv;  // V rows are copied as they are
+    }
+    if (live) *reinterpret_cast<uint4*>(dst + p * 8u) = res;
+}
+
 fk_status plan_rope_store(const RopeArgs& in, Launch* out) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
@@ -97,6 +180,22 @@ fk_status plan_rope_store(const RopeArgs& in, Launch* out) {
     if (!a.rows) a.rows = 1;
     if (a.rows > 65535) return set_error(FK_ERR_UNSUPPORTED, "rope: too many rows");
     if (a.n_kv && a.rows > a.capacity) return set_error(FK_ERR_INVALID, "rope: more rows than the cache holds");
+    const bool aligned = ((reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.k) | reinterpret_cast<uintptr_t>(a.v) |
+                           reinterpret_cast<uintptr_t>(a.cache_k) | reinterpret_cast<uintptr_t>(a.cache_v) |
+                           reinterpret_cast<uintptr_t>(a.q_norm) | reinterpret_cast<uintptr_t>(a.k_norm) |
+                           reinterpret_cast<uintptr_t>(a.rope_tab)) & 15u) == 0;
+    const uint32_t dim = a.n_q ? a.head_dim : a.k_dim;
+    if (a.rows >= 8 && a.rope_tab && a.rope_on && a.n_q && a.n_kv && (dim == 64 || dim == 128) && a.rope_dims == dim &&
+        a.k_dim == dim && a.v_dim == dim && aligned) {
+        const uint32_t hpw = dim == 128 ? 4u : 8u, heads = a.n_q + 2 * a.n_kv;
+        const uint64_t waves = (uint64_t)a.rows * ((heads + hpw - 1u) / hpw);
+        out->func = dim == 128 ? reinterpret_cast<const void*>(&rope_rows_fast_kernel<16>) : reinterpret_cast<const void*>(&rope_rows_fast_kernel<8>);
+        out->grid = dim3((uint32_t)((waves + 3u) / 4u), 1, 1);
+        out->block = dim3(256, 1, 1);
+        out->shmem = 0;
+        out->set_args(a);
+        return FK_OK;
+    }
     out->func = reinterpret_cast<const void*>(&rope_store_kernel);
     out->grid = dim3(a.n_q + 2 * a.n_kv, a.rows, 1);
     out->block = dim3(kWave, 1, 1);
