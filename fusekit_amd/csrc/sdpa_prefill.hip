@@ -85,6 +85,25 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The rescale of the output accumulators, in place in the accumulation registers of the matrix unit.
+// Written as plain C++ this multiply makes the compiler copy all of them to vector registers at the
+// head of EVERY pass, taken or not; spelled out, the copies stay inside the rare branch that calls
+// this (128 rows x 4096 positions: 112 -> 105 us).  The trailing s_nop covers the wait states a
+// matrix instruction needs after the write.
+template <int DT>
+__device__ __forceinline__ void rescale_accumulators(pf_f32x16_t (&oacc)[DT], float alpha) {
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float x = oacc[i][r], t;
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
+                         : "+a"(x), "=&v"(t)
+                         : "v"(alpha));
+            oacc[i][r] = x;
+        }
+}
+
 // One 64-position step of the running softmax of a lane's query.  Register r of score tile t is
 // cache position kv0 + 32 t + r % 4 + 8 (r / 4) + 4 kb; scores become base-2 exponents; positions
 // at or past q_limit are in the query's future (only steps with `mask` set can hold any).  Leaves
@@ -130,23 +149,7 @@ __device__ __forceinline__ void softmax_step(const pf_f32x16_t (&s)[2], float sc
     }
     l_run = l_run * alpha + psum;
     m_run = m_new;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-        // The accumulators live in the accumulation registers of the matrix unit.  Written as
-        // plain C++ this multiply makes the compiler copy all of them to vector registers at the
-        // head of EVERY pass, taken or not; spelled out, the copies stay inside this rare branch
-        // (128 rows x 4096 positions: 112 -> 105 us).  The trailing s_nop covers the wait states
-        // a matrix instruction needs after the write.
-#pragma unroll
-        for (int i = 0; i < DT; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float x = oacc[i][r], t;
-                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
-                             : "+a"(x), "=&v"(t)
-                             : "v"(alpha));
-                oacc[i][r] = x;
-            }
-    }
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) rescale_accumulators<DT>(oacc, alpha);
 }
 
 template <int D>
