@@ -161,39 +161,47 @@ def case_sdpa_prefill(d, reps, rows, kv_len):
           pool=pool)
 
 
-def case_moe(d, reps, bits=4):
+def case_moe(d, reps, bits=4, tokens=1):
+    """Config 5 routed experts: `tokens` active rows, top-6 of 64 experts each (tokens = 8: up to 48 distinct experts)."""
     import numpy as np
     E, hidden, inter, top_k, layers = 64, 2048, 1408, 6, 2
+    routes = tokens * top_k
     per = bits / 8 + 4 / 64
     rng = np.random.Generator(np.random.PCG64(5))
-    x, res = _bf16(hidden, 1), _bf16(hidden, 2)
-    row_idx = fk.DeviceBuffer.from_numpy(np.zeros(top_k, np.uint32))       # every route reads the one token
-    h_rows = fk.DeviceBuffer.from_numpy(np.arange(top_k, dtype=np.uint32))  # route r reads row r of the SwiGLU output
+    x, res = _bf16(tokens * hidden, 1), _bf16(tokens * hidden, 2)
+    row_idx = fk.DeviceBuffer.from_numpy(np.repeat(np.arange(tokens, dtype=np.uint32), top_k))  # route r reads its token's row
+    h_rows = fk.DeviceBuffer.from_numpy(np.arange(routes, dtype=np.uint32))  # route r reads row r of the SwiGLU output
     m1, m2, keep = [], [], []
     for L in range(layers):
         Wg, Wu = _rand_weight(inter, hidden, bits, 300 + 10 * L, experts=E), _rand_weight(inter, hidden, bits, 303 + 10 * L, experts=E)
         Wd = _rand_weight(hidden, inter, bits, 306 + 10 * L, experts=E)
         keep.append((Wg, Wu, Wd))
+    distinct = []
     for i in range(16):
         Wg, Wu, Wd = keep[i % layers]
-        eidx = fk.DeviceBuffer.from_numpy(rng.permutation(E)[:top_k].astype(np.uint32))
-        rwt = _bf16(top_k, 50 + i, 0.2)
-        h, out = fk.DeviceBuffer(top_k * inter * 2), fk.DeviceBuffer(hidden * 2)
-        ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(1, top_k, hidden))
+        ids = np.concatenate([rng.permutation(E)[:top_k] for _ in range(tokens)]).astype(np.uint32)
+        distinct.append(len(set(ids.tolist())))
+        eidx = fk.DeviceBuffer.from_numpy(ids)
+        rwt = _bf16(routes, 50 + i, 0.2)
+        h, out = fk.DeviceBuffer(routes * inter * 2), fk.DeviceBuffer(tokens * hidden * 2)
+        ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, hidden))
         keep.append((eidx, rwt, h, out, ws))
         m1.append(Dispatch("fusekit_routed_qmv_swiglu_f0",
                            [arg(x), arg(Wg.w), arg(Wg.scales), arg(Wg.biases), arg(Wu.w), arg(Wu.scales), arg(Wu.biases),
                             arg(row_idx), arg(eidx), arg(h)],
-                           {"bits": bits, "k": hidden, "o": inter, "experts": E, "routes": top_k, "x_rows": 1}))
+                           {"bits": bits, "k": hidden, "o": inter, "experts": E, "routes": routes, "x_rows": tokens}))
         m2.append(Dispatch("fusekit_routed_qmv_reduce_f0",
                            [arg(h), arg(Wd.w), arg(Wd.scales), arg(Wd.biases), arg(h_rows), arg(eidx), arg(rwt),
                             arg(res), arg(out), arg(ws)],
-                           {"bits": bits, "k": inter, "o": hidden, "experts": E, "tokens": 1, "top_k": top_k,
-                            "x_rows": top_k, "has_extra": 1}))
-    b1 = top_k * 2 * inter * hidden * per + hidden * 2 + top_k * inter * 2
-    b2 = top_k * hidden * inter * per + top_k * inter * 2 + 2 * hidden * 2
-    _emit(f"routed_qmv_swiglu_cfg5_q{bits}", _time_graph(d, m1, reps), b1, routes=top_k, experts=E)
-    _emit(f"routed_qmv_reduce_cfg5_q{bits}", _time_graph(d, m2, reps), b2, routes=top_k, experts=E,
+                           {"bits": bits, "k": inter, "o": hidden, "experts": E, "tokens": tokens, "top_k": top_k,
+                            "x_rows": routes, "has_extra": 1}))
+    uniq = sum(distinct) / len(distinct)  # an expert chosen by several rows is streamed once per route here
+    b1 = routes * 2 * inter * hidden * per + tokens * hidden * 2 + routes * inter * 2
+    b2 = routes * hidden * inter * per + routes * inter * 2 + 2 * tokens * hidden * 2
+    tag = f"cfg5_q{bits}" + (f"_rows{tokens}" if tokens > 1 else "")
+    _emit(f"routed_qmv_swiglu_{tag}", _time_graph(d, m1, reps), b1, flops=2.0 * routes * 2 * inter * hidden, routes=routes,
+          experts=E, distinct_experts=round(uniq, 1))
+    _emit(f"routed_qmv_reduce_{tag}", _time_graph(d, m2, reps), b2, flops=2.0 * routes * inter * hidden, routes=routes, experts=E,
           note="three kernels: routed GEMV, ordered reduction")
 
 
@@ -256,6 +264,7 @@ CASES = {
     "sdpa_prefill_r512_512": lambda d, r: case_sdpa_prefill(d, r, 512, 512),
     "sdpa_prefill_r512_4096": lambda d, r: case_sdpa_prefill(d, r, 512, 4096),
     "moe_cfg5": lambda d, r: case_moe(d, r),
+    "moe_cfg5_rows8": lambda d, r: case_moe(d, r, tokens=8),
     "qgemm_8": lambda d, r: case_qgemm(d, r, 8),
     "qgemm_32": lambda d, r: case_qgemm(d, r, 32),
     "qgemm_128": lambda d, r: case_qgemm(d, r, 128),
