@@ -420,6 +420,14 @@ fk_status fk_kv_cache_store_quant(const uint16_t* k, const uint16_t* v, const ui
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_kv_cache_dequant(const fk_kv_quant_cache* cache, uint32_t n_kv, uint32_t dim, uint32_t capacity, uint32_t bits,
+                              uint32_t group, uint32_t rows, uint16_t* out, uint32_t out_capacity, fk_stream s) {
+    if (!cache) return set_error(FK_ERR_INVALID, "fk_kv_cache_dequant: null cache");
+    Launch l;
+    FK_TRY(plan_kv_dequant(cache->packed, cache->scales, cache->biases, n_kv, dim, capacity, bits, group, rows, out, out_capacity, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_sdpa_decode_quant(const uint16_t* q, const fk_kv_quant_cache* cache_k, const fk_kv_quant_cache* cache_v,
                                uint16_t* out, const uint32_t* d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t rows,
                                uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity,

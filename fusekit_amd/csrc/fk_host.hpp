@@ -153,6 +153,10 @@ struct KvQuantStore {
     float eps, base_log2;
 };
 fk_status plan_kv_store_quant(const KvQuantStore& in, Launch* out);
+// rows [0, rows) of a quantised cache as bf16 [n_kv, out_capacity, dim] (operand of the prefill attention)
+fk_status plan_kv_dequant(const uint32_t* packed, const uint16_t* scales, const uint16_t* biases, uint32_t n_kv, uint32_t dim,
+                          uint32_t capacity, uint32_t bits, uint32_t group, uint32_t rows, uint16_t* out, uint32_t out_capacity,
+                          Launch* l);
 // RoPE (+ head norm) of q and the new k row, the cache append and the attention in one launch:
 // q / k_new / v_new are the raw projection outputs; the cache pointers of plan_sdpa_decode are
 // the cache the rows are appended to.

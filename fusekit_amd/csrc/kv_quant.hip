@@ -119,4 +119,63 @@ fk_status plan_kv_store_quant(const KvQuantStore& in, Launch* out) {
     return FK_OK;
 }
 
+// Rows [0, rows) of every head of a quantised cache as bf16, T(code * scale + bias): the operand
+// form the matrix-core prefill attention takes (a prompt pass dequantises the visible prefix once per
+// layer, a few MB, instead of running the single-row kernel once per row).  One thread per packed word.
+struct KvDequantArgs {
+    const uint32_t* packed;
+    const uint16_t* scales;
+    const uint16_t* biases;
+    uint16_t* out;  // [n_kv, out_capacity, dim]
+    uint32_t n_kv, dim, capacity, out_capacity, rows, bits, group;
+};
+
+__global__ __launch_bounds__(256) void kv_dequant_kernel(const KvDequantArgs a) {
+    const uint32_t per_word = 32u / a.bits, wpr = a.dim / per_word;
+    const size_t total = (size_t)a.n_kv * a.rows * wpr;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const uint32_t w = (uint32_t)(i % wpr);
+        const size_t hr = i / wpr;
+        const uint32_t row = (uint32_t)(hr % a.rows), h = (uint32_t)(hr / a.rows);
+        const size_t src_row = (size_t)h * a.capacity + row;
+        const uint32_t g = (w * per_word) / a.group;
+        const float s = bf16_bits_to_f32(a.scales[src_row * (a.dim / a.group) + g]);
+        const float b = bf16_bits_to_f32(a.biases[src_row * (a.dim / a.group) + g]);
+        const uint32_t word = a.packed[src_row * wpr + w];
+        uint16_t* dst = a.out + ((size_t)h * a.out_capacity + row) * a.dim + w * per_word;
+        auto dq = [&](uint32_t code) { return fmaf((float)code, s, b); };
+        if (a.bits == 4) {
+            *reinterpret_cast<uint4*>(dst) =
+                make_uint4(pack_bf16(dq(word & 15u), dq((word >> 4) & 15u)), pack_bf16(dq((word >> 8) & 15u), dq((word >> 12) & 15u)),
+                           pack_bf16(dq((word >> 16) & 15u), dq((word >> 20) & 15u)), pack_bf16(dq((word >> 24) & 15u), dq(word >> 28)));
+        } else {
+            *reinterpret_cast<uint2*>(dst) =
+                make_uint2(pack_bf16(dq(word & 255u), dq((word >> 8) & 255u)), pack_bf16(dq((word >> 16) & 255u), dq(word >> 24)));
+        }
+    }
+}
+
+fk_status plan_kv_dequant(const uint32_t* packed, const uint16_t* scales, const uint16_t* biases, uint32_t n_kv, uint32_t dim,
+                          uint32_t capacity, uint32_t bits, uint32_t group, uint32_t rows, uint16_t* out, uint32_t out_capacity,
+                          Launch* l) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!packed || !scales || !biases || !out) return set_error(FK_ERR_INVALID, "kv dequant: null pointer");
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, "kv dequant: bits must be 4 or 8");
+    if (group != 32 && group != 64 && group != 128) return set_error(FK_ERR_UNSUPPORTED, "kv dequant: group size must be 32, 64 or 128");
+    if (n_kv == 0 || dim == 0 || dim % group || dim % 8u) return set_error(FK_ERR_INVALID, "kv dequant: head dim must be a multiple of the group size");
+    if (rows == 0 || rows > capacity || rows > out_capacity) return set_error(FK_ERR_INVALID, "kv dequant: rows must fit both caches");
+    if (reinterpret_cast<uintptr_t>(out) & 15u) return set_error(FK_ERR_INVALID, "kv dequant: output must be 16-byte aligned");
+    KvDequantArgs a{packed, scales, biases, out, n_kv, dim, capacity, out_capacity, rows, bits, group};
+    const size_t total = (size_t)n_kv * rows * (dim * bits / 32u);
+    size_t blocks = (total + 255) / 256;
+    if (blocks > (size_t)dev->cus * 16) blocks = (size_t)dev->cus * 16;
+    l->func = reinterpret_cast<const void*>(&kv_dequant_kernel);
+    l->grid = dim3((uint32_t)blocks, 1, 1);
+    l->block = dim3(256, 1, 1);
+    l->shmem = 0;
+    l->set_args(a);
+    return FK_OK;
+}
+
 }  // namespace fk

@@ -345,13 +345,16 @@ class DecoderRuntime:
                      for n, k in ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
             # only the single-row attention kernel (quantised cache, other head dimensions) needs a workspace
             pb, cb = (native.sdpa_workspace_bytes(c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.capacity)
-                      if c.kv_bits or c.head_dim not in (64, 128) else (0, 0))
+                      if c.head_dim not in (64, 128) else (0, 0))
             self._rows = dict(
                 tok=DeviceBuffer(4 * R), x=DeviceBuffer(R * c.hidden * 2), x2=DeviceBuffer(R * c.hidden * 2),
                 xn=DeviceBuffer(R * c.hidden * 2), q=DeviceBuffer(R * c.n_q * 2), k=DeviceBuffer(R * c.n_kvd * 2),
                 v=DeviceBuffer(R * c.n_kvd * 2), att=DeviceBuffer(R * c.n_q * 2), mid=DeviceBuffer(R * c.inter * 2),
                 ws=DeviceBuffer(2 * ws), part=DeviceBuffer(max(pb, 4) * R), cnt=native.zeros(max(cb, 4) * R),
                 rope=DeviceBuffer(R * c.head_dim * 4))
+            if c.kv_bits and c.head_dim in (64, 128):  # the dequantised prefix of one layer's cache, reused by every layer
+                self._rows["kdq"] = DeviceBuffer(c.n_kv * c.capacity * c.head_dim * 2)
+                self._rows["vdq"] = DeviceBuffer(c.n_kv * c.capacity * c.head_dim * 2)
         b = self._rows
         emb = w.mats["embed_tokens"]
         head = w.mats.get("lm_head", emb)
@@ -376,8 +379,15 @@ class DecoderRuntime:
                                                c.theta, c.eps, m, pos, c.capacity, None, None, rope_tab=b["rope"])
                     native.kv_cache_store_quant(b["k"], b["v"], kn, c.n_kv, c.head_dim, c.head_dim, c.theta, c.eps,
                                                 None, pos, m, self.cache_k[l], self.cache_v[l])
-                    native.sdpa_decode_quant(b["q"], self.cache_k[l], self.cache_v[l], b["att"], None, pos + 1,
-                                             pos + m, m, c.n_heads, scale, b["part"], b["cnt"])
+                    if c.head_dim in (64, 128):
+                        # the visible prefix as bf16 (a few MB per layer), then the matrix-core attention
+                        native.kv_cache_dequant(self.cache_k[l], pos + m, b["kdq"], c.capacity)
+                        native.kv_cache_dequant(self.cache_v[l], pos + m, b["vdq"], c.capacity)
+                        native.sdpa_prefill(b["q"], b["kdq"], b["vdq"], b["att"], m, pos + m, c.n_heads, c.n_kv, c.head_dim,
+                                            c.capacity, scale)
+                    else:
+                        native.sdpa_decode_quant(b["q"], self.cache_k[l], self.cache_v[l], b["att"], None, pos + 1,
+                                                 pos + m, m, c.n_heads, scale, b["part"], b["cnt"])
                 else:
                     native.qkv_rope_store_rows(b["q"], b["k"], b["v"], qn, kn, c.n_heads, c.n_kv, c.head_dim, c.head_dim,
                                                c.theta, c.eps, m, pos, c.capacity, self.cache_k[l], self.cache_v[l],

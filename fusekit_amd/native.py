@@ -295,6 +295,13 @@ class QuantKvCache:
         return self.packed.nbytes + self.scales.nbytes + self.biases.nbytes
 
 
+def kv_cache_dequant(cache: "QuantKvCache", rows: int, out, out_capacity: int, stream=None):
+    """Rows [0, rows) of a quantised cache as bf16 [n_kv, out_capacity, dim]."""
+    check(lib.fk_kv_cache_dequant(C.byref(cache.c), C.c_uint32(cache.n_kv), C.c_uint32(cache.dim), C.c_uint32(cache.capacity),
+                                  C.c_uint32(cache.bits), C.c_uint32(cache.group), C.c_uint32(rows), _ptr(out),
+                                  C.c_uint32(out_capacity), _ptr(stream)))
+
+
 def kv_cache_store_quant(k, v, k_norm, n_kv, head_dim, rope_dims, theta, eps, d_offset, offset, rows, K: QuantKvCache,
                          V: QuantKvCache, stream=None):
     check(lib.fk_kv_cache_store_quant(_ptr(k), _ptr(v), _ptr(k_norm), C.c_uint32(n_kv), C.c_uint32(head_dim),

@@ -279,6 +279,12 @@ fk_status fk_kv_cache_store_quant(const uint16_t *k, const uint16_t *v, const ui
                                   const uint32_t *d_offset, uint32_t offset, uint32_t rows, uint32_t capacity,
                                   uint32_t bits, uint32_t group, const fk_kv_quant_cache *cache_k,
                                   const fk_kv_quant_cache *cache_v, fk_stream s);
+/* Rows [0, rows) of every head of a quantised cache as bf16 [n_kv, out_capacity, dim], T(code * scale + bias):
+ * the operand form of fk_sdpa_prefill, so that a prompt pass over a quantised cache runs the matrix-core
+ * attention on the dequantised prefix (an MI355X addition; the reference's prefill variants keep a bf16 cache). */
+fk_status fk_kv_cache_dequant(const fk_kv_quant_cache *cache, uint32_t n_kv, uint32_t dim, uint32_t capacity,
+                              uint32_t bits, uint32_t group, uint32_t rows, uint16_t *out, uint32_t out_capacity,
+                              fk_stream s);
 fk_status fk_sdpa_decode_quant(const uint16_t *q, const fk_kv_quant_cache *cache_k, const fk_kv_quant_cache *cache_v,
                                uint16_t *out, const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len,
                                uint32_t rows, uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim,

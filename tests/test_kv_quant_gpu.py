@@ -111,6 +111,37 @@ def test_attention_over_quantised_cache(fk, bits, n_heads, n_kv, dim, group, kv_
         assert np.max(np.abs(oracle.bf16_to_f32(got) - oracle.bf16_to_f32(want))) <= 2.0 ** -6 * np.max(np.abs(oracle.bf16_to_f32(want)))
 
 
+@pytest.mark.parametrize("bits,group,dim", [(4, 64, 128), (8, 64, 128), (4, 32, 64)])
+def test_dequantised_prefix_and_prefill_attention(fk, bits, group, dim):
+    """fk_kv_cache_dequant gives T(code * scale + bias) bit for bit (rows past the prefix untouched), and the
+    matrix-core prefill attention over it agrees with the quantised-cache oracle row by row."""
+    n_heads, n_kv, cap, rows, kv_len = 8, 2, 96, 40, 70
+    rs = rng(17)
+    oK, oV = oracle.QuantCache(n_kv, cap, dim, bits, group), oracle.QuantCache(n_kv, cap, dim, bits, group)
+    for c in (oK, oV):
+        c.packed[:] = rs.integers(0, 2 ** 32, c.packed.shape, dtype=np.uint32)
+        c.scales[:] = oracle.f32_to_bf16((rs.standard_normal(c.scales.shape) * 0.02 + (0.1 if bits == 4 else 0.008)).astype(np.float32))
+        c.biases[:] = oracle.f32_to_bf16((rs.standard_normal(c.biases.shape) * 0.3 - (0.7 if bits == 4 else 1.0)).astype(np.float32))
+    K, V = _caches(fk, n_kv, cap, dim, bits, group)
+    _upload(fk, oK, K), _upload(fk, oV, V)
+    kdq, vdq = fk.zeros(n_kv * cap * dim * 2), fk.zeros(n_kv * cap * dim * 2)
+    fk.kv_cache_dequant(K, kv_len, kdq, cap)
+    fk.kv_cache_dequant(V, kv_len, vdq, cap)
+    got_k = kdq.to_numpy(np.uint16).reshape(n_kv, cap, dim)
+    want_k = oracle.f32_to_bf16(oK.dequantize().astype(np.float32)).reshape(n_kv, cap, dim)
+    assert np.array_equal(got_k[:, :kv_len], want_k[:, :kv_len]) and not got_k[:, kv_len:].any()
+    q = normal_bf16(19, (rows, n_heads * dim))
+    out = fk.DeviceBuffer(rows * n_heads * dim * 2)
+    scale = dim ** -0.5
+    fk.sdpa_prefill(_dev(fk, q), kdq, vdq, out, rows, kv_len, n_heads, n_kv, dim, cap, scale)
+    got = out.to_numpy(np.uint16).reshape(rows, n_heads * dim)
+    for r in range(rows):
+        want = oracle.sdpa_decode_quant(q[r], oK, oV, n_heads, kv_len - rows + r + 1, scale)
+        assert rel_l2(got[r], oracle.bf16_to_f32(want)) <= 1e-2, r
+    with pytest.raises(fk.FusekitError):
+        fk.kv_cache_dequant(K, cap + 1, kdq, cap)
+
+
 def test_store_then_attend_matches_bf16_cache(fk):
     """Round trip at 8 bits: rows stored quantised and attended give the plain bf16-cache attention to
     within the quantisation noise (a size-independent property: no oracle involved)."""
