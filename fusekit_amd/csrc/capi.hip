@@ -381,6 +381,36 @@ fk_status fk_rope_kv_cache_store_decode(const uint16_t* k, const uint16_t* v, co
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_kv_cache_store_split_decode(uint16_t* q, uint32_t n_heads, uint32_t q0_dim, uint32_t q1_dim,
+                                         const uint16_t* k0, uint32_t k0_stride, const uint16_t* k1, uint32_t k1_heads,
+                                         const uint16_t* v, uint32_t v_stride, uint32_t n_kv, uint32_t k0_dim,
+                                         uint32_t k1_dim, uint32_t v_dim, uint32_t rope_dims, int traditional,
+                                         float theta, const uint32_t* d_offset, uint32_t offset,
+                                         const uint32_t* d_write_offset, uint32_t write_offset, uint32_t capacity,
+                                         uint16_t* cache_k, uint16_t* cache_v, fk_stream s) {
+    SplitStoreArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.n_heads = n_heads; a.q0_dim = q0_dim; a.q1_dim = q1_dim;
+    a.k0 = k0; a.k0_stride = k0_stride; a.k1 = k1; a.k1_heads = k1_heads; a.v = v; a.v_stride = v_stride;
+    a.n_kv = n_kv; a.k0_dim = k0_dim; a.k1_dim = k1_dim; a.v_dim = v_dim;
+    a.rope_dims = rope_dims; a.traditional = traditional ? 1u : 0u;
+    a.base_log2 = rope_dims ? theta_log2(theta) : 0.f;
+    a.offset_ptr = d_offset; a.offset_imm = offset;
+    a.write_offset_ptr = d_write_offset; a.write_offset_imm = write_offset; a.use_write_imm = 1;
+    a.capacity = capacity;
+    a.cache_k = cache_k; a.cache_v = cache_v;
+    Launch l;
+    FK_TRY(plan_split_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, int scale_per_route, uint32_t rows,
+                                uint32_t row_n, uint32_t top_k, uint32_t* idx, uint16_t* weight, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_softmax_topk_route(logits, scale, scale_per_route != 0, rows, row_n, top_k, idx, weight, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_qkv_rope_store_decode(uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_norm,
                                    const uint16_t* k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                    uint32_t rope_dims, float theta, float eps, const uint32_t* d_offset,

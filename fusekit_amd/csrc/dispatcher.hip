@@ -319,6 +319,76 @@ fk_status plan_rope_q(const Dispatch& d, Launch* l, SlotRW* rw, bool norm) {
     return plan_rope_store(a, l);
 }
 
+// [Q], K0, K1, V, cache_k, cache_v, offset, write_offset: the split-key form of kv_cache_store_decode
+// (kv_cache_store_decode.rs:206-214), with has_q = 1 also the in-place rotation of the query's second part.
+// Parameters: n_kv, k0_dim, k1_dim, v_dim, k1_n_kv, k0_stride, v_stride, rope_dims, traditional, theta,
+// capacity; with a query n_heads, q0_dim, q1_dim.
+fk_status plan_kv_store_split(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const bool has_q = d.u("has_q", 0) != 0;
+    const size_t b = has_q ? 1 : 0;
+    FK_TRY(need_args(d, b + 7));
+    SplitStoreArgs a;
+    memset(&a, 0, sizeof(a));
+    a.n_kv = d.u("n_kv");
+    a.k0_dim = d.u("k0_dim");
+    a.k1_dim = d.u("k1_dim");
+    a.v_dim = d.u("v_dim");
+    a.k1_heads = d.u("k1_n_kv", a.n_kv);
+    a.k0_stride = d.u("k0_stride", a.k0_dim);
+    a.v_stride = d.u("v_stride", a.v_dim);
+    a.rope_dims = d.u("rope_dims", 0);
+    a.traditional = d.u("traditional", 0);
+    a.capacity = d.u("capacity");
+    if (a.n_kv == 0 || a.k0_dim == 0 || a.k1_dim == 0 || a.v_dim == 0 || a.capacity == 0 || a.k1_heads == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_kv / k0_dim / k1_dim / v_dim / capacity parameters missing");
+    if (a.k0_stride < a.k0_dim || a.v_stride < a.v_dim) return set_error(FK_ERR_INVALID, d.kernel + ": stride below the row width");
+    if (has_q) {
+        a.n_heads = d.u("n_heads");
+        a.q0_dim = d.u("q0_dim");
+        a.q1_dim = d.u("q1_dim");
+        if (a.n_heads == 0) return set_error(FK_ERR_INVALID, d.kernel + ": n_heads parameter missing");
+        FK_TRY(need_bytes(d, 0, (size_t)a.n_heads * (a.q0_dim + a.q1_dim) * 2));
+        a.q = arg_ptr<uint16_t>(d, 0);
+    }
+    FK_TRY(need_bytes(d, b, ((size_t)(a.n_kv - 1) * a.k0_stride + a.k0_dim) * 2));
+    FK_TRY(need_bytes(d, b + 1, (size_t)a.k1_heads * a.k1_dim * 2));
+    FK_TRY(need_bytes(d, b + 2, ((size_t)(a.n_kv - 1) * a.v_stride + a.v_dim) * 2));
+    FK_TRY(need_bytes(d, b + 3, (size_t)a.n_kv * a.capacity * (a.k0_dim + a.k1_dim) * 2));
+    FK_TRY(need_bytes(d, b + 4, (size_t)a.n_kv * a.capacity * a.v_dim * 2));
+    FK_TRY(need_bytes(d, b + 5, 4));
+    FK_TRY(need_bytes(d, b + 6, 4));
+    a.k0 = arg_ptr<const uint16_t>(d, b);
+    a.k1 = arg_ptr<const uint16_t>(d, b + 1);
+    a.v = arg_ptr<const uint16_t>(d, b + 2);
+    a.cache_k = arg_ptr<uint16_t>(d, b + 3);
+    a.cache_v = arg_ptr<uint16_t>(d, b + 4);
+    a.offset_ptr = arg_ptr<const uint32_t>(d, b + 5);
+    a.write_offset_ptr = arg_ptr<const uint32_t>(d, b + 6);
+    a.base_log2 = a.rope_dims ? base_log2_of(d) : 0.f;
+    for (uint32_t i = 0; i < b + 7; ++i)
+        if (i != b + 3 && i != b + 4) rw->reads.push_back(i);
+    rw->writes = {(uint32_t)(b + 3), (uint32_t)(b + 4)};
+    if (has_q) rw->writes.push_back(0);
+    return plan_split_rope_store(a, l);
+}
+
+// logits, scale, idx, weight (SoftmaxTopKRoute, single.rs:2615-2760).  Parameters: row_n, top_k, rows,
+// scale_per_route.
+fk_status plan_softmax_topk_route_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 4));
+    const uint32_t row_n = d.u("row_n"), top_k = d.u("top_k"), rows = d.u("rows", 1);
+    const bool per_route = d.u("scale_per_route", 0) != 0;
+    if (row_n == 0 || top_k == 0 || rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": row_n / top_k parameters missing");
+    FK_TRY(need_bytes(d, 0, (size_t)rows * row_n * 2));
+    FK_TRY(need_bytes(d, 1, per_route ? (size_t)rows * top_k * 2 : 2));
+    FK_TRY(need_bytes(d, 2, (size_t)rows * top_k * 4));
+    FK_TRY(need_bytes(d, 3, (size_t)rows * top_k * 2));
+    rw->reads = {0, 1};
+    rw->writes = {2, 3};
+    return plan_softmax_topk_route(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), per_route, rows, row_n, top_k,
+                                   arg_ptr<uint32_t>(d, 2), arg_ptr<uint16_t>(d, 3), l);
+}
+
 // K, V, [k_weight], cache_k, cache_v, offset, write_offset
 fk_status plan_rope_kv(const Dispatch& d, Launch* l, SlotRW* rw, bool norm, bool rope) {
     const size_t n = norm ? 7 : 6;
@@ -791,7 +861,10 @@ const Family kFamilies[] = {
     {"fusekit_rope_kv_cache_store_decode",
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, true); }},
     {"fusekit_kv_cache_store_decode",
-     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv(d, l, rw, false, false); }},
+     [](const Dispatch& d, Launch* l, SlotRW* rw) {
+         return d.u("split_k", 0) ? plan_kv_store_split(d, l, rw) : plan_rope_kv(d, l, rw, false, false);
+     }},
+    {"fusekit_softmax_topk_route", plan_softmax_topk_route_d},
     {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
     {"fusekit_sdpa_decode", plan_sdpa_d},
     {"fusekit_sdpa_prefill", plan_sdpa_prefill_d},

@@ -131,6 +131,28 @@ fk_status plan_rope_store(const RopeArgs& in, Launch* out);
 // rope/store kernel would compute itself, filled once per prompt pass for all layers and heads.
 fk_status plan_rope_table(float* tab, uint32_t rope_dims, float base_log2, uint32_t offset, uint32_t rows, Launch* out);
 
+// Cache store of a key given as two parts [K0 | K1] with K1 rotated while written, plus the same
+// rotation of the query's second part in place (mla.hip).
+struct SplitStoreArgs {
+    uint16_t* q;             // packed [n_heads, q0_dim + q1_dim]; Q1 rotated in place; null with n_heads = 0
+    const uint16_t* k0;      // n_kv rows of k0_dim, k0_stride elements apart
+    const uint16_t* k1;      // [k1_heads, k1_dim], k1_heads = 1 (shared) or n_kv
+    const uint16_t* v;       // n_kv rows of v_dim, v_stride elements apart
+    uint16_t* cache_k;       // [n_kv, capacity, k0_dim + k1_dim]
+    uint16_t* cache_v;       // [n_kv, capacity, v_dim]
+    const uint32_t* offset_ptr;        // rotary position (device) or null -> offset_imm
+    const uint32_t* write_offset_ptr;  // cache row before the modulo, or null
+    uint32_t offset_imm, write_offset_imm;
+    uint32_t use_write_imm;  // with a null write_offset_ptr: 1 = write_offset_imm, 0 = the position
+    uint32_t n_heads, q0_dim, q1_dim;
+    uint32_t n_kv, k0_dim, k1_dim, v_dim, k0_stride, v_stride, k1_heads;
+    uint32_t rope_dims, traditional, capacity;
+    float base_log2;
+};
+fk_status plan_split_rope_store(const SplitStoreArgs& a, Launch* out);
+fk_status plan_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, bool scale_per_route, uint32_t rows,
+                                  uint32_t row_n, uint32_t top_k, uint32_t* idx, uint16_t* weight, Launch* out);
+
 // Quantised KV cache (mlx-lm QuantizedKVCache layout): packed uint32 [n_kv, capacity, dim*bits/32],
 // scales / biases bf16 [n_kv, capacity, dim/group].
 struct KvQuant {

@@ -1,0 +1,166 @@
+// The two small kernels a mixture-of-experts decoder with low-rank (MLA-style) keys needs next to
+// the streaming kernels: the cache store of a key given in two parts, and the router.
+// Both are launch-latency sized; what matters is one launch each and the reference's rounding.
+#include "fk_host.hpp"
+#include "fk_device.hpp"
+#include "rope_device.hpp"
+
+namespace fk {
+
+// ------------------------------------------------ split-key cache store (+ rotation of Q1)
+//
+// Cache K row = [K0 | K1] (src/codegen/kernels/kv_cache_store_decode.rs:268-352): K0 holds n_kv
+// heads, K1 n_kv heads or ONE head shared by all of them; the first rope_dims of K1 are rotated at
+// the token's position while written, as traditional (2i, 2i+1) or half-split (i, i + half) pairs.
+// K0 and V rows are k0_stride / v_stride elements apart, so both may alias one packed
+// [n_kv, k0_dim + v_dim] projection output (:103-140).  The query's second part, Q1 of the packed
+// [n_heads, q0_dim + q1_dim] rows, gets the same rotation in place and is rounded to T, which is
+// what the rotary op writes when it is not sunk into the attention kernel
+// (sdpa_decode.rs:592-660 keeps fp32 there).
+// One wave per head: blocks [0, n_heads) the query heads, then n_kv key heads, then n_kv value heads.
+__global__ __launch_bounds__(kWave) void split_rope_store_kernel(const SplitStoreArgs a) {
+    uint32_t b = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t pos = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
+    const uint32_t wpos = a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos);
+    const uint32_t row = wpos % a.capacity;
+    const uint32_t half = a.rope_dims / 2;
+
+    auto rotate = [&](const uint16_t* src, uint16_t* dst) __attribute__((always_inline)) {
+        for (uint32_t i = lane; i < half; i += kWave) {
+            const uint32_t lo_i = a.traditional ? 2 * i : i, hi_i = a.traditional ? 2 * i + 1 : i + half;
+            float lo, hi;
+            rope_rotate(bf16_bits_to_f32(src[lo_i]), bf16_bits_to_f32(src[hi_i]), i, half, pos, a.base_log2, lo, hi);
+            dst[lo_i] = (uint16_t)f32_to_bf16_bits(lo);
+            dst[hi_i] = (uint16_t)f32_to_bf16_bits(hi);
+        }
+    };
+    if (b < a.n_heads) {
+        uint16_t* q1 = a.q + (size_t)b * (a.q0_dim + a.q1_dim) + a.q0_dim;
+        rotate(q1, q1);
+        return;
+    }
+    b -= a.n_heads;
+    if (b < a.n_kv) {
+        uint16_t* dst = a.cache_k + ((size_t)b * a.capacity + row) * (a.k0_dim + a.k1_dim);
+        const uint16_t* k0 = a.k0 + (size_t)b * a.k0_stride;
+        for (uint32_t d = lane; d < a.k0_dim; d += kWave) dst[d] = k0[d];
+        const uint16_t* k1 = a.k1 + (size_t)(a.k1_heads == 1 ? 0 : b) * a.k1_dim;
+        rotate(k1, dst + a.k0_dim);
+        for (uint32_t d = 2 * half + lane; d < a.k1_dim; d += kWave) dst[a.k0_dim + d] = k1[d];
+        return;
+    }
+    b -= a.n_kv;
+    uint16_t* dst = a.cache_v + ((size_t)b * a.capacity + row) * a.v_dim;
+    const uint16_t* v = a.v + (size_t)b * a.v_stride;
+    for (uint32_t d = lane; d < a.v_dim; d += kWave) dst[d] = v[d];
+}
+
+fk_status plan_split_rope_store(const SplitStoreArgs& a, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!a.k0 || !a.k1 || !a.v || !a.cache_k || !a.cache_v) return set_error(FK_ERR_INVALID, "split store: null pointer");
+    if (a.n_heads && !a.q) return set_error(FK_ERR_INVALID, "split store: query heads without a query");
+    if (a.n_kv == 0 || a.k0_dim == 0 || a.k1_dim == 0 || a.v_dim == 0 || a.capacity == 0)
+        return set_error(FK_ERR_INVALID, "split store: empty shape");
+    if (a.k1_heads != 1 && a.k1_heads != a.n_kv)
+        return set_error(FK_ERR_INVALID, "split store: K1 has one head or one per KV head");
+    if (a.k0_stride < a.k0_dim || a.v_stride < a.v_dim) return set_error(FK_ERR_INVALID, "split store: stride below the row width");
+    if (a.rope_dims % 2 || a.rope_dims > a.k1_dim || (a.n_heads && a.rope_dims > a.q1_dim))
+        return set_error(FK_ERR_INVALID, "split store: rope_dims must be even and within K1 (and Q1)");
+    if (a.n_heads && a.q0_dim + a.q1_dim != a.k0_dim + a.k1_dim)
+        return set_error(FK_ERR_INVALID, "split store: query and key widths differ");
+    out->func = reinterpret_cast<const void*>(&split_rope_store_kernel);
+    out->grid = dim3(a.n_heads + 2 * a.n_kv, 1, 1);
+    out->block = dim3(kWave, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+// ------------------------------------------------------------------ softmax top-k route
+//
+// Router of a mixture-of-experts block (src/codegen/kernels/single.rs:2615-2760): softmax over
+// row_n logits, prob = float(T(exp(score - max) * (1 / sum))) rounded to T BEFORE the ordering,
+// the top_k largest in descending order with ties to the lower index, weight = T(prob * scale) with
+// one scale per row set or one per route.  row_n is a power of two of at most 256, top_k < row_n
+// and at most 32 (the reference's admission, :2636-2641).  One wave per row; a lane holds four
+// probabilities and the selection is top_k rounds of a wave-wide arg-max.
+struct RouteArgs {
+    const uint16_t* logits;
+    const uint16_t* scale;
+    uint32_t* idx;
+    uint16_t* weight;
+    uint32_t row_n, top_k, scale_per_route;
+};
+__global__ __launch_bounds__(kWave) void softmax_topk_route_kernel(const RouteArgs a) {
+    const uint32_t r = blockIdx.x, lane = threadIdx.x;
+    const uint16_t* l = a.logits + (size_t)r * a.row_n;
+    float x[4], p[4];
+    float m = -INFINITY;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t i = lane + j * kWave;
+        x[j] = i < a.row_n ? bf16_bits_to_f32(l[i]) : -INFINITY;
+        m = fmaxf(m, x[j]);
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        p[j] = lane + j * kWave < a.row_n ? expf(x[j] - m) : 0.f;
+        sum += p[j];
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) p[j] = lane + j * kWave < a.row_n ? round_bf16(p[j] * inv) : -1.f;  // -1: not a candidate
+    for (uint32_t k = 0; k < a.top_k; ++k) {
+        float best = -1.f;
+        uint32_t best_i = 0xffffffffu;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)   // ascending index within the lane: '>' keeps the lower one on ties
+            if (p[j] > best) {
+                best = p[j];
+                best_i = lane + j * kWave;
+            }
+#pragma unroll
+        for (uint32_t off = 1; off < kWave; off <<= 1) {
+            const float ob = __shfl_xor(best, off, kWave);
+            const uint32_t oi = __shfl_xor(best_i, off, kWave);
+            if (ob > best || (ob == best && oi < best_i)) {
+                best = ob;
+                best_i = oi;
+            }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (best_i == lane + j * kWave) p[j] = -1.f;
+        if (lane == 0) {
+            const size_t o = (size_t)r * a.top_k + k;
+            const float sc = bf16_bits_to_f32(a.scale[a.scale_per_route ? o : 0]);
+            a.idx[o] = best_i;
+            a.weight[o] = (uint16_t)f32_to_bf16_bits(best * sc);
+        }
+    }
+}
+
+fk_status plan_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, bool scale_per_route, uint32_t rows,
+                                  uint32_t row_n, uint32_t top_k, uint32_t* idx, uint16_t* weight, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!logits || !scale || !idx || !weight) return set_error(FK_ERR_INVALID, "softmax top-k route: null pointer");
+    if (rows == 0) return set_error(FK_ERR_INVALID, "softmax top-k route: no rows");
+    if (row_n < 2 || row_n > 256 || (row_n & (row_n - 1)) || top_k == 0 || top_k >= row_n || top_k > 32)
+        return set_error(FK_ERR_UNSUPPORTED,
+                         "softmax top-k route: row_n must be a power of two of at most 256, top_k below row_n and at most 32");
+    RouteArgs a{logits, scale, idx, weight, row_n, top_k, scale_per_route ? 1u : 0u};
+    out->func = reinterpret_cast<const void*>(&softmax_topk_route_kernel);
+    out->grid = dim3(rows, 1, 1);
+    out->block = dim3(kWave, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+}  // namespace fk

@@ -249,6 +249,23 @@ def rope_kv_cache_store_decode(k, v, k_norm, n_kv, k_dim, v_dim, rope_dims, thet
         _ptr(stream)))
 
 
+def kv_cache_store_split_decode(q, n_heads, q0_dim, q1_dim, k0, k0_stride, k1, k1_heads, v, v_stride, n_kv, k0_dim,
+                                k1_dim, v_dim, rope_dims, traditional, theta, d_offset, offset, d_write_offset,
+                                write_offset, capacity, cache_k, cache_v, stream=None):
+    """Cache K row = [K0 | rope(K1)], V row; with a query also rope(Q1) in place (fk_kv_cache_store_split_decode)."""
+    check(lib.fk_kv_cache_store_split_decode(
+        _ptr(q), C.c_uint32(n_heads), C.c_uint32(q0_dim), C.c_uint32(q1_dim), _ptr(k0), C.c_uint32(k0_stride), _ptr(k1),
+        C.c_uint32(k1_heads), _ptr(v), C.c_uint32(v_stride), C.c_uint32(n_kv), C.c_uint32(k0_dim), C.c_uint32(k1_dim),
+        C.c_uint32(v_dim), C.c_uint32(rope_dims), C.c_int(int(traditional)), C.c_float(theta), _ptr(d_offset),
+        C.c_uint32(offset), _ptr(d_write_offset), C.c_uint32(write_offset), C.c_uint32(capacity), _ptr(cache_k),
+        _ptr(cache_v), _ptr(stream)))
+
+
+def softmax_topk_route(logits, scale, scale_per_route, rows, row_n, top_k, idx, weight, stream=None):
+    check(lib.fk_softmax_topk_route(_ptr(logits), _ptr(scale), C.c_int(int(scale_per_route)), C.c_uint32(rows),
+                                    C.c_uint32(row_n), C.c_uint32(top_k), _ptr(idx), _ptr(weight), _ptr(stream)))
+
+
 def qkv_rope_store_decode(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope_dims, theta, eps, d_offset,
                           offset, capacity, cache_k, cache_v, stream=None):
     check(lib.fk_qkv_rope_store_decode(

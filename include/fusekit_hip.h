@@ -291,6 +291,33 @@ fk_status fk_sdpa_decode_quant(const uint16_t *q, const fk_kv_quant_cache *cache
                                uint32_t capacity, uint32_t bits, uint32_t group, float scale, float *partials,
                                uint32_t *counters, fk_stream s);
 
+/* ---- mixture-of-experts decoder with low-rank (MLA-style) keys: the glue around M1 / M2 / K4 ----
+ * fk_kv_cache_store_split_decode replaces the split-key form of KvCacheStoreDecode
+ * (src/codegen/kernels/kv_cache_store_decode.rs:84-352; attrs src/fusion/ir.rs:343-357): cache K row =
+ * [K0 | K1]; K0 has n_kv heads, K1 has k1_heads = n_kv heads or 1 head shared by all; the first rope_dims
+ * of K1 are rotated at `offset` while written (traditional != 0: pairs (2i, 2i+1), else (i, i + rope_dims/2)).
+ * K0 / V head rows start k0_stride / v_stride elements apart, so both may point into one packed
+ * [n_kv, k0_dim + v_dim] projection output (the reference's kv_transpose_split).  With n_heads > 0 the
+ * query's second part -- Q1 of the packed rows q [n_heads, q0_dim + q1_dim] -- gets the same rotation in
+ * place, rounded to bf16; the reference rotates Q1 inside its attention kernel and keeps fp32 there
+ * (src/codegen/kernels/sdpa_decode.rs:592-660), a difference of at most one bf16 rounding per rotated
+ * query element.  Offsets as in fk_rope_kv_cache_store_decode. */
+fk_status fk_kv_cache_store_split_decode(uint16_t *q, uint32_t n_heads, uint32_t q0_dim, uint32_t q1_dim,
+                                         const uint16_t *k0, uint32_t k0_stride, const uint16_t *k1, uint32_t k1_heads,
+                                         const uint16_t *v, uint32_t v_stride, uint32_t n_kv, uint32_t k0_dim,
+                                         uint32_t k1_dim, uint32_t v_dim, uint32_t rope_dims, int traditional,
+                                         float theta, const uint32_t *d_offset, uint32_t offset,
+                                         const uint32_t *d_write_offset, uint32_t write_offset, uint32_t capacity,
+                                         uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
+/* fk_softmax_topk_route replaces the router kernel SoftmaxTopKRoute (src/codegen/kernels/single.rs:2615-2760;
+ * matcher src/fusion/general.rs:6768-6880): per row softmax over row_n bf16 logits, probabilities rounded
+ * to bf16 BEFORE the ordering, the top_k largest in descending order with ties to the lower index;
+ * idx u32 [rows, top_k], weight bf16 [rows, top_k] = T(prob * scale).  scale: one bf16 value
+ * (scale_per_route = 0) or bf16 [rows, top_k].  row_n a power of two <= 256, top_k < row_n and <= 32
+ * (the reference's admission); anything else FK_ERR_UNSUPPORTED. */
+fk_status fk_softmax_topk_route(const uint16_t *logits, const uint16_t *scale, int scale_per_route, uint32_t rows,
+                                uint32_t row_n, uint32_t top_k, uint32_t *idx, uint16_t *weight, fk_stream s);
+
 /* ---- several active token rows (multi-token verification, chunked prefill) ----
  * The reference compiles such variants with active_m > 1 (src/target/mod.rs:170-200,
  * variants `prefill_mN`, src/patch.rs:103-150; causal attention

@@ -255,6 +255,40 @@ def sdpa_decode(q, cache_k, cache_v, n_heads, n_kv, qk_dim, v_dim, kv_len, capac
     return out
 
 
+def sdpa_decode_split_q(q, n_heads, q0_dim, q1_dim, rope_dims, traditional, theta, cache_k, cache_v, n_kv, v_dim,
+                        kv_len, capacity, scale) -> np.ndarray:
+    """q: packed [n_heads, q0_dim + q1_dim]; Q1's first rope_dims are rotated at kv_len - 1 in fp32."""
+    q = np.ascontiguousarray(q, dtype=np.uint16).reshape(-1)
+    out = np.empty(n_heads * v_dim, dtype=np.uint16)
+    stride = q0_dim + q1_dim
+    _lib.fko_sdpa_decode_split_q(_p(q, _u16p), C.c_int64(stride), _p(q[q0_dim:], _u16p), C.c_int64(stride),
+                                 C.c_int64(q0_dim), C.c_int64(q1_dim), C.c_int64(rope_dims), C.c_int(int(traditional)),
+                                 C.c_float(theta), _p(cache_k, _u16p), _p(cache_v, _u16p), C.c_int64(n_heads),
+                                 C.c_int64(n_kv), C.c_int64(v_dim), C.c_uint32(kv_len), C.c_uint32(capacity),
+                                 C.c_float(scale), _p(out, _u16p))
+    return out
+
+
+def kv_store_split(k0, k0_stride, k1, k1_heads, v, v_stride, n_kv, k0_dim, k1_dim, v_dim, rope_dims, traditional, theta,
+                   pos, write_offset, capacity, cache_k, cache_v):
+    """k0 / v: flat uint16 arrays whose head rows start k0_stride / v_stride elements apart."""
+    _lib.fko_kv_store_split(_p(k0, _u16p), C.c_int64(k0_stride), _p(k1, _u16p), C.c_int64(k1_heads), _p(v, _u16p),
+                            C.c_int64(v_stride), C.c_int64(n_kv), C.c_int64(k0_dim), C.c_int64(k1_dim), C.c_int64(v_dim),
+                            C.c_int64(rope_dims), C.c_int(int(traditional)), C.c_float(theta), C.c_uint32(pos),
+                            C.c_uint32(write_offset), C.c_uint32(capacity), _p(cache_k, _u16p), _p(cache_v, _u16p))
+
+
+def softmax_topk_route(logits, top_k, scale):
+    """logits bf16 [rows, row_n]; scale: one bf16 value or bf16 [rows, top_k].  Returns (idx u32, weight bf16)."""
+    logits = np.ascontiguousarray(logits, dtype=np.uint16)
+    rows, row_n = (1, logits.size) if logits.ndim == 1 else logits.shape
+    scale = np.ascontiguousarray(scale, dtype=np.uint16).reshape(-1)
+    idx, weight = np.empty(rows * top_k, np.uint32), np.empty(rows * top_k, np.uint16)
+    _lib.fko_softmax_topk_route(_p(logits, _u16p), C.c_int64(rows), C.c_int64(row_n), C.c_int64(top_k), _p(scale, _u16p),
+                                C.c_int(int(scale.size > 1)), _p(idx, C.POINTER(C.c_uint32)), _p(weight, _u16p))
+    return idx.reshape(rows, top_k), weight.reshape(rows, top_k)
+
+
 def sdpa_prefill(q, cache_k, cache_v, rows, n_heads, n_kv, dim, kv_len, capacity, scale) -> np.ndarray:
     """Causal attention of `rows` rows; kv_len counts them (row r sees kv_len - rows + r + 1 positions)."""
     out = np.empty(rows * n_heads * dim, dtype=np.uint16)

@@ -46,6 +46,14 @@
  *                                 scores before the product with V here and after it there;
  *                                 float64 causal softmax attention in numpy; row 0 of a fresh
  *                                 group returns V[0]; later cache rows never influence a row)
+ *   split-key cache store ....... pinned (equals the pinned rope + plain store on the assembled
+ *                                 [K0 | K1] row for half-split pairs; traditional pairs against
+ *                                 a numpy complex rotation; shared K1 head, packed source)
+ *   split-query attention ....... pinned (equals the pinned sdpa_decode on [Q0 | rope(Q1)] to one
+ *                                 bf16 step of the rotated query; position kv_len - 1)
+ *   softmax top-k route ......... pinned (equal logits -> 1/N exactly, indices 0..k-1; numpy
+ *                                 float64 softmax + stable sort; probabilities tie after the
+ *                                 rounding to T and the lower index wins)
  *   hand-derived known answers .. tests/golden/known_answers.json
  *   MLX-internal accumulation order, Metal fast::cos/sin/exp bit patterns:
  *                                 parity unpinned (cannot be observed here;
@@ -548,9 +556,9 @@ FKO_API void fko_sdpa_decode_quant(const uint16_t *q, const uint32_t *ck_packed,
  * rounded to T); o = sum p_j v_j / l; one final round
  * (src/codegen/kernels/sdpa_decode.rs:1064-1211); GQA kv_head = head /
  * (n_heads / n_kv) (:393); caches [n_kv, capacity, dim] (:799,868). */
-FKO_API void fko_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v,
-                             int64_t n_heads, int64_t n_kv, int64_t qk_dim, int64_t v_dim,
-                             uint32_t kv_len, uint32_t capacity, float scale, uint16_t *out) {
+static void sdpa_decode_core(const float *qf, const uint16_t *cache_k, const uint16_t *cache_v, int64_t n_heads,
+                             int64_t n_kv, int64_t qk_dim, int64_t v_dim, uint32_t kv_len, uint32_t capacity,
+                             float scale, uint16_t *out) {
     const int64_t per_kv = n_heads / n_kv;
 #pragma omp parallel for schedule(static)
     for (int64_t h = 0; h < n_heads; ++h) {
@@ -560,8 +568,7 @@ FKO_API void fko_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const u
         for (uint32_t j = 0; j < kv_len; ++j) {
             const uint16_t *kr = cache_k + (kvh * (int64_t)capacity + j) * qk_dim;
             double dot = 0.0;
-            for (int64_t d = 0; d < qk_dim; ++d)
-                dot += (double)bf16_to_f32(q[h * qk_dim + d]) * (double)bf16_to_f32(kr[d]);
+            for (int64_t d = 0; d < qk_dim; ++d) dot += (double)qf[h * qk_dim + d] * (double)bf16_to_f32(kr[d]);
             s[j] = (float)dot * scale;
             m = s[j] > m ? s[j] : m;
         }
@@ -578,6 +585,117 @@ FKO_API void fko_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const u
         }
         free(s);
     }
+}
+
+FKO_API void fko_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v,
+                             int64_t n_heads, int64_t n_kv, int64_t qk_dim, int64_t v_dim,
+                             uint32_t kv_len, uint32_t capacity, float scale, uint16_t *out) {
+    float *qf = (float *)malloc(sizeof(float) * (size_t)(n_heads * qk_dim));
+    for (int64_t i = 0; i < n_heads * qk_dim; ++i) qf[i] = bf16_to_f32(q[i]);
+    sdpa_decode_core(qf, cache_k, cache_v, n_heads, n_kv, qk_dim, v_dim, kv_len, capacity, scale, out);
+    free(qf);
+}
+
+/* One element of a rotated slice, written per element as the reference's emitters do
+ * (src/codegen/kernels/kv_cache_store_decode.rs:293-331, sdpa_decode.rs:622-652): traditional
+ * pairs are (2i, 2i+1), half-split pairs (i, i + half); inv_freq = exp2(-(i/half) * log2 base). */
+static float rope_slice_elem(const uint16_t *src, int64_t d1, int64_t rope_dims, int traditional, float base_log2,
+                             uint32_t pos) {
+    const int64_t half = rope_dims / 2;
+    const int64_t pair = traditional ? d1 / 2 : (d1 < half ? d1 : d1 - half);
+    const float d_norm = (float)pair / (float)half;
+    const float inv_freq = exp2f(-d_norm * base_log2);
+    const float angle = (float)pos * inv_freq;
+    const float c = cosf(angle), sn = sinf(angle);
+    const int64_t lo_idx = traditional ? pair * 2 : pair, hi_idx = traditional ? lo_idx + 1 : pair + half;
+    const float lo = bf16_to_f32(src[lo_idx]), hi = bf16_to_f32(src[hi_idx]);
+    const int lo_lane = traditional ? (d1 & 1) == 0 : d1 < half;
+    return lo_lane ? lo * c - hi * sn : hi * c + lo * sn;
+}
+
+/* Attention with the query given as two parts, Q = [Q0 | Q1] per head, Q1 rotated inside the
+ * kernel at position kv_len - 1 and kept in fp32 -- never rounded to T -- before the dot products
+ * (src/codegen/kernels/sdpa_decode.rs:283-294 buffers, :592-660 staging); the rest as
+ * fko_sdpa_decode.  q0 / q1 rows are q0_stride / q1_stride elements apart (one packed
+ * [n_heads, q0_dim + q1_dim] tensor: q1 = q0 + q0_dim, both strides q0_dim + q1_dim). */
+FKO_API void fko_sdpa_decode_split_q(const uint16_t *q0, int64_t q0_stride, const uint16_t *q1, int64_t q1_stride,
+                                     int64_t q0_dim, int64_t q1_dim, int64_t rope_dims, int traditional, float theta,
+                                     const uint16_t *cache_k, const uint16_t *cache_v, int64_t n_heads, int64_t n_kv,
+                                     int64_t v_dim, uint32_t kv_len, uint32_t capacity, float scale, uint16_t *out) {
+    const int64_t qk_dim = q0_dim + q1_dim;
+    const float base_log2 = (float)log2((double)theta);
+    const uint32_t pos = kv_len > 0 ? kv_len - 1 : 0;
+    float *qf = (float *)malloc(sizeof(float) * (size_t)(n_heads * qk_dim));
+    for (int64_t h = 0; h < n_heads; ++h)
+        for (int64_t d = 0; d < qk_dim; ++d) {
+            float v;
+            if (d < q0_dim)
+                v = bf16_to_f32(q0[h * q0_stride + d]);
+            else if (d - q0_dim >= rope_dims)
+                v = bf16_to_f32(q1[h * q1_stride + d - q0_dim]);
+            else
+                v = rope_slice_elem(q1 + h * q1_stride, d - q0_dim, rope_dims, traditional, base_log2, pos);
+            qf[h * qk_dim + d] = v;
+        }
+    sdpa_decode_core(qf, cache_k, cache_v, n_heads, n_kv, qk_dim, v_dim, kv_len, capacity, scale, out);
+    free(qf);
+}
+
+/* Cache store of a key given as two parts: cache K row = [K0 | K1]; K1 has n_kv heads or ONE
+ * head shared by all (MLA's rotary key) and its first rope_dims are rotated at `pos` while it is
+ * written; K0 and V rows are k0_stride / v_stride elements apart, so both may alias one packed
+ * [n_kv, k0_dim + v_dim] tensor (src/codegen/kernels/kv_cache_store_decode.rs:268-352; packed
+ * source :103-140). */
+FKO_API void fko_kv_store_split(const uint16_t *k0, int64_t k0_stride, const uint16_t *k1, int64_t k1_heads,
+                                const uint16_t *v, int64_t v_stride, int64_t n_kv, int64_t k0_dim, int64_t k1_dim,
+                                int64_t v_dim, int64_t rope_dims, int traditional, float theta, uint32_t pos,
+                                uint32_t write_offset, uint32_t capacity, uint16_t *cache_k, uint16_t *cache_v) {
+    const float base_log2 = (float)log2((double)theta);
+    const int64_t row = write_offset % capacity, k_dim = k0_dim + k1_dim;
+    for (int64_t h = 0; h < n_kv; ++h) {
+        uint16_t *ck = cache_k + (h * (int64_t)capacity + row) * k_dim;
+        uint16_t *cv = cache_v + (h * (int64_t)capacity + row) * v_dim;
+        const uint16_t *k1h = k1 + (k1_heads == 1 ? 0 : h) * k1_dim;
+        for (int64_t d = 0; d < k0_dim; ++d) ck[d] = k0[h * k0_stride + d];
+        for (int64_t d1 = 0; d1 < k1_dim; ++d1)
+            ck[k0_dim + d1] = d1 >= rope_dims ? k1h[d1]
+                                              : f32_to_bf16(rope_slice_elem(k1h, d1, rope_dims, traditional, base_log2, pos));
+        for (int64_t d = 0; d < v_dim; ++d) cv[d] = v[h * v_stride + d];
+    }
+}
+
+/* Router of a mixture-of-experts block: softmax over ROW_N logits, the top_k largest in
+ * descending order, ties to the lower index (src/codegen/kernels/single.rs:2615-2760):
+ * row_max and sum in fp32, prob = float(T(exp(score - row_max) * (1 / sum))) -- rounded to T
+ * BEFORE the sort (:2707-2709) -- sort key (-prob, index) (:2726-2728), weight = T(prob * scale)
+ * with one scale for the row or one per route (:2748-2750). */
+FKO_API void fko_softmax_topk_route(const uint16_t *logits, int64_t rows, int64_t row_n, int64_t top_k,
+                                    const uint16_t *scale, int scale_per_route, uint32_t *idx, uint16_t *weight) {
+    float *prob = (float *)malloc(sizeof(float) * (size_t)row_n);
+    char *taken = (char *)malloc((size_t)row_n);
+    for (int64_t r = 0; r < rows; ++r) {
+        const uint16_t *l = logits + r * row_n;
+        float m = -INFINITY;
+        for (int64_t i = 0; i < row_n; ++i) m = bf16_to_f32(l[i]) > m ? bf16_to_f32(l[i]) : m;
+        double sum = 0.0;
+        for (int64_t i = 0; i < row_n; ++i) sum += (double)expf(bf16_to_f32(l[i]) - m);
+        const float inv = 1.0f / (float)sum;
+        for (int64_t i = 0; i < row_n; ++i) {
+            prob[i] = bf16_to_f32(f32_to_bf16(expf(bf16_to_f32(l[i]) - m) * inv));
+            taken[i] = 0;
+        }
+        for (int64_t k = 0; k < top_k; ++k) {   /* selection = the first top_k of the (-prob, index) order */
+            int64_t best = -1;
+            for (int64_t i = 0; i < row_n; ++i)
+                if (!taken[i] && (best < 0 || prob[i] > prob[best])) best = i;
+            taken[best] = 1;
+            const float sc = bf16_to_f32(scale[scale_per_route ? r * top_k + k : 0]);
+            idx[r * top_k + k] = (uint32_t)best;
+            weight[r * top_k + k] = f32_to_bf16(prob[best] * sc);
+        }
+    }
+    free(prob);
+    free(taken);
 }
 
 /* Causal attention of a group of L rows (src/codegen/kernels/sdpa_prefill.rs): row l_q sits at

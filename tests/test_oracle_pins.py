@@ -499,3 +499,108 @@ def test_qgemm_with_weights_rounded_to_bf16(bits):
     bias = normal_bf16(92, n)
     yb = oracle.qgemm_bf16w(W, x, bias)
     assert np.array_equal(yb, oracle.f32_to_bf16(acc + oracle.bf16_to_f32(bias)))
+
+
+# ---------------------------------------------------------------- MLA glue and the router
+def _split_case(seed, n_kv, k0d, k1d, vd, k1_heads, packed):
+    if packed:
+        src = normal_bf16(seed, (n_kv, k0d + vd))
+        k0, v, k0s, vs = src.reshape(-1), src.reshape(-1)[k0d:], k0d + vd, k0d + vd
+        k0_rows, v_rows = src[:, :k0d], src[:, k0d:]
+    else:
+        k0_rows, v_rows = normal_bf16(seed, (n_kv, k0d)), normal_bf16(seed + 1, (n_kv, vd))
+        k0, v, k0s, vs = k0_rows.reshape(-1), v_rows.reshape(-1), k0d, vd
+    k1 = normal_bf16(seed + 2, (k1_heads, k1d))
+    return k0, k0s, k0_rows, k1, v, vs, v_rows
+
+
+@pytest.mark.parametrize("k1_heads,packed", [(1, True), (4, False), (1, False)])
+def test_split_key_store_equals_rope_and_plain_store_on_the_assembled_row(k1_heads, packed):
+    """Half-split pairs: [K0 | K1] with K1 rotated == the pinned rope + store applied to a key whose
+    FIRST dims are K1 (the pinned function rotates the leading dims), after moving the parts back."""
+    n_kv, k0d, k1d, vd, cap, pos, rope = 4, 32, 16, 24, 8, 13, 16
+    k0, k0s, k0_rows, k1, v, vs, v_rows = _split_case(300, n_kv, k0d, k1d, vd, k1_heads, packed)
+    ck, cv = np.zeros(n_kv * cap * (k0d + k1d), np.uint16), np.zeros(n_kv * cap * vd, np.uint16)
+    oracle.kv_store_split(k0, k0s, k1, k1_heads, v, vs, n_kv, k0d, k1d, vd, rope, False, 1e4, pos, pos + cap, cap, ck, cv)
+    k1_rows = np.repeat(k1, n_kv, 0) if k1_heads == 1 else k1
+    rot = oracle.rope_q(k1_rows.reshape(-1), n_kv, k1d, rope, 1e4, pos).reshape(n_kv, k1d)
+    want_k = np.concatenate([k0_rows, rot], 1)
+    got_k = ck.reshape(n_kv, cap, k0d + k1d)
+    assert np.array_equal(got_k[:, pos % cap], want_k)
+    assert np.array_equal(cv.reshape(n_kv, cap, vd)[:, pos % cap], v_rows)
+    keep = np.ones(cap, bool); keep[pos % cap] = False
+    assert not got_k[:, keep].any() and not cv.reshape(n_kv, cap, vd)[:, keep].any()
+
+
+def test_split_key_store_traditional_pairs_are_complex_rotations():
+    """Traditional pairs (2i, 2i+1): (lo + i hi) * exp(i pos theta^(-i/half)) in float64; dims beyond
+    rope_dims are copied; position 0 is the identity."""
+    n_kv, k0d, k1d, vd, cap, rope = 2, 8, 12, 8, 4, 8
+    k0, k0s, k0_rows, k1, v, vs, v_rows = _split_case(310, n_kv, k0d, k1d, vd, 1, False)
+    for pos in (0, 7):
+        ck, cv = np.zeros(n_kv * cap * (k0d + k1d), np.uint16), np.zeros(n_kv * cap * vd, np.uint16)
+        oracle.kv_store_split(k0, k0s, k1, 1, v, vs, n_kv, k0d, k1d, vd, rope, True, 100.0, pos, pos, cap, ck, cv)
+        got = oracle.bf16_to_f32(ck.reshape(n_kv, cap, k0d + k1d)[:, pos % cap, k0d:])
+        x = oracle.bf16_to_f32(k1[0]).astype(np.float64)
+        z = (x[0:rope:2] + 1j * x[1:rope:2]) * np.exp(1j * pos * 100.0 ** (-np.arange(rope // 2) / (rope // 2)))
+        want = x.copy()
+        want[0:rope:2], want[1:rope:2] = z.real, z.imag
+        for h in range(n_kv):
+            assert np.all(np.abs(got[h] - want) <= 2.0 ** -8 * np.abs(want) + 1e-6)
+            assert np.array_equal(got[h, rope:], oracle.bf16_to_f32(k1[0, rope:]))
+            if pos == 0:
+                assert np.array_equal(got[h], oracle.bf16_to_f32(k1[0]))
+
+
+@pytest.mark.parametrize("traditional", [False, True])
+def test_split_query_attention_is_attention_on_the_rotated_query(traditional):
+    """[Q0 | rope(Q1)] at position kv_len - 1 through the pinned sdpa_decode: equal up to the one bf16
+    rounding of the rotated elements that the split form does not make; with rope_dims = 0 bit-equal."""
+    n_heads, n_kv, q0d, q1d, vd, cap, kv_len, rope = 4, 2, 16, 8, 16, 16, 9, 8
+    q = normal_bf16(320, (n_heads, q0d + q1d))
+    ck, cv = normal_bf16(321, n_kv * cap * (q0d + q1d)), normal_bf16(322, n_kv * cap * vd)
+    scale = 0.2
+    got = oracle.sdpa_decode_split_q(q, n_heads, q0d, q1d, rope, traditional, 1e4, ck, cv, n_kv, vd, kv_len, cap, scale)
+    # rotate Q1 through the split store (one shared "key head" per query head, cache of one row)
+    qr = q.copy()
+    for h in range(n_heads):
+        row_k, row_v = np.zeros(q0d + q1d, np.uint16), np.zeros(1, np.uint16)
+        oracle.kv_store_split(q[h, :q0d].copy(), q0d, q[h, q0d:].copy(), 1, np.zeros(1, np.uint16), 1, 1, q0d, q1d, 1, rope,
+                              traditional, 1e4, kv_len - 1, 0, 1, row_k, row_v)
+        qr[h] = row_k
+    ref = oracle.sdpa_decode(qr.reshape(-1), ck, cv, n_heads, n_kv, q0d + q1d, vd, kv_len, cap, scale)
+    g, r = oracle.bf16_to_f32(got).astype(np.float64), oracle.bf16_to_f32(ref).astype(np.float64)
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) < 4e-3
+    plain = oracle.sdpa_decode_split_q(q, n_heads, q0d, q1d, 0, traditional, 1e4, ck, cv, n_kv, vd, kv_len, cap, scale)
+    assert np.array_equal(plain, oracle.sdpa_decode(q.reshape(-1), ck, cv, n_heads, n_kv, q0d + q1d, vd, kv_len, cap, scale))
+
+
+def test_softmax_topk_route_closed_forms_and_brute_force():
+    one = oracle.f32_to_bf16(np.array([1.0], np.float32))
+    # equal logits: every probability is 1/N exactly, ties resolve to the lowest indices in order
+    idx, w = oracle.softmax_topk_route(oracle.f32_to_bf16(np.full(64, 0.75, np.float32)), 6,
+                                       oracle.f32_to_bf16(np.array([2.5], np.float32)))
+    assert idx.tolist() == [[0, 1, 2, 3, 4, 5]]
+    assert np.array_equal(w, oracle.f32_to_bf16(np.full((1, 6), 2.5 / 64, np.float32)))
+    # logits 0 and ln 3 (bf16): probabilities 1/4 and 3/4 up to the logit's own rounding
+    l = oracle.f32_to_bf16(np.array([0.0, np.log(3.0)], np.float32))
+    idx, w = oracle.softmax_topk_route(l, 1, one)
+    assert idx.tolist() == [[1]] and abs(float(oracle.bf16_to_f32(w)[0, 0]) - 0.75) < 4e-3
+    # brute force: float64 softmax rounded to bf16, stable descending sort, per-route scales
+    rows, n, k = 7, 32, 5
+    logits = normal_bf16(330, (rows, n), 2.0)
+    scale = normal_bf16(331, (rows, k), 0.1, 1.0)
+    idx, w = oracle.softmax_topk_route(logits, k, scale)
+    f = oracle.bf16_to_f32(logits).astype(np.float64)
+    p = np.exp(f - f.max(1, keepdims=True)); p /= p.sum(1, keepdims=True)
+    pt = oracle.bf16_to_f32(oracle.f32_to_bf16(p.astype(np.float32)))
+    for r in range(rows):
+        order = sorted(range(n), key=lambda i: (-pt[r, i], i))[:k]
+        assert idx[r].tolist() == order
+        want = oracle.f32_to_bf16((pt[r, order] * oracle.bf16_to_f32(scale[r])).astype(np.float32))
+        assert np.array_equal(w[r], want)
+    # rounding to T comes before the ordering: two logits whose probabilities differ in fp32 but
+    # round to the same bf16 value are ordered by index
+    l = oracle.f32_to_bf16(np.array([0.0, 2.0 ** -10, -3.0, -3.0], np.float32))   # p = 0.47607 and 0.47653 -> 244 / 512 both
+    idx, w = oracle.softmax_topk_route(l, 2, one)
+    assert w[0, 0] == w[0, 1] and idx.tolist() == [[0, 1]]
