@@ -1,0 +1,326 @@
+"""Mixture-of-experts decoder with low-rank (MLA-style) keys and values on the MI355X backend:
+random-init weights in HBM, the per-token task list and the captured decode graph.
+
+The architecture is the DeepSeek-V2-Lite-like model of the reference's MoE benchmarks: per layer
+  RMSNorm -> q_proj [n_heads x (nope + rope)] and kv_a_proj [kv_lora_rank + rope] (one launch)
+  RMSNorm(latent) -> kv_b_proj [n_heads x (nope + v)]                              (one launch)
+  cache K row = [k_nope | rope(k_pe)] with ONE rotary key head shared by all heads, V row, and the
+  rotation of the query's rope part (the reference's split-key KvCacheStoreDecode,
+  src/codegen/kernels/kv_cache_store_decode.rs:84-352, and the Q1 rotation of its attention kernel,
+  sdpa_decode.rs:592-660)
+  attention at qk_dim = nope + rope, v_dim (sdpa_decode.rs:133-408) -> o_proj + residual
+  RMSNorm -> router logits -> SoftmaxTopKRoute (single.rs:2615-2760)
+  RoutedQmvSwiglu over the top_k experts (routed_qmv_swiglu.rs:20-452), the shared experts' gate/up,
+  RoutedQmvReduce + shared down projection + residual (routed_qmv_reduce.rs:11-543)
+with the first `first_dense` layers carrying a dense SwiGLU MLP instead of the experts.
+Every dispatch is a kernel family of the task-graph contract, so the list captures into one hipGraph
+and replays per token like the dense decoder's.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from . import native
+from .decoder import _synth, quantize_on_device
+from .native import DeviceBuffer, DeviceWeight
+from .runtime import FK_CHUNK, Dispatch, Dispatcher, arg, make_uniforms
+
+
+@dataclass
+class MoeConfig:
+    n_layers: int = 27
+    hidden: int = 2048
+    n_heads: int = 16
+    kv_lora_rank: int = 512
+    rope_dim: int = 64
+    nope_dim: int = 128
+    v_dim: int = 128
+    n_experts: int = 64
+    top_k: int = 6
+    moe_inter: int = 1408
+    n_shared: int = 2
+    dense_inter: int = 10944
+    first_dense: int = 1
+    vocab: int = 102400
+    eps: float = 1e-6
+    theta: float = 1e4
+    rope_traditional: bool = True
+    route_scale: float = 1.0
+    bits: int = 4
+    group: int = 64
+    swiglu_variant: int = 1
+    capacity: int = 1024
+
+    @property
+    def qk_dim(self) -> int:
+        return self.nope_dim + self.rope_dim
+
+    @property
+    def shared_inter(self) -> int:
+        return self.n_shared * self.moe_inter
+
+    def token_bytes(self, ctx: int) -> int:
+        """Algorithmic HBM bytes per decoded token at context `ctx`: the weights one token touches
+        (attention, top_k + shared experts or the dense MLP, bf16 router), the tied bf16 LM head and
+        the K / V rows attention reads."""
+        per = self.bits / 8 + 4 / self.group
+        attn = self.hidden * (self.n_heads * self.qk_dim + self.kv_lora_rank + self.rope_dim) \
+            + self.kv_lora_rank * self.n_heads * (self.nope_dim + self.v_dim) + self.n_heads * self.v_dim * self.hidden
+        moe = 3 * self.hidden * self.moe_inter * (self.top_k + self.n_shared)
+        dense = 3 * self.hidden * self.dense_inter
+        n_moe = self.n_layers - self.first_dense
+        weights = per * (self.n_layers * attn + n_moe * moe + self.first_dense * dense) + n_moe * self.n_experts * self.hidden * 2
+        kv = self.n_layers * self.n_heads * (self.qk_dim + self.v_dim) * 2 * ctx
+        return int(weights + self.vocab * self.hidden * 2 + kv)
+
+
+MOE_16B_LIKE = dict()   # the defaults above: 27 layers, hidden 2048, 64 experts of 1408, top-6, 2 shared
+
+
+class MoeWeights:
+    """Weights of one model in HBM, keyed by mlx-lm's parameter paths for this architecture."""
+
+    def __init__(self, cfg: MoeConfig):
+        self.cfg = cfg
+        self.mats: Dict[str, DeviceWeight] = {}
+        self.vecs: Dict[str, DeviceBuffer] = {}
+
+    @classmethod
+    def random_init(cls, cfg: MoeConfig, seed: int = 0, std: float = 0.02) -> "MoeWeights":
+        """Projections ~ N(0, std^2) quantised on the device (experts stacked [E, n, k]); the router and
+        the tied embedding stay bf16; norm weights ~ 1 + N(0, 0.1^2)."""
+        self = cls(cfg)
+        c = cfg
+        biggest = max(c.n_experts * c.moe_inter * c.hidden if c.n_layers > c.first_dense else 0,
+                      c.dense_inter * c.hidden if c.first_dense else 0, c.n_heads * c.qk_dim * c.hidden)
+        tmp = DeviceBuffer(biggest * 4)
+        counter = [seed * 100003 + 7]
+
+        def next_seed() -> int:
+            counter[0] += 1
+            return counter[0]
+
+        def matrix(name: str, n: int, k: int, experts: int = 0, sd: float = std) -> None:
+            rows = n * max(experts, 1)
+            _synth(tmp, rows * k, next_seed(), 0.0, sd, 0)
+            W = quantize_on_device(tmp, rows, k, c.bits, c.group)
+            if experts:
+                W.n, W.n_experts = n, experts
+            self.mats[name] = W
+
+        def dense_bf16(name: str, n: int, k: int, sd: float) -> None:
+            W = DeviceWeight.__new__(DeviceWeight)
+            W.n, W.k, W.bits, W.group = n, k, 16, 0
+            W.w, W.scales, W.biases = DeviceBuffer(n * k * 2), None, None
+            _synth(W.w, n * k, next_seed(), 0.0, sd, 1)
+            self.mats[name] = W
+
+        def vector(name: str, n: int, mean: float, sd: float) -> None:
+            b = DeviceBuffer(n * 2)
+            _synth(b, n, next_seed(), mean, sd, 1)
+            self.vecs[name] = b
+
+        dense_bf16("embed_tokens", c.vocab, c.hidden, std)
+        vector("final_norm", c.hidden, 1.0, 0.1)
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            vector(p + "input_layernorm", c.hidden, 1.0, 0.1)
+            vector(p + "post_attention_layernorm", c.hidden, 1.0, 0.1)
+            matrix(p + "self_attn.q_proj", c.n_heads * c.qk_dim, c.hidden)
+            matrix(p + "self_attn.kv_a_proj_with_mqa", c.kv_lora_rank + c.rope_dim, c.hidden)
+            vector(p + "self_attn.kv_a_layernorm", c.kv_lora_rank, 1.0, 0.1)
+            matrix(p + "self_attn.kv_b_proj", c.n_heads * (c.nope_dim + c.v_dim), c.kv_lora_rank)
+            matrix(p + "self_attn.o_proj", c.hidden, c.n_heads * c.v_dim)
+            if l < c.first_dense:
+                matrix(p + "mlp.gate_proj", c.dense_inter, c.hidden)
+                matrix(p + "mlp.up_proj", c.dense_inter, c.hidden)
+                matrix(p + "mlp.down_proj", c.hidden, c.dense_inter)
+            else:
+                dense_bf16(p + "mlp.gate", c.n_experts, c.hidden, 0.05)   # wider spread: distinct routes
+                for nm in ("gate_proj", "up_proj"):
+                    matrix(p + f"mlp.switch_mlp.{nm}", c.moe_inter, c.hidden, c.n_experts)
+                    matrix(p + f"mlp.shared_experts.{nm}", c.shared_inter, c.hidden)
+                matrix(p + "mlp.switch_mlp.down_proj", c.hidden, c.moe_inter, c.n_experts)
+                matrix(p + "mlp.shared_experts.down_proj", c.hidden, c.shared_inter)
+        native.sync()
+        return self
+
+    def nbytes(self) -> int:
+        return sum(m.nbytes for m in self.mats.values()) + sum(v.nbytes for v in self.vecs.values())
+
+
+def _rows(W: DeviceWeight, r0: int, r1: int):
+    """(packed, scales, biases) argument slices of rows r0 .. r1 of a quantised matrix."""
+    wb, sb = W.k * W.bits // 8, (W.k // W.group) * 2
+    return (arg(W.w, (r1 - r0) * wb, r0 * wb), arg(W.scales, (r1 - r0) * sb, r0 * sb), arg(W.biases, (r1 - r0) * sb, r0 * sb))
+
+
+class MoeRuntime:
+    """Scratch arena, KV caches, uniforms and the captured decode graph of one MoE model."""
+
+    def __init__(self, cfg: MoeConfig, weights: MoeWeights, dispatcher: Optional[Dispatcher] = None,
+                 hist_capacity: int = 4096):
+        c = cfg
+        if c.kv_lora_rank % 64 or c.hidden % 64 or c.moe_inter % 64 or (c.kv_lora_rank + c.rope_dim) % 2:
+            raise ValueError("widths must be multiples of the quantisation group")
+        self.cfg, self.w = cfg, weights
+        self.d = dispatcher or Dispatcher()
+        z, B = native.zeros, DeviceBuffer
+        self.token, self.step_counter = z(4), z(4)
+        self.offset, self.kv_len, self.hist_counter = z(4), z(4), z(4)
+        self.history = z(4 * hist_capacity)
+        self.x = [B(c.hidden * 2), B(c.hidden * 2)]
+        self.xn = B(c.hidden * 2)
+        self.q = B(c.n_heads * c.qk_dim * 2)
+        self.kva = B((c.kv_lora_rank + c.rope_dim) * 2)            # [latent | k_pe]
+        self.kvb = B(c.n_heads * (c.nope_dim + c.v_dim) * 2)       # per head [k_nope | v]
+        self.att = B(c.n_heads * c.v_dim * 2)
+        self.mid = B(max(c.dense_inter, c.shared_inter) * 2)
+        self.route_logits = B(c.n_experts * 2)
+        self.route_idx, self.route_weight = z(4 * c.top_k), z(2 * c.top_k)
+        self.route_scale = DeviceBuffer.from_numpy(_bf16(np.array([c.route_scale], np.float32)))
+        self.rows_x = z(4 * c.top_k)                                # every route reads activation row 0
+        self.rows_h = DeviceBuffer.from_numpy(np.arange(c.top_k, dtype=np.uint32))
+        self.h = B(c.top_k * c.moe_inter * 2)
+        self.moe_ws = B(max(native.routed_reduce_workspace_bytes(1, c.top_k, c.hidden), 4))
+        self.logits = B(c.vocab * 2)
+        self.cache_k = [z(c.n_heads * c.capacity * c.qk_dim * 2) for _ in range(c.n_layers)]
+        self.cache_v = [z(c.n_heads * c.capacity * c.v_dim * 2) for _ in range(c.n_layers)]
+        pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
+        self.sdpa_partials, self.sdpa_counters = B(max(pb, 4)), z(max(cb, 4))
+        self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
+        self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
+        self.tasks = self.build_tasks()
+        self.graph = self.d.build_graph(self.tasks)
+
+    def build_tasks(self) -> List[Dispatch]:
+        c, w = self.cfg, self.w
+        quant = dict(bits=c.bits, group=c.group)
+        t: List[Dispatch] = []
+        fid = [0]
+
+        def name(kind: str) -> str:
+            fid[0] += 1
+            return f"fusekit_{kind}_f{fid[0]}"
+
+        def wargs(W):
+            return [arg(W.w)] if W.bits == 16 else [arg(W.w), arg(W.scales), arg(W.biases)]
+
+        def fanout3(x, norm_w, hidden, parts, outs):
+            """RMSNorm + three row blocks of projections in one launch (the rmsnorm_qkv family)."""
+            (w0, s0, b0), (w1, s1, b1), (w2, s2, b2) = (p[0] for p in parts)
+            n_q, n_kv = parts[0][1], parts[1][1]
+            assert parts[2][1] == n_kv
+            t.append(Dispatch(name("rmsnorm_qkv"), [x, arg(norm_w), w0, w1, w2, s0, s1, s2, b0, b1, b2] + outs,
+                              dict(quant, hidden=hidden, n_q=n_q, n_kv=n_kv, eps=c.eps, has_norm=1, has_bias=0)))
+
+        t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
+        emb = w.mats["embed_tokens"]
+        t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token)] + wargs(emb) + [arg(self.x[0])],
+                          dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
+        n_a, half_a = c.kv_lora_rank + c.rope_dim, (c.kv_lora_rank + c.rope_dim) // 2
+        n_b = c.n_heads * (c.nope_dim + c.v_dim)
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            Wq, Wa, Wb = (w.mats[p + f"self_attn.{n}"] for n in ("q_proj", "kv_a_proj_with_mqa", "kv_b_proj"))
+            # q and the two halves of kv_a (latent | k_pe lands contiguously in kva)
+            fanout3(arg(self.x[0]), w.vecs[p + "input_layernorm"], c.hidden,
+                    [(_rows(Wq, 0, Wq.n), Wq.n), (_rows(Wa, 0, half_a), half_a), (_rows(Wa, half_a, n_a), half_a)],
+                    [arg(self.q), arg(self.kva, half_a * 2, 0), arg(self.kva, half_a * 2, half_a * 2)])
+            # kv_b on the normalised latent, as row blocks of one half and two quarters
+            fanout3(arg(self.kva, c.kv_lora_rank * 2, 0), w.vecs[p + "self_attn.kv_a_layernorm"], c.kv_lora_rank,
+                    [(_rows(Wb, 0, n_b // 2), n_b // 2), (_rows(Wb, n_b // 2, 3 * n_b // 4), n_b // 4),
+                     (_rows(Wb, 3 * n_b // 4, n_b), n_b // 4)],
+                    [arg(self.kvb, n_b, 0), arg(self.kvb, n_b // 2, n_b), arg(self.kvb, n_b // 2, n_b + n_b // 2)])
+            packed = c.nope_dim + c.v_dim
+            t.append(Dispatch(name("kv_cache_store_decode"),
+                              [arg(self.q), arg(self.kvb), arg(self.kva, c.rope_dim * 2, c.kv_lora_rank * 2),
+                               arg(self.kvb, self.kvb.nbytes - c.nope_dim * 2, c.nope_dim * 2),
+                               arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.offset), arg(self.offset)],
+                              dict(split_k=1, has_q=1, n_heads=c.n_heads, q0_dim=c.nope_dim, q1_dim=c.rope_dim, n_kv=c.n_heads,
+                                   k0_dim=c.nope_dim, k1_dim=c.rope_dim, v_dim=c.v_dim, k1_n_kv=1, k0_stride=packed,
+                                   v_stride=packed, rope_dims=c.rope_dim, traditional=int(c.rope_traditional), theta=c.theta,
+                                   capacity=c.capacity)))
+            t.append(Dispatch(name("sdpa_decode"),
+                              [arg(self.q), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len), arg(self.att),
+                               arg(self.sdpa_partials), arg(self.sdpa_counters)],
+                              dict(n_heads=c.n_heads, n_kv=c.n_heads, qk_dim=c.qk_dim, head_dim=c.qk_dim, v_dim=c.v_dim,
+                                   capacity=c.capacity, max_len=c.capacity)))
+            Wo = w.mats[p + "self_attn.o_proj"]
+            t.append(Dispatch(name("linear_residual"), [arg(self.att)] + wargs(Wo) + [arg(self.x[0]), arg(self.x[1])],
+                              dict(quant, m=Wo.k, n=c.hidden)))
+            post = w.vecs[p + "post_attention_layernorm"]
+            if l < c.first_dense:
+                Wg, Wu, Wd = (w.mats[p + f"mlp.{n}_proj"] for n in ("gate", "up", "down"))
+                t.append(Dispatch(name("rmsnorm_gateup_swiglu"),
+                                  [arg(self.x[1]), arg(post), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales),
+                                   arg(Wg.biases), arg(Wu.biases), arg(self.mid, c.dense_inter * 2)],
+                                  dict(quant, hidden=c.hidden, inter=c.dense_inter, eps=c.eps, variant=c.swiglu_variant,
+                                       has_norm=1)))
+                t.append(Dispatch(name("linear_residual"),
+                                  [arg(self.mid, c.dense_inter * 2)] + wargs(Wd) + [arg(self.x[1]), arg(self.x[0])],
+                                  dict(quant, m=c.dense_inter, n=c.hidden)))
+                continue
+            t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(post), arg(self.xn)],
+                              dict(rows=1, hidden=c.hidden, eps=c.eps)))
+            Wr = w.mats[p + "mlp.gate"]
+            t.append(Dispatch(name("qgemv"), [arg(self.xn), arg(Wr.w), arg(self.route_logits)],
+                              dict(bits=16, group=64, m=c.hidden, n=c.n_experts)))
+            t.append(Dispatch(name("softmax_topk_route"),
+                              [arg(self.route_logits), arg(self.route_scale), arg(self.route_idx), arg(self.route_weight)],
+                              dict(row_n=c.n_experts, top_k=c.top_k, rows=1)))
+            Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
+            t.append(Dispatch(name("routed_qmv_swiglu"),
+                              [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
+                               arg(self.rows_x), arg(self.route_idx), arg(self.h)],
+                              dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, x_rows=1)))
+            Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
+            t.append(Dispatch(name("qmv_swiglu"),
+                              [arg(self.xn), arg(Sg.w), arg(Su.w), arg(Sg.scales), arg(Su.scales), arg(Sg.biases), arg(Su.biases),
+                               arg(self.mid, c.shared_inter * 2)],
+                              dict(quant, hidden=c.hidden, inter=c.shared_inter, eps=c.eps, variant=c.swiglu_variant, has_norm=0)))
+            t.append(Dispatch(name("routed_qmv_reduce"),
+                              [arg(self.h), arg(Ed.w), arg(Ed.scales), arg(Ed.biases), arg(self.rows_h), arg(self.route_idx),
+                               arg(self.route_weight), arg(self.mid, c.shared_inter * 2), arg(Sd.w), arg(Sd.scales), arg(Sd.biases),
+                               arg(self.x[1]), arg(self.x[0]), arg(self.moe_ws)],
+                              dict(quant, k=c.moe_inter, o=c.hidden, experts=c.n_experts, tokens=1, top_k=c.top_k, x_rows=c.top_k,
+                                   has_shared=1, shared_k=c.shared_inter, has_extra=1)))
+        t.append(Dispatch(name("final_rmsnorm_lm_head"),
+                          [arg(self.x[0]), arg(w.vecs["final_norm"])] + wargs(emb) + [arg(self.logits)],
+                          dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
+        t.append(Dispatch(name("argmax_logits_decode"),
+                          [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history), arg(self.hist_counter)],
+                          dict(vocab=c.vocab)))
+        return t
+
+    # -- generation (the dense runtime's loop: prompt with forced tokens, then chunks fed back on the GPU)
+    def reset(self) -> None:
+        for b in (self.step_counter, self.offset, self.kv_len, self.hist_counter):
+            b.upload(np.zeros(1, np.uint32))
+
+    def prefill(self, prompt: Sequence[int], start_offset: int = 0) -> int:
+        preds, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
+        return preds[-1]
+
+    def generate(self, prompt: Sequence[int], max_tokens: int):
+        """Greedy decode: returns (tokens, seconds on the GPU for the decode chunks, decode steps)."""
+        if len(prompt) + max_tokens > self.cfg.capacity:
+            raise ValueError("prompt + max_tokens exceeds the KV-cache capacity")
+        out = [self.prefill(prompt)]
+        gpu_s, steps, offset = 0.0, 0, len(prompt)
+        while len(out) < max_tokens:
+            n = min(FK_CHUNK, max_tokens - len(out), self.uniforms.hist_capacity)
+            toks, sec = self.d.decode_chunk(self.graph, self.uniforms, offset, out[-1], n)
+            out += toks
+            gpu_s += sec
+            steps += n
+            offset += n
+        return out, gpu_s, steps
+
+
+def _bf16(a: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)

@@ -127,3 +127,86 @@ class OracleDecoder:
             toks.append(nxt); margins.append(m)
             off += 1
         return toks, margins
+
+
+class OracleMoeDecoder:
+    """CPU oracle of the mixture-of-experts decoder with low-rank keys, composed from the oracle's
+    per-kernel functions on the very bytes the GPU model holds, one call per dispatch of the GPU task list."""
+
+    def __init__(self, cfg, weights):
+        self.cfg = c = cfg
+        self.vec = {k: v.to_numpy(np.uint16) for k, v in weights.vecs.items()}
+        self.mat = {}
+        for k, dw in weights.mats.items():
+            E = getattr(dw, "n_experts", 0)
+            if not E:
+                self.mat[k] = host_weight(dw)
+                continue
+            per = 32 // dw.bits
+            wq = dw.w.to_numpy(np.uint32, (E, dw.n, dw.k // per))
+            sc = dw.scales.to_numpy(np.uint16, (E, dw.n, dw.k // dw.group))
+            bi = dw.biases.to_numpy(np.uint16, (E, dw.n, dw.k // dw.group))
+            S = oracle.StackedWeight.__new__(oracle.StackedWeight)     # the arrays are stacked already: no copy
+            oracle.QWeight.__init__(S, wq, sc, bi, dw.n, dw.k, dw.bits, dw.group)
+            S.n_experts = E
+            self.mat[k] = S
+        self.ck = [np.zeros(c.n_heads * c.capacity * c.qk_dim, np.uint16) for _ in range(c.n_layers)]
+        self.cv = [np.zeros(c.n_heads * c.capacity * c.v_dim, np.uint16) for _ in range(c.n_layers)]
+        self.route_scale = oracle.f32_to_bf16(np.array([c.route_scale], np.float32))
+        self.routes = []          # expert indices of the last step, per MoE layer
+
+    def step(self, token: int, offset: int, want_logits: bool = False):
+        c, m, v = self.cfg, self.mat, self.vec
+        x = oracle.embed_lookup(m["embed_tokens"], token)
+        packed = c.nope_dim + c.v_dim
+        self.routes = []
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            xn = oracle.rmsnorm(x, v[p + "input_layernorm"], c.eps)
+            q = oracle.qgemv(m[p + "self_attn.q_proj"], xn)
+            kva = oracle.qgemv(m[p + "self_attn.kv_a_proj_with_mqa"], xn)
+            lat = oracle.rmsnorm(kva[:c.kv_lora_rank].copy(), v[p + "self_attn.kv_a_layernorm"], c.eps)
+            kvb = oracle.qgemv(m[p + "self_attn.kv_b_proj"], lat)
+            k_pe = kva[c.kv_lora_rank:].copy().reshape(1, c.rope_dim)
+            oracle.kv_store_split(kvb, packed, k_pe, 1, kvb[c.nope_dim:], packed, c.n_heads, c.nope_dim, c.rope_dim, c.v_dim,
+                                  c.rope_dim, c.rope_traditional, c.theta, offset, offset, c.capacity, self.ck[l], self.cv[l])
+            # the GPU rotates the query's rope part in place (rounded to T) in the same launch
+            qh = q.reshape(c.n_heads, c.qk_dim).copy()
+            for h in range(c.n_heads):
+                row_k, row_v = np.zeros(c.qk_dim, np.uint16), np.zeros(1, np.uint16)
+                oracle.kv_store_split(qh[h, :c.nope_dim].copy(), c.nope_dim, qh[h, c.nope_dim:].copy(), 1, np.zeros(1, np.uint16), 1, 1,
+                                      c.nope_dim, c.rope_dim, 1, c.rope_dim, c.rope_traditional, c.theta, offset, 0, 1, row_k, row_v)
+                qh[h] = row_k
+            att = oracle.sdpa_decode(qh.reshape(-1), self.ck[l], self.cv[l], c.n_heads, c.n_heads, c.qk_dim, c.v_dim, offset + 1,
+                                     c.capacity, 1.0 / np.sqrt(c.qk_dim))
+            x1 = oracle.linear_residual(m[p + "self_attn.o_proj"], att, x)
+            post = v[p + "post_attention_layernorm"]
+            if l < c.first_dense:
+                mid = oracle.gateup_swiglu(x1, post, c.eps, m[p + "mlp.gate_proj"], m[p + "mlp.up_proj"], c.swiglu_variant)
+                x = oracle.linear_residual(m[p + "mlp.down_proj"], mid, x1)
+                continue
+            xn = oracle.rmsnorm(x1, post, c.eps)
+            logits = oracle.qgemv(m[p + "mlp.gate"], xn)
+            idx, rw = oracle.softmax_topk_route(logits, c.top_k, self.route_scale)
+            idx, rw = idx.reshape(-1), rw.reshape(-1)
+            self.routes.append(idx.copy())
+            h = oracle.routed_qmv_swiglu(xn.reshape(1, -1), m[p + "mlp.switch_mlp.gate_proj"], m[p + "mlp.switch_mlp.up_proj"],
+                                         np.zeros(c.top_k, np.uint32), idx, None)
+            smid = oracle.gateup_swiglu(xn, None, c.eps, m[p + "mlp.shared_experts.gate_proj"], m[p + "mlp.shared_experts.up_proj"],
+                                        c.swiglu_variant)
+            x = oracle.routed_qmv_reduce(h, m[p + "mlp.switch_mlp.down_proj"], idx, rw, x1.reshape(1, -1), 1, c.top_k,
+                                         np.arange(c.top_k, dtype=np.uint32), smid, m[p + "mlp.shared_experts.down_proj"]).reshape(-1)
+        logits = oracle.final_rmsnorm_lm_head(x, v["final_norm"], c.eps, m["embed_tokens"])
+        return oracle.argmax(logits), oracle.top2_margin(logits), (logits if want_logits else None)
+
+    def generate(self, prompt, max_tokens):
+        toks, margins, nxt = [], [], None
+        for i, t in enumerate(prompt):
+            nxt, mg, _ = self.step(int(t), i)
+        toks.append(nxt); margins.append(mg)
+        off = len(prompt)
+        while len(toks) < max_tokens:
+            nxt, mg, _ = self.step(toks[-1], off)
+            toks.append(nxt); margins.append(mg)
+            off += 1
+        return toks, margins
