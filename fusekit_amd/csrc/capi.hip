@@ -411,6 +411,14 @@ fk_status fk_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, i
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* w, const uint16_t* scale,
+                        uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t* xn, uint16_t* logits, uint32_t* idx,
+                        uint16_t* weight, uint32_t* workspace, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_moe_router(x, norm_w, eps, w, scale, hidden, experts, top_k, xn, logits, idx, weight, workspace, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_qkv_rope_store_decode(uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_norm,
                                    const uint16_t* k_norm, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                    uint32_t rope_dims, float theta, float eps, const uint32_t* d_offset,

@@ -389,6 +389,32 @@ fk_status plan_softmax_topk_route_d(const Dispatch& d, Launch* l, SlotRW* rw) {
                                    arg_ptr<uint32_t>(d, 2), arg_ptr<uint16_t>(d, 3), l);
 }
 
+// x, [norm_w], router_w, scale, xn, logits, idx, weight, workspace: norm + router projection + softmax top-k
+// route in one launch.  Parameters: hidden, experts, top_k, eps, has_norm.
+fk_status plan_moe_router_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const bool has_norm = d.u("has_norm", 1) != 0;
+    const size_t b = has_norm ? 2 : 1;
+    FK_TRY(need_args(d, b + 7));
+    const uint32_t hidden = d.u("hidden"), experts = d.u("experts"), top_k = d.u("top_k");
+    if (hidden == 0 || experts == 0 || top_k == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden / experts / top_k parameters missing");
+    FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
+    if (has_norm) FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, b, (size_t)experts * hidden * 2));
+    FK_TRY(need_bytes(d, b + 1, 2));
+    FK_TRY(need_bytes(d, b + 2, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, b + 3, (size_t)experts * 2));
+    FK_TRY(need_bytes(d, b + 4, (size_t)top_k * 4));
+    FK_TRY(need_bytes(d, b + 5, (size_t)top_k * 2));
+    FK_TRY(need_bytes(d, b + 6, ((size_t)experts + 1) * 4));
+    for (uint32_t i = 0; i < b + 2; ++i) rw->reads.push_back(i);
+    rw->reads.push_back((uint32_t)(b + 6));
+    for (uint32_t i = b + 2; i < b + 7; ++i) rw->writes.push_back(i);
+    return plan_moe_router(arg_ptr<const uint16_t>(d, 0), has_norm ? arg_ptr<const uint16_t>(d, 1) : nullptr,
+                           (float)d.param("eps", 1e-6), arg_ptr<const uint16_t>(d, b), arg_ptr<const uint16_t>(d, b + 1), hidden,
+                           experts, top_k, arg_ptr<uint16_t>(d, b + 2), arg_ptr<uint16_t>(d, b + 3), arg_ptr<uint32_t>(d, b + 4),
+                           arg_ptr<uint16_t>(d, b + 5), arg_ptr<uint32_t>(d, b + 6), l);
+}
+
 // K, V, [k_weight], cache_k, cache_v, offset, write_offset
 fk_status plan_rope_kv(const Dispatch& d, Launch* l, SlotRW* rw, bool norm, bool rope) {
     const size_t n = norm ? 7 : 6;
@@ -865,6 +891,7 @@ const Family kFamilies[] = {
          return d.u("split_k", 0) ? plan_kv_store_split(d, l, rw) : plan_rope_kv(d, l, rw, false, false);
      }},
     {"fusekit_softmax_topk_route", plan_softmax_topk_route_d},
+    {"fusekit_moe_router", plan_moe_router_d},
     {"fusekit_qkv_rope_store_decode", plan_qkv_rope_store},
     {"fusekit_sdpa_decode", plan_sdpa_d},
     {"fusekit_sdpa_prefill", plan_sdpa_prefill_d},

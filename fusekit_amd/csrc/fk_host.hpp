@@ -153,6 +153,12 @@ fk_status plan_split_rope_store(const SplitStoreArgs& a, Launch* out);
 fk_status plan_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, bool scale_per_route, uint32_t rows,
                                   uint32_t row_n, uint32_t top_k, uint32_t* idx, uint16_t* weight, Launch* out);
 
+// RMSNorm + router projection (bf16 [experts, hidden]) + softmax top-k route in one launch; xn (normalised
+// row) and logits are optional outputs; workspace: (experts + 1) words, zero before the first launch.
+fk_status plan_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* w, const uint16_t* scale,
+                          uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t* xn, uint16_t* logits, uint32_t* idx,
+                          uint16_t* weight, uint32_t* workspace, Launch* out);
+
 // Quantised KV cache (mlx-lm QuantizedKVCache layout): packed uint32 [n_kv, capacity, dim*bits/32],
 // scales / biases bf16 [n_kv, capacity, dim/group].
 struct KvQuant {

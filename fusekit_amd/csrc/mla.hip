@@ -163,4 +163,170 @@ fk_status plan_softmax_topk_route(const uint16_t* logits, const uint16_t* scale,
     return FK_OK;
 }
 
+// ------------------------------------------------------------------ router in one launch
+//
+// RMSNorm of the hidden row, the router projection (bf16 [experts, hidden]) and the softmax top-k
+// route as ONE launch: three launch-latency sized kernels become one.  The arithmetic is the
+// composition of the three (kernels/mod.rs:4424-4516 norm with its two roundings; a linear layer
+// with fp32 accumulation and one rounding to T; single.rs:2615-2760), and the normalised row is
+// written out for the expert projections that follow.
+// One wave per expert (a single CU cannot pull the whole matrix quickly: its requests in flight are
+// bounded, 256 KB took 15 us from one block): the wave requests its weight row, the activations and
+// the norm weights in the same 16-byte-per-lane layout, normalises in registers, reduces its dot
+// product and publishes the logit through an agent-scope store; the wave that arrives last at the
+// counter routes.  The counter returns to zero for the next launch.
+constexpr int kRouterChunks = 8;   // 16-byte pieces per lane and row: hidden <= 4096
+struct RouterArgs {
+    const uint16_t* x;
+    const uint16_t* norm_w;   // null: x is used as it is
+    const uint16_t* w;        // bf16 [experts, hidden]
+    const uint16_t* scale;    // one bf16 value
+    uint16_t* xn;             // [hidden] normalised row, or null
+    uint16_t* logits;         // [experts] or null
+    uint32_t* idx;
+    uint16_t* weight;
+    uint32_t* workspace;      // [experts] logits as fp32 bits, then the arrival counter
+    uint32_t hidden, experts, top_k;
+    float eps;
+};
+__global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
+    const uint32_t e = blockIdx.x, lane = threadIdx.x;
+    const uint32_t chunks = a.hidden / (8 * kWave);
+    uint4 wr[kRouterChunks], xr[kRouterChunks], nr[kRouterChunks];
+#pragma unroll
+    for (int c = 0; c < kRouterChunks; ++c) {
+        const uint32_t o = ((uint32_t)c < chunks ? c * kWave + lane : lane) * 8;   // beyond the row: a harmless repeat
+        wr[c] = *reinterpret_cast<const uint4*>(a.w + (size_t)e * a.hidden + o);
+        xr[c] = *reinterpret_cast<const uint4*>(a.x + o);
+        nr[c] = a.norm_w ? *reinterpret_cast<const uint4*>(a.norm_w + o) : make_uint4(0, 0, 0, 0);
+    }
+    float xf[kRouterChunks][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < kRouterChunks; ++c) {
+        const uint32_t p[4] = {xr[c].x, xr[c].y, xr[c].z, xr[c].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            xf[c][2 * i] = bf16_lo(p[i]);
+            xf[c][2 * i + 1] = bf16_hi(p[i]);
+        }
+        if ((uint32_t)c < chunks) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = fmaf(xf[c][i], xf[c][i], ss);
+        }
+    }
+    if (a.norm_w) {
+        ss = wave_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)a.hidden + a.eps);
+#pragma unroll
+        for (int c = 0; c < kRouterChunks; ++c) {
+            const uint32_t p[4] = {nr[c].x, nr[c].y, nr[c].z, nr[c].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                xf[c][2 * i] = round_bf16(bf16_lo(p[i]) * round_bf16(xf[c][2 * i] * r));
+                xf[c][2 * i + 1] = round_bf16(bf16_hi(p[i]) * round_bf16(xf[c][2 * i + 1] * r));
+            }
+        }
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < kRouterChunks; ++c) {
+        if ((uint32_t)c >= chunks) continue;
+        const uint32_t p[4] = {wr[c].x, wr[c].y, wr[c].z, wr[c].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc = fmaf(bf16_lo(p[i]), xf[c][2 * i], acc);
+            acc = fmaf(bf16_hi(p[i]), xf[c][2 * i + 1], acc);
+        }
+        if (e == 0 && a.xn) {
+            uint4 o;
+            o.x = pack_bf16(xf[c][0], xf[c][1]); o.y = pack_bf16(xf[c][2], xf[c][3]);
+            o.z = pack_bf16(xf[c][4], xf[c][5]); o.w = pack_bf16(xf[c][6], xf[c][7]);
+            *reinterpret_cast<uint4*>(a.xn + (c * kWave + lane) * 8) = o;
+        }
+    }
+    acc = round_bf16(wave_sum(acc));
+    uint32_t* counter = a.workspace + a.experts;
+    uint32_t last = 0;
+    if (lane == 0) {
+        __hip_atomic_store(&a.workspace[e], __float_as_uint(acc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (a.logits) a.logits[e] = (uint16_t)(__float_as_uint(acc) >> 16);
+        wait_memory_ops_done();
+        last = atomicAdd(counter, 1u) == a.experts - 1 ? 1u : 0u;
+    }
+    last = __builtin_amdgcn_readfirstlane(last);
+    if (!last) return;
+    if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // softmax top-k over the published logits: the arithmetic of softmax_topk_route_kernel
+    float x[4], p[4];
+    float m = -INFINITY;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t i = lane + j * kWave;
+        x[j] = i < a.experts ? __uint_as_float(__hip_atomic_load(&a.workspace[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                             : -INFINITY;
+        m = fmaxf(m, x[j]);
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        p[j] = lane + j * kWave < a.experts ? expf(x[j] - m) : 0.f;
+        sum += p[j];
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) p[j] = lane + j * kWave < a.experts ? round_bf16(p[j] * inv) : -1.f;
+    const float sc = bf16_bits_to_f32(a.scale[0]);
+    for (uint32_t k = 0; k < a.top_k; ++k) {
+        float best = -1.f;
+        uint32_t best_i = 0xffffffffu;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (p[j] > best) {
+                best = p[j];
+                best_i = lane + j * kWave;
+            }
+#pragma unroll
+        for (uint32_t off = 1; off < kWave; off <<= 1) {
+            const float ob = __shfl_xor(best, off, kWave);
+            const uint32_t oi = __shfl_xor(best_i, off, kWave);
+            if (ob > best || (ob == best && oi < best_i)) {
+                best = ob;
+                best_i = oi;
+            }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (best_i == lane + j * kWave) p[j] = -1.f;
+        if (lane == 0) {
+            a.idx[k] = best_i;
+            a.weight[k] = (uint16_t)f32_to_bf16_bits(best * sc);
+        }
+    }
+}
+
+fk_status plan_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* w, const uint16_t* scale,
+                          uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t* xn, uint16_t* logits, uint32_t* idx,
+                          uint16_t* weight, uint32_t* workspace, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!x || !w || !scale || !idx || !weight || !workspace) return set_error(FK_ERR_INVALID, "router: null pointer");
+    if (hidden == 0 || hidden % (8 * kWave) || hidden > (uint32_t)kRouterChunks * 8 * kWave)
+        return set_error(FK_ERR_UNSUPPORTED, "router: hidden must be a multiple of 512 of at most 4096");
+    if (experts < 2 || experts > 256 || (experts & (experts - 1)) || top_k == 0 || top_k >= experts || top_k > 32)
+        return set_error(FK_ERR_UNSUPPORTED, "router: experts must be a power of two of at most 256, top_k below it and at most 32");
+    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)norm_w | (uintptr_t)xn) & 15u)
+        return set_error(FK_ERR_INVALID, "router: activations and weights must be 16-byte aligned");
+    RouterArgs a{x, norm_w, w, scale, xn, logits, idx, weight, workspace, hidden, experts, top_k, eps};
+    out->func = reinterpret_cast<const void*>(&moe_router_kernel);
+    out->grid = dim3(experts, 1, 1);
+    out->block = dim3(kWave, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
 }  // namespace fk

@@ -88,7 +88,10 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     const uint32_t G = n_heads / n_kv;
     // Tiles of 1, 2 or 4 heads run the wave-local form, which needs a key row and its value row on
     // the same lanes (equal lanes per row); other shapes take the tile of 8, which goes through LDS.
-    const bool same_lanes = pow2_ceil(qk_dim / 8) == pow2_ceil(v_dim / 8);
+    // Rows of different widths (192 / 128) both take the lane count of the wider one -- the spare
+    // lanes of the narrower row idle -- as long as a row fits a wave; bf16 caches only.
+    const uint32_t lpk0 = pow2_ceil(qk_dim / 8), lpv0 = pow2_ceil(v_dim / 8), lp_wide = lpk0 > lpv0 ? lpk0 : lpv0;
+    const bool same_lanes = lpk0 == lpv0 || (!kvq && !fusion && lp_wide <= (uint32_t)kWave);
     const int gt = !same_lanes ? 8 : (G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1)));
     // Long contexts: a block walks several consecutive ranges (online softmax, the next
     // range's rows in flight), so that the grid stays near one to two blocks per CU and
@@ -128,8 +131,8 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         a.eps = fusion->eps; a.base_log2 = fusion->base_log2;
         a.rope_tab = fusion->rope_tab;
     }
-    a.lpk = pow2_ceil(qk_dim / 8);
-    a.lpv = pow2_ceil(v_dim / 8);
+    a.lpk = gt <= 4 ? lp_wide : lpk0;
+    a.lpv = gt <= 4 ? lp_wide : lpv0;
     a.scale = scale;
     a.partials = partials;
     a.counters = counters;

@@ -53,6 +53,7 @@ class MoeConfig:
     group: int = 64
     swiglu_variant: int = 1
     capacity: int = 1024
+    fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
 
     @property
     def qk_dim(self) -> int:
@@ -193,6 +194,9 @@ class MoeRuntime:
         self.sdpa_partials, self.sdpa_counters = B(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
+        # the single-launch router holds the hidden row in registers, 512 elements per piece, at most 8
+        self.fused_router = bool(c.fuse_router and c.hidden % 512 == 0 and c.hidden <= 4096)
+        self.router_ws = z(4 * (c.n_experts + 1))
         self.tasks = self.build_tasks()
         self.graph = self.d.build_graph(self.tasks)
 
@@ -264,14 +268,20 @@ class MoeRuntime:
                                   [arg(self.mid, c.dense_inter * 2)] + wargs(Wd) + [arg(self.x[1]), arg(self.x[0])],
                                   dict(quant, m=c.dense_inter, n=c.hidden)))
                 continue
-            t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(post), arg(self.xn)],
-                              dict(rows=1, hidden=c.hidden, eps=c.eps)))
             Wr = w.mats[p + "mlp.gate"]
-            t.append(Dispatch(name("qgemv"), [arg(self.xn), arg(Wr.w), arg(self.route_logits)],
-                              dict(bits=16, group=64, m=c.hidden, n=c.n_experts)))
-            t.append(Dispatch(name("softmax_topk_route"),
-                              [arg(self.route_logits), arg(self.route_scale), arg(self.route_idx), arg(self.route_weight)],
-                              dict(row_n=c.n_experts, top_k=c.top_k, rows=1)))
+            if self.fused_router:   # norm + router projection + top-k route in one single-block launch
+                t.append(Dispatch(name("moe_router"),
+                                  [arg(self.x[1]), arg(post), arg(Wr.w), arg(self.route_scale), arg(self.xn), arg(self.route_logits),
+                                   arg(self.route_idx), arg(self.route_weight), arg(self.router_ws)],
+                                  dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1)))
+            else:
+                t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(post), arg(self.xn)],
+                                  dict(rows=1, hidden=c.hidden, eps=c.eps)))
+                t.append(Dispatch(name("qgemv"), [arg(self.xn), arg(Wr.w), arg(self.route_logits)],
+                                  dict(bits=16, group=64, m=c.hidden, n=c.n_experts)))
+                t.append(Dispatch(name("softmax_topk_route"),
+                                  [arg(self.route_logits), arg(self.route_scale), arg(self.route_idx), arg(self.route_weight)],
+                                  dict(row_n=c.n_experts, top_k=c.top_k, rows=1)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             t.append(Dispatch(name("routed_qmv_swiglu"),
                               [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),

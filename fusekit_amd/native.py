@@ -266,6 +266,14 @@ def softmax_topk_route(logits, scale, scale_per_route, rows, row_n, top_k, idx, 
                                     C.c_uint32(row_n), C.c_uint32(top_k), _ptr(idx), _ptr(weight), _ptr(stream)))
 
 
+def moe_router(x, norm_w, eps, w, scale, hidden, experts, top_k, xn, logits, idx, weight, workspace, stream=None):
+    """RMSNorm + router projection (bf16 weights) + softmax top-k route in one launch (fk_moe_router);
+    workspace: zeros(4 * (experts + 1)), reusable by launches that do not overlap."""
+    check(lib.fk_moe_router(_ptr(x), _ptr(norm_w), C.c_float(eps), _ptr(w), _ptr(scale), C.c_uint32(hidden),
+                            C.c_uint32(experts), C.c_uint32(top_k), _ptr(xn), _ptr(logits), _ptr(idx), _ptr(weight),
+                            _ptr(workspace), _ptr(stream)))
+
+
 def qkv_rope_store_decode(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope_dims, theta, eps, d_offset,
                           offset, capacity, cache_k, cache_v, stream=None):
     check(lib.fk_qkv_rope_store_decode(

@@ -318,6 +318,19 @@ fk_status fk_kv_cache_store_split_decode(uint16_t *q, uint32_t n_heads, uint32_t
 fk_status fk_softmax_topk_route(const uint16_t *logits, const uint16_t *scale, int scale_per_route, uint32_t rows,
                                 uint32_t row_n, uint32_t top_k, uint32_t *idx, uint16_t *weight, fk_stream s);
 
+/* fk_moe_router: RMSNorm of one hidden row (norm_w may be NULL: x as it is), the router projection with
+ * bf16 weights w [experts, hidden] and fk_softmax_topk_route with one scale, as ONE launch (one wave per
+ * expert; the wave that finishes last routes).
+ * The reference runs these as three kernels (norm: src/codegen/kernels/mod.rs:4424-4516; linear: K1;
+ * SoftmaxTopKRoute: src/codegen/kernels/single.rs:2615-2760); the arithmetic here is their composition
+ * with the same roundings (normalised row and logits rounded to bf16).  xn [hidden] and logits [experts]
+ * are optional outputs (NULL to skip).  hidden a multiple of 512 up to 4096; experts / top_k as above.
+ * workspace: (experts + 1) 32-bit words, zero before the first launch, left zeroed by every launch; launches
+ * that share it must not overlap. */
+fk_status fk_moe_router(const uint16_t *x, const uint16_t *norm_w, float eps, const uint16_t *w, const uint16_t *scale,
+                        uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t *xn, uint16_t *logits,
+                        uint32_t *idx, uint16_t *weight, uint32_t *workspace, fk_stream s);
+
 /* ---- several active token rows (multi-token verification, chunked prefill) ----
  * The reference compiles such variants with active_m > 1 (src/target/mod.rs:170-200,
  * variants `prefill_mN`, src/patch.rs:103-150; causal attention

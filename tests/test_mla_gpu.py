@@ -125,6 +125,37 @@ def test_softmax_topk_route_ties_take_the_lower_index(fk):
     assert np.array_equal(got, ref_idx) and np.array_equal(w.to_numpy(np.uint16, (2, 6)), ref_w)
 
 
+@pytest.mark.parametrize("hidden,experts,top_k,norm", [(2048, 64, 6, True), (512, 8, 2, True), (1024, 256, 32, False),
+                                                       (3072, 16, 3, True)])
+def test_router_in_one_launch(fk, hidden, experts, top_k, norm):
+    """fk_moe_router = rmsnorm -> bf16 linear -> softmax top-k route of the oracle, outputs included."""
+    from helpers import make_qweight
+    x, nw = normal_bf16(40, hidden), normal_bf16(41, hidden, 0.1, 1.0)
+    W = make_qweight(42, experts, hidden, 16, std=0.05)
+    scale = oracle.f32_to_bf16(np.array([1.25], np.float32))
+    xn_ref = oracle.rmsnorm(x, nw, 1e-6) if norm else x
+    lg_ref = oracle.qgemv(W, xn_ref)
+    idx_ref, w_ref = oracle.softmax_topk_route(lg_ref, top_k, scale)
+    xn, lg, idx, w = fk.zeros(2 * hidden), fk.zeros(2 * experts), fk.zeros(4 * top_k), fk.zeros(2 * top_k)
+    ws = fk.zeros(4 * (experts + 1))
+    for _ in range(2):    # the second launch finds the counter back at zero
+        fk.moe_router(_dev(fk, x), _dev(fk, nw) if norm else None, 1e-6, _dev(fk, W.w), _dev(fk, scale), hidden, experts, top_k,
+                      xn, lg, idx, w, ws)
+        fk.sync()
+    assert ws.to_numpy(np.uint32)[experts] == 0
+    frac, ulps = bf16_mismatch(xn.to_numpy(np.uint16), xn_ref)
+    assert ulps <= 1.0 and frac <= 0.01
+    got_lg = lg.to_numpy(np.uint16)
+    frac, ulps = bf16_mismatch(got_lg, lg_ref)
+    assert ulps <= 1.0 and frac <= 0.1, (frac, ulps)
+    # the route is exactly the oracle's route of the logits the GPU produced (up to an edge flip of a probability)
+    idx2, w2 = oracle.softmax_topk_route(got_lg, top_k, scale)
+    got_idx, got_w = idx.to_numpy(np.uint32), w.to_numpy(np.uint16)
+    assert np.mean(got_idx == idx2.reshape(-1)) >= 0.9 and set(got_idx.tolist()) == set(idx2.reshape(-1).tolist())
+    assert bf16_mismatch(got_w, w2.reshape(-1))[1] <= 1.0
+    assert len(set(got_idx.tolist()) & set(idx_ref.reshape(-1).tolist())) >= top_k - 1
+
+
 def test_rejects(fk):
     b = fk.zeros(4096)
     with pytest.raises(fk.FusekitError):
