@@ -268,30 +268,14 @@ fk_status fk_routed_qmv_reduce(const uint16_t* h, uint32_t n_h_rows, const fk_we
                                const uint32_t* row_idx, const uint32_t* expert_idx, const uint16_t* route_weight,
                                const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual_extra,
                                uint32_t n_tokens, uint32_t top_k, uint16_t* out, void* workspace, fk_stream s) {
-    if (!Wd || !out || !workspace) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce: null weight, output or workspace");
-    if (n_tokens == 0 || top_k == 0) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce: empty route set");
-    if ((shared_x != nullptr) != (W_shared != nullptr))
-        return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce: shared_x and W_shared come together");
-    if (W_shared && (n_tokens != 1 || W_shared->n != Wd->n))
-        return set_error(FK_ERR_UNSUPPORTED, "fk_routed_qmv_reduce: shared expert needs one token and the same output width");
-    if ((uint64_t)n_tokens * top_k > 65536) return set_error(FK_ERR_UNSUPPORTED, "fk_routed_qmv_reduce: too many routes");
-    const uint32_t n_routes = n_tokens * top_k;
-    uint16_t* parts = static_cast<uint16_t*>(workspace);
-    Launch routed, shared, reduce;
-    FK_TRY(plan_routed_gemv(h, n_h_rows, Wd, nullptr, n_experts, row_idx, expert_idx, nullptr, n_routes, parts, &routed));
-    if (W_shared) {
-        GemvRequest rq;
-        rq.mats[0] = W_shared;
-        rq.y[0] = parts + (size_t)n_routes * Wd->n;
-        rq.x = shared_x;
-        FK_TRY(plan_gemv(rq, &shared));
-    }
-    FK_TRY(plan_route_reduce(parts, route_weight, residual_extra, out, n_tokens, top_k, Wd->n, W_shared != nullptr,
-                             &reduce));
-    FK_TRY(run_launch(routed, (hipStream_t)s));
-    if (W_shared) FK_TRY(run_launch(shared, (hipStream_t)s));
-    return run_launch(reduce, (hipStream_t)s);
+    if (!workspace) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce: null workspace");
+    Launch l;
+    FK_TRY(plan_routed_reduce_chain(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_weight, shared_x, W_shared,
+                                    residual_extra, n_tokens, top_k, out, static_cast<uint16_t*>(workspace), &l));
+    return run_launch(l, (hipStream_t)s);
 }
+
+void fk_set_routed_fused_reduce(int on) { set_routed_fused_reduce(on != 0); }
 
 fk_status fk_qgemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, uint32_t group, size_t* bytes) {
     if (!bytes) return set_error(FK_ERR_INVALID, "fk_qgemm_workspace_bytes: null output");

@@ -761,24 +761,11 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     rw->reads.push_back((uint32_t)ws_slot);
     rw->writes = {(uint32_t)out_slot, (uint32_t)ws_slot};
 
-    uint16_t* parts = arg_ptr<uint16_t>(d, ws_slot);
-    FK_TRY(plan_routed_gemv(arg_ptr<const uint16_t>(d, 0), x_rows, &Wd, nullptr, experts, arg_ptr<const uint32_t>(d, 4),
-                            arg_ptr<const uint32_t>(d, 5), nullptr, routes, parts, l));
-    if (has_shared) {
-        GemvRequest rq;
-        rq.mats[0] = &Ws;
-        rq.y[0] = parts + (size_t)routes * O;
-        rq.x = arg_ptr<const uint16_t>(d, shared_slot);
-        Launch shared;
-        FK_TRY(plan_gemv(rq, &shared));
-        l->then.push_back(shared);
-    }
-    Launch reduce;
-    FK_TRY(plan_route_reduce(parts, preweighted ? nullptr : arg_ptr<const uint16_t>(d, rw_slot),
-                             has_extra ? arg_ptr<const uint16_t>(d, extra_slot) : nullptr, arg_ptr<uint16_t>(d, out_slot),
-                             tokens, top_k, O, has_shared, &reduce));
-    l->then.push_back(reduce);
-    return FK_OK;
+    return plan_routed_reduce_chain(arg_ptr<const uint16_t>(d, 0), x_rows, &Wd, experts, arg_ptr<const uint32_t>(d, 4),
+                                    arg_ptr<const uint32_t>(d, 5), preweighted ? nullptr : arg_ptr<const uint16_t>(d, rw_slot),
+                                    has_shared ? arg_ptr<const uint16_t>(d, shared_slot) : nullptr, has_shared ? &Ws : nullptr,
+                                    has_extra ? arg_ptr<const uint16_t>(d, extra_slot) : nullptr, tokens, top_k,
+                                    arg_ptr<uint16_t>(d, out_slot), arg_ptr<uint16_t>(d, ws_slot), l);
 }
 
 // x, W, scales, biases, [bias], [residual], y, workspace.  Parameters: m (= K), n, rows, has_bias, has_residual.

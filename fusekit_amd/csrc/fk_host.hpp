@@ -85,6 +85,14 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out);
 fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
                            const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out);
+// Routed down projection + weighted reduction (+ shared expert + residual): one fused launch for one token
+// of int4 weights, else routed GEMV -> shared GEMV -> ordered reduction chained in out->then (`parts`,
+// (routes + tokens) * O bf16, is only touched by the chain).
+fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const fk_weight* Wd, uint32_t n_experts,
+                                   const uint32_t* row_idx, const uint32_t* expert_idx, const uint16_t* route_weight,
+                                   const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual,
+                                   uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out);
+void set_routed_fused_reduce(bool on);
 fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight, const uint16_t* residual,
                             uint16_t* out_ptr, uint32_t n_tokens, uint32_t top_k, uint32_t O, bool has_shared,
                             Launch* out);

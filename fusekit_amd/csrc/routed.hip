@@ -21,6 +21,8 @@
 
 namespace fk {
 
+static bool t_routed_fused_reduce = true;   // off: always the three launches (tests compare the two)
+
 struct RoutedArgs {
     GemvArgs g;                    // geometry of ONE route; pointers at expert 0 / activation row 0 / route 0
     const uint32_t* expert_idx;    // [n_routes]
@@ -116,6 +118,148 @@ __global__ __launch_bounds__(256) void route_reduce_kernel(const RouteReduceArgs
     if (a.has_shared) acc = __fadd_rn(acc, bf16_bits_to_f32(a.parts[(size_t)(a.n_tokens * a.top_k + t) * a.O + o]));
     if (a.residual) acc = __fadd_rn(acc, bf16_bits_to_f32(a.residual[i]));
     a.out[i] = (uint16_t)f32_to_bf16_bits(acc);
+}
+
+// ---------------------------------------------------------------- down + reduce in one launch
+//
+// One token, int4: out[o] = T(sum_slots rw_r * T(W_down[e_r][o, :] . h[r, :]) + T(W_shared[o, :] . shared_x)
+// + residual[o]), the sum in slot order with the reference's roundings (routed_qmv_reduce.rs:236-322),
+// without the per-route partial rows ever leaving the chip: a wave owns an output row, requests that row's
+// 16-byte pieces of every routed expert and of the shared matrix at once (lane c holds codes 32c .. 32c + 31),
+// reduces one dot product after the other across its lanes and adds them in slot order.  The activations of
+// all routes sit in LDS in the pairing the int4 dot wants, with the sum of every 32 of them for the bias term.
+constexpr int kDrBlock = 256, kDrWaves = kDrBlock / kWave, kDrRows = 2, kDrRoutes = 8, kDrSharedPasses = 2, kDrStage = 6;
+struct DownReduceArgs {
+    const uint16_t* h;             // [n_h_rows, K]
+    const uint4* w; const uint16_t* sc; const uint16_t* bi;      // stacked [E, O, ...]
+    const uint32_t* expert_idx;    // [top_k]
+    const uint32_t* row_idx;       // [top_k] row of h per slot, or null = the slot
+    const uint16_t* route_weight;  // [top_k] or null
+    const uint16_t* shared_x;      // [SK] or null
+    const uint4* sw; const uint16_t* ssc; const uint16_t* sbi;   // shared [O, SK]
+    const uint16_t* residual;      // [O] or null
+    uint16_t* out;                 // [O]
+    uint32_t K, SK, O, top_k, n_experts, n_h_rows, gdiv;         // gdiv: 32-code pieces per quantisation group
+};
+__global__ __launch_bounds__(kDrBlock) void routed_down_reduce_kernel(const DownReduceArgs a) {
+    extern __shared__ uint4 dr_lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t cpr = a.K / 32, scpr = a.SK / 32, gpr = cpr / a.gdiv, sgpr = scpr / a.gdiv;
+    const uint32_t routed8 = a.top_k * a.K / 8, total8 = routed8 + a.SK / 8;
+    uint4* xs = dr_lds;                                      // per route: [word slot 0..3][piece]
+    float* sx = reinterpret_cast<float*>(xs + total8);       // per route: [piece] sum of its 32 activations
+
+    uint32_t ex[kDrRoutes];
+#pragma unroll
+    for (int r = 0; r < kDrRoutes; ++r) {
+        const uint32_t e = a.expert_idx[(uint32_t)r < a.top_k ? r : 0u];
+        ex[r] = e < a.n_experts ? e : a.n_experts - 1;      // routed_qmv_swiglu.rs:138 clamps the same way
+    }
+    // every weight request of this wave's rows, before the activations are staged
+    // (scale and bias stay two raw values until they are used: combining them here would wait for each pair)
+    uint4 wq[kDrRows][kDrRoutes], wsq[kDrRows][kDrSharedPasses];
+    uint16_t sc_r[kDrRows][kDrRoutes], bi_r[kDrRows][kDrRoutes], sc_s[kDrRows][kDrSharedPasses], bi_s[kDrRows][kDrSharedPasses];
+#pragma unroll
+    for (int i = 0; i < kDrRows; ++i) {
+        const uint32_t o = blockIdx.x * (kDrRows * kDrWaves) + wave + i * kDrWaves;
+#pragma unroll
+        for (int r = 0; r < kDrRoutes; ++r) {
+            // a lane beyond the row repeats piece 0 (its result is dropped): no branch around the requests
+            const uint32_t c = lane < cpr ? lane : 0u;
+            const size_t row = (size_t)ex[r] * a.O + o;
+            const size_t g = row * gpr + c / a.gdiv;
+            wq[i][r] = a.w[row * cpr + c];
+            sc_r[i][r] = a.sc[g];
+            bi_r[i][r] = a.bi[g];
+        }
+#pragma unroll
+        for (int p = 0; p < kDrSharedPasses; ++p) {
+            const uint32_t c = lane + p * kWave;
+            wsq[i][p] = make_uint4(0, 0, 0, 0);
+            sc_s[i][p] = bi_s[i][p] = 0;
+            if (a.sw) {
+                const uint32_t cc = c < scpr ? c : 0u;
+                const size_t g = (size_t)o * sgpr + cc / a.gdiv;
+                wsq[i][p] = a.sw[(size_t)o * scpr + cc];
+                sc_s[i][p] = a.ssc[g];
+                bi_s[i][p] = a.sbi[g];
+            }
+        }
+    }
+    // activations: eight per thread and step, re-paired for the int4 dot, summed per 32.  The first
+    // kDrStage steps request all their rows before any is used (one memory round trip, not one per step).
+    auto source = [&](uint32_t j) __attribute__((always_inline)) {
+        if (j >= routed8) return a.shared_x + 8 * (j - routed8);
+        const uint32_t r = j / (a.K / 8), jl = j - r * (a.K / 8);
+        uint32_t row = a.row_idx ? a.row_idx[r] : r;
+        row = row < a.n_h_rows ? row : a.n_h_rows - 1;
+        return a.h + (size_t)row * a.K + 8 * jl;
+    };
+    auto place = [&](uint32_t j, const uint4& v) __attribute__((always_inline)) {
+        uint32_t base = routed8, jl = j - routed8, pieces = scpr;
+        if (j < routed8) {
+            const uint32_t r = j / (a.K / 8);
+            base = r * (a.K / 8); jl = j - base; pieces = cpr;
+        }
+        const uint32_t piece = jl >> 2, slot = jl & 3u;
+        uint4 pr;
+        pr.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);   // (x0, x2)
+        pr.y = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);   // (x4, x6)
+        pr.z = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);   // (x1, x3)
+        pr.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);   // (x5, x7)
+        xs[base + slot * pieces + piece] = pr;
+        float s8 = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+                   ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
+        s8 += __shfl_xor(s8, 1, kWave);
+        s8 += __shfl_xor(s8, 2, kWave);
+        if (slot == 0) sx[(base >> 2) + piece] = s8;
+    };
+    uint4 sv[kDrStage];
+#pragma unroll
+    for (int it = 0; it < kDrStage; ++it) {
+        const uint32_t j = tid + it * kDrBlock;
+        sv[it] = *reinterpret_cast<const uint4*>(source(j < total8 ? j : 0u));
+    }
+#pragma unroll
+    for (int it = 0; it < kDrStage; ++it) {
+        const uint32_t j = tid + it * kDrBlock;
+        if (j < total8) place(j, sv[it]);
+    }
+    for (uint32_t j = tid + kDrStage * kDrBlock; j < total8; j += kDrBlock) place(j, *reinterpret_cast<const uint4*>(source(j)));
+    __syncthreads();
+
+    auto piece_dot = [&](const uint4& wv, uint32_t scale, uint32_t bias, uint32_t base, uint32_t pieces, uint32_t c) __attribute__((always_inline)) {
+        float d0 = 0.f, d1 = 0.f;
+        d0 = q4_word_dot(wv.x, xs[base + c], d0);
+        d1 = q4_word_dot(wv.y, xs[base + pieces + c], d1);
+        d0 = q4_word_dot(wv.z, xs[base + 2 * pieces + c], d0);
+        d1 = q4_word_dot(wv.w, xs[base + 3 * pieces + c], d1);
+        return fmaf(bf16_bits_to_f32(scale), d0 + d1, bf16_bits_to_f32(bias) * sx[(base >> 2) + c]);
+    };
+#pragma unroll
+    for (int i = 0; i < kDrRows; ++i) {
+        const uint32_t o = blockIdx.x * (kDrRows * kDrWaves) + wave + i * kDrWaves;
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < kDrRoutes; ++r) {
+            if ((uint32_t)r >= a.top_k) break;
+            float d = lane < cpr ? piece_dot(wq[i][r], sc_r[i][r], bi_r[i][r], r * (a.K / 8), cpr, lane) : 0.f;
+            d = round_bf16(wave_sum(d));
+            const float rw = a.route_weight ? bf16_bits_to_f32(a.route_weight[r]) : 1.0f;
+            acc = __fadd_rn(acc, __fmul_rn(rw, d));
+        }
+        if (a.sw) {
+            float d = 0.f;
+#pragma unroll
+            for (int p = 0; p < kDrSharedPasses; ++p) {
+                const uint32_t c = lane + p * kWave;
+                if (c < scpr) d += piece_dot(wsq[i][p], sc_s[i][p], bi_s[i][p], routed8, scpr, c);
+            }
+            acc = __fadd_rn(acc, round_bf16(wave_sum(d)));
+        }
+        if (a.residual) acc = __fadd_rn(acc, bf16_bits_to_f32(a.residual[o]));
+        if (lane == 0) a.out[o] = (uint16_t)f32_to_bf16_bits(acc);
+    }
 }
 
 namespace {
@@ -240,5 +384,75 @@ fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight,
     out->set_args(a);
     return FK_OK;
 }
+
+// The fused form serves one token of int4 weights whose rows fit the lanes of a wave; anything else takes
+// the three launches.
+static bool down_reduce_fits(const fk_weight* Wd, const fk_weight* Ws, uint32_t n_tokens, uint32_t top_k) {
+    if (n_tokens != 1 || top_k > (uint32_t)kDrRoutes || Wd->bits != 4 || (Wd->group != 32 && Wd->group != 64 && Wd->group != 128))
+        return false;
+    if (Wd->k % Wd->group || Wd->k > 32u * kWave || Wd->n % (kDrRows * kDrWaves)) return false;
+    if (Ws && (Ws->bits != 4 || Ws->group != Wd->group || Ws->k % Ws->group || Ws->k > 32u * kWave * kDrSharedPasses)) return false;
+    const size_t lds = ((size_t)top_k * Wd->k + (Ws ? Ws->k : 0)) * (2 + 4.0 / 32);
+    return lds <= 60 * 1024;
+}
+
+fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const fk_weight* Wd, uint32_t n_experts,
+                                   const uint32_t* row_idx, const uint32_t* expert_idx, const uint16_t* route_weight,
+                                   const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual,
+                                   uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out) {
+    if (!Wd || !out_ptr || !h) return set_error(FK_ERR_INVALID, "routed reduce: null weight, input or output");
+    if (n_tokens == 0 || top_k == 0) return set_error(FK_ERR_INVALID, "routed reduce: empty route set");
+    if ((shared_x != nullptr) != (W_shared != nullptr))
+        return set_error(FK_ERR_INVALID, "routed reduce: shared_x and W_shared come together");
+    if (W_shared && (n_tokens != 1 || W_shared->n != Wd->n))
+        return set_error(FK_ERR_UNSUPPORTED, "routed reduce: shared expert needs one token and the same output width");
+    if ((uint64_t)n_tokens * top_k > 65536) return set_error(FK_ERR_UNSUPPORTED, "routed reduce: too many routes");
+    const uint32_t n_routes = n_tokens * top_k;
+    if (t_routed_fused_reduce && down_reduce_fits(Wd, W_shared, n_tokens, top_k)) {
+        const DeviceFacts* dev;
+        FK_TRY(device_facts(&dev));
+        if (!expert_idx) return set_error(FK_ERR_INVALID, "routed: null expert_idx");
+        if (n_experts == 0 || n_h_rows == 0) return set_error(FK_ERR_INVALID, "routed: experts and activation rows must be positive");
+        if (!Wd->w || !Wd->scales || !Wd->biases || (W_shared && (!W_shared->w || !W_shared->scales || !W_shared->biases)))
+            return set_error(FK_ERR_INVALID, "routed reduce: null weight arrays");
+        if (((uintptr_t)h | (uintptr_t)shared_x | (uintptr_t)Wd->w | (uintptr_t)(W_shared ? W_shared->w : nullptr)) & 15u)
+            return set_error(FK_ERR_INVALID, "routed reduce: activations and weights must be 16-byte aligned");
+        DownReduceArgs a;
+        memset(&a, 0, sizeof(a));
+        a.h = h;
+        a.w = static_cast<const uint4*>(Wd->w); a.sc = Wd->scales; a.bi = Wd->biases;
+        a.expert_idx = expert_idx; a.row_idx = row_idx; a.route_weight = route_weight;
+        a.shared_x = shared_x;
+        if (W_shared) { a.sw = static_cast<const uint4*>(W_shared->w); a.ssc = W_shared->scales; a.sbi = W_shared->biases; a.SK = W_shared->k; }
+        a.residual = residual; a.out = out_ptr;
+        a.K = Wd->k; a.O = Wd->n; a.top_k = top_k; a.n_experts = n_experts; a.n_h_rows = n_h_rows; a.gdiv = Wd->group / 32;
+        const size_t lds = ((size_t)top_k * a.K + a.SK) / 8 * 16 + ((size_t)top_k * a.K + a.SK) / 32 * 4;
+        out->func = reinterpret_cast<const void*>(&routed_down_reduce_kernel);
+        out->grid = dim3(a.O / (kDrRows * kDrWaves), 1, 1);
+        out->block = dim3(kDrBlock, 1, 1);
+        out->shmem = (uint32_t)lds;
+        out->set_args(a);
+        if (lds > 48 * 1024)
+            FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        return FK_OK;
+    }
+    if (!parts) return set_error(FK_ERR_INVALID, "routed reduce: workspace required");
+    FK_TRY(plan_routed_gemv(h, n_h_rows, Wd, nullptr, n_experts, row_idx, expert_idx, nullptr, n_routes, parts, out));
+    if (W_shared) {
+        GemvRequest rq;
+        rq.mats[0] = W_shared;
+        rq.y[0] = parts + (size_t)n_routes * Wd->n;
+        rq.x = shared_x;
+        Launch shared;
+        FK_TRY(plan_gemv(rq, &shared));
+        out->then.push_back(shared);
+    }
+    Launch reduce;
+    FK_TRY(plan_route_reduce(parts, route_weight, residual, out_ptr, n_tokens, top_k, Wd->n, W_shared != nullptr, &reduce));
+    out->then.push_back(reduce);
+    return FK_OK;
+}
+
+void set_routed_fused_reduce(bool on) { t_routed_fused_reduce = on; }
 
 }  // namespace fk

@@ -180,8 +180,9 @@ class MoeRuntime:
         self.kvb = B(c.n_heads * (c.nope_dim + c.v_dim) * 2)       # per head [k_nope | v]
         self.att = B(c.n_heads * c.v_dim * 2)
         self.mid = B(max(c.dense_inter, c.shared_inter) * 2)
-        self.route_logits = B(c.n_experts * 2)
-        self.route_idx, self.route_weight = z(4 * c.top_k), z(2 * c.top_k)
+        self.route_logits = z(c.n_experts * 2 * c.n_layers)   # one slot per layer, like the routes
+        # one slot per layer, so that the routes of a whole step can be read back after it
+        self.route_idx, self.route_weight = z(4 * c.top_k * c.n_layers), z(2 * c.top_k * c.n_layers)
         self.route_scale = DeviceBuffer.from_numpy(_bf16(np.array([c.route_scale], np.float32)))
         self.rows_x = z(4 * c.top_k)                                # every route reads activation row 0
         self.rows_h = DeviceBuffer.from_numpy(np.arange(c.top_k, dtype=np.uint32))
@@ -269,23 +270,26 @@ class MoeRuntime:
                                   dict(quant, m=c.dense_inter, n=c.hidden)))
                 continue
             Wr = w.mats[p + "mlp.gate"]
+            ridx = arg(self.route_idx, 4 * c.top_k, 4 * c.top_k * l)
+            rlg = arg(self.route_logits, 2 * c.n_experts, 2 * c.n_experts * l)
+            rwt = arg(self.route_weight, 2 * c.top_k, 2 * c.top_k * l)
             if self.fused_router:   # norm + router projection + top-k route in one single-block launch
                 t.append(Dispatch(name("moe_router"),
-                                  [arg(self.x[1]), arg(post), arg(Wr.w), arg(self.route_scale), arg(self.xn), arg(self.route_logits),
-                                   arg(self.route_idx), arg(self.route_weight), arg(self.router_ws)],
+                                  [arg(self.x[1]), arg(post), arg(Wr.w), arg(self.route_scale), arg(self.xn), rlg,
+                                   ridx, rwt, arg(self.router_ws)],
                                   dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1)))
             else:
                 t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(post), arg(self.xn)],
                                   dict(rows=1, hidden=c.hidden, eps=c.eps)))
-                t.append(Dispatch(name("qgemv"), [arg(self.xn), arg(Wr.w), arg(self.route_logits)],
+                t.append(Dispatch(name("qgemv"), [arg(self.xn), arg(Wr.w), rlg],
                                   dict(bits=16, group=64, m=c.hidden, n=c.n_experts)))
                 t.append(Dispatch(name("softmax_topk_route"),
-                                  [arg(self.route_logits), arg(self.route_scale), arg(self.route_idx), arg(self.route_weight)],
+                                  [rlg, arg(self.route_scale), ridx, rwt],
                                   dict(row_n=c.n_experts, top_k=c.top_k, rows=1)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             t.append(Dispatch(name("routed_qmv_swiglu"),
                               [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
-                               arg(self.rows_x), arg(self.route_idx), arg(self.h)],
+                               arg(self.rows_x), ridx, arg(self.h)],
                               dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, x_rows=1)))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
             t.append(Dispatch(name("qmv_swiglu"),
@@ -293,8 +297,8 @@ class MoeRuntime:
                                arg(self.mid, c.shared_inter * 2)],
                               dict(quant, hidden=c.hidden, inter=c.shared_inter, eps=c.eps, variant=c.swiglu_variant, has_norm=0)))
             t.append(Dispatch(name("routed_qmv_reduce"),
-                              [arg(self.h), arg(Ed.w), arg(Ed.scales), arg(Ed.biases), arg(self.rows_h), arg(self.route_idx),
-                               arg(self.route_weight), arg(self.mid, c.shared_inter * 2), arg(Sd.w), arg(Sd.scales), arg(Sd.biases),
+                              [arg(self.h), arg(Ed.w), arg(Ed.scales), arg(Ed.biases), arg(self.rows_h), ridx,
+                               rwt, arg(self.mid, c.shared_inter * 2), arg(Sd.w), arg(Sd.scales), arg(Sd.biases),
                                arg(self.x[1]), arg(self.x[0]), arg(self.moe_ws)],
                               dict(quant, k=c.moe_inter, o=c.hidden, experts=c.n_experts, tokens=1, top_k=c.top_k, x_rows=c.top_k,
                                    has_shared=1, shared_k=c.shared_inter, has_extra=1)))
@@ -305,6 +309,14 @@ class MoeRuntime:
                           [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history), arg(self.hist_counter)],
                           dict(vocab=c.vocab)))
         return t
+
+    def routes(self) -> np.ndarray:
+        """Expert indices the last replay chose, [n_layers, top_k] (rows of dense layers stay zero)."""
+        return self.route_idx.to_numpy(np.uint32, (self.cfg.n_layers, self.cfg.top_k))
+
+    def router_logits(self) -> np.ndarray:
+        """bf16 router logits of the last replay, [n_layers, n_experts]."""
+        return self.route_logits.to_numpy(np.uint16, (self.cfg.n_layers, self.cfg.n_experts))
 
     # -- generation (the dense runtime's loop: prompt with forced tokens, then chunks fed back on the GPU)
     def reset(self) -> None:

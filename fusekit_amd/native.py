@@ -213,6 +213,10 @@ def routed_qmv_reduce(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_wei
                                    _ptr(stream)))
 
 
+def set_routed_fused_reduce(on: bool) -> None:
+    lib.fk_set_routed_fused_reduce(C.c_int(int(on)))
+
+
 def qgemm_workspace_bytes(m, n, k, group=64) -> int:
     out = C.c_size_t(0)
     check(lib.fk_qgemm_workspace_bytes(C.c_uint32(m), C.c_uint32(n), C.c_uint32(k), C.c_uint32(group), C.byref(out)))

@@ -173,6 +173,10 @@ fk_status fk_routed_qmv_reduce(const uint16_t *h, uint32_t n_h_rows, const fk_we
                                const uint32_t *row_idx, const uint32_t *expert_idx, const uint16_t *route_weight,
                                const uint16_t *shared_x, const fk_weight *W_shared, const uint16_t *residual_extra,
                                uint32_t n_tokens, uint32_t top_k, uint16_t *out, void *workspace, fk_stream s);
+/* One token of int4 weights takes ONE launch (a wave per output row walks every route and the shared
+ * expert and adds them in slot order; the workspace is then not touched); other shapes take three
+ * (routed GEMV, shared GEMV, ordered reduction).  fk_set_routed_fused_reduce(0) forces the three. */
+void fk_set_routed_fused_reduce(int on);
 
 /* G   multi-row quantised matmul on the matrix cores: y[m, N] = T(x[m, K] @ dequant(W)^T
  *     (+ bias[N]) (+ residual[m, N])), fp32 accumulate, one round.  Replaces the

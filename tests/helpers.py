@@ -154,8 +154,15 @@ class OracleMoeDecoder:
         self.cv = [np.zeros(c.n_heads * c.capacity * c.v_dim, np.uint16) for _ in range(c.n_layers)]
         self.route_scale = oracle.f32_to_bf16(np.array([c.route_scale], np.float32))
         self.routes = []          # expert indices of the last step, per MoE layer
+        self.forced = 0           # layers (over all steps) where the forced routes differed from the oracle's own
+        self.router_drift = 0.0   # largest rel-L2 between the GPU's and the oracle's router logits of a layer
 
-    def step(self, token: int, offset: int, want_logits: bool = False):
+    def step(self, token: int, offset: int, want_logits: bool = False, forced_routes=None, gpu_router_logits=None):
+        """forced_routes [n_layers, top_k] with gpu_router_logits [n_layers, n_experts]: follow the GPU's routes.
+        Routing is a discrete function of the router logits, and those carry the stack's accumulated rounding
+        drift, so near the k-th probability the GPU and the oracle may choose differently.  Checked instead:
+        the GPU's logits are close to the oracle's, and its route is EXACTLY the oracle's router applied to the
+        GPU's own logits; the oracle then continues with those experts and its own probabilities for them."""
         c, m, v = self.cfg, self.mat, self.vec
         x = oracle.embed_lookup(m["embed_tokens"], token)
         packed = c.nope_dim + c.v_dim
@@ -189,6 +196,18 @@ class OracleMoeDecoder:
             logits = oracle.qgemv(m[p + "mlp.gate"], xn)
             idx, rw = oracle.softmax_topk_route(logits, c.top_k, self.route_scale)
             idx, rw = idx.reshape(-1), rw.reshape(-1)
+            if forced_routes is not None:
+                gl = np.ascontiguousarray(gpu_router_logits[l])
+                fg, fo = oracle.bf16_to_f32(gl).astype(np.float64), oracle.bf16_to_f32(logits).astype(np.float64)
+                self.router_drift = max(self.router_drift, float(np.linalg.norm(fg - fo) / np.linalg.norm(fo)))
+                own_idx, _ = oracle.softmax_topk_route(gl, c.top_k, self.route_scale)
+                assert set(own_idx.reshape(-1).tolist()) == set(forced_routes[l].tolist()), (l, own_idx, forced_routes[l])
+                if set(forced_routes[l].tolist()) != set(idx.tolist()):
+                    all_idx, all_w = oracle.softmax_topk_route(logits, c.n_experts - 1, self.route_scale)
+                    prob = dict(zip(all_idx.reshape(-1).tolist(), oracle.bf16_to_f32(all_w.reshape(-1)).tolist()))
+                    idx = forced_routes[l].astype(np.uint32)
+                    rw = oracle.f32_to_bf16(np.array([prob.get(int(e), 0.0) for e in idx], np.float32))
+                    self.forced += 1
             self.routes.append(idx.copy())
             h = oracle.routed_qmv_swiglu(xn.reshape(1, -1), m[p + "mlp.switch_mlp.gate_proj"], m[p + "mlp.switch_mlp.up_proj"],
                                          np.zeros(c.top_k, np.uint32), idx, None)

@@ -35,7 +35,7 @@ def test_greedy_tokens_and_routes_match_oracle(fk, bits, traditional, kw):
     for i, (g, r) in enumerate(zip(got, ref)):
         assert g == r, f"step {i}: gpu {g} oracle {r} (oracle margin {margins[i]})"
     # the routes of the last step (the last MoE layer's are still in the buffers)
-    assert sorted(rt.route_idx.to_numpy(np.uint32).tolist()) == sorted(od.routes[-1].tolist())
+    assert sorted(rt.routes()[-1].tolist()) == sorted(od.routes[-1].tolist())
     # replay determinism
     again, _, _ = rt.generate(prompt, n)
     assert again == got
@@ -57,34 +57,43 @@ def test_logits_close_after_each_prompt_token(fk):
 def test_full_size_model_32_greedy_tokens(fk):
     """The MoE benchmark model at full size (27 layers, hidden 2048, 64 experts of 1408, top-6 + 2 shared,
     16 heads of 128 + 64 / 128, vocab 102400, int4 g64): 32 greedy steps against the oracle on the same
-    weight bytes, teacher-forced on the oracle's tokens so that every step is checked.  As for the dense
-    model, a GPU token must be among the oracle's candidates within two bf16 steps of its maximum, and
-    must equal the oracle's wherever that set has one member; the last step's logits agree to 5e-2."""
+    weight bytes, teacher-forced on the oracle's tokens so that every step is checked.
+
+    Routing is discrete: where the sixth and seventh router probabilities are close, the rounding drift of
+    the stack (fp32 against double accumulation, ~3e-2 on the final logits as in the dense model) decides
+    which expert runs -- measured: 2 or 3 of the 26 layers per step -- and a different expert changes the
+    layer's output by far more than a rounding.  So the oracle follows the GPU's routes (read back per step,
+    one slot per layer) after checking that the GPU's router logits are close to its own (5e-2) and that the
+    GPU's route is exactly the oracle's router applied to the GPU's logits.  With equal routes the comparison
+    is the dense model's: a GPU token must be among the oracle's candidates within two bf16 steps of its
+    maximum, must equal the oracle's where that set has one member, and the last logits agree to 5e-2."""
     from fusekit_amd.moe_decoder import MoeConfig, MoeRuntime, MoeWeights
     cfg = MoeConfig(capacity=128)
     W = MoeWeights.random_init(cfg, seed=0)
     rt, od = MoeRuntime(cfg, W), OracleMoeDecoder(cfg, W)
     prompt = rng(0).integers(0, cfg.vocab, 4).tolist()
     n = 32
-    ref, cands, seq, route_match = [], [], list(prompt), []
+    ref, cands, preds, seq = [], [], [], list(prompt)
     for i in range(len(prompt) + n - 1):
-        nxt, m, logits = od.step(seq[i], i, want_logits=True)
+        got, _ = rt.d.decode_host_loop(rt.graph, rt.uniforms, i, [seq[i]])
+        nxt, m, logits = od.step(seq[i], i, want_logits=True, forced_routes=rt.routes(), gpu_router_logits=rt.router_logits())
         if i >= len(prompt) - 1:
             f = oracle.bf16_to_f32(logits)
             top = float(f.max())
             ulp = 2.0 ** (np.floor(np.log2(abs(top))) - 7)
-            ref.append(nxt); cands.append(set(np.nonzero(f >= top - 2 * ulp)[0].tolist()))
+            ref.append(nxt); cands.append(set(np.nonzero(f >= top - 2 * ulp)[0].tolist())); preds.append(got[0])
             seq.append(nxt)
-    preds, _ = rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, seq[:-1])
-    preds = preds[len(prompt) - 1:]
     exact = sum(int(g == r) for g, r in zip(preds, ref))
-    print(f"teacher-forced: {exact}/{n} steps pick the oracle's token; candidates per step {[len(c) for c in cands]}")
+    print(f"teacher-forced: {exact}/{n} steps pick the oracle's token; candidates per step {[len(c) for c in cands]}; "
+          f"{od.forced} of {(len(prompt) + n - 1) * (cfg.n_layers - cfg.first_dense)} layer routes differed by a near-tie")
     for i, (g, r) in enumerate(zip(preds, ref)):
         assert g in cands[i], f"step {i}: gpu {g} not among {sorted(cands[i])} (oracle {r})"
         if len(cands[i]) == 1:
             assert g == r
     assert exact >= n - 6
-    assert sorted(rt.route_idx.to_numpy(np.uint32).tolist()) == sorted(od.routes[-1].tolist())
+    print(f"largest router-logit drift of a layer {od.router_drift:.3e}")
+    assert od.router_drift <= 5e-2
+    assert od.forced <= 0.2 * (len(prompt) + n - 1) * (cfg.n_layers - cfg.first_dense)
     g = oracle.bf16_to_f32(rt.logits.to_numpy(np.uint16)).astype(np.float64)
     r = oracle.bf16_to_f32(logits).astype(np.float64)
     rel = np.linalg.norm(g - r) / np.linalg.norm(r)

@@ -120,6 +120,34 @@ def test_routed_reduce_one_token(fk, bits, preweighted, shared, residual):
     assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
 
 
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("E,O,K,top_k,SK,with_rows", [(16, 2048, 1408, 6, 2816, False), (8, 320, 448, 6, 256, True),
+                                                      (4, 64, 2048, 8, 4096, False), (4, 128, 64, 1, 0, False)])
+def test_routed_reduce_one_launch_and_three(fk, fused, E, O, K, top_k, SK, with_rows):
+    """One token of int4 weights: the single-launch form (a wave per output row, routes added in slot order)
+    and the three-launch form both meet the oracle; fk_set_routed_fused_reduce picks."""
+    Wd = _stack(2000, E, O, K, 4)
+    n_rows = top_k + 2 if with_rows else top_k
+    h = normal_bf16(30, (n_rows, K), 0.0, 0.5)
+    row_idx = rng(31).permutation(n_rows)[:top_k].astype(np.uint32) if with_rows else None
+    expert_idx = rng(32).integers(0, E + 2, top_k).astype(np.uint32)      # some beyond E: clamped
+    rw = normal_bf16(33, top_k, 0.15, 0.2)
+    Ws = make_qweight(2100, O, SK, 4) if SK else None
+    sx = normal_bf16(34, (1, SK)) if SK else None
+    res = normal_bf16(35, (1, O))
+    fk.set_routed_fused_reduce(fused)
+    try:
+        got = _run_m2(fk, h, Wd, row_idx, expert_idx, rw, sx, Ws, res, 1, top_k)
+    finally:
+        fk.set_routed_fused_reduce(True)
+    clamped = np.minimum(expert_idx, E - 1)
+    ref = oracle.routed_qmv_reduce(h, Wd, clamped, rw, res, 1, top_k, row_idx=row_idx, shared_x=sx, Wshared=Ws)
+    hh = h if row_idx is None else h[row_idx]
+    assert rel_l2(got, _m2_fp32(hh, Wd, clamped, rw, sx, Ws, res, 1, top_k)) <= REL_L2_BAR
+    frac, ulps = bf16_mismatch(got, ref)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+
+
 def test_routed_reduce_tokens_and_row_idx(fk):
     E, O, K, tokens, top_k = 4, 192, 256, 3, 2
     Wd = _stack(700, E, O, K, 4)
