@@ -260,6 +260,16 @@ fk_status fk_routed_qmv_swiglu(const uint16_t* x, uint32_t n_x_rows, const fk_we
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_routed_qmv_swiglu_shared(const uint16_t* x, const fk_weight* Wg, const fk_weight* Wu, uint32_t n_experts,
+                                      const uint32_t* expert_idx, const uint16_t* route_weight, uint32_t n_routes,
+                                      uint16_t* out0, const fk_weight* Sg, const fk_weight* Su, uint16_t* shared_out,
+                                      fk_stream s) {
+    if (!Wg || !Wu || !Sg || !Su) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_shared: null weight");
+    Launch l;
+    FK_TRY(plan_routed_gemv(x, 1, Wg, Wu, n_experts, nullptr, expert_idx, route_weight, n_routes, out0, &l, Sg, Su, shared_out));
+    return run_launch(l, (hipStream_t)s);
+}
+
 size_t fk_routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim) {
     return ((size_t)n_tokens * top_k + n_tokens) * out_dim * sizeof(uint16_t);
 }

@@ -701,9 +701,10 @@ fk_status plan_sdpa_quant_d(const Dispatch& d, Launch* l, SlotRW* rw, uint32_t b
 fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
     const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("k"), O = d.u("o");
     const uint32_t experts = d.u("experts"), routes = d.u("routes"), x_rows = d.u("x_rows", 1);
-    const bool pre_scale = d.u("pre_scale", 0) != 0;
+    const bool pre_scale = d.u("pre_scale", 0) != 0, has_shared = d.u("has_shared", 0) != 0;
     const size_t n_slots = pre_scale ? 11 : 10;
-    FK_TRY(need_args(d, n_slots));
+    // with has_shared = 1: + shared gate w / s / b, shared up w / s / b, shared_out (parameter shared_o rows)
+    FK_TRY(need_args(d, n_slots + (has_shared ? 7 : 0)));
     if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
     if (experts == 0 || routes == 0 || K == 0 || O == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": k / o / experts / routes parameters missing");
@@ -717,9 +718,22 @@ fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (pre_scale) FK_TRY(need_bytes(d, 9, (size_t)routes * 2));
     FK_TRY(need_bytes(d, n_slots - 1, (size_t)routes * O * 2));
     all_but_last(n_slots, 1, rw);
+    fk_weight Sg, Su;
+    uint16_t* shared_out = nullptr;
+    if (has_shared) {
+        const uint32_t so = d.u("shared_o");
+        if (so == 0) return set_error(FK_ERR_INVALID, d.kernel + ": shared_o parameter missing");
+        FK_TRY(bind_weight(d, bits, group, so, K, n_slots, n_slots + 1, n_slots + 2, &Sg));
+        FK_TRY(bind_weight(d, bits, group, so, K, n_slots + 3, n_slots + 4, n_slots + 5, &Su));
+        FK_TRY(need_bytes(d, n_slots + 6, (size_t)so * 2));
+        shared_out = arg_ptr<uint16_t>(d, n_slots + 6);
+        for (uint32_t i = 0; i < 6; ++i) rw->reads.push_back((uint32_t)n_slots + i);
+        rw->writes.push_back((uint32_t)n_slots + 6);
+    }
     return plan_routed_gemv(arg_ptr<const uint16_t>(d, 0), x_rows, &Wg, &Wu, experts, arg_ptr<const uint32_t>(d, 7),
                             arg_ptr<const uint32_t>(d, 8), pre_scale ? arg_ptr<const uint16_t>(d, 9) : nullptr, routes,
-                            arg_ptr<uint16_t>(d, n_slots - 1), l);
+                            arg_ptr<uint16_t>(d, n_slots - 1), l, has_shared ? &Sg : nullptr, has_shared ? &Su : nullptr,
+                            shared_out);
 }
 
 // x, wq, scales, biases, row_idx, expert_idx, [route_weight], [shared_x, shared_w, shared_s, shared_b],

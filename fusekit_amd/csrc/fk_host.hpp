@@ -84,7 +84,8 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out);
 // Mixture-of-experts routed projections (w_b non-null: gate/up pair with SwiGLU).
 fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
-                           const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out);
+                           const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out,
+                           const fk_weight* sh_a = nullptr, const fk_weight* sh_b = nullptr, uint16_t* sh_y = nullptr);
 // Routed down projection + weighted reduction (+ shared expert + residual): one fused launch for one token
 // of int4 weights, else routed GEMV -> shared GEMV -> ordered reduction chained in out->then (`parts`,
 // (routes + tokens) * O bf16, is only touched by the chain).

@@ -32,6 +32,14 @@ struct RoutedArgs {
     uint32_t w_stride;             // 16-byte chunks per expert
     uint32_t s_stride;             // scale (= bias) elements per expert
     uint32_t y_stride;             // output elements per route
+    // Shared experts as extra routes (one token): routes n_routes .. n_routes + x_routes - 1 read row block
+    // (route - n_routes) of these matrices -- [x_routes * O, K], i.e. a stack of their own -- unweighted,
+    // into xy [x_routes * O]: the shared gate/up pair rides in the routed launch.
+    const uint4* xw[2];
+    const uint16_t* xsc[2];
+    const uint16_t* xbi[2];
+    uint16_t* xy;
+    uint32_t n_routes, x_routes;
 };
 
 // GemvArgs as one route sees it.  n_mats is a compile-time 1 so that every index
@@ -60,19 +68,25 @@ template <WKind KIND, int NSEG>
 __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArgs a) {
     extern __shared__ uint4 lds_raw[];
     const uint32_t route = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - route * a.blocks_per_route;
-    uint32_t e = a.expert_idx[route];
+    const bool extra = route >= a.n_routes;     // uniform per block
+    const uint32_t lookup = extra ? 0u : route;
+    uint32_t e = a.expert_idx[lookup];
     e = e < a.n_experts ? e : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
-    uint32_t row = a.row_idx ? a.row_idx[route] : route;
+    uint32_t row = a.row_idx ? a.row_idx[lookup] : lookup;
     row = row < a.n_x_rows ? row : a.n_x_rows - 1;
+    if (extra) {
+        e = route - a.n_routes;
+        row = 0;
+    }
 
     RouteView v;
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
-        v.w[m] = a.g.w[m] + (size_t)e * a.w_stride;
-        v.sc[m] = a.g.sc[m] + (size_t)e * a.s_stride;
-        v.bi[m] = a.g.bi[m] + (size_t)e * a.s_stride;
+        v.w[m] = (extra ? a.xw[m] : a.g.w[m]) + (size_t)e * a.w_stride;
+        v.sc[m] = (extra ? a.xsc[m] : a.g.sc[m]) + (size_t)e * a.s_stride;
+        v.bi[m] = (extra ? a.xbi[m] : a.g.bi[m]) + (size_t)e * a.s_stride;
         v.bias[m] = nullptr;
-        v.y[m] = a.g.y[m] + (size_t)route * a.y_stride;
+        v.y[m] = extra ? a.xy + (size_t)e * a.y_stride : a.g.y[m] + (size_t)route * a.y_stride;
         v.n[m] = a.g.n[m];
         v.tile_start[m] = 0;
     }
@@ -84,7 +98,7 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
     v.res = nullptr;
     v.res2 = nullptr;
     v.swiglu_variant = 1;
-    v.y_scale = a.route_weight ? bf16_bits_to_f32(a.route_weight[route]) : 1.0f;
+    v.y_scale = (a.route_weight && !extra) ? bf16_bits_to_f32(a.route_weight[lookup]) : 1.0f;
 
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
@@ -301,10 +315,21 @@ uint32_t resident_blocks(const void* func, uint32_t lds_bytes, int cus) {
 // are the base of the stacked tensors.
 fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
-                           const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out) {
+                           const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out,
+                           const fk_weight* sh_a, const fk_weight* sh_b, uint16_t* sh_y) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!expert_idx) return set_error(FK_ERR_INVALID, "routed: null expert_idx");
+    uint32_t x_routes = 0;
+    if (sh_a) {
+        if (!w_b || !sh_b || !sh_y) return set_error(FK_ERR_INVALID, "routed: shared experts come as a gate/up pair with an output");
+        if (n_x_rows != 1) return set_error(FK_ERR_UNSUPPORTED, "routed: shared experts ride along for one token only");
+        for (const fk_weight* w : {sh_a, sh_b})
+            if (!w->w || w->k != w_a->k || w->bits != w_a->bits || w->group != w_a->group || w->n != sh_a->n || w->n == 0 ||
+                w->n % w_a->n || (w->bits != 16 && (!w->scales || !w->biases)))
+                return set_error(FK_ERR_INVALID, "routed: shared matrices must be whole row blocks of the expert shape");
+        x_routes = sh_a->n / w_a->n;
+    }
     if (n_experts == 0 || n_routes == 0 || n_x_rows == 0)
         return set_error(FK_ERR_INVALID, "routed: experts, routes and activation rows must be positive");
     if (n_routes > 65536) return set_error(FK_ERR_UNSUPPORTED, "routed: at most 65536 routes per launch");
@@ -324,13 +349,14 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
     // Two passes: the first sizes LDS with a nominal grid, the second plans the
     // tiles for the share of the resident blocks one route gets.
     Launch base;
-    uint32_t per_route = (uint32_t)dev->cus * 4u / n_routes;
+    const uint32_t all_routes = n_routes + x_routes;
+    uint32_t per_route = (uint32_t)dev->cus * 4u / all_routes;
     for (int pass = 0; pass < 2; ++pass) {
         t_gemv_grid_override = per_route ? per_route : 1u;
         const fk_status s = plan_gemv(rq, &base);
         t_gemv_grid_override = 0;
         FK_TRY(s);
-        per_route = resident_blocks(func, base.shmem, dev->cus) / n_routes;
+        per_route = resident_blocks(func, base.shmem, dev->cus) / all_routes;
     }
     GemvArgs g;
     memcpy(&g, base.args, sizeof(g));
@@ -351,9 +377,17 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
     a.w_stride = (uint32_t)w_stride;
     a.s_stride = (uint32_t)s_stride;
     a.y_stride = w_a->n;
+    a.n_routes = n_routes;
+    a.x_routes = x_routes;
+    if (sh_a) {
+        a.xw[0] = static_cast<const uint4*>(sh_a->w); a.xw[1] = static_cast<const uint4*>(sh_b->w);
+        a.xsc[0] = sh_a->scales; a.xsc[1] = sh_b->scales;
+        a.xbi[0] = sh_a->biases; a.xbi[1] = sh_b->biases;
+        a.xy = sh_y;
+    }
 
     out->func = func;
-    out->grid = dim3(base.grid.x * n_routes, 1, 1);
+    out->grid = dim3(base.grid.x * all_routes, 1, 1);
     out->block = dim3(kGemvBlock, 1, 1);
     out->shmem = base.shmem;
     out->set_args(a);

@@ -53,6 +53,7 @@ class MoeConfig:
     group: int = 64
     swiglu_variant: int = 1
     capacity: int = 1024
+    fuse_shared: bool = True   # the shared experts' gate/up pair as further routes of the routed launch
     fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
 
     @property
@@ -287,15 +288,21 @@ class MoeRuntime:
                                   [rlg, arg(self.route_scale), ridx, rwt],
                                   dict(row_n=c.n_experts, top_k=c.top_k, rows=1)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
-            t.append(Dispatch(name("routed_qmv_swiglu"),
-                              [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
-                               arg(self.rows_x), ridx, arg(self.h)],
-                              dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, x_rows=1)))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
-            t.append(Dispatch(name("qmv_swiglu"),
-                              [arg(self.xn), arg(Sg.w), arg(Su.w), arg(Sg.scales), arg(Su.scales), arg(Sg.biases), arg(Su.biases),
-                               arg(self.mid, c.shared_inter * 2)],
-                              dict(quant, hidden=c.hidden, inter=c.shared_inter, eps=c.eps, variant=c.swiglu_variant, has_norm=0)))
+            routed = [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
+                      arg(self.rows_x), ridx, arg(self.h)]
+            rparams = dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, x_rows=1)
+            if c.fuse_shared and c.swiglu_variant == 1:   # the shared pair as further routes of the routed launch
+                t.append(Dispatch(name("routed_qmv_swiglu"),
+                                  routed + [arg(Sg.w), arg(Sg.scales), arg(Sg.biases), arg(Su.w), arg(Su.scales), arg(Su.biases),
+                                            arg(self.mid, c.shared_inter * 2)],
+                                  dict(rparams, has_shared=1, shared_o=c.shared_inter)))
+            else:
+                t.append(Dispatch(name("routed_qmv_swiglu"), routed, rparams))
+                t.append(Dispatch(name("qmv_swiglu"),
+                                  [arg(self.xn), arg(Sg.w), arg(Su.w), arg(Sg.scales), arg(Su.scales), arg(Sg.biases), arg(Su.biases),
+                                   arg(self.mid, c.shared_inter * 2)],
+                                  dict(quant, hidden=c.hidden, inter=c.shared_inter, eps=c.eps, variant=c.swiglu_variant, has_norm=0)))
             t.append(Dispatch(name("routed_qmv_reduce"),
                               [arg(self.h), arg(Ed.w), arg(Ed.scales), arg(Ed.biases), arg(self.rows_h), ridx,
                                rwt, arg(self.mid, c.shared_inter * 2), arg(Sd.w), arg(Sd.scales), arg(Sd.biases),

@@ -197,6 +197,14 @@ def routed_qmv_swiglu(x, n_x_rows, Wg, Wu, n_experts, row_idx, expert_idx, route
                                    C.c_uint32(n_routes), _ptr(out0), _ptr(stream)))
 
 
+def routed_qmv_swiglu_shared(x, Wg, Wu, n_experts, expert_idx, route_weight, n_routes, out0, Sg, Su, shared_out,
+                             stream=None) -> None:
+    """One token: the routed gate/up + SwiGLU with the shared experts' pair as further routes of the same launch."""
+    check(lib.fk_routed_qmv_swiglu_shared(_ptr(x), C.byref(Wg.c), C.byref(Wu.c), C.c_uint32(n_experts), _ptr(expert_idx),
+                                          _ptr(route_weight), C.c_uint32(n_routes), _ptr(out0), C.byref(Sg.c), C.byref(Su.c),
+                                          _ptr(shared_out), _ptr(stream)))
+
+
 lib.fk_routed_reduce_workspace_bytes.restype = C.c_size_t
 
 

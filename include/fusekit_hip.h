@@ -159,6 +159,14 @@ fk_status fk_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps,
 fk_status fk_routed_qmv_swiglu(const uint16_t *x, uint32_t n_x_rows, const fk_weight *Wg, const fk_weight *Wu,
                                uint32_t n_experts, const uint32_t *row_idx, const uint32_t *expert_idx,
                                const uint16_t *route_weight, uint32_t n_routes, uint16_t *out0, fk_stream s);
+/* The same launch with the block's SHARED experts riding along (one token): Sg / Su [n_shared * O, K] are
+ * read as n_shared further routes -- row block j into shared_out [j * O ..) -- unweighted, with the same SwiGLU
+ * (the reference runs them as a separate qmv_swiglu launch, src/codegen/kernels/qmv_swiglu.rs:20-246; the
+ * arithmetic per output is that kernel's).  Every route reads the one activation row x [K]. */
+fk_status fk_routed_qmv_swiglu_shared(const uint16_t *x, const fk_weight *Wg, const fk_weight *Wu, uint32_t n_experts,
+                                      const uint32_t *expert_idx, const uint16_t *route_weight, uint32_t n_routes,
+                                      uint16_t *out0, const fk_weight *Sg, const fk_weight *Su, uint16_t *shared_out,
+                                      fk_stream s);
 
 /* M2  routed down projection + weighted reduction (+ shared expert + residual).
  *     Replaces src/codegen/kernels/routed_qmv_reduce.rs:14-460.  h is [n_h_rows, k]

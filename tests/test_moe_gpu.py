@@ -78,6 +78,29 @@ def test_routed_swiglu_rows_and_clamp(fk):
     assert np.array_equal(got2[-1], got[-1])  # the last route already read the last row
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_routed_swiglu_with_shared_experts_riding_along(fk, bits):
+    """fk_routed_qmv_swiglu_shared: the routed outputs are the plain routed launch's bits, the shared outputs
+    the dense gate/up + SwiGLU pair's (variant B, no norm) on the same activation row."""
+    E, O, K, top_k, n_shared = 8, 192, 256, 3, 2
+    Wg, Wu = _stack(2200, E, O, K, bits), _stack(2300, E, O, K, bits)
+    Sg, Su = make_qweight(2400, n_shared * O, K, bits), make_qweight(2500, n_shared * O, K, bits)
+    x = normal_bf16(40, (1, K))
+    expert_idx = np.array([5, 0, 7], np.uint32)
+    rw = normal_bf16(41, top_k, 0.2, 0.4)
+    out0, shared = fk.DeviceBuffer(2 * top_k * O), fk.DeviceBuffer(2 * n_shared * O)
+    fk.routed_qmv_swiglu_shared(_dev(fk, x), to_device(fk, Wg), to_device(fk, Wu), E, _dev(fk, expert_idx), _dev(fk, rw), top_k,
+                                out0, to_device(fk, Sg), to_device(fk, Su), shared)
+    plain = _run_m1(fk, x, Wg, Wu, np.zeros(top_k, np.uint32), expert_idx, rw)
+    assert np.array_equal(out0.to_numpy(np.uint16, (top_k, O)), plain)
+    ref = oracle.gateup_swiglu(x.reshape(-1), None, 0.0, Sg, Su, 1)
+    frac, ulps = bf16_mismatch(shared.to_numpy(np.uint16), ref)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+    with pytest.raises(fk.InvalidArgument):    # shared matrices must be whole row blocks of the expert shape
+        fk.routed_qmv_swiglu_shared(_dev(fk, x), to_device(fk, Wg), to_device(fk, Wu), E, _dev(fk, expert_idx), None, top_k,
+                                    out0, to_device(fk, make_qweight(1, O + 64, K, bits)), to_device(fk, make_qweight(2, O + 64, K, bits)), shared)
+
+
 def _run_m2(fk, h, Wd, row_idx, expert_idx, rw, shared_x, Ws, res, tokens, top_k):
     out = fk.DeviceBuffer(2 * tokens * Wd.n)
     ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, Wd.n))
