@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void route_reduce_kernel(const RouteReduceArgs
 // 16-byte pieces of every routed expert and of the shared matrix at once (lane c holds codes 32c .. 32c + 31),
 // reduces one dot product after the other across its lanes and adds them in slot order.  The activations of
 // all routes sit in LDS in the pairing the int4 dot wants, with the sum of every 32 of them for the bias term.
-constexpr int kDrBlock = 256, kDrWaves = kDrBlock / kWave, kDrRows = 2, kDrRoutes = 8, kDrSharedPasses = 2, kDrStage = 6;
+constexpr int kDrBlock = 512, kDrWaves = kDrBlock / kWave, kDrRows = 1, kDrRoutes = 8, kDrSharedPasses = 2, kDrStage = 3;
 struct DownReduceArgs {
     const uint16_t* h;             // [n_h_rows, K]
     const uint4* w; const uint16_t* sc; const uint16_t* bi;      // stacked [E, O, ...]
