@@ -604,6 +604,25 @@ fk_status fk_rope_store_sdpa_decode(const uint16_t* q, const uint16_t* k, const 
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_split_store_sdpa_decode(const uint16_t* q, uint32_t n_heads, uint32_t q0_dim, uint32_t q1_dim,
+                                     const uint16_t* k0, uint32_t k0_stride, const uint16_t* k1, uint32_t k1_heads,
+                                     const uint16_t* v, uint32_t v_stride, uint32_t n_kv, uint32_t v_dim, uint32_t rope_dims,
+                                     int traditional, float theta, const float* rope_tab, uint16_t* cache_k,
+                                     uint16_t* cache_v, uint16_t* out, const uint32_t* d_kv_len, uint32_t kv_len,
+                                     uint32_t max_len, uint32_t capacity, float scale, float* partials, uint32_t* counters,
+                                     fk_stream s) {
+    SdpaFusion f;
+    f.k_new = k0; f.k1_new = k1; f.v_new = v;
+    f.q0_dim = q0_dim; f.k0_stride = k0_stride; f.v_stride = v_stride; f.k1_heads = k1_heads;
+    f.traditional = traditional ? 1u : 0u;
+    f.rope_dims = rope_dims; f.base_log2 = rope_dims ? theta_log2(theta) : 0.f; f.rope_tab = rope_tab;
+    if (q0_dim == 0 || q1_dim == 0) return set_error(FK_ERR_INVALID, "fk_split_store_sdpa_decode: both head parts must be non-empty");
+    Launch l;
+    FK_TRY(plan_sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_kv, q0_dim + q1_dim, v_dim,
+                            capacity, scale, partials, counters, &l, 1, nullptr, &f));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_copy(void* dst, const void* src, size_t nbytes, fk_stream s) {
     Launch l;
     FK_TRY(plan_copy(dst, src, nbytes, &l));

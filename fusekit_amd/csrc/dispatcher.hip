@@ -608,6 +608,54 @@ fk_status plan_rope_store_sdpa(const Dispatch& d, Launch* l, SlotRW* rw) {
                             arg_ptr<float>(d, c0 + 4), arg_ptr<uint32_t>(d, c0 + 5), l, 1, nullptr, &f);
 }
 
+// Q, K0, K1, V, cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]: split-key store + attention of a
+// layer in one launch.  Parameters as the split form of kv_cache_store_decode (n_heads, q0_dim, q1_dim, n_kv,
+// v_dim, k1_n_kv, k0_stride, v_stride, rope_dims, traditional, theta, capacity) plus max_len, scale, has_table.
+fk_status plan_split_store_sdpa(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const bool table = d.u("has_table", 0) != 0;
+    const size_t n = 10 + (table ? 1 : 0);
+    FK_TRY(need_args(d, n));
+    const uint32_t n_heads = d.u("n_heads"), n_kv = d.u("n_kv"), q0 = d.u("q0_dim"), q1 = d.u("q1_dim"), vd = d.u("v_dim");
+    const uint32_t capacity = d.u("capacity"), max_len = d.u("max_len", capacity), qk = q0 + q1;
+    if (n_heads == 0 || n_kv == 0 || q0 == 0 || q1 == 0 || vd == 0 || capacity == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / q0_dim / q1_dim / v_dim / capacity parameters missing");
+    const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)qk);
+    SdpaFusion f;
+    f.q0_dim = q0;
+    f.k0_stride = d.u("k0_stride", q0);
+    f.v_stride = d.u("v_stride", vd);
+    f.k1_heads = d.u("k1_n_kv", n_kv);
+    f.traditional = d.u("traditional", 0);
+    f.rope_dims = d.u("rope_dims", 0);
+    f.base_log2 = f.rope_dims ? base_log2_of(d) : 0.f;
+    if (f.k0_stride < q0 || f.v_stride < vd || f.k1_heads == 0) return set_error(FK_ERR_INVALID, d.kernel + ": stride below the row width");
+    FK_TRY(need_bytes(d, 0, (size_t)n_heads * qk * 2));
+    FK_TRY(need_bytes(d, 1, ((size_t)(n_kv - 1) * f.k0_stride + q0) * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)f.k1_heads * q1 * 2));
+    FK_TRY(need_bytes(d, 3, ((size_t)(n_kv - 1) * f.v_stride + vd) * 2));
+    FK_TRY(need_bytes(d, 4, (size_t)n_kv * capacity * qk * 2));
+    FK_TRY(need_bytes(d, 5, (size_t)n_kv * capacity * vd * 2));
+    FK_TRY(need_bytes(d, 6, 4));
+    FK_TRY(need_bytes(d, 7, (size_t)n_heads * vd * 2));
+    size_t pb = 0, cb = 0;
+    FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, qk, vd, max_len, &pb, &cb));
+    FK_TRY(need_bytes(d, 8, pb));
+    FK_TRY(need_bytes(d, 9, cb));
+    f.k_new = arg_ptr<const uint16_t>(d, 1);
+    f.k1_new = arg_ptr<const uint16_t>(d, 2);
+    f.v_new = arg_ptr<const uint16_t>(d, 3);
+    if (table) {
+        FK_TRY(need_bytes(d, 10, (size_t)f.rope_dims * 4));
+        f.rope_tab = arg_ptr<const float>(d, 10);
+    }
+    for (uint32_t i = 0; i < n; ++i)
+        if (i != 7) rw->reads.push_back(i);
+    rw->writes = {4, 5, 7, 8, 9};
+    return plan_sdpa_decode(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 4), arg_ptr<const uint16_t>(d, 5),
+                            arg_ptr<uint16_t>(d, 7), arg_ptr<const uint32_t>(d, 6), 0, max_len, n_heads, n_kv, qk, vd, capacity,
+                            scale, arg_ptr<float>(d, 8), arg_ptr<uint32_t>(d, 9), l, 1, nullptr, &f);
+}
+
 // K, V, [k_weight], keys_packed, keys_scales, keys_biases, values_packed, values_scales, values_biases, offset,
 // write_offset (rope_kv_cache_store_decode_quant.rs:77-98; the capacity is a parameter here)
 fk_status plan_rope_kv_quant(const Dispatch& d, Launch* l, SlotRW* rw, uint32_t bits) {
@@ -898,6 +946,7 @@ const Family kFamilies[] = {
     {"fusekit_sdpa_prefill", plan_sdpa_prefill_d},
     {"fusekit_rmsnorm_rows", plan_rmsnorm_rows_d},
     {"fusekit_rope_store_sdpa_decode", plan_rope_store_sdpa},
+    {"fusekit_split_store_sdpa_decode", plan_split_store_sdpa},
     {"fusekit_rope_kv_cache_store_decode_q4",
      [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_rope_kv_quant(d, l, rw, 4); }},
     {"fusekit_rope_kv_cache_store_decode_q8",

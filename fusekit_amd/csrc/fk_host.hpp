@@ -205,6 +205,10 @@ struct SdpaFusion {
     uint32_t rope_dims = 0;
     float eps = 1e-6f, base_log2 = 0.f;
     const float* rope_tab = nullptr;   // (cos, sin) per pair at this token's position, or null
+    // heads as two parts (q0_dim != 0): q = [Q0 | Q1], new key = [k_new rows k0_stride apart | k1_new], rope_dims
+    // counted from the start of the second part, v_new rows v_stride apart; no head norm
+    const uint16_t* k1_new = nullptr;
+    uint32_t q0_dim = 0, k0_stride = 0, v_stride = 0, k1_heads = 1, traditional = 0;
 };
 uint32_t sdpa_chunk_len(uint32_t qk_dim, uint32_t v_dim, bool fused);
 fk_status sdpa_workspace_bytes(uint32_t n_heads, uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t max_len,

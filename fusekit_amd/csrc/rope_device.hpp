@@ -68,6 +68,33 @@ __device__ __forceinline__ void head_transform(const uint16_t* src, uint16_t* ds
         for (uint32_t d = 2 * half + lane; d < dim; d += kWave) dst[d] = (uint16_t)f32_to_bf16_bits(value(d));
 }
 
+// A head given as two parts: dst = [p0 (d0 dims) | p1 (d1 dims)], the first rope_dims of p1 rotated as
+// traditional (2i, 2i+1) or half-split (i, i + rope_dims / 2) pairs at `pos`; `tab` as in head_transform.
+// The arithmetic of the split-key cache store (mla.hip), for the attention kernel that appends the new
+// row itself.
+__device__ __forceinline__ void split_head_transform(const uint16_t* p0, const uint16_t* p1, uint16_t* dst, uint32_t d0,
+                                                     uint32_t d1, uint32_t rope_dims, bool traditional, uint32_t pos,
+                                                     float base_log2, uint32_t lane, const float* tab) {
+    for (uint32_t d = lane; d < d0; d += kWave) dst[d] = p0[d];
+    const uint32_t half = rope_dims / 2;
+    uint16_t* o = dst + d0;
+    for (uint32_t i = lane; i < half; i += kWave) {
+        const uint32_t lo_i = traditional ? 2 * i : i, hi_i = traditional ? 2 * i + 1 : i + half;
+        const float xl = bf16_bits_to_f32(p1[lo_i]), xh = bf16_bits_to_f32(p1[hi_i]);
+        float lo, hi;
+        if (tab) {
+            const float cs = tab[2 * i], sn = tab[2 * i + 1];
+            lo = xl * cs - xh * sn;
+            hi = xh * cs + xl * sn;
+        } else {
+            rope_rotate(xl, xh, i, half, pos, base_log2, lo, hi);
+        }
+        o[lo_i] = (uint16_t)f32_to_bf16_bits(lo);
+        o[hi_i] = (uint16_t)f32_to_bf16_bits(hi);
+    }
+    for (uint32_t d = 2 * half + lane; d < d1; d += kWave) o[d] = p1[d];
+}
+
 // The same transform for a head that is rotated over its whole width of at most 128 dims, split
 // in two so that a caller can put other memory requests between the loads and their use: lane
 // d < half owns the pair (d, d + half); head_pair_fetch issues every load (raw values, norm weights,

@@ -78,6 +78,14 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
             return set_error(FK_ERR_INVALID, "sdpa: rope_dims must be even and within the head");
         if ((fusion->q_norm == nullptr) != (fusion->k_norm == nullptr))
             return set_error(FK_ERR_INVALID, "sdpa: q and k head norms come together");
+        if (fusion->q0_dim) {
+            if (fusion->q0_dim >= qk_dim || fusion->rope_dims > qk_dim - fusion->q0_dim || !fusion->k1_new || fusion->q_norm)
+                return set_error(FK_ERR_INVALID, "sdpa: split heads need a second part that holds the rotated dims, a k1 row and no head norm");
+            if (fusion->k0_stride < fusion->q0_dim || fusion->v_stride < v_dim || (fusion->k1_heads != 1 && fusion->k1_heads != n_kv))
+                return set_error(FK_ERR_INVALID, "sdpa: split heads: strides below the row widths or a k1 head count other than 1 / n_kv");
+            if ((fusion->v_stride * 2) % 16 || ((uintptr_t)fusion->v_new & 15u))
+                return set_error(FK_ERR_INVALID, "sdpa: new value rows must be 16-byte aligned");
+        }
     }
     if (!kv_len_ptr && rows > 1 && kv_len_imm + rows - 1 > max_len)
         return set_error(FK_ERR_INVALID, "sdpa: the last row's kv length exceeds max_len");
@@ -91,7 +99,7 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     // Rows of different widths (192 / 128) both take the lane count of the wider one -- the spare
     // lanes of the narrower row idle -- as long as a row fits a wave; bf16 caches only.
     const uint32_t lpk0 = pow2_ceil(qk_dim / 8), lpv0 = pow2_ceil(v_dim / 8), lp_wide = lpk0 > lpv0 ? lpk0 : lpv0;
-    const bool same_lanes = lpk0 == lpv0 || (!kvq && !fusion && lp_wide <= (uint32_t)kWave);
+    const bool same_lanes = lpk0 == lpv0 || (!kvq && lp_wide <= (uint32_t)kWave);
     const int gt = !same_lanes ? 8 : (G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1)));
     // Long contexts: a block walks several consecutive ranges (online softmax, the next
     // range's rows in flight), so that the grid stays near one to two blocks per CU and
@@ -130,6 +138,10 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
         a.rope_dims = fusion->rope_dims;
         a.eps = fusion->eps; a.base_log2 = fusion->base_log2;
         a.rope_tab = fusion->rope_tab;
+        a.k1_new = fusion->k1_new;
+        a.q0_dim = fusion->q0_dim; a.k0_stride = fusion->k0_stride; a.k1_heads = fusion->k1_heads;
+        a.traditional = fusion->traditional;
+        a.v_stride = fusion->q0_dim ? fusion->v_stride : v_dim;
     }
     a.lpk = gt <= 4 ? lp_wide : lpk0;
     a.lpv = gt <= 4 ? lp_wide : lpv0;

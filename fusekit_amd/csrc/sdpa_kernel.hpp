@@ -57,6 +57,12 @@ struct SdpaArgs {
     uint32_t rope_dims;
     float eps, base_log2;
     const float* rope_tab;  // (cos, sin) per pair at this token's position, or null
+    // Heads given as two parts (low-rank keys): q0_dim != 0 means q = [Q0 | Q1] with the first rope_dims of
+    // Q1 rotated, the new key row = [k_new row (k0_stride apart) | k1_new (one shared head or one per KV
+    // head)] with the same rotation on its second part, v_new rows v_stride apart (both may point into one
+    // packed projection output); no head norm in this form.
+    const uint16_t* k1_new;
+    uint32_t q0_dim, k0_stride, v_stride, k1_heads, traditional;
 };
 
 // m[GT] at 0, l[GT] at 8 (GT <= 8), the last-block flag at 16, the per-range rescale factors at 24;
@@ -130,7 +136,17 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     auto transform_heads = [&](uint32_t h_first) {
         blk_owner = pos >= blk0 && pos < blk0 + blk_keys;
         for (uint32_t h = h_first + wave; h < gcount + (blk_owner ? 1u : 0u); h += kSdpaWaves) {
-            if (h < gcount) {
+            if (a.q0_dim) {
+                const uint32_t d1 = a.qk_dim - a.q0_dim;
+                if (h < gcount) {
+                    const uint16_t* qh = a.q + (size_t)(h0 + h) * a.qk_dim;
+                    split_head_transform(qh, qh + a.q0_dim, head_dst(h), a.q0_dim, d1, a.rope_dims, a.traditional != 0, pos,
+                                         a.base_log2, lane, a.rope_tab);
+                } else {
+                    split_head_transform(a.k_new + (size_t)kvh * a.k0_stride, a.k1_new + (size_t)(a.k1_heads == 1 ? 0 : kvh) * d1,
+                                         kn, a.q0_dim, d1, a.rope_dims, a.traditional != 0, pos, a.base_log2, lane, a.rope_tab);
+                }
+            } else if (h < gcount) {
                 head_transform(a.q + (size_t)(h0 + h) * a.qk_dim, head_dst(h), a.q_norm, a.qk_dim, a.rope_dims,
                                pos, a.base_log2, a.eps, true, lane, a.rope_tab);
             } else {
@@ -143,7 +159,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             const size_t row = (size_t)kvh * a.capacity + (pos % a.capacity);
             for (uint32_t d = tid; d < a.qk_dim; d += kSdpaBlock) a.cache_k_w[row * a.qk_dim + d] = kn[d];
             for (uint32_t d = tid; d < a.v_dim; d += kSdpaBlock)
-                a.cache_v_w[row * a.v_dim + d] = a.v_new[(size_t)kvh * a.v_dim + d];
+                a.cache_v_w[row * a.v_dim + d] = a.v_new[(size_t)kvh * (MODE == 2 ? a.v_stride : a.v_dim) + d];
         }
     };
     // Whole-token kernel: done before the K/V loads are issued: the trigonometry needs
@@ -311,7 +327,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         }
         request_rows(kc, vc, blk0, 0, false, 0);
         if constexpr (MODE == 2)
-            vnew = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_dim + (vcol_ok ? 8 * cv : 0u));
+            vnew = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_stride + (vcol_ok ? 8 * cv : 0u));
         settle();
         if (split >= n_active) return;  // uniform: whole block leaves before any barrier
         if constexpr (MODE == 2) {

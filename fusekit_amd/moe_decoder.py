@@ -53,6 +53,7 @@ class MoeConfig:
     group: int = 64
     swiglu_variant: int = 1
     capacity: int = 1024
+    fuse_attention: bool = True   # split-key cache store + attention of a layer in one launch
     fuse_shared: bool = True   # the shared experts' gate/up pair as further routes of the routed launch
     fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
 
@@ -195,6 +196,7 @@ class MoeRuntime:
         pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
         self.sdpa_partials, self.sdpa_counters = B(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
+        self.rope_tab = B(c.rope_dim * 4)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
         # the single-launch router holds the hidden row in registers, 512 elements per piece, at most 8
         self.fused_router = bool(c.fuse_router and c.hidden % 512 == 0 and c.hidden <= 4096)
@@ -223,7 +225,11 @@ class MoeRuntime:
             t.append(Dispatch(name("rmsnorm_qkv"), [x, arg(norm_w), w0, w1, w2, s0, s1, s2, b0, b1, b2] + outs,
                               dict(quant, hidden=hidden, n_q=n_q, n_kv=n_kv, eps=c.eps, has_norm=1, has_bias=0)))
 
-        t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
+        if c.fuse_attention:   # step_init also fills this token's (cos, sin) table, shared by all layers
+            t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len), arg(self.rope_tab)],
+                              dict(rope_dims=c.rope_dim, theta=c.theta)))
+        else:
+            t.append(Dispatch("fusekit_step_init", [arg(self.step_counter), arg(self.offset), arg(self.kv_len)]))
         emb = w.mats["embed_tokens"]
         t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token)] + wargs(emb) + [arg(self.x[0])],
                           dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
@@ -242,19 +248,25 @@ class MoeRuntime:
                      (_rows(Wb, 3 * n_b // 4, n_b), n_b // 4)],
                     [arg(self.kvb, n_b, 0), arg(self.kvb, n_b // 2, n_b), arg(self.kvb, n_b // 2, n_b + n_b // 2)])
             packed = c.nope_dim + c.v_dim
-            t.append(Dispatch(name("kv_cache_store_decode"),
-                              [arg(self.q), arg(self.kvb), arg(self.kva, c.rope_dim * 2, c.kv_lora_rank * 2),
-                               arg(self.kvb, self.kvb.nbytes - c.nope_dim * 2, c.nope_dim * 2),
-                               arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.offset), arg(self.offset)],
-                              dict(split_k=1, has_q=1, n_heads=c.n_heads, q0_dim=c.nope_dim, q1_dim=c.rope_dim, n_kv=c.n_heads,
-                                   k0_dim=c.nope_dim, k1_dim=c.rope_dim, v_dim=c.v_dim, k1_n_kv=1, k0_stride=packed,
-                                   v_stride=packed, rope_dims=c.rope_dim, traditional=int(c.rope_traditional), theta=c.theta,
-                                   capacity=c.capacity)))
-            t.append(Dispatch(name("sdpa_decode"),
-                              [arg(self.q), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len), arg(self.att),
-                               arg(self.sdpa_partials), arg(self.sdpa_counters)],
-                              dict(n_heads=c.n_heads, n_kv=c.n_heads, qk_dim=c.qk_dim, head_dim=c.qk_dim, v_dim=c.v_dim,
-                                   capacity=c.capacity, max_len=c.capacity)))
+            split = dict(n_heads=c.n_heads, q0_dim=c.nope_dim, q1_dim=c.rope_dim, n_kv=c.n_heads, v_dim=c.v_dim, k1_n_kv=1,
+                         k0_stride=packed, v_stride=packed, rope_dims=c.rope_dim, traditional=int(c.rope_traditional),
+                         theta=c.theta, capacity=c.capacity)
+            k0, k1 = arg(self.kvb), arg(self.kva, c.rope_dim * 2, c.kv_lora_rank * 2)
+            vv = arg(self.kvb, self.kvb.nbytes - c.nope_dim * 2, c.nope_dim * 2)
+            if c.fuse_attention:   # store + attention in one launch; the rotary table comes from step_init
+                t.append(Dispatch(name("split_store_sdpa_decode"),
+                                  [arg(self.q), k0, k1, vv, arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+                                   arg(self.att), arg(self.sdpa_partials), arg(self.sdpa_counters), arg(self.rope_tab)],
+                                  dict(split, has_table=1, max_len=c.capacity)))
+            else:
+                t.append(Dispatch(name("kv_cache_store_decode"),
+                                  [arg(self.q), k0, k1, vv, arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.offset),
+                                   arg(self.offset)], dict(split, split_k=1, has_q=1, k0_dim=c.nope_dim, k1_dim=c.rope_dim)))
+                t.append(Dispatch(name("sdpa_decode"),
+                                  [arg(self.q), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len), arg(self.att),
+                                   arg(self.sdpa_partials), arg(self.sdpa_counters)],
+                                  dict(n_heads=c.n_heads, n_kv=c.n_heads, qk_dim=c.qk_dim, head_dim=c.qk_dim, v_dim=c.v_dim,
+                                       capacity=c.capacity, max_len=c.capacity)))
             Wo = w.mats[p + "self_attn.o_proj"]
             t.append(Dispatch(name("linear_residual"), [arg(self.att)] + wargs(Wo) + [arg(self.x[0]), arg(self.x[1])],
                               dict(quant, m=Wo.k, n=c.hidden)))

@@ -273,6 +273,18 @@ def kv_cache_store_split_decode(q, n_heads, q0_dim, q1_dim, k0, k0_stride, k1, k
         _ptr(cache_v), _ptr(stream)))
 
 
+def split_store_sdpa_decode(q, n_heads, q0_dim, q1_dim, k0, k0_stride, k1, k1_heads, v, v_stride, n_kv, v_dim, rope_dims,
+                            traditional, theta, rope_tab, cache_k, cache_v, out, d_kv_len, kv_len, max_len, capacity, scale,
+                            partials, counters, stream=None):
+    """Split-key cache store + attention of a layer in one launch (fk_split_store_sdpa_decode)."""
+    check(lib.fk_split_store_sdpa_decode(
+        _ptr(q), C.c_uint32(n_heads), C.c_uint32(q0_dim), C.c_uint32(q1_dim), _ptr(k0), C.c_uint32(k0_stride), _ptr(k1),
+        C.c_uint32(k1_heads), _ptr(v), C.c_uint32(v_stride), C.c_uint32(n_kv), C.c_uint32(v_dim), C.c_uint32(rope_dims),
+        C.c_int(int(traditional)), C.c_float(theta), _ptr(rope_tab), _ptr(cache_k), _ptr(cache_v), _ptr(out), _ptr(d_kv_len),
+        C.c_uint32(kv_len), C.c_uint32(max_len), C.c_uint32(capacity), C.c_float(scale), _ptr(partials), _ptr(counters),
+        _ptr(stream)))
+
+
 def softmax_topk_route(logits, scale, scale_per_route, rows, row_n, top_k, idx, weight, stream=None):
     check(lib.fk_softmax_topk_route(_ptr(logits), _ptr(scale), C.c_int(int(scale_per_route)), C.c_uint32(rows),
                                     C.c_uint32(row_n), C.c_uint32(top_k), _ptr(idx), _ptr(weight), _ptr(stream)))

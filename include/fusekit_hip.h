@@ -321,6 +321,19 @@ fk_status fk_kv_cache_store_split_decode(uint16_t *q, uint32_t n_heads, uint32_t
                                          float theta, const uint32_t *d_offset, uint32_t offset,
                                          const uint32_t *d_write_offset, uint32_t write_offset, uint32_t capacity,
                                          uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
+/* The split-key store and the attention of a layer in ONE launch (one token): what fk_kv_cache_store_split_decode
+ * followed by fk_sdpa_decode computes, bit for bit.  Every block rotates its query heads itself (q is only
+ * read), the block whose range holds the new position assembles [K0 | rope(K1)], uses it and the new V row in
+ * place of the cache row and appends both to the caches.  kv_len counts the new token (its position is
+ * kv_len - 1).  rope_tab (may be NULL): (cos, sin) per rotary pair at that position as fk_step_init_rope fills
+ * it for rope_dims.  Workspace as fk_sdpa_decode (fk_sdpa_workspace_bytes). */
+fk_status fk_split_store_sdpa_decode(const uint16_t *q, uint32_t n_heads, uint32_t q0_dim, uint32_t q1_dim,
+                                     const uint16_t *k0, uint32_t k0_stride, const uint16_t *k1, uint32_t k1_heads,
+                                     const uint16_t *v, uint32_t v_stride, uint32_t n_kv, uint32_t v_dim,
+                                     uint32_t rope_dims, int traditional, float theta, const float *rope_tab,
+                                     uint16_t *cache_k, uint16_t *cache_v, uint16_t *out, const uint32_t *d_kv_len,
+                                     uint32_t kv_len, uint32_t max_len, uint32_t capacity, float scale,
+                                     float *partials, uint32_t *counters, fk_stream s);
 /* fk_softmax_topk_route replaces the router kernel SoftmaxTopKRoute (src/codegen/kernels/single.rs:2615-2760;
  * matcher src/fusion/general.rs:6768-6880): per row softmax over row_n bf16 logits, probabilities rounded
  * to bf16 BEFORE the ordering, the top_k largest in descending order with ties to the lower index;

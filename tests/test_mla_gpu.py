@@ -92,6 +92,46 @@ def test_split_query_attention_close_to_the_fp32_form(fk):
     assert rel_l2(out.to_numpy(np.uint16), oracle.bf16_to_f32(ref)) <= 1e-2
 
 
+@pytest.mark.parametrize("traditional,table", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("n_heads,k0d,k1d,vd,rope,kv_len,cap", [(16, 128, 64, 128, 64, 40, 64), (16, 128, 64, 128, 64, 700, 1024),
+                                                             (4, 64, 32, 64, 16, 1, 16), (2, 128, 64, 128, 64, 64, 64)])
+def test_split_store_and_attention_in_one_launch(fk, n_heads, k0d, k1d, vd, rope, kv_len, cap, traditional, table):
+    """fk_split_store_sdpa_decode == fk_kv_cache_store_split_decode followed by fk_sdpa_decode, bit for bit:
+    output, cache rows, and the query left untouched."""
+    theta, pos = 1e4, kv_len - 1
+    qk = k0d + k1d
+    q = normal_bf16(50, (n_heads, qk))
+    ck, cv = normal_bf16(51, n_heads * cap * qk), normal_bf16(52, n_heads * cap * vd)
+    src, k1 = normal_bf16(53, (n_heads, k0d + vd)), normal_bf16(54, (1, k1d))
+    scale = 1.0 / np.sqrt(qk)
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_heads, qk, vd, cap)
+
+    d_q, d_ck, d_cv, d_src, d_k1 = (_dev(fk, a) for a in (q, ck, cv, src, k1))
+    fk.kv_cache_store_split_decode(d_q, n_heads, k0d, k1d, d_src, k0d + vd, d_k1, 1, _Slice(d_src, k0d), k0d + vd, n_heads, k0d,
+                                   k1d, vd, rope, traditional, theta, None, pos, None, pos, cap, d_ck, d_cv)
+    ref = fk.DeviceBuffer(2 * n_heads * vd)
+    fk.sdpa_decode(d_q, d_ck, d_cv, ref, None, kv_len, cap, n_heads, n_heads, qk, vd, cap, scale, fk.DeviceBuffer(max(pb, 4)),
+                   fk.zeros(max(cb, 4)))
+
+    f_q, f_ck, f_cv = (_dev(fk, a) for a in (q, ck, cv))
+    tab = None
+    if table:
+        tab = fk.DeviceBuffer(4 * rope)
+        fk.step_init_rope(fk.zeros(4), fk.zeros(4), fk.zeros(4), tab, rope, theta)     # position 0 ...
+        cnt = _dev(fk, np.array([pos], np.uint32))
+        fk.step_init_rope(cnt, fk.zeros(4), fk.zeros(4), tab, rope, theta)             # ... then this token's
+    out = fk.DeviceBuffer(2 * n_heads * vd)
+    d_len = _dev(fk, np.array([kv_len], np.uint32))
+    for _ in range(2):   # counters are left zero: a second launch gives the same bits
+        fk.split_store_sdpa_decode(f_q, n_heads, k0d, k1d, d_src, k0d + vd, d_k1, 1, _Slice(d_src, k0d), k0d + vd, n_heads, vd,
+                                   rope, traditional, theta, tab, f_ck, f_cv, out, d_len, 0, cap, cap, scale,
+                                   fk.DeviceBuffer(max(pb, 4)), fk.zeros(max(cb, 4)))
+        assert np.array_equal(out.to_numpy(np.uint16), ref.to_numpy(np.uint16))
+    assert np.array_equal(f_ck.to_numpy(np.uint16), d_ck.to_numpy(np.uint16))
+    assert np.array_equal(f_cv.to_numpy(np.uint16), d_cv.to_numpy(np.uint16))
+    assert np.array_equal(f_q.to_numpy(np.uint16), q.reshape(-1))
+
+
 @pytest.mark.parametrize("rows,row_n,top_k,per_route", [(1, 64, 6, False), (8, 64, 6, True), (3, 256, 32, False),
                                                         (5, 2, 1, False), (2, 128, 8, True)])
 def test_softmax_topk_route(fk, rows, row_n, top_k, per_route):
