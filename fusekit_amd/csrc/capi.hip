@@ -271,7 +271,12 @@ fk_status fk_routed_qmv_swiglu_shared(const uint16_t* x, const fk_weight* Wg, co
 }
 
 size_t fk_routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim) {
-    return ((size_t)n_tokens * top_k + n_tokens) * out_dim * sizeof(uint16_t);
+    return routed_reduce_workspace_bytes(n_tokens, top_k, out_dim, 0, 0);
+}
+
+size_t fk_routed_reduce_workspace_bytes_shared(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim, uint32_t shared_k,
+                                               uint32_t group) {
+    return routed_reduce_workspace_bytes(n_tokens, top_k, out_dim, shared_k, group);
 }
 
 fk_status fk_routed_qmv_reduce(const uint16_t* h, uint32_t n_h_rows, const fk_weight* Wd, uint32_t n_experts,
@@ -398,6 +403,29 @@ fk_status fk_kv_cache_store_split_decode(uint16_t* q, uint32_t n_heads, uint32_t
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_kv_cache_store_split_rows(uint16_t* q, uint32_t n_heads, uint32_t q0_dim, uint32_t q1_dim, const uint16_t* k0,
+                                       uint32_t k0_stride, uint32_t k0_row_stride, const uint16_t* k1, uint32_t k1_heads,
+                                       uint32_t k1_row_stride, const uint16_t* v, uint32_t v_stride, uint32_t v_row_stride,
+                                       uint32_t n_kv, uint32_t k0_dim, uint32_t k1_dim, uint32_t v_dim, uint32_t rope_dims,
+                                       int traditional, float theta, uint32_t rows, uint32_t offset, uint32_t capacity,
+                                       uint16_t* cache_k, uint16_t* cache_v, fk_stream s) {
+    if (rows == 0) return set_error(FK_ERR_INVALID, "fk_kv_cache_store_split_rows: no rows");
+    SplitStoreArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.n_heads = n_heads; a.q0_dim = q0_dim; a.q1_dim = q1_dim;
+    a.k0 = k0; a.k0_stride = k0_stride; a.k1 = k1; a.k1_heads = k1_heads; a.v = v; a.v_stride = v_stride;
+    a.n_kv = n_kv; a.k0_dim = k0_dim; a.k1_dim = k1_dim; a.v_dim = v_dim;
+    a.rope_dims = rope_dims; a.traditional = traditional ? 1u : 0u;
+    a.base_log2 = rope_dims ? theta_log2(theta) : 0.f;
+    a.offset_imm = offset; a.write_offset_imm = offset; a.use_write_imm = 1;
+    a.capacity = capacity;
+    a.cache_k = cache_k; a.cache_v = cache_v;
+    a.rows = rows; a.k0_row_stride = k0_row_stride; a.k1_row_stride = k1_row_stride; a.v_row_stride = v_row_stride;
+    Launch l;
+    FK_TRY(plan_split_rope_store(a, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, int scale_per_route, uint32_t rows,
                                 uint32_t row_n, uint32_t top_k, uint32_t* idx, uint16_t* weight, fk_stream s) {
     Launch l;
@@ -407,9 +435,9 @@ fk_status fk_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, i
 
 fk_status fk_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* w, const uint16_t* scale,
                         uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t* xn, uint16_t* logits, uint32_t* idx,
-                        uint16_t* weight, uint32_t* workspace, fk_stream s) {
+                        uint16_t* weight, uint32_t* workspace, uint32_t rows, fk_stream s) {
     Launch l;
-    FK_TRY(plan_moe_router(x, norm_w, eps, w, scale, hidden, experts, top_k, xn, logits, idx, weight, workspace, &l));
+    FK_TRY(plan_moe_router(x, norm_w, eps, w, scale, hidden, experts, top_k, xn, logits, idx, weight, workspace, &l, rows));
     return run_launch(l, (hipStream_t)s);
 }
 

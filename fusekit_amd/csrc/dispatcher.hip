@@ -395,24 +395,24 @@ fk_status plan_moe_router_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const bool has_norm = d.u("has_norm", 1) != 0;
     const size_t b = has_norm ? 2 : 1;
     FK_TRY(need_args(d, b + 7));
-    const uint32_t hidden = d.u("hidden"), experts = d.u("experts"), top_k = d.u("top_k");
-    if (hidden == 0 || experts == 0 || top_k == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden / experts / top_k parameters missing");
-    FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
+    const uint32_t hidden = d.u("hidden"), experts = d.u("experts"), top_k = d.u("top_k"), rows = d.u("rows", 1);
+    if (hidden == 0 || experts == 0 || top_k == 0 || rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden / experts / top_k parameters missing");
+    FK_TRY(need_bytes(d, 0, (size_t)rows * hidden * 2));
     if (has_norm) FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
     FK_TRY(need_bytes(d, b, (size_t)experts * hidden * 2));
     FK_TRY(need_bytes(d, b + 1, 2));
-    FK_TRY(need_bytes(d, b + 2, (size_t)hidden * 2));
-    FK_TRY(need_bytes(d, b + 3, (size_t)experts * 2));
-    FK_TRY(need_bytes(d, b + 4, (size_t)top_k * 4));
-    FK_TRY(need_bytes(d, b + 5, (size_t)top_k * 2));
-    FK_TRY(need_bytes(d, b + 6, ((size_t)experts + 1) * 4));
+    FK_TRY(need_bytes(d, b + 2, (size_t)rows * hidden * 2));
+    FK_TRY(need_bytes(d, b + 3, (size_t)rows * experts * 2));
+    FK_TRY(need_bytes(d, b + 4, (size_t)rows * top_k * 4));
+    FK_TRY(need_bytes(d, b + 5, (size_t)rows * top_k * 2));
+    FK_TRY(need_bytes(d, b + 6, (size_t)rows * (experts + 1) * 4));
     for (uint32_t i = 0; i < b + 2; ++i) rw->reads.push_back(i);
     rw->reads.push_back((uint32_t)(b + 6));
     for (uint32_t i = b + 2; i < b + 7; ++i) rw->writes.push_back(i);
     return plan_moe_router(arg_ptr<const uint16_t>(d, 0), has_norm ? arg_ptr<const uint16_t>(d, 1) : nullptr,
                            (float)d.param("eps", 1e-6), arg_ptr<const uint16_t>(d, b), arg_ptr<const uint16_t>(d, b + 1), hidden,
                            experts, top_k, arg_ptr<uint16_t>(d, b + 2), arg_ptr<uint16_t>(d, b + 3), arg_ptr<uint32_t>(d, b + 4),
-                           arg_ptr<uint16_t>(d, b + 5), arg_ptr<uint32_t>(d, b + 6), l);
+                           arg_ptr<uint16_t>(d, b + 5), arg_ptr<uint32_t>(d, b + 6), l, rows);
 }
 
 // K, V, [k_weight], cache_k, cache_v, offset, write_offset
@@ -804,7 +804,6 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
     if (experts == 0 || routes == 0 || K == 0 || O == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": k / o / experts / top_k parameters missing");
-    if (has_shared && tokens != 1) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": shared expert needs one token");
     fk_weight Wd, Ws;
     FK_TRY(bind_weight(d, bits, group, O * experts, K, 1, 2, 3, &Wd));
     Wd.n = O;
@@ -818,7 +817,7 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     }
     if (has_extra) FK_TRY(need_bytes(d, extra_slot, (size_t)tokens * O * 2));
     FK_TRY(need_bytes(d, out_slot, (size_t)tokens * O * 2));
-    FK_TRY(need_bytes(d, ws_slot, ((size_t)routes + tokens) * O * 2));
+    FK_TRY(need_bytes(d, ws_slot, routed_reduce_workspace_bytes(tokens, top_k, O, has_shared ? shared_k : 0, group)));
     for (uint32_t i = 0; i < out_slot; ++i) rw->reads.push_back(i);
     rw->reads.push_back((uint32_t)ws_slot);
     rw->writes = {(uint32_t)out_slot, (uint32_t)ws_slot};

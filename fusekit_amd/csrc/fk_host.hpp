@@ -94,6 +94,10 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
                                    const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual,
                                    uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out);
 void set_routed_fused_reduce(bool on);
+// partial rows ((routes + tokens) * O bf16, rounded up to 256 bytes); with a shared expert and several tokens
+// the multi-row matmul's workspace follows them
+size_t routed_parts_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim);
+size_t routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim, uint32_t shared_k, uint32_t group);
 fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight, const uint16_t* residual,
                             uint16_t* out_ptr, uint32_t n_tokens, uint32_t top_k, uint32_t O, bool has_shared,
                             Launch* out);
@@ -157,6 +161,9 @@ struct SplitStoreArgs {
     uint32_t n_kv, k0_dim, k1_dim, v_dim, k0_stride, v_stride, k1_heads;
     uint32_t rope_dims, traditional, capacity;
     float base_log2;
+    // several active token rows (0 = 1): row r is position offset + r; its q row follows the previous one, its
+    // K0 / K1 / V rows start k0_row_stride / k1_row_stride / v_row_stride elements after the previous row's
+    uint32_t rows, k0_row_stride, k1_row_stride, v_row_stride;
 };
 fk_status plan_split_rope_store(const SplitStoreArgs& a, Launch* out);
 fk_status plan_softmax_topk_route(const uint16_t* logits, const uint16_t* scale, bool scale_per_route, uint32_t rows,
@@ -166,7 +173,7 @@ fk_status plan_softmax_topk_route(const uint16_t* logits, const uint16_t* scale,
 // row) and logits are optional outputs; workspace: (experts + 1) words, zero before the first launch.
 fk_status plan_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* w, const uint16_t* scale,
                           uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t* xn, uint16_t* logits, uint32_t* idx,
-                          uint16_t* weight, uint32_t* workspace, Launch* out);
+                          uint16_t* weight, uint32_t* workspace, Launch* out, uint32_t rows = 1);
 
 // Quantised KV cache (mlx-lm QuantizedKVCache layout): packed uint32 [n_kv, capacity, dim*bits/32],
 // scales / biases bf16 [n_kv, capacity, dim/group].

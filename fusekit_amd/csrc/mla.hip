@@ -20,9 +20,10 @@ namespace fk {
 // One wave per head: blocks [0, n_heads) the query heads, then n_kv key heads, then n_kv value heads.
 __global__ __launch_bounds__(kWave) void split_rope_store_kernel(const SplitStoreArgs a) {
     uint32_t b = blockIdx.x;
-    const uint32_t lane = threadIdx.x;
-    const uint32_t pos = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
-    const uint32_t wpos = a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos);
+    const uint32_t lane = threadIdx.x, tr = blockIdx.y;   // tr: active token row (position offset + tr)
+    const uint32_t pos0 = a.offset_ptr ? *a.offset_ptr : a.offset_imm;
+    const uint32_t pos = pos0 + tr;
+    const uint32_t wpos = (a.write_offset_ptr ? *a.write_offset_ptr : (a.use_write_imm ? a.write_offset_imm : pos0)) + tr;
     const uint32_t row = wpos % a.capacity;
     const uint32_t half = a.rope_dims / 2;
 
@@ -36,23 +37,23 @@ __global__ __launch_bounds__(kWave) void split_rope_store_kernel(const SplitStor
         }
     };
     if (b < a.n_heads) {
-        uint16_t* q1 = a.q + (size_t)b * (a.q0_dim + a.q1_dim) + a.q0_dim;
+        uint16_t* q1 = a.q + ((size_t)tr * a.n_heads + b) * (a.q0_dim + a.q1_dim) + a.q0_dim;
         rotate(q1, q1);
         return;
     }
     b -= a.n_heads;
     if (b < a.n_kv) {
         uint16_t* dst = a.cache_k + ((size_t)b * a.capacity + row) * (a.k0_dim + a.k1_dim);
-        const uint16_t* k0 = a.k0 + (size_t)b * a.k0_stride;
+        const uint16_t* k0 = a.k0 + (size_t)tr * a.k0_row_stride + (size_t)b * a.k0_stride;
         for (uint32_t d = lane; d < a.k0_dim; d += kWave) dst[d] = k0[d];
-        const uint16_t* k1 = a.k1 + (size_t)(a.k1_heads == 1 ? 0 : b) * a.k1_dim;
+        const uint16_t* k1 = a.k1 + (size_t)tr * a.k1_row_stride + (size_t)(a.k1_heads == 1 ? 0 : b) * a.k1_dim;
         rotate(k1, dst + a.k0_dim);
         for (uint32_t d = 2 * half + lane; d < a.k1_dim; d += kWave) dst[a.k0_dim + d] = k1[d];
         return;
     }
     b -= a.n_kv;
     uint16_t* dst = a.cache_v + ((size_t)b * a.capacity + row) * a.v_dim;
-    const uint16_t* v = a.v + (size_t)b * a.v_stride;
+    const uint16_t* v = a.v + (size_t)tr * a.v_row_stride + (size_t)b * a.v_stride;
     for (uint32_t d = lane; d < a.v_dim; d += kWave) dst[d] = v[d];
 }
 
@@ -71,7 +72,9 @@ fk_status plan_split_rope_store(const SplitStoreArgs& a, Launch* out) {
     if (a.n_heads && a.q0_dim + a.q1_dim != a.k0_dim + a.k1_dim)
         return set_error(FK_ERR_INVALID, "split store: query and key widths differ");
     out->func = reinterpret_cast<const void*>(&split_rope_store_kernel);
-    out->grid = dim3(a.n_heads + 2 * a.n_kv, 1, 1);
+    if (a.rows > 65535) return set_error(FK_ERR_UNSUPPORTED, "split store: at most 65535 rows per launch");
+    if (a.rows > 1 && a.rows > a.capacity) return set_error(FK_ERR_INVALID, "split store: more rows than cache rows");
+    out->grid = dim3(a.n_heads + 2 * a.n_kv, a.rows ? a.rows : 1, 1);
     out->block = dim3(kWave, 1, 1);
     out->shmem = 0;
     out->set_args(a);
@@ -190,14 +193,16 @@ struct RouterArgs {
     float eps;
 };
 __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
-    const uint32_t e = blockIdx.x, lane = threadIdx.x;
+    const uint32_t e = blockIdx.x, lane = threadIdx.x, tr = blockIdx.y;   // tr: token row
     const uint32_t chunks = a.hidden / (8 * kWave);
+    const uint16_t* xrow = a.x + (size_t)tr * a.hidden;
+    uint32_t* ws = a.workspace + (size_t)tr * (a.experts + 1);
     uint4 wr[kRouterChunks], xr[kRouterChunks], nr[kRouterChunks];
 #pragma unroll
     for (int c = 0; c < kRouterChunks; ++c) {
         const uint32_t o = ((uint32_t)c < chunks ? c * kWave + lane : lane) * 8;   // beyond the row: a harmless repeat
         wr[c] = *reinterpret_cast<const uint4*>(a.w + (size_t)e * a.hidden + o);
-        xr[c] = *reinterpret_cast<const uint4*>(a.x + o);
+        xr[c] = *reinterpret_cast<const uint4*>(xrow + o);
         nr[c] = a.norm_w ? *reinterpret_cast<const uint4*>(a.norm_w + o) : make_uint4(0, 0, 0, 0);
     }
     float xf[kRouterChunks][8];
@@ -242,15 +247,15 @@ __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
             uint4 o;
             o.x = pack_bf16(xf[c][0], xf[c][1]); o.y = pack_bf16(xf[c][2], xf[c][3]);
             o.z = pack_bf16(xf[c][4], xf[c][5]); o.w = pack_bf16(xf[c][6], xf[c][7]);
-            *reinterpret_cast<uint4*>(a.xn + (c * kWave + lane) * 8) = o;
+            *reinterpret_cast<uint4*>(a.xn + (size_t)tr * a.hidden + (c * kWave + lane) * 8) = o;
         }
     }
     acc = round_bf16(wave_sum(acc));
-    uint32_t* counter = a.workspace + a.experts;
+    uint32_t* counter = ws + a.experts;
     uint32_t last = 0;
     if (lane == 0) {
-        __hip_atomic_store(&a.workspace[e], __float_as_uint(acc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (a.logits) a.logits[e] = (uint16_t)(__float_as_uint(acc) >> 16);
+        __hip_atomic_store(&ws[e], __float_as_uint(acc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (a.logits) a.logits[(size_t)tr * a.experts + e] = (uint16_t)(__float_as_uint(acc) >> 16);
         wait_memory_ops_done();
         last = atomicAdd(counter, 1u) == a.experts - 1 ? 1u : 0u;
     }
@@ -264,7 +269,7 @@ __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
         const uint32_t i = lane + j * kWave;
-        x[j] = i < a.experts ? __uint_as_float(__hip_atomic_load(&a.workspace[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+        x[j] = i < a.experts ? __uint_as_float(__hip_atomic_load(&ws[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
                              : -INFINITY;
         m = fmaxf(m, x[j]);
     }
@@ -302,15 +307,15 @@ __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
         for (uint32_t j = 0; j < 4; ++j)
             if (best_i == lane + j * kWave) p[j] = -1.f;
         if (lane == 0) {
-            a.idx[k] = best_i;
-            a.weight[k] = (uint16_t)f32_to_bf16_bits(best * sc);
+            a.idx[(size_t)tr * a.top_k + k] = best_i;
+            a.weight[(size_t)tr * a.top_k + k] = (uint16_t)f32_to_bf16_bits(best * sc);
         }
     }
 }
 
 fk_status plan_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* w, const uint16_t* scale,
                           uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t* xn, uint16_t* logits, uint32_t* idx,
-                          uint16_t* weight, uint32_t* workspace, Launch* out) {
+                          uint16_t* weight, uint32_t* workspace, Launch* out, uint32_t rows) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!x || !w || !scale || !idx || !weight || !workspace) return set_error(FK_ERR_INVALID, "router: null pointer");
@@ -322,7 +327,8 @@ fk_status plan_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, 
         return set_error(FK_ERR_INVALID, "router: activations and weights must be 16-byte aligned");
     RouterArgs a{x, norm_w, w, scale, xn, logits, idx, weight, workspace, hidden, experts, top_k, eps};
     out->func = reinterpret_cast<const void*>(&moe_router_kernel);
-    out->grid = dim3(experts, 1, 1);
+    if (rows == 0 || rows > 65535) return set_error(FK_ERR_INVALID, "router: rows must lie in 1 .. 65535");
+    out->grid = dim3(experts, rows, 1);
     out->block = dim3(kWave, 1, 1);
     out->shmem = 0;
     out->set_args(a);

@@ -419,6 +419,19 @@ fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight,
     return FK_OK;
 }
 
+size_t routed_parts_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim) {
+    return (((size_t)n_tokens * top_k + n_tokens) * out_dim * sizeof(uint16_t) + 255) & ~(size_t)255;
+}
+
+size_t routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim, uint32_t shared_k, uint32_t group) {
+    size_t b = routed_parts_bytes(n_tokens, top_k, out_dim);
+    if (n_tokens > 1 && shared_k) {
+        size_t q = 0;
+        if (qgemm_workspace_bytes(n_tokens, out_dim, shared_k, group ? group : 64, &q) == FK_OK) b += q;
+    }
+    return b;
+}
+
 // The fused form serves one token of int4 weights whose rows fit the lanes of a wave; anything else takes
 // the three launches.
 static bool down_reduce_fits(const fk_weight* Wd, const fk_weight* Ws, uint32_t n_tokens, uint32_t top_k) {
@@ -438,8 +451,8 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
     if (n_tokens == 0 || top_k == 0) return set_error(FK_ERR_INVALID, "routed reduce: empty route set");
     if ((shared_x != nullptr) != (W_shared != nullptr))
         return set_error(FK_ERR_INVALID, "routed reduce: shared_x and W_shared come together");
-    if (W_shared && (n_tokens != 1 || W_shared->n != Wd->n))
-        return set_error(FK_ERR_UNSUPPORTED, "routed reduce: shared expert needs one token and the same output width");
+    if (W_shared && W_shared->n != Wd->n)
+        return set_error(FK_ERR_UNSUPPORTED, "routed reduce: the shared expert must have the routed experts' output width");
     if ((uint64_t)n_tokens * top_k > 65536) return set_error(FK_ERR_UNSUPPORTED, "routed reduce: too many routes");
     const uint32_t n_routes = n_tokens * top_k;
     if (t_routed_fused_reduce && down_reduce_fits(Wd, W_shared, n_tokens, top_k)) {
@@ -472,7 +485,7 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
     }
     if (!parts) return set_error(FK_ERR_INVALID, "routed reduce: workspace required");
     FK_TRY(plan_routed_gemv(h, n_h_rows, Wd, nullptr, n_experts, row_idx, expert_idx, nullptr, n_routes, parts, out));
-    if (W_shared) {
+    if (W_shared && n_tokens == 1) {
         GemvRequest rq;
         rq.mats[0] = W_shared;
         rq.y[0] = parts + (size_t)n_routes * Wd->n;
@@ -480,6 +493,14 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
         Launch shared;
         FK_TRY(plan_gemv(rq, &shared));
         out->then.push_back(shared);
+    } else if (W_shared) {
+        // several tokens: the shared expert's rows through the multi-row matmul, T(dot) per token into the
+        // rows behind the routes'; its own workspace follows the partial rows (routed_reduce_workspace_bytes)
+        unsigned char* qws = reinterpret_cast<unsigned char*>(parts) + routed_parts_bytes(n_tokens, top_k, Wd->n);
+        Launch main, red;
+        FK_TRY(plan_qgemm(W_shared, shared_x, n_tokens, nullptr, nullptr, parts + (size_t)n_routes * Wd->n, qws, &main, &red));
+        out->then.push_back(main);
+        out->then.push_back(red);
     }
     Launch reduce;
     FK_TRY(plan_route_reduce(parts, route_weight, residual, out_ptr, n_tokens, top_k, Wd->n, W_shared != nullptr, &reduce));

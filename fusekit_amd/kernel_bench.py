@@ -270,7 +270,29 @@ def case_moe_decode(d, reps, prompt_len=32, decode=512):
           flush=True)
 
 
+def case_moe_rows(d, reps, rows=8, offset=32):
+    """`rows` active token rows of the MoE benchmark model in one pass over the weights (direct calls)."""
+    import time
+    import numpy as np
+    from .moe_decoder import MoeConfig, MoeRuntime, MoeWeights
+    cfg = MoeConfig(capacity=1024)
+    W = MoeWeights.random_init(cfg, seed=0)
+    rt = MoeRuntime(cfg, W, dispatcher=d)
+    toks = np.random.Generator(np.random.PCG64(0)).integers(0, cfg.vocab, offset + rows).tolist()
+    rt.prefill(toks[:offset])
+    rt.forward_rows(toks[offset:], offset)
+    n = 5
+    t0 = time.perf_counter()
+    for _ in range(n):
+        rt.forward_rows(toks[offset:], offset)
+    sec = (time.perf_counter() - t0) / n
+    print(json.dumps({"case": f"moe_cfg5_rows{rows}_pass_q4", "rows": rows, "ms_per_pass": round(sec * 1e3, 3),
+                      "rows_per_s": round(rows / sec, 1), "note": "host-driven direct calls, wall clock"}), flush=True)
+
+
 CASES = {
+    "moe_cfg5_rows8_pass": lambda d, r: case_moe_rows(d, r, 8),
+    "moe_cfg5_rows64_pass": lambda d, r: case_moe_rows(d, r, 64),
     "moe_cfg5_decode": lambda d, r: case_moe_decode(d, r),
     "qgemv_cfg1": lambda d, r: case_qgemv(d, r, 4864, 896, 4, 512, "cfg1_4864x896"),
     "qgemv_big_q4": lambda d, r: case_qgemv(d, r, 9728, 2560, 4, 48, "9728x2560"),

@@ -337,6 +337,84 @@ class MoeRuntime:
         """bf16 router logits of the last replay, [n_layers, n_experts]."""
         return self.route_logits.to_numpy(np.uint16, (self.cfg.n_layers, self.cfg.n_experts))
 
+    # -- several active token rows (the reference's active_m > 1: multi-token verification, chunked prefill)
+    def forward_rows(self, tokens: Sequence[int], offset: int = 0) -> int:
+        """Processes len(tokens) rows at positions offset .. in ONE pass over the weights (direct calls, no graph):
+        multi-row matmuls for the dense projections, the row forms of the norm, the split-key store, the
+        attention and the router, routed experts over rows x top_k routes, the shared experts through the
+        multi-row matmul.  Fills the KV caches and returns the greedy token after the last row."""
+        c, w = self.cfg, self.w
+        m = len(tokens)
+        if m == 0 or offset + m > c.capacity:
+            raise ValueError("rows must be non-empty and fit the KV-cache capacity")
+        if c.hidden % 512 or c.hidden > 4096:
+            raise ValueError("the row form of the router needs hidden to be a multiple of 512 of at most 4096")
+        B, z = DeviceBuffer, native.zeros
+        n_q, n_a, n_b = c.n_heads * c.qk_dim, c.kv_lora_rank + c.rope_dim, c.n_heads * (c.nope_dim + c.v_dim)
+        toks = DeviceBuffer.from_numpy(np.asarray(tokens, np.uint32))
+        x, x1, xn = B(m * c.hidden * 2), B(m * c.hidden * 2), B(m * c.hidden * 2)
+        q, lat, kpe, latn = B(m * n_q * 2), B(m * c.kv_lora_rank * 2), B(m * c.rope_dim * 2), B(m * c.kv_lora_rank * 2)
+        kvb, att = B(m * n_b * 2), B(m * c.n_heads * c.v_dim * 2)
+        mid = B(m * max(c.dense_inter, c.shared_inter) * 2)
+        routes = m * c.top_k
+        ridx, rwt, rlg = z(4 * routes), z(2 * routes), z(2 * m * c.n_experts)
+        rows_x = DeviceBuffer.from_numpy(np.repeat(np.arange(m, dtype=np.uint32), c.top_k))
+        h = B(routes * c.moe_inter * 2)
+        rws = z(4 * m * (c.n_experts + 1))
+        shapes = [(n_q, c.hidden), (c.kv_lora_rank, c.hidden), (c.rope_dim, c.hidden), (n_b, c.kv_lora_rank),
+                  (c.hidden, c.n_heads * c.v_dim), (c.shared_inter, c.hidden), (c.dense_inter, c.hidden), (c.hidden, c.dense_inter)]
+        qws = B(2 * max(native.qgemm_workspace_bytes(m, n, k, c.group) for n, k in shapes))
+        mws = B(native.routed_reduce_workspace_bytes(m, c.top_k, c.hidden, c.shared_inter, c.group))
+        pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
+        parts, counters = B(max(pb, 4) * m), z(max(cb, 4) * m)
+        packed = c.nope_dim + c.v_dim
+
+        def rows_of(W, r0, r1):   # a view of rows r0 .. r1 of a quantised matrix
+            wb, sb = W.k * W.bits // 8, (W.k // W.group) * 2
+            V = DeviceWeight.__new__(DeviceWeight)
+            V.n, V.k, V.bits, V.group = r1 - r0, W.k, W.bits, W.group
+            V.w, V.scales, V.biases = _View(W.w, r0 * wb, (r1 - r0) * wb), _View(W.scales, r0 * sb, (r1 - r0) * sb), \
+                _View(W.biases, r0 * sb, (r1 - r0) * sb)
+            return V
+
+        native.embed_lookup_rows(w.mats["embed_tokens"], toks, m, 1.0, x)
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            Wa = w.mats[p + "self_attn.kv_a_proj_with_mqa"]
+            native.rmsnorm_rows(x, w.vecs[p + "input_layernorm"], c.eps, m, c.hidden, xn)
+            native.qgemm(w.mats[p + "self_attn.q_proj"], xn, m, None, None, q, qws)
+            native.qgemm(rows_of(Wa, 0, c.kv_lora_rank), xn, m, None, None, lat, qws)
+            native.qgemm(rows_of(Wa, c.kv_lora_rank, n_a), xn, m, None, None, kpe, qws)
+            native.rmsnorm_rows(lat, w.vecs[p + "self_attn.kv_a_layernorm"], c.eps, m, c.kv_lora_rank, latn)
+            native.qgemm(w.mats[p + "self_attn.kv_b_proj"], latn, m, None, None, kvb, qws)
+            native.kv_cache_store_split_rows(q, c.n_heads, c.nope_dim, c.rope_dim, kvb, packed, n_b, kpe, 1, c.rope_dim,
+                                             _View(kvb, c.nope_dim * 2, kvb.nbytes - c.nope_dim * 2), packed, n_b, c.n_heads,
+                                             c.nope_dim, c.rope_dim, c.v_dim, c.rope_dim, c.rope_traditional, c.theta, m, offset,
+                                             c.capacity, self.cache_k[l], self.cache_v[l])
+            native.sdpa_decode_rows(q, self.cache_k[l], self.cache_v[l], att, m, offset + 1, c.n_heads, c.n_heads, c.qk_dim, c.v_dim,
+                                    c.capacity, 1.0 / float(np.sqrt(c.qk_dim)), parts, counters)
+            native.qgemm(w.mats[p + "self_attn.o_proj"], att, m, None, x, x1, qws)
+            post = w.vecs[p + "post_attention_layernorm"]
+            if l < c.first_dense:
+                native.rmsnorm_rows(x1, post, c.eps, m, c.hidden, xn)
+                native.qgemm_swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], xn, m, c.swiglu_variant, mid, qws)
+                native.qgemm(w.mats[p + "mlp.down_proj"], mid, m, None, x1, x, qws)
+                continue
+            native.moe_router(x1, post, c.eps, w.mats[p + "mlp.gate"].w, self.route_scale, c.hidden, c.n_experts, c.top_k, xn, rlg,
+                              ridx, rwt, rws, rows=m)
+            Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
+            native.routed_qmv_swiglu(xn, m, Eg, Eu, c.n_experts, rows_x, ridx, None, routes, h)
+            native.qgemm_swiglu(w.mats[p + "mlp.shared_experts.gate_proj"], w.mats[p + "mlp.shared_experts.up_proj"], xn, m,
+                                c.swiglu_variant, mid, qws)
+            native.routed_qmv_reduce(h, routes, Ed, c.n_experts, None, ridx, rwt, mid, w.mats[p + "mlp.shared_experts.down_proj"],
+                                     x1, m, c.top_k, x, mws)
+        last = _View(x, (m - 1) * c.hidden * 2, c.hidden * 2)
+        native.final_rmsnorm_lm_head(last, w.vecs["final_norm"], c.eps, w.mats["embed_tokens"], self.logits)
+        native.argmax_logits_decode(self.logits, c.vocab, self.token, None, None, 0, self.argmax_ws)
+        native.sync()
+        self.rows_routes = ridx.to_numpy(np.uint32, (m, c.top_k))   # of the last expert layer
+        return int(self.token.to_numpy(np.uint32)[0])
+
     # -- generation (the dense runtime's loop: prompt with forced tokens, then chunks fed back on the GPU)
     def reset(self) -> None:
         for b in (self.step_counter, self.offset, self.kv_len, self.hist_counter):
@@ -360,6 +438,16 @@ class MoeRuntime:
             steps += n
             offset += n
         return out, gpu_s, steps
+
+
+class _View:
+    """`nbytes` bytes at `offset` into a DeviceBuffer, usable wherever the bindings take a buffer."""
+
+    def __init__(self, buf, offset: int, nbytes: int):
+        self.ptr, self.nbytes = buf.ptr + offset, nbytes
+
+    def __int__(self) -> int:
+        return self.ptr
 
 
 def _bf16(a: np.ndarray) -> np.ndarray:

@@ -208,8 +208,13 @@ def routed_qmv_swiglu_shared(x, Wg, Wu, n_experts, expert_idx, route_weight, n_r
 lib.fk_routed_reduce_workspace_bytes.restype = C.c_size_t
 
 
-def routed_reduce_workspace_bytes(n_tokens, top_k, out_dim) -> int:
-    return int(lib.fk_routed_reduce_workspace_bytes(C.c_uint32(n_tokens), C.c_uint32(top_k), C.c_uint32(out_dim)))
+lib.fk_routed_reduce_workspace_bytes_shared.restype = C.c_size_t
+
+
+def routed_reduce_workspace_bytes(n_tokens, top_k, out_dim, shared_k=0, group=64) -> int:
+    """shared_k: input width of a shared expert (several tokens then also need the multi-row matmul's workspace)."""
+    return int(lib.fk_routed_reduce_workspace_bytes_shared(C.c_uint32(n_tokens), C.c_uint32(top_k), C.c_uint32(out_dim),
+                                                           C.c_uint32(shared_k), C.c_uint32(group)))
 
 
 def routed_qmv_reduce(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_weight, shared_x, W_shared,
@@ -290,12 +295,23 @@ def softmax_topk_route(logits, scale, scale_per_route, rows, row_n, top_k, idx, 
                                     C.c_uint32(row_n), C.c_uint32(top_k), _ptr(idx), _ptr(weight), _ptr(stream)))
 
 
-def moe_router(x, norm_w, eps, w, scale, hidden, experts, top_k, xn, logits, idx, weight, workspace, stream=None):
+def moe_router(x, norm_w, eps, w, scale, hidden, experts, top_k, xn, logits, idx, weight, workspace, rows=1, stream=None):
     """RMSNorm + router projection (bf16 weights) + softmax top-k route in one launch (fk_moe_router);
-    workspace: zeros(4 * (experts + 1)), reusable by launches that do not overlap."""
+    workspace: zeros(4 * rows * (experts + 1)), reusable by launches that do not overlap."""
     check(lib.fk_moe_router(_ptr(x), _ptr(norm_w), C.c_float(eps), _ptr(w), _ptr(scale), C.c_uint32(hidden),
                             C.c_uint32(experts), C.c_uint32(top_k), _ptr(xn), _ptr(logits), _ptr(idx), _ptr(weight),
-                            _ptr(workspace), _ptr(stream)))
+                            _ptr(workspace), C.c_uint32(rows), _ptr(stream)))
+
+
+def kv_cache_store_split_rows(q, n_heads, q0_dim, q1_dim, k0, k0_stride, k0_row_stride, k1, k1_heads, k1_row_stride, v, v_stride,
+                              v_row_stride, n_kv, k0_dim, k1_dim, v_dim, rope_dims, traditional, theta, rows, offset, capacity,
+                              cache_k, cache_v, stream=None):
+    check(lib.fk_kv_cache_store_split_rows(
+        _ptr(q), C.c_uint32(n_heads), C.c_uint32(q0_dim), C.c_uint32(q1_dim), _ptr(k0), C.c_uint32(k0_stride),
+        C.c_uint32(k0_row_stride), _ptr(k1), C.c_uint32(k1_heads), C.c_uint32(k1_row_stride), _ptr(v), C.c_uint32(v_stride),
+        C.c_uint32(v_row_stride), C.c_uint32(n_kv), C.c_uint32(k0_dim), C.c_uint32(k1_dim), C.c_uint32(v_dim),
+        C.c_uint32(rope_dims), C.c_int(int(traditional)), C.c_float(theta), C.c_uint32(rows), C.c_uint32(offset),
+        C.c_uint32(capacity), _ptr(cache_k), _ptr(cache_v), _ptr(stream)))
 
 
 def qkv_rope_store_decode(q, k, v, q_norm, k_norm, n_heads, n_kv, head_dim, rope_dims, theta, eps, d_offset,

@@ -177,6 +177,10 @@ fk_status fk_routed_qmv_swiglu_shared(const uint16_t *x, const fk_weight *Wg, co
  *     n_tokens must be 1, as routed_qmv_reduce.rs:80) add the shared expert's down
  *     projection of shared_x.  workspace: fk_routed_reduce_workspace_bytes() bytes. */
 size_t fk_routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim);
+/* With a shared expert and SEVERAL tokens the shared rows go through the multi-row matmul, whose workspace
+ * follows the partial rows: size the buffer with this query (shared_k = the shared expert's input width). */
+size_t fk_routed_reduce_workspace_bytes_shared(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim, uint32_t shared_k,
+                                               uint32_t group);
 fk_status fk_routed_qmv_reduce(const uint16_t *h, uint32_t n_h_rows, const fk_weight *Wd, uint32_t n_experts,
                                const uint32_t *row_idx, const uint32_t *expert_idx, const uint16_t *route_weight,
                                const uint16_t *shared_x, const fk_weight *W_shared, const uint16_t *residual_extra,
@@ -321,6 +325,16 @@ fk_status fk_kv_cache_store_split_decode(uint16_t *q, uint32_t n_heads, uint32_t
                                          float theta, const uint32_t *d_offset, uint32_t offset,
                                          const uint32_t *d_write_offset, uint32_t write_offset, uint32_t capacity,
                                          uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
+/* Row form (several active token rows, row r at position offset + r, as the other _rows entry points): q is
+ * [rows, n_heads, q0_dim + q1_dim]; the K0 / K1 / V rows of token r start k0_row_stride / k1_row_stride /
+ * v_row_stride elements after those of token r - 1 (packed projection outputs [rows, n_kv, k0_dim + v_dim] and
+ * [rows, kv_lora_rank + k1_dim] are addressed without copies). */
+fk_status fk_kv_cache_store_split_rows(uint16_t *q, uint32_t n_heads, uint32_t q0_dim, uint32_t q1_dim, const uint16_t *k0,
+                                       uint32_t k0_stride, uint32_t k0_row_stride, const uint16_t *k1, uint32_t k1_heads,
+                                       uint32_t k1_row_stride, const uint16_t *v, uint32_t v_stride, uint32_t v_row_stride,
+                                       uint32_t n_kv, uint32_t k0_dim, uint32_t k1_dim, uint32_t v_dim, uint32_t rope_dims,
+                                       int traditional, float theta, uint32_t rows, uint32_t offset, uint32_t capacity,
+                                       uint16_t *cache_k, uint16_t *cache_v, fk_stream s);
 /* The split-key store and the attention of a layer in ONE launch (one token): what fk_kv_cache_store_split_decode
  * followed by fk_sdpa_decode computes, bit for bit.  Every block rotates its query heads itself (q is only
  * read), the block whose range holds the new position assembles [K0 | rope(K1)], uses it and the new V row in
@@ -350,11 +364,12 @@ fk_status fk_softmax_topk_route(const uint16_t *logits, const uint16_t *scale, i
  * SoftmaxTopKRoute: src/codegen/kernels/single.rs:2615-2760); the arithmetic here is their composition
  * with the same roundings (normalised row and logits rounded to bf16).  xn [hidden] and logits [experts]
  * are optional outputs (NULL to skip).  hidden a multiple of 512 up to 4096; experts / top_k as above.
- * workspace: (experts + 1) 32-bit words, zero before the first launch, left zeroed by every launch; launches
- * that share it must not overlap. */
+ * rows token rows at once: x / xn [rows, hidden], logits [rows, experts], idx / weight [rows, top_k].
+ * workspace: rows * (experts + 1) 32-bit words, zero before the first launch, left zeroed by every launch;
+ * launches that share it must not overlap. */
 fk_status fk_moe_router(const uint16_t *x, const uint16_t *norm_w, float eps, const uint16_t *w, const uint16_t *scale,
                         uint32_t hidden, uint32_t experts, uint32_t top_k, uint16_t *xn, uint16_t *logits,
-                        uint32_t *idx, uint16_t *weight, uint32_t *workspace, fk_stream s);
+                        uint32_t *idx, uint16_t *weight, uint32_t *workspace, uint32_t rows, fk_stream s);
 
 /* ---- several active token rows (multi-token verification, chunked prefill) ----
  * The reference compiles such variants with active_m > 1 (src/target/mod.rs:170-200,

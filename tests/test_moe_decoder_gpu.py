@@ -103,3 +103,34 @@ def test_full_size_model_32_greedy_tokens(fk):
     rel = np.linalg.norm(g - r) / np.linalg.norm(r)
     print(f"last-step logits rel-L2 {rel:.3e}")
     assert rel <= 5e-2
+
+
+@pytest.mark.parametrize("rows,offset", [(8, 0), (5, 8), (1, 3)])
+def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset):
+    """Several active token rows in one pass over the weights (multi-row matmuls, row forms of the store, the
+    attention and the router, routed experts over rows x top_k routes, shared experts with several tokens)
+    against the oracle stepping through the same tokens one by one: caches, routes, logits, next token."""
+    from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
+    cfg = _small_cfg(hidden=512, n_experts=16, top_k=4)
+    W = MoeWeights.random_init(cfg, seed=6)
+    rt, od = MoeRuntime(cfg, W), OracleMoeDecoder(cfg, W)
+    toks = rng(7).integers(0, cfg.vocab, offset + rows).tolist()
+    routes = []
+    for i, t in enumerate(toks):
+        if i < offset:       # the prefix through the decode graph, so that the caches hold it
+            rt.d.decode_host_loop(rt.graph, rt.uniforms, i, [t])
+        nxt, _, logits = od.step(t, i, want_logits=True)
+        routes.append(od.routes[-1].copy())
+    got = rt.forward_rows(toks[offset:], offset)
+    g = oracle.bf16_to_f32(rt.logits.to_numpy(np.uint16)).astype(np.float64)
+    r = oracle.bf16_to_f32(logits).astype(np.float64)
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+    assert got == nxt
+    same = sum(set(rt.rows_routes[j].tolist()) == set(routes[offset + j].tolist()) for j in range(rows))
+    assert same >= rows - 1, (rt.rows_routes, routes[offset:])
+    last = cfg.n_layers - 1
+    for cache, ref, dim in ((rt.cache_k[last], od.ck[last], cfg.qk_dim), (rt.cache_v[last], od.cv[last], cfg.v_dim)):
+        gk = oracle.bf16_to_f32(cache.to_numpy(np.uint16)).reshape(cfg.n_heads, cfg.capacity, dim)[:, :offset + rows].astype(np.float64)
+        rk = oracle.bf16_to_f32(ref).reshape(cfg.n_heads, cfg.capacity, dim)[:, :offset + rows].astype(np.float64)
+        assert np.linalg.norm(gk - rk) / np.linalg.norm(rk) <= 1e-2
+    assert not cache.to_numpy(np.uint16).reshape(cfg.n_heads, cfg.capacity, dim)[:, offset + rows:].any()   # later rows untouched

@@ -171,6 +171,28 @@ def test_routed_reduce_one_launch_and_three(fk, fused, E, O, K, top_k, SK, with_
     assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
 
 
+def test_routed_reduce_several_tokens_with_a_shared_expert(fk):
+    """tokens > 1 with a shared expert: its rows go through the multi-row matmul, T(dot) per token, and enter
+    the ordered sum after the routes (workspace sized by fk_routed_reduce_workspace_bytes_shared)."""
+    E, O, K, SK, tokens, top_k = 8, 256, 192, 384, 5, 3
+    Wd, Ws = _stack(2600, E, O, K, 4), make_qweight(2700, O, SK, 4)
+    h = normal_bf16(50, (tokens * top_k, K), 0.0, 0.5)
+    expert_idx = rng(51).integers(0, E, tokens * top_k).astype(np.uint32)
+    rw = normal_bf16(52, tokens * top_k, 0.2, 0.3)
+    sx, res = normal_bf16(53, (tokens, SK)), normal_bf16(54, (tokens, O))
+    out = fk.DeviceBuffer(2 * tokens * O)
+    ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, O, SK, 64))
+    fk.routed_qmv_reduce(_dev(fk, h), tokens * top_k, to_device(fk, Wd), E, None, _dev(fk, expert_idx), _dev(fk, rw), _dev(fk, sx),
+                         to_device(fk, Ws), _dev(fk, res), tokens, top_k, out, ws)
+    got = out.to_numpy(np.uint16, (tokens, O))
+    assert rel_l2(got, _m2_fp32(h, Wd, expert_idx, rw, sx, Ws, res, tokens, top_k)) <= REL_L2_BAR
+    ref = np.stack([oracle.routed_qmv_reduce(h[t * top_k:(t + 1) * top_k], Wd, expert_idx[t * top_k:(t + 1) * top_k],
+                                             rw[t * top_k:(t + 1) * top_k], res[t:t + 1], 1, top_k, shared_x=sx[t:t + 1], Wshared=Ws)[0]
+                    for t in range(tokens)])
+    frac, ulps = bf16_mismatch(got, ref)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+
+
 def test_routed_reduce_tokens_and_row_idx(fk):
     E, O, K, tokens, top_k = 4, 192, 256, 3, 2
     Wd = _stack(700, E, O, K, 4)
