@@ -270,6 +270,19 @@ fk_status fk_routed_qmv_swiglu_shared(const uint16_t* x, const fk_weight* Wg, co
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_routed_qmv_swiglu_routing(const uint16_t* x, const fk_weight* Wg, const fk_weight* Wu, uint32_t n_experts,
+                                       const uint16_t* logits, const uint16_t* scale, uint32_t top_k, int apply_weight,
+                                       uint32_t* idx_out, uint16_t* weight_out, uint16_t* out0, const fk_weight* Sg,
+                                       const fk_weight* Su, uint16_t* shared_out, fk_stream s) {
+    if (!Wg || !Wu) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_routing: null weight");
+    if ((Sg != nullptr) != (Su != nullptr)) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_routing: shared gate and up come together");
+    RouteInKernel rk;
+    rk.logits = logits; rk.scale = scale; rk.idx_out = idx_out; rk.weight_out = weight_out; rk.apply_weight = apply_weight != 0;
+    Launch l;
+    FK_TRY(plan_routed_gemv(x, 1, Wg, Wu, n_experts, nullptr, nullptr, nullptr, top_k, out0, &l, Sg, Su, shared_out, &rk));
+    return run_launch(l, (hipStream_t)s);
+}
+
 size_t fk_routed_reduce_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t out_dim) {
     return routed_reduce_workspace_bytes(n_tokens, top_k, out_dim, 0, 0);
 }

@@ -396,16 +396,18 @@ fk_status plan_moe_router_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const size_t b = has_norm ? 2 : 1;
     FK_TRY(need_args(d, b + 7));
     const uint32_t hidden = d.u("hidden"), experts = d.u("experts"), top_k = d.u("top_k"), rows = d.u("rows", 1);
-    if (hidden == 0 || experts == 0 || top_k == 0 || rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden / experts / top_k parameters missing");
+    if (hidden == 0 || experts == 0 || rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden / experts parameters missing");
     FK_TRY(need_bytes(d, 0, (size_t)rows * hidden * 2));
     if (has_norm) FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
     FK_TRY(need_bytes(d, b, (size_t)experts * hidden * 2));
     FK_TRY(need_bytes(d, b + 1, 2));
     FK_TRY(need_bytes(d, b + 2, (size_t)rows * hidden * 2));
     FK_TRY(need_bytes(d, b + 3, (size_t)rows * experts * 2));
-    FK_TRY(need_bytes(d, b + 4, (size_t)rows * top_k * 4));
-    FK_TRY(need_bytes(d, b + 5, (size_t)rows * top_k * 2));
-    FK_TRY(need_bytes(d, b + 6, (size_t)rows * (experts + 1) * 4));
+    if (top_k) {   // top_k = 0: the logits are the output and the last three slots are not touched
+        FK_TRY(need_bytes(d, b + 4, (size_t)rows * top_k * 4));
+        FK_TRY(need_bytes(d, b + 5, (size_t)rows * top_k * 2));
+        FK_TRY(need_bytes(d, b + 6, (size_t)rows * (experts + 1) * 4));
+    }
     for (uint32_t i = 0; i < b + 2; ++i) rw->reads.push_back(i);
     rw->reads.push_back((uint32_t)(b + 6));
     for (uint32_t i = b + 2; i < b + 7; ++i) rw->writes.push_back(i);
@@ -746,7 +748,53 @@ fk_status plan_sdpa_quant_d(const Dispatch& d, Launch* l, SlotRW* rw, uint32_t b
 
 // x, gate_w, gate_s, gate_b, up_w, up_s, up_b, row_idx, expert_idx, [route_weight], out0
 // (routed_qmv_swiglu.rs:99-112).  Parameters: k, o, experts, routes, x_rows, pre_scale.
+// route_in_kernel = 1: x, gate w / s / b, up w / s / b, logits, route_scale, idx_out, weight_out, out0,
+// [shared gate w / s / b, shared up w / s / b, shared_out]; parameters k, o, experts, routes (= top_k), pre_scale,
+// has_shared, shared_o.
+fk_status plan_routed_swiglu_routing(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("k"), O = d.u("o");
+    const uint32_t experts = d.u("experts"), routes = d.u("routes");
+    const bool has_shared = d.u("has_shared", 0) != 0;
+    const size_t n_slots = 12;
+    FK_TRY(need_args(d, n_slots + (has_shared ? 7 : 0)));
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
+    if (experts == 0 || routes == 0 || K == 0 || O == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": k / o / experts / routes parameters missing");
+    fk_weight Wg, Wu, Sg, Su;
+    FK_TRY(bind_weight(d, bits, group, O * experts, K, 1, 2, 3, &Wg));
+    FK_TRY(bind_weight(d, bits, group, O * experts, K, 4, 5, 6, &Wu));
+    Wg.n = Wu.n = O;
+    FK_TRY(need_bytes(d, 0, (size_t)K * 2));
+    FK_TRY(need_bytes(d, 7, (size_t)experts * 2));
+    FK_TRY(need_bytes(d, 8, 2));
+    FK_TRY(need_bytes(d, 9, (size_t)routes * 4));
+    FK_TRY(need_bytes(d, 10, (size_t)routes * 2));
+    FK_TRY(need_bytes(d, 11, (size_t)routes * O * 2));
+    for (uint32_t i = 0; i < 9; ++i) rw->reads.push_back(i);
+    rw->writes = {9, 10, 11};
+    uint16_t* shared_out = nullptr;
+    if (has_shared) {
+        const uint32_t so = d.u("shared_o");
+        if (so == 0) return set_error(FK_ERR_INVALID, d.kernel + ": shared_o parameter missing");
+        FK_TRY(bind_weight(d, bits, group, so, K, n_slots, n_slots + 1, n_slots + 2, &Sg));
+        FK_TRY(bind_weight(d, bits, group, so, K, n_slots + 3, n_slots + 4, n_slots + 5, &Su));
+        FK_TRY(need_bytes(d, n_slots + 6, (size_t)so * 2));
+        shared_out = arg_ptr<uint16_t>(d, n_slots + 6);
+        for (uint32_t i = 0; i < 6; ++i) rw->reads.push_back((uint32_t)n_slots + i);
+        rw->writes.push_back((uint32_t)n_slots + 6);
+    }
+    RouteInKernel rk;
+    rk.logits = arg_ptr<const uint16_t>(d, 7);
+    rk.scale = arg_ptr<const uint16_t>(d, 8);
+    rk.idx_out = arg_ptr<uint32_t>(d, 9);
+    rk.weight_out = arg_ptr<uint16_t>(d, 10);
+    rk.apply_weight = d.u("pre_scale", 0) != 0;
+    return plan_routed_gemv(arg_ptr<const uint16_t>(d, 0), 1, &Wg, &Wu, experts, nullptr, nullptr, nullptr, routes,
+                            arg_ptr<uint16_t>(d, 11), l, has_shared ? &Sg : nullptr, has_shared ? &Su : nullptr, shared_out, &rk);
+}
+
 fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
+    if (d.u("route_in_kernel", 0)) return plan_routed_swiglu_routing(d, l, rw);
     const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("k"), O = d.u("o");
     const uint32_t experts = d.u("experts"), routes = d.u("routes"), x_rows = d.u("x_rows", 1);
     const bool pre_scale = d.u("pre_scale", 0) != 0, has_shared = d.u("has_shared", 0) != 0;

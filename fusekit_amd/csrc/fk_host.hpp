@@ -82,10 +82,20 @@ struct GemvRequest {
 fk_status plan_gemv(const GemvRequest& rq, Launch* out);
 
 // Mixture-of-experts routed projections (w_b non-null: gate/up pair with SwiGLU).
+// Routing inside the routed launch (one token): logits bf16 [n_experts], one bf16 scale; the launch ranks them
+// per wave and writes the chosen experts and weights (bf16 [n_routes]) for the kernels that follow.
+struct RouteInKernel {
+    const uint16_t* logits = nullptr;
+    const uint16_t* scale = nullptr;
+    uint32_t* idx_out = nullptr;
+    uint16_t* weight_out = nullptr;
+    bool apply_weight = false;   // multiply this launch's outputs by the route weight (else a later kernel does)
+};
 fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
                            const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out,
-                           const fk_weight* sh_a = nullptr, const fk_weight* sh_b = nullptr, uint16_t* sh_y = nullptr);
+                           const fk_weight* sh_a = nullptr, const fk_weight* sh_b = nullptr, uint16_t* sh_y = nullptr,
+                           const RouteInKernel* rk = nullptr);
 // Routed down projection + weighted reduction (+ shared expert + residual): one fused launch for one token
 // of int4 weights, else routed GEMV -> shared GEMV -> ordered reduction chained in out->then (`parts`,
 // (routes + tokens) * O bf16, is only touched by the chain).

@@ -4,6 +4,7 @@
 #include "fk_host.hpp"
 #include "fk_device.hpp"
 #include "rope_device.hpp"
+#include "route_device.hpp"
 
 namespace fk {
 
@@ -100,45 +101,16 @@ __global__ __launch_bounds__(kWave) void softmax_topk_route_kernel(const RouteAr
     const uint32_t r = blockIdx.x, lane = threadIdx.x;
     const uint16_t* l = a.logits + (size_t)r * a.row_n;
     float x[4], p[4];
-    float m = -INFINITY;
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
         const uint32_t i = lane + j * kWave;
         x[j] = i < a.row_n ? bf16_bits_to_f32(l[i]) : -INFINITY;
-        m = fmaxf(m, x[j]);
     }
-    m = wave_max(m);
-    float sum = 0.f;
-#pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) {
-        p[j] = lane + j * kWave < a.row_n ? expf(x[j] - m) : 0.f;
-        sum += p[j];
-    }
-    sum = wave_sum(sum);
-    const float inv = 1.0f / sum;
-#pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) p[j] = lane + j * kWave < a.row_n ? round_bf16(p[j] * inv) : -1.f;  // -1: not a candidate
+    route_probabilities(x, a.row_n, lane, p);
     for (uint32_t k = 0; k < a.top_k; ++k) {
-        float best = -1.f;
-        uint32_t best_i = 0xffffffffu;
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)   // ascending index within the lane: '>' keeps the lower one on ties
-            if (p[j] > best) {
-                best = p[j];
-                best_i = lane + j * kWave;
-            }
-#pragma unroll
-        for (uint32_t off = 1; off < kWave; off <<= 1) {
-            const float ob = __shfl_xor(best, off, kWave);
-            const uint32_t oi = __shfl_xor(best_i, off, kWave);
-            if (ob > best || (ob == best && oi < best_i)) {
-                best = ob;
-                best_i = oi;
-            }
-        }
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (best_i == lane + j * kWave) p[j] = -1.f;
+        float best;
+        uint32_t best_i;
+        route_take_best(p, lane, best, best_i);
         if (lane == 0) {
             const size_t o = (size_t)r * a.top_k + k;
             const float sc = bf16_bits_to_f32(a.scale[a.scale_per_route ? o : 0]);
@@ -251,6 +223,10 @@ __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
         }
     }
     acc = round_bf16(wave_sum(acc));
+    if (a.top_k == 0) {   // the consumer routes for itself: publish the logit and leave
+        if (lane == 0) a.logits[(size_t)tr * a.experts + e] = (uint16_t)(__float_as_uint(acc) >> 16);
+        return;
+    }
     uint32_t* counter = ws + a.experts;
     uint32_t last = 0;
     if (lane == 0) {
@@ -265,47 +241,17 @@ __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
 
     // softmax top-k over the published logits: the arithmetic of softmax_topk_route_kernel
     float x[4], p[4];
-    float m = -INFINITY;
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
         const uint32_t i = lane + j * kWave;
-        x[j] = i < a.experts ? __uint_as_float(__hip_atomic_load(&ws[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-                             : -INFINITY;
-        m = fmaxf(m, x[j]);
+        x[j] = i < a.experts ? __uint_as_float(__hip_atomic_load(&ws[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) : -INFINITY;
     }
-    m = wave_max(m);
-    float sum = 0.f;
-#pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) {
-        p[j] = lane + j * kWave < a.experts ? expf(x[j] - m) : 0.f;
-        sum += p[j];
-    }
-    sum = wave_sum(sum);
-    const float inv = 1.0f / sum;
-#pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) p[j] = lane + j * kWave < a.experts ? round_bf16(p[j] * inv) : -1.f;
+    route_probabilities(x, a.experts, lane, p);
     const float sc = bf16_bits_to_f32(a.scale[0]);
     for (uint32_t k = 0; k < a.top_k; ++k) {
-        float best = -1.f;
-        uint32_t best_i = 0xffffffffu;
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (p[j] > best) {
-                best = p[j];
-                best_i = lane + j * kWave;
-            }
-#pragma unroll
-        for (uint32_t off = 1; off < kWave; off <<= 1) {
-            const float ob = __shfl_xor(best, off, kWave);
-            const uint32_t oi = __shfl_xor(best_i, off, kWave);
-            if (ob > best || (ob == best && oi < best_i)) {
-                best = ob;
-                best_i = oi;
-            }
-        }
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (best_i == lane + j * kWave) p[j] = -1.f;
+        float best;
+        uint32_t best_i;
+        route_take_best(p, lane, best, best_i);
         if (lane == 0) {
             a.idx[(size_t)tr * a.top_k + k] = best_i;
             a.weight[(size_t)tr * a.top_k + k] = (uint16_t)f32_to_bf16_bits(best * sc);
@@ -318,10 +264,12 @@ fk_status plan_moe_router(const uint16_t* x, const uint16_t* norm_w, float eps, 
                           uint16_t* weight, uint32_t* workspace, Launch* out, uint32_t rows) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
-    if (!x || !w || !scale || !idx || !weight || !workspace) return set_error(FK_ERR_INVALID, "router: null pointer");
+    if (!x || !w) return set_error(FK_ERR_INVALID, "router: null pointer");
+    if (top_k == 0 && !logits) return set_error(FK_ERR_INVALID, "router: without a route the logits are the output");
+    if (top_k != 0 && (!scale || !idx || !weight || !workspace)) return set_error(FK_ERR_INVALID, "router: null pointer");
     if (hidden == 0 || hidden % (8 * kWave) || hidden > (uint32_t)kRouterChunks * 8 * kWave)
         return set_error(FK_ERR_UNSUPPORTED, "router: hidden must be a multiple of 512 of at most 4096");
-    if (experts < 2 || experts > 256 || (experts & (experts - 1)) || top_k == 0 || top_k >= experts || top_k > 32)
+    if (experts < 2 || experts > 256 || (experts & (experts - 1)) || top_k >= experts || top_k > 32)
         return set_error(FK_ERR_UNSUPPORTED, "router: experts must be a power of two of at most 256, top_k below it and at most 32");
     if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)norm_w | (uintptr_t)xn) & 15u)
         return set_error(FK_ERR_INVALID, "router: activations and weights must be 16-byte aligned");

@@ -18,6 +18,7 @@
 
 #include "fk_host.hpp"
 #include "gemv_kernel.hpp"
+#include "route_device.hpp"
 
 namespace fk {
 
@@ -40,6 +41,14 @@ struct RoutedArgs {
     const uint16_t* xbi[2];
     uint16_t* xy;
     uint32_t n_routes, x_routes;
+    // Routing inside this launch (one token): with `logits` (bf16 [n_experts]) every wave ranks them itself --
+    // softmax, probabilities rounded to T, the n_routes largest, ties to the lower index -- and takes the
+    // route-th winner as its expert; the first block of a route writes idx_out / weight_out [n_routes] for the
+    // kernels that follow.  A router kernel then only publishes logits: no cross-block hand-over anywhere.
+    const uint16_t* logits;
+    const uint16_t* route_scale;   // one bf16 value
+    uint32_t* idx_out;
+    uint16_t* weight_out;
 };
 
 // GemvArgs as one route sees it.  n_mats is a compile-time 1 so that every index
@@ -70,10 +79,37 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
     const uint32_t route = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - route * a.blocks_per_route;
     const bool extra = route >= a.n_routes;     // uniform per block
     const uint32_t lookup = extra ? 0u : route;
-    uint32_t e = a.expert_idx[lookup];
-    e = e < a.n_experts ? e : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
-    uint32_t row = a.row_idx ? a.row_idx[lookup] : lookup;
-    row = row < a.n_x_rows ? row : a.n_x_rows - 1;
+    uint32_t e, row;
+    float routed_weight = 1.0f;
+    if (a.logits) {
+        row = 0;
+        e = 0;
+        if (!extra) {
+            const uint32_t lane = threadIdx.x & (kWave - 1);
+            float x[4], p[4];
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                const uint32_t i = lane + j * kWave;
+                x[j] = i < a.n_experts ? bf16_bits_to_f32(a.logits[i]) : -INFINITY;
+            }
+            route_probabilities(x, a.n_experts, lane, p);
+            float best = 0.f;
+            for (uint32_t k = 0; k <= route; ++k) route_take_best(p, lane, best, e);
+            const uint32_t wbits = f32_to_bf16_bits(best * bf16_bits_to_f32(a.route_scale[0]));
+            if (sub == 0 && threadIdx.x == 0) {
+                a.idx_out[route] = e;
+                a.weight_out[route] = (uint16_t)wbits;
+            }
+            e = __builtin_amdgcn_readfirstlane(e);
+            if (a.route_weight) routed_weight = bf16_bits_to_f32(wbits);   // any non-null pointer: apply the weight here
+        }
+    } else {
+        e = a.expert_idx[lookup];
+        e = e < a.n_experts ? e : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
+        row = a.row_idx ? a.row_idx[lookup] : lookup;
+        row = row < a.n_x_rows ? row : a.n_x_rows - 1;
+        if (a.route_weight && !extra) routed_weight = bf16_bits_to_f32(a.route_weight[lookup]);
+    }
     if (extra) {
         e = route - a.n_routes;
         row = 0;
@@ -98,7 +134,7 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
     v.res = nullptr;
     v.res2 = nullptr;
     v.swiglu_variant = 1;
-    v.y_scale = (a.route_weight && !extra) ? bf16_bits_to_f32(a.route_weight[lookup]) : 1.0f;
+    v.y_scale = routed_weight;
 
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
@@ -316,10 +352,17 @@ uint32_t resident_blocks(const void* func, uint32_t lds_bytes, int cus) {
 fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
                            const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out,
-                           const fk_weight* sh_a, const fk_weight* sh_b, uint16_t* sh_y) {
+                           const fk_weight* sh_a, const fk_weight* sh_b, uint16_t* sh_y, const RouteInKernel* rk) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
-    if (!expert_idx) return set_error(FK_ERR_INVALID, "routed: null expert_idx");
+    if (rk) {
+        if (!rk->logits || !rk->scale || !rk->idx_out || !rk->weight_out) return set_error(FK_ERR_INVALID, "routed: null routing tensor");
+        if (n_x_rows != 1) return set_error(FK_ERR_UNSUPPORTED, "routed: the launch routes for one token only");
+        if (n_experts < 2 || n_experts > 256 || (n_experts & (n_experts - 1)) || n_routes >= n_experts || n_routes > 32)
+            return set_error(FK_ERR_UNSUPPORTED, "routed: experts must be a power of two of at most 256, routes below it and at most 32");
+    } else if (!expert_idx) {
+        return set_error(FK_ERR_INVALID, "routed: null expert_idx");
+    }
     uint32_t x_routes = 0;
     if (sh_a) {
         if (!w_b || !sh_b || !sh_y) return set_error(FK_ERR_INVALID, "routed: shared experts come as a gate/up pair with an output");
@@ -379,6 +422,10 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
     a.y_stride = w_a->n;
     a.n_routes = n_routes;
     a.x_routes = x_routes;
+    if (rk) {
+        a.logits = rk->logits; a.route_scale = rk->scale; a.idx_out = rk->idx_out; a.weight_out = rk->weight_out;
+        a.route_weight = rk->apply_weight ? rk->scale : nullptr;
+    }
     if (sh_a) {
         a.xw[0] = static_cast<const uint4*>(sh_a->w); a.xw[1] = static_cast<const uint4*>(sh_b->w);
         a.xsc[0] = sh_a->scales; a.xsc[1] = sh_b->scales;

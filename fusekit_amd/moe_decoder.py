@@ -53,6 +53,7 @@ class MoeConfig:
     group: int = 64
     swiglu_variant: int = 1
     capacity: int = 1024
+    fuse_topk: bool = True        # the expert launch ranks the router logits itself (needs fuse_router and fuse_shared)
     fuse_attention: bool = True   # split-key cache store + attention of a layer in one launch
     fuse_shared: bool = True   # the shared experts' gate/up pair as further routes of the routed launch
     fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
@@ -286,11 +287,13 @@ class MoeRuntime:
             ridx = arg(self.route_idx, 4 * c.top_k, 4 * c.top_k * l)
             rlg = arg(self.route_logits, 2 * c.n_experts, 2 * c.n_experts * l)
             rwt = arg(self.route_weight, 2 * c.top_k, 2 * c.top_k * l)
-            if self.fused_router:   # norm + router projection + top-k route in one single-block launch
+            route_in_consumer = self.fused_router and c.fuse_topk and c.fuse_shared and c.swiglu_variant == 1
+            if self.fused_router:   # norm + router projection (+ top-k route unless the expert launch ranks the logits itself)
                 t.append(Dispatch(name("moe_router"),
                                   [arg(self.x[1]), arg(post), arg(Wr.w), arg(self.route_scale), arg(self.xn), rlg,
                                    ridx, rwt, arg(self.router_ws)],
-                                  dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1)))
+                                  dict(hidden=c.hidden, experts=c.n_experts, top_k=0 if route_in_consumer else c.top_k, eps=c.eps,
+                                       has_norm=1)))
             else:
                 t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(post), arg(self.xn)],
                                   dict(rows=1, hidden=c.hidden, eps=c.eps)))
@@ -304,7 +307,15 @@ class MoeRuntime:
             routed = [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
                       arg(self.rows_x), ridx, arg(self.h)]
             rparams = dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, x_rows=1)
-            if c.fuse_shared and c.swiglu_variant == 1:   # the shared pair as further routes of the routed launch
+            shared_slots = [arg(Sg.w), arg(Sg.scales), arg(Sg.biases), arg(Su.w), arg(Su.scales), arg(Su.biases),
+                            arg(self.mid, c.shared_inter * 2)]
+            if route_in_consumer:   # the expert launch ranks the logits itself and writes the route for the reduction
+                t.append(Dispatch(name("routed_qmv_swiglu"),
+                                  [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
+                                   rlg, arg(self.route_scale), ridx, rwt, arg(self.h)] + shared_slots,
+                                  dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, route_in_kernel=1,
+                                       has_shared=1, shared_o=c.shared_inter)))
+            elif c.fuse_shared and c.swiglu_variant == 1:   # the shared pair as further routes of the routed launch
                 t.append(Dispatch(name("routed_qmv_swiglu"),
                                   routed + [arg(Sg.w), arg(Sg.scales), arg(Sg.biases), arg(Su.w), arg(Su.scales), arg(Su.biases),
                                             arg(self.mid, c.shared_inter * 2)],

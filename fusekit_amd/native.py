@@ -205,6 +205,15 @@ def routed_qmv_swiglu_shared(x, Wg, Wu, n_experts, expert_idx, route_weight, n_r
                                           _ptr(shared_out), _ptr(stream)))
 
 
+def routed_qmv_swiglu_routing(x, Wg, Wu, n_experts, logits, scale, top_k, apply_weight, idx_out, weight_out, out0, Sg=None,
+                              Su=None, shared_out=None, stream=None) -> None:
+    """One token: the routed (+ shared) gate/up launch ranking the router logits itself (fk_routed_qmv_swiglu_routing)."""
+    check(lib.fk_routed_qmv_swiglu_routing(_ptr(x), C.byref(Wg.c), C.byref(Wu.c), C.c_uint32(n_experts), _ptr(logits), _ptr(scale),
+                                           C.c_uint32(top_k), C.c_int(int(apply_weight)), _ptr(idx_out), _ptr(weight_out),
+                                           _ptr(out0), C.byref(Sg.c) if Sg is not None else None,
+                                           C.byref(Su.c) if Su is not None else None, _ptr(shared_out), _ptr(stream)))
+
+
 lib.fk_routed_reduce_workspace_bytes.restype = C.c_size_t
 
 

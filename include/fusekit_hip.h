@@ -167,6 +167,16 @@ fk_status fk_routed_qmv_swiglu_shared(const uint16_t *x, const fk_weight *Wg, co
                                       const uint32_t *expert_idx, const uint16_t *route_weight, uint32_t n_routes,
                                       uint16_t *out0, const fk_weight *Sg, const fk_weight *Su, uint16_t *shared_out,
                                       fk_stream s);
+/* The routed (and optionally shared: Sg / Su / shared_out, or all three NULL) gate/up launch ROUTING FOR ITSELF,
+ * one token: instead of expert indices it takes the router logits (bf16 [n_experts]) and the bf16 scale; every
+ * wave evaluates fk_softmax_topk_route's arithmetic on them and the block of route r serves the r-th winner.
+ * idx_out u32 [top_k] / weight_out bf16 [top_k] are written for the kernels that follow (fk_routed_qmv_reduce);
+ * apply_weight != 0 multiplies this launch's outputs by the route weight as route_weight does above.  With
+ * fk_moe_router(top_k = 0), which then only publishes logits, no kernel of the block waits on another block. */
+fk_status fk_routed_qmv_swiglu_routing(const uint16_t *x, const fk_weight *Wg, const fk_weight *Wu, uint32_t n_experts,
+                                       const uint16_t *logits, const uint16_t *scale, uint32_t top_k, int apply_weight,
+                                       uint32_t *idx_out, uint16_t *weight_out, uint16_t *out0, const fk_weight *Sg,
+                                       const fk_weight *Su, uint16_t *shared_out, fk_stream s);
 
 /* M2  routed down projection + weighted reduction (+ shared expert + residual).
  *     Replaces src/codegen/kernels/routed_qmv_reduce.rs:14-460.  h is [n_h_rows, k]
@@ -364,6 +374,8 @@ fk_status fk_softmax_topk_route(const uint16_t *logits, const uint16_t *scale, i
  * SoftmaxTopKRoute: src/codegen/kernels/single.rs:2615-2760); the arithmetic here is their composition
  * with the same roundings (normalised row and logits rounded to bf16).  xn [hidden] and logits [experts]
  * are optional outputs (NULL to skip).  hidden a multiple of 512 up to 4096; experts / top_k as above.
+ * top_k = 0: no routing here -- the logits (then required) are the output, for a consumer that routes itself
+ * (fk_routed_qmv_swiglu_routing); scale, idx, weight and workspace may then be NULL.
  * rows token rows at once: x / xn [rows, hidden], logits [rows, experts], idx / weight [rows, top_k].
  * workspace: rows * (experts + 1) 32-bit words, zero before the first launch, left zeroed by every launch;
  * launches that share it must not overlap. */

@@ -19,6 +19,7 @@ def _small_cfg(**kw):
 
 
 @pytest.mark.parametrize("bits,traditional,kw", [(4, True, {}), (8, False, {}), (4, True, dict(hidden=512)),
+                                                 (4, True, dict(hidden=512, fuse_topk=False)),
                                                  (4, False, dict(hidden=512, fuse_router=False, fuse_shared=False, fuse_attention=False)),
                                                  (4, True, dict(n_heads=4, nope_dim=64, rope_dim=32, v_dim=64, n_experts=16, top_k=4))])
 def test_greedy_tokens_and_routes_match_oracle(fk, bits, traditional, kw):

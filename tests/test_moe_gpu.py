@@ -101,6 +101,32 @@ def test_routed_swiglu_with_shared_experts_riding_along(fk, bits):
                                     out0, to_device(fk, make_qweight(1, O + 64, K, bits)), to_device(fk, make_qweight(2, O + 64, K, bits)), shared)
 
 
+@pytest.mark.parametrize("apply_weight,shared", [(False, True), (True, False)])
+def test_routed_swiglu_routing_for_itself(fk, apply_weight, shared):
+    """fk_routed_qmv_swiglu_routing: the route written out is the oracle's router on the same logits, and the
+    outputs are the plain routed launch's bits for that route."""
+    E, O, K, top_k = 16, 192, 256, 4
+    Wg, Wu = _stack(2800, E, O, K, 4), _stack(2900, E, O, K, 4)
+    Sg, Su = make_qweight(3000, 2 * O, K, 4), make_qweight(3100, 2 * O, K, 4)
+    x = normal_bf16(60, (1, K))
+    logits = normal_bf16(61, E, 1.5)
+    scale = oracle.f32_to_bf16(np.array([1.5], np.float32))
+    ref_idx, ref_w = oracle.softmax_topk_route(logits, top_k, scale)
+    idx, w = fk.zeros(4 * top_k), fk.zeros(2 * top_k)
+    out0, sh = fk.DeviceBuffer(2 * top_k * O), fk.zeros(2 * 2 * O)
+    fk.routed_qmv_swiglu_routing(_dev(fk, x), to_device(fk, Wg), to_device(fk, Wu), E, _dev(fk, logits), _dev(fk, scale), top_k,
+                                 apply_weight, idx, w, out0, to_device(fk, Sg) if shared else None,
+                                 to_device(fk, Su) if shared else None, sh if shared else None)
+    got_idx, got_w = idx.to_numpy(np.uint32), w.to_numpy(np.uint16)
+    assert np.array_equal(got_idx, ref_idx.reshape(-1)) and np.array_equal(got_w, ref_w.reshape(-1))
+    plain = _run_m1(fk, x, Wg, Wu, np.zeros(top_k, np.uint32), got_idx, got_w if apply_weight else None)
+    assert np.array_equal(out0.to_numpy(np.uint16, (top_k, O)), plain)
+    if shared:
+        ref = oracle.gateup_swiglu(x.reshape(-1), None, 0.0, Sg, Su, 1)
+        frac, ulps = bf16_mismatch(sh.to_numpy(np.uint16), ref)
+        assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0
+
+
 def _run_m2(fk, h, Wd, row_idx, expert_idx, rw, shared_x, Ws, res, tokens, top_k):
     out = fk.DeviceBuffer(2 * tokens * Wd.n)
     ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, Wd.n))
