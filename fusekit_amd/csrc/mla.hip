@@ -100,17 +100,18 @@ struct RouteArgs {
 __global__ __launch_bounds__(kWave) void softmax_topk_route_kernel(const RouteArgs a) {
     const uint32_t r = blockIdx.x, lane = threadIdx.x;
     const uint16_t* l = a.logits + (size_t)r * a.row_n;
-    float x[4], p[4];
+    float x[4];
+    uint32_t p[4];
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
         const uint32_t i = lane + j * kWave;
         x[j] = i < a.row_n ? bf16_bits_to_f32(l[i]) : -INFINITY;
     }
-    route_probabilities(x, a.row_n, lane, p);
+    route_candidates(x, a.row_n, lane, p);
     for (uint32_t k = 0; k < a.top_k; ++k) {
         float best;
         uint32_t best_i;
-        route_take_best(p, lane, best, best_i);
+        route_take_best(p, best, best_i);
         if (lane == 0) {
             const size_t o = (size_t)r * a.top_k + k;
             const float sc = bf16_bits_to_f32(a.scale[a.scale_per_route ? o : 0]);
@@ -240,18 +241,19 @@ __global__ __launch_bounds__(kWave) void moe_router_kernel(const RouterArgs a) {
     if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // softmax top-k over the published logits: the arithmetic of softmax_topk_route_kernel
-    float x[4], p[4];
+    float x[4];
+    uint32_t p[4];
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
         const uint32_t i = lane + j * kWave;
         x[j] = i < a.experts ? __uint_as_float(__hip_atomic_load(&ws[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) : -INFINITY;
     }
-    route_probabilities(x, a.experts, lane, p);
+    route_candidates(x, a.experts, lane, p);
     const float sc = bf16_bits_to_f32(a.scale[0]);
     for (uint32_t k = 0; k < a.top_k; ++k) {
         float best;
         uint32_t best_i;
-        route_take_best(p, lane, best, best_i);
+        route_take_best(p, best, best_i);
         if (lane == 0) {
             a.idx[(size_t)tr * a.top_k + k] = best_i;
             a.weight[(size_t)tr * a.top_k + k] = (uint16_t)f32_to_bf16_bits(best * sc);

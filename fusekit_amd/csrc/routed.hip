@@ -86,15 +86,16 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
         e = 0;
         if (!extra) {
             const uint32_t lane = threadIdx.x & (kWave - 1);
-            float x[4], p[4];
+            float x[4];
+            uint32_t p[4];
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
                 const uint32_t i = lane + j * kWave;
                 x[j] = i < a.n_experts ? bf16_bits_to_f32(a.logits[i]) : -INFINITY;
             }
-            route_probabilities(x, a.n_experts, lane, p);
+            route_candidates(x, a.n_experts, lane, p);
             float best = 0.f;
-            for (uint32_t k = 0; k <= route; ++k) route_take_best(p, lane, best, e);
+            for (uint32_t k = 0; k <= route; ++k) route_take_best(p, best, e);
             const uint32_t wbits = f32_to_bf16_bits(best * bf16_bits_to_f32(a.route_scale[0]));
             if (sub == 0 && threadIdx.x == 0) {
                 a.idx_out[route] = e;
