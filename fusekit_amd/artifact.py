@@ -13,6 +13,7 @@ runtime whose graph replays the same decode.
 """
 from __future__ import annotations
 
+import dataclasses
 import json
 import os
 import re
@@ -37,6 +38,11 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
     def scratch(name: str, buf: DeviceBuffer, dtype: str, zero: bool = False):
         sym[buf.ptr] = dict(role="scratch", role_name=name, dtype=dtype, size_bytes=buf.nbytes, zero=zero)
 
+    if hasattr(rt, "scratch_symbols"):   # a runtime that names its own arena (the mixture-of-experts decoder)
+        for name, (buf, dtype, zero) in rt.scratch_symbols().items():
+            scratch(name, buf, dtype, zero)
+        _parameter_symbols(rt, sym)
+        return sym
     for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws"):
         scratch(name, getattr(rt, name), "uint32", zero=True)
     scratch("x.0", rt.x[0], "bfloat16")
@@ -55,24 +61,32 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
         else:
             scratch(f"cache_k.{l}", rt.cache_k[l], "bfloat16", zero=True)
             scratch(f"cache_v.{l}", rt.cache_v[l], "bfloat16", zero=True)
-    for path, W in rt.w.mats.items():
-        sym[W.w.ptr] = dict(role="external", source_path=path + ".weight", dtype="uint32" if W.bits != 16 else "bfloat16",
-                            shape=[W.n, W.k * W.bits // 32] if W.bits != 16 else [W.n, W.k])
-        if W.bits != 16:
-            sym[W.scales.ptr] = dict(role="external", source_path=path + ".scales", dtype="bfloat16", shape=[W.n, W.k // W.group])
-            sym[W.biases.ptr] = dict(role="external", source_path=path + ".biases", dtype="bfloat16", shape=[W.n, W.k // W.group])
-    for path, v in rt.w.vecs.items():
-        sym[v.ptr] = dict(role="external", source_path=path, dtype="bfloat16", shape=[v.nbytes // 2])
+    _parameter_symbols(rt, sym)
     return sym
 
 
+def _parameter_symbols(rt, sym: Dict[int, dict]) -> None:
+    for path, W in rt.w.mats.items():
+        lead = [W.n_experts] if getattr(W, "n_experts", 0) else []   # expert-stacked tensors [E, n, ...]
+        sym[W.w.ptr] = dict(role="external", source_path=path + ".weight", dtype="uint32" if W.bits != 16 else "bfloat16",
+                            shape=lead + ([W.n, W.k * W.bits // 32] if W.bits != 16 else [W.n, W.k]), size_bytes=W.w.nbytes)
+        if W.bits != 16:
+            sym[W.scales.ptr] = dict(role="external", source_path=path + ".scales", dtype="bfloat16",
+                                     shape=lead + [W.n, W.k // W.group], size_bytes=W.scales.nbytes)
+            sym[W.biases.ptr] = dict(role="external", source_path=path + ".biases", dtype="bfloat16",
+                                     shape=lead + [W.n, W.k // W.group], size_bytes=W.biases.nbytes)
+    for path, v in rt.w.vecs.items():
+        sym[v.ptr] = dict(role="external", source_path=path, dtype="bfloat16", shape=[v.nbytes // 2], size_bytes=v.nbytes)
+
+
 def _resolve(sym: Dict[int, dict], ptr: int):
-    """The symbol a slot points into, and the byte offset inside it (a slot may be a slice of a buffer)."""
+    """The symbol a slot points into, and the byte offset inside it (a slot may be a slice of a buffer:
+    part of an arena, or a block of rows of a parameter)."""
     s = sym.get(ptr)
     if s is not None:
         return s, 0
     for base, cand in sym.items():
-        if cand["role"] == "scratch" and base < ptr < base + cand["size_bytes"]:
+        if base < ptr < base + cand["size_bytes"]:
             return cand, ptr - base
     return None, 0
 
@@ -133,15 +147,13 @@ def _graph_dict(rt: DecoderRuntime, task_list: List[Dispatch], graph_id: int, sy
         decode_pipeline=[t["id"] for t in tasks],
         decode_capabilities=dict(dispatchable=True, reasons=[]),
         uniforms=uniforms,
-        model_config={k: getattr(c, k) for k in ("n_layers", "hidden", "n_heads", "n_kv", "head_dim", "inter", "vocab",
-                                                  "capacity", "bits", "group", "eps", "theta", "qk_norm", "qkv_bias",
-                                                  "fuse_rope_store", "swiglu_variant", "kv_bits", "kv_group", "fuse_attention")})
+        model_config=dict(dataclasses.asdict(c), config_class=type(c).__name__))
 
 
 def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "synthetic", prefill_variants=()) -> None:
     """`prefill_variants`: PrefillVariant objects of this runtime; each is written as
     `variants/prefill_mN/task_graph.json` and listed in the manifest (src/commands/patch.rs:112-150)."""
-    if rt.persistent:
+    if getattr(rt, "persistent", False):
         raise ValueError("write the artifact from a task-graph runtime (persistent=False)")
     os.makedirs(out_dir, exist_ok=True)
     sym = _symbols(rt)
@@ -169,9 +181,10 @@ def write_artifact(rt: DecoderRuntime, out_dir: str, model_name: str = "syntheti
     manifest = dict(
         schema_version=SCHEMA_VERSION, fusekit_version=BACKEND_VERSION,
         compiled_at=time.strftime("%Y-%m-%dT%H:%M:%SZ", time.gmtime()),
-        model=dict(name=model_name, model_type="dense-decoder", hidden_size=c.hidden, num_hidden_layers=c.n_layers,
-                   num_kv_shared_layers=0, num_attention_heads=c.n_heads, num_key_value_heads=c.n_kv,
-                   head_dim=c.head_dim, vocab_size=c.vocab),
+        model=dict(name=model_name, model_type="moe-decoder" if hasattr(c, "n_experts") else "dense-decoder",
+                   hidden_size=c.hidden, num_hidden_layers=c.n_layers, num_kv_shared_layers=0, num_attention_heads=c.n_heads,
+                   num_key_value_heads=getattr(c, "n_kv", c.n_heads), head_dim=getattr(c, "head_dim", None) or c.qk_dim,
+                   vocab_size=c.vocab),
         stats=dict(ops=len(tasks), fusions=len(tasks), tasks=len(tasks),
                    unique_kernels=len({re.sub(r"_f\d+$", "", t["kernel"]) for t in tasks})),
         variants=variants)

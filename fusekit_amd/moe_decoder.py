@@ -149,6 +149,10 @@ class MoeWeights:
                     matrix(p + f"mlp.shared_experts.{nm}", c.shared_inter, c.hidden)
                 matrix(p + "mlp.switch_mlp.down_proj", c.hidden, c.moe_inter, c.n_experts)
                 matrix(p + "mlp.shared_experts.down_proj", c.hidden, c.shared_inter)
+        # two constants the task list binds like parameters: the routing scale (bf16) and the identity map from
+        # a route to its row of expert outputs (uint32 0 .. top_k - 1)
+        self.vecs["mlp.route_scale"] = DeviceBuffer.from_numpy(_bf16(np.array([c.route_scale], np.float32)))
+        self.vecs["mlp.route_rows"] = DeviceBuffer.from_numpy(np.arange(c.top_k, dtype=np.uint32))
         native.sync()
         return self
 
@@ -186,9 +190,9 @@ class MoeRuntime:
         self.route_logits = z(c.n_experts * 2 * c.n_layers)   # one slot per layer, like the routes
         # one slot per layer, so that the routes of a whole step can be read back after it
         self.route_idx, self.route_weight = z(4 * c.top_k * c.n_layers), z(2 * c.top_k * c.n_layers)
-        self.route_scale = DeviceBuffer.from_numpy(_bf16(np.array([c.route_scale], np.float32)))
+        self.route_scale = weights.vecs["mlp.route_scale"]
         self.rows_x = z(4 * c.top_k)                                # every route reads activation row 0
-        self.rows_h = DeviceBuffer.from_numpy(np.arange(c.top_k, dtype=np.uint32))
+        self.rows_h = weights.vecs["mlp.route_rows"]
         self.h = B(c.top_k * c.moe_inter * 2)
         self.moe_ws = B(max(native.routed_reduce_workspace_bytes(1, c.top_k, c.hidden), 4))
         self.logits = B(c.vocab * 2)
@@ -339,6 +343,22 @@ class MoeRuntime:
                           [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history), arg(self.hist_counter)],
                           dict(vocab=c.vocab)))
         return t
+
+    def scratch_symbols(self):
+        """name -> (buffer, dtype, zero-initialised) of every arena buffer, as the artifact describes them."""
+        out = {}
+        for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws",
+                     "route_idx", "rows_x", "router_ws"):
+            out[name] = (getattr(self, name), "uint32", True)
+        out["x.0"], out["x.1"] = (self.x[0], "bfloat16", False), (self.x[1], "bfloat16", False)
+        for name in ("xn", "q", "kva", "kvb", "att", "mid", "h", "logits", "moe_ws"):
+            out[name] = (getattr(self, name), "bfloat16", False)
+        for name in ("route_logits", "route_weight"):
+            out[name] = (getattr(self, name), "bfloat16", True)
+        out["sdpa_partials"], out["rope_tab"] = (self.sdpa_partials, "float32", False), (self.rope_tab, "float32", False)
+        for l in range(self.cfg.n_layers):
+            out[f"cache_k.{l}"], out[f"cache_v.{l}"] = (self.cache_k[l], "bfloat16", True), (self.cache_v[l], "bfloat16", True)
+        return out
 
     def routes(self) -> np.ndarray:
         """Expert indices the last replay chose, [n_layers, top_k] (rows of dense layers stay zero)."""

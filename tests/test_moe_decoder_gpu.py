@@ -135,3 +135,29 @@ def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset):
         rk = oracle.bf16_to_f32(ref).reshape(cfg.n_heads, cfg.capacity, dim)[:, :offset + rows].astype(np.float64)
         assert np.linalg.norm(gk - rk) / np.linalg.norm(rk) <= 1e-2
     assert not cache.to_numpy(np.uint16).reshape(cfg.n_heads, cfg.capacity, dim)[:, offset + rows:].any()   # later rows untouched
+
+
+def test_artifact_round_trip(fk, tmp_path):
+    """task_graph.json / manifest.json written from the MoE runtime (row blocks of parameters carry offset_bytes,
+    expert-stacked tensors their leading dimension) and read back by the consumer that knows only the files
+    and the parameter tree: the same tokens."""
+    import json
+    from fusekit_amd.artifact import ArtifactRuntime, write_artifact
+    from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
+    cfg = _small_cfg(hidden=512)
+    W = MoeWeights.random_init(cfg, seed=9)
+    rt = MoeRuntime(cfg, W)
+    prompt = [3, 77, 1500, 9]
+    want, _, _ = rt.generate(prompt, 12)
+    write_artifact(rt, str(tmp_path), "moe-test")
+    g = json.load(open(tmp_path / "task_graph.json"))
+    man = json.load(open(tmp_path / "manifest.json"))
+    assert man["model"]["model_type"] == "moe-decoder" and g["model_config"]["n_experts"] == cfg.n_experts
+    kinds = {t["kernel"].rsplit("_f", 1)[0] for t in g["tasks"]}
+    assert {"fusekit_moe_router", "fusekit_routed_qmv_swiglu", "fusekit_routed_qmv_reduce", "fusekit_split_store_sdpa_decode"} <= kinds
+    sliced = [b for t in g["tasks"] for b in t["inputs"] if b["role"] == "external" and b.get("offset_bytes")]
+    assert sliced, "the kv_a / kv_b row blocks are slices of their parameters"
+    stacked = [p for p in g["model_params"] if "switch_mlp" in p["path"]]
+    assert stacked and all(p["shape"][0] == cfg.n_experts for p in stacked)
+    art = ArtifactRuntime(str(tmp_path), W)
+    assert art.generate(prompt, 12) == want
