@@ -100,7 +100,13 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     // lanes of the narrower row idle -- as long as a row fits a wave; bf16 caches only.
     const uint32_t lpk0 = pow2_ceil(qk_dim / 8), lpv0 = pow2_ceil(v_dim / 8), lp_wide = lpk0 > lpv0 ? lpk0 : lpv0;
     const bool same_lanes = lpk0 == lpv0 || (!kvq && lp_wide <= (uint32_t)kWave);
-    const int gt = !same_lanes ? 8 : (G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1)));
+    int gt = !same_lanes ? 8 : (G >= 8 ? 8 : (G >= 4 ? (G == 4 ? 4 : 8) : (G >= 2 ? (G == 2 ? 2 : 4) : 1)));
+    // Groups of 2 .. 4 query heads per KV head: smaller tiles mean more blocks with fewer registers each, and the
+    // repeated K / V reads of a KV head's tiles hit the L2.  Measured (32 q / 8 kv heads x 128, cold caches), tiles
+    // of 1 / 2 / 4 heads: 512 positions 7.9 / 8.5 / 9.1 us, 4096 16.5 / 14.6 / 16.0, 32768 53.8 / 42.0 / 41.7;
+    // the 4B decode loop at context 64 .. 576: 568 / 566 / 550 tokens/s.
+    // (a quantised cache keeps its larger tile beyond 2048 positions: int4 at 32768 ran 41.4 us with 4 heads, 44.4 with 2)
+    if (same_lanes && G >= 2 && G <= 4) gt = max_len <= 2048 ? 1 : (kvq ? gt : 2);
     // Long contexts: a block walks several consecutive ranges (online softmax, the next
     // range's rows in flight), so that the grid stays near one to two blocks per CU and
     // the final merge, which costs one memory round trip per 16 partials, stays short.
