@@ -4,8 +4,10 @@
   generate --model DIR --ids 1,2,3 [--max-tokens N] [--capacity C]
                                          greedy decode of an mlx-lm format checkpoint (token ids in,
                                          token ids out; no tokenizer is bundled)
-  export-random --out DIR [--bits 4] [--layers 2] ...
-                                         write a small random-init model in the mlx-lm file layout
+  export-random --out DIR [--bits 4] [--layers 2] [--moe] ...
+                                         write a small random-init model in the mlx-lm file layout (--moe: a
+                                         mixture-of-experts model in the deepseek_v2 layout; generate / patch
+                                         recognise it by config.json's model_type)
   patch --model DIR [--out DIR/.fusekit] [--prefill-m 32,128] [--capacity C]
                                          the reference's `fusekit patch`: write task_graph.json, manifest.json and
                                          variants/prefill_mN/task_graph.json for a checkpoint
@@ -42,6 +44,7 @@ def main() -> int:
     e.add_argument("--inter", type=int, default=512)
     e.add_argument("--vocab", type=int, default=2000)
     e.add_argument("--seed", type=int, default=0)
+    e.add_argument("--moe", action="store_true", help="a small mixture-of-experts model with low-rank keys (deepseek_v2 layout)")
     args = ap.parse_args()
 
     from . import native as fk
@@ -51,6 +54,15 @@ def main() -> int:
                           for f, _ in t._fields_}, indent=1))
         return 0
     from .decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    if args.cmd == "export-random" and args.moe:
+        from .checkpoint import save_moe_checkpoint
+        from .moe_decoder import MoeConfig, MoeWeights
+        mc = MoeConfig(n_layers=max(args.layers, 2), hidden=512, n_heads=args.heads, kv_lora_rank=128, rope_dim=64, nope_dim=128,
+                       v_dim=128, n_experts=8, top_k=2, moe_inter=128, n_shared=1, dense_inter=args.inter, first_dense=1,
+                       vocab=args.vocab, bits=args.bits if args.bits != 16 else 4)
+        save_moe_checkpoint(args.out, mc, MoeWeights.random_init(mc, seed=args.seed))
+        print(f"wrote {args.out}/config.json and model.safetensors (deepseek_v2 layout)")
+        return 0
     if args.cmd == "export-random":
         from .checkpoint import save_mlx_checkpoint
         cfg = DecoderConfig(n_layers=args.layers, hidden=args.hidden, n_heads=args.heads, n_kv=args.kv_heads,
@@ -58,6 +70,26 @@ def main() -> int:
                             swiglu_variant=1)
         save_mlx_checkpoint(args.out, cfg, DecoderWeights.random_init(cfg, seed=args.seed))
         print(f"wrote {args.out}/config.json and model.safetensors")
+        return 0
+    import os
+    model_type = json.load(open(os.path.join(args.model, "config.json"))).get("model_type", "")
+    if model_type.startswith("deepseek"):   # mixture-of-experts decoder with low-rank keys
+        from .artifact import ArtifactRuntime, write_artifact
+        from .checkpoint import load_moe_checkpoint
+        from .moe_decoder import MoeRuntime
+        cfg, w = load_moe_checkpoint(args.model, capacity=args.capacity)
+        if args.cmd == "patch":
+            rt = MoeRuntime(cfg, w)
+            out = args.out or os.path.join(args.model, ".fusekit")
+            write_artifact(rt, out, os.path.basename(os.path.normpath(args.model)))
+            print(json.dumps({"artifact": out, "tasks": len(rt.tasks), "variants": []}))
+            return 0
+        prompt = [int(t) for t in args.ids.split(",") if t.strip()]
+        if args.artifact:
+            print(json.dumps({"tokens": ArtifactRuntime(args.artifact, w).generate(prompt, args.max_tokens)}))
+            return 0
+        toks, gpu_s, steps = MoeRuntime(cfg, w).generate(prompt, args.max_tokens)
+        print(json.dumps({"tokens": toks, "decode_tok_per_s": round(steps / gpu_s, 1) if gpu_s else None}))
         return 0
     from .checkpoint import load_mlx_checkpoint
     cfg, w = load_mlx_checkpoint(args.model, capacity=args.capacity)

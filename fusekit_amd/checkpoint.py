@@ -205,3 +205,131 @@ def save_mlx_checkpoint(model_dir: str, cfg: DecoderConfig, w: DecoderWeights, m
     if cfg.bits != 16:
         conf["quantization"] = dict(group_size=cfg.group, bits=cfg.bits)
     json.dump(conf, open(os.path.join(model_dir, "config.json"), "w"), indent=1)
+
+
+# ---------------------------------------------------------------- mixture-of-experts layout (mlx-lm deepseek_v2)
+#
+# config.json keys as in DeepSeek-V2-Lite checkpoints: kv_lora_rank, qk_rope_head_dim, qk_nope_head_dim, v_head_dim,
+# n_routed_experts, num_experts_per_tok, moe_intermediate_size, n_shared_experts, intermediate_size (dense layers),
+# first_k_dense_replace, routed_scaling_factor; q_lora_rank must be absent / null (direct q_proj).  Expert matrices
+# are the stacked `mlp.switch_mlp.{gate,up,down}_proj` tensors [E, n, k*bits/32] mlx-lm writes; the router
+# `mlp.gate.weight` stays bf16.  The embedding is tied unless `lm_head.*` is present (then it must be bf16 too).
+
+def moe_config_from_json(c: dict, capacity: int = 1024):
+    from .moe_decoder import MoeConfig
+    if c.get("q_lora_rank"):
+        raise ValueError("low-rank query projections (q_lora_rank) are not supported: the model needs a direct q_proj")
+    q = c.get("quantization") or {}
+    return MoeConfig(
+        n_layers=int(c["num_hidden_layers"]), hidden=int(c["hidden_size"]), n_heads=int(c["num_attention_heads"]),
+        kv_lora_rank=int(c["kv_lora_rank"]), rope_dim=int(c["qk_rope_head_dim"]), nope_dim=int(c["qk_nope_head_dim"]),
+        v_dim=int(c["v_head_dim"]), n_experts=int(c["n_routed_experts"]), top_k=int(c["num_experts_per_tok"]),
+        moe_inter=int(c["moe_intermediate_size"]), n_shared=int(c.get("n_shared_experts") or 0),
+        dense_inter=int(c["intermediate_size"]), first_dense=int(c.get("first_k_dense_replace", 0)), vocab=int(c["vocab_size"]),
+        eps=float(c.get("rms_norm_eps", 1e-6)), theta=float(c.get("rope_theta", 1e4)),
+        rope_traditional=bool(c.get("rope_traditional", True)), route_scale=float(c.get("routed_scaling_factor", 1.0)),
+        bits=int(q.get("bits", 16)), group=int(q.get("group_size", 64)), capacity=capacity)
+
+
+def save_moe_checkpoint(model_dir: str, cfg, w) -> None:
+    """Writes a MoeWeights (downloaded from HBM) as config.json + model.safetensors in the mlx-lm deepseek_v2 layout."""
+    os.makedirs(model_dir, exist_ok=True)
+    tensors = []
+    for path, W in w.mats.items():
+        name = "model." + path
+        lead = (W.n_experts,) if getattr(W, "n_experts", 0) else ()
+        if W.bits == 16:
+            tensors.append((name + ".weight", "BF16", lead + (W.n, W.k), W.w.to_numpy(np.uint16)))
+        else:
+            tensors.append((name + ".weight", "U32", lead + (W.n, W.k * W.bits // 32), W.w.to_numpy(np.uint32)))
+            tensors.append((name + ".scales", "BF16", lead + (W.n, W.k // W.group), W.scales.to_numpy(np.uint16)))
+            tensors.append((name + ".biases", "BF16", lead + (W.n, W.k // W.group), W.biases.to_numpy(np.uint16)))
+    for path, v in w.vecs.items():
+        if path.startswith("mlp.route_"):
+            continue   # constants of the task list, rebuilt from the config on load
+        name = "model.norm.weight" if path == "final_norm" else "model." + path + ".weight"
+        tensors.append((name, "BF16", (v.nbytes // 2,), v.to_numpy(np.uint16)))
+    write_safetensors(os.path.join(model_dir, "model.safetensors"), tensors)
+    conf = dict(model_type="deepseek_v2", hidden_size=cfg.hidden, num_hidden_layers=cfg.n_layers, num_attention_heads=cfg.n_heads,
+                num_key_value_heads=cfg.n_heads, kv_lora_rank=cfg.kv_lora_rank, q_lora_rank=None, qk_rope_head_dim=cfg.rope_dim,
+                qk_nope_head_dim=cfg.nope_dim, v_head_dim=cfg.v_dim, n_routed_experts=cfg.n_experts,
+                num_experts_per_tok=cfg.top_k, moe_intermediate_size=cfg.moe_inter, n_shared_experts=cfg.n_shared,
+                intermediate_size=cfg.dense_inter, first_k_dense_replace=cfg.first_dense, vocab_size=cfg.vocab,
+                rms_norm_eps=cfg.eps, rope_theta=cfg.theta, rope_traditional=cfg.rope_traditional,
+                routed_scaling_factor=cfg.route_scale, tie_word_embeddings=True)
+    if cfg.bits != 16:
+        conf["quantization"] = dict(group_size=cfg.group, bits=cfg.bits)
+    json.dump(conf, open(os.path.join(model_dir, "config.json"), "w"), indent=1)
+
+
+def load_moe_checkpoint(model_dir: str, capacity: int = 1024):
+    """config.json (model_type deepseek_v2, no q_lora_rank) and every *.safetensors of `model_dir` into a
+    (MoeConfig, MoeWeights) pair in HBM; shapes are checked against the config tensor by tensor."""
+    from .moe_decoder import MoeWeights, _bf16
+    cfg = moe_config_from_json(json.load(open(os.path.join(model_dir, "config.json"))), capacity)
+    if cfg.bits == 16:
+        raise ValueError("the mixture-of-experts decoder takes 4- or 8-bit projections (config.json has no quantization block)")
+    files = [SafetensorsFile(os.path.join(model_dir, f)) for f in sorted(os.listdir(model_dir)) if f.endswith(".safetensors")]
+    if not files:
+        raise FileNotFoundError(f"no .safetensors file in {model_dir}")
+    where = {name: f for f in files for name in f.tensors}
+
+    def upload(name: str, want_dtype: str, want_shape) -> DeviceBuffer:
+        if name not in where:
+            raise KeyError(f"checkpoint has no tensor {name}")
+        data, dtype, shape = where[name].raw(name)
+        if dtype != want_dtype:
+            raise ValueError(f"{name}: dtype {dtype}, this backend needs {want_dtype}")
+        if tuple(shape) != tuple(want_shape):
+            raise ValueError(f"{name}: shape {tuple(shape)}, expected {tuple(want_shape)}")
+        return DeviceBuffer.from_numpy(data)
+
+    c, w = cfg, MoeWeights(cfg)
+
+    def matrix(path: str, n: int, k: int, experts: int = 0, dense: bool = False):
+        W = DeviceWeight.__new__(DeviceWeight)
+        W.n, W.k = n, k
+        lead = (experts,) if experts else ()
+        if dense:
+            W.bits, W.group, W.scales, W.biases = 16, 0, None, None
+            W.w = upload("model." + path + ".weight", "BF16", lead + (n, k))
+        else:
+            W.bits, W.group = c.bits, c.group
+            W.w = upload("model." + path + ".weight", "U32", lead + (n, k * c.bits // 32))
+            W.scales = upload("model." + path + ".scales", "BF16", lead + (n, k // c.group))
+            W.biases = upload("model." + path + ".biases", "BF16", lead + (n, k // c.group))
+        if experts:
+            W.n_experts = experts
+        w.mats[path] = W
+
+    def vector(path: str, n: int, name: str = None):
+        w.vecs[path] = upload(name or "model." + path + ".weight", "BF16", (n,))
+
+    matrix("embed_tokens", c.vocab, c.hidden, dense=True)
+    vector("final_norm", c.hidden, "model.norm.weight")
+    for l in range(c.n_layers):
+        p = f"layers.{l}."
+        vector(p + "input_layernorm", c.hidden)
+        vector(p + "post_attention_layernorm", c.hidden)
+        matrix(p + "self_attn.q_proj", c.n_heads * c.qk_dim, c.hidden)
+        matrix(p + "self_attn.kv_a_proj_with_mqa", c.kv_lora_rank + c.rope_dim, c.hidden)
+        vector(p + "self_attn.kv_a_layernorm", c.kv_lora_rank)
+        matrix(p + "self_attn.kv_b_proj", c.n_heads * (c.nope_dim + c.v_dim), c.kv_lora_rank)
+        matrix(p + "self_attn.o_proj", c.hidden, c.n_heads * c.v_dim)
+        if l < c.first_dense:
+            matrix(p + "mlp.gate_proj", c.dense_inter, c.hidden)
+            matrix(p + "mlp.up_proj", c.dense_inter, c.hidden)
+            matrix(p + "mlp.down_proj", c.hidden, c.dense_inter)
+        else:
+            matrix(p + "mlp.gate", c.n_experts, c.hidden, dense=True)
+            for nm in ("gate_proj", "up_proj"):
+                matrix(p + f"mlp.switch_mlp.{nm}", c.moe_inter, c.hidden, c.n_experts)
+                matrix(p + f"mlp.shared_experts.{nm}", c.shared_inter, c.hidden)
+            matrix(p + "mlp.switch_mlp.down_proj", c.hidden, c.moe_inter, c.n_experts)
+            matrix(p + "mlp.shared_experts.down_proj", c.hidden, c.shared_inter)
+    w.vecs["mlp.route_scale"] = DeviceBuffer.from_numpy(_bf16(np.array([c.route_scale], np.float32)))
+    w.vecs["mlp.route_rows"] = DeviceBuffer.from_numpy(np.arange(c.top_k, dtype=np.uint32))
+    for f in files:
+        f.close()
+    native.sync()
+    return cfg, w

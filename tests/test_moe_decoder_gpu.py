@@ -161,3 +161,31 @@ def test_artifact_round_trip(fk, tmp_path):
     assert stacked and all(p["shape"][0] == cfg.n_experts for p in stacked)
     art = ArtifactRuntime(str(tmp_path), W)
     assert art.generate(prompt, 12) == want
+
+
+def test_checkpoint_round_trip(fk, tmp_path):
+    """A MoE model written in the mlx-lm deepseek_v2 file layout (stacked expert tensors, bf16 router) and read
+    back tensor by tensor: same config, same bytes, same tokens; a wrong shape is refused by name."""
+    import json
+    from fusekit_amd.checkpoint import SafetensorsFile, load_moe_checkpoint, save_moe_checkpoint
+    from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
+    cfg = _small_cfg(hidden=512, route_scale=1.5)
+    W = MoeWeights.random_init(cfg, seed=10)
+    want, _, _ = MoeRuntime(cfg, W).generate([5, 6, 7], 10)
+    save_moe_checkpoint(str(tmp_path), cfg, W)
+    conf = json.load(open(tmp_path / "config.json"))
+    assert conf["model_type"] == "deepseek_v2" and conf["n_routed_experts"] == cfg.n_experts and conf["quantization"]["bits"] == 4
+    st = SafetensorsFile(str(tmp_path / "model.safetensors"))
+    _, dtype, shape = st.raw("model.layers.1.mlp.switch_mlp.gate_proj.weight")
+    assert dtype == "U32" and tuple(shape) == (cfg.n_experts, cfg.moe_inter, cfg.hidden * 4 // 32)
+    st.close()
+    cfg2, W2 = load_moe_checkpoint(str(tmp_path), capacity=cfg.capacity)
+    assert cfg2 == cfg
+    for k in W.mats:
+        assert np.array_equal(W.mats[k].w.to_numpy(np.uint8), W2.mats[k].w.to_numpy(np.uint8)), k
+    got, _, _ = MoeRuntime(cfg2, W2).generate([5, 6, 7], 10)
+    assert got == want
+    conf["moe_intermediate_size"] = cfg.moe_inter * 2
+    json.dump(conf, open(tmp_path / "config.json", "w"))
+    with pytest.raises(ValueError, match="switch_mlp"):
+        load_moe_checkpoint(str(tmp_path))
