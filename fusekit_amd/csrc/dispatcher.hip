@@ -342,17 +342,24 @@ fk_status plan_kv_store_split(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (a.n_kv == 0 || a.k0_dim == 0 || a.k1_dim == 0 || a.v_dim == 0 || a.capacity == 0 || a.k1_heads == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": n_kv / k0_dim / k1_dim / v_dim / capacity parameters missing");
     if (a.k0_stride < a.k0_dim || a.v_stride < a.v_dim) return set_error(FK_ERR_INVALID, d.kernel + ": stride below the row width");
+    // rows > 1 (row r at position offset + r): token rows k0_row_stride / k1_row_stride / v_row_stride elements apart
+    a.rows = d.u("rows", 1);
+    a.k0_row_stride = d.u("k0_row_stride", a.n_kv * a.k0_stride);
+    a.k1_row_stride = d.u("k1_row_stride", a.k1_heads * a.k1_dim);
+    a.v_row_stride = d.u("v_row_stride", a.n_kv * a.v_stride);
+    if (a.rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows must be positive");
+    const size_t more = a.rows - 1;
     if (has_q) {
         a.n_heads = d.u("n_heads");
         a.q0_dim = d.u("q0_dim");
         a.q1_dim = d.u("q1_dim");
         if (a.n_heads == 0) return set_error(FK_ERR_INVALID, d.kernel + ": n_heads parameter missing");
-        FK_TRY(need_bytes(d, 0, (size_t)a.n_heads * (a.q0_dim + a.q1_dim) * 2));
+        FK_TRY(need_bytes(d, 0, (size_t)a.rows * a.n_heads * (a.q0_dim + a.q1_dim) * 2));
         a.q = arg_ptr<uint16_t>(d, 0);
     }
-    FK_TRY(need_bytes(d, b, ((size_t)(a.n_kv - 1) * a.k0_stride + a.k0_dim) * 2));
-    FK_TRY(need_bytes(d, b + 1, (size_t)a.k1_heads * a.k1_dim * 2));
-    FK_TRY(need_bytes(d, b + 2, ((size_t)(a.n_kv - 1) * a.v_stride + a.v_dim) * 2));
+    FK_TRY(need_bytes(d, b, (more * a.k0_row_stride + (size_t)(a.n_kv - 1) * a.k0_stride + a.k0_dim) * 2));
+    FK_TRY(need_bytes(d, b + 1, (more * a.k1_row_stride + (size_t)a.k1_heads * a.k1_dim) * 2));
+    FK_TRY(need_bytes(d, b + 2, (more * a.v_row_stride + (size_t)(a.n_kv - 1) * a.v_stride + a.v_dim) * 2));
     FK_TRY(need_bytes(d, b + 3, (size_t)a.n_kv * a.capacity * (a.k0_dim + a.k1_dim) * 2));
     FK_TRY(need_bytes(d, b + 4, (size_t)a.n_kv * a.capacity * a.v_dim * 2));
     FK_TRY(need_bytes(d, b + 5, 4));
@@ -506,20 +513,23 @@ fk_status plan_sdpa_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (n_heads == 0 || n_kv == 0 || qk == 0 || capacity == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": n_heads / n_kv / head_dim / capacity parameters missing");
     const float scale = d.has("scale") ? (float)d.param("scale", 0) : 1.0f / sqrtf((float)qk);  // sdpa_decode.rs:248-252
-    FK_TRY(need_bytes(d, 0, (size_t)n_heads * qk * 2));
+    // rows > 1: row r of q / out attends to kv_len + r positions (kv_len is row 0's); workspace per row
+    const uint32_t rows = d.u("rows", 1);
+    if (rows == 0) return set_error(FK_ERR_INVALID, d.kernel + ": rows must be positive");
+    FK_TRY(need_bytes(d, 0, (size_t)rows * n_heads * qk * 2));
     FK_TRY(need_bytes(d, 1, (size_t)n_kv * capacity * qk * 2));
     FK_TRY(need_bytes(d, 2, (size_t)n_kv * capacity * vd * 2));
     FK_TRY(need_bytes(d, 3, 4));
-    FK_TRY(need_bytes(d, 4, (size_t)n_heads * vd * 2));
+    FK_TRY(need_bytes(d, 4, (size_t)rows * n_heads * vd * 2));
     size_t pb = 0, cb = 0;
     FK_TRY(sdpa_workspace_bytes(n_heads, n_kv, qk, vd, max_len, &pb, &cb));
-    FK_TRY(need_bytes(d, 5, pb));
-    FK_TRY(need_bytes(d, 6, cb));
+    FK_TRY(need_bytes(d, 5, pb * rows));
+    FK_TRY(need_bytes(d, 6, cb * rows));
     rw->reads = {0, 1, 2, 3, 5, 6};
     rw->writes = {4, 5, 6};
     return plan_sdpa_decode(arg_ptr<const uint16_t>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<const uint16_t>(d, 2),
                             arg_ptr<uint16_t>(d, 4), arg_ptr<const uint32_t>(d, 3), 0, max_len, n_heads, n_kv, qk, vd,
-                            capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l);
+                            capacity, scale, arg_ptr<float>(d, 5), arg_ptr<uint32_t>(d, 6), l, rows);
 }
 
 // Q, K, V, out: causal attention of `rows` token rows (sdpa_prefill.rs:11-21).  The reference binds

@@ -287,7 +287,7 @@ def case_moe_rows(d, reps, rows=8, offset=32):
         rt.forward_rows(toks[offset:], offset)
     sec = (time.perf_counter() - t0) / n
     print(json.dumps({"case": f"moe_cfg5_rows{rows}_pass_q4", "rows": rows, "ms_per_pass": round(sec * 1e3, 3),
-                      "rows_per_s": round(rows / sec, 1), "note": "host-driven direct calls, wall clock"}), flush=True)
+                      "rows_per_s": round(rows / sec, 1), "note": "one graph replay per pass, wall clock"}), flush=True)
 
 
 CASES = {

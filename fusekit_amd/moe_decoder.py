@@ -206,6 +206,7 @@ class MoeRuntime:
         # the single-launch router holds the hidden row in registers, 512 elements per piece, at most 8
         self.fused_router = bool(c.fuse_router and c.hidden % 512 == 0 and c.hidden <= 4096)
         self.router_ws = z(4 * (c.n_experts + 1))
+        self._rows_variants: Dict[int, "MoeRowsVariant"] = {}
         self.tasks = self.build_tasks()
         self.graph = self.d.build_graph(self.tasks)
 
@@ -370,81 +371,16 @@ class MoeRuntime:
 
     # -- several active token rows (the reference's active_m > 1: multi-token verification, chunked prefill)
     def forward_rows(self, tokens: Sequence[int], offset: int = 0) -> int:
-        """Processes len(tokens) rows at positions offset .. in ONE pass over the weights (direct calls, no graph):
-        multi-row matmuls for the dense projections, the row forms of the norm, the split-key store, the
-        attention and the router, routed experts over rows x top_k routes, the shared experts through the
-        multi-row matmul.  Fills the KV caches and returns the greedy token after the last row."""
-        c, w = self.cfg, self.w
+        """Processes len(tokens) rows at positions offset .. in ONE pass over the weights: the replay of a
+        `MoeRowsVariant` graph for that row count (built on first use).  Fills the KV caches and returns the
+        greedy token after the last row."""
         m = len(tokens)
-        if m == 0 or offset + m > c.capacity:
-            raise ValueError("rows must be non-empty and fit the KV-cache capacity")
-        if c.hidden % 512 or c.hidden > 4096:
-            raise ValueError("the row form of the router needs hidden to be a multiple of 512 of at most 4096")
-        B, z = DeviceBuffer, native.zeros
-        n_q, n_a, n_b = c.n_heads * c.qk_dim, c.kv_lora_rank + c.rope_dim, c.n_heads * (c.nope_dim + c.v_dim)
-        toks = DeviceBuffer.from_numpy(np.asarray(tokens, np.uint32))
-        x, x1, xn = B(m * c.hidden * 2), B(m * c.hidden * 2), B(m * c.hidden * 2)
-        q, lat, kpe, latn = B(m * n_q * 2), B(m * c.kv_lora_rank * 2), B(m * c.rope_dim * 2), B(m * c.kv_lora_rank * 2)
-        kvb, att = B(m * n_b * 2), B(m * c.n_heads * c.v_dim * 2)
-        mid = B(m * max(c.dense_inter, c.shared_inter) * 2)
-        routes = m * c.top_k
-        ridx, rwt, rlg = z(4 * routes), z(2 * routes), z(2 * m * c.n_experts)
-        rows_x = DeviceBuffer.from_numpy(np.repeat(np.arange(m, dtype=np.uint32), c.top_k))
-        h = B(routes * c.moe_inter * 2)
-        rws = z(4 * m * (c.n_experts + 1))
-        shapes = [(n_q, c.hidden), (c.kv_lora_rank, c.hidden), (c.rope_dim, c.hidden), (n_b, c.kv_lora_rank),
-                  (c.hidden, c.n_heads * c.v_dim), (c.shared_inter, c.hidden), (c.dense_inter, c.hidden), (c.hidden, c.dense_inter)]
-        qws = B(2 * max(native.qgemm_workspace_bytes(m, n, k, c.group) for n, k in shapes))
-        mws = B(native.routed_reduce_workspace_bytes(m, c.top_k, c.hidden, c.shared_inter, c.group))
-        pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
-        parts, counters = B(max(pb, 4) * m), z(max(cb, 4) * m)
-        packed = c.nope_dim + c.v_dim
-
-        def rows_of(W, r0, r1):   # a view of rows r0 .. r1 of a quantised matrix
-            wb, sb = W.k * W.bits // 8, (W.k // W.group) * 2
-            V = DeviceWeight.__new__(DeviceWeight)
-            V.n, V.k, V.bits, V.group = r1 - r0, W.k, W.bits, W.group
-            V.w, V.scales, V.biases = _View(W.w, r0 * wb, (r1 - r0) * wb), _View(W.scales, r0 * sb, (r1 - r0) * sb), \
-                _View(W.biases, r0 * sb, (r1 - r0) * sb)
-            return V
-
-        native.embed_lookup_rows(w.mats["embed_tokens"], toks, m, 1.0, x)
-        for l in range(c.n_layers):
-            p = f"layers.{l}."
-            Wa = w.mats[p + "self_attn.kv_a_proj_with_mqa"]
-            native.rmsnorm_rows(x, w.vecs[p + "input_layernorm"], c.eps, m, c.hidden, xn)
-            native.qgemm(w.mats[p + "self_attn.q_proj"], xn, m, None, None, q, qws)
-            native.qgemm(rows_of(Wa, 0, c.kv_lora_rank), xn, m, None, None, lat, qws)
-            native.qgemm(rows_of(Wa, c.kv_lora_rank, n_a), xn, m, None, None, kpe, qws)
-            native.rmsnorm_rows(lat, w.vecs[p + "self_attn.kv_a_layernorm"], c.eps, m, c.kv_lora_rank, latn)
-            native.qgemm(w.mats[p + "self_attn.kv_b_proj"], latn, m, None, None, kvb, qws)
-            native.kv_cache_store_split_rows(q, c.n_heads, c.nope_dim, c.rope_dim, kvb, packed, n_b, kpe, 1, c.rope_dim,
-                                             _View(kvb, c.nope_dim * 2, kvb.nbytes - c.nope_dim * 2), packed, n_b, c.n_heads,
-                                             c.nope_dim, c.rope_dim, c.v_dim, c.rope_dim, c.rope_traditional, c.theta, m, offset,
-                                             c.capacity, self.cache_k[l], self.cache_v[l])
-            native.sdpa_decode_rows(q, self.cache_k[l], self.cache_v[l], att, m, offset + 1, c.n_heads, c.n_heads, c.qk_dim, c.v_dim,
-                                    c.capacity, 1.0 / float(np.sqrt(c.qk_dim)), parts, counters)
-            native.qgemm(w.mats[p + "self_attn.o_proj"], att, m, None, x, x1, qws)
-            post = w.vecs[p + "post_attention_layernorm"]
-            if l < c.first_dense:
-                native.rmsnorm_rows(x1, post, c.eps, m, c.hidden, xn)
-                native.qgemm_swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], xn, m, c.swiglu_variant, mid, qws)
-                native.qgemm(w.mats[p + "mlp.down_proj"], mid, m, None, x1, x, qws)
-                continue
-            native.moe_router(x1, post, c.eps, w.mats[p + "mlp.gate"].w, self.route_scale, c.hidden, c.n_experts, c.top_k, xn, rlg,
-                              ridx, rwt, rws, rows=m)
-            Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
-            native.routed_qmv_swiglu(xn, m, Eg, Eu, c.n_experts, rows_x, ridx, None, routes, h)
-            native.qgemm_swiglu(w.mats[p + "mlp.shared_experts.gate_proj"], w.mats[p + "mlp.shared_experts.up_proj"], xn, m,
-                                c.swiglu_variant, mid, qws)
-            native.routed_qmv_reduce(h, routes, Ed, c.n_experts, None, ridx, rwt, mid, w.mats[p + "mlp.shared_experts.down_proj"],
-                                     x1, m, c.top_k, x, mws)
-        last = _View(x, (m - 1) * c.hidden * 2, c.hidden * 2)
-        native.final_rmsnorm_lm_head(last, w.vecs["final_norm"], c.eps, w.mats["embed_tokens"], self.logits)
-        native.argmax_logits_decode(self.logits, c.vocab, self.token, None, None, 0, self.argmax_ws)
-        native.sync()
-        self.rows_routes = ridx.to_numpy(np.uint32, (m, c.top_k))   # of the last expert layer
-        return int(self.token.to_numpy(np.uint32)[0])
+        v = self._rows_variants.get(m)
+        if v is None:
+            v = self._rows_variants[m] = MoeRowsVariant(self, m)
+        nxt = v.run(tokens, offset)
+        self.rows_routes = v.ridx.to_numpy(np.uint32, (self.cfg.n_layers, m, self.cfg.top_k))[-1]   # of the last expert layer
+        return nxt
 
     # -- generation (the dense runtime's loop: prompt with forced tokens, then chunks fed back on the GPU)
     def reset(self) -> None:
@@ -469,6 +405,144 @@ class MoeRuntime:
             steps += n
             offset += n
         return out, gpu_s, steps
+
+
+class MoeRowsVariant:
+    """The whole MoE model for `m` active token rows as ONE task list / hipGraph (the reference's `active_m = m`
+    variants, src/commands/patch.rs:112-150): multi-row matmuls for the dense projections and the shared experts,
+    the row forms of the norm, the split-key store, the attention and the router, routed experts over
+    m x top_k routes, the ordered reduction with the shared expert's rows.  `offset` (position of row 0) and
+    `kv_len` (= offset + 1, row 0's) are device words the host writes before a replay; caches, token, history
+    and logits are the decode graph's."""
+
+    def __init__(self, rt: "MoeRuntime", m: int):
+        c = rt.cfg
+        if not 1 <= m <= c.capacity:
+            raise ValueError("rows must lie in 1 .. capacity")
+        if c.hidden % 512 or c.hidden > 4096:
+            raise ValueError("the row form of the router needs hidden to be a multiple of 512 of at most 4096")
+        self.rt, self.m, self.name = rt, m, f"prefill_m{m}"
+        B, z = DeviceBuffer, native.zeros
+        n_q, n_b = c.n_heads * c.qk_dim, c.n_heads * (c.nope_dim + c.v_dim)
+        self.tokens, self.offset, self.kv_len = z(4 * m), z(4), z(4)
+        self.x = [B(m * c.hidden * 2), B(m * c.hidden * 2)]
+        self.xn = B(m * c.hidden * 2)
+        self.q, self.lat, self.kpe, self.latn = B(m * n_q * 2), B(m * c.kv_lora_rank * 2), B(m * c.rope_dim * 2), B(m * c.kv_lora_rank * 2)
+        self.kvb, self.att = B(m * n_b * 2), B(m * c.n_heads * c.v_dim * 2)
+        self.mid = B(m * max(c.dense_inter, c.shared_inter) * 2)
+        routes = m * c.top_k
+        self.ridx, self.rwt = z(4 * routes * c.n_layers), z(2 * routes * c.n_layers)
+        self.rlg = z(2 * m * c.n_experts)
+        self.rows_x = DeviceBuffer.from_numpy(np.repeat(np.arange(m, dtype=np.uint32), c.top_k))
+        self.rows_h = DeviceBuffer.from_numpy(np.arange(routes, dtype=np.uint32))
+        self.h = B(routes * c.moe_inter * 2)
+        self.router_ws = z(4 * m * (c.n_experts + 1))
+        shapes = [(n_q, c.hidden), (c.kv_lora_rank, c.hidden), (c.rope_dim, c.hidden), (n_b, c.kv_lora_rank),
+                  (c.hidden, c.n_heads * c.v_dim), (c.shared_inter, c.hidden), (c.dense_inter, c.hidden), (c.hidden, c.dense_inter)]
+        self.qws = B(2 * max(native.qgemm_workspace_bytes(m, n, k, c.group) for n, k in shapes))
+        self.moe_ws = B(native.routed_reduce_workspace_bytes(m, c.top_k, c.hidden, c.shared_inter, c.group))
+        pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
+        self.parts, self.counters = B(max(pb, 4) * m), z(max(cb, 4) * m)
+        self.tasks = self._build()
+        self.graph = rt.d.build_graph(self.tasks)
+
+    def _build(self) -> List[Dispatch]:
+        rt, c, w, m = self.rt, self.rt.cfg, self.rt.w, self.m
+        quant = dict(bits=c.bits, group=c.group)
+        t: List[Dispatch] = []
+        fid = [0]
+
+        def name(kind: str) -> str:
+            fid[0] += 1
+            return f"fusekit_{kind}_f{fid[0]}"
+
+        def matmul(x, wargs, k, n, out, res=None):
+            a = [arg(x)] + list(wargs) + ([arg(res)] if res is not None else []) + [arg(out), arg(self.qws)]
+            t.append(Dispatch(name("qgemm"), a, dict(quant, m=k, n=n, rows=m, has_bias=0, has_residual=int(res is not None))))
+
+        def full(W):
+            return [arg(W.w), arg(W.scales), arg(W.biases)]
+
+        def norm_rows(x, nw, hidden, out):
+            t.append(Dispatch(name("rmsnorm_rows"), [arg(x), arg(nw), arg(out)], dict(rows=m, hidden=hidden, eps=c.eps)))
+
+        def swiglu(Wg, Wu, inter):
+            t.append(Dispatch(name("qgemm_swiglu"),
+                              [arg(self.xn), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases),
+                               arg(self.mid, m * inter * 2), arg(self.qws)],
+                              dict(quant, hidden=c.hidden, inter=inter, rows=m, variant=c.swiglu_variant)))
+
+        emb = w.mats["embed_tokens"]
+        t.append(Dispatch(name("embed_lookup_decode"), [arg(self.tokens), arg(emb.w), arg(self.x[0])],
+                          dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0, rows=m)))
+        n_q, n_a, n_b = c.n_heads * c.qk_dim, c.kv_lora_rank + c.rope_dim, c.n_heads * (c.nope_dim + c.v_dim)
+        packed, routes = c.nope_dim + c.v_dim, m * c.top_k
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            Wq, Wa, Wb, Wo = (w.mats[p + f"self_attn.{n}"] for n in ("q_proj", "kv_a_proj_with_mqa", "kv_b_proj", "o_proj"))
+            norm_rows(self.x[0], w.vecs[p + "input_layernorm"], c.hidden, self.xn)
+            matmul(self.xn, full(Wq), c.hidden, n_q, self.q)
+            matmul(self.xn, _rows(Wa, 0, c.kv_lora_rank), c.hidden, c.kv_lora_rank, self.lat)
+            matmul(self.xn, _rows(Wa, c.kv_lora_rank, n_a), c.hidden, c.rope_dim, self.kpe)
+            norm_rows(self.lat, w.vecs[p + "self_attn.kv_a_layernorm"], c.kv_lora_rank, self.latn)
+            matmul(self.latn, full(Wb), c.kv_lora_rank, n_b, self.kvb)
+            t.append(Dispatch(name("kv_cache_store_decode"),
+                              [arg(self.q), arg(self.kvb), arg(self.kpe), arg(self.kvb, self.kvb.nbytes - c.nope_dim * 2, c.nope_dim * 2),
+                               arg(rt.cache_k[l]), arg(rt.cache_v[l]), arg(self.offset), arg(self.offset)],
+                              dict(split_k=1, has_q=1, n_heads=c.n_heads, q0_dim=c.nope_dim, q1_dim=c.rope_dim, n_kv=c.n_heads,
+                                   k0_dim=c.nope_dim, k1_dim=c.rope_dim, v_dim=c.v_dim, k1_n_kv=1, k0_stride=packed, v_stride=packed,
+                                   rope_dims=c.rope_dim, traditional=int(c.rope_traditional), theta=c.theta, capacity=c.capacity,
+                                   rows=m, k0_row_stride=n_b, k1_row_stride=c.rope_dim, v_row_stride=n_b)))
+            t.append(Dispatch(name("sdpa_decode"),
+                              [arg(self.q), arg(rt.cache_k[l]), arg(rt.cache_v[l]), arg(self.kv_len), arg(self.att), arg(self.parts),
+                               arg(self.counters)],
+                              dict(n_heads=c.n_heads, n_kv=c.n_heads, qk_dim=c.qk_dim, head_dim=c.qk_dim, v_dim=c.v_dim,
+                                   capacity=c.capacity, max_len=c.capacity, rows=m)))
+            matmul(self.att, full(Wo), c.n_heads * c.v_dim, c.hidden, self.x[1], res=self.x[0])
+            post = w.vecs[p + "post_attention_layernorm"]
+            if l < c.first_dense:
+                norm_rows(self.x[1], post, c.hidden, self.xn)
+                swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], c.dense_inter)
+                matmul(self.mid, full(w.mats[p + "mlp.down_proj"]), c.dense_inter, c.hidden, self.x[0], res=self.x[1])
+                continue
+            ridx = arg(self.ridx, 4 * routes, 4 * routes * l)
+            rwt = arg(self.rwt, 2 * routes, 2 * routes * l)
+            t.append(Dispatch(name("moe_router"),
+                              [arg(self.x[1]), arg(post), arg(w.mats[p + "mlp.gate"].w), arg(rt.route_scale), arg(self.xn), arg(self.rlg),
+                               ridx, rwt, arg(self.router_ws)],
+                              dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1, rows=m)))
+            Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
+            Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
+            t.append(Dispatch(name("routed_qmv_swiglu"),
+                              [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
+                               arg(self.rows_x), ridx, arg(self.h)],
+                              dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=routes, x_rows=m)))
+            swiglu(Sg, Su, c.shared_inter)
+            t.append(Dispatch(name("routed_qmv_reduce"),
+                              [arg(self.h), arg(Ed.w), arg(Ed.scales), arg(Ed.biases), arg(self.rows_h), ridx, rwt,
+                               arg(self.mid, m * c.shared_inter * 2), arg(Sd.w), arg(Sd.scales), arg(Sd.biases), arg(self.x[1]),
+                               arg(self.x[0]), arg(self.moe_ws)],
+                              dict(quant, k=c.moe_inter, o=c.hidden, experts=c.n_experts, tokens=m, top_k=c.top_k, x_rows=routes,
+                                   has_shared=1, shared_k=c.shared_inter, has_extra=1)))
+        last = arg(self.x[0], c.hidden * 2, (m - 1) * c.hidden * 2)
+        t.append(Dispatch(name("final_rmsnorm_lm_head"), [last, arg(w.vecs["final_norm"]), arg(emb.w), arg(rt.logits)],
+                          dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
+        t.append(Dispatch(name("argmax_logits_decode"),
+                          [arg(rt.logits), arg(rt.token), arg(rt.argmax_ws), arg(rt.history), arg(rt.hist_counter)], dict(vocab=c.vocab)))
+        return t
+
+    def run(self, tokens: Sequence[int], offset: int) -> int:
+        rt = self.rt
+        tokens = list(tokens)
+        if len(tokens) != self.m:
+            raise ValueError(f"a variant of {self.m} rows processes exactly {self.m} tokens")
+        if offset + self.m > rt.cfg.capacity:
+            raise ValueError("rows exceed the KV-cache capacity")
+        self.tokens.upload(np.asarray(tokens, np.uint32))
+        self.offset.upload(np.array([offset], np.uint32))
+        self.kv_len.upload(np.array([offset + 1], np.uint32))     # row 0's length; row r attends to kv_len + r positions
+        rt.d.execute_graph(self.graph)
+        return int(rt.token.to_numpy(np.uint32)[0])
 
 
 class _View:
