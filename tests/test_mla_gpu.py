@@ -243,3 +243,27 @@ def test_families_in_a_graph(fk):
 
     for a, b in zip(run(True), run(False)):
         assert np.array_equal(a, b)
+
+
+def test_split_key_store_rows_wrap_around_the_cache(fk):
+    """Row form: token r at position offset + r lands in cache row (offset + r) % capacity with its own rotation;
+    the oracle stores the rows one by one."""
+    n_heads, k0d, k1d, vd, cap, rows, offset, theta = 4, 64, 32, 64, 8, 5, 6, 1e4
+    kvb = normal_bf16(70, (rows, n_heads, k0d + vd))
+    kpe = normal_bf16(71, (rows, k1d))
+    q = normal_bf16(72, (rows, n_heads, k0d + k1d))
+    ck0, cv0 = normal_bf16(73, n_heads * cap * (k0d + k1d)), normal_bf16(74, n_heads * cap * vd)
+    ck, cv = ck0.copy(), cv0.copy()
+    for r in range(rows):
+        flat = kvb[r].reshape(-1)
+        oracle.kv_store_split(flat, k0d + vd, kpe[r:r + 1], 1, flat[k0d:], k0d + vd, n_heads, k0d, k1d, vd, k1d, True, theta,
+                              offset + r, offset + r, cap, ck, cv)
+    d_kvb, d_q, d_ck, d_cv = _dev(fk, kvb), _dev(fk, q), _dev(fk, ck0), _dev(fk, cv0)
+    fk.kv_cache_store_split_rows(d_q, n_heads, k0d, k1d, d_kvb, k0d + vd, n_heads * (k0d + vd), _dev(fk, kpe), 1, k1d,
+                                 _Slice(d_kvb, k0d), k0d + vd, n_heads * (k0d + vd), n_heads, k0d, k1d, vd, k1d, True, theta, rows,
+                                 offset, cap, d_ck, d_cv)
+    assert np.array_equal(d_cv.to_numpy(np.uint16), cv)
+    frac, ulps = bf16_mismatch(d_ck.to_numpy(np.uint16), ck)
+    assert ulps <= 1.0 and frac <= 0.01, (frac, ulps)
+    gq = d_q.to_numpy(np.uint16).reshape(rows, n_heads, -1)
+    assert np.array_equal(gq[:, :, :k0d], q[:, :, :k0d]) and not np.array_equal(gq[1:, :, k0d:], q[1:, :, k0d:])

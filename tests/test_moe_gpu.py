@@ -127,6 +127,29 @@ def test_routed_swiglu_routing_for_itself(fk, apply_weight, shared):
         assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0
 
 
+def test_routed_swiglu_routing_ties_and_the_largest_admitted_shape(fk):
+    """256 experts, 32 routes: equal logits route to experts 0 .. 31 in order (ties to the lower index), each with
+    probability 1/256; then a seeded row against the oracle's router."""
+    E, O, K, top_k = 256, 64, 128, 32
+    Wg, Wu = _stack(3200, E, O, K, 4), _stack(3300, E, O, K, 4)
+    x = normal_bf16(62, (1, K))
+    one = oracle.f32_to_bf16(np.array([1.0], np.float32))
+    idx, w, out0 = fk.zeros(4 * top_k), fk.zeros(2 * top_k), fk.DeviceBuffer(2 * top_k * O)
+    dWg, dWu = to_device(fk, Wg), to_device(fk, Wu)
+    flat = oracle.f32_to_bf16(np.full(E, 0.25, np.float32))
+    fk.routed_qmv_swiglu_routing(_dev(fk, x), dWg, dWu, E, _dev(fk, flat), _dev(fk, one), top_k, False, idx, w, out0)
+    assert idx.to_numpy(np.uint32).tolist() == list(range(top_k))
+    assert np.array_equal(w.to_numpy(np.uint16), oracle.f32_to_bf16(np.full(top_k, 1.0 / E, np.float32)))
+    logits = normal_bf16(63, E, 2.0)
+    fk.routed_qmv_swiglu_routing(_dev(fk, x), dWg, dWu, E, _dev(fk, logits), _dev(fk, one), top_k, False, idx, w, out0)
+    ref_idx, ref_w = oracle.softmax_topk_route(logits, top_k, one)
+    got_idx = idx.to_numpy(np.uint32)
+    assert set(got_idx.tolist()) == set(ref_idx.reshape(-1).tolist()) and np.mean(got_idx == ref_idx.reshape(-1)) >= 0.9
+    assert bf16_mismatch(w.to_numpy(np.uint16), ref_w.reshape(-1))[1] <= 1.0
+    plain = _run_m1(fk, x, Wg, Wu, np.zeros(top_k, np.uint32), got_idx, None)
+    assert np.array_equal(out0.to_numpy(np.uint16, (top_k, O)), plain)
+
+
 def _run_m2(fk, h, Wd, row_idx, expert_idx, rw, shared_x, Ws, res, tokens, top_k):
     out = fk.DeviceBuffer(2 * tokens * Wd.n)
     ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, Wd.n))
