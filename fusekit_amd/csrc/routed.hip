@@ -13,6 +13,7 @@
 //                             out[tok, o] = T(sum_slots rw * part + shared + residual)
 // The weighted sum runs in slot order in fp32 in a second small kernel, so the
 // result does not depend on which block finishes first.
+#include <atomic>
 #include <map>
 #include <mutex>
 
@@ -22,7 +23,7 @@
 
 namespace fk {
 
-static bool t_routed_fused_reduce = true;   // off: always the three launches (tests compare the two)
+static std::atomic<bool> g_routed_fused_reduce{true};   // off: always the three launches (tests compare the two)
 
 struct RoutedArgs {
     GemvArgs g;                    // geometry of ONE route; pointers at expert 0 / activation row 0 / route 0
@@ -503,7 +504,7 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
         return set_error(FK_ERR_UNSUPPORTED, "routed reduce: the shared expert must have the routed experts' output width");
     if ((uint64_t)n_tokens * top_k > 65536) return set_error(FK_ERR_UNSUPPORTED, "routed reduce: too many routes");
     const uint32_t n_routes = n_tokens * top_k;
-    if (t_routed_fused_reduce && down_reduce_fits(Wd, W_shared, n_tokens, top_k)) {
+    if (g_routed_fused_reduce && down_reduce_fits(Wd, W_shared, n_tokens, top_k)) {
         const DeviceFacts* dev;
         FK_TRY(device_facts(&dev));
         if (!expert_idx) return set_error(FK_ERR_INVALID, "routed: null expert_idx");
@@ -556,6 +557,6 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
     return FK_OK;
 }
 
-void set_routed_fused_reduce(bool on) { t_routed_fused_reduce = on; }
+void set_routed_fused_reduce(bool on) { g_routed_fused_reduce = on; }
 
 }  // namespace fk
