@@ -305,6 +305,10 @@ fk_status fk_routed_qmv_reduce(const uint16_t* h, uint32_t n_h_rows, const fk_we
 
 void fk_set_routed_fused_reduce(int on) { set_routed_fused_reduce(on != 0); }
 
+int fk_gemm_library_available(void) { return gemm_library_available() ? 1 : 0; }
+
+fk_status fk_dequantize_bf16(const fk_weight* W, uint16_t* out, fk_stream s) { return run_dequantize_bf16(W, out, (hipStream_t)s); }
+
 fk_status fk_qgemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, uint32_t group, size_t* bytes) {
     if (!bytes) return set_error(FK_ERR_INVALID, "fk_qgemm_workspace_bytes: null output");
     return qgemm_workspace_bytes(m, n, k, group, bytes);

@@ -121,6 +121,7 @@ fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint
 
 // Large row counts, direct calls only: dequantise to bf16 once, library GEMM, the same epilogue.
 void set_gemm_library_rows(uint32_t rows);  // 0: never
+fk_status run_dequantize_bf16(const fk_weight* W, uint16_t* out, hipStream_t s);
 bool qgemm_takes_library(uint32_t m);
 bool gemm_library_available();
 size_t qgemm_library_sums_bytes(uint32_t m, uint32_t n, uint32_t k);

@@ -180,6 +180,19 @@ bool shape_ok(const fk_weight* W, uint32_t m) {
 
 }  // namespace
 
+// An MLX-affine matrix as bf16 [n, k], every element T(code * scale + bias): the values the library route of the
+// multi-row matmul works on.  A caller with memory to spare keeps the result and passes it as a dense weight.
+fk_status run_dequantize_bf16(const fk_weight* W, uint16_t* out, hipStream_t s) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!W || !W->w || !W->scales || !W->biases || !out) return set_error(FK_ERR_INVALID, "dequantize: null tensor");
+    if ((W->bits != 4 && W->bits != 8) || (W->group != 64 && W->group != 128) || W->k % W->group || W->n == 0)
+        return set_error(FK_ERR_UNSUPPORTED, "dequantize: bits must be 4 or 8, group 64 or 128 dividing k");
+    Launch l;
+    FK_TRY(plan_dequant(dev, W, out, &l));
+    return run_launch(l, s);
+}
+
 void set_gemm_library_rows(uint32_t rows) { g_library_rows = rows; }
 
 bool qgemm_takes_library(uint32_t m) {

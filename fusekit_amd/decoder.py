@@ -193,6 +193,7 @@ class DecoderRuntime:
         # fuses them itself and is built from the plain task list)
         self.fused_attention = bool(cfg.fuse_attention and not persistent and not cfg.kv_bits)
         self.rope_tab = DeviceBuffer(cfg.head_dim * 4) if self.fused_attention else None
+        self._bf16_weights: Dict[str, DeviceWeight] = {}   # resident bf16 copies for prompt passes (prefill_rows)
         self.tasks = self.build_tasks()
         # persistent: the same task list, run by one whole-token kernel per replay
         self.graph = (self.d.build_decode_graph(self.tasks, True, spin_limit) if persistent
@@ -321,7 +322,8 @@ class DecoderRuntime:
         nxt, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
         return nxt[-1]
 
-    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 4096) -> int:
+    def prefill_rows(self, prompt: Sequence[int], start_offset: int = 0, rows_per_pass: int = 4096,
+                     keep_bf16_weights: bool = False) -> int:
         """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
         active_m > 1 variants): the projections of up to `rows_per_pass` (<= 4096) tokens share ONE pass over each weight
         matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form, from 256 rows
@@ -329,7 +331,10 @@ class DecoderRuntime:
         causal inside the group (fk_sdpa_prefill for the bf16 cache with head dimension 64 or 128,
         else the single-row kernel once per row).  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy
-        first token.  Dense bf16 weights take the library GEMM for every row count."""
+        first token.  Dense bf16 weights take the library GEMM for every row count.
+        keep_bf16_weights: passes of at least 256 rows multiply with a bf16 copy of every projection that stays
+        resident after its first use (2 bytes per weight: 7.3 GB for the 4B-class model) instead of
+        dequantising each matrix again in every pass; same results bit for bit."""
         c, w = self.cfg, self.w
         prompt = list(prompt)
         if start_offset + len(prompt) > c.capacity:
@@ -360,6 +365,15 @@ class DecoderRuntime:
         head = w.mats.get("lm_head", emb)
         pos = start_offset
         scale = 1.0 / float(np.sqrt(c.head_dim))
+
+        def mat(name: str, m: int):
+            W = w.mats[name]
+            if not keep_bf16_weights or W.bits == 16 or m < 256 or not native.gemm_library_available():
+                return W
+            if name not in self._bf16_weights:
+                self._bf16_weights[name] = native.dequantize_bf16(W)
+            return self._bf16_weights[name]
+
         while pos < start_offset + len(prompt):
             chunk = prompt[pos - start_offset: pos - start_offset + R]
             m = len(chunk)
@@ -371,7 +385,7 @@ class DecoderRuntime:
                 native.rmsnorm_rows(b["x"], w.vecs[p + "input_layernorm"], c.eps, m, c.hidden, b["xn"])
                 for nm, dst in (("q", b["q"]), ("k", b["k"]), ("v", b["v"])):
                     bias = w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None
-                    native.qgemm(w.mats[p + f"self_attn.{nm}_proj"], b["xn"], m, bias, None, dst, b["ws"])
+                    native.qgemm(mat(p + f"self_attn.{nm}_proj", m), b["xn"], m, bias, None, dst, b["ws"])
                 qn = w.vecs.get(p + "self_attn.q_norm") if c.qk_norm else None
                 kn = w.vecs.get(p + "self_attn.k_norm") if c.qk_norm else None
                 if c.kv_bits:
@@ -398,11 +412,11 @@ class DecoderRuntime:
                     else:
                         native.sdpa_decode_rows(b["q"], self.cache_k[l], self.cache_v[l], b["att"], m, pos + 1, c.n_heads,
                                                 c.n_kv, c.head_dim, c.head_dim, c.capacity, scale, b["part"], b["cnt"])
-                native.qgemm(w.mats[p + "self_attn.o_proj"], b["att"], m, None, b["x"], b["x2"], b["ws"])
+                native.qgemm(mat(p + "self_attn.o_proj", m), b["att"], m, None, b["x"], b["x2"], b["ws"])
                 native.rmsnorm_rows(b["x2"], w.vecs[p + "post_attention_layernorm"], c.eps, m, c.hidden, b["xn"])
-                native.qgemm_swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], b["xn"], m, c.swiglu_variant,
+                native.qgemm_swiglu(mat(p + "mlp.gate_proj", m), mat(p + "mlp.up_proj", m), b["xn"], m, c.swiglu_variant,
                                     b["mid"], b["ws"])
-                native.qgemm(w.mats[p + "mlp.down_proj"], b["mid"], m, None, b["x2"], b["x"], b["ws"])
+                native.qgemm(mat(p + "mlp.down_proj", m), b["mid"], m, None, b["x2"], b["x"], b["ws"])
             pos += m
         # the last row's hidden state -> logits -> greedy token, and the decode loop's uniforms
         last = DeviceBuffer(c.hidden * 2)

@@ -221,7 +221,7 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
           note="two kernels: MFMA main + split-k reduction")
 
 
-def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_bits=0):
+def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_bits=0, keep=False):
     """Chunked prefill of the 4B-class model: `rows_per_pass` prompt tokens per pass over the weights."""
     import time
     import numpy as np
@@ -230,15 +230,15 @@ def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_
     W = DecoderWeights.random_init(cfg, seed=0)
     rt = DecoderRuntime(cfg, W, dispatcher=d)
     prompt = np.random.Generator(np.random.PCG64(0)).integers(0, cfg.vocab, prompt_len).tolist()
-    rt.prefill_rows(prompt, rows_per_pass=rows_per_pass)
+    rt.prefill_rows(prompt, rows_per_pass=rows_per_pass, keep_bf16_weights=keep)
     t0 = time.perf_counter()
-    rt.prefill_rows(prompt, rows_per_pass=rows_per_pass)
+    rt.prefill_rows(prompt, rows_per_pass=rows_per_pass, keep_bf16_weights=keep)
     rows_s = time.perf_counter() - t0
     t0 = time.perf_counter()
     rt.prefill(prompt[:64])
     single_s = (time.perf_counter() - t0) / 64 * prompt_len
     flops = 2.0 * prompt_len * (cfg.n_layers * (cfg.hidden * (cfg.n_q + 2 * cfg.n_kvd) + cfg.n_q * cfg.hidden + 3 * cfg.inter * cfg.hidden))
-    print(json.dumps({"case": f"prefill_4b_q4_{prompt_len}_tokens" + (f"_kv{kv_bits}" if kv_bits else ""), "rows_per_pass": rows_per_pass,
+    print(json.dumps({"case": f"prefill_4b_q4_{prompt_len}_tokens" + (f"_kv{kv_bits}" if kv_bits else "") + ("_bf16_copy" if keep else ""), "rows_per_pass": rows_per_pass,
                       "prompt_tok_per_s": round(prompt_len / rows_s, 1), "ms": round(rows_s * 1e3, 2),
                       "token_by_token_tok_per_s": round(prompt_len / single_s, 1),
                       "TFLOPs": round(flops / rows_s / 1e12, 2)}), flush=True)
@@ -325,6 +325,8 @@ CASES = {
     "prefill_4b_4096_tokens": lambda d, r: case_prefill(d, r, 4096, 512, 4608),
     "prefill_4b_4096_tokens_1024": lambda d, r: case_prefill(d, r, 4096, 1024, 4608),
     "prefill_4b_4096_tokens_4096": lambda d, r: case_prefill(d, r, 4096, 4096, 4608),
+    "prefill_4b_4096_tokens_bf16_copy": lambda d, r: case_prefill(d, r, 4096, 4096, 4608, keep=True),
+    "prefill_4b_512_tokens_bf16_copy": lambda d, r: case_prefill(d, r, 512, 512, 1024, keep=True),
     "prefill_4b_4096_tokens_kv4": lambda d, r: case_prefill(d, r, 4096, 4096, 4608, kv_bits=4),
 }
 

@@ -429,6 +429,19 @@ def sdpa_prefill(q, cache_k, cache_v, out, rows, kv_len, n_heads, n_kv, head_dim
                               C.c_float(scale), _ptr(stream)))
 
 
+def gemm_library_available() -> bool:
+    return bool(lib.fk_gemm_library_available())
+
+
+def dequantize_bf16(W: DeviceWeight, stream=None) -> DeviceWeight:
+    """The bf16 copy of a quantised matrix (fk_dequantize_bf16) as a bits-16 DeviceWeight."""
+    D = DeviceWeight.__new__(DeviceWeight)
+    D.n, D.k, D.bits, D.group, D.scales, D.biases = W.n, W.k, 16, 0, None, None
+    D.w = DeviceBuffer(W.n * W.k * 2)
+    check(lib.fk_dequantize_bf16(C.byref(W.c), _ptr(D.w), _ptr(stream)))
+    return D
+
+
 def set_gemm_library_rows(rows: int):
     """Row count from which qgemm / qgemm_swiglu take the dequantise + library-GEMM route (0: never)."""
     check(lib.fk_set_gemm_library_rows(C.c_uint32(rows)))

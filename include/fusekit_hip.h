@@ -605,6 +605,15 @@ fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks);
  * product to rocBLAS (opened on first use; absent: the fused kernel is kept).  Default 256; 0 = never.
  * Set it BEFORE sizing workspaces: fk_qgemm_workspace_bytes covers the route that will be taken. */
 fk_status fk_set_gemm_library_rows(uint32_t rows);
+/* An MLX-affine matrix (bits 4 / 8, group 64 / 128) as dense bf16 [n, k], every element T(code * scale + bias):
+ * the values the library route of fk_qgemm multiplies with.  With 288 GB of HBM a runtime may keep the bf16 copy
+ * of a model's projections resident for its prompt passes and hand it to fk_qgemm as a bits-16 weight, which
+ * then skips the per-pass dequantisation; the results are the library route's, bit for bit.  No counterpart in
+ * the reference (its qMM dequantises inside the kernel, src/codegen/msl.rs:2318-2440). */
+fk_status fk_dequantize_bf16(const fk_weight *W, uint16_t *out, fk_stream s);
+/* 1 when the GEMM library (rocBLAS, loaded at first use) is present: bits-16 weights and the route from
+ * fk_set_gemm_library_rows rows up need it. */
+int fk_gemm_library_available(void);
 
 #pragma GCC visibility pop
 #ifdef __cplusplus
