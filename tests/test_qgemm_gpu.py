@@ -128,9 +128,10 @@ def test_qgemm_many_rows_both_routes(fk, m, n, k, bits, group, route):
         fk.set_gemm_library_rows(256)
 
 
-@pytest.mark.parametrize("route", ["kernel", "library"])
-def test_qgemm_swiglu_many_rows_both_routes(fk, route):
-    m, hidden, inter, variant = 512, 896, 1216, 2
+@pytest.mark.parametrize("route,m", [("kernel", 512), ("library", 512), ("library", 2048)])
+def test_qgemm_swiglu_many_rows_both_routes(fk, route, m):
+    """From 2048 rows the library route lets the GEMM round gate and up to bf16 itself and runs SwiGLU over bf16."""
+    hidden, inter, variant = 896, 1216, 2
     fk.set_gemm_library_rows(0 if route == "kernel" else 256)
     try:
         Wg, Wu = make_qweight(76, inter, hidden, 4), make_qweight(77, inter, hidden, 4)
@@ -141,9 +142,10 @@ def test_qgemm_swiglu_many_rows_both_routes(fk, route):
         got = out.to_numpy(np.uint16, (m, inter))
         _, g = oracle.qgemm_bf16w(Wg, x, None, want_acc=True)
         _, u = oracle.qgemm_bf16w(Wu, x, None, want_acc=True)
-        want = np.array([[oracle.swiglu_scalar(float(a), float(b), variant) for a, b in zip(g[r], u[r])] for r in range(0, m, 37)],
+        step = 37 * (m // 512)
+        want = np.array([[oracle.swiglu_scalar(float(a), float(b), variant) for a, b in zip(g[r], u[r])] for r in range(0, m, step)],
                         dtype=np.uint16)
-        sel = got[::37]
+        sel = got[::step]
         gf, wf = oracle.bf16_to_f32(sel).astype(np.float64), oracle.bf16_to_f32(want).astype(np.float64)
         assert np.linalg.norm(gf - wf) / np.linalg.norm(wf) <= 1e-2
         assert np.mean(sel != want) <= 0.05          # fp32 summation order may cross a bf16 rounding edge
