@@ -298,6 +298,11 @@ CASES = {
     "qgemv_big_q4": lambda d, r: case_qgemv(d, r, 9728, 2560, 4, 48, "9728x2560"),
     "qgemv_big_q8": lambda d, r: case_qgemv(d, r, 9728, 2560, 8, 28, "9728x2560"),
     "qgemv_big_bf16": lambda d, r: case_qgemv(d, r, 9728, 2560, 16, 14, "9728x2560"),
+    # Vocabulary-sized matrices: hundreds of MB per launch, so the start-up chain of a launch is
+    # amortised and the figure is the kernel's steady streaming rate.
+    "qgemv_vocab_q4": lambda d, r: case_qgemv(d, r, 151936, 2560, 4, 3, "151936x2560"),
+    "qgemv_vocab_q8": lambda d, r: case_qgemv(d, r, 151936, 2560, 8, 2, "151936x2560"),
+    "qgemv_wide_q4": lambda d, r: case_qgemv(d, r, 65536, 8192, 4, 2, "65536x8192"),
     "sdpa_512": lambda d, r: case_sdpa(d, r, 512),
     "sdpa_4096": lambda d, r: case_sdpa(d, r, 4096),
     "sdpa_32768": lambda d, r: case_sdpa(d, r, 32768),
