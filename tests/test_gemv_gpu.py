@@ -67,6 +67,17 @@ def test_qgemv_matches_oracle(fk, n, k, bits):
     assert rel_l2(got, ref64) <= REL_L2_BAR
 
 
+def test_qgemv_vocab_sized_matches_oracle(fk):
+    """The 219 MB shape whose streaming rate the kernel bench reports (1536 blocks, many tiles per block)."""
+    n, k = 151936, 2560
+    W = make_qweight(4242, n, k, 4)
+    x = normal_bf16(9, k)
+    dW, dx = to_device(fk, W), fk.DeviceBuffer.from_numpy(x)
+    dy = fk.DeviceBuffer(2 * n)
+    fk.qgemv(dW, dx, None, dy)
+    _check(dy.to_numpy(np.uint16), oracle.qgemv(W, x), oracle.linear_acc(W, x), W, x)
+
+
 @pytest.mark.parametrize("group", [32, 128])
 @pytest.mark.parametrize("bits", [4, 8])
 def test_qgemv_other_group_sizes(fk, bits, group):
