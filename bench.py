@@ -1,18 +1,24 @@
 #!/usr/bin/env python3
-"""Headline benchmark: hipGraph-replayed batch-1 greedy decode of the 4B-class dense model,
-4-bit g64 MLX-affine weights, 512 generated tokens, on one MI355X.
+"""Headline benchmark: hipGraph-replayed batch-1 greedy decode of the 4B-class dense model
+(configs[3]: 36 layers, hidden 2560, 4-bit g64 MLX-affine weights) at context 512, on one MI355X.
 
-One "step" = one decoded token = one replay of the captured decode graph (step_init, embed,
-36 x [rmsnorm_qkv, rope + kv-store + sdpa (one launch), o_proj+residual,
-rmsnorm_gateup_swiglu, down_proj+residual], final norm + LM head, argmax).  Weights are random-init (seeded, generated
-and quantised in HBM); inputs are resident before the timed region.
+One "step" = one decoded token = one replay of the captured decode graph.  Weights are random-init
+(seeded, generated and quantised in HBM); everything is resident before the timed region.
+
+The K timed steps always sit around context 512: after the 32-token prompt the script decodes
+untimed (at least --warmup steps) until the cache holds 512 - K/2 positions, then times exactly K
+steps, so the window is [512 - K/2, 512 + K/2] whatever K is (K <= 960).
 
 Prints ONE JSON line: value = generated tokens/s (wall clock around the K timed steps), plus
-  roofline     -- the dominant kernel (int4 gate/up SwiGLU qGEMV): algorithmic bytes per launch /
-                  its average launch duration, measured here with HIP events on the launch stream
-                  over the 36 layers' distinct weights (985 MB, larger than any cache),
+  roofline     -- the kernel symbol that holds the largest share of a token's GPU time: algorithmic
+                  bytes of its launches / their summed average durations, measured here with HIP
+                  events on the launch stream over serialised graphs of the 36 layers' own nodes
+                  (distinct weights, 2 GB in all: nothing stays in a cache); `by_launch` lists every
+                  launch shape of the token the same way,
+  qgemv_cfg1   -- configs[0]/[1]'s int4 qGEMV (4864 x 896, g64) over a rotating pool of 512 weight
+                  sets (1.26 GB), GB/s and fraction of the 8 TB/s peak,
   cpu_baseline -- the CPU oracle (C restatement of the reference semantics) decoding the same
-                  model on the host cores, bounded to --cpu-tokens decode steps (about 10 s of CPU work).
+                  model at the same context on the host cores, bounded to --cpu-tokens steps.
 """
 import argparse
 import json
@@ -24,10 +30,24 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E published peak
-# HBM bytes per launch of the int4 gate/up kernel of the 4B-class model, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE (two counter runs of this script, each scaled by what the same counter reads for the plain
-# 256 MiB copies of --calibrate-copy: 1.99989 and 1.0).  Counters cannot be read from inside this process.
-GATEUP_Q4_4B_TRAFFIC_BYTES = 28590500
+CONTEXT = 512
+
+# task family -> (HIP kernel symbol as rocprofv3 prints it, short label)
+SYMBOLS = {
+    "rmsnorm_qkv": "gemv_stream_kernel<Q4, 1 segment>",
+    "linear_residual": "gemv_stream_kernel<Q4, 1 segment>",
+    "rmsnorm_gateup_swiglu": "gemv_stream_kernel<Q4, gate/up pair>",
+    "rope_store_sdpa_decode": "sdpa_rope_store_kernel",
+    "final_rmsnorm_lm_head": "gemv_stream_kernel<BF16, 1 segment>",
+    "argmax_logits_decode": "argmax_kernel",
+    "embed_lookup_decode": "embed_lookup_kernel",
+    "step_init": "step_init_kernel",
+}
+
+
+def family(kernel: str) -> str:
+    name = kernel[len("fusekit_"):] if kernel.startswith("fusekit_") else kernel
+    return name.rsplit("_f", 1)[0] if "_f" in name else name
 
 
 def main() -> int:
@@ -38,8 +58,9 @@ def main() -> int:
     ap.add_argument("--bits", type=int, default=4, choices=[4, 8, 16])
     ap.add_argument("--prompt", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-tokens", type=int, default=24,
-                    help="decode steps the CPU oracle runs for cpu_baseline (about 10 s on 16 cores)")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-launch measurements (roofline, qgemv_cfg1)")
+    ap.add_argument("--cpu-tokens", type=int, default=48,
+                    help="decode steps the CPU oracle runs for cpu_baseline (10-30 s on the box's cores)")
     ap.add_argument("--per-kernel", action="store_true", help="print per-family GPU time of one token to stderr")
     ap.add_argument("--layers", type=int, default=0, help="experiment only: override the layer count (not the headline config)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -60,14 +81,15 @@ def main() -> int:
     from fusekit_amd.runtime import Dispatch, arg
 
     props = fk.device_props()
-    total = args.prompt + args.warmup + args.steps
+    start = max(args.prompt + args.warmup, CONTEXT - args.steps // 2)   # context of the first timed step
+    total = start + args.steps
     capacity = max(1024, 1 << (total - 1).bit_length())
     cfg = DecoderConfig(**DENSE_4B, bits=args.bits, capacity=capacity)
     if args.layers:
         cfg.n_layers = args.layers
     t0 = time.time()
     W = DecoderWeights.random_init(cfg, seed=0)
-    rt = DecoderRuntime(cfg, W, hist_capacity=max(4096, args.steps + args.warmup),
+    rt = DecoderRuntime(cfg, W, hist_capacity=max(4096, total),
                         persistent=(args.mode == "persistent"))
     setup_s = time.time() - t0
 
@@ -84,12 +106,11 @@ def main() -> int:
     first = rt.prefill(prompt)
     offset = len(prompt)
     tok = first
-    # warm-up: W untimed decode steps
-    done = 0
-    while done < args.warmup:
-        n = min(64, args.warmup - done)
+    # untimed: decode until the cache holds `start` positions (>= W steps; this is the warm-up)
+    while offset < start:
+        n = min(64, start - offset)
         toks, _ = rt.d.decode_chunk(rt.graph, rt.uniforms, offset, tok, n)
-        tok, offset, done = toks[-1], offset + n, done + n
+        tok, offset = toks[-1], offset + n
     fk.sync()
     # timed: exactly K steps, all chunks enqueued by the native loop, sync on both sides
     gpu_s = 0.0
@@ -102,39 +123,12 @@ def main() -> int:
     fk.sync()
     wall_s = time.perf_counter() - t0
     tok_s = args.steps / wall_s
-    ctx_mid = args.prompt + args.warmup + args.steps // 2
+    ctx_mid = start + args.steps // 2
     bytes_per_token = cfg.token_bytes(ctx_mid)
     roofline_tok_s = HBM_PEAK_GBPS * 1e9 / bytes_per_token
 
-    # ---- dominant kernel: gate/up SwiGLU qGEMV over the 36 layers' distinct weights ----
-    gateup = [t for t in rt.tasks if t.kernel.startswith("fusekit_rmsnorm_gateup_swiglu")]
-    per = cfg.bits / 8 + (0 if cfg.bits == 16 else 4 / cfg.group)
-    gateup_bytes = int(2 * cfg.inter * cfg.hidden * per) + 2 * cfg.hidden * 2 + cfg.inter * 2
-    g2 = rt.d.build_graph(gateup, barriers=[True] * len(gateup))   # serialised, one launch after another
-    rt.d.execute_graph(g2)
-    reps = 20
-    sec = rt.d.execute_graph(g2, repeat=reps)
-    gateup_us = sec / (reps * len(gateup)) * 1e6
-    achieved = gateup_bytes / (gateup_us * 1e-6) / 1e9
-
-    per_kernel = {}
-    if args.per_kernel and args.mode == "persistent":
-        tr = rt.d.graph_phase_trace(rt.graph)
-        names = ["embed"] + ["qkv", "attention", "o_proj", "gateup", "down"] * cfg.n_layers + ["lm_head", "argmax_scan", "argmax_final"]
-        for nm, s_ in zip(names, tr):
-            per_kernel[nm] = per_kernel.get(nm, 0.0) + s_
-        print("[bench:per-phase] " + " ".join(f"{k}={v * 1e3:.3f}ms" for k, v in per_kernel.items())
-              + f" | layer0: " + " ".join(f"{n}={t * 1e6:.1f}us" for n, t in zip(names[1:6], tr[1:6])), file=sys.stderr)
-    elif args.per_kernel:
-        times = rt.d.profile_graph_nodes(rt.graph)
-        for t, s in zip(rt.tasks, times):
-            fam = t.kernel.rsplit("_f", 1)[0]
-            per_kernel[fam] = per_kernel.get(fam, 0.0) + s
-        print("[bench:per-kernel] " + " ".join(f"{k}={v * 1e3:.3f}ms" for k, v in per_kernel.items()),
-              file=sys.stderr)
-
     out = {
-        "metric": "decode tok/s, 4B-class %d-bit @ L=%d (int4 qGEMV HBM GB/s in roofline)" % (cfg.bits, args.steps),
+        "metric": "decode tok/s, 4B-class %d-bit @ L=%d (int4 qGEMV HBM GB/s in qgemv_cfg1 and roofline)" % (cfg.bits, ctx_mid),
         "value": round(tok_s, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -150,7 +144,9 @@ def main() -> int:
             "workload": "configs[3]: 36-layer dense decoder, hidden 2560, inter 9728, 32q/8kv heads x128, vocab 151936 "
                         "tied bf16 head, %d-token prompt, greedy decode, one hipGraph per token" % args.prompt,
             "weights": "%d-bit g%d MLX-affine" % (cfg.bits, cfg.group) if cfg.bits != 16 else "bf16",
-            "context_range": [args.prompt + args.warmup, args.prompt + args.warmup + args.steps],
+            "context": ctx_mid,
+            "context_range": [start, start + args.steps],
+            "untimed_steps_before": start - args.prompt,
             "graph_nodes": len(rt.tasks),
         },
         "gpu_ms_per_step": round(gpu_s / args.steps * 1e3, 4),
@@ -159,19 +155,101 @@ def main() -> int:
         "frac_of_roofline_tok_s": round(tok_s / roofline_tok_s, 4),
         "device": props.name.decode().strip() or props.arch.decode(),
         "setup_s": round(setup_s, 1),
-        "roofline": {
-            "kernel": "gemv_stream_kernel<Q4, gate/up SwiGLU, fused RMSNorm> (fusekit_rmsnorm_gateup_swiglu)",
+    }
+
+    # ---- per launch shape: serialised graphs of the token's own nodes, HIP events on the dispatcher's stream ----
+    if not args.no_kernels and args.mode == "graph":
+        # the attention launches read kv_len from the device: hold the measurement at context 512
+        rt.kv_len.upload(np.array([CONTEXT], np.uint32))
+        rt.offset.upload(np.array([CONTEXT - 1], np.uint32))
+        rt.step_counter.upload(np.array([CONTEXT - 1], np.uint32))
+        kv_row_bytes = 2 * cfg.n_kv * cfg.head_dim * 2
+        groups = {}   # (family, position of the launch among its family inside a layer) -> tasks
+        seen = {}
+        for t in rt.tasks:
+            fam = family(t.kernel)
+            if fam in ("step_init",):
+                continue
+            idx = seen.get(fam, 0)
+            seen[fam] = idx + 1
+            per_layer = 2 if fam == "linear_residual" else 1
+            groups.setdefault((fam, idx % per_layer), []).append(t)
+        by_launch, by_symbol = [], {}
+        for (fam, pos), tasks in groups.items():
+            if fam == "rope_store_sdpa_decode" or fam.startswith("sdpa_decode"):
+                nbytes = kv_row_bytes * CONTEXT + 2 * (cfg.n_q * 2)          # K/V rows read + q in, out
+                label = "rope/store + attention @%d" % CONTEXT
+            else:
+                nbytes = sum(n for _, n in tasks[0].args)                    # weights + scales + biases + vectors in/out
+                label = {("linear_residual", 0): "o_proj + residual", ("linear_residual", 1): "down_proj + residual"}.get(
+                    (fam, pos), fam)
+            reps = max(2, 720 // len(tasks))
+            g = rt.d.build_graph(tasks, barriers=[True] * len(tasks))
+            rt.d.execute_graph(g)
+            us = rt.d.execute_graph(g, repeat=reps) / (reps * len(tasks)) * 1e6
+            sym = SYMBOLS.get(fam, fam)
+            e = {"launch": label, "kernel": sym, "per_token": len(tasks), "bytes_per_launch": int(nbytes),
+                 "avg_launch_us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),
+                 "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            by_launch.append(e)
+            s = by_symbol.setdefault(sym, {"us": 0.0, "bytes": 0, "launches": 0})
+            s["us"] += us * len(tasks)
+            s["bytes"] += nbytes * len(tasks)
+            s["launches"] += len(tasks)
+        dom = max(by_symbol, key=lambda k: by_symbol[k]["us"])
+        s = by_symbol[dom]
+        achieved = s["bytes"] / s["us"] / 1e3
+        out["roofline"] = {
+            "kernel": dom,
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": GATEUP_Q4_4B_TRAFFIC_BYTES if (cfg.bits == 4 and not args.layers) else None,
-            "bytes_per_launch": gateup_bytes,
-            "avg_launch_us": round(gateup_us, 3),
-            "launches_timed": reps * len(gateup),
-        },
-    }
+            "traffic": None,
+            "bytes_per_launch": int(s["bytes"] / s["launches"]),
+            "avg_launch_us": round(s["us"] / s["launches"], 3),
+            "launches_per_token": s["launches"],
+            "share_of_token_gpu_time": round(s["us"] / sum(v["us"] for v in by_symbol.values()), 4),
+            "by_launch": sorted(by_launch, key=lambda e: -e["avg_launch_us"] * e["per_token"]),
+        }
+        if args.per_kernel:
+            for e in out["roofline"]["by_launch"]:
+                print("[bench:launch] %-34s x%-3d %8.2f us  %7.1f GB/s  %.3f of peak" % (
+                    e["launch"], e["per_token"], e["avg_launch_us"], e["GBps"], e["frac"]), file=sys.stderr)
+
+        # ---- configs[0]/[1]: the single int4 qGEMV 4864 x 896 over a rotating pool of 512 weight sets ----
+        if cfg.bits == 4:
+            from fusekit_amd.kernel_bench import _bf16, _rand_weight, _wargs
+            n, k, pool = 4864, 896, 512
+            nbytes = int(n * k * 0.5625) + k * 2 + n * 2
+            Ws = [_rand_weight(n, k, 4, 100 + 3 * i) for i in range(pool)]
+            x, ys = _bf16(k, 7), [fk.DeviceBuffer(n * 2) for _ in range(pool)]
+            tasks = [Dispatch("fusekit_qgemv_f0", [arg(x)] + _wargs(Wi) + [arg(y)], {"bits": 4, "group": 64, "m": k, "n": n})
+                     for Wi, y in zip(Ws, ys)]
+            res = {}
+            for name, serial in (("serial", True), ("overlapped", False)):
+                g = rt.d.build_graph(tasks, barriers=[serial] * pool)
+                rt.d.execute_graph(g)
+                us = rt.d.execute_graph(g, repeat=4) / (4 * pool) * 1e6
+                res[name] = us
+            out["qgemv_cfg1"] = {
+                "shape": "4864 x 896 int4 g64, bf16 x and y", "pool": pool, "bytes_per_launch": nbytes,
+                "serial_us": round(res["serial"], 3), "serial_GBps": round(nbytes / res["serial"] / 1e3, 1),
+                "serial_frac": round(nbytes / res["serial"] / 1e3 / HBM_PEAK_GBPS, 4),
+                "overlapped_us": round(res["overlapped"], 3), "overlapped_GBps": round(nbytes / res["overlapped"] / 1e3, 1),
+                "overlapped_frac": round(nbytes / res["overlapped"] / 1e3 / HBM_PEAK_GBPS, 4),
+                "note": "serial: dependent graph nodes, launch to launch; overlapped: independent nodes of one graph",
+            }
+            del Ws, ys, tasks
+
+    if args.per_kernel and args.mode == "persistent":
+        per_kernel = {}
+        tr = rt.d.graph_phase_trace(rt.graph)
+        names = ["embed"] + ["qkv", "attention", "o_proj", "gateup", "down"] * cfg.n_layers + ["lm_head", "argmax_scan", "argmax_final"]
+        for nm, s_ in zip(names, tr):
+            per_kernel[nm] = per_kernel.get(nm, 0.0) + s_
+        print("[bench:per-phase] " + " ".join(f"{k}={v * 1e3:.3f}ms" for k, v in per_kernel.items()), file=sys.stderr)
 
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -179,18 +257,20 @@ def main() -> int:
         from helpers import OracleDecoder
         od = OracleDecoder(cfg, W)
         threads = oracle.num_threads()
+        od.step(prompt[0], CONTEXT - 1)                    # untimed: pages the weights in
         t0 = time.perf_counter()
         t = prompt[0]
         for i in range(args.cpu_tokens):
-            t, _, _ = od.step(t, i)
+            t, _, _ = od.step(t, CONTEXT + i)
         cpu_s = time.perf_counter() - t0
         out["cpu_baseline"] = {
             "value": round(args.cpu_tokens / cpu_s, 4),
             "unit": "tokens/s",
             "cores": threads,
             "kind": "port",
-            "sample": "%d decode steps of the same model at context 1..%d with the CPU oracle (OpenMP over rows/heads)"
-                      % (args.cpu_tokens, args.cpu_tokens),
+            "sample": "%d decode steps of the same model at context %d..%d with the CPU oracle (OpenMP over rows / heads; "
+                      "the cache rows before the sample are zeros, which costs the same arithmetic)"
+                      % (args.cpu_tokens, CONTEXT + 1, CONTEXT + args.cpu_tokens),
         }
     print(json.dumps(out))
     return 0

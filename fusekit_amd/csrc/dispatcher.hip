@@ -1068,6 +1068,7 @@ struct Graph {
     std::vector<Node> nodes;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    std::vector<uint8_t> barriers;  // as given to fk_build_graph (empty: none forced)
     // persistent whole-token mode: one kernel node; device-side tables it reads
     bool persistent = false;
     Launch token_launch;
@@ -1075,6 +1076,15 @@ struct Graph {
     uint32_t* d_abort = nullptr;
     unsigned long long* d_trace = nullptr;
     uint32_t trace_len = 0;
+    Graph() = default;
+    Graph(const Graph&) = delete;
+    Graph& operator=(const Graph&) = delete;
+    // a graph that fails half-way through its construction is dropped by its builder: release what it holds
+    ~Graph() {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
+        if (d_tables) (void)hipFree(d_tables);
+    }
 };
 
 struct DispatcherState {
@@ -1118,6 +1128,20 @@ hipKernelNodeParams launch_params(Launch& l, void** slot) {
 }
 hipKernelNodeParams node_params(Node& n, void** slot) { return launch_params(n.launch, slot); }
 
+// Does the later dispatch `b` have to wait for the earlier `a` (RAW / WAW / WAR on overlapping byte ranges)?
+bool direct_dep(const std::vector<fk_arg>& aa, const SlotRW& arw, const std::vector<fk_arg>& ba, const SlotRW& brw) {
+    for (uint32_t ws : arw.writes) {
+        for (uint32_t s : brw.reads)
+            if (overlap(aa[ws], ba[s])) return true;
+        for (uint32_t s : brw.writes)
+            if (overlap(aa[ws], ba[s])) return true;
+    }
+    for (uint32_t rs : arw.reads)
+        for (uint32_t s : brw.writes)
+            if (overlap(aa[rs], ba[s])) return true;
+    return false;
+}
+
 // RAW / WAW / WAR edges on overlapping byte ranges, transitively reduced.
 void derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
     const size_t n = nodes.size();
@@ -1126,21 +1150,8 @@ void derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
     for (size_t i = 0; i < n; ++i) {
         std::vector<uint32_t> cand;
         for (size_t j = 0; j < i; ++j) {
-            bool dep = barriers && barriers[i];
             const Node &a = nodes[j], &b = nodes[i];
-            for (uint32_t ws : a.rw.writes) {
-                if (dep) break;
-                for (uint32_t s : b.rw.reads)
-                    if (overlap(a.d.args[ws], b.d.args[s])) { dep = true; break; }
-                if (dep) break;
-                for (uint32_t s : b.rw.writes)
-                    if (overlap(a.d.args[ws], b.d.args[s])) { dep = true; break; }
-            }
-            for (uint32_t rs : a.rw.reads) {
-                if (dep) break;
-                for (uint32_t s : b.rw.writes)
-                    if (overlap(a.d.args[rs], b.d.args[s])) { dep = true; break; }
-            }
+            const bool dep = (barriers && barriers[i]) || direct_dep(a.d.args, a.rw, b.d.args, b.rw);
             if (dep) cand.push_back((uint32_t)j);
         }
         // keep a candidate only if no later candidate already descends from it
@@ -1443,7 +1454,11 @@ fk_status check_abort(Graph* g) {
     if (!g->persistent) return FK_OK;
     uint32_t flag = 0;
     FK_HIP(hipMemcpy(&flag, g->d_abort, 4, hipMemcpyDeviceToHost));
-    if (flag) return set_error(FK_ERR_HIP, "persistent decode kernel: a grid barrier wait exceeded its spin limit; results are invalid");
+    // The flag and the barrier counters stay as the aborted launch left them: the graph is unusable from here
+    // on and every later call reports the same error until the caller builds a new one.
+    if (flag)
+        return set_error(FK_ERR_HIP, "persistent decode kernel: a grid barrier wait exceeded its spin limit; results are "
+                                     "invalid and this graph stays unusable: rebuild it with fk_build_decode_graph");
     return FK_OK;
 }
 
@@ -1581,6 +1596,7 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
         FK_TRY(plan_dispatch(g->nodes[i].d, &g->nodes[i].launch, &g->nodes[i].rw));
     }
     derive_edges(g->nodes, barriers);
+    if (barriers) g->barriers.assign(barriers, barriers + n);
     FK_HIP(hipGraphCreate(&g->graph, 0));
     for (size_t i = 0; i < n; ++i) {
         Node& nd = g->nodes[i];
@@ -1696,7 +1712,7 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
     Graph* g;
     FK_TRY(get_graph(ds, graph_id, &g));
     if (g->persistent) return set_error(FK_ERR_UNSUPPORTED, "a persistent decode graph holds its bindings in device tables; rebuild it instead");
-    // validate all, then apply (a failed update leaves the graph untouched)
+    // validate everything first: a refused update leaves the graph untouched
     std::vector<Dispatch> patched;
     std::vector<uint32_t> touched;
     for (size_t i = 0; i < n; ++i) {
@@ -1717,16 +1733,51 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
         patched[k].args[u.slot] = fk_arg{u.ptr, u.nbytes};
     }
     std::vector<Launch> launches(touched.size());
+    std::vector<SlotRW> rws(touched.size());
     for (size_t k = 0; k < touched.size(); ++k) {
-        SlotRW rw;
-        FK_TRY(plan_dispatch(patched[k], &launches[k], &rw));
+        FK_TRY(plan_dispatch(patched[k], &launches[k], &rws[k]));
+        if (launches[k].then.size() != g->nodes[touched[k]].tail.size())
+            return set_error(FK_ERR_UNSUPPORTED, "binding update changes the number of kernels of a task");
     }
+    // The graph's edges were derived from the byte ranges of the ORIGINAL bindings.  A rebinding that makes two
+    // dispatches overlap where they did not (or stop overlapping) would need other edges: refuse it, the caller
+    // rebuilds the graph.  Compared pair by pair on the direct dependency predicate, before anything is applied.
+    {
+        auto view = [&](size_t idx, const std::vector<fk_arg>** args, const SlotRW** rw, bool patched_view) {
+            auto it = std::find(touched.begin(), touched.end(), (uint32_t)idx);
+            if (patched_view && it != touched.end()) {
+                const size_t k = (size_t)(it - touched.begin());
+                *args = &patched[k].args;
+                *rw = &rws[k];
+            } else {
+                *args = &g->nodes[idx].d.args;
+                *rw = &g->nodes[idx].rw;
+            }
+        };
+        for (uint32_t t : touched)
+            for (size_t o = 0; o < g->nodes.size(); ++o) {
+                if (o == t) continue;
+                const size_t first = o < t ? o : t, second = o < t ? t : o;
+                if (!g->barriers.empty() && g->barriers[second]) continue;  // forced edge either way
+                const std::vector<fk_arg>*a0, *b0, *a1, *b1;
+                const SlotRW *ar0, *br0, *ar1, *br1;
+                view(first, &a0, &ar0, false);
+                view(second, &b0, &br0, false);
+                view(first, &a1, &ar1, true);
+                view(second, &b1, &br1, true);
+                if (direct_dep(*a0, *ar0, *b0, *br0) != direct_dep(*a1, *ar1, *b1, *br1))
+                    return set_error(FK_ERR_UNSUPPORTED,
+                                     "binding update changes which dispatches overlap (the graph's dependency edges "
+                                     "would change); rebuild the graph with fk_build_graph");
+            }
+    }
+    // all checks passed: apply.  A HIP failure below can still leave the executable graph partly updated;
+    // the error is reported and the caller must rebuild.
     for (size_t k = 0; k < touched.size(); ++k) {
         Node& nd = g->nodes[touched[k]];
-        if (launches[k].then.size() != nd.tail.size())
-            return set_error(FK_ERR_UNSUPPORTED, "binding update changes the number of kernels of a task");
         nd.d = patched[k];
         nd.launch = launches[k];
+        nd.rw = rws[k];
         void* slot = nullptr;
         hipKernelNodeParams p = node_params(nd, &slot);
         FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.node, &p));

@@ -81,8 +81,10 @@ struct SynthArgs {
     size_t count;
     uint64_t seed;
     float mean, std;
-    uint32_t kind;  // 0: fp32 normal, 1: bf16 normal, 2: uint32 uniform in [0, bound)
+    uint32_t kind;  // 0: fp32 normal, 1: bf16 normal, 2: uint32 uniform in [0, bound); 3 / 4: see synth_exact
     uint32_t bound;
+    uint64_t row_len;  // kinds 3 / 4: elements per row for the row-norm spread (0: none)
+    float tau;
 };
 
 __device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
@@ -92,13 +94,46 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
     return z ^ (z >> 31);
 }
 
+// Kinds 3 (fp32) and 4 (bf16): values a host can reproduce bit for bit, because only integer
+// arithmetic, exact int -> float conversions and single IEEE operations are involved (no
+// transcendental function, the one multiply-add written as a fused one):
+//   z(seed, i) = (2 * S - 524280) * (1 / 107019.84), S = the sum of the eight 16-bit fields of two
+//                splitmix64 words keyed by (seed, i): mean 0, variance 1, |z| < 4.9
+//   value      = fma(std, z, mean) * rowscale(i / row_len)
+//   rowscale(j), when row_len and tau are non-zero: u = floor(tau * z(seed ^ K, j) * 8),
+//                (1 + (u & 7) / 8) * 2^(u >> 3): row norms spread like a log-normal.
+__device__ __forceinline__ float ih_normal(uint64_t seed, uint64_t i) {
+    const uint64_t r0 = splitmix64(seed * 0xD1342543DE82EF95ull + i), r1 = splitmix64(r0);
+    int32_t sum = 0;
+#pragma unroll
+    for (int f = 0; f < 4; ++f) sum += (int32_t)((r0 >> (16 * f)) & 0xFFFF) + (int32_t)((r1 >> (16 * f)) & 0xFFFF);
+    return __fmul_rn((float)(2 * sum - 524280), 9.3440616e-06f);
+}
+__device__ __forceinline__ float synth_exact(const SynthArgs& a, size_t i) {
+    float v = __fmaf_rn(a.std, ih_normal(a.seed, i), a.mean);
+    if (a.row_len && a.tau != 0.0f) {
+        const float t = floorf(__fmul_rn(__fmul_rn(a.tau, ih_normal(a.seed ^ 0x5DEECE66Dull, i / a.row_len)), 8.0f));
+        const int u = (int)t;
+        v = __fmul_rn(v, ldexpf(__fmaf_rn((float)(u & 7), 0.125f, 1.0f), u >> 3));
+    }
+    return v;
+}
+
 // Counter-based: element i depends only on (seed, i), so any launch shape gives
-// the same bytes.  Normals by Box-Muller on two 24-bit uniforms.
+// the same bytes.  Normals by Box-Muller on two 24-bit uniforms (kinds 0 / 1).
 __global__ __launch_bounds__(256) void synth_kernel(const SynthArgs a) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < a.count; i += (size_t)gridDim.x * 256) {
         const uint64_t r = splitmix64(a.seed * 0xD1342543DE82EF95ull + i);
         if (a.kind == 2) {
             reinterpret_cast<uint32_t*>(a.out)[i] = (uint32_t)(((r >> 32) * (uint64_t)a.bound) >> 32);
+            continue;
+        }
+        if (a.kind >= 3) {
+            const float e = synth_exact(a, i);
+            if (a.kind == 3)
+                reinterpret_cast<float*>(a.out)[i] = e;
+            else
+                reinterpret_cast<uint16_t*>(a.out)[i] = (uint16_t)f32_to_bf16_bits(e);
             continue;
         }
         const float u1 = ((float)((r >> 40) & 0xFFFFFF) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
@@ -113,12 +148,12 @@ __global__ __launch_bounds__(256) void synth_kernel(const SynthArgs a) {
 }
 
 fk_status plan_synth(void* out_ptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind, uint32_t bound,
-                     Launch* out) {
+                     Launch* out, uint64_t row_len, float tau) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!out_ptr || count == 0) return set_error(FK_ERR_INVALID, "synth: null pointer or zero count");
-    if (kind > 2 || (kind == 2 && bound == 0)) return set_error(FK_ERR_INVALID, "synth: bad kind or bound");
-    SynthArgs a{out_ptr, count, seed, mean, std, kind, bound};
+    if (kind > 4 || (kind == 2 && bound == 0)) return set_error(FK_ERR_INVALID, "synth: bad kind or bound");
+    SynthArgs a{out_ptr, count, seed, mean, std, kind, bound, row_len, tau};
     size_t blocks = (count + 255) / 256;
     if (blocks > (size_t)dev->cus * 16) blocks = (size_t)dev->cus * 16;
     out->func = reinterpret_cast<const void*>(&synth_kernel);

@@ -107,7 +107,13 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     // caller issued); nothing below touches it until the first K/V rows have been
     // requested, so that round trip overlaps the cache reads.
     uint32_t n_active = 0, blk_keys = 0, n_chunks = 0;
+    uint32_t pos = 0;  // fused: position of the new token
     auto settle = [&]() {
+        // a device scalar is not trusted: a length beyond what the launch was sized for would leave ranges
+        // without a block (the last-arrival count would never complete), zero would divide by an empty sum
+        const uint32_t covered = a.n_splits * span < a.capacity ? a.n_splits * span : a.capacity;
+        kv_len = kv_len < 1u ? 1u : (kv_len > covered ? covered : kv_len);
+        pos = XFORM ? kv_len - 1 : 0u;
         n_active = (kv_len + span - 1) / span;
         if (split < n_active) {
             blk_keys = (kv_len - blk0) < span ? (kv_len - blk0) : span;
@@ -126,7 +132,6 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     float* stat = red + (kSdpaBlock / a.lpv) * GT * a.v_dim;  // m[GT], l[GT], misc
     uint16_t* qn = reinterpret_cast<uint16_t*>(stat + kSdpaStatFloats);  // fused: [GT][qk_dim] + k row
     uint16_t* kn = qn + GT * a.qk_dim;
-    const uint32_t pos = XFORM ? kv_len - 1 : 0u;  // fused: position of the new token
     bool blk_owner = false;
 
     // Head norm + RoPE of this block's q heads (one wave per head), and of the new k row

@@ -44,6 +44,7 @@ class DecoderConfig:
     fuse_attention: bool = True    # graph mode, bf16 cache: rope/store + attention of a layer in one launch
     kv_bits: int = 0         # 0: bf16 KV cache; 4 / 8: quantised cache (mlx-lm QuantizedKVCache layout)
     kv_group: int = 64
+    embed_scale: float = 1.0  # output_scale of the embedding lookup (embed_lookup_decode.rs:74-99)
 
     @property
     def n_q(self) -> int:
@@ -72,7 +73,14 @@ QWEN25_05B_LIKE = dict(n_layers=24, hidden=896, n_heads=14, n_kv=2, head_dim=64,
 DENSE_4B = dict(n_layers=36, hidden=2560, n_heads=32, n_kv=8, head_dim=128, inter=9728, vocab=151936, qk_norm=True)
 
 
-def _synth(buf: DeviceBuffer, count: int, seed: int, mean: float, std: float, kind: int, bound: int = 0) -> None:
+def _synth(buf: DeviceBuffer, count: int, seed: int, mean: float, std: float, kind: int, bound: int = 0,
+           row_len: int = 0, tau: float = 0.0) -> None:
+    """kind 0 / 1: fp32 / bf16 normal, 2: uniform uint32 below `bound`; 3 / 4: fp32 / bf16 values a host can
+    reproduce bit for bit (fk_synth_fill_exact), optionally with a log-normal-like spread of the row norms."""
+    if kind >= 3:
+        check(lib.fk_synth_fill_exact(C.c_void_p(buf.ptr), C.c_size_t(count), C.c_uint64(seed), C.c_float(mean),
+                                      C.c_float(std), C.c_uint32(kind), C.c_size_t(row_len), C.c_float(tau), None))
+        return
     check(lib.fk_synth_fill(C.c_void_p(buf.ptr), C.c_size_t(count), C.c_uint64(seed), C.c_float(mean),
                             C.c_float(std), C.c_uint32(kind), C.c_uint32(bound), None))
 
@@ -100,10 +108,15 @@ class DecoderWeights:
         self.vecs: Dict[str, DeviceBuffer] = {}
 
     @classmethod
-    def random_init(cls, cfg: DecoderConfig, seed: int = 0, std: float = 0.02) -> "DecoderWeights":
+    def random_init(cls, cfg: DecoderConfig, seed: int = 0, std: float = 0.02, exact: bool = False,
+                    embed_seed: Optional[int] = None, embed_tau: float = 0.0) -> "DecoderWeights":
         """Projections ~ N(0, std^2) quantised on the device; norm weights ~ 1 + N(0, 0.1^2);
-        tied bf16 embedding ~ N(0, std^2); biases ~ N(0, 0.5^2)."""
+        tied bf16 embedding ~ N(0, std^2); biases ~ N(0, 0.5^2).
+        exact: draw every value with the host-reproducible generator (fk_synth_fill_exact), so a CPU
+        build of the same model from the same seeds holds the same bytes.  embed_seed / embed_tau
+        (exact only): own seed of the embedding, and the spread of its row norms."""
         self = cls(cfg)
+        f32_kind, bf16_kind = (3, 4) if exact else (0, 1)
         biggest = max(cfg.inter * cfg.hidden, cfg.n_q * cfg.hidden)
         tmp = DeviceBuffer(biggest * 4) if cfg.bits != 16 else None
         counter = [seed * 100003 + 1]
@@ -117,21 +130,26 @@ class DecoderWeights:
                 W = DeviceWeight.__new__(DeviceWeight)
                 W.n, W.k, W.bits, W.group = n, k, 16, 0
                 W.w, W.scales, W.biases = DeviceBuffer(n * k * 2), None, None
-                _synth(W.w, n * k, next_seed(), 0.0, std, 1)
+                _synth(W.w, n * k, next_seed(), 0.0, std, bf16_kind)
             else:
-                _synth(tmp, n * k, next_seed(), 0.0, std, 0)
+                _synth(tmp, n * k, next_seed(), 0.0, std, f32_kind)
                 W = quantize_on_device(tmp, n, k, cfg.bits, cfg.group)
             self.mats[name] = W
 
         def vector(name: str, n: int, mean: float, sd: float) -> None:
             b = DeviceBuffer(n * 2)
-            _synth(b, n, next_seed(), mean, sd, 1)
+            _synth(b, n, next_seed(), mean, sd, bf16_kind)
             self.vecs[name] = b
 
         emb = DeviceWeight.__new__(DeviceWeight)
         emb.n, emb.k, emb.bits, emb.group = cfg.vocab, cfg.hidden, 16, 0
         emb.w, emb.scales, emb.biases = DeviceBuffer(cfg.vocab * cfg.hidden * 2), None, None
-        _synth(emb.w, cfg.vocab * cfg.hidden, next_seed(), 0.0, std, 1)
+        es = next_seed()
+        if exact:
+            _synth(emb.w, cfg.vocab * cfg.hidden, es if embed_seed is None else embed_seed, 0.0, std, 4,
+                   row_len=cfg.hidden, tau=embed_tau)
+        else:
+            _synth(emb.w, cfg.vocab * cfg.hidden, es, 0.0, std, 1)
         self.mats["embed_tokens"] = emb
         vector("final_norm", cfg.hidden, 1.0, 0.1)
         for l in range(cfg.n_layers):
@@ -221,7 +239,8 @@ class DecoderRuntime:
         emb = w.mats["embed_tokens"]       # dense bf16 or MLX-affine (4-bit checkpoints quantise it too)
         head = w.mats.get("lm_head", emb)  # untied output projection when the checkpoint has one
         t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token)] + self._wargs(emb) + [arg(self.x[0])],
-                          dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
+                          dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab,
+                               output_scale=c.embed_scale)))
         for l in range(c.n_layers):
             p = f"layers.{l}."
             Wq, Wk, Wv = (w.mats[p + f"self_attn.{n}_proj"] for n in "qkv")
@@ -378,7 +397,7 @@ class DecoderRuntime:
             chunk = prompt[pos - start_offset: pos - start_offset + R]
             m = len(chunk)
             b["tok"].upload(np.asarray(chunk, np.uint32))
-            native.embed_lookup_rows(emb, b["tok"], m, 1.0, b["x"])
+            native.embed_lookup_rows(emb, b["tok"], m, c.embed_scale, b["x"])
             native.rope_table_rows(b["rope"], c.head_dim, c.theta, pos, m)  # once per pass, for every layer and head
             for l in range(c.n_layers):
                 p = f"layers.{l}."

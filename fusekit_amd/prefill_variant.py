@@ -74,7 +74,7 @@ class PrefillVariant:
         emb = w.mats["embed_tokens"]
         head = w.mats.get("lm_head", emb)
         t.append(Dispatch(name("embed_lookup_decode"), [arg(self.tokens)] + rt._wargs(emb) + [arg(self.x[0])],
-                          dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0, rows=m)))
+                          dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab, output_scale=c.embed_scale, rows=m)))
         for l in range(c.n_layers):
             p = f"layers.{l}."
             t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(self.xn)],

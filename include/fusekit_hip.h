@@ -237,6 +237,15 @@ fk_status fk_quantize_affine(const float *d_w, size_t n, size_t k, uint32_t bits
  * kind 0: fp32 N(mean, std^2); 1: bf16 N(mean, std^2); 2: uint32 uniform in [0, bound). */
 fk_status fk_synth_fill(void *dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind,
                         uint32_t bound, fk_stream s);
+/* The same for values a host can reproduce bit for bit (parity tests build the very model on the
+ * CPU): kind 3 fp32, kind 4 bf16; value = fma(std, z, mean) with z a sum of eight 16-bit uniform
+ * integers, centred and scaled to unit variance (integer arithmetic and single IEEE operations
+ * only).  With row_len and tau non-zero every row of row_len elements is multiplied by
+ * (1 + (u & 7) / 8) * 2^(u >> 3), u = floor(8 * tau * z_row): row norms spread like a log-normal,
+ * which gives a tied embedding / LM head the peaked logits of a trained model.  Like
+ * fk_synth_fill this has no counterpart in the reference, which loads real checkpoints. */
+fk_status fk_synth_fill_exact(void *dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind,
+                              size_t row_len, float tau, fk_stream s);
 
 /* Per-token scalars (rotary position, cache row, KV length) come either from a
  * device scalar `d_*` (so a captured hipGraph can be replayed while a step

@@ -62,7 +62,9 @@
  * Conventions: activations "T" are bfloat16 held as uint16_t bit patterns;
  * every T(...) in the reference is a round-to-nearest-even fp32->bf16 here.
  * Dot products accumulate in double and are narrowed to float once, so the
- * oracle is the closest fp32 value any summation order may aim for.
+ * oracle is the closest fp32 value any summation order may aim for; two fp32
+ * summation orders of the projections can be switched on (fko_set_accum_mode)
+ * to measure the envelope fp32 arithmetic leaves around those values.
  */
 #include <math.h>
 #include <stdint.h>
@@ -192,6 +194,48 @@ FKO_API void fko_dequantize(const uint32_t *packed, const uint16_t *scales, cons
         }
 }
 
+/* ------------------------------------------------ seeded synthetic data */
+/*
+ * Test-data generator that the GPU library's synthetic fill (kinds 3 / 4) reproduces bit for bit:
+ * only integer arithmetic, exact int -> float conversions and single IEEE operations (one fused
+ * multiply-add, written as such on both sides), so a model instantiated in HBM and one built on
+ * the host from the same seeds hold the same bytes.  Not part of the reference: it replaces
+ * "weights drawn N(0, 0.02^2) from a seed" (MLX's generator cannot run here).
+ *   z(seed, i) = (2 * S - 524280) * (1 / 107019.84),  S = sum of eight 16-bit fields of two
+ *                splitmix64 words keyed by (seed, i): mean 0, variance 1, |z| < 4.9
+ *   value      = fma(std, z, mean) * rowscale(i / row_len)
+ *   rowscale(j) (row_len != 0 and tau != 0): u = floor(tau * z(seed ^ K, j) * 8),
+ *                rowscale = (1 + (u & 7) / 8) * 2^(u >> 3): a log-normal-like spread of row norms
+ */
+static inline uint64_t splitmix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static inline float ih_normal(uint64_t seed, uint64_t i) {
+    const uint64_t r0 = splitmix64(seed * 0xD1342543DE82EF95ull + i), r1 = splitmix64(r0);
+    int32_t sum = 0;
+    for (int f = 0; f < 4; ++f) sum += (int32_t)((r0 >> (16 * f)) & 0xFFFF) + (int32_t)((r1 >> (16 * f)) & 0xFFFF);
+    return (float)(2 * sum - 524280) * 9.3440616e-06f;
+}
+static inline float row_scale(uint64_t seed, uint64_t row, float tau) {
+    const float t = floorf((tau * ih_normal(seed ^ 0x5DEECE66Dull, row)) * 8.0f);
+    const int u = (int)t;
+    return ldexpf(1.0f + (float)(u & 7) * 0.125f, u >> 3);
+}
+/* kind 3: fp32 out, kind 4: bf16 out */
+FKO_API void fko_synth_fill(void *out, int64_t count, uint64_t seed, float mean, float std, int kind,
+                            int64_t row_len, float tau) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < count; ++i) {
+        float v = fmaf(std, ih_normal(seed, (uint64_t)i), mean);
+        if (row_len && tau != 0.0f) v = v * row_scale(seed, (uint64_t)(i / row_len), tau);
+        if (kind == 3) ((float *)out)[i] = v;
+        else ((uint16_t *)out)[i] = f32_to_bf16(v);
+    }
+}
+
 /* --------------------------------------------------------- K1: linear */
 /*
  * One weight matrix [n, k] in one of three storage kinds:
@@ -206,20 +250,54 @@ typedef struct {
     int bits, group;
 } fko_weight;
 
+/* Accumulation mode of every projection (linear_acc), process-wide; tests switch it to measure how far fp32
+ * summation orders -- which the reference's own kernels use -- sit from the double sums:
+ *   0  double accumulation, narrowed to float once (default: the value any fp32 order aims for)
+ *   1  fp32, the per-element form in element order: acc += x[k] * (q*s + b)
+ *      (src/codegen/kernels/mod.rs:2850-2908 read literally, one accumulator)
+ *   2  fp32, the qdot form per quantisation group, acc += s * sum(x*q) + b * sum(x), groups in order
+ *      (src/codegen/kernels/mod.rs:2634-2713); dense rows: 32 interleaved partial sums added as a
+ *      simdgroup sum does (pairwise tree), src/codegen/msl.rs:310-440 */
+static int g_accum_mode = 0;
+FKO_API void fko_set_accum_mode(int mode) { g_accum_mode = mode; }
+FKO_API int fko_get_accum_mode(void) { return g_accum_mode; }
+
+static inline uint32_t code_at(const uint32_t *prow, int64_t j, int bits, int per_word, uint32_t mask) {
+    return (prow[j / per_word] >> ((j % per_word) * bits)) & mask;
+}
+
 /* acc[i] = sum_k x[k] * (q*s + b), the per-element form of
  * src/codegen/kernels/mod.rs:2850-2908 (q4) and :3053-3104 (q8); dense rows
  * as src/codegen/kernels/linear_residual.rs:342-346.  x is fp32 holding values
- * the caller already rounded to T where the reference does. */
+ * the caller already rounded to T where the reference does.  Mode 0 keeps four
+ * double accumulators (elements j = 0..3 mod 4), added (a0 + a1) + (a2 + a3). */
 static void linear_acc(const fko_weight *W, const float *x, float *acc) {
     const int64_t n = W->n, k = W->k;
+    const int mode = g_accum_mode;
     if (W->bits == 16) {
         const uint16_t *d = (const uint16_t *)W->w;
 #pragma omp parallel for schedule(static)
         for (int64_t r = 0; r < n; ++r) {
-            double a = 0.0;
             const uint16_t *row = d + r * k;
-            for (int64_t j = 0; j < k; ++j) a += (double)x[j] * (double)bf16_to_f32(row[j]);
-            acc[r] = (float)a;
+            if (mode == 0) {
+                double a[4] = {0.0, 0.0, 0.0, 0.0};
+                int64_t j = 0;
+                for (; j + 4 <= k; j += 4)
+                    for (int e = 0; e < 4; ++e) a[e] += (double)x[j + e] * (double)bf16_to_f32(row[j + e]);
+                for (; j < k; ++j) a[0] += (double)x[j] * (double)bf16_to_f32(row[j]);
+                acc[r] = (float)((a[0] + a[1]) + (a[2] + a[3]));
+            } else if (mode == 1) {
+                float a = 0.0f;
+                for (int64_t j = 0; j < k; ++j) a += x[j] * bf16_to_f32(row[j]);
+                acc[r] = a;
+            } else {
+                float lane[32];
+                for (int i = 0; i < 32; ++i) lane[i] = 0.0f;
+                for (int64_t j = 0; j < k; ++j) lane[j & 31] += x[j] * bf16_to_f32(row[j]);
+                for (int w = 16; w >= 1; w >>= 1)
+                    for (int i = 0; i < w; ++i) lane[i] += lane[i + w];
+                acc[r] = lane[0];
+            }
         }
         return;
     }
@@ -229,19 +307,54 @@ static void linear_acc(const fko_weight *W, const float *x, float *acc) {
     const uint32_t *p = (const uint32_t *)W->w;
 #pragma omp parallel for schedule(static)
     for (int64_t r = 0; r < n; ++r) {
-        double a = 0.0;
         const uint32_t *prow = p + r * words;
-        for (int64_t g = 0; g < groups; ++g) {
-            const float s = bf16_to_f32(W->scales[r * groups + g]);
-            const float b = bf16_to_f32(W->biases[r * groups + g]);
-            for (int i = 0; i < group; ++i) {
-                int64_t j = g * group + i;
-                uint32_t q = (prow[j / per_word] >> ((j % per_word) * bits)) & mask;
-                float wv = (float)q * s + b; /* fp32 dequant as in the reference */
-                a += (double)x[j] * (double)wv;
+        if (mode == 0) {
+            double a[4] = {0.0, 0.0, 0.0, 0.0};
+            float wv[128];
+            for (int64_t g = 0; g < groups; ++g) {
+                const float s = bf16_to_f32(W->scales[r * groups + g]);
+                const float b = bf16_to_f32(W->biases[r * groups + g]);
+                const float *xg = x + g * group;
+                const uint32_t *pw = prow + g * (group / per_word);
+                /* fp32 dequant as in the reference: float(q) * s + b, two roundings */
+                if (bits == 4) {
+                    for (int w = 0; w < group / 8; ++w)
+                        for (int e = 0; e < 8; ++e) wv[w * 8 + e] = (float)((pw[w] >> (4 * e)) & 15u) * s + b;
+                } else {
+                    for (int w = 0; w < group / 4; ++w)
+                        for (int e = 0; e < 4; ++e) wv[w * 4 + e] = (float)((pw[w] >> (8 * e)) & 255u) * s + b;
+                }
+                for (int i = 0; i < group; i += 4)
+                    for (int e = 0; e < 4; ++e) a[e] += (double)xg[i + e] * (double)wv[i + e];
             }
+            acc[r] = (float)((a[0] + a[1]) + (a[2] + a[3]));
+        } else if (mode == 1) {
+            float a = 0.0f;
+            for (int64_t g = 0; g < groups; ++g) {
+                const float s = bf16_to_f32(W->scales[r * groups + g]);
+                const float b = bf16_to_f32(W->biases[r * groups + g]);
+                for (int i = 0; i < group; ++i) {
+                    const int64_t j = g * group + i;
+                    const float wvj = (float)code_at(prow, j, bits, per_word, mask) * s + b;
+                    a += x[j] * wvj;
+                }
+            }
+            acc[r] = a;
+        } else {
+            float a = 0.0f;
+            for (int64_t g = 0; g < groups; ++g) {
+                const float s = bf16_to_f32(W->scales[r * groups + g]);
+                const float b = bf16_to_f32(W->biases[r * groups + g]);
+                float dq = 0.0f, sx = 0.0f;
+                for (int i = 0; i < group; ++i) {
+                    const int64_t j = g * group + i;
+                    dq += x[j] * (float)code_at(prow, j, bits, per_word, mask);
+                    sx += x[j];
+                }
+                a += s * dq + b * sx;
+            }
+            acc[r] = a;
         }
-        acc[r] = (float)a;
     }
 }
 

@@ -46,8 +46,67 @@ def to_device(fk, W: oracle.QWeight):
 
 
 # ---------------------------------------------------------------- whole-model oracle
+class HostDecoderWeights:
+    """A dense decoder's weights built on the HOST with the oracle's copy of the library's
+    host-reproducible generator and the oracle's quantiser: the bytes
+    `DecoderWeights.random_init(cfg, seed, exact=True, ...)` puts into HBM (same seed sequence)."""
+
+    def __init__(self, cfg, seed: int = 0, std: float = 0.02, embed_seed=None, embed_tau: float = 0.0,
+                 with_embedding: bool = True):
+        self.cfg = cfg
+        self.mats, self.vecs = {}, {}
+        self.std = std
+        counter = [seed * 100003 + 1]
+
+        def next_seed():
+            counter[0] += 1
+            return counter[0]
+
+        def matrix(name, n, k):
+            sd = next_seed()
+            if cfg.bits == 16:
+                self.mats[name] = oracle.dense(oracle.synth_fill(n * k, sd, 0.0, std, 4).reshape(n, k))
+            else:
+                self.mats[name] = oracle.quantize(oracle.synth_fill(n * k, sd, 0.0, std, 3).reshape(n, k), cfg.bits, cfg.group)
+
+        def vector(name, n, mean, sd_):
+            self.vecs[name] = oracle.synth_fill(n, next_seed(), mean, sd_, 4)
+
+        es = next_seed()
+        self.embed_seed = es if embed_seed is None else embed_seed
+        if with_embedding:
+            self.set_embedding(self.embed_seed, embed_tau)
+        vector("final_norm", cfg.hidden, 1.0, 0.1)
+        for l in range(cfg.n_layers):
+            p = f"layers.{l}."
+            matrix(p + "self_attn.q_proj", cfg.n_q, cfg.hidden)
+            matrix(p + "self_attn.k_proj", cfg.n_kvd, cfg.hidden)
+            matrix(p + "self_attn.v_proj", cfg.n_kvd, cfg.hidden)
+            matrix(p + "self_attn.o_proj", cfg.hidden, cfg.n_q)
+            matrix(p + "mlp.gate_proj", cfg.inter, cfg.hidden)
+            matrix(p + "mlp.up_proj", cfg.inter, cfg.hidden)
+            matrix(p + "mlp.down_proj", cfg.hidden, cfg.inter)
+            vector(p + "input_layernorm", cfg.hidden, 1.0, 0.1)
+            vector(p + "post_attention_layernorm", cfg.hidden, 1.0, 0.1)
+            if cfg.qk_norm:
+                vector(p + "self_attn.q_norm", cfg.head_dim, 1.0, 0.1)
+                vector(p + "self_attn.k_norm", cfg.head_dim, 1.0, 0.1)
+            if cfg.qkv_bias:
+                vector(p + "self_attn.q_proj.bias", cfg.n_q, 0.0, 0.5)
+                vector(p + "self_attn.k_proj.bias", cfg.n_kvd, 0.0, 0.5)
+                vector(p + "self_attn.v_proj.bias", cfg.n_kvd, 0.0, 0.5)
+
+    def set_embedding(self, embed_seed: int, embed_tau: float) -> None:
+        c = self.cfg
+        self.mats["embed_tokens"] = oracle.dense(
+            oracle.synth_fill(c.vocab * c.hidden, embed_seed, 0.0, self.std, 4, row_len=c.hidden, tau=embed_tau)
+            .reshape(c.vocab, c.hidden))
+
+
 def host_weight(dw) -> oracle.QWeight:
-    """Download a fusekit_amd DeviceWeight into an oracle QWeight."""
+    """Download a fusekit_amd DeviceWeight into an oracle QWeight (host weights pass through)."""
+    if isinstance(dw, oracle.QWeight):
+        return dw
     if dw.bits == 16:
         return oracle.dense(dw.w.to_numpy(np.uint16, (dw.n, dw.k)))
     per = 32 // dw.bits
@@ -66,7 +125,8 @@ class OracleDecoder:
         u16p = C.POINTER(C.c_uint16)
 
         def vec(name):
-            a = weights.vecs[name].to_numpy(np.uint16)
+            a = weights.vecs[name]
+            a = a if isinstance(a, np.ndarray) else a.to_numpy(np.uint16)
             self.keep.append(a)
             return a.ctypes.data_as(u16p)
 
@@ -105,7 +165,7 @@ class OracleDecoder:
         emb = mat("embed_tokens")
         head = mat("lm_head") if "lm_head" in weights.mats else emb
         self.model = oracle.Model(cfg.n_layers, cfg.hidden, cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab,
-                                  cfg.eps, cfg.theta, 1.0 / np.sqrt(cfg.head_dim), 1.0, cfg.swiglu_variant,
+                                  cfg.eps, cfg.theta, 1.0 / np.sqrt(cfg.head_dim), getattr(cfg, "embed_scale", 1.0), cfg.swiglu_variant,
                                   cfg.capacity, emb, head, vec("final_norm"), self.layers,
                                   getattr(cfg, "kv_bits", 0), getattr(cfg, "kv_group", 64))
 
