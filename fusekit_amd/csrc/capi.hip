@@ -6,6 +6,7 @@
 #include <mutex>
 
 #include "fk_host.hpp"
+#include "xcd_layer.hpp"
 
 namespace fk {
 
@@ -700,6 +701,33 @@ fk_status fk_synth_fill_exact(void* dptr, size_t count, uint64_t seed, float mea
     Launch l;
     FK_TRY(plan_synth(dptr, count, seed, mean, std, kind, 0, &l, row_len, tau));
     return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_xcd_layer_supported(uint32_t hidden, uint32_t inter, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                 uint32_t capacity, uint32_t bits, uint32_t group) {
+    return xcd_layer_supported(XcdLayerShape{hidden, inter, n_heads, n_kv, head_dim, capacity, bits, group});
+}
+
+fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t* control_bytes, size_t* attention_partial_bytes) {
+    if (!control_bytes || !attention_partial_bytes) return set_error(FK_ERR_INVALID, "fk_xcd_workspace_bytes: null out");
+    XcdLayerShape s{};
+    s.n_heads = n_heads;
+    s.head_dim = head_dim;
+    *control_bytes = xcd_workspace_bytes();
+    *attention_partial_bytes = xcd_attn_partials_bytes(s);
+    return FK_OK;
+}
+
+fk_status fk_xcd_check(void* workspace, fk_stream s) {
+    if (!workspace) return set_error(FK_ERR_INVALID, "fk_xcd_check: null workspace");
+    FK_HIP(hipStreamSynchronize((hipStream_t)s));
+    XcdControl* c = reinterpret_cast<XcdControl*>(workspace);
+    uint32_t flag = 0;
+    FK_HIP(hipMemcpy(&flag, &c->abort_flag, 4, hipMemcpyDeviceToHost));
+    if (!flag) return FK_OK;
+    // the arrival words of an aborted launch are inconsistent: start over from zero
+    FK_HIP(hipMemset(workspace, 0, sizeof(XcdControl)));
+    return set_error(FK_ERR_HIP, "xcd layer: a hand-over wait exceeded its spin limit; results are invalid (the workspace was reset)");
 }
 
 }  // extern "C"

@@ -26,6 +26,7 @@
 #include "decode_token.hpp"
 #include "fk_host.hpp"
 #include "fk_json.hpp"
+#include "xcd_layer.hpp"
 
 namespace fk {
 namespace {
@@ -620,6 +621,167 @@ fk_status plan_rope_store_sdpa(const Dispatch& d, Launch* l, SlotRW* rw) {
                             arg_ptr<float>(d, c0 + 4), arg_ptr<uint32_t>(d, c0 + 5), l, 1, nullptr, &f);
 }
 
+// ---- XCD-resident layer (xcd_layer.hpp): two launches per layer -------------------------------------
+XcdLayerShape xcd_shape(const Dispatch& d) {
+    XcdLayerShape s;
+    s.hidden = d.u("hidden");
+    s.inter = d.u("inter");
+    s.n_heads = d.u("n_heads");
+    s.n_kv = d.u("n_kv");
+    s.head_dim = d.u("head_dim");
+    s.capacity = d.u("capacity");
+    s.bits = d.u("bits", 4);
+    s.group = d.u("group", 64);
+    return s;
+}
+
+// [partials_in], residual, x_out, norm_w, W_q, W_k, W_v, [s_q, s_k, s_v, b_q, b_k, b_v], W_o, [s_o, b_o],
+// [q_norm, k_norm], q, k, v, cache_k, cache_v, kv_len, rope_tab, att_partials, out_partials, workspace
+// Parameters: the layer shape (hidden, inter, n_heads, n_kv, head_dim, capacity, bits, group), eps, theta,
+// has_partials, has_norm, residual_per_xcd, spin_limit.
+fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const XcdLayerShape s = xcd_shape(d);
+    const bool has_p = d.u("has_partials", 1) != 0, norm = d.u("has_norm", 0) != 0, q = s.bits != 16;
+    size_t i = 0;
+    const size_t p_slot = has_p ? i++ : 0, res_slot = i++, x_slot = i++, nw_slot = i++, w_slot = i;
+    i += 3;
+    const size_t meta_slot = i;
+    if (q) i += 6;
+    const size_t wo_slot = i++;
+    const size_t wo_meta = i;
+    if (q) i += 2;
+    const size_t hn_slot = i;
+    if (norm) i += 2;
+    const size_t q_slot = i;
+    i += 3;
+    const size_t ck_slot = i++, cv_slot = i++, len_slot = i++, tab_slot = i++, ap_slot = i++, op_slot = i++, ws_slot = i++;
+    FK_TRY(need_args(d, i));
+    if (s.hidden == 0 || s.n_heads == 0 || s.n_kv == 0 || s.head_dim == 0 || s.capacity == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": layer shape parameters missing");
+    const uint32_t n_q = s.n_heads * s.head_dim, n_kvd = s.n_kv * s.head_dim;
+    XcdAttnRequest rq;
+    memset(&rq, 0, sizeof(rq));
+    rq.shape = s;
+    const bool per_xcd = d.u("residual_per_xcd", 0) != 0;
+    if (has_p) {
+        FK_TRY(need_bytes(d, p_slot, (size_t)kXcds * s.hidden * 4));
+        rq.partials_in = arg_ptr<const float>(d, p_slot);
+    }
+    FK_TRY(need_bytes(d, res_slot, (size_t)(per_xcd ? kXcds : 1) * s.hidden * 2));
+    FK_TRY(need_bytes(d, x_slot, (size_t)kXcds * s.hidden * 2));
+    FK_TRY(need_bytes(d, nw_slot, (size_t)s.hidden * 2));
+    rq.residual = arg_ptr<const uint16_t>(d, res_slot);
+    rq.residual_stride = per_xcd ? s.hidden : 0;
+    rq.x_out = arg_ptr<uint16_t>(d, x_slot);
+    rq.norm_w = arg_ptr<const uint16_t>(d, nw_slot);
+    rq.eps = (float)d.param("eps", 1e-6);
+    fk_weight W[4];
+    const uint32_t ns[3] = {n_q, n_kvd, n_kvd};
+    for (int m = 0; m < 3; ++m)
+        FK_TRY(bind_weight(d, s.bits, s.group, ns[m], s.hidden, w_slot + m, meta_slot + m, meta_slot + 3 + m, &W[m]));
+    FK_TRY(bind_weight(d, s.bits, s.group, s.hidden, n_q, wo_slot, wo_meta, wo_meta + 1, &W[3]));
+    rq.wq = &W[0];
+    rq.wk = &W[1];
+    rq.wv = &W[2];
+    rq.wo = &W[3];
+    if (norm) {
+        FK_TRY(need_bytes(d, hn_slot, (size_t)s.head_dim * 2));
+        FK_TRY(need_bytes(d, hn_slot + 1, (size_t)s.head_dim * 2));
+        rq.q_norm = arg_ptr<const uint16_t>(d, hn_slot);
+        rq.k_norm = arg_ptr<const uint16_t>(d, hn_slot + 1);
+    }
+    FK_TRY(need_bytes(d, q_slot, (size_t)n_q * 2));
+    FK_TRY(need_bytes(d, q_slot + 1, (size_t)n_kvd * 2));
+    FK_TRY(need_bytes(d, q_slot + 2, (size_t)n_kvd * 2));
+    rq.q = arg_ptr<uint16_t>(d, q_slot);
+    rq.k = arg_ptr<uint16_t>(d, q_slot + 1);
+    rq.v = arg_ptr<uint16_t>(d, q_slot + 2);
+    FK_TRY(need_bytes(d, ck_slot, (size_t)s.n_kv * s.capacity * s.head_dim * 2));
+    FK_TRY(need_bytes(d, cv_slot, (size_t)s.n_kv * s.capacity * s.head_dim * 2));
+    rq.cache_k = arg_ptr<uint16_t>(d, ck_slot);
+    rq.cache_v = arg_ptr<uint16_t>(d, cv_slot);
+    FK_TRY(need_bytes(d, len_slot, 4));
+    rq.kv_len = arg_ptr<const uint32_t>(d, len_slot);
+    FK_TRY(need_bytes(d, tab_slot, (size_t)s.head_dim * 4));
+    rq.rope_tab = arg_ptr<const float>(d, tab_slot);
+    rq.theta = (float)d.param("theta", 10000.0);
+    FK_TRY(need_bytes(d, ap_slot, xcd_attn_partials_bytes(s)));
+    rq.att_partials = arg_ptr<float>(d, ap_slot);
+    FK_TRY(need_bytes(d, op_slot, (size_t)kXcds * s.hidden * 4));
+    rq.out_partials = arg_ptr<float>(d, op_slot);
+    FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
+    rq.workspace = d.args[ws_slot].ptr;
+    rq.spin_limit = d.u("spin_limit", 0);
+    for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
+    rw->writes = {(uint32_t)x_slot, (uint32_t)q_slot, (uint32_t)q_slot + 1, (uint32_t)q_slot + 2, (uint32_t)ck_slot,
+                  (uint32_t)cv_slot, (uint32_t)ap_slot, (uint32_t)op_slot, (uint32_t)ws_slot};
+    return plan_xcd_attn(rq, l);
+}
+
+// [partials_in], residual, x_out, norm_w, W_gate, W_up, [s_g, s_u, b_g, b_u], W_down, [s_d, b_d], mid, out_partials, workspace
+fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const XcdLayerShape s = xcd_shape(d);
+    const bool has_p = d.u("has_partials", 1) != 0, q = s.bits != 16;
+    size_t i = 0;
+    const size_t p_slot = has_p ? i++ : 0, res_slot = i++, x_slot = i++, nw_slot = i++, w_slot = i;
+    i += 2;
+    const size_t meta_slot = i;
+    if (q) i += 4;
+    const size_t wd_slot = i++;
+    const size_t wd_meta = i;
+    if (q) i += 2;
+    const size_t mid_slot = i++, op_slot = i++, ws_slot = i++;
+    FK_TRY(need_args(d, i));
+    if (s.hidden == 0 || s.inter == 0) return set_error(FK_ERR_INVALID, d.kernel + ": layer shape parameters missing");
+    XcdMlpRequest rq;
+    memset(&rq, 0, sizeof(rq));
+    rq.shape = s;
+    const bool per_xcd = d.u("residual_per_xcd", 0) != 0;
+    if (has_p) {
+        FK_TRY(need_bytes(d, p_slot, (size_t)kXcds * s.hidden * 4));
+        rq.partials_in = arg_ptr<const float>(d, p_slot);
+    }
+    FK_TRY(need_bytes(d, res_slot, (size_t)(per_xcd ? kXcds : 1) * s.hidden * 2));
+    FK_TRY(need_bytes(d, x_slot, (size_t)kXcds * s.hidden * 2));
+    FK_TRY(need_bytes(d, nw_slot, (size_t)s.hidden * 2));
+    rq.residual = arg_ptr<const uint16_t>(d, res_slot);
+    rq.residual_stride = per_xcd ? s.hidden : 0;
+    rq.x_out = arg_ptr<uint16_t>(d, x_slot);
+    rq.norm_w = arg_ptr<const uint16_t>(d, nw_slot);
+    rq.eps = (float)d.param("eps", 1e-6);
+    fk_weight W[3];
+    for (int m = 0; m < 2; ++m)
+        FK_TRY(bind_weight(d, s.bits, s.group, s.inter, s.hidden, w_slot + m, meta_slot + m, meta_slot + 2 + m, &W[m]));
+    FK_TRY(bind_weight(d, s.bits, s.group, s.hidden, s.inter, wd_slot, wd_meta, wd_meta + 1, &W[2]));
+    rq.wgate = &W[0];
+    rq.wup = &W[1];
+    rq.wdown = &W[2];
+    rq.swiglu_variant = (int)d.param("variant", 0);
+    FK_TRY(need_bytes(d, mid_slot, (size_t)s.inter * 2));
+    rq.mid = arg_ptr<uint16_t>(d, mid_slot);
+    FK_TRY(need_bytes(d, op_slot, (size_t)kXcds * s.hidden * 4));
+    rq.out_partials = arg_ptr<float>(d, op_slot);
+    FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
+    rq.workspace = d.args[ws_slot].ptr;
+    rq.spin_limit = d.u("spin_limit", 0);
+    for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
+    rw->writes = {(uint32_t)x_slot, (uint32_t)mid_slot, (uint32_t)op_slot, (uint32_t)ws_slot};
+    return plan_xcd_mlp(rq, l);
+}
+
+// partials [8][hidden] fp32, residual [hidden] bf16, x [hidden] bf16 (parameter hidden)
+fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 3));
+    const uint32_t hidden = d.u("hidden");
+    if (hidden == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden parameter missing");
+    FK_TRY(need_bytes(d, 0, (size_t)kXcds * hidden * 4));
+    FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, 2, (size_t)hidden * 2));
+    rw->reads = {0, 1};
+    rw->writes = {2};
+    return plan_xcd_reduce(arg_ptr<const float>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<uint16_t>(d, 2), hidden, l);
+}
+
 // Q, K0, K1, V, cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]: split-key store + attention of a
 // layer in one launch.  Parameters as the split form of kv_cache_store_decode (n_heads, q0_dim, q1_dim, n_kv,
 // v_dim, k1_n_kv, k0_stride, v_stride, rope_dims, traditional, theta, capacity) plus max_len, scale, has_table.
@@ -1011,6 +1173,9 @@ const Family kFamilies[] = {
     {"fusekit_sdpa_decode_q4", [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_sdpa_quant_d(d, l, rw, 4); }},
     {"fusekit_sdpa_decode_q8", [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_sdpa_quant_d(d, l, rw, 8); }},
     {"fusekit_argmax_logits_decode", plan_argmax_d},
+    {"fusekit_xcd_attn_block", plan_xcd_attn_d},
+    {"fusekit_xcd_mlp_block", plan_xcd_mlp_d},
+    {"fusekit_xcd_reduce", plan_xcd_reduce_d},
 };
 
 const Family* find_family(const std::string& kernel) {
@@ -1069,6 +1234,7 @@ struct Graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     std::vector<uint8_t> barriers;  // as given to fk_build_graph (empty: none forced)
+    std::vector<void*> xcd_controls;  // control blocks of XCD-resident launches in this graph (abort words)
     // persistent whole-token mode: one kernel node; device-side tables it reads
     bool persistent = false;
     Launch token_launch;
@@ -1451,6 +1617,16 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
 }
 
 fk_status check_abort(Graph* g) {
+    for (void* ws : g->xcd_controls) {
+        uint32_t flag = 0;
+        XcdControl* c = reinterpret_cast<XcdControl*>(ws);
+        FK_HIP(hipMemcpy(&flag, &c->abort_flag, 4, hipMemcpyDeviceToHost));
+        if (flag) {
+            // the arrival words of an aborted launch are inconsistent: start over from zero
+            FK_HIP(hipMemset(ws, 0, sizeof(XcdControl)));
+            return set_error(FK_ERR_HIP, "xcd layer: a hand-over wait exceeded its spin limit; results are invalid (the control block was reset)");
+        }
+    }
     if (!g->persistent) return FK_OK;
     uint32_t flag = 0;
     FK_HIP(hipMemcpy(&flag, g->d_abort, 4, hipMemcpyDeviceToHost));
@@ -1597,6 +1773,13 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
     }
     derive_edges(g->nodes, barriers);
     if (barriers) g->barriers.assign(barriers, barriers + n);
+    for (size_t i = 0; i < n; ++i) {
+        const Node& nd = g->nodes[i];
+        if (nd.d.kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || nd.d.kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0) {
+            void* ws = nd.d.args.back().ptr;
+            if (std::find(g->xcd_controls.begin(), g->xcd_controls.end(), ws) == g->xcd_controls.end()) g->xcd_controls.push_back(ws);
+        }
+    }
     FK_HIP(hipGraphCreate(&g->graph, 0));
     for (size_t i = 0; i < n; ++i) {
         Node& nd = g->nodes[i];

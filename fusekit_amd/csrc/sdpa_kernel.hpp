@@ -86,7 +86,9 @@ __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk,
 // the cache row and appends both to the cache.
 // FASTHEAD (mode 2): heads rotated over their whole width of at most 128 dims with a rotary table;
 // the transforms' loads are issued ahead of the cache rows and used after them.
-template <int GT, int MODE, typename ARGS, int KVQ = 0, bool FASTHEAD = false>
+// NOMERGE: the caller merges the ranges' results itself: every active block writes its (m, l, o) partial with
+// ordinary stores -- also when one range covers the context -- and returns; no arrival counter is touched.
+template <int GT, int MODE, typename ARGS, int KVQ = 0, bool FASTHEAD = false, bool NOMERGE = false>
 __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
                                            uint32_t gz, uint32_t gz_count, float* lds) {
     constexpr bool FUSED = MODE == 1;   // inside the whole-token kernel
@@ -649,7 +651,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 
     FK_SDPA_STAMP(6);
     const uint32_t n_out = gcount * a.v_dim;
-    const bool direct = (n_active == 1);
+    const bool direct = !NOMERGE && (n_active == 1);
     for (uint32_t e = tid; e < n_out; e += kSdpaBlock) {
         const uint32_t h = e / a.v_dim, d = e - h * a.v_dim;
         float o = 0.f;
@@ -658,15 +660,15 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
             st_u16<FUSED>(a.out + (size_t)(h0 + h) * a.v_dim + d, f32_to_bf16_bits(o / stat[8 + h]));
         } else {
             float* p = a.partials + ((size_t)(h0 + h) * a.n_splits + split) * (a.v_dim + 2);
-            st_f32<true>(p + 2 + d, o);
+            st_f32<!NOMERGE>(p + 2 + d, o);
             if (d == 0) {
-                st_f32<true>(p, stat[h]);
-                st_f32<true>(p + 1, stat[8 + h]);
+                st_f32<!NOMERGE>(p, stat[h]);
+                st_f32<!NOMERGE>(p + 1, stat[8 + h]);
             }
         }
     }
     FK_SDPA_STAMP(7);
-    if (direct) return;
+    if (direct || NOMERGE) return;
 
     // ---------------- last block merges the partials ----------------
     // Partials and the arrival counter move through agent-scope (write-through /

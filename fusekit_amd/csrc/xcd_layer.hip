@@ -1,0 +1,723 @@
+// XCD-resident decoder layer: the attention launch and the MLP launch (see xcd_layer.hpp for the scheme).
+#include "xcd_layer.hpp"
+
+namespace fk {
+namespace {
+
+constexpr int kBlock = kGemvBlock;  // 256 threads
+
+__device__ __forceinline__ uint32_t xcc_id() {
+    uint32_t v;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+    return v & 0xfu;
+}
+
+// ---- hand-over inside an XCD ------------------------------------------------------------------
+struct XcdSync {
+    XcdControl* ctl;
+    uint32_t xcd, slot, epoch, spin_limit;
+    bool aborted;
+};
+
+// Ordinary stores of this block that other blocks of the XCD will read must have been acknowledged before
+// the flag is published: every wave waits for its own memory counter, the block barrier collects the
+// waves, thread 0 publishes.  Wave 0 then polls the XCD's 64 flag words (one per lane, L1-bypassing
+// loads that are served by the XCD's L2) until every one has reached the epoch.
+__device__ __forceinline__ void xcd_barrier(XcdSync& s, uint32_t* abort_lds) {
+    s.epoch += 1;
+    wait_memory_ops_done();
+    __syncthreads();
+    uint32_t* flags = s.ctl->flags + s.xcd * kXcdSlots;
+    if (threadIdx.x == 0) __hip_atomic_store(flags + s.slot, s.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (threadIdx.x < kWave) {
+        uint32_t spins = 0;
+        bool bad = false;
+        for (;;) {
+            const uint32_t v = __hip_atomic_load(flags + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (__all((int)((int32_t)(v - s.epoch) >= 0))) break;
+            ++spins;
+            if ((spins & 255u) == 0u &&
+                __hip_atomic_load(&s.ctl->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+                bad = true;
+                break;
+            }
+            if (spins > s.spin_limit) {
+                if (threadIdx.x == 0)
+                    __hip_atomic_store(&s.ctl->abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                bad = true;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if (threadIdx.x == 0) *abort_lds = bad ? 1u : 0u;
+    }
+    __syncthreads();
+    s.aborted = s.aborted || (*abort_lds != 0u);
+}
+
+// ---- activation staging (the chunk-interleaved LDS layout of the streaming GEMV) -------------------
+// Group t holds elements 8t .. 8t+7 of the vector: v = their bf16 bits, wv the norm weights' (NORM).
+// With NORM the staged value is T(w * T(x * r)) (src/codegen/kernels/mod.rs:4464-4472).  Every lane of a
+// wave must call this together (the chunk sums are quad butterflies); `live` masks lanes past the end.
+template <WKind KIND>
+__device__ __forceinline__ void stage_emit(uint4* xs, float* sx, uint32_t cs, uint32_t t, bool live, uint4 v, uint4 wv,
+                                           float r, bool NORM) {
+    uint32_t nb[4] = {v.x, v.y, v.z, v.w};
+    if (NORM) {
+        const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t xr_ = pack_bf16(bf16_lo(nb[i]) * r, bf16_hi(nb[i]) * r);
+            nb[i] = pack_bf16(bf16_lo(q[i]) * bf16_lo(xr_), bf16_hi(q[i]) * bf16_hi(xr_));
+        }
+    }
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = bf16_lo(nb[i]);
+        f[2 * i + 1] = bf16_hi(nb[i]);
+    }
+    float s8 = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+    if constexpr (KIND == W_Q4) {
+        const uint32_t c = t >> 2, j = t & 3u;
+        if (live)
+            xs[j * cs + c] = make_uint4(__builtin_amdgcn_perm(nb[1], nb[0], 0x05040100u),
+                                        __builtin_amdgcn_perm(nb[3], nb[2], 0x05040100u),
+                                        __builtin_amdgcn_perm(nb[1], nb[0], 0x07060302u),
+                                        __builtin_amdgcn_perm(nb[3], nb[2], 0x07060302u));
+        s8 = group_sum(s8, 4);
+        if (live && j == 0) sx[c] = s8;
+    } else if constexpr (KIND == W_Q8) {
+        const uint32_t c = t >> 1, j = (t & 1u) * 2u;
+        if (live) {
+            xs[j * cs + c] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                                        __float_as_uint(f[3]));
+            xs[(j + 1) * cs + c] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]), __float_as_uint(f[6]),
+                                              __float_as_uint(f[7]));
+        }
+        s8 = group_sum(s8, 2);
+        if (live && j == 0) sx[c] = s8;
+    } else {
+        if (live) xs[t] = make_uint4(nb[0], nb[1], nb[2], nb[3]);
+    }
+}
+
+// A vector of n8 groups of 8 bf16 values that other blocks of this XCD wrote: L1-bypassing loads, staged as is.
+template <WKind KIND>
+__device__ __forceinline__ void stage_vector(const uint16_t* src, uint32_t n8, uint32_t cs, uint4* xs, float* sx) {
+    const uint4* s8 = reinterpret_cast<const uint4*>(src);
+    const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
+    for (uint32_t t = threadIdx.x; t < n8_up; t += kBlock) {
+        const bool live = t < n8;
+        const uint4 v = ld_u128<true>(s8 + (live ? t : 0u));
+        stage_emit<KIND>(xs, sx, cs, t, live, v, v, 1.0f, false);
+    }
+}
+
+// ---- the input of a launch -------------------------------------------------------------------
+constexpr int kInRegs = 2;  // groups of 8 hidden elements per thread kept in registers (hidden <= 4096)
+
+struct InputFetch {
+    float p[kXcds];
+    uint32_t res;
+    uint4 nw[kInRegs];
+};
+
+// Issues the loads of this block's share of the reduction and of the norm weights.  Called first in the
+// kernel: loads return in issue order and these are needed first.
+__device__ __forceinline__ void input_fetch(const XcdInput& in, uint32_t xcd, uint32_t slot, InputFetch& f) {
+    const uint32_t r0 = slot * in.rows_per_block;
+    uint32_t row = r0 + threadIdx.x;
+    if (threadIdx.x >= in.rows_per_block || row >= in.hidden) row = r0 < in.hidden ? r0 : 0u;  // clamped: straight-line loads
+    const float* p = in.partials ? in.partials : reinterpret_cast<const float*>(in.residual);
+#pragma unroll
+    for (uint32_t j = 0; j < kXcds; ++j) f.p[j] = in.partials ? p[(size_t)j * in.hidden + row] : 0.f;
+    f.res = in.residual[(size_t)xcd * in.residual_stride + row];
+    const uint4* w8 = reinterpret_cast<const uint4*>(in.norm_w);
+    const uint32_t n8 = in.hidden >> 3;
+#pragma unroll
+    for (int i = 0; i < kInRegs; ++i) {
+        const uint32_t t = threadIdx.x + i * kBlock;
+        f.nw[i] = w8[t < n8 ? t : 0u];
+    }
+}
+
+// Stage A: this block's rows of x = T(sum of the partial rows + residual), written to this XCD's copy, and the
+// block's sum of squares.  Then the hand-over, then stage B: every block stages the whole normalised vector.
+template <WKind KIND>
+__device__ __forceinline__ void input_finish(const XcdInput& in, XcdSync& sync, const InputFetch& f, uint4* xs, float* sx,
+                                             float* scratch, uint32_t cs) {
+    const uint32_t r0 = sync.slot * in.rows_per_block;
+    const uint32_t row = r0 + threadIdx.x;
+    const bool mine = threadIdx.x < in.rows_per_block && row < in.hidden;
+    float sq = 0.f;
+    if (mine) {
+        // fixed order: ((p0 + p1) + (p2 + p3)) + ((p4 + p5) + (p6 + p7)), then the residual, one rounding
+        const float acc = ((f.p[0] + f.p[1]) + (f.p[2] + f.p[3])) + ((f.p[4] + f.p[5]) + (f.p[6] + f.p[7]));
+        const uint32_t xb = f32_to_bf16_bits(acc + bf16_bits_to_f32(f.res));
+        in.x_out[(size_t)sync.xcd * in.hidden + row] = (uint16_t)xb;
+        const float xv = bf16_bits_to_f32(xb);
+        sq = xv * xv;
+    }
+    sq = block_sum<kBlock>(sq, scratch);
+    if (threadIdx.x == 0) sync.ctl->ssq[sync.xcd * kXcdSlots + sync.slot] = sq;
+    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+    // sum of squares over the whole vector: every wave adds the 64 block sums in the same order
+    float ss = ld_f32<true>(&sync.ctl->ssq[sync.xcd * kXcdSlots + (threadIdx.x & (kWave - 1))]);
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)in.hidden + in.eps);
+    const uint4* x8 = reinterpret_cast<const uint4*>(in.x_out + (size_t)sync.xcd * in.hidden);
+    const uint32_t n8 = in.hidden >> 3;
+    const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
+#pragma unroll
+    for (int i = 0; i < kInRegs; ++i) {
+        const uint32_t t = threadIdx.x + i * kBlock;
+        if ((threadIdx.x & ~(uint32_t)(kWave - 1)) + i * kBlock < n8_up) {
+            const bool live = t < n8;
+            const uint4 v = ld_u128<true>(x8 + (live ? t : 0u));
+            stage_emit<KIND>(xs, sx, cs, t, live, v, f.nw[i], r, true);
+        }
+    }
+    __syncthreads();
+}
+
+// ---- projection tiles ----------------------------------------------------------------------------
+// A tile: rows [row0, row0 + rows) x chunks [col0, col0 + cs) of a matrix; flat position p = row * cs + col.
+// A pass covers NL * 256 positions; positions past the tile read the tile's first chunk (in bounds).
+template <int NL>
+struct TileRegs {
+    uint4 w[NL];
+    uint32_t sc[NL], bi[NL];
+};
+
+struct Tile {
+    uint32_t row0, rows, col0, cs;
+    float inv_cs;
+};
+
+template <WKind KIND, int NL>
+__device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, uint32_t pass, TileRegs<NL>& r) {
+    const uint32_t total = t.rows * t.cs;
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const uint32_t pos = (pass * NL + j) * kBlock + threadIdx.x;
+        const uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
+        const uint32_t col = pos - row * t.cs;
+        const size_t idx = pos < total ? (size_t)(t.row0 + row) * m.cpr + t.col0 + col : (size_t)t.row0 * m.cpr + t.col0;
+        r.w[j] = m.w[idx];
+        if constexpr (KIND != W_BF16) {
+            const size_t g = idx >> m.gshift;
+            r.sc[j] = m.sc[g];
+            r.bi[j] = m.bi[g];
+        }
+    }
+}
+
+// One fp32 partial per chunk into part[pos] (padded to whole passes, so no guard is needed).
+template <WKind KIND, int NL>
+__device__ __forceinline__ void tile_partials(const Tile& t, uint32_t pass, const TileRegs<NL>& r, const uint4* xs,
+                                              const float* sx, float* part) {
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const uint32_t pos = (pass * NL + j) * kBlock + threadIdx.x;
+        const uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
+        uint32_t col = pos - row * t.cs;
+        col = col < t.cs ? col : 0u;
+        part[pos] = chunk_partial<KIND>(r.w[j], r.sc[j], r.bi[j], xs, sx, col, t.cs);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// All passes of a tile whose first pass is already in `r`.
+template <WKind KIND, int NL>
+__device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, TileRegs<NL>& r, const uint4* xs, const float* sx,
+                                         float* part) {
+    const uint32_t n_pass = (t.rows * t.cs + NL * kBlock - 1) / (NL * kBlock);
+    for (uint32_t p = 0; p < n_pass; ++p) {
+        if (p) tile_load<KIND, NL>(m, t, p, r);
+        tile_partials<KIND, NL>(t, p, r, xs, sx, part);
+    }
+}
+
+__device__ __forceinline__ uint32_t lanes_per_row(uint32_t cs) {
+    uint32_t lr = 1;
+    while (lr * 2 <= cs && lr < 64) lr <<= 1;
+    return lr;
+}
+
+// Adds each row's partials in a fixed order; f(row, sum0, sum1) runs in one lane per row.
+template <bool TWO, typename F>
+__device__ __forceinline__ void tile_rows(const Tile& t, const float* part, const float* part1, F f) {
+    const uint32_t lr = lanes_per_row(t.cs), lane = threadIdx.x & (lr - 1);
+    const uint32_t rows_up = (t.rows + (kBlock / lr) - 1) / (kBlock / lr) * (kBlock / lr);
+    for (uint32_t rr = threadIdx.x / lr; rr < rows_up; rr += kBlock / lr) {
+        const bool ok = rr < t.rows;
+        float s0 = 0.f, s1 = 0.f;
+        if (ok)
+            for (uint32_t i = lane; i < t.cs; i += lr) {
+                s0 += part[rr * t.cs + i];
+                if constexpr (TWO) s1 += part1[rr * t.cs + i];
+            }
+        s0 = group_sum(s0, lr);
+        if constexpr (TWO) s1 = group_sum(s1, lr);
+        if (ok && lane == 0) f(rr, s0, s1);
+    }
+}
+
+// An empty tile (a block without work in this projection) still issues its loads, clamped to the tile's
+// first chunk: it is moved to row 0 so that those loads stay inside the matrix.
+__device__ __forceinline__ Tile make_tile(uint32_t row0, uint32_t rows, uint32_t col0, uint32_t cs) {
+    Tile t;
+    t.row0 = rows ? row0 : 0u;
+    t.rows = rows;
+    t.col0 = col0;
+    t.cs = cs;
+    t.inv_cs = 1.0f / (float)cs;
+    return t;
+}
+
+// LDS layout shared by both kernels (floats unless noted):
+//   xs   uint4 [PIECES * cs_max]      staged activations
+//   sx   [cs_max]                     per-chunk sums
+//   work [work_floats]                chunk partials of a tile (two segments for gate / up), or the attention's LDS
+//   att  uint16 [att_elems]           merged attention rows (attention launch)
+//   scratch [16]
+struct LdsPlan {
+    uint32_t cs_max, work_floats, att_elems;
+};
+template <WKind KIND>
+__host__ __device__ inline uint32_t xcd_lds_bytes(const LdsPlan& p) {
+    return ChunkTraits<KIND>::kPieces * p.cs_max * 16u + p.cs_max * 4u + p.work_floats * 4u +
+           ((p.att_elems * 2u + 15u) & ~15u) + 64u;
+}
+
+}  // namespace
+
+// =============================================================================================== MLP launch
+template <WKind KIND, int NLA, int NLB>
+__global__ __launch_bounds__(kBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    const uint32_t cs_max = a.cs_max, work_floats = a.work_floats;
+    constexpr int PIECES = ChunkTraits<KIND>::kPieces;
+    uint4* xs = lds_raw;
+    float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
+    float* work = sx + cs_max;
+    float* scratch = work + work_floats;
+
+    XcdSync sync;
+    sync.ctl = a.ctl;
+    // Workgroups are dealt to the XCDs round-robin, starting wherever the previous dispatch stopped: the XCD is
+    // read from the hardware, and workgroups i and i + 8 land on the same XCD, so i / 8 numbers the 64 blocks of
+    // each XCD.  (Were the dealing ever different, two blocks would share a flag word, a hand-over wait would
+    // run into its spin limit and the launch would report it.)
+    sync.xcd = xcc_id() & (kXcds - 1);
+    sync.slot = blockIdx.x / kXcds;
+    sync.spin_limit = a.spin_limit;
+    sync.aborted = false;
+    sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    InputFetch fin;
+    input_fetch(a.in, sync.xcd, sync.slot, fin);
+
+    const uint32_t per_xcd = a.inter / kXcds;
+    const uint32_t gu0 = sync.slot * a.gu_rows;
+    const uint32_t gu_n = gu0 < per_xcd ? ((per_xcd - gu0) < a.gu_rows ? (per_xcd - gu0) : a.gu_rows) : 0u;
+    const Tile tg = make_tile(sync.xcd * per_xcd + gu0, gu_n, 0, a.gate.cpr);
+    const uint32_t d0 = sync.slot * a.down_rows;
+    const uint32_t d_n = d0 < a.in.hidden ? ((a.in.hidden - d0) < a.down_rows ? (a.in.hidden - d0) : a.down_rows) : 0u;
+    const Tile td = make_tile(d0, d_n, sync.xcd * a.down_cs, a.down_cs);
+
+    // every weight this block will use is requested now; the hand-overs below only gate arithmetic
+    TileRegs<NLA> rg, ru;
+    TileRegs<NLB> rd;
+    tile_load<KIND, NLA>(a.gate, tg, 0, rg);
+    tile_load<KIND, NLA>(a.up, tg, 0, ru);
+    tile_load<KIND, NLB>(a.down, td, 0, rd);
+
+    input_finish<KIND>(a.in, sync, fin, xs, sx, scratch, a.gate.cpr);
+
+    // ---- gate / up rows of this XCD's slice, SwiGLU ----
+    const uint32_t seg = (gu_n * a.gate.cpr + NLA * kBlock - 1) / (NLA * kBlock) * (NLA * kBlock);
+    if (gu_n) {
+        tile_run<KIND, NLA>(a.gate, tg, rg, xs, sx, work);
+        tile_run<KIND, NLA>(a.up, tg, ru, xs, sx, work + seg);
+    }
+    __syncthreads();
+    if (gu_n) {
+        uint16_t* mid = a.mid + (size_t)sync.xcd * per_xcd + gu0;
+        const int variant = a.swiglu_variant;
+        tile_rows<true>(tg, work, work + seg,
+                        [&](uint32_t r, float s0, float s1) { mid[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
+    }
+    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+
+    // ---- down_proj over this XCD's K-slice: fp32 partial row ----
+    stage_vector<KIND>(a.mid + (size_t)sync.xcd * per_xcd, per_xcd >> 3, a.down_cs, xs, sx);
+    __syncthreads();
+    if (d_n) tile_run<KIND, NLB>(a.down, td, rd, xs, sx, work);
+    __syncthreads();
+    if (d_n) {
+        float* out = a.out_partials + (size_t)sync.xcd * a.in.hidden + d0;
+        tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { out[r] = s0; });
+    }
+}
+
+// =============================================================================================== attention launch
+template <WKind KIND, int NLA, int NLB>
+__global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    const uint32_t cs_max = a.cs_max, work_floats = a.work_floats, att_elems = a.att_elems;
+    constexpr int PIECES = ChunkTraits<KIND>::kPieces;
+    uint4* xs = lds_raw;
+    float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
+    float* work = sx + cs_max;
+    uint16_t* att = reinterpret_cast<uint16_t*>(work + work_floats);
+    float* scratch = reinterpret_cast<float*>(reinterpret_cast<char*>(att) + ((att_elems * 2u + 15u) & ~15u));
+
+    XcdSync sync;
+    sync.ctl = a.ctl;
+    sync.xcd = xcc_id() & (kXcds - 1);   // see xcd_mlp_kernel
+    sync.slot = blockIdx.x / kXcds;
+    sync.spin_limit = a.spin_limit;
+    sync.aborted = false;
+    sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t kv_len0 = *a.sdpa.kv_len_ptr;
+
+    InputFetch fin;
+    input_fetch(a.in, sync.xcd, sync.slot, fin);
+
+    // tile of the q / k / v projections: the XCD's q rows first, then its k rows, then its v rows
+    const uint32_t R = a.qkv_tile_rows, ti = sync.slot;
+    const bool has_tile = ti < a.q_tiles + 2 * a.kv_tiles;
+    const uint32_t part_id = ti < a.q_tiles ? 0u : (ti < a.q_tiles + a.kv_tiles ? 1u : 2u);
+    const uint32_t tl = part_id == 0 ? ti : (part_id == 1 ? ti - a.q_tiles : ti - a.q_tiles - a.kv_tiles);
+    const uint32_t part_rows = part_id == 0 ? a.q_rows : a.kv_rows;
+    const uint32_t pr0 = tl * R;
+    const uint32_t pr_n = has_tile ? ((part_rows - pr0) < R ? (part_rows - pr0) : R) : 0u;
+    const XcdMat& mq = part_id == 0 ? a.wq : (part_id == 1 ? a.wk : a.wv);
+    const Tile tq = make_tile(sync.xcd * part_rows + pr0, pr_n, 0, a.wq.cpr);
+    const uint32_t o0 = sync.slot * a.o_rows;
+    const uint32_t o_n = o0 < a.in.hidden ? ((a.in.hidden - o0) < a.o_rows ? (a.in.hidden - o0) : a.o_rows) : 0u;
+    const Tile to = make_tile(o0, o_n, sync.xcd * a.o_cs, a.o_cs);
+
+    TileRegs<NLA> rq;
+    TileRegs<NLB> ro;
+    tile_load<KIND, NLA>(mq, tq, 0, rq);
+    tile_load<KIND, NLB>(a.wo, to, 0, ro);
+
+    input_finish<KIND>(a.in, sync, fin, xs, sx, scratch, a.wq.cpr);
+
+    // ---- q / k / v rows of this XCD's KV head ----
+    if (pr_n) tile_run<KIND, NLA>(mq, tq, rq, xs, sx, work);
+    __syncthreads();
+    if (pr_n) {
+        uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
+        tile_rows<false>(tq, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
+    }
+    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+
+    // ---- head norm + RoPE + cache append + attention: block = (query head of the group, key range) ----
+    const uint32_t G = a.sdpa.n_heads / a.sdpa.n_kv;
+    {
+        const uint32_t gz = sync.slot % G, split = sync.slot / G;
+        if (split < a.sdpa.n_splits)
+            sdpa_block<1, 2, SdpaArgs, 0, true, true>(a.sdpa, kv_len0, split, sync.xcd, gz, G, work);
+    }
+    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+
+    // ---- merge the ranges of each of the group's heads (range order), rows to LDS ----
+    {
+        const uint32_t span = a.sdpa.chunk_len * a.sdpa.chunks_per_block;
+        const uint32_t covered = a.sdpa.n_splits * span < a.sdpa.capacity ? a.sdpa.n_splits * span : a.sdpa.capacity;
+        const uint32_t kv_len = kv_len0 < 1u ? 1u : (kv_len0 > covered ? covered : kv_len0);
+        const uint32_t n_active = (kv_len + span - 1) / span;
+        const uint32_t row = a.sdpa.v_dim + 2;
+        const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+        for (uint32_t h = wave; h < G; h += kBlock / kWave) {
+            const float* ph = a.sdpa.partials + (size_t)(sync.xcd * G + h) * a.sdpa.n_splits * row;
+            for (uint32_t d2 = lane; d2 < ((a.sdpa.v_dim >> 1) + kWave - 1) / kWave * kWave; d2 += kWave) {
+                const bool live = d2 < (a.sdpa.v_dim >> 1);
+                const float* pd = ph + 2 + 2 * (live ? d2 : 0u);
+                float2 ml[kXcdMaxRanges], po[kXcdMaxRanges];
+#pragma unroll
+                for (uint32_t i = 0; i < kXcdMaxRanges; ++i) {
+                    const uint32_t idx = i < n_active ? i : 0u;
+                    ml[i] = ld_f32x2<true>(ph + (size_t)idx * row);
+                    po[i] = ld_f32x2<true>(pd + (size_t)idx * row);
+                }
+                float M = ml[0].x;
+#pragma unroll
+                for (uint32_t i = 1; i < kXcdMaxRanges; ++i) M = i < n_active ? fmaxf(M, ml[i].x) : M;
+                float L = 0.f, o0_ = 0.f, o1_ = 0.f;
+#pragma unroll
+                for (uint32_t i = 0; i < kXcdMaxRanges; ++i) {
+                    const float w = i < n_active ? expf(ml[i].x - M) : 0.f;
+                    L = fmaf(ml[i].y, w, L);
+                    o0_ = fmaf(po[i].x, w, o0_);
+                    o1_ = fmaf(po[i].y, w, o1_);
+                }
+                const float inv_l = 1.0f / L;
+                if (live) {
+                    att[h * a.sdpa.v_dim + 2 * d2] = (uint16_t)f32_to_bf16_bits(o0_ * inv_l);
+                    att[h * a.sdpa.v_dim + 2 * d2 + 1] = (uint16_t)f32_to_bf16_bits(o1_ * inv_l);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // ---- o_proj over this XCD's K-slice (its heads' columns): fp32 partial row ----
+    {
+        const uint32_t n8 = (G * a.sdpa.v_dim) >> 3, n8_up = (n8 + kWave - 1) / kWave * kWave;
+        const uint4* a8 = reinterpret_cast<const uint4*>(att);
+        for (uint32_t t = threadIdx.x; t < n8_up; t += kBlock) {
+            const bool live = t < n8;
+            const uint4 v = a8[live ? t : 0u];
+            stage_emit<KIND>(xs, sx, a.o_cs, t, live, v, v, 1.0f, false);
+        }
+    }
+    __syncthreads();
+    if (o_n) tile_run<KIND, NLB>(a.wo, to, ro, xs, sx, work);
+    __syncthreads();
+    if (o_n) {
+        float* out = a.out_partials + (size_t)sync.xcd * a.in.hidden + o0;
+        tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { out[r] = s0; });
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.hidden) return;
+    float p[kXcds];
+#pragma unroll
+    for (uint32_t j = 0; j < kXcds; ++j) p[j] = a.partials[(size_t)j * a.hidden + i];
+    const float acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+    a.x[i] = (uint16_t)f32_to_bf16_bits(acc + bf16_bits_to_f32(a.residual[i]));
+}
+
+// =============================================================================================== host side
+namespace {
+
+constexpr int kNlQkv = 5, kNlO = 3, kNlGu = 6, kNlDown = 6;
+
+uint32_t ilog2u(uint32_t v) {
+    uint32_t r = 0;
+    while ((1u << (r + 1)) <= v) ++r;
+    return r;
+}
+uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+uint32_t chunk_values(uint32_t bits) { return bits == 4 ? 32u : (bits == 8 ? 16u : 8u); }
+
+fk_status bind_mat(const fk_weight* w, uint32_t n, uint32_t k, const XcdLayerShape& s, XcdMat* m, const char* what) {
+    if (!w || !w->w) return set_error(FK_ERR_INVALID, std::string("xcd layer: null weight ") + what);
+    if (w->n != n || w->k != k || w->bits != s.bits || (s.bits != 16 && w->group != s.group))
+        return set_error(FK_ERR_INVALID, std::string("xcd layer: weight ") + what + " does not match the layer shape");
+    if (s.bits != 16 && (!w->scales || !w->biases)) return set_error(FK_ERR_INVALID, std::string("xcd layer: null scales / biases of ") + what);
+    m->w = reinterpret_cast<const uint4*>(w->w);
+    m->sc = w->scales;
+    m->bi = w->biases;
+    m->cpr = k / chunk_values(s.bits);
+    m->gshift = s.bits == 16 ? 0 : ilog2u(s.group / chunk_values(s.bits));
+    return FK_OK;
+}
+
+template <WKind KIND>
+const void* mlp_func() { return reinterpret_cast<const void*>(&xcd_mlp_kernel<KIND, kNlGu, kNlDown>); }
+template <WKind KIND>
+const void* attn_func() { return reinterpret_cast<const void*>(&xcd_attn_kernel<KIND, kNlQkv, kNlO>); }
+
+uint32_t lds_for(uint32_t bits, const LdsPlan& p) {
+    return bits == 4 ? xcd_lds_bytes<W_Q4>(p) : (bits == 8 ? xcd_lds_bytes<W_Q8>(p) : xcd_lds_bytes<W_BF16>(p));
+}
+
+fk_status fill_input(const XcdLayerShape& s, const float* partials, const uint16_t* residual, uint32_t residual_stride,
+                     uint16_t* x_out, const uint16_t* norm_w, float eps, XcdInput* in) {
+    if (!residual || !x_out || !norm_w) return set_error(FK_ERR_INVALID, "xcd layer: null residual, x_out or norm weight");
+    if (residual_stride != 0 && residual_stride != s.hidden)
+        return set_error(FK_ERR_INVALID, "xcd layer: residual stride must be 0 (one row) or hidden (a copy per XCD)");
+    in->partials = partials;
+    in->residual = residual;
+    in->residual_stride = residual_stride;
+    in->x_out = x_out;
+    in->norm_w = norm_w;
+    in->eps = eps;
+    in->hidden = s.hidden;
+    in->rows_per_block = ceil_div(s.hidden, kXcdSlots);
+    return FK_OK;
+}
+
+fk_status set_lds_limit(const void* func, uint32_t lds) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if ((int)lds > dev->max_dyn_lds) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: LDS need exceeds the CU");
+    if (lds > 48 * 1024) FK_HIP(hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    return FK_OK;
+}
+
+}  // namespace
+
+fk_status xcd_layer_supported(const XcdLayerShape& s) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (dev->cus != (int)(kXcds * 32)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: needs 8 XCDs of 32 CUs");
+    if (s.bits != 4 && s.bits != 8 && s.bits != 16) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: bits must be 4, 8 or 16");
+    const uint32_t cv = chunk_values(s.bits), unit = s.bits == 16 ? cv : (s.group > cv ? s.group : cv);
+    if (s.bits != 16 && s.group != 32 && s.group != 64 && s.group != 128)
+        return set_error(FK_ERR_UNSUPPORTED, "xcd layer: group size must be 32, 64 or 128");
+    if (s.n_kv != kXcds) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: needs exactly 8 KV heads (one per XCD)");
+    if (s.n_heads % s.n_kv) return set_error(FK_ERR_INVALID, "xcd layer: n_heads must be a multiple of n_kv");
+    const uint32_t G = s.n_heads / s.n_kv;
+    if (G != 1 && G != 2 && G != 4 && G != 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: 1, 2, 4 or 8 query heads per KV head");
+    if (s.head_dim != 64 && s.head_dim != 128) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: head_dim must be 64 or 128");
+    if (s.hidden % 64 || s.hidden > (uint32_t)kInRegs * kBlock * 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: hidden must be a multiple of 64, at most 4096");
+    if ((G * s.head_dim) % unit) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a KV head's query columns must be whole quantisation groups");
+    if (s.inter % (kXcds * unit) || s.inter % (kXcds * 8)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: intermediate / 8 must be whole quantisation groups");
+    if (s.capacity == 0) return set_error(FK_ERR_INVALID, "xcd layer: zero cache capacity");
+    return FK_OK;
+}
+
+size_t xcd_workspace_bytes() { return sizeof(XcdControl); }
+
+size_t xcd_attn_partials_bytes(const XcdLayerShape& s) {
+    return (size_t)s.n_heads * kXcdMaxRanges * (s.head_dim + 2) * sizeof(float);
+}
+
+fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
+    const XcdLayerShape& s = rq.shape;
+    FK_TRY(xcd_layer_supported(s));
+    if (!rq.mid || !rq.out_partials || !rq.workspace) return set_error(FK_ERR_INVALID, "xcd mlp: null mid, partial rows or workspace");
+    if (rq.swiglu_variant < 0 || rq.swiglu_variant > 2) return set_error(FK_ERR_INVALID, "xcd mlp: swiglu variant must be 0, 1 or 2");
+    XcdMlpArgs a;
+    memset(&a, 0, sizeof(a));
+    FK_TRY(fill_input(s, rq.partials_in, rq.residual, rq.residual_stride, rq.x_out, rq.norm_w, rq.eps, &a.in));
+    FK_TRY(bind_mat(rq.wgate, s.inter, s.hidden, s, &a.gate, "gate_proj"));
+    FK_TRY(bind_mat(rq.wup, s.inter, s.hidden, s, &a.up, "up_proj"));
+    FK_TRY(bind_mat(rq.wdown, s.hidden, s.inter, s, &a.down, "down_proj"));
+    a.inter = s.inter;
+    a.gu_rows = ceil_div(s.inter / kXcds, kXcdSlots);
+    a.down_rows = ceil_div(s.hidden, kXcdSlots);
+    a.down_cs = a.down.cpr / kXcds;
+    a.swiglu_variant = rq.swiglu_variant;
+    a.mid = rq.mid;
+    a.out_partials = rq.out_partials;
+    a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
+    a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
+    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
+    LdsPlan lp;
+    lp.cs_max = a.gate.cpr > a.down_cs ? a.gate.cpr : a.down_cs;
+    const uint32_t gu = 2 * padded(a.gu_rows * a.gate.cpr, kNlGu), dn = padded(a.down_rows * a.down_cs, kNlDown);
+    lp.work_floats = gu > dn ? gu : dn;
+    lp.att_elems = 0;
+    const uint32_t lds = lds_for(s.bits, lp);
+    out->func = s.bits == 4 ? mlp_func<W_Q4>() : (s.bits == 8 ? mlp_func<W_Q8>() : mlp_func<W_BF16>());
+    FK_TRY(set_lds_limit(out->func, lds));
+    out->grid = dim3(kXcdGrid, 1, 1);
+    out->block = dim3(kBlock, 1, 1);
+    out->shmem = lds;
+    a.cs_max = lp.cs_max;
+    a.work_floats = lp.work_floats;
+    out->set_args(a);
+    return FK_OK;
+}
+
+fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
+    const XcdLayerShape& s = rq.shape;
+    FK_TRY(xcd_layer_supported(s));
+    if (!rq.q || !rq.k || !rq.v || !rq.cache_k || !rq.cache_v || !rq.kv_len || !rq.rope_tab || !rq.att_partials ||
+        !rq.out_partials || !rq.workspace)
+        return set_error(FK_ERR_INVALID, "xcd attention: null buffer");
+    if ((rq.q_norm == nullptr) != (rq.k_norm == nullptr)) return set_error(FK_ERR_INVALID, "xcd attention: q and k head norms come together");
+    const uint32_t G = s.n_heads / s.n_kv, n_q = s.n_heads * s.head_dim, n_kvd = s.n_kv * s.head_dim;
+    XcdAttnArgs a;
+    memset(&a, 0, sizeof(a));
+    FK_TRY(fill_input(s, rq.partials_in, rq.residual, rq.residual_stride, rq.x_out, rq.norm_w, rq.eps, &a.in));
+    FK_TRY(bind_mat(rq.wq, n_q, s.hidden, s, &a.wq, "q_proj"));
+    FK_TRY(bind_mat(rq.wk, n_kvd, s.hidden, s, &a.wk, "k_proj"));
+    FK_TRY(bind_mat(rq.wv, n_kvd, s.hidden, s, &a.wv, "v_proj"));
+    FK_TRY(bind_mat(rq.wo, s.hidden, n_q, s, &a.wo, "o_proj"));
+    a.q_rows = G * s.head_dim;
+    a.kv_rows = s.head_dim;
+    uint32_t R = 1;
+    while (ceil_div(a.q_rows, R) + 2 * ceil_div(a.kv_rows, R) > kXcdSlots) ++R;
+    a.qkv_tile_rows = R;
+    a.q_tiles = ceil_div(a.q_rows, R);
+    a.kv_tiles = ceil_div(a.kv_rows, R);
+    a.o_rows = ceil_div(s.hidden, kXcdSlots);
+    a.o_cs = a.wo.cpr / kXcds;
+    a.q = rq.q;
+    a.k = rq.k;
+    a.v = rq.v;
+    // attention of one KV head per XCD: blocks = (query head of the group) x (key range)
+    SdpaArgs& sd = a.sdpa;
+    sd.q = rq.q;
+    sd.k = rq.cache_k;
+    sd.v = rq.cache_v;
+    sd.out = nullptr;
+    sd.kv_len_ptr = rq.kv_len;
+    sd.n_heads = s.n_heads;
+    sd.n_kv = s.n_kv;
+    sd.qk_dim = sd.v_dim = s.head_dim;
+    sd.capacity = s.capacity;
+    sd.chunk_len = sdpa_chunk_len(s.head_dim, s.head_dim, false);
+    uint32_t splits = kXcdSlots / G;
+    if (splits > kXcdMaxRanges) splits = kXcdMaxRanges;
+    const uint32_t n_chunks = ceil_div(s.capacity, sd.chunk_len);
+    sd.chunks_per_block = ceil_div(n_chunks, splits);
+    sd.n_splits = ceil_div(n_chunks, sd.chunks_per_block);
+    sd.rows = 1;
+    uint32_t lp_ = 1;
+    while (lp_ < s.head_dim / 8) lp_ <<= 1;
+    sd.lpk = sd.lpv = lp_;
+    sd.scale = 1.0f / sqrtf((float)s.head_dim);
+    sd.partials = rq.att_partials;
+    sd.counters = nullptr;
+    sd.k_new = rq.k;
+    sd.v_new = rq.v;
+    sd.q_norm = rq.q_norm;
+    sd.k_norm = rq.k_norm;
+    sd.cache_k_w = rq.cache_k;
+    sd.cache_v_w = rq.cache_v;
+    sd.rope_dims = s.head_dim;
+    sd.eps = rq.eps;
+    sd.base_log2 = (float)log2((double)rq.theta);
+    sd.rope_tab = rq.rope_tab;
+    sd.v_stride = s.head_dim;
+    sd.k1_heads = 1;
+    a.out_partials = rq.out_partials;
+    a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
+    a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
+    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
+    LdsPlan lp;
+    lp.cs_max = a.wq.cpr > a.o_cs ? a.wq.cpr : a.o_cs;
+    uint32_t wf = padded(R * a.wq.cpr, kNlQkv);
+    const uint32_t wo_ = padded(a.o_rows * a.o_cs, kNlO);
+    wf = wf > wo_ ? wf : wo_;
+    const uint32_t sf = sdpa_lds_floats(1, sd.chunk_len, s.head_dim, s.head_dim, true);
+    lp.work_floats = wf > sf ? wf : sf;
+    lp.att_elems = G * s.head_dim;
+    const uint32_t lds = lds_for(s.bits, lp);
+    out->func = s.bits == 4 ? attn_func<W_Q4>() : (s.bits == 8 ? attn_func<W_Q8>() : attn_func<W_BF16>());
+    FK_TRY(set_lds_limit(out->func, lds));
+    out->grid = dim3(kXcdGrid, 1, 1);
+    out->block = dim3(kBlock, 1, 1);
+    out->shmem = lds;
+    a.cs_max = lp.cs_max;
+    a.work_floats = lp.work_floats;
+    a.att_elems = lp.att_elems;
+    out->set_args(a);
+    return FK_OK;
+}
+
+fk_status plan_xcd_reduce(const float* partials, const uint16_t* residual, uint16_t* x, uint32_t hidden, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!partials || !residual || !x || hidden == 0) return set_error(FK_ERR_INVALID, "xcd reduce: null buffer or zero width");
+    XcdReduceArgs a{partials, residual, x, hidden};
+    out->func = reinterpret_cast<const void*>(&xcd_reduce_kernel);
+    out->grid = dim3(ceil_div(hidden, kBlock), 1, 1);
+    out->block = dim3(kBlock, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
+
+}  // namespace fk

@@ -45,6 +45,8 @@ class DecoderConfig:
     kv_bits: int = 0         # 0: bf16 KV cache; 4 / 8: quantised cache (mlx-lm QuantizedKVCache layout)
     kv_group: int = 64
     embed_scale: float = 1.0  # output_scale of the embedding lookup (embed_lookup_decode.rs:74-99)
+    xcd_layers: bool = True   # graph mode: run a layer as two XCD-resident launches where the shape allows it
+    xcd_spin_limit: int = 0   # bound of the XCD hand-over waits in polls (0: the library's default)
 
     @property
     def n_q(self) -> int:
@@ -211,6 +213,16 @@ class DecoderRuntime:
         # fuses them itself and is built from the plain task list)
         self.fused_attention = bool(cfg.fuse_attention and not persistent and not cfg.kv_bits)
         self.rope_tab = DeviceBuffer(cfg.head_dim * 4) if self.fused_attention else None
+        # a layer as two XCD-resident launches (8 KV heads, one per XCD): graph mode, bf16 cache, no projection bias
+        self.xcd = bool(cfg.xcd_layers and self.fused_attention and not cfg.qkv_bias and
+                        native.xcd_layer_supported(cfg.hidden, cfg.inter, cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.capacity,
+                                                   cfg.bits, cfg.group))
+        if self.xcd:
+            ctl, ap = native.xcd_workspace_bytes(cfg.n_heads, cfg.head_dim)
+            self.xcd_ctl = z(ctl)
+            self.xcd_att_partials = DeviceBuffer(ap)
+            self.xcd_xa, self.xcd_xb = DeviceBuffer(8 * cfg.hidden * 2), DeviceBuffer(8 * cfg.hidden * 2)
+            self.xcd_o_part, self.xcd_down_part = DeviceBuffer(8 * cfg.hidden * 4), DeviceBuffer(8 * cfg.hidden * 4)
         self._bf16_weights: Dict[str, DeviceWeight] = {}   # resident bf16 copies for prompt passes (prefill_rows)
         self.tasks = self.build_tasks()
         # persistent: the same task list, run by one whole-token kernel per replay
@@ -241,7 +253,9 @@ class DecoderRuntime:
         t.append(Dispatch(name("embed_lookup_decode"), [arg(self.token)] + self._wargs(emb) + [arg(self.x[0])],
                           dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab,
                                output_scale=c.embed_scale)))
-        for l in range(c.n_layers):
+        if self.xcd:
+            self._xcd_layer_tasks(t, name)
+        for l in range(0 if not self.xcd else c.n_layers, c.n_layers):
             p = f"layers.{l}."
             Wq, Wk, Wv = (w.mats[p + f"self_attn.{n}_proj"] for n in "qkv")
             qkv_args = [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(Wq.w), arg(Wk.w), arg(Wv.w)]
@@ -329,6 +343,40 @@ class DecoderRuntime:
                           [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history),
                            arg(self.hist_counter)], dict(vocab=c.vocab)))
         return t
+
+    def _xcd_layer_tasks(self, t: List[Dispatch], name) -> None:
+        """Two launches per layer (families fusekit_xcd_attn_block / fusekit_xcd_mlp_block), then the reduction of
+        the last layer's partial rows into x[0] for the LM head."""
+        c, w = self.cfg, self.w
+        shape = dict(hidden=c.hidden, inter=c.inter, n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim,
+                     capacity=c.capacity, bits=c.bits, group=c.group, eps=c.eps, theta=c.theta,
+                     spin_limit=c.xcd_spin_limit)
+        quant = c.bits != 16
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            Wq, Wk, Wv, Wo = (w.mats[p + f"self_attn.{n}_proj"] for n in "qkvo")
+            a = [] if l == 0 else [arg(self.xcd_down_part)]
+            a += [arg(self.x[0]) if l == 0 else arg(self.xcd_xb), arg(self.xcd_xa), arg(w.vecs[p + "input_layernorm"]),
+                  arg(Wq.w), arg(Wk.w), arg(Wv.w)]
+            if quant:
+                a += [arg(m.scales) for m in (Wq, Wk, Wv)] + [arg(m.biases) for m in (Wq, Wk, Wv)]
+            a += self._wargs(Wo)
+            if c.qk_norm:
+                a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
+            a += [arg(self.q), arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+                  arg(self.rope_tab), arg(self.xcd_att_partials), arg(self.xcd_o_part), arg(self.xcd_ctl)]
+            t.append(Dispatch(name("xcd_attn_block"), a,
+                              dict(shape, has_partials=int(l > 0), residual_per_xcd=int(l > 0), has_norm=int(c.qk_norm))))
+            Wg, Wu, Wd = (w.mats[p + f"mlp.{n}_proj"] for n in ("gate", "up", "down"))
+            m = [arg(self.xcd_o_part), arg(self.xcd_xa), arg(self.xcd_xb), arg(w.vecs[p + "post_attention_layernorm"]),
+                 arg(Wg.w), arg(Wu.w)]
+            if quant:
+                m += [arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases)]
+            m += self._wargs(Wd) + [arg(self.mid), arg(self.xcd_down_part), arg(self.xcd_ctl)]
+            t.append(Dispatch(name("xcd_mlp_block"), m,
+                              dict(shape, has_partials=1, residual_per_xcd=1, variant=c.swiglu_variant)))
+        t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_down_part), arg(self.xcd_xb, c.hidden * 2), arg(self.x[0])],
+                          dict(hidden=c.hidden)))
 
     # -- generation ------------------------------------------------------------------
     def reset(self) -> None:

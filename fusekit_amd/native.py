@@ -479,6 +479,23 @@ def rope_store_sdpa_decode(q, k, v, q_norm, k_norm, cache_k, cache_v, out, d_kv_
         _ptr(partials), _ptr(counters), _ptr(stream)))
 
 
+def xcd_layer_supported(hidden, inter, n_heads, n_kv, head_dim, capacity, bits, group) -> bool:
+    """Can a layer of this shape run as two XCD-resident launches (fk_xcd_layer_supported)?"""
+    return lib.fk_xcd_layer_supported(C.c_uint32(hidden), C.c_uint32(inter), C.c_uint32(n_heads), C.c_uint32(n_kv),
+                                      C.c_uint32(head_dim), C.c_uint32(capacity), C.c_uint32(bits), C.c_uint32(group)) == 0
+
+
+def xcd_workspace_bytes(n_heads, head_dim):
+    """(bytes of the control block, bytes of the attention partial rows)."""
+    a, b = C.c_size_t(), C.c_size_t()
+    check(lib.fk_xcd_workspace_bytes(C.c_uint32(n_heads), C.c_uint32(head_dim), C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
+def xcd_check(workspace, stream=None) -> None:
+    check(lib.fk_xcd_check(_ptr(workspace), _ptr(stream)))
+
+
 def copy(dst, src, nbytes, stream=None):
     check(lib.fk_copy(_ptr(dst), _ptr(src), C.c_size_t(nbytes), _ptr(stream)))
 

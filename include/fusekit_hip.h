@@ -466,6 +466,25 @@ fk_status fk_rope_store_sdpa_decode(const uint16_t *q, const uint16_t *k, const 
                                     uint32_t capacity, float scale, const float *rope_tab, float *partials,
                                     uint32_t *counters, fk_stream s);
 
+/* ---- XCD-resident layer: a decoder layer as TWO launches -------------------------------------
+ *
+ * Dispatch families `fusekit_xcd_attn_block` (replaces, for one layer, the dispatches
+ * rmsnorm_qkv.rs + rope_q_decode.rs / rope_kv_cache_store_decode.rs (or their head-norm forms) +
+ * sdpa_decode.rs + linear_residual.rs of the attention half) and `fusekit_xcd_mlp_block` (replaces
+ * rmsnorm_gateup_swiglu.rs + linear_residual.rs of the MLP half); `fusekit_xcd_reduce` finishes the last
+ * layer's output row for final_rmsnorm_lm_head.rs.  Same arithmetic and rounding points per output
+ * (fp32 accumulation, one rounding to bf16 after the residual is added); the K dimension of o_proj and
+ * down_proj is summed as 8 slices, one per XCD, added in a fixed order.  Slot orders are documented at
+ * the planners (fusekit_amd/csrc/dispatcher.hip).  Requires 8 KV heads (one per XCD), 1 / 2 / 4 / 8 query
+ * heads per KV head, head_dim 64 or 128, hidden <= 4096; other layers use the per-dispatch families. */
+fk_status fk_xcd_layer_supported(uint32_t hidden, uint32_t inter, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                 uint32_t capacity, uint32_t bits, uint32_t group);
+/* Bytes of the control block (arrival words, abort word; zero it once) and of the attention partial rows. */
+fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t *control_bytes, size_t *attention_partial_bytes);
+/* Synchronises the stream and reports whether a launch gave up on a hand-over wait (FK_ERR_HIP; the control
+ * block is reset).  The dispatcher calls it after every graph execution that holds such launches. */
+fk_status fk_xcd_check(void *workspace, fk_stream s);
+
 /* ---- dispatcher: replaces `_fusekit_runtime_native` ------------------------
  *
  * A dispatch names a kernel family by prefix ("fusekit_rmsnorm_qkv_f12" ->

@@ -1,0 +1,228 @@
+"""XCD-resident layer launches (families fusekit_xcd_attn_block / fusekit_xcd_mlp_block / fusekit_xcd_reduce)
+against the oracle, through the C ABI (dispatcher).
+
+Bar: the outputs are sums of 8 K-slices in fp32 added in a fixed order, so they are held to the per-kernel
+bar of the streaming GEMV: relative L2 <= 1e-2 against the oracle's fp32 values, element-wise equal to the
+oracle's bf16 except where the summation order crosses a rounding edge (<= 1 ulp on <= 2 % of elements)."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
+
+pytestmark = pytest.mark.gpu
+
+EPS = 1e-6
+
+
+def _dev(fk, a):
+    return fk.DeviceBuffer.from_numpy(np.ascontiguousarray(a))
+
+
+def _wargs(arg, W):
+    return [arg(W.w)] + ([] if W.bits == 16 else [arg(W.scales), arg(W.biases)])
+
+
+def _reduce_ref(partials, residual):
+    """x = T(((p0+p1)+(p2+p3)) + ((p4+p5)+(p6+p7)) + float(res)) in fp32, the launch's fixed order."""
+    p = partials.astype(np.float32)
+    acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))
+    return oracle.f32_to_bf16((acc + oracle.bf16_to_f32(residual)).astype(np.float32))
+
+
+def _close_bf16(got, ref_bits, ref_f32=None, frac=0.02, ulps=1.0):
+    f, u = bf16_mismatch(got, ref_bits)
+    assert f <= frac and u <= ulps, (f, u)
+    if ref_f32 is not None:
+        assert rel_l2(got, ref_f32) <= 1e-2
+
+
+@pytest.mark.parametrize("bits", [4, 8, 16])
+@pytest.mark.parametrize("hidden,inter,variant", [(512, 1024, 0), (2560, 9728, 1), (1024, 3072, 2)])
+def test_xcd_mlp_block(fk, bits, hidden, inter, variant):
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    if not fk.xcd_layer_supported(hidden, inter, 32, 8, 128, 256, bits, 64):
+        pytest.skip("shape not supported: " + fk.lib.fk_last_error().decode())
+    d = Dispatcher()
+    Wg, Wu, Wd = make_qweight(1, inter, hidden, bits), make_qweight(2, inter, hidden, bits), make_qweight(3, hidden, inter, bits)
+    norm_w = normal_bf16(4, hidden, 0.1, 1.0)
+    partials = (rng(5).standard_normal((8, hidden), dtype=np.float32) * 0.3).astype(np.float32)
+    res = np.stack([normal_bf16(6, hidden)] * 8)          # one copy per XCD, as a previous launch leaves it
+    dWg, dWu, dWd = (to_device(fk, W) for W in (Wg, Wu, Wd))
+    ctl_bytes, _ = fk.xcd_workspace_bytes(32, 128)
+    ctl = fk.zeros(ctl_bytes)
+    b = dict(p=_dev(fk, partials), res=_dev(fk, res), x=fk.DeviceBuffer(8 * hidden * 2), nw=_dev(fk, norm_w),
+             mid=fk.DeviceBuffer(inter * 2), out=fk.DeviceBuffer(8 * hidden * 4))
+    a = [arg(b["p"]), arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dWg.w), arg(dWu.w)]
+    if bits != 16:
+        a += [arg(dWg.scales), arg(dWu.scales), arg(dWg.biases), arg(dWu.biases)]
+    a += _wargs(arg, dWd) + [arg(b["mid"]), arg(b["out"]), arg(ctl)]
+    task = Dispatch("fusekit_xcd_mlp_block_f1", a,
+                    dict(hidden=hidden, inter=inter, n_heads=32, n_kv=8, head_dim=128, capacity=256, bits=bits, group=64,
+                         eps=EPS, variant=variant, has_partials=1, residual_per_xcd=1))
+    for rep in range(2):                                  # twice: the arrival words carry over between launches
+        d.dispatch_kernel(task)
+        fk.xcd_check(ctl)
+        x1 = _reduce_ref(partials, res[0])
+        got_x = b["x"].to_numpy(np.uint16, (8, hidden))
+        for c in range(8):
+            assert np.array_equal(got_x[c], x1), f"copy {c} of the reduced input differs"
+        mid_ref = oracle.gateup_swiglu(x1, norm_w, EPS, Wg, Wu, variant)
+        got_mid = b["mid"].to_numpy(np.uint16)
+        _close_bf16(got_mid, mid_ref, frac=0.03, ulps=2.0)   # gate and up may each sit on a rounding edge
+        # the 8 partial rows are the K-slices of W_down . mid (mid as the GPU produced it)
+        out = b["out"].to_numpy(np.float32, (8, hidden))
+        wd = oracle.dequantize(Wd).astype(np.float64) if bits != 16 else oracle.bf16_to_f32(Wd.w).astype(np.float64)
+        m64 = oracle.bf16_to_f32(got_mid).astype(np.float64)
+        sl = inter // 8
+        for c in range(8):
+            ref = wd[:, c * sl:(c + 1) * sl] @ m64[c * sl:(c + 1) * sl]
+            scale = np.abs(wd[:, c * sl:(c + 1) * sl]) @ np.abs(m64[c * sl:(c + 1) * sl])
+            assert np.all(np.abs(out[c] - ref) <= 2e-6 * scale + 1e-30), f"K-slice {c}"
+        # and the next launch's reduction of them is the down projection + residual
+        y = _reduce_ref(out, x1)
+        y_ref = oracle.linear_residual(Wd, got_mid, x1)
+        _close_bf16(y, y_ref, oracle.linear_acc(Wd, got_mid) + oracle.bf16_to_f32(x1))
+        partials = (partials * 0.5).astype(np.float32)   # second round on other inputs
+        b["p"].upload(partials)
+
+
+@pytest.mark.parametrize("bits", [4, 16])
+@pytest.mark.parametrize("n_heads,head_dim,qk_norm", [(32, 128, True), (16, 64, False), (8, 128, True), (64, 64, True)])
+def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
+    """Several decode steps through the attention launch: q / k / v rows, head norm + RoPE, cache append,
+    attention over the growing context, o_proj partial rows; against the oracle's composition of the same
+    dispatches.  Context crosses several key ranges (capacity 256 -> ranges of 64 or 128 positions)."""
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    n_kv, hidden, inter, capacity, theta = 8, 1024, 1024, 256, 1e6
+    if not fk.xcd_layer_supported(hidden, inter, n_heads, n_kv, head_dim, capacity, bits, 64):
+        pytest.skip("shape not supported: " + fk.lib.fk_last_error().decode())
+    d = Dispatcher()
+    n_q, n_kvd = n_heads * head_dim, n_kv * head_dim
+    Wq, Wk, Wv = make_qweight(1, n_q, hidden, bits, std=0.05), make_qweight(2, n_kvd, hidden, bits, std=0.05), make_qweight(3, n_kvd, hidden, bits, std=0.05)
+    Wo = make_qweight(4, hidden, n_q, bits)
+    norm_w = normal_bf16(5, hidden, 0.1, 1.0)
+    qn, kn = (normal_bf16(6, head_dim, 0.1, 1.0), normal_bf16(7, head_dim, 0.1, 1.0)) if qk_norm else (None, None)
+    dW = [to_device(fk, W) for W in (Wq, Wk, Wv, Wo)]
+    ctl_bytes, ap_bytes = fk.xcd_workspace_bytes(n_heads, head_dim)
+    ctl = fk.zeros(ctl_bytes)
+    cache_bytes = n_kv * capacity * head_dim * 2
+    b = dict(res=fk.DeviceBuffer(hidden * 2), x=fk.DeviceBuffer(8 * hidden * 2), nw=_dev(fk, norm_w),
+             q=fk.DeviceBuffer(n_q * 2), k=fk.DeviceBuffer(n_kvd * 2), v=fk.DeviceBuffer(n_kvd * 2),
+             ck=fk.zeros(cache_bytes), cv=fk.zeros(cache_bytes), kv_len=fk.zeros(4), off=fk.zeros(4), step=fk.zeros(4),
+             tab=fk.DeviceBuffer(head_dim * 4), ap=fk.DeviceBuffer(ap_bytes), out=fk.DeviceBuffer(8 * hidden * 4))
+    a = [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dW[0].w), arg(dW[1].w), arg(dW[2].w)]
+    if bits != 16:
+        a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]]
+    a += _wargs(arg, dW[3])
+    if qk_norm:
+        b["qn"], b["kn"] = _dev(fk, qn), _dev(fk, kn)
+        a += [arg(b["qn"]), arg(b["kn"])]
+    a += [arg(b["q"]), arg(b["k"]), arg(b["v"]), arg(b["ck"]), arg(b["cv"]), arg(b["kv_len"]), arg(b["tab"]), arg(b["ap"]),
+          arg(b["out"]), arg(ctl)]
+    task = Dispatch("fusekit_xcd_attn_block_f1", a,
+                    dict(hidden=hidden, inter=inter, n_heads=n_heads, n_kv=n_kv, head_dim=head_dim, capacity=capacity,
+                         bits=bits, group=64, eps=EPS, theta=theta, has_partials=0, residual_per_xcd=0, has_norm=int(qk_norm)))
+    step = Dispatch("fusekit_step_init", [arg(b["step"]), arg(b["off"]), arg(b["kv_len"]), arg(b["tab"])],
+                    dict(rope_dims=head_dim, theta=theta))
+    ck = np.zeros(n_kv * capacity * head_dim, np.uint16)
+    cv = np.zeros(n_kv * capacity * head_dim, np.uint16)
+    scale = 1.0 / np.sqrt(head_dim)
+    worst = 0.0
+    for pos in range(200):
+        x = normal_bf16(100 + pos, hidden)
+        b["res"].upload(x)
+        d.dispatch_batch([step, task])
+        if pos % 16 and pos < 190:
+            # the oracle still has to append this position's rows: it follows the GPU's own q/k/v rows, checked
+            # against the oracle's at the sampled positions below
+            qg, kg, vg = b["q"].to_numpy(np.uint16), b["k"].to_numpy(np.uint16), b["v"].to_numpy(np.uint16)
+            kr = oracle.headnorm_rope(kg, kn, n_kv, head_dim, head_dim, EPS, theta, pos) if qk_norm else \
+                oracle.rope_q(kg, n_kv, head_dim, head_dim, theta, pos)
+            oracle.kv_store(kr, vg, n_kv, head_dim, head_dim, pos, capacity, ck, cv)
+            continue
+        fk.xcd_check(ctl)
+        got_x = b["x"].to_numpy(np.uint16, (8, hidden))
+        assert all(np.array_equal(got_x[c], x) for c in range(8))
+        q_ref, k_ref, v_ref = oracle.rmsnorm_qkv(x, norm_w, EPS, Wq, Wk, Wv)
+        qg, kg, vg = b["q"].to_numpy(np.uint16), b["k"].to_numpy(np.uint16), b["v"].to_numpy(np.uint16)
+        for g, r in ((qg, q_ref), (kg, k_ref), (vg, v_ref)):
+            _close_bf16(g, r)
+        # downstream of the GPU's own projection rows, as the per-kernel tests do
+        if qk_norm:
+            qr = oracle.headnorm_rope(qg, qn, n_heads, head_dim, head_dim, EPS, theta, pos)
+            kr = oracle.headnorm_rope(kg, kn, n_kv, head_dim, head_dim, EPS, theta, pos)
+        else:
+            qr = oracle.rope_q(qg, n_heads, head_dim, head_dim, theta, pos)
+            kr = oracle.rope_q(kg, n_kv, head_dim, head_dim, theta, pos)
+        oracle.kv_store(kr, vg, n_kv, head_dim, head_dim, pos, capacity, ck, cv)
+        gck, gcv = b["ck"].to_numpy(np.uint16), b["cv"].to_numpy(np.uint16)
+        assert np.array_equal(gcv, cv), "V cache rows differ"
+        # RoPE: a normalised value that sits on a rounding edge may differ by one bf16 ulp between the fp32 and
+        # the double sum of squares, and the rotation (lo * cos - hi * sin) can nearly cancel: bound the difference by
+        # one ulp of the ROW's largest magnitude, not of the element's
+        fg, fo = oracle.bf16_to_f32(gck).reshape(-1, head_dim), oracle.bf16_to_f32(ck).reshape(-1, head_dim)
+        row_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(fo).max(axis=1, keepdims=True), 1e-30))) - 7)
+        assert np.all(np.abs(fg - fo) <= row_ulp), float(np.max(np.abs(fg - fo) / row_ulp))
+        assert np.mean(gck != ck) <= 0.01
+        ck = gck.copy()                                  # keep both sides on the same cache bits
+        att = oracle.sdpa_decode(qr, ck, cv, n_heads, n_kv, head_dim, head_dim, pos + 1, capacity, scale)
+        y_ref_acc = oracle.linear_acc(Wo, att)
+        out = b["out"].to_numpy(np.float32, (8, hidden))
+        acc = ((out[0] + out[1]) + (out[2] + out[3])) + ((out[4] + out[5]) + (out[6] + out[7]))
+        rel = float(np.linalg.norm(acc.astype(np.float64) - y_ref_acc) / np.linalg.norm(y_ref_acc))
+        worst = max(worst, rel)
+        assert rel <= 1e-2, (pos, rel)
+    print("worst rel-L2 of the o_proj sums over the sampled positions: %.3e" % worst)
+
+
+def test_xcd_reduce(fk):
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    d = Dispatcher()
+    hidden = 2560
+    partials = (rng(1).standard_normal((8, hidden), dtype=np.float32)).astype(np.float32)
+    res = normal_bf16(2, hidden)
+    bp, br, bx = _dev(fk, partials), _dev(fk, res), fk.DeviceBuffer(hidden * 2)
+    d.dispatch_kernel(Dispatch("fusekit_xcd_reduce_f1", [arg(bp), arg(br), arg(bx)], dict(hidden=hidden)))
+    assert np.array_equal(bx.to_numpy(np.uint16), _reduce_ref(partials, res))
+
+
+def test_xcd_wait_gives_up_and_reports(fk):
+    """A hand-over wait that exceeds its spin limit (forced from the host: one poll) must not hang: every
+    block drains, the error is reported and the control block is reset."""
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    cfg = DecoderConfig(n_layers=2, hidden=512, n_heads=16, n_kv=8, head_dim=64, inter=1024, vocab=512, capacity=64,
+                        qk_norm=True, xcd_spin_limit=1)
+    rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=1))
+    assert rt.xcd
+    with pytest.raises(fk.FusekitError) as e:
+        for _ in range(50):          # one poll may well succeed now and then: the limit has to bite within a few launches
+            rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, [5])
+    assert "spin limit" in str(e.value)
+    assert not rt.xcd_ctl.to_numpy(np.uint32).any()
+
+
+@pytest.mark.parametrize("bits", [4, 8, 16])
+@pytest.mark.parametrize("n_heads,head_dim,qk_norm", [(16, 64, True), (32, 128, False)])
+def test_xcd_decoder_tokens_match_oracle_and_the_per_dispatch_path(fk, bits, n_heads, head_dim, qk_norm):
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    from helpers import OracleDecoder
+    kw = dict(n_layers=3, hidden=512, n_heads=n_heads, n_kv=8, head_dim=head_dim, inter=1024, vocab=2000, capacity=128,
+              qk_norm=qk_norm, bits=bits)
+    cfg = DecoderConfig(**kw)
+    W = DecoderWeights.random_init(cfg, seed=11)
+    rt = DecoderRuntime(cfg, W)
+    assert rt.xcd and len(rt.tasks) == 2 + 2 * cfg.n_layers + 3
+    prompt = [7, 1500, 42, 3, 99]
+    got, _, _ = rt.generate(prompt, 40)
+    ref, margins = OracleDecoder(cfg, W).generate(prompt, 40)
+    old = DecoderRuntime(DecoderConfig(**kw, xcd_layers=False), W)
+    assert not old.xcd
+    got_old, _, _ = old.generate(prompt, 40)
+    print("margins:", ["%.3g" % m for m in margins])
+    # identical tokens as long as the oracle's own top-2 margin is more than one bf16 ulp of these logits (the two
+    # GPU paths sum in different orders; at a one-ulp margin either may legitimately pick the other candidate)
+    clear = next((i for i, m in enumerate(margins) if m < 0.01), len(ref))
+    assert clear >= 5
+    assert got[:clear] == ref[:clear], (got, ref)
+    assert got_old[:clear] == ref[:clear]
