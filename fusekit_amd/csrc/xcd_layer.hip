@@ -1,6 +1,21 @@
 // XCD-resident decoder layer: the attention launch and the MLP launch (see xcd_layer.hpp for the scheme).
 #include "xcd_layer.hpp"
 
+// Hook for timing probes: a probe build defines FK_PROBE_STAMPS and records a clock per block at the phase
+// boundaries of both launches; the library build leaves the macro empty.
+#ifdef FK_PROBE_STAMPS
+__device__ unsigned long long g_fk_xcd_stamp[2][512 * 16];
+#define FK_XCD_STAMP(k, i)                                                                      \
+    do {                                                                                        \
+        if (threadIdx.x == 0 || threadIdx.x == 256) g_fk_xcd_stamp[k][blockIdx.x * 16 + (i)] = wall_clock64(); \
+    } while (0)
+extern "C" __attribute__((visibility("default"))) int fk_probe_read_xcd_stamps(unsigned long long* out) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fk_xcd_stamp), sizeof(unsigned long long) * 2 * 512 * 16);
+}
+#else
+#define FK_XCD_STAMP(k, i)
+#endif
+
 namespace fk {
 namespace {
 
@@ -23,36 +38,34 @@ struct XcdSync {
 // the flag is published: every wave waits for its own memory counter, the block barrier collects the
 // waves, thread 0 publishes.  Wave 0 then polls the XCD's 64 flag words (one per lane, L1-bypassing
 // loads that are served by the XCD's L2) until every one has reached the epoch.
-__device__ __forceinline__ void xcd_barrier(XcdSync& s, uint32_t* abort_lds) {
+// One wave publishes this block's arrival (its stores of the stage must be complete) and polls the XCD's 64
+// flag words, one per lane, until every block has reached the epoch; returns false when it gave up.
+__device__ __forceinline__ bool xcd_publish_and_wait(const XcdSync& s, uint32_t lane) {
+    uint32_t* flags = s.ctl->flags + s.xcd * kXcdSlots;
+    if (lane == 0) __hip_atomic_store(flags + s.slot, s.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    uint32_t spins = 0;
+    for (;;) {
+        const uint32_t v = __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__all((int)((int32_t)(v - s.epoch) >= 0))) return true;
+        ++spins;
+        if ((spins & 255u) == 0u && __hip_atomic_load(&s.ctl->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
+            return false;
+        if (spins > s.spin_limit) {
+            if (lane == 0) __hip_atomic_store(&s.ctl->abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// Whole block; the wave that starts at thread POLL publishes and polls.
+template <int POLL>
+__device__ __forceinline__ void xcd_barrier(XcdSync& s) {
     s.epoch += 1;
     wait_memory_ops_done();
     __syncthreads();
-    uint32_t* flags = s.ctl->flags + s.xcd * kXcdSlots;
-    if (threadIdx.x == 0) __hip_atomic_store(flags + s.slot, s.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (threadIdx.x < kWave) {
-        uint32_t spins = 0;
-        bool bad = false;
-        for (;;) {
-            const uint32_t v = __hip_atomic_load(flags + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (__all((int)((int32_t)(v - s.epoch) >= 0))) break;
-            ++spins;
-            if ((spins & 255u) == 0u &&
-                __hip_atomic_load(&s.ctl->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
-                bad = true;
-                break;
-            }
-            if (spins > s.spin_limit) {
-                if (threadIdx.x == 0)
-                    __hip_atomic_store(&s.ctl->abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                bad = true;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-        if (threadIdx.x == 0) *abort_lds = bad ? 1u : 0u;
-    }
+    if (threadIdx.x >= POLL && threadIdx.x < POLL + kWave) (void)xcd_publish_and_wait(s, threadIdx.x - POLL);
     __syncthreads();
-    s.aborted = s.aborted || (*abort_lds != 0u);
 }
 
 // ---- activation staging (the chunk-interleaved LDS layout of the streaming GEMV) -------------------
@@ -115,79 +128,80 @@ __device__ __forceinline__ void stage_vector(const uint16_t* src, uint32_t n8, u
 }
 
 // ---- the input of a launch -------------------------------------------------------------------
-constexpr int kInRegs = 2;  // groups of 8 hidden elements per thread kept in registers (hidden <= 4096)
+// Run by ONE wave of the block (the control wave), while the other waves request the block's weights: a wave
+// issues its memory instructions in order, and a wave that is busy requesting megabytes of weights (the requests
+// are accepted at the rate memory delivers) would not get to the hand-over before they have all gone out.
+//   stage A  this block's rows of x = T(sum of the partial rows + residual) -> this XCD's copy; their sum of squares
+//   hand-over (every block of the XCD has published its rows)
+//   stage B  the whole normalised vector, T(w * T(x * r)), staged into LDS for the projections
+constexpr int kCtlRegs = 8;  // groups of 8 hidden elements per lane of the control wave (hidden <= 4096)
 
-struct InputFetch {
-    float p[kXcds];
-    uint32_t res;
-    uint4 nw[kInRegs];
-};
-
-// Issues the loads of this block's share of the reduction and of the norm weights.  Called first in the
-// kernel: loads return in issue order and these are needed first.
-__device__ __forceinline__ void input_fetch(const XcdInput& in, uint32_t xcd, uint32_t slot, InputFetch& f) {
+template <WKind KIND, int PROBE>
+__device__ __forceinline__ void input_control(const XcdInput& in, XcdSync& sync, uint32_t xcd, uint32_t slot, uint32_t lane,
+                                              uint4* xs, float* sx, uint32_t cs) {
     const uint32_t r0 = slot * in.rows_per_block;
-    uint32_t row = r0 + threadIdx.x;
-    if (threadIdx.x >= in.rows_per_block || row >= in.hidden) row = r0 < in.hidden ? r0 : 0u;  // clamped: straight-line loads
-    const float* p = in.partials ? in.partials : reinterpret_cast<const float*>(in.residual);
+    const bool mine = lane < in.rows_per_block && r0 + lane < in.hidden;
+    const uint32_t row = mine ? r0 + lane : (r0 < in.hidden ? r0 : 0u);  // clamped: straight-line loads
+    float p[kXcds];
 #pragma unroll
-    for (uint32_t j = 0; j < kXcds; ++j) f.p[j] = in.partials ? p[(size_t)j * in.hidden + row] : 0.f;
-    f.res = in.residual[(size_t)xcd * in.residual_stride + row];
+    for (uint32_t j = 0; j < kXcds; ++j) p[j] = in.partials ? in.partials[(size_t)j * in.hidden + row] : 0.f;
+    const uint32_t res = in.residual[(size_t)xcd * in.residual_stride + row];
     const uint4* w8 = reinterpret_cast<const uint4*>(in.norm_w);
     const uint32_t n8 = in.hidden >> 3;
+    uint4 nw[kCtlRegs];
 #pragma unroll
-    for (int i = 0; i < kInRegs; ++i) {
-        const uint32_t t = threadIdx.x + i * kBlock;
-        f.nw[i] = w8[t < n8 ? t : 0u];
+    for (int i = 0; i < kCtlRegs; ++i) {
+        const uint32_t t = lane + i * kWave;
+        nw[i] = w8[t < n8 ? t : 0u];
     }
-}
-
-// Stage A: this block's rows of x = T(sum of the partial rows + residual), written to this XCD's copy, and the
-// block's sum of squares.  Then the hand-over, then stage B: every block stages the whole normalised vector.
-template <WKind KIND>
-__device__ __forceinline__ void input_finish(const XcdInput& in, XcdSync& sync, const InputFetch& f, uint4* xs, float* sx,
-                                             float* scratch, uint32_t cs) {
-    const uint32_t r0 = sync.slot * in.rows_per_block;
-    const uint32_t row = r0 + threadIdx.x;
-    const bool mine = threadIdx.x < in.rows_per_block && row < in.hidden;
     float sq = 0.f;
     if (mine) {
         // fixed order: ((p0 + p1) + (p2 + p3)) + ((p4 + p5) + (p6 + p7)), then the residual, one rounding
-        const float acc = ((f.p[0] + f.p[1]) + (f.p[2] + f.p[3])) + ((f.p[4] + f.p[5]) + (f.p[6] + f.p[7]));
-        const uint32_t xb = f32_to_bf16_bits(acc + bf16_bits_to_f32(f.res));
-        in.x_out[(size_t)sync.xcd * in.hidden + row] = (uint16_t)xb;
+        const float acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+        const uint32_t xb = f32_to_bf16_bits(acc + bf16_bits_to_f32(res));
+        in.x_out[(size_t)xcd * in.hidden + row] = (uint16_t)xb;
         const float xv = bf16_bits_to_f32(xb);
         sq = xv * xv;
     }
-    sq = block_sum<kBlock>(sq, scratch);
-    if (threadIdx.x == 0) sync.ctl->ssq[sync.xcd * kXcdSlots + sync.slot] = sq;
-    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
-    // sum of squares over the whole vector: every wave adds the 64 block sums in the same order
-    float ss = ld_f32<true>(&sync.ctl->ssq[sync.xcd * kXcdSlots + (threadIdx.x & (kWave - 1))]);
+    FK_XCD_STAMP(PROBE, 2);
+    sq = wave_sum(sq);
+    if (lane == 0) sync.ctl->ssq[xcd * kXcdSlots + slot] = sq;
+    wait_memory_ops_done();
+    FK_XCD_STAMP(PROBE, 3);
+    (void)xcd_publish_and_wait(sync, lane);
+    FK_XCD_STAMP(PROBE, 4);
+    // sum of squares over the whole vector: the 64 block sums in a fixed order
+    float ss = ld_f32<true>(&sync.ctl->ssq[xcd * kXcdSlots + lane]);
     ss = wave_sum(ss);
     const float r = 1.0f / sqrtf(ss / (float)in.hidden + in.eps);
-    const uint4* x8 = reinterpret_cast<const uint4*>(in.x_out + (size_t)sync.xcd * in.hidden);
-    const uint32_t n8 = in.hidden >> 3;
-    const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
+    const uint4* x8 = reinterpret_cast<const uint4*>(in.x_out + (size_t)xcd * in.hidden);
+    uint4 xv[kCtlRegs];
 #pragma unroll
-    for (int i = 0; i < kInRegs; ++i) {
-        const uint32_t t = threadIdx.x + i * kBlock;
-        if ((threadIdx.x & ~(uint32_t)(kWave - 1)) + i * kBlock < n8_up) {
-            const bool live = t < n8;
-            const uint4 v = ld_u128<true>(x8 + (live ? t : 0u));
-            stage_emit<KIND>(xs, sx, cs, t, live, v, f.nw[i], r, true);
-        }
+    for (int i = 0; i < kCtlRegs; ++i) {
+        const uint32_t t = lane + i * kWave;
+        xv[i] = ld_u128<true>(x8 + (t < n8 ? t : 0u));
     }
-    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kCtlRegs; ++i) {
+        const uint32_t t = lane + i * kWave;
+        if ((uint32_t)i * kWave < n8) stage_emit<KIND>(xs, sx, cs, t, t < n8, xv[i], nw[i], r, true);
+    }
 }
 
 // ---- projection tiles ----------------------------------------------------------------------------
 // A tile: rows [row0, row0 + rows) x chunks [col0, col0 + cs) of a matrix; flat position p = row * cs + col.
 // A pass covers NL * 256 positions; positions past the tile read the tile's first chunk (in bounds).
+// Weights are requested as 16-byte chunks, one per lane and position (1 KiB contiguous per wave instruction).
+// Scales and biases are NOT fetched per chunk (two more memory instructions per chunk, each as expensive to
+// issue as the 16-byte one): the block fetches the tile's groups once, kMetaRegs per thread, and parks them
+// in LDS as (scale | bias << 16) words.
 template <int NL>
 struct TileRegs {
     uint4 w[NL];
-    uint32_t sc[NL], bi[NL];
+};
+constexpr int kMetaRegs = 3;  // quantisation groups of a tile per thread: tiles of at most 768 groups per matrix
+struct MetaRegs {
+    uint32_t s[kMetaRegs], b[kMetaRegs];
 };
 
 struct Tile {
@@ -195,47 +209,105 @@ struct Tile {
     float inv_cs;
 };
 
-template <WKind KIND, int NL>
-__device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, uint32_t pass, TileRegs<NL>& r) {
+// SN threads stream a tile; `ti` is the calling thread's index among them.
+template <WKind KIND, int NL, int SN>
+__device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, uint32_t pass, uint32_t ti, TileRegs<NL>& r) {
     const uint32_t total = t.rows * t.cs;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-        const uint32_t pos = (pass * NL + j) * kBlock + threadIdx.x;
+        const uint32_t pos = (pass * NL + j) * SN + ti;
         const uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
         const uint32_t col = pos - row * t.cs;
         const size_t idx = pos < total ? (size_t)(t.row0 + row) * m.cpr + t.col0 + col : (size_t)t.row0 * m.cpr + t.col0;
         r.w[j] = m.w[idx];
-        if constexpr (KIND != W_BF16) {
-            const size_t g = idx >> m.gshift;
-            r.sc[j] = m.sc[g];
-            r.bi[j] = m.bi[g];
+    }
+}
+
+// Group gi of the tile = (row gi / gpr, group gi % gpr of the row's slice), gpr groups per row slice.
+template <WKind KIND, int SN>
+__device__ __forceinline__ void meta_fetch(const XcdMat& m, const Tile& t, uint32_t ti, MetaRegs& r) {
+    if constexpr (KIND != W_BF16) {
+        const uint32_t gpr = t.cs >> m.gshift, total = t.rows * gpr;
+        const float inv = 1.0f / (float)gpr;
+        const size_t g0 = (size_t)t.row0 * (m.cpr >> m.gshift) + (t.col0 >> m.gshift);
+#pragma unroll
+        for (int k = 0; k < kMetaRegs; ++k) {
+            const uint32_t gi = k * SN + ti;
+            const uint32_t row = (uint32_t)(((float)gi + 0.5f) * inv);
+            const size_t e = gi < total ? g0 + (size_t)row * (m.cpr >> m.gshift) + (gi - row * gpr) : g0;
+            r.s[k] = m.sc[e];
+            r.b[k] = m.bi[e];
         }
+    }
+}
+template <WKind KIND, int SN>
+__device__ __forceinline__ void meta_store(const MetaRegs& r, uint32_t ti, uint32_t* meta) {
+    if constexpr (KIND != W_BF16) {
+#pragma unroll
+        for (int k = 0; k < kMetaRegs; ++k) meta[k * SN + ti] = r.s[k] | (r.b[k] << 16);
     }
 }
 
 // One fp32 partial per chunk into part[pos] (padded to whole passes, so no guard is needed).
-template <WKind KIND, int NL>
-__device__ __forceinline__ void tile_partials(const Tile& t, uint32_t pass, const TileRegs<NL>& r, const uint4* xs,
-                                              const float* sx, float* part) {
+template <WKind KIND, int NL, int SN>
+__device__ __forceinline__ void tile_partials(const XcdMat& m, const Tile& t, uint32_t pass, uint32_t ti, const TileRegs<NL>& r,
+                                              const uint4* xs, const float* sx, const uint32_t* meta, float* part) {
+    const uint32_t gpr = t.cs >> m.gshift;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-        const uint32_t pos = (pass * NL + j) * kBlock + threadIdx.x;
-        const uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
+        const uint32_t pos = (pass * NL + j) * SN + ti;
+        uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
         uint32_t col = pos - row * t.cs;
-        col = col < t.cs ? col : 0u;
-        part[pos] = chunk_partial<KIND>(r.w[j], r.sc[j], r.bi[j], xs, sx, col, t.cs);
+        if (row >= t.rows) row = 0u, col = 0u;
+        uint32_t sb = 0, bb = 0;
+        if constexpr (KIND != W_BF16) {
+            const uint32_t mw = meta[row * gpr + (col >> m.gshift)];
+            sb = mw & 0xffffu;
+            bb = mw >> 16;
+        }
+        part[pos] = chunk_partial<KIND>(r.w[j], sb, bb, xs, sx, col, t.cs);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
 
-// All passes of a tile whose first pass is already in `r`.
-template <WKind KIND, int NL>
-__device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, TileRegs<NL>& r, const uint4* xs, const float* sx,
-                                         float* part) {
-    const uint32_t n_pass = (t.rows * t.cs + NL * kBlock - 1) / (NL * kBlock);
-    for (uint32_t p = 0; p < n_pass; ++p) {
-        if (p) tile_load<KIND, NL>(m, t, p, r);
-        tile_partials<KIND, NL>(t, p, r, xs, sx, part);
+// All passes of a tile whose first pass is already in `r0`: pass p + 1 is requested before pass p is consumed.
+template <WKind KIND, int NL, int SN>
+__device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, uint32_t ti, TileRegs<NL>& r0, const uint4* xs,
+                                         const float* sx, const uint32_t* meta, float* part) {
+    const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
+    TileRegs<NL> r1;
+    for (uint32_t p = 0; p < n_pass; p += 2) {
+        if (p + 1 < n_pass) tile_load<KIND, NL, SN>(m, t, p + 1, ti, r1);
+        tile_partials<KIND, NL, SN>(m, t, p, ti, r0, xs, sx, meta, part);
+        if (p + 1 < n_pass) {
+            if (p + 2 < n_pass) tile_load<KIND, NL, SN>(m, t, p + 2, ti, r0);
+            tile_partials<KIND, NL, SN>(m, t, p + 1, ti, r1, xs, sx, meta, part);
+        }
+    }
+}
+
+// The gate / up pair: both matrices' passes interleaved, so that one pass of each is in flight while one is consumed.
+template <WKind KIND, int NL, int SN>
+__device__ __forceinline__ void tile_run_pair(const XcdMat& ma, const XcdMat& mb, const Tile& t, uint32_t ti, TileRegs<NL>& a0,
+                                              TileRegs<NL>& b0, const uint4* xs, const float* sx, const uint32_t* meta_a,
+                                              const uint32_t* meta_b, float* part_a, float* part_b) {
+    const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
+    TileRegs<NL> a1, b1;
+    for (uint32_t p = 0; p < n_pass; p += 2) {
+        if (p + 1 < n_pass) {
+            tile_load<KIND, NL, SN>(ma, t, p + 1, ti, a1);
+            tile_load<KIND, NL, SN>(mb, t, p + 1, ti, b1);
+        }
+        tile_partials<KIND, NL, SN>(ma, t, p, ti, a0, xs, sx, meta_a, part_a);
+        tile_partials<KIND, NL, SN>(mb, t, p, ti, b0, xs, sx, meta_b, part_b);
+        if (p + 1 < n_pass) {
+            if (p + 2 < n_pass) {
+                tile_load<KIND, NL, SN>(ma, t, p + 2, ti, a0);
+                tile_load<KIND, NL, SN>(mb, t, p + 2, ti, b0);
+            }
+            tile_partials<KIND, NL, SN>(ma, t, p + 1, ti, a1, xs, sx, meta_a, part_a);
+            tile_partials<KIND, NL, SN>(mb, t, p + 1, ti, b1, xs, sx, meta_b, part_b);
+        }
     }
 }
 
@@ -280,29 +352,34 @@ __device__ __forceinline__ Tile make_tile(uint32_t row0, uint32_t rows, uint32_t
 //   xs   uint4 [PIECES * cs_max]      staged activations
 //   sx   [cs_max]                     per-chunk sums
 //   work [work_floats]                chunk partials of a tile (two segments for gate / up), or the attention's LDS
+//   meta uint32 [3][kMetaRegs * 256]  (scale | bias << 16) of the groups of up to three tiles
 //   att  uint16 [att_elems]           merged attention rows (attention launch)
 //   scratch [16]
 struct LdsPlan {
     uint32_t cs_max, work_floats, att_elems;
 };
+constexpr uint32_t kMetaWords = kMetaRegs * kBlock;  // per matrix (the streaming threads never exceed kBlock)
 template <WKind KIND>
 __host__ __device__ inline uint32_t xcd_lds_bytes(const LdsPlan& p) {
-    return ChunkTraits<KIND>::kPieces * p.cs_max * 16u + p.cs_max * 4u + p.work_floats * 4u +
+    return ChunkTraits<KIND>::kPieces * p.cs_max * 16u + p.cs_max * 4u + p.work_floats * 4u + 3u * kMetaWords * 4u +
            ((p.att_elems * 2u + 15u) & ~15u) + 64u;
 }
 
 }  // namespace
 
 // =============================================================================================== MLP launch
+// 320 threads: waves 0..3 stream and multiply, wave 4 is the control wave (input reduction, hand-over polls).
+constexpr int kMlpBlock = kBlock + kWave;
+
 template <WKind KIND, int NLA, int NLB>
-__global__ __launch_bounds__(kBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) {
+__global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) {
     extern __shared__ uint4 lds_raw[];
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     uint4* xs = lds_raw;
     float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
     float* work = sx + cs_max;
-    float* scratch = work + work_floats;
+    uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]
 
     XcdSync sync;
     sync.ctl = a.ctl;
@@ -315,10 +392,10 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) 
     sync.spin_limit = a.spin_limit;
     sync.aborted = false;
     sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t tid = threadIdx.x;
+    const bool streams = tid < (uint32_t)kBlock;
 
-    InputFetch fin;
-    input_fetch(a.in, sync.xcd, sync.slot, fin);
-
+    FK_XCD_STAMP(1, 0);
     const uint32_t per_xcd = a.inter / kXcds;
     const uint32_t gu0 = sync.slot * a.gu_rows;
     const uint32_t gu_n = gu0 < per_xcd ? ((per_xcd - gu0) < a.gu_rows ? (per_xcd - gu0) : a.gu_rows) : 0u;
@@ -327,52 +404,76 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) 
     const uint32_t d_n = d0 < a.in.hidden ? ((a.in.hidden - d0) < a.down_rows ? (a.in.hidden - d0) : a.down_rows) : 0u;
     const Tile td = make_tile(d0, d_n, sync.xcd * a.down_cs, a.down_cs);
 
-    // every weight this block will use is requested now; the hand-overs below only gate arithmetic
+    MetaRegs mg, mu, md;
     TileRegs<NLA> rg, ru;
     TileRegs<NLB> rd;
-    tile_load<KIND, NLA>(a.gate, tg, 0, rg);
-    tile_load<KIND, NLA>(a.up, tg, 0, ru);
-    tile_load<KIND, NLB>(a.down, td, 0, rd);
-
-    input_finish<KIND>(a.in, sync, fin, xs, sx, scratch, a.gate.cpr);
+    sync.epoch += 1;  // the input hand-over
+    if (streams) {
+        // Requested now, in the order of use: the groups' scales and biases, the first pass of gate / up, all of
+        // this block's down_proj slice.  The hand-overs only gate arithmetic; the later passes of gate / up
+        // stream while the earlier ones are consumed.
+        meta_fetch<KIND, kBlock>(a.gate, tg, tid, mg);
+        meta_fetch<KIND, kBlock>(a.up, tg, tid, mu);
+        meta_fetch<KIND, kBlock>(a.down, td, tid, md);
+        tile_load<KIND, NLA, kBlock>(a.gate, tg, 0, tid, rg);
+        tile_load<KIND, NLA, kBlock>(a.up, tg, 0, tid, ru);
+        tile_load<KIND, NLB, kBlock>(a.down, td, 0, tid, rd);
+        FK_XCD_STAMP(1, 1);
+        meta_store<KIND, kBlock>(mg, tid, meta);
+        meta_store<KIND, kBlock>(mu, tid, meta + kMetaWords);
+        meta_store<KIND, kBlock>(md, tid, meta + 2 * kMetaWords);
+    } else {
+        input_control<KIND, 1>(a.in, sync, sync.xcd, sync.slot, tid - kBlock, xs, sx, a.gate.cpr);
+    }
+    __syncthreads();
+    FK_XCD_STAMP(1, 5);
 
     // ---- gate / up rows of this XCD's slice, SwiGLU ----
     const uint32_t seg = (gu_n * a.gate.cpr + NLA * kBlock - 1) / (NLA * kBlock) * (NLA * kBlock);
-    if (gu_n) {
-        tile_run<KIND, NLA>(a.gate, tg, rg, xs, sx, work);
-        tile_run<KIND, NLA>(a.up, tg, ru, xs, sx, work + seg);
-    }
+    if (streams && gu_n)
+        tile_run_pair<KIND, NLA, kBlock>(a.gate, a.up, tg, tid, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg);
+    FK_XCD_STAMP(1, 6);
     __syncthreads();
-    if (gu_n) {
+    if (streams && gu_n) {
         uint16_t* mid = a.mid + (size_t)sync.xcd * per_xcd + gu0;
         const int variant = a.swiglu_variant;
         tile_rows<true>(tg, work, work + seg,
                         [&](uint32_t r, float s0, float s1) { mid[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
     }
-    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+    FK_XCD_STAMP(1, 7);
+    xcd_barrier<kBlock>(sync);
+    FK_XCD_STAMP(1, 8);
 
     // ---- down_proj over this XCD's K-slice: fp32 partial row ----
-    stage_vector<KIND>(a.mid + (size_t)sync.xcd * per_xcd, per_xcd >> 3, a.down_cs, xs, sx);
+    if (streams) stage_vector<KIND>(a.mid + (size_t)sync.xcd * per_xcd, per_xcd >> 3, a.down_cs, xs, sx);
     __syncthreads();
-    if (d_n) tile_run<KIND, NLB>(a.down, td, rd, xs, sx, work);
+    FK_XCD_STAMP(1, 9);
+    if (streams && d_n) tile_run<KIND, NLB, kBlock>(a.down, td, tid, rd, xs, sx, meta + 2 * kMetaWords, work);
     __syncthreads();
-    if (d_n) {
+    FK_XCD_STAMP(1, 10);
+    if (streams && d_n) {
         float* out = a.out_partials + (size_t)sync.xcd * a.in.hidden + d0;
         tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { out[r] = s0; });
     }
+    FK_XCD_STAMP(1, 11);
 }
 
 // =============================================================================================== attention launch
+// 256 threads (the attention phase wants exactly four waves): until the input is staged wave 0 is the control
+// wave and waves 1..3 request the weights; afterwards all four are peers.
+constexpr int kAttnStream = kBlock - kWave;
+
 template <WKind KIND, int NLA, int NLB>
 __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a) {
     extern __shared__ uint4 lds_raw[];
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats, att_elems = a.att_elems;
+    (void)att_elems;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     uint4* xs = lds_raw;
     float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
     float* work = sx + cs_max;
-    uint16_t* att = reinterpret_cast<uint16_t*>(work + work_floats);
-    float* scratch = reinterpret_cast<float*>(reinterpret_cast<char*>(att) + ((att_elems * 2u + 15u) & ~15u));
+    uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]; two used
+    uint16_t* att = reinterpret_cast<uint16_t*>(meta + 3 * kMetaWords);
 
     XcdSync sync;
     sync.ctl = a.ctl;
@@ -382,15 +483,16 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     sync.aborted = false;
     sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t kv_len0 = *a.sdpa.kv_len_ptr;
+    const uint32_t tid = threadIdx.x;
+    const bool streams = tid >= (uint32_t)kWave;
+    const uint32_t ti = tid - kWave;  // index among the streaming threads
 
-    InputFetch fin;
-    input_fetch(a.in, sync.xcd, sync.slot, fin);
-
+    FK_XCD_STAMP(0, 0);
     // tile of the q / k / v projections: the XCD's q rows first, then its k rows, then its v rows
-    const uint32_t R = a.qkv_tile_rows, ti = sync.slot;
-    const bool has_tile = ti < a.q_tiles + 2 * a.kv_tiles;
-    const uint32_t part_id = ti < a.q_tiles ? 0u : (ti < a.q_tiles + a.kv_tiles ? 1u : 2u);
-    const uint32_t tl = part_id == 0 ? ti : (part_id == 1 ? ti - a.q_tiles : ti - a.q_tiles - a.kv_tiles);
+    const uint32_t R = a.qkv_tile_rows, tix = sync.slot;
+    const bool has_tile = tix < a.q_tiles + 2 * a.kv_tiles;
+    const uint32_t part_id = tix < a.q_tiles ? 0u : (tix < a.q_tiles + a.kv_tiles ? 1u : 2u);
+    const uint32_t tl = part_id == 0 ? tix : (part_id == 1 ? tix - a.q_tiles : tix - a.q_tiles - a.kv_tiles);
     const uint32_t part_rows = part_id == 0 ? a.q_rows : a.kv_rows;
     const uint32_t pr0 = tl * R;
     const uint32_t pr_n = has_tile ? ((part_rows - pr0) < R ? (part_rows - pr0) : R) : 0u;
@@ -400,21 +502,34 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     const uint32_t o_n = o0 < a.in.hidden ? ((a.in.hidden - o0) < a.o_rows ? (a.in.hidden - o0) : a.o_rows) : 0u;
     const Tile to = make_tile(o0, o_n, sync.xcd * a.o_cs, a.o_cs);
 
+    MetaRegs mmq, mmo;
     TileRegs<NLA> rq;
     TileRegs<NLB> ro;
-    tile_load<KIND, NLA>(mq, tq, 0, rq);
-    tile_load<KIND, NLB>(a.wo, to, 0, ro);
-
-    input_finish<KIND>(a.in, sync, fin, xs, sx, scratch, a.wq.cpr);
+    sync.epoch += 1;  // the input hand-over
+    if (streams) {
+        meta_fetch<KIND, kAttnStream>(mq, tq, ti, mmq);
+        meta_fetch<KIND, kAttnStream>(a.wo, to, ti, mmo);
+        tile_load<KIND, NLA, kAttnStream>(mq, tq, 0, ti, rq);
+        tile_load<KIND, NLB, kAttnStream>(a.wo, to, 0, ti, ro);
+        FK_XCD_STAMP(0, 1);
+        meta_store<KIND, kAttnStream>(mmq, ti, meta);
+        meta_store<KIND, kAttnStream>(mmo, ti, meta + kMetaWords);
+    } else {
+        input_control<KIND, 0>(a.in, sync, sync.xcd, sync.slot, tid, xs, sx, a.wq.cpr);
+    }
+    __syncthreads();
+    FK_XCD_STAMP(0, 5);
 
     // ---- q / k / v rows of this XCD's KV head ----
-    if (pr_n) tile_run<KIND, NLA>(mq, tq, rq, xs, sx, work);
+    if (streams && pr_n) tile_run<KIND, NLA, kAttnStream>(mq, tq, ti, rq, xs, sx, meta, work);
     __syncthreads();
     if (pr_n) {
         uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
         tile_rows<false>(tq, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
     }
-    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+    FK_XCD_STAMP(0, 6);
+    xcd_barrier<0>(sync);
+    FK_XCD_STAMP(0, 7);
 
     // ---- head norm + RoPE + cache append + attention: block = (query head of the group, key range) ----
     const uint32_t G = a.sdpa.n_heads / a.sdpa.n_kv;
@@ -423,7 +538,9 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
         if (split < a.sdpa.n_splits)
             sdpa_block<1, 2, SdpaArgs, 0, true, true>(a.sdpa, kv_len0, split, sync.xcd, gz, G, work);
     }
-    xcd_barrier(sync, reinterpret_cast<uint32_t*>(scratch + 8));
+    FK_XCD_STAMP(0, 8);
+    xcd_barrier<0>(sync);
+    FK_XCD_STAMP(0, 9);
 
     // ---- merge the ranges of each of the group's heads (range order), rows to LDS ----
     {
@@ -465,6 +582,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
         }
     }
     __syncthreads();
+    FK_XCD_STAMP(0, 10);
     // ---- o_proj over this XCD's K-slice (its heads' columns): fp32 partial row ----
     {
         const uint32_t n8 = (G * a.sdpa.v_dim) >> 3, n8_up = (n8 + kWave - 1) / kWave * kWave;
@@ -476,12 +594,14 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
         }
     }
     __syncthreads();
-    if (o_n) tile_run<KIND, NLB>(a.wo, to, ro, xs, sx, work);
+    if (streams && o_n) tile_run<KIND, NLB, kAttnStream>(a.wo, to, ti, ro, xs, sx, meta + kMetaWords, work);
     __syncthreads();
+    FK_XCD_STAMP(0, 11);
     if (o_n) {
         float* out = a.out_partials + (size_t)sync.xcd * a.in.hidden + o0;
         tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { out[r] = s0; });
     }
+    FK_XCD_STAMP(0, 12);
 }
 
 __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
@@ -497,7 +617,7 @@ __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs 
 // =============================================================================================== host side
 namespace {
 
-constexpr int kNlQkv = 5, kNlO = 3, kNlGu = 6, kNlDown = 6;
+constexpr int kNlQkv = 6, kNlO = 4, kNlGu = 2, kNlDown = 6;  // 16-byte requests per streaming thread and pass
 
 uint32_t ilog2u(uint32_t v) {
     uint32_t r = 0;
@@ -568,10 +688,20 @@ fk_status xcd_layer_supported(const XcdLayerShape& s) {
     const uint32_t G = s.n_heads / s.n_kv;
     if (G != 1 && G != 2 && G != 4 && G != 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: 1, 2, 4 or 8 query heads per KV head");
     if (s.head_dim != 64 && s.head_dim != 128) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: head_dim must be 64 or 128");
-    if (s.hidden % 64 || s.hidden > (uint32_t)kInRegs * kBlock * 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: hidden must be a multiple of 64, at most 4096");
+    if (s.hidden % 64 || s.hidden > (uint32_t)kCtlRegs * kWave * 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: hidden must be a multiple of 64, at most 4096");
     if ((G * s.head_dim) % unit) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a KV head's query columns must be whole quantisation groups");
     if (s.inter % (kXcds * unit) || s.inter % (kXcds * 8)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: intermediate / 8 must be whole quantisation groups");
     if (s.capacity == 0) return set_error(FK_ERR_INVALID, "xcd layer: zero cache capacity");
+    if (s.bits != 16) {
+        // a tile's quantisation groups are fetched kMetaRegs per thread
+        const uint32_t budget = kMetaRegs * kBlock, n_q = s.n_heads * s.head_dim;
+        uint32_t R = 1;
+        while (ceil_div(G * s.head_dim, R) + 2 * ceil_div(s.head_dim, R) > kXcdSlots) ++R;
+        if (R * (s.hidden / s.group) > budget || ceil_div(s.hidden, kXcdSlots) * (n_q / kXcds / s.group) > budget ||
+            ceil_div(s.inter / kXcds, kXcdSlots) * (s.hidden / s.group) > budget ||
+            ceil_div(s.hidden, kXcdSlots) * (s.inter / kXcds / s.group) > budget)
+            return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a block's tile holds more quantisation groups than the kernel fetches");
+    }
     return FK_OK;
 }
 
@@ -611,7 +741,7 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     out->func = s.bits == 4 ? mlp_func<W_Q4>() : (s.bits == 8 ? mlp_func<W_Q8>() : mlp_func<W_BF16>());
     FK_TRY(set_lds_limit(out->func, lds));
     out->grid = dim3(kXcdGrid, 1, 1);
-    out->block = dim3(kBlock, 1, 1);
+    out->block = dim3(kMlpBlock, 1, 1);
     out->shmem = lds;
     a.cs_max = lp.cs_max;
     a.work_floats = lp.work_floats;
@@ -685,7 +815,7 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     a.out_partials = rq.out_partials;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
-    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
+    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kAttnStream) * nl * kAttnStream; };
     LdsPlan lp;
     lp.cs_max = a.wq.cpr > a.o_cs ? a.wq.cpr : a.o_cs;
     uint32_t wf = padded(R * a.wq.cpr, kNlQkv);

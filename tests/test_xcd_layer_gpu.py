@@ -220,9 +220,9 @@ def test_xcd_decoder_tokens_match_oracle_and_the_per_dispatch_path(fk, bits, n_h
     assert not old.xcd
     got_old, _, _ = old.generate(prompt, 40)
     print("margins:", ["%.3g" % m for m in margins])
-    # identical tokens as long as the oracle's own top-2 margin is more than one bf16 ulp of these logits (the two
-    # GPU paths sum in different orders; at a one-ulp margin either may legitimately pick the other candidate)
-    clear = next((i for i, m in enumerate(margins) if m < 0.01), len(ref))
-    assert clear >= 5
-    assert got[:clear] == ref[:clear], (got, ref)
-    assert got_old[:clear] == ref[:clear]
+    # identical tokens; the runs may part only at a step where the oracle's own top-2 margin is at most one bf16 ulp
+    # of these logits (the two GPU paths and the oracle sum in different orders: at such a step any of them may
+    # legitimately pick the other candidate, and the continuations then differ)
+    for name_, seq in (("xcd", got), ("per-dispatch", got_old)):
+        i = next((i for i, (g, r) in enumerate(zip(seq, ref)) if g != r), None)
+        assert i is None or margins[i] < 0.01, f"{name_}: step {i}: gpu {seq[i]} oracle {ref[i]} at margin {margins[i]}"
