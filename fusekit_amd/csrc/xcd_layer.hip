@@ -170,10 +170,7 @@ __device__ __forceinline__ void input_control(const XcdInput& in, XcdSync& sync,
     FK_XCD_STAMP(PROBE, 3);
     (void)xcd_publish_and_wait(sync, lane);
     FK_XCD_STAMP(PROBE, 4);
-    // sum of squares over the whole vector: the 64 block sums in a fixed order
-    float ss = ld_f32<true>(&sync.ctl->ssq[xcd * kXcdSlots + lane]);
-    ss = wave_sum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)in.hidden + in.eps);
+    // the whole vector and the 64 block sums of squares (added in a fixed order) are requested together
     const uint4* x8 = reinterpret_cast<const uint4*>(in.x_out + (size_t)xcd * in.hidden);
     uint4 xv[kCtlRegs];
 #pragma unroll
@@ -181,6 +178,9 @@ __device__ __forceinline__ void input_control(const XcdInput& in, XcdSync& sync,
         const uint32_t t = lane + i * kWave;
         xv[i] = ld_u128<true>(x8 + (t < n8 ? t : 0u));
     }
+    float ss = ld_f32<true>(&sync.ctl->ssq[xcd * kXcdSlots + lane]);
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)in.hidden + in.eps);
 #pragma unroll
     for (int i = 0; i < kCtlRegs; ++i) {
         const uint32_t t = lane + i * kWave;
@@ -209,16 +209,38 @@ struct Tile {
     float inv_cs;
 };
 
-// SN threads stream a tile; `ti` is the calling thread's index among them.
-template <WKind KIND, int NL, int SN>
-__device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, uint32_t pass, uint32_t ti, TileRegs<NL>& r) {
-    const uint32_t total = t.rows * t.cs;
+// SN threads stream a tile; `ti` is the calling thread's index among them.  A thread's position in pass p is
+// (p * NL + j) * SN + ti; its (row, column) is worked out once per tile and advanced from pass to pass.
+template <int NL>
+struct TilePos {
+    uint32_t row[NL], col[NL];
+};
+template <int NL, int SN>
+__device__ __forceinline__ void tile_pos_init(const Tile& t, uint32_t ti, TilePos<NL>& p) {
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-        const uint32_t pos = (pass * NL + j) * SN + ti;
-        const uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
-        const uint32_t col = pos - row * t.cs;
-        const size_t idx = pos < total ? (size_t)(t.row0 + row) * m.cpr + t.col0 + col : (size_t)t.row0 * m.cpr + t.col0;
+        const uint32_t pos = j * SN + ti;
+        p.row[j] = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
+        p.col[j] = pos - p.row[j] * t.cs;
+    }
+}
+template <int NL, int SN>
+__device__ __forceinline__ void tile_pos_next(const Tile& t, uint32_t step_r, uint32_t step_c, TilePos<NL>& p) {
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const uint32_t c = p.col[j] + step_c;
+        const bool wrap = c >= t.cs;
+        p.col[j] = wrap ? c - t.cs : c;
+        p.row[j] += step_r + (wrap ? 1u : 0u);
+    }
+}
+
+template <WKind KIND, int NL>
+__device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, const TilePos<NL>& p, TileRegs<NL>& r) {
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const bool in = p.row[j] < t.rows;
+        const size_t idx = (size_t)(t.row0 + (in ? p.row[j] : 0u)) * m.cpr + t.col0 + (in ? p.col[j] : 0u);
         r.w[j] = m.w[idx];
     }
 }
@@ -248,72 +270,98 @@ __device__ __forceinline__ void meta_store(const MetaRegs& r, uint32_t ti, uint3
     }
 }
 
-// One fp32 partial per chunk into part[pos] (padded to whole passes, so no guard is needed).
-template <WKind KIND, int NL, int SN>
-__device__ __forceinline__ void tile_partials(const XcdMat& m, const Tile& t, uint32_t pass, uint32_t ti, const TileRegs<NL>& r,
+// One fp32 partial per chunk into part[row * cs + col]; positions past the tile are dropped.
+template <WKind KIND, int NL>
+__device__ __forceinline__ void tile_partials(const XcdMat& m, const Tile& t, const TilePos<NL>& p, const TileRegs<NL>& r,
                                               const uint4* xs, const float* sx, const uint32_t* meta, float* part) {
     const uint32_t gpr = t.cs >> m.gshift;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-        const uint32_t pos = (pass * NL + j) * SN + ti;
-        uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
-        uint32_t col = pos - row * t.cs;
-        if (row >= t.rows) row = 0u, col = 0u;
+        const bool in = p.row[j] < t.rows;
+        const uint32_t row = in ? p.row[j] : 0u, col = in ? p.col[j] : 0u;
         uint32_t sb = 0, bb = 0;
         if constexpr (KIND != W_BF16) {
             const uint32_t mw = meta[row * gpr + (col >> m.gshift)];
             sb = mw & 0xffffu;
             bb = mw >> 16;
         }
-        part[pos] = chunk_partial<KIND>(r.w[j], sb, bb, xs, sx, col, t.cs);
+        const float v = chunk_partial<KIND>(r.w[j], sb, bb, xs, sx, col, t.cs);
+        if (in) part[row * t.cs + col] = v;
         __builtin_amdgcn_sched_barrier(0);
     }
 }
 
-// All passes of a tile whose first pass is already in `r0`: pass p + 1 is requested before pass p is consumed.
-template <WKind KIND, int NL, int SN>
-__device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, uint32_t ti, TileRegs<NL>& r0, const uint4* xs,
-                                         const float* sx, const uint32_t* meta, float* part) {
+// All passes of a tile whose first pass is already in `r0` (positions `p` at pass 0): pass k + 1 is requested
+// before pass k is consumed.  `after_last_request` runs once the tile's last pass has been requested (the caller
+// queues what it needs next behind it).
+template <WKind KIND, int NL, int SN, typename F>
+__device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
+                                         const float* sx, const uint32_t* meta, float* part, F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
+    const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs;
     TileRegs<NL> r1;
-    for (uint32_t p = 0; p < n_pass; p += 2) {
-        if (p + 1 < n_pass) tile_load<KIND, NL, SN>(m, t, p + 1, ti, r1);
-        tile_partials<KIND, NL, SN>(m, t, p, ti, r0, xs, sx, meta, part);
-        if (p + 1 < n_pass) {
-            if (p + 2 < n_pass) tile_load<KIND, NL, SN>(m, t, p + 2, ti, r0);
-            tile_partials<KIND, NL, SN>(m, t, p + 1, ti, r1, xs, sx, meta, part);
+    TilePos<NL> q = p;
+    if (n_pass <= 1) after_last_request();
+    for (uint32_t k = 0; k < n_pass; k += 2) {
+        if (k + 1 < n_pass) {
+            tile_pos_next<NL, SN>(t, step_r, step_c, q);
+            tile_load<KIND, NL>(m, t, q, r1);
+            if (k + 2 >= n_pass) after_last_request();
+        }
+        tile_partials<KIND, NL>(m, t, p, r0, xs, sx, meta, part);
+        if (k + 1 < n_pass) {
+            p = q;
+            if (k + 2 < n_pass) {
+                tile_pos_next<NL, SN>(t, step_r, step_c, q);
+                tile_load<KIND, NL>(m, t, q, r0);
+                if (k + 3 >= n_pass) after_last_request();
+            }
+            tile_partials<KIND, NL>(m, t, p, r1, xs, sx, meta, part);
+            p = q;
         }
     }
 }
 
 // The gate / up pair: both matrices' passes interleaved, so that one pass of each is in flight while one is consumed.
-template <WKind KIND, int NL, int SN>
-__device__ __forceinline__ void tile_run_pair(const XcdMat& ma, const XcdMat& mb, const Tile& t, uint32_t ti, TileRegs<NL>& a0,
-                                              TileRegs<NL>& b0, const uint4* xs, const float* sx, const uint32_t* meta_a,
-                                              const uint32_t* meta_b, float* part_a, float* part_b) {
+template <WKind KIND, int NL, int SN, typename F>
+__device__ __forceinline__ void tile_run_pair(const XcdMat& ma, const XcdMat& mb, const Tile& t, TilePos<NL>& p,
+                                              TileRegs<NL>& a0, TileRegs<NL>& b0, const uint4* xs, const float* sx,
+                                              const uint32_t* meta_a, const uint32_t* meta_b, float* part_a, float* part_b,
+                                              F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
+    const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs;
     TileRegs<NL> a1, b1;
-    for (uint32_t p = 0; p < n_pass; p += 2) {
-        if (p + 1 < n_pass) {
-            tile_load<KIND, NL, SN>(ma, t, p + 1, ti, a1);
-            tile_load<KIND, NL, SN>(mb, t, p + 1, ti, b1);
+    TilePos<NL> q = p;
+    if (n_pass <= 1) after_last_request();
+    for (uint32_t k = 0; k < n_pass; k += 2) {
+        if (k + 1 < n_pass) {
+            tile_pos_next<NL, SN>(t, step_r, step_c, q);
+            tile_load<KIND, NL>(ma, t, q, a1);
+            tile_load<KIND, NL>(mb, t, q, b1);
+            if (k + 2 >= n_pass) after_last_request();
         }
-        tile_partials<KIND, NL, SN>(ma, t, p, ti, a0, xs, sx, meta_a, part_a);
-        tile_partials<KIND, NL, SN>(mb, t, p, ti, b0, xs, sx, meta_b, part_b);
-        if (p + 1 < n_pass) {
-            if (p + 2 < n_pass) {
-                tile_load<KIND, NL, SN>(ma, t, p + 2, ti, a0);
-                tile_load<KIND, NL, SN>(mb, t, p + 2, ti, b0);
+        tile_partials<KIND, NL>(ma, t, p, a0, xs, sx, meta_a, part_a);
+        tile_partials<KIND, NL>(mb, t, p, b0, xs, sx, meta_b, part_b);
+        if (k + 1 < n_pass) {
+            p = q;
+            if (k + 2 < n_pass) {
+                tile_pos_next<NL, SN>(t, step_r, step_c, q);
+                tile_load<KIND, NL>(ma, t, q, a0);
+                tile_load<KIND, NL>(mb, t, q, b0);
+                if (k + 3 >= n_pass) after_last_request();
             }
-            tile_partials<KIND, NL, SN>(ma, t, p + 1, ti, a1, xs, sx, meta_a, part_a);
-            tile_partials<KIND, NL, SN>(mb, t, p + 1, ti, b1, xs, sx, meta_b, part_b);
+            tile_partials<KIND, NL>(ma, t, p, a1, xs, sx, meta_a, part_a);
+            tile_partials<KIND, NL>(mb, t, p, b1, xs, sx, meta_b, part_b);
+            p = q;
         }
     }
 }
 
+// Lanes that share a row in the row-sum phase: about four to eight partials per lane, at most 16 lanes (so that
+// the cross-lane sum stays inside a 16-lane row of the wave).
 __device__ __forceinline__ uint32_t lanes_per_row(uint32_t cs) {
     uint32_t lr = 1;
-    while (lr * 2 <= cs && lr < 64) lr <<= 1;
+    while (lr < 16 && lr * 8 <= cs) lr <<= 1;
     return lr;
 }
 
@@ -407,17 +455,20 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
     MetaRegs mg, mu, md;
     TileRegs<NLA> rg, ru;
     TileRegs<NLB> rd;
+    TilePos<NLA> pg;
+    TilePos<NLB> pd;
     sync.epoch += 1;  // the input hand-over
     if (streams) {
-        // Requested now, in the order of use: the groups' scales and biases, the first pass of gate / up, all of
-        // this block's down_proj slice.  The hand-overs only gate arithmetic; the later passes of gate / up
-        // stream while the earlier ones are consumed.
+        // Requested now: the groups' scales and biases and the first pass of gate / up -- a few KiB per CU, so
+        // that the control wave's small requests are not queued behind megabytes.  The later passes stream
+        // while the earlier ones are consumed; the down_proj slice is queued behind the last of them.
+        tile_pos_init<NLA, kBlock>(tg, tid, pg);
+        tile_pos_init<NLB, kBlock>(td, tid, pd);
         meta_fetch<KIND, kBlock>(a.gate, tg, tid, mg);
         meta_fetch<KIND, kBlock>(a.up, tg, tid, mu);
         meta_fetch<KIND, kBlock>(a.down, td, tid, md);
-        tile_load<KIND, NLA, kBlock>(a.gate, tg, 0, tid, rg);
-        tile_load<KIND, NLA, kBlock>(a.up, tg, 0, tid, ru);
-        tile_load<KIND, NLB, kBlock>(a.down, td, 0, tid, rd);
+        tile_load<KIND, NLA>(a.gate, tg, pg, rg);
+        tile_load<KIND, NLA>(a.up, tg, pg, ru);
         FK_XCD_STAMP(1, 1);
         meta_store<KIND, kBlock>(mg, tid, meta);
         meta_store<KIND, kBlock>(mu, tid, meta + kMetaWords);
@@ -430,8 +481,14 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
 
     // ---- gate / up rows of this XCD's slice, SwiGLU ----
     const uint32_t seg = (gu_n * a.gate.cpr + NLA * kBlock - 1) / (NLA * kBlock) * (NLA * kBlock);
-    if (streams && gu_n)
-        tile_run_pair<KIND, NLA, kBlock>(a.gate, a.up, tg, tid, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg);
+    if (streams) {
+        auto request_down = [&]() { tile_load<KIND, NLB>(a.down, td, pd, rd); };
+        if (gu_n)
+            tile_run_pair<KIND, NLA, kBlock>(a.gate, a.up, tg, pg, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg,
+                                             request_down);
+        else
+            request_down();
+    }
     FK_XCD_STAMP(1, 6);
     __syncthreads();
     if (streams && gu_n) {
@@ -448,7 +505,7 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
     if (streams) stage_vector<KIND>(a.mid + (size_t)sync.xcd * per_xcd, per_xcd >> 3, a.down_cs, xs, sx);
     __syncthreads();
     FK_XCD_STAMP(1, 9);
-    if (streams && d_n) tile_run<KIND, NLB, kBlock>(a.down, td, tid, rd, xs, sx, meta + 2 * kMetaWords, work);
+    if (streams && d_n) tile_run<KIND, NLB, kBlock>(a.down, td, pd, rd, xs, sx, meta + 2 * kMetaWords, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(1, 10);
     if (streams && d_n) {
@@ -505,12 +562,15 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     MetaRegs mmq, mmo;
     TileRegs<NLA> rq;
     TileRegs<NLB> ro;
+    TilePos<NLA> pq;
+    TilePos<NLB> po;
     sync.epoch += 1;  // the input hand-over
     if (streams) {
+        tile_pos_init<NLA, kAttnStream>(tq, ti, pq);
+        tile_pos_init<NLB, kAttnStream>(to, ti, po);
         meta_fetch<KIND, kAttnStream>(mq, tq, ti, mmq);
         meta_fetch<KIND, kAttnStream>(a.wo, to, ti, mmo);
-        tile_load<KIND, NLA, kAttnStream>(mq, tq, 0, ti, rq);
-        tile_load<KIND, NLB, kAttnStream>(a.wo, to, 0, ti, ro);
+        tile_load<KIND, NLA>(mq, tq, pq, rq);
         FK_XCD_STAMP(0, 1);
         meta_store<KIND, kAttnStream>(mmq, ti, meta);
         meta_store<KIND, kAttnStream>(mmo, ti, meta + kMetaWords);
@@ -520,8 +580,14 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     __syncthreads();
     FK_XCD_STAMP(0, 5);
 
-    // ---- q / k / v rows of this XCD's KV head ----
-    if (streams && pr_n) tile_run<KIND, NLA, kAttnStream>(mq, tq, ti, rq, xs, sx, meta, work);
+    // ---- q / k / v rows of this XCD's KV head; the o_proj slice is requested behind their last pass ----
+    if (streams) {
+        auto request_o = [&]() { tile_load<KIND, NLB>(a.wo, to, po, ro); };
+        if (pr_n)
+            tile_run<KIND, NLA, kAttnStream>(mq, tq, pq, rq, xs, sx, meta, work, request_o);
+        else
+            request_o();
+    }
     __syncthreads();
     if (pr_n) {
         uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
@@ -555,24 +621,33 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
             for (uint32_t d2 = lane; d2 < ((a.sdpa.v_dim >> 1) + kWave - 1) / kWave * kWave; d2 += kWave) {
                 const bool live = d2 < (a.sdpa.v_dim >> 1);
                 const float* pd = ph + 2 + 2 * (live ? d2 : 0u);
-                float2 ml[kXcdMaxRanges], po[kXcdMaxRanges];
+                float M = -INFINITY, L = 0.f, o0_ = 0.f, o1_ = 0.f;
+                // all requests first (clamped indices: straight-line), then the fold in range order; up to 8 ranges
+                // (a context of 8 x the range length) take half the requests
+                auto merge = [&](auto n_const) {
+                    constexpr uint32_t N = decltype(n_const)::value;
+                    float2 ml[N], po[N];
 #pragma unroll
-                for (uint32_t i = 0; i < kXcdMaxRanges; ++i) {
-                    const uint32_t idx = i < n_active ? i : 0u;
-                    ml[i] = ld_f32x2<true>(ph + (size_t)idx * row);
-                    po[i] = ld_f32x2<true>(pd + (size_t)idx * row);
-                }
-                float M = ml[0].x;
+                    for (uint32_t i = 0; i < N; ++i) {
+                        const uint32_t idx = i < n_active ? i : 0u;
+                        ml[i] = ld_f32x2<true>(ph + (size_t)idx * row);
+                        po[i] = ld_f32x2<true>(pd + (size_t)idx * row);
+                    }
+                    M = ml[0].x;
 #pragma unroll
-                for (uint32_t i = 1; i < kXcdMaxRanges; ++i) M = i < n_active ? fmaxf(M, ml[i].x) : M;
-                float L = 0.f, o0_ = 0.f, o1_ = 0.f;
+                    for (uint32_t i = 1; i < N; ++i) M = i < n_active ? fmaxf(M, ml[i].x) : M;
 #pragma unroll
-                for (uint32_t i = 0; i < kXcdMaxRanges; ++i) {
-                    const float w = i < n_active ? expf(ml[i].x - M) : 0.f;
-                    L = fmaf(ml[i].y, w, L);
-                    o0_ = fmaf(po[i].x, w, o0_);
-                    o1_ = fmaf(po[i].y, w, o1_);
-                }
+                    for (uint32_t i = 0; i < N; ++i) {
+                        const float w = i < n_active ? expf(ml[i].x - M) : 0.f;
+                        L = fmaf(ml[i].y, w, L);
+                        o0_ = fmaf(po[i].x, w, o0_);
+                        o1_ = fmaf(po[i].y, w, o1_);
+                    }
+                };
+                if (n_active <= kXcdMaxRanges / 2)
+                    merge(std::integral_constant<uint32_t, kXcdMaxRanges / 2>{});
+                else
+                    merge(std::integral_constant<uint32_t, kXcdMaxRanges>{});
                 const float inv_l = 1.0f / L;
                 if (live) {
                     att[h * a.sdpa.v_dim + 2 * d2] = (uint16_t)f32_to_bf16_bits(o0_ * inv_l);
@@ -594,7 +669,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
         }
     }
     __syncthreads();
-    if (streams && o_n) tile_run<KIND, NLB, kAttnStream>(a.wo, to, ti, ro, xs, sx, meta + kMetaWords, work);
+    if (streams && o_n) tile_run<KIND, NLB, kAttnStream>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(0, 11);
     if (o_n) {
