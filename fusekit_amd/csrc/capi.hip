@@ -696,10 +696,10 @@ fk_status fk_synth_fill(void* dptr, size_t count, uint64_t seed, float mean, flo
 }
 
 fk_status fk_synth_fill_exact(void* dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind,
-                              size_t row_len, float tau, fk_stream s) {
+                              size_t row_len, float tau, size_t loud_rows, float loud_gain, fk_stream s) {
     if (kind != 3 && kind != 4) return set_error(FK_ERR_INVALID, "synth_fill_exact: kind must be 3 (fp32) or 4 (bf16)");
     Launch l;
-    FK_TRY(plan_synth(dptr, count, seed, mean, std, kind, 0, &l, row_len, tau));
+    FK_TRY(plan_synth(dptr, count, seed, mean, std, kind, 0, &l, row_len, tau, loud_rows, loud_gain));
     return run_launch(l, (hipStream_t)s);
 }
 

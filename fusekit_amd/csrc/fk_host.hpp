@@ -257,6 +257,6 @@ fk_status plan_copy(void* dst, const void* src, size_t nbytes, Launch* out);
 fk_status plan_quantize(const float* w, size_t n, size_t k, uint32_t bits, uint32_t group, uint32_t* packed,
                         uint16_t* scales, uint16_t* biases, Launch* out);
 fk_status plan_synth(void* out_ptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind, uint32_t bound,
-                     Launch* out, uint64_t row_len = 0, float tau = 0.f);
+                     Launch* out, uint64_t row_len = 0, float tau = 0.f, uint64_t loud_rows = 0, float loud_gain = 1.f);
 
 }  // namespace fk

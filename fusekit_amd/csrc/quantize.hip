@@ -85,6 +85,8 @@ struct SynthArgs {
     uint32_t bound;
     uint64_t row_len;  // kinds 3 / 4: elements per row for the row-norm spread (0: none)
     float tau;
+    uint64_t loud_rows;  // kinds 3 / 4: the first loud_rows rows are multiplied by loud_gain instead
+    float loud_gain;
 };
 
 __device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
@@ -101,7 +103,8 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
 //                splitmix64 words keyed by (seed, i): mean 0, variance 1, |z| < 4.9
 //   value      = fma(std, z, mean) * rowscale(i / row_len)
 //   rowscale(j), when row_len and tau are non-zero: u = floor(tau * z(seed ^ K, j) * 8),
-//                (1 + (u & 7) / 8) * 2^(u >> 3): row norms spread like a log-normal.
+//                (1 + (u & 7) / 8) * 2^(u >> 3): row norms spread like a log-normal;
+//                rows j < loud_rows are multiplied by loud_gain instead (a few dominant rows).
 __device__ __forceinline__ float ih_normal(uint64_t seed, uint64_t i) {
     const uint64_t r0 = splitmix64(seed * 0xD1342543DE82EF95ull + i), r1 = splitmix64(r0);
     int32_t sum = 0;
@@ -111,7 +114,9 @@ __device__ __forceinline__ float ih_normal(uint64_t seed, uint64_t i) {
 }
 __device__ __forceinline__ float synth_exact(const SynthArgs& a, size_t i) {
     float v = __fmaf_rn(a.std, ih_normal(a.seed, i), a.mean);
-    if (a.row_len && a.tau != 0.0f) {
+    if (a.row_len && i / a.row_len < a.loud_rows) {
+        v = __fmul_rn(v, a.loud_gain);
+    } else if (a.row_len && a.tau != 0.0f) {
         const float t = floorf(__fmul_rn(__fmul_rn(a.tau, ih_normal(a.seed ^ 0x5DEECE66Dull, i / a.row_len)), 8.0f));
         const int u = (int)t;
         v = __fmul_rn(v, ldexpf(__fmaf_rn((float)(u & 7), 0.125f, 1.0f), u >> 3));
@@ -148,12 +153,12 @@ __global__ __launch_bounds__(256) void synth_kernel(const SynthArgs a) {
 }
 
 fk_status plan_synth(void* out_ptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind, uint32_t bound,
-                     Launch* out, uint64_t row_len, float tau) {
+                     Launch* out, uint64_t row_len, float tau, uint64_t loud_rows, float loud_gain) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!out_ptr || count == 0) return set_error(FK_ERR_INVALID, "synth: null pointer or zero count");
     if (kind > 4 || (kind == 2 && bound == 0)) return set_error(FK_ERR_INVALID, "synth: bad kind or bound");
-    SynthArgs a{out_ptr, count, seed, mean, std, kind, bound, row_len, tau};
+    SynthArgs a{out_ptr, count, seed, mean, std, kind, bound, row_len, tau, loud_rows, loud_gain};
     size_t blocks = (count + 255) / 256;
     if (blocks > (size_t)dev->cus * 16) blocks = (size_t)dev->cus * 16;
     out->func = reinterpret_cast<const void*>(&synth_kernel);

@@ -76,12 +76,13 @@ DENSE_4B = dict(n_layers=36, hidden=2560, n_heads=32, n_kv=8, head_dim=128, inte
 
 
 def _synth(buf: DeviceBuffer, count: int, seed: int, mean: float, std: float, kind: int, bound: int = 0,
-           row_len: int = 0, tau: float = 0.0) -> None:
+           row_len: int = 0, tau: float = 0.0, loud_rows: int = 0, loud_gain: float = 1.0) -> None:
     """kind 0 / 1: fp32 / bf16 normal, 2: uniform uint32 below `bound`; 3 / 4: fp32 / bf16 values a host can
     reproduce bit for bit (fk_synth_fill_exact), optionally with a log-normal-like spread of the row norms."""
     if kind >= 3:
         check(lib.fk_synth_fill_exact(C.c_void_p(buf.ptr), C.c_size_t(count), C.c_uint64(seed), C.c_float(mean),
-                                      C.c_float(std), C.c_uint32(kind), C.c_size_t(row_len), C.c_float(tau), None))
+                                      C.c_float(std), C.c_uint32(kind), C.c_size_t(row_len), C.c_float(tau),
+                                      C.c_size_t(loud_rows), C.c_float(loud_gain), None))
         return
     check(lib.fk_synth_fill(C.c_void_p(buf.ptr), C.c_size_t(count), C.c_uint64(seed), C.c_float(mean),
                             C.c_float(std), C.c_uint32(kind), C.c_uint32(bound), None))
@@ -111,12 +112,14 @@ class DecoderWeights:
 
     @classmethod
     def random_init(cls, cfg: DecoderConfig, seed: int = 0, std: float = 0.02, exact: bool = False,
-                    embed_seed: Optional[int] = None, embed_tau: float = 0.0) -> "DecoderWeights":
+                    embed_seed: Optional[int] = None, embed_tau: float = 0.0, embed_loud_rows: int = 0,
+                    embed_loud_gain: float = 1.0) -> "DecoderWeights":
         """Projections ~ N(0, std^2) quantised on the device; norm weights ~ 1 + N(0, 0.1^2);
         tied bf16 embedding ~ N(0, std^2); biases ~ N(0, 0.5^2).
         exact: draw every value with the host-reproducible generator (fk_synth_fill_exact), so a CPU
-        build of the same model from the same seeds holds the same bytes.  embed_seed / embed_tau
-        (exact only): own seed of the embedding, and the spread of its row norms."""
+        build of the same model from the same seeds holds the same bytes.  embed_seed / embed_tau /
+        embed_loud_rows / embed_loud_gain (exact only): own seed of the embedding, the spread of its row
+        norms, and a few dominant rows (token ids 0 .. loud_rows - 1)."""
         self = cls(cfg)
         f32_kind, bf16_kind = (3, 4) if exact else (0, 1)
         biggest = max(cfg.inter * cfg.hidden, cfg.n_q * cfg.hidden)
@@ -149,7 +152,7 @@ class DecoderWeights:
         es = next_seed()
         if exact:
             _synth(emb.w, cfg.vocab * cfg.hidden, es if embed_seed is None else embed_seed, 0.0, std, 4,
-                   row_len=cfg.hidden, tau=embed_tau)
+                   row_len=cfg.hidden, tau=embed_tau, loud_rows=embed_loud_rows, loud_gain=embed_loud_gain)
         else:
             _synth(emb.w, cfg.vocab * cfg.hidden, es, 0.0, std, 1)
         self.mats["embed_tokens"] = emb

@@ -118,13 +118,14 @@ def get_accum_mode() -> int:
     return int(_lib.fko_get_accum_mode())
 
 
-def synth_fill(count: int, seed: int, mean: float, std: float, kind: int, row_len: int = 0, tau: float = 0.0) -> np.ndarray:
+def synth_fill(count: int, seed: int, mean: float, std: float, kind: int, row_len: int = 0, tau: float = 0.0,
+               loud_rows: int = 0, loud_gain: float = 1.0) -> np.ndarray:
     """The GPU library's host-reproducible synthetic fill (fk_synth_fill_exact), bit for bit:
     kind 3 -> float32 array, kind 4 -> bf16 bit patterns (uint16)."""
     assert kind in (3, 4)
     out = np.empty(count, dtype=np.float32 if kind == 3 else np.uint16)
     _lib.fko_synth_fill(C.c_void_p(out.ctypes.data), C.c_int64(count), C.c_uint64(seed), C.c_float(mean), C.c_float(std),
-                        C.c_int(kind), C.c_int64(row_len), C.c_float(tau))
+                        C.c_int(kind), C.c_int64(row_len), C.c_float(tau), C.c_int64(loud_rows), C.c_float(loud_gain))
     return out
 
 

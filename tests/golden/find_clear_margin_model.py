@@ -59,7 +59,9 @@ def run(cfg, W, prompt, forced=None, want_logits=False):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--model-seed", type=int, default=0)
-    ap.add_argument("--grid", nargs="+", default=["2.0:0.02"], help="tau:embed_scale pairs")
+    ap.add_argument("--grid", nargs="+", default=["0:0.02"], help="tau:embed_scale pairs")
+    ap.add_argument("--loud-rows", type=int, default=0, help="token ids 0 .. N-1 get the row gain instead of the spread")
+    ap.add_argument("--loud-gain", type=float, default=1.0)
     ap.add_argument("--seeds", type=int, default=8, help="embedding seeds tried per (tau, scale)")
     ap.add_argument("--first-seed", type=int, default=1000)
     ap.add_argument("--safety", type=float, default=3.0)
@@ -83,12 +85,13 @@ def main():
         if True:
             for es in range(args.first_seed, args.first_seed + args.seeds):
                 cfg.embed_scale = scale
-                W.set_embedding(es, tau)
+                W.set_embedding(es, tau, args.loud_rows, args.loud_gain)
                 oracle.set_accum_mode(0)
                 t0 = time.time()
                 toks, margins, lg0 = run(cfg, W, prompt, want_logits=True)
                 distinct = len(set(toks))
-                rec = dict(tau=tau, embed_scale=scale, embed_seed=es, tokens=toks, distinct=distinct,
+                rec = dict(tau=tau, embed_scale=scale, embed_seed=es, loud_rows=args.loud_rows, loud_gain=args.loud_gain,
+                           tokens=toks, distinct=distinct,
                            min_margin=float(min(margins)), margins=[float(m) for m in margins])
                 line = "tau %.2f scale %.3g seed %d: distinct %d, min margin %.4g, %.0f s" % (
                     tau, scale, es, distinct, min(margins), time.time() - t0)

@@ -52,7 +52,7 @@ class HostDecoderWeights:
     `DecoderWeights.random_init(cfg, seed, exact=True, ...)` puts into HBM (same seed sequence)."""
 
     def __init__(self, cfg, seed: int = 0, std: float = 0.02, embed_seed=None, embed_tau: float = 0.0,
-                 with_embedding: bool = True):
+                 with_embedding: bool = True, embed_loud_rows: int = 0, embed_loud_gain: float = 1.0):
         self.cfg = cfg
         self.mats, self.vecs = {}, {}
         self.std = std
@@ -75,7 +75,7 @@ class HostDecoderWeights:
         es = next_seed()
         self.embed_seed = es if embed_seed is None else embed_seed
         if with_embedding:
-            self.set_embedding(self.embed_seed, embed_tau)
+            self.set_embedding(self.embed_seed, embed_tau, embed_loud_rows, embed_loud_gain)
         vector("final_norm", cfg.hidden, 1.0, 0.1)
         for l in range(cfg.n_layers):
             p = f"layers.{l}."
@@ -96,11 +96,11 @@ class HostDecoderWeights:
                 vector(p + "self_attn.k_proj.bias", cfg.n_kvd, 0.0, 0.5)
                 vector(p + "self_attn.v_proj.bias", cfg.n_kvd, 0.0, 0.5)
 
-    def set_embedding(self, embed_seed: int, embed_tau: float) -> None:
+    def set_embedding(self, embed_seed: int, embed_tau: float, loud_rows: int = 0, loud_gain: float = 1.0) -> None:
         c = self.cfg
         self.mats["embed_tokens"] = oracle.dense(
-            oracle.synth_fill(c.vocab * c.hidden, embed_seed, 0.0, self.std, 4, row_len=c.hidden, tau=embed_tau)
-            .reshape(c.vocab, c.hidden))
+            oracle.synth_fill(c.vocab * c.hidden, embed_seed, 0.0, self.std, 4, row_len=c.hidden, tau=embed_tau,
+                              loud_rows=loud_rows, loud_gain=loud_gain).reshape(c.vocab, c.hidden))
 
 
 def host_weight(dw) -> oracle.QWeight:
