@@ -346,6 +346,15 @@ def sdpa_decode(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_
                              _ptr(partials), _ptr(counters), _ptr(stream)))
 
 
+def sdpa_decode_static(q, cache_k, cache_v, out, d_kv_len, kv_len, max_len, n_heads, n_kv, qk_dim, v_dim, capacity,
+                       scale, stream=None):
+    """fk_sdpa_decode with the split-K workspace in the library's static device array: allocates nothing."""
+    check(lib.fk_sdpa_decode_static(_ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(out), _ptr(d_kv_len),
+                                    C.c_uint32(kv_len), C.c_uint32(max_len), C.c_uint32(n_heads), C.c_uint32(n_kv),
+                                    C.c_uint32(qk_dim), C.c_uint32(v_dim), C.c_uint32(capacity), C.c_float(scale),
+                                    _ptr(stream)))
+
+
 class _KvQuantCache(C.Structure):
     _fields_ = [("packed", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
 

@@ -241,11 +241,12 @@ fk_status fk_synth_fill(void *dptr, size_t count, uint64_t seed, float mean, flo
  * CPU): kind 3 fp32, kind 4 bf16; value = fma(std, z, mean) with z a sum of eight 16-bit uniform
  * integers, centred and scaled to unit variance (integer arithmetic and single IEEE operations
  * only).  With row_len and tau non-zero every row of row_len elements is multiplied by
- * (1 + (u & 7) / 8) * 2^(u >> 3), u = floor(8 * tau * z_row): row norms spread like a log-normal,
- * which gives a tied embedding / LM head the peaked logits of a trained model.  Like
+ * (1 + (u & 7) / 8) * 2^(u >> 3), u = floor(8 * tau * z_row): row norms spread like a log-normal;
+ * the first loud_rows rows are multiplied by loud_gain instead.  Either gives a tied embedding / LM
+ * head the peaked logits of a trained model (a random one is near-uniform over the vocabulary).  Like
  * fk_synth_fill this has no counterpart in the reference, which loads real checkpoints. */
 fk_status fk_synth_fill_exact(void *dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind,
-                              size_t row_len, float tau, fk_stream s);
+                              size_t row_len, float tau, size_t loud_rows, float loud_gain, fk_stream s);
 
 /* Per-token scalars (rotary position, cache row, KV length) come either from a
  * device scalar `d_*` (so a captured hipGraph can be replayed while a step
@@ -295,6 +296,19 @@ fk_status fk_sdpa_decode(const uint16_t *q, const uint16_t *cache_k, const uint1
                          const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
                          uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
                          float *partials, uint32_t *counters, fk_stream s);
+
+/*     The same attention for callers that cannot allocate device memory (code under hipGraph capture,
+ *     tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference: the
+ *     split-K workspace (partial rows + arrival counters) is a device array inside the library,
+ *     fk_sdpa_static_scratch_bytes() = 9 MiB per GPU for the life of the process, found once per device
+ *     with hipGetSymbolAddress.  The call allocates nothing; problems whose workspace
+ *     (fk_sdpa_workspace_bytes) does not fit are refused with FK_ERR_UNSUPPORTED.  All calls on one GPU
+ *     share the array: calls that overlap on one GPU race and must be serialised by the caller. */
+size_t fk_sdpa_static_scratch_bytes(void);
+fk_status fk_sdpa_decode_static(const uint16_t *q, const uint16_t *cache_k, const uint16_t *cache_v, uint16_t *out,
+                                const uint32_t *d_kv_len, uint32_t kv_len, uint32_t max_len, uint32_t n_heads,
+                                uint32_t n_kv, uint32_t qk_dim, uint32_t v_dim, uint32_t capacity, float scale,
+                                fk_stream s);
 
 /* ---- quantised KV cache (mlx-lm QuantizedKVCache: kv_bits = 4 | 8) ----------------
  * Layout: packed uint32 [n_kv, capacity, dim*bits/32], scales / biases bf16
