@@ -2,8 +2,11 @@
 """Headline benchmark: hipGraph-replayed batch-1 greedy decode of the 4B-class dense model
 (configs[3]: 36 layers, hidden 2560, 4-bit g64 MLX-affine weights) at context 512, on one MI355X.
 
-One "step" = one decoded token = one replay of the captured decode graph.  Weights are random-init
-(seeded, generated and quantised in HBM); everything is resident before the timed region.
+One "step" = one decoded token = one replay of the captured decode graph: step_init, embedding, 36 x
+[attention launch | MLP launch] (the XCD-resident layer: RMSNorm + q/k/v + head norm + RoPE + cache append +
+attention + o_proj, then RMSNorm + gate/up + SwiGLU + down_proj, residuals folded into the next launch's
+input), the last layer's reduction, final norm + LM head, argmax.  Weights are random-init (seeded,
+generated and quantised in HBM); everything is resident before the timed region.
 
 The K timed steps always sit around context 512: after the 32-token prompt the script decodes
 untimed (at least --warmup steps) until the cache holds 512 - K/2 positions, then times exactly K
@@ -38,6 +41,9 @@ SYMBOLS = {
     "linear_residual": "gemv_stream_kernel<Q4, 1 segment>",
     "rmsnorm_gateup_swiglu": "gemv_stream_kernel<Q4, gate/up pair>",
     "rope_store_sdpa_decode": "sdpa_rope_store_kernel",
+    "xcd_attn_block": "xcd_attn_kernel<Q4>",
+    "xcd_mlp_block": "xcd_mlp_kernel<Q4>",
+    "xcd_reduce": "xcd_reduce_kernel",
     "final_rmsnorm_lm_head": "gemv_stream_kernel<BF16, 1 segment>",
     "argmax_logits_decode": "argmax_kernel",
     "embed_lookup_decode": "embed_lookup_kernel",
@@ -175,18 +181,29 @@ def main() -> int:
             per_layer = 2 if fam == "linear_residual" else 1
             groups.setdefault((fam, idx % per_layer), []).append(t)
         by_launch, by_symbol = [], {}
+        cache_bytes = cfg.n_kv * cfg.capacity * cfg.head_dim * 2
         for (fam, pos), tasks in groups.items():
             if fam == "rope_store_sdpa_decode" or fam.startswith("sdpa_decode"):
                 nbytes = kv_row_bytes * CONTEXT + 2 * (cfg.n_q * 2)          # K/V rows read + q in, out
                 label = "rope/store + attention @%d" % CONTEXT
+            elif fam == "xcd_attn_block":
+                # q/k/v/o weights + vectors + partial rows, and the K/V rows of the context instead of the whole caches
+                nbytes = sum(n for _, n in tasks[0].args if n != cache_bytes) + kv_row_bytes * CONTEXT
+                label = "attention launch (norm, q/k/v, rope, append, attention @%d, o_proj)" % CONTEXT
+            elif fam == "xcd_mlp_block":
+                nbytes = sum(n for _, n in tasks[0].args)
+                label = "MLP launch (norm, gate/up, SwiGLU, down_proj)"
             else:
                 nbytes = sum(n for _, n in tasks[0].args)                    # weights + scales + biases + vectors in/out
                 label = {("linear_residual", 0): "o_proj + residual", ("linear_residual", 1): "down_proj + residual"}.get(
                     (fam, pos), fam)
-            reps = max(2, 720 // len(tasks))
-            g = rt.d.build_graph(tasks, barriers=[True] * len(tasks))
+            # a launch that occurs once per token is chained 32 times, so that the cost of starting a graph is not
+            # charged to one small kernel
+            chain = tasks if len(tasks) > 1 else tasks * 32
+            reps = max(2, 720 // len(chain))
+            g = rt.d.build_graph(chain, barriers=[True] * len(chain))
             rt.d.execute_graph(g)
-            us = rt.d.execute_graph(g, repeat=reps) / (reps * len(tasks)) * 1e6
+            us = rt.d.execute_graph(g, repeat=reps) / (reps * len(chain)) * 1e6
             sym = SYMBOLS.get(fam, fam)
             e = {"launch": label, "kernel": sym, "per_token": len(tasks), "bytes_per_launch": int(nbytes),
                  "avg_launch_us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),

@@ -85,7 +85,7 @@ struct SynthArgs {
     uint32_t bound;
     uint64_t row_len;  // kinds 3 / 4: elements per row for the row-norm spread (0: none)
     float tau;
-    uint64_t loud_rows;  // kinds 3 / 4: the first loud_rows rows are multiplied by loud_gain instead
+    uint64_t loud_rows;  // kinds 3 / 4: row j < loud_rows is multiplied by loud_gain * 2^-j instead
     float loud_gain;
 };
 
@@ -104,7 +104,8 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
 //   value      = fma(std, z, mean) * rowscale(i / row_len)
 //   rowscale(j), when row_len and tau are non-zero: u = floor(tau * z(seed ^ K, j) * 8),
 //                (1 + (u & 7) / 8) * 2^(u >> 3): row norms spread like a log-normal;
-//                rows j < loud_rows are multiplied by loud_gain instead (a few dominant rows).
+//                rows j < loud_rows are multiplied by loud_gain * 2^-j instead (a few dominant rows,
+//                each half as loud as the one before).
 __device__ __forceinline__ float ih_normal(uint64_t seed, uint64_t i) {
     const uint64_t r0 = splitmix64(seed * 0xD1342543DE82EF95ull + i), r1 = splitmix64(r0);
     int32_t sum = 0;
@@ -115,7 +116,7 @@ __device__ __forceinline__ float ih_normal(uint64_t seed, uint64_t i) {
 __device__ __forceinline__ float synth_exact(const SynthArgs& a, size_t i) {
     float v = __fmaf_rn(a.std, ih_normal(a.seed, i), a.mean);
     if (a.row_len && i / a.row_len < a.loud_rows) {
-        v = __fmul_rn(v, a.loud_gain);
+        v = __fmul_rn(v, ldexpf(a.loud_gain, -(int)(i / a.row_len)));
     } else if (a.row_len && a.tau != 0.0f) {
         const float t = floorf(__fmul_rn(__fmul_rn(a.tau, ih_normal(a.seed ^ 0x5DEECE66Dull, i / a.row_len)), 8.0f));
         const int u = (int)t;

@@ -242,7 +242,7 @@ fk_status fk_synth_fill(void *dptr, size_t count, uint64_t seed, float mean, flo
  * integers, centred and scaled to unit variance (integer arithmetic and single IEEE operations
  * only).  With row_len and tau non-zero every row of row_len elements is multiplied by
  * (1 + (u & 7) / 8) * 2^(u >> 3), u = floor(8 * tau * z_row): row norms spread like a log-normal;
- * the first loud_rows rows are multiplied by loud_gain instead.  Either gives a tied embedding / LM
+ * row j of the first loud_rows rows is multiplied by loud_gain * 2^-j instead.  Either gives a tied embedding / LM
  * head the peaked logits of a trained model (a random one is near-uniform over the vocabulary).  Like
  * fk_synth_fill this has no counterpart in the reference, which loads real checkpoints. */
 fk_status fk_synth_fill_exact(void *dptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind,

@@ -206,7 +206,8 @@ FKO_API void fko_dequantize(const uint32_t *packed, const uint16_t *scales, cons
  *   value      = fma(std, z, mean) * rowscale(i / row_len)
  *   rowscale(j) (row_len != 0 and tau != 0): u = floor(tau * z(seed ^ K, j) * 8),
  *                rowscale = (1 + (u & 7) / 8) * 2^(u >> 3): a log-normal-like spread of row norms
- *   rows j < loud_rows are multiplied by loud_gain instead (a few dominant rows)
+ *   rows j < loud_rows are multiplied by loud_gain * 2^-j instead (a few dominant rows, each half as loud
+ *                as the one before, so that two of them rarely compete at equal strength)
  */
 static inline uint64_t splitmix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;
@@ -231,7 +232,7 @@ FKO_API void fko_synth_fill(void *out, int64_t count, uint64_t seed, float mean,
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < count; ++i) {
         float v = fmaf(std, ih_normal(seed, (uint64_t)i), mean);
-        if (row_len && i / row_len < loud_rows) v = v * loud_gain;
+        if (row_len && i / row_len < loud_rows) v = v * ldexpf(loud_gain, -(int)(i / row_len));
         else if (row_len && tau != 0.0f) v = v * row_scale(seed, (uint64_t)(i / row_len), tau);
         if (kind == 3) ((float *)out)[i] = v;
         else ((uint16_t *)out)[i] = f32_to_bf16(v);

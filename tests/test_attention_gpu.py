@@ -236,6 +236,39 @@ def test_rope_store_sdpa_in_one_launch(fk, norm, table, n_heads, n_kv, dim, rope
     assert np.array_equal(ck3.to_numpy(np.uint16), ck1.to_numpy(np.uint16))
 
 
+@pytest.mark.parametrize("kv_len", [512, 4096, 32768])
+def test_config3_rope_append_attention_chain_against_the_oracle(fk, kv_len):
+    """configs[2] as stated: 32 q / 8 kv heads x 128, bf16 cache ~ N(0, 1) of kv_len - 1 positions, RoPE (theta 1e6) on
+    q and on the new k, the new k / v rows appended at position kv_len - 1, then attention over kv_len rows --
+    the one-launch form against the ORACLE's chain (rope_q, rope + cache store, attention), cache rows included."""
+    n_heads, n_kv, dim, theta, eps = 32, 8, 128, 1e6, 1e-6
+    cap, pos, scale = kv_len, kv_len - 1, dim ** -0.5
+    q, k, v = normal_bf16(11, n_heads * dim), normal_bf16(12, n_kv * dim), normal_bf16(13, n_kv * dim)
+    ck, cv = normal_bf16(14, n_kv * cap * dim), normal_bf16(15, n_kv * cap * dim)
+    dev = lambda a: fk.DeviceBuffer.from_numpy(a)
+    pb, cb = fk.sdpa_workspace_bytes(n_heads, n_kv, dim, dim, cap)
+    part, cnt = fk.DeviceBuffer(max(pb, 16)), fk.zeros(max(cb, 16))
+    dck, dcv, out = dev(ck), dev(cv), fk.DeviceBuffer(n_heads * dim * 2)
+    tab = fk.DeviceBuffer(dim * 4)
+    fk.step_init_rope(_u32(fk, pos), fk.zeros(4), fk.zeros(4), tab, dim, theta)
+    fk.rope_store_sdpa_decode(dev(q), dev(k), dev(v), None, None, dck, dcv, out, _u32(fk, kv_len), 0, cap, n_heads, n_kv,
+                              dim, dim, theta, eps, cap, scale, tab, part, cnt)
+    # the oracle's chain on the same inputs
+    rq = oracle.rope_q(q, n_heads, dim, dim, theta, pos)
+    ock, ocv = ck.copy(), cv.copy()
+    oracle.rope_kv_store(k, v, n_kv, dim, dim, theta, pos, pos, cap, ock, ocv)
+    got_ck, got_cv = dck.to_numpy(np.uint16), dcv.to_numpy(np.uint16)
+    assert np.array_equal(got_cv, ocv)                                    # V is a pure copy: bit-exact
+    rows = lambda a: a.reshape(n_kv, cap, dim)
+    keep = np.arange(cap) != pos
+    assert np.array_equal(rows(got_ck)[:, keep], rows(ock)[:, keep])      # no other row touched
+    frac, ulps = bf16_mismatch(rows(got_ck)[:, pos], rows(ock)[:, pos])
+    assert ulps <= 1.0 and frac <= 0.02                                   # fp32 sin / cos products on a rounding edge
+    ref = oracle.sdpa_decode(rq, ock, ocv, n_heads, n_kv, dim, dim, kv_len, cap, scale)
+    assert rel_l2(out.to_numpy(np.uint16), oracle.bf16_to_f32(ref)) <= REL_L2_BAR
+    assert not cnt.to_numpy(np.uint32).any()
+
+
 def test_rope_store_sdpa_rejects_bad_arguments(fk):
     b = fk.DeviceBuffer(1 << 16)
     args = dict(n_heads=8, n_kv=2, dim=64)

@@ -176,6 +176,63 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
     print("worst rel-L2 of the o_proj sums over the sampled positions: %.3e" % worst)
 
 
+@pytest.mark.parametrize("kv_len", [512, 4096, 32768])
+def test_xcd_attn_block_at_the_config3_contexts(fk, kv_len):
+    """The attention launch at 32 q / 8 kv heads x 128 over a cache ~ N(0, 1) of kv_len - 1 positions (blocks walk
+    several key ranges at 4096 and 32768): cache append and o_proj sums against the oracle's chain."""
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    n_heads, n_kv, head_dim, hidden, inter, bits, theta = 32, 8, 128, 1024, 1024, 4, 1e6
+    capacity, pos = kv_len, kv_len - 1
+    assert fk.xcd_layer_supported(hidden, inter, n_heads, n_kv, head_dim, capacity, bits, 64)
+    d = Dispatcher()
+    n_q, n_kvd = n_heads * head_dim, n_kv * head_dim
+    Wq, Wk, Wv = (make_qweight(s_, n, hidden, bits, std=0.05) for s_, n in ((1, n_q), (2, n_kvd), (3, n_kvd)))
+    Wo = make_qweight(4, hidden, n_q, bits)
+    norm_w, x = normal_bf16(5, hidden, 0.1, 1.0), normal_bf16(6, hidden)
+    ck, cv = normal_bf16(7, n_kv * capacity * head_dim), normal_bf16(8, n_kv * capacity * head_dim)
+    dW = [to_device(fk, W) for W in (Wq, Wk, Wv, Wo)]
+    ctl_bytes, ap_bytes = fk.xcd_workspace_bytes(n_heads, head_dim)
+    ctl = fk.zeros(ctl_bytes)
+    b = dict(res=_dev(fk, x), x=fk.DeviceBuffer(8 * hidden * 2), nw=_dev(fk, norm_w), q=fk.DeviceBuffer(n_q * 2),
+             k=fk.DeviceBuffer(n_kvd * 2), v=fk.DeviceBuffer(n_kvd * 2), ck=_dev(fk, ck), cv=_dev(fk, cv),
+             kv_len=fk.zeros(4), off=fk.zeros(4), step=_dev(fk, np.array([pos], np.uint32)), tab=fk.DeviceBuffer(head_dim * 4),
+             ap=fk.DeviceBuffer(ap_bytes), out=fk.DeviceBuffer(8 * hidden * 4))
+    a = [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dW[0].w), arg(dW[1].w), arg(dW[2].w)]
+    a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]] + _wargs(arg, dW[3])
+    a += [arg(b["q"]), arg(b["k"]), arg(b["v"]), arg(b["ck"]), arg(b["cv"]), arg(b["kv_len"]), arg(b["tab"]), arg(b["ap"]),
+          arg(b["out"]), arg(ctl)]
+    task = Dispatch("fusekit_xcd_attn_block_f1", a,
+                    dict(hidden=hidden, inter=inter, n_heads=n_heads, n_kv=n_kv, head_dim=head_dim, capacity=capacity,
+                         bits=bits, group=64, eps=EPS, theta=theta, has_partials=0, residual_per_xcd=0, has_norm=0))
+    step = Dispatch("fusekit_step_init", [arg(b["step"]), arg(b["off"]), arg(b["kv_len"]), arg(b["tab"])],
+                    dict(rope_dims=head_dim, theta=theta))
+    d.dispatch_batch([step, task])
+    fk.xcd_check(ctl)
+    assert int(b["kv_len"].to_numpy(np.uint32)[0]) == kv_len
+    qg, kg, vg = b["q"].to_numpy(np.uint16), b["k"].to_numpy(np.uint16), b["v"].to_numpy(np.uint16)
+    q_ref, k_ref, v_ref = oracle.rmsnorm_qkv(x, norm_w, EPS, Wq, Wk, Wv)
+    for g, r in ((qg, q_ref), (kg, k_ref), (vg, v_ref)):
+        _close_bf16(g, r)
+    qr = oracle.rope_q(qg, n_heads, head_dim, head_dim, theta, pos)
+    ock, ocv = ck.copy(), cv.copy()
+    oracle.rope_kv_store(kg, vg, n_kv, head_dim, head_dim, theta, pos, pos, capacity, ock, ocv)
+    gck, gcv = b["ck"].to_numpy(np.uint16), b["cv"].to_numpy(np.uint16)
+    assert np.array_equal(gcv, ocv)
+    rows = lambda t: t.reshape(n_kv, capacity, head_dim)
+    keep = np.arange(capacity) != pos
+    assert np.array_equal(rows(gck)[:, keep], rows(ock)[:, keep])
+    fg, fo = oracle.bf16_to_f32(rows(gck)[:, pos]), oracle.bf16_to_f32(rows(ock)[:, pos])
+    row_ulp = 2.0 ** (np.floor(np.log2(np.abs(fo).max(axis=1, keepdims=True))) - 7)
+    assert np.all(np.abs(fg - fo) <= row_ulp)
+    att = oracle.sdpa_decode(qr, gck, gcv, n_heads, n_kv, head_dim, head_dim, kv_len, capacity, 1.0 / np.sqrt(head_dim))
+    y_ref = oracle.linear_acc(Wo, att)
+    out = b["out"].to_numpy(np.float32, (8, hidden))
+    acc = ((out[0] + out[1]) + (out[2] + out[3])) + ((out[4] + out[5]) + (out[6] + out[7]))
+    rel = float(np.linalg.norm(acc.astype(np.float64) - y_ref) / np.linalg.norm(y_ref))
+    print(f"kv_len {kv_len}: o_proj sums rel-L2 {rel:.3e}")
+    assert rel <= 1e-2
+
+
 def test_xcd_reduce(fk):
     from fusekit_amd.runtime import Dispatch, Dispatcher, arg
     d = Dispatcher()
