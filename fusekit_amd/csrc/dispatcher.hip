@@ -635,13 +635,15 @@ XcdLayerShape xcd_shape(const Dispatch& d) {
     return s;
 }
 
-// [partials_in], residual, x_out, norm_w, W_q, W_k, W_v, [s_q, s_k, s_v, b_q, b_k, b_v], W_o, [s_o, b_o],
-// [q_norm, k_norm], q, k, v, cache_k, cache_v, kv_len, rope_tab, att_partials, out_partials, workspace
+// [sums_in], residual, x_out, norm_w, W_q, W_k, W_v, [s_q, s_k, s_v, b_q, b_k, b_v], W_o, [s_o, b_o],
+// [q_norm, k_norm], q, k, v, cache_k, cache_v, kv_len, rope_tab, att_partials, out_sums, clear_sums, workspace
+// (sums_in: the sum row the previous launch added into; out_sums: the row this launch adds into, zero on entry;
+// clear_sums: the row this launch zeroes; residual and x_out: one bf16 row each.)
 // Parameters: the layer shape (hidden, inter, n_heads, n_kv, head_dim, capacity, bits, group), eps, theta,
-// has_partials, has_norm, residual_per_xcd, spin_limit.
+// has_sums, has_norm, spin_limit.
 fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const XcdLayerShape s = xcd_shape(d);
-    const bool has_p = d.u("has_partials", 1) != 0, norm = d.u("has_norm", 0) != 0, q = s.bits != 16;
+    const bool has_p = d.u("has_sums", 1) != 0, norm = d.u("has_norm", 0) != 0, q = s.bits != 16;
     size_t i = 0;
     const size_t p_slot = has_p ? i++ : 0, res_slot = i++, x_slot = i++, nw_slot = i++, w_slot = i;
     i += 3;
@@ -654,7 +656,8 @@ fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (norm) i += 2;
     const size_t q_slot = i;
     i += 3;
-    const size_t ck_slot = i++, cv_slot = i++, len_slot = i++, tab_slot = i++, ap_slot = i++, op_slot = i++, ws_slot = i++;
+    const size_t ck_slot = i++, cv_slot = i++, len_slot = i++, tab_slot = i++, ap_slot = i++, op_slot = i++, clr_slot = i++,
+                 ws_slot = i++;
     FK_TRY(need_args(d, i));
     if (s.hidden == 0 || s.n_heads == 0 || s.n_kv == 0 || s.head_dim == 0 || s.capacity == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": layer shape parameters missing");
@@ -662,16 +665,14 @@ fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     XcdAttnRequest rq;
     memset(&rq, 0, sizeof(rq));
     rq.shape = s;
-    const bool per_xcd = d.u("residual_per_xcd", 0) != 0;
     if (has_p) {
-        FK_TRY(need_bytes(d, p_slot, (size_t)kXcds * s.hidden * 4));
-        rq.partials_in = arg_ptr<const float>(d, p_slot);
+        FK_TRY(need_bytes(d, p_slot, xcd_sum_row_bytes(s.hidden)));
+        rq.sums_in = arg_ptr<const long long>(d, p_slot);
     }
-    FK_TRY(need_bytes(d, res_slot, (size_t)(per_xcd ? kXcds : 1) * s.hidden * 2));
-    FK_TRY(need_bytes(d, x_slot, (size_t)kXcds * s.hidden * 2));
+    FK_TRY(need_bytes(d, res_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, x_slot, (size_t)s.hidden * 2));
     FK_TRY(need_bytes(d, nw_slot, (size_t)s.hidden * 2));
     rq.residual = arg_ptr<const uint16_t>(d, res_slot);
-    rq.residual_stride = per_xcd ? s.hidden : 0;
     rq.x_out = arg_ptr<uint16_t>(d, x_slot);
     rq.norm_w = arg_ptr<const uint16_t>(d, nw_slot);
     rq.eps = (float)d.param("eps", 1e-6);
@@ -707,21 +708,24 @@ fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     rq.theta = (float)d.param("theta", 10000.0);
     FK_TRY(need_bytes(d, ap_slot, xcd_attn_partials_bytes(s)));
     rq.att_partials = arg_ptr<float>(d, ap_slot);
-    FK_TRY(need_bytes(d, op_slot, (size_t)kXcds * s.hidden * 4));
-    rq.out_partials = arg_ptr<float>(d, op_slot);
+    FK_TRY(need_bytes(d, op_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.out_sums = arg_ptr<long long>(d, op_slot);
+    FK_TRY(need_bytes(d, clr_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.clear = arg_ptr<long long>(d, clr_slot);
     FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
     rq.workspace = d.args[ws_slot].ptr;
     rq.spin_limit = d.u("spin_limit", 0);
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
     rw->writes = {(uint32_t)x_slot, (uint32_t)q_slot, (uint32_t)q_slot + 1, (uint32_t)q_slot + 2, (uint32_t)ck_slot,
-                  (uint32_t)cv_slot, (uint32_t)ap_slot, (uint32_t)op_slot, (uint32_t)ws_slot};
+                  (uint32_t)cv_slot, (uint32_t)ap_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
     return plan_xcd_attn(rq, l);
 }
 
-// [partials_in], residual, x_out, norm_w, W_gate, W_up, [s_g, s_u, b_g, b_u], W_down, [s_d, b_d], mid, out_partials, workspace
+// [sums_in], residual, x_out, norm_w, W_gate, W_up, [s_g, s_u, b_g, b_u], W_down, [s_d, b_d], mid, out_sums, clear_sums,
+// workspace
 fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const XcdLayerShape s = xcd_shape(d);
-    const bool has_p = d.u("has_partials", 1) != 0, q = s.bits != 16;
+    const bool has_p = d.u("has_sums", 1) != 0, q = s.bits != 16;
     size_t i = 0;
     const size_t p_slot = has_p ? i++ : 0, res_slot = i++, x_slot = i++, nw_slot = i++, w_slot = i;
     i += 2;
@@ -730,22 +734,20 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const size_t wd_slot = i++;
     const size_t wd_meta = i;
     if (q) i += 2;
-    const size_t mid_slot = i++, op_slot = i++, ws_slot = i++;
+    const size_t mid_slot = i++, op_slot = i++, clr_slot = i++, ws_slot = i++;
     FK_TRY(need_args(d, i));
     if (s.hidden == 0 || s.inter == 0) return set_error(FK_ERR_INVALID, d.kernel + ": layer shape parameters missing");
     XcdMlpRequest rq;
     memset(&rq, 0, sizeof(rq));
     rq.shape = s;
-    const bool per_xcd = d.u("residual_per_xcd", 0) != 0;
     if (has_p) {
-        FK_TRY(need_bytes(d, p_slot, (size_t)kXcds * s.hidden * 4));
-        rq.partials_in = arg_ptr<const float>(d, p_slot);
+        FK_TRY(need_bytes(d, p_slot, xcd_sum_row_bytes(s.hidden)));
+        rq.sums_in = arg_ptr<const long long>(d, p_slot);
     }
-    FK_TRY(need_bytes(d, res_slot, (size_t)(per_xcd ? kXcds : 1) * s.hidden * 2));
-    FK_TRY(need_bytes(d, x_slot, (size_t)kXcds * s.hidden * 2));
+    FK_TRY(need_bytes(d, res_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, x_slot, (size_t)s.hidden * 2));
     FK_TRY(need_bytes(d, nw_slot, (size_t)s.hidden * 2));
     rq.residual = arg_ptr<const uint16_t>(d, res_slot);
-    rq.residual_stride = per_xcd ? s.hidden : 0;
     rq.x_out = arg_ptr<uint16_t>(d, x_slot);
     rq.norm_w = arg_ptr<const uint16_t>(d, nw_slot);
     rq.eps = (float)d.param("eps", 1e-6);
@@ -759,27 +761,31 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     rq.swiglu_variant = (int)d.param("variant", 0);
     FK_TRY(need_bytes(d, mid_slot, (size_t)s.inter * 2));
     rq.mid = arg_ptr<uint16_t>(d, mid_slot);
-    FK_TRY(need_bytes(d, op_slot, (size_t)kXcds * s.hidden * 4));
-    rq.out_partials = arg_ptr<float>(d, op_slot);
+    FK_TRY(need_bytes(d, op_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.out_sums = arg_ptr<long long>(d, op_slot);
+    FK_TRY(need_bytes(d, clr_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.clear = arg_ptr<long long>(d, clr_slot);
     FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
     rq.workspace = d.args[ws_slot].ptr;
     rq.spin_limit = d.u("spin_limit", 0);
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
-    rw->writes = {(uint32_t)x_slot, (uint32_t)mid_slot, (uint32_t)op_slot, (uint32_t)ws_slot};
+    rw->writes = {(uint32_t)x_slot, (uint32_t)mid_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
     return plan_xcd_mlp(rq, l);
 }
 
-// partials [8][hidden] fp32, residual [hidden] bf16, x [hidden] bf16 (parameter hidden)
+// sum row, residual [hidden] bf16, x [hidden] bf16, sum row to clear (may be the one read) (parameter hidden)
 fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
-    FK_TRY(need_args(d, 3));
+    FK_TRY(need_args(d, 4));
     const uint32_t hidden = d.u("hidden");
     if (hidden == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden parameter missing");
-    FK_TRY(need_bytes(d, 0, (size_t)kXcds * hidden * 4));
+    FK_TRY(need_bytes(d, 0, xcd_sum_row_bytes(hidden)));
     FK_TRY(need_bytes(d, 1, (size_t)hidden * 2));
     FK_TRY(need_bytes(d, 2, (size_t)hidden * 2));
+    FK_TRY(need_bytes(d, 3, xcd_sum_row_bytes(hidden)));
     rw->reads = {0, 1};
-    rw->writes = {2};
-    return plan_xcd_reduce(arg_ptr<const float>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<uint16_t>(d, 2), hidden, l);
+    rw->writes = {2, 3};
+    return plan_xcd_reduce(arg_ptr<const long long>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<uint16_t>(d, 2),
+                           arg_ptr<long long>(d, 3), hidden, l);
 }
 
 // Q, K0, K1, V, cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]: split-key store + attention of a

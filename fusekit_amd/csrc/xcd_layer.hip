@@ -128,64 +128,94 @@ __device__ __forceinline__ void stage_vector(const uint16_t* src, uint32_t n8, u
 }
 
 // ---- the input of a launch -------------------------------------------------------------------
-// Run by ONE wave of the block (the control wave), while the other waves request the block's weights: a wave
-// issues its memory instructions in order, and a wave that is busy requesting megabytes of weights (the requests
-// are accepted at the rate memory delivers) would not get to the hand-over before they have all gone out.
-//   stage A  this block's rows of x = T(sum of the partial rows + residual) -> this XCD's copy; their sum of squares
-//   hand-over (every block of the XCD has published its rows)
-//   stage B  the whole normalised vector, T(w * T(x * r)), staged into LDS for the projections
-constexpr int kCtlRegs = 8;  // groups of 8 hidden elements per lane of the control wave (hidden <= 4096)
+//   x = T(f32(sum row) + residual) for the WHOLE vector (every block computes all of it: one round trip, no
+//   hand-over), its sum of squares, then T(w * T(x * r)) staged into LDS for the projections.
+// Thread t of the block takes the groups of eight elements t and t + 256 (hidden <= 4096).  The requests go out
+// first (input_request), the block's first weight requests behind them, then the values are used (input_stage).
+constexpr int kInGroups = 2;
 
-template <WKind KIND, int PROBE>
-__device__ __forceinline__ void input_control(const XcdInput& in, XcdSync& sync, uint32_t xcd, uint32_t slot, uint32_t lane,
-                                              uint4* xs, float* sx, uint32_t cs) {
-    const uint32_t r0 = slot * in.rows_per_block;
-    const bool mine = lane < in.rows_per_block && r0 + lane < in.hidden;
-    const uint32_t row = mine ? r0 + lane : (r0 < in.hidden ? r0 : 0u);  // clamped: straight-line loads
-    float p[kXcds];
-#pragma unroll
-    for (uint32_t j = 0; j < kXcds; ++j) p[j] = in.partials ? in.partials[(size_t)j * in.hidden + row] : 0.f;
-    const uint32_t res = in.residual[(size_t)xcd * in.residual_stride + row];
+__device__ __forceinline__ float xcd_sum_to_f32(uint32_t lo, uint32_t hi) {
+    return fmaf((float)lo, kXcdSumInv, (float)(int32_t)hi);
+}
+__device__ __forceinline__ void xcd_sum_add(long long* row, uint32_t e, float v) {
+    const long long q = __float2ll_rn(v * kXcdSumScale);
+    (void)__hip_atomic_fetch_add(reinterpret_cast<unsigned long long*>(row) + xcd_sum_index(e), (unsigned long long)q,
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct InputRegs {
+    uint4 sv[kInGroups][4], rv[kInGroups], nw[kInGroups];
+};
+
+__device__ __forceinline__ void input_request(const XcdInput& in, InputRegs& r) {
+    const uint32_t n8 = in.hidden >> 3, lane = threadIdx.x & (kWave - 1);
+    const uint4* s16 = reinterpret_cast<const uint4*>(in.sums);
+    const uint4* r8 = reinterpret_cast<const uint4*>(in.residual);
     const uint4* w8 = reinterpret_cast<const uint4*>(in.norm_w);
-    const uint32_t n8 = in.hidden >> 3;
-    uint4 nw[kCtlRegs];
-#pragma unroll
-    for (int i = 0; i < kCtlRegs; ++i) {
-        const uint32_t t = lane + i * kWave;
-        nw[i] = w8[t < n8 ? t : 0u];
+    if (in.clear) {  // 16-byte units of the row to clear, spread over the grid
+        const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
+        if (u < in.row_elems / 2) reinterpret_cast<uint4*>(in.clear)[u] = make_uint4(0, 0, 0, 0);
     }
+#pragma unroll
+    for (int i = 0; i < kInGroups; ++i) {
+        const uint32_t t = threadIdx.x + i * kBlock, sec = t >> 6;  // the wave's section of 64 groups
+        if (sec * kWave < n8) {                                      // wave-uniform
+            const uint32_t tc = t < n8 ? t : 0u;
+            if (in.sums) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) r.sv[i][k] = s16[(sec * 4 + k) * kWave + lane];  // padded row: in bounds
+            }
+            r.rv[i] = r8[tc];
+            r.nw[i] = w8[tc];
+        }
+    }
+}
+
+// Whole block (two block barriers inside); `red`: 4 floats of LDS.
+template <WKind KIND, int PROBE>
+__device__ __forceinline__ void input_stage(const XcdInput& in, const InputRegs& r, uint4* xs, float* sx, uint32_t cs,
+                                            float* red) {
+    const uint32_t n8 = in.hidden >> 3;
+    uint4 xv[kInGroups];
     float sq = 0.f;
-    if (mine) {
-        // fixed order: ((p0 + p1) + (p2 + p3)) + ((p4 + p5) + (p6 + p7)), then the residual, one rounding
-        const float acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
-        const uint32_t xb = f32_to_bf16_bits(acc + bf16_bits_to_f32(res));
-        in.x_out[(size_t)xcd * in.hidden + row] = (uint16_t)xb;
-        const float xv = bf16_bits_to_f32(xb);
-        sq = xv * xv;
+#pragma unroll
+    for (int i = 0; i < kInGroups; ++i) {
+        const uint32_t t = threadIdx.x + i * kBlock, sec = t >> 6;
+        if (sec * kWave < n8) {
+            uint32_t xb[4] = {r.rv[i].x, r.rv[i].y, r.rv[i].z, r.rv[i].w};
+            if (in.sums) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float lo = xcd_sum_to_f32(r.sv[i][k].x, r.sv[i][k].y) + bf16_lo(xb[k]);
+                    const float hi = xcd_sum_to_f32(r.sv[i][k].z, r.sv[i][k].w) + bf16_hi(xb[k]);
+                    xb[k] = pack_bf16(lo, hi);
+                }
+            }
+            xv[i] = make_uint4(xb[0], xb[1], xb[2], xb[3]);
+            if (t < n8) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float lo = bf16_lo(xb[k]), hi = bf16_hi(xb[k]);
+                    sq = fmaf(lo, lo, sq);
+                    sq = fmaf(hi, hi, sq);
+                }
+                if (blockIdx.x == 0) reinterpret_cast<uint4*>(in.x_out)[t] = xv[i];
+            }
+        }
     }
     FK_XCD_STAMP(PROBE, 2);
     sq = wave_sum(sq);
-    if (lane == 0) sync.ctl->ssq[xcd * kXcdSlots + slot] = sq;
-    wait_memory_ops_done();
+    if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = sq;
+    __syncthreads();
+    sq = (red[0] + red[1]) + (red[2] + red[3]);
+    const float rr = 1.0f / sqrtf(sq / (float)in.hidden + in.eps);
     FK_XCD_STAMP(PROBE, 3);
-    (void)xcd_publish_and_wait(sync, lane);
-    FK_XCD_STAMP(PROBE, 4);
-    // the whole vector and the 64 block sums of squares (added in a fixed order) are requested together
-    const uint4* x8 = reinterpret_cast<const uint4*>(in.x_out + (size_t)xcd * in.hidden);
-    uint4 xv[kCtlRegs];
 #pragma unroll
-    for (int i = 0; i < kCtlRegs; ++i) {
-        const uint32_t t = lane + i * kWave;
-        xv[i] = ld_u128<true>(x8 + (t < n8 ? t : 0u));
+    for (int i = 0; i < kInGroups; ++i) {
+        const uint32_t t = threadIdx.x + i * kBlock, sec = t >> 6;
+        if (sec * kWave < n8) stage_emit<KIND>(xs, sx, cs, t, t < n8, xv[i], r.nw[i], rr, true);
     }
-    float ss = ld_f32<true>(&sync.ctl->ssq[xcd * kXcdSlots + lane]);
-    ss = wave_sum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)in.hidden + in.eps);
-#pragma unroll
-    for (int i = 0; i < kCtlRegs; ++i) {
-        const uint32_t t = lane + i * kWave;
-        if ((uint32_t)i * kWave < n8) stage_emit<KIND>(xs, sx, cs, t, t < n8, xv[i], nw[i], r, true);
-    }
+    __syncthreads();
 }
 
 // ---- projection tiles ----------------------------------------------------------------------------
@@ -246,27 +276,49 @@ __device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, const 
 }
 
 // Group gi of the tile = (row gi / gpr, group gi % gpr of the row's slice), gpr groups per row slice.
-template <WKind KIND, int SN>
+// A vector memory instruction costs the CU about as much to issue whether it moves 2 or 16 bytes per lane, so
+// a tile of whole rows whose row holds a multiple of four groups (its groups are then one contiguous,
+// 8-byte-aligned run of the scale and of the bias array) is fetched four groups per lane and instruction.
+// RUN: the tile spans whole rows of a multiple of four groups (the host plans it so).
+template <WKind KIND, int SN, bool RUN>
 __device__ __forceinline__ void meta_fetch(const XcdMat& m, const Tile& t, uint32_t ti, MetaRegs& r) {
     if constexpr (KIND != W_BF16) {
         const uint32_t gpr = t.cs >> m.gshift, total = t.rows * gpr;
-        const float inv = 1.0f / (float)gpr;
         const size_t g0 = (size_t)t.row0 * (m.cpr >> m.gshift) + (t.col0 >> m.gshift);
+        if constexpr (RUN) {
+            // kMetaRegs * SN groups at most: lane ti takes groups 4 ti .. 4 ti + 3 (s[0..1] / b[0..1] hold them)
+            const uint32_t gi = 4u * ti;
+            const size_t e = gi < total ? g0 + gi : g0;
+            const uint2 sv = *reinterpret_cast<const uint2*>(m.sc + e), bv = *reinterpret_cast<const uint2*>(m.bi + e);
+            r.s[0] = sv.x;
+            r.s[1] = sv.y;
+            r.b[0] = bv.x;
+            r.b[1] = bv.y;
+        } else {
+            const float inv = 1.0f / (float)gpr;
 #pragma unroll
-        for (int k = 0; k < kMetaRegs; ++k) {
-            const uint32_t gi = k * SN + ti;
-            const uint32_t row = (uint32_t)(((float)gi + 0.5f) * inv);
-            const size_t e = gi < total ? g0 + (size_t)row * (m.cpr >> m.gshift) + (gi - row * gpr) : g0;
-            r.s[k] = m.sc[e];
-            r.b[k] = m.bi[e];
+            for (int k = 0; k < kMetaRegs; ++k) {
+                const uint32_t gi = k * SN + ti;
+                const uint32_t row = (uint32_t)(((float)gi + 0.5f) * inv);
+                const size_t e = gi < total ? g0 + (size_t)row * (m.cpr >> m.gshift) + (gi - row * gpr) : g0;
+                r.s[k] = m.sc[e];
+                r.b[k] = m.bi[e];
+            }
         }
     }
 }
-template <WKind KIND, int SN>
+template <WKind KIND, int SN, bool RUN>
 __device__ __forceinline__ void meta_store(const MetaRegs& r, uint32_t ti, uint32_t* meta) {
     if constexpr (KIND != W_BF16) {
+        if constexpr (RUN) {
+            if (4u * ti < (uint32_t)kMetaRegs * SN)
+                *reinterpret_cast<uint4*>(meta + 4u * ti) =
+                    make_uint4((r.s[0] & 0xffffu) | (r.b[0] << 16), (r.s[0] >> 16) | (r.b[0] & 0xffff0000u),
+                               (r.s[1] & 0xffffu) | (r.b[1] << 16), (r.s[1] >> 16) | (r.b[1] & 0xffff0000u));
+        } else {
 #pragma unroll
-        for (int k = 0; k < kMetaRegs; ++k) meta[k * SN + ti] = r.s[k] | (r.b[k] << 16);
+            for (int k = 0; k < kMetaRegs; ++k) meta[k * SN + ti] = r.s[k] | (r.b[k] << 16);
+        }
     }
 }
 
@@ -416,11 +468,10 @@ __host__ __device__ inline uint32_t xcd_lds_bytes(const LdsPlan& p) {
 }  // namespace
 
 // =============================================================================================== MLP launch
-// 320 threads: waves 0..3 stream and multiply, wave 4 is the control wave (input reduction, hand-over polls).
-constexpr int kMlpBlock = kBlock + kWave;
+constexpr int kMlpBlock = kBlock;
 
 template <WKind KIND, int NLA, int NLB>
-__global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) {
+__global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) {
     extern __shared__ uint4 lds_raw[];
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
@@ -428,6 +479,7 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
     float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
     float* work = sx + cs_max;
     uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]
+    float* red = reinterpret_cast<float*>(meta + 3 * kMetaWords);      // [16]
 
     XcdSync sync;
     sync.ctl = a.ctl;
@@ -441,7 +493,7 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
     sync.aborted = false;
     sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t tid = threadIdx.x;
-    const bool streams = tid < (uint32_t)kBlock;
+    constexpr bool streams = true;
 
     FK_XCD_STAMP(1, 0);
     const uint32_t per_xcd = a.inter / kXcds;
@@ -457,27 +509,24 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
     TileRegs<NLB> rd;
     TilePos<NLA> pg;
     TilePos<NLB> pd;
-    sync.epoch += 1;  // the input hand-over
-    if (streams) {
-        // Requested now: the groups' scales and biases and the first pass of gate / up -- a few KiB per CU, so
-        // that the control wave's small requests are not queued behind megabytes.  The later passes stream
-        // while the earlier ones are consumed; the down_proj slice is queued behind the last of them.
-        tile_pos_init<NLA, kBlock>(tg, tid, pg);
-        tile_pos_init<NLB, kBlock>(td, tid, pd);
-        meta_fetch<KIND, kBlock>(a.gate, tg, tid, mg);
-        meta_fetch<KIND, kBlock>(a.up, tg, tid, mu);
-        meta_fetch<KIND, kBlock>(a.down, td, tid, md);
-        tile_load<KIND, NLA>(a.gate, tg, pg, rg);
-        tile_load<KIND, NLA>(a.up, tg, pg, ru);
-        FK_XCD_STAMP(1, 1);
-        meta_store<KIND, kBlock>(mg, tid, meta);
-        meta_store<KIND, kBlock>(mu, tid, meta + kMetaWords);
-        meta_store<KIND, kBlock>(md, tid, meta + 2 * kMetaWords);
-    } else {
-        input_control<KIND, 1>(a.in, sync, sync.xcd, sync.slot, tid - kBlock, xs, sx, a.gate.cpr);
-    }
-    __syncthreads();
+    InputRegs inr;
+    // Requested now, behind the input: the groups' scales and biases and the first pass of gate / up -- a few
+    // KiB per CU.  The later passes stream while the earlier ones are consumed; the down_proj slice is queued
+    // behind the last of them.
+    input_request(a.in, inr);
+    tile_pos_init<NLA, kBlock>(tg, tid, pg);
+    tile_pos_init<NLB, kBlock>(td, tid, pd);
+    meta_fetch<KIND, kBlock, true>(a.gate, tg, tid, mg);
+    meta_fetch<KIND, kBlock, true>(a.up, tg, tid, mu);
+    tile_load<KIND, NLA>(a.gate, tg, pg, rg);
+    tile_load<KIND, NLA>(a.up, tg, pg, ru);
+    FK_XCD_STAMP(1, 1);
+    input_stage<KIND, 1>(a.in, inr, xs, sx, a.gate.cpr, red);
     FK_XCD_STAMP(1, 5);
+    meta_store<KIND, kBlock, true>(mg, tid, meta);
+    meta_store<KIND, kBlock, true>(mu, tid, meta + kMetaWords);
+    meta_fetch<KIND, kBlock, false>(a.down, td, tid, md);  // not needed before the hand-over: kept off the start-up path
+    __syncthreads();
 
     // ---- gate / up rows of this XCD's slice, SwiGLU ----
     const uint32_t seg = (gu_n * a.gate.cpr + NLA * kBlock - 1) / (NLA * kBlock) * (NLA * kBlock);
@@ -490,6 +539,7 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
             request_down();
     }
     FK_XCD_STAMP(1, 6);
+    meta_store<KIND, kBlock, false>(md, tid, meta + 2 * kMetaWords);
     __syncthreads();
     if (streams && gu_n) {
         uint16_t* mid = a.mid + (size_t)sync.xcd * per_xcd + gu0;
@@ -498,7 +548,7 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
                         [&](uint32_t r, float s0, float s1) { mid[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
     }
     FK_XCD_STAMP(1, 7);
-    xcd_barrier<kBlock>(sync);
+    xcd_barrier<0>(sync);
     FK_XCD_STAMP(1, 8);
 
     // ---- down_proj over this XCD's K-slice: fp32 partial row ----
@@ -509,16 +559,14 @@ __global__ __launch_bounds__(kMlpBlock) void xcd_mlp_kernel(const XcdMlpArgs a) 
     __syncthreads();
     FK_XCD_STAMP(1, 10);
     if (streams && d_n) {
-        float* out = a.out_partials + (size_t)sync.xcd * a.in.hidden + d0;
-        tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { out[r] = s0; });
+        long long* out = a.out_sums;
+        tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, d0 + r, s0); });
     }
     FK_XCD_STAMP(1, 11);
 }
 
 // =============================================================================================== attention launch
-// 256 threads (the attention phase wants exactly four waves): until the input is staged wave 0 is the control
-// wave and waves 1..3 request the weights; afterwards all four are peers.
-constexpr int kAttnStream = kBlock - kWave;
+constexpr int kAttnStream = kBlock;
 
 template <WKind KIND, int NLA, int NLB>
 __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a) {
@@ -540,9 +588,9 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     sync.aborted = false;
     sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t kv_len0 = *a.sdpa.kv_len_ptr;
-    const uint32_t tid = threadIdx.x;
-    const bool streams = tid >= (uint32_t)kWave;
-    const uint32_t ti = tid - kWave;  // index among the streaming threads
+    const uint32_t tid = threadIdx.x, ti = tid;
+    constexpr bool streams = true;
+    float* red = reinterpret_cast<float*>(att + ((att_elems + 7u) & ~7u));  // [16]
 
     FK_XCD_STAMP(0, 0);
     // tile of the q / k / v projections: the XCD's q rows first, then its k rows, then its v rows
@@ -564,21 +612,18 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     TileRegs<NLB> ro;
     TilePos<NLA> pq;
     TilePos<NLB> po;
-    sync.epoch += 1;  // the input hand-over
-    if (streams) {
-        tile_pos_init<NLA, kAttnStream>(tq, ti, pq);
-        tile_pos_init<NLB, kAttnStream>(to, ti, po);
-        meta_fetch<KIND, kAttnStream>(mq, tq, ti, mmq);
-        meta_fetch<KIND, kAttnStream>(a.wo, to, ti, mmo);
-        tile_load<KIND, NLA>(mq, tq, pq, rq);
-        FK_XCD_STAMP(0, 1);
-        meta_store<KIND, kAttnStream>(mmq, ti, meta);
-        meta_store<KIND, kAttnStream>(mmo, ti, meta + kMetaWords);
-    } else {
-        input_control<KIND, 0>(a.in, sync, sync.xcd, sync.slot, tid, xs, sx, a.wq.cpr);
-    }
-    __syncthreads();
+    InputRegs inr;
+    input_request(a.in, inr);
+    tile_pos_init<NLA, kAttnStream>(tq, ti, pq);
+    tile_pos_init<NLB, kAttnStream>(to, ti, po);
+    meta_fetch<KIND, kAttnStream, true>(mq, tq, ti, mmq);
+    tile_load<KIND, NLA>(mq, tq, pq, rq);
+    FK_XCD_STAMP(0, 1);
+    input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red);
     FK_XCD_STAMP(0, 5);
+    meta_store<KIND, kAttnStream, true>(mmq, ti, meta);
+    meta_fetch<KIND, kAttnStream, false>(a.wo, to, ti, mmo);  // not needed before the attention is done
+    __syncthreads();
 
     // ---- q / k / v rows of this XCD's KV head; the o_proj slice is requested behind their last pass ----
     if (streams) {
@@ -588,6 +633,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
         else
             request_o();
     }
+    meta_store<KIND, kAttnStream, false>(mmo, ti, meta + kMetaWords);
     __syncthreads();
     if (pr_n) {
         uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
@@ -673,8 +719,8 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     __syncthreads();
     FK_XCD_STAMP(0, 11);
     if (o_n) {
-        float* out = a.out_partials + (size_t)sync.xcd * a.in.hidden + o0;
-        tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { out[r] = s0; });
+        long long* out = a.out_sums;
+        tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, o0 + r, s0); });
     }
     FK_XCD_STAMP(0, 12);
 }
@@ -682,11 +728,10 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
 __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= a.hidden) return;
-    float p[kXcds];
-#pragma unroll
-    for (uint32_t j = 0; j < kXcds; ++j) p[j] = a.partials[(size_t)j * a.hidden + i];
-    const float acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
-    a.x[i] = (uint16_t)f32_to_bf16_bits(acc + bf16_bits_to_f32(a.residual[i]));
+    const uint32_t at = xcd_sum_index(i);
+    const unsigned long long s = (unsigned long long)a.sums[at];
+    a.x[i] = (uint16_t)f32_to_bf16_bits(xcd_sum_to_f32((uint32_t)s, (uint32_t)(s >> 32)) + bf16_bits_to_f32(a.residual[i]));
+    if (a.clear) a.clear[at] = 0;
 }
 
 // =============================================================================================== host side
@@ -707,6 +752,8 @@ fk_status bind_mat(const fk_weight* w, uint32_t n, uint32_t k, const XcdLayerSha
     if (w->n != n || w->k != k || w->bits != s.bits || (s.bits != 16 && w->group != s.group))
         return set_error(FK_ERR_INVALID, std::string("xcd layer: weight ") + what + " does not match the layer shape");
     if (s.bits != 16 && (!w->scales || !w->biases)) return set_error(FK_ERR_INVALID, std::string("xcd layer: null scales / biases of ") + what);
+    if (((uintptr_t)w->w & 15u) || (s.bits != 16 && (((uintptr_t)w->scales | (uintptr_t)w->biases) & 7u)))
+        return set_error(FK_ERR_INVALID, std::string("xcd layer: ") + what + " needs 16-byte aligned weights and 8-byte aligned scales / biases");
     m->w = reinterpret_cast<const uint4*>(w->w);
     m->sc = w->scales;
     m->bi = w->biases;
@@ -724,19 +771,20 @@ uint32_t lds_for(uint32_t bits, const LdsPlan& p) {
     return bits == 4 ? xcd_lds_bytes<W_Q4>(p) : (bits == 8 ? xcd_lds_bytes<W_Q8>(p) : xcd_lds_bytes<W_BF16>(p));
 }
 
-fk_status fill_input(const XcdLayerShape& s, const float* partials, const uint16_t* residual, uint32_t residual_stride,
-                     uint16_t* x_out, const uint16_t* norm_w, float eps, XcdInput* in) {
+fk_status fill_input(const XcdLayerShape& s, const long long* sums, const uint16_t* residual, uint16_t* x_out,
+                     long long* clear, const long long* out_sums, const uint16_t* norm_w, float eps, XcdInput* in) {
     if (!residual || !x_out || !norm_w) return set_error(FK_ERR_INVALID, "xcd layer: null residual, x_out or norm weight");
-    if (residual_stride != 0 && residual_stride != s.hidden)
-        return set_error(FK_ERR_INVALID, "xcd layer: residual stride must be 0 (one row) or hidden (a copy per XCD)");
-    in->partials = partials;
+    if (residual == x_out) return set_error(FK_ERR_INVALID, "xcd layer: x_out must not be the residual row");
+    if (out_sums == sums || out_sums == clear || (clear && clear == sums))
+        return set_error(FK_ERR_INVALID, "xcd layer: the sum rows read, added into and cleared must be three different rows");
+    in->sums = sums;
     in->residual = residual;
-    in->residual_stride = residual_stride;
     in->x_out = x_out;
+    in->clear = clear;
     in->norm_w = norm_w;
     in->eps = eps;
     in->hidden = s.hidden;
-    in->rows_per_block = ceil_div(s.hidden, kXcdSlots);
+    in->row_elems = xcd_sum_row_elems(s.hidden);
     return FK_OK;
 }
 
@@ -763,7 +811,8 @@ fk_status xcd_layer_supported(const XcdLayerShape& s) {
     const uint32_t G = s.n_heads / s.n_kv;
     if (G != 1 && G != 2 && G != 4 && G != 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: 1, 2, 4 or 8 query heads per KV head");
     if (s.head_dim != 64 && s.head_dim != 128) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: head_dim must be 64 or 128");
-    if (s.hidden % 64 || s.hidden > (uint32_t)kCtlRegs * kWave * 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: hidden must be a multiple of 64, at most 4096");
+    if (s.hidden % 64 || s.hidden > (uint32_t)kInGroups * kBlock * 8) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: hidden must be a multiple of 64, at most 4096");
+    if (s.bits != 16 && (s.hidden / s.group) % 4) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: hidden must hold a multiple of four quantisation groups");
     if ((G * s.head_dim) % unit) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a KV head's query columns must be whole quantisation groups");
     if (s.inter % (kXcds * unit) || s.inter % (kXcds * 8)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: intermediate / 8 must be whole quantisation groups");
     if (s.capacity == 0) return set_error(FK_ERR_INVALID, "xcd layer: zero cache capacity");
@@ -781,6 +830,7 @@ fk_status xcd_layer_supported(const XcdLayerShape& s) {
 }
 
 size_t xcd_workspace_bytes() { return sizeof(XcdControl); }
+size_t xcd_sum_row_bytes(uint32_t hidden) { return (size_t)xcd_sum_row_elems(hidden) * sizeof(long long); }
 
 size_t xcd_attn_partials_bytes(const XcdLayerShape& s) {
     return (size_t)s.n_heads * kXcdMaxRanges * (s.head_dim + 2) * sizeof(float);
@@ -789,11 +839,11 @@ size_t xcd_attn_partials_bytes(const XcdLayerShape& s) {
 fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     const XcdLayerShape& s = rq.shape;
     FK_TRY(xcd_layer_supported(s));
-    if (!rq.mid || !rq.out_partials || !rq.workspace) return set_error(FK_ERR_INVALID, "xcd mlp: null mid, partial rows or workspace");
+    if (!rq.mid || !rq.out_sums || !rq.workspace) return set_error(FK_ERR_INVALID, "xcd mlp: null mid, sum row or workspace");
     if (rq.swiglu_variant < 0 || rq.swiglu_variant > 2) return set_error(FK_ERR_INVALID, "xcd mlp: swiglu variant must be 0, 1 or 2");
     XcdMlpArgs a;
     memset(&a, 0, sizeof(a));
-    FK_TRY(fill_input(s, rq.partials_in, rq.residual, rq.residual_stride, rq.x_out, rq.norm_w, rq.eps, &a.in));
+    FK_TRY(fill_input(s, rq.sums_in, rq.residual, rq.x_out, rq.clear, rq.out_sums, rq.norm_w, rq.eps, &a.in));
     FK_TRY(bind_mat(rq.wgate, s.inter, s.hidden, s, &a.gate, "gate_proj"));
     FK_TRY(bind_mat(rq.wup, s.inter, s.hidden, s, &a.up, "up_proj"));
     FK_TRY(bind_mat(rq.wdown, s.hidden, s.inter, s, &a.down, "down_proj"));
@@ -803,7 +853,7 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     a.down_cs = a.down.cpr / kXcds;
     a.swiglu_variant = rq.swiglu_variant;
     a.mid = rq.mid;
-    a.out_partials = rq.out_partials;
+    a.out_sums = rq.out_sums;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
     auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
@@ -828,13 +878,13 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     const XcdLayerShape& s = rq.shape;
     FK_TRY(xcd_layer_supported(s));
     if (!rq.q || !rq.k || !rq.v || !rq.cache_k || !rq.cache_v || !rq.kv_len || !rq.rope_tab || !rq.att_partials ||
-        !rq.out_partials || !rq.workspace)
+        !rq.out_sums || !rq.workspace)
         return set_error(FK_ERR_INVALID, "xcd attention: null buffer");
     if ((rq.q_norm == nullptr) != (rq.k_norm == nullptr)) return set_error(FK_ERR_INVALID, "xcd attention: q and k head norms come together");
     const uint32_t G = s.n_heads / s.n_kv, n_q = s.n_heads * s.head_dim, n_kvd = s.n_kv * s.head_dim;
     XcdAttnArgs a;
     memset(&a, 0, sizeof(a));
-    FK_TRY(fill_input(s, rq.partials_in, rq.residual, rq.residual_stride, rq.x_out, rq.norm_w, rq.eps, &a.in));
+    FK_TRY(fill_input(s, rq.sums_in, rq.residual, rq.x_out, rq.clear, rq.out_sums, rq.norm_w, rq.eps, &a.in));
     FK_TRY(bind_mat(rq.wq, n_q, s.hidden, s, &a.wq, "q_proj"));
     FK_TRY(bind_mat(rq.wk, n_kvd, s.hidden, s, &a.wk, "k_proj"));
     FK_TRY(bind_mat(rq.wv, n_kvd, s.hidden, s, &a.wv, "v_proj"));
@@ -887,7 +937,7 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     sd.rope_tab = rq.rope_tab;
     sd.v_stride = s.head_dim;
     sd.k1_heads = 1;
-    a.out_partials = rq.out_partials;
+    a.out_sums = rq.out_sums;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
     auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kAttnStream) * nl * kAttnStream; };
@@ -912,11 +962,12 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     return FK_OK;
 }
 
-fk_status plan_xcd_reduce(const float* partials, const uint16_t* residual, uint16_t* x, uint32_t hidden, Launch* out) {
+fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
+                          Launch* out) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
-    if (!partials || !residual || !x || hidden == 0) return set_error(FK_ERR_INVALID, "xcd reduce: null buffer or zero width");
-    XcdReduceArgs a{partials, residual, x, hidden};
+    if (!sums || !residual || !x || hidden == 0) return set_error(FK_ERR_INVALID, "xcd reduce: null buffer or zero width");
+    XcdReduceArgs a{sums, residual, x, clear, hidden};
     out->func = reinterpret_cast<const void*>(&xcd_reduce_kernel);
     out->grid = dim3(ceil_div(hidden, kBlock), 1, 1);
     out->block = dim3(kBlock, 1, 1);

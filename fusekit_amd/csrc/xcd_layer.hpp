@@ -10,18 +10,23 @@
 //
 // The layer is cut so that every hand-over but two stays inside an XCD:
 //
-//   attention launch   x = T(sum of the previous launch's 8 partial rows + residual); RMSNorm;
+//   attention launch   x = T(sum row of the previous launch + residual); RMSNorm;
 //                      XCD h: q / k / v rows of KV head h  ->  head norm + RoPE + cache append +
 //                      attention of KV head h (its G query heads, S key ranges)  ->  merge  ->
-//                      o_proj restricted to the K-slice of those heads, ALL output rows: fp32 partial
-//                      row h of 8.
-//   MLP launch         x1 = T(sum of the 8 o_proj partial rows + residual); RMSNorm;
+//                      o_proj restricted to the K-slice of those heads, ALL output rows, each added
+//                      into the launch's sum row.
+//   MLP launch         x1 = T(sum row of the attention launch + residual); RMSNorm;
 //                      XCD h: gate / up rows [h I/8, (h+1) I/8) + SwiGLU  ->  down_proj restricted to
-//                      that K-slice, ALL output rows: fp32 partial row h of 8.
+//                      that K-slice, ALL output rows, each added into the launch's sum row.
 //
-// The sum over the 8 partial rows is taken in a fixed order by the NEXT launch (the kernel boundary makes
-// them visible), so results do not depend on timing.  Every block issues the weight loads of BOTH of its
-// projections when it starts; the hand-overs only gate arithmetic.
+// The sum row: every output element receives eight contributions, one per XCD.  They are added as 64-bit
+// fixed-point integers (2^-32 units) with memory-side atomic adds -- integer addition is associative, so the
+// row does not depend on the order of arrival, and a contribution of magnitude >= 2^-8 is carried exactly.
+// The NEXT launch reads the finished row behind the kernel boundary: every block takes the whole row (20 KB at
+// hidden 2560), adds the residual, and has the vector and its sum of squares without waiting for any other
+// block.  Three rows rotate: a launch reads one, adds into the second and clears the third for the launch
+// after it.  Every block requests the weights of BOTH of its projections when it starts; the hand-overs only
+// gate arithmetic.
 //
 // Hand-over protocol inside an XCD: block (xcd, slot) owns one 32-bit flag word.  It reads the word when
 // it starts (base), and publishes base + k with an ordinary store after the stores of stage k have been
@@ -42,14 +47,24 @@ constexpr uint32_t kXcdMaxRanges = 16;              // key ranges merged per que
 
 // Control words of the protocol, one allocation per decoder (fk_xcd_workspace_bytes):
 //   flags[8][64]   uint32   arrival word of block (xcd, slot)
-//   ssq[8][64]     float    per-block sums of squares of the rows a block reduced
 //   abort          uint32   set when a wait ran into the spin limit
 struct XcdControl {
     uint32_t flags[kXcds * kXcdSlots];
-    float ssq[kXcds * kXcdSlots];
     uint32_t abort_flag;
     uint32_t pad[63];
 };
+
+// A sum row: hidden 64-bit fixed-point sums (value * 2^32), padded to whole 512-element sections.  Inside a
+// section the elements are permuted so that the control wave of a block, whose lane l takes the eight
+// elements 8 (l + 64 i) .. + 7 in step i, reads 1 KiB contiguous per instruction: element e sits at
+// xcd_sum_index(e).
+constexpr float kXcdSumScale = 4294967296.0f;
+constexpr float kXcdSumInv = 1.0f / 4294967296.0f;
+__host__ __device__ inline uint32_t xcd_sum_index(uint32_t e) {
+    const uint32_t t = e >> 3;
+    return (((((t >> 6) * 4u + ((e & 7u) >> 1)) * 64u + (t & 63u)) << 1) | (e & 1u));
+}
+inline uint32_t xcd_sum_row_elems(uint32_t hidden) { return (hidden + 511u) / 512u * 512u; }
 
 // One projection restricted to a row block and a K-slice: rows [row0, row0 + rows) of a [n, K] matrix,
 // chunks [col0, col0 + cs) of each row's cpr 16-byte chunks.
@@ -61,17 +76,18 @@ struct XcdMat {
     uint32_t gshift;   // chunk index >> gshift = quantisation group
 };
 
-// The input of a launch: hidden = T(sum_j partial[j][i] + residual[i]) (n_partials = 0: the residual alone),
-// written to x_out (one copy per XCD) and RMS-normalised with norm_w for the projections.
+// The input of a launch: x[i] = T(f32(sums[i]) + residual[i]) (sums null: the residual alone), written to x_out
+// by workgroup 0 and RMS-normalised with norm_w for the projections; f32(s) = fma(f32(low word), 2^-32,
+// f32(high word)).
 struct XcdInput {
-    const float* partials;      // [8][hidden] or null
-    const uint16_t* residual;   // [hidden] (stride 0) or one copy per XCD (stride hidden)
-    uint32_t residual_stride;
-    uint16_t* x_out;            // [8][hidden]
+    const long long* sums;      // sum row of the previous launch, or null
+    const uint16_t* residual;   // [hidden]
+    uint16_t* x_out;            // [hidden]
+    long long* clear;           // sum row this launch zeroes (the one the launch after it adds into), or null
     const uint16_t* norm_w;
     float eps;
     uint32_t hidden;
-    uint32_t rows_per_block;    // hidden rows one block reduces (ceil(hidden / 64))
+    uint32_t row_elems;         // elements of a (padded) sum row
 };
 
 struct XcdMlpArgs {
@@ -83,7 +99,7 @@ struct XcdMlpArgs {
     uint32_t down_cs;           // chunks of one XCD's K-slice of a down_proj row
     int swiglu_variant;
     uint16_t* mid;              // [inter] bf16, every XCD touches only its slice
-    float* out_partials;        // [8][hidden] fp32
+    long long* out_sums;        // sum row the down_proj outputs are added into
     XcdControl* ctl;
     uint32_t spin_limit;
     uint32_t cs_max, work_floats;  // LDS layout: chunks of the longest staged vector, floats of the work area
@@ -101,17 +117,19 @@ struct XcdAttnArgs {
     uint16_t* k;                // [n_kv * head_dim]
     uint16_t* v;
     SdpaArgs sdpa;              // attention of one KV head per XCD: n_splits ranges x G heads = 64 blocks
-    float* out_partials;        // [8][hidden] fp32
+    long long* out_sums;        // sum row the o_proj outputs are added into
     XcdControl* ctl;
     uint32_t spin_limit;
     uint32_t cs_max, work_floats, att_elems;  // LDS layout (att_elems: bf16 elements of the merged attention rows)
 };
 
-// x = T(sum of 8 partial rows + residual): the last layer's output for the LM head.
+// x = T(f32(sums) + residual): the last layer's output for the LM head.  `clear` (may be the row read, or null)
+// is zeroed element by element behind the read: the row the next token's first launch adds into.
 struct XcdReduceArgs {
-    const float* partials;
-    const uint16_t* residual;   // one copy per XCD: copy 0 is read
+    const long long* sums;
+    const uint16_t* residual;
     uint16_t* x;
+    long long* clear;
     uint32_t hidden;
 };
 
@@ -123,14 +141,15 @@ struct XcdLayerShape {
 // whole quantisation groups, tiles that fit the per-thread load budget.)  Sets an error message if not.
 fk_status xcd_layer_supported(const XcdLayerShape& s);
 size_t xcd_workspace_bytes();
+size_t xcd_sum_row_bytes(uint32_t hidden);
 size_t xcd_attn_partials_bytes(const XcdLayerShape& s);
 
 struct XcdAttnRequest {
     XcdLayerShape shape;
-    const float* partials_in;        // previous MLP launch's partial rows, or null (first layer)
+    const long long* sums_in;        // previous MLP launch's sum row, or null (first layer)
     const uint16_t* residual;
-    uint32_t residual_stride;
     uint16_t* x_out;
+    long long* clear;
     const uint16_t* norm_w;
     float eps;
     const fk_weight *wq, *wk, *wv, *wo;
@@ -141,7 +160,7 @@ struct XcdAttnRequest {
     const float* rope_tab;
     float theta;
     float* att_partials;
-    float* out_partials;
+    long long* out_sums;
     void* workspace;
     uint32_t spin_limit;
 };
@@ -149,20 +168,21 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out);
 
 struct XcdMlpRequest {
     XcdLayerShape shape;
-    const float* partials_in;
+    const long long* sums_in;
     const uint16_t* residual;
-    uint32_t residual_stride;
     uint16_t* x_out;
+    long long* clear;
     const uint16_t* norm_w;
     float eps;
     const fk_weight *wgate, *wup, *wdown;
     int swiglu_variant;
     uint16_t* mid;
-    float* out_partials;
+    long long* out_sums;
     void* workspace;
     uint32_t spin_limit;
 };
 fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out);
-fk_status plan_xcd_reduce(const float* partials, const uint16_t* residual, uint16_t* x, uint32_t hidden, Launch* out);
+fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
+                          Launch* out);
 
 }  // namespace fk

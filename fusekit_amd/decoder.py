@@ -224,8 +224,9 @@ class DecoderRuntime:
             ctl, ap = native.xcd_workspace_bytes(cfg.n_heads, cfg.head_dim)
             self.xcd_ctl = z(ctl)
             self.xcd_att_partials = DeviceBuffer(ap)
-            self.xcd_xa, self.xcd_xb = DeviceBuffer(8 * cfg.hidden * 2), DeviceBuffer(8 * cfg.hidden * 2)
-            self.xcd_o_part, self.xcd_down_part = DeviceBuffer(8 * cfg.hidden * 4), DeviceBuffer(8 * cfg.hidden * 4)
+            self.xcd_xa, self.xcd_xb = DeviceBuffer(cfg.hidden * 2), DeviceBuffer(cfg.hidden * 2)
+            # three rotating sum rows: a launch reads one, adds into the next and clears the third
+            self.xcd_sums = [z(native.xcd_sum_row_bytes(cfg.hidden)) for _ in range(3)]
         self._bf16_weights: Dict[str, DeviceWeight] = {}   # resident bf16 copies for prompt passes (prefill_rows)
         self.tasks = self.build_tasks()
         # persistent: the same task list, run by one whole-token kernel per replay
@@ -348,8 +349,10 @@ class DecoderRuntime:
         return t
 
     def _xcd_layer_tasks(self, t: List[Dispatch], name) -> None:
-        """Two launches per layer (families fusekit_xcd_attn_block / fusekit_xcd_mlp_block), then the reduction of
-        the last layer's partial rows into x[0] for the LM head."""
+        """Two launches per layer (families fusekit_xcd_attn_block / fusekit_xcd_mlp_block), then the last layer's
+        sum row + residual into x[0] for the LM head.  Launch i of the token reads sum row i % 3, adds into row
+        (i + 1) % 3 and clears row (i + 2) % 3; the first launch adds into row 1, which the closing reduction
+        leaves cleared for the next token."""
         c, w = self.cfg, self.w
         shape = dict(hidden=c.hidden, inter=c.inter, n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim,
                      capacity=c.capacity, bits=c.bits, group=c.group, eps=c.eps, theta=c.theta,
@@ -358,7 +361,8 @@ class DecoderRuntime:
         for l in range(c.n_layers):
             p = f"layers.{l}."
             Wq, Wk, Wv, Wo = (w.mats[p + f"self_attn.{n}_proj"] for n in "qkvo")
-            a = [] if l == 0 else [arg(self.xcd_down_part)]
+            S = lambda i: arg(self.xcd_sums[i % 3])
+            a = [] if l == 0 else [S(2 * l)]
             a += [arg(self.x[0]) if l == 0 else arg(self.xcd_xb), arg(self.xcd_xa), arg(w.vecs[p + "input_layernorm"]),
                   arg(Wq.w), arg(Wk.w), arg(Wv.w)]
             if quant:
@@ -367,24 +371,25 @@ class DecoderRuntime:
             if c.qk_norm:
                 a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
             a += [arg(self.q), arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
-                  arg(self.rope_tab), arg(self.xcd_att_partials), arg(self.xcd_o_part), arg(self.xcd_ctl)]
-            t.append(Dispatch(name("xcd_attn_block"), a,
-                              dict(shape, has_partials=int(l > 0), residual_per_xcd=int(l > 0), has_norm=int(c.qk_norm))))
+                  arg(self.rope_tab), arg(self.xcd_att_partials), S(2 * l + 1), S(2 * l + 2), arg(self.xcd_ctl)]
+            t.append(Dispatch(name("xcd_attn_block"), a, dict(shape, has_sums=int(l > 0), has_norm=int(c.qk_norm))))
             Wg, Wu, Wd = (w.mats[p + f"mlp.{n}_proj"] for n in ("gate", "up", "down"))
-            m = [arg(self.xcd_o_part), arg(self.xcd_xa), arg(self.xcd_xb), arg(w.vecs[p + "post_attention_layernorm"]),
+            m = [S(2 * l + 1), arg(self.xcd_xa), arg(self.xcd_xb), arg(w.vecs[p + "post_attention_layernorm"]),
                  arg(Wg.w), arg(Wu.w)]
             if quant:
                 m += [arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases)]
-            m += self._wargs(Wd) + [arg(self.mid), arg(self.xcd_down_part), arg(self.xcd_ctl)]
-            t.append(Dispatch(name("xcd_mlp_block"), m,
-                              dict(shape, has_partials=1, residual_per_xcd=1, variant=c.swiglu_variant)))
-        t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_down_part), arg(self.xcd_xb, c.hidden * 2), arg(self.x[0])],
-                          dict(hidden=c.hidden)))
+            m += self._wargs(Wd) + [arg(self.mid), S(2 * l + 2), S(2 * l + 3), arg(self.xcd_ctl)]
+            t.append(Dispatch(name("xcd_mlp_block"), m, dict(shape, has_sums=1, variant=c.swiglu_variant)))
+        t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_sums[(2 * c.n_layers) % 3]), arg(self.xcd_xb), arg(self.x[0]),
+                                               arg(self.xcd_sums[1])], dict(hidden=c.hidden)))
 
     # -- generation ------------------------------------------------------------------
     def reset(self) -> None:
         for b in (self.step_counter, self.offset, self.kv_len, self.hist_counter):
             b.upload(np.zeros(1, np.uint32))
+        if self.xcd:
+            for b in self.xcd_sums:
+                b.upload(np.zeros(b.nbytes, np.uint8))
 
     def prefill(self, prompt: Sequence[int], start_offset: int = 0) -> int:
         """Feeds the prompt through the decode graph with forced tokens; returns the greedy

@@ -501,6 +501,21 @@ def xcd_workspace_bytes(n_heads, head_dim):
     return a.value, b.value
 
 
+lib.fk_xcd_sum_row_bytes.restype = C.c_size_t
+
+
+def xcd_sum_row_bytes(hidden: int) -> int:
+    return int(lib.fk_xcd_sum_row_bytes(C.c_uint32(hidden)))
+
+
+def xcd_sum_index(hidden: int):
+    """Index of element e of a hidden-wide vector inside a sum row (numpy array of hidden indices)."""
+    import numpy as np
+    e = np.arange(hidden, dtype=np.int64)
+    t = e >> 3
+    return ((((t >> 6) * 4 + ((e & 7) >> 1)) * 64 + (t & 63)) << 1) | (e & 1)
+
+
 def xcd_check(workspace, stream=None) -> None:
     check(lib.fk_xcd_check(_ptr(workspace), _ptr(stream)))
 

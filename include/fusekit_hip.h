@@ -488,13 +488,23 @@ fk_status fk_rope_store_sdpa_decode(const uint16_t *q, const uint16_t *k, const 
  * rmsnorm_gateup_swiglu.rs + linear_residual.rs of the MLP half); `fusekit_xcd_reduce` finishes the last
  * layer's output row for final_rmsnorm_lm_head.rs.  Same arithmetic and rounding points per output
  * (fp32 accumulation, one rounding to bf16 after the residual is added); the K dimension of o_proj and
- * down_proj is summed as 8 slices, one per XCD, added in a fixed order.  Slot orders are documented at
- * the planners (fusekit_amd/csrc/dispatcher.hip).  Requires 8 KV heads (one per XCD), 1 / 2 / 4 / 8 query
- * heads per KV head, head_dim 64 or 128, hidden <= 4096; other layers use the per-dispatch families. */
+ * down_proj is summed as 8 slices, one per XCD, whose fp32 sums are added as 64-bit fixed-point integers
+ * (2^-32 units, memory-side atomic adds) into a "sum row": integer addition is associative, so the result
+ * does not depend on the order of arrival.  A sum row holds fk_xcd_sum_row_bytes(hidden) bytes; element e
+ * of the vector sits at index ((((t >> 6) * 4 + ((e & 7) >> 1)) * 64 + (t & 63)) << 1) | (e & 1), t = e >> 3.
+ * Three rows rotate through the launches of a token: a launch reads one (the previous launch's), adds into
+ * the second and clears the third (the one the launch after it adds into); the row the first launch of a
+ * token adds into must hold zeros (fusekit_xcd_reduce clears it at the end of the previous token; zero all
+ * three once after allocation, and again after a launch has reported an abort).  Non-finite projection
+ * outputs are not carried through a sum row.  Slot orders are documented at the planners
+ * (fusekit_amd/csrc/dispatcher.hip).  Requires 8 KV heads (one per XCD), 1 / 2 / 4 / 8 query heads per KV
+ * head, head_dim 64 or 128, hidden <= 4096; other layers use the per-dispatch families. */
 fk_status fk_xcd_layer_supported(uint32_t hidden, uint32_t inter, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                  uint32_t capacity, uint32_t bits, uint32_t group);
 /* Bytes of the control block (arrival words, abort word; zero it once) and of the attention partial rows. */
 fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t *control_bytes, size_t *attention_partial_bytes);
+/* Bytes of one sum row of a hidden-wide vector (0 for hidden == 0). */
+size_t fk_xcd_sum_row_bytes(uint32_t hidden);
 /* Synchronises the stream and reports whether a launch gave up on a hand-over wait (FK_ERR_HIP; the control
  * block is reset).  The dispatcher calls it after every graph execution that holds such launches. */
 fk_status fk_xcd_check(void *workspace, fk_stream s);

@@ -23,11 +23,29 @@ def _wargs(arg, W):
     return [arg(W.w)] + ([] if W.bits == 16 else [arg(W.scales), arg(W.biases)])
 
 
-def _reduce_ref(partials, residual):
-    """x = T(((p0+p1)+(p2+p3)) + ((p4+p5)+(p6+p7)) + float(res)) in fp32, the launch's fixed order."""
-    p = partials.astype(np.float32)
-    acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))
-    return oracle.f32_to_bf16((acc + oracle.bf16_to_f32(residual)).astype(np.float32))
+def _sum_row(fk, hidden, contributions=None):
+    """A sum row as the launches keep it: 64-bit fixed point (2^-32 units), elements permuted (fk.xcd_sum_index),
+    padded to whole 512-element sections; `contributions` [n][hidden] fp32 are added the way a launch adds its
+    outputs (each rounded to the nearest unit)."""
+    row = np.zeros(fk.xcd_sum_row_bytes(hidden) // 8, np.int64)
+    if contributions is not None:
+        q = np.rint(np.asarray(contributions, np.float32).astype(np.float64) * 2.0 ** 32).astype(np.int64)
+        row[fk.xcd_sum_index(hidden)] = q.sum(axis=0)
+    return row
+
+
+def _row_values(fk, row, hidden):
+    """The sums of a row as exact doubles, in vector order."""
+    return row[fk.xcd_sum_index(hidden)].astype(np.float64) / 2.0 ** 32
+
+
+def _input_ref(fk, row, hidden, residual):
+    """x = T(f32(sum) + float(res)), f32(sum) = fma(f32(low word), 2^-32, f32(high word)): the launches' input."""
+    v = row[fk.xcd_sum_index(hidden)]
+    lo = (v & 0xffffffff).astype(np.uint32).astype(np.float32).astype(np.float64)
+    hi = (v >> 32).astype(np.int32).astype(np.float32).astype(np.float64)
+    f = (lo * 2.0 ** -32 + hi).astype(np.float32)            # exact in double, one rounding: the fma
+    return oracle.f32_to_bf16((f + oracle.bf16_to_f32(residual)).astype(np.float32))
 
 
 def _close_bf16(got, ref_bits, ref_f32=None, frac=0.02, ulps=1.0):
@@ -47,44 +65,49 @@ def test_xcd_mlp_block(fk, bits, hidden, inter, variant):
     Wg, Wu, Wd = make_qweight(1, inter, hidden, bits), make_qweight(2, inter, hidden, bits), make_qweight(3, hidden, inter, bits)
     norm_w = normal_bf16(4, hidden, 0.1, 1.0)
     partials = (rng(5).standard_normal((8, hidden), dtype=np.float32) * 0.3).astype(np.float32)
-    res = np.stack([normal_bf16(6, hidden)] * 8)          # one copy per XCD, as a previous launch leaves it
+    res = normal_bf16(6, hidden)
     dWg, dWu, dWd = (to_device(fk, W) for W in (Wg, Wu, Wd))
     ctl_bytes, _ = fk.xcd_workspace_bytes(32, 128)
     ctl = fk.zeros(ctl_bytes)
-    b = dict(p=_dev(fk, partials), res=_dev(fk, res), x=fk.DeviceBuffer(8 * hidden * 2), nw=_dev(fk, norm_w),
-             mid=fk.DeviceBuffer(inter * 2), out=fk.DeviceBuffer(8 * hidden * 4))
+    row_in = _sum_row(fk, hidden, partials)
+    junk = np.full_like(row_in, 0x0123456789abcdef)
+    b = dict(p=_dev(fk, row_in), res=_dev(fk, res), x=fk.DeviceBuffer(hidden * 2), nw=_dev(fk, norm_w),
+             mid=fk.DeviceBuffer(inter * 2), out=_dev(fk, _sum_row(fk, hidden)), clr=_dev(fk, junk))
     a = [arg(b["p"]), arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dWg.w), arg(dWu.w)]
     if bits != 16:
         a += [arg(dWg.scales), arg(dWu.scales), arg(dWg.biases), arg(dWu.biases)]
-    a += _wargs(arg, dWd) + [arg(b["mid"]), arg(b["out"]), arg(ctl)]
+    a += _wargs(arg, dWd) + [arg(b["mid"]), arg(b["out"]), arg(b["clr"]), arg(ctl)]
     task = Dispatch("fusekit_xcd_mlp_block_f1", a,
                     dict(hidden=hidden, inter=inter, n_heads=32, n_kv=8, head_dim=128, capacity=256, bits=bits, group=64,
-                         eps=EPS, variant=variant, has_partials=1, residual_per_xcd=1))
+                         eps=EPS, variant=variant, has_sums=1))
     for rep in range(2):                                  # twice: the arrival words carry over between launches
         d.dispatch_kernel(task)
         fk.xcd_check(ctl)
-        x1 = _reduce_ref(partials, res[0])
-        got_x = b["x"].to_numpy(np.uint16, (8, hidden))
-        for c in range(8):
-            assert np.array_equal(got_x[c], x1), f"copy {c} of the reduced input differs"
+        x1 = _input_ref(fk, row_in, hidden, res)
+        assert np.array_equal(b["x"].to_numpy(np.uint16), x1), "the launch's input row differs"
+        assert not b["clr"].to_numpy(np.int64).any(), "the third sum row was not cleared"
         mid_ref = oracle.gateup_swiglu(x1, norm_w, EPS, Wg, Wu, variant)
         got_mid = b["mid"].to_numpy(np.uint16)
         _close_bf16(got_mid, mid_ref, frac=0.03, ulps=2.0)   # gate and up may each sit on a rounding edge
-        # the 8 partial rows are the K-slices of W_down . mid (mid as the GPU produced it)
-        out = b["out"].to_numpy(np.float32, (8, hidden))
+        # the sum row holds W_down . mid (mid as the GPU produced it): eight fp32 K-slice sums per element
+        row_out = b["out"].to_numpy(np.int64)
+        out = _row_values(fk, row_out, hidden)
         wd = oracle.dequantize(Wd).astype(np.float64) if bits != 16 else oracle.bf16_to_f32(Wd.w).astype(np.float64)
         m64 = oracle.bf16_to_f32(got_mid).astype(np.float64)
-        sl = inter // 8
-        for c in range(8):
-            ref = wd[:, c * sl:(c + 1) * sl] @ m64[c * sl:(c + 1) * sl]
-            scale = np.abs(wd[:, c * sl:(c + 1) * sl]) @ np.abs(m64[c * sl:(c + 1) * sl])
-            assert np.all(np.abs(out[c] - ref) <= 2e-6 * scale + 1e-30), f"K-slice {c}"
-        # and the next launch's reduction of them is the down projection + residual
-        y = _reduce_ref(out, x1)
+        ref, scale = wd @ m64, np.abs(wd) @ np.abs(m64)
+        assert np.all(np.abs(out - ref) <= 2e-6 * scale + 8 * 2.0 ** -33)
+        pad = np.ones(row_out.size, bool)
+        pad[fk.xcd_sum_index(hidden)] = False
+        assert not row_out[pad].any()
+        # and the next launch's input from it is the down projection + residual
+        y = _input_ref(fk, row_out, hidden, x1)
         y_ref = oracle.linear_residual(Wd, got_mid, x1)
         _close_bf16(y, y_ref, oracle.linear_acc(Wd, got_mid) + oracle.bf16_to_f32(x1))
         partials = (partials * 0.5).astype(np.float32)   # second round on other inputs
-        b["p"].upload(partials)
+        row_in = _sum_row(fk, hidden, partials)
+        b["p"].upload(row_in)
+        b["out"].upload(_sum_row(fk, hidden))
+        b["clr"].upload(junk)
 
 
 @pytest.mark.parametrize("bits", [4, 16])
@@ -107,10 +130,11 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
     ctl_bytes, ap_bytes = fk.xcd_workspace_bytes(n_heads, head_dim)
     ctl = fk.zeros(ctl_bytes)
     cache_bytes = n_kv * capacity * head_dim * 2
-    b = dict(res=fk.DeviceBuffer(hidden * 2), x=fk.DeviceBuffer(8 * hidden * 2), nw=_dev(fk, norm_w),
+    zero_row = _sum_row(fk, hidden)
+    b = dict(res=fk.DeviceBuffer(hidden * 2), x=fk.DeviceBuffer(hidden * 2), nw=_dev(fk, norm_w),
              q=fk.DeviceBuffer(n_q * 2), k=fk.DeviceBuffer(n_kvd * 2), v=fk.DeviceBuffer(n_kvd * 2),
              ck=fk.zeros(cache_bytes), cv=fk.zeros(cache_bytes), kv_len=fk.zeros(4), off=fk.zeros(4), step=fk.zeros(4),
-             tab=fk.DeviceBuffer(head_dim * 4), ap=fk.DeviceBuffer(ap_bytes), out=fk.DeviceBuffer(8 * hidden * 4))
+             tab=fk.DeviceBuffer(head_dim * 4), ap=fk.DeviceBuffer(ap_bytes), out=_dev(fk, zero_row), clr=_dev(fk, zero_row))
     a = [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dW[0].w), arg(dW[1].w), arg(dW[2].w)]
     if bits != 16:
         a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]]
@@ -119,10 +143,10 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
         b["qn"], b["kn"] = _dev(fk, qn), _dev(fk, kn)
         a += [arg(b["qn"]), arg(b["kn"])]
     a += [arg(b["q"]), arg(b["k"]), arg(b["v"]), arg(b["ck"]), arg(b["cv"]), arg(b["kv_len"]), arg(b["tab"]), arg(b["ap"]),
-          arg(b["out"]), arg(ctl)]
+          arg(b["out"]), arg(b["clr"]), arg(ctl)]
     task = Dispatch("fusekit_xcd_attn_block_f1", a,
                     dict(hidden=hidden, inter=inter, n_heads=n_heads, n_kv=n_kv, head_dim=head_dim, capacity=capacity,
-                         bits=bits, group=64, eps=EPS, theta=theta, has_partials=0, residual_per_xcd=0, has_norm=int(qk_norm)))
+                         bits=bits, group=64, eps=EPS, theta=theta, has_sums=0, has_norm=int(qk_norm)))
     step = Dispatch("fusekit_step_init", [arg(b["step"]), arg(b["off"]), arg(b["kv_len"]), arg(b["tab"])],
                     dict(rope_dims=head_dim, theta=theta))
     ck = np.zeros(n_kv * capacity * head_dim, np.uint16)
@@ -132,6 +156,7 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
     for pos in range(200):
         x = normal_bf16(100 + pos, hidden)
         b["res"].upload(x)
+        b["out"].upload(zero_row)
         d.dispatch_batch([step, task])
         if pos % 16 and pos < 190:
             # the oracle still has to append this position's rows: it follows the GPU's own q/k/v rows, checked
@@ -142,8 +167,7 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
             oracle.kv_store(kr, vg, n_kv, head_dim, head_dim, pos, capacity, ck, cv)
             continue
         fk.xcd_check(ctl)
-        got_x = b["x"].to_numpy(np.uint16, (8, hidden))
-        assert all(np.array_equal(got_x[c], x) for c in range(8))
+        assert np.array_equal(b["x"].to_numpy(np.uint16), x)
         q_ref, k_ref, v_ref = oracle.rmsnorm_qkv(x, norm_w, EPS, Wq, Wk, Wv)
         qg, kg, vg = b["q"].to_numpy(np.uint16), b["k"].to_numpy(np.uint16), b["v"].to_numpy(np.uint16)
         for g, r in ((qg, q_ref), (kg, k_ref), (vg, v_ref)):
@@ -168,9 +192,8 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
         ck = gck.copy()                                  # keep both sides on the same cache bits
         att = oracle.sdpa_decode(qr, ck, cv, n_heads, n_kv, head_dim, head_dim, pos + 1, capacity, scale)
         y_ref_acc = oracle.linear_acc(Wo, att)
-        out = b["out"].to_numpy(np.float32, (8, hidden))
-        acc = ((out[0] + out[1]) + (out[2] + out[3])) + ((out[4] + out[5]) + (out[6] + out[7]))
-        rel = float(np.linalg.norm(acc.astype(np.float64) - y_ref_acc) / np.linalg.norm(y_ref_acc))
+        acc = _row_values(fk, b["out"].to_numpy(np.int64), hidden)
+        rel = float(np.linalg.norm(acc - y_ref_acc) / np.linalg.norm(y_ref_acc))
         worst = max(worst, rel)
         assert rel <= 1e-2, (pos, rel)
     print("worst rel-L2 of the o_proj sums over the sampled positions: %.3e" % worst)
@@ -193,17 +216,17 @@ def test_xcd_attn_block_at_the_config3_contexts(fk, kv_len):
     dW = [to_device(fk, W) for W in (Wq, Wk, Wv, Wo)]
     ctl_bytes, ap_bytes = fk.xcd_workspace_bytes(n_heads, head_dim)
     ctl = fk.zeros(ctl_bytes)
-    b = dict(res=_dev(fk, x), x=fk.DeviceBuffer(8 * hidden * 2), nw=_dev(fk, norm_w), q=fk.DeviceBuffer(n_q * 2),
+    b = dict(res=_dev(fk, x), x=fk.DeviceBuffer(hidden * 2), nw=_dev(fk, norm_w), q=fk.DeviceBuffer(n_q * 2),
              k=fk.DeviceBuffer(n_kvd * 2), v=fk.DeviceBuffer(n_kvd * 2), ck=_dev(fk, ck), cv=_dev(fk, cv),
              kv_len=fk.zeros(4), off=fk.zeros(4), step=_dev(fk, np.array([pos], np.uint32)), tab=fk.DeviceBuffer(head_dim * 4),
-             ap=fk.DeviceBuffer(ap_bytes), out=fk.DeviceBuffer(8 * hidden * 4))
+             ap=fk.DeviceBuffer(ap_bytes), out=_dev(fk, _sum_row(fk, hidden)), clr=_dev(fk, _sum_row(fk, hidden)))
     a = [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dW[0].w), arg(dW[1].w), arg(dW[2].w)]
     a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]] + _wargs(arg, dW[3])
     a += [arg(b["q"]), arg(b["k"]), arg(b["v"]), arg(b["ck"]), arg(b["cv"]), arg(b["kv_len"]), arg(b["tab"]), arg(b["ap"]),
-          arg(b["out"]), arg(ctl)]
+          arg(b["out"]), arg(b["clr"]), arg(ctl)]
     task = Dispatch("fusekit_xcd_attn_block_f1", a,
                     dict(hidden=hidden, inter=inter, n_heads=n_heads, n_kv=n_kv, head_dim=head_dim, capacity=capacity,
-                         bits=bits, group=64, eps=EPS, theta=theta, has_partials=0, residual_per_xcd=0, has_norm=0))
+                         bits=bits, group=64, eps=EPS, theta=theta, has_sums=0, has_norm=0))
     step = Dispatch("fusekit_step_init", [arg(b["step"]), arg(b["off"]), arg(b["kv_len"]), arg(b["tab"])],
                     dict(rope_dims=head_dim, theta=theta))
     d.dispatch_batch([step, task])
@@ -226,9 +249,8 @@ def test_xcd_attn_block_at_the_config3_contexts(fk, kv_len):
     assert np.all(np.abs(fg - fo) <= row_ulp)
     att = oracle.sdpa_decode(qr, gck, gcv, n_heads, n_kv, head_dim, head_dim, kv_len, capacity, 1.0 / np.sqrt(head_dim))
     y_ref = oracle.linear_acc(Wo, att)
-    out = b["out"].to_numpy(np.float32, (8, hidden))
-    acc = ((out[0] + out[1]) + (out[2] + out[3])) + ((out[4] + out[5]) + (out[6] + out[7]))
-    rel = float(np.linalg.norm(acc.astype(np.float64) - y_ref) / np.linalg.norm(y_ref))
+    acc = _row_values(fk, b["out"].to_numpy(np.int64), hidden)
+    rel = float(np.linalg.norm(acc - y_ref) / np.linalg.norm(y_ref))
     print(f"kv_len {kv_len}: o_proj sums rel-L2 {rel:.3e}")
     assert rel <= 1e-2
 
@@ -236,12 +258,21 @@ def test_xcd_attn_block_at_the_config3_contexts(fk, kv_len):
 def test_xcd_reduce(fk):
     from fusekit_amd.runtime import Dispatch, Dispatcher, arg
     d = Dispatcher()
-    hidden = 2560
-    partials = (rng(1).standard_normal((8, hidden), dtype=np.float32)).astype(np.float32)
-    res = normal_bf16(2, hidden)
-    bp, br, bx = _dev(fk, partials), _dev(fk, res), fk.DeviceBuffer(hidden * 2)
-    d.dispatch_kernel(Dispatch("fusekit_xcd_reduce_f1", [arg(bp), arg(br), arg(bx)], dict(hidden=hidden)))
-    assert np.array_equal(bx.to_numpy(np.uint16), _reduce_ref(partials, res))
+    for hidden in (2560, 1088):                          # 1088: a row with a partly filled last section
+        partials = (rng(1).standard_normal((8, hidden), dtype=np.float32) * 40).astype(np.float32)
+        partials[:, :7] = [-3e5, 1e-9, -1e-9, 0.5, 2.0 ** -33, -2.0 ** -33, 70000.25]
+        res = normal_bf16(2, hidden)
+        row = _sum_row(fk, hidden, partials)
+        bp, br, bx = _dev(fk, row), _dev(fk, res), fk.DeviceBuffer(hidden * 2)
+        other = _dev(fk, np.full_like(row, -1))
+        d.dispatch_kernel(Dispatch("fusekit_xcd_reduce_f1", [arg(bp), arg(br), arg(bx), arg(other)], dict(hidden=hidden)))
+        assert np.array_equal(bx.to_numpy(np.uint16), _input_ref(fk, row, hidden, res))
+        assert not other.to_numpy(np.int64)[fk.xcd_sum_index(hidden)].any()
+        assert np.array_equal(bp.to_numpy(np.int64), row)
+        # clearing the row that is read: read first, then cleared
+        d.dispatch_kernel(Dispatch("fusekit_xcd_reduce_f1", [arg(bp), arg(br), arg(bx), arg(bp)], dict(hidden=hidden)))
+        assert np.array_equal(bx.to_numpy(np.uint16), _input_ref(fk, row, hidden, res))
+        assert not bp.to_numpy(np.int64)[fk.xcd_sum_index(hidden)].any()
 
 
 def test_xcd_wait_gives_up_and_reports(fk):
