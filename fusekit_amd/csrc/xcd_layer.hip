@@ -239,40 +239,45 @@ struct Tile {
     float inv_cs;
 };
 
-// SN threads stream a tile; `ti` is the calling thread's index among them.  A thread's position in pass p is
-// (p * NL + j) * SN + ti; its (row, column) is worked out once per tile and advanced from pass to pass.
+// SN threads stream a tile; `ti` is the calling thread's index among them.  A thread's j-th position in pass p is
+// pos = (p * NL + j) * SN + ti = row * cs + col.  The thread keeps, per j, the column (it addresses the staged
+// activations) and the chunk's index in the matrix (the request); both are worked out once per tile and advanced
+// from pass to pass without a multiplication.  The flat position itself indexes the partials, and pos >> gshift
+// the tile's quantisation groups (cs is a whole number of groups).
 template <int NL>
 struct TilePos {
-    uint32_t row[NL], col[NL];
+    uint32_t p0;            // position of j = 0
+    uint32_t col[NL], gidx[NL];
 };
 template <int NL, int SN>
-__device__ __forceinline__ void tile_pos_init(const Tile& t, uint32_t ti, TilePos<NL>& p) {
+__device__ __forceinline__ void tile_pos_init(const XcdMat& m, const Tile& t, uint32_t ti, TilePos<NL>& p) {
+    p.p0 = ti;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
         const uint32_t pos = j * SN + ti;
-        p.row[j] = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
-        p.col[j] = pos - p.row[j] * t.cs;
+        const uint32_t row = (uint32_t)(((float)pos + 0.5f) * t.inv_cs);
+        p.col[j] = pos - row * t.cs;
+        p.gidx[j] = (t.row0 + row) * m.cpr + t.col0 + p.col[j];
     }
 }
 template <int NL, int SN>
-__device__ __forceinline__ void tile_pos_next(const Tile& t, uint32_t step_r, uint32_t step_c, TilePos<NL>& p) {
+__device__ __forceinline__ void tile_pos_next(const XcdMat& m, const Tile& t, uint32_t step_c, uint32_t step_g, TilePos<NL>& p) {
+    p.p0 += NL * SN;
+    const uint32_t skip = m.cpr - t.cs;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
         const uint32_t c = p.col[j] + step_c;
         const bool wrap = c >= t.cs;
         p.col[j] = wrap ? c - t.cs : c;
-        p.row[j] += step_r + (wrap ? 1u : 0u);
+        p.gidx[j] += step_g + (wrap ? skip : 0u);
     }
 }
 
-template <WKind KIND, int NL>
+template <WKind KIND, int NL, int SN>
 __device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, const TilePos<NL>& p, TileRegs<NL>& r) {
+    const uint32_t total = t.rows * t.cs, first = t.row0 * m.cpr + t.col0;
 #pragma unroll
-    for (int j = 0; j < NL; ++j) {
-        const bool in = p.row[j] < t.rows;
-        const size_t idx = (size_t)(t.row0 + (in ? p.row[j] : 0u)) * m.cpr + t.col0 + (in ? p.col[j] : 0u);
-        r.w[j] = m.w[idx];
-    }
+    for (int j = 0; j < NL; ++j) r.w[j] = m.w[p.p0 + j * SN < total ? p.gidx[j] : first];
 }
 
 // Group gi of the tile = (row gi / gpr, group gi % gpr of the row's slice), gpr groups per row slice.
@@ -322,23 +327,22 @@ __device__ __forceinline__ void meta_store(const MetaRegs& r, uint32_t ti, uint3
     }
 }
 
-// One fp32 partial per chunk into part[row * cs + col]; positions past the tile are dropped.
-template <WKind KIND, int NL>
+// One fp32 partial per chunk into part[pos]; positions past the tile land in the padding of `part` (it holds whole
+// passes) and read group 0's scale and bias.
+template <WKind KIND, int NL, int SN>
 __device__ __forceinline__ void tile_partials(const XcdMat& m, const Tile& t, const TilePos<NL>& p, const TileRegs<NL>& r,
                                               const uint4* xs, const float* sx, const uint32_t* meta, float* part) {
-    const uint32_t gpr = t.cs >> m.gshift;
+    const uint32_t total = t.rows * t.cs;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-        const bool in = p.row[j] < t.rows;
-        const uint32_t row = in ? p.row[j] : 0u, col = in ? p.col[j] : 0u;
+        const uint32_t pos = p.p0 + j * SN;
         uint32_t sb = 0, bb = 0;
         if constexpr (KIND != W_BF16) {
-            const uint32_t mw = meta[row * gpr + (col >> m.gshift)];
+            const uint32_t mw = meta[(pos < total ? pos : 0u) >> m.gshift];
             sb = mw & 0xffffu;
             bb = mw >> 16;
         }
-        const float v = chunk_partial<KIND>(r.w[j], sb, bb, xs, sx, col, t.cs);
-        if (in) part[row * t.cs + col] = v;
+        part[pos] = chunk_partial<KIND>(r.w[j], sb, bb, xs, sx, p.col[j], t.cs);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
@@ -350,60 +354,61 @@ template <WKind KIND, int NL, int SN, typename F>
 __device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
                                          const float* sx, const uint32_t* meta, float* part, F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
-    const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs;
+    const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * m.cpr + step_c;
     TileRegs<NL> r1;
     TilePos<NL> q = p;
     if (n_pass <= 1) after_last_request();
     for (uint32_t k = 0; k < n_pass; k += 2) {
         if (k + 1 < n_pass) {
-            tile_pos_next<NL, SN>(t, step_r, step_c, q);
-            tile_load<KIND, NL>(m, t, q, r1);
+            tile_pos_next<NL, SN>(m, t, step_c, step_g, q);
+            tile_load<KIND, NL, SN>(m, t, q, r1);
             if (k + 2 >= n_pass) after_last_request();
         }
-        tile_partials<KIND, NL>(m, t, p, r0, xs, sx, meta, part);
+        tile_partials<KIND, NL, SN>(m, t, p, r0, xs, sx, meta, part);
         if (k + 1 < n_pass) {
             p = q;
             if (k + 2 < n_pass) {
-                tile_pos_next<NL, SN>(t, step_r, step_c, q);
-                tile_load<KIND, NL>(m, t, q, r0);
+                tile_pos_next<NL, SN>(m, t, step_c, step_g, q);
+                tile_load<KIND, NL, SN>(m, t, q, r0);
                 if (k + 3 >= n_pass) after_last_request();
             }
-            tile_partials<KIND, NL>(m, t, p, r1, xs, sx, meta, part);
+            tile_partials<KIND, NL, SN>(m, t, p, r1, xs, sx, meta, part);
             p = q;
         }
     }
 }
 
 // The gate / up pair: both matrices' passes interleaved, so that one pass of each is in flight while one is consumed.
+// (Same shape and tile: one set of positions serves both.)
 template <WKind KIND, int NL, int SN, typename F>
 __device__ __forceinline__ void tile_run_pair(const XcdMat& ma, const XcdMat& mb, const Tile& t, TilePos<NL>& p,
                                               TileRegs<NL>& a0, TileRegs<NL>& b0, const uint4* xs, const float* sx,
                                               const uint32_t* meta_a, const uint32_t* meta_b, float* part_a, float* part_b,
                                               F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
-    const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs;
+    const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * ma.cpr + step_c;
     TileRegs<NL> a1, b1;
     TilePos<NL> q = p;
     if (n_pass <= 1) after_last_request();
     for (uint32_t k = 0; k < n_pass; k += 2) {
         if (k + 1 < n_pass) {
-            tile_pos_next<NL, SN>(t, step_r, step_c, q);
-            tile_load<KIND, NL>(ma, t, q, a1);
-            tile_load<KIND, NL>(mb, t, q, b1);
+            tile_pos_next<NL, SN>(ma, t, step_c, step_g, q);
+            tile_load<KIND, NL, SN>(ma, t, q, a1);
+            tile_load<KIND, NL, SN>(mb, t, q, b1);
             if (k + 2 >= n_pass) after_last_request();
         }
-        tile_partials<KIND, NL>(ma, t, p, a0, xs, sx, meta_a, part_a);
-        tile_partials<KIND, NL>(mb, t, p, b0, xs, sx, meta_b, part_b);
+        tile_partials<KIND, NL, SN>(ma, t, p, a0, xs, sx, meta_a, part_a);
+        tile_partials<KIND, NL, SN>(mb, t, p, b0, xs, sx, meta_b, part_b);
         if (k + 1 < n_pass) {
             p = q;
             if (k + 2 < n_pass) {
-                tile_pos_next<NL, SN>(t, step_r, step_c, q);
-                tile_load<KIND, NL>(ma, t, q, a0);
-                tile_load<KIND, NL>(mb, t, q, b0);
+                tile_pos_next<NL, SN>(ma, t, step_c, step_g, q);
+                tile_load<KIND, NL, SN>(ma, t, q, a0);
+                tile_load<KIND, NL, SN>(mb, t, q, b0);
                 if (k + 3 >= n_pass) after_last_request();
             }
-            tile_partials<KIND, NL>(ma, t, p, a1, xs, sx, meta_a, part_a);
-            tile_partials<KIND, NL>(mb, t, p, b1, xs, sx, meta_b, part_b);
+            tile_partials<KIND, NL, SN>(ma, t, p, a1, xs, sx, meta_a, part_a);
+            tile_partials<KIND, NL, SN>(mb, t, p, b1, xs, sx, meta_b, part_b);
             p = q;
         }
     }
@@ -514,12 +519,12 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     // KiB per CU.  The later passes stream while the earlier ones are consumed; the down_proj slice is queued
     // behind the last of them.
     input_request(a.in, inr);
-    tile_pos_init<NLA, kBlock>(tg, tid, pg);
-    tile_pos_init<NLB, kBlock>(td, tid, pd);
+    tile_pos_init<NLA, kBlock>(a.gate, tg, tid, pg);
+    tile_pos_init<NLB, kBlock>(a.down, td, tid, pd);
     meta_fetch<KIND, kBlock, true>(a.gate, tg, tid, mg);
     meta_fetch<KIND, kBlock, true>(a.up, tg, tid, mu);
-    tile_load<KIND, NLA>(a.gate, tg, pg, rg);
-    tile_load<KIND, NLA>(a.up, tg, pg, ru);
+    tile_load<KIND, NLA, kBlock>(a.gate, tg, pg, rg);
+    tile_load<KIND, NLA, kBlock>(a.up, tg, pg, ru);
     FK_XCD_STAMP(1, 1);
     input_stage<KIND, 1>(a.in, inr, xs, sx, a.gate.cpr, red);
     FK_XCD_STAMP(1, 5);
@@ -531,7 +536,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     // ---- gate / up rows of this XCD's slice, SwiGLU ----
     const uint32_t seg = (gu_n * a.gate.cpr + NLA * kBlock - 1) / (NLA * kBlock) * (NLA * kBlock);
     if (streams) {
-        auto request_down = [&]() { tile_load<KIND, NLB>(a.down, td, pd, rd); };
+        auto request_down = [&]() { tile_load<KIND, NLB, kBlock>(a.down, td, pd, rd); };
         if (gu_n)
             tile_run_pair<KIND, NLA, kBlock>(a.gate, a.up, tg, pg, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg,
                                              request_down);
@@ -614,10 +619,10 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     TilePos<NLB> po;
     InputRegs inr;
     input_request(a.in, inr);
-    tile_pos_init<NLA, kAttnStream>(tq, ti, pq);
-    tile_pos_init<NLB, kAttnStream>(to, ti, po);
+    tile_pos_init<NLA, kAttnStream>(mq, tq, ti, pq);
+    tile_pos_init<NLB, kAttnStream>(a.wo, to, ti, po);
     meta_fetch<KIND, kAttnStream, true>(mq, tq, ti, mmq);
-    tile_load<KIND, NLA>(mq, tq, pq, rq);
+    tile_load<KIND, NLA, kAttnStream>(mq, tq, pq, rq);
     FK_XCD_STAMP(0, 1);
     input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red);
     FK_XCD_STAMP(0, 5);
@@ -627,7 +632,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
 
     // ---- q / k / v rows of this XCD's KV head; the o_proj slice is requested behind their last pass ----
     if (streams) {
-        auto request_o = [&]() { tile_load<KIND, NLB>(a.wo, to, po, ro); };
+        auto request_o = [&]() { tile_load<KIND, NLB, kAttnStream>(a.wo, to, po, ro); };
         if (pr_n)
             tile_run<KIND, NLA, kAttnStream>(mq, tq, pq, rq, xs, sx, meta, work, request_o);
         else
@@ -737,7 +742,7 @@ __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs 
 // =============================================================================================== host side
 namespace {
 
-constexpr int kNlQkv = 6, kNlO = 4, kNlGu = 2, kNlDown = 6;  // 16-byte requests per streaming thread and pass
+constexpr int kNlQkv = 6, kNlO = 4, kNlGu = 6, kNlDown = 6;  // 16-byte requests per streaming thread and pass
 
 uint32_t ilog2u(uint32_t v) {
     uint32_t r = 0;
