@@ -12,6 +12,10 @@
                                          the reference's `fusekit patch`: write task_graph.json, manifest.json and
                                          variants/prefill_mN/task_graph.json for a checkpoint
   generate --model DIR --artifact DIR ... decode from the artifact's task graphs instead of a fresh runtime
+  bench DIR [--tokens 64] [--prompt TEXT | --ids 1,2,3] [--repeat 1] [--max-kv-size N] [--kv-bits 4|8]
+        [--kv-group-size 64] [--per-kernel] [--dump-tokens]
+                                         the reference's `fusekit bench`: fixed-length generation, `[bench:N] key=value`
+                                         lines (prompt_tokens, generated_tokens, stream_tps, wall_s, wall_tps, peak_gb)
 """
 import argparse
 import json
@@ -45,8 +49,12 @@ def main() -> int:
     e.add_argument("--vocab", type=int, default=2000)
     e.add_argument("--seed", type=int, default=0)
     e.add_argument("--moe", action="store_true", help="a small mixture-of-experts model with low-rank keys (deepseek_v2 layout)")
+    from . import bench_cli
+    bench_cli.add_arguments(sub)
     args = ap.parse_args()
 
+    if args.cmd == "bench":
+        return bench_cli.run(args)
     from . import native as fk
     if args.cmd == "info":
         t = fk.target_describe()

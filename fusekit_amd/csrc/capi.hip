@@ -123,6 +123,14 @@ fk_status fk_alloc(size_t nbytes, void** dptr) {
     return FK_OK;
 }
 
+fk_status fk_mem_info(size_t* free_bytes, size_t* total_bytes) {
+    if (!free_bytes || !total_bytes) return set_error(FK_ERR_INVALID, "fk_mem_info: null out pointer");
+    const DeviceFacts* d;
+    FK_TRY(device_facts(&d));
+    FK_HIP(hipMemGetInfo(free_bytes, total_bytes));
+    return FK_OK;
+}
+
 fk_status fk_free(void* dptr) {
     if (!dptr) return FK_OK;
     FK_HIP(hipFree(dptr));

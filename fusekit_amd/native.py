@@ -83,6 +83,13 @@ def device_props() -> DeviceProps:
     return p
 
 
+def mem_info():
+    """(free, total) device memory in bytes."""
+    a, b = C.c_size_t(), C.c_size_t()
+    check(lib.fk_mem_info(C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
 def has_device() -> bool:
     p = DeviceProps()
     return lib.fk_device_props_get(C.byref(p)) == FK_OK

@@ -72,8 +72,13 @@ typedef struct fk_device_props {
 } fk_device_props;
 
 fk_status fk_device_props_get(fk_device_props *out);
+/* Device memory (hipMalloc).  The reference's buffers carry a storage mode (shared / private); here every
+ * buffer is device-private HBM and the host reaches it through fk_upload / fk_download only, so there is no
+ * memory-kind argument. */
 fk_status fk_alloc(size_t nbytes, void **dptr);
 fk_status fk_free(void *dptr);
+/* Free and total device memory in bytes (what `peak_gb` of the bench driver is taken from; scripts/bench.py:148). */
+fk_status fk_mem_info(size_t *free_bytes, size_t *total_bytes);
 fk_status fk_upload(void *dptr, const void *host, size_t nbytes);
 fk_status fk_download(void *host, const void *dptr, size_t nbytes);
 fk_status fk_fill_u32(void *dptr, uint32_t value, size_t count, fk_stream s);
