@@ -193,6 +193,9 @@ def main() -> int:
             elif fam == "xcd_mlp_block":
                 nbytes = sum(n for _, n in tasks[0].args)
                 label = "MLP launch (norm, gate/up, SwiGLU, down_proj)"
+            elif fam == "embed_lookup_decode":
+                nbytes = 4 + 2 * cfg.hidden * 2                               # the token, one table row in, one row out
+                label = fam
             else:
                 nbytes = sum(n for _, n in tasks[0].args)                    # weights + scales + biases + vectors in/out
                 label = {("linear_residual", 0): "o_proj + residual", ("linear_residual", 1): "down_proj + residual"}.get(

@@ -638,7 +638,6 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
         else
             request_o();
     }
-    meta_store<KIND, kAttnStream, false>(mmo, ti, meta + kMetaWords);
     __syncthreads();
     if (pr_n) {
         uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
@@ -674,15 +673,19 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
                 const float* pd = ph + 2 + 2 * (live ? d2 : 0u);
                 float M = -INFINITY, L = 0.f, o0_ = 0.f, o1_ = 0.f;
                 // all requests first (clamped indices: straight-line), then the fold in range order; up to 8 ranges
-                // (a context of 8 x the range length) take half the requests
+                // (a context of 8 x the range length) take half the requests.  The (maximum, sum) pair of range i is
+                // fetched by lane i alone and handed to the wave through scalar registers: one request, not N.
                 auto merge = [&](auto n_const) {
                     constexpr uint32_t N = decltype(n_const)::value;
-                    float2 ml[N], po[N];
+                    float2 po[N];
+                    const float2 mine = ld_f32x2<true>(ph + (size_t)(lane < n_active ? lane : 0u) * row);
+#pragma unroll
+                    for (uint32_t i = 0; i < N; ++i) po[i] = ld_f32x2<true>(pd + (size_t)(i < n_active ? i : 0u) * row);
+                    float2 ml[N];
 #pragma unroll
                     for (uint32_t i = 0; i < N; ++i) {
-                        const uint32_t idx = i < n_active ? i : 0u;
-                        ml[i] = ld_f32x2<true>(ph + (size_t)idx * row);
-                        po[i] = ld_f32x2<true>(pd + (size_t)idx * row);
+                        ml[i].x = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mine.x), i));
+                        ml[i].y = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mine.y), i));
                     }
                     M = ml[0].x;
 #pragma unroll
@@ -719,6 +722,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
             stage_emit<KIND>(xs, sx, a.o_cs, t, live, v, v, 1.0f, false);
         }
     }
+    meta_store<KIND, kAttnStream, false>(mmo, ti, meta + kMetaWords);
     __syncthreads();
     if (streams && o_n) tile_run<KIND, NLB, kAttnStream>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
     __syncthreads();
