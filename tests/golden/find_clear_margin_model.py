@@ -5,10 +5,10 @@ Random-init weights give near-uniform logits: among 151936 candidates the two la
 bf16 ulps at roughly one step in ten, and no arithmetic (fp32 in any order, double) agrees with another
 across such a step.  A trained model has peaked logits.  This script instantiates configs[3] (36 layers,
 hidden 2560, 32 q / 8 kv heads x 128, intermediate 9728, vocab 151936, int4 g64) ON THE HOST with the
-oracle's copy of the library's host-reproducible generator, gives the tied embedding a log-normal-like
-spread of row norms (rowscale = 2^(tau z), see fko_synth_fill) and an embedding output scale, and keeps a
-candidate (embedding seed, tau, embed_scale) when, over the 32-token prompt + 32 greedy steps of the
-double-accumulating oracle,
+oracle's copy of the library's host-reproducible generator, gives the tied embedding either a
+log-normal-like spread of row norms (rowscale = 2^(tau z)) or a few dominant rows (row j < loud_rows scaled by
+loud_gain * 2^-j; see fko_synth_fill) and an embedding output scale, and keeps a candidate (embedding seed,
+tau, embed_scale) when, over the 32-token prompt + 32 greedy steps of the double-accumulating oracle,
 
   * at every step, for each of the 16 leading competitors j of the chosen token t, the gap
     logit[t] - logit[j] is at least `--safety` times the largest change of that gap that the two fp32
@@ -20,7 +20,13 @@ The winner is written to clear_margin_4b.json (parameters, prompt, the 32 expect
 fp32 envelope per step); tests/test_decoder_gpu.py builds the same model in HBM from the same seeds and
 asserts plain free-running equality.  Runs only the oracle: no GPU, no reference code.
 
-    python tests/golden/find_clear_margin_model.py --taus 2.0 2.5 --scales 0.05 0.1 --seeds 20
+The committed fixture came from
+
+    python tests/golden/find_clear_margin_model.py --grid 0:0.004 --loud-rows 12 --loud-gain 256 \
+        --first-seed 3007 --seeds 1 --safety 2 --min-distinct 3
+
+after a sweep over --grid 0:0.002 0:0.004 0:0.006 0:0.02 and seeds 3000..3007 (about a minute per candidate on
+8 cores; most candidates hold at least one near-tie among their 32 steps and are skipped).
 """
 import argparse
 import json
