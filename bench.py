@@ -69,6 +69,10 @@ def main() -> int:
                     help="decode steps the CPU oracle runs for cpu_baseline (10-30 s on the box's cores)")
     ap.add_argument("--per-kernel", action="store_true", help="print per-family GPU time of one token to stderr")
     ap.add_argument("--layers", type=int, default=0, help="experiment only: override the layer count (not the headline config)")
+    ap.add_argument("--sync-steps", action="store_true",
+                    help="counter runs: one synchronised graph launch per token instead of chunks of queued launches "
+                         "(a profiler that rewrites every dispatch packet needs the queue kept short); the rate "
+                         "printed is then not the headline figure")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain 256 MiB device copies (outside the timed region): the known-traffic "
                          "kernel that rocprofv3 byte counters of the same run are scaled by")
@@ -113,9 +117,20 @@ def main() -> int:
     offset = len(prompt)
     tok = first
     # untimed: decode until the cache holds `start` positions (>= W steps; this is the warm-up)
+    def chunk(offset, tok, n):
+        if not args.sync_steps:
+            return rt.d.decode_chunk(rt.graph, rt.uniforms, offset, tok, n)
+        out, sec = [], 0.0
+        for i in range(n):
+            nxt, s1 = rt.d.decode_host_loop(rt.graph, rt.uniforms, offset + i, [tok])
+            tok = nxt[0]
+            out.append(tok)
+            sec += s1
+        return out, sec
+
     while offset < start:
         n = min(64, start - offset)
-        toks, _ = rt.d.decode_chunk(rt.graph, rt.uniforms, offset, tok, n)
+        toks, _ = chunk(offset, tok, n)
         tok, offset = toks[-1], offset + n
     fk.sync()
     # timed: exactly K steps, all chunks enqueued by the native loop, sync on both sides
@@ -124,7 +139,7 @@ def main() -> int:
     done = 0
     while done < args.steps:
         n = min(rt.uniforms.hist_capacity, args.steps - done)
-        toks, sec = rt.d.decode_chunk(rt.graph, rt.uniforms, offset, tok, n)
+        toks, sec = chunk(offset, tok, n)
         tok, offset, done, gpu_s = toks[-1], offset + n, done + n, gpu_s + sec
     fk.sync()
     wall_s = time.perf_counter() - t0
