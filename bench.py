@@ -56,6 +56,12 @@ def family(kernel: str) -> str:
     return name.rsplit("_f", 1)[0] if "_f" in name else name
 
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the counter reads for a plain
+# 256 MiB copy); the runs and their commands are kept in profiles/xcd_layer_q4_4b.pmc_traffic.md.  Counters cannot be
+# read inside this process, so the figure is the recorded one for the kernel as built there.
+TRAFFIC_BYTES = {"xcd_mlp_kernel<Q4>": 44981900}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -241,7 +247,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": TRAFFIC_BYTES.get(dom),
             "bytes_per_launch": int(s["bytes"] / s["launches"]),
             "avg_launch_us": round(s["us"] / s["launches"], 3),
             "launches_per_token": s["launches"],

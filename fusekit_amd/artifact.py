@@ -52,6 +52,13 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
     scratch("sdpa_partials", rt.sdpa_partials, "float32")
     if rt.rope_tab is not None:
         scratch("rope_tab", rt.rope_tab, "float32")
+    if getattr(rt, "xcd", False):   # a layer as two launches: control words, sum rows, the rows between the launches
+        scratch("xcd.control", rt.xcd_ctl, "uint32", zero=True)
+        scratch("xcd.attention_partials", rt.xcd_att_partials, "float32")
+        scratch("xcd.x.0", rt.xcd_xa, "bfloat16")
+        scratch("xcd.x.1", rt.xcd_xb, "bfloat16")
+        for i, b in enumerate(rt.xcd_sums):
+            scratch(f"xcd.sums.{i}", b, "uint32", zero=True)
     for l in range(rt.cfg.n_layers):
         if rt.cfg.kv_bits:
             for nm, c in (("cache_k", rt.cache_k[l]), ("cache_v", rt.cache_v[l])):
@@ -62,6 +69,13 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
             scratch(f"cache_k.{l}", rt.cache_k[l], "bfloat16", zero=True)
             scratch(f"cache_v.{l}", rt.cache_v[l], "bfloat16", zero=True)
     _parameter_symbols(rt, sym)
+    # scales / biases of o_proj and down_proj as the two-launch layer binds them: a parameter behind a load-time
+    # re-layout, named by the parameter and the transform
+    for path, (sc, bi) in getattr(rt, "xcd_kmeta", {}).items():
+        W = rt.w.mats[path]
+        for buf, leaf in ((sc, ".scales"), (bi, ".biases")):
+            sym[buf.ptr] = dict(role="external", source_path=path + leaf, dtype="bfloat16", transform="xcd_kslice",
+                                shape=[W.n, W.k // W.group], size_bytes=buf.nbytes)
     return sym
 
 
@@ -111,6 +125,8 @@ def _graph_dict(rt: DecoderRuntime, task_list: List[Dispatch], graph_id: int, sy
                 b["offset_bytes"] = off
             if s["role"] == "external":
                 b.update(source_path=s["source_path"], shape=s["shape"], role_name=s["source_path"].rsplit(".", 1)[-1])
+                if s.get("transform"):
+                    b["transform"] = s["transform"]
             else:
                 name = s["role_name"]
                 if name not in scratch_ids:
@@ -142,7 +158,8 @@ def _graph_dict(rt: DecoderRuntime, task_list: List[Dispatch], graph_id: int, sy
         version=SCHEMA_VERSION, active_m=active_m, backend="hip-gfx950", tasks=tasks,
         events=[dict(id=t["id"], num_triggers=1, fires=[u["id"] for u in tasks if t["id"] in u["depends_on"]]) for t in tasks],
         scratch_buffers=scratch_buffers, initial_tasks=[t["id"] for t in tasks if not t["depends_on"]],
-        model_params=[dict(path=s["source_path"], shape=s["shape"], dtype=s["dtype"]) for s in sym.values() if s["role"] == "external"],
+        model_params=[dict(path=s["source_path"], shape=s["shape"], dtype=s["dtype"]) for s in sym.values()
+                      if s["role"] == "external" and not s.get("transform")],
         layer_groups=[dict(region=r, task_ids=ids) for r, ids in groups.items()],
         decode_pipeline=[t["id"] for t in tasks],
         decode_capabilities=dict(dispatchable=True, reasons=[]),
@@ -247,7 +264,16 @@ class ArtifactRuntime:
             slots = sorted(t["inputs"] + t["outputs"], key=lambda b: b["slot"])
             args = []
             for b in slots:
-                buf = self._params[b["source_path"]] if b["role"] == "external" else self.scratch[b["role_name"]]
+                if b["role"] == "external" and b.get("transform") == "xcd_kslice":
+                    key = b["source_path"] + "@xcd_kslice"
+                    if key not in self._params:   # [n, groups] -> [8][n][groups / 8], once per parameter
+                        n, groups = b["shape"]
+                        self._params[key] = native.xcd_kslice_meta(self._params[b["source_path"]], n, groups)
+                    buf = self._params[key]
+                elif b["role"] == "external" and b.get("transform"):
+                    raise ValueError(f"task {tid} slot {b['slot']}: unknown parameter transform {b['transform']}")
+                else:
+                    buf = self._params[b["source_path"]] if b["role"] == "external" else self.scratch[b["role_name"]]
                 off = int(b.get("offset_bytes", 0))
                 if off + b["nbytes"] > buf.nbytes:
                     raise ValueError(f"task {tid} slot {b['slot']}: binding wants {off + b['nbytes']} bytes, buffer has {buf.nbytes}")

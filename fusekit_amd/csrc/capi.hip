@@ -728,6 +728,10 @@ fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t* co
 
 size_t fk_xcd_sum_row_bytes(uint32_t hidden) { return xcd_sum_row_bytes(hidden); }
 
+fk_status fk_xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint16_t* dst, fk_stream s) {
+    return xcd_kslice_meta(src, n, groups, dst, (hipStream_t)s);
+}
+
 fk_status fk_xcd_check(void* workspace, fk_stream s) {
     if (!workspace) return set_error(FK_ERR_INVALID, "fk_xcd_check: null workspace");
     FK_HIP(hipStreamSynchronize((hipStream_t)s));

@@ -284,12 +284,14 @@ __device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, const 
 // A vector memory instruction costs the CU about as much to issue whether it moves 2 or 16 bytes per lane, so
 // a tile of whole rows whose row holds a multiple of four groups (its groups are then one contiguous,
 // 8-byte-aligned run of the scale and of the bias array) is fetched four groups per lane and instruction.
-// RUN: the tile spans whole rows of a multiple of four groups (the host plans it so).
+// RUN: the tile's groups are one contiguous, 8-byte aligned run of a multiple of four entries of the scale and of
+// the bias array (the host plans it so): a tile of whole rows, or a K-slice tile of a matrix whose scales and
+// biases were re-laid out per XCD (fk_xcd_kslice_meta: [xcd][row][groups of the slice]; `xcd` then selects the copy).
 template <WKind KIND, int SN, bool RUN>
-__device__ __forceinline__ void meta_fetch(const XcdMat& m, const Tile& t, uint32_t ti, MetaRegs& r) {
+__device__ __forceinline__ void meta_fetch(const XcdMat& m, const Tile& t, uint32_t ti, MetaRegs& r, uint32_t xcd = 0) {
     if constexpr (KIND != W_BF16) {
         const uint32_t gpr = t.cs >> m.gshift, total = t.rows * gpr;
-        const size_t g0 = (size_t)t.row0 * (m.cpr >> m.gshift) + (t.col0 >> m.gshift);
+        const size_t g0 = t.cs == m.cpr ? (size_t)t.row0 * gpr : ((size_t)xcd * m.rows + t.row0) * gpr;
         if constexpr (RUN) {
             // kMetaRegs * SN groups at most: lane ti takes groups 4 ti .. 4 ti + 3 (s[0..1] / b[0..1] hold them)
             const uint32_t gi = 4u * ti;
@@ -530,7 +532,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     FK_XCD_STAMP(1, 5);
     meta_store<KIND, kBlock, true>(mg, tid, meta);
     meta_store<KIND, kBlock, true>(mu, tid, meta + kMetaWords);
-    meta_fetch<KIND, kBlock, false>(a.down, td, tid, md);  // not needed before the hand-over: kept off the start-up path
+    meta_fetch<KIND, kBlock, true>(a.down, td, tid, md, sync.xcd);  // not needed before the hand-over: kept off the start-up path
     __syncthreads();
 
     // ---- gate / up rows of this XCD's slice, SwiGLU ----
@@ -544,7 +546,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
             request_down();
     }
     FK_XCD_STAMP(1, 6);
-    meta_store<KIND, kBlock, false>(md, tid, meta + 2 * kMetaWords);
+    meta_store<KIND, kBlock, true>(md, tid, meta + 2 * kMetaWords);
     __syncthreads();
     if (streams && gu_n) {
         uint16_t* mid = a.mid + (size_t)sync.xcd * per_xcd + gu0;
@@ -627,7 +629,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red);
     FK_XCD_STAMP(0, 5);
     meta_store<KIND, kAttnStream, true>(mmq, ti, meta);
-    meta_fetch<KIND, kAttnStream, false>(a.wo, to, ti, mmo);  // not needed before the attention is done
+    meta_fetch<KIND, kAttnStream, true>(a.wo, to, ti, mmo, sync.xcd);  // not needed before the attention is done
     __syncthreads();
 
     // ---- q / k / v rows of this XCD's KV head; the o_proj slice is requested behind their last pass ----
@@ -722,7 +724,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
             stage_emit<KIND>(xs, sx, a.o_cs, t, live, v, v, 1.0f, false);
         }
     }
-    meta_store<KIND, kAttnStream, false>(mmo, ti, meta + kMetaWords);
+    meta_store<KIND, kAttnStream, true>(mmo, ti, meta + kMetaWords);
     __syncthreads();
     if (streams && o_n) tile_run<KIND, NLB, kAttnStream>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
     __syncthreads();
@@ -743,7 +745,27 @@ __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs 
     if (a.clear) a.clear[at] = 0;
 }
 
+// dst[(h * n + r) * gl + g] = src[r * groups + h * gl + g]: the scales (or biases) of a [n, groups] matrix, the
+// K dimension cut into 8 slices of gl = groups / 8 groups, one contiguous copy per slice.
+__global__ __launch_bounds__(kBlock) void xcd_kslice_meta_kernel(const uint16_t* src, uint16_t* dst, uint32_t n, uint32_t groups) {
+    const uint32_t gl = groups / kXcds;
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= (size_t)n * groups) return;
+    const uint32_t g = (uint32_t)(i % gl), r = (uint32_t)((i / gl) % n), h = (uint32_t)(i / ((size_t)gl * n));
+    dst[i] = src[(size_t)r * groups + h * gl + g];
+}
+
 // =============================================================================================== host side
+fk_status xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint16_t* dst, hipStream_t stream) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!src || !dst || n == 0 || groups == 0 || groups % kXcds) return set_error(FK_ERR_INVALID, "xcd k-slice scales: null buffer, or groups per row not a multiple of 8");
+    const size_t total = (size_t)n * groups;
+    hipLaunchKernelGGL(xcd_kslice_meta_kernel, dim3((unsigned)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0, stream, src, dst, n, groups);
+    FK_HIP(hipGetLastError());
+    return FK_OK;
+}
+
 namespace {
 
 constexpr int kNlQkv = 6, kNlO = 4, kNlGu = 6, kNlDown = 6;  // 16-byte requests per streaming thread and pass
@@ -766,6 +788,7 @@ fk_status bind_mat(const fk_weight* w, uint32_t n, uint32_t k, const XcdLayerSha
     m->w = reinterpret_cast<const uint4*>(w->w);
     m->sc = w->scales;
     m->bi = w->biases;
+    m->rows = n;
     m->cpr = k / chunk_values(s.bits);
     m->gshift = s.bits == 16 ? 0 : ilog2u(s.group / chunk_values(s.bits));
     return FK_OK;
@@ -834,6 +857,10 @@ fk_status xcd_layer_supported(const XcdLayerShape& s) {
             ceil_div(s.inter / kXcds, kXcdSlots) * (s.hidden / s.group) > budget ||
             ceil_div(s.hidden, kXcdSlots) * (s.inter / kXcds / s.group) > budget)
             return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a block's tile holds more quantisation groups than the kernel fetches");
+        // the groups of a block's o_proj / down_proj tile are fetched four per lane from the per-XCD copies
+        const uint32_t rpb = ceil_div(s.hidden, kXcdSlots);
+        if (s.hidden % kXcdSlots || (rpb * (n_q / kXcds / s.group)) % 4 || (rpb * (s.inter / kXcds / s.group)) % 4)
+            return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a block's o_proj / down_proj tile must hold a multiple of four quantisation groups");
     }
     return FK_OK;
 }

@@ -70,8 +70,9 @@ inline uint32_t xcd_sum_row_elems(uint32_t hidden) { return (hidden + 511u) / 51
 // chunks [col0, col0 + cs) of each row's cpr 16-byte chunks.
 struct XcdMat {
     const uint4* w;
-    const uint16_t* sc;
+    const uint16_t* sc;   // o_proj / down_proj: the per-XCD re-laid-out copies (fk_xcd_kslice_meta)
     const uint16_t* bi;
+    uint32_t rows;     // rows of the matrix
     uint32_t cpr;      // chunks per full row
     uint32_t gshift;   // chunk index >> gshift = quantisation group
 };
@@ -142,6 +143,8 @@ struct XcdLayerShape {
 fk_status xcd_layer_supported(const XcdLayerShape& s);
 size_t xcd_workspace_bytes();
 size_t xcd_sum_row_bytes(uint32_t hidden);
+// Scales (or biases) [n, groups] -> [8][n][groups / 8]: what the o_proj / down_proj slots of the launches take.
+fk_status xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint16_t* dst, hipStream_t stream);
 size_t xcd_attn_partials_bytes(const XcdLayerShape& s);
 
 struct XcdAttnRequest {

@@ -227,6 +227,14 @@ class DecoderRuntime:
             self.xcd_xa, self.xcd_xb = DeviceBuffer(cfg.hidden * 2), DeviceBuffer(cfg.hidden * 2)
             # three rotating sum rows: a launch reads one, adds into the next and clears the third
             self.xcd_sums = [z(native.xcd_sum_row_bytes(cfg.hidden)) for _ in range(3)]
+            # scales / biases of o_proj and down_proj, one contiguous copy per K-slice (once, at load time)
+            self.xcd_kmeta: Dict[str, tuple] = {}
+            if cfg.bits != 16:
+                for l in range(cfg.n_layers):
+                    for name in (f"layers.{l}.self_attn.o_proj", f"layers.{l}.mlp.down_proj"):
+                        W = weights.mats[name]
+                        self.xcd_kmeta[name] = (native.xcd_kslice_meta(W.scales, W.n, W.k // W.group),
+                                                native.xcd_kslice_meta(W.biases, W.n, W.k // W.group))
         self._bf16_weights: Dict[str, DeviceWeight] = {}   # resident bf16 copies for prompt passes (prefill_rows)
         self.tasks = self.build_tasks()
         # persistent: the same task list, run by one whole-token kernel per replay
@@ -348,6 +356,12 @@ class DecoderRuntime:
                            arg(self.hist_counter)], dict(vocab=c.vocab)))
         return t
 
+    def _xcd_kslice_args(self, name: str, W: DeviceWeight):
+        if W.bits == 16:
+            return [arg(W.w)]
+        sc, bi = self.xcd_kmeta[name]
+        return [arg(W.w), arg(sc), arg(bi)]
+
     def _xcd_layer_tasks(self, t: List[Dispatch], name) -> None:
         """Two launches per layer (families fusekit_xcd_attn_block / fusekit_xcd_mlp_block), then the last layer's
         sum row + residual into x[0] for the LM head.  Launch i of the token reads sum row i % 3, adds into row
@@ -367,7 +381,7 @@ class DecoderRuntime:
                   arg(Wq.w), arg(Wk.w), arg(Wv.w)]
             if quant:
                 a += [arg(m.scales) for m in (Wq, Wk, Wv)] + [arg(m.biases) for m in (Wq, Wk, Wv)]
-            a += self._wargs(Wo)
+            a += self._xcd_kslice_args(p + "self_attn.o_proj", Wo)
             if c.qk_norm:
                 a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
             a += [arg(self.q), arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
@@ -378,7 +392,7 @@ class DecoderRuntime:
                  arg(Wg.w), arg(Wu.w)]
             if quant:
                 m += [arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases)]
-            m += self._wargs(Wd) + [arg(self.mid), S(2 * l + 2), S(2 * l + 3), arg(self.xcd_ctl)]
+            m += self._xcd_kslice_args(p + "mlp.down_proj", Wd) + [arg(self.mid), S(2 * l + 2), S(2 * l + 3), arg(self.xcd_ctl)]
             t.append(Dispatch(name("xcd_mlp_block"), m, dict(shape, has_sums=1, variant=c.swiglu_variant)))
         t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_sums[(2 * c.n_layers) % 3]), arg(self.xcd_xb), arg(self.x[0]),
                                                arg(self.xcd_sums[1])], dict(hidden=c.hidden)))

@@ -515,6 +515,13 @@ def xcd_sum_row_bytes(hidden: int) -> int:
     return int(lib.fk_xcd_sum_row_bytes(C.c_uint32(hidden)))
 
 
+def xcd_kslice_meta(src: "DeviceBuffer", n: int, groups: int, stream=None) -> "DeviceBuffer":
+    """The per-XCD re-laid-out copy of a scale or bias array [n, groups] (fk_xcd_kslice_meta)."""
+    dst = DeviceBuffer(n * groups * 2)
+    check(lib.fk_xcd_kslice_meta(_ptr(src), C.c_uint32(n), C.c_uint32(groups), _ptr(dst), _ptr(stream)))
+    return dst
+
+
 def xcd_sum_index(hidden: int):
     """Index of element e of a hidden-wide vector inside a sum row (numpy array of hidden indices)."""
     import numpy as np

@@ -510,6 +510,12 @@ fk_status fk_xcd_layer_supported(uint32_t hidden, uint32_t inter, uint32_t n_hea
 fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t *control_bytes, size_t *attention_partial_bytes);
 /* Bytes of one sum row of a hidden-wide vector (0 for hidden == 0). */
 size_t fk_xcd_sum_row_bytes(uint32_t hidden);
+/* The o_proj and down_proj slots of the two families take their scales and biases re-laid out per K-slice:
+ * dst[(h * n + r) * (groups / 8) + g] = src[r * groups + h * (groups / 8) + g] for the [n, groups] array of a
+ * matrix (same size as the source).  An XCD then reads its slice of every row as one contiguous stream; in the
+ * MLX layout its 16..38 bytes of every row drag whole 128-byte lines into all eight L2s.  Done once per matrix
+ * at load time; the weights themselves stay in the MLX layout (src/fusion/ir.rs:236-242). */
+fk_status fk_xcd_kslice_meta(const uint16_t *src, uint32_t n, uint32_t groups, uint16_t *dst, fk_stream s);
 /* Synchronises the stream and reports whether a launch gave up on a hand-over wait (FK_ERR_HIP; the control
  * block is reset).  The dispatcher calls it after every graph execution that holds such launches. */
 fk_status fk_xcd_check(void *workspace, fk_stream s);

@@ -23,6 +23,23 @@ def _wargs(arg, W):
     return [arg(W.w)] + ([] if W.bits == 16 else [arg(W.scales), arg(W.biases)])
 
 
+def _kslice_args(fk, arg, W, keep):
+    """o_proj / down_proj slots: the weights as they are, scales and biases re-laid out per K-slice
+    (fk_xcd_kslice_meta), checked here against the plain numpy statement of that layout."""
+    if W.bits == 16:
+        return [arg(W.w)]
+    out = [arg(W.w)]
+    groups = W.k // W.group
+    for src in (W.scales, W.biases):
+        dst = fk.xcd_kslice_meta(src, W.n, groups)
+        fk.sync()
+        want = src.to_numpy(np.uint16, (W.n, 8, groups // 8)).transpose(1, 0, 2)
+        assert np.array_equal(dst.to_numpy(np.uint16, (8, W.n, groups // 8)), want)
+        keep.append(dst)
+        out.append(arg(dst))
+    return out
+
+
 def _sum_row(fk, hidden, contributions=None):
     """A sum row as the launches keep it: 64-bit fixed point (2^-32 units), elements permuted (fk.xcd_sum_index),
     padded to whole 512-element sections; `contributions` [n][hidden] fp32 are added the way a launch adds its
@@ -76,7 +93,8 @@ def test_xcd_mlp_block(fk, bits, hidden, inter, variant):
     a = [arg(b["p"]), arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dWg.w), arg(dWu.w)]
     if bits != 16:
         a += [arg(dWg.scales), arg(dWu.scales), arg(dWg.biases), arg(dWu.biases)]
-    a += _wargs(arg, dWd) + [arg(b["mid"]), arg(b["out"]), arg(b["clr"]), arg(ctl)]
+    keep = []
+    a += _kslice_args(fk, arg, dWd, keep) + [arg(b["mid"]), arg(b["out"]), arg(b["clr"]), arg(ctl)]
     task = Dispatch("fusekit_xcd_mlp_block_f1", a,
                     dict(hidden=hidden, inter=inter, n_heads=32, n_kv=8, head_dim=128, capacity=256, bits=bits, group=64,
                          eps=EPS, variant=variant, has_sums=1))
@@ -138,7 +156,8 @@ def test_xcd_attn_block(fk, bits, n_heads, head_dim, qk_norm):
     a = [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dW[0].w), arg(dW[1].w), arg(dW[2].w)]
     if bits != 16:
         a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]]
-    a += _wargs(arg, dW[3])
+    keep = []
+    a += _kslice_args(fk, arg, dW[3], keep)
     if qk_norm:
         b["qn"], b["kn"] = _dev(fk, qn), _dev(fk, kn)
         a += [arg(b["qn"]), arg(b["kn"])]
@@ -221,7 +240,8 @@ def test_xcd_attn_block_at_the_config3_contexts(fk, kv_len):
              kv_len=fk.zeros(4), off=fk.zeros(4), step=_dev(fk, np.array([pos], np.uint32)), tab=fk.DeviceBuffer(head_dim * 4),
              ap=fk.DeviceBuffer(ap_bytes), out=_dev(fk, _sum_row(fk, hidden)), clr=_dev(fk, _sum_row(fk, hidden)))
     a = [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(dW[0].w), arg(dW[1].w), arg(dW[2].w)]
-    a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]] + _wargs(arg, dW[3])
+    keep = []
+    a += [arg(m.scales) for m in dW[:3]] + [arg(m.biases) for m in dW[:3]] + _kslice_args(fk, arg, dW[3], keep)
     a += [arg(b["q"]), arg(b["k"]), arg(b["v"]), arg(b["ck"]), arg(b["cv"]), arg(b["kv_len"]), arg(b["tab"]), arg(b["ap"]),
           arg(b["out"]), arg(b["clr"]), arg(ctl)]
     task = Dispatch("fusekit_xcd_attn_block_f1", a,
