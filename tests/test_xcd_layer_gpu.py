@@ -334,3 +334,29 @@ def test_xcd_decoder_tokens_match_oracle_and_the_per_dispatch_path(fk, bits, n_h
     for name_, seq in (("xcd", got), ("per-dispatch", got_old)):
         i = next((i for i, (g, r) in enumerate(zip(seq, ref)) if g != r), None)
         assert i is None or margins[i] < 0.01, f"{name_}: step {i}: gpu {seq[i]} oracle {ref[i]} at margin {margins[i]}"
+
+
+def test_artifact_round_trip_of_a_two_launch_layer_model(fk, tmp_path):
+    """task_graph.json written from a runtime on the two-launch layer path (control words, sum rows, the
+    per-K-slice copies of o_proj / down_proj scales and biases recorded as a parameter + transform) and replayed
+    by a consumer that knows only the files and the parameter tree: same tokens."""
+    import json
+    from fusekit_amd.artifact import ArtifactRuntime, write_artifact
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    cfg = DecoderConfig(n_layers=2, hidden=512, n_heads=16, n_kv=8, head_dim=64, inter=1024, vocab=1000, capacity=128,
+                        qk_norm=True)
+    W = DecoderWeights.random_init(cfg, seed=9)
+    rt = DecoderRuntime(cfg, W)
+    assert rt.xcd
+    prompt = [3, 700, 41, 12]
+    want, _, _ = rt.generate(prompt, 12)
+    write_artifact(rt, str(tmp_path), "tiny8")
+    tg = json.load(open(tmp_path / "task_graph.json"))
+    kinds = [t["kernel"].rsplit("_f", 1)[0] for t in tg["tasks"]]
+    assert kinds.count("fusekit_xcd_attn_block") == 2 and kinds.count("fusekit_xcd_mlp_block") == 2
+    attn = next(t for t in tg["tasks"] if t["kernel"].startswith("fusekit_xcd_attn_block"))
+    moved = [b for b in attn["inputs"] if b.get("transform") == "xcd_kslice"]
+    assert sorted(b["source_path"] for b in moved) == ["layers.0.self_attn.o_proj.biases", "layers.0.self_attn.o_proj.scales"]
+    assert not any("@" in p["path"] for p in tg["model_params"])
+    got = ArtifactRuntime(str(tmp_path), W).generate(prompt, 12)
+    assert got == want
