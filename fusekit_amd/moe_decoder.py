@@ -93,11 +93,16 @@ class MoeWeights:
         self.vecs: Dict[str, DeviceBuffer] = {}
 
     @classmethod
-    def random_init(cls, cfg: MoeConfig, seed: int = 0, std: float = 0.02) -> "MoeWeights":
+    def random_init(cls, cfg: MoeConfig, seed: int = 0, std: float = 0.02, exact: bool = False,
+                    embed_loud_rows: int = 0, embed_loud_gain: float = 1.0) -> "MoeWeights":
         """Projections ~ N(0, std^2) quantised on the device (experts stacked [E, n, k]); the router and
-        the tied embedding stay bf16; norm weights ~ 1 + N(0, 0.1^2)."""
+        the tied embedding stay bf16; norm weights ~ 1 + N(0, 0.1^2).
+        exact: every value from the host-reproducible generator (fk_synth_fill_exact), so that a CPU build of the
+        same model from the same seeds holds the same bytes; embed_loud_rows / embed_loud_gain (exact only): a few
+        dominant embedding rows (token ids 0 .. loud_rows - 1)."""
         self = cls(cfg)
         c = cfg
+        f32_kind, bf16_kind = (3, 4) if exact else (0, 1)
         biggest = max(c.n_experts * c.moe_inter * c.hidden if c.n_layers > c.first_dense else 0,
                       c.dense_inter * c.hidden if c.first_dense else 0, c.n_heads * c.qk_dim * c.hidden)
         tmp = DeviceBuffer(biggest * 4)
@@ -109,7 +114,7 @@ class MoeWeights:
 
         def matrix(name: str, n: int, k: int, experts: int = 0, sd: float = std) -> None:
             rows = n * max(experts, 1)
-            _synth(tmp, rows * k, next_seed(), 0.0, sd, 0)
+            _synth(tmp, rows * k, next_seed(), 0.0, sd, f32_kind)
             W = quantize_on_device(tmp, rows, k, c.bits, c.group)
             if experts:
                 W.n, W.n_experts = n, experts
@@ -119,12 +124,15 @@ class MoeWeights:
             W = DeviceWeight.__new__(DeviceWeight)
             W.n, W.k, W.bits, W.group = n, k, 16, 0
             W.w, W.scales, W.biases = DeviceBuffer(n * k * 2), None, None
-            _synth(W.w, n * k, next_seed(), 0.0, sd, 1)
+            if exact and name == "embed_tokens":
+                _synth(W.w, n * k, next_seed(), 0.0, sd, 4, row_len=k, loud_rows=embed_loud_rows, loud_gain=embed_loud_gain)
+            else:
+                _synth(W.w, n * k, next_seed(), 0.0, sd, bf16_kind)
             self.mats[name] = W
 
         def vector(name: str, n: int, mean: float, sd: float) -> None:
             b = DeviceBuffer(n * 2)
-            _synth(b, n, next_seed(), mean, sd, 1)
+            _synth(b, n, next_seed(), mean, sd, bf16_kind)
             self.vecs[name] = b
 
         dense_bf16("embed_tokens", c.vocab, c.hidden, std)

@@ -189,15 +189,104 @@ class OracleDecoder:
         return toks, margins
 
 
+class HostMoeWeights:
+    """The mixture-of-experts decoder's weights built on the HOST with the oracle's copy of the library's
+    host-reproducible generator and the oracle's quantiser: the bytes `MoeWeights.random_init(cfg, seed, std,
+    exact=True, ...)` puts into HBM (same seed sequence).  `mats`: oracle QWeight / StackedWeight, `vecs`: bf16 bits."""
+
+    def __init__(self, cfg, seed: int = 0, std: float = 0.02, embed_loud_rows: int = 0, embed_loud_gain: float = 1.0):
+        self.cfg = c = cfg
+        self.mats, self.vecs = {}, {}
+        counter = [seed * 100003 + 7]
+
+        def next_seed():
+            counter[0] += 1
+            return counter[0]
+
+        def matrix(name, n, k, experts=0, sd=std):
+            rows = n * max(experts, 1)
+            W = oracle.quantize(oracle.synth_fill(rows * k, next_seed(), 0.0, sd, 3).reshape(rows, k), c.bits, c.group)
+            if experts:
+                S = oracle.StackedWeight.__new__(oracle.StackedWeight)
+                oracle.QWeight.__init__(S, np.asarray(W.w).reshape(experts, n, -1), np.asarray(W.scales).reshape(experts, n, -1),
+                                        np.asarray(W.biases).reshape(experts, n, -1), n, k, c.bits, c.group)
+                S.n_experts = experts
+                W = S
+            self.mats[name] = W
+
+        def dense_bf16(name, n, k, sd):
+            if name == "embed_tokens":
+                a = oracle.synth_fill(n * k, next_seed(), 0.0, sd, 4, row_len=k, loud_rows=embed_loud_rows, loud_gain=embed_loud_gain)
+            else:
+                a = oracle.synth_fill(n * k, next_seed(), 0.0, sd, 4)
+            self.mats[name] = oracle.dense(a.reshape(n, k))
+
+        def vector(name, n, mean, sd):
+            self.vecs[name] = oracle.synth_fill(n, next_seed(), mean, sd, 4)
+
+        dense_bf16("embed_tokens", c.vocab, c.hidden, std)
+        vector("final_norm", c.hidden, 1.0, 0.1)
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            vector(p + "input_layernorm", c.hidden, 1.0, 0.1)
+            vector(p + "post_attention_layernorm", c.hidden, 1.0, 0.1)
+            matrix(p + "self_attn.q_proj", c.n_heads * c.qk_dim, c.hidden)
+            matrix(p + "self_attn.kv_a_proj_with_mqa", c.kv_lora_rank + c.rope_dim, c.hidden)
+            vector(p + "self_attn.kv_a_layernorm", c.kv_lora_rank, 1.0, 0.1)
+            matrix(p + "self_attn.kv_b_proj", c.n_heads * (c.nope_dim + c.v_dim), c.kv_lora_rank)
+            matrix(p + "self_attn.o_proj", c.hidden, c.n_heads * c.v_dim)
+            if l < c.first_dense:
+                matrix(p + "mlp.gate_proj", c.dense_inter, c.hidden)
+                matrix(p + "mlp.up_proj", c.dense_inter, c.hidden)
+                matrix(p + "mlp.down_proj", c.hidden, c.dense_inter)
+            else:
+                dense_bf16(p + "mlp.gate", c.n_experts, c.hidden, 0.05)
+                for nm in ("gate_proj", "up_proj"):
+                    matrix(p + f"mlp.switch_mlp.{nm}", c.moe_inter, c.hidden, c.n_experts)
+                    matrix(p + f"mlp.shared_experts.{nm}", c.shared_inter, c.hidden)
+                matrix(p + "mlp.switch_mlp.down_proj", c.hidden, c.moe_inter, c.n_experts)
+                matrix(p + "mlp.shared_experts.down_proj", c.hidden, c.shared_inter)
+
+
+def moe_stable_channel(cfg, mats, vecs, channel: int, level: float, route_logits, route_noise: float):
+    """Gives a mixture-of-experts model what a trained one has and a random one lacks: a persistent large
+    activation in one hidden channel, and routers that read it.  On the bf16 arrays of `mats` / `vecs` (oracle
+    weights), in place:
+      * the tied embedding's column `channel` becomes `level` for every token (it dominates every RMS norm input of
+        the stack), and the final norm's weight of that channel becomes 0, so that the head never sees it (the same
+        huge amount in every logit would cost the logits their resolution);
+      * each router keeps its random rows scaled by `route_noise` and gets column `channel` = route_logits[j] / u,
+        u = sqrt(hidden) (the channel's normalised value when it dominates): expert j's logit is about
+        route_logits[j] whatever the token, plus noise.
+    Returns the names of the arrays it changed (the caller uploads those to the device model)."""
+    changed = ["embed_tokens", "final_norm"]
+    E = np.asarray(mats["embed_tokens"].w).reshape(cfg.vocab, cfg.hidden)
+    E[:, channel] = oracle.f32_to_bf16(np.array([level], np.float32))[0]
+    vecs["final_norm"][channel] = 0
+    u = float(np.sqrt(cfg.hidden))
+    col = oracle.f32_to_bf16((np.asarray(route_logits, np.float32) / u).astype(np.float32))
+    for l in range(cfg.first_dense, cfg.n_layers):
+        name = f"layers.{l}.mlp.gate"
+        R = np.asarray(mats[name].w).reshape(cfg.n_experts, cfg.hidden)
+        R[:] = oracle.f32_to_bf16((oracle.bf16_to_f32(R) * np.float32(route_noise)).astype(np.float32))
+        R[:, channel] = col
+        changed.append(name)
+    return changed
+
+
 class OracleMoeDecoder:
     """CPU oracle of the mixture-of-experts decoder with low-rank keys, composed from the oracle's
     per-kernel functions on the very bytes the GPU model holds, one call per dispatch of the GPU task list."""
 
     def __init__(self, cfg, weights):
         self.cfg = c = cfg
-        self.vec = {k: v.to_numpy(np.uint16) for k, v in weights.vecs.items()}
+        host = isinstance(weights, HostMoeWeights)
+        self.vec = dict(weights.vecs) if host else {k: v.to_numpy(np.uint16) for k, v in weights.vecs.items()}
         self.mat = {}
         for k, dw in weights.mats.items():
+            if host:
+                self.mat[k] = dw
+                continue
             E = getattr(dw, "n_experts", 0)
             if not E:
                 self.mat[k] = host_weight(dw)
