@@ -59,6 +59,9 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
         scratch("xcd.x.1", rt.xcd_xb, "bfloat16")
         for i, b in enumerate(rt.xcd_sums):
             scratch(f"xcd.sums.{i}", b, "uint32", zero=True)
+        for l, bufs in enumerate(getattr(rt, "xcd_qkv", [])):
+            for nm, b in zip("qkv", bufs):
+                scratch(f"xcd.{nm}.{l}", b, "bfloat16")
     for l in range(rt.cfg.n_layers):
         if rt.cfg.kv_bits:
             for nm, c in (("cache_k", rt.cache_k[l]), ("cache_v", rt.cache_v[l])):

@@ -768,6 +768,7 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
     rq.workspace = d.args[ws_slot].ptr;
     rq.spin_limit = d.u("spin_limit", 0);
+    rq.for_token = d.u("token", 0) != 0;
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
     rw->writes = {(uint32_t)x_slot, (uint32_t)mid_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
     return plan_xcd_mlp(rq, l);
@@ -1241,6 +1242,18 @@ struct Graph {
     hipGraphExec_t exec = nullptr;
     std::vector<uint8_t> barriers;  // as given to fk_build_graph (empty: none forced)
     std::vector<void*> xcd_controls;  // control blocks of XCD-resident launches in this graph (abort words)
+    // Runs of alternating xcd_attn / xcd_mlp dispatches (parameter token_launch = 1) executed as ONE launch each:
+    // the nodes keep their own launches (eager execution, profiling), the executable graph holds one kernel node
+    // per run, whose per-layer argument blocks sit in device tables.
+    struct FusedRun {
+        size_t first = 0, count = 0;
+        Launch launch;
+        void* d_attn = nullptr;
+        void* d_mlp = nullptr;
+        hipGraphNode_t node = nullptr;
+    };
+    std::vector<FusedRun> fused;
+    std::vector<int> fused_of;  // per node: index into `fused`, or -1
     // persistent whole-token mode: one kernel node; device-side tables it reads
     bool persistent = false;
     Launch token_launch;
@@ -1256,6 +1269,10 @@ struct Graph {
         if (exec) (void)hipGraphExecDestroy(exec);
         if (graph) (void)hipGraphDestroy(graph);
         if (d_tables) (void)hipFree(d_tables);
+        for (FusedRun& r : fused) {
+            if (r.d_attn) (void)hipFree(r.d_attn);
+            if (r.d_mlp) (void)hipFree(r.d_mlp);
+        }
     }
 };
 
@@ -1766,6 +1783,72 @@ fk_status fk_plan_geometry(fk_handle h, const fk_dispatch* d, fk_launch_geometry
     return FK_OK;
 }
 
+// The argument block a member of a fused run contributes to the run's device tables: the dispatch planned once
+// more with the parameter `token` (the one launch sizes some tiles differently).
+fk_status plan_for_token(const Dispatch& d, Launch* l) {
+    Dispatch t = d;
+    t.params.emplace_back("token", 1.0);
+    SlotRW rw;
+    return plan_dispatch(t, l, &rw);
+}
+
+bool is_family(const Dispatch& d, const char* fam) {
+    const size_t n = strlen(fam);
+    return d.kernel.compare(0, n, fam) == 0 && (d.kernel.size() == n || d.kernel[n] == '_');
+}
+
+fk_status find_fused_runs(Graph* g) {
+    const size_t n = g->nodes.size();
+    g->fused_of.assign(n, -1);
+    size_t i = 0;
+    while (i < n) {
+        const Dispatch& d = g->nodes[i].d;
+        if (!(is_family(d, "fusekit_xcd_attn_block") && d.u("token_launch", 0) != 0)) {
+            ++i;
+            continue;
+        }
+        size_t j = i;
+        while (j + 1 < n && is_family(g->nodes[j].d, "fusekit_xcd_attn_block") && g->nodes[j].d.u("token_launch", 0) != 0 &&
+               is_family(g->nodes[j + 1].d, "fusekit_xcd_mlp_block") && g->nodes[j + 1].d.u("token_launch", 0) != 0 &&
+               g->nodes[j].d.u("bits", 4) == d.u("bits", 4))
+            j += 2;
+        const size_t count = j - i;
+        if (count < 2) {
+            ++i;
+            continue;
+        }
+        const uint32_t layers = (uint32_t)(count / 2);
+        std::vector<XcdAttnArgs> ha(layers);
+        std::vector<XcdMlpArgs> hm(layers);
+        uint32_t attn_lds = 0, mlp_lds = 0;
+        for (uint32_t l = 0; l < layers; ++l) {
+            Launch la, lm;
+            FK_TRY(plan_for_token(g->nodes[i + 2 * l].d, &la));
+            FK_TRY(plan_for_token(g->nodes[i + 2 * l + 1].d, &lm));
+            if (la.args_size != sizeof(XcdAttnArgs) || lm.args_size != sizeof(XcdMlpArgs))
+                return set_error(FK_ERR_INVALID, "fused layer run: unexpected argument block");
+            memcpy(&ha[l], la.args, sizeof(XcdAttnArgs));
+            memcpy(&hm[l], lm.args, sizeof(XcdMlpArgs));
+            attn_lds = std::max(attn_lds, la.shmem);
+            mlp_lds = std::max(mlp_lds, lm.shmem);
+        }
+        Graph::FusedRun run;
+        run.first = i;
+        run.count = count;
+        g->fused.push_back(run);
+        Graph::FusedRun& r = g->fused.back();
+        FK_HIP(hipMalloc(&r.d_attn, layers * sizeof(XcdAttnArgs)));
+        FK_HIP(hipMalloc(&r.d_mlp, layers * sizeof(XcdMlpArgs)));
+        FK_HIP(hipMemcpy(r.d_attn, ha.data(), layers * sizeof(XcdAttnArgs), hipMemcpyHostToDevice));
+        FK_HIP(hipMemcpy(r.d_mlp, hm.data(), layers * sizeof(XcdMlpArgs), hipMemcpyHostToDevice));
+        FK_TRY(plan_xcd_token(ha.data(), hm.data(), layers, d.u("bits", 4), reinterpret_cast<const XcdAttnArgs*>(r.d_attn),
+                              reinterpret_cast<const XcdMlpArgs*>(r.d_mlp), attn_lds, mlp_lds, &r.launch));
+        for (size_t m = i; m < j; ++m) g->fused_of[m] = (int)g->fused.size() - 1;
+        i = j;
+    }
+    return FK_OK;
+}
+
 fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const uint8_t* barriers, uint32_t* graph_id) {
     DispatcherState* ds;
     FK_TRY(get_dispatcher(h, &ds));
@@ -1786,11 +1869,35 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
             if (std::find(g->xcd_controls.begin(), g->xcd_controls.end(), ws) == g->xcd_controls.end()) g->xcd_controls.push_back(ws);
         }
     }
+    FK_TRY(find_fused_runs(g.get()));
     FK_HIP(hipGraphCreate(&g->graph, 0));
     for (size_t i = 0; i < n; ++i) {
         Node& nd = g->nodes[i];
+        const int fr = g->fused_of[i];
+        if (fr >= 0) {
+            Graph::FusedRun& run = g->fused[fr];
+            if (i != run.first) {
+                nd.node = run.node;  // later dispatches that depend on any member wait for the run's launch
+                continue;
+            }
+            std::vector<hipGraphNode_t> deps;
+            for (size_t m = run.first; m < run.first + run.count; ++m)
+                for (uint32_t j : g->nodes[m].deps)
+                    if (j < run.first) {
+                        hipGraphNode_t dn = g->nodes[j].last();
+                        if (std::find(deps.begin(), deps.end(), dn) == deps.end()) deps.push_back(dn);
+                    }
+            void* slot = nullptr;
+            hipKernelNodeParams p = launch_params(run.launch, &slot);
+            FK_HIP(hipGraphAddKernelNode(&run.node, g->graph, deps.data(), deps.size(), &p));
+            nd.node = run.node;
+            continue;
+        }
         std::vector<hipGraphNode_t> deps;
-        for (uint32_t j : nd.deps) deps.push_back(g->nodes[j].last());
+        for (uint32_t j : nd.deps) {
+            hipGraphNode_t dn = g->nodes[j].last();
+            if (std::find(deps.begin(), deps.end(), dn) == deps.end()) deps.push_back(dn);
+        }
         void* slot = nullptr;
         hipKernelNodeParams p = node_params(nd, &slot);
         FK_HIP(hipGraphAddKernelNode(&nd.node, g->graph, deps.data(), deps.size(), &p));
@@ -1967,6 +2074,17 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
         nd.d = patched[k];
         nd.launch = launches[k];
         nd.rw = rws[k];
+        const int fr = g->fused_of.empty() ? -1 : g->fused_of[touched[k]];
+        if (fr >= 0) {
+            // member of a run that executes as one launch: its argument block in the run's device table is replaced
+            Graph::FusedRun& run = g->fused[fr];
+            Launch lt;
+            FK_TRY(plan_for_token(nd.d, &lt));
+            const size_t pos = touched[k] - run.first;
+            char* dst = (pos & 1) ? (char*)run.d_mlp + (pos / 2) * sizeof(XcdMlpArgs) : (char*)run.d_attn + (pos / 2) * sizeof(XcdAttnArgs);
+            FK_HIP(hipMemcpy(dst, lt.args, lt.args_size, hipMemcpyHostToDevice));
+            continue;
+        }
         void* slot = nullptr;
         hipKernelNodeParams p = node_params(nd, &slot);
         FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.node, &p));

@@ -147,15 +147,34 @@ struct InputRegs {
     uint4 sv[kInGroups][4], rv[kInGroups], nw[kInGroups];
 };
 
-__device__ __forceinline__ void input_request(const XcdInput& in, InputRegs& r) {
+// Zeroes the sum row the launch after this one adds into (16-byte units spread over the grid).  Called once the
+// input has been consumed: a wave's memory counter completes in order, and in the whole-token launch these are
+// write-through stores (a line left dirty in this XCD's L2 would later overwrite the other XCDs' additions) that
+// take a trip to memory.
+template <bool TOKEN, typename IN>
+__device__ __forceinline__ void input_clear(const IN& in) {
+    if (!in.clear) return;
+    const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
+    if (u < in.row_elems / 2) {
+        if constexpr (TOKEN) {
+            unsigned long long* c = reinterpret_cast<unsigned long long*>(in.clear) + 2 * (size_t)u;
+            __hip_atomic_store(c, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(c + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            reinterpret_cast<uint4*>(in.clear)[u] = make_uint4(0, 0, 0, 0);
+        }
+    }
+}
+
+// TOKEN: the launch runs every layer of a token (xcd_token_kernel).  The sum row was then written memory-side by
+// other XCDs earlier in the SAME launch: it is read with L1-bypassing loads.  `xres`, if given, is the block's own
+// copy of the residual row in LDS (every block computes the whole row in every phase).
+template <bool TOKEN, typename IN>
+__device__ __forceinline__ void input_request(const IN& in, InputRegs& r, const uint4* xres) {
     const uint32_t n8 = in.hidden >> 3, lane = threadIdx.x & (kWave - 1);
     const uint4* s16 = reinterpret_cast<const uint4*>(in.sums);
     const uint4* r8 = reinterpret_cast<const uint4*>(in.residual);
     const uint4* w8 = reinterpret_cast<const uint4*>(in.norm_w);
-    if (in.clear) {  // 16-byte units of the row to clear, spread over the grid
-        const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
-        if (u < in.row_elems / 2) reinterpret_cast<uint4*>(in.clear)[u] = make_uint4(0, 0, 0, 0);
-    }
 #pragma unroll
     for (int i = 0; i < kInGroups; ++i) {
         const uint32_t t = threadIdx.x + i * kBlock, sec = t >> 6;  // the wave's section of 64 groups
@@ -163,18 +182,19 @@ __device__ __forceinline__ void input_request(const XcdInput& in, InputRegs& r) 
             const uint32_t tc = t < n8 ? t : 0u;
             if (in.sums) {
 #pragma unroll
-                for (int k = 0; k < 4; ++k) r.sv[i][k] = s16[(sec * 4 + k) * kWave + lane];  // padded row: in bounds
+                for (int k = 0; k < 4; ++k) r.sv[i][k] = ld_u128<TOKEN>(s16 + (sec * 4 + k) * kWave + lane);  // padded row: in bounds
             }
-            r.rv[i] = r8[tc];
+            r.rv[i] = (TOKEN && xres) ? xres[tc] : r8[tc];
             r.nw[i] = w8[tc];
         }
     }
 }
 
-// Whole block (two block barriers inside); `red`: 4 floats of LDS.
-template <WKind KIND, int PROBE>
-__device__ __forceinline__ void input_stage(const XcdInput& in, const InputRegs& r, uint4* xs, float* sx, uint32_t cs,
-                                            float* red) {
+// Whole block (two block barriers inside); `red`: 4 floats of LDS; `xres_out` (LDS, or null): where the block keeps
+// the row for the next phase of the same launch.
+template <WKind KIND, int PROBE, typename IN>
+__device__ __forceinline__ void input_stage(const IN& in, const InputRegs& r, uint4* xs, float* sx, uint32_t cs,
+                                            float* red, uint4* xres_out = nullptr) {
     const uint32_t n8 = in.hidden >> 3;
     uint4 xv[kInGroups];
     float sq = 0.f;
@@ -200,6 +220,7 @@ __device__ __forceinline__ void input_stage(const XcdInput& in, const InputRegs&
                     sq = fmaf(hi, hi, sq);
                 }
                 if (blockIdx.x == 0) reinterpret_cast<uint4*>(in.x_out)[t] = xv[i];
+                if (xres_out) xres_out[t] = xv[i];
             }
         }
     }
@@ -249,8 +270,8 @@ struct TilePos {
     uint32_t p0;            // position of j = 0
     uint32_t col[NL], gidx[NL];
 };
-template <int NL, int SN>
-__device__ __forceinline__ void tile_pos_init(const XcdMat& m, const Tile& t, uint32_t ti, TilePos<NL>& p) {
+template <int NL, int SN, typename MAT>
+__device__ __forceinline__ void tile_pos_init(const MAT& m, const Tile& t, uint32_t ti, TilePos<NL>& p) {
     p.p0 = ti;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
@@ -260,8 +281,8 @@ __device__ __forceinline__ void tile_pos_init(const XcdMat& m, const Tile& t, ui
         p.gidx[j] = (t.row0 + row) * m.cpr + t.col0 + p.col[j];
     }
 }
-template <int NL, int SN>
-__device__ __forceinline__ void tile_pos_next(const XcdMat& m, const Tile& t, uint32_t step_c, uint32_t step_g, TilePos<NL>& p) {
+template <int NL, int SN, typename MAT>
+__device__ __forceinline__ void tile_pos_next(const MAT& m, const Tile& t, uint32_t step_c, uint32_t step_g, TilePos<NL>& p) {
     p.p0 += NL * SN;
     const uint32_t skip = m.cpr - t.cs;
 #pragma unroll
@@ -273,8 +294,8 @@ __device__ __forceinline__ void tile_pos_next(const XcdMat& m, const Tile& t, ui
     }
 }
 
-template <WKind KIND, int NL, int SN>
-__device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, const TilePos<NL>& p, TileRegs<NL>& r) {
+template <WKind KIND, int NL, int SN, typename MAT>
+__device__ __forceinline__ void tile_load(const MAT& m, const Tile& t, const TilePos<NL>& p, TileRegs<NL>& r) {
     const uint32_t total = t.rows * t.cs, first = t.row0 * m.cpr + t.col0;
 #pragma unroll
     for (int j = 0; j < NL; ++j) r.w[j] = m.w[p.p0 + j * SN < total ? p.gidx[j] : first];
@@ -287,8 +308,8 @@ __device__ __forceinline__ void tile_load(const XcdMat& m, const Tile& t, const 
 // RUN: the tile's groups are one contiguous, 8-byte aligned run of a multiple of four entries of the scale and of
 // the bias array (the host plans it so): a tile of whole rows, or a K-slice tile of a matrix whose scales and
 // biases were re-laid out per XCD (fk_xcd_kslice_meta: [xcd][row][groups of the slice]; `xcd` then selects the copy).
-template <WKind KIND, int SN, bool RUN>
-__device__ __forceinline__ void meta_fetch(const XcdMat& m, const Tile& t, uint32_t ti, MetaRegs& r, uint32_t xcd = 0) {
+template <WKind KIND, int SN, bool RUN, typename MAT>
+__device__ __forceinline__ void meta_fetch(const MAT& m, const Tile& t, uint32_t ti, MetaRegs& r, uint32_t xcd = 0) {
     if constexpr (KIND != W_BF16) {
         const uint32_t gpr = t.cs >> m.gshift, total = t.rows * gpr;
         const size_t g0 = t.cs == m.cpr ? (size_t)t.row0 * gpr : ((size_t)xcd * m.rows + t.row0) * gpr;
@@ -331,8 +352,8 @@ __device__ __forceinline__ void meta_store(const MetaRegs& r, uint32_t ti, uint3
 
 // One fp32 partial per chunk into part[pos]; positions past the tile land in the padding of `part` (it holds whole
 // passes) and read group 0's scale and bias.
-template <WKind KIND, int NL, int SN>
-__device__ __forceinline__ void tile_partials(const XcdMat& m, const Tile& t, const TilePos<NL>& p, const TileRegs<NL>& r,
+template <WKind KIND, int NL, int SN, typename MAT>
+__device__ __forceinline__ void tile_partials(const MAT& m, const Tile& t, const TilePos<NL>& p, const TileRegs<NL>& r,
                                               const uint4* xs, const float* sx, const uint32_t* meta, float* part) {
     const uint32_t total = t.rows * t.cs;
 #pragma unroll
@@ -352,8 +373,8 @@ __device__ __forceinline__ void tile_partials(const XcdMat& m, const Tile& t, co
 // All passes of a tile whose first pass is already in `r0` (positions `p` at pass 0): pass k + 1 is requested
 // before pass k is consumed.  `after_last_request` runs once the tile's last pass has been requested (the caller
 // queues what it needs next behind it).
-template <WKind KIND, int NL, int SN, typename F>
-__device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
+template <WKind KIND, int NL, int SN, typename MAT, typename F>
+__device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
                                          const float* sx, const uint32_t* meta, float* part, F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * m.cpr + step_c;
@@ -382,8 +403,8 @@ __device__ __forceinline__ void tile_run(const XcdMat& m, const Tile& t, TilePos
 
 // The gate / up pair: both matrices' passes interleaved, so that one pass of each is in flight while one is consumed.
 // (Same shape and tile: one set of positions serves both.)
-template <WKind KIND, int NL, int SN, typename F>
-__device__ __forceinline__ void tile_run_pair(const XcdMat& ma, const XcdMat& mb, const Tile& t, TilePos<NL>& p,
+template <WKind KIND, int NL, int SN, typename MAT, typename F>
+__device__ __forceinline__ void tile_run_pair(const MAT& ma, const MAT& mb, const Tile& t, TilePos<NL>& p,
                                               TileRegs<NL>& a0, TileRegs<NL>& b0, const uint4* xs, const float* sx,
                                               const uint32_t* meta_a, const uint32_t* meta_b, float* part_a, float* part_b,
                                               F after_last_request) {
@@ -477,9 +498,11 @@ __host__ __device__ inline uint32_t xcd_lds_bytes(const LdsPlan& p) {
 // =============================================================================================== MLP launch
 constexpr int kMlpBlock = kBlock;
 
-template <WKind KIND, int NLA, int NLB>
-__global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) {
-    extern __shared__ uint4 lds_raw[];
+// One MLP phase of one block.  `sync` carries the block's XCD, slot and hand-over epoch; `xres_in` / `xres_out`:
+// the residual row in LDS (token kernel only).
+template <WKind KIND, int NLA, int NLB, bool TOKEN, typename ARGS>
+__device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, XcdSync& sync, uint4* lds_raw, const uint4* xres_in,
+                                              uint4* xres_out) {
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     uint4* xs = lds_raw;
@@ -487,18 +510,6 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     float* work = sx + cs_max;
     uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]
     float* red = reinterpret_cast<float*>(meta + 3 * kMetaWords);      // [16]
-
-    XcdSync sync;
-    sync.ctl = a.ctl;
-    // Workgroups are dealt to the XCDs round-robin, starting wherever the previous dispatch stopped: the XCD is
-    // read from the hardware, and workgroups i and i + 8 land on the same XCD, so i / 8 numbers the 64 blocks of
-    // each XCD.  (Were the dealing ever different, two blocks would share a flag word, a hand-over wait would
-    // run into its spin limit and the launch would report it.)
-    sync.xcd = xcc_id() & (kXcds - 1);
-    sync.slot = blockIdx.x / kXcds;
-    sync.spin_limit = a.spin_limit;
-    sync.aborted = false;
-    sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t tid = threadIdx.x;
     constexpr bool streams = true;
 
@@ -520,7 +531,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     // Requested now, behind the input: the groups' scales and biases and the first pass of gate / up -- a few
     // KiB per CU.  The later passes stream while the earlier ones are consumed; the down_proj slice is queued
     // behind the last of them.
-    input_request(a.in, inr);
+    input_request<TOKEN>(a.in, inr, xres_in);
     tile_pos_init<NLA, kBlock>(a.gate, tg, tid, pg);
     tile_pos_init<NLB, kBlock>(a.down, td, tid, pd);
     meta_fetch<KIND, kBlock, true>(a.gate, tg, tid, mg);
@@ -528,8 +539,9 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     tile_load<KIND, NLA, kBlock>(a.gate, tg, pg, rg);
     tile_load<KIND, NLA, kBlock>(a.up, tg, pg, ru);
     FK_XCD_STAMP(1, 1);
-    input_stage<KIND, 1>(a.in, inr, xs, sx, a.gate.cpr, red);
+    input_stage<KIND, 1>(a.in, inr, xs, sx, a.gate.cpr, red, xres_out);
     FK_XCD_STAMP(1, 5);
+    input_clear<TOKEN>(a.in);
     meta_store<KIND, kBlock, true>(mg, tid, meta);
     meta_store<KIND, kBlock, true>(mu, tid, meta + kMetaWords);
     meta_fetch<KIND, kBlock, true>(a.down, td, tid, md, sync.xcd);  // not needed before the hand-over: kept off the start-up path
@@ -572,12 +584,34 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs 
     FK_XCD_STAMP(1, 11);
 }
 
+// Workgroups are dealt to the XCDs round-robin, starting wherever the previous dispatch stopped: the XCD is read
+// from the hardware, and workgroups i and i + 8 land on the same XCD, so i / 8 numbers the 64 blocks of each XCD.
+// (Were the dealing ever different, two blocks would share a flag word, a hand-over wait would run into its spin
+// limit and the launch would report it.)
+__device__ __forceinline__ XcdSync xcd_sync_init(XcdControl* ctl, uint32_t spin_limit) {
+    XcdSync sync;
+    sync.ctl = ctl;
+    sync.xcd = xcc_id() & (kXcds - 1);
+    sync.slot = blockIdx.x / kXcds;
+    sync.spin_limit = spin_limit;
+    sync.aborted = false;
+    sync.epoch = __hip_atomic_load(ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return sync;
+}
+
+template <WKind KIND, int NLA, int NLB>
+__global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
+    xcd_mlp_phase<KIND, NLA, NLB, false>(a, sync, lds_raw, nullptr, nullptr);
+}
+
 // =============================================================================================== attention launch
 constexpr int kAttnStream = kBlock;
 
-template <WKind KIND, int NLA, int NLB>
-__global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a) {
-    extern __shared__ uint4 lds_raw[];
+template <WKind KIND, int NLA, int NLB, bool TOKEN, typename ARGS>
+__device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uint4* lds_raw, const uint4* xres_in,
+                                               uint4* xres_out) {
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats, att_elems = a.att_elems;
     (void)att_elems;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
@@ -587,13 +621,6 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]; two used
     uint16_t* att = reinterpret_cast<uint16_t*>(meta + 3 * kMetaWords);
 
-    XcdSync sync;
-    sync.ctl = a.ctl;
-    sync.xcd = xcc_id() & (kXcds - 1);   // see xcd_mlp_kernel
-    sync.slot = blockIdx.x / kXcds;
-    sync.spin_limit = a.spin_limit;
-    sync.aborted = false;
-    sync.epoch = __hip_atomic_load(a.ctl->flags + sync.xcd * kXcdSlots + sync.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t kv_len0 = *a.sdpa.kv_len_ptr;
     const uint32_t tid = threadIdx.x, ti = tid;
     constexpr bool streams = true;
@@ -608,7 +635,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     const uint32_t part_rows = part_id == 0 ? a.q_rows : a.kv_rows;
     const uint32_t pr0 = tl * R;
     const uint32_t pr_n = has_tile ? ((part_rows - pr0) < R ? (part_rows - pr0) : R) : 0u;
-    const XcdMat& mq = part_id == 0 ? a.wq : (part_id == 1 ? a.wk : a.wv);
+    const auto& mq = part_id == 0 ? a.wq : (part_id == 1 ? a.wk : a.wv);
     const Tile tq = make_tile(sync.xcd * part_rows + pr0, pr_n, 0, a.wq.cpr);
     const uint32_t o0 = sync.slot * a.o_rows;
     const uint32_t o_n = o0 < a.in.hidden ? ((a.in.hidden - o0) < a.o_rows ? (a.in.hidden - o0) : a.o_rows) : 0u;
@@ -620,14 +647,15 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     TilePos<NLA> pq;
     TilePos<NLB> po;
     InputRegs inr;
-    input_request(a.in, inr);
+    input_request<TOKEN>(a.in, inr, xres_in);
     tile_pos_init<NLA, kAttnStream>(mq, tq, ti, pq);
     tile_pos_init<NLB, kAttnStream>(a.wo, to, ti, po);
     meta_fetch<KIND, kAttnStream, true>(mq, tq, ti, mmq);
     tile_load<KIND, NLA, kAttnStream>(mq, tq, pq, rq);
     FK_XCD_STAMP(0, 1);
-    input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red);
+    input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red, xres_out);
     FK_XCD_STAMP(0, 5);
+    input_clear<TOKEN>(a.in);
     meta_store<KIND, kAttnStream, true>(mmq, ti, meta);
     meta_fetch<KIND, kAttnStream, true>(a.wo, to, ti, mmo, sync.xcd);  // not needed before the attention is done
     __syncthreads();
@@ -654,7 +682,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     {
         const uint32_t gz = sync.slot % G, split = sync.slot / G;
         if (split < a.sdpa.n_splits)
-            sdpa_block<1, 2, SdpaArgs, 0, true, true>(a.sdpa, kv_len0, split, sync.xcd, gz, G, work);
+            sdpa_block<1, 2, std::remove_cv_t<std::remove_reference_t<decltype((a.sdpa))>>, 0, true, true>(a.sdpa, kv_len0, split, sync.xcd, gz, G, work);
     }
     FK_XCD_STAMP(0, 8);
     xcd_barrier<0>(sync);
@@ -736,6 +764,107 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a
     FK_XCD_STAMP(0, 12);
 }
 
+template <WKind KIND, int NLA, int NLB>
+__global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
+    xcd_attn_phase<KIND, NLA, NLB, false>(a, sync, lds_raw, nullptr, nullptr);
+}
+
+// ---- the whole token in one launch --------------------------------------------------------------------------
+// Device-wide barrier in two levels: every block publishes its arrival word as in a hand-over; the leader block of
+// each XCD (slot 0) waits for its 64 blocks, adds one to `arrivals` (a memory-side add) and waits until all eight
+// leaders have (L1-bypassing loads see memory-side additions), then releases its XCD through `release[xcd]`, which
+// the other 63 blocks poll.  Counters only grow; every wait is bounded.  Returns false after an abort.
+struct XcdGlobalSync {
+    uint32_t arrivals_base, release_base, k;
+};
+__device__ __forceinline__ XcdGlobalSync xcd_global_init(const XcdSync& s) {
+    XcdGlobalSync g;
+    // a fast leader may already have arrived at the first barrier: it completes only with all eight, so the count
+    // read here lies within 7 of the last completed multiple of 8
+    g.arrivals_base = __hip_atomic_load(&s.ctl->arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & ~7u;
+    g.release_base = __hip_atomic_load(&s.ctl->release[s.xcd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    g.k = 0;
+    return g;
+}
+__device__ __forceinline__ bool xcd_global_barrier(XcdSync& s, XcdGlobalSync& g) {
+    s.epoch += 1;
+    g.k += 1;
+    wait_memory_ops_done();
+    __syncthreads();
+    if (threadIdx.x < (uint32_t)kWave) {
+        const uint32_t lane = threadIdx.x;
+        bool ok = true;
+        if (s.slot == 0) {
+            ok = xcd_publish_and_wait(s, lane);
+            if (ok) {
+                if (lane == 0) (void)__hip_atomic_fetch_add(&s.ctl->arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t target = g.arrivals_base + kXcds * g.k;
+                uint32_t spins = 0;
+                for (;;) {
+                    const uint32_t v = __hip_atomic_load(&s.ctl->arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if ((int32_t)(v - target) >= 0) break;
+                    if (++spins > s.spin_limit || ((spins & 255u) == 0u &&
+                                                   __hip_atomic_load(&s.ctl->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+                        if (lane == 0) __hip_atomic_store(&s.ctl->abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        ok = false;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            // released also after a failure, so that the XCD's blocks leave their wait at once and see the abort word
+            if (lane == 0) __hip_atomic_store(&s.ctl->release[s.xcd], g.release_base + g.k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+            if (lane == 0) __hip_atomic_store(s.ctl->flags + s.xcd * kXcdSlots + s.slot, s.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t target = g.release_base + g.k;
+            uint32_t spins = 0;
+            for (;;) {
+                const uint32_t v = __hip_atomic_load(&s.ctl->release[s.xcd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((int32_t)(v - target) >= 0) break;
+                if (++spins > s.spin_limit) {
+                    if (lane == 0) __hip_atomic_store(&s.ctl->abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+    }
+    __syncthreads();
+    return __hip_atomic_load(&s.ctl->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u;
+}
+
+template <WKind KIND, int NLQ, int NLO, int NLG, int NLD>
+__global__ __launch_bounds__(kBlock, 2) void xcd_token_kernel(const XcdTokenArgs t) {
+    extern __shared__ uint4 lds_raw[];
+    uint4* xres = lds_raw + t.xres_off;
+    XcdSync sync = xcd_sync_init(t.ctl, t.spin_limit);
+    XcdGlobalSync gs = xcd_global_init(sync);
+    // The argument blocks never change while the kernel runs: read through the constant address space, every field
+    // is a scalar load, as for kernel arguments.
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((address_space(4))) XcdAttnArgs ConstAttn;
+    typedef __attribute__((address_space(4))) XcdMlpArgs ConstMlp;
+#else
+    typedef XcdAttnArgs ConstAttn;
+    typedef XcdMlpArgs ConstMlp;
+#endif
+    // The next phase's argument block is pulled into this XCD's L2 while the current phase runs (one request per
+    // 64 bytes by a few lanes), so that its scalar loads do not start the phase with a trip to memory.
+    auto touch = [&](const void* p, uint32_t bytes) {
+        if (threadIdx.x * 64u < bytes) (void)*reinterpret_cast<const volatile uint32_t*>(reinterpret_cast<const char*>(p) + threadIdx.x * 64u);
+    };
+    for (uint32_t l = 0; l < t.n_layers; ++l) {
+        touch(t.mlp + l, sizeof(XcdMlpArgs));
+        xcd_attn_phase<KIND, NLQ, NLO, true>(*(const ConstAttn*)(t.attn + l), sync, lds_raw, l ? xres : nullptr, xres);
+        if (!xcd_global_barrier(sync, gs)) return;
+        if (l + 1 < t.n_layers) touch(t.attn + l + 1, sizeof(XcdAttnArgs));
+        xcd_mlp_phase<KIND, NLG, NLD, true>(*(const ConstMlp*)(t.mlp + l), sync, lds_raw, xres, xres);
+        if (l + 1 < t.n_layers && !xcd_global_barrier(sync, gs)) return;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= a.hidden) return;
@@ -769,6 +898,7 @@ fk_status xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint
 namespace {
 
 constexpr int kNlQkv = 6, kNlO = 4, kNlGu = 6, kNlDown = 6;  // 16-byte requests per streaming thread and pass
+constexpr int kNlGuToken = 4;  // the whole-token launch holds both phases' registers: shallower gate / up passes
 
 uint32_t ilog2u(uint32_t v) {
     uint32_t r = 0;
@@ -895,7 +1025,7 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
     LdsPlan lp;
     lp.cs_max = a.gate.cpr > a.down_cs ? a.gate.cpr : a.down_cs;
-    const uint32_t gu = 2 * padded(a.gu_rows * a.gate.cpr, kNlGu), dn = padded(a.down_rows * a.down_cs, kNlDown);
+    const uint32_t gu = 2 * padded(a.gu_rows * a.gate.cpr, rq.for_token ? kNlGuToken : kNlGu), dn = padded(a.down_rows * a.down_cs, kNlDown);
     lp.work_floats = gu > dn ? gu : dn;
     lp.att_elems = 0;
     const uint32_t lds = lds_for(s.bits, lp);
@@ -995,6 +1125,42 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     a.work_floats = lp.work_floats;
     a.att_elems = lp.att_elems;
     out->set_args(a);
+    return FK_OK;
+}
+
+fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uint32_t n_layers, uint32_t bits,
+                         const XcdAttnArgs* d_attn, const XcdMlpArgs* d_mlp, uint32_t attn_lds, uint32_t mlp_lds, Launch* out) {
+    if (!h_attn || !h_mlp || !d_attn || !d_mlp || n_layers == 0) return set_error(FK_ERR_INVALID, "xcd token: empty layer list");
+    for (uint32_t l = 0; l < n_layers; ++l) {
+        if (h_attn[l].ctl != h_attn[0].ctl || h_mlp[l].ctl != h_attn[0].ctl)
+            return set_error(FK_ERR_INVALID, "xcd token: every launch of the run must use the same control block");
+        if (h_attn[l].in.hidden != h_attn[0].in.hidden || h_mlp[l].in.hidden != h_attn[0].in.hidden)
+            return set_error(FK_ERR_INVALID, "xcd token: layers of different width");
+        for (uint32_t m = 0; m < l; ++m)
+            if (h_attn[l].q == h_attn[m].q || h_attn[l].k == h_attn[m].k || h_attn[l].v == h_attn[m].v)
+                return set_error(FK_ERR_UNSUPPORTED, "xcd token: every layer needs its own q / k / v rows inside one launch");
+    }
+    XcdTokenArgs t;
+    memset(&t, 0, sizeof(t));
+    t.attn = d_attn;
+    t.mlp = d_mlp;
+    t.n_layers = n_layers;
+    t.ctl = h_attn[0].ctl;
+    t.spin_limit = h_attn[0].spin_limit;
+    const uint32_t phase_lds = ((attn_lds > mlp_lds ? attn_lds : mlp_lds) + 15u) & ~15u;
+    t.xres_off = phase_lds / 16u;
+    const uint32_t lds = phase_lds + h_attn[0].in.hidden * 2u;
+    auto func = [&]() -> const void* {
+        if (bits == 4) return reinterpret_cast<const void*>(&xcd_token_kernel<W_Q4, kNlQkv, kNlO, kNlGuToken, kNlDown>);
+        if (bits == 8) return reinterpret_cast<const void*>(&xcd_token_kernel<W_Q8, kNlQkv, kNlO, kNlGuToken, kNlDown>);
+        return reinterpret_cast<const void*>(&xcd_token_kernel<W_BF16, kNlQkv, kNlO, kNlGuToken, kNlDown>);
+    };
+    out->func = func();
+    FK_TRY(set_lds_limit(out->func, lds));
+    out->grid = dim3(kXcdGrid, 1, 1);
+    out->block = dim3(kBlock, 1, 1);
+    out->shmem = lds;
+    out->set_args(t);
     return FK_OK;
 }
 

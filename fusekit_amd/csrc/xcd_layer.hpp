@@ -48,10 +48,14 @@ constexpr uint32_t kXcdMaxRanges = 16;              // key ranges merged per que
 // Control words of the protocol, one allocation per decoder (fk_xcd_workspace_bytes):
 //   flags[8][64]   uint32   arrival word of block (xcd, slot)
 //   abort          uint32   set when a wait ran into the spin limit
+//   arrivals       uint32   device-wide barrier of the whole-token launch: XCD leaders arrived (memory-side adds)
+//   release[8]     uint32   ... and the word each XCD's leader releases its XCD with
 struct XcdControl {
     uint32_t flags[kXcds * kXcdSlots];
     uint32_t abort_flag;
-    uint32_t pad[63];
+    uint32_t arrivals;
+    uint32_t release[kXcds];
+    uint32_t pad[54];
 };
 
 // A sum row: hidden 64-bit fixed-point sums (value * 2^32), padded to whole 512-element sections.  Inside a
@@ -124,6 +128,18 @@ struct XcdAttnArgs {
     uint32_t cs_max, work_floats, att_elems;  // LDS layout (att_elems: bf16 elements of the merged attention rows)
 };
 
+// Every layer of a token in ONE launch: the attention and MLP phases of the two kernels above, layer after layer,
+// with a device-wide barrier where the separate launches have a kernel boundary.  The per-layer argument blocks
+// (exactly what the separate launches take) sit in device memory.
+struct XcdTokenArgs {
+    const XcdAttnArgs* attn;   // [n_layers]
+    const XcdMlpArgs* mlp;     // [n_layers]
+    uint32_t n_layers;
+    XcdControl* ctl;
+    uint32_t spin_limit;
+    uint32_t xres_off;         // LDS offset (16-byte units) of the block's copy of the residual row
+};
+
 // x = T(f32(sums) + residual): the last layer's output for the LM head.  `clear` (may be the row read, or null)
 // is zeroed element by element behind the read: the row the next token's first launch adds into.
 struct XcdReduceArgs {
@@ -183,8 +199,15 @@ struct XcdMlpRequest {
     long long* out_sums;
     void* workspace;
     uint32_t spin_limit;
+    bool for_token;   // the block is meant for the whole-token launch (its gate / up passes are shallower)
 };
 fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out);
+// One launch for a run of alternating attention / MLP launches (as planned by plan_xcd_attn / plan_xcd_mlp, same
+// weight kind): `d_attn` / `d_mlp` are device copies of their argument blocks.  Requirements beyond the separate
+// launches': every layer has its own q / k / v rows (a block reads them with ordinary loads, and inside one launch
+// a line of the previous layer's row may still sit in its L1).
+fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uint32_t n_layers, uint32_t bits,
+                         const XcdAttnArgs* d_attn, const XcdMlpArgs* d_mlp, uint32_t attn_lds, uint32_t mlp_lds, Launch* out);
 fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
                           Launch* out);
 

@@ -47,6 +47,7 @@ class DecoderConfig:
     embed_scale: float = 1.0  # output_scale of the embedding lookup (embed_lookup_decode.rs:74-99)
     xcd_layers: bool = True   # graph mode: run a layer as two XCD-resident launches where the shape allows it
     xcd_spin_limit: int = 0   # bound of the XCD hand-over waits in polls (0: the library's default)
+    xcd_token_launch: bool = False  # the layers' launches of a token as ONE launch (device-wide barriers between them); slower at present
 
     @property
     def n_q(self) -> int:
@@ -225,6 +226,10 @@ class DecoderRuntime:
             self.xcd_ctl = z(ctl)
             self.xcd_att_partials = DeviceBuffer(ap)
             self.xcd_xa, self.xcd_xb = DeviceBuffer(cfg.hidden * 2), DeviceBuffer(cfg.hidden * 2)
+            # one launch per token: every layer needs its own q / k / v rows (read with ordinary loads inside the launch)
+            if cfg.xcd_token_launch:
+                self.xcd_qkv = [(DeviceBuffer(cfg.n_q * 2), DeviceBuffer(cfg.n_kvd * 2), DeviceBuffer(cfg.n_kvd * 2))
+                                for _ in range(cfg.n_layers)]
             # three rotating sum rows: a launch reads one, adds into the next and clears the third
             self.xcd_sums = [z(native.xcd_sum_row_bytes(cfg.hidden)) for _ in range(3)]
             # scales / biases of o_proj and down_proj, one contiguous copy per K-slice (once, at load time)
@@ -370,7 +375,7 @@ class DecoderRuntime:
         c, w = self.cfg, self.w
         shape = dict(hidden=c.hidden, inter=c.inter, n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim,
                      capacity=c.capacity, bits=c.bits, group=c.group, eps=c.eps, theta=c.theta,
-                     spin_limit=c.xcd_spin_limit)
+                     spin_limit=c.xcd_spin_limit, token_launch=int(c.xcd_token_launch))
         quant = c.bits != 16
         for l in range(c.n_layers):
             p = f"layers.{l}."
@@ -384,7 +389,8 @@ class DecoderRuntime:
             a += self._xcd_kslice_args(p + "self_attn.o_proj", Wo)
             if c.qk_norm:
                 a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
-            a += [arg(self.q), arg(self.k), arg(self.v), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+            q_, k_, v_ = self.xcd_qkv[l] if c.xcd_token_launch else (self.q, self.k, self.v)
+            a += [arg(q_), arg(k_), arg(v_), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
                   arg(self.rope_tab), arg(self.xcd_att_partials), S(2 * l + 1), S(2 * l + 2), arg(self.xcd_ctl)]
             t.append(Dispatch(name("xcd_attn_block"), a, dict(shape, has_sums=int(l > 0), has_norm=int(c.qk_norm))))
             Wg, Wu, Wd = (w.mats[p + f"mlp.{n}_proj"] for n in ("gate", "up", "down"))

@@ -123,10 +123,7 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
     bit-reproducible generator from the fixture's seeds; the host builds the same bytes (checked on two quantised
     tensors), applies the structure and uploads the few arrays it changes."""
     from fusekit_amd.moe_decoder import MoeConfig, MoeRuntime, MoeWeights
-    path = os.path.join(os.path.dirname(__file__), "golden", "clear_margin_moe.json")
-    if not os.path.exists(path):
-        pytest.skip("tests/golden/clear_margin_moe.json has not been produced yet (tests/golden/find_clear_margin_moe.py)")
-    fx = json.load(open(path))
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "clear_margin_moe.json")))
     cfg = MoeConfig(capacity=128)
     assert fx["n_layers"] == cfg.n_layers and len(fx["prompt"]) == 32 and len(fx["tokens"]) == 32
     kw = dict(seed=fx["model_seed"], std=fx["std"], embed_loud_rows=fx["loud_rows"], embed_loud_gain=fx["loud_gain"])
