@@ -44,7 +44,7 @@ SYMBOLS = {
     "xcd_attn_block": "xcd_attn_kernel<Q4>",
     "xcd_mlp_block": "xcd_mlp_kernel<Q4>",
     "xcd_reduce": "xcd_reduce_kernel",
-    "final_rmsnorm_lm_head": "gemv_stream_kernel<BF16, 1 segment>",
+    "final_rmsnorm_lm_head": "gemv_rows_kernel<BF16, batches of 5 column blocks>",
     "argmax_logits_decode": "argmax_kernel",
     "embed_lookup_decode": "embed_lookup_kernel",
     "step_init": "step_init_kernel",

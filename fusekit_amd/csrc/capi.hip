@@ -203,6 +203,13 @@ fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks) {
     return FK_OK;
 }
 
+int fk_gemv_form(uint32_t n, uint32_t k, uint32_t bits, uint32_t group) { return gemv_rows_batch(n, k, bits, group) ? 1 : 0; }
+
+fk_status fk_set_gemv_flat_only(int flat_only) {
+    g_gemv_policy.flat_only = flat_only != 0;
+    return FK_OK;
+}
+
 fk_status fk_qgemv(const fk_weight* W, const uint16_t* x, const uint16_t* bias, uint16_t* y, fk_stream s) {
     GemvRequest rq;
     rq.mats[0] = W;

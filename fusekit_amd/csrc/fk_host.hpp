@@ -60,8 +60,12 @@ fk_status run_launch(const Launch& l, hipStream_t s);
 // ---- planners (one per kernel family); each validates shapes on the host ----
 struct GemvPolicy {
     uint32_t rows_per_tile = 0, grid_blocks = 0;
+    bool flat_only = false;  // never pick the row-group form
 };
 extern GemvPolicy g_gemv_policy;
+// Column blocks per batch (3, 4 or 5) of the row-group GEMV form for one [n, k] matrix without bias or residual, or
+// 0 when the shape stays on the flat form.
+uint32_t gemv_rows_batch(uint32_t n, uint32_t k, uint32_t bits, uint32_t group);
 // When non-zero, plan_gemv on this thread sizes its tiles for exactly this many
 // blocks (the persistent whole-token kernel plans every phase for its own grid).
 extern thread_local uint32_t t_gemv_grid_override;

@@ -1,4 +1,6 @@
 // Launch planner and template instances of the flat-stream GEMV.
+#include <stdlib.h>
+
 #include <map>
 #include <mutex>
 
@@ -21,10 +23,16 @@ extern "C" __attribute__((visibility("default"))) int fk_probe_read_gemv_stamps(
 }
 #endif
 #include "gemv_kernel.hpp"
+#include "gemv_rows.hpp"
 
 namespace fk {
 
-GemvPolicy g_gemv_policy;
+GemvPolicy g_gemv_policy = [] {
+    GemvPolicy p;
+    const char* e = getenv("FUSEKIT_GEMV_FLAT_ONLY");  // "1": never pick the row-group form (measurements, tests)
+    p.flat_only = e && e[0] == '1';
+    return p;
+}();
 thread_local uint32_t t_gemv_grid_override = 0;
 
 namespace {
@@ -42,6 +50,40 @@ const void* select_gemv(WKind kind, bool swiglu) {
     }
 }
 
+template <WKind KIND, bool TAIL>
+const void* rows_func(uint32_t nb) {
+    switch (nb) {
+        case 3: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 3, TAIL>);
+        case 4: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 4, TAIL>);
+        default: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 5, TAIL>);
+    }
+}
+const void* rows_func(WKind kind, uint32_t nb, bool tail) {
+    switch (kind) {
+        case W_Q4: return tail ? rows_func<W_Q4, true>(nb) : rows_func<W_Q4, false>(nb);
+        case W_Q8: return tail ? rows_func<W_Q8, true>(nb) : rows_func<W_Q8, false>(nb);
+        default: return tail ? rows_func<W_BF16, true>(nb) : rows_func<W_BF16, false>(nb);
+    }
+}
+
+// Blocks of `func` one CU holds at once (registers and LDS decide); cached per (kernel, LDS bytes).
+uint32_t blocks_per_cu(const void* func, uint32_t lds_bytes) {
+    static std::mutex mu;
+    static std::map<std::pair<const void*, uint32_t>, int> cache;
+    std::lock_guard<std::mutex> lk(mu);
+    auto key = std::make_pair(func, lds_bytes);
+    auto it = cache.find(key);
+    if (it == cache.end()) {
+        if (lds_bytes > 48 * 1024)
+            (void)hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, func, kGemvBlock, lds_bytes) != hipSuccess || per_cu < 1)
+            per_cu = 1;
+        it = cache.emplace(key, per_cu).first;
+    }
+    return (uint32_t)it->second;
+}
+
 uint32_t ilog2(uint32_t v) {
     uint32_t r = 0;
     while ((1u << (r + 1)) <= v) ++r;
@@ -49,6 +91,28 @@ uint32_t ilog2(uint32_t v) {
 }
 
 }  // namespace
+
+// Shapes of the row-group form: rows of whole 256-byte blocks that the staging registers cover, group size 64,
+// 32-bit byte offsets into the matrix, and enough rows that every CU gets at least two blocks of four-row passes.
+// Batches of 5, 4 or 3 column blocks, whichever leaves the fewest unused slots in a row's last batch (at most 7 %).
+uint32_t gemv_rows_batch(uint32_t n, uint32_t k, uint32_t bits, uint32_t group) {
+    if (g_gemv_policy.flat_only || (bits != 4 && bits != 8 && bits != 16) || (bits != 16 && group != 64)) return 0;
+    const uint32_t values = bits == 4 ? 32u : (bits == 8 ? 16u : 8u);
+    if (k == 0 || k % values != 0) return 0;
+    const uint32_t cpr = k / values;
+    if (cpr % kRowLanes != 0 || k > (uint32_t)kStageRegs * kGemvBlock * 8u) return 0;
+    const DeviceFacts* dev;
+    if (device_facts(&dev) != FK_OK) return 0;
+    const uint64_t passes = ((uint64_t)n + kPassRows - 1) / kPassRows;
+    if (passes < 2ull * kBlockWaves * dev->cus || (uint64_t)n * cpr * 16ull > 0xffffffffull) return 0;
+    const uint32_t cpl = cpr / kRowLanes;
+    uint32_t nb = 0, best_slots = ~0u;
+    for (uint32_t c : {5u, 4u, 3u}) {
+        const uint32_t slots = (cpl + c - 1) / c * c;
+        if (slots < best_slots) best_slots = slots, nb = c;
+    }
+    return best_slots * 100u <= cpl * 107u ? nb : 0u;
+}
 
 fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     const DeviceFacts* dev;
@@ -81,6 +145,64 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     const uint32_t cpr = K / values;
     const uint32_t nseg = rq.swiglu ? 2u : 1u;
 
+    // Row-group form (gemv_rows.hpp): see gemv_rows_batch for the shapes.
+    const uint32_t rows_nb = (!rq.swiglu && nm == 1 && !t_gemv_grid_override && !g_gemv_policy.rows_per_tile && !rq.res &&
+                              !rq.res2 && !rq.bias[0])
+                                 ? gemv_rows_batch(rq.mats[0]->n, K, bits, bits == 16 ? 64 : group)
+                                 : 0u;
+    if (rows_nb) {
+        const uint32_t cpl = cpr / kRowLanes, nb = rows_nb;
+        const uint32_t mb = bits == 4 ? 16u : 8u;
+        bool ok = true;
+        const uint64_t passes = (rq.mats[0]->n + kPassRows - 1) / kPassRows;
+        if (bits != 16 && (((uintptr_t)rq.mats[0]->scales | (uintptr_t)rq.mats[0]->biases) & (mb - 1)) != 0) ok = false;
+        if (((uintptr_t)rq.mats[0]->w & 15u) != 0) ok = false;
+        const uint32_t lds = kind == W_Q4 ? gemv_rows_lds_bytes<W_Q4>(cpr)
+                             : (kind == W_Q8 ? gemv_rows_lds_bytes<W_Q8>(cpr) : gemv_rows_lds_bytes<W_BF16>(cpr));
+        if (ok && (int)lds <= dev->max_dyn_lds) {
+            const void* f = rows_func(kind, nb, cpl % nb != 0);
+            // whole rounds: every wave of the grid gets the same number of passes (to within one)
+            const uint64_t cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : (uint64_t)blocks_per_cu(f, lds) * dev->cus;
+            const uint64_t block_passes = (passes + kBlockWaves - 1) / kBlockWaves;
+            const uint64_t rounds = (block_passes + cap - 1) / cap;
+            const uint64_t blocks = (block_passes + rounds - 1) / rounds;
+            GemvArgs a;
+            memset(&a, 0, sizeof(a));
+            uint32_t t0 = 0;
+            for (int m = 0; m < nm; ++m) {
+                a.w[m] = reinterpret_cast<const uint4*>(rq.mats[m]->w);
+                a.sc[m] = rq.mats[m]->scales;
+                a.bi[m] = rq.mats[m]->biases;
+                a.bias[m] = rq.bias[m];
+                a.y[m] = rq.y[m];
+                a.n[m] = rq.mats[m]->n;
+                a.tile_start[m] = t0;
+                t0 += (rq.mats[m]->n + kPassRows - 1) / kPassRows;
+            }
+            a.tile_start[nm] = t0;
+            a.n_mats = nm;
+            a.K = K;
+            a.cpr = cpr;
+            a.gshift = bits == 16 ? 0 : ilog2(group / values);
+            a.R = kPassRows;
+            a.n_tiles = (uint32_t)passes;
+            a.lr = kRowLanes;
+            a.inv_cpr = 1.0f / (float)cpr;
+            a.x = rq.x;
+            a.norm_w = rq.norm_w;
+            a.eps = rq.eps;
+            a.res = rq.res;
+            a.res2 = rq.res2;
+            a.y_scale = 1.0f;
+            out->func = f;
+            out->grid = dim3((uint32_t)blocks, 1, 1);
+            out->block = dim3(kGemvBlock, 1, 1);
+            out->shmem = lds;
+            out->set_args(a);
+            if (lds > 48 * 1024) FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            return FK_OK;
+        }
+    }
     const void* func = select_gemv(kind, rq.swiglu);
     auto tiles_for = [&](uint32_t r) {
         uint64_t t = 0;
@@ -99,23 +221,7 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     // exceeds it, so no block waits for a slot and then pays the whole start-up chain
     // (stage x, first loads) a second time; surplus tiles go to the persistent loop,
     // whose next batch is already in flight while the current one is consumed.
-    auto resident_for = [&](uint32_t lds_bytes) -> uint32_t {
-        static std::mutex mu;
-        static std::map<std::pair<const void*, uint32_t>, int> cache;
-        std::lock_guard<std::mutex> lk(mu);
-        auto key = std::make_pair(func, lds_bytes);
-        auto it = cache.find(key);
-        if (it == cache.end()) {
-            if (lds_bytes > 48 * 1024)
-                (void)hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            int per_cu = 0;
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, func, kGemvBlock, lds_bytes) != hipSuccess ||
-                per_cu < 1)
-                per_cu = 1;
-            it = cache.emplace(key, per_cu).first;
-        }
-        return (uint32_t)it->second * (uint32_t)dev->cus;
-    };
+    auto resident_for = [&](uint32_t lds_bytes) -> uint32_t { return blocks_per_cu(func, lds_bytes) * (uint32_t)dev->cus; };
 
     // Rows per tile.  A batch (4 x 16-byte loads per lane) costs the same whether its
     // lanes are full or not, and the blocks resident on a CU share its issue slots, so

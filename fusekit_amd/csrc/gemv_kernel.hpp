@@ -168,7 +168,13 @@ __device__ __forceinline__ void stage_fetch(const ARGS& a, uint4 (&xr)[kStageReg
     }
 }
 
-template <WKind KIND, typename ARGS>
+// BLOCKED: the layout of the row-group kernel (gemv_rows.hpp): piece j of chunk c at uint4 index
+// ((c / 16) * PIECES + j) * 16 + c % 16, so that the 16 lanes sharing a row read 256 contiguous bytes and a
+// chunk's pieces sit at fixed distances from each other.
+// SHORT: the caller guarantees K <= kStageRegs * kGemvBlock * 8, so the loops over the rest of a long row are
+// left out (their loads, conditional and issued after the caller's prefetch, blur the compiler's account of which
+// registers still have a load outstanding).
+template <WKind KIND, typename ARGS, bool BLOCKED = false, bool SHORT = false>
 __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, float* sx, float* scratch,
                                                   uint4 (&xr)[kStageRegs], uint4 (&wr)[kStageRegs]) {
     const bool NORM = a.norm_w != nullptr;  // uniform; one code path serves both
@@ -190,7 +196,8 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
 #pragma unroll
         for (int i = 0; i < kStageRegs; ++i)
             if (threadIdx.x + i * kGemvBlock < n8) add_sq(xr[i]);
-        for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8; t += kGemvBlock) add_sq(x8[t]);
+        if constexpr (!SHORT)
+            for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8; t += kGemvBlock) add_sq(x8[t]);
         FK_GEMV_STAMP(5);
         ss = block_sum<kGemvBlock>(ss, scratch);
         r = 1.0f / sqrtf(ss / (float)K + a.eps);
@@ -220,7 +227,8 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
             // word j of chunk c; activation pairs (0,2) (4,6) (1,3) (5,7) as q4_word_dot wants
             const uint32_t c = t >> 2, j = t & 3u;
             if (live)
-                xs[j * cpr + c] = make_uint4(__builtin_amdgcn_perm(nb[1], nb[0], 0x05040100u),
+                xs[BLOCKED ? ((c >> 4) * 4 + j) * 16 + (c & 15u) : j * cpr + c] =
+                                  make_uint4(__builtin_amdgcn_perm(nb[1], nb[0], 0x05040100u),
                                              __builtin_amdgcn_perm(nb[3], nb[2], 0x05040100u),
                                              __builtin_amdgcn_perm(nb[1], nb[0], 0x07060302u),
                                              __builtin_amdgcn_perm(nb[3], nb[2], 0x07060302u));
@@ -229,10 +237,11 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
         } else if constexpr (KIND == W_Q8) {
             const uint32_t c = t >> 1, j = (t & 1u) * 2u;
             if (live) {
-                xs[j * cpr + c] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
-                                             __float_as_uint(f[3]));
-                xs[(j + 1) * cpr + c] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]),
-                                                   __float_as_uint(f[6]), __float_as_uint(f[7]));
+                const uint32_t at = BLOCKED ? ((c >> 4) * 4 + j) * 16 + (c & 15u) : j * cpr + c;
+                xs[at] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                                    __float_as_uint(f[3]));
+                xs[at + (BLOCKED ? 16u : cpr)] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]),
+                                                            __float_as_uint(f[6]), __float_as_uint(f[7]));
             }
             s8 = group_sum(s8, 2);
             if (live && j == 0) sx[c] = s8;
@@ -246,14 +255,16 @@ __device__ __forceinline__ void stage_activations(const ARGS& a, uint4* xs, floa
         if ((threadIdx.x & ~(uint32_t)(kWave - 1)) + i * kGemvBlock < n8) emit(threadIdx.x + i * kGemvBlock, xr[i], wr[i]);
     // long rows: the rest is fetched again (whole waves stay in the loop so the
     // butterflies above see all their lanes)
-    const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
-    for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8_up; t += kGemvBlock) {
-        uint4 v = make_uint4(0, 0, 0, 0), wv = make_uint4(0, 0, 0, 0);
-        if (t < n8) {
-            v = x8[t];
-            if (NORM) wv = w8[t];
+    if constexpr (!SHORT) {
+        const uint32_t n8_up = (n8 + kWave - 1) / kWave * kWave;
+        for (uint32_t t = threadIdx.x + kStageRegs * kGemvBlock; t < n8_up; t += kGemvBlock) {
+            uint4 v = make_uint4(0, 0, 0, 0), wv = make_uint4(0, 0, 0, 0);
+            if (t < n8) {
+                v = x8[t];
+                if (NORM) wv = w8[t];
+            }
+            emit(t, v, wv);
         }
-        emit(t, v, wv);
     }
     FK_GEMV_STAMP(7);
     __syncthreads();

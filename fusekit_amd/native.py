@@ -552,6 +552,15 @@ def set_gemv_policy(rows_per_tile: int = 0, grid_blocks: int = 0) -> None:
     check(lib.fk_set_gemv_policy(C.c_uint32(rows_per_tile), C.c_uint32(grid_blocks)))
 
 
+def gemv_form(n: int, k: int, bits: int, group: int = 64) -> int:
+    """1 when a plain GEMV over an [n, k] matrix runs the row-group kernel form, 0 for the flat stream."""
+    return int(lib.fk_gemv_form(C.c_uint32(n), C.c_uint32(k), C.c_uint32(bits), C.c_uint32(group)))
+
+
+def set_gemv_flat_only(flat_only: bool) -> None:
+    check(lib.fk_set_gemv_flat_only(C.c_int(1 if flat_only else 0)))
+
+
 def sync(stream=None) -> None:
     check(lib.fk_stream_sync(_ptr(stream)))
 

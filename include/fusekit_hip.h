@@ -664,6 +664,14 @@ fk_status fk_decode_chunk_host_loop(fk_handle h, uint32_t graph_id, const fk_dec
 /* Launch-geometry overrides for experiments (0 = library policy): rows per
  * tile and grid blocks of the streaming GEMV.  Process-wide. */
 fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks);
+/* The streaming GEMV has two kernel forms: the flat stream (any K that is a multiple of 64, fused epilogues, up to
+ * three matrices) and the row-group form (sixteen lanes per row, one accumulator per lane; a single matrix without
+ * bias or residual whose rows are whole 256-byte blocks, group size 64, K <= 10240, at least eight rows per
+ * compute unit pair).  fk_gemv_form answers which one a plain fk_qgemv / fk_final_rmsnorm_lm_head over an
+ * [n, k] matrix would run: 1 = row-group, 0 = flat.  fk_set_gemv_flat_only(1) keeps every launch planned from then
+ * on on the flat form (measurements, tests); 0 restores the library's choice.  Process-wide. */
+int fk_gemv_form(uint32_t n, uint32_t k, uint32_t bits, uint32_t group);
+fk_status fk_set_gemv_flat_only(int flat_only);
 /* Row count from which fk_qgemm / fk_qgemm_swiglu dequantise the matrix to bf16 once and hand the
  * product to rocBLAS (opened on first use; absent: the fused kernel is kept).  Default 256; 0 = never.
  * Set it BEFORE sizing workspaces: fk_qgemm_workspace_bytes covers the route that will be taken. */

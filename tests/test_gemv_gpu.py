@@ -78,6 +78,59 @@ def test_qgemv_vocab_sized_matches_oracle(fk):
     _check(dy.to_numpy(np.uint16), oracle.qgemv(W, x), oracle.linear_acc(W, x), W, x)
 
 
+# Shapes of the row-group kernel form (sixteen lanes per row, four rows per wave and pass): batches of 5, 4 and 3
+# column blocks, rows whose last batch has unused slots (9728 / int4: 19 column blocks in batches of 5; 9728 / int8:
+# 38 in batches of 3; 2432 / bf16: 19 in batches of 5), a row count that is not a multiple of four.
+ROW_GROUP_SHAPES = [
+    (8201, 2560, 4), (8201, 9728, 4), (8196, 4096, 4), (8202, 2048, 8), (8201, 9728, 8), (8201, 2560, 16),
+    (8199, 1536, 16), (8203, 2432, 16), (8201, 1536, 4),
+]
+
+
+@pytest.mark.parametrize("n,k,bits", ROW_GROUP_SHAPES)
+def test_qgemv_row_group_form_matches_oracle_and_flat_form(fk, n, k, bits):
+    assert fk.gemv_form(n, k, bits) == 1, "the planner is expected to pick the row-group form for this shape"
+    W = make_qweight(300 + n + k, n, k, bits)
+    x = normal_bf16(17, k)
+    dW, dx = to_device(fk, W), fk.DeviceBuffer.from_numpy(x)
+    dy = fk.DeviceBuffer(2 * n)
+    fk.qgemv(dW, dx, None, dy)
+    got = dy.to_numpy(np.uint16)
+    _check(got, oracle.qgemv(W, x), oracle.linear_acc(W, x), W, x)
+    # the flat form on the same operands: both forms share every rounding boundary and differ in summation order only
+    fk.set_gemv_flat_only(True)
+    try:
+        assert fk.gemv_form(n, k, bits) == 0
+        dz = fk.DeviceBuffer(2 * n)
+        fk.qgemv(dW, dx, None, dz)
+    finally:
+        fk.set_gemv_flat_only(False)
+    flat = dz.to_numpy(np.uint16)
+    _check(got, flat, oracle.bf16_to_f32(flat), W, x)
+
+
+def test_row_group_form_with_fused_final_norm(fk):
+    hidden, vocab = 2560, 20011
+    assert fk.gemv_form(vocab, hidden, 4) == 1
+    W = make_qweight(61, vocab, hidden, 4)
+    x = normal_bf16(1, hidden, 3.0)
+    gamma = normal_bf16(2, hidden, 0.1, 1.0)
+    dl = fk.DeviceBuffer(2 * vocab)
+    fk.final_rmsnorm_lm_head(fk.DeviceBuffer.from_numpy(x), fk.DeviceBuffer.from_numpy(gamma), 1e-6,
+                             to_device(fk, W), dl)
+    ref = oracle.final_rmsnorm_lm_head(x, gamma, 1e-6, W)
+    ny = oracle.rmsnorm(x, gamma, 1e-6)
+    _check(dl.to_numpy(np.uint16), ref, oracle.linear_acc(W, ny), W, ny)
+
+
+def test_row_group_form_is_kept_for_the_shapes_it_was_built_for(fk):
+    assert fk.gemv_form(151936, 2560, 4) == 1 and fk.gemv_form(151936, 2560, 16) == 1
+    assert fk.gemv_form(2560, 2560, 4) == 0          # too few rows to fill the chip four rows a wave
+    assert fk.gemv_form(20000, 896, 4) == 0          # rows are not whole 256-byte blocks
+    assert fk.gemv_form(20000, 2560, 4, 32) == 0     # group size
+    assert fk.gemv_form(20000, 12288, 4) == 0        # longer than the staging registers cover
+
+
 @pytest.mark.parametrize("group", [32, 128])
 @pytest.mark.parametrize("bits", [4, 8])
 def test_qgemv_other_group_sizes(fk, bits, group):
