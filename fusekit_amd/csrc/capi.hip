@@ -53,6 +53,7 @@ fk_status device_facts(const DeviceFacts** out) {
 }
 
 fk_status run_launch(const Launch& l, hipStream_t s) {
+    if (!l.func) return FK_OK;  // an empty launch (a planner that needed fewer kernels than its caller offers)
     void* params[1] = {const_cast<unsigned char*>(l.args)};
     FK_HIP(hipLaunchKernel(l.func, l.grid, l.block, params, l.shmem, s));
     for (const Launch& f : l.then) FK_TRY(run_launch(f, s));
@@ -189,6 +190,11 @@ fk_status fk_event_elapsed_ms(fk_event start, fk_event stop, float* ms) {
     if (!start || !stop || !ms) return set_error(FK_ERR_INVALID, "null event or out pointer");
     FK_HIP(hipEventSynchronize((hipEvent_t)stop));
     FK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return FK_OK;
+}
+
+fk_status fk_set_qgemm_wide(int enabled) {
+    set_qgemm_wide(enabled != 0);
     return FK_OK;
 }
 

@@ -1082,7 +1082,7 @@ fk_status plan_qgemm_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(plan_qgemm(&W, arg_ptr<const uint16_t>(d, 0), rows, has_bias ? arg_ptr<const uint16_t>(d, bias_slot) : nullptr,
                       has_res ? arg_ptr<const uint16_t>(d, res_slot) : nullptr, arg_ptr<uint16_t>(d, out_slot),
                       d.args[ws_slot].ptr, l, &reduce));
-    l->then.push_back(reduce);
+    if (reduce.func) l->then.push_back(reduce);
     return FK_OK;
 }
 
@@ -1106,8 +1106,8 @@ fk_status plan_qgemm_swiglu_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     Launch up, reduce;
     FK_TRY(plan_qgemm_swiglu(&Wg, &Wu, arg_ptr<const uint16_t>(d, 0), rows, (int)d.param("variant", 2),
                              arg_ptr<uint16_t>(d, 7), d.args[8].ptr, l, &up, &reduce));
-    l->then.push_back(up);
-    l->then.push_back(reduce);
+    if (up.func) l->then.push_back(up);
+    if (reduce.func) l->then.push_back(reduce);
     return FK_OK;
 }
 

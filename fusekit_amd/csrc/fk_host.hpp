@@ -127,6 +127,13 @@ fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint
 void set_gemm_library_rows(uint32_t rows);  // 0: never
 fk_status run_dequantize_bf16(const fk_weight* W, uint16_t* out, hipStream_t s);
 bool qgemm_takes_library(uint32_t m);
+// 2..10 activation rows at group size 64 run the shared-stream kernel (qgemm_wide.hip): one launch, epilogue
+// included.  plan_qgemm / plan_qgemm_swiglu then leave their other launches empty (func == nullptr), which
+// run_launch and the graph builder skip.
+bool qgemm_takes_wide(uint32_t M, uint32_t group);
+void set_qgemm_wide(bool on);
+fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16_t* x, uint32_t M, const uint16_t* bias,
+                          const uint16_t* res, int variant, uint16_t* y, Launch* out);
 bool gemm_library_available();
 size_t qgemm_library_sums_bytes(uint32_t m, uint32_t n, uint32_t k);
 size_t qgemm_library_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);

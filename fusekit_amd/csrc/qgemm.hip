@@ -470,6 +470,10 @@ fk_status plan_qgemm(const fk_weight* W, const uint16_t* x, uint32_t M, const ui
     FK_TRY(device_facts(&dev));
     FK_TRY(check_weight(W, "qgemm"));
     if (!x || !y || !workspace) return set_error(FK_ERR_INVALID, "qgemm: null activation, output or workspace");
+    if (qgemm_takes_wide(M, W->group)) {  // 2..10 rows: one launch, no split-k sums (reduce stays empty)
+        *reduce = Launch();
+        return plan_qgemm_wide(W, nullptr, x, M, bias, res, 0, y, main);
+    }
     QgemmShape s;
     FK_TRY(plan_qgemm_main(dev, W, x, M, static_cast<float*>(workspace), &s, main));
     plan_reduce(static_cast<float*>(workspace), nullptr, bias, res, y, M, W->n, s.ksplit, 0, reduce);
@@ -486,6 +490,11 @@ fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint
         return set_error(FK_ERR_INVALID, "qgemm_swiglu: gate and up need the same shape and group size");
     if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, "qgemm_swiglu: variant must be 0, 1 or 2");
     if (!x || !out || !workspace) return set_error(FK_ERR_INVALID, "qgemm_swiglu: null activation, output or workspace");
+    if (qgemm_takes_wide(M, Wg->group)) {  // 2..10 rows: gate, up and SwiGLU in one launch (up, reduce stay empty)
+        *up = Launch();
+        *reduce = Launch();
+        return plan_qgemm_wide(Wg, Wu, x, M, nullptr, nullptr, variant, out, gate);
+    }
     QgemmShape s;
     float* p0 = static_cast<float*>(workspace);
     FK_TRY(plan_qgemm_main(dev, Wg, x, M, p0, &s, gate));

@@ -1,0 +1,345 @@
+// Shared-stream matmul for 2 .. 10 activation rows: y[M, N] = epilogue(x[M, K] @ dequant(W)^T) in ONE launch,
+// the weight matrix read once for all rows.  Replaces the reference's small-M kernels (fusekit_qmv_wide_impl,
+// src/codegen/msl.rs:462-546; fusekit_qmv_fast_m_impl, :1307-1485; policy kernels/mod.rs:164-186: 2..10 rows,
+// group 64, 4 or 8 bits) -- there up to five activation vectors share a dequantised weight fragment in
+// registers and the stream is read ceil(M / 5) times; here the ten rows share it through the matrix cores and
+// the stream is read once.
+//
+// Same arithmetic as the exact form of qgemm_kernel (qgemm.hip): the integer codes go into
+// v_mfma_f32_32x32x16_bf16 as exact bf16 values with the WEIGHTS as the B operand, the integer dot of a
+// quantisation group is accumulated in a zeroed C tile and folded into the fp32 accumulators as
+// s * dot + b * Sx(row, group).  What differs is the cut: a block owns 32 weight rows over ALL of K and its
+// waves (4 or 8) split K between them in slabs of 256, so there is no split-k workspace and no second kernel --
+// the waves' accumulators meet in LDS, are added in wave order, and the epilogue (bias, residual, or SwiGLU of a
+// gate / up pair streamed side by side) runs in the same launch.  Every wave stages the activation slab it is
+// about to use in its OWN piece of LDS (M <= 10 rows x 256 k = 5 KB; LDS operations of one wave execute in order),
+// so the main loop has no block barrier at all; rows 10 .. 31 of the matrix operand read one zero row.
+// Matrices with few rows run eight waves per block instead of four (N / 32 blocks of four waves would leave most
+// of the chip without a wave).
+#include "fk_host.hpp"
+#include "gemv_kernel.hpp"
+
+#ifdef FK_PROBE_STAMPS
+// Timing-probe build only: clocks of the first wave of every block at the phase boundaries.
+__device__ unsigned long long g_fk_wide_stamp[2048 * 8];
+#define FK_WIDE_STAMP(i)                                                                                  \
+    do {                                                                                                  \
+        if (threadIdx.x == 0 && blockIdx.x < 2048) g_fk_wide_stamp[blockIdx.x * 8 + (i)] = wall_clock64(); \
+    } while (0)
+extern "C" __attribute__((visibility("default"))) int fk_probe_read_wide_stamps(unsigned long long* out) {
+    const size_t bytes = sizeof(unsigned long long) * 2048 * 8;
+    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fk_wide_stamp), bytes);
+    if (e != hipSuccess) return (int)e;
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_fk_wide_stamp));
+    return (int)(e != hipSuccess ? e : hipMemset(p, 0, bytes));
+}
+#else
+#define FK_WIDE_STAMP(i)
+#endif
+
+namespace fk {
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kWideMaxRows = 10;             // activation rows (the reference's upper bound for this path)
+constexpr uint32_t kWideSlab = 256;               // k per wave and step
+constexpr uint32_t kWideXS = kWideSlab / 8 + 1;   // uint4 per staged activation row (+1: bank spread)
+constexpr uint32_t kWideXRows = kWideMaxRows + 1; // staged rows + the zero row
+constexpr int kWideXPT = kWideMaxRows * (kWideSlab / 8) / kWave;  // 16-byte pieces of x per lane and slab
+
+struct QgemmWideArgs {
+    const uint4* w[2];
+    const uint16_t* sc[2];
+    const uint16_t* bi[2];
+    const uint16_t* x;     // [M, K] bf16
+    const uint16_t* bias;  // [N] or null (single matrix)
+    const uint16_t* res;   // [M, N] or null (single matrix)
+    uint16_t* y;           // [M, N]
+    uint32_t M, N, K;
+    uint32_t cpr, gpr;
+    int variant;           // SwiGLU rounding variant (pair)
+};
+
+// LDS per wave: staged activations [kWideXRows][kWideXS] uint4, group sums [4][32] floats; per block
+// additionally the waves' results [waves][mats][kWideMaxRows][32] floats.
+__host__ __device__ constexpr uint32_t wide_wave_lds() { return kWideXRows * kWideXS * 16u + 4u * 32u * 4u; }
+__host__ __device__ constexpr uint32_t wide_lds_bytes(uint32_t waves, uint32_t mats) {
+    return waves * wide_wave_lds() + waves * mats * kWideMaxRows * 32u * 4u;
+}
+
+template <WKind KIND, int MATS, int WAVES>
+__global__ __launch_bounds__(WAVES* kWave) void qgemm_wide_kernel(const QgemmWideArgs a) {
+    constexpr uint32_t VPL = KIND == W_Q4 ? 32u : 16u;  // codes per 16-byte lane load
+    constexpr int MF = VPL / 8;                         // MFMA steps per load
+    constexpr int LOADS = kWideSlab / (2u * VPL);       // 16-byte weight loads per lane, matrix and slab
+    constexpr int UNITS = kWideSlab / 64u;              // groups per slab
+    constexpr uint32_t LPG = 64u / (2u * VPL);          // loads per group
+    extern __shared__ uint4 lds_raw[];
+    const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), kb = lane >> 5, nl = lane & 31u;
+    uint4* xs = reinterpret_cast<uint4*>(reinterpret_cast<char*>(lds_raw) + wave * wide_wave_lds());  // [kWideXRows][kWideXS]
+    float* sxs = reinterpret_cast<float*>(xs + kWideXRows * kWideXS);                                  // [UNITS][32]
+    float* meet = reinterpret_cast<float*>(reinterpret_cast<char*>(lds_raw) + WAVES * wide_wave_lds()); // [WAVES][MATS][rows][32]
+
+    const uint32_t M = a.M, n = blockIdx.x * 32u + nl, nc = n < a.N ? n : a.N - 1;  // rows past the end repeat the last
+    const uint32_t n_slabs = (a.K + kWideSlab - 1) / kWideSlab;
+
+    // the zero row and the group sums of rows that do not exist (read by the fold, never stored)
+    for (uint32_t i = lane; i < kWideXS; i += kWave) xs[kWideMaxRows * kWideXS + i] = make_uint4(0, 0, 0, 0);
+    for (uint32_t i = lane; i < UNITS * 32u; i += kWave) sxs[i] = 0.f;
+    const uint32_t arow = nl < M ? nl : kWideMaxRows;  // this lane's row of the A operand
+
+    const uint4* wrow[MATS];
+    const uint16_t *srow[MATS], *brow[MATS];
+#pragma unroll
+    for (int q = 0; q < MATS; ++q) {
+        wrow[q] = a.w[q] + (size_t)nc * a.cpr;
+        srow[q] = a.sc[q] + (size_t)nc * a.gpr;
+        brow[q] = a.bi[q] + (size_t)nc * a.gpr;
+    }
+
+    f32x16_t acc[MATS];
+#pragma unroll
+    for (int q = 0; q < MATS; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[q][r] = 0.f;
+
+    // A slab's requests: weights, scale / bias pairs and this lane's pieces of the activations.  Straight-line (a
+    // branch around requests makes the compiler wait for everything outstanding where the paths join): a slab past
+    // the end (`live` false) reads the first bytes of the arrays.
+    struct Slab {
+        uint4 w[MATS][LOADS], x[kWideXPT];
+        uint32_t sb[MATS][UNITS];
+    };
+    auto fetch = [&](uint32_t slab, Slab& B) {
+        const bool live = slab < n_slabs;
+        const uint32_t ks0 = live ? slab * kWideSlab : 0u;
+        const uint32_t slab_k = a.K - ks0 < kWideSlab ? a.K - ks0 : kWideSlab;
+        const uint32_t loads = live ? slab_k / (2u * VPL) : 0u, units = live ? slab_k >> 6 : 0u, s8 = live ? slab_k >> 3 : 0u;
+#pragma unroll
+        for (int q = 0; q < MATS; ++q) {
+            const uint4* wp = (live ? wrow[q] : a.w[q]) + ks0 / VPL + (live ? kb : 0u);
+#pragma unroll
+            for (int t = 0; t < LOADS; ++t) B.w[q][t] = wp[2u * ((uint32_t)t < loads ? (uint32_t)t : 0u)];
+#pragma unroll
+            for (int u = 0; u < UNITS; ++u) {
+                const uint32_t g = (ks0 >> 6) + ((uint32_t)u < units ? (uint32_t)u : 0u);
+                B.sb[q][u] = (uint32_t)(live ? srow[q] : a.sc[q])[g] | ((uint32_t)(live ? brow[q] : a.bi[q])[g] << 16);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kWideXPT; ++i) {
+            const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
+            const bool have = m < M && k8 < s8;
+            B.x[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(have ? m : 0u) * a.K + ks0 + (have ? k8 : 0u) * 8u);
+        }
+    };
+    auto consume = [&](uint32_t slab, const Slab& B) {
+        const uint32_t ks0 = slab * kWideSlab;
+        const uint32_t slab_k = a.K - ks0 < kWideSlab ? a.K - ks0 : kWideSlab;
+        // park the slab's activations (the previous slab's fragments have been read: LDS operations of a wave are
+        // executed in order)
+#pragma unroll
+        for (int i = 0; i < kWideXPT; ++i) {
+            const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
+            uint4 v = (m < M && k8 < (slab_k >> 3)) ? B.x[i] : make_uint4(0, 0, 0, 0);
+            if constexpr (KIND == W_Q4) {
+                // nibble pairing of the int4 unpack: (x0,x2) (x4,x6) (x1,x3) (x5,x7)
+                v = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
+                               (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
+            }
+            xs[m * kWideXS + k8] = v;
+        }
+        __builtin_amdgcn_wave_barrier();
+        // group sums of the staged rows: lane (g, m) = (lane / 16, lane % 16) adds the 64 values of its group
+        {
+            const uint32_t g = lane >> 4, m = lane & 15u;
+            if (m < M) {
+                // (pairs of bf16 against a pair of ones: v_dot2_f32_bf16, no unpacking; two chains)
+                float s0 = 0.f, s1 = 0.f;
+                if (g < (slab_k >> 6)) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 8; ++i) {
+                        const uint4 v = xs[m * kWideXS + g * 8u + i];
+                        s0 = dot2_bf16(v.x, 0x3F803F80u, s0);
+                        s1 = dot2_bf16(v.y, 0x3F803F80u, s1);
+                        s0 = dot2_bf16(v.z, 0x3F803F80u, s0);
+                        s1 = dot2_bf16(v.w, 0x3F803F80u, s1);
+                    }
+                }
+                sxs[g * 32u + m] = s0 + s1;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        const uint32_t loads = slab_k / (2u * VPL);
+        // two C tiles per matrix, used alternately: consecutive matrix instructions do not wait for each other
+        // (a group's first instruction on a tile starts from a constant zero operand instead of a cleared tile)
+        f32x16_t c[MATS][2];
+        const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < LOADS; ++t) {
+            if ((uint32_t)t < loads) {  // wave-uniform
+                const uint4* xa = xs + arow * kWideXS + (((uint32_t)t * 2u + kb) * VPL >> 3);
+#pragma unroll
+                for (int j = 0; j < MF; ++j) {
+                    const uint4 av = xa[j];
+#pragma unroll
+                    for (int q = 0; q < MATS; ++q) {
+                        const uint32_t wd[4] = {B.w[q][t].x, B.w[q][t].y, B.w[q][t].z, B.w[q][t].w};
+                        uint4 bw;
+                        if constexpr (KIND == W_Q4) {
+                            const uint32_t even = wd[j] & 0x0F0F0F0Fu, odd = (wd[j] >> 4) & 0x0F0F0F0Fu;
+                            bw.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false));
+                            bw.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, true));
+                            bw.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, false));
+                            bw.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, true));
+                        } else {
+                            const uint32_t w0 = wd[(2 * j) & 3], w1 = wd[(2 * j + 1) & 3];
+                            auto pair = [](float lo, float hi) {
+                                const bf16x2_t p = {(__bf16)lo, (__bf16)hi};  // integers <= 255 are exact in bf16
+                                return __builtin_bit_cast(uint32_t, p);
+                            };
+                            bw.x = pair((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu));
+                            bw.y = pair((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24));
+                            bw.z = pair((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu));
+                            bw.w = pair((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24));
+                        }
+                        // step (t % LPG) * MF + j of its group: the first two start their tiles
+                        const bool first = ((uint32_t)t & (LPG - 1u)) * MF + j < 2;
+                        c[q][j & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                              __builtin_bit_cast(bf16x8_t, bw),
+                                                                              first ? zero : c[q][j & 1], 0, 0, 0);
+                    }
+                }
+                if (((uint32_t)t & (LPG - 1u)) == LPG - 1u) {
+                    // group complete: fold the integer dot into the accumulators.  Register r of this lane is
+                    // activation row (r % 4) + 8 * (r / 4) + 4 * kb; rows 16 .. 31 do not exist here (r >= 8).
+                    const uint32_t gl = ((uint32_t)t * 2u * VPL) >> 6;
+                    const float* sxg = sxs + gl * 32u + 4u * kb;
+                    const float4 sx0 = *reinterpret_cast<const float4*>(sxg), sx1 = *reinterpret_cast<const float4*>(sxg + 8);
+#pragma unroll
+                    for (int q = 0; q < MATS; ++q) {
+                        const uint32_t sb = B.sb[q][gl];
+                        const float sf = bf16_bits_to_f32(sb & 0xffffu), bf = bf16_bits_to_f32(sb >> 16);
+                        acc[q][0] += fmaf(sf, c[q][0][0] + c[q][1][0], bf * sx0.x);
+                        acc[q][1] += fmaf(sf, c[q][0][1] + c[q][1][1], bf * sx0.y);
+                        acc[q][2] += fmaf(sf, c[q][0][2] + c[q][1][2], bf * sx0.z);
+                        acc[q][3] += fmaf(sf, c[q][0][3] + c[q][1][3], bf * sx0.w);
+                        acc[q][4] += fmaf(sf, c[q][0][4] + c[q][1][4], bf * sx1.x);
+                        acc[q][5] += fmaf(sf, c[q][0][5] + c[q][1][5], bf * sx1.y);
+                        acc[q][6] += fmaf(sf, c[q][0][6] + c[q][1][6], bf * sx1.z);
+                        acc[q][7] += fmaf(sf, c[q][0][7] + c[q][1][7], bf * sx1.w);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();  // the next slab's pieces are written behind these reads
+    };
+
+    // Two sets of registers: slab i + 1 is requested before slab i is touched.  (One loop exit per pair of steps,
+    // so that the compiler does not have to assume, at the loop's top, that the set it is about to refill is
+    // still being loaded.)
+    Slab A, B;
+    FK_WIDE_STAMP(0);
+    fetch(wave, A);
+    FK_WIDE_STAMP(1);
+    for (uint32_t slab = wave; slab < n_slabs; slab += 2 * WAVES) {
+        fetch(slab + WAVES, B);
+        consume(slab, A);
+        if (slab == wave) FK_WIDE_STAMP(2);
+        fetch(slab + 2 * WAVES, A);
+        if (slab + WAVES < n_slabs) consume(slab + WAVES, B);
+        if (slab == wave) FK_WIDE_STAMP(3);
+    }
+    FK_WIDE_STAMP(4);
+
+    // The waves meet: every wave parks its sums of the rows that exist, [wave][matrix][row][weight row of the block].
+#pragma unroll
+    for (int q = 0; q < MATS; ++q)
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const uint32_t m = (uint32_t)(r % 4 + 8 * (r / 4)) + 4u * kb;
+            if (m < M) meet[((wave * MATS + q) * kWideMaxRows + m) * 32u + nl] = acc[q][r];
+        }
+    __syncthreads();
+    FK_WIDE_STAMP(5);
+    for (uint32_t e = threadIdx.x; e < M * 32u; e += WAVES * kWave) {
+        const uint32_t m = e >> 5, col = e & 31u, nn = blockIdx.x * 32u + col;
+        if (nn >= a.N) continue;
+        float s[MATS];
+#pragma unroll
+        for (int q = 0; q < MATS; ++q) {
+            s[q] = 0.f;
+            for (int w = 0; w < WAVES; ++w) s[q] += meet[((w * MATS + q) * kWideMaxRows + m) * 32u + col];
+        }
+        uint32_t o;
+        if constexpr (MATS == 2) {
+            o = swiglu_bits(s[0], s[1], a.variant, 1.0f);
+        } else {
+            float v = s[0];
+            if (a.bias) v += bf16_bits_to_f32(a.bias[nn]);
+            if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * a.N + nn]);
+            o = f32_to_bf16_bits(v);
+        }
+        a.y[(size_t)m * a.N + nn] = (uint16_t)o;
+    }
+    FK_WIDE_STAMP(6);
+}
+
+template <WKind KIND, int MATS>
+const void* wide_func(uint32_t waves) {
+    return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide_kernel<KIND, MATS, 8>)
+                      : reinterpret_cast<const void*>(&qgemm_wide_kernel<KIND, MATS, 4>);
+}
+
+}  // namespace
+
+static bool g_wide_on = true;
+void set_qgemm_wide(bool on) { g_wide_on = on; }
+bool qgemm_takes_wide(uint32_t M, uint32_t group) { return g_wide_on && M >= 2 && M <= kWideMaxRows && group == 64; }
+
+// W1 (and SwiGLU of the pair) or bias / res (single matrix).
+fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16_t* x, uint32_t M, const uint16_t* bias,
+                          const uint16_t* res, int variant, uint16_t* y, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!qgemm_takes_wide(M, W0->group)) return set_error(FK_ERR_UNSUPPORTED, "qgemm (shared stream): 2..10 rows, group size 64");
+    if (W0->k % 64u) return set_error(FK_ERR_UNSUPPORTED, "qgemm (shared stream): K must be a multiple of 64");
+    QgemmWideArgs a;
+    memset(&a, 0, sizeof(a));
+    const fk_weight* Ws[2] = {W0, W1};
+    for (int q = 0; q < (W1 ? 2 : 1); ++q) {
+        a.w[q] = reinterpret_cast<const uint4*>(Ws[q]->w);
+        a.sc[q] = Ws[q]->scales;
+        a.bi[q] = Ws[q]->biases;
+    }
+    a.x = x; a.bias = bias; a.res = res; a.y = y;
+    a.M = M; a.N = W0->n; a.K = W0->k;
+    a.cpr = W0->k / (W0->bits == 4 ? 32u : 16u);
+    a.gpr = W0->k / 64u;
+    a.variant = variant;
+    // Eight waves per block (K split eight ways) while every block still finds a CU of its own; four beyond
+    // (registers allow one eight-wave block per CU).  Measured, 8 rows of int4, serialised graph, against the
+    // split-k kernel + reduction: 6144 x 2560 8.5 us (15.6), 2560 x 4096 11.2 (18.4), 2048 x 1408 5.8 (10.2),
+    // 1408 x 2048 6.9 (11.4), 9728 x 2560 14.0 (16.3), 2560 x 9728 21.0 (21.7): per 16-byte chunk the kernel spends
+    // ~150 vector instructions and four matrix instructions (three quarters of whose rows are padding), so the
+    // 14 MB matrices are bound by that, not by the stream.
+    const uint32_t blocks = (W0->n + 31u) / 32u, n_slabs = (W0->k + kWideSlab - 1) / kWideSlab;
+    const uint32_t waves = (blocks <= (uint32_t)dev->cus && n_slabs >= 5u) ? 8u : 4u;
+    const bool q4 = W0->bits == 4;
+    out->func = W1 ? (q4 ? wide_func<W_Q4, 2>(waves) : wide_func<W_Q8, 2>(waves))
+                   : (q4 ? wide_func<W_Q4, 1>(waves) : wide_func<W_Q8, 1>(waves));
+    out->grid = dim3(blocks, 1, 1);
+    out->block = dim3(waves * kWave, 1, 1);
+    out->shmem = wide_lds_bytes(waves, W1 ? 2u : 1u);
+    out->set_args(a);
+    if (out->shmem > 48 * 1024)
+        FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)out->shmem));
+    return FK_OK;
+}
+
+}  // namespace fk

@@ -549,7 +549,7 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
         Launch main, red;
         FK_TRY(plan_qgemm(W_shared, shared_x, n_tokens, nullptr, nullptr, parts + (size_t)n_routes * Wd->n, qws, &main, &red));
         out->then.push_back(main);
-        out->then.push_back(red);
+        if (red.func) out->then.push_back(red);
     }
     Launch reduce;
     FK_TRY(plan_route_reduce(parts, route_weight, residual, out_ptr, n_tokens, top_k, Wd->n, W_shared != nullptr, &reduce));

@@ -218,7 +218,7 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
                               {"bits": bits, "group": 64, "m": k, "n": n, "rows": rows}))
     nbytes = n * k * per + rows * k * 2 + rows * n * 2
     _emit(f"qgemm_rows{rows}_{n}x{k}_q{bits}", _time_graph(d, tasks, reps), nbytes, flops=2.0 * rows * n * k, pool=pool,
-          note="two kernels: MFMA main + split-k reduction")
+          note="2..10 rows: one shared-stream launch; more rows: MFMA main + split-k reduction")
 
 
 def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_bits=0, keep=False):

@@ -557,6 +557,10 @@ def gemv_form(n: int, k: int, bits: int, group: int = 64) -> int:
     return int(lib.fk_gemv_form(C.c_uint32(n), C.c_uint32(k), C.c_uint32(bits), C.c_uint32(group)))
 
 
+def set_qgemm_wide(enabled: bool) -> None:
+    check(lib.fk_set_qgemm_wide(C.c_int(1 if enabled else 0)))
+
+
 def set_gemv_flat_only(flat_only: bool) -> None:
     check(lib.fk_set_gemv_flat_only(C.c_int(1 if flat_only else 0)))
 

@@ -676,6 +676,12 @@ fk_status fk_set_gemv_flat_only(int flat_only);
  * product to rocBLAS (opened on first use; absent: the fused kernel is kept).  Default 256; 0 = never.
  * Set it BEFORE sizing workspaces: fk_qgemm_workspace_bytes covers the route that will be taken. */
 fk_status fk_set_gemm_library_rows(uint32_t rows);
+/* 2..10 activation rows at group size 64 run fk_qgemm / fk_qgemm_swiglu as ONE launch that streams the weights
+ * once for all rows and includes the epilogue (the reference's small-M kernels: src/codegen/msl.rs:462-546,
+ * :1307-1485, policy src/codegen/kernels/mod.rs:164-186).  fk_set_qgemm_wide(0) sends those row counts through
+ * the split-k kernel + reduction instead (measurements, tests); 1 restores the default.  Process-wide; takes
+ * effect for launches planned afterwards. */
+fk_status fk_set_qgemm_wide(int enabled);
 /* An MLX-affine matrix (bits 4 / 8, group 64 / 128) as dense bf16 [n, k], every element T(code * scale + bias):
  * the values the library route of fk_qgemm multiplies with.  With 288 GB of HBM a runtime may keep the bf16 copy
  * of a model's projections resident for its prompt passes and hand it to fk_qgemm as a bits-16 weight, which

@@ -149,6 +149,17 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
     routes = rt.routes()[cfg.first_dense:]
     assert [sorted(r.tolist()) for r in routes] == fx["routes_last_step"]
 
+    # The same model at full size with EIGHT active token rows in one pass over the weights (shared-stream matmuls
+    # for the dense projections and the shared experts, row forms of the store, the attention and the router,
+    # routed experts over 48 routes): the oracle's tokens 23 .. 30 as rows at positions 55 .. 62, behind a cache
+    # filled step by step, must give the oracle's token 31 and, for the last row, the oracle's routes of its last step.
+    rt.reset()
+    head, _, _ = rt.generate(fx["prompt"], 24)
+    assert head == fx["tokens"][:24]
+    nxt = rt.forward_rows(fx["tokens"][23:31], 32 + 23)
+    assert nxt == fx["tokens"][31]
+    assert sorted(rt.rows_routes[-1].tolist()) == fx["routes_last_step"][-1]
+
 
 @pytest.mark.parametrize("rows,offset", [(8, 0), (5, 8), (1, 3)])
 def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset):

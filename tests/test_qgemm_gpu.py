@@ -65,6 +65,50 @@ def test_qgemm_matches_oracle(fk, m, n, k, bits):
         _check(got[r], ref[r], acc[r], W, x[r])
 
 
+# The shared-stream kernel for 2..10 activation rows (one launch, no split-k sums): every row count of its range,
+# the projections of the 4B-class decoder and of the mixture-of-experts model (K = 1408 ends in half a slab),
+# a ragged N, few weight rows with a long K (16 waves per block), bias and residual, and the split-k route on the
+# same operands (both keep the single-row arithmetic: rounding-edge flips only).
+WIDE_SHAPES = [(2, 2560, 2560), (3, 6144, 2560), (4, 333, 1408), (5, 2560, 9728), (6, 2048, 1408), (7, 1408, 2048),
+               (8, 9728, 2560), (9, 70, 4096), (10, 2560, 4096)]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,n,k", WIDE_SHAPES)
+def test_shared_stream_rows_match_oracle_and_the_split_k_route(fk, m, n, k, bits):
+    W = make_qweight(150 + bits + m, n, k, bits)
+    x = normal_bf16(151 + m, (m, k))
+    bias, res = normal_bf16(152, n), normal_bf16(153, (m, n))
+    got = _run(fk, W, x)
+    ref, acc = _reference(W, x)
+    for r in range(m):
+        _check(got[r], ref[r], acc[r], W, x[r])
+    got_b = _run(fk, W, x, bias=bias, res=res)
+    fk.set_qgemm_wide(False)
+    try:
+        split_k = _run(fk, W, x)
+        split_k_b = _run(fk, W, x, bias=bias, res=res)
+    finally:
+        fk.set_qgemm_wide(True)
+    for r in range(m):
+        _check(got[r], split_k[r], oracle.bf16_to_f32(split_k[r]), W, x[r])
+        _check(got_b[r], split_k_b[r], oracle.bf16_to_f32(split_k_b[r]), W, x[r])
+    assert not np.array_equal(got_b, got)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("m,hidden,inter,bits", [(2, 2560, 9728, 4), (10, 2048, 1408, 4), (5, 896, 4864, 8)])
+def test_shared_stream_gate_up_swiglu(fk, m, hidden, inter, bits, variant):
+    Wg, Wu = make_qweight(166, inter, hidden, bits), make_qweight(167, inter, hidden, bits)
+    x = normal_bf16(168, (m, hidden))
+    out = fk.DeviceBuffer(2 * m * inter)
+    ws = fk.DeviceBuffer(2 * fk.qgemm_workspace_bytes(m, inter, hidden, 64))
+    fk.qgemm_swiglu(to_device(fk, Wg), to_device(fk, Wu), _dev(fk, x), m, variant, out, ws)
+    got = out.to_numpy(np.uint16, (m, inter))
+    for r in range(m):
+        _check_swiglu(got[r], oracle.gateup_swiglu(x[r], None, 0.0, Wg, Wu, variant), x[r], Wg, Wu, variant)
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("m", [9, 100])
 def test_qgemm_group_128(fk, bits, m):
