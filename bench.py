@@ -45,6 +45,7 @@ SYMBOLS = {
     "xcd_mlp_block": "xcd_mlp_kernel<Q4>",
     "xcd_reduce": "xcd_reduce_kernel",
     "final_rmsnorm_lm_head": "gemv_rows_kernel<BF16, batches of 5 column blocks>",
+    "final_rmsnorm_lm_head_argmax": "gemv_rows_kernel<BF16, batches of 5 column blocks, greedy token>",
     "argmax_logits_decode": "argmax_kernel",
     "embed_lookup_decode": "embed_lookup_kernel",
     "step_init": "step_init_kernel",

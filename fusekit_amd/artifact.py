@@ -43,7 +43,8 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
             scratch(name, buf, dtype, zero)
         _parameter_symbols(rt, sym)
         return sym
-    for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws"):
+    for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws",
+                 "head_argmax_ws"):
         scratch(name, getattr(rt, name), "uint32", zero=True)
     scratch("x.0", rt.x[0], "bfloat16")
     scratch("x.1", rt.x[1], "bfloat16")

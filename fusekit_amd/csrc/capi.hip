@@ -381,6 +381,31 @@ fk_status fk_final_rmsnorm_lm_head(const uint16_t* x, const uint16_t* norm_w, fl
     return run_launch(l, (hipStream_t)s);
 }
 
+static_assert(FK_HEAD_ARGMAX_WORKSPACE_BYTES == kHeadArgmaxWorkspaceBytes, "header and kernel disagree");
+
+fk_status fk_final_rmsnorm_lm_head_argmax(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* W,
+                                          uint16_t* logits, uint32_t* next_token, uint32_t* history,
+                                          uint32_t* hist_counter, uint32_t hist_capacity, void* workspace,
+                                          fk_stream s) {
+    if (!norm_w) return set_error(FK_ERR_INVALID, "fk_final_rmsnorm_lm_head_argmax: null norm weight");
+    HeadArgmax am;
+    am.next_token = next_token;
+    am.history = history;
+    am.hist_counter = hist_counter;
+    am.hist_capacity = hist_capacity;
+    am.workspace = workspace;
+    GemvRequest rq;
+    rq.mats[0] = W;
+    rq.y[0] = logits;
+    rq.x = x;
+    rq.norm_w = norm_w;
+    rq.eps = eps;
+    rq.argmax = &am;
+    Launch l;
+    FK_TRY(plan_gemv(rq, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 static float theta_log2(float theta) { return (float)log2((double)theta); }
 
 fk_status fk_rope_q_decode(uint16_t* q, const uint16_t* q_norm, uint32_t n_heads, uint32_t head_dim,

@@ -6,6 +6,7 @@
 #include "fk_host.hpp"
 #include "fk_device.hpp"
 #include "rope_device.hpp"
+#include "argmax_tail.hpp"
 
 namespace fk {
 
@@ -266,76 +267,20 @@ fk_status plan_embed(const fk_weight* E, const uint32_t* token_ptr, uint32_t tok
 struct ArgmaxArgs {
     const uint16_t* logits;
     uint32_t n;
-    uint32_t* next_token;
-    uint32_t* history;        // optional: history[(*hist_counter)++] = token
-    uint32_t* hist_counter;
-    uint32_t hist_capacity;
-    uint64_t* partial;        // [grid] packed (order-preserving key << 32) | ~index
-    uint32_t* counter;        // zero before the first launch
+    ArgmaxTail tail;
 };
 
-// Order-preserving key of a bf16-as-float value; NaN maps below everything so it
-// never wins (the reference's `v > max` comparison, argmax_logits_decode.rs:63-95).
-__device__ __forceinline__ uint32_t order_key(float v) {
-    if (v != v) return 0u;
-    const uint32_t u = __float_as_uint(v);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-// Two stages in one launch: every block reduces a slice to one packed 64-bit
-// candidate (value key in the high word, inverted index in the low word, so the
-// maximum of the packed value is the largest logit with the LOWEST index); the
-// last block to finish reduces the candidates.
+// Two stages in one launch (argmax_tail.hpp): every block reduces a slice to one packed candidate, the last block
+// to finish reduces the candidates.
 __global__ __launch_bounds__(256) void argmax_kernel(const ArgmaxArgs a) {
     __shared__ uint64_t sm[256 / kWave];
     __shared__ uint32_t is_last;
     uint64_t best = 0;
     for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < a.n; i += gridDim.x * 256) {
-        const uint64_t cand = ((uint64_t)order_key(bf16_bits_to_f32(a.logits[i])) << 32) | (uint32_t)(~i);
+        const uint64_t cand = argmax_candidate(a.logits[i], i);
         best = cand > best ? cand : best;
     }
-    auto block_best = [&](uint64_t v) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const uint64_t other = __shfl_xor(v, o, kWave);
-            v = other > v ? other : v;
-        }
-        if ((threadIdx.x & (kWave - 1)) == 0) sm[threadIdx.x / kWave] = v;
-        __syncthreads();
-        uint64_t r = sm[0];
-#pragma unroll
-        for (int w = 1; w < 256 / kWave; ++w) r = sm[w] > r ? sm[w] : r;
-        __syncthreads();
-        return r;
-    };
-    best = block_best(best);
-    // The candidate is stored write-through (agent scope) and its arrival awaited
-    // before the block counts itself in; the last block reads the candidates past
-    // the caches.  No device-wide fence (which would write back a whole L2).
-    if (threadIdx.x == 0) {
-        __hip_atomic_store(&a.partial[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        wait_memory_ops_done();
-        is_last = (atomicAdd(a.counter, 1u) == gridDim.x - 1) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (!is_last) return;
-    uint64_t fin = 0;
-    for (uint32_t i = threadIdx.x; i < gridDim.x; i += 256) {
-        const uint64_t c = __hip_atomic_load(&a.partial[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        fin = c > fin ? c : fin;
-    }
-    fin = block_best(fin);
-    if (threadIdx.x == 0) {
-        // all-NaN / empty rows fall back to index 0 like the reference's initial local_idx
-        const uint32_t tok = (fin >> 32) ? ~(uint32_t)fin : 0u;
-        *a.next_token = tok;
-        if (a.history && a.hist_counter) {
-            const uint32_t slot = *a.hist_counter;
-            if (slot < a.hist_capacity) a.history[slot] = tok;
-            *a.hist_counter = slot + 1;
-        }
-        __hip_atomic_store(a.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    argmax_block_finish<256>(a.tail, best, sm, &is_last);
 }
 
 fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, uint32_t* history,
@@ -348,10 +293,10 @@ fk_status plan_argmax(const uint16_t* logits, uint32_t n, uint32_t* next_token, 
     if (grid > 160) grid = 160;
     ArgmaxArgs a;
     memset(&a, 0, sizeof(a));
-    a.logits = logits; a.n = n; a.next_token = next_token;
-    a.history = history; a.hist_counter = hist_counter; a.hist_capacity = hist_capacity;
-    a.counter = reinterpret_cast<uint32_t*>(workspace);
-    a.partial = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(workspace) + 8);
+    a.logits = logits; a.n = n; a.tail.next_token = next_token;
+    a.tail.history = history; a.tail.hist_counter = hist_counter; a.tail.hist_capacity = hist_capacity;
+    a.tail.counter = reinterpret_cast<uint32_t*>(workspace);
+    a.tail.partial = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(workspace) + 8);
     out->func = reinterpret_cast<const void*>(&argmax_kernel);
     out->grid = dim3(grid, 1, 1);
     out->block = dim3(256, 1, 1);

@@ -271,12 +271,33 @@ fk_status plan_qgemv_d(const Dispatch& d, Launch* l, SlotRW* rw) {
 }
 
 // x, norm_w, W, [scales, biases], logits
-fk_status plan_lm_head(const Dispatch& d, Launch* l, SlotRW* rw) {
+// argmax: the direct head; slots behind the logits are next_tok, workspace [, history, hist_counter].
+fk_status plan_lm_head(const Dispatch& d, Launch* l, SlotRW* rw, bool argmax) {
     const uint32_t bits = d.u("bits", 16), group = d.u("group", 64), hidden = d.u("hidden"), vocab = d.u("vocab");
     size_t s = 3;
     if (bits != 16) s += 2;
     const size_t out_slot = s++;
-    FK_TRY(need_args(d, s));
+    HeadArgmax am;
+    if (argmax) {
+        const bool hist = d.args.size() == s + 4;
+        FK_TRY(need_args(d, s + (hist ? 4 : 2)));
+        FK_TRY(need_bytes(d, s, 4));
+        FK_TRY(need_bytes(d, s + 1, kHeadArgmaxWorkspaceBytes));
+        am.next_token = arg_ptr<uint32_t>(d, s);
+        am.workspace = d.args[s + 1].ptr;
+        if (hist) {
+            FK_TRY(need_bytes(d, s + 3, 4));
+            am.history = arg_ptr<uint32_t>(d, s + 2);
+            am.hist_counter = arg_ptr<uint32_t>(d, s + 3);
+            am.hist_capacity = (uint32_t)(d.args[s + 2].nbytes / 4);
+        }
+        for (size_t i = 0; i < out_slot; ++i) rw->reads.push_back((uint32_t)i);
+        rw->reads.push_back((uint32_t)(s + 1));
+        for (size_t i = out_slot; i < d.args.size(); ++i) rw->writes.push_back((uint32_t)i);
+        if (hist) rw->reads.push_back((uint32_t)(s + 3));
+    } else {
+        FK_TRY(need_args(d, s));
+    }
     GemvRequest rq;
     fk_weight W;
     FK_TRY(bind_weight(d, bits, group, vocab, hidden, 2, 3, 4, &W));
@@ -288,7 +309,10 @@ fk_status plan_lm_head(const Dispatch& d, Launch* l, SlotRW* rw) {
     rq.norm_w = arg_ptr<const uint16_t>(d, 1);
     rq.eps = (float)d.param("eps", 1e-6);
     rq.y[0] = arg_ptr<uint16_t>(d, out_slot);
-    all_but_last(s, 1, rw);
+    if (argmax)
+        rq.argmax = &am;
+    else
+        all_but_last(s, 1, rw);
     return plan_gemv(rq, l);
 }
 
@@ -1148,7 +1172,10 @@ const Family kFamilies[] = {
     {"fusekit_rmsnorm_gateup_swiglu", plan_gateup},
     {"fusekit_qmv_swiglu", plan_gateup},
     {"fusekit_linear_residual", plan_linres},
-    {"fusekit_final_rmsnorm_lm_head", plan_lm_head},
+    {"fusekit_final_rmsnorm_lm_head_argmax",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_lm_head(d, l, rw, true); }},
+    {"fusekit_final_rmsnorm_lm_head",
+     [](const Dispatch& d, Launch* l, SlotRW* rw) { return plan_lm_head(d, l, rw, false); }},
     {"fusekit_qgemv", plan_qgemv_d},
     {"fusekit_qgemm", plan_qgemm_d},
     {"fusekit_qgemm_swiglu", plan_qgemm_swiglu_d},

@@ -70,6 +70,19 @@ uint32_t gemv_rows_batch(uint32_t n, uint32_t k, uint32_t bits, uint32_t group);
 // blocks (the persistent whole-token kernel plans every phase for its own grid).
 extern thread_local uint32_t t_gemv_grid_override;
 
+// Greedy selection fused into the GEMV that produces the logits (row-group form only): the launch writes y as usual
+// and also the index of its largest bf16 output, lowest index on ties, like plan_argmax.  `workspace` holds
+// kHeadArgmaxWorkspaceBytes, zero before the first launch.
+struct HeadArgmax {
+    uint32_t* next_token = nullptr;
+    uint32_t* history = nullptr;  // optional, with hist_counter: history[(*hist_counter)++] = token
+    uint32_t* hist_counter = nullptr;
+    uint32_t hist_capacity = 0;
+    void* workspace = nullptr;
+};
+constexpr uint32_t kHeadArgmaxMaxBlocks = 4096;
+constexpr size_t kHeadArgmaxWorkspaceBytes = 8 + 8 * (size_t)kHeadArgmaxMaxBlocks;
+
 struct GemvRequest {
     const fk_weight* mats[3] = {nullptr, nullptr, nullptr};
     const uint16_t* bias[3] = {nullptr, nullptr, nullptr};
@@ -82,6 +95,7 @@ struct GemvRequest {
     float eps = 0.f;
     const uint16_t* res = nullptr;
     const uint16_t* res2 = nullptr;
+    const HeadArgmax* argmax = nullptr;  // FK_ERR_UNSUPPORTED when the shape does not take the row-group form
 };
 fk_status plan_gemv(const GemvRequest& rq, Launch* out);
 

@@ -50,19 +50,24 @@ const void* select_gemv(WKind kind, bool swiglu) {
     }
 }
 
-template <WKind KIND, bool TAIL>
+template <WKind KIND, bool TAIL, bool ARGMAX>
 const void* rows_func(uint32_t nb) {
     switch (nb) {
-        case 3: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 3, TAIL>);
-        case 4: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 4, TAIL>);
-        default: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 5, TAIL>);
+        case 3: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 3, TAIL, ARGMAX>);
+        case 4: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 4, TAIL, ARGMAX>);
+        default: return reinterpret_cast<const void*>(&gemv_rows_kernel<KIND, 5, TAIL, ARGMAX>);
     }
 }
-const void* rows_func(WKind kind, uint32_t nb, bool tail) {
+template <WKind KIND>
+const void* rows_func(uint32_t nb, bool tail, bool argmax) {
+    if (argmax) return tail ? rows_func<KIND, true, true>(nb) : rows_func<KIND, false, true>(nb);
+    return tail ? rows_func<KIND, true, false>(nb) : rows_func<KIND, false, false>(nb);
+}
+const void* rows_func(WKind kind, uint32_t nb, bool tail, bool argmax) {
     switch (kind) {
-        case W_Q4: return tail ? rows_func<W_Q4, true>(nb) : rows_func<W_Q4, false>(nb);
-        case W_Q8: return tail ? rows_func<W_Q8, true>(nb) : rows_func<W_Q8, false>(nb);
-        default: return tail ? rows_func<W_BF16, true>(nb) : rows_func<W_BF16, false>(nb);
+        case W_Q4: return rows_func<W_Q4>(nb, tail, argmax);
+        case W_Q8: return rows_func<W_Q8>(nb, tail, argmax);
+        default: return rows_func<W_BF16>(nb, tail, argmax);
     }
 }
 
@@ -140,6 +145,8 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
         if (rq.mats[0]->n != rq.mats[1]->n) return set_error(FK_ERR_INVALID, "gemv: gate and up need equal rows");
         if (!rq.y[0]) return set_error(FK_ERR_INVALID, "gemv: null output");
     }
+    if (rq.argmax && (!rq.argmax->next_token || !rq.argmax->workspace))
+        return set_error(FK_ERR_INVALID, "gemv: head argmax needs a token slot and a workspace");
     const WKind kind = bits == 4 ? W_Q4 : (bits == 8 ? W_Q8 : W_BF16);
     const uint32_t values = bits == 4 ? 32u : (bits == 8 ? 16u : 8u);
     const uint32_t cpr = K / values;
@@ -160,14 +167,24 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
         const uint32_t lds = kind == W_Q4 ? gemv_rows_lds_bytes<W_Q4>(cpr)
                              : (kind == W_Q8 ? gemv_rows_lds_bytes<W_Q8>(cpr) : gemv_rows_lds_bytes<W_BF16>(cpr));
         if (ok && (int)lds <= dev->max_dyn_lds) {
-            const void* f = rows_func(kind, nb, cpl % nb != 0);
+            const void* f = rows_func(kind, nb, cpl % nb != 0, rq.argmax != nullptr);
             // whole rounds: every wave of the grid gets the same number of passes (to within one)
             const uint64_t cap = g_gemv_policy.grid_blocks ? g_gemv_policy.grid_blocks : (uint64_t)blocks_per_cu(f, lds) * dev->cus;
             const uint64_t block_passes = (passes + kBlockWaves - 1) / kBlockWaves;
             const uint64_t rounds = (block_passes + cap - 1) / cap;
             const uint64_t blocks = (block_passes + rounds - 1) / rounds;
-            GemvArgs a;
+            if (rq.argmax && blocks > kHeadArgmaxMaxBlocks)
+                return set_error(FK_ERR_UNSUPPORTED, "gemv: head argmax over more blocks than its workspace holds");
+            GemvArgmaxArgs a;
             memset(&a, 0, sizeof(a));
+            if (rq.argmax) {
+                a.tail.next_token = rq.argmax->next_token;
+                a.tail.history = rq.argmax->history;
+                a.tail.hist_counter = rq.argmax->hist_counter;
+                a.tail.hist_capacity = rq.argmax->hist_capacity;
+                a.tail.counter = reinterpret_cast<uint32_t*>(rq.argmax->workspace);
+                a.tail.partial = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(rq.argmax->workspace) + 8);
+            }
             uint32_t t0 = 0;
             for (int m = 0; m < nm; ++m) {
                 a.w[m] = reinterpret_cast<const uint4*>(rq.mats[m]->w);
@@ -198,11 +215,15 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
             out->grid = dim3((uint32_t)blocks, 1, 1);
             out->block = dim3(kGemvBlock, 1, 1);
             out->shmem = lds;
-            out->set_args(a);
+            if (rq.argmax)
+                out->set_args(a);
+            else
+                out->set_args(static_cast<const GemvArgs&>(a));
             if (lds > 48 * 1024) FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             return FK_OK;
         }
     }
+    if (rq.argmax) return set_error(FK_ERR_UNSUPPORTED, "gemv: head argmax needs a shape the row-group form takes");
     const void* func = select_gemv(kind, rq.swiglu);
     auto tiles_for = [&](uint32_t r) {
         uint64_t t = 0;

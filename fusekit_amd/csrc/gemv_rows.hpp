@@ -19,6 +19,9 @@
 // Batches (NB column blocks of one pass) are double-buffered in registers: batch k + 1 is requested before batch k
 // is consumed.  Work is dealt to waves pass by pass: pass (k * gridDim.x + block) * 4 + wave.
 #pragma once
+#include <type_traits>
+
+#include "argmax_tail.hpp"
 #include "gemv_kernel.hpp"
 
 namespace fk {
@@ -89,8 +92,16 @@ __device__ __forceinline__ float rows_chunk_dot(uint4 wv, const uint4* xp, float
 // The loop body is straight-line as far as memory requests go: a branch around a request makes the compiler wait
 // for EVERY outstanding load where the paths join, which would serialise the prefetch.  A wave that has run out of
 // passes therefore still issues its NB + 1 requests once more, all lanes at the first bytes of the arrays.
-template <WKind KIND, int NB, bool TAIL>
-__global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const GemvArgs a) {
+//
+// ARGMAX: the rows are logits and the launch also selects the greedy token (argmax_tail.hpp): a lane keeps the best
+// (value, row) candidate of the rows it has stored, on the bf16 value it stored, and the block hands its best to
+// argmax_block_finish once its waves have run out of passes -- the only block barrier after staging.
+struct GemvArgmaxArgs : GemvArgs {
+    ArgmaxTail tail;
+};
+
+template <WKind KIND, int NB, bool TAIL, bool ARGMAX = false>
+__global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const std::conditional_t<ARGMAX, GemvArgmaxArgs, GemvArgs> a) {
     extern __shared__ uint4 lds_raw[];
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     constexpr bool QUANT = KIND != W_BF16;
@@ -157,9 +168,12 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const GemvArgs a)
     // registers, as if the load were still outstanding -- and with it for the batch just requested).
 #pragma unroll
     for (int i = 0; i < kStageRegs; ++i) asm volatile("" ::"v"(xr[i].x), "v"(wr[i].x));
-    if (!any) return;
+    if constexpr (!ARGMAX) {
+        if (!any) return;
+    }
 
     float acc = 0.f;
+    [[maybe_unused]] uint64_t best = 0;
     // Value and offset of the last output stored.  Stores and loads complete in issue order on one counter, so
     // overwriting a store's registers before the loads issued ahead of it have been waited for anyway would make
     // the compiler wait for all of those loads early, before the next batch is requested: the two are kept alive
@@ -217,6 +231,10 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const GemvArgs a)
             // (one would make the compiler restructure the whole loop around a single exit, and the paths it
             // then has to assume make it wait for the newest batch where it need not).
             *reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(ybase) + held_o) = (uint16_t)held_v;
+            if constexpr (ARGMAX) {
+                const uint64_t cand = argmax_candidate(held_v, row_c);
+                best = cand > best ? cand : best;
+            }
             acc = 0.f;
         }
         pass = npass;
@@ -227,10 +245,15 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const GemvArgs a)
     // and must then assume, at the loop's top, that the batch requested by the first step may still be in flight
     // in the registers it is about to reuse -- it waits for it, and the prefetch is gone.  A wave with an odd
     // number of batches therefore consumes one dead batch (requested with live = false) whose result is dropped.
-    bool more = true;
+    bool more = any;
     while (more) {
         step(wa, ma, wb, mb);
         more = step(wb, mb, wa, ma);
+    }
+    if constexpr (ARGMAX) {
+        __shared__ uint64_t best_of_wave[kBlockWaves];
+        __shared__ uint32_t is_last;
+        argmax_block_finish<kGemvBlock>(a.tail, best, best_of_wave, &is_last);
     }
 }
 

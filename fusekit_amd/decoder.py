@@ -47,6 +47,7 @@ class DecoderConfig:
     embed_scale: float = 1.0  # output_scale of the embedding lookup (embed_lookup_decode.rs:74-99)
     xcd_layers: bool = True   # graph mode: run a layer as two XCD-resident launches where the shape allows it
     xcd_spin_limit: int = 0   # bound of the XCD hand-over waits in polls (0: the library's default)
+    direct_head_argmax: bool = True  # graph mode: the LM head selects the greedy token itself where its shape allows
     xcd_token_launch: bool = False  # the layers' launches of a token as ONE launch (device-wide barriers between them); slower at present
 
     @property
@@ -211,6 +212,7 @@ class DecoderRuntime:
         pb, cb = native.sdpa_workspace_bytes(cfg.n_heads, cfg.n_kv, cfg.head_dim, cfg.head_dim, cfg.capacity)
         self.sdpa_partials, self.sdpa_counters = DeviceBuffer(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
+        self.head_argmax_ws = z(native.HEAD_ARGMAX_WORKSPACE_BYTES)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
         self.persistent = persistent
         # one launch per layer for rope/store + attention: the task graph only (the whole-token kernel
@@ -353,9 +355,18 @@ class DecoderRuntime:
             t.append(Dispatch(name("linear_residual"),
                               [arg(self.mid)] + self._wargs(Wd) + [arg(self.x[1]), arg(self.x[0])],
                               dict(q, m=c.inter, n=c.hidden)))
-        t.append(Dispatch(name("final_rmsnorm_lm_head"),
-                          [arg(self.x[0]), arg(w.vecs["final_norm"])] + self._wargs(head) + [arg(self.logits)],
-                          dict(bits=head.bits, group=head.group or 64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
+        head_args = [arg(self.x[0]), arg(w.vecs["final_norm"])] + self._wargs(head) + [arg(self.logits)]
+        head_params = dict(bits=head.bits, group=head.group or 64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)
+        # The direct head (the reference's `<head>_argmax` + `_argmax_finalize`, dispatch.py:3458-3505, greedy
+        # decode only) as one launch; the whole-token kernel keeps the canonical two tasks.
+        self.direct_head = bool(c.direct_head_argmax and not self.persistent and
+                                native.gemv_form(c.vocab, c.hidden, head.bits, head.group or 64) == 1)
+        if self.direct_head:
+            t.append(Dispatch(name("final_rmsnorm_lm_head_argmax"),
+                              head_args + [arg(self.token), arg(self.head_argmax_ws), arg(self.history),
+                                           arg(self.hist_counter)], head_params))
+            return t
+        t.append(Dispatch(name("final_rmsnorm_lm_head"), head_args, head_params))
         t.append(Dispatch(name("argmax_logits_decode"),
                           [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history),
                            arg(self.hist_counter)], dict(vocab=c.vocab)))

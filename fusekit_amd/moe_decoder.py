@@ -57,6 +57,7 @@ class MoeConfig:
     fuse_attention: bool = True   # split-key cache store + attention of a layer in one launch
     fuse_shared: bool = True   # the shared experts' gate/up pair as further routes of the routed launch
     fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
+    direct_head_argmax: bool = True  # the LM head selects the greedy token itself where its shape allows
 
     @property
     def qk_dim(self) -> int:
@@ -209,6 +210,7 @@ class MoeRuntime:
         pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
         self.sdpa_partials, self.sdpa_counters = B(max(pb, 4)), z(max(cb, 4))
         self.argmax_ws = z(native.ARGMAX_WORKSPACE_BYTES)
+        self.head_argmax_ws = z(native.HEAD_ARGMAX_WORKSPACE_BYTES)
         self.rope_tab = B(c.rope_dim * 4)
         self.uniforms = make_uniforms(self.token, self.step_counter, self.hist_counter, self.history)
         # the single-launch router holds the hidden row in registers, 512 elements per piece, at most 8
@@ -345,9 +347,16 @@ class MoeRuntime:
                                arg(self.x[1]), arg(self.x[0]), arg(self.moe_ws)],
                               dict(quant, k=c.moe_inter, o=c.hidden, experts=c.n_experts, tokens=1, top_k=c.top_k, x_rows=c.top_k,
                                    has_shared=1, shared_k=c.shared_inter, has_extra=1)))
-        t.append(Dispatch(name("final_rmsnorm_lm_head"),
-                          [arg(self.x[0]), arg(w.vecs["final_norm"])] + wargs(emb) + [arg(self.logits)],
-                          dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))
+        head_args = [arg(self.x[0]), arg(w.vecs["final_norm"])] + wargs(emb) + [arg(self.logits)]
+        head_params = dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)
+        # the direct head (dispatch.py:3458-3505) as one launch where the vocabulary matrix takes the row-group GEMV
+        self.direct_head = bool(c.direct_head_argmax and native.gemv_form(c.vocab, c.hidden, 16, 64) == 1)
+        if self.direct_head:
+            t.append(Dispatch(name("final_rmsnorm_lm_head_argmax"),
+                              head_args + [arg(self.token), arg(self.head_argmax_ws), arg(self.history), arg(self.hist_counter)],
+                              head_params))
+            return t
+        t.append(Dispatch(name("final_rmsnorm_lm_head"), head_args, head_params))
         t.append(Dispatch(name("argmax_logits_decode"),
                           [arg(self.logits), arg(self.token), arg(self.argmax_ws), arg(self.history), arg(self.hist_counter)],
                           dict(vocab=c.vocab)))
@@ -357,7 +366,7 @@ class MoeRuntime:
         """name -> (buffer, dtype, zero-initialised) of every arena buffer, as the artifact describes them."""
         out = {}
         for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws",
-                     "route_idx", "rows_x", "router_ws"):
+                     "head_argmax_ws", "route_idx", "rows_x", "router_ws"):
             out[name] = (getattr(self, name), "uint32", True)
         out["x.0"], out["x.1"] = (self.x[0], "bfloat16", False), (self.x[1], "bfloat16", False)
         for name in ("xn", "q", "kva", "kvb", "att", "mid", "h", "logits", "moe_ws"):

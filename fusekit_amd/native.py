@@ -267,6 +267,17 @@ def final_rmsnorm_lm_head(x, norm_w, eps, W, logits, stream=None) -> None:
                                        _ptr(stream)))
 
 
+HEAD_ARGMAX_WORKSPACE_BYTES = 32776
+
+
+def final_rmsnorm_lm_head_argmax(x, norm_w, eps, W, logits, next_token, history, hist_counter, hist_capacity, workspace,
+                                 stream=None) -> None:
+    """The LM head that also selects the greedy token (one launch); UnsupportedError unless gemv_form(...) == 1."""
+    check(lib.fk_final_rmsnorm_lm_head_argmax(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(W.c), _ptr(logits),
+                                              _ptr(next_token), _ptr(history), _ptr(hist_counter),
+                                              C.c_uint32(hist_capacity), _ptr(workspace), _ptr(stream)))
+
+
 def rope_q_decode(q, q_norm, n_heads, head_dim, rope_dims, theta, eps=0.0, d_offset=None, offset=0, stream=None):
     check(lib.fk_rope_q_decode(_ptr(q), _ptr(q_norm), C.c_uint32(n_heads), C.c_uint32(head_dim),
                                C.c_uint32(rope_dims), C.c_float(theta), C.c_float(eps), _ptr(d_offset),

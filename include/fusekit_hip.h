@@ -228,6 +228,20 @@ fk_status fk_qgemm_swiglu(const fk_weight *Wg, const fk_weight *Wu, const uint16
  *     src/codegen/kernels/final_rmsnorm_lm_head.rs:144-629. */
 fk_status fk_final_rmsnorm_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *W,
                                    uint16_t *logits, fk_stream s);
+/* H+A the same launch also selects the greedy token: next_token = index of the largest bf16 logit, lowest
+ *     index on ties, NaN never wins, and optionally history[(*hist_counter)++] = token, exactly as
+ *     fk_argmax_logits_decode over the logits it writes.  Replaces the reference's direct head
+ *     (`<head kernel>_argmax` + `_argmax_finalize`, src/codegen/msl.rs:1674-1890, enabled per
+ *     python/fusekit_runtime/dispatch.py:1846-1866 and bound at 3458-3505) -- as ONE launch whose last block
+ *     finishes the selection; unlike the reference's form the logits are still written (300 KB beside a matrix
+ *     of hundreds of MB).  Only for matrices that fk_gemv_form reports as row-group form; anything else
+ *     FK_ERR_UNSUPPORTED (the caller keeps the two launches).  Workspace: FK_HEAD_ARGMAX_WORKSPACE_BYTES,
+ *     zeroed once; launches that share a workspace must not overlap. */
+#define FK_HEAD_ARGMAX_WORKSPACE_BYTES 32776
+fk_status fk_final_rmsnorm_lm_head_argmax(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *W,
+                                          uint16_t *logits, uint32_t *next_token, uint32_t *history,
+                                          uint32_t *hist_counter, uint32_t hist_capacity, void *workspace,
+                                          fk_stream s);
 
 /* Q0  MLX-affine quantiser on the device: w fp32 [n, k] -> packed uint32
  *     [n, k*bits/32], scales / biases bf16 [n, k/group].  Arithmetic of the
@@ -549,6 +563,8 @@ fk_status fk_xcd_check(void *workspace, fk_stream s);
  *   fusekit_rmsnorm_gateup_swiglu | fusekit_qmv_swiglu(has_norm=0)
  *       x, [norm_w], W_gate, W_up, [s_g, s_u, b_g, b_u], out   {bits, group, hidden, inter, eps, variant=0, has_norm=1}
  *   fusekit_final_rmsnorm_lm_head     x, norm_w, W [, scales, biases], logits   {bits=16, group, hidden, vocab, eps}
+ *   fusekit_final_rmsnorm_lm_head_argmax   x, norm_w, W [, scales, biases], logits, next_tok, workspace
+ *                                     [, history, hist_counter]   {bits=16, group, hidden, vocab, eps}
  *   fusekit_qgemv                     x, W [, scales, biases], [bias], y        {bits, group, m, n, has_bias=0}
  *   fusekit_argmax_logits_decode      logits, next_tok, workspace [, history, hist_counter]   {vocab}
  * Read/write slots per family follow the reference's table

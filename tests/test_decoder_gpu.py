@@ -1,6 +1,7 @@
 """Whole-decoder parity on the GPU: greedy tokens of the hipGraph-replayed decode loop
 against the CPU oracle run on the same weight bytes; plus the device quantiser (Q0) and the
 dispatcher's graph / error behaviour."""
+import dataclasses
 import os
 
 import numpy as np
@@ -194,6 +195,28 @@ def test_update_graph_bindings_repoints_kv_cache(fk, fuse_attention):
     assert "depend" in str(e.value)
     got, _, _ = rt.generate(prompt, 12)                                   # the graph is as it was
     assert got == want
+
+
+@pytest.mark.parametrize("bits,hidden", [(16, 512), (4, 2048), (8, 1024)])
+def test_direct_head_argmax_decodes_the_same_tokens(fk, bits, hidden):
+    """Vocabulary matrices that take the row-group GEMV get the LM head that selects the token itself (one task
+    instead of two); tokens and history equal those of the two-task list and of the oracle."""
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    cfg = _small_cfg(bits=bits, hidden=hidden, n_layers=2, inter=512, vocab=9001, head_dim=64, n_heads=4, n_kv=2)
+    W = DecoderWeights.random_init(cfg, seed=21)
+    prompt = rng(5).integers(0, cfg.vocab, 6).tolist()
+    a = DecoderRuntime(cfg, W)
+    assert a.direct_head and a.tasks[-1].kernel.startswith("fusekit_final_rmsnorm_lm_head_argmax")
+    b = DecoderRuntime(dataclasses.replace(cfg, direct_head_argmax=False), W)
+    assert not b.direct_head and len(b.tasks) == len(a.tasks) + 1
+    ta, _, _ = a.generate(prompt, 24)
+    tb, _, _ = b.generate(prompt, 24)
+    ref, margins = OracleDecoder(cfg, W).generate(prompt, 24)
+    assert ta == tb == ref, (ta, tb, ref, margins)
+    n = int(a.hist_counter.to_numpy(np.uint32)[0])
+    assert n == int(b.hist_counter.to_numpy(np.uint32)[0])
+    assert np.array_equal(a.history.to_numpy(np.uint32)[:n], b.history.to_numpy(np.uint32)[:n])
+    assert np.array_equal(a.logits.to_numpy(np.uint16), b.logits.to_numpy(np.uint16))
 
 
 # ---------------------------------------------------------------- persistent whole-token kernel

@@ -123,6 +123,74 @@ def test_row_group_form_with_fused_final_norm(fk):
     _check(dl.to_numpy(np.uint16), ref, oracle.linear_acc(W, ny), W, ny)
 
 
+def _greedy(logits_bf16: np.ndarray) -> int:
+    """Largest bf16 logit, lowest index on ties, NaN never wins (argmax_logits_decode.rs:63-95)."""
+    v = oracle.bf16_to_f32(logits_bf16).astype(np.float64)
+    v = np.where(np.isnan(v), -np.inf, v)
+    return int(np.argmax(v)) if np.isfinite(v).any() or np.isinf(v).any() else 0
+
+
+@pytest.mark.parametrize("bits,hidden", [(16, 2560), (4, 2560), (8, 1024), (4, 3072), (16, 2432), (4, 9728)])
+def test_direct_head_argmax_matches_the_two_launches(fk, bits, hidden):
+    """The LM head that selects the token itself: same logits, bit for bit, as the plain head, and the token the
+    stand-alone argmax picks over them -- with the winning row repeated (lowest index must win, also against a copy
+    in the last, partial group of four rows), twice in a row on one workspace, then with another winner."""
+    vocab = 20011
+    assert fk.gemv_form(vocab, hidden, bits) == 1
+    W = make_qweight(62, vocab, hidden, bits)
+    x = normal_bf16(1, hidden, 3.0)
+    gamma = normal_bf16(2, hidden, 0.1, 1.0)
+    dx, dg = fk.DeviceBuffer.from_numpy(x), fk.DeviceBuffer.from_numpy(gamma)
+    base = oracle.final_rmsnorm_lm_head(x, gamma, 1e-6, W)
+    win = _greedy(base)
+    copies = sorted({win, (win + 4097) % vocab, vocab - 1, (win + 13) % vocab})
+    for r in copies:                                      # identical rows -> identical logits
+        W.w[r] = W.w[win]
+        if bits != 16:
+            W.scales[r], W.biases[r] = W.scales[win], W.biases[win]
+    if bits == 16:
+        W.w[(copies[0] + 1) % vocab, 5] = 0x7FC0         # a NaN logit never wins
+    dW = to_device(fk, W)
+    plain = fk.DeviceBuffer(2 * vocab)
+    fk.final_rmsnorm_lm_head(dx, dg, 1e-6, dW, plain)
+    want_logits = plain.to_numpy(np.uint16)
+    tok2, ws2 = fk.zeros(4), fk.zeros(fk.ARGMAX_WORKSPACE_BYTES)
+    fk.argmax_logits_decode(plain, vocab, tok2, None, None, 0, ws2)
+    want = int(tok2.to_numpy(np.uint32)[0])
+    assert want == copies[0] == _greedy(want_logits)
+
+    ws = fk.zeros(fk.HEAD_ARGMAX_WORKSPACE_BYTES)
+    tok, hist, cnt = fk.zeros(4), fk.zeros(4 * 4), fk.zeros(4)
+    for rep in range(2):
+        dl = fk.DeviceBuffer(2 * vocab)
+        fk.final_rmsnorm_lm_head_argmax(dx, dg, 1e-6, dW, dl, tok, hist, cnt, 4, ws)
+        assert np.array_equal(dl.to_numpy(np.uint16), want_logits)
+        assert int(tok.to_numpy(np.uint32)[0]) == want
+        assert int(cnt.to_numpy(np.uint32)[0]) == rep + 1
+    assert hist.to_numpy(np.uint32).tolist() == [want, want, 0, 0]
+    assert int(ws.to_numpy(np.uint32)[0]) == 0           # the block counter is back at zero
+
+    # another activation vector: another winner through the same workspace, no history
+    x2 = normal_bf16(9, hidden, 3.0)
+    dl = fk.DeviceBuffer(2 * vocab)
+    fk.final_rmsnorm_lm_head_argmax(fk.DeviceBuffer.from_numpy(x2), dg, 1e-6, dW, dl, tok, None, None, 0, ws)
+    assert int(tok.to_numpy(np.uint32)[0]) == _greedy(dl.to_numpy(np.uint16))
+    assert int(cnt.to_numpy(np.uint32)[0]) == 2
+
+
+def test_direct_head_argmax_refuses_shapes_of_the_flat_form(fk):
+    W = make_qweight(63, 2000, 896, 4)
+    assert fk.gemv_form(2000, 896, 4) == 0
+    with pytest.raises(fk.FusekitError) as e:
+        fk.final_rmsnorm_lm_head_argmax(fk.DeviceBuffer(896 * 2), fk.DeviceBuffer(896 * 2), 1e-6, to_device(fk, W),
+                                        fk.DeviceBuffer(4000), fk.zeros(4), None, None, 0,
+                                        fk.zeros(fk.HEAD_ARGMAX_WORKSPACE_BYTES))
+    assert e.value.status == 5 and "row-group" in str(e.value)
+    with pytest.raises(fk.InvalidArgument):
+        fk.final_rmsnorm_lm_head_argmax(fk.DeviceBuffer(896 * 2), fk.DeviceBuffer(896 * 2), 1e-6, to_device(fk, W),
+                                        fk.DeviceBuffer(4000), None, None, None, 0, None)
+
+
 def test_row_group_form_is_kept_for_the_shapes_it_was_built_for(fk):
     assert fk.gemv_form(151936, 2560, 4) == 1 and fk.gemv_form(151936, 2560, 16) == 1
     assert fk.gemv_form(2560, 2560, 4) == 0          # too few rows to fill the chip four rows a wave
