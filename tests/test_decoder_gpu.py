@@ -281,32 +281,23 @@ def test_persistent_kernel_barrier_timeout_drains_and_reports(fk):
     assert "spin limit" in str(e.value)
 
 
-def test_4b_class_greedy_32_tokens_match_oracle(fk):
-    """The headline model at full size (36 layers, hidden 2560, vocab 151936, int4 g64), 32 greedy
-    steps against the oracle on the same weight bytes.
+def _teacher_forced_against_oracle(cfg, W, prompt, n, min_exact, logits_bar, window_ulps=2.0, min_in_two_ulps=1.0):
+    """n greedy steps of the full-size model against the oracle on the same weight bytes.
 
     Logits are bf16 and the weights are random, so among 151936 candidates the two largest logits
     are often equal or one bf16 ulp apart (margins are printed).  Free-running equality is required
     as long as the oracle's margin is clear; at a near-tie the GPU token must be one of the oracle's
     candidates within two ulps of its maximum (either logit may sit on a rounding edge and move by
     one ulp with the fp32 summation order), and the run continues teacher-forced on the oracle's
-    tokens so that every one of the 32 steps is checked.
-
-    The per-kernel bar (rel-L2 <= 1e-2) does not carry over to 36 stacked layers: at K = 2560..9728
-    fp32 accumulation (any order) and the oracle's double accumulation round ~1-2 % of a GEMV's
-    outputs to neighbouring bf16 values, which measures 1.7e-3 on the logits after one layer and
-    grows to ~3e-2 after 36 (the same stack at hidden 256 agrees bit for bit).  The last step's
-    logits are held to 5e-2."""
-    from fusekit_amd.decoder import DENSE_4B, DecoderConfig, DecoderRuntime, DecoderWeights
-    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=128)
-    W = DecoderWeights.random_init(cfg, seed=0)
+    tokens so that every one of the n steps is checked.  window_ulps > 2 (long runs): the oracle's logit of the
+    GPU's token lies within that many ulps of the oracle's maximum at every step, and within 2 at the fraction
+    min_in_two_ulps of them."""
+    from fusekit_amd.decoder import DecoderRuntime
     rt = DecoderRuntime(cfg, W)
     od = OracleDecoder(cfg, W)
-    prompt = rng(0).integers(0, cfg.vocab, 4).tolist()
-    n = 32
-    got_free, _, _ = rt.generate(prompt, n)
+    got_free, _, _ = rt.generate(prompt, min(n, 32))
 
-    ref, margins, cands = [], [], []
+    ref, margins, cands, wide = [], [], [], []
     seq = list(prompt)
     for i in range(len(prompt) + n - 1):
         nxt, m, logits = od.step(seq[i], i, want_logits=True)
@@ -315,27 +306,74 @@ def test_4b_class_greedy_32_tokens_match_oracle(fk):
             top = float(f.max())
             ulp = 2.0 ** (np.floor(np.log2(abs(top))) - 7)
             ref.append(nxt); margins.append(m); cands.append(set(np.nonzero(f >= top - 2 * ulp)[0].tolist()))
+            wide.append({int(t): (top - float(f[t])) / ulp for t in np.nonzero(f >= top - window_ulps * ulp)[0]})
             seq.append(nxt)
-    print("oracle margins:", ["%.3g" % m for m in margins])
-    print("candidates per step:", [len(c) for c in cands])
+    print("oracle margins:", ["%.3g" % m for m in margins[:48]])
+    print("candidates per step:", [len(c) for c in cands[:48]])
 
     preds, _ = rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, seq[:-1])
     preds = preds[len(prompt) - 1:]
     exact = sum(int(g == r) for g, r in zip(preds, ref))
     print(f"teacher-forced: {exact}/{n} steps pick the oracle's token")
+    in_two = 0
     for i, (g, r) in enumerate(zip(preds, ref)):
-        assert g in cands[i], f"step {i}: gpu {g} is not among the oracle's near-maximal tokens {sorted(cands[i])} (oracle {r})"
-        if len(cands[i]) == 1:
+        assert g in wide[i], f"step {i}: gpu {g} is not among the oracle's near-maximal tokens {wide[i]} (oracle {r})"
+        in_two += int(g in cands[i])
+        if len(wide[i]) == 1:
             assert g == r
+    print(f"within two ulps of the oracle's maximum: {in_two}/{n}; largest deficit "
+          f"{max(wide[i][g] for i, g in enumerate(preds)):.1f} ulps")
+    assert in_two >= min_in_two_ulps * n
     # free-running: identical up to the first step that has more than one candidate
     first_tie = next((i for i, c in enumerate(cands) if len(c) > 1), n)
-    assert got_free[:first_tie] == ref[:first_tie]
-    assert exact >= n - 6
+    k = min(first_tie, len(got_free))
+    assert got_free[:k] == ref[:k]
+    assert exact >= min_exact
     f_got = oracle.bf16_to_f32(rt.logits.to_numpy(np.uint16)).astype(np.float64)
     f_ref = oracle.bf16_to_f32(logits).astype(np.float64)
     rel = np.linalg.norm(f_got - f_ref) / np.linalg.norm(f_ref)
     print(f"last-step logits rel-L2 {rel:.3e}")
-    assert rel <= 5e-2
+    assert rel <= logits_bar
+    return rt
+
+
+def test_4b_class_greedy_32_tokens_match_oracle(fk):
+    """The headline model at full size (36 layers, hidden 2560, vocab 151936, int4 g64), 32 greedy
+    steps against the oracle on the same weight bytes (see _teacher_forced_against_oracle).
+
+    The per-kernel bar (rel-L2 <= 1e-2) does not carry over to 36 stacked layers: at K = 2560..9728
+    fp32 accumulation (any order) and the oracle's double accumulation round ~1-2 % of a GEMV's
+    outputs to neighbouring bf16 values, which measures 1.7e-3 on the logits after one layer and
+    grows to ~3e-2 after 36 (the same stack at hidden 256 agrees bit for bit).  The last step's
+    logits are held to 5e-2."""
+    from fusekit_amd.decoder import DENSE_4B, DecoderConfig, DecoderWeights
+    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=128)
+    W = DecoderWeights.random_init(cfg, seed=0)
+    _teacher_forced_against_oracle(cfg, W, rng(0).integers(0, cfg.vocab, 4).tolist(), 32, 26, 5e-2)
+
+
+@pytest.mark.parametrize("bits", [8, 16])
+def test_4b_class_int8_and_bf16_weights_match_oracle(fk, bits):
+    """The same model with 8-bit g64 and with dense bf16 weights at full size (4.3 / 8 GB): 12 greedy steps, every
+    one checked against the oracle as above."""
+    from fusekit_amd.decoder import DENSE_4B, DecoderConfig, DecoderWeights
+    cfg = DecoderConfig(**DENSE_4B, bits=bits, capacity=128)
+    W = DecoderWeights.random_init(cfg, seed=1)
+    rt = _teacher_forced_against_oracle(cfg, W, rng(1).integers(0, cfg.vocab, 4).tolist(), 12, 9, 5e-2)
+    assert rt.xcd and rt.direct_head
+
+
+def test_4b_class_512_tokens_at_full_size_follow_the_oracle(fk):
+    """The 512-token run of the headline configuration at full size: a 4-token prompt and 512 decode steps (context
+    up to 515 in a 1024-row cache), the GPU fed the oracle's tokens, every step's choice checked against the
+    oracle's near-maximal set; at least 85 % of the steps pick the oracle's very token.  The stack's fp32-versus-
+    double drift (3e-2 relative L2 on the logits, about 1.3 bf16 ulps rms at the top of the distribution) makes the
+    two-ulp window a statistical one over 512 steps: it is asserted for 99 % of them (measured: 511 of 512, the other step 4 ulps), six ulps for all."""
+    from fusekit_amd.decoder import DENSE_4B, DecoderConfig, DecoderWeights
+    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=1024)
+    W = DecoderWeights.random_init(cfg, seed=0)
+    _teacher_forced_against_oracle(cfg, W, rng(2).integers(0, cfg.vocab, 4).tolist(), 512, 435, 5e-2, window_ulps=6.0,
+                                   min_in_two_ulps=0.99)
 
 
 def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk):
