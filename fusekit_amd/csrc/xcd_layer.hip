@@ -659,6 +659,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uin
     meta_store<KIND, kAttnStream, true>(mmq, ti, meta);
     meta_fetch<KIND, kAttnStream, true>(a.wo, to, ti, mmo, sync.xcd);  // not needed before the attention is done
     __syncthreads();
+    FK_XCD_STAMP(0, 13);
 
     // ---- q / k / v rows of this XCD's KV head; the o_proj slice is requested behind their last pass ----
     if (streams) {
@@ -668,7 +669,9 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uin
         else
             request_o();
     }
+    FK_XCD_STAMP(0, 14);
     __syncthreads();
+    FK_XCD_STAMP(0, 15);
     if (pr_n) {
         uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
         tile_rows<false>(tq, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
@@ -897,7 +900,7 @@ fk_status xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint
 
 namespace {
 
-constexpr int kNlQkv = 6, kNlO = 4, kNlGu = 6, kNlDown = 6;  // 16-byte requests per streaming thread and pass
+constexpr int kNlQkv = 5, kNlO = 3, kNlGu = 6, kNlDown = 6;  // 16-byte requests per streaming thread and pass
 constexpr int kNlGuToken = 4;  // the whole-token launch holds both phases' registers: shallower gate / up passes
 
 uint32_t ilog2u(uint32_t v) {
