@@ -238,7 +238,7 @@ class ArtifactRuntime:
         u = graph["uniforms"]
         self.uniforms = make_uniforms(self.scratch[u["token"]], self.scratch[u["step_counter"]],
                                       self.scratch[u["hist_counter"]], self.scratch[u["history"]])
-        self.graph = self.d.build_graph(self.tasks)
+        self.graph = self.d.build_decode_graph(self.tasks, False)
         self.model_config = graph["model_config"]
         self._weights = weights  # keeps the parameter buffers alive
         # prefill_mN variants (manifest `variants`, one task graph each): scratch buffers are shared by role
@@ -258,7 +258,7 @@ class ArtifactRuntime:
                     raise ValueError(f"variant {v['name']}: scratch {sb['role_name']} is larger than in the decode graph")
             vu = vg["uniforms"]
             self.variants[int(v["active_m"])] = dict(
-                graph=self.d.build_graph(self._tasks_of(vg)), tokens=self.scratch[vu["tokens"]],
+                graph=self.d.build_decode_graph(self._tasks_of(vg), False), tokens=self.scratch[vu["tokens"]],
                 offset=self.scratch[vu["offset"]], kv_len=self.scratch[vu["kv_len"]], token=self.scratch[vu["token"]])
 
     def _tasks_of(self, graph: dict) -> List[Dispatch]:

@@ -1943,7 +1943,14 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
 
 fk_status fk_build_decode_graph(fk_handle h, const fk_dispatch* list, size_t n, int persistent, uint32_t spin_limit,
                                 uint32_t* graph_id) {
-    if (!persistent) return fk_build_graph(h, list, n, nullptr, graph_id);
+    if (!persistent) {
+        // List order, one node behind the other.  Every launch of a decode pipeline fills the chip, so independent
+        // tasks gain nothing from running side by side, while a graph that forks anywhere (step_init beside the
+        // embedding lookup is enough) is replayed through several queues and costs about 70 us more per replay.
+        if (!list || n == 0) return set_error(FK_ERR_INVALID, "empty dispatch list or null out");
+        const std::vector<uint8_t> chain(n, 1);
+        return fk_build_graph(h, list, n, chain.data(), graph_id);
+    }
     DispatcherState* ds;
     FK_TRY(get_dispatcher(h, &ds));
     if (!list || n == 0 || !graph_id) return set_error(FK_ERR_INVALID, "empty dispatch list or null out");

@@ -246,7 +246,7 @@ class DecoderRuntime:
         self.tasks = self.build_tasks()
         # persistent: the same task list, run by one whole-token kernel per replay
         self.graph = (self.d.build_decode_graph(self.tasks, True, spin_limit) if persistent
-                      else self.d.build_graph(self.tasks))
+                      else self.d.build_decode_graph(self.tasks, False))
 
     # -- task list -------------------------------------------------------------------
     def _wargs(self, W: DeviceWeight):

@@ -218,7 +218,7 @@ class MoeRuntime:
         self.router_ws = z(4 * (c.n_experts + 1))
         self._rows_variants: Dict[int, "MoeRowsVariant"] = {}
         self.tasks = self.build_tasks()
-        self.graph = self.d.build_graph(self.tasks)
+        self.graph = self.d.build_decode_graph(self.tasks, False)
 
     def build_tasks(self) -> List[Dispatch]:
         c, w = self.cfg, self.w
@@ -461,7 +461,7 @@ class MoeRowsVariant:
         pb, cb = native.sdpa_workspace_bytes(c.n_heads, c.n_heads, c.qk_dim, c.v_dim, c.capacity)
         self.parts, self.counters = B(max(pb, 4) * m), z(max(cb, 4) * m)
         self.tasks = self._build()
-        self.graph = rt.d.build_graph(self.tasks)
+        self.graph = rt.d.build_decode_graph(self.tasks, False)
 
     def _build(self) -> List[Dispatch]:
         rt, c, w, m = self.rt, self.rt.cfg, self.rt.w, self.m

@@ -44,7 +44,7 @@ class PrefillVariant:
                  for n, k in ((c.n_q, c.hidden), (c.n_kvd, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
         self.ws = B(2 * ws)
         self.tasks = self._build()
-        self.graph = rt.d.build_graph(self.tasks)
+        self.graph = rt.d.build_decode_graph(self.tasks, False)
 
     def scratch(self) -> Dict[str, DeviceBuffer]:
         """Buffers private to the variant, by the role name the artifact gives them."""

@@ -119,12 +119,15 @@ def test_graph_edges_follow_hazards(fk):
     idx = {n.rsplit("_f", 1)[0]: i for i, n in enumerate(names)}
     qkv, rq, rkv, sd = (idx[f"fusekit_{k}"] for k in ("rmsnorm_qkv", "rope_q_decode", "rope_kv_cache_store_decode",
                                                        "sdpa_decode"))
-    deps = {i: rt.d.node_deps(rt.graph, i) for i in range(len(names))}
+    g = rt.d.build_graph(rt.tasks)                      # edges from the read/write tables
+    deps = {i: rt.d.node_deps(g, i) for i in range(len(names))}
     assert qkv in deps[rq] and qkv in deps[rkv]
     assert rq not in deps[rkv] and rkv not in deps[rq]
     assert rq in deps[sd] and rkv in deps[sd]
-    n, e = rt.d.graph_info(rt.graph)
+    n, e = rt.d.graph_info(g)
     assert n == len(names) and e < 3 * n
+    # the decoder's own graph runs the same tasks in list order: one node behind the other
+    assert [rt.d.node_deps(rt.graph, i) for i in range(len(names))] == [[]] + [[i] for i in range(len(names) - 1)]
 
 
 def test_dispatcher_error_paths(fk, tmp_path):
@@ -190,10 +193,11 @@ def test_update_graph_bindings_repoints_kv_cache(fk, fuse_attention):
     prod = next(i for i, t in enumerate(rt.tasks) if "final_rmsnorm_lm_head" in t.kernel)
     slot = next(s for s, (p, n) in enumerate(rt.tasks[prod].args) if p == rt.logits.ptr)
     other = fk.zeros(rt.logits.nbytes)
+    derived = rt.d.build_graph(rt.tasks)                                  # edges from the read/write tables
     with pytest.raises(fk.FusekitError) as e:
-        rt.d.update_graph_bindings(rt.graph, [(prod, slot, other.ptr, rt.logits.nbytes)])
+        rt.d.update_graph_bindings(derived, [(prod, slot, other.ptr, rt.logits.nbytes)])
     assert "depend" in str(e.value)
-    got, _, _ = rt.generate(prompt, 12)                                   # the graph is as it was
+    got, _, _ = rt.generate(prompt, 12)                                   # the decoder's graph is as it was
     assert got == want
 
 
