@@ -54,7 +54,8 @@ fk_status device_facts(const DeviceFacts** out) {
 
 fk_status run_launch(const Launch& l, hipStream_t s) {
     if (!l.func) return FK_OK;  // an empty launch (a planner that needed fewer kernels than its caller offers)
-    void* params[1] = {const_cast<unsigned char*>(l.args)};
+    void* params[kMaxKernelParams];
+    const_cast<Launch&>(l).params(params);
     FK_HIP(hipLaunchKernel(l.func, l.grid, l.block, params, l.shmem, s));
     for (const Launch& f : l.then) FK_TRY(run_launch(f, s));
     return FK_OK;

@@ -1337,7 +1337,7 @@ hipKernelNodeParams launch_params(Launch& l, void** slot) {
     p.gridDim = l.grid;
     p.blockDim = l.block;
     p.sharedMemBytes = l.shmem;
-    *slot = l.args;
+    l.params(slot);  // `slot` holds kMaxKernelParams entries
     p.kernelParams = slot;
     p.extra = nullptr;
     return p;
@@ -1914,8 +1914,8 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
                         hipGraphNode_t dn = g->nodes[j].last();
                         if (std::find(deps.begin(), deps.end(), dn) == deps.end()) deps.push_back(dn);
                     }
-            void* slot = nullptr;
-            hipKernelNodeParams p = launch_params(run.launch, &slot);
+            void* slot[kMaxKernelParams];
+            hipKernelNodeParams p = launch_params(run.launch, slot);
             FK_HIP(hipGraphAddKernelNode(&run.node, g->graph, deps.data(), deps.size(), &p));
             nd.node = run.node;
             continue;
@@ -1925,13 +1925,13 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
             hipGraphNode_t dn = g->nodes[j].last();
             if (std::find(deps.begin(), deps.end(), dn) == deps.end()) deps.push_back(dn);
         }
-        void* slot = nullptr;
-        hipKernelNodeParams p = node_params(nd, &slot);
+        void* slot[kMaxKernelParams];
+        hipKernelNodeParams p = node_params(nd, slot);
         FK_HIP(hipGraphAddKernelNode(&nd.node, g->graph, deps.data(), deps.size(), &p));
         nd.tail.resize(nd.launch.then.size());
         for (size_t f = 0; f < nd.launch.then.size(); ++f) {
             hipGraphNode_t prev = f ? nd.tail[f - 1] : nd.node;
-            hipKernelNodeParams fp = launch_params(nd.launch.then[f], &slot);
+            hipKernelNodeParams fp = launch_params(nd.launch.then[f], slot);
             FK_HIP(hipGraphAddKernelNode(&nd.tail[f], g->graph, &prev, 1, &fp));
         }
     }
@@ -2119,11 +2119,11 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
             FK_HIP(hipMemcpy(dst, lt.args, lt.args_size, hipMemcpyHostToDevice));
             continue;
         }
-        void* slot = nullptr;
-        hipKernelNodeParams p = node_params(nd, &slot);
+        void* slot[kMaxKernelParams];
+        hipKernelNodeParams p = node_params(nd, slot);
         FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.node, &p));
         for (size_t f = 0; f < nd.tail.size(); ++f) {
-            hipKernelNodeParams fp = launch_params(nd.launch.then[f], &slot);
+            hipKernelNodeParams fp = launch_params(nd.launch.then[f], slot);
             FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.tail[f], &fp));
         }
     }

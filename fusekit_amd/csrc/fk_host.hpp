@@ -24,13 +24,33 @@ struct Launch {
     // builder treat the chain as one unit.
     std::vector<Launch> then;
 
+    // Kernel parameters AHEAD of the argument block (at most kMaxLead, 8 bytes or less each): what a kernel needs for
+    // its very first requests.  Leading scalar parameters can be handed to a wave in registers at its launch (kernel
+    // argument preload), a by-value block cannot: its fields arrive with a load, one trip to memory into the kernel.
+    static constexpr int kMaxLead = 4;
+    uint32_t n_lead = 0;
+    uint64_t lead[kMaxLead] = {0, 0, 0, 0};
+
     template <typename T>
     void set_args(const T& a) {
         static_assert(sizeof(T) <= sizeof(args), "argument block too large");
         memcpy(args, &a, sizeof(T));
         args_size = sizeof(T);
     }
+    template <typename T>
+    void add_lead(T v) {
+        static_assert(sizeof(T) <= 8, "a leading parameter is a pointer or a scalar");
+        uint64_t w = 0;
+        memcpy(&w, &v, sizeof(T));
+        lead[n_lead++] = w;
+    }
+    // The kernelParams array of this launch (kMaxLead + 1 entries at most); valid while the Launch is.
+    void params(void** out) {
+        for (uint32_t i = 0; i < n_lead; ++i) out[i] = &lead[i];
+        out[n_lead] = args;
+    }
 };
+constexpr int kMaxKernelParams = Launch::kMaxLead + 1;
 
 struct DeviceFacts {
     int cus = 0;

@@ -147,6 +147,16 @@ struct InputRegs {
     uint4 sv[kInGroups][4], rv[kInGroups], nw[kInGroups];
 };
 
+// What input_request reads of a launch's input, as leading kernel parameters: they reach a wave in registers when it
+// starts (kernel argument preload), so the sum row is requested before the argument block -- one trip to memory
+// away -- has arrived.
+struct XcdInputLead {
+    const long long* sums;
+    const uint16_t* residual;
+    const uint16_t* norm_w;
+    uint32_t hidden;
+};
+
 // Zeroes the sum row the launch after this one adds into (16-byte units spread over the grid).  Called once the
 // input has been consumed: a wave's memory counter completes in order, and in the whole-token launch these are
 // write-through stores (a line left dirty in this XCD's L2 would later overwrite the other XCDs' additions) that
@@ -186,6 +196,35 @@ __device__ __forceinline__ void input_request(const IN& in, InputRegs& r, const 
             }
             r.rv[i] = (TOKEN && xres) ? xres[tc] : r8[tc];
             r.nw[i] = w8[tc];
+        }
+    }
+}
+
+// Placed behind the LAST request of a launch's start-up, before input_stage.  input_request and input_stage test
+// the same (wave-uniform) conditions, and without this the compiler merges the two regions: the conversion of the
+// sum row ends up directly behind its loads, inside the first condition, and the wave then sits out a whole trip
+// to memory -- twice, once per group -- before it requests the residual, the scales and biases and its first pass
+// of weights.  The empty statement makes every input register a value that exists only from here on, so the
+// arithmetic cannot move ahead of the requests in between.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void pin128(uint4& v) {  // as ONE 128-bit register operand: the load's tuple stays whole
+    u32x4_t t = {v.x, v.y, v.z, v.w};
+    asm volatile("" : "+v"(t));
+    v = make_uint4(t.x, t.y, t.z, t.w);
+}
+template <typename IN>
+__device__ __forceinline__ void input_pin(const IN& in, InputRegs& r) {
+    const uint32_t n8 = in.hidden >> 3;
+#pragma unroll
+    for (int i = 0; i < kInGroups; ++i) {
+        const uint32_t t = threadIdx.x + i * kBlock, sec = t >> 6;
+        if (sec * kWave < n8) {  // as in input_request / input_stage: registers of a skipped group hold nothing
+            if (in.sums) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) pin128(r.sv[i][k]);
+            }
+            pin128(r.rv[i]);
+            pin128(r.nw[i]);
         }
     }
 }
@@ -500,9 +539,11 @@ constexpr int kMlpBlock = kBlock;
 
 // One MLP phase of one block.  `sync` carries the block's XCD, slot and hand-over epoch; `xres_in` / `xres_out`:
 // the residual row in LDS (token kernel only).
-template <WKind KIND, int NLA, int NLB, bool TOKEN, typename ARGS>
-__device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, XcdSync& sync, uint4* lds_raw, const uint4* xres_in,
-                                              uint4* xres_out) {
+// EARLY: the caller has already issued input_request into `inr` (the stand-alone launch does so before anything
+// else, from its leading parameters).
+template <WKind KIND, int NLA, int NLB, bool TOKEN, bool EARLY, typename ARGS, typename LEAD>
+__device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, InputRegs& inr, XcdSync& sync, uint4* lds_raw,
+                                              const uint4* xres_in, uint4* xres_out) {
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     uint4* xs = lds_raw;
@@ -527,11 +568,10 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, XcdSync& sync, uint
     TileRegs<NLB> rd;
     TilePos<NLA> pg;
     TilePos<NLB> pd;
-    InputRegs inr;
     // Requested now, behind the input: the groups' scales and biases and the first pass of gate / up -- a few
     // KiB per CU.  The later passes stream while the earlier ones are consumed; the down_proj slice is queued
     // behind the last of them.
-    input_request<TOKEN>(a.in, inr, xres_in);
+    if constexpr (!EARLY) input_request<TOKEN>(lead, inr, xres_in);
     tile_pos_init<NLA, kBlock>(a.gate, tg, tid, pg);
     tile_pos_init<NLB, kBlock>(a.down, td, tid, pd);
     meta_fetch<KIND, kBlock, true>(a.gate, tg, tid, mg);
@@ -539,6 +579,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, XcdSync& sync, uint
     tile_load<KIND, NLA, kBlock>(a.gate, tg, pg, rg);
     tile_load<KIND, NLA, kBlock>(a.up, tg, pg, ru);
     FK_XCD_STAMP(1, 1);
+    input_pin(lead, inr);
     input_stage<KIND, 1>(a.in, inr, xs, sx, a.gate.cpr, red, xres_out);
     FK_XCD_STAMP(1, 5);
     input_clear<TOKEN>(a.in);
@@ -600,18 +641,23 @@ __device__ __forceinline__ XcdSync xcd_sync_init(XcdControl* ctl, uint32_t spin_
 }
 
 template <WKind KIND, int NLA, int NLB>
-__global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const XcdMlpArgs a) {
+__global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const long long* sums, const uint16_t* residual,
+                                                               const uint16_t* norm_w, uint32_t hidden, const XcdMlpArgs a) {
     extern __shared__ uint4 lds_raw[];
+    // The input is requested from the leading parameters before the argument block is touched.
+    const XcdInputLead lead{sums, residual, norm_w, hidden};
+    InputRegs inr;
+    input_request<false>(lead, inr, nullptr);
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
-    xcd_mlp_phase<KIND, NLA, NLB, false>(a, sync, lds_raw, nullptr, nullptr);
+    xcd_mlp_phase<KIND, NLA, NLB, false, true>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
 }
 
 // =============================================================================================== attention launch
 constexpr int kAttnStream = kBlock;
 
-template <WKind KIND, int NLA, int NLB, bool TOKEN, typename ARGS>
-__device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uint4* lds_raw, const uint4* xres_in,
-                                               uint4* xres_out) {
+template <WKind KIND, int NLA, int NLB, bool TOKEN, bool EARLY, typename ARGS, typename LEAD>
+__device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, InputRegs& inr, XcdSync& sync, uint4* lds_raw,
+                                               const uint4* xres_in, uint4* xres_out) {
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats, att_elems = a.att_elems;
     (void)att_elems;
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
@@ -621,7 +667,9 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uin
     uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]; two used
     uint16_t* att = reinterpret_cast<uint16_t*>(meta + 3 * kMetaWords);
 
-    const uint32_t kv_len0 = *a.sdpa.kv_len_ptr;
+    // Requested now, looked at only behind the start-up requests (the pin below): used at once, the wave would sit
+    // out this load's trip to memory before it has asked for anything else.
+    uint32_t kv_len_raw = *a.sdpa.kv_len_ptr;
     const uint32_t tid = threadIdx.x, ti = tid;
     constexpr bool streams = true;
     float* red = reinterpret_cast<float*>(att + ((att_elems + 7u) & ~7u));  // [16]
@@ -646,13 +694,15 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uin
     TileRegs<NLB> ro;
     TilePos<NLA> pq;
     TilePos<NLB> po;
-    InputRegs inr;
-    input_request<TOKEN>(a.in, inr, xres_in);
+    if constexpr (!EARLY) input_request<TOKEN>(lead, inr, xres_in);
     tile_pos_init<NLA, kAttnStream>(mq, tq, ti, pq);
     tile_pos_init<NLB, kAttnStream>(a.wo, to, ti, po);
     meta_fetch<KIND, kAttnStream, true>(mq, tq, ti, mmq);
     tile_load<KIND, NLA, kAttnStream>(mq, tq, pq, rq);
     FK_XCD_STAMP(0, 1);
+    asm volatile("" : "+v"(kv_len_raw));
+    const uint32_t kv_len0 = __builtin_amdgcn_readfirstlane(kv_len_raw);
+    input_pin(lead, inr);
     input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red, xres_out);
     FK_XCD_STAMP(0, 5);
     input_clear<TOKEN>(a.in);
@@ -768,10 +818,14 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, XcdSync& sync, uin
 }
 
 template <WKind KIND, int NLA, int NLB>
-__global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const XcdAttnArgs a) {
+__global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const long long* sums, const uint16_t* residual,
+                                                             const uint16_t* norm_w, uint32_t hidden, const XcdAttnArgs a) {
     extern __shared__ uint4 lds_raw[];
+    const XcdInputLead lead{sums, residual, norm_w, hidden};
+    InputRegs inr;
+    input_request<false>(lead, inr, nullptr);
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
-    xcd_attn_phase<KIND, NLA, NLB, false>(a, sync, lds_raw, nullptr, nullptr);
+    xcd_attn_phase<KIND, NLA, NLB, false, true>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
 }
 
 // ---- the whole token in one launch --------------------------------------------------------------------------
@@ -860,10 +914,16 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_token_kernel(const XcdTokenArgs
     };
     for (uint32_t l = 0; l < t.n_layers; ++l) {
         touch(t.mlp + l, sizeof(XcdMlpArgs));
-        xcd_attn_phase<KIND, NLQ, NLO, true>(*(const ConstAttn*)(t.attn + l), sync, lds_raw, l ? xres : nullptr, xres);
+        {
+            InputRegs inr;
+            xcd_attn_phase<KIND, NLQ, NLO, true, false>(*(const ConstAttn*)(t.attn + l), ((const ConstAttn*)(t.attn + l))->in, inr, sync, lds_raw, l ? xres : nullptr, xres);
+        }
         if (!xcd_global_barrier(sync, gs)) return;
         if (l + 1 < t.n_layers) touch(t.attn + l + 1, sizeof(XcdAttnArgs));
-        xcd_mlp_phase<KIND, NLG, NLD, true>(*(const ConstMlp*)(t.mlp + l), sync, lds_raw, xres, xres);
+        {
+            InputRegs inr;
+            xcd_mlp_phase<KIND, NLG, NLD, true, false>(*(const ConstMlp*)(t.mlp + l), ((const ConstMlp*)(t.mlp + l))->in, inr, sync, lds_raw, xres, xres);
+        }
         if (l + 1 < t.n_layers && !xcd_global_barrier(sync, gs)) return;
     }
 }
@@ -1040,6 +1100,11 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     a.cs_max = lp.cs_max;
     a.work_floats = lp.work_floats;
     out->set_args(a);
+    out->n_lead = 0;
+    out->add_lead(a.in.sums);
+    out->add_lead(a.in.residual);
+    out->add_lead(a.in.norm_w);
+    out->add_lead(a.in.hidden);
     return FK_OK;
 }
 
@@ -1128,6 +1193,11 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     a.work_floats = lp.work_floats;
     a.att_elems = lp.att_elems;
     out->set_args(a);
+    out->n_lead = 0;
+    out->add_lead(a.in.sums);
+    out->add_lead(a.in.residual);
+    out->add_lead(a.in.norm_w);
+    out->add_lead(a.in.hidden);
     return FK_OK;
 }
 
