@@ -219,6 +219,10 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
                 out->set_args(a);
             else
                 out->set_args(static_cast<const GemvArgs&>(a));
+            out->n_lead = 0;
+            out->add_lead(a.x);
+            out->add_lead(a.norm_w);
+            out->add_lead(a.K);
             if (lds > 48 * 1024) FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             return FK_OK;
         }
@@ -332,6 +336,10 @@ fk_status plan_gemv(const GemvRequest& rq, Launch* out) {
     out->block = dim3(kGemvBlock, 1, 1);
     out->shmem = lds;
     out->set_args(a);
+    out->n_lead = 0;
+    out->add_lead(a.x);
+    out->add_lead(a.norm_w);
+    out->add_lead(a.K);
     if (lds > 48 * 1024) {
         FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     }

@@ -151,6 +151,11 @@ constexpr int kStageRegs = 5;
 // stand-alone kernel calls this BEFORE the weight prefetch: loads return in issue
 // order, so x queued behind a batch of weight rows would wait for HBM although it
 // sits in cache.
+struct StageLead {  // what stage_fetch reads, as a kernel's leading parameters
+    const uint16_t* x;
+    const uint16_t* norm_w;
+    uint32_t K;
+};
 template <typename ARGS>
 __device__ __forceinline__ void stage_fetch(const ARGS& a, uint4 (&xr)[kStageRegs], uint4 (&wr)[kStageRegs]) {
     // Straight-line on purpose (clamped index, the norm weight replaced by x itself
@@ -478,14 +483,17 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
     gemv_run<KIND, NSEG, COH, ARGS>(a, block_id, n_blocks, lds_raw, wa, sa, ba, xr, wr);
 }
 
+// x, norm_w and K also travel as LEADING parameters: those reach a wave in registers at its launch (kernel argument
+// preload), so the activations are requested before the argument block -- one trip to memory away -- has arrived.
 template <WKind KIND, int NSEG>
-__global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const GemvArgs a) {
+__global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const uint16_t* x, const uint16_t* norm_w, uint32_t K,
+                                                                 const GemvArgs a) {
     extern __shared__ uint4 lds_raw[];
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
     uint4 xr[kStageRegs], wr[kStageRegs];
     FK_GEMV_STAMP(0);
-    stage_fetch(a, xr, wr);                                // activations first: they return first
+    stage_fetch(StageLead{x, norm_w, K}, xr, wr);          // activations first: they return first
     gemv_prefetch<KIND, NSEG>(a, blockIdx.x, wa, sa, ba);  // weights stream while x is staged
     gemv_run<KIND, NSEG, false>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba, xr, wr);
 }

@@ -101,7 +101,8 @@ struct GemvArgmaxArgs : GemvArgs {
 };
 
 template <WKind KIND, int NB, bool TAIL, bool ARGMAX = false>
-__global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const std::conditional_t<ARGMAX, GemvArgmaxArgs, GemvArgs> a) {
+__global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const uint16_t* x, const uint16_t* norm_w, uint32_t K,
+                                                               const std::conditional_t<ARGMAX, GemvArgmaxArgs, GemvArgs> a) {
     extern __shared__ uint4 lds_raw[];
     constexpr int PIECES = ChunkTraits<KIND>::kPieces;
     constexpr bool QUANT = KIND != W_BF16;
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const std::condit
     constexpr uint32_t GPB = 16u >> GSH;  // groups per column block
 
     uint4 xr[kStageRegs], wr[kStageRegs];
-    stage_fetch(a, xr, wr);
+    stage_fetch(StageLead{x, norm_w, K}, xr, wr);  // from the leading parameters: before the argument block arrives
 
     const uint32_t lane = threadIdx.x & (kWave - 1), l16 = lane & (kRowLanes - 1), rg = lane / kRowLanes;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
