@@ -80,42 +80,44 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
     const uint32_t route = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - route * a.blocks_per_route;
     const bool extra = route >= a.n_routes;     // uniform per block
     const uint32_t lookup = extra ? 0u : route;
-    uint32_t e, row;
+    uint32_t e = 0, row = 0;
     float routed_weight = 1.0f;
-    if (a.logits) {
-        row = 0;
-        e = 0;
-        if (!extra) {
-            const uint32_t lane = threadIdx.x & (kWave - 1);
-            float x[4];
-            uint32_t p[4];
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                const uint32_t i = lane + j * kWave;
-                x[j] = i < a.n_experts ? bf16_bits_to_f32(a.logits[i]) : -INFINITY;
-            }
-            route_candidates(x, a.n_experts, lane, p);
-            float best = 0.f;
-            for (uint32_t k = 0; k <= route; ++k) route_take_best(p, best, e);
-            const uint32_t wbits = f32_to_bf16_bits(best * bf16_bits_to_f32(a.route_scale[0]));
-            if (sub == 0 && threadIdx.x == 0) {
-                a.idx_out[route] = e;
-                a.weight_out[route] = (uint16_t)wbits;
-            }
-            e = __builtin_amdgcn_readfirstlane(e);
-            if (a.route_weight) routed_weight = bf16_bits_to_f32(wbits);   // any non-null pointer: apply the weight here
-        }
-    } else {
+    if (!a.logits) {
         e = a.expert_idx[lookup];
         e = e < a.n_experts ? e : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
         row = a.row_idx ? a.row_idx[lookup] : lookup;
         row = row < a.n_x_rows ? row : a.n_x_rows - 1;
         if (a.route_weight && !extra) routed_weight = bf16_bits_to_f32(a.route_weight[lookup]);
     }
-    if (extra) {
-        e = route - a.n_routes;
-        row = 0;
+    if (extra) row = 0;
+    // The activation row is known here in both forms (row 0 when the launch ranks the logits itself): it is
+    // requested BEFORE the ranking, whose logits cost a trip to memory and whose result only the weight addresses
+    // need.
+    uint4 xr[kStageRegs], wr[kStageRegs];
+    stage_fetch(StageLead{a.g.x + (size_t)row * a.g.K, nullptr, a.g.K}, xr, wr);
+    if (a.logits && !extra) {
+        const uint32_t lane = threadIdx.x & (kWave - 1);
+        float x[4];
+        uint32_t p[4];
+        const uint32_t scale_bits = a.route_scale[0];  // requested with the logits, used behind the ranking
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {  // clamped index, straight-line: four requests, one wait
+            const uint32_t i = lane + j * kWave;
+            const float v = bf16_bits_to_f32(a.logits[i < a.n_experts ? i : 0u]);
+            x[j] = i < a.n_experts ? v : -INFINITY;
+        }
+        route_candidates(x, a.n_experts, lane, p);
+        float best = 0.f;
+        for (uint32_t k = 0; k <= route; ++k) route_take_best(p, best, e);
+        const uint32_t wbits = f32_to_bf16_bits(best * bf16_bits_to_f32(scale_bits));
+        if (sub == 0 && threadIdx.x == 0) {
+            a.idx_out[route] = e;
+            a.weight_out[route] = (uint16_t)wbits;
+        }
+        e = __builtin_amdgcn_readfirstlane(e);
+        if (a.route_weight) routed_weight = bf16_bits_to_f32(wbits);   // any non-null pointer: apply the weight here
     }
+    if (extra) e = route - a.n_routes;
 
     RouteView v;
 #pragma unroll
@@ -140,8 +142,6 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
 
     uint4 wa[kGemvUnroll];
     uint32_t sa[kGemvUnroll], ba[kGemvUnroll];
-    uint4 xr[kStageRegs], wr[kStageRegs];
-    stage_fetch(v, xr, wr);
     gemv_prefetch<KIND, NSEG>(v, sub, wa, sa, ba);
     gemv_run<KIND, NSEG, false>(v, sub, a.blocks_per_route, lds_raw, wa, sa, ba, xr, wr);
 }
