@@ -103,6 +103,16 @@ __device__ __forceinline__ float q4_word_dot(uint32_t w, uint4 xp, float d) {
     return d;
 }
 
+// An empty statement that takes a 128-bit value as ONE register operand: whatever computes with the value afterwards
+// cannot be scheduled ahead of this point, and the four registers of a load stay one tuple (separate operands per
+// component make the compiler copy the tuple apart, and wait for the load to do so).
+typedef uint32_t fk_u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void pin_u128(uint4& v) {
+    fk_u32x4_t t = {v.x, v.y, v.z, v.w};
+    asm volatile("" : "+v"(t));
+    v = make_uint4(t.x, t.y, t.z, t.w);
+}
+
 // Blocks until every global store and load this wave has issued is complete
 // (s_waitcnt vmcnt(0) lgkmcnt(0)).  With write-through (agent-scope) stores this is
 // the whole "release" a block needs before it signals other blocks through an

@@ -89,8 +89,12 @@ __host__ __device__ inline uint32_t sdpa_lds_floats(uint32_t gt, uint32_t chunk,
 // NOMERGE: the caller merges the ranges' results itself: every active block writes its (m, l, o) partial with
 // ordinary stores -- also when one range covers the context -- and returns; no arrival counter is touched.
 template <int GT, int MODE, typename ARGS, int KVQ = 0, bool FASTHEAD = false, bool NOMERGE = false>
-__device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint32_t split, uint32_t kvh,
-                                           uint32_t gz, uint32_t gz_count, float* lds) {
+__device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_raw, uint32_t split, uint32_t kvh,
+                                           uint32_t gz, uint32_t gz_count, float* lds, uint32_t kv_add = 0) {
+    // kv_raw + kv_add positions are visible (kv_add: the row's index among several active rows).  The sum is formed
+    // inside settle(), behind the points where the length is first allowed to be looked at: formed by the caller, it
+    // is a use of the loaded length at the very top of the kernel.
+    uint32_t kv_len = 0;
     constexpr bool FUSED = MODE == 1;   // inside the whole-token kernel
     constexpr bool XFORM = MODE != 0;   // q / new-row transforms happen here
     // Tiles of up to 4 heads outside the whole-token kernel: every wave runs the online softmax
@@ -114,7 +118,8 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         // a device scalar is not trusted: a length beyond what the launch was sized for would leave ranges
         // without a block (the last-arrival count would never complete), zero would divide by an empty sum
         const uint32_t covered = a.n_splits * span < a.capacity ? a.n_splits * span : a.capacity;
-        kv_len = kv_len < 1u ? 1u : (kv_len > covered ? covered : kv_len);
+        const uint32_t given = kv_raw + kv_add;
+        kv_len = given < 1u ? 1u : (given > covered ? covered : given);
         pos = XFORM ? kv_len - 1 : 0u;
         n_active = (kv_len + span - 1) / span;
         if (split < n_active) {
@@ -202,33 +207,39 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
 
     // This lane's 8 dims of each query head; fetched before the K/V rows so that the
     // scores can start as soon as the first keys arrive (loads return in order).
+    // The request is straight-line (a lane past the head width or a head past the tile reads a valid address and
+    // is zeroed afterwards): with the load under a condition the compiler waits for it where the paths join, i.e.
+    // before the K/V rows are requested -- a whole trip to memory at the start of every block.  settle_q zeroes the
+    // unused lanes and derives what the quantised forms need; it runs behind the first K/V request.
     uint4 qf[GT];
+    float sq[GT];  // quantised K: sum of this lane's 8 query dims (the affine bias term b * sum q)
     auto load_q = [&]() {
 #pragma unroll
         for (int h = 0; h < GT; ++h) {
-            qf[h] = make_uint4(0, 0, 0, 0);
-            if (kcol_ok && (uint32_t)h < gcount) {
-                if constexpr (XFORM)
-                    qf[h] = *reinterpret_cast<const uint4*>(qn + h * a.qk_dim + 8 * ck);
-                else
-                    qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + h) * a.qk_dim + 8 * ck);
+            const uint32_t hc = (uint32_t)h < gcount ? (uint32_t)h : 0u, cc = kcol_ok ? ck : 0u;
+            if constexpr (XFORM)
+                qf[h] = *reinterpret_cast<const uint4*>(qn + hc * a.qk_dim + 8 * cc);
+            else
+                qf[h] = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + hc) * a.qk_dim + 8 * cc);
+        }
+    };
+    auto settle_q = [&]() {
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+            pin_u128(qf[h]);  // looked at only from here on
+            if (!(kcol_ok && (uint32_t)h < gcount)) qf[h] = make_uint4(0, 0, 0, 0);
+            if constexpr (KVQ != 0) {
+                const uint4 v = qf[h];
+                sq[h] = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+                        ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
+                if constexpr (KVQ == 4)  // nibble pairing of q4_word_dot: (x0,x2) (x4,x6) (x1,x3) (x5,x7)
+                    qf[h] = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
+                                       (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
             }
         }
     };
     if constexpr (MODE != 2) load_q();
-
-    float sq[GT];  // quantised K: sum of this lane's 8 query dims (the affine bias term b * sum q)
-    if constexpr (KVQ != 0) {
-#pragma unroll
-        for (int h = 0; h < GT; ++h) {
-            const uint4 v = qf[h];
-            sq[h] = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
-                    ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
-            if constexpr (KVQ == 4)  // nibble pairing of q4_word_dot: (x0,x2) (x4,x6) (x1,x3) (x5,x7)
-                qf[h] = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
-                                   (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
-        }
-    }
+    if constexpr (MODE == 1) settle_q();  // whole-token kernel: q comes from LDS, its rows are requested per range
 
     // All K and V loads of a range are issued up front (the range is sized so that
     // each lane owns kSteps rows of each), so one HBM round trip covers both phases.
@@ -328,13 +339,19 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
         // ranges wait for it (it was the kernel's first request and is long back by now):
         // a fixed grid sized for the whole cache would otherwise read every range's rows
         // each launch, megabytes of traffic for a context of a few hundred tokens.
+        // (kv_len is made opaque at both places where it is first looked at: settle() runs on both paths, and
+        // the compiler otherwise computes its common part once, AHEAD of the branch -- the first range's request
+        // then waits for the length after all)
         if (split != 0) {
+            asm volatile("" : "+v"(kv_raw));
             settle();
             if (split >= n_active) return;
         }
         request_rows(kc, vc, blk0, 0, false, 0);
+        if constexpr (MODE == 0) settle_q();
         if constexpr (MODE == 2)
             vnew = *reinterpret_cast<const uint4*>(a.v_new + (size_t)kvh * a.v_stride + (vcol_ok ? 8 * cv : 0u));
+        asm volatile("" : "+v"(kv_raw));
         settle();
         if (split >= n_active) return;  // uniform: whole block leaves before any barrier
         if constexpr (MODE == 2) {
@@ -351,6 +368,7 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
                 transform_heads(0);
             }
             load_q();
+            settle_q();
         }
     }
 
@@ -755,19 +773,29 @@ __device__ __forceinline__ void sdpa_block(const ARGS& a, uint32_t kv_len, uint3
     FK_SDPA_STAMP(9);
 }
 
+// The context length of a stand-alone launch: ONE unconditional load (a load under a branch would be waited for at
+// the join, ahead of the cache reads it is meant to overlap) through a GLOBAL pointer -- the device scalar, or the
+// immediate's own place in the kernel-argument segment.  (Selected as generic pointers the two make a flat load,
+// and a flat load's completion can only be awaited with vmcnt(0): every cache row requested behind it would be
+// waited for with it.)
+__device__ __forceinline__ uint32_t sdpa_load_kv_len(const SdpaArgs& a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const __attribute__((address_space(1))) uint32_t* global_u32;
+    const global_u32 imm = (global_u32)((uintptr_t)__builtin_amdgcn_kernarg_segment_ptr() + offsetof(SdpaArgs, kv_len_imm));
+    const global_u32 dev = (global_u32)(uintptr_t)a.kv_len_ptr;
+    return *(a.kv_len_ptr ? dev : imm);
+#else
+    return a.kv_len_ptr ? *a.kv_len_ptr : a.kv_len_imm;
+#endif
+}
+
 template <int GT, int KVQ = 0>
 __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs a) {
     extern __shared__ __align__(16) float lds[];
     // One unconditional load (the immediate is read from the kernel-argument segment
     // when there is no device scalar): a load under a branch would be waited for at
     // the join, ahead of the cache reads it is meant to overlap.
-#if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t* imm = (const uint32_t*)((const char*)__builtin_amdgcn_kernarg_segment_ptr() +
-                                            offsetof(SdpaArgs, kv_len_imm));
-#else
-    const uint32_t* imm = &a.kv_len_imm;
-#endif
-    const uint32_t kv_len0 = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
+    const uint32_t kv_len0 = sdpa_load_kv_len(a);
     if (a.rows <= 1) {
         sdpa_block<GT, false, SdpaArgs, KVQ>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
         return;
@@ -782,7 +810,7 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     r.out = a.out + (size_t)tr * a.n_heads * a.v_dim;
     r.partials = a.partials + (size_t)tr * a.n_heads * a.n_splits * (a.v_dim + 2);
     r.counters = a.counters + (size_t)tr * a.n_kv * gz_count;
-    sdpa_block<GT, false, SdpaArgs, KVQ>(r, kv_len0 + tr, blockIdx.x, blockIdx.y, gz, gz_count, lds);
+    sdpa_block<GT, false, SdpaArgs, KVQ>(r, kv_len0, blockIdx.x, blockIdx.y, gz, gz_count, lds, tr);
 }
 
 // RoPE (+ head norm) of q and of the new k row, the cache append and the attention in one
@@ -791,13 +819,7 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
 template <int GT, bool FASTHEAD>
 __global__ __launch_bounds__(kSdpaBlock) void sdpa_rope_store_kernel(const SdpaArgs a) {
     extern __shared__ __align__(16) float lds[];
-#if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t* imm = (const uint32_t*)((const char*)__builtin_amdgcn_kernarg_segment_ptr() +
-                                            offsetof(SdpaArgs, kv_len_imm));
-#else
-    const uint32_t* imm = &a.kv_len_imm;
-#endif
-    const uint32_t kv_len0 = *(a.kv_len_ptr ? a.kv_len_ptr : imm);
+    const uint32_t kv_len0 = sdpa_load_kv_len(a);
     sdpa_block<GT, 2, SdpaArgs, 0, FASTHEAD>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
 }
 
