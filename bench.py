@@ -85,9 +85,6 @@ def main() -> int:
                          "kernel that rocprofv3 byte counters of the same run are scaled by")
     ap.add_argument("--five-launches", action="store_true",
                     help="experiment only: the per-dispatch task list (five launches per layer) instead of the two-launch layer")
-    ap.add_argument("--hazard-graph", action="store_true",
-                    help="profiling only: build the token's graph from the read/write tables (one fork at its start) instead "
-                         "of the chain the decoder uses; rocprofv3's kernel trace crashes in hipGraphLaunch on the chain")
     ap.add_argument("--mode", choices=["persistent", "graph"], default="graph",
                     help="persistent: one whole-token kernel per replay; graph: one kernel node per task")
     args = ap.parse_args()
@@ -113,8 +110,6 @@ def main() -> int:
     W = DecoderWeights.random_init(cfg, seed=0)
     rt = DecoderRuntime(cfg, W, hist_capacity=max(4096, total),
                         persistent=(args.mode == "persistent"))
-    if args.hazard_graph and args.mode == "graph":
-        rt.graph = rt.d.build_graph(rt.tasks)
     setup_s = time.time() - t0
 
     if args.calibrate_copy:

@@ -25,7 +25,6 @@ from .runtime import Dispatch, Dispatcher, arg
 
 HBM_PEAK = 8.0e12
 MFMA_BF16_PEAK = 2.5e15
-HAZARD_GRAPH = False  # --hazard-graph
 
 
 def _rand_weight(n, k, bits, seed, group=64, experts=1):
@@ -253,8 +252,6 @@ def case_moe_decode(d, reps, prompt_len=32, decode=512):
     cfg = MoeConfig(capacity=1024)
     W = MoeWeights.random_init(cfg, seed=0)
     rt = MoeRuntime(cfg, W, dispatcher=d)
-    if HAZARD_GRAPH:   # profiling only: rocprofv3's kernel trace crashes in hipGraphLaunch on the decoder's chain graph
-        rt.graph = rt.d.build_graph(rt.tasks)
     prompt = np.random.Generator(np.random.PCG64(0)).integers(0, cfg.vocab, prompt_len).tolist()
     rt.generate(prompt, 9)
     toks, gpu_s, steps = rt.generate(prompt, decode + 1)
@@ -343,11 +340,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--case", action="append", choices=sorted(CASES), help="default: all")
     ap.add_argument("--reps", type=int, default=20)
-    ap.add_argument("--hazard-graph", action="store_true",
-                    help="profiling only (moe_cfg5_decode): the token's graph from the read/write tables instead of the chain")
     args = ap.parse_args()
-    global HAZARD_GRAPH
-    HAZARD_GRAPH = args.hazard_graph
     d = Dispatcher()
     for name in (args.case or list(CASES)):
         print(f"[kernel_bench] {name}", file=sys.stderr, flush=True)
