@@ -130,6 +130,23 @@ def test_graph_edges_follow_hazards(fk):
     assert [rt.d.node_deps(rt.graph, i) for i in range(len(names))] == [[]] + [[i] for i in range(len(names) - 1)]
 
 
+def test_chain_graph_and_hazard_graph_decode_the_same_tokens(fk):
+    """The decoder replays its tasks as a chain (fk_build_decode_graph); the same tasks with edges from the
+    read/write tables (fk_build_graph) -- where independent tasks may overlap -- produce the same tokens."""
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    cfg = _small_cfg(bits=4, qk_norm=True, n_layers=2)
+    rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=13))
+    prompt = [3, 1500, 77]
+    want, _, _ = rt.generate(prompt, 16)
+    chain = rt.graph
+    rt.graph = rt.d.build_graph(rt.tasks)
+    n, e = rt.d.graph_info(rt.graph)
+    assert any(len(rt.d.node_deps(rt.graph, i)) != 1 for i in range(1, n))   # not a chain: a fork or a join
+    got, _, _ = rt.generate(prompt, 16)
+    rt.graph = chain
+    assert got == want
+
+
 def test_dispatcher_error_paths(fk, tmp_path):
     from fusekit_amd.runtime import Dispatch, Dispatcher
     d = Dispatcher()
