@@ -120,6 +120,24 @@ __device__ __forceinline__ void pin_u128(uint4& v) {
 // and an agent-scope fence adds a write-back of the whole L2.
 __device__ __forceinline__ void wait_memory_ops_done() { __builtin_amdgcn_s_waitcnt(0x0070); }
 
+// Reads one word of every 64-byte line of the kernel's argument block (BYTES from its start) and makes the wave wait
+// for them once.  A long kernel otherwise fetches its arguments where it first uses them, phase by phase, and each
+// first touch of a line is a scalar-cache miss -- a trip to the L2 -- in the middle of that phase; after this the
+// later fetches hit.  Call it where the wave waits for its first arguments anyway.
+template <int BYTES>
+__device__ __forceinline__ void kernarg_warm() {
+    typedef const uint32_t __attribute__((address_space(4))) * karg_t;
+    karg_t ka = (karg_t)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr int LINES = (BYTES + 63) / 64;
+    static_assert(LINES <= 12, "argument block larger than this helper covers");
+    uint32_t v[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) v[i] = ka[(i < LINES ? i : 0) * 16];
+    // one statement that takes them all: every request goes out before the one wait
+    asm volatile("" ::"s"(v[0]), "s"(v[1]), "s"(v[2]), "s"(v[3]), "s"(v[4]), "s"(v[5]), "s"(v[6]), "s"(v[7]), "s"(v[8]),
+                 "s"(v[9]), "s"(v[10]), "s"(v[11]));
+}
+
 // v + (v of the lane selected by a DPP control): cross-lane adds inside a row of
 // 16 lanes without going through the LDS crossbar.
 template <int CTRL>

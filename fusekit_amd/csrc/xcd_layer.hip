@@ -417,9 +417,17 @@ __device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL
                                          const float* sx, const uint32_t* meta, float* part, F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * m.cpr + step_c;
+    if (n_pass <= 1) {
+        // One pass: a path of its own, so that the waits for `r0` are counted with the caller's requests behind them.
+        // Joined with the loop below, where those requests sit under a condition, the compiler counts without them,
+        // and every chunk of the pass then also waits for as many of the caller's requests as it has passes in
+        // flight -- at the end for all of them.
+        after_last_request();
+        tile_partials<KIND, NL, SN>(m, t, p, r0, xs, sx, meta, part);
+        return;
+    }
     TileRegs<NL> r1;
     TilePos<NL> q = p;
-    if (n_pass <= 1) after_last_request();
     for (uint32_t k = 0; k < n_pass; k += 2) {
         if (k + 1 < n_pass) {
             tile_pos_next<NL, SN>(m, t, step_c, step_g, q);
@@ -449,9 +457,14 @@ __device__ __forceinline__ void tile_run_pair(const MAT& ma, const MAT& mb, cons
                                               F after_last_request) {
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * ma.cpr + step_c;
+    if (n_pass <= 1) {  // a path of its own: see tile_run
+        after_last_request();
+        tile_partials<KIND, NL, SN>(ma, t, p, a0, xs, sx, meta_a, part_a);
+        tile_partials<KIND, NL, SN>(mb, t, p, b0, xs, sx, meta_b, part_b);
+        return;
+    }
     TileRegs<NL> a1, b1;
     TilePos<NL> q = p;
-    if (n_pass <= 1) after_last_request();
     for (uint32_t k = 0; k < n_pass; k += 2) {
         if (k + 1 < n_pass) {
             tile_pos_next<NL, SN>(ma, t, step_c, step_g, q);
@@ -648,6 +661,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const long long* 
     const XcdInputLead lead{sums, residual, norm_w, hidden};
     InputRegs inr;
     input_request<false>(lead, inr, nullptr);
+    kernarg_warm<32 + (int)sizeof(XcdMlpArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
     xcd_mlp_phase<KIND, NLA, NLB, false, true>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
 }
@@ -824,6 +838,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const long long* su
     const XcdInputLead lead{sums, residual, norm_w, hidden};
     InputRegs inr;
     input_request<false>(lead, inr, nullptr);
+    kernarg_warm<32 + (int)sizeof(XcdAttnArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
     xcd_attn_phase<KIND, NLA, NLB, false, true>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
 }
