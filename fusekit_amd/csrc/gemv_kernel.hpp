@@ -494,6 +494,7 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_stream_kernel(const uint16_t*
     uint4 xr[kStageRegs], wr[kStageRegs];
     FK_GEMV_STAMP(0);
     stage_fetch(StageLead{x, norm_w, K}, xr, wr);          // activations first: they return first
+    kernarg_warm<24 + (int)sizeof(GemvArgs)>();
     gemv_prefetch<KIND, NSEG>(a, blockIdx.x, wa, sa, ba);  // weights stream while x is staged
     gemv_run<KIND, NSEG, false>(a, blockIdx.x, gridDim.x, lds_raw, wa, sa, ba, xr, wr);
 }

@@ -113,6 +113,7 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_rows_kernel(const uint16_t* x
 
     uint4 xr[kStageRegs], wr[kStageRegs];
     stage_fetch(StageLead{x, norm_w, K}, xr, wr);  // from the leading parameters: before the argument block arrives
+    kernarg_warm<24 + (int)sizeof(a)>();
 
     const uint32_t lane = threadIdx.x & (kWave - 1), l16 = lane & (kRowLanes - 1), rg = lane / kRowLanes;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);

@@ -77,6 +77,7 @@ struct RouteView {
 template <WKind KIND, int NSEG>
 __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArgs a) {
     extern __shared__ uint4 lds_raw[];
+    kernarg_warm<(int)sizeof(RoutedArgs)>();
     const uint32_t route = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - route * a.blocks_per_route;
     const bool extra = route >= a.n_routes;     // uniform per block
     const uint32_t lookup = extra ? 0u : route;
@@ -195,6 +196,7 @@ struct DownReduceArgs {
 };
 __global__ __launch_bounds__(kDrBlock) void routed_down_reduce_kernel(const DownReduceArgs a) {
     extern __shared__ uint4 dr_lds[];
+    kernarg_warm<(int)sizeof(DownReduceArgs)>();
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t cpr = a.K / 32, scpr = a.SK / 32, gpr = cpr / a.gdiv, sgpr = scpr / a.gdiv;
     const uint32_t routed8 = a.top_k * a.K / 8, total8 = routed8 + a.SK / 8;

@@ -795,6 +795,7 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
     // One unconditional load (the immediate is read from the kernel-argument segment
     // when there is no device scalar): a load under a branch would be waited for at
     // the join, ahead of the cache reads it is meant to overlap.
+    kernarg_warm<(int)sizeof(SdpaArgs)>();
     const uint32_t kv_len0 = sdpa_load_kv_len(a);
     if (a.rows <= 1) {
         sdpa_block<GT, false, SdpaArgs, KVQ>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
@@ -819,6 +820,7 @@ __global__ __launch_bounds__(kSdpaBlock) void sdpa_decode_kernel(const SdpaArgs 
 template <int GT, bool FASTHEAD>
 __global__ __launch_bounds__(kSdpaBlock) void sdpa_rope_store_kernel(const SdpaArgs a) {
     extern __shared__ __align__(16) float lds[];
+    kernarg_warm<(int)sizeof(SdpaArgs)>();
     const uint32_t kv_len0 = sdpa_load_kv_len(a);
     sdpa_block<GT, 2, SdpaArgs, 0, FASTHEAD>(a, kv_len0, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z, lds);
 }
