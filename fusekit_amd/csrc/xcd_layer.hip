@@ -412,9 +412,16 @@ __device__ __forceinline__ void tile_partials(const MAT& m, const Tile& t, const
 // All passes of a tile whose first pass is already in `r0` (positions `p` at pass 0): pass k + 1 is requested
 // before pass k is consumed.  `after_last_request` runs once the tile's last pass has been requested (the caller
 // queues what it needs next behind it).
-template <WKind KIND, int NL, int SN, typename MAT, typename F>
+// ONE: the launch was planned with every tile within one pass; the loop (and the second set of registers it keeps)
+// is then not compiled at all.
+template <WKind KIND, int NL, int SN, bool ONE = false, typename MAT, typename F>
 __device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
                                          const float* sx, const uint32_t* meta, float* part, F after_last_request) {
+    if constexpr (ONE) {
+        after_last_request();
+        tile_partials<KIND, NL, SN>(m, t, p, r0, xs, sx, meta, part);
+        return;
+    }
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * m.cpr + step_c;
     if (n_pass <= 1) {
@@ -450,11 +457,17 @@ __device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL
 
 // The gate / up pair: both matrices' passes interleaved, so that one pass of each is in flight while one is consumed.
 // (Same shape and tile: one set of positions serves both.)
-template <WKind KIND, int NL, int SN, typename MAT, typename F>
+template <WKind KIND, int NL, int SN, bool ONE = false, typename MAT, typename F>
 __device__ __forceinline__ void tile_run_pair(const MAT& ma, const MAT& mb, const Tile& t, TilePos<NL>& p,
                                               TileRegs<NL>& a0, TileRegs<NL>& b0, const uint4* xs, const float* sx,
                                               const uint32_t* meta_a, const uint32_t* meta_b, float* part_a, float* part_b,
                                               F after_last_request) {
+    if constexpr (ONE) {
+        after_last_request();
+        tile_partials<KIND, NL, SN>(ma, t, p, a0, xs, sx, meta_a, part_a);
+        tile_partials<KIND, NL, SN>(mb, t, p, b0, xs, sx, meta_b, part_b);
+        return;
+    }
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * ma.cpr + step_c;
     if (n_pass <= 1) {  // a path of its own: see tile_run
@@ -554,7 +567,7 @@ constexpr int kMlpBlock = kBlock;
 // the residual row in LDS (token kernel only).
 // EARLY: the caller has already issued input_request into `inr` (the stand-alone launch does so before anything
 // else, from its leading parameters).
-template <WKind KIND, int NLA, int NLB, bool TOKEN, bool EARLY, typename ARGS, typename LEAD>
+template <WKind KIND, int NLA, int NLB, bool TOKEN, bool EARLY, bool ONE = false, typename ARGS, typename LEAD>
 __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, InputRegs& inr, XcdSync& sync, uint4* lds_raw,
                                               const uint4* xres_in, uint4* xres_out) {
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats;
@@ -606,7 +619,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if (streams) {
         auto request_down = [&]() { tile_load<KIND, NLB, kBlock>(a.down, td, pd, rd); };
         if (gu_n)
-            tile_run_pair<KIND, NLA, kBlock>(a.gate, a.up, tg, pg, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg,
+            tile_run_pair<KIND, NLA, kBlock, ONE>(a.gate, a.up, tg, pg, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg,
                                              request_down);
         else
             request_down();
@@ -628,7 +641,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if (streams) stage_vector<KIND>(a.mid + (size_t)sync.xcd * per_xcd, per_xcd >> 3, a.down_cs, xs, sx);
     __syncthreads();
     FK_XCD_STAMP(1, 9);
-    if (streams && d_n) tile_run<KIND, NLB, kBlock>(a.down, td, pd, rd, xs, sx, meta + 2 * kMetaWords, work, []() {});
+    if (streams && d_n) tile_run<KIND, NLB, kBlock, ONE>(a.down, td, pd, rd, xs, sx, meta + 2 * kMetaWords, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(1, 10);
     if (streams && d_n) {
@@ -653,7 +666,7 @@ __device__ __forceinline__ XcdSync xcd_sync_init(XcdControl* ctl, uint32_t spin_
     return sync;
 }
 
-template <WKind KIND, int NLA, int NLB>
+template <WKind KIND, int NLA, int NLB, bool ONE>
 __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const long long* sums, const uint16_t* residual,
                                                                const uint16_t* norm_w, uint32_t hidden, const XcdMlpArgs a) {
     extern __shared__ uint4 lds_raw[];
@@ -663,13 +676,13 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const long long* 
     input_request<false>(lead, inr, nullptr);
     kernarg_warm<32 + (int)sizeof(XcdMlpArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
-    xcd_mlp_phase<KIND, NLA, NLB, false, true>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
+    xcd_mlp_phase<KIND, NLA, NLB, false, true, ONE>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
 }
 
 // =============================================================================================== attention launch
 constexpr int kAttnStream = kBlock;
 
-template <WKind KIND, int NLA, int NLB, bool TOKEN, bool EARLY, typename ARGS, typename LEAD>
+template <WKind KIND, int NLA, int NLB, bool TOKEN, bool EARLY, bool ONE = false, typename ARGS, typename LEAD>
 __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, InputRegs& inr, XcdSync& sync, uint4* lds_raw,
                                                const uint4* xres_in, uint4* xres_out) {
     const uint32_t cs_max = a.cs_max, work_floats = a.work_floats, att_elems = a.att_elems;
@@ -729,7 +742,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     if (streams) {
         auto request_o = [&]() { tile_load<KIND, NLB, kAttnStream>(a.wo, to, po, ro); };
         if (pr_n)
-            tile_run<KIND, NLA, kAttnStream>(mq, tq, pq, rq, xs, sx, meta, work, request_o);
+            tile_run<KIND, NLA, kAttnStream, ONE>(mq, tq, pq, rq, xs, sx, meta, work, request_o);
         else
             request_o();
     }
@@ -821,7 +834,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     }
     meta_store<KIND, kAttnStream, true>(mmo, ti, meta + kMetaWords);
     __syncthreads();
-    if (streams && o_n) tile_run<KIND, NLB, kAttnStream>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
+    if (streams && o_n) tile_run<KIND, NLB, kAttnStream, ONE>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(0, 11);
     if (o_n) {
@@ -831,7 +844,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     FK_XCD_STAMP(0, 12);
 }
 
-template <WKind KIND, int NLA, int NLB>
+template <WKind KIND, int NLA, int NLB, bool ONE>
 __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const long long* sums, const uint16_t* residual,
                                                              const uint16_t* norm_w, uint32_t hidden, const XcdAttnArgs a) {
     extern __shared__ uint4 lds_raw[];
@@ -840,7 +853,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const long long* su
     input_request<false>(lead, inr, nullptr);
     kernarg_warm<32 + (int)sizeof(XcdAttnArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
-    xcd_attn_phase<KIND, NLA, NLB, false, true>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
+    xcd_attn_phase<KIND, NLA, NLB, false, true, ONE>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
 }
 
 // ---- the whole token in one launch --------------------------------------------------------------------------
@@ -1003,9 +1016,15 @@ fk_status bind_mat(const fk_weight* w, uint32_t n, uint32_t k, const XcdLayerSha
 }
 
 template <WKind KIND>
-const void* mlp_func() { return reinterpret_cast<const void*>(&xcd_mlp_kernel<KIND, kNlGu, kNlDown>); }
+const void* mlp_func(bool one) {
+    return one ? reinterpret_cast<const void*>(&xcd_mlp_kernel<KIND, kNlGu, kNlDown, true>)
+               : reinterpret_cast<const void*>(&xcd_mlp_kernel<KIND, kNlGu, kNlDown, false>);
+}
 template <WKind KIND>
-const void* attn_func() { return reinterpret_cast<const void*>(&xcd_attn_kernel<KIND, kNlQkv, kNlO>); }
+const void* attn_func(bool one) {
+    return one ? reinterpret_cast<const void*>(&xcd_attn_kernel<KIND, kNlQkv, kNlO, true>)
+               : reinterpret_cast<const void*>(&xcd_attn_kernel<KIND, kNlQkv, kNlO, false>);
+}
 
 uint32_t lds_for(uint32_t bits, const LdsPlan& p) {
     return bits == 4 ? xcd_lds_bytes<W_Q4>(p) : (bits == 8 ? xcd_lds_bytes<W_Q8>(p) : xcd_lds_bytes<W_BF16>(p));
@@ -1107,7 +1126,9 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     lp.work_floats = gu > dn ? gu : dn;
     lp.att_elems = 0;
     const uint32_t lds = lds_for(s.bits, lp);
-    out->func = s.bits == 4 ? mlp_func<W_Q4>() : (s.bits == 8 ? mlp_func<W_Q8>() : mlp_func<W_BF16>());
+    // every tile within one pass (the 4B-class shapes): the flavour compiled without the pass loop
+    const bool one = !rq.for_token && a.gu_rows * a.gate.cpr <= (uint32_t)kNlGu * kBlock && a.down_rows * a.down_cs <= (uint32_t)kNlDown * kBlock;
+    out->func = s.bits == 4 ? mlp_func<W_Q4>(one) : (s.bits == 8 ? mlp_func<W_Q8>(one) : mlp_func<W_BF16>(one));
     FK_TRY(set_lds_limit(out->func, lds));
     out->grid = dim3(kXcdGrid, 1, 1);
     out->block = dim3(kMlpBlock, 1, 1);
@@ -1199,7 +1220,8 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     lp.work_floats = wf > sf ? wf : sf;
     lp.att_elems = G * s.head_dim;
     const uint32_t lds = lds_for(s.bits, lp);
-    out->func = s.bits == 4 ? attn_func<W_Q4>() : (s.bits == 8 ? attn_func<W_Q8>() : attn_func<W_BF16>());
+    const bool one = R * a.wq.cpr <= (uint32_t)kNlQkv * kAttnStream && a.o_rows * a.o_cs <= (uint32_t)kNlO * kAttnStream;
+    out->func = s.bits == 4 ? attn_func<W_Q4>(one) : (s.bits == 8 ? attn_func<W_Q8>(one) : attn_func<W_BF16>(one));
     FK_TRY(set_lds_limit(out->func, lds));
     out->grid = dim3(kXcdGrid, 1, 1);
     out->block = dim3(kBlock, 1, 1);
