@@ -413,7 +413,10 @@ __device__ __forceinline__ void tile_partials(const MAT& m, const Tile& t, const
 // before pass k is consumed.  `after_last_request` runs once the tile's last pass has been requested (the caller
 // queues what it needs next behind it).
 // ONE: the launch was planned with every tile within one pass; the loop (and the second set of registers it keeps)
-// is then not compiled at all.
+// is then not compiled at all, and the waits for `r0` are counted with the caller's requests behind them.  (In the
+// loop those requests sit under a condition; the compiler then counts without them, and every chunk of a pass also
+// waits for as many of the caller's requests as the pass has chunks in flight -- at the end for all of them.  A
+// run-time test for one pass inside this general form costs it registers: 26-31 spilled in the MLP kernel.)
 template <WKind KIND, int NL, int SN, bool ONE = false, typename MAT, typename F>
 __device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
                                          const float* sx, const uint32_t* meta, float* part, F after_last_request) {
@@ -424,17 +427,9 @@ __device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL
     }
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * m.cpr + step_c;
-    if (n_pass <= 1) {
-        // One pass: a path of its own, so that the waits for `r0` are counted with the caller's requests behind them.
-        // Joined with the loop below, where those requests sit under a condition, the compiler counts without them,
-        // and every chunk of the pass then also waits for as many of the caller's requests as it has passes in
-        // flight -- at the end for all of them.
-        after_last_request();
-        tile_partials<KIND, NL, SN>(m, t, p, r0, xs, sx, meta, part);
-        return;
-    }
     TileRegs<NL> r1;
     TilePos<NL> q = p;
+    if (n_pass <= 1) after_last_request();
     for (uint32_t k = 0; k < n_pass; k += 2) {
         if (k + 1 < n_pass) {
             tile_pos_next<NL, SN>(m, t, step_c, step_g, q);
@@ -470,14 +465,9 @@ __device__ __forceinline__ void tile_run_pair(const MAT& ma, const MAT& mb, cons
     }
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
     const uint32_t step_r = (NL * SN) / t.cs, step_c = (NL * SN) - step_r * t.cs, step_g = step_r * ma.cpr + step_c;
-    if (n_pass <= 1) {  // a path of its own: see tile_run
-        after_last_request();
-        tile_partials<KIND, NL, SN>(ma, t, p, a0, xs, sx, meta_a, part_a);
-        tile_partials<KIND, NL, SN>(mb, t, p, b0, xs, sx, meta_b, part_b);
-        return;
-    }
     TileRegs<NL> a1, b1;
     TilePos<NL> q = p;
+    if (n_pass <= 1) after_last_request();
     for (uint32_t k = 0; k < n_pass; k += 2) {
         if (k + 1 < n_pass) {
             tile_pos_next<NL, SN>(ma, t, step_c, step_g, q);
