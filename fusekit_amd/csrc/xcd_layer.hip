@@ -133,6 +133,7 @@ __device__ __forceinline__ void stage_vector(const uint16_t* src, uint32_t n8, u
 // Thread t of the block takes the groups of eight elements t and t + 256 (hidden <= 4096).  The requests go out
 // first (input_request), the block's first weight requests behind them, then the values are used (input_stage).
 constexpr int kInGroups = 2;
+constexpr int kGuAhead = 4;  // gate requests of the MLP launch that go out ahead of its input's staging
 
 __device__ __forceinline__ float xcd_sum_to_f32(uint32_t lo, uint32_t hi) {
     return fmaf((float)lo, kXcdSumInv, (float)(int32_t)hi);
@@ -333,11 +334,11 @@ __device__ __forceinline__ void tile_pos_next(const MAT& m, const Tile& t, uint3
     }
 }
 
-template <WKind KIND, int NL, int SN, typename MAT>
+template <WKind KIND, int NL, int SN, int J0 = 0, int J1 = NL, typename MAT>
 __device__ __forceinline__ void tile_load(const MAT& m, const Tile& t, const TilePos<NL>& p, TileRegs<NL>& r) {
     const uint32_t total = t.rows * t.cs, first = t.row0 * m.cpr + t.col0;
 #pragma unroll
-    for (int j = 0; j < NL; ++j) r.w[j] = m.w[p.p0 + j * SN < total ? p.gidx[j] : first];
+    for (int j = J0; j < J1; ++j) r.w[j] = m.w[p.p0 + j * SN < total ? p.gidx[j] : first];
 }
 
 // Group gi of the tile = (row gi / gpr, group gi % gpr of the row's slice), gpr groups per row slice.
@@ -592,11 +593,18 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     tile_pos_init<NLB, kBlock>(a.down, td, tid, pd);
     meta_fetch<KIND, kBlock, true>(a.gate, tg, tid, mg);
     meta_fetch<KIND, kBlock, true>(a.up, tg, tid, mu);
-    tile_load<KIND, NLA, kBlock>(a.gate, tg, pg, rg);
-    tile_load<KIND, NLA, kBlock>(a.up, tg, pg, ru);
+    // Only kGuAhead requests of the gate matrix go out ahead of the input's staging, the rest of the pass and the up
+    // matrix's behind it: a wave cannot stage before it has ISSUED what stands in front, issue stalls once the CU's
+    // request queue is full, and the block's staging waits for its slowest wave.  With all twelve in front the
+    // median block had its activations staged 1.3 us later than the attention launch has; with none the stream
+    // starts too late (4B int4, tok/s by requests in front: 12: 780, 6: 791, 4: 796, 3: 796, 2: 790, 1: 781, 0: 774).
+    constexpr int GP = kGuAhead < NLA ? kGuAhead : NLA;
+    tile_load<KIND, NLA, kBlock, 0, GP>(a.gate, tg, pg, rg);
     FK_XCD_STAMP(1, 1);
     input_pin(lead, inr);
     input_stage<KIND, 1>(a.in, inr, xs, sx, a.gate.cpr, red, xres_out);
+    tile_load<KIND, NLA, kBlock, GP, NLA>(a.gate, tg, pg, rg);
+    tile_load<KIND, NLA, kBlock>(a.up, tg, pg, ru);
     FK_XCD_STAMP(1, 5);
     input_clear<TOKEN>(a.in);
     meta_store<KIND, kBlock, true>(mg, tid, meta);
@@ -715,7 +723,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     tile_pos_init<NLA, kAttnStream>(mq, tq, ti, pq);
     tile_pos_init<NLB, kAttnStream>(a.wo, to, ti, po);
     meta_fetch<KIND, kAttnStream, true>(mq, tq, ti, mmq);
-    tile_load<KIND, NLA, kAttnStream>(mq, tq, pq, rq);
+    tile_load<KIND, NLA, kAttnStream>(mq, tq, pq, rq);  // all of it ahead of the staging: 2 or 3 of 5 were no faster here
     FK_XCD_STAMP(0, 1);
     asm volatile("" : "+v"(kv_len_raw));
     const uint32_t kv_len0 = __builtin_amdgcn_readfirstlane(kv_len_raw);
