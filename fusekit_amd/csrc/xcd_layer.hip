@@ -422,7 +422,7 @@ template <WKind KIND, int NL, int SN, bool ONE = false, typename MAT, typename F
 __device__ __forceinline__ void tile_run(const MAT& m, const Tile& t, TilePos<NL>& p, TileRegs<NL>& r0, const uint4* xs,
                                          const float* sx, const uint32_t* meta, float* part, F after_last_request) {
     if constexpr (ONE) {
-        after_last_request();
+        after_last_request();  // (the o_proj slice: in front of or behind the arithmetic made no difference)
         tile_partials<KIND, NL, SN>(m, t, p, r0, xs, sx, meta, part);
         return;
     }
@@ -459,9 +459,12 @@ __device__ __forceinline__ void tile_run_pair(const MAT& ma, const MAT& mb, cons
                                               const uint32_t* meta_a, const uint32_t* meta_b, float* part_a, float* part_b,
                                               F after_last_request) {
     if constexpr (ONE) {
-        after_last_request();
+        // The caller's requests (the down_proj slice) go out BEHIND the arithmetic of both matrices: they are not
+        // needed before the hand-over that follows, and in front they only lengthen the queue the gate / up chunks
+        // stand in (4B int4, same box: in front 798 tok/s, between the two matrices 809, behind 821).
         tile_partials<KIND, NL, SN>(ma, t, p, a0, xs, sx, meta_a, part_a);
         tile_partials<KIND, NL, SN>(mb, t, p, b0, xs, sx, meta_b, part_b);
+        after_last_request();
         return;
     }
     const uint32_t n_pass = (t.rows * t.cs + NL * SN - 1) / (NL * SN);
