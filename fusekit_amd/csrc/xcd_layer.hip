@@ -133,7 +133,7 @@ __device__ __forceinline__ void stage_vector(const uint16_t* src, uint32_t n8, u
 // Thread t of the block takes the groups of eight elements t and t + 256 (hidden <= 4096).  The requests go out
 // first (input_request), the block's first weight requests behind them, then the values are used (input_stage).
 constexpr int kInGroups = 2;
-constexpr int kGuAhead = 4;  // gate requests of the MLP launch that go out ahead of its input's staging
+constexpr int kGuAhead = 3;  // gate requests of the MLP launch that go out ahead of its input's staging
 
 __device__ __forceinline__ float xcd_sum_to_f32(uint32_t lo, uint32_t hi) {
     return fmaf((float)lo, kXcdSumInv, (float)(int32_t)hi);
@@ -600,7 +600,8 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     // matrix's behind it: a wave cannot stage before it has ISSUED what stands in front, issue stalls once the CU's
     // request queue is full, and the block's staging waits for its slowest wave.  With all twelve in front the
     // median block had its activations staged 1.3 us later than the attention launch has; with none the stream
-    // starts too late (4B int4, tok/s by requests in front: 12: 780, 6: 791, 4: 796, 3: 796, 2: 790, 1: 781, 0: 774).
+    // starts too late (4B int4, tok/s by requests in front: 12: 780, 6: 791, 4: 796, 3: 796, 2: 790, 1: 781, 0: 774; with the
+    // down_proj slice requested behind the arithmetic: 6: 802, 4: 819, 3: 828, 2: 820).
     constexpr int GP = kGuAhead < NLA ? kGuAhead : NLA;
     tile_load<KIND, NLA, kBlock, 0, GP>(a.gate, tg, pg, rg);
     FK_XCD_STAMP(1, 1);
