@@ -508,8 +508,8 @@ __device__ __forceinline__ uint32_t lanes_per_row(uint32_t cs) {
 template <bool TWO, typename F>
 __device__ __forceinline__ void tile_rows(const Tile& t, const float* part, const float* part1, F f) {
     const uint32_t lr = lanes_per_row(t.cs), lane = threadIdx.x & (lr - 1);
-    const uint32_t rows_up = (t.rows + (kBlock / lr) - 1) / (kBlock / lr) * (kBlock / lr);
-    for (uint32_t rr = threadIdx.x / lr; rr < rows_up; rr += kBlock / lr) {
+    const uint32_t step = kBlock / lr, rows_up = (t.rows + step - 1) / step * step;
+    auto one = [&](uint32_t rr) {
         const bool ok = rr < t.rows;
         float s0 = 0.f, s1 = 0.f;
         if (ok)
@@ -520,7 +520,16 @@ __device__ __forceinline__ void tile_rows(const Tile& t, const float* part, cons
         s0 = group_sum(s0, lr);
         if constexpr (TWO) s1 = group_sum(s1, lr);
         if (ok && lane == 0) f(rr, s0, s1);
+    };
+    // Up to two rounds (the 4B-class tiles) run straight-line: f stores to memory, and in front of a LOOP with
+    // stores in it the compiler waits for every request still in flight -- here the next projection's weights,
+    // requested just before, whose trip to memory the row sums and the hand-over are meant to cover.
+    if (rows_up <= 2 * step) {
+        one(threadIdx.x / lr);
+        if (rows_up > step) one(threadIdx.x / lr + step);
+        return;
     }
+    for (uint32_t rr = threadIdx.x / lr; rr < rows_up; rr += step) one(rr);
 }
 
 // An empty tile (a block without work in this projection) still issues its loads, clamped to the tile's
