@@ -774,13 +774,7 @@ fk_status fk_xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, u
 fk_status fk_xcd_check(void* workspace, fk_stream s) {
     if (!workspace) return set_error(FK_ERR_INVALID, "fk_xcd_check: null workspace");
     FK_HIP(hipStreamSynchronize((hipStream_t)s));
-    XcdControl* c = reinterpret_cast<XcdControl*>(workspace);
-    uint32_t flag = 0;
-    FK_HIP(hipMemcpy(&flag, &c->abort_flag, 4, hipMemcpyDeviceToHost));
-    if (!flag) return FK_OK;
-    // the arrival words of an aborted launch are inconsistent: start over from zero
-    FK_HIP(hipMemset(workspace, 0, sizeof(XcdControl)));
-    return set_error(FK_ERR_HIP, "xcd layer: a hand-over wait exceeded its spin limit; results are invalid (the workspace was reset)");
+    return xcd_check_control(workspace);
 }
 
 }  // extern "C"

@@ -1269,6 +1269,7 @@ struct Graph {
     hipGraphExec_t exec = nullptr;
     std::vector<uint8_t> barriers;  // as given to fk_build_graph (empty: none forced)
     std::vector<void*> xcd_controls;  // control blocks of XCD-resident launches in this graph (abort words)
+    std::vector<std::pair<void*, size_t>> xcd_sum_rows;  // the sum rows those launches read, add into and clear
     // Runs of alternating xcd_attn / xcd_mlp dispatches (parameter token_launch = 1) executed as ONE launch each:
     // the nodes keep their own launches (eager execution, profiling), the executable graph holds one kernel node
     // per run, whose per-layer argument blocks sit in device tables.
@@ -1312,6 +1313,7 @@ struct DispatcherState {
     std::vector<const char*> kernel_name_ptrs;
     std::string task_graph_path;
     bool pending = false;
+    Graph* pending_graph = nullptr;  // the graph of the launch in flight (graphs live as long as their dispatcher)
 };
 
 std::mutex g_mu;
@@ -1359,7 +1361,8 @@ bool direct_dep(const std::vector<fk_arg>& aa, const SlotRW& arw, const std::vec
 }
 
 // RAW / WAW / WAR edges on overlapping byte ranges, transitively reduced.
-void derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
+// Returns the ancestor sets (bit j of anc[i]: node j runs before node i).
+std::vector<std::vector<uint64_t>> derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
     const size_t n = nodes.size();
     const size_t words = (n + 63) / 64;
     std::vector<std::vector<uint64_t>> anc(n, std::vector<uint64_t>(words, 0));
@@ -1381,6 +1384,29 @@ void derive_edges(std::vector<Node>& nodes, const uint8_t* barriers) {
         }
         std::sort(nodes[i].deps.begin(), nodes[i].deps.end());
     }
+    return anc;
+}
+
+// An XCD-resident launch needs the whole device to itself: its 512 workgroups must all be resident at once, two per
+// CU, and a kernel running beside it would hold CUs and leave some of them waiting (the hand-over waits would then
+// run into their spin limit).  Inside a graph that means every other node must be ordered before or after it.
+fk_status require_xcd_nodes_ordered(const std::vector<Node>& nodes, const std::vector<std::vector<uint64_t>>& anc) {
+    auto is_xcd = [](const Node& nd) {
+        return nd.d.kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || nd.d.kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0;
+    };
+    for (size_t i = 0; i < nodes.size(); ++i) {
+        if (!is_xcd(nodes[i])) continue;
+        for (size_t j = 0; j < nodes.size(); ++j) {
+            if (j == i) continue;
+            const bool ordered = j < i ? (anc[i][j / 64] >> (j % 64) & 1) != 0 : (anc[j][i / 64] >> (i % 64) & 1) != 0;
+            if (!ordered)
+                return set_error(FK_ERR_UNSUPPORTED, "graph: dispatch " + std::to_string(i) + " (" + nodes[i].d.kernel +
+                                                         ") needs the device to itself, but dispatch " + std::to_string(j) + " (" +
+                                                         nodes[j].d.kernel + ") is not ordered against it; pass barriers that "
+                                                         "order them (a decode graph built as a chain does)");
+        }
+    }
+    return FK_OK;
 }
 
 fk_status timed(DispatcherState* ds, double* gpu_seconds, const std::function<fk_status()>& body) {
@@ -1666,15 +1692,16 @@ fk_status build_token_kernel(std::vector<Node>& nodes, uint32_t spin_limit, Grap
     return FK_OK;
 }
 
+// Called with the stream idle.  A failed XCD-resident launch leaves partial sums behind: the control block is reset
+// by the check, the graph's sum rows are zeroed here (every token starts from zero rows), and the error text tells the
+// caller to decode the token again, which rewrites the cache rows of its position.
 fk_status check_abort(Graph* g) {
     for (void* ws : g->xcd_controls) {
-        uint32_t flag = 0;
-        XcdControl* c = reinterpret_cast<XcdControl*>(ws);
-        FK_HIP(hipMemcpy(&flag, &c->abort_flag, 4, hipMemcpyDeviceToHost));
-        if (flag) {
-            // the arrival words of an aborted launch are inconsistent: start over from zero
-            FK_HIP(hipMemset(ws, 0, sizeof(XcdControl)));
-            return set_error(FK_ERR_HIP, "xcd layer: a hand-over wait exceeded its spin limit; results are invalid (the control block was reset)");
+        const fk_status st = xcd_check_control(ws);
+        if (st != FK_OK) {
+            const std::string msg = fk_last_error();
+            for (const auto& row : g->xcd_sum_rows) FK_HIP(hipMemset(row.first, 0, row.second));
+            return set_error(st, msg + " [the graph's sum rows were zeroed]");
         }
     }
     if (!g->persistent) return FK_OK;
@@ -1887,13 +1914,24 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
         FK_TRY(copy_dispatch(list[i], &g->nodes[i].d));
         FK_TRY(plan_dispatch(g->nodes[i].d, &g->nodes[i].launch, &g->nodes[i].rw));
     }
-    derive_edges(g->nodes, barriers);
+    const auto anc = derive_edges(g->nodes, barriers);
+    FK_TRY(require_xcd_nodes_ordered(g->nodes, anc));
     if (barriers) g->barriers.assign(barriers, barriers + n);
     for (size_t i = 0; i < n; ++i) {
         const Node& nd = g->nodes[i];
         if (nd.d.kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || nd.d.kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0) {
             void* ws = nd.d.args.back().ptr;
             if (std::find(g->xcd_controls.begin(), g->xcd_controls.end(), ws) == g->xcd_controls.end()) g->xcd_controls.push_back(ws);
+            // slots: [sums_in], ..., out_sums, clear_sums, workspace (the planners have checked count and sizes)
+            const size_t na = nd.d.args.size(), row_bytes = xcd_sum_row_bytes(nd.d.u("hidden"));
+            auto add_row = [&](void* p) {
+                for (const auto& r : g->xcd_sum_rows)
+                    if (r.first == p) return;
+                g->xcd_sum_rows.emplace_back(p, row_bytes);
+            };
+            add_row(nd.d.args[na - 3].ptr);
+            add_row(nd.d.args[na - 2].ptr);
+            if (nd.d.u("has_sums", 1) != 0) add_row(nd.d.args[0].ptr);
         }
     }
     FK_TRY(find_fused_runs(g.get()));
@@ -2165,10 +2203,11 @@ fk_status fk_execute_graph_range(fk_handle h, uint32_t graph_id, uint32_t start,
     Graph* g;
     FK_TRY(get_graph(ds, graph_id, &g));
     if (start > end || end > g->nodes.size()) return set_error(FK_ERR_INVALID, "graph range out of bounds");  // lib.rs:781-786
-    return timed(ds, gpu_seconds, [&]() -> fk_status {
+    FK_TRY(timed(ds, gpu_seconds, [&]() -> fk_status {
         for (uint32_t i = start; i < end; ++i) FK_TRY(run_launch(g->nodes[i].launch, ds->stream));
         return FK_OK;
-    });
+    }));
+    return check_abort(g);
 }
 
 fk_status fk_profile_graph_nodes(fk_handle h, uint32_t graph_id, double* per_node_seconds, size_t n) {
@@ -2181,7 +2220,7 @@ fk_status fk_profile_graph_nodes(fk_handle h, uint32_t graph_id, double* per_nod
     for (size_t i = 0; i < g->nodes.size(); ++i) {
         FK_TRY(timed(ds, &per_node_seconds[i], [&]() -> fk_status { return run_launch(g->nodes[i].launch, ds->stream); }));
     }
-    return FK_OK;
+    return check_abort(g);
 }
 
 fk_status fk_submit_graph_async(fk_handle h, uint32_t graph_id) {
@@ -2195,6 +2234,7 @@ fk_status fk_submit_graph_async(fk_handle h, uint32_t graph_id) {
     FK_HIP(hipGraphLaunch(g->exec, ds->stream));
     FK_HIP(hipEventRecord(ds->ev1, ds->stream));
     ds->pending = true;
+    ds->pending_graph = g;
     return FK_OK;
 }
 
@@ -2211,7 +2251,9 @@ fk_status fk_wait_pending(fk_handle h, double* gpu_seconds) {
     FK_HIP(hipEventElapsedTime(&ms, ds->ev0, ds->ev1));
     if (gpu_seconds) *gpu_seconds = ms * 1e-3;
     ds->pending = false;
-    return FK_OK;
+    Graph* g = ds->pending_graph;
+    ds->pending_graph = nullptr;
+    return g ? check_abort(g) : FK_OK;
 }
 
 fk_status fk_decode_chunk(fk_handle h, uint32_t graph_id, const fk_decode_uniforms* u, uint32_t start_offset,

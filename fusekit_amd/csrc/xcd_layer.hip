@@ -58,14 +58,27 @@ __device__ __forceinline__ bool xcd_publish_and_wait(const XcdSync& s, uint32_t 
     }
 }
 
-// Whole block; the wave that starts at thread POLL publishes and polls.
+// Whole block; the wave that starts at thread POLL publishes and polls.  `okw`: one word of LDS through which that
+// wave tells the block how the wait ended.  Returns false (to every thread alike) when the wait gave up or another
+// block had raised the abort word: the caller leaves the launch at once, so that nothing computed from rows that were
+// never finished is appended to a cache or added into a sum row.
 template <int POLL>
-__device__ __forceinline__ void xcd_barrier(XcdSync& s) {
+__device__ __forceinline__ bool xcd_barrier(XcdSync& s, uint32_t* okw) {
     s.epoch += 1;
     wait_memory_ops_done();
     __syncthreads();
-    if (threadIdx.x >= POLL && threadIdx.x < POLL + kWave) (void)xcd_publish_and_wait(s, threadIdx.x - POLL);
+    if (threadIdx.x >= POLL && threadIdx.x < POLL + kWave) {
+        const bool ok = xcd_publish_and_wait(s, threadIdx.x - POLL);
+        if (threadIdx.x == POLL) *okw = ok ? 1u : 0u;
+    }
     __syncthreads();
+    return *okw != 0u;
+}
+
+// Last thing a block does: flip its bit of its XCD's placement word (see XcdControl).
+__device__ __forceinline__ void xcd_mark_placement(const XcdSync& s) {
+    if (threadIdx.x == 0)
+        (void)__hip_atomic_fetch_xor(&s.ctl->placement[s.xcd].bits, 1ull << s.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- activation staging (the chunk-interleaved LDS layout of the streaming GEMV) -------------------
@@ -138,7 +151,11 @@ constexpr int kGuAhead = 3;  // gate requests of the MLP launch that go out ahea
 __device__ __forceinline__ float xcd_sum_to_f32(uint32_t lo, uint32_t hi) {
     return fmaf((float)lo, kXcdSumInv, (float)(int32_t)hi);
 }
-__device__ __forceinline__ void xcd_sum_add(long long* row, uint32_t e, float v) {
+__device__ __forceinline__ void xcd_sum_add(long long* row, uint32_t e, float v, XcdControl* ctl) {
+    if (!(fabsf(v) < kXcdSumLimit)) {  // beyond the fixed-point range, or not finite: clamp and tell the host
+        __hip_atomic_store(&ctl->overflow, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v = v != v ? 0.f : (v < 0.f ? -kXcdSumLimit : kXcdSumLimit);
+    }
     const long long q = __float2ll_rn(v * kXcdSumScale);
     (void)__hip_atomic_fetch_add(reinterpret_cast<unsigned long long*>(row) + xcd_sum_index(e), (unsigned long long)q,
                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -645,7 +662,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
                         [&](uint32_t r, float s0, float s1) { mid[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
     }
     FK_XCD_STAMP(1, 7);
-    xcd_barrier<0>(sync);
+    if (!xcd_barrier<0>(sync, reinterpret_cast<uint32_t*>(red) + 8)) return;
     FK_XCD_STAMP(1, 8);
 
     // ---- down_proj over this XCD's K-slice: fp32 partial row ----
@@ -657,7 +674,8 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     FK_XCD_STAMP(1, 10);
     if (streams && d_n) {
         long long* out = a.out_sums;
-        tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, d0 + r, s0); });
+        XcdControl* ctl = sync.ctl;
+        tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, d0 + r, s0, ctl); });
     }
     FK_XCD_STAMP(1, 11);
 }
@@ -688,6 +706,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const long long* 
     kernarg_warm<32 + (int)sizeof(XcdMlpArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
     xcd_mlp_phase<KIND, NLA, NLB, false, true, ONE>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
+    xcd_mark_placement(sync);
 }
 
 // =============================================================================================== attention launch
@@ -765,7 +784,8 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
         tile_rows<false>(tq, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
     }
     FK_XCD_STAMP(0, 6);
-    xcd_barrier<0>(sync);
+    uint32_t* okw = reinterpret_cast<uint32_t*>(red) + 8;
+    if (!xcd_barrier<0>(sync, okw)) return;
     FK_XCD_STAMP(0, 7);
 
     // ---- head norm + RoPE + cache append + attention: block = (query head of the group, key range) ----
@@ -776,7 +796,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
             sdpa_block<1, 2, std::remove_cv_t<std::remove_reference_t<decltype((a.sdpa))>>, 0, true, true>(a.sdpa, kv_len0, split, sync.xcd, gz, G, work);
     }
     FK_XCD_STAMP(0, 8);
-    xcd_barrier<0>(sync);
+    if (!xcd_barrier<0>(sync, okw)) return;
     FK_XCD_STAMP(0, 9);
 
     // ---- merge the ranges of each of the group's heads (range order), rows to LDS ----
@@ -850,7 +870,8 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     FK_XCD_STAMP(0, 11);
     if (o_n) {
         long long* out = a.out_sums;
-        tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, o0 + r, s0); });
+        XcdControl* ctl = sync.ctl;
+        tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, o0 + r, s0, ctl); });
     }
     FK_XCD_STAMP(0, 12);
 }
@@ -865,6 +886,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const long long* su
     kernarg_warm<32 + (int)sizeof(XcdAttnArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
     xcd_attn_phase<KIND, NLA, NLB, false, true, ONE>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
+    xcd_mark_placement(sync);
 }
 
 // ---- the whole token in one launch --------------------------------------------------------------------------
@@ -965,6 +987,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_token_kernel(const XcdTokenArgs
         }
         if (l + 1 < t.n_layers && !xcd_global_barrier(sync, gs)) return;
     }
+    xcd_mark_placement(sync);
 }
 
 __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
@@ -1078,12 +1101,110 @@ fk_status set_lds_limit(const void* func, uint32_t lds) {
     return FK_OK;
 }
 
-}  // namespace
-
-fk_status xcd_layer_supported(const XcdLayerShape& s) {
+// Both launches need their 512 workgroups resident TOGETHER, two per CU: a block that has not started cannot publish
+// its arrival, and the blocks that did would poll until their spin limit.  First the plain budget (two blocks' LDS in
+// the 160 KiB of a gfx950 CU, whatever device is present -- this part also runs without one), then the device's own
+// answer for the kernel as compiled (registers included).
+constexpr uint32_t kCuLdsBytes = 160u * 1024u;
+fk_status require_two_blocks_per_cu(const void* func, uint32_t lds, const char* what) {
+    if (2u * ((lds + 1023u) & ~1023u) > kCuLdsBytes)
+        return set_error(FK_ERR_UNSUPPORTED, std::string("xcd layer: the ") + what + " launch needs " + std::to_string(lds) +
+                                                 " bytes of LDS per workgroup; two workgroups do not fit one CU, so its 512 "
+                                                 "workgroups cannot all be resident");
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
-    if (dev->cus != (int)(kXcds * 32)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: needs 8 XCDs of 32 CUs");
+    if ((int)lds > dev->max_dyn_lds) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: LDS need exceeds the CU");
+    if (lds > 48 * 1024) FK_HIP(hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    int per_cu = 0;
+    FK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, func, kBlock, lds));
+    if ((long long)per_cu * dev->cus < (long long)kXcdGrid)
+        return set_error(FK_ERR_UNSUPPORTED, std::string("xcd layer: only ") + std::to_string(per_cu) + " workgroup(s) of the " + what +
+                                                 " launch fit one CU on this device; its 512 workgroups cannot all be resident");
+    return FK_OK;
+}
+
+// What a launch's shape decides: tiles, kernel flavour, LDS.
+struct MlpGeometry {
+    uint32_t gate_cpr, down_cpr, gu_rows, down_rows, down_cs;
+    bool one;
+    LdsPlan lp;
+    uint32_t lds;
+    const void* func;
+};
+MlpGeometry mlp_geometry(const XcdLayerShape& s, bool for_token) {
+    MlpGeometry g;
+    const uint32_t cv = chunk_values(s.bits);
+    g.gate_cpr = s.hidden / cv;
+    g.down_cpr = s.inter / cv;
+    g.gu_rows = ceil_div(s.inter / kXcds, kXcdSlots);
+    g.down_rows = ceil_div(s.hidden, kXcdSlots);
+    g.down_cs = g.down_cpr / kXcds;
+    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
+    g.lp.cs_max = g.gate_cpr > g.down_cs ? g.gate_cpr : g.down_cs;
+    const PassDepth deep = depth_of_bits(s.bits);
+    // every tile within one pass (the 4B-class shapes): the flavour compiled without the pass loop
+    g.one = !for_token && g.gu_rows * g.gate_cpr <= (uint32_t)deep.gu * kBlock && g.down_rows * g.down_cs <= (uint32_t)deep.down * kBlock;
+    const PassDepth depth = for_token ? PassDepth{kNlQkv, kNlO, kNlGuToken, kNlDown} : (g.one ? deep : PassDepth{kNlQkv, kNlO, kNlGu, kNlDown});
+    const uint32_t gu = 2 * padded(g.gu_rows * g.gate_cpr, depth.gu), dn = padded(g.down_rows * g.down_cs, depth.down);
+    g.lp.work_floats = gu > dn ? gu : dn;
+    g.lp.att_elems = 0;
+    g.lds = lds_for(s.bits, g.lp);
+    g.func = s.bits == 4 ? mlp_func<W_Q4>(g.one) : (s.bits == 8 ? mlp_func<W_Q8>(g.one) : mlp_func<W_BF16>(g.one));
+    return g;
+}
+
+struct AttnGeometry {
+    uint32_t wq_cpr, wo_cpr, q_rows, kv_rows, R, q_tiles, kv_tiles, o_rows, o_cs;
+    uint32_t chunk_len, chunks_per_block, n_splits;
+    bool one;
+    LdsPlan lp;
+    uint32_t lds;
+    const void* func;
+};
+AttnGeometry attn_geometry(const XcdLayerShape& s) {
+    AttnGeometry g;
+    const uint32_t cv = chunk_values(s.bits), G = s.n_heads / s.n_kv;
+    g.wq_cpr = s.hidden / cv;
+    g.wo_cpr = s.n_heads * s.head_dim / cv;
+    g.q_rows = G * s.head_dim;
+    g.kv_rows = s.head_dim;
+    uint32_t R = 1;
+    while (ceil_div(g.q_rows, R) + 2 * ceil_div(g.kv_rows, R) > kXcdSlots) ++R;
+    g.R = R;
+    g.q_tiles = ceil_div(g.q_rows, R);
+    g.kv_tiles = ceil_div(g.kv_rows, R);
+    g.o_rows = ceil_div(s.hidden, kXcdSlots);
+    g.o_cs = g.wo_cpr / kXcds;
+    // attention of one KV head per XCD: blocks = (query head of the group) x (key range)
+    g.chunk_len = sdpa_chunk_len(s.head_dim, s.head_dim, false);
+    uint32_t splits = kXcdSlots / G;
+    if (splits > kXcdMaxRanges) splits = kXcdMaxRanges;
+    const uint32_t n_chunks = ceil_div(s.capacity, g.chunk_len);
+    g.chunks_per_block = ceil_div(n_chunks, splits);
+    g.n_splits = ceil_div(n_chunks, g.chunks_per_block);
+    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kAttnStream) * nl * kAttnStream; };
+    g.lp.cs_max = g.wq_cpr > g.o_cs ? g.wq_cpr : g.o_cs;
+    // partial rows padded to whole passes: of this launch's depths and of the whole-token launch's (it shares this plan)
+    const PassDepth deep = depth_of_bits(s.bits);
+    g.one = R * g.wq_cpr <= (uint32_t)deep.qkv * kAttnStream && g.o_rows * g.o_cs <= (uint32_t)deep.o * kAttnStream;
+    const PassDepth depth = g.one ? deep : PassDepth{kNlQkv, kNlO, kNlGu, kNlDown};
+    auto larger = [](uint32_t x, uint32_t y) { return x > y ? x : y; };
+    uint32_t wf = larger(padded(R * g.wq_cpr, depth.qkv), padded(R * g.wq_cpr, kNlQkv));
+    const uint32_t wo_ = larger(padded(g.o_rows * g.o_cs, depth.o), padded(g.o_rows * g.o_cs, kNlO));
+    wf = wf > wo_ ? wf : wo_;
+    const uint32_t sf = sdpa_lds_floats(1, g.chunk_len, s.head_dim, s.head_dim, true);
+    g.lp.work_floats = wf > sf ? wf : sf;
+    g.lp.att_elems = G * s.head_dim;
+    g.lds = lds_for(s.bits, g.lp);
+    g.func = s.bits == 4 ? attn_func<W_Q4>(g.one) : (s.bits == 8 ? attn_func<W_Q8>(g.one) : attn_func<W_BF16>(g.one));
+    return g;
+}
+
+}  // namespace
+
+// The shape rules and the LDS budget come first and need no device; the device's CU count and its occupancy answer for
+// the two kernels come last.
+fk_status xcd_layer_supported(const XcdLayerShape& s) {
     if (s.bits != 4 && s.bits != 8 && s.bits != 16) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: bits must be 4, 8 or 16");
     const uint32_t cv = chunk_values(s.bits), unit = s.bits == 16 ? cv : (s.group > cv ? s.group : cv);
     if (s.bits != 16 && s.group != 32 && s.group != 64 && s.group != 128)
@@ -1112,10 +1233,51 @@ fk_status xcd_layer_supported(const XcdLayerShape& s) {
         if (s.hidden % kXcdSlots || (rpb * (n_q / kXcds / s.group)) % 4 || (rpb * (s.inter / kXcds / s.group)) % 4)
             return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a block's o_proj / down_proj tile must hold a multiple of four quantisation groups");
     }
+    const MlpGeometry mg = mlp_geometry(s, false);
+    const AttnGeometry ag = attn_geometry(s);
+    if (2u * ((mg.lds + 1023u) & ~1023u) > kCuLdsBytes || 2u * ((ag.lds + 1023u) & ~1023u) > kCuLdsBytes)
+        return set_error(FK_ERR_UNSUPPORTED, "xcd layer: two workgroups of a launch must fit the LDS of one CU (MLP launch " +
+                                                 std::to_string(mg.lds) + " bytes, attention launch " + std::to_string(ag.lds) +
+                                                 " bytes per workgroup): its 512 workgroups could not all be resident");
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (dev->cus != (int)(kXcds * 32)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: needs 8 XCDs of 32 CUs");
+    FK_TRY(require_two_blocks_per_cu(mg.func, mg.lds, "MLP"));
+    FK_TRY(require_two_blocks_per_cu(ag.func, ag.lds, "attention"));
     return FK_OK;
 }
 
 size_t xcd_workspace_bytes() { return sizeof(XcdControl); }
+
+fk_status xcd_check_control(void* workspace) {
+    if (!workspace) return set_error(FK_ERR_INVALID, "xcd layer: null control block");
+    static_assert(offsetof(XcdControl, abort_flag) == sizeof(uint32_t) * kXcds * kXcdSlots, "control block layout");
+    // everything behind the arrival words in one copy
+    constexpr size_t off = offsetof(XcdControl, abort_flag);
+    alignas(8) unsigned char tail[sizeof(XcdControl) - off];
+    FK_HIP(hipMemcpy(tail, reinterpret_cast<const char*>(workspace) + off, sizeof(tail), hipMemcpyDeviceToHost));
+    auto word = [&](size_t o) {
+        uint32_t v;
+        memcpy(&v, tail + (o - off), 4);
+        return v;
+    };
+    const char* what = nullptr;
+    if (word(offsetof(XcdControl, abort_flag)))
+        what = "a hand-over wait exceeded its spin limit";
+    else if (word(offsetof(XcdControl, overflow)))
+        what = "a contribution to a sum row was not finite or reached 2^27 in magnitude (the fixed-point range)";
+    else
+        for (uint32_t x = 0; x < kXcds; ++x) {
+            unsigned long long bits;
+            memcpy(&bits, tail + (offsetof(XcdControl, placement) + x * sizeof(XcdPlacement) - off), 8);
+            if (bits != 0ull && bits != ~0ull) what = "two workgroups of a launch ran in the same (XCD, slot): the dispatch order is not the round-robin dealing the layer cut relies on";
+        }
+    if (!what) return FK_OK;
+    // the arrival words of a failed launch are inconsistent: start over from zero
+    FK_HIP(hipMemset(workspace, 0, sizeof(XcdControl)));
+    return set_error(FK_ERR_HIP, std::string("xcd layer: ") + what +
+                                     "; results are invalid (the control block was reset; zero the sum rows and decode the token again)");
+}
 size_t xcd_sum_row_bytes(uint32_t hidden) { return (size_t)xcd_sum_row_elems(hidden) * sizeof(long long); }
 
 size_t xcd_attn_partials_bytes(const XcdLayerShape& s) {
@@ -1133,28 +1295,23 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     FK_TRY(bind_mat(rq.wgate, s.inter, s.hidden, s, &a.gate, "gate_proj"));
     FK_TRY(bind_mat(rq.wup, s.inter, s.hidden, s, &a.up, "up_proj"));
     FK_TRY(bind_mat(rq.wdown, s.hidden, s.inter, s, &a.down, "down_proj"));
+    const MlpGeometry g = mlp_geometry(s, rq.for_token);
     a.inter = s.inter;
-    a.gu_rows = ceil_div(s.inter / kXcds, kXcdSlots);
-    a.down_rows = ceil_div(s.hidden, kXcdSlots);
-    a.down_cs = a.down.cpr / kXcds;
+    a.gu_rows = g.gu_rows;
+    a.down_rows = g.down_rows;
+    a.down_cs = g.down_cs;
     a.swiglu_variant = rq.swiglu_variant;
     a.mid = rq.mid;
     a.out_sums = rq.out_sums;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
-    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kBlock) * nl * kBlock; };
-    LdsPlan lp;
-    lp.cs_max = a.gate.cpr > a.down_cs ? a.gate.cpr : a.down_cs;
-    const PassDepth deep = depth_of_bits(s.bits);
-    // every tile within one pass (the 4B-class shapes): the flavour compiled without the pass loop
-    const bool one = !rq.for_token && a.gu_rows * a.gate.cpr <= (uint32_t)deep.gu * kBlock && a.down_rows * a.down_cs <= (uint32_t)deep.down * kBlock;
-    const PassDepth depth = rq.for_token ? PassDepth{kNlQkv, kNlO, kNlGuToken, kNlDown} : (one ? deep : PassDepth{kNlQkv, kNlO, kNlGu, kNlDown});
-    const uint32_t gu = 2 * padded(a.gu_rows * a.gate.cpr, depth.gu), dn = padded(a.down_rows * a.down_cs, depth.down);
-    lp.work_floats = gu > dn ? gu : dn;
-    lp.att_elems = 0;
-    const uint32_t lds = lds_for(s.bits, lp);
-    out->func = s.bits == 4 ? mlp_func<W_Q4>(one) : (s.bits == 8 ? mlp_func<W_Q8>(one) : mlp_func<W_BF16>(one));
-    FK_TRY(set_lds_limit(out->func, lds));
+    const LdsPlan lp = g.lp;
+    const uint32_t lds = g.lds;
+    out->func = g.func;
+    if (rq.for_token)
+        FK_TRY(set_lds_limit(out->func, lds));  // an argument block for the whole-token launch, which is planned (and checked) as a whole
+    else
+        FK_TRY(require_two_blocks_per_cu(out->func, lds, "MLP"));
     out->grid = dim3(kXcdGrid, 1, 1);
     out->block = dim3(kMlpBlock, 1, 1);
     out->shmem = lds;
@@ -1176,7 +1333,7 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
         !rq.out_sums || !rq.workspace)
         return set_error(FK_ERR_INVALID, "xcd attention: null buffer");
     if ((rq.q_norm == nullptr) != (rq.k_norm == nullptr)) return set_error(FK_ERR_INVALID, "xcd attention: q and k head norms come together");
-    const uint32_t G = s.n_heads / s.n_kv, n_q = s.n_heads * s.head_dim, n_kvd = s.n_kv * s.head_dim;
+    const uint32_t n_q = s.n_heads * s.head_dim, n_kvd = s.n_kv * s.head_dim;
     XcdAttnArgs a;
     memset(&a, 0, sizeof(a));
     FK_TRY(fill_input(s, rq.sums_in, rq.residual, rq.x_out, rq.clear, rq.out_sums, rq.norm_w, rq.eps, &a.in));
@@ -1184,15 +1341,14 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     FK_TRY(bind_mat(rq.wk, n_kvd, s.hidden, s, &a.wk, "k_proj"));
     FK_TRY(bind_mat(rq.wv, n_kvd, s.hidden, s, &a.wv, "v_proj"));
     FK_TRY(bind_mat(rq.wo, s.hidden, n_q, s, &a.wo, "o_proj"));
-    a.q_rows = G * s.head_dim;
-    a.kv_rows = s.head_dim;
-    uint32_t R = 1;
-    while (ceil_div(a.q_rows, R) + 2 * ceil_div(a.kv_rows, R) > kXcdSlots) ++R;
-    a.qkv_tile_rows = R;
-    a.q_tiles = ceil_div(a.q_rows, R);
-    a.kv_tiles = ceil_div(a.kv_rows, R);
-    a.o_rows = ceil_div(s.hidden, kXcdSlots);
-    a.o_cs = a.wo.cpr / kXcds;
+    const AttnGeometry g = attn_geometry(s);
+    a.q_rows = g.q_rows;
+    a.kv_rows = g.kv_rows;
+    a.qkv_tile_rows = g.R;
+    a.q_tiles = g.q_tiles;
+    a.kv_tiles = g.kv_tiles;
+    a.o_rows = g.o_rows;
+    a.o_cs = g.o_cs;
     a.q = rq.q;
     a.k = rq.k;
     a.v = rq.v;
@@ -1207,12 +1363,9 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     sd.n_kv = s.n_kv;
     sd.qk_dim = sd.v_dim = s.head_dim;
     sd.capacity = s.capacity;
-    sd.chunk_len = sdpa_chunk_len(s.head_dim, s.head_dim, false);
-    uint32_t splits = kXcdSlots / G;
-    if (splits > kXcdMaxRanges) splits = kXcdMaxRanges;
-    const uint32_t n_chunks = ceil_div(s.capacity, sd.chunk_len);
-    sd.chunks_per_block = ceil_div(n_chunks, splits);
-    sd.n_splits = ceil_div(n_chunks, sd.chunks_per_block);
+    sd.chunk_len = g.chunk_len;
+    sd.chunks_per_block = g.chunks_per_block;
+    sd.n_splits = g.n_splits;
     sd.rows = 1;
     uint32_t lp_ = 1;
     while (lp_ < s.head_dim / 8) lp_ <<= 1;
@@ -1235,23 +1388,10 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     a.out_sums = rq.out_sums;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
-    auto padded = [](uint32_t chunks, int nl) { return ceil_div(chunks, nl * kAttnStream) * nl * kAttnStream; };
-    LdsPlan lp;
-    lp.cs_max = a.wq.cpr > a.o_cs ? a.wq.cpr : a.o_cs;
-    // partial rows padded to whole passes: of this launch's depths and of the whole-token launch's (it shares this plan)
-    const PassDepth deep = depth_of_bits(s.bits);
-    const bool one = R * a.wq.cpr <= (uint32_t)deep.qkv * kAttnStream && a.o_rows * a.o_cs <= (uint32_t)deep.o * kAttnStream;
-    const PassDepth depth = one ? deep : PassDepth{kNlQkv, kNlO, kNlGu, kNlDown};
-    auto larger = [](uint32_t x, uint32_t y) { return x > y ? x : y; };
-    uint32_t wf = larger(padded(R * a.wq.cpr, depth.qkv), padded(R * a.wq.cpr, kNlQkv));
-    const uint32_t wo_ = larger(padded(a.o_rows * a.o_cs, depth.o), padded(a.o_rows * a.o_cs, kNlO));
-    wf = wf > wo_ ? wf : wo_;
-    const uint32_t sf = sdpa_lds_floats(1, sd.chunk_len, s.head_dim, s.head_dim, true);
-    lp.work_floats = wf > sf ? wf : sf;
-    lp.att_elems = G * s.head_dim;
-    const uint32_t lds = lds_for(s.bits, lp);
-    out->func = s.bits == 4 ? attn_func<W_Q4>(one) : (s.bits == 8 ? attn_func<W_Q8>(one) : attn_func<W_BF16>(one));
-    FK_TRY(set_lds_limit(out->func, lds));
+    const LdsPlan lp = g.lp;
+    const uint32_t lds = g.lds;
+    out->func = g.func;
+    FK_TRY(require_two_blocks_per_cu(out->func, lds, "attention"));
     out->grid = dim3(kXcdGrid, 1, 1);
     out->block = dim3(kBlock, 1, 1);
     out->shmem = lds;
@@ -1295,7 +1435,7 @@ fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uin
         return reinterpret_cast<const void*>(&xcd_token_kernel<W_BF16, kNlQkv, kNlO, kNlGuToken, kNlDown>);
     };
     out->func = func();
-    FK_TRY(set_lds_limit(out->func, lds));
+    FK_TRY(require_two_blocks_per_cu(out->func, lds, "whole-token"));
     out->grid = dim3(kXcdGrid, 1, 1);
     out->block = dim3(kBlock, 1, 1);
     out->shmem = lds;

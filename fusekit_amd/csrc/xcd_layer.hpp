@@ -50,13 +50,28 @@ constexpr uint32_t kXcdMaxRanges = 16;              // key ranges merged per que
 //   abort          uint32   set when a wait ran into the spin limit
 //   arrivals       uint32   device-wide barrier of the whole-token launch: XCD leaders arrived (memory-side adds)
 //   release[8]     uint32   ... and the word each XCD's leader releases its XCD with
+//   overflow       uint32   set when a contribution to a sum row was not finite or lay beyond the fixed-point range
+//   placement[8]   uint64   one word per XCD, each in a 256-byte line of its own: every block of a launch flips bit
+//                           `slot` of its XCD's word when it ends (a memory-side xor that returns nothing).  With one
+//                           block per (XCD, slot) all 64 bits of a word flip together, so between launches every word
+//                           is all zeros or all ones; anything else means two blocks shared a slot and the host
+//                           reports it.  (Two blocks in one slot also leave some slot of another XCD empty, whose
+//                           arrival word then never advances: the hand-over waits of that XCD give up and the launch
+//                           already reports through the abort word.  The placement words name the cause.)
+struct XcdPlacement {
+    unsigned long long bits;
+    uint32_t pad[62];
+};
 struct XcdControl {
     uint32_t flags[kXcds * kXcdSlots];
     uint32_t abort_flag;
     uint32_t arrivals;
     uint32_t release[kXcds];
-    uint32_t pad[54];
+    uint32_t overflow;
+    uint32_t pad[53];
+    XcdPlacement placement[kXcds];
 };
+static_assert(sizeof(XcdControl) == 2304 + 8 * 256, "control block layout");
 
 // A sum row: hidden 64-bit fixed-point sums (value * 2^32), padded to whole 512-element sections.  Inside a
 // section the elements are permuted so that the control wave of a block, whose lane l takes the eight
@@ -64,6 +79,11 @@ struct XcdControl {
 // xcd_sum_index(e).
 constexpr float kXcdSumScale = 4294967296.0f;
 constexpr float kXcdSumInv = 1.0f / 4294967296.0f;
+// Range of one contribution: |v| < 2^27, so that eight of them (one per XCD) stay far inside 64 bits.  A contribution
+// at or beyond it, or one that is not finite, is clamped and raises XcdControl::overflow, which the host reports as
+// an error (the reference's bf16 row would carry such a value on; a row of fixed-point sums cannot).  Resolution:
+// 2^-32 per contribution, i.e. below half a bf16 step of any result of magnitude >= 2^-24.
+constexpr float kXcdSumLimit = 134217728.0f;
 __host__ __device__ inline uint32_t xcd_sum_index(uint32_t e) {
     const uint32_t t = e >> 3;
     return (((((t >> 6) * 4u + ((e & 7u) >> 1)) * 64u + (t & 63u)) << 1) | (e & 1u));
@@ -158,6 +178,13 @@ struct XcdLayerShape {
 // whole quantisation groups, tiles that fit the per-thread load budget.)  Sets an error message if not.
 fk_status xcd_layer_supported(const XcdLayerShape& s);
 size_t xcd_workspace_bytes();
+// Reads the control block after the launches that use it have completed (the caller has synchronised).  FK_OK when
+// nothing was raised; otherwise the block is reset to zeros and FK_ERR_HIP says which of the three it was: a hand-over
+// wait that gave up, a sum-row contribution outside the fixed-point range, two blocks of a launch in one slot.  After
+// an error the sum rows the launches added into hold partial sums and the cache rows of the token's position may hold
+// values built from unfinished rows: the caller zeroes the sum rows and decodes that token again (which rewrites the
+// cache rows).
+fk_status xcd_check_control(void* workspace);
 size_t xcd_sum_row_bytes(uint32_t hidden);
 // Scales (or biases) [n, groups] -> [8][n][groups / 8]: what the o_proj / down_proj slots of the launches take.
 fk_status xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint16_t* dst, hipStream_t stream);

@@ -514,13 +514,26 @@ fk_status fk_rope_store_sdpa_decode(const uint16_t *q, const uint16_t *k, const 
  * Three rows rotate through the launches of a token: a launch reads one (the previous launch's), adds into
  * the second and clears the third (the one the launch after it adds into); the row the first launch of a
  * token adds into must hold zeros (fusekit_xcd_reduce clears it at the end of the previous token; zero all
- * three once after allocation, and again after a launch has reported an abort).  Non-finite projection
- * outputs are not carried through a sum row.  Slot orders are documented at the planners
+ * three once after allocation, and again after a launch has reported an error -- the dispatcher does that
+ * for the rows bound to a graph).  One contribution must be finite and below 2^27 in magnitude; a launch that
+ * meets another clamps it and raises a word of the control block, reported as FK_ERR_HIP by the next check
+ * (resolution: 2^-32 per contribution).  Slot orders are documented at the planners
  * (fusekit_amd/csrc/dispatcher.hip).  Requires 8 KV heads (one per XCD), 1 / 2 / 4 / 8 query heads per KV
- * head, head_dim 64 or 128, hidden <= 4096; other layers use the per-dispatch families. */
+ * head, head_dim 64 or 128, hidden <= 4096, and a shape whose workgroups fit two per CU (LDS and registers:
+ * answered from the shape where possible, else by the device's occupancy query); other layers use the
+ * per-dispatch families.
+ *
+ * EXCLUSIVE USE OF THE DEVICE.  A launch of these families is 512 workgroups that wait for one another inside
+ * the launch, so all of them must be resident at once, two per CU of all 256 CUs, dealt to the XCDs round-robin.
+ * Nothing else may run on the device while such a launch runs: no kernel of another stream, process or graph
+ * branch.  fk_build_graph refuses a graph in which any other node is not ordered before or after such a
+ * launch.  A launch that cannot make progress does not hang: every wait is bounded (parameter spin_limit),
+ * gives up, and the error is reported by fk_xcd_check / by the dispatcher call that executed the graph;
+ * the results of that token are then invalid -- decode it again (the retry rewrites the cache rows). */
 fk_status fk_xcd_layer_supported(uint32_t hidden, uint32_t inter, uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                  uint32_t capacity, uint32_t bits, uint32_t group);
-/* Bytes of the control block (arrival words, abort word; zero it once) and of the attention partial rows. */
+/* Bytes of the control block (arrival words, abort / overflow words, placement words; zero it once) and of the
+ * attention partial rows. */
 fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t *control_bytes, size_t *attention_partial_bytes);
 /* Bytes of one sum row of a hidden-wide vector (0 for hidden == 0). */
 size_t fk_xcd_sum_row_bytes(uint32_t hidden);
@@ -530,8 +543,11 @@ size_t fk_xcd_sum_row_bytes(uint32_t hidden);
  * MLX layout its 16..38 bytes of every row drag whole 128-byte lines into all eight L2s.  Done once per matrix
  * at load time; the weights themselves stay in the MLX layout (src/fusion/ir.rs:236-242). */
 fk_status fk_xcd_kslice_meta(const uint16_t *src, uint32_t n, uint32_t groups, uint16_t *dst, fk_stream s);
-/* Synchronises the stream and reports whether a launch gave up on a hand-over wait (FK_ERR_HIP; the control
- * block is reset).  The dispatcher calls it after every graph execution that holds such launches. */
+/* Synchronises the stream and reports (FK_ERR_HIP, control block reset to zeros) whether a launch gave up on a
+ * hand-over wait, met a contribution outside the sum rows' range, or ran two workgroups in one (XCD, slot).  The
+ * dispatcher does the same check after every execution of a graph that holds such launches -- synchronous,
+ * range, per-node profile, decode chunks, and in fk_wait_pending for the asynchronous pair -- and zeroes the
+ * graph's sum rows when it fails. */
 fk_status fk_xcd_check(void *workspace, fk_stream s);
 
 /* ---- dispatcher: replaces `_fusekit_runtime_native` ------------------------

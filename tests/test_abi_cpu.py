@@ -96,3 +96,20 @@ def test_target_description_without_a_gpu():
     if not t.from_device:
         assert (t.compute_units, t.xcds, t.lds_bytes_per_cu) == (256, 8, 160 * 1024)
         assert t.hbm_peak_bytes_per_s == 8.0e12 and t.hbm_bytes == 288 << 30
+
+
+def test_two_launch_layer_admission_rules_need_no_device():
+    """The shape rules of the two-launch layer, the LDS budget among them, are checked before any device is asked:
+    a bf16 layer of hidden 4096 / intermediate 14336 needs more than half a CU's LDS per workgroup, so its 512
+    workgroups could not all be resident (the hand-overs need that) -- refused as unsupported, on any machine."""
+    import fusekit_amd.native as fk
+    u = C.c_uint32
+    st = fk.lib.fk_xcd_layer_supported(u(4096), u(14336), u(32), u(8), u(128), u(1024), u(16), u(64))
+    assert st == fk.FK_ERR_UNSUPPORTED and b"resident" in fk.lib.fk_last_error()
+    st = fk.lib.fk_xcd_layer_supported(u(4096), u(12288), u(32), u(8), u(128), u(1024), u(16), u(64))
+    assert st == fk.FK_ERR_UNSUPPORTED and b"resident" in fk.lib.fk_last_error()
+    st = fk.lib.fk_xcd_layer_supported(u(2560), u(9728), u(32), u(4), u(128), u(1024), u(4), u(64))
+    assert st == fk.FK_ERR_UNSUPPORTED and b"8 KV heads" in fk.lib.fk_last_error()
+    # the 4B-class shape passes every rule; without a device the answer is then "no HIP device"
+    st = fk.lib.fk_xcd_layer_supported(u(2560), u(9728), u(32), u(8), u(128), u(1024), u(4), u(64))
+    assert st == (fk.FK_OK if fk.has_device() else fk.FK_ERR_HIP), fk.lib.fk_last_error()

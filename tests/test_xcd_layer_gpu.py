@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
+from helpers import OracleDecoder, bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
 
 pytestmark = pytest.mark.gpu
 
@@ -75,12 +75,35 @@ def _close_bf16(got, ref_bits, ref_f32=None, frac=0.02, ulps=1.0):
 @pytest.mark.parametrize("bits", [4, 8, 16])
 @pytest.mark.parametrize("hidden,inter,variant", [(512, 1024, 0), (2560, 9728, 1), (1024, 3072, 2)])
 def test_xcd_mlp_block(fk, bits, hidden, inter, variant):
+    _run_mlp_block(fk, bits, hidden, inter, variant)
+
+
+@pytest.mark.parametrize("gain,lo,hi", [(3.0e3, 2.0 ** 20, 2.0 ** 27), (1.5e-6, 0.0, 2.0 ** -26)])
+def test_xcd_sum_row_carries_large_and_tiny_contributions(fk, gain, lo, hi):
+    """The kernel's own add path at the ends of the fixed-point range: a norm weight scaled by `gain` puts the
+    down_proj K-slice sums of the 4B-class shape near 2^26 (the range of one contribution ends at 2^27), resp. near
+    the 2^-32 resolution.  Same checks as the plain test: the row equals the float64 product to 2e-6 of its
+    absolute terms + 8 half-units, and the next input equals the oracle's down projection + residual."""
+    peak = _run_mlp_block(fk, 4, 2560, 9728, 1, norm_gain=gain)
+    assert lo <= peak <= hi, peak
+
+
+def test_xcd_sum_row_reports_a_contribution_beyond_its_range(fk):
+    """A K-slice sum of 2^27 or more cannot be carried by the fixed-point row: the launch clamps it, raises the
+    overflow word, and the host reports an error instead of handing on a wrong row."""
+    with pytest.raises(fk.FusekitError) as e:
+        _run_mlp_block(fk, 4, 2560, 9728, 1, norm_gain=4.0e4)
+    assert "fixed-point range" in str(e.value)
+
+
+def _run_mlp_block(fk, bits, hidden, inter, variant, norm_gain=1.0):
     from fusekit_amd.runtime import Dispatch, Dispatcher, arg
     if not fk.xcd_layer_supported(hidden, inter, 32, 8, 128, 256, bits, 64):
         pytest.skip("shape not supported: " + fk.lib.fk_last_error().decode())
     d = Dispatcher()
     Wg, Wu, Wd = make_qweight(1, inter, hidden, bits), make_qweight(2, inter, hidden, bits), make_qweight(3, hidden, inter, bits)
-    norm_w = normal_bf16(4, hidden, 0.1, 1.0)
+    norm_w = oracle.f32_to_bf16((oracle.bf16_to_f32(normal_bf16(4, hidden, 0.1, 1.0)) * np.float32(norm_gain)).astype(np.float32))
+    peak = 0.0
     partials = (rng(5).standard_normal((8, hidden), dtype=np.float32) * 0.3).astype(np.float32)
     res = normal_bf16(6, hidden)
     dWg, dWu, dWd = (to_device(fk, W) for W in (Wg, Wu, Wd))
@@ -114,6 +137,7 @@ def test_xcd_mlp_block(fk, bits, hidden, inter, variant):
         m64 = oracle.bf16_to_f32(got_mid).astype(np.float64)
         ref, scale = wd @ m64, np.abs(wd) @ np.abs(m64)
         assert np.all(np.abs(out - ref) <= 2e-6 * scale + 8 * 2.0 ** -33)
+        peak = max(peak, float(np.abs(out).max()))
         pad = np.ones(row_out.size, bool)
         pad[fk.xcd_sum_index(hidden)] = False
         assert not row_out[pad].any()
@@ -126,6 +150,7 @@ def test_xcd_mlp_block(fk, bits, hidden, inter, variant):
         b["p"].upload(row_in)
         b["out"].upload(_sum_row(fk, hidden))
         b["clr"].upload(junk)
+    return peak
 
 
 @pytest.mark.parametrize("bits", [4, 16])
@@ -308,6 +333,57 @@ def test_xcd_wait_gives_up_and_reports(fk):
             rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, [5])
     assert "spin limit" in str(e.value)
     assert not rt.xcd_ctl.to_numpy(np.uint32).any()
+    # the partial sums the failed launch left behind are gone as well: the next token starts from zero rows
+    assert not any(row.to_numpy(np.int64).any() for row in rt.xcd_sums)
+    # the asynchronous pair reports it too (the error belongs to the wait)
+    with pytest.raises(fk.FusekitError) as e2:
+        for _ in range(50):
+            rt.d.submit_graph_async(rt.graph)
+            rt.d.wait_pending()
+    assert "spin limit" in str(e2.value)
+    assert not any(row.to_numpy(np.int64).any() for row in rt.xcd_sums)
+
+
+def test_placement_words_flip_together(fk):
+    """Every block of a launch flips its bit of its XCD's placement word as it ends: after any number of launches
+    each of the eight words is all zeros or all ones (one block per (XCD, slot)), which is what the host checks."""
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    cfg = DecoderConfig(n_layers=3, hidden=512, n_heads=16, n_kv=8, head_dim=64, inter=1024, vocab=512, capacity=64, qk_norm=True)
+    rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=2))
+    assert rt.xcd
+    seen = set()
+    for n in (1, 2, 5):
+        rt.generate([7, 8, 9], n)
+        ctl = rt.xcd_ctl.to_numpy(np.uint8)
+        words = [int(np.frombuffer(ctl[2304 + 256 * x: 2304 + 256 * x + 8].tobytes(), np.uint64)[0]) for x in range(8)]
+        assert all(w in (0, 2 ** 64 - 1) for w in words), [hex(w) for w in words]
+        assert len(set(words)) == 1
+        seen.add(words[0])
+    # a word in any other state is reported
+    ctl = rt.xcd_ctl.to_numpy(np.uint8).copy()
+    ctl[2304 + 256 * 3] ^= 1
+    rt.xcd_ctl.upload(ctl)
+    with pytest.raises(fk.FusekitError) as e:
+        fk.xcd_check(rt.xcd_ctl)
+    assert "same (XCD, slot)" in str(e.value)
+    assert not rt.xcd_ctl.to_numpy(np.uint8).any()
+
+
+def test_shapes_whose_workgroups_cannot_all_be_resident_are_refused(fk):
+    """Two workgroups per CU are a precondition of the hand-overs.  A bf16 8B-class layer (hidden 4096, intermediate
+    14336) needs more than half a CU's LDS per workgroup in the MLP launch: refused at plan time, and the decoder
+    takes the per-dispatch path.  Nothing of that shape is launched XCD-resident here."""
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    assert not fk.xcd_layer_supported(4096, 14336, 32, 8, 128, 1024, 16, 64)
+    assert "resident" in fk.lib.fk_last_error().decode()
+    cfg = DecoderConfig(n_layers=1, hidden=4096, n_heads=32, n_kv=8, head_dim=128, inter=14336, vocab=512, capacity=64,
+                        qk_norm=True, bits=16)
+    W = DecoderWeights.random_init(cfg, seed=3)
+    rt = DecoderRuntime(cfg, W)
+    assert not rt.xcd
+    toks, _, _ = rt.generate([1, 2, 3], 4)
+    ref, _ = OracleDecoder(cfg, W).generate([1, 2, 3], 4)
+    assert toks == ref
 
 
 @pytest.mark.parametrize("bits", [4, 8, 16])
