@@ -664,7 +664,8 @@ XcdLayerShape xcd_shape(const Dispatch& d) {
 // (sums_in: the sum row the previous launch added into; out_sums: the row this launch adds into, zero on entry;
 // clear_sums: the row this launch zeroes; residual and x_out: one bf16 row each.)
 // Parameters: the layer shape (hidden, inter, n_heads, n_kv, head_dim, capacity, bits, group), eps, theta,
-// has_sums, has_norm, spin_limit.
+// has_sums, has_norm, spin_limit, mark_placement (every block flips its bit of its XCD's placement word as it ends;
+// set on one launch per token).
 fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const XcdLayerShape s = xcd_shape(d);
     const bool has_p = d.u("has_sums", 1) != 0, norm = d.u("has_norm", 0) != 0, q = s.bits != 16;
@@ -739,6 +740,7 @@ fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
     rq.workspace = d.args[ws_slot].ptr;
     rq.spin_limit = d.u("spin_limit", 0);
+    rq.mark_placement = d.u("mark_placement", 0) != 0;
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
     rw->writes = {(uint32_t)x_slot, (uint32_t)q_slot, (uint32_t)q_slot + 1, (uint32_t)q_slot + 2, (uint32_t)ck_slot,
                   (uint32_t)cv_slot, (uint32_t)ap_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
@@ -792,6 +794,7 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
     rq.workspace = d.args[ws_slot].ptr;
     rq.spin_limit = d.u("spin_limit", 0);
+    rq.mark_placement = d.u("mark_placement", 0) != 0;
     rq.for_token = d.u("token", 0) != 0;
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
     rw->writes = {(uint32_t)x_slot, (uint32_t)mid_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};

@@ -6,22 +6,9 @@
 
 #include "fk_host.hpp"
 
-#ifdef FK_PROBE_STAMPS
-// Timing-probe build only: per-block clocks at the phase boundaries of the GEMV.
-__device__ unsigned long long g_fk_gemv_stamp[2048 * 8];
-#define FK_GEMV_STAMP(i)                                                                   \
-    do {                                                                                   \
-        if (threadIdx.x == 0 && blockIdx.x < 2048) g_fk_gemv_stamp[blockIdx.x * 8 + (i)] = wall_clock64(); \
-    } while (0)
-extern "C" __attribute__((visibility("default"))) int fk_probe_read_gemv_stamps(unsigned long long* out) {
-    const size_t bytes = sizeof(unsigned long long) * 2048 * 8;
-    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fk_gemv_stamp), bytes);
-    if (e != hipSuccess) return (int)e;
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_fk_gemv_stamp));  // cleared for the next launch
-    return (int)(e != hipSuccess ? e : hipMemset(p, 0, bytes));
-}
-#endif
+#include "fk_probe.hpp"
+FK_PROBE_DEFINE(gemv, 2048, 8)
+#define FK_GEMV_STAMP(i) FK_PROBE_STAMP(gemv, 2048, 8, blockIdx.x, threadIdx.x == 0, i)
 #include "gemv_kernel.hpp"
 #include "gemv_rows.hpp"
 

@@ -19,24 +19,9 @@
 #include "fk_host.hpp"
 #include "gemv_kernel.hpp"
 
-#ifdef FK_PROBE_STAMPS
-// Timing-probe build only: clocks of the first wave of every block at the phase boundaries.
-__device__ unsigned long long g_fk_wide_stamp[2048 * 8];
-#define FK_WIDE_STAMP(i)                                                                                  \
-    do {                                                                                                  \
-        if (threadIdx.x == 0 && blockIdx.x < 2048) g_fk_wide_stamp[blockIdx.x * 8 + (i)] = wall_clock64(); \
-    } while (0)
-extern "C" __attribute__((visibility("default"))) int fk_probe_read_wide_stamps(unsigned long long* out) {
-    const size_t bytes = sizeof(unsigned long long) * 2048 * 8;
-    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fk_wide_stamp), bytes);
-    if (e != hipSuccess) return (int)e;
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_fk_wide_stamp));
-    return (int)(e != hipSuccess ? e : hipMemset(p, 0, bytes));
-}
-#else
-#define FK_WIDE_STAMP(i)
-#endif
+#include "fk_probe.hpp"
+FK_PROBE_DEFINE(wide, 2048, 8)
+#define FK_WIDE_STAMP(i) FK_PROBE_STAMP(wide, 2048, 8, blockIdx.x, threadIdx.x == 0, i)
 
 namespace fk {
 

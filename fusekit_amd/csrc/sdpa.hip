@@ -18,23 +18,10 @@
 // arrival order) and resets the counter for the next launch.
 #include "fk_host.hpp"
 
-#ifdef FK_PROBE_STAMPS
-// Timing-probe build only: per-block clocks at the phase boundaries of the decode attention.
-__device__ unsigned long long g_fk_sdpa_stamp[4096 * 10];
-#define FK_SDPA_STAMP(i)                                                                                  \
-    do {                                                                                                  \
-        const uint32_t b_ = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);               \
-        if (threadIdx.x == 0 && b_ < 4096) g_fk_sdpa_stamp[b_ * 10 + (i)] = wall_clock64();               \
-    } while (0)
-extern "C" __attribute__((visibility("default"))) int fk_probe_read_sdpa_stamps(unsigned long long* out) {
-    const size_t bytes = sizeof(unsigned long long) * 4096 * 10;
-    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fk_sdpa_stamp), bytes);
-    if (e != hipSuccess) return (int)e;
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_fk_sdpa_stamp));  // cleared for the next launch
-    return (int)(e != hipSuccess ? e : hipMemset(p, 0, bytes));
-}
-#endif
+#include "fk_probe.hpp"
+FK_PROBE_DEFINE(sdpa, 4096, 10)
+#define FK_SDPA_STAMP(i) \
+    FK_PROBE_STAMP(sdpa, 4096, 10, blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), threadIdx.x == 0, i)
 #include "sdpa_kernel.hpp"
 
 namespace fk {

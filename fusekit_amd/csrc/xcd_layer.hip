@@ -1,20 +1,11 @@
 // XCD-resident decoder layer: the attention launch and the MLP launch (see xcd_layer.hpp for the scheme).
 #include "xcd_layer.hpp"
 
-// Hook for timing probes: a probe build defines FK_PROBE_STAMPS and records a clock per block at the phase
-// boundaries of both launches; the library build leaves the macro empty.
-#ifdef FK_PROBE_STAMPS
-__device__ unsigned long long g_fk_xcd_stamp[2][512 * 16];
-#define FK_XCD_STAMP(k, i)                                                                      \
-    do {                                                                                        \
-        if (threadIdx.x == 0 || threadIdx.x == 256) g_fk_xcd_stamp[k][blockIdx.x * 16 + (i)] = wall_clock64(); \
-    } while (0)
-extern "C" __attribute__((visibility("default"))) int fk_probe_read_xcd_stamps(unsigned long long* out) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fk_xcd_stamp), sizeof(unsigned long long) * 2 * 512 * 16);
-}
-#else
-#define FK_XCD_STAMP(k, i)
-#endif
+// Timing probes (empty in the library build): launch k (0 attention, 1 MLP), boundary i, by the first thread of
+// the block's first and last wave-pair.
+#include "fk_probe.hpp"
+FK_PROBE_DEFINE(xcd, 1024, 16)
+#define FK_XCD_STAMP(k, i) FK_PROBE_STAMP(xcd, 1024, 16, (k) * 512 + blockIdx.x, threadIdx.x == 0 || threadIdx.x == 256, i)
 
 namespace fk {
 namespace {
@@ -59,11 +50,13 @@ __device__ __forceinline__ bool xcd_publish_and_wait(const XcdSync& s, uint32_t 
 }
 
 // Whole block; the wave that starts at thread POLL publishes and polls.  `okw`: one word of LDS through which that
-// wave tells the block how the wait ended.  Returns false (to every thread alike) when the wait gave up or another
-// block had raised the abort word: the caller leaves the launch at once, so that nothing computed from rows that were
-// never finished is appended to a cache or added into a sum row.
+// wave tells the block how the wait ended: 0 when it gave up or another block had raised the abort word.  The caller
+// reads the word after the barrier (xcd_wait_ok) and, once it is 0, does nothing that outlives the launch -- no cache
+// append, no addition into a sum row -- with values built from rows that were never finished.  Where nothing of that
+// kind follows at once, the word is read at the barrier and tested only in front of those effects, so that the LDS
+// round trip is not on the path.
 template <int POLL>
-__device__ __forceinline__ bool xcd_barrier(XcdSync& s, uint32_t* okw) {
+__device__ __forceinline__ void xcd_barrier(XcdSync& s, uint32_t* okw) {
     s.epoch += 1;
     wait_memory_ops_done();
     __syncthreads();
@@ -72,12 +65,14 @@ __device__ __forceinline__ bool xcd_barrier(XcdSync& s, uint32_t* okw) {
         if (threadIdx.x == POLL) *okw = ok ? 1u : 0u;
     }
     __syncthreads();
-    return *okw != 0u;
 }
+__device__ __forceinline__ bool xcd_wait_ok(const uint32_t* okw) { return *reinterpret_cast<const volatile uint32_t*>(okw) != 0u; }
 
-// Last thing a block does: flip its bit of its XCD's placement word (see XcdControl).
-__device__ __forceinline__ void xcd_mark_placement(const XcdSync& s) {
-    if (threadIdx.x == 0)
+// Last thing a block does in a launch that was asked to (parameter mark_placement: one launch per token is enough to
+// watch how the device deals workgroups, and the memory-side operation at the very end of EVERY launch cost 0.1-0.3 us
+// each): flip its bit of its XCD's placement word (see XcdControl).
+__device__ __forceinline__ void xcd_mark_placement(const XcdSync& s, uint32_t wanted) {
+    if (wanted && threadIdx.x == 0)
         (void)__hip_atomic_fetch_xor(&s.ctl->placement[s.xcd].bits, 1ull << s.slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -152,9 +147,11 @@ __device__ __forceinline__ float xcd_sum_to_f32(uint32_t lo, uint32_t hi) {
     return fmaf((float)lo, kXcdSumInv, (float)(int32_t)hi);
 }
 __device__ __forceinline__ void xcd_sum_add(long long* row, uint32_t e, float v, XcdControl* ctl) {
-    if (!(fabsf(v) < kXcdSumLimit)) {  // beyond the fixed-point range, or not finite: clamp and tell the host
-        __hip_atomic_store(&ctl->overflow, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        v = v != v ? 0.f : (v < 0.f ? -kXcdSumLimit : kXcdSumLimit);
+    // beyond the fixed-point range, or not finite: clamp and tell the host (branch-free but for the rare store)
+    const bool bad = !(fabsf(v) < kXcdSumLimit);
+    v = v != v ? 0.f : fminf(fmaxf(v, -kXcdSumLimit), kXcdSumLimit);
+    if (__any((int)bad)) {
+        if (bad) __hip_atomic_store(&ctl->overflow, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     const long long q = __float2ll_rn(v * kXcdSumScale);
     (void)__hip_atomic_fetch_add(reinterpret_cast<unsigned long long*>(row) + xcd_sum_index(e), (unsigned long long)q,
@@ -662,7 +659,9 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
                         [&](uint32_t r, float s0, float s1) { mid[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
     }
     FK_XCD_STAMP(1, 7);
-    if (!xcd_barrier<0>(sync, reinterpret_cast<uint32_t*>(red) + 8)) return;
+    uint32_t* okw = reinterpret_cast<uint32_t*>(red) + 8;
+    xcd_barrier<0>(sync, okw);
+    const bool ok = xcd_wait_ok(okw);  // tested in front of the additions into the sum row
     FK_XCD_STAMP(1, 8);
 
     // ---- down_proj over this XCD's K-slice: fp32 partial row ----
@@ -672,7 +671,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if (streams && d_n) tile_run<KIND, NLB, kBlock, ONE>(a.down, td, pd, rd, xs, sx, meta + 2 * kMetaWords, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(1, 10);
-    if (streams && d_n) {
+    if (streams && d_n && ok) {
         long long* out = a.out_sums;
         XcdControl* ctl = sync.ctl;
         tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, d0 + r, s0, ctl); });
@@ -706,7 +705,7 @@ __global__ __launch_bounds__(kMlpBlock, 2) void xcd_mlp_kernel(const long long* 
     kernarg_warm<32 + (int)sizeof(XcdMlpArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
     xcd_mlp_phase<KIND, NLA, NLB, false, true, ONE>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
-    xcd_mark_placement(sync);
+    xcd_mark_placement(sync, a.mark_placement);
 }
 
 // =============================================================================================== attention launch
@@ -785,7 +784,8 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     }
     FK_XCD_STAMP(0, 6);
     uint32_t* okw = reinterpret_cast<uint32_t*>(red) + 8;
-    if (!xcd_barrier<0>(sync, okw)) return;
+    xcd_barrier<0>(sync, okw);
+    if (!xcd_wait_ok(okw)) return;  // the attention phase appends to the cache
     FK_XCD_STAMP(0, 7);
 
     // ---- head norm + RoPE + cache append + attention: block = (query head of the group, key range) ----
@@ -796,7 +796,8 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
             sdpa_block<1, 2, std::remove_cv_t<std::remove_reference_t<decltype((a.sdpa))>>, 0, true, true>(a.sdpa, kv_len0, split, sync.xcd, gz, G, work);
     }
     FK_XCD_STAMP(0, 8);
-    if (!xcd_barrier<0>(sync, okw)) return;
+    xcd_barrier<0>(sync, okw);
+    const bool ok2 = xcd_wait_ok(okw);  // tested in front of the additions into the sum row
     FK_XCD_STAMP(0, 9);
 
     // ---- merge the ranges of each of the group's heads (range order), rows to LDS ----
@@ -868,7 +869,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     if (streams && o_n) tile_run<KIND, NLB, kAttnStream, ONE>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(0, 11);
-    if (o_n) {
+    if (o_n && ok2) {
         long long* out = a.out_sums;
         XcdControl* ctl = sync.ctl;
         tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, o0 + r, s0, ctl); });
@@ -886,7 +887,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_attn_kernel(const long long* su
     kernarg_warm<32 + (int)sizeof(XcdAttnArgs)>();
     XcdSync sync = xcd_sync_init(a.ctl, a.spin_limit);
     xcd_attn_phase<KIND, NLA, NLB, false, true, ONE>(a, lead, inr, sync, lds_raw, nullptr, nullptr);
-    xcd_mark_placement(sync);
+    xcd_mark_placement(sync, a.mark_placement);
 }
 
 // ---- the whole token in one launch --------------------------------------------------------------------------
@@ -987,7 +988,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_token_kernel(const XcdTokenArgs
         }
         if (l + 1 < t.n_layers && !xcd_global_barrier(sync, gs)) return;
     }
-    xcd_mark_placement(sync);
+    xcd_mark_placement(sync, t.mark_placement);
 }
 
 __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
@@ -1305,6 +1306,7 @@ fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out) {
     a.out_sums = rq.out_sums;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
+    a.mark_placement = rq.mark_placement ? 1u : 0u;
     const LdsPlan lp = g.lp;
     const uint32_t lds = g.lds;
     out->func = g.func;
@@ -1388,6 +1390,7 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     a.out_sums = rq.out_sums;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
+    a.mark_placement = rq.mark_placement ? 1u : 0u;
     const LdsPlan lp = g.lp;
     const uint32_t lds = g.lds;
     out->func = g.func;
@@ -1426,6 +1429,7 @@ fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uin
     t.n_layers = n_layers;
     t.ctl = h_attn[0].ctl;
     t.spin_limit = h_attn[0].spin_limit;
+    t.mark_placement = h_attn[0].mark_placement;
     const uint32_t phase_lds = ((attn_lds > mlp_lds ? attn_lds : mlp_lds) + 15u) & ~15u;
     t.xres_off = phase_lds / 16u;
     const uint32_t lds = phase_lds + h_attn[0].in.hidden * 2u;

@@ -128,6 +128,7 @@ struct XcdMlpArgs {
     XcdControl* ctl;
     uint32_t spin_limit;
     uint32_t cs_max, work_floats;  // LDS layout: chunks of the longest staged vector, floats of the work area
+    uint32_t mark_placement;       // every block flips its bit of its XCD's placement word when it ends
 };
 
 struct XcdAttnArgs {
@@ -146,6 +147,7 @@ struct XcdAttnArgs {
     XcdControl* ctl;
     uint32_t spin_limit;
     uint32_t cs_max, work_floats, att_elems;  // LDS layout (att_elems: bf16 elements of the merged attention rows)
+    uint32_t mark_placement;
 };
 
 // Every layer of a token in ONE launch: the attention and MLP phases of the two kernels above, layer after layer,
@@ -158,6 +160,7 @@ struct XcdTokenArgs {
     XcdControl* ctl;
     uint32_t spin_limit;
     uint32_t xres_off;         // LDS offset (16-byte units) of the block's copy of the residual row
+    uint32_t mark_placement;
 };
 
 // x = T(f32(sums) + residual): the last layer's output for the LM head.  `clear` (may be the row read, or null)
@@ -209,6 +212,7 @@ struct XcdAttnRequest {
     long long* out_sums;
     void* workspace;
     uint32_t spin_limit;
+    bool mark_placement;
 };
 fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out);
 
@@ -226,6 +230,7 @@ struct XcdMlpRequest {
     long long* out_sums;
     void* workspace;
     uint32_t spin_limit;
+    bool mark_placement;
     bool for_token;   // the block is meant for the whole-token launch (its gate / up passes are shallower)
 };
 fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out);

@@ -403,7 +403,9 @@ class DecoderRuntime:
             q_, k_, v_ = self.xcd_qkv[l] if c.xcd_token_launch else (self.q, self.k, self.v)
             a += [arg(q_), arg(k_), arg(v_), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
                   arg(self.rope_tab), arg(self.xcd_att_partials), S(2 * l + 1), S(2 * l + 2), arg(self.xcd_ctl)]
-            t.append(Dispatch(name("xcd_attn_block"), a, dict(shape, has_sums=int(l > 0), has_norm=int(c.qk_norm))))
+            # the first launch of a token also flips the placement words (the watch on how workgroups are dealt)
+            t.append(Dispatch(name("xcd_attn_block"), a, dict(shape, has_sums=int(l > 0), has_norm=int(c.qk_norm),
+                                                              mark_placement=int(l == 0))))
             Wg, Wu, Wd = (w.mats[p + f"mlp.{n}_proj"] for n in ("gate", "up", "down"))
             m = [S(2 * l + 1), arg(self.xcd_xa), arg(self.xcd_xb), arg(w.vecs[p + "post_attention_layernorm"]),
                  arg(Wg.w), arg(Wu.w)]
