@@ -20,6 +20,10 @@ Prints ONE JSON line: value = generated tokens/s (wall clock around the K timed 
                   launch shape of the token the same way,
   qgemv_cfg1   -- configs[0]/[1]'s int4 qGEMV (4864 x 896, g64) over a rotating pool of 512 weight
                   sets (1.26 GB), GB/s and fraction of the 8 TB/s peak,
+  qgemv_steady -- the same kernel family on a vocabulary-sized int4 matrix (151936 x 2560, 219 MB per
+                  launch, three sets in rotation): the steady streaming rate of the int4 qGEMV,
+  hbm_read_ceiling -- a plain read-and-XOR kernel over 1 GiB buffers: what a read-only kernel gets from
+                  HBM on this device, the bound the GEMV figures are also stated against,
   cpu_baseline -- the CPU oracle (C restatement of the reference semantics) decoding the same
                   model at the same context on the host cores, bounded to --cpu-tokens steps.
 """
@@ -286,6 +290,49 @@ def main() -> int:
                 "note": "serial: dependent graph nodes, launch to launch; overlapped: independent nodes of one graph",
             }
             del Ws, ys, tasks
+
+            # ---- the same kernel family at steady state: a vocabulary-sized int4 matrix (151936 x 2560, 219 MB per
+            # launch), three weight sets in rotation (657 MB: past the 256 MB last-level cache), dependent graph
+            # nodes, launch to launch; median and best of nine graph executions ----
+            n, k, pool, rounds = 151936, 2560, 3, 8
+            nbytes = int(n * k * 0.5625) + k * 2 + n * 2
+            Ws = [_rand_weight(n, k, 4, 900 + 3 * i) for i in range(pool)]
+            x, ys = _bf16(k, 8), [fk.DeviceBuffer(n * 2) for _ in range(pool)]
+            tasks = [Dispatch("fusekit_qgemv_f0", [arg(x)] + _wargs(Wi) + [arg(y)], {"bits": 4, "group": 64, "m": k, "n": n})
+                     for Wi, y in zip(Ws, ys)] * rounds
+            g = rt.d.build_graph(tasks, barriers=[True] * len(tasks))
+            rt.d.execute_graph(g)
+            runs = sorted(rt.d.execute_graph(g) / len(tasks) * 1e6 for _ in range(9))
+            med, best = runs[len(runs) // 2], runs[0]
+            out["qgemv_steady"] = {
+                "shape": "151936 x 2560 int4 g64, bf16 x and y", "pool": pool, "bytes_per_launch": nbytes,
+                "median_us": round(med, 2), "median_GBps": round(nbytes / med / 1e3, 1),
+                "median_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBPS, 4),
+                "best_us": round(best, 2), "best_frac": round(nbytes / best / 1e3 / HBM_PEAK_GBPS, 4),
+                "note": "gemv_rows_kernel<Q4>; dependent graph nodes, launch to launch, %d launches per graph execution" % len(tasks),
+            }
+            del Ws, ys, tasks
+
+        # ---- what a plain read-only kernel gets from HBM on this device: 16 bytes per lane, 1 KiB contiguous per wave
+        # instruction, eight requests in flight per lane, XOR only; two 1 GiB buffers in rotation ----
+        gib = 1 << 30
+        bufs = [fk.DeviceBuffer(gib) for _ in range(2)]
+        for i, b in enumerate(bufs):
+            fk.fill_u32(b, 0x3f803f80 + i, gib // 4)
+        sink = fk.DeviceBuffer(fk.read_reduce_out_bytes())
+        tasks = [Dispatch("fusekit_read_reduce_f0", [arg(b), arg(sink)], {}) for b in bufs] * 4
+        g = rt.d.build_graph(tasks, barriers=[True] * len(tasks))
+        rt.d.execute_graph(g)
+        runs = sorted(rt.d.execute_graph(g) / len(tasks) * 1e6 for _ in range(5))
+        med = runs[len(runs) // 2]
+        out["hbm_read_ceiling"] = {
+            "kernel": "read_reduce_kernel (plain 16-byte loads, XOR)", "bytes_per_launch": gib,
+            "median_us": round(med, 2), "GBps": round(gib / med / 1e3, 1), "frac_of_published_peak": round(gib / med / 1e3 / HBM_PEAK_GBPS, 4),
+            "best_us": round(runs[0], 2),
+        }
+        if "qgemv_steady" in out:
+            out["qgemv_steady"]["median_frac_of_read_ceiling"] = round(out["qgemv_steady"]["median_GBps"] / out["hbm_read_ceiling"]["GBps"], 4)
+        del bufs
 
     if args.per_kernel and args.mode == "persistent":
         per_kernel = {}

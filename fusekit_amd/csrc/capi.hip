@@ -722,6 +722,14 @@ fk_status fk_copy(void* dst, const void* src, size_t nbytes, fk_stream s) {
     return run_launch(l, (hipStream_t)s);
 }
 
+size_t fk_read_reduce_out_bytes(void) { return (size_t)256 * 8 * 8; }
+
+fk_status fk_read_reduce(const void* src, size_t nbytes, void* out, size_t out_bytes, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_read_reduce(src, nbytes, out, out_bytes, 0, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_fill_u32(void* dptr, uint32_t value, size_t count, fk_stream s) {
     Launch l;
     FK_TRY(plan_fill_u32(dptr, value, count, &l));

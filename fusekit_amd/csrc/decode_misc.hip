@@ -441,4 +441,64 @@ fk_status plan_copy(void* dst, const void* src, size_t nbytes, Launch* out) {
     return FK_OK;
 }
 
+// ---------------------------------------------------------------- plain read (measurement aid)
+// Streams `count` 16-byte pieces through the chip and keeps only their XOR: the upper bound of what ANY read-only
+// kernel of this access pattern (1 KiB contiguous per wave instruction, several requests in flight per lane) gets
+// from HBM on the device at hand.  The streaming GEMVs are priced against the published peak AND against this.
+struct ReadArgs {
+    const uint4* src;
+    size_t count;
+    unsigned long long* out;  // [grid] one word per block
+    size_t span;              // pieces per block (a multiple of 8 * 256), blocks walk contiguous spans
+};
+__global__ __launch_bounds__(256) void read_reduce_kernel(const ReadArgs a) {
+    uint4 acc = make_uint4(0, 0, 0, 0);
+    auto fold = [&](const uint4& v) {
+        acc.x ^= v.x;
+        acc.y ^= v.y;
+        acc.z ^= v.z;
+        acc.w ^= v.w;
+    };
+    // a block reads its own contiguous span, 32 KiB (8 requests per lane) per round
+    const size_t begin = (size_t)blockIdx.x * a.span;
+    const size_t end = begin + a.span < a.count ? begin + a.span : a.count;
+    size_t i = begin + threadIdx.x;
+    for (; i + 7 * 256 < end; i += 8 * 256) {
+        uint4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = a.src[i + j * 256];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) fold(v[j]);
+    }
+    for (; i < end; i += 256) fold(a.src[i]);
+    unsigned long long w = ((unsigned long long)(acc.x ^ acc.z) << 32) | (acc.y ^ acc.w);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) w ^= __shfl_xor(w, off);
+    __shared__ unsigned long long part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = w;
+    __syncthreads();
+    if (threadIdx.x == 0) a.out[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
+}
+
+fk_status plan_read_reduce(const void* src, size_t nbytes, void* out, size_t out_bytes, uint32_t blocks_per_cu, Launch* l) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!src || !out || nbytes == 0) return set_error(FK_ERR_INVALID, "read: null pointer or zero size");
+    if (nbytes % 16 || reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(out) % 8)
+        return set_error(FK_ERR_INVALID, "read: source and size must be multiples of 16 bytes, the output 8-byte aligned");
+    if (blocks_per_cu == 0) blocks_per_cu = 4;  // 2, 4 and 8 read 1 GiB at 5.99, 6.04 and 6.04 TB/s; 1: 5.55
+    if (blocks_per_cu > 8) return set_error(FK_ERR_INVALID, "read: at most 8 workgroups per CU");
+    ReadArgs a{reinterpret_cast<const uint4*>(src), nbytes / 16, reinterpret_cast<unsigned long long*>(out), 0};
+    size_t blocks = (a.count + 8 * 256 - 1) / (8 * 256);
+    if (blocks > (size_t)dev->cus * blocks_per_cu) blocks = (size_t)dev->cus * blocks_per_cu;
+    a.span = ((a.count + blocks - 1) / blocks + 8 * 256 - 1) / (8 * 256) * (8 * 256);
+    if (out_bytes < blocks * 8) return set_error(FK_ERR_INVALID, "read: the output needs 8 bytes per workgroup (fk_read_reduce_out_bytes)");
+    l->func = reinterpret_cast<const void*>(&read_reduce_kernel);
+    l->grid = dim3((uint32_t)blocks, 1, 1);
+    l->block = dim3(256, 1, 1);
+    l->shmem = 0;
+    l->set_args(a);
+    return FK_OK;
+}
+
 }  // namespace fk

@@ -801,6 +801,14 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     return plan_xcd_mlp(rq, l);
 }
 
+// src, out (8 bytes per workgroup): the plain read kernel (parameter blocks_per_cu)
+fk_status plan_read_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 2));
+    rw->reads = {0};
+    rw->writes = {1};
+    return plan_read_reduce(d.args[0].ptr, d.args[0].nbytes, d.args[1].ptr, d.args[1].nbytes, d.u("blocks_per_cu", 0), l);
+}
+
 // sum row, residual [hidden] bf16, x [hidden] bf16, sum row to clear (may be the one read) (parameter hidden)
 fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_args(d, 4));
@@ -1213,6 +1221,7 @@ const Family kFamilies[] = {
     {"fusekit_xcd_attn_block", plan_xcd_attn_d},
     {"fusekit_xcd_mlp_block", plan_xcd_mlp_d},
     {"fusekit_xcd_reduce", plan_xcd_reduce_d},
+    {"fusekit_read_reduce", plan_read_reduce_d},
 };
 
 const Family* find_family(const std::string& kernel) {

@@ -299,6 +299,7 @@ fk_status plan_step_init(uint32_t* step_counter, uint32_t* offset, uint32_t* kv_
                          float* rope_tab = nullptr, uint32_t rope_dims = 0, float base_log2 = 0.f);
 fk_status plan_fill_u32(void* p, uint32_t value, size_t count, Launch* out);
 fk_status plan_copy(void* dst, const void* src, size_t nbytes, Launch* out);
+fk_status plan_read_reduce(const void* src, size_t nbytes, void* out, size_t out_bytes, uint32_t blocks_per_cu, Launch* l);
 fk_status plan_quantize(const float* w, size_t n, size_t k, uint32_t bits, uint32_t group, uint32_t* packed,
                         uint16_t* scales, uint16_t* biases, Launch* out);
 fk_status plan_synth(void* out_ptr, size_t count, uint64_t seed, float mean, float std, uint32_t kind, uint32_t bound,

@@ -526,6 +526,27 @@ __device__ __forceinline__ void tile_rows(const Tile& t, const float* part, cons
     auto one = [&](uint32_t rr) {
         const bool ok = rr < t.rows;
         float s0 = 0.f, s1 = 0.f;
+#ifdef FK_AB_ROWS8
+        if (t.cs <= 8u * lr) {
+            // at most eight partials per lane (every 4B-class tile): all reads first, with clamped positions, then
+            // the additions in the loop's order -- one trip to the LDS instead of one per partial
+            const uint32_t base = (ok ? rr : 0u) * t.cs;
+            float v0[8], v1[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t i = lane + k * lr;
+                const uint32_t at = base + (i < t.cs ? i : 0u);
+                v0[k] = part[at];
+                if constexpr (TWO) v1[k] = part1[at];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const bool in = ok && lane + k * lr < t.cs;
+                s0 += in ? v0[k] : 0.f;
+                if constexpr (TWO) s1 += in ? v1[k] : 0.f;
+            }
+        } else
+#endif
         if (ok)
             for (uint32_t i = lane; i < t.cs; i += lr) {
                 s0 += part[rr * t.cs + i];
@@ -840,7 +861,9 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
                         o1_ = fmaf(po[i].y, w, o1_);
                     }
                 };
-                if (n_active <= kXcdMaxRanges / 2)
+                if (n_active <= kXcdMaxRanges / 4)
+                    merge(std::integral_constant<uint32_t, kXcdMaxRanges / 4>{});
+                else if (n_active <= kXcdMaxRanges / 2)
                     merge(std::integral_constant<uint32_t, kXcdMaxRanges / 2>{});
                 else
                     merge(std::integral_constant<uint32_t, kXcdMaxRanges>{});
@@ -1180,6 +1203,9 @@ AttnGeometry attn_geometry(const XcdLayerShape& s) {
     g.chunk_len = sdpa_chunk_len(s.head_dim, s.head_dim, false);
     uint32_t splits = kXcdSlots / G;
     if (splits > kXcdMaxRanges) splits = kXcdMaxRanges;
+#ifdef FK_AB_SPLITS
+    if (splits > FK_AB_SPLITS) splits = FK_AB_SPLITS;
+#endif
     const uint32_t n_chunks = ceil_div(s.capacity, g.chunk_len);
     g.chunks_per_block = ceil_div(n_chunks, splits);
     g.n_splits = ceil_div(n_chunks, g.chunks_per_block);

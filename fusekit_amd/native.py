@@ -549,6 +549,18 @@ def copy(dst, src, nbytes, stream=None):
     check(lib.fk_copy(_ptr(dst), _ptr(src), C.c_size_t(nbytes), _ptr(stream)))
 
 
+lib.fk_read_reduce_out_bytes.restype = C.c_size_t
+
+
+def read_reduce_out_bytes() -> int:
+    return int(lib.fk_read_reduce_out_bytes())
+
+
+def read_reduce(src, nbytes, out, stream=None):
+    """XOR of nbytes read with plain 16-byte loads, one word per workgroup into `out` (fk_read_reduce)."""
+    check(lib.fk_read_reduce(_ptr(src), C.c_size_t(nbytes), _ptr(out), C.c_size_t(out.nbytes), _ptr(stream)))
+
+
 def fill_u32(buf, value, count, stream=None):
     check(lib.fk_fill_u32(_ptr(buf), C.c_uint32(value), C.c_size_t(count), _ptr(stream)))
 

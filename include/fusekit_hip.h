@@ -86,6 +86,14 @@ fk_status fk_fill_u32(void *dptr, uint32_t value, size_t count, fk_stream s);
  * moves buffers inside a stream / graph and is the known-traffic kernel against
  * which hardware byte counters are calibrated. */
 fk_status fk_copy(void *dst, const void *src, size_t nbytes, fk_stream s);
+/* Measurement aid with no counterpart in the reference: reads nbytes (a multiple of 16, 16-byte aligned) with
+ * plain 16-byte-per-lane loads (every workgroup walks its own contiguous span, 1 KiB per wave instruction, eight requests in flight per lane) and
+ * keeps only the XOR of what it read, one 64-bit word per workgroup in `out` (fk_read_reduce_out_bytes() bytes).
+ * Over a buffer larger than the 256 MB last-level cache its rate is what a read-only streaming kernel gets from
+ * HBM on the device at hand: the bench prices the GEMVs against the published 8 TB/s and against this.  Also the
+ * dispatch family `fusekit_read_reduce` (slots: src, out; parameter blocks_per_cu, default 4). */
+fk_status fk_read_reduce(const void *src, size_t nbytes, void *out, size_t out_bytes, fk_stream s);
+size_t fk_read_reduce_out_bytes(void);
 fk_status fk_stream_create(fk_stream *out);
 fk_status fk_stream_destroy(fk_stream s);
 fk_status fk_stream_sync(fk_stream s);

@@ -26,7 +26,9 @@ The committed fixture came from
         --first-seed 3007 --seeds 1 --safety 2 --min-distinct 3
 
 after a sweep over --grid 0:0.002 0:0.004 0:0.006 0:0.02 and seeds 3000..3007 (about a minute per candidate on
-8 cores; most candidates hold at least one near-tie among their 32 steps and are skipped).
+8 cores; most candidates hold at least one near-tie among their 32 steps and are skipped).  The 8-bit and bf16
+fixtures (clear_margin_4b_q8.json, clear_margin_4b_bf16.json: configs[3] names both variants) come from the same
+command with --bits 8 / --bits 16 --min-distinct 4 over seeds 3000..; the seed each one took is in its file.
 """
 import argparse
 import json
@@ -73,11 +75,14 @@ def main():
     ap.add_argument("--safety", type=float, default=3.0)
     ap.add_argument("--min-distinct", type=int, default=3)
     ap.add_argument("--layers", type=int, default=0, help="experiments only: fewer layers")
-    ap.add_argument("--out", default=os.path.join(HERE, "clear_margin_4b.json"))
+    ap.add_argument("--bits", type=int, default=4, choices=[4, 8, 16], help="weights: 4- / 8-bit g64 MLX-affine, or bf16")
+    ap.add_argument("--out", default="", help="default: clear_margin_4b.json (4-bit), clear_margin_4b_q8.json, clear_margin_4b_bf16.json")
     ap.add_argument("--log", default="")
     args = ap.parse_args()
 
-    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=128)
+    if not args.out:
+        args.out = os.path.join(HERE, {4: "clear_margin_4b.json", 8: "clear_margin_4b_q8.json", 16: "clear_margin_4b_bf16.json"}[args.bits])
+    cfg = DecoderConfig(**DENSE_4B, bits=args.bits, capacity=128)
     if args.layers:
         cfg.n_layers = args.layers
     t0 = time.time()
@@ -137,7 +142,7 @@ def main():
                     log.write(json.dumps(rec) + "\n"); log.flush()
                 if same and ratio.min() >= args.safety and not args.layers:
                     rec.update(model_seed=args.model_seed, std=0.02, prompt=prompt, n_layers=cfg.n_layers,
-                               safety=args.safety,
+                               safety=args.safety, bits=args.bits,
                                note="written by tests/golden/find_clear_margin_model.py (oracle only)")
                     with open(args.out, "w") as f:
                         json.dump(rec, f, indent=1)

@@ -248,30 +248,57 @@ class HostMoeWeights:
                 matrix(p + "mlp.shared_experts.down_proj", c.hidden, c.shared_inter)
 
 
-def moe_stable_channel(cfg, mats, vecs, channel: int, level: float, route_logits, route_noise: float):
-    """Gives a mixture-of-experts model what a trained one has and a random one lacks: a persistent large
-    activation in one hidden channel, and routers that read it.  On the bf16 arrays of `mats` / `vecs` (oracle
-    weights), in place:
-      * the tied embedding's column `channel` becomes `level` for every token (it dominates every RMS norm input of
-        the stack), and the final norm's weight of that channel becomes 0, so that the head never sees it (the same
-        huge amount in every logit would cost the logits their resolution);
-      * each router keeps its random rows scaled by `route_noise` and gets column `channel` = route_logits[j] / u,
-        u = sqrt(hidden) (the channel's normalised value when it dominates): expert j's logit is about
-        route_logits[j] whatever the token, plus noise.
-    Returns the names of the arrays it changed (the caller uploads those to the device model)."""
+def moe_class_channels(cfg, mats, vecs, n_classes: int, first_channel: int, level: float, ladder, route_noise: float,
+                       perm_seed: int, loud_rows: int, loud_gain: float, loud_ratio: float):
+    """Gives a mixture-of-experts model what a trained one has and a random one lacks -- persistent large
+    activations and routers that read them -- in a form whose routes VARY: by token, by layer, and so by step.
+    On the bf16 arrays of `mats` / `vecs` (oracle weights), in place:
+      * token t belongs to class t % n_classes; the tied embedding's column first_channel + k holds `level` for the
+        tokens of class k and 0 for the others (the class channel dominates every RMS norm input of the stack: its
+        normalised value is about sqrt(hidden)); the final norm's weight of those channels becomes 0, so that the
+        head never sees them;
+      * each router keeps its random rows scaled by `route_noise`; in layer l the experts are cut into n_classes
+        blocks of n_experts / n_classes by a permutation drawn from (perm_seed, l), and column first_channel + k
+        holds ladder[i] / sqrt(hidden) for the i-th expert of block k (i < top_k) and 0 elsewhere: a token of class
+        k routes to block k's first top_k experts in layer l, whatever else the stack has computed, with the
+        ladder's gaps between the probabilities;
+      * rows j < loud_rows of the embedding are scaled by loud_gain * loud_ratio^-j (a few dominant rows, as trained
+        embeddings have; the class columns are written afterwards).
+    Classes of the top_k experts never overlap inside a layer, so a group of tokens of c different classes touches
+    c * top_k distinct experts there.  Returns (names of the arrays changed, expected routes [n_layers][n_classes]
+    as sorted expert lists; entries of dense layers are None)."""
+    assert cfg.n_experts % n_classes == 0 and cfg.n_experts // n_classes >= cfg.top_k and len(ladder) == cfg.top_k
     changed = ["embed_tokens", "final_norm"]
     E = np.asarray(mats["embed_tokens"].w).reshape(cfg.vocab, cfg.hidden)
-    E[:, channel] = oracle.f32_to_bf16(np.array([level], np.float32))[0]
-    vecs["final_norm"][channel] = 0
+    for j in range(loud_rows):
+        g = np.float32(loud_gain * loud_ratio ** -j)
+        E[j] = oracle.f32_to_bf16((oracle.bf16_to_f32(E[j]) * g).astype(np.float32))
+    lvl = oracle.f32_to_bf16(np.array([level], np.float32))[0]
+    cls = np.arange(cfg.vocab) % n_classes
+    for k in range(n_classes):
+        E[:, first_channel + k] = np.where(cls == k, lvl, np.uint16(0))
+        vecs["final_norm"][first_channel + k] = 0
     u = float(np.sqrt(cfg.hidden))
-    col = oracle.f32_to_bf16((np.asarray(route_logits, np.float32) / u).astype(np.float32))
-    for l in range(cfg.first_dense, cfg.n_layers):
+    per = cfg.n_experts // n_classes
+    expected = []
+    for l in range(cfg.n_layers):
+        if l < cfg.first_dense:
+            expected.append(None)
+            continue
         name = f"layers.{l}.mlp.gate"
         R = np.asarray(mats[name].w).reshape(cfg.n_experts, cfg.hidden)
         R[:] = oracle.f32_to_bf16((oracle.bf16_to_f32(R) * np.float32(route_noise)).astype(np.float32))
-        R[:, channel] = col
+        perm = rng(perm_seed * 1000 + l).permutation(cfg.n_experts)
+        rows = []
+        for k in range(n_classes):
+            col = np.zeros(cfg.n_experts, np.float32)
+            chosen = perm[k * per: k * per + cfg.top_k]
+            col[chosen] = np.asarray(ladder, np.float32) / np.float32(u)
+            R[:, first_channel + k] = oracle.f32_to_bf16(col)
+            rows.append(sorted(int(e) for e in chosen))
+        expected.append(rows)
         changed.append(name)
-    return changed
+    return changed, expected
 
 
 class OracleMoeDecoder:

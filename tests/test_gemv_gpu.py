@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import bf16_mismatch, make_qweight, normal_bf16, rel_l2, to_device
+from helpers import bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
 
 pytestmark = pytest.mark.gpu
 
@@ -340,3 +340,20 @@ def test_rejects_bad_shapes(fk):
     dW.k, dW.bits = 64, 3
     with pytest.raises(fk.FusekitError):
         fk.qgemv(dW, fk.DeviceBuffer(256), None, fk.DeviceBuffer(16))
+
+
+def test_plain_read_kernel_returns_the_xor_of_what_it_read(fk):
+    """fk_read_reduce (the measurement aid behind bench.py's hbm_read_ceiling): every 16-byte piece is read exactly
+    once -- the XOR over the per-workgroup words equals numpy's over the buffer, for sizes around the unrolled
+    loop's edges."""
+    for nbytes in (16, 4096 * 16, (256 * 8 * 256 * 8 + 3) * 16, 3 * 1000 * 1000 * 16):
+        a = rng(nbytes % 1000).integers(0, 2 ** 32, nbytes // 4, dtype=np.uint32)
+        src = fk.DeviceBuffer.from_numpy(a)
+        out = fk.zeros(fk.read_reduce_out_bytes())
+        fk.read_reduce(src, nbytes, out)
+        fk.sync()
+        q = a.reshape(-1, 4)
+        x, y, z, w = (int(np.bitwise_xor.reduce(q[:, i])) for i in range(4))
+        want = ((x ^ z) << 32) | (y ^ w)
+        got = int(np.bitwise_xor.reduce(out.to_numpy(np.uint64)))
+        assert got == want, nbytes

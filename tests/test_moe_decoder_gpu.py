@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import HostMoeWeights, OracleMoeDecoder, moe_stable_channel, rng
+from helpers import HostMoeWeights, OracleMoeDecoder, moe_class_channels, rng
 
 pytestmark = pytest.mark.gpu
 
@@ -111,22 +111,34 @@ def test_full_size_model_32_greedy_tokens(fk):
 
 def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk):
     """Plain free-running equality at full size for the mixture-of-experts model: 32-token prompt, 32 greedy
-    tokens, every expert route chosen by the GPU itself -- `got == expected`, no forced routes, no candidate sets.
+    tokens, every expert route chosen by the GPU itself -- `got == expected` for the tokens AND for the route sets
+    of all 63 steps x 26 expert layers, no forced routes, no candidate sets.
 
     With random weights the sixth and seventh router probabilities are within the stack's rounding drift in a few
     layers of every step (test_full_size_model_32_greedy_tokens follows the GPU's routes for that reason).  The
-    fixture's model has what a trained model has: a persistent large activation in one hidden channel (the tied
-    embedding's column at a constant level, hidden from the head by a zero in the final norm weight), routers that
-    read it (their random part scaled down) and a few dominant embedding rows; tests/golden/find_clear_margin_moe.py
-    found the parameters on the CPU with the oracle alone: every 6th-7th router gap and every logit gap is at
-    least `safety` times what two fp32 summation orders change it by.  The model is built in HBM by the library's
-    bit-reproducible generator from the fixture's seeds; the host builds the same bytes (checked on two quantised
-    tensors), applies the structure and uploads the few arrays it changes."""
+    fixture's model has what a trained model has -- persistent large activations and routers that read them -- in
+    a form whose routes vary (helpers.moe_class_channels): a token's class lights one of eight hidden channels,
+    every layer's router sends each class to its own six experts through a per-layer permutation, a few embedding
+    rows dominate the head.  tests/golden/find_clear_margin_moe.py found the parameters on the CPU with the oracle
+    alone: every 6th-7th router gap and every logit gap is at least `safety` times what two fp32 summation orders
+    change it by.  A build that skipped experts, ignored the context or mis-ranked a router would fail here: the
+    route sets differ between layers and between steps (8 different ones per layer over the run), the expected
+    tokens take several values.  The model is built in HBM by the library's bit-reproducible generator from the
+    fixture's seeds; the host builds the same bytes (checked on two quantised tensors), applies the structure and
+    uploads the arrays it changes."""
     from fusekit_amd.moe_decoder import MoeConfig, MoeRuntime, MoeWeights
     fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "clear_margin_moe.json")))
     cfg = MoeConfig(capacity=128)
-    assert fx["n_layers"] == cfg.n_layers and len(fx["prompt"]) == 32 and len(fx["tokens"]) == 32
-    kw = dict(seed=fx["model_seed"], std=fx["std"], embed_loud_rows=fx["loud_rows"], embed_loud_gain=fx["loud_gain"])
+    n_moe = cfg.n_layers - cfg.first_dense
+    prompt, want = fx["prompt"], fx["tokens"]
+    assert fx["n_layers"] == cfg.n_layers and len(prompt) == 32 and len(want) == 32
+    # the fixture can fail a wrong build: several tokens, routes that move between layers and steps
+    assert len(set(want)) >= 4
+    assert len(fx["routes"]) == 63 and all(len(st) == n_moe for st in fx["routes"])
+    for l in range(n_moe):
+        assert len({tuple(st[l]) for st in fx["routes"]}) >= 4, l
+    assert all(len({tuple(r) for r in st}) >= n_moe // 2 for st in fx["routes"])   # a step's layers differ
+    kw = dict(seed=fx["model_seed"], std=fx["std"])
     W = MoeWeights.random_init(cfg, exact=True, **kw)
     H = HostMoeWeights(cfg, **kw)
     for name in ("layers.0.self_attn.q_proj", "layers.26.mlp.switch_mlp.down_proj"):
@@ -135,30 +147,59 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
         assert np.array_equal(d.scales.to_numpy(np.uint16), np.asarray(h.scales).reshape(-1)), name
         assert np.array_equal(d.biases.to_numpy(np.uint16), np.asarray(h.biases).reshape(-1)), name
     assert np.array_equal(W.mats["embed_tokens"].w.to_numpy(np.uint16), np.asarray(H.mats["embed_tokens"].w).reshape(-1))
-    for name in moe_stable_channel(cfg, H.mats, H.vecs, fx["channel"], fx["level"], fx["route_logits"], fx["route_noise"]):
+    changed, _ = moe_class_channels(cfg, H.mats, H.vecs, fx["classes"], fx["first_channel"], fx["level"], fx["ladder"],
+                                    fx["route_noise"], fx["perm_seed"], fx["loud_rows"], fx["loud_gain"], fx["loud_ratio"])
+    for name in changed:
         if name in H.vecs:
             W.vecs[name].upload(np.ascontiguousarray(H.vecs[name]))
         else:
             W.mats[name].w.upload(np.ascontiguousarray(np.asarray(H.mats[name].w).reshape(-1)))
     rt = MoeRuntime(cfg, W)
-    got, _, _ = rt.generate(fx["prompt"], 32)
+    # step by step through the decode graph, so that every step's routes can be read: the prompt is fed as it is,
+    # then the GPU's own tokens (free running)
+    got, tok, bad_routes = [], prompt[0], []
+    for i in range(63):
+        nxt, _ = rt.d.decode_host_loop(rt.graph, rt.uniforms, i, [tok])
+        routes = rt.routes()[cfg.first_dense:]
+        for l in range(n_moe):
+            if sorted(routes[l].tolist()) != fx["routes"][i][l]:
+                bad_routes.append((i, l, sorted(routes[l].tolist()), fx["routes"][i][l]))
+        if i >= 31:
+            got.append(nxt[0])
+        tok = prompt[i + 1] if i + 1 < 32 else nxt[0]
     print("tokens:", got)
-    print("fixture: min logit margin %.1f bf16 ulps, logit margin / fp32 envelope %.2f, router gap / fp32 envelope %.2f" %
-          (fx["min_margin_ulps"], fx["min_ratio"], fx["min_router_ratio"]))
-    assert got == fx["tokens"]
-    routes = rt.routes()[cfg.first_dense:]
-    assert [sorted(r.tolist()) for r in routes] == fx["routes_last_step"]
+    print("fixture: %d distinct tokens, route sets per layer %d..%d, min logit margin %.1f bf16 ulps, logit margin / fp32 envelope "
+          "%.2f, router gap / fp32 envelope %.2f" % (fx["distinct"], min(fx["route_sets_per_layer"]), max(fx["route_sets_per_layer"]),
+                                                       fx["min_margin_ulps"], fx["min_ratio"], fx["min_router_ratio"]))
+    assert got == want
+    assert not bad_routes, bad_routes[:4]
+    # the chunked loop (tokens fed back on the GPU) decides the same
+    rt.reset()
+    again, _, _ = rt.generate(prompt, 32)
+    assert again == want
 
     # The same model at full size with EIGHT active token rows in one pass over the weights (shared-stream matmuls
     # for the dense projections and the shared experts, row forms of the store, the attention and the router,
-    # routed experts over 48 routes): the oracle's tokens 23 .. 30 as rows at positions 55 .. 62, behind a cache
-    # filled step by step, must give the oracle's token 31 and, for the last row, the oracle's routes of its last step.
+    # routed experts over 48 routes).  The eight consecutive positions of the run whose tokens span the most classes
+    # are taken as rows behind a cache filled step by step: the pass must give the oracle's next token and, for
+    # every row and every layer, the oracle's routes of that step -- at least 20 distinct experts per layer.
+    seq = prompt + want
+    # (windows that end at position 31 or later: the token after the window is then one of the expected ones)
+    first = max(range(24, 55), key=lambda p: len({t % fx["classes"] for t in seq[p:p + 8]}))
+    n_classes = len({t % fx["classes"] for t in seq[first:first + 8]})
+    assert n_classes >= 4, n_classes
     rt.reset()
-    head, _, _ = rt.generate(fx["prompt"], 24)
-    assert head == fx["tokens"][:24]
-    nxt = rt.forward_rows(fx["tokens"][23:31], 32 + 23)
-    assert nxt == fx["tokens"][31]
-    assert sorted(rt.rows_routes[-1].tolist()) == fx["routes_last_step"][-1]
+    if first:
+        rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, seq[:first])
+    nxt = rt.forward_rows(seq[first:first + 8], first)
+    assert nxt == seq[first + 8]
+    ridx = rt._rows_variants[8].ridx.to_numpy(np.uint32, (cfg.n_layers, 8, cfg.top_k))[cfg.first_dense:]
+    for l in range(n_moe):
+        for r in range(8):
+            assert sorted(ridx[l, r].tolist()) == fx["routes"][first + r][l], (l, r)
+        assert len(set(ridx[l].reshape(-1).tolist())) >= 20
+    print("eight-row pass at positions %d..%d: %d classes, %d distinct experts per layer" % (
+        first, first + 7, n_classes, len(set(ridx[0].reshape(-1).tolist()))))
 
 
 @pytest.mark.parametrize("rows,offset", [(8, 0), (5, 8), (1, 3)])
