@@ -326,6 +326,37 @@ fk_status fk_routed_qmv_reduce(const uint16_t* h, uint32_t n_h_rows, const fk_we
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_route_order(const uint32_t* expert_idx, uint32_t n_routes, uint32_t n_experts, uint32_t* order, fk_stream s) {
+    Launch l;
+    FK_TRY(plan_route_order(expert_idx, n_routes, n_experts, order, &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_routed_qmv_swiglu_ordered(const uint16_t* x, uint32_t n_x_rows, const fk_weight* Wg, const fk_weight* Wu,
+                                       uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
+                                       const uint16_t* route_weight, uint32_t n_routes, const uint32_t* order,
+                                       uint16_t* out0, fk_stream s) {
+    if (!Wg || !Wu) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_ordered: null weight");
+    if (!order) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_ordered: null order");
+    Launch l;
+    FK_TRY(plan_routed_gemv(x, n_x_rows, Wg, Wu, n_experts, row_idx, expert_idx, route_weight, n_routes, out0, &l, nullptr,
+                            nullptr, nullptr, nullptr, order));
+    return run_launch(l, (hipStream_t)s);
+}
+
+fk_status fk_routed_qmv_reduce_ordered(const uint16_t* h, uint32_t n_h_rows, const fk_weight* Wd, uint32_t n_experts,
+                                       const uint32_t* row_idx, const uint32_t* expert_idx, const uint16_t* route_weight,
+                                       const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual_extra,
+                                       uint32_t n_tokens, uint32_t top_k, const uint32_t* order, uint16_t* out, void* workspace,
+                                       fk_stream s) {
+    if (!workspace) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce_ordered: null workspace");
+    if (!order) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce_ordered: null order");
+    Launch l;
+    FK_TRY(plan_routed_reduce_chain(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_weight, shared_x, W_shared,
+                                    residual_extra, n_tokens, top_k, out, static_cast<uint16_t*>(workspace), &l, order));
+    return run_launch(l, (hipStream_t)s);
+}
+
 void fk_set_routed_fused_reduce(int on) { set_routed_fused_reduce(on != 0); }
 
 int fk_gemm_library_available(void) { return gemm_library_available() ? 1 : 0; }

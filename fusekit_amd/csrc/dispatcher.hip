@@ -1013,8 +1013,10 @@ fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
     const uint32_t experts = d.u("experts"), routes = d.u("routes"), x_rows = d.u("x_rows", 1);
     const bool pre_scale = d.u("pre_scale", 0) != 0, has_shared = d.u("has_shared", 0) != 0;
     const size_t n_slots = pre_scale ? 11 : 10;
-    // with has_shared = 1: + shared gate w / s / b, shared up w / s / b, shared_out (parameter shared_o rows)
-    FK_TRY(need_args(d, n_slots + (has_shared ? 7 : 0)));
+    // with has_shared = 1: + shared gate w / s / b, shared up w / s / b, shared_out (parameter shared_o rows);
+    // with has_order = 1 (several tokens, no shared pair): + order (uint32 [routes], from fusekit_route_order)
+    const bool has_order = d.u("has_order", 0) != 0;
+    FK_TRY(need_args(d, n_slots + (has_shared ? 7 : 0) + (has_order ? 1 : 0)));
     if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
     if (experts == 0 || routes == 0 || K == 0 || O == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": k / o / experts / routes parameters missing");
@@ -1040,10 +1042,17 @@ fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
         for (uint32_t i = 0; i < 6; ++i) rw->reads.push_back((uint32_t)n_slots + i);
         rw->writes.push_back((uint32_t)n_slots + 6);
     }
+    const uint32_t* order = nullptr;
+    if (has_order) {
+        const size_t os = n_slots + (has_shared ? 7 : 0);
+        FK_TRY(need_bytes(d, os, (size_t)routes * 4));
+        order = arg_ptr<const uint32_t>(d, os);
+        rw->reads.push_back((uint32_t)os);
+    }
     return plan_routed_gemv(arg_ptr<const uint16_t>(d, 0), x_rows, &Wg, &Wu, experts, arg_ptr<const uint32_t>(d, 7),
                             arg_ptr<const uint32_t>(d, 8), pre_scale ? arg_ptr<const uint16_t>(d, 9) : nullptr, routes,
                             arg_ptr<uint16_t>(d, n_slots - 1), l, has_shared ? &Sg : nullptr, has_shared ? &Su : nullptr,
-                            shared_out);
+                            shared_out, nullptr, order);
 }
 
 // x, wq, scales, biases, row_idx, expert_idx, [route_weight], [shared_x, shared_w, shared_s, shared_b],
@@ -1062,6 +1071,8 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     if (has_shared) s += 4;
     const size_t extra_slot = has_extra ? s++ : 0;
     const size_t out_slot = s++, ws_slot = s++;
+    const bool has_order = d.u("has_order", 0) != 0;   // + order (uint32 [routes], from fusekit_route_order) as the last slot
+    const size_t order_slot = has_order ? s++ : 0;
     FK_TRY(need_args(d, s));
     if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
     if (experts == 0 || routes == 0 || K == 0 || O == 0)
@@ -1083,12 +1094,31 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     for (uint32_t i = 0; i < out_slot; ++i) rw->reads.push_back(i);
     rw->reads.push_back((uint32_t)ws_slot);
     rw->writes = {(uint32_t)out_slot, (uint32_t)ws_slot};
+    const uint32_t* order = nullptr;
+    if (has_order) {
+        FK_TRY(need_bytes(d, order_slot, (size_t)routes * 4));
+        order = arg_ptr<const uint32_t>(d, order_slot);
+        rw->reads.push_back((uint32_t)order_slot);
+    }
 
     return plan_routed_reduce_chain(arg_ptr<const uint16_t>(d, 0), x_rows, &Wd, experts, arg_ptr<const uint32_t>(d, 4),
                                     arg_ptr<const uint32_t>(d, 5), preweighted ? nullptr : arg_ptr<const uint16_t>(d, rw_slot),
                                     has_shared ? arg_ptr<const uint16_t>(d, shared_slot) : nullptr, has_shared ? &Ws : nullptr,
                                     has_extra ? arg_ptr<const uint16_t>(d, extra_slot) : nullptr, tokens, top_k,
-                                    arg_ptr<uint16_t>(d, out_slot), arg_ptr<uint16_t>(d, ws_slot), l);
+                                    arg_ptr<uint16_t>(d, out_slot), arg_ptr<uint16_t>(d, ws_slot), l, order);
+}
+
+// expert_idx (uint32 [routes]), order (uint32 [routes], written): the routes sorted by expert, stable (parameters
+// routes, experts).  No counterpart among the reference's kernels: its routed kernels serve routes as listed.
+fk_status plan_route_order_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    FK_TRY(need_args(d, 2));
+    const uint32_t routes = d.u("routes"), experts = d.u("experts");
+    if (routes == 0 || experts == 0) return set_error(FK_ERR_INVALID, d.kernel + ": routes / experts parameters missing");
+    FK_TRY(need_bytes(d, 0, (size_t)routes * 4));
+    FK_TRY(need_bytes(d, 1, (size_t)routes * 4));
+    rw->reads = {0};
+    rw->writes = {1};
+    return plan_route_order(arg_ptr<const uint32_t>(d, 0), routes, experts, arg_ptr<uint32_t>(d, 1), l);
 }
 
 // x, W, scales, biases, [bias], [residual], y, workspace.  Parameters: m (= K), n, rows, has_bias, has_residual.
@@ -1222,6 +1252,7 @@ const Family kFamilies[] = {
     {"fusekit_xcd_mlp_block", plan_xcd_mlp_d},
     {"fusekit_xcd_reduce", plan_xcd_reduce_d},
     {"fusekit_read_reduce", plan_read_reduce_d},
+    {"fusekit_route_order", plan_route_order_d},
 };
 
 const Family* find_family(const std::string& kernel) {

@@ -133,14 +133,17 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
                            const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out,
                            const fk_weight* sh_a = nullptr, const fk_weight* sh_b = nullptr, uint16_t* sh_y = nullptr,
-                           const RouteInKernel* rk = nullptr);
+                           const RouteInKernel* rk = nullptr, const uint32_t* order = nullptr);
+// order[position] = route: the routes sorted by expert (stable), for the `order` argument of the routed launches.
+fk_status plan_route_order(const uint32_t* expert_idx, uint32_t n_routes, uint32_t n_experts, uint32_t* order, Launch* out);
 // Routed down projection + weighted reduction (+ shared expert + residual): one fused launch for one token
 // of int4 weights, else routed GEMV -> shared GEMV -> ordered reduction chained in out->then (`parts`,
 // (routes + tokens) * O bf16, is only touched by the chain).
 fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const fk_weight* Wd, uint32_t n_experts,
                                    const uint32_t* row_idx, const uint32_t* expert_idx, const uint16_t* route_weight,
                                    const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual,
-                                   uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out);
+                                   uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out,
+                                   const uint32_t* order = nullptr);
 void set_routed_fused_reduce(bool on);
 // partial rows ((routes + tokens) * O bf16, rounded up to 256 bytes); with a shared expert and several tokens
 // the multi-row matmul's workspace follows them

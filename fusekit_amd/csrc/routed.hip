@@ -50,6 +50,12 @@ struct RoutedArgs {
     const uint16_t* route_scale;   // one bf16 value
     uint32_t* idx_out;
     uint16_t* weight_out;
+    // Several tokens: the routes in the order they are SERVED, order[position] = route (plan_route_order sorts them
+    // by expert), or null = as listed.  Routes that chose the same expert then sit next to each other in the grid, and
+    // with a multiple of eight blocks per route the blocks that walk the same tiles of the same slice land on the same
+    // XCD at the same time: the slice comes from HBM once and from that XCD's L2 for the other rows.  Inputs,
+    // outputs and arithmetic of a route are untouched.
+    const uint32_t* order;
 };
 
 // GemvArgs as one route sees it.  n_mats is a compile-time 1 so that every index
@@ -78,7 +84,12 @@ template <WKind KIND, int NSEG>
 __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArgs a) {
     extern __shared__ uint4 lds_raw[];
     kernarg_warm<(int)sizeof(RoutedArgs)>();
-    const uint32_t route = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - route * a.blocks_per_route;
+    const uint32_t pos = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - pos * a.blocks_per_route;
+    uint32_t route = pos;
+    if (a.order && pos < a.n_routes) {
+        route = a.order[pos];
+        route = route < a.n_routes ? route : pos;   // a device array is not trusted with addresses
+    }
     const bool extra = route >= a.n_routes;     // uniform per block
     const uint32_t lookup = extra ? 0u : route;
     uint32_t e = 0, row = 0;
@@ -356,9 +367,11 @@ uint32_t resident_blocks(const void* func, uint32_t lds_bytes, int cus) {
 fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight* w_a, const fk_weight* w_b,
                            uint32_t n_experts, const uint32_t* row_idx, const uint32_t* expert_idx,
                            const uint16_t* route_weight, uint32_t n_routes, uint16_t* y, Launch* out,
-                           const fk_weight* sh_a, const fk_weight* sh_b, uint16_t* sh_y, const RouteInKernel* rk) {
+                           const fk_weight* sh_a, const fk_weight* sh_b, uint16_t* sh_y, const RouteInKernel* rk,
+                           const uint32_t* order) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
+    if (order && (rk || sh_a)) return set_error(FK_ERR_UNSUPPORTED, "routed: a serving order goes with listed routes of several tokens only");
     if (rk) {
         if (!rk->logits || !rk->scale || !rk->idx_out || !rk->weight_out) return set_error(FK_ERR_INVALID, "routed: null routing tensor");
         if (n_x_rows != 1) return set_error(FK_ERR_UNSUPPORTED, "routed: the launch routes for one token only");
@@ -404,6 +417,9 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
         t_gemv_grid_override = 0;
         FK_TRY(s);
         per_route = resident_blocks(func, base.shmem, dev->cus) / all_routes;
+        // served in expert order: a whole number of XCD rounds per route, so that block (position, i) and block
+        // (position + 1, i) share an XCD
+        if (order && per_route >= 8) per_route &= ~7u;
     }
     GemvArgs g;
     memcpy(&g, base.args, sizeof(g));
@@ -426,6 +442,7 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
     a.y_stride = w_a->n;
     a.n_routes = n_routes;
     a.x_routes = x_routes;
+    a.order = order;
     if (rk) {
         a.logits = rk->logits; a.route_scale = rk->scale; a.idx_out = rk->idx_out; a.weight_out = rk->weight_out;
         a.route_weight = rk->apply_weight ? rk->scale : nullptr;
@@ -497,7 +514,8 @@ static bool down_reduce_fits(const fk_weight* Wd, const fk_weight* Ws, uint32_t 
 fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const fk_weight* Wd, uint32_t n_experts,
                                    const uint32_t* row_idx, const uint32_t* expert_idx, const uint16_t* route_weight,
                                    const uint16_t* shared_x, const fk_weight* W_shared, const uint16_t* residual,
-                                   uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out) {
+                                   uint32_t n_tokens, uint32_t top_k, uint16_t* out_ptr, uint16_t* parts, Launch* out,
+                                   const uint32_t* order) {
     if (!Wd || !out_ptr || !h) return set_error(FK_ERR_INVALID, "routed reduce: null weight, input or output");
     if (n_tokens == 0 || top_k == 0) return set_error(FK_ERR_INVALID, "routed reduce: empty route set");
     if ((shared_x != nullptr) != (W_shared != nullptr))
@@ -535,7 +553,8 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
         return FK_OK;
     }
     if (!parts) return set_error(FK_ERR_INVALID, "routed reduce: workspace required");
-    FK_TRY(plan_routed_gemv(h, n_h_rows, Wd, nullptr, n_experts, row_idx, expert_idx, nullptr, n_routes, parts, out));
+    FK_TRY(plan_routed_gemv(h, n_h_rows, Wd, nullptr, n_experts, row_idx, expert_idx, nullptr, n_routes, parts, out, nullptr,
+                            nullptr, nullptr, nullptr, order));
     if (W_shared && n_tokens == 1) {
         GemvRequest rq;
         rq.mats[0] = W_shared;
@@ -560,5 +579,43 @@ fk_status plan_routed_reduce_chain(const uint16_t* h, uint32_t n_h_rows, const f
 }
 
 void set_routed_fused_reduce(bool on) { g_routed_fused_reduce = on; }
+
+// ---------------------------------------------------------------- routes in expert order
+// order[position] = route, the routes sorted by expert index (clamped as the routed kernels clamp it), routes of one
+// expert in their listed order: a stable counting sort by one block.  Each thread ranks its routes against the
+// list in LDS: rank = routes with a smaller expert + earlier routes with the same one.
+constexpr uint32_t kOrderMaxRoutes = 2048;
+struct RouteOrderArgs {
+    const uint32_t* expert_idx;
+    uint32_t* order;
+    uint32_t n_routes, n_experts;
+};
+__global__ __launch_bounds__(256) void route_order_kernel(const RouteOrderArgs a) {
+    __shared__ uint32_t ex[kOrderMaxRoutes];
+    for (uint32_t r = threadIdx.x; r < a.n_routes; r += 256) {
+        const uint32_t e = a.expert_idx[r];
+        ex[r] = e < a.n_experts ? e : a.n_experts - 1;
+    }
+    __syncthreads();
+    for (uint32_t r = threadIdx.x; r < a.n_routes; r += 256) {
+        const uint32_t e = ex[r];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < a.n_routes; ++j) rank += (ex[j] < e || (ex[j] == e && j < r)) ? 1u : 0u;
+        a.order[rank] = r;
+    }
+}
+
+fk_status plan_route_order(const uint32_t* expert_idx, uint32_t n_routes, uint32_t n_experts, uint32_t* order, Launch* out) {
+    if (!expert_idx || !order) return set_error(FK_ERR_INVALID, "route order: null array");
+    if (n_routes == 0 || n_experts == 0) return set_error(FK_ERR_INVALID, "route order: routes and experts must be positive");
+    if (n_routes > kOrderMaxRoutes) return set_error(FK_ERR_UNSUPPORTED, "route order: at most 2048 routes");
+    RouteOrderArgs a{expert_idx, order, n_routes, n_experts};
+    out->func = reinterpret_cast<const void*>(&route_order_kernel);
+    out->grid = dim3(1, 1, 1);
+    out->block = dim3(256, 1, 1);
+    out->shmem = 0;
+    out->set_args(a);
+    return FK_OK;
+}
 
 }  // namespace fk

@@ -171,7 +171,7 @@ def case_moe(d, reps, bits=4, tokens=1):
     x, res = _bf16(tokens * hidden, 1), _bf16(tokens * hidden, 2)
     row_idx = fk.DeviceBuffer.from_numpy(np.repeat(np.arange(tokens, dtype=np.uint32), top_k))  # route r reads its token's row
     h_rows = fk.DeviceBuffer.from_numpy(np.arange(routes, dtype=np.uint32))  # route r reads row r of the SwiGLU output
-    m1, m2, keep = [], [], []
+    m1, m2, o1, o2, keep = [], [], [], [], []
     for L in range(layers):
         Wg, Wu = _rand_weight(inter, hidden, bits, 300 + 10 * L, experts=E), _rand_weight(inter, hidden, bits, 303 + 10 * L, experts=E)
         Wd = _rand_weight(hidden, inter, bits, 306 + 10 * L, experts=E)
@@ -195,6 +195,12 @@ def case_moe(d, reps, bits=4, tokens=1):
                             arg(res), arg(out), arg(ws)],
                            {"bits": bits, "k": inter, "o": hidden, "experts": E, "tokens": tokens, "top_k": top_k,
                             "x_rows": routes, "has_extra": 1}))
+        if tokens > 1:   # the same launches with the routes served in expert order (fusekit_route_order)
+            order = fk.zeros(4 * routes)
+            fk.route_order(eidx, routes, E, order)
+            keep.append(order)
+            o1.append(Dispatch(m1[-1].kernel, list(m1[-1].args) + [arg(order)], dict(m1[-1].params, has_order=1)))
+            o2.append(Dispatch(m2[-1].kernel, list(m2[-1].args) + [arg(order)], dict(m2[-1].params, has_order=1)))
     uniq = sum(distinct) / len(distinct)  # an expert chosen by several rows is streamed once per route here
     b1 = routes * 2 * inter * hidden * per + tokens * hidden * 2 + routes * inter * 2
     b2 = routes * hidden * inter * per + routes * inter * 2 + 2 * tokens * hidden * 2
@@ -203,6 +209,11 @@ def case_moe(d, reps, bits=4, tokens=1):
           experts=E, distinct_experts=round(uniq, 1))
     _emit(f"routed_qmv_reduce_{tag}", _time_graph(d, m2, reps), b2, flops=2.0 * routes * inter * hidden, routes=routes, experts=E,
           note="three kernels: routed GEMV, ordered reduction")
+    if o1:
+        fk.sync()
+        _emit(f"routed_qmv_swiglu_{tag}_expert_order", _time_graph(d, o1, reps), b1, routes=routes, experts=E,
+              distinct_experts=round(uniq, 1), note="bytes as if every route streamed its slice")
+        _emit(f"routed_qmv_reduce_{tag}_expert_order", _time_graph(d, o2, reps), b2, routes=routes, experts=E)
 
 
 def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):

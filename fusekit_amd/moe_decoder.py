@@ -179,8 +179,9 @@ class MoeRuntime:
     """Scratch arena, KV caches, uniforms and the captured decode graph of one MoE model."""
 
     def __init__(self, cfg: MoeConfig, weights: MoeWeights, dispatcher: Optional[Dispatcher] = None,
-                 hist_capacity: int = 4096):
+                 hist_capacity: int = 4096, route_order: bool = True):
         c = cfg
+        self.route_order = route_order   # passes over several token rows serve their routes sorted by expert
         if c.kv_lora_rank % 64 or c.hidden % 64 or c.moe_inter % 64 or (c.kv_lora_rank + c.rope_dim) % 2:
             raise ValueError("widths must be multiples of the quantisation group")
         self.cfg, self.w = cfg, weights
@@ -452,6 +453,8 @@ class MoeRowsVariant:
         self.rlg = z(2 * m * c.n_experts)
         self.rows_x = DeviceBuffer.from_numpy(np.repeat(np.arange(m, dtype=np.uint32), c.top_k))
         self.rows_h = DeviceBuffer.from_numpy(np.arange(routes, dtype=np.uint32))
+        # the routes of a layer in the order the routed launches serve them: sorted by expert (fusekit_route_order)
+        self.order = z(4 * routes) if (rt.route_order and 1 < routes <= 2048) else None
         self.h = B(routes * c.moe_inter * 2)
         self.router_ws = z(4 * m * (c.n_experts + 1))
         shapes = [(n_q, c.hidden), (c.kv_lora_rank, c.hidden), (c.rope_dim, c.hidden), (n_b, c.kv_lora_rank),
@@ -530,17 +533,20 @@ class MoeRowsVariant:
                               dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1, rows=m)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
+            order, ordered = ([arg(self.order)], dict(has_order=1)) if self.order is not None else ([], {})
+            if order:
+                t.append(Dispatch(name("route_order"), [ridx, arg(self.order)], dict(routes=routes, experts=c.n_experts)))
             t.append(Dispatch(name("routed_qmv_swiglu"),
                               [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
-                               arg(self.rows_x), ridx, arg(self.h)],
-                              dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=routes, x_rows=m)))
+                               arg(self.rows_x), ridx, arg(self.h)] + order,
+                              dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=routes, x_rows=m, **ordered)))
             swiglu(Sg, Su, c.shared_inter)
             t.append(Dispatch(name("routed_qmv_reduce"),
                               [arg(self.h), arg(Ed.w), arg(Ed.scales), arg(Ed.biases), arg(self.rows_h), ridx, rwt,
                                arg(self.mid, m * c.shared_inter * 2), arg(Sd.w), arg(Sd.scales), arg(Sd.biases), arg(self.x[1]),
-                               arg(self.x[0]), arg(self.moe_ws)],
+                               arg(self.x[0]), arg(self.moe_ws)] + order,
                               dict(quant, k=c.moe_inter, o=c.hidden, experts=c.n_experts, tokens=m, top_k=c.top_k, x_rows=routes,
-                                   has_shared=1, shared_k=c.shared_inter, has_extra=1)))
+                                   has_shared=1, shared_k=c.shared_inter, has_extra=1, **ordered)))
         last = arg(self.x[0], c.hidden * 2, (m - 1) * c.hidden * 2)
         t.append(Dispatch(name("final_rmsnorm_lm_head"), [last, arg(w.vecs["final_norm"]), arg(emb.w), arg(rt.logits)],
                           dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)))

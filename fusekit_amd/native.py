@@ -242,6 +242,23 @@ def routed_qmv_reduce(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_wei
                                    _ptr(stream)))
 
 
+def routed_qmv_swiglu_ordered(x, n_x_rows, Wg, Wu, n_experts, row_idx, expert_idx, route_weight, n_routes, order, out0,
+                              stream=None) -> None:
+    """fk_routed_qmv_swiglu with the routes served in `order` (fk_route_order): same results, shared slices read once."""
+    check(lib.fk_routed_qmv_swiglu_ordered(_ptr(x), C.c_uint32(n_x_rows), C.byref(Wg.c), C.byref(Wu.c), C.c_uint32(n_experts),
+                                           _ptr(row_idx), _ptr(expert_idx), _ptr(route_weight), C.c_uint32(n_routes), _ptr(order),
+                                           _ptr(out0), _ptr(stream)))
+
+
+def routed_qmv_reduce_ordered(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_weight, shared_x, W_shared,
+                              residual_extra, n_tokens, top_k, order, out, workspace, stream=None) -> None:
+    check(lib.fk_routed_qmv_reduce_ordered(_ptr(h), C.c_uint32(n_h_rows), C.byref(Wd.c), C.c_uint32(n_experts),
+                                           _ptr(row_idx), _ptr(expert_idx), _ptr(route_weight), _ptr(shared_x),
+                                           C.byref(W_shared.c) if W_shared is not None else None, _ptr(residual_extra),
+                                           C.c_uint32(n_tokens), C.c_uint32(top_k), _ptr(order), _ptr(out), _ptr(workspace),
+                                           _ptr(stream)))
+
+
 def set_routed_fused_reduce(on: bool) -> None:
     lib.fk_set_routed_fused_reduce(C.c_int(int(on)))
 
@@ -547,6 +564,11 @@ def xcd_check(workspace, stream=None) -> None:
 
 def copy(dst, src, nbytes, stream=None):
     check(lib.fk_copy(_ptr(dst), _ptr(src), C.c_size_t(nbytes), _ptr(stream)))
+
+
+def route_order(expert_idx, n_routes: int, n_experts: int, order, stream=None) -> None:
+    """order[position] = route, the routes sorted by expert index, stable (fk_route_order)."""
+    check(lib.fk_route_order(_ptr(expert_idx), C.c_uint32(n_routes), C.c_uint32(n_experts), _ptr(order), _ptr(stream)))
 
 
 lib.fk_read_reduce_out_bytes.restype = C.c_size_t

@@ -172,6 +172,28 @@ fk_status fk_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps,
 fk_status fk_routed_qmv_swiglu(const uint16_t *x, uint32_t n_x_rows, const fk_weight *Wg, const fk_weight *Wu,
                                uint32_t n_experts, const uint32_t *row_idx, const uint32_t *expert_idx,
                                const uint16_t *route_weight, uint32_t n_routes, uint16_t *out0, fk_stream s);
+/* Several tokens whose routes share experts: `order` [n_routes] lists the routes in the order they are served
+ * (fk_route_order: sorted by expert, stable).  Inputs, outputs and arithmetic per route are those of
+ * fk_routed_qmv_swiglu (a route gets a multiple of eight blocks, so its tiles -- and the order in which a row's
+ * partial sums are added -- may differ from the listed launch's: equal to rounding-edge flips); routes of one
+ * expert sit next to each other in the grid and their blocks share an XCD, so an expert's slice is streamed
+ * from HBM once instead of once per route (the
+ * reference's kernels serve routes as listed, src/codegen/kernels/routed_qmv_swiglu.rs:104-160: row_idx /
+ * expert_idx per route).  Dispatch families fusekit_routed_qmv_swiglu / fusekit_routed_qmv_reduce take the same
+ * array as a last slot with the parameter has_order = 1; fusekit_route_order (slots expert_idx, order;
+ * parameters routes, experts) writes it. */
+fk_status fk_route_order(const uint32_t *expert_idx, uint32_t n_routes, uint32_t n_experts, uint32_t *order, fk_stream s);
+fk_status fk_routed_qmv_swiglu_ordered(const uint16_t *x, uint32_t n_x_rows, const fk_weight *Wg, const fk_weight *Wu,
+                                       uint32_t n_experts, const uint32_t *row_idx, const uint32_t *expert_idx,
+                                       const uint16_t *route_weight, uint32_t n_routes, const uint32_t *order,
+                                       uint16_t *out0, fk_stream s);
+/* fk_routed_qmv_reduce with the routed down projections served in `order` (several tokens); the weighted sums
+ * stay in slot order per token (src/codegen/kernels/routed_qmv_reduce.rs:240, 315-322). */
+fk_status fk_routed_qmv_reduce_ordered(const uint16_t *h, uint32_t n_h_rows, const fk_weight *Wd, uint32_t n_experts,
+                                       const uint32_t *row_idx, const uint32_t *expert_idx, const uint16_t *route_weight,
+                                       const uint16_t *shared_x, const fk_weight *W_shared, const uint16_t *residual_extra,
+                                       uint32_t n_tokens, uint32_t top_k, const uint32_t *order, uint16_t *out,
+                                       void *workspace, fk_stream s);
 /* The same launch with the block's SHARED experts riding along (one token): Sg / Su [n_shared * O, K] are
  * read as n_shared further routes -- row block j into shared_out [j * O ..) -- unweighted, with the same SwiGLU
  * (the reference runs them as a separate qmv_swiglu launch, src/codegen/kernels/qmv_swiglu.rs:20-246; the

@@ -256,6 +256,66 @@ def test_routed_reduce_tokens_and_row_idx(fk):
     assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
 
 
+def test_routes_served_in_expert_order_give_the_same_bits(fk):
+    """Several tokens whose routes share experts (config-5 widths, 8 tokens x top-6 over 16 experts): fk_route_order
+    is numpy's stable sort by (clamped) expert, and the routed launches served in that order -- an expert's slice
+    then comes from HBM once -- give the listed order's results (to rounding-edge flips: the tiles differ) and the
+    oracle's, for M1 and for M2 with a shared expert and a residual."""
+    E, O, K, tokens, top_k = 16, 1408, 2048, 8, 6
+    routes = tokens * top_k
+    Wg, Wu, Wd = _stack(3100, E, O, K, 4), _stack(3200, E, O, K, 4), _stack(3300, E, K, O, 4)
+    Ws = make_qweight(3400, K, 2816, 4)
+    x = normal_bf16(60, (tokens, K))
+    expert_idx = rng(61).integers(0, E, routes).astype(np.uint32)
+    expert_idx[5] = 4000                                       # clamps to E - 1, and sorts as E - 1
+    row_idx = np.repeat(np.arange(tokens, dtype=np.uint32), top_k)
+    rw = normal_bf16(62, routes, 0.2, 0.2)
+    d_e, order = _dev(fk, expert_idx), fk.zeros(4 * routes)
+    fk.route_order(d_e, routes, E, order)
+    fk.sync()
+    want_order = np.argsort(np.minimum(expert_idx, E - 1), kind="stable").astype(np.uint32)
+    assert np.array_equal(order.to_numpy(np.uint32), want_order)
+    dWg, dWu, dWd, dWs = (to_device(fk, W) for W in (Wg, Wu, Wd, Ws))
+    dx, dr, dw = _dev(fk, x), _dev(fk, row_idx), _dev(fk, rw)
+    h0, h1 = fk.DeviceBuffer(2 * routes * O), fk.DeviceBuffer(2 * routes * O)
+    fk.routed_qmv_swiglu(dx, tokens, dWg, dWu, E, dr, d_e, None, routes, h0)
+    fk.routed_qmv_swiglu_ordered(dx, tokens, dWg, dWu, E, dr, d_e, None, routes, order, h1)
+    fk.sync()
+    a, b = h0.to_numpy(np.uint16, (routes, O)), h1.to_numpy(np.uint16, (routes, O))
+    # same chunks, same products; the tile geometry follows the blocks a route gets (a multiple of eight when
+    # served in order), and with it the order in which a row's partial sums are added: rounding-edge flips only
+    frac, ulps = bf16_mismatch(b, a)
+    print("ordered against listed: %.4f of the outputs differ, by at most %.1f ulp" % (frac, ulps))
+    assert frac <= FLIP_FRACTION_BAR, (frac, ulps)
+    ref = oracle.routed_qmv_swiglu(x, Wg, Wu, row_idx, expert_idx, None)
+    for r in range(routes):
+        e = min(int(expert_idx[r]), E - 1)
+        _check_swiglu(b[r], ref[r], x[row_idx[r]], Wg.expert(e), Wu.expert(e), 1)
+    sx, res = normal_bf16(63, (tokens, 2816)), normal_bf16(64, (tokens, K))
+    outs = []
+    for ordered in (False, True):
+        out = fk.DeviceBuffer(2 * tokens * K)
+        ws = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, K, 2816, 64))
+        args = (h0, routes, dWd, E, None, d_e, dw, _dev(fk, sx), dWs, _dev(fk, res), tokens, top_k)
+        if ordered:
+            fk.routed_qmv_reduce_ordered(*args, order, out, ws)
+        else:
+            fk.routed_qmv_reduce(*args, out, ws)
+        fk.sync()
+        outs.append(out.to_numpy(np.uint16, (tokens, K)))
+    frac, ulps = bf16_mismatch(outs[1], outs[0])
+    assert frac <= FLIP_FRACTION_BAR, (frac, ulps)
+    ref2 = np.stack([oracle.routed_qmv_reduce(a[t * top_k:(t + 1) * top_k], Wd, expert_idx[t * top_k:(t + 1) * top_k],
+                                              rw[t * top_k:(t + 1) * top_k], res[t:t + 1], 1, top_k, shared_x=sx[t:t + 1], Wshared=Ws)[0]
+                     for t in range(tokens)])
+    frac, ulps = bf16_mismatch(outs[1], ref2)
+    assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
+    # an order that is not a permutation of the routes is refused where it can be seen (null), and a wild entry
+    # falls back to the position (never an address)
+    with pytest.raises(fk.FusekitError):
+        fk.routed_qmv_swiglu_ordered(dx, tokens, dWg, dWu, E, dr, d_e, None, routes, None, h1)
+
+
 def test_moe_block_full_size(fk):
     """Config-5 shapes (hidden 2048, expert width 1408, 6 of 16 experts, int4): M1 feeds M2."""
     E, hidden, inter, top_k = 16, 2048, 1408, 6
