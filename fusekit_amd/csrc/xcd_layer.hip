@@ -519,34 +519,46 @@ __device__ __forceinline__ uint32_t lanes_per_row(uint32_t cs) {
 }
 
 // Adds each row's partials in a fixed order; f(row, sum0, sum1) runs in one lane per row.
-template <bool TWO, typename F>
+// ONCE (the one-pass flavour): when a row group of 16, 8, ... lanes covers every row of the tile in ONE round and a lane
+// then holds at most ten partials per matrix, all its LDS reads go out first (clamped positions) and a row's epilogue
+// runs once -- instead of rounds of a read-wait-add loop (gate / up rows of the 4B-class MLP launch: two rounds of
+// sixteen lanes and five dependent LDS trips each took 1.65 us; one round of eight lanes 1.1).
+template <bool TWO, bool ONCE = false, typename F>
 __device__ __forceinline__ void tile_rows(const Tile& t, const float* part, const float* part1, F f) {
+    if constexpr (ONCE) {
+        // the widest row group (at most 16 lanes) with which every row of the tile fits one round
+        uint32_t lr1 = 16;
+        while (lr1 > 1 && t.rows * lr1 > (uint32_t)kBlock) lr1 >>= 1;
+        if (t.rows * lr1 <= (uint32_t)kBlock && t.cs <= 10u * lr1) {
+            const uint32_t lane1 = threadIdx.x & (lr1 - 1), rr = threadIdx.x / lr1;
+            const bool ok = rr < t.rows;
+            const uint32_t base = (ok ? rr : 0u) * t.cs;
+            float v0[10], v1[10];
+#pragma unroll
+            for (int k = 0; k < 10; ++k) {
+                const uint32_t i = lane1 + lr1 * k;
+                const uint32_t at = base + (i < t.cs ? i : 0u);
+                v0[k] = part[at];
+                if constexpr (TWO) v1[k] = part1[at];
+            }
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int k = 0; k < 10; ++k) {
+                const bool in = lane1 + lr1 * k < t.cs;
+                s0 += in ? v0[k] : 0.f;
+                if constexpr (TWO) s1 += in ? v1[k] : 0.f;
+            }
+            s0 = group_sum(s0, lr1);
+            if constexpr (TWO) s1 = group_sum(s1, lr1);
+            if (ok && lane1 == 0) f(rr, s0, s1);
+            return;
+        }
+    }
     const uint32_t lr = lanes_per_row(t.cs), lane = threadIdx.x & (lr - 1);
     const uint32_t step = kBlock / lr, rows_up = (t.rows + step - 1) / step * step;
     auto one = [&](uint32_t rr) {
         const bool ok = rr < t.rows;
         float s0 = 0.f, s1 = 0.f;
-#ifdef FK_AB_ROWS8
-        if (t.cs <= 8u * lr) {
-            // at most eight partials per lane (every 4B-class tile): all reads first, with clamped positions, then
-            // the additions in the loop's order -- one trip to the LDS instead of one per partial
-            const uint32_t base = (ok ? rr : 0u) * t.cs;
-            float v0[8], v1[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const uint32_t i = lane + k * lr;
-                const uint32_t at = base + (i < t.cs ? i : 0u);
-                v0[k] = part[at];
-                if constexpr (TWO) v1[k] = part1[at];
-            }
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const bool in = ok && lane + k * lr < t.cs;
-                s0 += in ? v0[k] : 0.f;
-                if constexpr (TWO) s1 += in ? v1[k] : 0.f;
-            }
-        } else
-#endif
         if (ok)
             for (uint32_t i = lane; i < t.cs; i += lr) {
                 s0 += part[rr * t.cs + i];
@@ -673,11 +685,13 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     FK_XCD_STAMP(1, 6);
     meta_store<KIND, kBlock, true>(md, tid, meta + 2 * kMetaWords);
     __syncthreads();
+    FK_XCD_STAMP(1, 12);
     if (streams && gu_n) {
         uint16_t* mid = a.mid + (size_t)sync.xcd * per_xcd + gu0;
         const int variant = a.swiglu_variant;
-        tile_rows<true>(tg, work, work + seg,
+        tile_rows<true, ONE>(tg, work, work + seg,
                         [&](uint32_t r, float s0, float s1) { mid[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
+
     }
     FK_XCD_STAMP(1, 7);
     uint32_t* okw = reinterpret_cast<uint32_t*>(red) + 8;
@@ -695,7 +709,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if (streams && d_n && ok) {
         long long* out = a.out_sums;
         XcdControl* ctl = sync.ctl;
-        tile_rows<false>(td, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, d0 + r, s0, ctl); });
+        tile_rows<false, ONE>(td, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, d0 + r, s0, ctl); });
     }
     FK_XCD_STAMP(1, 11);
 }
@@ -801,7 +815,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     FK_XCD_STAMP(0, 15);
     if (pr_n) {
         uint16_t* dst = (part_id == 0 ? a.q : (part_id == 1 ? a.k : a.v)) + (size_t)sync.xcd * part_rows + pr0;
-        tile_rows<false>(tq, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
+        tile_rows<false, ONE>(tq, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
     }
     FK_XCD_STAMP(0, 6);
     uint32_t* okw = reinterpret_cast<uint32_t*>(red) + 8;
@@ -895,6 +909,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     if (o_n && ok2) {
         long long* out = a.out_sums;
         XcdControl* ctl = sync.ctl;
+        // (the one-round form was slower here: 835 against 837 tok/s; the o_proj slice has 16 chunks per row)
         tile_rows<false>(to, work, work, [&](uint32_t r, float s0, float) { xcd_sum_add(out, o0 + r, s0, ctl); });
     }
     FK_XCD_STAMP(0, 12);
