@@ -423,7 +423,22 @@ __device__ __forceinline__ void gemv_run(const ARGS& a, uint32_t block_id, uint3
             const uint32_t lr = a.lr, lane = threadIdx.x & (lr - 1);
             for (uint32_t rr = threadIdx.x / lr; rr < R; rr += kGemvBlock / lr) {
                 float s0 = 0.f, s1 = 0.f;
-                for (uint32_t i = lane; i < cpr; i += lr) {
+                uint32_t i_first = lane;
+                if constexpr (NSEG == 1) {
+                    // the first eight partials of a lane are read in one go (clamped positions, masked additions in the
+                    // loop's order, so the sums keep their bits): one trip to the LDS instead of one per partial
+                    // (4864 x 896 int4: 4.59 -> 4.50 us; with the gate / up pair's two sums it gained nothing)
+                    float v0[8];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const uint32_t i = lane + (uint32_t)k * lr;
+                        v0[k] = part[rr * cpr + (i < cpr ? i : 0u)];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) s0 += lane + (uint32_t)k * lr < cpr ? v0[k] : 0.f;
+                    i_first = lane + 8u * lr;
+                }
+                for (uint32_t i = i_first; i < cpr; i += lr) {
                     s0 += part[rr * cpr + i];
                     if constexpr (NSEG == 2) s1 += part[seg_pad + rr * cpr + i];
                 }
