@@ -64,7 +64,7 @@ def family(kernel: str) -> str:
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the counter reads for a plain
 # 256 MiB copy); the runs and their commands are kept in profiles/xcd_layer_q4_4b.pmc_traffic.md.  Counters cannot be
 # read inside this process, so the figure is the recorded one for the kernel as built there.
-TRAFFIC_BYTES = {"xcd_mlp_kernel<Q4>": 44984200, "xcd_attn_kernel<Q4>": 18303200}  # the latter at context 505..520
+TRAFFIC_BYTES = {"xcd_mlp_kernel<Q4>": 44944500, "xcd_attn_kernel<Q4>": 18298100}  # the latter at context 505..520
 
 
 def main() -> int:

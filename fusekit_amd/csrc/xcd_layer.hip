@@ -1218,9 +1218,6 @@ AttnGeometry attn_geometry(const XcdLayerShape& s) {
     g.chunk_len = sdpa_chunk_len(s.head_dim, s.head_dim, false);
     uint32_t splits = kXcdSlots / G;
     if (splits > kXcdMaxRanges) splits = kXcdMaxRanges;
-#ifdef FK_AB_SPLITS
-    if (splits > FK_AB_SPLITS) splits = FK_AB_SPLITS;
-#endif
     const uint32_t n_chunks = ceil_div(s.capacity, g.chunk_len);
     g.chunks_per_block = ceil_div(n_chunks, splits);
     g.n_splits = ceil_div(n_chunks, g.chunks_per_block);
