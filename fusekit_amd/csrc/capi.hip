@@ -337,10 +337,9 @@ fk_status fk_routed_qmv_swiglu_ordered(const uint16_t* x, uint32_t n_x_rows, con
                                        const uint16_t* route_weight, uint32_t n_routes, const uint32_t* order,
                                        uint16_t* out0, fk_stream s) {
     if (!Wg || !Wu) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_ordered: null weight");
-    if (!order) return set_error(FK_ERR_INVALID, "fk_routed_qmv_swiglu_ordered: null order");
-    Launch l;
+    Launch l;   // no order array: the launch ranks its routes itself
     FK_TRY(plan_routed_gemv(x, n_x_rows, Wg, Wu, n_experts, row_idx, expert_idx, route_weight, n_routes, out0, &l, nullptr,
-                            nullptr, nullptr, nullptr, order));
+                            nullptr, nullptr, nullptr, order ? order : kOrderInKernel));
     return run_launch(l, (hipStream_t)s);
 }
 
@@ -350,10 +349,10 @@ fk_status fk_routed_qmv_reduce_ordered(const uint16_t* h, uint32_t n_h_rows, con
                                        uint32_t n_tokens, uint32_t top_k, const uint32_t* order, uint16_t* out, void* workspace,
                                        fk_stream s) {
     if (!workspace) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce_ordered: null workspace");
-    if (!order) return set_error(FK_ERR_INVALID, "fk_routed_qmv_reduce_ordered: null order");
     Launch l;
     FK_TRY(plan_routed_reduce_chain(h, n_h_rows, Wd, n_experts, row_idx, expert_idx, route_weight, shared_x, W_shared,
-                                    residual_extra, n_tokens, top_k, out, static_cast<uint16_t*>(workspace), &l, order));
+                                    residual_extra, n_tokens, top_k, out, static_cast<uint16_t*>(workspace), &l,
+                                    order ? order : kOrderInKernel));
     return run_launch(l, (hipStream_t)s);
 }
 

@@ -1014,8 +1014,10 @@ fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
     const bool pre_scale = d.u("pre_scale", 0) != 0, has_shared = d.u("has_shared", 0) != 0;
     const size_t n_slots = pre_scale ? 11 : 10;
     // with has_shared = 1: + shared gate w / s / b, shared up w / s / b, shared_out (parameter shared_o rows);
-    // with has_order = 1 (several tokens, no shared pair): + order (uint32 [routes], from fusekit_route_order)
-    const bool has_order = d.u("has_order", 0) != 0;
+    // with has_order = 1 (several tokens, no shared pair): + order (uint32 [routes], from fusekit_route_order);
+    // with expert_order = 1 instead (no slot, up to 64 routes): the launch finds the same order itself
+    const bool has_order = d.u("has_order", 0) != 0, expert_order = d.u("expert_order", 0) != 0;
+    if (has_order && expert_order) return set_error(FK_ERR_INVALID, d.kernel + ": has_order and expert_order exclude each other");
     FK_TRY(need_args(d, n_slots + (has_shared ? 7 : 0) + (has_order ? 1 : 0)));
     if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
     if (experts == 0 || routes == 0 || K == 0 || O == 0)
@@ -1042,7 +1044,7 @@ fk_status plan_routed_swiglu(const Dispatch& d, Launch* l, SlotRW* rw) {
         for (uint32_t i = 0; i < 6; ++i) rw->reads.push_back((uint32_t)n_slots + i);
         rw->writes.push_back((uint32_t)n_slots + 6);
     }
-    const uint32_t* order = nullptr;
+    const uint32_t* order = expert_order ? kOrderInKernel : nullptr;
     if (has_order) {
         const size_t os = n_slots + (has_shared ? 7 : 0);
         FK_TRY(need_bytes(d, os, (size_t)routes * 4));
@@ -1072,6 +1074,8 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     const size_t extra_slot = has_extra ? s++ : 0;
     const size_t out_slot = s++, ws_slot = s++;
     const bool has_order = d.u("has_order", 0) != 0;   // + order (uint32 [routes], from fusekit_route_order) as the last slot
+    const bool expert_order = d.u("expert_order", 0) != 0;   // no slot, up to 64 routes: the launch finds that order itself
+    if (has_order && expert_order) return set_error(FK_ERR_INVALID, d.kernel + ": has_order and expert_order exclude each other");
     const size_t order_slot = has_order ? s++ : 0;
     FK_TRY(need_args(d, s));
     if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
@@ -1094,7 +1098,7 @@ fk_status plan_routed_reduce(const Dispatch& d, Launch* l, SlotRW* rw) {
     for (uint32_t i = 0; i < out_slot; ++i) rw->reads.push_back(i);
     rw->reads.push_back((uint32_t)ws_slot);
     rw->writes = {(uint32_t)out_slot, (uint32_t)ws_slot};
-    const uint32_t* order = nullptr;
+    const uint32_t* order = expert_order ? kOrderInKernel : nullptr;
     if (has_order) {
         FK_TRY(need_bytes(d, order_slot, (size_t)routes * 4));
         order = arg_ptr<const uint32_t>(d, order_slot);

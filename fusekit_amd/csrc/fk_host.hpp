@@ -135,6 +135,9 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
                            const fk_weight* sh_a = nullptr, const fk_weight* sh_b = nullptr, uint16_t* sh_y = nullptr,
                            const RouteInKernel* rk = nullptr, const uint32_t* order = nullptr);
 // order[position] = route: the routes sorted by expert (stable), for the `order` argument of the routed launches.
+// kOrderInKernel in place of an array: every wave of the launch ranks the routes itself (up to 64 routes); the value
+// is a tag and is never dereferenced.
+static const uint32_t* const kOrderInKernel = reinterpret_cast<const uint32_t*>(uintptr_t(1));
 fk_status plan_route_order(const uint32_t* expert_idx, uint32_t n_routes, uint32_t n_experts, uint32_t* order, Launch* out);
 // Routed down projection + weighted reduction (+ shared expert + residual): one fused launch for one token
 // of int4 weights, else routed GEMV -> shared GEMV -> ordered reduction chained in out->then (`parts`,

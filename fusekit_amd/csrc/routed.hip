@@ -56,6 +56,11 @@ struct RoutedArgs {
     // XCD at the same time: the slice comes from HBM once and from that XCD's L2 for the other rows.  Inputs,
     // outputs and arithmetic of a route are untouched.
     const uint32_t* order;
+    // The same serving order found by every wave for itself (up to 64 routes): lane i takes expert_idx[i], ranks the
+    // key (expert, i) among all routes, and the lane whose rank is the block's position names the route.  No order
+    // array, no launch in front to write one, and the expert and the activation row of the route come out of the same
+    // trip to memory.
+    uint32_t rank_in_kernel;
 };
 
 // GemvArgs as one route sees it.  n_mats is a compile-time 1 so that every index
@@ -86,19 +91,36 @@ __global__ __launch_bounds__(kGemvBlock) void routed_gemv_kernel(const RoutedArg
     kernarg_warm<(int)sizeof(RoutedArgs)>();
     const uint32_t pos = blockIdx.x / a.blocks_per_route, sub = blockIdx.x - pos * a.blocks_per_route;
     uint32_t route = pos;
+    uint32_t e = 0, row = 0;
     if (a.order && pos < a.n_routes) {
         route = a.order[pos];
         route = route < a.n_routes ? route : pos;   // a device array is not trusted with addresses
     }
+    const bool ranked = a.rank_in_kernel && pos < a.n_routes;   // uniform per block
+    if (ranked) {
+        const uint32_t lane = threadIdx.x & (kWave - 1), li = lane < a.n_routes ? lane : 0u;
+        uint32_t ei = a.expert_idx[li];
+        uint32_t ri = a.row_idx ? a.row_idx[li] : li;
+        ei = ei < a.n_experts ? ei : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
+        const uint32_t key = lane < a.n_routes ? ei * kWave + lane : 0xffffffffu;   // distinct per route
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < a.n_routes; ++j) rank += (uint32_t)__builtin_amdgcn_readlane((int)key, (int)j) < key ? 1u : 0u;
+        const unsigned long long hit = __ballot(rank == pos && lane < a.n_routes);   // exactly one lane
+        route = hit ? (uint32_t)__builtin_ctzll(hit) : pos;
+        e = (uint32_t)__builtin_amdgcn_readlane((int)ei, (int)route);
+        row = (uint32_t)__builtin_amdgcn_readlane((int)ri, (int)route);
+        row = row < a.n_x_rows ? row : a.n_x_rows - 1;
+    }
     const bool extra = route >= a.n_routes;     // uniform per block
     const uint32_t lookup = extra ? 0u : route;
-    uint32_t e = 0, row = 0;
     float routed_weight = 1.0f;
     if (!a.logits) {
-        e = a.expert_idx[lookup];
-        e = e < a.n_experts ? e : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
-        row = a.row_idx ? a.row_idx[lookup] : lookup;
-        row = row < a.n_x_rows ? row : a.n_x_rows - 1;
+        if (!ranked) {
+            e = a.expert_idx[lookup];
+            e = e < a.n_experts ? e : a.n_experts - 1;  // routed_qmv_swiglu.rs:138
+            row = a.row_idx ? a.row_idx[lookup] : lookup;
+            row = row < a.n_x_rows ? row : a.n_x_rows - 1;
+        }
         if (a.route_weight && !extra) routed_weight = bf16_bits_to_f32(a.route_weight[lookup]);
     }
     if (extra) row = 0;
@@ -372,6 +394,9 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (order && (rk || sh_a)) return set_error(FK_ERR_UNSUPPORTED, "routed: a serving order goes with listed routes of several tokens only");
+    const bool rank_in_kernel = order == kOrderInKernel;
+    if (rank_in_kernel && (n_routes > 64 || n_experts > (1u << 24)))
+        return set_error(FK_ERR_UNSUPPORTED, "routed: the launch ranks up to 64 routes itself; more take an order array (fk_route_order)");
     if (rk) {
         if (!rk->logits || !rk->scale || !rk->idx_out || !rk->weight_out) return set_error(FK_ERR_INVALID, "routed: null routing tensor");
         if (n_x_rows != 1) return set_error(FK_ERR_UNSUPPORTED, "routed: the launch routes for one token only");
@@ -442,7 +467,8 @@ fk_status plan_routed_gemv(const uint16_t* x, uint32_t n_x_rows, const fk_weight
     a.y_stride = w_a->n;
     a.n_routes = n_routes;
     a.x_routes = x_routes;
-    a.order = order;
+    a.order = rank_in_kernel ? nullptr : order;
+    a.rank_in_kernel = rank_in_kernel ? 1u : 0u;
     if (rk) {
         a.logits = rk->logits; a.route_scale = rk->scale; a.idx_out = rk->idx_out; a.weight_out = rk->weight_out;
         a.route_weight = rk->apply_weight ? rk->scale : nullptr;

@@ -179,7 +179,7 @@ class MoeRuntime:
     """Scratch arena, KV caches, uniforms and the captured decode graph of one MoE model."""
 
     def __init__(self, cfg: MoeConfig, weights: MoeWeights, dispatcher: Optional[Dispatcher] = None,
-                 hist_capacity: int = 4096, route_order: bool = True):
+                 hist_capacity: int = 4096, route_order: bool = False):
         c = cfg
         self.route_order = route_order   # passes over several token rows serve their routes sorted by expert
         if c.kv_lora_rank % 64 or c.hidden % 64 or c.moe_inter % 64 or (c.kv_lora_rank + c.rope_dim) % 2:
@@ -454,7 +454,8 @@ class MoeRowsVariant:
         self.rows_x = DeviceBuffer.from_numpy(np.repeat(np.arange(m, dtype=np.uint32), c.top_k))
         self.rows_h = DeviceBuffer.from_numpy(np.arange(routes, dtype=np.uint32))
         # the routes of a layer in the order the routed launches serve them: sorted by expert (fusekit_route_order)
-        self.order = z(4 * routes) if (rt.route_order and 1 < routes <= 2048) else None
+        self.rank_in_launch = rt.route_order and 1 < routes <= 64      # the routed launches rank the routes themselves
+        self.order = z(4 * routes) if (rt.route_order and 64 < routes <= 2048) else None
         self.h = B(routes * c.moe_inter * 2)
         self.router_ws = z(4 * m * (c.n_experts + 1))
         shapes = [(n_q, c.hidden), (c.kv_lora_rank, c.hidden), (c.rope_dim, c.hidden), (n_b, c.kv_lora_rank),
@@ -534,6 +535,8 @@ class MoeRowsVariant:
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
             order, ordered = ([arg(self.order)], dict(has_order=1)) if self.order is not None else ([], {})
+            if self.rank_in_launch:
+                ordered = dict(expert_order=1)
             if order:
                 t.append(Dispatch(name("route_order"), [ridx, arg(self.order)], dict(routes=routes, experts=c.n_experts)))
             t.append(Dispatch(name("routed_qmv_swiglu"),

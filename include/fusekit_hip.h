@@ -181,7 +181,9 @@ fk_status fk_routed_qmv_swiglu(const uint16_t *x, uint32_t n_x_rows, const fk_we
  * reference's kernels serve routes as listed, src/codegen/kernels/routed_qmv_swiglu.rs:104-160: row_idx /
  * expert_idx per route).  Dispatch families fusekit_routed_qmv_swiglu / fusekit_routed_qmv_reduce take the same
  * array as a last slot with the parameter has_order = 1; fusekit_route_order (slots expert_idx, order;
- * parameters routes, experts) writes it. */
+ * parameters routes, experts) writes it.  order = NULL (families: parameter expert_order = 1, no slot): up to 64
+ * routes, every wave of the launch ranks the routes by (expert, route) itself -- the same order without an array
+ * and without the launch that writes one (one graph node less per layer; more than 64 routes: FK_ERR_UNSUPPORTED). */
 fk_status fk_route_order(const uint32_t *expert_idx, uint32_t n_routes, uint32_t n_experts, uint32_t *order, fk_stream s);
 fk_status fk_routed_qmv_swiglu_ordered(const uint16_t *x, uint32_t n_x_rows, const fk_weight *Wg, const fk_weight *Wu,
                                        uint32_t n_experts, const uint32_t *row_idx, const uint32_t *expert_idx,

@@ -202,15 +202,17 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
         first, first + 7, n_classes, len(set(ridx[0].reshape(-1).tolist()))))
 
 
-@pytest.mark.parametrize("rows,offset", [(8, 0), (5, 8), (1, 3)])
-def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset):
+@pytest.mark.parametrize("rows,offset,route_order", [(8, 0, False), (5, 8, False), (1, 3, False), (8, 0, True), (20, 4, True)])
+def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset, route_order):
     """Several active token rows in one pass over the weights (multi-row matmuls, row forms of the store, the
     attention and the router, routed experts over rows x top_k routes, shared experts with several tokens)
-    against the oracle stepping through the same tokens one by one: caches, routes, logits, next token."""
+    against the oracle stepping through the same tokens one by one: caches, routes, logits, next token.  With
+    `route_order` the routed launches serve their routes sorted by expert: up to 64 routes they rank them
+    themselves (8 rows x 4), beyond that a small launch writes the order first (20 rows x 4)."""
     from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
     cfg = _small_cfg(hidden=512, n_experts=16, top_k=4)
     W = MoeWeights.random_init(cfg, seed=6)
-    rt, od = MoeRuntime(cfg, W), OracleMoeDecoder(cfg, W)
+    rt, od = MoeRuntime(cfg, W, route_order=route_order), OracleMoeDecoder(cfg, W)
     toks = rng(7).integers(0, cfg.vocab, offset + rows).tolist()
     routes = []
     for i, t in enumerate(toks):
@@ -223,6 +225,9 @@ def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset):
     r = oracle.bf16_to_f32(logits).astype(np.float64)
     assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
     assert got == nxt
+    if route_order:
+        v = rt._rows_variants[rows]
+        assert v.rank_in_launch == (rows * cfg.top_k <= 64) and (v.order is not None) == (rows * cfg.top_k > 64)
     same = sum(set(rt.rows_routes[j].tolist()) == set(routes[offset + j].tolist()) for j in range(rows))
     assert same >= rows - 1, (rt.rows_routes, routes[offset:])
     last = cfg.n_layers - 1

@@ -260,7 +260,8 @@ def test_routes_served_in_expert_order_give_the_same_bits(fk):
     """Several tokens whose routes share experts (config-5 widths, 8 tokens x top-6 over 16 experts): fk_route_order
     is numpy's stable sort by (clamped) expert, and the routed launches served in that order -- an expert's slice
     then comes from HBM once -- give the listed order's results (to rounding-edge flips: the tiles differ) and the
-    oracle's, for M1 and for M2 with a shared expert and a residual."""
+    oracle's, for M1 and for M2 with a shared expert and a residual.  The launches that rank the routes themselves
+    (no order array) give the bits of the launches that read the array."""
     E, O, K, tokens, top_k = 16, 1408, 2048, 8, 6
     routes = tokens * top_k
     Wg, Wu, Wd = _stack(3100, E, O, K, 4), _stack(3200, E, O, K, 4), _stack(3300, E, K, O, 4)
@@ -310,10 +311,21 @@ def test_routes_served_in_expert_order_give_the_same_bits(fk):
                      for t in range(tokens)])
     frac, ulps = bf16_mismatch(outs[1], ref2)
     assert frac <= FLIP_FRACTION_BAR and ulps <= 2.0, (frac, ulps)
-    # an order that is not a permutation of the routes is refused where it can be seen (null), and a wild entry
-    # falls back to the position (never an address)
+    # without an order array (up to 64 routes) every wave of the launch ranks the routes itself: the same order,
+    # the same grid, hence the same bits as with the array
+    h2 = fk.DeviceBuffer(2 * routes * O)
+    fk.routed_qmv_swiglu_ordered(dx, tokens, dWg, dWu, E, dr, d_e, None, routes, None, h2)
+    out2 = fk.DeviceBuffer(2 * tokens * K)
+    ws2 = fk.DeviceBuffer(fk.routed_reduce_workspace_bytes(tokens, top_k, K, 2816, 64))
+    fk.routed_qmv_reduce_ordered(h0, routes, dWd, E, None, d_e, dw, _dev(fk, sx), dWs, _dev(fk, res), tokens, top_k, None, out2, ws2)
+    fk.sync()
+    assert np.array_equal(h2.to_numpy(np.uint16, (routes, O)), b)
+    assert np.array_equal(out2.to_numpy(np.uint16, (tokens, K)), outs[1])
+    # more than 64 routes need the array
+    many = 66
     with pytest.raises(fk.FusekitError):
-        fk.routed_qmv_swiglu_ordered(dx, tokens, dWg, dWu, E, dr, d_e, None, routes, None, h1)
+        fk.routed_qmv_swiglu_ordered(dx, tokens, dWg, dWu, E, _dev(fk, np.zeros(many, np.uint32)), _dev(fk, np.zeros(many, np.uint32)),
+                                     None, many, None, fk.DeviceBuffer(2 * many * O))
 
 
 def test_moe_block_full_size(fk):
