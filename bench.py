@@ -87,6 +87,8 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain 256 MiB device copies (outside the timed region): the known-traffic "
                          "kernel that rocprofv3 byte counters of the same run are scaled by")
+    ap.add_argument("--layer-launch", action="store_true",
+                    help="a layer's attention and MLP launches as ONE launch with a device-wide barrier between the phases")
     ap.add_argument("--five-launches", action="store_true",
                     help="experiment only: the per-dispatch task list (five launches per layer) instead of the two-launch layer")
     ap.add_argument("--mode", choices=["persistent", "graph"], default="graph",
@@ -107,7 +109,8 @@ def main() -> int:
     start = max(args.prompt + args.warmup, CONTEXT - args.steps // 2)   # context of the first timed step
     total = start + args.steps
     capacity = max(1024, 1 << (total - 1).bit_length())
-    cfg = DecoderConfig(**DENSE_4B, bits=args.bits, capacity=capacity, xcd_layers=not args.five_launches)
+    cfg = DecoderConfig(**DENSE_4B, bits=args.bits, capacity=capacity, xcd_layers=not args.five_launches,
+                        xcd_layer_launch=args.layer_launch)
     if args.layers:
         cfg.n_layers = args.layers
     t0 = time.time()

@@ -1908,9 +1908,29 @@ fk_status find_fused_runs(Graph* g) {
             ++i;
             continue;
         }
+        if (d.u("token_launch", 0) == 2) {
+            // one launch per LAYER: this attention launch and the MLP launch behind it, as they were planned
+            if (i + 1 < n && is_family(g->nodes[i + 1].d, "fusekit_xcd_mlp_block") && g->nodes[i + 1].d.u("token_launch", 0) == 2) {
+                Graph::FusedRun run;
+                run.first = i;
+                run.count = 2;
+                const fk_status st = plan_xcd_layer(g->nodes[i].launch, g->nodes[i + 1].launch, &run.launch);
+                if (st == FK_ERR_UNSUPPORTED) {  // e.g. a shape whose tiles need the pass loop: the two launches stay
+                    i += 2;
+                    continue;
+                }
+                FK_TRY(st);
+                g->fused.push_back(run);
+                g->fused_of[i] = g->fused_of[i + 1] = (int)g->fused.size() - 1;
+                i += 2;
+            } else {
+                ++i;
+            }
+            continue;
+        }
         size_t j = i;
-        while (j + 1 < n && is_family(g->nodes[j].d, "fusekit_xcd_attn_block") && g->nodes[j].d.u("token_launch", 0) != 0 &&
-               is_family(g->nodes[j + 1].d, "fusekit_xcd_mlp_block") && g->nodes[j + 1].d.u("token_launch", 0) != 0 &&
+        while (j + 1 < n && is_family(g->nodes[j].d, "fusekit_xcd_attn_block") && g->nodes[j].d.u("token_launch", 0) == 1 &&
+               is_family(g->nodes[j + 1].d, "fusekit_xcd_mlp_block") && g->nodes[j + 1].d.u("token_launch", 0) == 1 &&
                g->nodes[j].d.u("bits", 4) == d.u("bits", 4))
             j += 2;
         const size_t count = j - i;
@@ -2188,12 +2208,17 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
     }
     // all checks passed: apply.  A HIP failure below can still leave the executable graph partly updated;
     // the error is reported and the caller must rebuild.
+    std::vector<int> replan;
     for (size_t k = 0; k < touched.size(); ++k) {
         Node& nd = g->nodes[touched[k]];
         nd.d = patched[k];
         nd.launch = launches[k];
         nd.rw = rws[k];
         const int fr = g->fused_of.empty() ? -1 : g->fused_of[touched[k]];
+        if (fr >= 0 && !g->fused[fr].d_attn) {
+            replan.push_back(fr);  // a layer launch carries both argument blocks by value: planned again below
+            continue;
+        }
         if (fr >= 0) {
             // member of a run that executes as one launch: its argument block in the run's device table is replaced
             Graph::FusedRun& run = g->fused[fr];
@@ -2211,6 +2236,15 @@ fk_status fk_update_graph_bindings(fk_handle h, uint32_t graph_id, const fk_bind
             hipKernelNodeParams fp = launch_params(nd.launch.then[f], slot);
             FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, nd.tail[f], &fp));
         }
+    }
+    std::sort(replan.begin(), replan.end());
+    replan.erase(std::unique(replan.begin(), replan.end()), replan.end());
+    for (int fr : replan) {
+        Graph::FusedRun& run = g->fused[fr];
+        FK_TRY(plan_xcd_layer(g->nodes[run.first].launch, g->nodes[run.first + 1].launch, &run.launch));
+        void* slot[kMaxKernelParams];
+        hipKernelNodeParams p = launch_params(run.launch, slot);
+        FK_HIP(hipGraphExecKernelNodeSetParams(g->exec, run.node, &p));
     }
     return FK_OK;
 }

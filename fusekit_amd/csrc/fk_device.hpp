@@ -124,15 +124,16 @@ __device__ __forceinline__ void wait_memory_ops_done() { __builtin_amdgcn_s_wait
 // for them once.  A long kernel otherwise fetches its arguments where it first uses them, phase by phase, and each
 // first touch of a line is a scalar-cache miss -- a trip to the L2 -- in the middle of that phase; after this the
 // later fetches hit.  Call it where the wave waits for its first arguments anyway.
-template <int BYTES>
+// (FROM: the first line covered; a block of more than twelve lines takes a second call with FROM = 12.)
+template <int BYTES, int FROM = 0>
 __device__ __forceinline__ void kernarg_warm() {
     typedef const uint32_t __attribute__((address_space(4))) * karg_t;
     karg_t ka = (karg_t)__builtin_amdgcn_kernarg_segment_ptr();
-    constexpr int LINES = (BYTES + 63) / 64;
-    static_assert(LINES <= 12, "argument block larger than this helper covers");
+    constexpr int LINES = (BYTES + 63) / 64 - FROM;
+    static_assert(LINES >= 1 && LINES <= 12, "argument block larger than this helper covers");
     uint32_t v[12];
 #pragma unroll
-    for (int i = 0; i < 12; ++i) v[i] = ka[(i < LINES ? i : 0) * 16];
+    for (int i = 0; i < 12; ++i) v[i] = ka[(FROM + (i < LINES ? i : 0)) * 16];
     // one statement that takes them all: every request goes out before the one wait
     asm volatile("" ::"s"(v[0]), "s"(v[1]), "s"(v[2]), "s"(v[3]), "s"(v[4]), "s"(v[5]), "s"(v[6]), "s"(v[7]), "s"(v[8]),
                  "s"(v[9]), "s"(v[10]), "s"(v[11]));

@@ -18,7 +18,7 @@ struct Launch {
     dim3 grid{1, 1, 1}, block{1, 1, 1};
     uint32_t shmem = 0;
     size_t args_size = 0;
-    alignas(16) unsigned char args[640];
+    alignas(16) unsigned char args[896];
     // Kernels that complete the same operation and must run after this one, in
     // order (a split-k reduction, a routed reduction).  run_launch and the graph
     // builder treat the chain as one unit.

@@ -1029,6 +1029,33 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_token_kernel(const XcdTokenArgs
     xcd_mark_placement(sync, t.mark_placement);
 }
 
+// ---- a whole layer in one launch ------------------------------------------------------------------------------
+// Attention phase (the stand-alone launch's, input requested from the leading parameters), a device-wide barrier,
+// MLP phase.  What crosses the barrier: the sum row the attention phase added into (memory-side additions, read with
+// L1-bypassing loads), the residual row (every block holds its own copy in LDS) and the row the attention phase
+// cleared for the MLP phase to add into (write-through stores).  Everything else is private to an XCD as in the
+// separate launches.
+template <WKind KIND, int NLQ, int NLO, int NLG, int NLD>
+__global__ __launch_bounds__(kBlock, 2) void xcd_layer_kernel(const long long* sums, const uint16_t* residual,
+                                                              const uint16_t* norm_w, uint32_t hidden, const XcdLayerArgs t) {
+    extern __shared__ uint4 lds_raw[];
+    const XcdInputLead lead{sums, residual, norm_w, hidden};
+    InputRegs inr;
+    input_request<false>(lead, inr, nullptr);
+    kernarg_warm<768>();
+    kernarg_warm<32 + (int)sizeof(XcdLayerArgs), 12>();
+    uint4* xres = lds_raw + t.xres_off;
+    XcdSync sync = xcd_sync_init(t.attn.ctl, t.attn.spin_limit);
+    XcdGlobalSync gs = xcd_global_init(sync);
+    xcd_attn_phase<KIND, NLQ, NLO, true, true, true>(t.attn, lead, inr, sync, lds_raw, nullptr, xres);
+    if (!xcd_global_barrier(sync, gs)) return;
+    {
+        InputRegs inm;
+        xcd_mlp_phase<KIND, NLG, NLD, true, false, true>(t.mlp, t.mlp.in, inm, sync, lds_raw, xres, nullptr);
+    }
+    xcd_mark_placement(sync, t.mark_placement);
+}
+
 __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs a) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= a.hidden) return;
@@ -1109,6 +1136,12 @@ const void* attn_func(bool one) {
     constexpr PassDepth d = depth_of(KIND);
     return one ? reinterpret_cast<const void*>(&xcd_attn_kernel<KIND, d.qkv, d.o, true>)
                : reinterpret_cast<const void*>(&xcd_attn_kernel<KIND, kNlQkv, kNlO, false>);
+}
+
+template <WKind KIND>
+const void* layer_func() {
+    constexpr PassDepth d = depth_of(KIND);
+    return reinterpret_cast<const void*>(&xcd_layer_kernel<KIND, d.qkv, d.o, d.gu, d.down>);
 }
 
 uint32_t lds_for(uint32_t bits, const LdsPlan& p) {
@@ -1445,6 +1478,42 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     out->add_lead(a.in.residual);
     out->add_lead(a.in.norm_w);
     out->add_lead(a.in.hidden);
+    return FK_OK;
+}
+
+fk_status plan_xcd_layer(const Launch& la, const Launch& lm, Launch* out) {
+    if (la.args_size != sizeof(XcdAttnArgs) || lm.args_size != sizeof(XcdMlpArgs))
+        return set_error(FK_ERR_INVALID, "xcd layer launch: not an attention launch followed by an MLP launch");
+    XcdLayerArgs t;
+    memset(&t, 0, sizeof(t));
+    memcpy(&t.attn, la.args, sizeof(XcdAttnArgs));
+    memcpy(&t.mlp, lm.args, sizeof(XcdMlpArgs));
+    const void* func = nullptr;
+    if (la.func == attn_func<W_Q4>(true) && lm.func == mlp_func<W_Q4>(true)) func = layer_func<W_Q4>();
+    if (la.func == attn_func<W_Q8>(true) && lm.func == mlp_func<W_Q8>(true)) func = layer_func<W_Q8>();
+    if (la.func == attn_func<W_BF16>(true) && lm.func == mlp_func<W_BF16>(true)) func = layer_func<W_BF16>();
+    if (!func) return set_error(FK_ERR_UNSUPPORTED, "xcd layer launch: both launches must take their one-pass flavour, same weight kind");
+    if (t.attn.ctl != t.mlp.ctl) return set_error(FK_ERR_INVALID, "xcd layer launch: the two launches use different control blocks");
+    if (!t.mlp.in.sums || t.mlp.in.sums != t.attn.out_sums || t.mlp.in.residual != t.attn.in.x_out ||
+        t.mlp.in.hidden != t.attn.in.hidden)
+        return set_error(FK_ERR_INVALID, "xcd layer launch: the MLP launch must read the sum row the attention launch adds into and the row it writes");
+    if (t.attn.in.clear != t.mlp.out_sums)
+        return set_error(FK_ERR_INVALID, "xcd layer launch: the attention launch must clear the row the MLP launch adds into");
+    const uint32_t phase_lds = ((la.shmem > lm.shmem ? la.shmem : lm.shmem) + 15u) & ~15u;
+    t.xres_off = phase_lds / 16u;
+    t.mark_placement = (t.attn.mark_placement | t.mlp.mark_placement) ? 1u : 0u;
+    const uint32_t lds = phase_lds + t.attn.in.hidden * 2u;
+    out->func = func;
+    FK_TRY(require_two_blocks_per_cu(out->func, lds, "whole-layer"));
+    out->grid = dim3(kXcdGrid, 1, 1);
+    out->block = dim3(kBlock, 1, 1);
+    out->shmem = lds;
+    out->set_args(t);
+    out->n_lead = 0;
+    out->add_lead(t.attn.in.sums);
+    out->add_lead(t.attn.in.residual);
+    out->add_lead(t.attn.in.norm_w);
+    out->add_lead(t.attn.in.hidden);
     return FK_OK;
 }
 

@@ -163,6 +163,15 @@ struct XcdTokenArgs {
     uint32_t mark_placement;
 };
 
+// A whole layer in one launch: the attention phase, a device-wide barrier, the MLP phase (xcd_layer_kernel).  The two
+// blocks are those of the stand-alone launches, by value.
+struct XcdLayerArgs {
+    XcdAttnArgs attn;
+    XcdMlpArgs mlp;
+    uint32_t xres_off;         // LDS offset (16-byte units) of the block's copy of the residual row
+    uint32_t mark_placement;
+};
+
 // x = T(f32(sums) + residual): the last layer's output for the LM head.  `clear` (may be the row read, or null)
 // is zeroed element by element behind the read: the row the next token's first launch adds into.
 struct XcdReduceArgs {
@@ -234,6 +243,11 @@ struct XcdMlpRequest {
     bool for_token;   // the block is meant for the whole-token launch (its gate / up passes are shallower)
 };
 fk_status plan_xcd_mlp(const XcdMlpRequest& rq, Launch* out);
+// One launch for an attention launch and the MLP launch that follows it (both as planned by plan_xcd_attn /
+// plan_xcd_mlp in their one-pass flavours, the MLP launch reading the sum row the attention launch adds into and the
+// row it writes as x_out): attention phase, device-wide barrier, MLP phase.  The MLP phase's first weight requests go
+// out in front of the barrier.
+fk_status plan_xcd_layer(const Launch& attn, const Launch& mlp, Launch* out);
 // One launch for a run of alternating attention / MLP launches (as planned by plan_xcd_attn / plan_xcd_mlp, same
 // weight kind): `d_attn` / `d_mlp` are device copies of their argument blocks.  Requirements beyond the separate
 // launches': every layer has its own q / k / v rows (a block reads them with ordinary loads, and inside one launch

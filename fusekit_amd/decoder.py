@@ -49,6 +49,7 @@ class DecoderConfig:
     xcd_spin_limit: int = 0   # bound of the XCD hand-over waits in polls (0: the library's default)
     direct_head_argmax: bool = True  # graph mode: the LM head selects the greedy token itself where its shape allows
     xcd_token_launch: bool = False  # the layers' launches of a token as ONE launch (device-wide barriers between them); slower at present
+    xcd_layer_launch: bool = False  # a layer's two launches as ONE launch (attention phase, device-wide barrier, MLP phase)
 
     @property
     def n_q(self) -> int:
@@ -386,7 +387,7 @@ class DecoderRuntime:
         c, w = self.cfg, self.w
         shape = dict(hidden=c.hidden, inter=c.inter, n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim,
                      capacity=c.capacity, bits=c.bits, group=c.group, eps=c.eps, theta=c.theta,
-                     spin_limit=c.xcd_spin_limit, token_launch=int(c.xcd_token_launch))
+                     spin_limit=c.xcd_spin_limit, token_launch=1 if c.xcd_token_launch else (2 if c.xcd_layer_launch else 0))
         quant = c.bits != 16
         for l in range(c.n_layers):
             p = f"layers.{l}."

@@ -439,6 +439,11 @@ def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk)
     rt2 = DecoderRuntime(cfg2, W)
     got2, _, _ = rt2.generate(fx["prompt"], 32)
     assert got2 == fx["tokens"]
+    # and so does the form with ONE launch per layer (attention phase, device-wide barrier, MLP phase)
+    del rt2
+    cfg3 = DecoderConfig(**DENSE_4B, bits=4, capacity=128, embed_scale=fx["embed_scale"], xcd_layer_launch=True)
+    got3, _, _ = DecoderRuntime(cfg3, W).generate(fx["prompt"], 32)
+    assert got3 == fx["tokens"]
 
 
 def test_bench_command_prints_the_reference_lines(fk, tmp_path, capsys):

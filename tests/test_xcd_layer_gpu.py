@@ -458,6 +458,37 @@ def test_artifact_round_trip_of_a_two_launch_layer_model(fk, tmp_path):
 
 
 @pytest.mark.parametrize("bits", [4, 16])
+def test_one_launch_per_layer_gives_the_same_tokens(fk, bits):
+    """DecoderConfig.xcd_layer_launch: the dispatcher fuses each attention launch with the MLP launch behind it
+    (attention phase, device-wide barrier, MLP phase; both argument blocks by value) where both take their one-pass
+    flavour (the 4-bit model here; the bf16 one keeps its two launches).  Same tokens as the separate launches, same
+    graph node list for the caller, and a rebinding of a member's buffer reaches the fused launch."""
+    from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
+    kw = dict(n_layers=3, hidden=1024, n_heads=32, n_kv=8, head_dim=128, inter=2048, vocab=3000, capacity=128, qk_norm=True, bits=bits)
+    W = DecoderWeights.random_init(DecoderConfig(**kw), seed=5)
+    prompt = [11, 2222, 333, 4]
+    want, _, _ = DecoderRuntime(DecoderConfig(**kw), W).generate(prompt, 24)
+    rt = DecoderRuntime(DecoderConfig(**kw, xcd_layer_launch=True), W)
+    assert rt.xcd
+    got, _, _ = rt.generate(prompt, 24)
+    assert got == want
+    new_k, new_v = fk.zeros(rt.cache_k[1].nbytes), fk.zeros(rt.cache_v[1].nbytes)
+    ups = []
+    for i, t in enumerate(rt.tasks):
+        for s_, (p, n) in enumerate(t.args):
+            if p == rt.cache_k[1].ptr:
+                ups.append((i, s_, new_k.ptr, n))
+            if p == rt.cache_v[1].ptr:
+                ups.append((i, s_, new_v.ptr, n))
+    assert len(ups) == 2
+    rt.d.update_graph_bindings(rt.graph, ups)
+    old = rt.cache_k[1].to_numpy(np.uint16).copy()
+    got2, _, _ = rt.generate(prompt, 24)
+    assert got2 == want
+    assert np.array_equal(rt.cache_k[1].to_numpy(np.uint16), old) and new_k.to_numpy(np.uint16).any()
+
+
+@pytest.mark.parametrize("bits", [4, 16])
 def test_one_launch_per_token_gives_the_same_tokens(fk, bits):
     """DecoderConfig.xcd_token_launch: the 2 x n_layers launches of a token fused by the dispatcher into ONE launch
     (device-wide barriers where the separate launches have kernel boundaries, per-layer argument blocks in device
