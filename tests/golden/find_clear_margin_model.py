@@ -45,7 +45,7 @@ import numpy as np  # noqa: E402
 
 import oracle  # noqa: E402
 from fusekit_amd.decoder import DENSE_4B, DecoderConfig  # noqa: E402  (a plain dataclass: no GPU needed)
-from helpers import HostDecoderWeights, OracleDecoder, rng  # noqa: E402
+from helpers import HostDecoderWeights, OracleDecoder, loud_rows_equal, rng  # noqa: E402
 
 N_PROMPT, N_GEN = 32, 32
 
@@ -70,6 +70,9 @@ def main():
     ap.add_argument("--grid", nargs="+", default=["0:0.02"], help="tau:embed_scale pairs")
     ap.add_argument("--loud-rows", type=int, default=0, help="token ids 0 .. N-1 get the row gain instead of the spread")
     ap.add_argument("--loud-gain", type=float, default=1.0)
+    ap.add_argument("--loud-equal", action="store_true",
+                    help="the loud rows all get the gain (a power of two; applied on the host, helpers.loud_rows_equal) "
+                         "instead of the generator's gain * 2^-j")
     ap.add_argument("--seeds", type=int, default=8, help="embedding seeds tried per (tau, scale)")
     ap.add_argument("--first-seed", type=int, default=1000)
     ap.add_argument("--safety", type=float, default=3.0)
@@ -96,12 +99,17 @@ def main():
         if True:
             for es in range(args.first_seed, args.first_seed + args.seeds):
                 cfg.embed_scale = scale
-                W.set_embedding(es, tau, args.loud_rows, args.loud_gain)
+                if args.loud_equal:
+                    W.set_embedding(es, tau, 0, 1.0)
+                    loud_rows_equal(W, args.loud_rows, args.loud_gain)
+                else:
+                    W.set_embedding(es, tau, args.loud_rows, args.loud_gain)
                 oracle.set_accum_mode(0)
                 t0 = time.time()
                 toks, margins, lg0 = run(cfg, W, prompt, want_logits=True)
                 distinct = len(set(toks))
                 rec = dict(tau=tau, embed_scale=scale, embed_seed=es, loud_rows=args.loud_rows, loud_gain=args.loud_gain,
+                           loud_equal=bool(args.loud_equal),
                            tokens=toks, distinct=distinct,
                            min_margin=float(min(margins)), margins=[float(m) for m in margins])
                 line = "tau %.2f scale %.3g seed %d: distinct %d, min margin %.4g, %.0f s" % (

@@ -103,6 +103,17 @@ class HostDecoderWeights:
                               loud_rows=loud_rows, loud_gain=loud_gain).reshape(c.vocab, c.hidden))
 
 
+def loud_rows_equal(host_weights, rows: int, gain: float) -> np.ndarray:
+    """Multiplies the first `rows` rows of a host model's (bf16, tied) embedding by `gain`, a power of two so that
+    the product is exact: equally loud rows, where the generator's own loud rows halve from row to row.  Returns
+    the changed rows (bf16 bits, [rows, hidden]) for the upload into the device model."""
+    assert gain > 0 and float(np.log2(gain)).is_integer()
+    emb = host_weights.mats["embed_tokens"]
+    w = np.asarray(emb.w).reshape(emb.n, emb.k)
+    w[:rows] = oracle.f32_to_bf16((oracle.bf16_to_f32(w[:rows]) * np.float32(gain)).astype(np.float32))
+    return w[:rows].copy()
+
+
 def host_weight(dw) -> oracle.QWeight:
     """Download a fusekit_amd DeviceWeight into an oracle QWeight (host weights pass through)."""
     if isinstance(dw, oracle.QWeight):
