@@ -29,6 +29,7 @@ namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kWideMaxRows = 10;             // activation rows (the reference's upper bound for this path)
 constexpr uint32_t kWideSlab = 256;               // k per wave and step
@@ -275,8 +276,233 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide_kernel(const QgemmWid
     FK_WIDE_STAMP(6);
 }
 
+
+// ---- up to 8 rows: 16 x 16 x 32 tiles ---------------------------------------------------------------------------
+// v_mfma_f32_16x16x32_bf16: lane (c = lane % 16, kq = lane / 16) supplies 8 values of k block kq for row / column c
+// and holds C[4 * kq + r][c].  A quantisation group is 64 codes = two k blocks of 32, so one instruction would mix
+// two groups; instead the A operand carries every activation row TWICE -- row m with only the k blocks 0, 1, row
+// m + 8 with only the k blocks 2, 3 -- and one instruction yields the integer dots of two groups side by side:
+// lanes kq 0, 1 hold the even group's dots of rows 0..7, lanes kq 2, 3 the odd group's.  A lane therefore folds
+// exactly the group whose codes it loaded (one scale / bias pair per lane and double group), and the two halves
+// meet once at the end.  Against the 32 x 32 x 16 form: no padding rows beyond 8 of 16 (there 22 of 32), four
+// accumulator registers per tile instead of sixteen, a fold of 4 values instead of 8 x 2.
+// A block still owns 32 weight rows (two tiles of 16) over all of K, its waves split K in slabs of 256.
+template <WKind KIND, int MATS, int WAVES>
+__global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmWideArgs a) {
+    constexpr uint32_t VPL = KIND == W_Q4 ? 32u : 16u;  // codes per 16-byte lane load
+    constexpr int MF = VPL / 8;                         // matrix instructions per load
+    constexpr int LU = 32 / VPL;                        // loads per lane, tile and double group
+    constexpr int DGS = kWideSlab / 128u;               // double groups per slab
+    constexpr int UNITS = kWideSlab / 64u;
+    extern __shared__ uint4 lds_raw[];
+    const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t c16 = lane & 15u, kq = lane >> 4, gsel = kq >> 1, hf = kq & 1u;
+    uint4* xs = reinterpret_cast<uint4*>(reinterpret_cast<char*>(lds_raw) + wave * wide_wave_lds());
+    float* sxs = reinterpret_cast<float*>(xs + kWideXRows * kWideXS);
+    float* meet = reinterpret_cast<float*>(reinterpret_cast<char*>(lds_raw) + WAVES * wide_wave_lds());
+
+    const uint32_t M = a.M;
+    const uint32_t n_slabs = (a.K + kWideSlab - 1) / kWideSlab;
+    for (uint32_t i = lane; i < kWideXS; i += kWave) xs[kWideMaxRows * kWideXS + i] = make_uint4(0, 0, 0, 0);
+    for (uint32_t i = lane; i < UNITS * 32u; i += kWave) sxs[i] = 0.f;
+    // A operand row c16: activation row c16 % 8, live only in the k blocks of group half c16 / 8
+    const uint32_t am = c16 & 7u;
+    const uint32_t arow = (am < M && (c16 >> 3) == gsel) ? am : kWideMaxRows;
+
+    const uint4* wrow[MATS][2];
+    const uint16_t *srow[MATS][2], *brow[MATS][2];
+#pragma unroll
+    for (int q = 0; q < MATS; ++q)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t n = blockIdx.x * 32u + (uint32_t)h * 16u + c16, nc = n < a.N ? n : a.N - 1;
+            wrow[q][h] = a.w[q] + (size_t)nc * a.cpr;
+            srow[q][h] = a.sc[q] + (size_t)nc * a.gpr;
+            brow[q][h] = a.bi[q] + (size_t)nc * a.gpr;
+        }
+
+    f32x4_t acc[MATS][2];
+#pragma unroll
+    for (int q = 0; q < MATS; ++q)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) acc[q][h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    struct Slab {
+        uint4 w[MATS][2][DGS * LU], x[kWideXPT];
+        uint32_t sb[MATS][2][DGS];
+    };
+    // code offset inside a slab of this lane's load u of double group d
+    auto k_of = [&](int d, int u) { return (uint32_t)d * 128u + gsel * 64u + (hf + 2u * (uint32_t)u) * VPL; };
+    auto fetch = [&](uint32_t slab, Slab& B) {
+        const bool live = slab < n_slabs;
+        const uint32_t ks0 = live ? slab * kWideSlab : 0u;
+        const uint32_t slab_k = a.K - ks0 < kWideSlab ? a.K - ks0 : kWideSlab;
+        const uint32_t s8 = live ? slab_k >> 3 : 0u;
+#pragma unroll
+        for (int q = 0; q < MATS; ++q)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int d = 0; d < DGS; ++d) {
+#pragma unroll
+                    for (int u = 0; u < LU; ++u) {
+                        const bool have = live && k_of(d, u) < slab_k;   // K is whole groups: a group is inside or outside
+                        B.w[q][h][d * LU + u] = (have ? wrow[q][h] : a.w[q])[have ? (ks0 + k_of(d, u)) / VPL : 0u];
+                    }
+                    const uint32_t gl = 2u * (uint32_t)d + gsel;
+                    const bool have = live && gl * 64u < slab_k;
+                    const uint32_t g = have ? (ks0 >> 6) + gl : 0u;
+                    B.sb[q][h][d] = (uint32_t)(have ? srow[q][h] : a.sc[q])[g] | ((uint32_t)(have ? brow[q][h] : a.bi[q])[g] << 16);
+                }
+            }
+#pragma unroll
+        for (int i = 0; i < kWideXPT; ++i) {
+            const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
+            const bool have = m < M && k8 < s8;
+            B.x[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(have ? m : 0u) * a.K + ks0 + (have ? k8 : 0u) * 8u);
+        }
+    };
+    auto consume = [&](uint32_t slab, const Slab& B) {
+        const uint32_t ks0 = slab * kWideSlab;
+        const uint32_t slab_k = a.K - ks0 < kWideSlab ? a.K - ks0 : kWideSlab;
+#pragma unroll
+        for (int i = 0; i < kWideXPT; ++i) {
+            const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
+            uint4 v = (m < M && k8 < (slab_k >> 3)) ? B.x[i] : make_uint4(0, 0, 0, 0);
+            if constexpr (KIND == W_Q4) {
+                v = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
+                               (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
+            }
+            if (m < kWideMaxRows) xs[m * kWideXS + k8] = v;
+        }
+        __builtin_amdgcn_wave_barrier();
+        {
+            const uint32_t g = lane >> 4, m = lane & 15u;
+            if (m < M) {
+                float s0 = 0.f, s1 = 0.f;
+                if (g < (slab_k >> 6)) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 8; ++i) {
+                        const uint4 v = xs[m * kWideXS + g * 8u + i];
+                        s0 = dot2_bf16(v.x, 0x3F803F80u, s0);
+                        s1 = dot2_bf16(v.y, 0x3F803F80u, s1);
+                        s0 = dot2_bf16(v.z, 0x3F803F80u, s0);
+                        s1 = dot2_bf16(v.w, 0x3F803F80u, s1);
+                    }
+                }
+                sxs[g * 32u + m] = s0 + s1;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 0; d < DGS; ++d) {
+            if ((uint32_t)d * 128u < slab_k) {  // wave-uniform; a lane whose group lies past the slab multiplies zeros
+                f32x4_t c[MATS][2];
+#pragma unroll
+                for (int u = 0; u < LU; ++u) {
+                    const uint4* xa = xs + arow * kWideXS + (k_of(d, u) >> 3);
+#pragma unroll
+                    for (int j = 0; j < MF; ++j) {
+                        const uint4 av = xa[j];
+#pragma unroll
+                        for (int q = 0; q < MATS; ++q)
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                const uint4 wv = B.w[q][h][d * LU + u];
+                                const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+                                uint4 bw;
+                                if constexpr (KIND == W_Q4) {
+                                    const uint32_t even = wd[j] & 0x0F0F0F0Fu, odd = (wd[j] >> 4) & 0x0F0F0F0Fu;
+                                    bw.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, false));
+                                    bw.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(even, 512.0f, true));
+                                    bw.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, false));
+                                    bw.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(odd, 512.0f, true));
+                                } else {
+                                    const uint32_t w0 = wd[(2 * j) & 3], w1 = wd[(2 * j + 1) & 3];
+                                    auto pair = [](float lo, float hi) {
+                                        const bf16x2_t p = {(__bf16)lo, (__bf16)hi};  // integers <= 255 are exact in bf16
+                                        return __builtin_bit_cast(uint32_t, p);
+                                    };
+                                    bw.x = pair((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu));
+                                    bw.y = pair((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24));
+                                    bw.z = pair((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu));
+                                    bw.w = pair((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24));
+                                }
+                                const bool first = u * MF + j == 0;
+                                c[q][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                                 __builtin_bit_cast(bf16x8_t, bw),
+                                                                                 first ? zero : c[q][h], 0, 0, 0);
+                            }
+                    }
+                }
+                // fold this lane's group (2 d + gsel): C register r is activation row 4 * hf + r
+                const float4 sx = *reinterpret_cast<const float4*>(sxs + (2u * (uint32_t)d + gsel) * 32u + 4u * hf);
+#pragma unroll
+                for (int q = 0; q < MATS; ++q)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const uint32_t sb = B.sb[q][h][d];
+                        const float sf = bf16_bits_to_f32(sb & 0xffffu), bf = bf16_bits_to_f32(sb >> 16);
+                        acc[q][h][0] += fmaf(sf, c[q][h][0], bf * sx.x);
+                        acc[q][h][1] += fmaf(sf, c[q][h][1], bf * sx.y);
+                        acc[q][h][2] += fmaf(sf, c[q][h][2], bf * sx.z);
+                        acc[q][h][3] += fmaf(sf, c[q][h][3], bf * sx.w);
+                    }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    Slab A, B;
+    fetch(wave, A);
+    for (uint32_t slab = wave; slab < n_slabs; slab += 2 * WAVES) {
+        fetch(slab + WAVES, B);
+        consume(slab, A);
+        fetch(slab + 2 * WAVES, A);
+        if (slab + WAVES < n_slabs) consume(slab + WAVES, B);
+    }
+
+    // the two group halves of a row meet (lane ^ 32), then the waves as in the 32 x 32 form
+#pragma unroll
+    for (int q = 0; q < MATS; ++q)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = acc[q][h][r] + __shfl_xor(acc[q][h][r], 32);
+                const uint32_t m = 4u * hf + (uint32_t)r;
+                if (gsel == 0 && m < M) meet[((wave * MATS + q) * kWideMaxRows + m) * 32u + (uint32_t)h * 16u + c16] = v;
+            }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < M * 32u; e += WAVES * kWave) {
+        const uint32_t m = e >> 5, col = e & 31u, nn = blockIdx.x * 32u + col;
+        if (nn >= a.N) continue;
+        float s[MATS];
+#pragma unroll
+        for (int q = 0; q < MATS; ++q) {
+            s[q] = 0.f;
+            for (int w = 0; w < WAVES; ++w) s[q] += meet[((w * MATS + q) * kWideMaxRows + m) * 32u + col];
+        }
+        uint32_t o;
+        if constexpr (MATS == 2) {
+            o = swiglu_bits(s[0], s[1], a.variant, 1.0f);
+        } else {
+            float v = s[0];
+            if (a.bias) v += bf16_bits_to_f32(a.bias[nn]);
+            if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * a.N + nn]);
+            o = f32_to_bf16_bits(v);
+        }
+        a.y[(size_t)m * a.N + nn] = (uint16_t)o;
+    }
+}
+
 template <WKind KIND, int MATS>
-const void* wide_func(uint32_t waves) {
+const void* wide_func(uint32_t waves, bool tiles16) {
+    if (tiles16)
+        return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 8>)
+                          : reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 4>);
     return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide_kernel<KIND, MATS, 8>)
                       : reinterpret_cast<const void*>(&qgemm_wide_kernel<KIND, MATS, 4>);
 }
@@ -284,6 +510,7 @@ const void* wide_func(uint32_t waves) {
 }  // namespace
 
 static bool g_wide_on = true;
+static const bool g_wide_tiles16 = true;   // 9728 x 2560 int4, 8 rows: 13.86 us with 32 x 32 x 16 tiles, 12.51 with 16 x 16 x 32
 void set_qgemm_wide(bool on) { g_wide_on = on; }
 bool qgemm_takes_wide(uint32_t M, uint32_t group) { return g_wide_on && M >= 2 && M <= kWideMaxRows && group == 64; }
 
@@ -316,8 +543,9 @@ fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16
     const uint32_t blocks = (W0->n + 31u) / 32u, n_slabs = (W0->k + kWideSlab - 1) / kWideSlab;
     const uint32_t waves = (blocks <= (uint32_t)dev->cus && n_slabs >= 5u) ? 8u : 4u;
     const bool q4 = W0->bits == 4;
-    out->func = W1 ? (q4 ? wide_func<W_Q4, 2>(waves) : wide_func<W_Q8, 2>(waves))
-                   : (q4 ? wide_func<W_Q4, 1>(waves) : wide_func<W_Q8, 1>(waves));
+    const bool t16 = g_wide_tiles16 && M <= 8;   // up to 8 rows: the 16 x 16 x 32 tiling
+    out->func = W1 ? (q4 ? wide_func<W_Q4, 2>(waves, t16) : wide_func<W_Q8, 2>(waves, t16))
+                   : (q4 ? wide_func<W_Q4, 1>(waves, t16) : wide_func<W_Q8, 1>(waves, t16));
     out->grid = dim3(blocks, 1, 1);
     out->block = dim3(waves * kWave, 1, 1);
     out->shmem = wide_lds_bytes(waves, W1 ? 2u : 1u);

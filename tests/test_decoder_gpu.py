@@ -397,9 +397,11 @@ def test_4b_class_512_tokens_at_full_size_follow_the_oracle(fk):
                                    min_in_two_ulps=0.99)
 
 
-def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk):
-    """Plain free-running equality at full size: prompt of 32 tokens, 32 greedy tokens, no teacher forcing, no
-    window, no candidate sets -- `got == expected`.
+@pytest.mark.parametrize("bits,fixture", [(4, "clear_margin_4b.json"), (8, "clear_margin_4b_q8.json"),
+                                          (16, "clear_margin_4b_bf16.json")])
+def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk, bits, fixture):
+    """Plain free-running equality at full size, for 4-bit, 8-bit and bf16 weights: prompt of 32 tokens, 32 greedy
+    tokens, no teacher forcing, no window, no candidate sets -- `got == expected`.
 
     Random-init weights make the logits near-uniform, and no two arithmetics agree across a step whose two best
     logits are a bf16 ulp apart.  tests/golden/find_clear_margin_model.py therefore searched, on the CPU with
@@ -412,9 +414,10 @@ def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk)
     import json
     from fusekit_amd.decoder import DENSE_4B, DecoderConfig, DecoderRuntime, DecoderWeights
     from helpers import HostDecoderWeights
-    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "clear_margin_4b.json")))
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", fixture)))
     assert fx["n_layers"] == DENSE_4B["n_layers"] and len(fx["prompt"]) == 32 and len(fx["tokens"]) == 32
-    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=128, embed_scale=fx["embed_scale"])
+    assert fx.get("bits", 4) == bits and len(set(fx["tokens"])) >= 4 and not fx.get("loud_equal", False)
+    cfg = DecoderConfig(**DENSE_4B, bits=bits, capacity=128, embed_scale=fx["embed_scale"])
     W = DecoderWeights.random_init(cfg, seed=fx["model_seed"], std=fx["std"], exact=True, embed_seed=fx["embed_seed"],
                                    embed_tau=fx["tau"], embed_loud_rows=fx["loud_rows"], embed_loud_gain=fx["loud_gain"])
     # the same model as the fixture's: the host generator's bytes against what sits in HBM
@@ -424,6 +427,9 @@ def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk)
     assert np.array_equal(emb_dev.w.to_numpy(np.uint16), np.asarray(H.mats["embed_tokens"].w).reshape(-1))
     for name in ("layers.0.self_attn.q_proj", "layers.35.mlp.down_proj"):
         d, h = W.mats[name], H.mats[name]
+        if bits == 16:
+            assert np.array_equal(d.w.to_numpy(np.uint16), np.asarray(h.w).reshape(-1))
+            continue
         assert np.array_equal(d.w.to_numpy(np.uint32), np.asarray(h.w).reshape(-1).view(np.uint32))
         assert np.array_equal(d.scales.to_numpy(np.uint16), np.asarray(h.scales).reshape(-1))
         assert np.array_equal(d.biases.to_numpy(np.uint16), np.asarray(h.biases).reshape(-1))
@@ -431,17 +437,17 @@ def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk)
     assert rt.xcd, "the headline model runs on the two-launch layer path"
     got, _, _ = rt.generate(fx["prompt"], 32)
     print("tokens:", got)
-    print("oracle margins (bf16 ulps of the top logit), min %.1f; margin / fp32 envelope, min %.2f" %
-          (fx["min_margin_ulps"], fx["min_ratio"]))
+    print("%d distinct tokens; oracle margins (bf16 ulps of the top logit), min %.1f; margin / fp32 envelope, min %.2f" %
+          (len(set(fx["tokens"])), fx["min_margin_ulps"], fx["min_ratio"]))
     assert got == fx["tokens"]
     # the per-dispatch task list (five launches per layer) decides the same 32 tokens
-    cfg2 = DecoderConfig(**DENSE_4B, bits=4, capacity=128, embed_scale=fx["embed_scale"], xcd_layers=False)
+    cfg2 = DecoderConfig(**DENSE_4B, bits=bits, capacity=128, embed_scale=fx["embed_scale"], xcd_layers=False)
     rt2 = DecoderRuntime(cfg2, W)
     got2, _, _ = rt2.generate(fx["prompt"], 32)
     assert got2 == fx["tokens"]
     # and so does the form with ONE launch per layer (attention phase, device-wide barrier, MLP phase)
     del rt2
-    cfg3 = DecoderConfig(**DENSE_4B, bits=4, capacity=128, embed_scale=fx["embed_scale"], xcd_layer_launch=True)
+    cfg3 = DecoderConfig(**DENSE_4B, bits=bits, capacity=128, embed_scale=fx["embed_scale"], xcd_layer_launch=True)
     got3, _, _ = DecoderRuntime(cfg3, W).generate(fx["prompt"], 32)
     assert got3 == fx["tokens"]
 
