@@ -287,7 +287,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide_kernel(const QgemmWid
 // meet once at the end.  Against the 32 x 32 x 16 form: no padding rows beyond 8 of 16 (there 22 of 32), four
 // accumulator registers per tile instead of sixteen, a fold of 4 values instead of 8 x 2.
 // A block still owns 32 weight rows (two tiles of 16) over all of K, its waves split K in slabs of 256.
-template <WKind KIND, int MATS, int WAVES>
+template <WKind KIND, int MATS, int WAVES, int TILES>
 __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmWideArgs a) {
     constexpr uint32_t VPL = KIND == W_Q4 ? 32u : 16u;  // codes per 16-byte lane load
     constexpr int MF = VPL / 8;                         // matrix instructions per load
@@ -309,27 +309,27 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
     const uint32_t am = c16 & 7u;
     const uint32_t arow = (am < M && (c16 >> 3) == gsel) ? am : kWideMaxRows;
 
-    const uint4* wrow[MATS][2];
-    const uint16_t *srow[MATS][2], *brow[MATS][2];
+    const uint4* wrow[MATS][TILES];
+    const uint16_t *srow[MATS][TILES], *brow[MATS][TILES];
 #pragma unroll
     for (int q = 0; q < MATS; ++q)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const uint32_t n = blockIdx.x * 32u + (uint32_t)h * 16u + c16, nc = n < a.N ? n : a.N - 1;
+        for (int h = 0; h < TILES; ++h) {
+            const uint32_t n = blockIdx.x * (16u * TILES) + (uint32_t)h * 16u + c16, nc = n < a.N ? n : a.N - 1;
             wrow[q][h] = a.w[q] + (size_t)nc * a.cpr;
             srow[q][h] = a.sc[q] + (size_t)nc * a.gpr;
             brow[q][h] = a.bi[q] + (size_t)nc * a.gpr;
         }
 
-    f32x4_t acc[MATS][2];
+    f32x4_t acc[MATS][TILES];
 #pragma unroll
     for (int q = 0; q < MATS; ++q)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) acc[q][h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int h = 0; h < TILES; ++h) acc[q][h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     struct Slab {
-        uint4 w[MATS][2][DGS * LU], x[kWideXPT];
-        uint32_t sb[MATS][2][DGS];
+        uint4 w[MATS][TILES][DGS * LU], x[kWideXPT];
+        uint32_t sb[MATS][TILES][DGS];
     };
     // code offset inside a slab of this lane's load u of double group d
     auto k_of = [&](int d, int u) { return (uint32_t)d * 128u + gsel * 64u + (hf + 2u * (uint32_t)u) * VPL; };
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 #pragma unroll
         for (int q = 0; q < MATS; ++q)
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < TILES; ++h) {
 #pragma unroll
                 for (int d = 0; d < DGS; ++d) {
 #pragma unroll
@@ -399,7 +399,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 #pragma unroll
         for (int d = 0; d < DGS; ++d) {
             if ((uint32_t)d * 128u < slab_k) {  // wave-uniform; a lane whose group lies past the slab multiplies zeros
-                f32x4_t c[MATS][2];
+                f32x4_t c[MATS][TILES];
 #pragma unroll
                 for (int u = 0; u < LU; ++u) {
                     const uint4* xa = xs + arow * kWideXS + (k_of(d, u) >> 3);
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 #pragma unroll
                         for (int q = 0; q < MATS; ++q)
 #pragma unroll
-                            for (int h = 0; h < 2; ++h) {
+                            for (int h = 0; h < TILES; ++h) {
                                 const uint4 wv = B.w[q][h][d * LU + u];
                                 const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
                                 uint4 bw;
@@ -442,7 +442,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 #pragma unroll
                 for (int q = 0; q < MATS; ++q)
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) {
+                    for (int h = 0; h < TILES; ++h) {
                         const uint32_t sb = B.sb[q][h][d];
                         const float sf = bf16_bits_to_f32(sb & 0xffffu), bf = bf16_bits_to_f32(sb >> 16);
                         acc[q][h][0] += fmaf(sf, c[q][h][0], bf * sx.x);
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 #pragma unroll
     for (int q = 0; q < MATS; ++q)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < TILES; ++h)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float v = acc[q][h][r] + __shfl_xor(acc[q][h][r], 32);
@@ -476,8 +476,9 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
                 if (gsel == 0 && m < M) meet[((wave * MATS + q) * kWideMaxRows + m) * 32u + (uint32_t)h * 16u + c16] = v;
             }
     __syncthreads();
-    for (uint32_t e = threadIdx.x; e < M * 32u; e += WAVES * kWave) {
-        const uint32_t m = e >> 5, col = e & 31u, nn = blockIdx.x * 32u + col;
+    constexpr uint32_t COLS = 16u * TILES;
+    for (uint32_t e = threadIdx.x; e < M * COLS; e += WAVES * kWave) {
+        const uint32_t m = e / COLS, col = e % COLS, nn = blockIdx.x * COLS + col;
         if (nn >= a.N) continue;
         float s[MATS];
 #pragma unroll
@@ -499,10 +500,13 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 }
 
 template <WKind KIND, int MATS>
-const void* wide_func(uint32_t waves, bool tiles16) {
+const void* wide_func(uint32_t waves, bool tiles16, bool one_tile) {
+    if (tiles16 && one_tile)
+        return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 8, 1>)
+                          : reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 4, 1>);
     if (tiles16)
-        return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 8>)
-                          : reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 4>);
+        return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 8, 2>)
+                          : reinterpret_cast<const void*>(&qgemm_wide16_kernel<KIND, MATS, 4, 2>);
     return waves == 8 ? reinterpret_cast<const void*>(&qgemm_wide_kernel<KIND, MATS, 8>)
                       : reinterpret_cast<const void*>(&qgemm_wide_kernel<KIND, MATS, 4>);
 }
@@ -535,17 +539,24 @@ fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16
     a.gpr = W0->k / 64u;
     a.variant = variant;
     // Eight waves per block (K split eight ways) while every block still finds a CU of its own; four beyond
-    // (registers allow one eight-wave block per CU).  Measured, 8 rows of int4, serialised graph, against the
-    // split-k kernel + reduction: 6144 x 2560 8.5 us (15.6), 2560 x 4096 11.2 (18.4), 2048 x 1408 5.8 (10.2),
-    // 1408 x 2048 6.9 (11.4), 9728 x 2560 14.0 (16.3), 2560 x 9728 21.0 (21.7): per 16-byte chunk the kernel spends
-    // ~150 vector instructions and four matrix instructions (three quarters of whose rows are padding), so the
-    // 14 MB matrices are bound by that, not by the stream.
-    const uint32_t blocks = (W0->n + 31u) / 32u, n_slabs = (W0->k + kWideSlab - 1) / kWideSlab;
-    const uint32_t waves = (blocks <= (uint32_t)dev->cus && n_slabs >= 5u) ? 8u : 4u;
-    const bool q4 = W0->bits == 4;
+    // (registers allow one eight-wave block per CU).  Measured with the 32 x 32 x 16 form, 8 rows of int4, serialised
+    // graph, against the split-k kernel + reduction: 6144 x 2560 8.5 us (15.6), 2560 x 4096 11.2 (18.4),
+    // 2048 x 1408 5.8 (10.2), 1408 x 2048 6.9 (11.4), 9728 x 2560 14.0 (16.3), 2560 x 9728 21.0 (21.7).
     const bool t16 = g_wide_tiles16 && M <= 8;   // up to 8 rows: the 16 x 16 x 32 tiling
-    out->func = W1 ? (q4 ? wide_func<W_Q4, 2>(waves, t16) : wide_func<W_Q8, 2>(waves, t16))
-                   : (q4 ? wide_func<W_Q4, 1>(waves, t16) : wide_func<W_Q8, 1>(waves, t16));
+    // The 16-row form may give a block ONE tile: twice the blocks, each wave half the arithmetic per slab.  What these
+    // launches lack is waves to hide their LDS round trips behind, not bandwidth, so the smaller block wins wherever
+    // the grid is short (8 rows of int4, one / two tiles: 2048 x 2048 5.8 / 7.7 us, 3072 x 2048 6.0 / 7.7,
+    // 2560 x 9728 13.3 / 18.8, 9728 x 2560 11.8 / 12.6) and loses where the two-tile grid already fills the chip or
+    // the eight-wave form would be lost (6144 x 2560 9.6 / 8.1, 19456 x 2560 17.3 / 16.3, 77824 x 2560 54 / 46).
+    const uint32_t n_slabs = (W0->k + kWideSlab - 1) / kWideSlab, b16 = (W0->n + 15u) / 16u, b32 = (W0->n + 31u) / 32u;
+    const uint32_t cus = (uint32_t)dev->cus;
+    const bool deep = n_slabs >= 5u;
+    const bool one_tile = t16 && ((deep && b16 <= cus) || (!(deep && b32 <= cus) && b16 <= 3u * cus));
+    const uint32_t blocks = one_tile ? b16 : b32;
+    const uint32_t waves = (blocks <= cus && deep) ? 8u : 4u;
+    const bool q4 = W0->bits == 4;
+    out->func = W1 ? (q4 ? wide_func<W_Q4, 2>(waves, t16, one_tile) : wide_func<W_Q8, 2>(waves, t16, one_tile))
+                   : (q4 ? wide_func<W_Q4, 1>(waves, t16, one_tile) : wide_func<W_Q8, 1>(waves, t16, one_tile));
     out->grid = dim3(blocks, 1, 1);
     out->block = dim3(waves * kWave, 1, 1);
     out->shmem = wide_lds_bytes(waves, W1 ? 2u : 1u);
