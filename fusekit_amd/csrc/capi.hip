@@ -258,6 +258,18 @@ fk_status fk_rmsnorm_qkv(const uint16_t* x, const uint16_t* norm_w, float eps, c
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_rmsnorm_qkv_rows(const uint16_t* x, uint32_t rows, uint32_t x_row_stride, const uint16_t* norm_w, float eps,
+                              const fk_weight* Wq, const fk_weight* Wk, const fk_weight* Wv, uint16_t* q,
+                              uint32_t q_row_stride, uint16_t* k, uint32_t k_row_stride, uint16_t* v, uint32_t v_row_stride,
+                              fk_stream s) {
+    if (!Wq) return set_error(FK_ERR_INVALID, "fk_rmsnorm_qkv_rows: null Wq");
+    if (!Wk && Wv) return set_error(FK_ERR_INVALID, "fk_rmsnorm_qkv_rows: Wv without Wk");
+    WideSeg segs[3] = {{Wq, q, q_row_stride}, {Wk, k, k_row_stride}, {Wv, v, v_row_stride}};
+    Launch l;
+    FK_TRY(plan_qgemm_wide_fan(x, x_row_stride, rows, norm_w, eps, segs, Wv ? 3u : (Wk ? 2u : 1u), &l));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_gateup_swiglu(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* Wg,
                            const fk_weight* Wu, int variant, uint16_t* out, fk_stream s) {
     if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, "fk_gateup_swiglu: variant must be 0, 1 or 2");

@@ -171,6 +171,30 @@ fk_status plan_qkv(const Dispatch& d, Launch* l, SlotRW* rw) {
         rq.y[m] = arg_ptr<uint16_t>(d, out_slot + m);
     }
     rq.n_mats = 3;
+    const uint32_t rows = d.u("rows", 1);
+    if (rows > 1) {
+        // Row form (2 .. 8 token rows, the prefill_mN variants' and the multi-row passes' shape): x [rows, x_row_stride],
+        // outputs [rows, q / k / v_row_stride] (defaults: dense rows), one shared-stream launch for the three matrices
+        // with the norm applied while the rows are staged.
+        if (has_bias) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": the row form takes no bias");
+        const uint32_t xs = d.u("x_row_stride", hidden);
+        const uint32_t ys[3] = {d.u("q_row_stride", n_q), d.u("k_row_stride", n_kv), d.u("v_row_stride", n_kv)};
+        if (xs < hidden) return set_error(FK_ERR_INVALID, d.kernel + ": x_row_stride below hidden");
+        FK_TRY(need_bytes(d, 0, ((size_t)(rows - 1) * xs + hidden) * 2));
+        WideSeg segs[3];
+        for (int m = 0; m < 3; ++m) {
+            if (ys[m] < ns[m]) return set_error(FK_ERR_INVALID, d.kernel + ": output row stride below the matrix's rows");
+            FK_TRY(need_bytes(d, out_slot + m, ((size_t)(rows - 1) * ys[m] + ns[m]) * 2));
+            segs[m] = WideSeg{&W[m], arg_ptr<uint16_t>(d, out_slot + m), ys[m]};
+        }
+        const uint16_t* nw = nullptr;
+        if (has_norm) {
+            FK_TRY(need_bytes(d, norm_slot, (size_t)hidden * 2));
+            nw = arg_ptr<const uint16_t>(d, norm_slot);
+        }
+        all_but_last(s, 3, rw);
+        return plan_qgemm_wide_fan(arg_ptr<const uint16_t>(d, 0), xs, rows, nw, (float)d.param("eps", 1e-6), segs, 3, l);
+    }
     FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
     rq.x = arg_ptr<const uint16_t>(d, 0);
     if (has_norm) {

@@ -172,6 +172,13 @@ bool qgemm_takes_library(uint32_t m);
 // run_launch and the graph builder skip.
 bool qgemm_takes_wide(uint32_t M, uint32_t group);
 void set_qgemm_wide(bool on);
+struct WideSeg {
+    const fk_weight* W;
+    uint16_t* y;
+    uint32_t y_stride;   // elements between the rows of y
+};
+fk_status plan_qgemm_wide_fan(const uint16_t* x, uint32_t x_stride, uint32_t M, const uint16_t* norm_w, float eps,
+                              const WideSeg* segs, uint32_t n_seg, Launch* out);
 fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16_t* x, uint32_t M, const uint16_t* bias,
                           const uint16_t* res, int variant, uint16_t* y, Launch* out);
 bool gemm_library_available();

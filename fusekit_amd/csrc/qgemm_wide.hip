@@ -38,23 +38,31 @@ constexpr uint32_t kWideXRows = kWideMaxRows + 1; // staged rows + the zero row
 constexpr int kWideXPT = kWideMaxRows * (kWideSlab / 8) / kWave;  // 16-byte pieces of x per lane and slab
 
 struct QgemmWideArgs {
-    const uint4* w[2];
-    const uint16_t* sc[2];
-    const uint16_t* bi[2];
-    const uint16_t* x;     // [M, K] bf16
+    const uint4* w[3];     // the matrix, the gate / up pair, or up to three matrices served side by side (segments)
+    const uint16_t* sc[3];
+    const uint16_t* bi[3];
+    const uint16_t* x;     // [M, x_stride] bf16
     const uint16_t* bias;  // [N] or null (single matrix)
     const uint16_t* res;   // [M, N] or null (single matrix)
     uint16_t* y;           // [M, N]
     uint32_t M, N, K;
     uint32_t cpr, gpr;
     int variant;           // SwiGLU rounding variant (pair)
+    // 16-row form with one matrix per block: segment s owns blocks [blk0[s], blk0[s + 1]) and writes ys[s] with its own
+    // row stride; norm_w: the activations are RMS-normalised as they are staged, T(w * T(x * r)) per element
+    uint32_t n_seg, x_stride;
+    uint32_t ns[3], blk0[3], y_stride[3];
+    uint16_t* ys[3];
+    const uint16_t* norm_w;
+    float eps;
 };
 
 // LDS per wave: staged activations [kWideXRows][kWideXS] uint4, group sums [4][32] floats; per block
 // additionally the waves' results [waves][mats][kWideMaxRows][32] floats.
 __host__ __device__ constexpr uint32_t wide_wave_lds() { return kWideXRows * kWideXS * 16u + 4u * 32u * 4u; }
+__host__ __device__ constexpr uint32_t wide_meet_bytes(uint32_t waves, uint32_t mats) { return waves * mats * kWideMaxRows * 32u * 4u; }
 __host__ __device__ constexpr uint32_t wide_lds_bytes(uint32_t waves, uint32_t mats) {
-    return waves * wide_wave_lds() + waves * mats * kWideMaxRows * 32u * 4u;
+    return waves * wide_wave_lds() + wide_meet_bytes(waves, mats) + 64u;   // + one 1/rms per activation row
 }
 
 template <WKind KIND, int MATS, int WAVES>
@@ -120,7 +128,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide_kernel(const QgemmWid
         for (int i = 0; i < kWideXPT; ++i) {
             const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
             const bool have = m < M && k8 < s8;
-            B.x[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(have ? m : 0u) * a.K + ks0 + (have ? k8 : 0u) * 8u);
+            B.x[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(have ? m : 0u) * a.x_stride + ks0 + (have ? k8 : 0u) * 8u);
         }
     };
     auto consume = [&](uint32_t slab, const Slab& B) {
@@ -301,8 +309,47 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
     float* sxs = reinterpret_cast<float*>(xs + kWideXRows * kWideXS);
     float* meet = reinterpret_cast<float*>(reinterpret_cast<char*>(lds_raw) + WAVES * wide_wave_lds());
 
+    float* rrs = reinterpret_cast<float*>(reinterpret_cast<char*>(meet) + wide_meet_bytes(WAVES, MATS));  // [rows] 1 / rms
+
     const uint32_t M = a.M;
     const uint32_t n_slabs = (a.K + kWideSlab - 1) / kWideSlab;
+    // one matrix per block: which of the (up to three) matrices this block serves
+    uint32_t seg = 0, blk = blockIdx.x;
+    if constexpr (MATS == 1) {
+        if (a.n_seg > 1 && blockIdx.x >= a.blk0[1]) seg = 1;
+        if (a.n_seg > 2 && blockIdx.x >= a.blk0[2]) seg = 2;
+        blk = blockIdx.x - a.blk0[seg];
+    }
+    const uint32_t N = MATS == 1 ? a.ns[seg] : a.N;
+    const uint4* wb[MATS];
+    const uint16_t *scb[MATS], *bib[MATS];
+#pragma unroll
+    for (int q = 0; q < MATS; ++q) {
+        wb[q] = a.w[MATS == 1 ? seg : (uint32_t)q];
+        scb[q] = a.sc[MATS == 1 ? seg : (uint32_t)q];
+        bib[q] = a.bi[MATS == 1 ? seg : (uint32_t)q];
+    }
+    const bool normed = a.norm_w != nullptr;
+    if (normed) {
+        // 1 / rms of every activation row: wave w takes rows w, w + WAVES, ...
+        for (uint32_t m = wave; m < M; m += WAVES) {
+            const uint4* xr = reinterpret_cast<const uint4*>(a.x + (size_t)m * a.x_stride);
+            float ss = 0.f;
+            for (uint32_t i = lane; i < (a.K >> 3); i += kWave) {
+                const uint4 v = xr[i];
+                const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const float lo = bf16_lo(wd[t]), hi = bf16_hi(wd[t]);
+                    ss = fmaf(lo, lo, ss);
+                    ss = fmaf(hi, hi, ss);
+                }
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) rrs[m] = 1.0f / sqrtf(ss / (float)a.K + a.eps);
+        }
+        __syncthreads();
+    }
     for (uint32_t i = lane; i < kWideXS; i += kWave) xs[kWideMaxRows * kWideXS + i] = make_uint4(0, 0, 0, 0);
     for (uint32_t i = lane; i < UNITS * 32u; i += kWave) sxs[i] = 0.f;
     // A operand row c16: activation row c16 % 8, live only in the k blocks of group half c16 / 8
@@ -315,10 +362,10 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
     for (int q = 0; q < MATS; ++q)
 #pragma unroll
         for (int h = 0; h < TILES; ++h) {
-            const uint32_t n = blockIdx.x * (16u * TILES) + (uint32_t)h * 16u + c16, nc = n < a.N ? n : a.N - 1;
-            wrow[q][h] = a.w[q] + (size_t)nc * a.cpr;
-            srow[q][h] = a.sc[q] + (size_t)nc * a.gpr;
-            brow[q][h] = a.bi[q] + (size_t)nc * a.gpr;
+            const uint32_t n = blk * (16u * TILES) + (uint32_t)h * 16u + c16, nc = n < N ? n : N - 1;
+            wrow[q][h] = wb[q] + (size_t)nc * a.cpr;
+            srow[q][h] = scb[q] + (size_t)nc * a.gpr;
+            brow[q][h] = bib[q] + (size_t)nc * a.gpr;
         }
 
     f32x4_t acc[MATS][TILES];
@@ -328,7 +375,7 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
         for (int h = 0; h < TILES; ++h) acc[q][h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     struct Slab {
-        uint4 w[MATS][TILES][DGS * LU], x[kWideXPT];
+        uint4 w[MATS][TILES][DGS * LU], x[kWideXPT], nw;
         uint32_t sb[MATS][TILES][DGS];
     };
     // code offset inside a slab of this lane's load u of double group d
@@ -347,19 +394,25 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
 #pragma unroll
                     for (int u = 0; u < LU; ++u) {
                         const bool have = live && k_of(d, u) < slab_k;   // K is whole groups: a group is inside or outside
-                        B.w[q][h][d * LU + u] = (have ? wrow[q][h] : a.w[q])[have ? (ks0 + k_of(d, u)) / VPL : 0u];
+                        B.w[q][h][d * LU + u] = (have ? wrow[q][h] : wb[q])[have ? (ks0 + k_of(d, u)) / VPL : 0u];
                     }
                     const uint32_t gl = 2u * (uint32_t)d + gsel;
                     const bool have = live && gl * 64u < slab_k;
                     const uint32_t g = have ? (ks0 >> 6) + gl : 0u;
-                    B.sb[q][h][d] = (uint32_t)(have ? srow[q][h] : a.sc[q])[g] | ((uint32_t)(have ? brow[q][h] : a.bi[q])[g] << 16);
+                    B.sb[q][h][d] = (uint32_t)(have ? srow[q][h] : scb[q])[g] | ((uint32_t)(have ? brow[q][h] : bib[q])[g] << 16);
                 }
             }
 #pragma unroll
         for (int i = 0; i < kWideXPT; ++i) {
             const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
             const bool have = m < M && k8 < s8;
-            B.x[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(have ? m : 0u) * a.K + ks0 + (have ? k8 : 0u) * 8u);
+            B.x[i] = *reinterpret_cast<const uint4*>(a.x + (size_t)(have ? m : 0u) * a.x_stride + ks0 + (have ? k8 : 0u) * 8u);
+        }
+        // the norm weights of this lane's pieces: k8 = lane % 32 for every one of them (straight-line: without a norm
+        // the request reads the activations' first bytes)
+        {
+            const uint32_t k8 = lane & (kWideSlab / 8 - 1);
+            B.nw = *reinterpret_cast<const uint4*>((normed ? a.norm_w : a.x) + (normed ? ks0 + (k8 < s8 ? k8 : 0u) * 8u : 0u));
         }
     };
     auto consume = [&](uint32_t slab, const Slab& B) {
@@ -369,6 +422,17 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
         for (int i = 0; i < kWideXPT; ++i) {
             const uint32_t idx = lane + (uint32_t)i * kWave, m = idx / (kWideSlab / 8), k8 = idx % (kWideSlab / 8);
             uint4 v = (m < M && k8 < (slab_k >> 3)) ? B.x[i] : make_uint4(0, 0, 0, 0);
+            if (normed) {  // block-uniform
+                const float r = rrs[m < M ? m : 0u];
+                const uint32_t xv[4] = {v.x, v.y, v.z, v.w}, wv[4] = {B.nw.x, B.nw.y, B.nw.z, B.nw.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint32_t xr2 = pack_bf16(bf16_lo(xv[t]) * r, bf16_hi(xv[t]) * r);   // T(x * r)
+                    o[t] = pack_bf16(bf16_lo(wv[t]) * bf16_lo(xr2), bf16_hi(wv[t]) * bf16_hi(xr2));  // T(w * .)
+                }
+                v = make_uint4(o[0], o[1], o[2], o[3]);
+            }
             if constexpr (KIND == W_Q4) {
                 v = make_uint4((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16),
                                (v.x >> 16) | (v.y & 0xffff0000u), (v.z >> 16) | (v.w & 0xffff0000u));
@@ -477,9 +541,11 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
             }
     __syncthreads();
     constexpr uint32_t COLS = 16u * TILES;
+    uint16_t* yo = MATS == 1 ? a.ys[seg] : a.y;
+    const uint32_t yst = MATS == 1 ? a.y_stride[seg] : a.N;
     for (uint32_t e = threadIdx.x; e < M * COLS; e += WAVES * kWave) {
-        const uint32_t m = e / COLS, col = e % COLS, nn = blockIdx.x * COLS + col;
-        if (nn >= a.N) continue;
+        const uint32_t m = e / COLS, col = e % COLS, nn = blk * COLS + col;
+        if (nn >= N) continue;
         float s[MATS];
 #pragma unroll
         for (int q = 0; q < MATS; ++q) {
@@ -492,10 +558,10 @@ __global__ __launch_bounds__(WAVES* kWave) void qgemm_wide16_kernel(const QgemmW
         } else {
             float v = s[0];
             if (a.bias) v += bf16_bits_to_f32(a.bias[nn]);
-            if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * a.N + nn]);
+            if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * N + nn]);
             o = f32_to_bf16_bits(v);
         }
-        a.y[(size_t)m * a.N + nn] = (uint16_t)o;
+        yo[(size_t)m * yst + nn] = (uint16_t)o;
     }
 }
 
@@ -535,6 +601,8 @@ fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16
     }
     a.x = x; a.bias = bias; a.res = res; a.y = y;
     a.M = M; a.N = W0->n; a.K = W0->k;
+    a.n_seg = 1; a.x_stride = W0->k;
+    a.ns[0] = W0->n; a.blk0[0] = 0; a.y_stride[0] = W0->n; a.ys[0] = y;
     a.cpr = W0->k / (W0->bits == 4 ? 32u : 16u);
     a.gpr = W0->k / 64u;
     a.variant = variant;
@@ -560,6 +628,62 @@ fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16
     out->grid = dim3(blocks, 1, 1);
     out->block = dim3(waves * kWave, 1, 1);
     out->shmem = wide_lds_bytes(waves, W1 ? 2u : 1u);
+    out->set_args(a);
+    if (out->shmem > 48 * 1024)
+        FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)out->shmem));
+    return FK_OK;
+}
+
+// Up to three matrices over the same activations in ONE launch of the 16-row form (2 .. 8 rows), each with its own
+// output and row stride; with norm_w the rows are RMS-normalised while they are staged.  The row form of the
+// RMSNorm -> Q, K, V fan-out (src/codegen/kernels/rmsnorm_qkv.rs:53-736 with active_m > 1).
+fk_status plan_qgemm_wide_fan(const uint16_t* x, uint32_t x_stride, uint32_t M, const uint16_t* norm_w, float eps,
+                              const WideSeg* segs, uint32_t n_seg, Launch* out) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    if (!x || !segs || n_seg == 0 || n_seg > 3) return set_error(FK_ERR_INVALID, "qgemm fan-out: one to three matrices");
+    const fk_weight* W0 = segs[0].W;
+    if (!W0) return set_error(FK_ERR_INVALID, "qgemm fan-out: null weight");
+    if (!g_wide_on || M < 2 || M > 8 || W0->group != 64 || (W0->bits != 4 && W0->bits != 8))
+        return set_error(FK_ERR_UNSUPPORTED, "qgemm fan-out: 2..8 rows, 4- or 8-bit weights, group size 64");
+    if (W0->k % 64u || x_stride < W0->k || x_stride % 8u || ((uintptr_t)x & 15u) || (norm_w && ((uintptr_t)norm_w & 15u)))
+        return set_error(FK_ERR_INVALID, "qgemm fan-out: K must be whole groups, rows and norm weights 16-byte aligned");
+    QgemmWideArgs a;
+    memset(&a, 0, sizeof(a));
+    uint32_t b16 = 0, b32 = 0;
+    for (uint32_t i = 0; i < n_seg; ++i) {
+        const fk_weight* W = segs[i].W;
+        if (!W || !W->w || !W->scales || !W->biases || !segs[i].y) return set_error(FK_ERR_INVALID, "qgemm fan-out: null matrix or output");
+        if (W->k != W0->k || W->bits != W0->bits || W->group != W0->group || W->n == 0)
+            return set_error(FK_ERR_INVALID, "qgemm fan-out: the matrices must share K, bits and group size");
+        if (segs[i].y_stride < W->n) return set_error(FK_ERR_INVALID, "qgemm fan-out: output row stride below the matrix's rows");
+        a.w[i] = reinterpret_cast<const uint4*>(W->w);
+        a.sc[i] = W->scales;
+        a.bi[i] = W->biases;
+        a.ns[i] = W->n;
+        a.ys[i] = segs[i].y;
+        a.y_stride[i] = segs[i].y_stride;
+        b16 += (W->n + 15u) / 16u;
+        b32 += (W->n + 31u) / 32u;
+    }
+    a.x = x; a.M = M; a.N = W0->n; a.K = W0->k;
+    a.cpr = W0->k / (W0->bits == 4 ? 32u : 16u);
+    a.gpr = W0->k / 64u;
+    a.n_seg = n_seg; a.x_stride = x_stride;
+    a.norm_w = norm_w; a.eps = eps;
+    const uint32_t n_slabs = (W0->k + kWideSlab - 1) / kWideSlab, cus = (uint32_t)dev->cus;
+    const bool deep = n_slabs >= 5u;
+    const bool one_tile = (deep && b16 <= cus) || (!(deep && b32 <= cus) && b16 <= 3u * cus);   // as plan_qgemm_wide
+    uint32_t blocks = 0;
+    for (uint32_t i = 0; i < n_seg; ++i) {
+        a.blk0[i] = blocks;
+        blocks += one_tile ? (a.ns[i] + 15u) / 16u : (a.ns[i] + 31u) / 32u;
+    }
+    const uint32_t waves = (blocks <= cus && deep) ? 8u : 4u;
+    out->func = W0->bits == 4 ? wide_func<W_Q4, 1>(waves, true, one_tile) : wide_func<W_Q8, 1>(waves, true, one_tile);
+    out->grid = dim3(blocks, 1, 1);
+    out->block = dim3(waves * kWave, 1, 1);
+    out->shmem = wide_lds_bytes(waves, 1u);
     out->set_args(a);
     if (out->shmem > 48 * 1024)
         FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)out->shmem));

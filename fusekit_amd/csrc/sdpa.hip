@@ -117,7 +117,9 @@ fk_status plan_sdpa_decode(const uint16_t* q, const uint16_t* k, const uint16_t*
     // the final merge, which costs one memory round trip per 16 partials, stays short.
     // Measured (32 q / 8 kv heads x 128): 4096 positions are fastest with 32 splits,
     // 32768 with 64.
-    const uint32_t tiles = n_kv * ((G + gt - 1) / gt);
+    // (several active rows multiply the tiles: each row then needs fewer ranges to fill the chip; 8 rows x 16 heads at
+    // a capacity of 1024 ran 16 ranges per row and head -- 2048 blocks, most of them past the context -- in 14.4 us)
+    const uint32_t tiles = n_kv * ((G + gt - 1) / gt) * rows;
     uint32_t want = (n_chunks > 128 ? 2u : 1u) * (uint32_t)dev->cus / tiles;
     if (want < 1) want = 1;
     if (want > 256) want = 256;

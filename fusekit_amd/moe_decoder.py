@@ -447,6 +447,10 @@ class MoeRowsVariant:
         self.xn = B(m * c.hidden * 2)
         self.q, self.lat, self.kpe, self.latn = B(m * n_q * 2), B(m * c.kv_lora_rank * 2), B(m * c.rope_dim * 2), B(m * c.kv_lora_rank * 2)
         self.kvb, self.att = B(m * n_b * 2), B(m * c.n_heads * c.v_dim * 2)
+        # 2..8 rows: RMSNorm + q / kv_a, and RMSNorm(latent) + kv_b, are ONE launch each (the row form of the
+        # rmsnorm_qkv family); kv_a's output rows are [latent | k_pe], as in the single-token list
+        self.fan = 2 <= m <= 8 and c.bits in (4, 8) and c.group == 64
+        self.kva = B(m * (c.kv_lora_rank + c.rope_dim) * 2)
         self.mid = B(m * max(c.dense_inter, c.shared_inter) * 2)
         routes = m * c.top_k
         self.ridx, self.rwt = z(4 * routes * c.n_layers), z(2 * routes * c.n_layers)
@@ -487,6 +491,17 @@ class MoeRowsVariant:
         def norm_rows(x, nw, hidden, out):
             t.append(Dispatch(name("rmsnorm_rows"), [arg(x), arg(nw), arg(out)], dict(rows=m, hidden=hidden, eps=c.eps)))
 
+        def fan3(x, x_stride, norm_w, hidden, parts, outs):
+            """RMSNorm + three row blocks of projections of the m rows in one launch (row form of rmsnorm_qkv);
+            outs: (buffer, first column, row stride in elements) per block."""
+            (w0, s0, b0), (w1, s1, b1), (w2, s2, b2) = (pt[0] for pt in parts)
+            n0, n1 = parts[0][1], parts[1][1]
+            assert parts[2][1] == n1
+            o = [arg(buf, ((m - 1) * st + n) * 2, col * 2) for (buf, col, st), n in zip(outs, (n0, n1, n1))]
+            t.append(Dispatch(name("rmsnorm_qkv"), [x, arg(norm_w), w0, w1, w2, s0, s1, s2, b0, b1, b2] + o,
+                              dict(quant, hidden=hidden, n_q=n0, n_kv=n1, eps=c.eps, has_norm=1, has_bias=0, rows=m,
+                                   x_row_stride=x_stride, q_row_stride=outs[0][2], k_row_stride=outs[1][2], v_row_stride=outs[2][2])))
+
         def swiglu(Wg, Wu, inter):
             t.append(Dispatch(name("qgemm_swiglu"),
                               [arg(self.xn), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases),
@@ -501,19 +516,31 @@ class MoeRowsVariant:
         for l in range(c.n_layers):
             p = f"layers.{l}."
             Wq, Wa, Wb, Wo = (w.mats[p + f"self_attn.{n}"] for n in ("q_proj", "kv_a_proj_with_mqa", "kv_b_proj", "o_proj"))
-            norm_rows(self.x[0], w.vecs[p + "input_layernorm"], c.hidden, self.xn)
-            matmul(self.xn, full(Wq), c.hidden, n_q, self.q)
-            matmul(self.xn, _rows(Wa, 0, c.kv_lora_rank), c.hidden, c.kv_lora_rank, self.lat)
-            matmul(self.xn, _rows(Wa, c.kv_lora_rank, n_a), c.hidden, c.rope_dim, self.kpe)
-            norm_rows(self.lat, w.vecs[p + "self_attn.kv_a_layernorm"], c.kv_lora_rank, self.latn)
-            matmul(self.latn, full(Wb), c.kv_lora_rank, n_b, self.kvb)
+            if self.fan:
+                half_a = n_a // 2
+                fan3(arg(self.x[0]), c.hidden, w.vecs[p + "input_layernorm"], c.hidden,
+                     [(_rows(Wq, 0, n_q), n_q), (_rows(Wa, 0, half_a), half_a), (_rows(Wa, half_a, n_a), half_a)],
+                     [(self.q, 0, n_q), (self.kva, 0, n_a), (self.kva, half_a, n_a)])
+                fan3(arg(self.kva, ((m - 1) * n_a + c.kv_lora_rank) * 2, 0), n_a, w.vecs[p + "self_attn.kv_a_layernorm"], c.kv_lora_rank,
+                     [(_rows(Wb, 0, n_b // 2), n_b // 2), (_rows(Wb, n_b // 2, 3 * n_b // 4), n_b // 4),
+                      (_rows(Wb, 3 * n_b // 4, n_b), n_b // 4)],
+                     [(self.kvb, 0, n_b), (self.kvb, n_b // 2, n_b), (self.kvb, 3 * n_b // 4, n_b)])
+                kpe, kpe_stride = arg(self.kva, ((m - 1) * n_a + c.rope_dim) * 2, c.kv_lora_rank * 2), n_a
+            else:
+                norm_rows(self.x[0], w.vecs[p + "input_layernorm"], c.hidden, self.xn)
+                matmul(self.xn, full(Wq), c.hidden, n_q, self.q)
+                matmul(self.xn, _rows(Wa, 0, c.kv_lora_rank), c.hidden, c.kv_lora_rank, self.lat)
+                matmul(self.xn, _rows(Wa, c.kv_lora_rank, n_a), c.hidden, c.rope_dim, self.kpe)
+                norm_rows(self.lat, w.vecs[p + "self_attn.kv_a_layernorm"], c.kv_lora_rank, self.latn)
+                matmul(self.latn, full(Wb), c.kv_lora_rank, n_b, self.kvb)
+                kpe, kpe_stride = arg(self.kpe), c.rope_dim
             t.append(Dispatch(name("kv_cache_store_decode"),
-                              [arg(self.q), arg(self.kvb), arg(self.kpe), arg(self.kvb, self.kvb.nbytes - c.nope_dim * 2, c.nope_dim * 2),
+                              [arg(self.q), arg(self.kvb), kpe, arg(self.kvb, self.kvb.nbytes - c.nope_dim * 2, c.nope_dim * 2),
                                arg(rt.cache_k[l]), arg(rt.cache_v[l]), arg(self.offset), arg(self.offset)],
                               dict(split_k=1, has_q=1, n_heads=c.n_heads, q0_dim=c.nope_dim, q1_dim=c.rope_dim, n_kv=c.n_heads,
                                    k0_dim=c.nope_dim, k1_dim=c.rope_dim, v_dim=c.v_dim, k1_n_kv=1, k0_stride=packed, v_stride=packed,
                                    rope_dims=c.rope_dim, traditional=int(c.rope_traditional), theta=c.theta, capacity=c.capacity,
-                                   rows=m, k0_row_stride=n_b, k1_row_stride=c.rope_dim, v_row_stride=n_b)))
+                                   rows=m, k0_row_stride=n_b, k1_row_stride=kpe_stride, v_row_stride=n_b)))
             t.append(Dispatch(name("sdpa_decode"),
                               [arg(self.q), arg(rt.cache_k[l]), arg(rt.cache_v[l]), arg(self.kv_len), arg(self.att), arg(self.parts),
                                arg(self.counters)],

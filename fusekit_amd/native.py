@@ -191,6 +191,16 @@ def rmsnorm_qkv(x, norm_w, eps, Wq, Wk, Wv, bq, bk, bv, q, k, v, stream=None) ->
                              _ptr(bq), _ptr(bk), _ptr(bv), _ptr(q), _ptr(k), _ptr(v), _ptr(stream)))
 
 
+def rmsnorm_qkv_rows(x, rows, x_row_stride, norm_w, eps, Wq, Wk, Wv, q, q_row_stride, k=None, k_row_stride=0, v=None,
+                     v_row_stride=0, stream=None) -> None:
+    """fk_rmsnorm_qkv_rows: RMSNorm + one to three projections of 2..8 token rows in one launch."""
+    wk = C.byref(Wk.c) if Wk is not None else None
+    wv = C.byref(Wv.c) if Wv is not None else None
+    check(lib.fk_rmsnorm_qkv_rows(_ptr(x), C.c_uint32(rows), C.c_uint32(x_row_stride), _ptr(norm_w), C.c_float(eps),
+                                  C.byref(Wq.c), wk, wv, _ptr(q), C.c_uint32(q_row_stride), _ptr(k), C.c_uint32(k_row_stride),
+                                  _ptr(v), C.c_uint32(v_row_stride), _ptr(stream)))
+
+
 def gateup_swiglu(x, norm_w, eps, Wg, Wu, variant, out, stream=None) -> None:
     check(lib.fk_gateup_swiglu(_ptr(x), _ptr(norm_w), C.c_float(eps), C.byref(Wg.c), C.byref(Wu.c),
                                C.c_int(variant), _ptr(out), _ptr(stream)))

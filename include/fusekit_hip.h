@@ -153,6 +153,17 @@ fk_status fk_rmsnorm_qkv(const uint16_t *x, const uint16_t *norm_w, float eps, c
                          const fk_weight *Wk, const fk_weight *Wv, const uint16_t *bq, const uint16_t *bk,
                          const uint16_t *bv, uint16_t *q, uint16_t *k, uint16_t *v, fk_stream s);
 
+/* K2 for 2..8 token rows (the reference compiles the same emitter with active_m = N for its prefill_mN variants,
+ *     src/commands/patch.rs:112-150, src/codegen/kernels/rmsnorm_qkv.rs:53-736): x [rows, x_row_stride], outputs
+ *     [rows, *_row_stride]; ONE launch streams the one to three matrices once for all rows (Wk, Wv may be NULL from
+ *     the end; 4- or 8-bit, group 64, no bias) and applies the norm while the rows are staged (norm_w NULL: none).
+ *     Row strides let the outputs be column blocks of a wider row.  Dispatch family fusekit_rmsnorm_qkv with the
+ *     parameter rows (and x_row_stride, q_ / k_ / v_row_stride). */
+fk_status fk_rmsnorm_qkv_rows(const uint16_t *x, uint32_t rows, uint32_t x_row_stride, const uint16_t *norm_w, float eps,
+                              const fk_weight *Wq, const fk_weight *Wk, const fk_weight *Wv, uint16_t *q,
+                              uint32_t q_row_stride, uint16_t *k, uint32_t k_row_stride, uint16_t *v, uint32_t v_row_stride,
+                              fk_stream s);
+
 /* K3a (RMSNorm ->) gate/up projections -> SwiGLU.  variant 0: every op in T
  *     (src/codegen/kernels/rmsnorm_gateup_swiglu.rs:236-257); 1: fp32 sigmoid,
  *     one round (src/codegen/msl.rs:1286-1294); 2: rounded sigmoid and gate

@@ -110,6 +110,39 @@ def test_shared_stream_gate_up_swiglu(fk, m, hidden, inter, bits, variant):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,hidden,ns,normed", [(8, 2048, (3072, 288, 288), True), (5, 512, (2048, 1024, 1024), True),
+                                                (2, 896, (333, 64, None), False), (8, 2560, (4096, None, None), True)])
+def test_norm_and_fan_out_of_several_rows_in_one_launch(fk, bits, m, hidden, ns, normed):
+    """fk_rmsnorm_qkv_rows: 2..8 token rows, RMSNorm applied while the rows are staged, one to three matrices served by
+    one launch, inputs and outputs with row strides (column blocks of wider rows).  Every row equals the oracle's
+    RMSNorm followed by its single-row projection (to rounding-edge flips), and the launch equals the separate
+    rmsnorm_rows + fk_qgemm launches to the same bar; what lies between the column blocks is not touched."""
+    Ws = [make_qweight(700 + i + bits, n, hidden, bits) if n else None for i, n in enumerate(ns)]
+    xs_, pad = hidden + 64, 40                       # activations are the first `hidden` columns of wider rows
+    xw = normal_bf16(710 + m, (m, xs_))
+    nw = normal_bf16(711, hidden, 0.1, 1.0) if normed else None
+    outs = [fk.DeviceBuffer.from_numpy(np.full((m, n + pad), 0xAAAA, np.uint16)) if n else None for n in ns]
+    dW = [to_device(fk, W) if W is not None else None for W in Ws]
+    fk.rmsnorm_qkv_rows(_dev(fk, xw), m, xs_, _dev(fk, nw), 1e-6, dW[0], dW[1], dW[2],
+                        outs[0], ns[0] + pad, outs[1], (ns[1] or 0) + pad, outs[2], (ns[2] or 0) + pad)
+    fk.sync()
+    x = np.ascontiguousarray(xw[:, :hidden])
+    xn = np.stack([oracle.rmsnorm(x[r], nw, 1e-6) for r in range(m)]) if normed else x
+    for W, o, n in zip(Ws, outs, ns):
+        if W is None:
+            continue
+        got = o.to_numpy(np.uint16, (m, n + pad))
+        assert (got[:, n:] == 0xAAAA).all()
+        sep = _run(fk, W, xn)                         # the separate launches on the oracle's normalised rows
+        for r in range(m):
+            _check(got[r, :n], oracle.qgemv(W, xn[r], None), oracle.linear_acc(W, xn[r]), W, xn[r])
+            _check(got[r, :n], sep[r], oracle.bf16_to_f32(sep[r]), W, xn[r])
+    with pytest.raises(fk.FusekitError):               # nine rows take the plain matmul
+        fk.rmsnorm_qkv_rows(_dev(fk, normal_bf16(1, (9, xs_))), 9, xs_, _dev(fk, nw), 1e-6, dW[0], None, None,
+                            fk.DeviceBuffer(2 * 9 * (ns[0] + pad)), ns[0] + pad)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("m", [9, 100])
 def test_qgemm_group_128(fk, bits, m):
     W = make_qweight(60, 384, 1024, bits, group=128)
