@@ -20,15 +20,19 @@ The winner is written to clear_margin_4b.json (parameters, prompt, the 32 expect
 fp32 envelope per step); tests/test_decoder_gpu.py builds the same model in HBM from the same seeds and
 asserts plain free-running equality.  Runs only the oracle: no GPU, no reference code.
 
-The committed fixture came from
+The committed fixtures came from
 
-    python tests/golden/find_clear_margin_model.py --grid 0:0.004 --loud-rows 12 --loud-gain 256 \
-        --first-seed 3007 --seeds 1 --safety 2 --min-distinct 3
+    python tests/golden/find_clear_margin_model.py --bits 4  --grid 0:0.004 --loud-rows 12 --loud-gain 256 \
+        --first-seed SEED4 --seeds 1 --safety 2 --min-distinct 4          # clear_margin_4b.json
+    python tests/golden/find_clear_margin_model.py --bits 8  ... --first-seed 5511 --seeds 1 ...   # clear_margin_4b_q8.json
+    python tests/golden/find_clear_margin_model.py --bits 16 ... --first-seed 5600 --seeds 1 ...   # clear_margin_4b_bf16.json
 
-after a sweep over --grid 0:0.002 0:0.004 0:0.006 0:0.02 and seeds 3000..3007 (about a minute per candidate on
-8 cores; most candidates hold at least one near-tie among their 32 steps and are skipped).  The 8-bit and bf16
-fixtures (clear_margin_4b_q8.json, clear_margin_4b_bf16.json: configs[3] names both variants) come from the same
-command with --bits 8 / --bits 16 --min-distinct 4 over seeds 3000..; the seed each one took is in its file.
+(configs[3] names the 4-bit, 8-bit and bf16 variants; the seed each fixture took is in its file).  About one candidate
+in fifteen passes -- most hold at least one near-tie among their 32 steps -- and a candidate costs one to three minutes
+on 8 cores, so the seeds tried were ranked beforehand with the library itself: the GPU decoder ran thousands of seeds
+through the two-launch and the five-launch task lists and sorted them by the smallest ratio of a logit gap to what the
+other list changes it by.  That ranking only chose WHICH seeds this script examined; every number in a fixture is the
+CPU oracle's, and the commands above reproduce the files without a GPU.
 """
 import argparse
 import json
