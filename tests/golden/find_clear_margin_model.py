@@ -23,7 +23,7 @@ asserts plain free-running equality.  Runs only the oracle: no GPU, no reference
 The committed fixtures came from
 
     python tests/golden/find_clear_margin_model.py --bits 4  --grid 0:0.004 --loud-rows 12 --loud-gain 256 \
-        --first-seed SEED4 --seeds 1 --safety 2 --min-distinct 4          # clear_margin_4b.json
+        --first-seed 6328 --seeds 1 --safety 2 --min-distinct 4          # clear_margin_4b.json
     python tests/golden/find_clear_margin_model.py --bits 8  ... --first-seed 5511 --seeds 1 ...   # clear_margin_4b_q8.json
     python tests/golden/find_clear_margin_model.py --bits 16 ... --first-seed 5600 --seeds 1 ...   # clear_margin_4b_bf16.json
 

@@ -397,9 +397,8 @@ def test_4b_class_512_tokens_at_full_size_follow_the_oracle(fk):
                                    min_in_two_ulps=0.99)
 
 
-@pytest.mark.parametrize("bits,fixture", [(b, f) for b, f in ((4, "clear_margin_4b.json"), (8, "clear_margin_4b_q8.json"),
-                                                              (16, "clear_margin_4b_bf16.json"))
-                                          if os.path.exists(os.path.join(os.path.dirname(__file__), "golden", f))])
+@pytest.mark.parametrize("bits,fixture", [(4, "clear_margin_4b.json"), (8, "clear_margin_4b_q8.json"),
+                                          (16, "clear_margin_4b_bf16.json")])
 def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk, bits, fixture):
     """Plain free-running equality at full size, for 4-bit, 8-bit and bf16 weights: prompt of 32 tokens, 32 greedy
     tokens, no teacher forcing, no window, no candidate sets -- `got == expected`.
@@ -417,7 +416,7 @@ def test_4b_class_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk,
     from helpers import HostDecoderWeights
     fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", fixture)))
     assert fx["n_layers"] == DENSE_4B["n_layers"] and len(fx["prompt"]) == 32 and len(fx["tokens"]) == 32
-    assert fx.get("bits", 4) == bits and len(set(fx["tokens"])) >= 3 and not fx.get("loud_equal", False)
+    assert fx.get("bits", 4) == bits and len(set(fx["tokens"])) >= 4 and not fx.get("loud_equal", False)
     cfg = DecoderConfig(**DENSE_4B, bits=bits, capacity=128, embed_scale=fx["embed_scale"])
     W = DecoderWeights.random_init(cfg, seed=fx["model_seed"], std=fx["std"], exact=True, embed_seed=fx["embed_seed"],
                                    embed_tau=fx["tau"], embed_loud_rows=fx["loud_rows"], embed_loud_gain=fx["loud_gain"])

@@ -8,16 +8,13 @@ import pytest
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
-DENSE = [(n, b) for n, b in (("clear_margin_4b.json", 4), ("clear_margin_4b_q8.json", 8), ("clear_margin_4b_bf16.json", 16))
-         if os.path.exists(os.path.join(GOLDEN, n))]
-
-
-@pytest.mark.parametrize("name,bits", DENSE)
+@pytest.mark.parametrize("name,bits", [("clear_margin_4b.json", 4), ("clear_margin_4b_q8.json", 8),
+                                       ("clear_margin_4b_bf16.json", 16)])
 def test_dense_fixture_decides_every_token_clearly(name, bits):
     fx = json.load(open(os.path.join(GOLDEN, name)))
     assert fx.get("bits", 4) == bits and fx["n_layers"] == 36
     assert len(fx["prompt"]) == 32 and len(fx["tokens"]) == 32 and len(fx["margins"]) == 32 and len(fx["envelope"]) == 32
-    assert len(set(fx["tokens"])) == fx["distinct"] >= 3          # a continuation that moves
+    assert len(set(fx["tokens"])) == fx["distinct"] >= 4          # a continuation that moves
     assert fx["fp32_orders_agree"] is True                        # both fp32 summation orders pick these tokens
     assert fx["min_ratio"] >= fx["safety"] >= 2.0                 # every gap >= safety x what the orders change it by
     assert fx["min_margin_ulps"] >= 3.0
