@@ -70,7 +70,9 @@ def test_qgemm_matches_oracle(fk, m, n, k, bits):
 # a ragged N, few weight rows with a long K (16 waves per block), bias and residual, and the split-k route on the
 # same operands (both keep the single-row arithmetic: rounding-edge flips only).
 WIDE_SHAPES = [(2, 2560, 2560), (3, 6144, 2560), (4, 333, 1408), (5, 2560, 9728), (6, 2048, 1408), (7, 1408, 2048),
-               (8, 9728, 2560), (9, 70, 4096), (10, 2560, 4096)]
+               (8, 9728, 2560), (9, 70, 4096), (10, 2560, 4096),
+               # K of one, three and five groups (a slab's second double group partly or wholly past the end), few rows
+               (8, 48, 64), (3, 100, 192), (2, 17, 320), (8, 40000, 512)]
 
 
 @pytest.mark.parametrize("bits", [4, 8])
