@@ -768,6 +768,7 @@ fk_status plan_xcd_attn_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
     rw->writes = {(uint32_t)x_slot, (uint32_t)q_slot, (uint32_t)q_slot + 1, (uint32_t)q_slot + 2, (uint32_t)ck_slot,
                   (uint32_t)cv_slot, (uint32_t)ap_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
+    rq.for_token = d.u("token", 0) != 0;
     return plan_xcd_attn(rq, l);
 }
 

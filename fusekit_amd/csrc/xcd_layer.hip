@@ -304,9 +304,14 @@ template <int NL>
 struct TileRegs {
     uint4 w[NL];
 };
-constexpr int kMetaRegs = 3;  // quantisation groups of a tile per thread: tiles of at most 768 groups per matrix
+constexpr int kMetaRegs = 3;  // one-pass flavour: a tile holds at most 3 * 256 = 768 quantisation groups per matrix
+// The flavour with the pass loop serves larger tiles (an 8B-class int4 gate / up tile is 28 rows x 64 groups): there a
+// thread fetches a second run of four groups, 2048 per tile and matrix.
+constexpr uint32_t kMetaWords = kMetaRegs * 256u, kMetaWordsBig = 8u * 256u;
+template <bool ONE>
+constexpr uint32_t meta_words() { return ONE ? kMetaWords : kMetaWordsBig; }
 struct MetaRegs {
-    uint32_t s[kMetaRegs], b[kMetaRegs];
+    uint32_t s[4], b[4];   // [0..1]: groups 4 ti .. 4 ti + 3; [2..3] (BIG): groups 4 (ti + SN) .. + 3
 };
 
 struct Tile {
@@ -362,7 +367,7 @@ __device__ __forceinline__ void tile_load(const MAT& m, const Tile& t, const Til
 // RUN: the tile's groups are one contiguous, 8-byte aligned run of a multiple of four entries of the scale and of
 // the bias array (the host plans it so): a tile of whole rows, or a K-slice tile of a matrix whose scales and
 // biases were re-laid out per XCD (fk_xcd_kslice_meta: [xcd][row][groups of the slice]; `xcd` then selects the copy).
-template <WKind KIND, int SN, bool RUN, typename MAT>
+template <WKind KIND, int SN, bool RUN, bool BIG = false, typename MAT>
 __device__ __forceinline__ void meta_fetch(const MAT& m, const Tile& t, uint32_t ti, MetaRegs& r, uint32_t xcd = 0) {
     if constexpr (KIND != W_BF16) {
         const uint32_t gpr = t.cs >> m.gshift, total = t.rows * gpr;
@@ -376,6 +381,15 @@ __device__ __forceinline__ void meta_fetch(const MAT& m, const Tile& t, uint32_t
             r.s[1] = sv.y;
             r.b[0] = bv.x;
             r.b[1] = bv.y;
+            if constexpr (BIG) {  // straight-line: a lane past the tile's groups repeats the first entries
+                const uint32_t gi2 = 4u * (ti + (uint32_t)SN);
+                const size_t e2 = gi2 < total ? g0 + gi2 : g0;
+                const uint2 sv2 = *reinterpret_cast<const uint2*>(m.sc + e2), bv2 = *reinterpret_cast<const uint2*>(m.bi + e2);
+                r.s[2] = sv2.x;
+                r.s[3] = sv2.y;
+                r.b[2] = bv2.x;
+                r.b[3] = bv2.y;
+            }
         } else {
             const float inv = 1.0f / (float)gpr;
 #pragma unroll
@@ -389,14 +403,18 @@ __device__ __forceinline__ void meta_fetch(const MAT& m, const Tile& t, uint32_t
         }
     }
 }
-template <WKind KIND, int SN, bool RUN>
+template <WKind KIND, int SN, bool RUN, bool BIG = false>
 __device__ __forceinline__ void meta_store(const MetaRegs& r, uint32_t ti, uint32_t* meta) {
     if constexpr (KIND != W_BF16) {
         if constexpr (RUN) {
-            if (4u * ti < (uint32_t)kMetaRegs * SN)
+            if (BIG || 4u * ti < (uint32_t)kMetaRegs * SN)
                 *reinterpret_cast<uint4*>(meta + 4u * ti) =
                     make_uint4((r.s[0] & 0xffffu) | (r.b[0] << 16), (r.s[0] >> 16) | (r.b[0] & 0xffff0000u),
                                (r.s[1] & 0xffffu) | (r.b[1] << 16), (r.s[1] >> 16) | (r.b[1] & 0xffff0000u));
+            if constexpr (BIG)
+                *reinterpret_cast<uint4*>(meta + 4u * (ti + (uint32_t)SN)) =
+                    make_uint4((r.s[2] & 0xffffu) | (r.b[2] << 16), (r.s[2] >> 16) | (r.b[2] & 0xffff0000u),
+                               (r.s[3] & 0xffffu) | (r.b[3] << 16), (r.s[3] >> 16) | (r.b[3] & 0xffff0000u));
         } else {
 #pragma unroll
             for (int k = 0; k < kMetaRegs; ++k) meta[k * SN + ti] = r.s[k] | (r.b[k] << 16);
@@ -600,11 +618,12 @@ __device__ __forceinline__ Tile make_tile(uint32_t row0, uint32_t rows, uint32_t
 //   scratch [16]
 struct LdsPlan {
     uint32_t cs_max, work_floats, att_elems;
+    uint32_t meta_words;   // per matrix: kMetaWords (one-pass flavour) or kMetaWordsBig
 };
-constexpr uint32_t kMetaWords = kMetaRegs * kBlock;  // per matrix (the streaming threads never exceed kBlock)
+static_assert(kBlock == 256, "the metadata areas are sized for 256 streaming threads");
 template <WKind KIND>
 __host__ __device__ inline uint32_t xcd_lds_bytes(const LdsPlan& p) {
-    return ChunkTraits<KIND>::kPieces * p.cs_max * 16u + p.cs_max * 4u + p.work_floats * 4u + 3u * kMetaWords * 4u +
+    return ChunkTraits<KIND>::kPieces * p.cs_max * 16u + p.cs_max * 4u + p.work_floats * 4u + 3u * p.meta_words * 4u +
            ((p.att_elems * 2u + 15u) & ~15u) + 64u;
 }
 
@@ -625,8 +644,9 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     uint4* xs = lds_raw;
     float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
     float* work = sx + cs_max;
-    uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]
-    float* red = reinterpret_cast<float*>(meta + 3 * kMetaWords);      // [16]
+    constexpr uint32_t MW = meta_words<ONE>();
+    uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][MW]
+    float* red = reinterpret_cast<float*>(meta + 3 * MW);              // [16]
     const uint32_t tid = threadIdx.x;
     constexpr bool streams = true;
 
@@ -650,8 +670,8 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if constexpr (!EARLY) input_request<TOKEN>(lead, inr, xres_in);
     tile_pos_init<NLA, kBlock>(a.gate, tg, tid, pg);
     tile_pos_init<NLB, kBlock>(a.down, td, tid, pd);
-    meta_fetch<KIND, kBlock, true>(a.gate, tg, tid, mg);
-    meta_fetch<KIND, kBlock, true>(a.up, tg, tid, mu);
+    meta_fetch<KIND, kBlock, true, !ONE>(a.gate, tg, tid, mg);
+    meta_fetch<KIND, kBlock, true, !ONE>(a.up, tg, tid, mu);
     // Only kGuAhead requests of the gate matrix go out ahead of the input's staging, the rest of the pass and the up
     // matrix's behind it: a wave cannot stage before it has ISSUED what stands in front, issue stalls once the CU's
     // request queue is full, and the block's staging waits for its slowest wave.  With all twelve in front the
@@ -667,9 +687,9 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     tile_load<KIND, NLA, kBlock>(a.up, tg, pg, ru);
     FK_XCD_STAMP(1, 5);
     input_clear<TOKEN>(a.in);
-    meta_store<KIND, kBlock, true>(mg, tid, meta);
-    meta_store<KIND, kBlock, true>(mu, tid, meta + kMetaWords);
-    meta_fetch<KIND, kBlock, true>(a.down, td, tid, md, sync.xcd);  // not needed before the hand-over: kept off the start-up path
+    meta_store<KIND, kBlock, true, !ONE>(mg, tid, meta);
+    meta_store<KIND, kBlock, true, !ONE>(mu, tid, meta + MW);
+    meta_fetch<KIND, kBlock, true, !ONE>(a.down, td, tid, md, sync.xcd);  // not needed before the hand-over: kept off the start-up path
     __syncthreads();
 
     // ---- gate / up rows of this XCD's slice, SwiGLU ----
@@ -677,13 +697,13 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if (streams) {
         auto request_down = [&]() { tile_load<KIND, NLB, kBlock>(a.down, td, pd, rd); };
         if (gu_n)
-            tile_run_pair<KIND, NLA, kBlock, ONE>(a.gate, a.up, tg, pg, rg, ru, xs, sx, meta, meta + kMetaWords, work, work + seg,
+            tile_run_pair<KIND, NLA, kBlock, ONE>(a.gate, a.up, tg, pg, rg, ru, xs, sx, meta, meta + MW, work, work + seg,
                                              request_down);
         else
             request_down();
     }
     FK_XCD_STAMP(1, 6);
-    meta_store<KIND, kBlock, true>(md, tid, meta + 2 * kMetaWords);
+    meta_store<KIND, kBlock, true, !ONE>(md, tid, meta + 2 * MW);
     __syncthreads();
     FK_XCD_STAMP(1, 12);
     if (streams && gu_n) {
@@ -703,7 +723,7 @@ __device__ __forceinline__ void xcd_mlp_phase(const ARGS& a, const LEAD& lead, I
     if (streams) stage_vector<KIND>(a.mid + (size_t)sync.xcd * per_xcd, per_xcd >> 3, a.down_cs, xs, sx);
     __syncthreads();
     FK_XCD_STAMP(1, 9);
-    if (streams && d_n) tile_run<KIND, NLB, kBlock, ONE>(a.down, td, pd, rd, xs, sx, meta + 2 * kMetaWords, work, []() {});
+    if (streams && d_n) tile_run<KIND, NLB, kBlock, ONE>(a.down, td, pd, rd, xs, sx, meta + 2 * MW, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(1, 10);
     if (streams && d_n && ok) {
@@ -755,8 +775,9 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     uint4* xs = lds_raw;
     float* sx = reinterpret_cast<float*>(xs + PIECES * cs_max);
     float* work = sx + cs_max;
-    uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][kMetaWords]; two used
-    uint16_t* att = reinterpret_cast<uint16_t*>(meta + 3 * kMetaWords);
+    constexpr uint32_t MW = meta_words<ONE>();
+    uint32_t* meta = reinterpret_cast<uint32_t*>(work + work_floats);  // [3][MW]; two used
+    uint16_t* att = reinterpret_cast<uint16_t*>(meta + 3 * MW);
 
     // Requested now, looked at only behind the start-up requests (the pin below): used at once, the wave would sit
     // out this load's trip to memory before it has asked for anything else.
@@ -788,7 +809,7 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     if constexpr (!EARLY) input_request<TOKEN>(lead, inr, xres_in);
     tile_pos_init<NLA, kAttnStream>(mq, tq, ti, pq);
     tile_pos_init<NLB, kAttnStream>(a.wo, to, ti, po);
-    meta_fetch<KIND, kAttnStream, true>(mq, tq, ti, mmq);
+    meta_fetch<KIND, kAttnStream, true, !ONE>(mq, tq, ti, mmq);
     tile_load<KIND, NLA, kAttnStream>(mq, tq, pq, rq);  // all of it ahead of the staging: 2 or 3 of 5 were no faster here
     FK_XCD_STAMP(0, 1);
     asm volatile("" : "+v"(kv_len_raw));
@@ -797,8 +818,8 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
     input_stage<KIND, 0>(a.in, inr, xs, sx, a.wq.cpr, red, xres_out);
     FK_XCD_STAMP(0, 5);
     input_clear<TOKEN>(a.in);
-    meta_store<KIND, kAttnStream, true>(mmq, ti, meta);
-    meta_fetch<KIND, kAttnStream, true>(a.wo, to, ti, mmo, sync.xcd);  // not needed before the attention is done
+    meta_store<KIND, kAttnStream, true, !ONE>(mmq, ti, meta);
+    meta_fetch<KIND, kAttnStream, true, !ONE>(a.wo, to, ti, mmo, sync.xcd);  // not needed before the attention is done
     __syncthreads();
     FK_XCD_STAMP(0, 13);
 
@@ -901,9 +922,9 @@ __device__ __forceinline__ void xcd_attn_phase(const ARGS& a, const LEAD& lead, 
             stage_emit<KIND>(xs, sx, a.o_cs, t, live, v, v, 1.0f, false);
         }
     }
-    meta_store<KIND, kAttnStream, true>(mmo, ti, meta + kMetaWords);
+    meta_store<KIND, kAttnStream, true, !ONE>(mmo, ti, meta + MW);
     __syncthreads();
-    if (streams && o_n) tile_run<KIND, NLB, kAttnStream, ONE>(a.wo, to, po, ro, xs, sx, meta + kMetaWords, work, []() {});
+    if (streams && o_n) tile_run<KIND, NLB, kAttnStream, ONE>(a.wo, to, po, ro, xs, sx, meta + MW, work, []() {});
     __syncthreads();
     FK_XCD_STAMP(0, 11);
     if (o_n && ok2) {
@@ -1220,6 +1241,7 @@ MlpGeometry mlp_geometry(const XcdLayerShape& s, bool for_token) {
     const uint32_t gu = 2 * padded(g.gu_rows * g.gate_cpr, depth.gu), dn = padded(g.down_rows * g.down_cs, depth.down);
     g.lp.work_floats = gu > dn ? gu : dn;
     g.lp.att_elems = 0;
+    g.lp.meta_words = g.one ? kMetaWords : kMetaWordsBig;
     g.lds = lds_for(s.bits, g.lp);
     g.func = s.bits == 4 ? mlp_func<W_Q4>(g.one) : (s.bits == 8 ? mlp_func<W_Q8>(g.one) : mlp_func<W_BF16>(g.one));
     return g;
@@ -1233,7 +1255,7 @@ struct AttnGeometry {
     uint32_t lds;
     const void* func;
 };
-AttnGeometry attn_geometry(const XcdLayerShape& s) {
+AttnGeometry attn_geometry(const XcdLayerShape& s, bool for_token = false) {
     AttnGeometry g;
     const uint32_t cv = chunk_values(s.bits), G = s.n_heads / s.n_kv;
     g.wq_cpr = s.hidden / cv;
@@ -1258,7 +1280,7 @@ AttnGeometry attn_geometry(const XcdLayerShape& s) {
     g.lp.cs_max = g.wq_cpr > g.o_cs ? g.wq_cpr : g.o_cs;
     // partial rows padded to whole passes: of this launch's depths and of the whole-token launch's (it shares this plan)
     const PassDepth deep = depth_of_bits(s.bits);
-    g.one = R * g.wq_cpr <= (uint32_t)deep.qkv * kAttnStream && g.o_rows * g.o_cs <= (uint32_t)deep.o * kAttnStream;
+    g.one = !for_token && R * g.wq_cpr <= (uint32_t)deep.qkv * kAttnStream && g.o_rows * g.o_cs <= (uint32_t)deep.o * kAttnStream;
     const PassDepth depth = g.one ? deep : PassDepth{kNlQkv, kNlO, kNlGu, kNlDown};
     auto larger = [](uint32_t x, uint32_t y) { return x > y ? x : y; };
     uint32_t wf = larger(padded(R * g.wq_cpr, depth.qkv), padded(R * g.wq_cpr, kNlQkv));
@@ -1267,6 +1289,7 @@ AttnGeometry attn_geometry(const XcdLayerShape& s) {
     const uint32_t sf = sdpa_lds_floats(1, g.chunk_len, s.head_dim, s.head_dim, true);
     g.lp.work_floats = wf > sf ? wf : sf;
     g.lp.att_elems = G * s.head_dim;
+    g.lp.meta_words = g.one ? kMetaWords : kMetaWordsBig;   // the whole-token launch runs the flavour with the pass loop
     g.lds = lds_for(s.bits, g.lp);
     g.func = s.bits == 4 ? attn_func<W_Q4>(g.one) : (s.bits == 8 ? attn_func<W_Q8>(g.one) : attn_func<W_BF16>(g.one));
     return g;
@@ -1291,22 +1314,24 @@ fk_status xcd_layer_supported(const XcdLayerShape& s) {
     if ((G * s.head_dim) % unit) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a KV head's query columns must be whole quantisation groups");
     if (s.inter % (kXcds * unit) || s.inter % (kXcds * 8)) return set_error(FK_ERR_UNSUPPORTED, "xcd layer: intermediate / 8 must be whole quantisation groups");
     if (s.capacity == 0) return set_error(FK_ERR_INVALID, "xcd layer: zero cache capacity");
+    const MlpGeometry mg = mlp_geometry(s, false);
+    const AttnGeometry ag = attn_geometry(s);
     if (s.bits != 16) {
-        // a tile's quantisation groups are fetched kMetaRegs per thread
-        const uint32_t budget = kMetaRegs * kBlock, n_q = s.n_heads * s.head_dim;
+        // a tile's quantisation groups are fetched once per block: 768 per matrix in the one-pass flavour, 2048 in the
+        // flavour with the pass loop
+        const uint32_t n_q = s.n_heads * s.head_dim;
+        const uint32_t budget_a = ag.lp.meta_words, budget_m = mg.lp.meta_words;
         uint32_t R = 1;
         while (ceil_div(G * s.head_dim, R) + 2 * ceil_div(s.head_dim, R) > kXcdSlots) ++R;
-        if (R * (s.hidden / s.group) > budget || ceil_div(s.hidden, kXcdSlots) * (n_q / kXcds / s.group) > budget ||
-            ceil_div(s.inter / kXcds, kXcdSlots) * (s.hidden / s.group) > budget ||
-            ceil_div(s.hidden, kXcdSlots) * (s.inter / kXcds / s.group) > budget)
+        if (R * (s.hidden / s.group) > budget_a || ceil_div(s.hidden, kXcdSlots) * (n_q / kXcds / s.group) > budget_a ||
+            ceil_div(s.inter / kXcds, kXcdSlots) * (s.hidden / s.group) > budget_m ||
+            ceil_div(s.hidden, kXcdSlots) * (s.inter / kXcds / s.group) > budget_m)
             return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a block's tile holds more quantisation groups than the kernel fetches");
         // the groups of a block's o_proj / down_proj tile are fetched four per lane from the per-XCD copies
         const uint32_t rpb = ceil_div(s.hidden, kXcdSlots);
         if (s.hidden % kXcdSlots || (rpb * (n_q / kXcds / s.group)) % 4 || (rpb * (s.inter / kXcds / s.group)) % 4)
             return set_error(FK_ERR_UNSUPPORTED, "xcd layer: a block's o_proj / down_proj tile must hold a multiple of four quantisation groups");
     }
-    const MlpGeometry mg = mlp_geometry(s, false);
-    const AttnGeometry ag = attn_geometry(s);
     if (2u * ((mg.lds + 1023u) & ~1023u) > kCuLdsBytes || 2u * ((ag.lds + 1023u) & ~1023u) > kCuLdsBytes)
         return set_error(FK_ERR_UNSUPPORTED, "xcd layer: two workgroups of a launch must fit the LDS of one CU (MLP launch " +
                                                  std::to_string(mg.lds) + " bytes, attention launch " + std::to_string(ag.lds) +
@@ -1414,7 +1439,7 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     FK_TRY(bind_mat(rq.wk, n_kvd, s.hidden, s, &a.wk, "k_proj"));
     FK_TRY(bind_mat(rq.wv, n_kvd, s.hidden, s, &a.wv, "v_proj"));
     FK_TRY(bind_mat(rq.wo, s.hidden, n_q, s, &a.wo, "o_proj"));
-    const AttnGeometry g = attn_geometry(s);
+    const AttnGeometry g = attn_geometry(s, rq.for_token);
     a.q_rows = g.q_rows;
     a.kv_rows = g.kv_rows;
     a.qkv_tile_rows = g.R;
@@ -1465,7 +1490,10 @@ fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out) {
     const LdsPlan lp = g.lp;
     const uint32_t lds = g.lds;
     out->func = g.func;
-    FK_TRY(require_two_blocks_per_cu(out->func, lds, "attention"));
+    if (rq.for_token)
+        FK_TRY(set_lds_limit(out->func, lds));  // an argument block for the whole-token launch, which is checked as a whole
+    else
+        FK_TRY(require_two_blocks_per_cu(out->func, lds, "attention"));
     out->grid = dim3(kXcdGrid, 1, 1);
     out->block = dim3(kBlock, 1, 1);
     out->shmem = lds;

@@ -222,6 +222,7 @@ struct XcdAttnRequest {
     void* workspace;
     uint32_t spin_limit;
     bool mark_placement;
+    bool for_token = false;   // the block is meant for the whole-token launch (which runs the flavour with the pass loop)
 };
 fk_status plan_xcd_attn(const XcdAttnRequest& rq, Launch* out);
 

@@ -113,3 +113,12 @@ def test_two_launch_layer_admission_rules_need_no_device():
     # the 4B-class shape passes every rule; without a device the answer is then "no HIP device"
     st = fk.lib.fk_xcd_layer_supported(u(2560), u(9728), u(32), u(8), u(128), u(1024), u(4), u(64))
     assert st == (fk.FK_OK if fk.has_device() else fk.FK_ERR_HIP), fk.lib.fk_last_error()
+    # the 8B class: in 4 bits its tiles (up to 1792 quantisation groups) fit the flavour with the pass loop; in 8 bits
+    # two workgroups of the MLP launch do not fit a CU
+    st = fk.lib.fk_xcd_layer_supported(u(4096), u(14336), u(32), u(8), u(128), u(1024), u(4), u(64))
+    assert st == (fk.FK_OK if fk.has_device() else fk.FK_ERR_HIP), fk.lib.fk_last_error()
+    st = fk.lib.fk_xcd_layer_supported(u(4096), u(14336), u(32), u(8), u(128), u(1024), u(8), u(64))
+    assert st == fk.FK_ERR_UNSUPPORTED and b"resident" in fk.lib.fk_last_error()
+    # a tile beyond 2048 groups per matrix is refused (hidden 4096 in groups of 32: 28 rows x 128 groups)
+    st = fk.lib.fk_xcd_layer_supported(u(4096), u(14336), u(32), u(8), u(128), u(1024), u(4), u(32))
+    assert st == fk.FK_ERR_UNSUPPORTED and b"quantisation groups" in fk.lib.fk_last_error()
