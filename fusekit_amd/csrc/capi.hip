@@ -270,6 +270,19 @@ fk_status fk_rmsnorm_qkv_rows(const uint16_t* x, uint32_t rows, uint32_t x_row_s
     return run_launch(l, (hipStream_t)s);
 }
 
+fk_status fk_gateup_swiglu_rows(const uint16_t* x, uint32_t rows, const uint16_t* norm_w, float eps, const fk_weight* Wg,
+                                const fk_weight* Wu, int variant, uint16_t* out, fk_stream s) {
+    if (!Wg || !Wu || !x || !out) return set_error(FK_ERR_INVALID, "fk_gateup_swiglu_rows: null weight, input or output");
+    if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, "fk_gateup_swiglu_rows: variant must be 0, 1 or 2");
+    if (Wg->n != Wu->n || Wg->k != Wu->k || Wg->group != Wu->group || Wg->bits != Wu->bits)
+        return set_error(FK_ERR_INVALID, "fk_gateup_swiglu_rows: gate and up need the same shape, bits and group size");
+    if (rows < 2 || rows > 8 || Wg->group != 64 || (Wg->bits != 4 && Wg->bits != 8))
+        return set_error(FK_ERR_UNSUPPORTED, "fk_gateup_swiglu_rows: 2..8 rows, 4- or 8-bit weights, group size 64");
+    Launch l;
+    FK_TRY(plan_qgemm_wide(Wg, Wu, x, rows, nullptr, nullptr, variant, out, &l, norm_w, eps));
+    return run_launch(l, (hipStream_t)s);
+}
+
 fk_status fk_gateup_swiglu(const uint16_t* x, const uint16_t* norm_w, float eps, const fk_weight* Wg,
                            const fk_weight* Wu, int variant, uint16_t* out, fk_stream s) {
     if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, "fk_gateup_swiglu: variant must be 0, 1 or 2");

@@ -228,6 +228,23 @@ fk_status plan_gateup(const Dispatch& d, Launch* l, SlotRW* rw) {
     const int variant = (int)d.param("variant", 0);
     if (variant < 0 || variant > 2) return set_error(FK_ERR_INVALID, d.kernel + ": swiglu variant must be 0, 1 or 2");
     rq.swiglu_variant = variant;
+    const uint32_t rows = d.u("rows", 1);
+    if (rows > 1) {
+        // Row form (2 .. 8 token rows): x [rows, hidden], out [rows, inter]; the pair streamed once for all rows by the
+        // shared-stream matmul, the norm applied while the rows are staged.
+        if (bits == 16) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": the row form takes 4- or 8-bit weights");
+        FK_TRY(need_bytes(d, 0, (size_t)rows * hidden * 2));
+        FK_TRY(need_bytes(d, out_slot, (size_t)rows * inter * 2));
+        const uint16_t* nw = nullptr;
+        if (has_norm) {
+            FK_TRY(need_bytes(d, norm_slot, (size_t)hidden * 2));
+            nw = arg_ptr<const uint16_t>(d, norm_slot);
+        }
+        all_but_last(s, 1, rw);
+        if (rows > 8 || group != 64) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": the row form takes 2..8 rows and group size 64");
+        return plan_qgemm_wide(&W[0], &W[1], arg_ptr<const uint16_t>(d, 0), rows, nullptr, nullptr, variant,
+                               arg_ptr<uint16_t>(d, out_slot), l, nw, (float)d.param("eps", 1e-6));
+    }
     FK_TRY(need_bytes(d, 0, (size_t)hidden * 2));
     FK_TRY(need_bytes(d, out_slot, (size_t)inter * 2));
     rq.x = arg_ptr<const uint16_t>(d, 0);

@@ -180,7 +180,8 @@ struct WideSeg {
 fk_status plan_qgemm_wide_fan(const uint16_t* x, uint32_t x_stride, uint32_t M, const uint16_t* norm_w, float eps,
                               const WideSeg* segs, uint32_t n_seg, Launch* out);
 fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16_t* x, uint32_t M, const uint16_t* bias,
-                          const uint16_t* res, int variant, uint16_t* y, Launch* out);
+                          const uint16_t* res, int variant, uint16_t* y, Launch* out, const uint16_t* norm_w = nullptr,
+                          float eps = 0.f);
 bool gemm_library_available();
 size_t qgemm_library_sums_bytes(uint32_t m, uint32_t n, uint32_t k);
 size_t qgemm_library_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);

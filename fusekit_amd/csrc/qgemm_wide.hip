@@ -586,7 +586,7 @@ bool qgemm_takes_wide(uint32_t M, uint32_t group) { return g_wide_on && M >= 2 &
 
 // W1 (and SwiGLU of the pair) or bias / res (single matrix).
 fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16_t* x, uint32_t M, const uint16_t* bias,
-                          const uint16_t* res, int variant, uint16_t* y, Launch* out) {
+                          const uint16_t* res, int variant, uint16_t* y, Launch* out, const uint16_t* norm_w, float eps) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!qgemm_takes_wide(M, W0->group)) return set_error(FK_ERR_UNSUPPORTED, "qgemm (shared stream): 2..10 rows, group size 64");
@@ -603,6 +603,12 @@ fk_status plan_qgemm_wide(const fk_weight* W0, const fk_weight* W1, const uint16
     a.M = M; a.N = W0->n; a.K = W0->k;
     a.n_seg = 1; a.x_stride = W0->k;
     a.ns[0] = W0->n; a.blk0[0] = 0; a.y_stride[0] = W0->n; a.ys[0] = y;
+    if (norm_w) {  // the activations are RMS-normalised while they are staged: the 16-row form only
+        if (M > 8 || !g_wide_tiles16) return set_error(FK_ERR_UNSUPPORTED, "qgemm (shared stream): a fused norm takes 2..8 rows");
+        if (((uintptr_t)norm_w | (uintptr_t)x) & 15u) return set_error(FK_ERR_INVALID, "qgemm (shared stream): rows and norm weights must be 16-byte aligned");
+        a.norm_w = norm_w;
+        a.eps = eps;
+    }
     a.cpr = W0->k / (W0->bits == 4 ? 32u : 16u);
     a.gpr = W0->k / 64u;
     a.variant = variant;

@@ -549,8 +549,16 @@ class MoeRowsVariant:
             matmul(self.att, full(Wo), c.n_heads * c.v_dim, c.hidden, self.x[1], res=self.x[0])
             post = w.vecs[p + "post_attention_layernorm"]
             if l < c.first_dense:
-                norm_rows(self.x[1], post, c.hidden, self.xn)
-                swiglu(w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"], c.dense_inter)
+                Wg, Wu = w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"]
+                if self.fan:    # the norm rides in the gate / up launch (row form of rmsnorm_gateup_swiglu)
+                    t.append(Dispatch(name("rmsnorm_gateup_swiglu"),
+                                      [arg(self.x[1]), arg(post), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales), arg(Wg.biases),
+                                       arg(Wu.biases), arg(self.mid, m * c.dense_inter * 2)],
+                                      dict(quant, hidden=c.hidden, inter=c.dense_inter, eps=c.eps, variant=c.swiglu_variant,
+                                           has_norm=1, rows=m)))
+                else:
+                    norm_rows(self.x[1], post, c.hidden, self.xn)
+                    swiglu(Wg, Wu, c.dense_inter)
                 matmul(self.mid, full(w.mats[p + "mlp.down_proj"]), c.dense_inter, c.hidden, self.x[0], res=self.x[1])
                 continue
             ridx = arg(self.ridx, 4 * routes, 4 * routes * l)

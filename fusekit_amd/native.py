@@ -191,6 +191,12 @@ def rmsnorm_qkv(x, norm_w, eps, Wq, Wk, Wv, bq, bk, bv, q, k, v, stream=None) ->
                              _ptr(bq), _ptr(bk), _ptr(bv), _ptr(q), _ptr(k), _ptr(v), _ptr(stream)))
 
 
+def gateup_swiglu_rows(x, rows, norm_w, eps, Wg, Wu, variant, out, stream=None) -> None:
+    """fk_gateup_swiglu_rows: RMSNorm + gate / up + SwiGLU of 2..8 token rows in one launch."""
+    check(lib.fk_gateup_swiglu_rows(_ptr(x), C.c_uint32(rows), _ptr(norm_w), C.c_float(eps), C.byref(Wg.c), C.byref(Wu.c),
+                                    C.c_int(variant), _ptr(out), _ptr(stream)))
+
+
 def rmsnorm_qkv_rows(x, rows, x_row_stride, norm_w, eps, Wq, Wk, Wv, q, q_row_stride, k=None, k_row_stride=0, v=None,
                      v_row_stride=0, stream=None) -> None:
     """fk_rmsnorm_qkv_rows: RMSNorm + one to three projections of 2..8 token rows in one launch."""

@@ -10,6 +10,9 @@ uniforms and the logits with the decode graph:
     causal attention (kv_len read on the device), o matmul + residual, RMSNorm rows,
     gate/up matmul + SwiGLU, down matmul + residual] -> final norm + LM head on the last row -> argmax
 
+(for 2..8 rows of 4- / 8-bit weights the norms ride in the launches behind them: RMSNorm + q / k / v is one launch,
+RMSNorm + gate/up + SwiGLU another)
+
 `offset` (position of row 0) and `kv_len` (= offset + N) are device words the host writes before a
 replay, so one graph serves any position.  Every node is a kernel of this library (the fused
 multi-row matmul; a library GEMM cannot be a node), quantised weights and a bf16 KV cache only.
@@ -75,13 +78,24 @@ class PrefillVariant:
         head = w.mats.get("lm_head", emb)
         t.append(Dispatch(name("embed_lookup_decode"), [arg(self.tokens)] + rt._wargs(emb) + [arg(self.x[0])],
                           dict(bits=emb.bits, group=emb.group or 64, hidden=c.hidden, vocab=c.vocab, output_scale=c.embed_scale, rows=m)))
+        # 2..8 rows of 4- / 8-bit weights: the norm and the projections behind it are ONE launch (row forms of the
+        # rmsnorm_qkv and rmsnorm_gateup_swiglu families: the norm is applied while the rows are staged)
+        fused = 2 <= m <= 8 and c.bits in (4, 8) and c.group == 64
         for l in range(c.n_layers):
             p = f"layers.{l}."
-            t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(self.xn)],
-                              dict(rows=m, hidden=c.hidden, eps=c.eps)))
-            for nm, dst in (("q", self.q), ("k", self.k), ("v", self.v)):
-                matmul(self.xn, w.mats[p + f"self_attn.{nm}_proj"], dst,
-                       bias=w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None)
+            if fused and not c.qkv_bias:
+                Wq, Wk, Wv = (w.mats[p + f"self_attn.{nm}_proj"] for nm in "qkv")
+                t.append(Dispatch(name("rmsnorm_qkv"),
+                                  [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(Wq.w), arg(Wk.w), arg(Wv.w),
+                                   arg(Wq.scales), arg(Wk.scales), arg(Wv.scales), arg(Wq.biases), arg(Wk.biases), arg(Wv.biases),
+                                   arg(self.q), arg(self.k), arg(self.v)],
+                                  dict(quant, hidden=c.hidden, n_q=Wq.n, n_kv=Wk.n, eps=c.eps, has_norm=1, has_bias=0, rows=m)))
+            else:
+                t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(self.xn)],
+                                  dict(rows=m, hidden=c.hidden, eps=c.eps)))
+                for nm, dst in (("q", self.q), ("k", self.k), ("v", self.v)):
+                    matmul(self.xn, w.mats[p + f"self_attn.{nm}_proj"], dst,
+                           bias=w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None)
             a = [arg(self.q), arg(self.k), arg(self.v)]
             if c.qk_norm:
                 a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]
@@ -93,13 +107,19 @@ class PrefillVariant:
                               [arg(self.q), arg(rt.cache_k[l]), arg(rt.cache_v[l]), arg(self.kv_len), arg(self.att)],
                               dict(n_heads=c.n_heads, n_kv=c.n_kv, head_dim=c.head_dim, capacity=c.capacity, rows=m)))
             matmul(self.att, w.mats[p + "self_attn.o_proj"], self.x[1], res=self.x[0])
-            t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(w.vecs[p + "post_attention_layernorm"]), arg(self.xn)],
-                              dict(rows=m, hidden=c.hidden, eps=c.eps)))
             Wg, Wu = w.mats[p + "mlp.gate_proj"], w.mats[p + "mlp.up_proj"]
-            t.append(Dispatch(name("qgemm_swiglu"),
-                              [arg(self.xn), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases),
-                               arg(self.mid), arg(self.ws)],
-                              dict(quant, hidden=c.hidden, inter=c.inter, rows=m, variant=c.swiglu_variant)))
+            if fused:
+                t.append(Dispatch(name("rmsnorm_gateup_swiglu"),
+                                  [arg(self.x[1]), arg(w.vecs[p + "post_attention_layernorm"]), arg(Wg.w), arg(Wu.w), arg(Wg.scales),
+                                   arg(Wu.scales), arg(Wg.biases), arg(Wu.biases), arg(self.mid)],
+                                  dict(quant, hidden=c.hidden, inter=c.inter, eps=c.eps, variant=c.swiglu_variant, has_norm=1, rows=m)))
+            else:
+                t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[1]), arg(w.vecs[p + "post_attention_layernorm"]), arg(self.xn)],
+                                  dict(rows=m, hidden=c.hidden, eps=c.eps)))
+                t.append(Dispatch(name("qgemm_swiglu"),
+                                  [arg(self.xn), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales), arg(Wg.biases), arg(Wu.biases),
+                                   arg(self.mid), arg(self.ws)],
+                                  dict(quant, hidden=c.hidden, inter=c.inter, rows=m, variant=c.swiglu_variant)))
             matmul(self.mid, w.mats[p + "mlp.down_proj"], self.x[0], res=self.x[1])
         last = arg(self.x[0], c.hidden * 2, (m - 1) * c.hidden * 2)  # the last row's hidden state
         t.append(Dispatch(name("final_rmsnorm_lm_head"), [last, arg(w.vecs["final_norm"])] + rt._wargs(head) + [arg(rt.logits)],

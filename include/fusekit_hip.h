@@ -171,6 +171,12 @@ fk_status fk_rmsnorm_qkv_rows(const uint16_t *x, uint32_t rows, uint32_t x_row_s
  *     (src/codegen/kernels/qmv_swiglu.rs:20-246). */
 fk_status fk_gateup_swiglu(const uint16_t *x, const uint16_t *norm_w, float eps, const fk_weight *Wg,
                            const fk_weight *Wu, int variant, uint16_t *out, fk_stream s);
+/* K3a for 2..8 token rows (the emitter compiled with active_m = N, src/codegen/kernels/rmsnorm_gateup_swiglu.rs:20-330,
+ *     src/commands/patch.rs:112-150): x [rows, hidden], out [rows, inter]; ONE launch streams the pair once for all rows
+ *     and applies the norm while the rows are staged (norm_w NULL: none); 4- or 8-bit, group 64.  Dispatch family
+ *     fusekit_rmsnorm_gateup_swiglu with the parameter rows. */
+fk_status fk_gateup_swiglu_rows(const uint16_t *x, uint32_t rows, const uint16_t *norm_w, float eps, const fk_weight *Wg,
+                                const fk_weight *Wu, int variant, uint16_t *out, fk_stream s);
 
 /* M1  routed gate/up + SwiGLU over expert-stacked weights.  Replaces
  *     src/codegen/kernels/routed_qmv_swiglu.rs:20-450 (slots x, gate w/s/b, up w/s/b,

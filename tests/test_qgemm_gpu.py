@@ -145,6 +145,24 @@ def test_norm_and_fan_out_of_several_rows_in_one_launch(fk, bits, m, hidden, ns,
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,hidden,inter,variant,normed", [(8, 2560, 9728, 1, True), (3, 896, 4864, 0, True), (2, 512, 1408, 2, False)])
+def test_norm_gate_up_and_swiglu_of_several_rows_in_one_launch(fk, bits, m, hidden, inter, variant, normed):
+    """fk_gateup_swiglu_rows: every row equals the oracle's single-row RMSNorm -> gate / up -> SwiGLU."""
+    Wg, Wu = make_qweight(720 + bits, inter, hidden, bits), make_qweight(730 + bits, inter, hidden, bits)
+    x = normal_bf16(740 + m, (m, hidden))
+    nw = normal_bf16(741, hidden, 0.1, 1.0) if normed else None
+    out = fk.DeviceBuffer(2 * m * inter)
+    fk.gateup_swiglu_rows(_dev(fk, x), m, _dev(fk, nw), 1e-6, to_device(fk, Wg), to_device(fk, Wu), variant, out)
+    got = out.to_numpy(np.uint16, (m, inter))
+    for r in range(m):
+        xn = oracle.rmsnorm(x[r], nw, 1e-6) if normed else x[r]
+        _check_swiglu(got[r], oracle.gateup_swiglu(x[r], nw, 1e-6, Wg, Wu, variant), xn, Wg, Wu, variant)
+    with pytest.raises(fk.FusekitError):
+        fk.gateup_swiglu_rows(_dev(fk, normal_bf16(1, (9, hidden))), 9, _dev(fk, nw), 1e-6, to_device(fk, Wg), to_device(fk, Wu),
+                              variant, fk.DeviceBuffer(2 * 9 * inter))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("m", [9, 100])
 def test_qgemm_group_128(fk, bits, m):
     W = make_qweight(60, 384, 1024, bits, group=128)
