@@ -301,7 +301,28 @@ def case_moe_rows(d, reps, rows=8, offset=32):
                       "rows_per_s": round(rows / sec, 1), "note": "one graph replay per pass, wall clock"}), flush=True)
 
 
+def case_dense_rows(d, reps, rows=8, offset=32):
+    """`rows` active token rows of the 4B-class dense model (int4) in one pass: its prefill_m<rows> variant."""
+    import time
+    from .decoder import DENSE_4B, DecoderConfig, DecoderRuntime, DecoderWeights
+    from .prefill_variant import PrefillVariant
+    cfg = DecoderConfig(**DENSE_4B, bits=4, capacity=1024)
+    rt = DecoderRuntime(cfg, DecoderWeights.random_init(cfg, seed=0), dispatcher=d)
+    v = PrefillVariant(rt, rows)
+    rt.prefill(list(range(200, 200 + offset)))
+    toks = list(range(100, 100 + rows))
+    v.run(toks, offset)
+    n = 10
+    t0 = time.perf_counter()
+    for _ in range(n):
+        v.run(toks, offset)
+    sec = (time.perf_counter() - t0) / n
+    print(json.dumps({"case": f"dense4b_rows{rows}_pass_q4", "rows": rows, "ms_per_pass": round(sec * 1e3, 3), "launches": len(v.tasks),
+                      "rows_per_s": round(rows / sec, 1), "note": "one graph replay per pass, wall clock"}), flush=True)
+
+
 CASES = {
+    "dense4b_rows8_pass": lambda d, r: case_dense_rows(d, r, 8),
     "moe_cfg5_rows8_pass": lambda d, r: case_moe_rows(d, r, 8),
     "moe_cfg5_rows64_pass": lambda d, r: case_moe_rows(d, r, 64),
     "moe_cfg5_decode": lambda d, r: case_moe_decode(d, r),
