@@ -570,7 +570,11 @@ fk_status fk_rope_store_sdpa_decode(const uint16_t *q, const uint16_t *k, const 
  * (fusekit_amd/csrc/dispatcher.hip).  Requires 8 KV heads (one per XCD), 1 / 2 / 4 / 8 query heads per KV
  * head, head_dim 64 or 128, hidden <= 4096, and a shape whose workgroups fit two per CU (LDS and registers:
  * answered from the shape where possible, else by the device's occupancy query); other layers use the
- * per-dispatch families.
+ * per-dispatch families.  Parameter token_launch on the dispatches of a run: 1 -- fk_build_graph executes the
+ * whole run attention, MLP, attention, ... as ONE kernel node (device-wide barriers between the phases; every
+ * layer then needs its own q / k / v rows); 2 -- each attention dispatch and the MLP dispatch behind it as one
+ * node where both take their one-pass flavour.  Both are off by default: on this part a kernel boundary costs
+ * less than the barrier that replaces it.
  *
  * EXCLUSIVE USE OF THE DEVICE.  A launch of these families is 512 workgroups that wait for one another inside
  * the launch, so all of them must be resident at once, two per CU of all 256 CUs, dealt to the XCDs round-robin.
