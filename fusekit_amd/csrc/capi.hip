@@ -830,6 +830,19 @@ fk_status fk_xcd_workspace_bytes(uint32_t n_heads, uint32_t head_dim, size_t* co
 
 size_t fk_xcd_sum_row_bytes(uint32_t hidden) { return xcd_sum_row_bytes(hidden); }
 
+fk_status fk_xcd_moe_supported(uint32_t hidden, uint32_t inter, uint32_t shared_inter, uint32_t experts, uint32_t top_k,
+                               uint32_t bits, uint32_t group) {
+    return xcd_moe_supported(XcdMoeShape{hidden, inter, shared_inter, experts, top_k, bits, group});
+}
+
+size_t fk_xcd_moe_scratch_bytes(uint32_t inter, uint32_t shared_inter, uint32_t top_k) {
+    XcdMoeShape s{};
+    s.inter = inter;
+    s.shared_inter = shared_inter;
+    s.top_k = top_k;
+    return xcd_moe_scratch_bytes(s);
+}
+
 fk_status fk_xcd_kslice_meta(const uint16_t* src, uint32_t n, uint32_t groups, uint16_t* dst, fk_stream s) {
     return xcd_kslice_meta(src, n, groups, dst, (hipStream_t)s);
 }

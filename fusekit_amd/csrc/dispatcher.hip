@@ -843,6 +843,82 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     return plan_xcd_mlp(rq, l);
 }
 
+// The expert block of a mixture-of-experts layer as one XCD-resident launch (xcd_moe_kernel):
+// [sums_in], residual, x_out, norm_w, W_router (bf16 [experts, hidden]), route_scale, then (w, scales, biases) of the
+// expert gate, up, down stacks and of the shared gate, up, down matrices, logits_out [experts] bf16, idx_out [top_k]
+// uint32, weight_out [top_k] bf16, scratch (fk_xcd_moe_scratch_bytes), out_sums, clear_sums, workspace.
+// Parameters: hidden, inter, shared_inter, experts, top_k, bits, group, eps, variant, has_sums, spin_limit,
+// mark_placement.
+fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    XcdMoeShape s;
+    s.hidden = d.u("hidden");
+    s.inter = d.u("inter");
+    s.shared_inter = d.u("shared_inter");
+    s.experts = d.u("experts");
+    s.top_k = d.u("top_k");
+    s.bits = d.u("bits", 4);
+    s.group = d.u("group", 64);
+    const bool has_p = d.u("has_sums", 1) != 0;
+    size_t i = 0;
+    const size_t p_slot = has_p ? i++ : 0, res_slot = i++, x_slot = i++, nw_slot = i++, rw_slot = i++, rs_slot = i++, w_slot = i;
+    i += 18;
+    const size_t lo_slot = i++, io_slot = i++, wo_slot = i++, sc_slot = i++, op_slot = i++, clr_slot = i++, ws_slot = i++;
+    FK_TRY(need_args(d, i));
+    if (s.hidden == 0 || s.inter == 0 || s.shared_inter == 0 || s.experts == 0 || s.top_k == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": shape parameters missing");
+    if (s.bits != 4) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": 4-bit weights only");
+    XcdMoeRequest rq;
+    memset(&rq, 0, sizeof(rq));
+    rq.shape = s;
+    if (has_p) {
+        FK_TRY(need_bytes(d, p_slot, xcd_sum_row_bytes(s.hidden)));
+        rq.sums_in = arg_ptr<const long long>(d, p_slot);
+    }
+    FK_TRY(need_bytes(d, res_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, x_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, nw_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, rw_slot, (size_t)s.experts * s.hidden * 2));
+    FK_TRY(need_bytes(d, rs_slot, 2));
+    rq.residual = arg_ptr<const uint16_t>(d, res_slot);
+    rq.x_out = arg_ptr<uint16_t>(d, x_slot);
+    rq.norm_w = arg_ptr<const uint16_t>(d, nw_slot);
+    rq.eps = (float)d.param("eps", 1e-6);
+    rq.router_w = arg_ptr<const uint16_t>(d, rw_slot);
+    rq.route_scale = arg_ptr<const uint16_t>(d, rs_slot);
+    fk_weight W[6];
+    const uint32_t ns[6] = {s.experts * s.inter, s.experts * s.inter, s.experts * s.hidden, s.shared_inter, s.shared_inter, s.hidden};
+    const uint32_t ks[6] = {s.hidden, s.hidden, s.inter, s.hidden, s.hidden, s.shared_inter};
+    for (int m = 0; m < 6; ++m)
+        FK_TRY(bind_weight(d, s.bits, s.group, ns[m], ks[m], w_slot + 3 * m, w_slot + 3 * m + 1, w_slot + 3 * m + 2, &W[m]));
+    rq.gate = &W[0];
+    rq.up = &W[1];
+    rq.down = &W[2];
+    rq.sgate = &W[3];
+    rq.sup = &W[4];
+    rq.sdown = &W[5];
+    rq.swiglu_variant = (int)d.param("variant", 1);
+    FK_TRY(need_bytes(d, lo_slot, (size_t)s.experts * 2));
+    FK_TRY(need_bytes(d, io_slot, (size_t)s.top_k * 4));
+    FK_TRY(need_bytes(d, wo_slot, (size_t)s.top_k * 2));
+    rq.logits_out = arg_ptr<uint16_t>(d, lo_slot);
+    rq.idx_out = arg_ptr<uint32_t>(d, io_slot);
+    rq.weight_out = arg_ptr<uint16_t>(d, wo_slot);
+    FK_TRY(need_bytes(d, sc_slot, xcd_moe_scratch_bytes(s)));
+    rq.scratch = d.args[sc_slot].ptr;
+    FK_TRY(need_bytes(d, op_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.out_sums = arg_ptr<long long>(d, op_slot);
+    FK_TRY(need_bytes(d, clr_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.clear = arg_ptr<long long>(d, clr_slot);
+    FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
+    rq.workspace = d.args[ws_slot].ptr;
+    rq.spin_limit = d.u("spin_limit", 0);
+    rq.mark_placement = d.u("mark_placement", 0) != 0;
+    for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
+    rw->writes = {(uint32_t)x_slot, (uint32_t)lo_slot, (uint32_t)io_slot, (uint32_t)wo_slot, (uint32_t)sc_slot, (uint32_t)op_slot,
+                  (uint32_t)clr_slot, (uint32_t)ws_slot};
+    return plan_xcd_moe(rq, l);
+}
+
 // src, out (8 bytes per workgroup): the plain read kernel (parameter blocks_per_cu)
 fk_status plan_read_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_args(d, 2));
@@ -1297,6 +1373,7 @@ const Family kFamilies[] = {
     {"fusekit_xcd_attn_block", plan_xcd_attn_d},
     {"fusekit_xcd_mlp_block", plan_xcd_mlp_d},
     {"fusekit_xcd_reduce", plan_xcd_reduce_d},
+    {"fusekit_xcd_moe_block", plan_xcd_moe_d},
     {"fusekit_read_reduce", plan_read_reduce_d},
     {"fusekit_route_order", plan_route_order_d},
 };
@@ -1476,13 +1553,17 @@ std::vector<std::vector<uint64_t>> derive_edges(std::vector<Node>& nodes, const 
     return anc;
 }
 
+// The families whose launches are 512 workgroups that wait for one another (slots end: out_sums, clear_sums, workspace).
+bool is_xcd_launch(const std::string& kernel) {
+    return kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0 ||
+           kernel.compare(0, 21, "fusekit_xcd_moe_block") == 0;
+}
+
 // An XCD-resident launch needs the whole device to itself: its 512 workgroups must all be resident at once, two per
 // CU, and a kernel running beside it would hold CUs and leave some of them waiting (the hand-over waits would then
 // run into their spin limit).  Inside a graph that means every other node must be ordered before or after it.
 fk_status require_xcd_nodes_ordered(const std::vector<Node>& nodes, const std::vector<std::vector<uint64_t>>& anc) {
-    auto is_xcd = [](const Node& nd) {
-        return nd.d.kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || nd.d.kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0;
-    };
+    auto is_xcd = [](const Node& nd) { return is_xcd_launch(nd.d.kernel); };
     for (size_t i = 0; i < nodes.size(); ++i) {
         if (!is_xcd(nodes[i])) continue;
         for (size_t j = 0; j < nodes.size(); ++j) {
@@ -2028,7 +2109,7 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
     if (barriers) g->barriers.assign(barriers, barriers + n);
     for (size_t i = 0; i < n; ++i) {
         const Node& nd = g->nodes[i];
-        if (nd.d.kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || nd.d.kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0) {
+        if (is_xcd_launch(nd.d.kernel)) {
             void* ws = nd.d.args.back().ptr;
             if (std::find(g->xcd_controls.begin(), g->xcd_controls.end(), ws) == g->xcd_controls.end()) g->xcd_controls.push_back(ws);
             // slots: [sums_in], ..., out_sums, clear_sums, workspace (the planners have checked count and sizes)

@@ -172,6 +172,72 @@ struct XcdLayerArgs {
     uint32_t mark_placement;
 };
 
+// ---- the expert block of a mixture-of-experts layer as ONE launch ----------------------------------------------
+// router + routed gate / up + shared gate / up + routed down + shared down + weighted sum, cut BY ROUTE: XCD u < top_k
+// serves the u-th winner of the ranking entirely (its expert's gate / up rows, then its down_proj rows over the whole
+// intermediate width), the remaining XCDs serve the shared expert.  A route's FULL dot product is therefore formed,
+// rounded to T and weighted inside one XCD, exactly as the reference's reduction does it
+// (routed_qmv_reduce.rs:236-322); only the final sum over the routes crosses XCDs, through the sum row.
+//   every XCD      x1 = T(sum row + residual); RMSNorm; staged
+//   XCD u < top_k  block `slot` forms router logit `slot` (bf16 router row . normalised x) -> hand-over -> every wave
+//                  ranks the 64 logits (softmax, top-k) and takes winner u: expert e, weight w
+//                  -> gate / up rows [slot I/64, (slot+1) I/64) of expert e, SwiGLU -> hand-over
+//                  -> down_proj rows [slot H/64, ..) of expert e over all of I: w * T(dot) added into the sum row
+//   XCD u >= top_k (shared unit h = u - top_k of n_shared = 8 - top_k): ALL gate / up rows of the shared expert (every
+//                  shared XCD repeats them: no hand-over between XCDs), SwiGLU -> hand-over -> shared down_proj rows
+//                  [h H/n_shared, (h+1) H/n_shared) over the whole shared width: T(dot) added into the sum row
+// The shared XCDs do not wait for the ranking and start streaming at once, which offsets their larger gate / up share.
+struct XcdMoeArgs {
+    XcdInput in;
+    const uint16_t* router_w;      // bf16 [experts, hidden]
+    const uint16_t* route_scale;   // one bf16 value
+    XcdMat gate, up, down;         // expert stacks: [experts * inter, hidden] twice, [experts * hidden, inter]
+    XcdMat sgate, sup, sdown;      // shared expert: [shared_inter, hidden] twice, [hidden, shared_inter]
+    uint32_t experts, top_k, n_shared, inter;
+    uint32_t gu_rows;              // gate (and up) rows per block and unit: inter / 64
+    uint32_t down_rows;            // routed down_proj rows per block: hidden / 64
+    uint32_t sdown_rows;           // shared down_proj rows per block: hidden / (64 n_shared)
+    int swiglu_variant;
+    uint32_t* logits_xcd;          // [8][64] fp32 bits of the bf16 logits, every XCD its own copy
+    uint16_t* mid;                 // [top_k][inter], then per shared XCD [n_shared * inter]
+    uint16_t* logits_out;          // [experts] bf16, or null   } what the host reads back; written by one block
+    uint32_t* idx_out;             // [top_k] or null            }
+    uint16_t* weight_out;          // [top_k] or null            }
+    long long* out_sums;
+    XcdControl* ctl;
+    uint32_t spin_limit;
+    uint32_t cs_max, work_floats;
+    uint32_t mark_placement;
+};
+
+struct XcdMoeShape {
+    uint32_t hidden, inter, shared_inter, experts, top_k, bits, group;
+};
+fk_status xcd_moe_supported(const XcdMoeShape& s);
+size_t xcd_moe_scratch_bytes(const XcdMoeShape& s);   // logits_xcd + mid
+struct XcdMoeRequest {
+    XcdMoeShape shape;
+    const long long* sums_in;
+    const uint16_t* residual;
+    uint16_t* x_out;
+    long long* clear;
+    const uint16_t* norm_w;
+    float eps;
+    const uint16_t* router_w;
+    const uint16_t* route_scale;
+    const fk_weight *gate, *up, *down, *sgate, *sup, *sdown;
+    int swiglu_variant;
+    uint16_t* logits_out;
+    uint32_t* idx_out;
+    uint16_t* weight_out;
+    void* scratch;
+    long long* out_sums;
+    void* workspace;
+    uint32_t spin_limit;
+    bool mark_placement;
+};
+fk_status plan_xcd_moe(const XcdMoeRequest& rq, Launch* out);
+
 // x = T(f32(sums) + residual): the last layer's output for the LM head.  `clear` (may be the row read, or null)
 // is zeroed element by element behind the read: the row the next token's first launch adds into.
 struct XcdReduceArgs {

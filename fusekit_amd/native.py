@@ -559,6 +559,19 @@ def xcd_sum_row_bytes(hidden: int) -> int:
     return int(lib.fk_xcd_sum_row_bytes(C.c_uint32(hidden)))
 
 
+def xcd_moe_supported(hidden, inter, shared_inter, experts, top_k, bits, group) -> bool:
+    """Can the expert block of a layer of this shape run as one XCD-resident launch (fk_xcd_moe_supported)?"""
+    return lib.fk_xcd_moe_supported(C.c_uint32(hidden), C.c_uint32(inter), C.c_uint32(shared_inter), C.c_uint32(experts),
+                                    C.c_uint32(top_k), C.c_uint32(bits), C.c_uint32(group)) == FK_OK
+
+
+lib.fk_xcd_moe_scratch_bytes.restype = C.c_size_t
+
+
+def xcd_moe_scratch_bytes(inter: int, shared_inter: int, top_k: int) -> int:
+    return int(lib.fk_xcd_moe_scratch_bytes(C.c_uint32(inter), C.c_uint32(shared_inter), C.c_uint32(top_k)))
+
+
 def xcd_kslice_meta(src: "DeviceBuffer", n: int, groups: int, stream=None) -> "DeviceBuffer":
     """The per-XCD re-laid-out copy of a scale or bias array [n, groups] (fk_xcd_kslice_meta)."""
     dst = DeviceBuffer(n * groups * 2)

@@ -1,0 +1,146 @@
+"""The expert block of a mixture-of-experts layer as ONE XCD-resident launch (family fusekit_xcd_moe_block: router,
+ranking, routed + shared gate / up with SwiGLU, routed + shared down_proj, weighted sum into a sum row) against the
+oracle's composition of the reference's kernels, through the C ABI (dispatcher).
+
+Bars: the router logits are fp32 dot products rounded once (equal to the oracle's except on a rounding edge); the routes
+must be EXACTLY the oracle's ranking of the GPU's own logits; SwiGLU rows to the bar of the routed kernels (equal to the
+oracle's except where gate or up sits on a rounding edge or nearly cancels); the block's output (sum row + residual, rounded once)
+equals the oracle's reduction over the GPU's own SwiGLU rows except on a rounding edge (<= 1 ulp on <= 2 %)."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import bf16_mismatch, make_qweight, normal_bf16, rel_l2, rng, to_device
+from test_gemv_gpu import _check_swiglu
+from test_xcd_layer_gpu import _dev, _input_ref, _row_values, _sum_row
+
+pytestmark = pytest.mark.gpu
+
+EPS = 1e-6
+SHAPES = [  # hidden, inter, shared_inter, experts, top_k
+    (512, 128, 256, 16, 6),
+    (1024, 256, 512, 64, 6),
+    (512, 128, 128, 8, 7),          # one shared unit
+    (2048, 1408, 2816, 64, 6),      # the benchmark model's expert layers
+]
+
+
+def _stack(seed, n_experts, n, k):
+    return oracle.StackedWeight([make_qweight(seed + e, n, k, 4) for e in range(n_experts)])
+
+
+def _wargs(arg, W):
+    return [arg(W.w), arg(W.scales), arg(W.biases)]
+
+
+@pytest.mark.parametrize("hidden,inter,shared,experts,top_k", SHAPES)
+@pytest.mark.parametrize("has_sums", [0, 1])
+def test_xcd_moe_block(fk, hidden, inter, shared, experts, top_k, has_sums):
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    if not fk.xcd_moe_supported(hidden, inter, shared, experts, top_k, 4, 64):
+        pytest.skip("shape not supported: " + fk.lib.fk_last_error().decode())
+    d = Dispatcher()
+    n_shared = shared // inter
+    Eg, Eu, Ed = _stack(100, experts, inter, hidden), _stack(300, experts, inter, hidden), _stack(500, experts, hidden, inter)
+    Sg, Su, Sd = make_qweight(701, shared, hidden, 4), make_qweight(702, shared, hidden, 4), make_qweight(703, hidden, shared, 4)
+    Wr = normal_bf16(704, (experts, hidden), 0.05)
+    norm_w = normal_bf16(705, hidden, 0.1, 1.0)
+    scale = oracle.f32_to_bf16(np.array([1.5], np.float32))
+    res = normal_bf16(706, hidden)
+    partials = (rng(707).standard_normal((8, hidden), dtype=np.float32) * 0.3).astype(np.float32)
+    dE = [to_device(fk, W) for W in (Eg, Eu, Ed, Sg, Su, Sd)]
+    ctl_bytes, _ = fk.xcd_workspace_bytes(32, 128)
+    ctl = fk.zeros(ctl_bytes)
+    row_in = _sum_row(fk, hidden, partials)
+    junk = np.full_like(row_in, 0x0123456789abcdef)
+    scratch_bytes = fk.xcd_moe_scratch_bytes(inter, shared, top_k)
+    assert scratch_bytes == 8 * 64 * 4 + (top_k * inter + n_shared * shared) * 2
+    b = dict(p=_dev(fk, row_in), res=_dev(fk, res), x=fk.DeviceBuffer(hidden * 2), nw=_dev(fk, norm_w), wr=_dev(fk, Wr),
+             rs=_dev(fk, scale), lo=fk.zeros(experts * 2), io=fk.zeros(top_k * 4), wo=fk.zeros(top_k * 2),
+             sc=fk.zeros(scratch_bytes), out=_dev(fk, _sum_row(fk, hidden)), clr=_dev(fk, junk))
+    a = ([arg(b["p"])] if has_sums else []) + [arg(b["res"]), arg(b["x"]), arg(b["nw"]), arg(b["wr"]), arg(b["rs"])]
+    for W in dE:
+        a += _wargs(arg, W)
+    a += [arg(b["lo"]), arg(b["io"]), arg(b["wo"]), arg(b["sc"]), arg(b["out"]), arg(b["clr"]), arg(ctl)]
+    task = Dispatch("fusekit_xcd_moe_block_f1", a,
+                    dict(hidden=hidden, inter=inter, shared_inter=shared, experts=experts, top_k=top_k, bits=4, group=64,
+                         eps=EPS, variant=1, has_sums=has_sums))
+    for rep in range(2):                                  # twice: the arrival words carry over between launches
+        d.dispatch_kernel(task)
+        fk.xcd_check(ctl)
+        x1 = _input_ref(fk, row_in, hidden, res) if has_sums else res
+        assert np.array_equal(b["x"].to_numpy(np.uint16), x1), "the launch's input row differs"
+        assert not b["clr"].to_numpy(np.int64).any(), "the third sum row was not cleared"
+        xn = oracle.rmsnorm(x1, norm_w, EPS)
+        # router logits: fp32 dot products of bf16 rows, rounded once
+        logits = b["lo"].to_numpy(np.uint16)
+        logits_ref = oracle.qgemv(oracle.dense(Wr), xn)
+        f, u = bf16_mismatch(logits, logits_ref)
+        assert f <= 0.1 and u <= 1.0, (f, u)
+        # every XCD that ranks holds the same logits
+        per_xcd = b["sc"].to_numpy(np.uint8)[:8 * 64 * 4].view(np.uint32).reshape(8, 64)
+        for xcd in range(top_k):
+            assert np.array_equal((per_xcd[xcd, :experts] >> 16).astype(np.uint16), logits)
+            assert not (per_xcd[xcd, :experts] & 0xffff).any()
+        # the routes: the oracle's ranking of the GPU's logits, bit for bit
+        idx_ref, w_ref = oracle.softmax_topk_route(logits, top_k, scale)
+        idx, rw = b["io"].to_numpy(np.uint32), b["wo"].to_numpy(np.uint16)
+        assert np.array_equal(idx, idx_ref[0]) and np.array_equal(rw, w_ref[0])
+        # SwiGLU rows of the routes and of the shared expert (every shared XCD its own copy)
+        mid = b["sc"].to_numpy(np.uint8)[8 * 64 * 4:].view(np.uint16)
+        h = mid[:top_k * inter].reshape(top_k, inter)
+        h_ref = oracle.routed_qmv_swiglu(xn.reshape(1, -1), Eg, Eu, np.zeros(top_k, np.uint32), idx, None)
+        for r in range(top_k):
+            _check_swiglu(h[r], h_ref[r], xn, Eg.expert(int(idx[r])), Eu.expert(int(idx[r])), 1)
+        sh_ref = oracle.gateup_swiglu(xn, None, 0.0, Sg, Su, 1)
+        sh = mid[top_k * inter:].reshape(n_shared, shared)
+        for c in range(n_shared):
+            _check_swiglu(sh[c], sh_ref, xn, Sg, Su, 1)
+        for c in range(1, n_shared):
+            assert np.array_equal(sh[c], sh[0]), "the shared XCDs must agree on the shared expert's rows"
+        # the sum row: every term is w * T(dot) resp. T(dot), added exactly -- against float64 on the GPU's own rows
+        row_out = b["out"].to_numpy(np.int64)
+        out = _row_values(fk, row_out, hidden)
+        ref64 = np.zeros(hidden)
+        term_ulp = np.zeros(hidden)
+        for r in range(top_k):
+            w = float(oracle.bf16_to_f32(rw[r:r + 1])[0])
+            dot = oracle.bf16_to_f32(oracle.qgemv(Ed.expert(int(idx[r])), h[r])).astype(np.float64)
+            ref64 += w * dot
+            term_ulp += w * 2.0 ** (np.floor(np.log2(np.maximum(np.abs(dot), 1e-30))) - 7)
+        dot = oracle.bf16_to_f32(oracle.qgemv(Sd, sh[0])).astype(np.float64)
+        ref64 += dot
+        term_ulp += 2.0 ** (np.floor(np.log2(np.maximum(np.abs(dot), 1e-30))) - 7)
+        # a term whose dot product sat on a rounding edge may differ by one bf16 step of that term
+        assert np.all(np.abs(out - ref64) <= term_ulp + 1e-6 * np.abs(ref64) + 8 * 2.0 ** -32)
+        assert np.mean(np.abs(out - ref64) > 1e-6 * np.abs(ref64) + 8 * 2.0 ** -32) <= 0.05
+        pad = np.ones(row_out.size, bool)
+        pad[fk.xcd_sum_index(hidden)] = False
+        assert not row_out[pad].any()
+        # and what the next launch reads from it: the reference's reduction (routes in slot order, shared expert, residual)
+        y = _input_ref(fk, row_out, hidden, x1)
+        y_ref = oracle.routed_qmv_reduce(h, Ed, idx, rw, x1.reshape(1, -1), 1, top_k, shared_x=sh[0].reshape(1, -1), Wshared=Sd)[0]
+        # (a route whose dot product sat on a rounding edge moves the sum by one bf16 step of THAT TERM, which may exceed
+        # a step of a smaller result)
+        yf, rf = oracle.bf16_to_f32(y).astype(np.float64), oracle.bf16_to_f32(y_ref).astype(np.float64)
+        step = 2.0 ** (np.floor(np.log2(np.maximum(np.maximum(np.abs(yf), np.abs(rf)), 1e-30))) - 7)
+        assert np.mean(y != y_ref) <= 0.02 and np.all(np.abs(yf - rf) <= step + term_ulp)
+        assert rel_l2(y, ref64 + oracle.bf16_to_f32(x1)) <= 1e-2
+        # second round on other inputs
+        partials = (partials * 0.5).astype(np.float32)
+        row_in = _sum_row(fk, hidden, partials)
+        res = normal_bf16(710 + rep, hidden)
+        b["p"].upload(row_in)
+        b["res"].upload(res)
+        b["out"].upload(_sum_row(fk, hidden))
+        b["clr"].upload(junk)
+
+
+def test_xcd_moe_admission_needs_no_device_for_the_shape_rules(fk):
+    u = fk.xcd_moe_supported
+    assert u(2048, 1408, 2816, 64, 6, 4, 64), fk.lib.fk_last_error().decode()
+    assert not u(2048, 1408, 2816, 64, 6, 8, 64) and b"4-bit" in fk.lib.fk_last_error()
+    assert not u(2048, 1408, 2816, 128, 6, 4, 64) and b"64 experts" in fk.lib.fk_last_error()
+    assert not u(2048, 1408, 1408, 64, 6, 4, 64) and b"must be 8" in fk.lib.fk_last_error()
+    assert not u(2048, 1400, 2800, 64, 6, 4, 64) and b"multiples of 64" in fk.lib.fk_last_error()
+    assert not u(4096, 2048, 4096, 64, 6, 4, 64) and b"chunks" in fk.lib.fk_last_error()
