@@ -835,11 +835,9 @@ fk_status fk_xcd_moe_supported(uint32_t hidden, uint32_t inter, uint32_t shared_
     return xcd_moe_supported(XcdMoeShape{hidden, inter, shared_inter, experts, top_k, bits, group});
 }
 
-size_t fk_xcd_moe_scratch_bytes(uint32_t inter, uint32_t shared_inter, uint32_t top_k) {
+size_t fk_xcd_moe_scratch_bytes(uint32_t inter) {
     XcdMoeShape s{};
     s.inter = inter;
-    s.shared_inter = shared_inter;
-    s.top_k = top_k;
     return xcd_moe_scratch_bytes(s);
 }
 

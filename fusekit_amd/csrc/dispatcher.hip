@@ -846,7 +846,8 @@ fk_status plan_xcd_mlp_d(const Dispatch& d, Launch* l, SlotRW* rw) {
 // The expert block of a mixture-of-experts layer as one XCD-resident launch (xcd_moe_kernel):
 // [sums_in], residual, x_out, norm_w, W_router (bf16 [experts, hidden]), route_scale, then (w, scales, biases) of the
 // expert gate, up, down stacks and of the shared gate, up, down matrices, logits_out [experts] bf16, idx_out [top_k]
-// uint32, weight_out [top_k] bf16, scratch (fk_xcd_moe_scratch_bytes), out_sums, clear_sums, workspace.
+// uint32, weight_out [top_k] bf16, scratch (fk_xcd_moe_scratch_bytes), shared_sums (the sum row of the shared expert's
+// dot products, zero on entry), out_sums, clear_sums, workspace.
 // Parameters: hidden, inter, shared_inter, experts, top_k, bits, group, eps, variant, has_sums, spin_limit,
 // mark_placement.
 fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
@@ -862,7 +863,7 @@ fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     size_t i = 0;
     const size_t p_slot = has_p ? i++ : 0, res_slot = i++, x_slot = i++, nw_slot = i++, rw_slot = i++, rs_slot = i++, w_slot = i;
     i += 18;
-    const size_t lo_slot = i++, io_slot = i++, wo_slot = i++, sc_slot = i++, op_slot = i++, clr_slot = i++, ws_slot = i++;
+    const size_t lo_slot = i++, io_slot = i++, wo_slot = i++, sc_slot = i++, op2_slot = i++, op_slot = i++, clr_slot = i++, ws_slot = i++;
     FK_TRY(need_args(d, i));
     if (s.hidden == 0 || s.inter == 0 || s.shared_inter == 0 || s.experts == 0 || s.top_k == 0)
         return set_error(FK_ERR_INVALID, d.kernel + ": shape parameters missing");
@@ -905,6 +906,8 @@ fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     rq.weight_out = arg_ptr<uint16_t>(d, wo_slot);
     FK_TRY(need_bytes(d, sc_slot, xcd_moe_scratch_bytes(s)));
     rq.scratch = d.args[sc_slot].ptr;
+    FK_TRY(need_bytes(d, op2_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.out_sums2 = arg_ptr<long long>(d, op2_slot);
     FK_TRY(need_bytes(d, op_slot, xcd_sum_row_bytes(s.hidden)));
     rq.out_sums = arg_ptr<long long>(d, op_slot);
     FK_TRY(need_bytes(d, clr_slot, xcd_sum_row_bytes(s.hidden)));
@@ -914,8 +917,8 @@ fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     rq.spin_limit = d.u("spin_limit", 0);
     rq.mark_placement = d.u("mark_placement", 0) != 0;
     for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
-    rw->writes = {(uint32_t)x_slot, (uint32_t)lo_slot, (uint32_t)io_slot, (uint32_t)wo_slot, (uint32_t)sc_slot, (uint32_t)op_slot,
-                  (uint32_t)clr_slot, (uint32_t)ws_slot};
+    rw->writes = {(uint32_t)x_slot, (uint32_t)lo_slot, (uint32_t)io_slot, (uint32_t)wo_slot, (uint32_t)sc_slot, (uint32_t)op2_slot,
+                  (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
     return plan_xcd_moe(rq, l);
 }
 
@@ -927,9 +930,12 @@ fk_status plan_read_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     return plan_read_reduce(d.args[0].ptr, d.args[0].nbytes, d.args[1].ptr, d.args[1].nbytes, d.u("blocks_per_cu", 0), l);
 }
 
-// sum row, residual [hidden] bf16, x [hidden] bf16, sum row to clear (may be the one read) (parameter hidden)
+// sum row, residual [hidden] bf16, x [hidden] bf16, sum row to clear (may be the one read) [, second sum row, second row
+// to clear]: x = T(f32(row) + residual), with a second row x = T((f32(row) + T(f32(second row))) + residual)
+// (parameter hidden)
 fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
-    FK_TRY(need_args(d, 4));
+    const bool two = d.args.size() >= 6;
+    FK_TRY(need_args(d, two ? 6 : 4));
     const uint32_t hidden = d.u("hidden");
     if (hidden == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden parameter missing");
     FK_TRY(need_bytes(d, 0, xcd_sum_row_bytes(hidden)));
@@ -938,8 +944,15 @@ fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_bytes(d, 3, xcd_sum_row_bytes(hidden)));
     rw->reads = {0, 1};
     rw->writes = {2, 3};
+    if (two) {
+        FK_TRY(need_bytes(d, 4, xcd_sum_row_bytes(hidden)));
+        FK_TRY(need_bytes(d, 5, xcd_sum_row_bytes(hidden)));
+        rw->reads.push_back(4);
+        rw->writes.push_back(5);
+    }
     return plan_xcd_reduce(arg_ptr<const long long>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<uint16_t>(d, 2),
-                           arg_ptr<long long>(d, 3), hidden, l);
+                           arg_ptr<long long>(d, 3), hidden, l, two ? arg_ptr<const long long>(d, 4) : nullptr,
+                           two ? arg_ptr<long long>(d, 5) : nullptr);
 }
 
 // Q, K0, K1, V, cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]: split-key store + attention of a
@@ -2121,6 +2134,7 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
             };
             add_row(nd.d.args[na - 3].ptr);
             add_row(nd.d.args[na - 2].ptr);
+            if (nd.d.kernel.compare(0, 21, "fusekit_xcd_moe_block") == 0) add_row(nd.d.args[na - 4].ptr);  // the shared expert's row
             if (nd.d.u("has_sums", 1) != 0) add_row(nd.d.args[0].ptr);
         }
     }

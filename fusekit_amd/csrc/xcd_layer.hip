@@ -449,7 +449,13 @@ __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs 
     if (i >= a.hidden) return;
     const uint32_t at = xcd_sum_index(i);
     const unsigned long long s = (unsigned long long)a.sums[at];
-    a.x[i] = (uint16_t)f32_to_bf16_bits(xcd_sum_to_f32((uint32_t)s, (uint32_t)(s >> 32)) + bf16_bits_to_f32(a.residual[i]));
+    float v = xcd_sum_to_f32((uint32_t)s, (uint32_t)(s >> 32));
+    if (a.sums2) {
+        const unsigned long long s2 = (unsigned long long)a.sums2[at];
+        v = __fadd_rn(v, round_bf16(xcd_sum_to_f32((uint32_t)s2, (uint32_t)(s2 >> 32))));
+        if (a.clear2) a.clear2[at] = 0;
+    }
+    a.x[i] = (uint16_t)f32_to_bf16_bits(v + bf16_bits_to_f32(a.residual[i]));
     if (a.clear) a.clear[at] = 0;
 }
 
@@ -884,11 +890,11 @@ fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uin
 }
 
 fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
-                          Launch* out) {
+                          Launch* out, const long long* sums2, long long* clear2) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!sums || !residual || !x || hidden == 0) return set_error(FK_ERR_INVALID, "xcd reduce: null buffer or zero width");
-    XcdReduceArgs a{sums, residual, x, clear, hidden};
+    XcdReduceArgs a{sums, residual, x, clear, hidden, sums2, clear2};
     out->func = reinterpret_cast<const void*>(&xcd_reduce_kernel);
     out->grid = dim3(ceil_div(hidden, kBlock), 1, 1);
     out->block = dim3(kBlock, 1, 1);

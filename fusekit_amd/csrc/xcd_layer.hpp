@@ -175,18 +175,19 @@ struct XcdLayerArgs {
 // ---- the expert block of a mixture-of-experts layer as ONE launch ----------------------------------------------
 // router + routed gate / up + shared gate / up + routed down + shared down + weighted sum, cut BY ROUTE: XCD u < top_k
 // serves the u-th winner of the ranking entirely (its expert's gate / up rows, then its down_proj rows over the whole
-// intermediate width), the remaining XCDs serve the shared expert.  A route's FULL dot product is therefore formed,
-// rounded to T and weighted inside one XCD, exactly as the reference's reduction does it
-// (routed_qmv_reduce.rs:236-322); only the final sum over the routes crosses XCDs, through the sum row.
+// intermediate width).  A route's FULL dot product is therefore formed, rounded to T and weighted inside one XCD,
+// exactly as the reference's reduction does it (routed_qmv_reduce.rs:236-322); only the final sum over the routes
+// crosses XCDs, through the sum row.  The shared expert (width n_shared x an expert's) is n_shared more units of the
+// same size on the following XCDs: unit h takes its gate / up rows [h I, (h+1) I) and the K-slice of the shared
+// down_proj that those rows feed; its partial dot products go UNROUNDED into a second sum row, whose finished element
+// is the shared expert's full dot product -- rounded to T where the row is read.  Every XCD streams the same bytes.
 //   every XCD      x1 = T(sum row + residual); RMSNorm; staged
 //   XCD u < top_k  block `slot` forms router logit `slot` (bf16 router row . normalised x) -> hand-over -> every wave
 //                  ranks the 64 logits (softmax, top-k) and takes winner u: expert e, weight w
-//                  -> gate / up rows [slot I/64, (slot+1) I/64) of expert e, SwiGLU -> hand-over
-//                  -> down_proj rows [slot H/64, ..) of expert e over all of I: w * T(dot) added into the sum row
-//   XCD u >= top_k (shared unit h = u - top_k of n_shared = 8 - top_k): ALL gate / up rows of the shared expert (every
-//                  shared XCD repeats them: no hand-over between XCDs), SwiGLU -> hand-over -> shared down_proj rows
-//                  [h H/n_shared, (h+1) H/n_shared) over the whole shared width: T(dot) added into the sum row
-// The shared XCDs do not wait for the ranking and start streaming at once, which offsets their larger gate / up share.
+//   every unit     gate / up rows [slot I/64, (slot+1) I/64) of the unit, SwiGLU -> hand-over
+//                  -> down_proj rows [slot H/64, ..) over the unit's intermediate row:
+//                  routed: w * T(dot) into the sum row; shared: the partial dot into the second sum row
+// What reads the rows forms x2 = T((f32(row) + T(f32(second row))) + residual): the reference's order of additions.
 struct XcdMoeArgs {
     XcdInput in;
     const uint16_t* router_w;      // bf16 [experts, hidden]
@@ -194,16 +195,16 @@ struct XcdMoeArgs {
     XcdMat gate, up, down;         // expert stacks: [experts * inter, hidden] twice, [experts * hidden, inter]
     XcdMat sgate, sup, sdown;      // shared expert: [shared_inter, hidden] twice, [hidden, shared_inter]
     uint32_t experts, top_k, n_shared, inter;
-    uint32_t gu_rows;              // gate (and up) rows per block and unit: inter / 64
-    uint32_t down_rows;            // routed down_proj rows per block: hidden / 64
-    uint32_t sdown_rows;           // shared down_proj rows per block: hidden / (64 n_shared)
+    uint32_t gu_rows;              // gate (and up) rows per block: inter / 64
+    uint32_t down_rows;            // down_proj rows per block: hidden / 64
     int swiglu_variant;
     uint32_t* logits_xcd;          // [8][64] fp32 bits of the bf16 logits, every XCD its own copy
-    uint16_t* mid;                 // [top_k][inter], then per shared XCD [n_shared * inter]
+    uint16_t* mid;                 // [8][inter]: the SwiGLU row of every unit
     uint16_t* logits_out;          // [experts] bf16, or null   } what the host reads back; written by one block
     uint32_t* idx_out;             // [top_k] or null            }
     uint16_t* weight_out;          // [top_k] or null            }
-    long long* out_sums;
+    long long* out_sums;           // the routes' weighted outputs
+    long long* out_sums2;          // the shared expert's dot products
     XcdControl* ctl;
     uint32_t spin_limit;
     uint32_t cs_max, work_floats;
@@ -232,6 +233,7 @@ struct XcdMoeRequest {
     uint16_t* weight_out;
     void* scratch;
     long long* out_sums;
+    long long* out_sums2;
     void* workspace;
     uint32_t spin_limit;
     bool mark_placement;
@@ -246,6 +248,9 @@ struct XcdReduceArgs {
     uint16_t* x;
     long long* clear;
     uint32_t hidden;
+    // with a second row (the shared expert's of the expert launch): x = T((f32(sums) + T(f32(sums2))) + residual)
+    const long long* sums2;
+    long long* clear2;
 };
 
 struct XcdLayerShape {
@@ -322,6 +327,6 @@ fk_status plan_xcd_layer(const Launch& attn, const Launch& mlp, Launch* out);
 fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uint32_t n_layers, uint32_t bits,
                          const XcdAttnArgs* d_attn, const XcdMlpArgs* d_mlp, uint32_t attn_lds, uint32_t mlp_lds, Launch* out);
 fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
-                          Launch* out);
+                          Launch* out, const long long* sums2 = nullptr, long long* clear2 = nullptr);
 
 }  // namespace fk

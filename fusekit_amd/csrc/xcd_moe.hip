@@ -15,7 +15,6 @@ FK_PROBE_DEFINE(xcd_moe, 512, 16)
 namespace fk {
 
 constexpr int kMoeNl = 6;        // 16-byte requests per thread and tile: a tile holds at most 6 * 256 chunks
-constexpr uint32_t kMoeMaxShared = 2;
 
 namespace {
 
@@ -53,6 +52,22 @@ __device__ __forceinline__ XcdMat pick_mat(bool first, const XcdMat& a, const Xc
     m.cpr = first ? a.cpr : b.cpr;
     m.gshift = first ? a.gshift : b.gshift;
     return m;
+}
+
+// Scales and biases of a tile that may be a K-slice of the matrix's rows (MLX layout: [row][groups of the row]), one
+// group per lane and request: group gi of the tile = (row gi / gpr, group gi % gpr of the slice).
+template <WKind KIND, int SN, typename MAT>
+__device__ __forceinline__ void meta_fetch_slice(const MAT& m, const Tile& t, uint32_t ti, MetaRegs& r) {
+    const uint32_t gpr = t.cs >> m.gshift, total = t.rows * gpr, full = m.cpr >> m.gshift, g0 = t.col0 >> m.gshift;
+    const float inv = 1.0f / (float)gpr;
+#pragma unroll
+    for (int k = 0; k < kMetaRegs; ++k) {
+        const uint32_t gi = k * SN + ti;
+        const uint32_t row = (uint32_t)(((float)gi + 0.5f) * inv);
+        const size_t e = gi < total ? (size_t)(t.row0 + row) * full + g0 + (gi - row * gpr) : (size_t)t.row0 * full + g0;
+        r.s[k] = m.sc[e];
+        r.b[k] = m.bi[e];
+    }
 }
 
 // input_stage of the dense launches, with the router's dot product taken on the way: x = T(sums + residual), its sum
@@ -136,27 +151,17 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
     const bool routed = unit < a.top_k;                   // block-uniform
     const uint32_t sh = routed ? 0u : unit - a.top_k;     // shared unit
     const bool idle = !routed && sh >= a.n_shared;        // an XCD without a unit (top_k + n_shared < 8)
-    const uint32_t n_sub = routed ? 1u : a.n_shared;      // gate / up sub-tiles of this block
     const XcdMat G = pick_mat(routed, a.gate, a.sgate), U = pick_mat(routed, a.up, a.sup), D = pick_mat(routed, a.down, a.sdown);
 
-    // Every set of weight registers has ONE point in the program where it is requested (a set requested at either of
-    // two points ends up in private memory).  Set E ("early") is used by the shared XCDs only: the first half of the
-    // shared expert's rows, requested at once.  Set L ("late") is requested by everyone behind the ranking: a routed
-    // XCD's expert rows, a shared XCD's second half (or, with one shared unit per XCD's worth of rows, its only half).
-    TileRegs<NL> rgE, ruE, rgL, ruL, rd;
-    MetaRegs mgE, muE, mgL, muL, md;
-    TilePos<NL> pgE, pgL, pd;
+    // A shared unit is served like a route: unit h of the shared expert is its gate / up rows [h I, (h+1) I) and, in
+    // down_proj, the K-slice of those rows' outputs -- a partial dot product per output row, added UNROUNDED into the
+    // second sum row, whose finished element is the shared expert's full dot product (rounded to T where it is read).
+    // Every XCD therefore streams the same number of bytes.
+    TileRegs<NL> rg, ru, rd;
+    MetaRegs mg, mu, md;
+    TilePos<NL> pg, pd;
 
     const uint32_t gu0 = sync.slot * a.gu_rows;
-    const bool two = !routed && !idle && a.n_shared > 1;   // block-uniform: this block walks two gate / up sub-tiles
-    const Tile tgE = make_tile(gu0, two ? a.gu_rows : 0u, 0, G.cpr);
-    tile_pos_init<NL, kBlock>(G, tgE, tid, pgE);
-    if (two) {
-        meta_fetch<KIND, kBlock, true>(G, tgE, tid, mgE);
-        meta_fetch<KIND, kBlock, true>(U, tgE, tid, muE);
-        tile_load<KIND, NL, kBlock>(G, tgE, pgE, rgE);
-        tile_load<KIND, NL, kBlock>(U, tgE, pgE, ruE);
-    }
     const bool with_router = routed && sync.slot < a.experts;
     uint4 rw[kInGroups];
     {
@@ -169,6 +174,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
             if (routed && (t >> 6) * kWave < n8) rw[i] = w8[t < n8 ? t : 0u];
         }
     }
+    const float sc = bf16_bits_to_f32(a.route_scale[0]);
     FK_XCD_STAMP(0, 1);
     input_pin(lead, inr);
     float dot = moe_input_stage<KIND>(a.in, inr, rw, with_router, xs, sx, G.cpr, red);
@@ -197,7 +203,6 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
         if (lane < a.experts) x[0] = __uint_as_float(__hip_atomic_load(lg + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
         uint32_t key[4];
         route_candidates(x, a.experts, lane, key);
-        const float sc = bf16_bits_to_f32(a.route_scale[0]);
         const bool reporter = unit == 0 && sync.slot == 0 && tid == 0;
         for (uint32_t k = 0; k < a.top_k; ++k) {
             float best;
@@ -215,70 +220,58 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
         }
         expert = __builtin_amdgcn_readfirstlane(expert);
     }
-    // ---- set L: the expert's rows (routed), the shared expert's remaining rows (shared) ----
-    const uint32_t rowL = routed ? expert * a.inter + gu0 : (two ? a.inter : 0u) + gu0;
-    const Tile tgL = make_tile(rowL, idle ? 0u : a.gu_rows, 0, G.cpr);
-    tile_pos_init<NL, kBlock>(G, tgL, tid, pgL);
-    meta_fetch<KIND, kBlock, true>(G, tgL, tid, mgL);
-    meta_fetch<KIND, kBlock, true>(U, tgL, tid, muL);
-    tile_load<KIND, NL, kBlock>(G, tgL, pgL, rgL);
-    tile_load<KIND, NL, kBlock>(U, tgL, pgL, ruL);
+    // ---- the unit's gate / up rows: the expert's (routed), rows [h I, (h+1) I) of the shared expert (shared) ----
+    const uint32_t row_gu = (routed ? expert : sh) * a.inter + gu0;
+    const Tile tg = make_tile(row_gu, idle ? 0u : a.gu_rows, 0, G.cpr);
+    tile_pos_init<NL, kBlock>(G, tg, tid, pg);
+    meta_fetch<KIND, kBlock, true>(G, tg, tid, mg);
+    meta_fetch<KIND, kBlock, true>(U, tg, tid, mu);
+    tile_load<KIND, NL, kBlock>(G, tg, pg, rg);
+    tile_load<KIND, NL, kBlock>(U, tg, pg, ru);
     FK_XCD_STAMP(0, 4);
 
-    // down_proj tile of this block
-    const uint32_t drows = routed ? a.down_rows : a.sdown_rows;
-    const uint32_t out0 = routed ? sync.slot * a.down_rows : sh * (hidden / (a.n_shared ? a.n_shared : 1u)) + sync.slot * a.sdown_rows;
-    const Tile td = make_tile(routed ? expert * hidden + out0 : out0, idle ? 0u : drows, 0, D.cpr);
+    // down_proj tile of this block: its output rows x the unit's intermediate columns (all of an expert's row, the
+    // unit's K-slice of the shared expert's)
+    const uint32_t out0 = sync.slot * a.down_rows, dcs = a.down.cpr;
+    const Tile td = make_tile(routed ? expert * hidden + out0 : out0, idle ? 0u : a.down_rows, routed ? 0u : sh * dcs, dcs);
     tile_pos_init<NL, kBlock>(D, td, tid, pd);
 
-    uint16_t* mid = routed ? a.mid + (size_t)unit * a.inter : a.mid + (size_t)a.top_k * a.inter + (size_t)sh * a.n_shared * a.inter;
+    uint16_t* mid = a.mid + (size_t)unit * a.inter;
     const int variant = a.swiglu_variant;
     constexpr uint32_t seg = NL * kBlock;
-    if (two) {   // first half of the shared rows
-        meta_store<KIND, kBlock, true>(mgE, tid, meta);
-        meta_store<KIND, kBlock, true>(muE, tid, meta + MW);
-        __syncthreads();
-        tile_partials<KIND, NL, kBlock>(G, tgE, pgE, rgE, xs, sx, meta, work);
-        tile_partials<KIND, NL, kBlock>(U, tgE, pgE, ruE, xs, sx, meta + MW, work + seg);
-        __syncthreads();
-        tile_rows<true, true>(tgE, work, work + seg,
-                              [&](uint32_t r, float s0, float s1) { mid[gu0 + r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
-    }
-    meta_store<KIND, kBlock, true>(mgL, tid, meta);
-    meta_store<KIND, kBlock, true>(muL, tid, meta + MW);
+    meta_store<KIND, kBlock, true>(mg, tid, meta);
+    meta_store<KIND, kBlock, true>(mu, tid, meta + MW);
     __syncthreads();
-    tile_partials<KIND, NL, kBlock>(G, tgL, pgL, rgL, xs, sx, meta, work);
-    tile_partials<KIND, NL, kBlock>(U, tgL, pgL, ruL, xs, sx, meta + MW, work + seg);
+    tile_partials<KIND, NL, kBlock>(G, tg, pg, rg, xs, sx, meta, work);
+    tile_partials<KIND, NL, kBlock>(U, tg, pg, ru, xs, sx, meta + MW, work + seg);
     // the down_proj rows are requested behind the gate / up arithmetic: not needed before the hand-over
-    meta_fetch<KIND, kBlock, true>(D, td, tid, md);
+    meta_fetch_slice<KIND, kBlock>(D, td, tid, md);
     tile_load<KIND, NL, kBlock>(D, td, pd, rd);
     FK_XCD_STAMP(0, 5);
     __syncthreads();
-    if (!idle) {
-        uint16_t* m2 = mid + (two ? a.inter : 0u) + gu0;
-        tile_rows<true, true>(tgL, work, work + seg,
-                              [&](uint32_t r, float s0, float s1) { m2[r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
-    }
+    if (!idle)
+        tile_rows<true, true>(tg, work, work + seg,
+                              [&](uint32_t r, float s0, float s1) { mid[gu0 + r] = (uint16_t)swiglu_bits(s0, s1, variant, 1.0f); });
     FK_XCD_STAMP(0, 6);
-    meta_store<KIND, kBlock, true>(md, tid, meta + 2 * MW);
+    meta_store<KIND, kBlock, false>(md, tid, meta + 2 * MW);
     xcd_barrier<0>(sync, okw);
-    const bool ok = xcd_wait_ok(okw);  // tested in front of the additions into the sum row
+    const bool ok = xcd_wait_ok(okw);  // tested in front of the additions into the sum rows
     FK_XCD_STAMP(0, 7);
 
-    // ---- down_proj of the unit over its whole intermediate row ----
-    if (!idle) stage_vector<KIND>(mid, (n_sub * a.inter) >> 3, D.cpr, xs, sx);
+    // ---- down_proj of the unit over its intermediate row ----
+    if (!idle) stage_vector<KIND>(mid, a.inter >> 3, dcs, xs, sx);
     __syncthreads();
     FK_XCD_STAMP(0, 8);
     tile_partials<KIND, NL, kBlock>(D, td, pd, rd, xs, sx, meta + 2 * MW, work);
     __syncthreads();
     FK_XCD_STAMP(0, 9);
     if (!idle && ok) {
-        long long* out = a.out_sums;
+        long long* out = routed ? a.out_sums : a.out_sums2;
         XcdControl* ctl = sync.ctl;
-        // a route's (and the shared expert's) full dot product is rounded to T before it is weighted and summed
-        // (routed_qmv_reduce.rs:236-322)
+        // a route's full dot product is rounded to T before it is weighted and summed (routed_qmv_reduce.rs:236-322);
+        // a shared unit contributes its K-slice of the shared expert's dot product as it is
         tile_rows<false, true>(td, work, work, [&](uint32_t r, float s0, float) {
-            xcd_sum_add(out, out0 + r, __fmul_rn(route_w, round_bf16(s0)), ctl);
+            xcd_sum_add(out, out0 + r, routed ? __fmul_rn(route_w, round_bf16(s0)) : s0, ctl);
         });
     }
     FK_XCD_STAMP(0, 10);
@@ -289,7 +282,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
 namespace {
 
 struct MoeGeometry {
-    uint32_t n_shared, gu_rows, down_rows, sdown_rows, gate_cpr, down_cpr, sdown_cpr;
+    uint32_t n_shared, gu_rows, down_rows, gate_cpr, down_cpr;
     LdsPlan lp;
     uint32_t lds;
 };
@@ -299,12 +292,9 @@ MoeGeometry moe_geometry(const XcdMoeShape& s) {
     g.n_shared = s.inter ? s.shared_inter / s.inter : 0u;
     g.gu_rows = s.inter / kXcdSlots;
     g.down_rows = s.hidden / kXcdSlots;
-    g.sdown_rows = g.n_shared ? s.hidden / (kXcdSlots * g.n_shared) : 0u;
     g.gate_cpr = s.hidden / cv;
     g.down_cpr = s.inter / cv;
-    g.sdown_cpr = s.shared_inter / cv;
-    g.lp.cs_max = g.gate_cpr > g.sdown_cpr ? g.gate_cpr : g.sdown_cpr;
-    if (g.down_cpr > g.lp.cs_max) g.lp.cs_max = g.down_cpr;
+    g.lp.cs_max = g.gate_cpr > g.down_cpr ? g.gate_cpr : g.down_cpr;
     g.lp.work_floats = 2u * kMoeNl * kBlock;
     g.lp.att_elems = 0;
     g.lp.meta_words = kMetaWords;
@@ -322,25 +312,23 @@ fk_status xcd_moe_supported(const XcdMoeShape& s) {
     if (s.experts > kXcdSlots || s.top_k > s.experts) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: at most 64 experts (one router logit per block of an XCD)");
     if (s.shared_inter % s.inter) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: the shared width must be a multiple of an expert's");
     const MoeGeometry g = moe_geometry(s);
-    if (g.n_shared < 1 || g.n_shared > kMoeMaxShared || s.top_k + g.n_shared != kXcds)
-        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: routes + shared units (shared width / expert width, 1 or 2) must be 8, one per XCD");
-    if (s.hidden % 64 || s.hidden > (uint32_t)kInGroups * kBlock * 8) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: hidden must be a multiple of 64, at most 4096");
-    if (s.inter % kXcdSlots || s.hidden % (kXcdSlots * g.n_shared))
-        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: expert width and hidden / shared units must be multiples of 64 (whole rows per block)");
+    if (g.n_shared < 1 || s.top_k + g.n_shared > kXcds)
+        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: routes + shared units (shared width / expert width) must be at most 8, one per XCD");
+    if (s.hidden % 128 || s.inter % 128 || s.hidden > (uint32_t)kInGroups * kBlock * 8)
+        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: widths must be multiples of 128, hidden at most 4096");
+    if (s.inter % kXcdSlots || s.hidden % kXcdSlots)
+        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: expert width and hidden must be multiples of 64 (whole rows per block)");
     if (s.hidden % s.group || s.inter % s.group) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: widths must be whole quantisation groups");
-    // a tile is one pass of 6 requests per thread; its groups are fetched four per lane as one aligned run
+    // a tile is one pass of 6 requests per thread; the groups of a gate / up tile are fetched four per lane as one
+    // aligned run
     const uint32_t budget = (uint32_t)kMoeNl * kBlock;
-    const uint32_t gg = s.hidden / s.group, dg = s.inter / s.group, sg = s.shared_inter / s.group;
-    if (g.gu_rows * g.gate_cpr > budget || g.down_rows * g.down_cpr > budget || g.sdown_rows * g.sdown_cpr > budget)
+    const uint32_t gg = s.hidden / s.group, dg = s.inter / s.group;
+    if (g.gu_rows * g.gate_cpr > budget || g.down_rows * g.down_cpr > budget)
         return set_error(FK_ERR_UNSUPPORTED, "xcd moe: a block's tile holds more than 1536 16-byte chunks");
-    if (g.gu_rows * gg > kMetaWords || g.down_rows * dg > kMetaWords || g.sdown_rows * sg > kMetaWords)
+    if (g.gu_rows * gg > kMetaWords || g.down_rows * dg > kMetaWords)
         return set_error(FK_ERR_UNSUPPORTED, "xcd moe: a block's tile holds more than 768 quantisation groups");
-    if ((g.gu_rows * gg) % 4 || (g.down_rows * dg) % 4 || (g.sdown_rows * sg) % 4)
-        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: a block's tile must hold a multiple of four quantisation groups");
-    if (g.gate_cpr % 4 || g.down_cpr % 4 || g.sdown_cpr % 4)
-        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: widths must be multiples of 128");
-    if (g.gu_rows * g.gate_cpr == 0 || g.lp.cs_max > 10u * 16u)
-        return set_error(FK_ERR_UNSUPPORTED, "xcd moe: rows of more than 160 chunks are not served");
+    if ((g.gu_rows * gg) % 4) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: a block's gate / up tile must hold a multiple of four quantisation groups");
+    if (g.lp.cs_max > 10u * 16u) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: rows of more than 160 chunks are not served");
     if (2u * ((g.lds + 1023u) & ~1023u) > kCuLdsBytes) return set_error(FK_ERR_UNSUPPORTED, "xcd moe: two workgroups must fit the LDS of one CU");
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
@@ -348,16 +336,15 @@ fk_status xcd_moe_supported(const XcdMoeShape& s) {
     return require_two_blocks_per_cu(reinterpret_cast<const void*>(&xcd_moe_kernel<W_Q4>), g.lds, "expert");
 }
 
-size_t xcd_moe_scratch_bytes(const XcdMoeShape& s) {
-    const uint32_t n_shared = s.inter ? s.shared_inter / s.inter : 0u;
-    return (size_t)kXcds * kXcdSlots * 4 + ((size_t)s.top_k * s.inter + (size_t)n_shared * s.shared_inter) * 2;
-}
+size_t xcd_moe_scratch_bytes(const XcdMoeShape& s) { return (size_t)kXcds * kXcdSlots * 4 + (size_t)kXcds * s.inter * 2; }
 
 fk_status plan_xcd_moe(const XcdMoeRequest& rq, Launch* out) {
     const XcdMoeShape& s = rq.shape;
     FK_TRY(xcd_moe_supported(s));
-    if (!rq.router_w || !rq.route_scale || !rq.scratch || !rq.out_sums || !rq.workspace)
+    if (!rq.router_w || !rq.route_scale || !rq.scratch || !rq.out_sums || !rq.out_sums2 || !rq.workspace)
         return set_error(FK_ERR_INVALID, "xcd moe: null router, scratch, sum row or workspace");
+    if (rq.out_sums2 == rq.out_sums || rq.out_sums2 == rq.sums_in || rq.out_sums2 == rq.clear)
+        return set_error(FK_ERR_INVALID, "xcd moe: the shared expert's sum row must be a row of its own");
     if (((uintptr_t)rq.router_w | (uintptr_t)rq.scratch) & 15u) return set_error(FK_ERR_INVALID, "xcd moe: router rows and scratch must be 16-byte aligned");
     if (rq.swiglu_variant < 0 || rq.swiglu_variant > 2) return set_error(FK_ERR_INVALID, "xcd moe: swiglu variant must be 0, 1 or 2");
     const MoeGeometry g = moe_geometry(s);
@@ -383,7 +370,6 @@ fk_status plan_xcd_moe(const XcdMoeRequest& rq, Launch* out) {
     a.inter = s.inter;
     a.gu_rows = g.gu_rows;
     a.down_rows = g.down_rows;
-    a.sdown_rows = g.sdown_rows;
     a.swiglu_variant = rq.swiglu_variant;
     a.logits_xcd = reinterpret_cast<uint32_t*>(rq.scratch);
     a.mid = reinterpret_cast<uint16_t*>(reinterpret_cast<unsigned char*>(rq.scratch) + (size_t)kXcds * kXcdSlots * 4);
@@ -391,6 +377,7 @@ fk_status plan_xcd_moe(const XcdMoeRequest& rq, Launch* out) {
     a.idx_out = rq.idx_out;
     a.weight_out = rq.weight_out;
     a.out_sums = rq.out_sums;
+    a.out_sums2 = rq.out_sums2;
     a.ctl = reinterpret_cast<XcdControl*>(rq.workspace);
     a.spin_limit = rq.spin_limit ? rq.spin_limit : (1u << 20);
     a.cs_max = g.lp.cs_max;

@@ -58,6 +58,8 @@ class MoeConfig:
     fuse_shared: bool = True   # the shared experts' gate/up pair as further routes of the routed launch
     fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
     direct_head_argmax: bool = True  # the LM head selects the greedy token itself where its shape allows
+    xcd_moe: bool = False      # router + routed / shared experts + reduction of a layer as ONE XCD-resident launch
+    xcd_spin_limit: int = 0    # hand-over wait bound of that launch (0: the library's default)
 
     @property
     def qk_dim(self) -> int:
@@ -217,6 +219,16 @@ class MoeRuntime:
         # the single-launch router holds the hidden row in registers, 512 elements per piece, at most 8
         self.fused_router = bool(c.fuse_router and c.hidden % 512 == 0 and c.hidden <= 4096)
         self.router_ws = z(4 * (c.n_experts + 1))
+        # the expert block as one launch, cut by route over the XCDs (where the shape admits it)
+        self.xcd = bool(c.xcd_moe and c.swiglu_variant == 1 and c.first_dense < c.n_layers and
+                        native.xcd_moe_supported(c.hidden, c.moe_inter, c.shared_inter, c.n_experts, c.top_k, c.bits, c.group))
+        if c.xcd_moe and not self.xcd:
+            raise native.FusekitError(native.FK_ERR_UNSUPPORTED, "xcd_moe: " + native.lib.fk_last_error().decode())
+        if self.xcd:
+            self.xcd_ctl = z(native.xcd_workspace_bytes(c.n_heads, c.qk_dim)[0])
+            self.xcd_sums = [z(native.xcd_sum_row_bytes(c.hidden)) for _ in range(3)]   # routes, shared expert, cleared
+            self.xcd_x = B(c.hidden * 2)
+            self.xcd_scratch = z(native.xcd_moe_scratch_bytes(c.moe_inter))
         self._rows_variants: Dict[int, "MoeRowsVariant"] = {}
         self.tasks = self.build_tasks()
         self.graph = self.d.build_decode_graph(self.tasks, False)
@@ -304,7 +316,9 @@ class MoeRuntime:
             rlg = arg(self.route_logits, 2 * c.n_experts, 2 * c.n_experts * l)
             rwt = arg(self.route_weight, 2 * c.top_k, 2 * c.top_k * l)
             route_in_consumer = self.fused_router and c.fuse_topk and c.fuse_shared and c.swiglu_variant == 1
-            if self.fused_router:   # norm + router projection (+ top-k route unless the expert launch ranks the logits itself)
+            if self.xcd:            # the expert launch below forms and ranks the logits itself
+                pass
+            elif self.fused_router:   # norm + router projection (+ top-k route unless the expert launch ranks the logits itself)
                 t.append(Dispatch(name("moe_router"),
                                   [arg(self.x[1]), arg(post), arg(Wr.w), arg(self.route_scale), arg(self.xn), rlg,
                                    ridx, rwt, arg(self.router_ws)],
@@ -320,6 +334,19 @@ class MoeRuntime:
                                   dict(row_n=c.n_experts, top_k=c.top_k, rows=1)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
+            if self.xcd:   # one launch into a sum row, then sum row + residual -> x[0]
+                a = [arg(self.x[1]), arg(self.xcd_x), arg(post), arg(Wr.w), arg(self.route_scale)]
+                for W in (Eg, Eu, Ed, Sg, Su, Sd):
+                    a += wargs(W)
+                a += [rlg, ridx, rwt, arg(self.xcd_scratch), arg(self.xcd_sums[1]), arg(self.xcd_sums[0]), arg(self.xcd_sums[2]),
+                      arg(self.xcd_ctl)]
+                t.append(Dispatch(name("xcd_moe_block"), a,
+                                  dict(quant, hidden=c.hidden, inter=c.moe_inter, shared_inter=c.shared_inter, experts=c.n_experts,
+                                       top_k=c.top_k, eps=c.eps, variant=c.swiglu_variant, has_sums=0,
+                                       spin_limit=c.xcd_spin_limit, mark_placement=int(l == c.first_dense))))
+                t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_sums[0]), arg(self.x[1]), arg(self.x[0]), arg(self.xcd_sums[0]),
+                                                       arg(self.xcd_sums[1]), arg(self.xcd_sums[1])], dict(hidden=c.hidden)))
+                continue
             routed = [arg(self.xn), arg(Eg.w), arg(Eg.scales), arg(Eg.biases), arg(Eu.w), arg(Eu.scales), arg(Eu.biases),
                       arg(self.rows_x), ridx, arg(self.h)]
             rparams = dict(quant, k=c.hidden, o=c.moe_inter, experts=c.n_experts, routes=c.top_k, x_rows=1)
@@ -377,6 +404,11 @@ class MoeRuntime:
         out["sdpa_partials"], out["rope_tab"] = (self.sdpa_partials, "float32", False), (self.rope_tab, "float32", False)
         for l in range(self.cfg.n_layers):
             out[f"cache_k.{l}"], out[f"cache_v.{l}"] = (self.cache_k[l], "bfloat16", True), (self.cache_v[l], "bfloat16", True)
+        if self.xcd:
+            out["xcd.control"], out["xcd.scratch"] = (self.xcd_ctl, "uint32", True), (self.xcd_scratch, "uint32", True)
+            out["xcd.x"] = (self.xcd_x, "bfloat16", False)
+            for i, b in enumerate(self.xcd_sums):
+                out[f"xcd.sums.{i}"] = (b, "uint32", True)
         return out
 
     def routes(self) -> np.ndarray:
@@ -404,6 +436,9 @@ class MoeRuntime:
     def reset(self) -> None:
         for b in (self.step_counter, self.offset, self.kv_len, self.hist_counter):
             b.upload(np.zeros(1, np.uint32))
+        if self.xcd:
+            for b in self.xcd_sums:
+                b.upload(np.zeros(b.nbytes, np.uint8))
 
     def prefill(self, prompt: Sequence[int], start_offset: int = 0) -> int:
         preds, _ = self.d.decode_host_loop(self.graph, self.uniforms, start_offset, list(prompt))
@@ -569,6 +604,19 @@ class MoeRowsVariant:
                               dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1, rows=m)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
+            if self.xcd:   # one launch into a sum row, then sum row + residual -> x[0]
+                a = [arg(self.x[1]), arg(self.xcd_x), arg(post), arg(Wr.w), arg(self.route_scale)]
+                for W in (Eg, Eu, Ed, Sg, Su, Sd):
+                    a += wargs(W)
+                a += [rlg, ridx, rwt, arg(self.xcd_scratch), arg(self.xcd_sums[1]), arg(self.xcd_sums[0]), arg(self.xcd_sums[2]),
+                      arg(self.xcd_ctl)]
+                t.append(Dispatch(name("xcd_moe_block"), a,
+                                  dict(quant, hidden=c.hidden, inter=c.moe_inter, shared_inter=c.shared_inter, experts=c.n_experts,
+                                       top_k=c.top_k, eps=c.eps, variant=c.swiglu_variant, has_sums=0,
+                                       spin_limit=c.xcd_spin_limit, mark_placement=int(l == c.first_dense))))
+                t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_sums[0]), arg(self.x[1]), arg(self.x[0]), arg(self.xcd_sums[0]),
+                                                       arg(self.xcd_sums[1]), arg(self.xcd_sums[1])], dict(hidden=c.hidden)))
+                continue
             order, ordered = ([arg(self.order)], dict(has_order=1)) if self.order is not None else ([], {})
             if self.rank_in_launch:
                 ordered = dict(expert_order=1)

@@ -568,8 +568,8 @@ def xcd_moe_supported(hidden, inter, shared_inter, experts, top_k, bits, group) 
 lib.fk_xcd_moe_scratch_bytes.restype = C.c_size_t
 
 
-def xcd_moe_scratch_bytes(inter: int, shared_inter: int, top_k: int) -> int:
-    return int(lib.fk_xcd_moe_scratch_bytes(C.c_uint32(inter), C.c_uint32(shared_inter), C.c_uint32(top_k)))
+def xcd_moe_scratch_bytes(inter: int) -> int:
+    return int(lib.fk_xcd_moe_scratch_bytes(C.c_uint32(inter)))
 
 
 def xcd_kslice_meta(src: "DeviceBuffer", n: int, groups: int, stream=None) -> "DeviceBuffer":

@@ -596,20 +596,21 @@ size_t fk_xcd_sum_row_bytes(uint32_t hidden);
  * routed_qmv_reduce.rs (with the shared expert's down_proj).  The cut is BY ROUTE: XCD u < top_k serves the u-th winner
  * of the ranking -- its 64 workgroups form the 64 router logits, hand them over inside the XCD, every wave ranks them,
  * then the expert's gate / up rows, SwiGLU, a second hand-over, and the expert's down_proj over the whole intermediate
- * width; the other XCDs serve the shared expert (every one of them all its gate / up rows, a share of its down_proj
- * rows).  A route's full dot product is formed, rounded to bf16 and weighted inside one XCD, as the reference's
- * reduction does it (routed_qmv_reduce.rs:236-322); the weighted routes, the shared output and (in the launch that
- * reads the row) the residual are then added exactly, in 64-bit fixed point, where the reference adds them one by one
- * in fp32, and rounded to bf16 once.  Output: a sum row (finish it with fusekit_xcd_reduce or hand it to the next
- * launch of these families); the logits, the routes and their weights are also written out for the host.  Slot
- * order at the planner (fusekit_amd/csrc/dispatcher.hip).  Requires 4-bit weights, at most 64 experts,
- * top_k + shared_inter / inter == 8 with one or two shared units, widths that give every workgroup whole rows
- * (inter % 64 == 0, hidden % (64 * shared units) == 0), tiles of at most 1536 16-byte chunks and 768 quantisation
- * groups; other layers use the per-dispatch families.  The exclusive-use rule below applies. */
+ * width.  A route's full dot product is formed, rounded to bf16 and weighted inside one XCD, as the reference's
+ * reduction does it (routed_qmv_reduce.rs:236-322).  The shared expert, n = shared_inter / inter times as wide as a
+ * routed one, is n more units of the same size on the next XCDs (gate / up rows [h inter, (h+1) inter) and the K-slice
+ * of the shared down_proj they feed); their partial dot products are added unrounded into a second sum row.  Outputs:
+ * the two sum rows -- x = T((f32(row) + T(f32(shared row))) + residual) is the reference's result with its additions in
+ * its order, the weighted routes being added exactly, in 64-bit fixed point, where the reference adds them one by one
+ * in fp32; fusekit_xcd_reduce with six slots forms it -- and the logits, the routes and their weights for the host.
+ * Slot order at the planner (fusekit_amd/csrc/dispatcher.hip).  Requires 4-bit weights, at most 64 experts,
+ * top_k + n <= 8, widths that are multiples of 128 and give every workgroup whole rows (inter % 64 == 0,
+ * hidden % 64 == 0), tiles of at most 1536 16-byte chunks and 768 quantisation groups; other layers use the
+ * per-dispatch families.  The exclusive-use rule below applies. */
 fk_status fk_xcd_moe_supported(uint32_t hidden, uint32_t inter, uint32_t shared_inter, uint32_t experts, uint32_t top_k,
                                uint32_t bits, uint32_t group);
 /* Bytes of the launch's scratch slot: per-XCD copies of the router logits and the SwiGLU rows of the eight units. */
-size_t fk_xcd_moe_scratch_bytes(uint32_t inter, uint32_t shared_inter, uint32_t top_k);
+size_t fk_xcd_moe_scratch_bytes(uint32_t inter);
 /* The o_proj and down_proj slots of the two families take their scales and biases re-laid out per K-slice:
  * dst[(h * n + r) * (groups / 8) + g] = src[r * groups + h * (groups / 8) + g] for the [n, groups] array of a
  * matrix (same size as the source).  An XCD then reads its slice of every row as one contiguous stream; in the
