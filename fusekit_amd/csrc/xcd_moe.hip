@@ -149,9 +149,11 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
 
     const uint32_t unit = sync.xcd;
     const bool routed = unit < a.top_k;                   // block-uniform
-    const uint32_t sh = routed ? 0u : unit - a.top_k;     // shared unit
-    const bool idle = !routed && sh >= a.n_shared;        // an XCD without a unit (top_k + n_shared < 8)
-    const XcdMat G = pick_mat(routed, a.gate, a.sgate), U = pick_mat(routed, a.up, a.sup), D = pick_mat(routed, a.down, a.sdown);
+    const bool idle = !routed && unit - a.top_k >= a.n_shared;   // an XCD without a unit (top_k + n_shared < 8)
+    // shared unit; an idle XCD walks the same code with empty tiles, whose (clamped) requests must stay inside the
+    // matrices: it addresses unit 0
+    const uint32_t sh = (routed || idle) ? 0u : unit - a.top_k;
+    XcdMat G = pick_mat(routed, a.gate, a.sgate), U = pick_mat(routed, a.up, a.sup), D = pick_mat(routed, a.down, a.sdown);
 
     // A shared unit is served like a route: unit h of the shared expert is its gate / up rows [h I, (h+1) I) and, in
     // down_proj, the K-slice of those rows' outputs -- a partial dot product per output row, added UNROUNDED into the
@@ -161,7 +163,14 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
     MetaRegs mg, mu, md;
     TilePos<NL> pg, pd;
 
+    // Tile geometry does not depend on the expert: positions are worked out now, relative to the unit's first row, and
+    // the ranking only moves the matrices' base pointers to that row (scalar work).
     const uint32_t gu0 = sync.slot * a.gu_rows;
+    const Tile tg = make_tile(gu0, idle ? 0u : a.gu_rows, 0, G.cpr);
+    tile_pos_init<NL, kBlock>(G, tg, tid, pg);
+    const uint32_t out0 = sync.slot * a.down_rows, dcs = a.down.cpr;
+    const Tile td = make_tile(out0, idle ? 0u : a.down_rows, routed ? 0u : sh * dcs, dcs);
+    tile_pos_init<NL, kBlock>(D, td, tid, pd);
     const bool with_router = routed && sync.slot < a.experts;
     uint4 rw[kInGroups];
     {
@@ -199,42 +208,60 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_moe_kernel(const long long* sum
         if (!xcd_wait_ok(okw)) return;
         FK_XCD_STAMP(0, 3);
         // ---- every wave ranks the logits and takes winner `unit` ----
-        float x[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-        if (lane < a.experts) x[0] = __uint_as_float(__hip_atomic_load(lg + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        uint32_t key[4];
-        route_candidates(x, a.experts, lane, key);
-        const bool reporter = unit == 0 && sync.slot == 0 && tid == 0;
-        for (uint32_t k = 0; k < a.top_k; ++k) {
-            float best;
-            uint32_t best_i;
-            route_take_best(key, best, best_i);
-            const uint32_t wbits = f32_to_bf16_bits(best * sc);
-            if (k == unit) {
-                expert = best_i < a.experts ? best_i : a.experts - 1;
-                route_w = bf16_bits_to_f32((uint16_t)wbits);
-            }
-            if (reporter) {
-                if (a.idx_out) a.idx_out[k] = best_i;
-                if (a.weight_out) a.weight_out[k] = (uint16_t)wbits;
-            }
+        // (route_candidates / route_take_best with one logit per lane: at most 64 experts here; same arithmetic)
+        const bool has = lane < a.experts;
+        const float xl = has ? __uint_as_float(__hip_atomic_load(lg + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) : -INFINITY;
+        const float mx = wave_max(xl);
+        FK_XCD_STAMP(0, 11);
+        const float pl = has ? expf(xl - mx) : 0.f;
+        const float inv = 1.0f / wave_sum(pl);
+        uint32_t key = has ? (__float_as_uint(round_bf16(pl * inv)) | (256u - lane)) : 0u;
+        // Rank of every lane's key = number of larger keys (keys of live lanes are distinct: the index is part of the
+        // key): 64 independent compares instead of top_k dependent rounds of a wave-wide maximum.  The lane of rank
+        // `unit` is the unit's expert -- the lane index IS the expert index.
+        uint32_t c0 = 0, c1 = 0;
+#pragma unroll
+        for (int i = 0; i < (int)kWave; i += 2) {
+            const uint32_t s0 = (uint32_t)__builtin_amdgcn_readlane((int)key, i), s1 = (uint32_t)__builtin_amdgcn_readlane((int)key, i + 1);
+            c0 += s0 > key ? 1u : 0u;
+            c1 += s1 > key ? 1u : 0u;
+        }
+        const uint32_t rank = c0 + c1;
+        const uint32_t wbits = f32_to_bf16_bits(__uint_as_float(key & 0xffff0000u) * sc);
+        const unsigned long long mine = __ballot(has && rank == unit);
+        const uint32_t win = mine ? (uint32_t)__builtin_ctzll(mine) : 0u;   // (always one lane: top_k <= experts)
+        expert = win;
+        route_w = bf16_bits_to_f32((uint16_t)__builtin_amdgcn_readlane((int)wbits, win));
+        if (unit == 0 && sync.slot == 0 && tid < kWave && has && rank < a.top_k) {   // the host's copy of the route
+            if (a.idx_out) a.idx_out[rank] = lane;
+            if (a.weight_out) a.weight_out[rank] = (uint16_t)wbits;
         }
         expert = __builtin_amdgcn_readfirstlane(expert);
+        FK_XCD_STAMP(0, 12);
     }
     // ---- the unit's gate / up rows: the expert's (routed), rows [h I, (h+1) I) of the shared expert (shared) ----
-    const uint32_t row_gu = (routed ? expert : sh) * a.inter + gu0;
-    const Tile tg = make_tile(row_gu, idle ? 0u : a.gu_rows, 0, G.cpr);
-    tile_pos_init<NL, kBlock>(G, tg, tid, pg);
+    {
+        const size_t urow = (size_t)(routed ? expert : sh) * a.inter;   // first gate / up row of the unit
+        const uint32_t ggr = G.cpr >> G.gshift;
+        G.w += urow * G.cpr;
+        U.w += urow * U.cpr;
+        G.sc += urow * ggr;
+        G.bi += urow * ggr;
+        U.sc += urow * ggr;
+        U.bi += urow * ggr;
+        if (routed) {   // an expert's down_proj rows; the shared units take a K-slice of the one shared matrix
+            const size_t drow = (size_t)expert * hidden;
+            D.w += drow * D.cpr;
+            D.sc += drow * (D.cpr >> D.gshift);
+            D.bi += drow * (D.cpr >> D.gshift);
+        }
+    }
     meta_fetch<KIND, kBlock, true>(G, tg, tid, mg);
     meta_fetch<KIND, kBlock, true>(U, tg, tid, mu);
+    FK_XCD_STAMP(0, 13);
     tile_load<KIND, NL, kBlock>(G, tg, pg, rg);
     tile_load<KIND, NL, kBlock>(U, tg, pg, ru);
     FK_XCD_STAMP(0, 4);
-
-    // down_proj tile of this block: its output rows x the unit's intermediate columns (all of an expert's row, the
-    // unit's K-slice of the shared expert's)
-    const uint32_t out0 = sync.slot * a.down_rows, dcs = a.down.cpr;
-    const Tile td = make_tile(routed ? expert * hidden + out0 : out0, idle ? 0u : a.down_rows, routed ? 0u : sh * dcs, dcs);
-    tile_pos_init<NL, kBlock>(D, td, tid, pd);
 
     uint16_t* mid = a.mid + (size_t)unit * a.inter;
     const int variant = a.swiglu_variant;

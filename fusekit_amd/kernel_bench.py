@@ -255,7 +255,7 @@ def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_
                       "TFLOPs": round(flops / rows_s / 1e12, 2)}), flush=True)
 
 
-def case_moe_decode(d, reps, prompt_len=32, decode=512, xcd_moe=False):
+def case_moe_decode(d, reps, prompt_len=32, decode=512, xcd_moe=True):
     """Decode loop of the MoE benchmark model (27 layers, 64 experts top-6 + 2 shared, low-rank keys, int4):
     a 32-token prompt, then 512 greedy tokens from the captured graph; per-node times of one replay."""
     import numpy as np
@@ -273,7 +273,7 @@ def case_moe_decode(d, reps, prompt_len=32, decode=512, xcd_moe=False):
     for t, sec in zip(rt.tasks, per_node):
         k = t.kernel.rsplit("_f", 1)[0].replace("fusekit_", "")
         kinds[k] = kinds.get(k, 0.0) + sec * 1e6
-    print(json.dumps({"case": "moe_cfg5_decode_q4" + ("_expert_launch" if xcd_moe else ""), "tok_per_s": round(steps / gpu_s, 1), "ms_per_token": round(gpu_s / steps * 1e3, 3),
+    print(json.dumps({"case": "moe_cfg5_decode_q4" + ("" if xcd_moe else "_per_dispatch"), "tok_per_s": round(steps / gpu_s, 1), "ms_per_token": round(gpu_s / steps * 1e3, 3),
                       "graph_nodes": len(rt.tasks), "token_MB": round(cfg.token_bytes(ctx) / 1e6, 1),
                       "roofline_tok_per_s": round(roof, 1), "frac": round(steps / gpu_s / roof, 4),
                       "weights_GB": round(W.nbytes() / 1e9, 2),
@@ -326,7 +326,7 @@ CASES = {
     "moe_cfg5_rows8_pass": lambda d, r: case_moe_rows(d, r, 8),
     "moe_cfg5_rows64_pass": lambda d, r: case_moe_rows(d, r, 64),
     "moe_cfg5_decode": lambda d, r: case_moe_decode(d, r),
-    "moe_cfg5_decode_expert_launch": lambda d, r: case_moe_decode(d, r, xcd_moe=True),
+    "moe_cfg5_decode_per_dispatch": lambda d, r: case_moe_decode(d, r, xcd_moe=False),
     "qgemv_cfg1": lambda d, r: case_qgemv(d, r, 4864, 896, 4, 512, "cfg1_4864x896"),
     "qgemv_big_q4": lambda d, r: case_qgemv(d, r, 9728, 2560, 4, 48, "9728x2560"),
     "qgemv_big_q8": lambda d, r: case_qgemv(d, r, 9728, 2560, 8, 28, "9728x2560"),

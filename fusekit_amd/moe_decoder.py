@@ -58,7 +58,8 @@ class MoeConfig:
     fuse_shared: bool = True   # the shared experts' gate/up pair as further routes of the routed launch
     fuse_router: bool = True   # norm + router projection + top-k route as one launch (hidden % 512 == 0)
     direct_head_argmax: bool = True  # the LM head selects the greedy token itself where its shape allows
-    xcd_moe: bool = False      # router + routed / shared experts + reduction of a layer as ONE XCD-resident launch
+    xcd_moe: bool = True       # router + routed / shared experts + reduction of a layer as ONE XCD-resident launch, where
+                               # the shape admits it (MoeRuntime.xcd tells); off: the per-dispatch families
     xcd_spin_limit: int = 0    # hand-over wait bound of that launch (0: the library's default)
 
     @property
@@ -222,8 +223,6 @@ class MoeRuntime:
         # the expert block as one launch, cut by route over the XCDs (where the shape admits it)
         self.xcd = bool(c.xcd_moe and c.swiglu_variant == 1 and c.first_dense < c.n_layers and
                         native.xcd_moe_supported(c.hidden, c.moe_inter, c.shared_inter, c.n_experts, c.top_k, c.bits, c.group))
-        if c.xcd_moe and not self.xcd:
-            raise native.FusekitError(native.FK_ERR_UNSUPPORTED, "xcd_moe: " + native.lib.fk_last_error().decode())
         if self.xcd:
             self.xcd_ctl = z(native.xcd_workspace_bytes(c.n_heads, c.qk_dim)[0])
             self.xcd_sums = [z(native.xcd_sum_row_bytes(c.hidden)) for _ in range(3)]   # routes, shared expert, cleared
@@ -604,19 +603,6 @@ class MoeRowsVariant:
                               dict(hidden=c.hidden, experts=c.n_experts, top_k=c.top_k, eps=c.eps, has_norm=1, rows=m)))
             Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
             Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
-            if self.xcd:   # one launch into a sum row, then sum row + residual -> x[0]
-                a = [arg(self.x[1]), arg(self.xcd_x), arg(post), arg(Wr.w), arg(self.route_scale)]
-                for W in (Eg, Eu, Ed, Sg, Su, Sd):
-                    a += wargs(W)
-                a += [rlg, ridx, rwt, arg(self.xcd_scratch), arg(self.xcd_sums[1]), arg(self.xcd_sums[0]), arg(self.xcd_sums[2]),
-                      arg(self.xcd_ctl)]
-                t.append(Dispatch(name("xcd_moe_block"), a,
-                                  dict(quant, hidden=c.hidden, inter=c.moe_inter, shared_inter=c.shared_inter, experts=c.n_experts,
-                                       top_k=c.top_k, eps=c.eps, variant=c.swiglu_variant, has_sums=0,
-                                       spin_limit=c.xcd_spin_limit, mark_placement=int(l == c.first_dense))))
-                t.append(Dispatch(name("xcd_reduce"), [arg(self.xcd_sums[0]), arg(self.x[1]), arg(self.x[0]), arg(self.xcd_sums[0]),
-                                                       arg(self.xcd_sums[1]), arg(self.xcd_sums[1])], dict(hidden=c.hidden)))
-                continue
             order, ordered = ([arg(self.order)], dict(has_order=1)) if self.order is not None else ([], {})
             if self.rank_in_launch:
                 ordered = dict(expert_order=1)

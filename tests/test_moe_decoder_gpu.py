@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 def _small_cfg(**kw):
     from fusekit_amd.moe_decoder import MoeConfig
     base = dict(n_layers=3, hidden=256, n_heads=2, kv_lora_rank=128, rope_dim=64, nope_dim=128, v_dim=128, n_experts=8,
-                top_k=2, moe_inter=128, n_shared=1, dense_inter=512, first_dense=1, vocab=2000, capacity=64)
+                top_k=2, moe_inter=128, n_shared=1, dense_inter=512, first_dense=1, vocab=2000, capacity=64, xcd_moe=False)
     base.update(kw)
     return MoeConfig(**base)
 
@@ -24,12 +24,16 @@ def _small_cfg(**kw):
 @pytest.mark.parametrize("bits,traditional,kw", [(4, True, {}), (8, False, {}), (4, True, dict(hidden=512)),
                                                  (4, True, dict(hidden=512, fuse_topk=False)),
                                                  (4, False, dict(hidden=512, fuse_router=False, fuse_shared=False, fuse_attention=False)),
-                                                 (4, True, dict(n_heads=4, nope_dim=64, rope_dim=32, v_dim=64, n_experts=16, top_k=4))])
+                                                 (4, True, dict(n_heads=4, nope_dim=64, rope_dim=32, v_dim=64, n_experts=16, top_k=4)),
+                                                 # the expert block as one launch: 3 of 8 XCDs busy, then all 8
+                                                 (4, True, dict(hidden=512, xcd_moe=True)),
+                                                 (4, False, dict(hidden=512, n_experts=16, top_k=6, n_shared=2, xcd_moe=True))])
 def test_greedy_tokens_and_routes_match_oracle(fk, bits, traditional, kw):
     from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
     cfg = _small_cfg(bits=bits, rope_traditional=traditional, **kw)
     W = MoeWeights.random_init(cfg, seed=2)
     rt = MoeRuntime(cfg, W)
+    assert rt.xcd == bool(kw.get("xcd_moe", False)), fk.lib.fk_last_error().decode()
     od = OracleMoeDecoder(cfg, W)
     prompt = rng(1).integers(0, cfg.vocab, 6).tolist()
     n = 20
@@ -74,7 +78,7 @@ def test_full_size_model_32_greedy_tokens(fk):
     the oracle's candidates within six bf16 steps of its maximum, must equal the oracle's where that set has
     one member, and at least 26 of the 32 steps pick the oracle's token outright."""
     from fusekit_amd.moe_decoder import MoeConfig, MoeRuntime, MoeWeights
-    cfg = MoeConfig(capacity=128)
+    cfg = MoeConfig(capacity=128, xcd_moe=False)
     W = MoeWeights.random_init(cfg, seed=0)
     rt, od = MoeRuntime(cfg, W), OracleMoeDecoder(cfg, W)
     prompt = rng(0).integers(0, cfg.vocab, 4).tolist()
@@ -128,7 +132,7 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
     uploads the arrays it changes."""
     from fusekit_amd.moe_decoder import MoeConfig, MoeRuntime, MoeWeights
     fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "clear_margin_moe.json")))
-    cfg = MoeConfig(capacity=128)
+    cfg = MoeConfig(capacity=128, xcd_moe=False)
     n_moe = cfg.n_layers - cfg.first_dense
     prompt, want = fx["prompt"], fx["tokens"]
     assert fx["n_layers"] == cfg.n_layers and len(prompt) == 32 and len(want) == 32
@@ -177,6 +181,26 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
     rt.reset()
     again, _, _ = rt.generate(prompt, 32)
     assert again == want
+
+    # The same run with every layer's expert block as ONE launch (router, ranking, routed and shared experts, weighted
+    # sum: family fusekit_xcd_moe_block): the same tokens and, step by step and layer by layer, the same route sets.
+    import dataclasses
+    rx = MoeRuntime(dataclasses.replace(cfg, xcd_moe=True), W)
+    assert rx.xcd and sum(t.kernel.startswith("fusekit_xcd_moe_block") for t in rx.tasks) == n_moe
+    got_x, tok = [], prompt[0]
+    for i in range(63):
+        nxt, _ = rx.d.decode_host_loop(rx.graph, rx.uniforms, i, [tok])
+        routes = rx.routes()[cfg.first_dense:]
+        for l in range(n_moe):
+            assert sorted(routes[l].tolist()) == fx["routes"][i][l], (i, l)
+        if i >= 31:
+            got_x.append(nxt[0])
+        tok = prompt[i + 1] if i + 1 < 32 else nxt[0]
+    assert got_x == want
+    rx.reset()
+    again, _, _ = rx.generate(prompt, 32)
+    assert again == want
+    del rx
 
     # The same model at full size with EIGHT active token rows in one pass over the weights (shared-stream matmuls
     # for the dense projections and the shared experts, row forms of the store, the attention and the router,
@@ -238,16 +262,18 @@ def test_rows_pass_matches_sequential_oracle_steps(fk, rows, offset, route_order
     assert not cache.to_numpy(np.uint16).reshape(cfg.n_heads, cfg.capacity, dim)[:, offset + rows:].any()   # later rows untouched
 
 
-def test_artifact_round_trip(fk, tmp_path):
+@pytest.mark.parametrize("expert_launch", [False, True])
+def test_artifact_round_trip(fk, tmp_path, expert_launch):
     """task_graph.json / manifest.json written from the MoE runtime (row blocks of parameters carry offset_bytes,
     expert-stacked tensors their leading dimension) and read back by the consumer that knows only the files
     and the parameter tree: the same tokens."""
     import json
     from fusekit_amd.artifact import ArtifactRuntime, write_artifact
     from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
-    cfg = _small_cfg(hidden=512)
+    cfg = _small_cfg(hidden=512, xcd_moe=expert_launch)
     W = MoeWeights.random_init(cfg, seed=9)
     rt = MoeRuntime(cfg, W)
+    assert rt.xcd == expert_launch
     prompt = [3, 77, 1500, 9]
     want, _, _ = rt.generate(prompt, 12)
     write_artifact(rt, str(tmp_path), "moe-test")
@@ -255,7 +281,11 @@ def test_artifact_round_trip(fk, tmp_path):
     man = json.load(open(tmp_path / "manifest.json"))
     assert man["model"]["model_type"] == "moe-decoder" and g["model_config"]["n_experts"] == cfg.n_experts
     kinds = {t["kernel"].rsplit("_f", 1)[0] for t in g["tasks"]}
-    assert {"fusekit_moe_router", "fusekit_routed_qmv_swiglu", "fusekit_routed_qmv_reduce", "fusekit_split_store_sdpa_decode"} <= kinds
+    if expert_launch:   # the expert block of a layer as one launch and the row that finishes its output
+        assert {"fusekit_xcd_moe_block", "fusekit_xcd_reduce", "fusekit_split_store_sdpa_decode"} <= kinds
+        assert not {"fusekit_moe_router", "fusekit_routed_qmv_swiglu", "fusekit_routed_qmv_reduce"} & kinds
+    else:
+        assert {"fusekit_moe_router", "fusekit_routed_qmv_swiglu", "fusekit_routed_qmv_reduce", "fusekit_split_store_sdpa_decode"} <= kinds
     sliced = [b for t in g["tasks"] for b in t["inputs"] if b["role"] == "external" and b.get("offset_bytes")]
     assert sliced, "the kv_a / kv_b row blocks are slices of their parameters"
     stacked = [p for p in g["model_params"] if "switch_mlp" in p["path"]]
@@ -281,6 +311,8 @@ def test_checkpoint_round_trip(fk, tmp_path):
     assert dtype == "U32" and tuple(shape) == (cfg.n_experts, cfg.moe_inter, cfg.hidden * 4 // 32)
     st.close()
     cfg2, W2 = load_moe_checkpoint(str(tmp_path), capacity=cfg.capacity)
+    import dataclasses
+    cfg2 = dataclasses.replace(cfg2, xcd_moe=cfg.xcd_moe)   # a run-time choice, not part of the model's files
     assert cfg2 == cfg
     for k in W.mats:
         assert np.array_equal(W.mats[k].w.to_numpy(np.uint8), W2.mats[k].w.to_numpy(np.uint8)), k
