@@ -835,6 +835,24 @@ fk_status fk_xcd_moe_supported(uint32_t hidden, uint32_t inter, uint32_t shared_
     return xcd_moe_supported(XcdMoeShape{hidden, inter, shared_inter, experts, top_k, bits, group});
 }
 
+fk_status fk_xcd_mla_supported(uint32_t hidden, uint32_t n_heads, uint32_t rank, uint32_t rope_dim, uint32_t nope_dim,
+                               uint32_t v_dim, uint32_t capacity, uint32_t bits, uint32_t group) {
+    return xcd_mla_supported(XcdMlaShape{hidden, n_heads, rank, rope_dim, nope_dim, v_dim, capacity, bits, group});
+}
+
+fk_status fk_xcd_mla_workspace_bytes(uint32_t n_heads, uint32_t rank, uint32_t rope_dim, uint32_t v_dim, size_t* latent_bytes,
+                                     size_t* attention_partial_bytes) {
+    if (!latent_bytes || !attention_partial_bytes) return set_error(FK_ERR_INVALID, "fk_xcd_mla_workspace_bytes: null out");
+    XcdMlaShape s{};
+    s.n_heads = n_heads;
+    s.rank = rank;
+    s.rope_dim = rope_dim;
+    s.v_dim = v_dim;
+    *latent_bytes = xcd_mla_latent_bytes(s);
+    *attention_partial_bytes = xcd_mla_partials_bytes(s);
+    return FK_OK;
+}
+
 size_t fk_xcd_moe_scratch_bytes(uint32_t inter) {
     XcdMoeShape s{};
     s.inter = inter;

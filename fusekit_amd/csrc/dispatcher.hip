@@ -922,6 +922,103 @@ fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     return plan_xcd_moe(rq, l);
 }
 
+// The attention half of a layer with low-rank keys as one XCD-resident launch (xcd_mla_kernel):
+// [sums_in, shared_sums_in], residual, x_out, norm_w, W_q, s_q, b_q, W_kv_a, s_a, b_a, latent_norm_w, W_kv_b, s_b, b_b,
+// W_o, s_o, b_o (o_proj's scales and biases re-laid out per K-slice: fk_xcd_kslice_meta), q, kva (fk_xcd_mla_latent_bytes),
+// kvb, cache_k, cache_v, kv_len, rope_tab, att_partials, [clear2_sums], out_sums, clear_sums, workspace.
+// Parameters: hidden, n_heads, rank, rope_dim, nope_dim, v_dim, capacity, bits, group, eps, theta, traditional, scale,
+// has_sums (0: the input is the residual row alone; 2: the two rows of an expert launch), has_clear2, spin_limit,
+// mark_placement.
+fk_status plan_xcd_mla_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    XcdMlaShape s;
+    s.hidden = d.u("hidden");
+    s.n_heads = d.u("n_heads");
+    s.rank = d.u("rank");
+    s.rope_dim = d.u("rope_dim");
+    s.nope_dim = d.u("nope_dim");
+    s.v_dim = d.u("v_dim");
+    s.capacity = d.u("capacity");
+    s.bits = d.u("bits", 4);
+    s.group = d.u("group", 64);
+    const uint32_t has_p = d.u("has_sums", 0);
+    const bool has_c2 = d.u("has_clear2", 0) != 0;
+    if (has_p != 0 && has_p != 2) return set_error(FK_ERR_INVALID, d.kernel + ": has_sums must be 0 or 2");
+    size_t i = has_p;
+    const size_t res_slot = i++, x_slot = i++, nw_slot = i++, wq_slot = i, wa_slot = i + 3, an_slot = i + 6, wb_slot = i + 7, wo_slot = i + 10;
+    i += 13;
+    const size_t q_slot = i++, kva_slot = i++, kvb_slot = i++, ck_slot = i++, cv_slot = i++, len_slot = i++, tab_slot = i++, ap_slot = i++;
+    const size_t c2_slot = has_c2 ? i++ : 0;
+    const size_t op_slot = i++, clr_slot = i++, ws_slot = i++;
+    FK_TRY(need_args(d, i));
+    if (s.hidden == 0 || s.n_heads == 0 || s.rank == 0 || s.rope_dim == 0 || s.nope_dim == 0 || s.v_dim == 0 || s.capacity == 0)
+        return set_error(FK_ERR_INVALID, d.kernel + ": shape parameters missing");
+    if (s.bits != 4) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": 4-bit weights only");
+    const uint32_t qk = s.nope_dim + s.rope_dim, n_a = s.rank + s.rope_dim, n_b = s.n_heads * (s.nope_dim + s.v_dim);
+    XcdMlaRequest rq;
+    memset(&rq, 0, sizeof(rq));
+    rq.shape = s;
+    if (has_p) {
+        FK_TRY(need_bytes(d, 0, xcd_sum_row_bytes(s.hidden)));
+        FK_TRY(need_bytes(d, 1, xcd_sum_row_bytes(s.hidden)));
+        rq.sums_in = arg_ptr<const long long>(d, 0);
+        rq.sums2_in = arg_ptr<const long long>(d, 1);
+    }
+    FK_TRY(need_bytes(d, res_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, x_slot, (size_t)s.hidden * 2));
+    FK_TRY(need_bytes(d, nw_slot, (size_t)s.hidden * 2));
+    rq.residual = arg_ptr<const uint16_t>(d, res_slot);
+    rq.x_out = arg_ptr<uint16_t>(d, x_slot);
+    rq.norm_w = arg_ptr<const uint16_t>(d, nw_slot);
+    rq.eps = (float)d.param("eps", 1e-6);
+    fk_weight W[4];
+    FK_TRY(bind_weight(d, s.bits, s.group, s.n_heads * qk, s.hidden, wq_slot, wq_slot + 1, wq_slot + 2, &W[0]));
+    FK_TRY(bind_weight(d, s.bits, s.group, n_a, s.hidden, wa_slot, wa_slot + 1, wa_slot + 2, &W[1]));
+    FK_TRY(bind_weight(d, s.bits, s.group, n_b, s.rank, wb_slot, wb_slot + 1, wb_slot + 2, &W[2]));
+    FK_TRY(bind_weight(d, s.bits, s.group, s.hidden, s.n_heads * s.v_dim, wo_slot, wo_slot + 1, wo_slot + 2, &W[3]));
+    rq.wq = &W[0];
+    rq.wa = &W[1];
+    rq.wb = &W[2];
+    rq.wo = &W[3];
+    FK_TRY(need_bytes(d, an_slot, (size_t)s.rank * 2));
+    rq.a_norm = arg_ptr<const uint16_t>(d, an_slot);
+    FK_TRY(need_bytes(d, q_slot, (size_t)s.n_heads * qk * 2));
+    FK_TRY(need_bytes(d, kva_slot, xcd_mla_latent_bytes(s)));
+    FK_TRY(need_bytes(d, kvb_slot, (size_t)n_b * 2));
+    rq.q = arg_ptr<uint16_t>(d, q_slot);
+    rq.kva = arg_ptr<uint16_t>(d, kva_slot);
+    rq.kvb = arg_ptr<uint16_t>(d, kvb_slot);
+    FK_TRY(need_bytes(d, ck_slot, (size_t)s.n_heads * s.capacity * qk * 2));
+    FK_TRY(need_bytes(d, cv_slot, (size_t)s.n_heads * s.capacity * s.v_dim * 2));
+    rq.cache_k = arg_ptr<uint16_t>(d, ck_slot);
+    rq.cache_v = arg_ptr<uint16_t>(d, cv_slot);
+    FK_TRY(need_bytes(d, len_slot, 4));
+    rq.kv_len = arg_ptr<const uint32_t>(d, len_slot);
+    FK_TRY(need_bytes(d, tab_slot, (size_t)s.rope_dim * 4));
+    rq.rope_tab = arg_ptr<const float>(d, tab_slot);
+    rq.theta = (float)d.param("theta", 10000.0);
+    rq.scale = (float)d.param("scale", 0.0);
+    rq.traditional = d.u("traditional", 0) != 0;
+    FK_TRY(need_bytes(d, ap_slot, xcd_mla_partials_bytes(s)));
+    rq.att_partials = arg_ptr<float>(d, ap_slot);
+    if (has_c2) {
+        FK_TRY(need_bytes(d, c2_slot, xcd_sum_row_bytes(s.hidden)));
+        rq.clear2 = arg_ptr<long long>(d, c2_slot);
+    }
+    FK_TRY(need_bytes(d, op_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.out_sums = arg_ptr<long long>(d, op_slot);
+    FK_TRY(need_bytes(d, clr_slot, xcd_sum_row_bytes(s.hidden)));
+    rq.clear = arg_ptr<long long>(d, clr_slot);
+    FK_TRY(need_bytes(d, ws_slot, xcd_workspace_bytes()));
+    rq.workspace = d.args[ws_slot].ptr;
+    rq.spin_limit = d.u("spin_limit", 0);
+    rq.mark_placement = d.u("mark_placement", 0) != 0;
+    for (uint32_t j = 0; j < i; ++j) rw->reads.push_back(j);
+    rw->writes = {(uint32_t)x_slot, (uint32_t)q_slot, (uint32_t)kva_slot, (uint32_t)kvb_slot, (uint32_t)ck_slot, (uint32_t)cv_slot,
+                  (uint32_t)ap_slot, (uint32_t)op_slot, (uint32_t)clr_slot, (uint32_t)ws_slot};
+    if (has_c2) rw->writes.push_back((uint32_t)c2_slot);
+    return plan_xcd_mla(rq, l);
+}
+
 // src, out (8 bytes per workgroup): the plain read kernel (parameter blocks_per_cu)
 fk_status plan_read_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     FK_TRY(need_args(d, 2));
@@ -931,11 +1028,11 @@ fk_status plan_read_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
 }
 
 // sum row, residual [hidden] bf16, x [hidden] bf16, sum row to clear (may be the one read) [, second sum row, second row
-// to clear]: x = T(f32(row) + residual), with a second row x = T((f32(row) + T(f32(second row))) + residual)
+// to clear [, a third row to clear]]: x = T(f32(row) + residual), with a second row x = T((f32(row) + T(f32(second row))) + residual)
 // (parameter hidden)
 fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
-    const bool two = d.args.size() >= 6;
-    FK_TRY(need_args(d, two ? 6 : 4));
+    const bool two = d.args.size() >= 6, three = d.args.size() >= 7;
+    FK_TRY(need_args(d, three ? 7 : (two ? 6 : 4)));
     const uint32_t hidden = d.u("hidden");
     if (hidden == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden parameter missing");
     FK_TRY(need_bytes(d, 0, xcd_sum_row_bytes(hidden)));
@@ -950,9 +1047,13 @@ fk_status plan_xcd_reduce_d(const Dispatch& d, Launch* l, SlotRW* rw) {
         rw->reads.push_back(4);
         rw->writes.push_back(5);
     }
+    if (three) {
+        FK_TRY(need_bytes(d, 6, xcd_sum_row_bytes(hidden)));
+        rw->writes.push_back(6);
+    }
     return plan_xcd_reduce(arg_ptr<const long long>(d, 0), arg_ptr<const uint16_t>(d, 1), arg_ptr<uint16_t>(d, 2),
                            arg_ptr<long long>(d, 3), hidden, l, two ? arg_ptr<const long long>(d, 4) : nullptr,
-                           two ? arg_ptr<long long>(d, 5) : nullptr);
+                           two ? arg_ptr<long long>(d, 5) : nullptr, three ? arg_ptr<long long>(d, 6) : nullptr);
 }
 
 // Q, K0, K1, V, cache_k, cache_v, kv_len, out, partials, counters, [rope_tab]: split-key store + attention of a
@@ -1387,6 +1488,7 @@ const Family kFamilies[] = {
     {"fusekit_xcd_mlp_block", plan_xcd_mlp_d},
     {"fusekit_xcd_reduce", plan_xcd_reduce_d},
     {"fusekit_xcd_moe_block", plan_xcd_moe_d},
+    {"fusekit_xcd_mla_block", plan_xcd_mla_d},
     {"fusekit_read_reduce", plan_read_reduce_d},
     {"fusekit_route_order", plan_route_order_d},
 };
@@ -1569,7 +1671,7 @@ std::vector<std::vector<uint64_t>> derive_edges(std::vector<Node>& nodes, const 
 // The families whose launches are 512 workgroups that wait for one another (slots end: out_sums, clear_sums, workspace).
 bool is_xcd_launch(const std::string& kernel) {
     return kernel.compare(0, 22, "fusekit_xcd_attn_block") == 0 || kernel.compare(0, 21, "fusekit_xcd_mlp_block") == 0 ||
-           kernel.compare(0, 21, "fusekit_xcd_moe_block") == 0;
+           kernel.compare(0, 21, "fusekit_xcd_moe_block") == 0 || kernel.compare(0, 21, "fusekit_xcd_mla_block") == 0;
 }
 
 // An XCD-resident launch needs the whole device to itself: its 512 workgroups must all be resident at once, two per
@@ -2135,6 +2237,10 @@ fk_status fk_build_graph(fk_handle h, const fk_dispatch* list, size_t n, const u
             add_row(nd.d.args[na - 3].ptr);
             add_row(nd.d.args[na - 2].ptr);
             if (nd.d.kernel.compare(0, 21, "fusekit_xcd_moe_block") == 0) add_row(nd.d.args[na - 4].ptr);  // the shared expert's row
+            if (nd.d.kernel.compare(0, 21, "fusekit_xcd_mla_block") == 0) {
+                if (nd.d.u("has_sums", 0) != 0) add_row(nd.d.args[1].ptr);
+                if (nd.d.u("has_clear2", 0) != 0) add_row(nd.d.args[na - 4].ptr);
+            }
             if (nd.d.u("has_sums", 1) != 0) add_row(nd.d.args[0].ptr);
         }
     }

@@ -457,6 +457,7 @@ __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs 
     }
     a.x[i] = (uint16_t)f32_to_bf16_bits(v + bf16_bits_to_f32(a.residual[i]));
     if (a.clear) a.clear[at] = 0;
+    if (a.clear3) a.clear3[at] = 0;
 }
 
 // dst[(h * n + r) * gl + g] = src[r * groups + h * gl + g]: the scales (or biases) of a [n, groups] matrix, the
@@ -890,11 +891,11 @@ fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uin
 }
 
 fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
-                          Launch* out, const long long* sums2, long long* clear2) {
+                          Launch* out, const long long* sums2, long long* clear2, long long* clear3) {
     const DeviceFacts* dev;
     FK_TRY(device_facts(&dev));
     if (!sums || !residual || !x || hidden == 0) return set_error(FK_ERR_INVALID, "xcd reduce: null buffer or zero width");
-    XcdReduceArgs a{sums, residual, x, clear, hidden, sums2, clear2};
+    XcdReduceArgs a{sums, residual, x, clear, hidden, sums2, clear2, clear3};
     out->func = reinterpret_cast<const void*>(&xcd_reduce_kernel);
     out->grid = dim3(ceil_div(hidden, kBlock), 1, 1);
     out->block = dim3(kBlock, 1, 1);

@@ -240,6 +240,75 @@ struct XcdMoeRequest {
 };
 fk_status plan_xcd_moe(const XcdMoeRequest& rq, Launch* out);
 
+// ---- the attention half of a layer with low-rank keys as ONE launch -------------------------------------------
+// (q = [q_nope | q_pe] per head from q_proj; kv_a -> [latent | k_pe]; RMSNorm(latent) -> kv_b -> per head [k_nope | v];
+// K = [k_nope | rope(k_pe)], the rotated k_pe shared by all heads; n_heads / 8 heads per XCD.)
+//   every XCD   x = T((f32(row) + T(f32(second row))) + residual) -- the rows of the previous layer's expert launch --
+//               or a plain row; RMSNorm; staged
+//   XCD u       q rows of its heads AND the whole kv_a row (every XCD forms the latent row itself: no hand-over
+//               between XCDs; its copy lies in its own part of `kva`)  -> hand-over
+//               -> latent RMSNorm, kv_b rows of its heads -> hand-over
+//               -> rotation of q_pe / k_pe, cache append, attention: block = (head of the XCD, key range) -> hand-over
+//               -> merge of the ranges -> o_proj restricted to the K-slice of its heads, all output rows, added into
+//               the launch's sum row
+struct XcdMlaArgs {
+    XcdInput in;                // in.sums: the routes' row of the previous expert launch, or null
+    const long long* sums2;     // the shared expert's row (with in.sums), or null
+    long long* clear2;          // a second row this launch zeroes, or null
+    XcdMat wq, wa, wb, wo;      // q_proj, kv_a_proj, kv_b_proj, o_proj (o_proj: per-XCD re-laid-out scales / biases)
+    const uint16_t* a_norm;     // [rank] latent norm weight
+    uint32_t hl;                // heads per XCD
+    uint32_t q_rows;            // q rows of one XCD: hl * (nope + rope)
+    uint32_t a_rows;            // rank + rope
+    uint32_t rank;
+    uint32_t b_total;           // kv_b rows of one XCD: hl * (nope + v)
+    uint32_t tile_rows;         // rows per block tile of the q / kv_a projections
+    uint32_t q_tiles, a_tiles;
+    uint32_t b_rows;            // kv_b rows per block
+    uint32_t o_rows, o_cs;      // o_proj output rows per block, chunks of one XCD's K-slice of an o_proj row
+    uint16_t* q;                // [n_heads * (nope + rope)] raw projection outputs
+    uint16_t* kva;              // [8][rank + rope]: every XCD's own copy of the latent row
+    uint16_t* kvb;              // [n_heads * (nope + v)]
+    SdpaArgs sdpa;              // split-head form; k1_new points at XCD 0's k_pe, the kernel moves it to its own copy
+    long long* out_sums;
+    XcdControl* ctl;
+    uint32_t spin_limit;
+    uint32_t cs_max, work_floats, att_elems;
+    uint32_t mark_placement;
+};
+
+struct XcdMlaShape {
+    uint32_t hidden, n_heads, rank, rope_dim, nope_dim, v_dim, capacity, bits, group;
+};
+fk_status xcd_mla_supported(const XcdMlaShape& s);
+size_t xcd_mla_partials_bytes(const XcdMlaShape& s);
+size_t xcd_mla_latent_bytes(const XcdMlaShape& s);   // the `kva` slot
+struct XcdMlaRequest {
+    XcdMlaShape shape;
+    const long long* sums_in;
+    const long long* sums2_in;
+    const uint16_t* residual;
+    uint16_t* x_out;
+    long long* clear;
+    long long* clear2;
+    const uint16_t* norm_w;
+    float eps;
+    const fk_weight *wq, *wa, *wb, *wo;
+    const uint16_t* a_norm;
+    uint16_t *q, *kva, *kvb;
+    uint16_t *cache_k, *cache_v;
+    const uint32_t* kv_len;
+    const float* rope_tab;
+    float theta, scale;
+    bool traditional;
+    float* att_partials;
+    long long* out_sums;
+    void* workspace;
+    uint32_t spin_limit;
+    bool mark_placement;
+};
+fk_status plan_xcd_mla(const XcdMlaRequest& rq, Launch* out);
+
 // x = T(f32(sums) + residual): the last layer's output for the LM head.  `clear` (may be the row read, or null)
 // is zeroed element by element behind the read: the row the next token's first launch adds into.
 struct XcdReduceArgs {
@@ -251,6 +320,7 @@ struct XcdReduceArgs {
     // with a second row (the shared expert's of the expert launch): x = T((f32(sums) + T(f32(sums2))) + residual)
     const long long* sums2;
     long long* clear2;
+    long long* clear3;   // one more row to zero, or null
 };
 
 struct XcdLayerShape {
@@ -327,6 +397,6 @@ fk_status plan_xcd_layer(const Launch& attn, const Launch& mlp, Launch* out);
 fk_status plan_xcd_token(const XcdAttnArgs* h_attn, const XcdMlpArgs* h_mlp, uint32_t n_layers, uint32_t bits,
                          const XcdAttnArgs* d_attn, const XcdMlpArgs* d_mlp, uint32_t attn_lds, uint32_t mlp_lds, Launch* out);
 fk_status plan_xcd_reduce(const long long* sums, const uint16_t* residual, uint16_t* x, long long* clear, uint32_t hidden,
-                          Launch* out, const long long* sums2 = nullptr, long long* clear2 = nullptr);
+                          Launch* out, const long long* sums2 = nullptr, long long* clear2 = nullptr, long long* clear3 = nullptr);
 
 }  // namespace fk

@@ -565,6 +565,21 @@ def xcd_moe_supported(hidden, inter, shared_inter, experts, top_k, bits, group) 
                                     C.c_uint32(top_k), C.c_uint32(bits), C.c_uint32(group)) == FK_OK
 
 
+def xcd_mla_supported(hidden, n_heads, rank, rope_dim, nope_dim, v_dim, capacity, bits, group) -> bool:
+    """Can the attention half of a layer with low-rank keys run as one XCD-resident launch (fk_xcd_mla_supported)?"""
+    u = C.c_uint32
+    return lib.fk_xcd_mla_supported(u(hidden), u(n_heads), u(rank), u(rope_dim), u(nope_dim), u(v_dim), u(capacity), u(bits),
+                                    u(group)) == FK_OK
+
+
+def xcd_mla_workspace_bytes(n_heads, rank, rope_dim, v_dim):
+    """(bytes of the `kva` slot, bytes of the attention partial rows) of fusekit_xcd_mla_block."""
+    a, b = C.c_size_t(), C.c_size_t()
+    check(lib.fk_xcd_mla_workspace_bytes(C.c_uint32(n_heads), C.c_uint32(rank), C.c_uint32(rope_dim), C.c_uint32(v_dim),
+                                         C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
 lib.fk_xcd_moe_scratch_bytes.restype = C.c_size_t
 
 

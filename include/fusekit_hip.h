@@ -611,6 +611,20 @@ fk_status fk_xcd_moe_supported(uint32_t hidden, uint32_t inter, uint32_t shared_
                                uint32_t bits, uint32_t group);
 /* Bytes of the launch's scratch slot: per-XCD copies of the router logits and the SwiGLU rows of the eight units. */
 size_t fk_xcd_moe_scratch_bytes(uint32_t inter);
+/* The attention half of a layer with low-rank keys as ONE such launch, dispatch family `fusekit_xcd_mla_block`:
+ * replaces, for one layer and one token, the two rmsnorm_qkv.rs launches (norm + q / kv_a, latent norm + kv_b), the
+ * split-key cache store with its rotations, sdpa_decode.rs and linear_residual.rs (o_proj).  n_heads / 8 heads per XCD;
+ * every XCD forms the whole kv_a row itself (its own copy in the `kva` slot), so the latent norm and kv_b need no
+ * exchange between XCDs; o_proj is cut along K by XCD as in fusekit_xcd_attn_block and added into a sum row.  The input
+ * is a plain row or the two rows of the previous layer's fusekit_xcd_moe_block (x = T((f32(row) + T(f32(shared row))) +
+ * residual)).  Same arithmetic and rounding points per output as the launches it replaces.  Requires 4-bit weights,
+ * 8 .. 32 heads in multiples of 8, hidden a multiple of 256 up to 4096, a latent width that is a multiple of 128;
+ * slot order at the planner (fusekit_amd/csrc/dispatcher.hip).  The exclusive-use rule below applies. */
+fk_status fk_xcd_mla_supported(uint32_t hidden, uint32_t n_heads, uint32_t rank, uint32_t rope_dim, uint32_t nope_dim,
+                               uint32_t v_dim, uint32_t capacity, uint32_t bits, uint32_t group);
+/* Bytes of that family's `kva` slot (eight copies of the latent row) and of its attention partial rows. */
+fk_status fk_xcd_mla_workspace_bytes(uint32_t n_heads, uint32_t rank, uint32_t rope_dim, uint32_t v_dim, size_t *latent_bytes,
+                                     size_t *attention_partial_bytes);
 /* The o_proj and down_proj slots of the two families take their scales and biases re-laid out per K-slice:
  * dst[(h * n + r) * (groups / 8) + g] = src[r * groups + h * (groups / 8) + g] for the [n, groups] array of a
  * matrix (same size as the source).  An XCD then reads its slice of every row as one contiguous stream; in the
