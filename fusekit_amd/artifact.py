@@ -42,6 +42,7 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
         for name, (buf, dtype, zero) in rt.scratch_symbols().items():
             scratch(name, buf, dtype, zero)
         _parameter_symbols(rt, sym)
+        _kslice_symbols(rt, sym)
         return sym
     for name in ("token", "step_counter", "offset", "kv_len", "hist_counter", "history", "sdpa_counters", "argmax_ws",
                  "head_argmax_ws"):
@@ -73,14 +74,18 @@ def _symbols(rt: DecoderRuntime) -> Dict[int, dict]:
             scratch(f"cache_k.{l}", rt.cache_k[l], "bfloat16", zero=True)
             scratch(f"cache_v.{l}", rt.cache_v[l], "bfloat16", zero=True)
     _parameter_symbols(rt, sym)
-    # scales / biases of o_proj and down_proj as the two-launch layer binds them: a parameter behind a load-time
-    # re-layout, named by the parameter and the transform
+    _kslice_symbols(rt, sym)
+    return sym
+
+
+def _kslice_symbols(rt, sym: Dict[int, dict]) -> None:
+    """Scales / biases of o_proj and down_proj as the XCD-resident launches bind them: a parameter behind a load-time
+    re-layout, named by the parameter and the transform."""
     for path, (sc, bi) in getattr(rt, "xcd_kmeta", {}).items():
         W = rt.w.mats[path]
         for buf, leaf in ((sc, ".scales"), (bi, ".biases")):
             sym[buf.ptr] = dict(role="external", source_path=path + leaf, dtype="bfloat16", transform="xcd_kslice",
                                 shape=[W.n, W.k // W.group], size_bytes=buf.nbytes)
-    return sym
 
 
 def _parameter_symbols(rt, sym: Dict[int, dict]) -> None:

@@ -60,7 +60,8 @@ class MoeConfig:
     direct_head_argmax: bool = True  # the LM head selects the greedy token itself where its shape allows
     xcd_moe: bool = True       # router + routed / shared experts + reduction of a layer as ONE XCD-resident launch, where
                                # the shape admits it (MoeRuntime.xcd tells); off: the per-dispatch families
-    xcd_spin_limit: int = 0    # hand-over wait bound of that launch (0: the library's default)
+    xcd_attn: bool = True      # with xcd_moe: the attention half of every layer as ONE launch too (two launches per layer)
+    xcd_spin_limit: int = 0    # hand-over wait bound of these launches (0: the library's default)
 
     @property
     def qk_dim(self) -> int:
@@ -223,11 +224,28 @@ class MoeRuntime:
         # the expert block as one launch, cut by route over the XCDs (where the shape admits it)
         self.xcd = bool(c.xcd_moe and c.swiglu_variant == 1 and c.first_dense < c.n_layers and
                         native.xcd_moe_supported(c.hidden, c.moe_inter, c.shared_inter, c.n_experts, c.top_k, c.bits, c.group))
+        # ... and the attention half (low-rank keys) as one launch: then a layer is two launches
+        self.xcd_attn = bool(self.xcd and c.xcd_attn and c.fuse_attention and
+                             native.xcd_mla_supported(c.hidden, c.n_heads, c.kv_lora_rank, c.rope_dim, c.nope_dim, c.v_dim,
+                                                      c.capacity, c.bits, c.group))
         if self.xcd:
             self.xcd_ctl = z(native.xcd_workspace_bytes(c.n_heads, c.qk_dim)[0])
-            self.xcd_sums = [z(native.xcd_sum_row_bytes(c.hidden)) for _ in range(3)]   # routes, shared expert, cleared
+            # expert launch alone: routes, shared expert, a row to clear; with the attention launch six rows rotate:
+            # P0, P1 (attention outputs), then the (routes, shared expert) pairs of even and of odd layers
+            self.xcd_sums = [z(native.xcd_sum_row_bytes(c.hidden)) for _ in range(6 if self.xcd_attn else 3)]
             self.xcd_x = B(c.hidden * 2)
             self.xcd_scratch = z(native.xcd_moe_scratch_bytes(c.moe_inter))
+        self.xcd_kmeta: Dict[str, tuple] = {}
+        if self.xcd_attn:
+            lat, part = native.xcd_mla_workspace_bytes(c.n_heads, c.kv_lora_rank, c.rope_dim, c.v_dim)
+            self.xcd_kva, self.xcd_att_partials = z(lat), B(part)
+            self.xcd_xb = B(c.hidden * 2)
+            for l in range(c.n_layers):   # o_proj's scales and biases per K-slice, once per matrix
+                name = f"layers.{l}.self_attn.o_proj"
+                Wo = weights.mats[name]
+                self.xcd_kmeta[name] = (native.xcd_kslice_meta(Wo.scales, Wo.n, Wo.k // Wo.group),
+                                        native.xcd_kslice_meta(Wo.biases, Wo.n, Wo.k // Wo.group))
+            native.sync()
         self._rows_variants: Dict[int, "MoeRowsVariant"] = {}
         self.tasks = self.build_tasks()
         self.graph = self.d.build_decode_graph(self.tasks, False)
@@ -263,6 +281,9 @@ class MoeRuntime:
                           dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, output_scale=1.0)))
         n_a, half_a = c.kv_lora_rank + c.rope_dim, (c.kv_lora_rank + c.rope_dim) // 2
         n_b = c.n_heads * (c.nope_dim + c.v_dim)
+        if self.xcd_attn:
+            self._two_launch_tasks(t, name, wargs, quant)
+            return self._head_tasks(t, name, wargs, emb)
         for l in range(c.n_layers):
             p = f"layers.{l}."
             Wq, Wa, Wb = (w.mats[p + f"self_attn.{n}"] for n in ("q_proj", "kv_a_proj_with_mqa", "kv_b_proj"))
@@ -374,6 +395,67 @@ class MoeRuntime:
                                arg(self.x[1]), arg(self.x[0]), arg(self.moe_ws)],
                               dict(quant, k=c.moe_inter, o=c.hidden, experts=c.n_experts, tokens=1, top_k=c.top_k, x_rows=c.top_k,
                                    has_shared=1, shared_k=c.shared_inter, has_extra=1)))
+        return self._head_tasks(t, name, wargs, emb)
+
+    def _two_launch_tasks(self, t, name, wargs, quant) -> None:
+        """A layer as TWO launches (families fusekit_xcd_mla_block / fusekit_xcd_moe_block; a dense layer keeps its
+        per-dispatch MLP behind fusekit_xcd_reduce).  Sum rows: the attention launch of layer l adds into P[l % 2] and
+        clears the pair Q[l % 2] its expert launch adds into; the expert launch reads P[l % 2], adds into Q[l % 2] and
+        clears P[(l + 1) % 2]; the next attention launch reads Q[l % 2].  The closing fusekit_xcd_reduce clears what the
+        last layer left, so that every row a token's first launches add into holds zeros."""
+        c, w = self.cfg, self.w
+        P = lambda i: arg(self.xcd_sums[i % 2])
+        Q = lambda i: (arg(self.xcd_sums[2 + 2 * (i % 2)]), arg(self.xcd_sums[3 + 2 * (i % 2)]))
+        mla = dict(quant, hidden=c.hidden, n_heads=c.n_heads, rank=c.kv_lora_rank, rope_dim=c.rope_dim, nope_dim=c.nope_dim,
+                   v_dim=c.v_dim, capacity=c.capacity, eps=c.eps, theta=c.theta, traditional=int(c.rope_traditional),
+                   spin_limit=c.xcd_spin_limit)
+        from_experts = False          # the previous layer ended in an expert launch (two sum rows + the row in xcd_xb)
+        for l in range(c.n_layers):
+            p = f"layers.{l}."
+            Wq, Wa, Wb, Wo = (w.mats[p + f"self_attn.{n}"] for n in ("q_proj", "kv_a_proj_with_mqa", "kv_b_proj", "o_proj"))
+            sc, bi = self.xcd_kmeta[p + "self_attn.o_proj"]
+            a = list(Q(l - 1)) if from_experts else []
+            a += [arg(self.xcd_xb) if from_experts else arg(self.x[0]), arg(self.xcd_x), arg(w.vecs[p + "input_layernorm"])]
+            a += wargs(Wq) + wargs(Wa) + [arg(w.vecs[p + "self_attn.kv_a_layernorm"])] + wargs(Wb) + [arg(Wo.w), arg(sc), arg(bi)]
+            a += [arg(self.q), arg(self.xcd_kva), arg(self.kvb), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+                  arg(self.rope_tab), arg(self.xcd_att_partials)]
+            qr, qs = Q(l)
+            a += [qs, P(l), qr, arg(self.xcd_ctl)]      # clear2 = the shared row, out, clear = the routes' row
+            t.append(Dispatch(name("xcd_mla_block"), a, dict(mla, has_sums=2 if from_experts else 0, has_clear2=1,
+                                                            mark_placement=int(l == 0))))
+            post = w.vecs[p + "post_attention_layernorm"]
+            if l < c.first_dense:   # x1 = T(P + x) as a row, then the per-dispatch MLP
+                t.append(Dispatch(name("xcd_reduce"), [P(l), arg(self.xcd_x), arg(self.x[1]), P(l)], dict(hidden=c.hidden)))
+                Wg, Wu, Wd = (w.mats[p + f"mlp.{n}_proj"] for n in ("gate", "up", "down"))
+                t.append(Dispatch(name("rmsnorm_gateup_swiglu"),
+                                  [arg(self.x[1]), arg(post), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales),
+                                   arg(Wg.biases), arg(Wu.biases), arg(self.mid, c.dense_inter * 2)],
+                                  dict(quant, hidden=c.hidden, inter=c.dense_inter, eps=c.eps, variant=c.swiglu_variant,
+                                       has_norm=1)))
+                t.append(Dispatch(name("linear_residual"),
+                                  [arg(self.mid, c.dense_inter * 2)] + wargs(Wd) + [arg(self.x[1]), arg(self.x[0])],
+                                  dict(quant, m=c.dense_inter, n=c.hidden)))
+                from_experts = False
+                continue
+            Wr = w.mats[p + "mlp.gate"]
+            Eg, Eu, Ed = (w.mats[p + f"mlp.switch_mlp.{n}_proj"] for n in ("gate", "up", "down"))
+            Sg, Su, Sd = (w.mats[p + f"mlp.shared_experts.{n}_proj"] for n in ("gate", "up", "down"))
+            m = [P(l), arg(self.xcd_x), arg(self.xcd_xb), arg(post), arg(Wr.w), arg(self.route_scale)]
+            for W in (Eg, Eu, Ed, Sg, Su, Sd):
+                m += wargs(W)
+            m += [arg(self.route_logits, 2 * c.n_experts, 2 * c.n_experts * l), arg(self.route_idx, 4 * c.top_k, 4 * c.top_k * l),
+                  arg(self.route_weight, 2 * c.top_k, 2 * c.top_k * l), arg(self.xcd_scratch), qs, qr, P(l + 1), arg(self.xcd_ctl)]
+            t.append(Dispatch(name("xcd_moe_block"), m,
+                              dict(quant, hidden=c.hidden, inter=c.moe_inter, shared_inter=c.shared_inter, experts=c.n_experts,
+                                   top_k=c.top_k, eps=c.eps, variant=c.swiglu_variant, has_sums=1, spin_limit=c.xcd_spin_limit)))
+            from_experts = True
+        if from_experts:   # the last layer's rows + its residual row -> x[0] for the LM head; leaves every row zero
+            qr, qs = Q(c.n_layers - 1)
+            t.append(Dispatch(name("xcd_reduce"), [qr, arg(self.xcd_xb), arg(self.x[0]), qr, qs, qs, P(c.n_layers - 1)],
+                              dict(hidden=c.hidden)))
+
+    def _head_tasks(self, t, name, wargs, emb) -> List[Dispatch]:
+        c, w = self.cfg, self.w
         head_args = [arg(self.x[0]), arg(w.vecs["final_norm"])] + wargs(emb) + [arg(self.logits)]
         head_params = dict(bits=16, group=64, hidden=c.hidden, vocab=c.vocab, eps=c.eps)
         # the direct head (dispatch.py:3458-3505) as one launch where the vocabulary matrix takes the row-group GEMV
@@ -406,6 +488,9 @@ class MoeRuntime:
         if self.xcd:
             out["xcd.control"], out["xcd.scratch"] = (self.xcd_ctl, "uint32", True), (self.xcd_scratch, "uint32", True)
             out["xcd.x"] = (self.xcd_x, "bfloat16", False)
+            if self.xcd_attn:
+                out["xcd.x.1"], out["xcd.kva"] = (self.xcd_xb, "bfloat16", False), (self.xcd_kva, "bfloat16", True)
+                out["xcd.attention_partials"] = (self.xcd_att_partials, "float32", False)
             for i, b in enumerate(self.xcd_sums):
                 out[f"xcd.sums.{i}"] = (b, "uint32", True)
         return out

@@ -27,13 +27,17 @@ def _small_cfg(**kw):
                                                  (4, True, dict(n_heads=4, nope_dim=64, rope_dim=32, v_dim=64, n_experts=16, top_k=4)),
                                                  # the expert block as one launch: 3 of 8 XCDs busy, then all 8
                                                  (4, True, dict(hidden=512, xcd_moe=True)),
-                                                 (4, False, dict(hidden=512, n_experts=16, top_k=6, n_shared=2, xcd_moe=True))])
+                                                 (4, False, dict(hidden=512, n_experts=16, top_k=6, n_shared=2, xcd_moe=True)),
+                                                 # ... and the attention half as one launch too: two launches per layer
+                                                 (4, True, dict(hidden=512, n_heads=8, n_experts=16, top_k=6, n_shared=2, xcd_moe=True)),
+                                                 (4, False, dict(hidden=512, n_heads=8, n_layers=4, first_dense=2, xcd_moe=True))])
 def test_greedy_tokens_and_routes_match_oracle(fk, bits, traditional, kw):
     from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
     cfg = _small_cfg(bits=bits, rope_traditional=traditional, **kw)
     W = MoeWeights.random_init(cfg, seed=2)
     rt = MoeRuntime(cfg, W)
     assert rt.xcd == bool(kw.get("xcd_moe", False)), fk.lib.fk_last_error().decode()
+    assert rt.xcd_attn == (rt.xcd and cfg.n_heads % 8 == 0), fk.lib.fk_last_error().decode()
     od = OracleMoeDecoder(cfg, W)
     prompt = rng(1).integers(0, cfg.vocab, 6).tolist()
     n = 20
@@ -183,24 +187,28 @@ def test_full_size_clear_margin_model_32_free_running_tokens_equal_the_oracle(fk
     assert again == want
 
     # The same run with every layer's expert block as ONE launch (router, ranking, routed and shared experts, weighted
-    # sum: family fusekit_xcd_moe_block): the same tokens and, step by step and layer by layer, the same route sets.
+    # sum: family fusekit_xcd_moe_block), then with the attention half as one launch as well (fusekit_xcd_mla_block: two
+    # launches per layer): the same tokens and, step by step and layer by layer, the same route sets.
     import dataclasses
-    rx = MoeRuntime(dataclasses.replace(cfg, xcd_moe=True), W)
-    assert rx.xcd and sum(t.kernel.startswith("fusekit_xcd_moe_block") for t in rx.tasks) == n_moe
-    got_x, tok = [], prompt[0]
-    for i in range(63):
-        nxt, _ = rx.d.decode_host_loop(rx.graph, rx.uniforms, i, [tok])
-        routes = rx.routes()[cfg.first_dense:]
-        for l in range(n_moe):
-            assert sorted(routes[l].tolist()) == fx["routes"][i][l], (i, l)
-        if i >= 31:
-            got_x.append(nxt[0])
-        tok = prompt[i + 1] if i + 1 < 32 else nxt[0]
-    assert got_x == want
-    rx.reset()
-    again, _, _ = rx.generate(prompt, 32)
-    assert again == want
-    del rx
+    for attn in (False, True):
+        rx = MoeRuntime(dataclasses.replace(cfg, xcd_moe=True, xcd_attn=attn), W)
+        assert rx.xcd and rx.xcd_attn == attn
+        assert sum(t.kernel.startswith("fusekit_xcd_moe_block") for t in rx.tasks) == n_moe
+        assert sum(t.kernel.startswith("fusekit_xcd_mla_block") for t in rx.tasks) == (cfg.n_layers if attn else 0)
+        got_x, tok = [], prompt[0]
+        for i in range(63):
+            nxt, _ = rx.d.decode_host_loop(rx.graph, rx.uniforms, i, [tok])
+            routes = rx.routes()[cfg.first_dense:]
+            for l in range(n_moe):
+                assert sorted(routes[l].tolist()) == fx["routes"][i][l], (attn, i, l)
+            if i >= 31:
+                got_x.append(nxt[0])
+            tok = prompt[i + 1] if i + 1 < 32 else nxt[0]
+        assert got_x == want, attn
+        rx.reset()
+        again, _, _ = rx.generate(prompt, 32)
+        assert again == want, attn
+        del rx
 
     # The same model at full size with EIGHT active token rows in one pass over the weights (shared-stream matmuls
     # for the dense projections and the shared experts, row forms of the store, the attention and the router,
