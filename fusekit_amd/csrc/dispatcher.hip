@@ -924,7 +924,8 @@ fk_status plan_xcd_moe_d(const Dispatch& d, Launch* l, SlotRW* rw) {
 
 // The attention half of a layer with low-rank keys as one XCD-resident launch (xcd_mla_kernel):
 // [sums_in, shared_sums_in], residual, x_out, norm_w, W_q, s_q, b_q, W_kv_a, s_a, b_a, latent_norm_w, W_kv_b, s_b, b_b,
-// W_o, s_o, b_o (o_proj's scales and biases re-laid out per K-slice: fk_xcd_kslice_meta), q, kva (fk_xcd_mla_latent_bytes),
+// W_o, s_o, b_o (o_proj's scales and biases re-laid out per K-slice: fk_xcd_kslice_meta), q (twice n_heads * (nope + rope)
+// elements: the raw rows, then the rows with q_pe rotated), kva (fk_xcd_mla_latent_bytes),
 // kvb, cache_k, cache_v, kv_len, rope_tab, att_partials, [clear2_sums], out_sums, clear_sums, workspace.
 // Parameters: hidden, n_heads, rank, rope_dim, nope_dim, v_dim, capacity, bits, group, eps, theta, traditional, scale,
 // has_sums (0: the input is the residual row alone; 2: the two rows of an expert launch), has_clear2, spin_limit,
@@ -981,7 +982,7 @@ fk_status plan_xcd_mla_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     rq.wo = &W[3];
     FK_TRY(need_bytes(d, an_slot, (size_t)s.rank * 2));
     rq.a_norm = arg_ptr<const uint16_t>(d, an_slot);
-    FK_TRY(need_bytes(d, q_slot, (size_t)s.n_heads * qk * 2));
+    FK_TRY(need_bytes(d, q_slot, (size_t)2 * s.n_heads * qk * 2));   // raw rows, then the rows with q_pe rotated
     FK_TRY(need_bytes(d, kva_slot, xcd_mla_latent_bytes(s)));
     FK_TRY(need_bytes(d, kvb_slot, (size_t)n_b * 2));
     rq.q = arg_ptr<uint16_t>(d, q_slot);

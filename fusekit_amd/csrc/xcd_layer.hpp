@@ -266,10 +266,10 @@ struct XcdMlaArgs {
     uint32_t q_tiles, a_tiles;
     uint32_t b_rows;            // kv_b rows per block
     uint32_t o_rows, o_cs;      // o_proj output rows per block, chunks of one XCD's K-slice of an o_proj row
-    uint16_t* q;                // [n_heads * (nope + rope)] raw projection outputs
+    uint16_t* q;                // [2][n_heads * (nope + rope)]: raw projection outputs, then the rows with q_pe rotated
     uint16_t* kva;              // [8][rank + rope]: every XCD's own copy of the latent row
     uint16_t* kvb;              // [n_heads * (nope + v)]
-    SdpaArgs sdpa;              // split-head form; k1_new points at XCD 0's k_pe, the kernel moves it to its own copy
+    SdpaArgs sdpa;              // geometry of the attention phase and the split-head parameters of the rotations
     long long* out_sums;
     XcdControl* ctl;
     uint32_t spin_limit;

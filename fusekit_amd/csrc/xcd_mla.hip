@@ -211,6 +211,25 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
     if (!xcd_wait_ok(okw)) return;
     FK_XCD_STAMP(0, 4);
 
+    // position of the new token, as the attention blocks settle it
+    const uint32_t span = a.sdpa.chunk_len * a.sdpa.chunks_per_block;
+    const uint32_t covered = a.sdpa.n_splits * span < a.sdpa.capacity ? a.sdpa.n_splits * span : a.sdpa.capacity;
+    const uint32_t kv_len = kv_len0 < 1u ? 1u : (kv_len0 > covered ? covered : kv_len0);
+    const uint32_t pos = kv_len - 1, cache_row = pos % a.sdpa.capacity;
+    // ---- rotations: one wave per head of the XCD (in the last blocks, which hold no q / kv_a tile) writes the head's q
+    // with its second part rotated into the second half of `q`, and the rotated k_pe into the head's new cache row ----
+    if (slot >= kXcdSlots - a.hl && wave == 3) {
+        const uint32_t head = xcd * a.hl + (kXcdSlots - 1 - slot);
+        const uint32_t d0 = a.sdpa.q0_dim, d1 = a.sdpa.qk_dim - d0;
+        const uint16_t* qh = a.q + (size_t)head * a.sdpa.qk_dim;
+        uint16_t* qr = a.q + (size_t)a.sdpa.n_heads * a.sdpa.qk_dim + (size_t)head * a.sdpa.qk_dim;
+        split_head_transform(qh, qh + d0, qr, d0, d1, a.sdpa.rope_dims, a.sdpa.traditional != 0, pos, a.sdpa.base_log2, lane,
+                             a.sdpa.rope_tab);
+        const uint16_t* kpe = a.kva + (size_t)xcd * a.a_rows + a.rank;
+        uint16_t* krow = a.sdpa.cache_k_w + ((size_t)head * a.sdpa.capacity + cache_row) * a.sdpa.qk_dim + d0;
+        split_head_transform(kpe, kpe, krow, 0u, d1, a.sdpa.rope_dims, a.sdpa.traditional != 0, pos, a.sdpa.base_log2, lane,
+                             a.sdpa.rope_tab);
+    }
     // ---- latent RMSNorm, kv_b rows of the XCD's heads ----
     {
         const uint32_t n8 = a.rank >> 3;   // at most 256 groups: one per thread
@@ -243,9 +262,22 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
     }
     tile_partials<KIND, NLB, kBlock>(a.wb, tb, pb, rb, xs, sx, meta + MW, work);
     __syncthreads();
-    if (b_n) {
+    if (b_n) {   // [k_nope | v] of a head: into `kvb` and straight into the head's new cache rows
         uint16_t* dst = a.kvb + (size_t)xcd * a.b_total + b0;
-        tile_rows<false, true>(tb, work, work, [&](uint32_t r, float s0, float) { dst[r] = (uint16_t)f32_to_bf16_bits(s0); });
+        const uint32_t d0 = a.sdpa.q0_dim, packed = d0 + a.sdpa.v_dim, qkd = a.sdpa.qk_dim, vd = a.sdpa.v_dim, cap = a.sdpa.capacity;
+        uint16_t* ck = a.sdpa.cache_k_w;
+        uint16_t* cv = a.sdpa.cache_v_w;
+        const uint32_t head0 = xcd * a.hl;
+        tile_rows<false, true>(tb, work, work, [&](uint32_t r, float s0, float) {
+            const uint16_t v16 = (uint16_t)f32_to_bf16_bits(s0);
+            dst[r] = v16;
+            const uint32_t rr = b0 + r, hl_ = rr / packed, w = rr - hl_ * packed;
+            const size_t crow = (size_t)(head0 + hl_) * cap + cache_row;
+            if (w < d0)
+                ck[crow * qkd + w] = v16;
+            else
+                cv[crow * vd + (w - d0)] = v16;
+        });
     }
     FK_XCD_STAMP(0, 5);
     xcd_barrier<0>(sync, okw);
@@ -255,10 +287,10 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
     // ---- rotation + cache append + attention: block = (head of the XCD, key range) ----
     {
         const uint32_t head = slot % a.hl, split = slot / a.hl;
-        if (split < a.sdpa.n_splits) {
+        if (split < a.sdpa.n_splits) {   // q rotated and the new rows cached by the phase before: plain attention
             SdpaArgs sd = a.sdpa;
-            sd.k1_new += (size_t)xcd * a.a_rows;   // this XCD's copy of the latent row
-            sdpa_block<1, 2, SdpaArgs, 0, false, true>(sd, kv_len0, split, xcd * a.hl + head, 0u, 1u, work);
+            sd.q += (size_t)a.sdpa.n_heads * a.sdpa.qk_dim;   // the rotated copy
+            sdpa_block<1, 0, SdpaArgs, 0, false, true>(sd, kv_len0, split, xcd * a.hl + head, 0u, 1u, work);
         }
     }
     FK_XCD_STAMP(0, 7);
@@ -268,9 +300,6 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
 
     // ---- merge the ranges of each of the XCD's heads (range order), rows to LDS ----
     {
-        const uint32_t span = a.sdpa.chunk_len * a.sdpa.chunks_per_block;
-        const uint32_t covered = a.sdpa.n_splits * span < a.sdpa.capacity ? a.sdpa.n_splits * span : a.sdpa.capacity;
-        const uint32_t kv_len = kv_len0 < 1u ? 1u : (kv_len0 > covered ? covered : kv_len0);
         const uint32_t n_active = (kv_len + span - 1) / span;
         const uint32_t row = a.sdpa.v_dim + 2;
         for (uint32_t h = wave; h < a.hl; h += kBlock / kWave) {

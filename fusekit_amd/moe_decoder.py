@@ -239,6 +239,7 @@ class MoeRuntime:
         if self.xcd_attn:
             lat, part = native.xcd_mla_workspace_bytes(c.n_heads, c.kv_lora_rank, c.rope_dim, c.v_dim)
             self.xcd_kva, self.xcd_att_partials = z(lat), B(part)
+            self.xcd_q = B(2 * c.n_heads * c.qk_dim * 2)     # raw q rows, then the rows with q_pe rotated
             self.xcd_xb = B(c.hidden * 2)
             for l in range(c.n_layers):   # o_proj's scales and biases per K-slice, once per matrix
                 name = f"layers.{l}.self_attn.o_proj"
@@ -417,7 +418,7 @@ class MoeRuntime:
             a = list(Q(l - 1)) if from_experts else []
             a += [arg(self.xcd_xb) if from_experts else arg(self.x[0]), arg(self.xcd_x), arg(w.vecs[p + "input_layernorm"])]
             a += wargs(Wq) + wargs(Wa) + [arg(w.vecs[p + "self_attn.kv_a_layernorm"])] + wargs(Wb) + [arg(Wo.w), arg(sc), arg(bi)]
-            a += [arg(self.q), arg(self.xcd_kva), arg(self.kvb), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
+            a += [arg(self.xcd_q), arg(self.xcd_kva), arg(self.kvb), arg(self.cache_k[l]), arg(self.cache_v[l]), arg(self.kv_len),
                   arg(self.rope_tab), arg(self.xcd_att_partials)]
             qr, qs = Q(l)
             a += [qs, P(l), qr, arg(self.xcd_ctl)]      # clear2 = the shared row, out, clear = the routes' row
@@ -490,7 +491,7 @@ class MoeRuntime:
             out["xcd.x"] = (self.xcd_x, "bfloat16", False)
             if self.xcd_attn:
                 out["xcd.x.1"], out["xcd.kva"] = (self.xcd_xb, "bfloat16", False), (self.xcd_kva, "bfloat16", True)
-                out["xcd.attention_partials"] = (self.xcd_att_partials, "float32", False)
+                out["xcd.attention_partials"], out["xcd.q"] = (self.xcd_att_partials, "float32", False), (self.xcd_q, "bfloat16", False)
             for i, b in enumerate(self.xcd_sums):
                 out[f"xcd.sums.{i}"] = (b, "uint32", True)
         return out

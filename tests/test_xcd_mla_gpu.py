@@ -58,7 +58,7 @@ def test_xcd_mla_block(fk, hidden, n_heads, rank, capacity, steps, traditional, 
     zero_row = _sum_row(fk, hidden)
     junk = np.full_like(zero_row, 0x0123456789abcdef)
     b = dict(res=fk.DeviceBuffer(hidden * 2), x=fk.DeviceBuffer(hidden * 2), nw=_dev(fk, norm_w), an=_dev(fk, a_norm),
-             q=fk.DeviceBuffer(n_heads * qk * 2), kva=fk.zeros(lat_bytes), kvb=fk.DeviceBuffer(n_b * 2),
+             q=fk.DeviceBuffer(2 * n_heads * qk * 2), kva=fk.zeros(lat_bytes), kvb=fk.DeviceBuffer(n_b * 2),
              ck=fk.zeros(n_heads * capacity * qk * 2), cv=fk.zeros(n_heads * capacity * vd * 2), kv_len=fk.zeros(4), off=fk.zeros(4),
              step=fk.zeros(4), tab=fk.DeviceBuffer(rope * 4), ap=fk.DeviceBuffer(ap_bytes), out=_dev(fk, zero_row),
              clr=_dev(fk, junk), clr2=_dev(fk, junk), p1=_dev(fk, zero_row), p2=_dev(fk, zero_row))
@@ -96,7 +96,8 @@ def test_xcd_mla_block(fk, hidden, n_heads, rank, capacity, steps, traditional, 
             x = oracle.f32_to_bf16(((_row_f32(fk, r1, hidden) + shared).astype(np.float32) + oracle.bf16_to_f32(res)).astype(np.float32))
         d.dispatch_batch([step, task])
         sampled = pos % 16 == 0 or pos >= steps - 10
-        qg, ag, bg = b["q"].to_numpy(np.uint16), b["kva"].to_numpy(np.uint16, (8, n_a)), b["kvb"].to_numpy(np.uint16)
+        q2 = b["q"].to_numpy(np.uint16, (2, n_heads * qk))    # raw rows, then the rows with their second part rotated
+        qg, ag, bg = q2[0], b["kva"].to_numpy(np.uint16, (8, n_a)), b["kvb"].to_numpy(np.uint16)
         k_pe = ag[0, rank:].copy().reshape(1, rope)
         if not sampled:   # the oracle still appends this position's rows: it follows the GPU's own, checked when sampled
             oracle.kv_store_split(bg, packed, k_pe, 1, bg[nope:], packed, n_heads, nope, rope, vd, rope, traditional, theta, pos, pos,
@@ -130,7 +131,11 @@ def test_xcd_mla_block(fk, hidden, n_heads, rank, capacity, steps, traditional, 
             oracle.kv_store_split(qh[h, :nope].copy(), nope, qh[h, nope:].copy(), 1, np.zeros(1, np.uint16), 1, 1, nope, rope, 1, rope,
                                   traditional, theta, pos, 0, 1, row_k, row_v)
             qh[h] = row_k
-        att = oracle.sdpa_decode(qh.reshape(-1), ck, cv, n_heads, n_heads, qk, vd, pos + 1, capacity, scale)
+        fq, fr = oracle.bf16_to_f32(q2[1]).reshape(n_heads, qk), oracle.bf16_to_f32(qh.reshape(-1)).reshape(n_heads, qk)
+        q_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(fr).max(axis=1, keepdims=True), 1e-30))) - 7)
+        assert np.all(np.abs(fq - fr) <= q_ulp) and np.mean(q2[1] != qh.reshape(-1)) <= 0.01
+        assert np.array_equal(q2[1].reshape(n_heads, qk)[:, :nope], qg.reshape(n_heads, qk)[:, :nope])
+        att = oracle.sdpa_decode(q2[1].copy(), ck, cv, n_heads, n_heads, qk, vd, pos + 1, capacity, scale)
         y_ref_acc = oracle.linear_acc(Wo, att)
         acc = _row_values(fk, b["out"].to_numpy(np.int64), hidden)
         rel = float(np.linalg.norm(acc - y_ref_acc) / np.linalg.norm(y_ref_acc))
