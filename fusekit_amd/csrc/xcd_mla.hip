@@ -159,8 +159,11 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
     const XcdMat A = pick_mat2(is_q, a.wq, a.wa);
     const Tile ta = make_tile((is_q ? xcd * a.q_rows : 0u) + pr0, pr_n, 0, A.cpr);
     // kv_b: the XCD's heads' rows ([k_nope | v] per head), all of the latent width
+    // (the last 2 hl blocks of the XCD take no kv_b rows: they rotate q_pe / k_pe of its heads meanwhile)
+    const uint32_t n_rot = 2u * a.hl;
+    const bool is_rot = slot >= kXcdSlots - n_rot;
     const uint32_t b0 = slot * a.b_rows;
-    const uint32_t b_n = b0 < a.b_total ? ((a.b_total - b0) < a.b_rows ? (a.b_total - b0) : a.b_rows) : 0u;
+    const uint32_t b_n = (!is_rot && b0 < a.b_total) ? ((a.b_total - b0) < a.b_rows ? (a.b_total - b0) : a.b_rows) : 0u;
     const Tile tb = make_tile(xcd * a.b_total + b0, b_n, 0, a.wb.cpr);
     // o_proj: this block's output rows x the K-slice of the XCD's heads
     const uint32_t o0 = slot * a.o_rows;
@@ -216,68 +219,75 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
     const uint32_t covered = a.sdpa.n_splits * span < a.sdpa.capacity ? a.sdpa.n_splits * span : a.sdpa.capacity;
     const uint32_t kv_len = kv_len0 < 1u ? 1u : (kv_len0 > covered ? covered : kv_len0);
     const uint32_t pos = kv_len - 1, cache_row = pos % a.sdpa.capacity;
-    // ---- rotations: one wave per head of the XCD (in the last blocks, which hold no q / kv_a tile) writes the head's q
-    // with its second part rotated into the second half of `q`, and the rotated k_pe into the head's new cache row ----
-    if (slot >= kXcdSlots - a.hl && wave == 3) {
-        const uint32_t head = xcd * a.hl + (kXcdSlots - 1 - slot);
-        const uint32_t d0 = a.sdpa.q0_dim, d1 = a.sdpa.qk_dim - d0;
-        const uint16_t* qh = a.q + (size_t)head * a.sdpa.qk_dim;
-        uint16_t* qr = a.q + (size_t)a.sdpa.n_heads * a.sdpa.qk_dim + (size_t)head * a.sdpa.qk_dim;
-        split_head_transform(qh, qh + d0, qr, d0, d1, a.sdpa.rope_dims, a.sdpa.traditional != 0, pos, a.sdpa.base_log2, lane,
-                             a.sdpa.rope_tab);
-        const uint16_t* kpe = a.kva + (size_t)xcd * a.a_rows + a.rank;
-        uint16_t* krow = a.sdpa.cache_k_w + ((size_t)head * a.sdpa.capacity + cache_row) * a.sdpa.qk_dim + d0;
-        split_head_transform(kpe, kpe, krow, 0u, d1, a.sdpa.rope_dims, a.sdpa.traditional != 0, pos, a.sdpa.base_log2, lane,
-                             a.sdpa.rope_tab);
-    }
-    // ---- latent RMSNorm, kv_b rows of the XCD's heads ----
-    {
-        const uint32_t n8 = a.rank >> 3;   // at most 256 groups: one per thread
-        const uint4* l8 = reinterpret_cast<const uint4*>(a.kva + (size_t)xcd * a.a_rows);
-        const uint4* w8 = reinterpret_cast<const uint4*>(a.a_norm);
-        const bool live = tid < n8;
-        const bool wave_live = (tid & ~(kWave - 1u)) < n8;   // wave-uniform
-        uint4 v = make_uint4(0, 0, 0, 0), wv = v;
-        if (wave_live) {
-            v = ld_u128<true>(l8 + (live ? tid : 0u));
-            wv = w8[live ? tid : 0u];
-        }
-        float sq = 0.f;
-        if (live) {
-            const uint32_t xb[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float lo = bf16_lo(xb[k]), hi = bf16_hi(xb[k]);
-                sq = fmaf(lo, lo, sq);
-                sq = fmaf(hi, hi, sq);
+    if (is_rot) {
+        // ---- rotations, one wave each: unit 2 h -> the head's q with its second part rotated, into the second half of
+        // `q`; unit 2 h + 1 -> the rotated k_pe into the head's new cache row.  They run beside the other blocks' kv_b
+        // rows and meet them at the hand-over. ----
+        if (wave == 0) {
+            const uint32_t unit = kXcdSlots - 1 - slot, head = xcd * a.hl + (unit >> 1);
+            const uint32_t d0 = a.sdpa.q0_dim, d1 = a.sdpa.qk_dim - d0;
+            if ((unit & 1u) == 0) {
+                const uint16_t* qh = a.q + (size_t)head * a.sdpa.qk_dim;
+                uint16_t* qr = a.q + (size_t)a.sdpa.n_heads * a.sdpa.qk_dim + (size_t)head * a.sdpa.qk_dim;
+                split_head_transform(qh, qh + d0, qr, d0, d1, a.sdpa.rope_dims, a.sdpa.traditional != 0, pos, a.sdpa.base_log2, lane,
+                                     a.sdpa.rope_tab);
+            } else {
+                const uint16_t* kpe = a.kva + (size_t)xcd * a.a_rows + a.rank;
+                uint16_t* krow = a.sdpa.cache_k_w + ((size_t)head * a.sdpa.capacity + cache_row) * a.sdpa.qk_dim + d0;
+                split_head_transform(kpe, kpe, krow, 0u, d1, a.sdpa.rope_dims, a.sdpa.traditional != 0, pos, a.sdpa.base_log2, lane,
+                                     a.sdpa.rope_tab);
             }
         }
-        sq = wave_sum(sq);
-        if (lane == 0) red[wave] = sq;
+    } else {
+        // ---- latent RMSNorm, kv_b rows of the XCD's heads ----
+        {
+            const uint32_t n8 = a.rank >> 3;   // at most 256 groups: one per thread
+            const uint4* l8 = reinterpret_cast<const uint4*>(a.kva + (size_t)xcd * a.a_rows);
+            const uint4* w8 = reinterpret_cast<const uint4*>(a.a_norm);
+            const bool live = tid < n8;
+            const bool wave_live = (tid & ~(kWave - 1u)) < n8;   // wave-uniform
+            uint4 v = make_uint4(0, 0, 0, 0), wv = v;
+            if (wave_live) {
+                v = ld_u128<true>(l8 + (live ? tid : 0u));
+                wv = w8[live ? tid : 0u];
+            }
+            float sq = 0.f;
+            if (live) {
+                const uint32_t xb[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float lo = bf16_lo(xb[k]), hi = bf16_hi(xb[k]);
+                    sq = fmaf(lo, lo, sq);
+                    sq = fmaf(hi, hi, sq);
+                }
+            }
+            sq = wave_sum(sq);
+            if (lane == 0) red[wave] = sq;
+            __syncthreads();
+            sq = (red[0] + red[1]) + (red[2] + red[3]);
+            const float rr = 1.0f / sqrtf(sq / (float)a.rank + a.in.eps);
+            if (wave_live) stage_emit<KIND>(xs, sx, a.wb.cpr, tid, live, v, wv, rr, true);
+            __syncthreads();
+        }
+        tile_partials<KIND, NLB, kBlock>(a.wb, tb, pb, rb, xs, sx, meta + MW, work);
         __syncthreads();
-        sq = (red[0] + red[1]) + (red[2] + red[3]);
-        const float rr = 1.0f / sqrtf(sq / (float)a.rank + a.in.eps);
-        if (wave_live) stage_emit<KIND>(xs, sx, a.wb.cpr, tid, live, v, wv, rr, true);
-        __syncthreads();
-    }
-    tile_partials<KIND, NLB, kBlock>(a.wb, tb, pb, rb, xs, sx, meta + MW, work);
-    __syncthreads();
-    if (b_n) {   // [k_nope | v] of a head: into `kvb` and straight into the head's new cache rows
-        uint16_t* dst = a.kvb + (size_t)xcd * a.b_total + b0;
-        const uint32_t d0 = a.sdpa.q0_dim, packed = d0 + a.sdpa.v_dim, qkd = a.sdpa.qk_dim, vd = a.sdpa.v_dim, cap = a.sdpa.capacity;
-        uint16_t* ck = a.sdpa.cache_k_w;
-        uint16_t* cv = a.sdpa.cache_v_w;
-        const uint32_t head0 = xcd * a.hl;
-        tile_rows<false, true>(tb, work, work, [&](uint32_t r, float s0, float) {
-            const uint16_t v16 = (uint16_t)f32_to_bf16_bits(s0);
-            dst[r] = v16;
-            const uint32_t rr = b0 + r, hl_ = rr / packed, w = rr - hl_ * packed;
-            const size_t crow = (size_t)(head0 + hl_) * cap + cache_row;
-            if (w < d0)
-                ck[crow * qkd + w] = v16;
-            else
-                cv[crow * vd + (w - d0)] = v16;
-        });
+        if (b_n) {   // [k_nope | v] of a head: into `kvb` and straight into the head's new cache rows
+            uint16_t* dst = a.kvb + (size_t)xcd * a.b_total + b0;
+            const uint32_t d0 = a.sdpa.q0_dim, packed = d0 + a.sdpa.v_dim, qkd = a.sdpa.qk_dim, vd = a.sdpa.v_dim, cap = a.sdpa.capacity;
+            uint16_t* ck = a.sdpa.cache_k_w;
+            uint16_t* cv = a.sdpa.cache_v_w;
+            const uint32_t head0 = xcd * a.hl;
+            tile_rows<false, true>(tb, work, work, [&](uint32_t r, float s0, float) {
+                const uint16_t v16 = (uint16_t)f32_to_bf16_bits(s0);
+                dst[r] = v16;
+                const uint32_t rr_ = b0 + r, hl_ = rr_ / packed, w = rr_ - hl_ * packed;
+                const size_t crow = (size_t)(head0 + hl_) * cap + cache_row;
+                if (w < d0)
+                    ck[crow * qkd + w] = v16;
+                else
+                    cv[crow * vd + (w - d0)] = v16;
+            });
+        }
     }
     FK_XCD_STAMP(0, 5);
     xcd_barrier<0>(sync, okw);
@@ -394,7 +404,14 @@ MlaGeometry mla_geometry(const XcdMlaShape& s) {
     g.R = R;
     g.q_tiles = ceil_div(g.q_rows, R);
     g.a_tiles = ceil_div(g.a_rows, R);
-    g.b_rows = ceil_div(g.b_total, kXcdSlots);
+    // the last 2 hl blocks of an XCD rotate instead; a tile's quantisation groups are fetched four per lane, so its rows
+    // are rounded up to a whole number of such runs
+    g.b_rows = ceil_div(g.b_total, kXcdSlots - 2u * g.hl);
+    {
+        const uint32_t gb = s.group ? s.rank / s.group : 1u;
+        const uint32_t unit = (gb % 4u == 0) ? 1u : ((gb % 2u == 0) ? 2u : 4u);
+        g.b_rows = ceil_div(g.b_rows, unit) * unit;
+    }
     g.o_rows = ceil_div(s.hidden, kXcdSlots);
     g.o_cs = s.n_heads * s.v_dim / cv / kXcds;
     g.chunk_len = sdpa_chunk_len(g.qk_dim, s.v_dim, false);
@@ -444,7 +461,7 @@ fk_status xcd_mla_supported(const XcdMlaShape& s) {
         return set_error(FK_ERR_UNSUPPORTED, "xcd mla: a block's tile holds more chunks than the kernel requests in one pass");
     if (g.R * gq > kMetaWords || g.b_rows * gb > kMetaWords || g.o_rows * go > kMetaWords)
         return set_error(FK_ERR_UNSUPPORTED, "xcd mla: a block's tile holds more than 768 quantisation groups");
-    if (gq % 4 || (g.b_rows * gb) % 4 || (g.b_total * gb) % 4 || (g.o_rows * go) % 4 || g.b_total % g.b_rows)
+    if (gq % 4 || (g.b_rows * gb) % 4 || (g.b_total * gb) % 4 || (g.o_rows * go) % 4)
         return set_error(FK_ERR_UNSUPPORTED, "xcd mla: a block's tile must hold a multiple of four quantisation groups");
     if (g.lp_.cs_max % 4 || g.lp_.cs_max > 160u) return set_error(FK_ERR_UNSUPPORTED, "xcd mla: rows of more than 160 chunks are not served");
     if (2u * ((g.lds + 1023u) & ~1023u) > kCuLdsBytes) return set_error(FK_ERR_UNSUPPORTED, "xcd mla: two workgroups must fit the LDS of one CU");

@@ -43,8 +43,7 @@ def _normed(x, w, rows, W):
 def test_xcd_mla_block(fk, hidden, n_heads, rank, capacity, steps, traditional, two_rows):
     from fusekit_amd.runtime import Dispatch, Dispatcher, arg
     rope, nope, vd, theta = 64, 128, 128, 1e4
-    if not fk.xcd_mla_supported(hidden, n_heads, rank, rope, nope, vd, capacity, 4, 64):
-        pytest.skip("shape not supported: " + fk.lib.fk_last_error().decode())
+    assert fk.xcd_mla_supported(hidden, n_heads, rank, rope, nope, vd, capacity, 4, 64), fk.lib.fk_last_error().decode()
     d = Dispatcher()
     qk, n_a, packed = nope + rope, rank + rope, nope + vd
     n_b = n_heads * packed
