@@ -122,3 +122,24 @@ def test_two_launch_layer_admission_rules_need_no_device():
     # a tile beyond 2048 groups per matrix is refused (hidden 4096 in groups of 32: 28 rows x 128 groups)
     st = fk.lib.fk_xcd_layer_supported(u(4096), u(14336), u(32), u(8), u(128), u(1024), u(4), u(32))
     assert st == fk.FK_ERR_UNSUPPORTED and b"quantisation groups" in fk.lib.fk_last_error()
+
+
+def test_expert_and_low_rank_attention_launch_admission_rules_need_no_device():
+    """fk_xcd_moe_supported / fk_xcd_mla_supported answer the shape rules on any machine; a shape that passes them all is
+    then asked of the device."""
+    import fusekit_amd.native as fk
+    u = C.c_uint32
+    ok = fk.FK_OK if fk.has_device() else fk.FK_ERR_HIP
+    moe = lambda *a: fk.lib.fk_xcd_moe_supported(*[u(v) for v in a])
+    assert moe(2048, 1408, 2816, 64, 6, 4, 64) == ok, fk.lib.fk_last_error()
+    assert moe(2048, 1408, 2816, 64, 6, 8, 64) == fk.FK_ERR_UNSUPPORTED and b"4-bit" in fk.lib.fk_last_error()
+    assert moe(2048, 1408, 2816, 128, 6, 4, 64) == fk.FK_ERR_UNSUPPORTED and b"64 experts" in fk.lib.fk_last_error()
+    assert moe(2048, 1408, 4224, 64, 6, 4, 64) == fk.FK_ERR_UNSUPPORTED and b"at most 8" in fk.lib.fk_last_error()
+    assert moe(2048, 1400, 2800, 64, 6, 4, 64) == fk.FK_ERR_UNSUPPORTED and b"multiples of 128" in fk.lib.fk_last_error()
+    assert moe(4096, 2048, 4096, 64, 6, 4, 64) == fk.FK_ERR_UNSUPPORTED and b"chunks" in fk.lib.fk_last_error()
+    mla = lambda *a: fk.lib.fk_xcd_mla_supported(*[u(v) for v in a])
+    assert mla(2048, 16, 512, 64, 128, 128, 1024, 4, 64) == ok, fk.lib.fk_last_error()
+    assert mla(2048, 12, 512, 64, 128, 128, 1024, 4, 64) == fk.FK_ERR_UNSUPPORTED and b"heads" in fk.lib.fk_last_error()
+    assert mla(2048, 16, 512, 64, 128, 128, 1024, 8, 64) == fk.FK_ERR_UNSUPPORTED and b"4-bit" in fk.lib.fk_last_error()
+    assert mla(2048, 16, 448, 64, 128, 128, 1024, 4, 64) == fk.FK_ERR_UNSUPPORTED and b"latent" in fk.lib.fk_last_error()
+    assert fk.xcd_moe_scratch_bytes(1408) == 8 * 64 * 4 + 8 * 1408 * 2

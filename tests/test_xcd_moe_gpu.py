@@ -156,11 +156,3 @@ def _row_f32(fk, row, hidden):
     return (lo * 2.0 ** -32 + hi).astype(np.float32)
 
 
-def test_xcd_moe_admission_needs_no_device_for_the_shape_rules(fk):
-    u = fk.xcd_moe_supported
-    assert u(2048, 1408, 2816, 64, 6, 4, 64), fk.lib.fk_last_error().decode()
-    assert not u(2048, 1408, 2816, 64, 6, 8, 64) and b"4-bit" in fk.lib.fk_last_error()
-    assert not u(2048, 1408, 2816, 128, 6, 4, 64) and b"64 experts" in fk.lib.fk_last_error()
-    assert not u(2048, 1408, 4224, 64, 6, 4, 64) and b"at most 8" in fk.lib.fk_last_error()
-    assert not u(2048, 1400, 2800, 64, 6, 4, 64) and b"multiples of 128" in fk.lib.fk_last_error()
-    assert not u(4096, 2048, 4096, 64, 6, 4, 64) and b"chunks" in fk.lib.fk_last_error()
