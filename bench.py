@@ -337,6 +337,27 @@ def main() -> int:
             out["qgemv_steady"]["median_frac_of_read_ceiling"] = round(out["qgemv_steady"]["median_GBps"] / out["hbm_read_ceiling"]["GBps"], 4)
         del bufs
 
+        # ---- the mixture-of-experts benchmark model (BASELINE configs[4]: 27 layers, hidden 2048, 64 experts of 1408
+        # top-6 + 2 shared, low-rank keys 16 heads x 192 / 128, vocab 102400, int4 g64; 9 GB of weights): 32-token
+        # prompt, 512 greedy tokens at context 32..544, one hipGraph replay per token (two launches per layer) ----
+        from fusekit_amd.moe_decoder import MoeConfig, MoeRuntime, MoeWeights
+        mcfg = MoeConfig(capacity=1024)
+        mW = MoeWeights.random_init(mcfg, seed=0)
+        mrt = MoeRuntime(mcfg, mW)
+        mprompt = np.random.Generator(np.random.PCG64(0)).integers(0, mcfg.vocab, 32).tolist()
+        mrt.generate(mprompt, 9)
+        mrt.reset()
+        _, m_s, m_steps = mrt.generate(mprompt, 513)
+        m_bytes = mcfg.token_bytes(32 + 256)
+        out["moe_cfg5_decode"] = {
+            "workload": "configs[4]: 27-layer mixture-of-experts decoder, 64 experts top-6 + 2 shared, int4 g64, context 32..544",
+            "tok_per_s": round(m_steps / m_s, 1), "ms_per_token": round(m_s / m_steps * 1e3, 4), "graph_nodes": len(mrt.tasks),
+            "launches_per_expert_layer": 2 if mrt.xcd_attn else (5 if mrt.xcd else 7),
+            "bytes_per_token": m_bytes, "weight_streaming_roofline_tok_s": round(HBM_PEAK_GBPS * 1e9 / m_bytes, 1),
+            "frac_of_roofline_tok_s": round(m_steps / m_s / (HBM_PEAK_GBPS * 1e9 / m_bytes), 4),
+        }
+        del mrt, mW
+
     if args.per_kernel and args.mode == "persistent":
         per_kernel = {}
         tr = rt.d.graph_phase_trace(rt.graph)

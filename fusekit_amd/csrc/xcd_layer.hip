@@ -448,15 +448,15 @@ __global__ __launch_bounds__(kBlock) void xcd_reduce_kernel(const XcdReduceArgs 
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= a.hidden) return;
     const uint32_t at = xcd_sum_index(i);
+    // every request first (a row that is not given repeats the first: no branch between the loads)
     const unsigned long long s = (unsigned long long)a.sums[at];
+    const unsigned long long s2 = (unsigned long long)(a.sums2 ? a.sums2 : a.sums)[at];
+    const uint16_t res = a.residual[i];
     float v = xcd_sum_to_f32((uint32_t)s, (uint32_t)(s >> 32));
-    if (a.sums2) {
-        const unsigned long long s2 = (unsigned long long)a.sums2[at];
-        v = __fadd_rn(v, round_bf16(xcd_sum_to_f32((uint32_t)s2, (uint32_t)(s2 >> 32))));
-        if (a.clear2) a.clear2[at] = 0;
-    }
-    a.x[i] = (uint16_t)f32_to_bf16_bits(v + bf16_bits_to_f32(a.residual[i]));
+    if (a.sums2) v = __fadd_rn(v, round_bf16(xcd_sum_to_f32((uint32_t)s2, (uint32_t)(s2 >> 32))));
+    a.x[i] = (uint16_t)f32_to_bf16_bits(v + bf16_bits_to_f32(res));
     if (a.clear) a.clear[at] = 0;
+    if (a.clear2) a.clear2[at] = 0;
     if (a.clear3) a.clear3[at] = 0;
 }
 
