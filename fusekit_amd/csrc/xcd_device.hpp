@@ -625,6 +625,20 @@ __host__ __device__ inline uint32_t xcd_lds_bytes(const LdsPlan& p) {
            ((p.att_elems * 2u + 15u) & ~15u) + 64u;
 }
 
+// One of two matrices, chosen by a block-uniform condition.  Field by field, so that the choice stays in scalar
+// registers (a reference chosen between two members of the argument block makes the compiler copy both to private
+// memory).
+__device__ __forceinline__ XcdMat pick_mat(bool first, const XcdMat& a, const XcdMat& b) {
+    XcdMat m;
+    m.w = first ? a.w : b.w;
+    m.sc = first ? a.sc : b.sc;
+    m.bi = first ? a.bi : b.bi;
+    m.rows = first ? a.rows : b.rows;
+    m.cpr = first ? a.cpr : b.cpr;
+    m.gshift = first ? a.gshift : b.gshift;
+    return m;
+}
+
 // Workgroups are dealt to the XCDs round-robin, starting wherever the previous dispatch stopped: the XCD is read
 // from the hardware, and workgroups i and i + 8 land on the same XCD, so i / 8 numbers the 64 blocks of each XCD.
 // (Were the dealing ever different, two blocks would share a flag word, a hand-over wait would run into its spin

@@ -20,18 +20,6 @@ constexpr int kMlaNlO = 3;   // ... an o_proj tile
 
 namespace {
 
-__device__ __forceinline__ XcdMat pick_mat2(bool first, const XcdMat& a, const XcdMat& b) {
-    XcdMat m;
-    m.w = first ? a.w : b.w;
-    m.sc = first ? a.sc : b.sc;
-    m.bi = first ? a.bi : b.bi;
-    m.rows = first ? a.rows : b.rows;
-    m.cpr = first ? a.cpr : b.cpr;
-    m.gshift = first ? a.gshift : b.gshift;
-    return m;
-}
-
-
 // The second sum row of the input (the shared expert's dot products of the previous layer's expert launch): requested
 // like the first.
 struct InputRegs2 {
@@ -156,7 +144,7 @@ __global__ __launch_bounds__(kBlock, 2) void xcd_mla_kernel(const long long* sum
     const uint32_t part_rows = is_q ? a.q_rows : a.a_rows;
     const uint32_t pr0 = tl * R;
     const uint32_t pr_n = has_tile ? ((part_rows - pr0) < R ? (part_rows - pr0) : R) : 0u;
-    const XcdMat A = pick_mat2(is_q, a.wq, a.wa);
+    const XcdMat A = pick_mat(is_q, a.wq, a.wa);
     const Tile ta = make_tile((is_q ? xcd * a.q_rows : 0u) + pr0, pr_n, 0, A.cpr);
     // kv_b: the XCD's heads' rows ([k_nope | v] per head), all of the latent width
     // (the last 2 hl blocks of the XCD take no kv_b rows: they rotate q_pe / k_pe of its heads meanwhile)

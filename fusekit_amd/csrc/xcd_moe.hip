@@ -41,19 +41,6 @@ __device__ __forceinline__ float dot8_bf16(uint4 w, uint4 x, float acc) {
     return acc;
 }
 
-// Field by field, so that the choice stays in scalar registers (a reference chosen between two members of the argument
-// block makes the compiler copy both to private memory).
-__device__ __forceinline__ XcdMat pick_mat(bool first, const XcdMat& a, const XcdMat& b) {
-    XcdMat m;
-    m.w = first ? a.w : b.w;
-    m.sc = first ? a.sc : b.sc;
-    m.bi = first ? a.bi : b.bi;
-    m.rows = first ? a.rows : b.rows;
-    m.cpr = first ? a.cpr : b.cpr;
-    m.gshift = first ? a.gshift : b.gshift;
-    return m;
-}
-
 // Scales and biases of a tile that may be a K-slice of the matrix's rows (MLX layout: [row][groups of the row]), one
 // group per lane and request: group gi of the tile = (row gi / gpr, group gi % gpr of the slice).
 template <WKind KIND, int SN, typename MAT>
