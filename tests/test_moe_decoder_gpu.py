@@ -330,3 +330,28 @@ def test_checkpoint_round_trip(fk, tmp_path):
     json.dump(conf, open(tmp_path / "config.json", "w"))
     with pytest.raises(ValueError, match="switch_mlp"):
         load_moe_checkpoint(str(tmp_path))
+
+
+def test_two_launch_layer_wait_gives_up_and_reports(fk):
+    """A hand-over wait of the attention or the expert launch that exceeds its spin limit (forced from the host: one poll)
+    must not hang: every block drains, the error is reported, the control block and the graph's six sum rows are reset,
+    and the same model decodes the oracle's tokens afterwards with the default limit."""
+    from fusekit_amd.moe_decoder import MoeRuntime, MoeWeights
+    kw = dict(hidden=512, n_heads=8, n_experts=16, top_k=6, n_shared=2, xcd_moe=True)
+    cfg = _small_cfg(xcd_spin_limit=1, **kw)
+    W = MoeWeights.random_init(cfg, seed=3)
+    rt = MoeRuntime(cfg, W)
+    assert rt.xcd and rt.xcd_attn and len(rt.xcd_sums) == 6
+    with pytest.raises(fk.FusekitError) as e:
+        for _ in range(50):          # one poll may well succeed now and then: the limit has to bite within a few launches
+            rt.d.decode_host_loop(rt.graph, rt.uniforms, 0, [5])
+    assert "spin limit" in str(e.value)
+    assert not rt.xcd_ctl.to_numpy(np.uint32).any()
+    assert not any(row.to_numpy(np.int64).any() for row in rt.xcd_sums)
+    del rt
+    cfg = _small_cfg(**kw)
+    rt, od = MoeRuntime(cfg, W), OracleMoeDecoder(cfg, W)
+    prompt = rng(2).integers(0, cfg.vocab, 5).tolist()
+    got, _, _ = rt.generate(prompt, 10)
+    ref, _ = od.generate(prompt, 10)
+    assert got == ref
