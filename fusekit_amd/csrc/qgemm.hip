@@ -67,6 +67,10 @@ struct QgemmArgs {
     uint32_t group;        // 64 or 128
     uint32_t k_per_split;  // multiple of group
     uint32_t n_blocks;     // blocks along N
+    // the tile form with one k split writes finished outputs (null: partial sums as above)
+    uint16_t* y;
+    const uint16_t* bias;
+    const uint16_t* res;
 };
 
 template <WKind KIND, int MT>
@@ -271,6 +275,186 @@ __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
     }
 }
 
+// ---- the tile form: from 256 activation rows ---------------------------------------------------------------------
+// A block of EIGHT waves owns 256 activation rows x 128 weight rows and walks k in slabs of 64.  Both operands of a slab
+// are staged in LDS once per block -- the activations as they lie, the weights dequantised to bf16 (w = T(s q + b), the
+// arithmetic of the form above) by the one thread that loaded their 16 codes -- and every wave multiplies a 64 x 64
+// part of the tile from there (four accumulators, 4 fragment reads per 4 matrix instructions).  Two waves share a SIMD:
+// while one unpacks, stages or waits, the other one's matrix instructions keep the pipe busy (one wave per SIMD with
+// everything interleaved by hand ran its phases one after the other: 65 us for 512 x 9728 x 2560, of which the matrix
+// instructions alone are 21).  Two LDS buffers; a slab is requested two passes before it is staged (parked in named
+// registers, one set for even and one for odd slabs), one barrier per slab.  Staged rows are 9 pieces of 16 bytes
+// apart (8 used), which spreads the fragment reads of 8 neighbouring lanes over all banks.
+// With one k split the block finishes its outputs itself (bias, residual, one rounding: the arithmetic of the second
+// kernel below for one split); otherwise partial sums go out in the layout of the form above.
+constexpr int kTileBlock = 512;
+constexpr uint32_t kTileM = 256, kTileN = 128, kTileK = 64;
+constexpr uint32_t kTileStride = kTileK / 8 + 1;                            // uint4 per staged row
+constexpr uint32_t kTileBufPieces = (kTileM + kTileN) * kTileStride;        // one buffer: x rows, then weight rows
+constexpr uint32_t kTileLdsBytes = 2u * kTileBufPieces * 16u;
+
+// Piece p (codes 8 p .. 8 p + 7, element order) of the 16 codes one thread loaded (int4: w.x, w.y; int8: all of w) as
+// eight bf16 weights T(s q + b).
+template <WKind KIND>
+__device__ __forceinline__ uint4 tile_unpack_piece(int p, const uint4 w, float sf, float bf) {
+    uint4 bw;
+    if constexpr (KIND == W_Q4) {
+        const uint32_t word = p ? w.y : w.x;
+        const uint32_t lo = word & 0x0F0F0F0Fu, hi = (word >> 4) & 0x0F0F0F0Fu;
+        bw.x = pack_bf16(fmaf((float)(lo & 0xffu), sf, bf), fmaf((float)(hi & 0xffu), sf, bf));
+        bw.y = pack_bf16(fmaf((float)((lo >> 8) & 0xffu), sf, bf), fmaf((float)((hi >> 8) & 0xffu), sf, bf));
+        bw.z = pack_bf16(fmaf((float)((lo >> 16) & 0xffu), sf, bf), fmaf((float)((hi >> 16) & 0xffu), sf, bf));
+        bw.w = pack_bf16(fmaf((float)(lo >> 24), sf, bf), fmaf((float)(hi >> 24), sf, bf));
+    } else {
+        const uint32_t lo = p ? w.z : w.x, hi = p ? w.w : w.y;
+        bw.x = pack_bf16(fmaf((float)(lo & 0xffu), sf, bf), fmaf((float)((lo >> 8) & 0xffu), sf, bf));
+        bw.y = pack_bf16(fmaf((float)((lo >> 16) & 0xffu), sf, bf), fmaf((float)(lo >> 24), sf, bf));
+        bw.z = pack_bf16(fmaf((float)(hi & 0xffu), sf, bf), fmaf((float)((hi >> 8) & 0xffu), sf, bf));
+        bw.w = pack_bf16(fmaf((float)((hi >> 16) & 0xffu), sf, bf), fmaf((float)(hi >> 24), sf, bf));
+    }
+    return bw;
+}
+
+template <WKind KIND>
+__global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs a) {
+    extern __shared__ uint4 lds_raw[];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, kb = lane >> 5, nl = lane & 31u;
+    const uint32_t wm = wave >> 1, wn = wave & 1u;   // the wave's 64 x 64 part: rows 64 wm, weight rows 64 wn
+    const uint32_t nb = blockIdx.x % a.n_blocks, ks = blockIdx.x / a.n_blocks;
+    const uint32_t m0 = blockIdx.y * kTileM, n0 = nb * kTileN;
+    const uint32_t k0 = ks * a.k_per_split;
+    const uint32_t k1 = k0 + a.k_per_split < a.K ? k0 + a.k_per_split : a.K;
+    const uint32_t gshift = a.group == 128 ? 7u : 6u;
+    const uint32_t slabs = (k1 - k0) / kTileK;
+
+    // staging roles: x pieces (row tid / 8 + 64 i, piece tid % 8), i < 4; 16 codes of weight row tid / 4, quarter
+    // tid % 4 of the slab (8 bytes of int4, 16 of int8)
+    const uint32_t xr = tid >> 3, xp = tid & 7u;
+    const uint32_t wr = tid >> 2, wq = tid & 3u;
+    const uint32_t wrow = n0 + wr < a.N ? n0 + wr : a.N - 1;   // rows past the end read the last row; never stored
+    const unsigned char* wsrc = reinterpret_cast<const unsigned char*>(a.w + (size_t)wrow * a.cpr) + wq * (KIND == W_Q4 ? 8u : 16u);
+    const uint16_t* srow = a.sc + (size_t)wrow * a.gpr;
+    const uint16_t* brow = a.bi + (size_t)wrow * a.gpr;
+    const uint16_t* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t m = m0 + xr + 64u * (uint32_t)i;
+        xsrc[i] = a.x + (size_t)(m < a.M ? m : a.M - 1) * a.K + xp * 8u;
+    }
+
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // (Macros over named registers, not lambdas over a struct or arrays: an object whose address a closure holds, or an
+    // array, stays in scratch once a fence stands between its writes and its reads.)
+#define FK_TILE_DECLARE(S) uint4 S##x0, S##x1, S##x2, S##x3, S##w; uint16_t S##sc, S##bi
+#define FK_TILE_REQUEST(S, slab)                                                                                      \
+    {                                                                                                                 \
+        const uint32_t kf = k0 + ((slab) < slabs ? (slab) : 0u) * kTileK; /* past the end: the first slab (unused) */ \
+        S##x0 = *reinterpret_cast<const uint4*>(xsrc[0] + kf);                                                        \
+        S##x1 = *reinterpret_cast<const uint4*>(xsrc[1] + kf);                                                        \
+        S##x2 = *reinterpret_cast<const uint4*>(xsrc[2] + kf);                                                        \
+        S##x3 = *reinterpret_cast<const uint4*>(xsrc[3] + kf);                                                        \
+        if constexpr (KIND == W_Q4) {                                                                                 \
+            const uint2 v = *reinterpret_cast<const uint2*>(wsrc + (kf >> 1));                                        \
+            S##w = make_uint4(v.x, v.y, 0u, 0u);                                                                      \
+        } else {                                                                                                      \
+            S##w = *reinterpret_cast<const uint4*>(wsrc + kf);                                                        \
+        }                                                                                                             \
+        const uint32_t g = kf >> gshift;                                                                              \
+        S##sc = srow[g]; /* kept apart: combining the two here would wait for both loads on the spot */              \
+        S##bi = brow[g];                                                                                              \
+        /* keeps the requests where they are written: left alone, the compiler moves them down to their first use */  \
+        asm volatile("" ::: "memory");                                                                                \
+    }
+#define FK_TILE_STAGE(S, to)                                                                                          \
+    {                                                                                                                 \
+        uint4* xs_w = lds_raw + (to) * kTileBufPieces;                                                                \
+        uint4* xd = xs_w + xr * kTileStride + xp;                                                                     \
+        xd[0 * 64 * kTileStride] = S##x0; xd[1 * 64 * kTileStride] = S##x1;                                           \
+        xd[2 * 64 * kTileStride] = S##x2; xd[3 * 64 * kTileStride] = S##x3;                                           \
+        const float sf = bf16_bits_to_f32(S##sc), bf = bf16_bits_to_f32(S##bi);                                       \
+        uint4* wd = xs_w + kTileM * kTileStride + wr * kTileStride + wq * 2u;                                         \
+        wd[0] = tile_unpack_piece<KIND>(0, S##w, sf, bf);                                                             \
+        wd[1] = tile_unpack_piece<KIND>(1, S##w, sf, bf);                                                             \
+    }
+    auto multiply = [&](uint32_t from) {
+        const uint4* xs = lds_raw + from * kTileBufPieces;
+        const uint4* xa = xs + (wm * 64u + nl) * kTileStride + kb;
+        const uint4* wb = xs + (kTileM + wn * 64u + nl) * kTileStride + kb;
+#pragma unroll
+        for (int st = 0; st < (int)kTileK / 16; ++st) {
+            uint4 af[2], bfr[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = xa[(uint32_t)i * 32u * kTileStride + 2u * (uint32_t)st];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bfr[j] = wb[(uint32_t)j * 32u * kTileStride + 2u * (uint32_t)st];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
+                                                                        __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
+        }
+    };
+    FK_TILE_DECLARE(e_);
+    FK_TILE_DECLARE(o_);
+    // slab s parks in the set of its parity; pass q stages slab q, requests slab q + 2 into the set it has just emptied
+    // and multiplies slab q - 1
+    FK_TILE_REQUEST(e_, 0u);
+    FK_TILE_REQUEST(o_, 1u);
+    FK_TILE_STAGE(e_, 0u);
+    FK_TILE_REQUEST(e_, 2u);
+    __syncthreads();
+    uint32_t buf = 0;   // a pass multiplies from `buf` and stages into the other one
+    uint32_t q = 1;
+    for (; q + 1 <= slabs; q += 2) {
+        FK_TILE_STAGE(o_, buf ^ 1u);
+        FK_TILE_REQUEST(o_, q + 2u);
+        multiply(buf);
+        __syncthreads();
+        buf ^= 1u;
+        FK_TILE_STAGE(e_, buf ^ 1u);
+        FK_TILE_REQUEST(e_, q + 3u);
+        multiply(buf);
+        __syncthreads();
+        buf ^= 1u;
+    }
+    if (q <= slabs) multiply(buf);   // the last slab of an odd count
+#undef FK_TILE_DECLARE
+#undef FK_TILE_REQUEST
+#undef FK_TILE_STAGE
+
+    // register r of a lane is activation row (r % 4) + 8 (r / 4) + 4 kb of its 32 x 32 tile, column nl
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t n = n0 + wn * 64u + (uint32_t)j * 32u + nl;
+        if (n >= a.N) continue;
+        const float bias = (a.y && a.bias) ? bf16_bits_to_f32(a.bias[n]) : 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t m = m0 + wm * 64u + (uint32_t)(i * 32 + r % 4 + 8 * (r / 4)) + 4u * kb;
+                if (m >= a.M) continue;
+                if (a.y) {   // one k split: finished here, in the order of additions of the second kernel
+                    float v = acc[i][j][r];
+                    if (a.bias) v += bias;
+                    if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * a.N + n]);
+                    a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
+                } else {
+                    a.partial[((size_t)ks * a.M + m) * a.N + n] = acc[i][j][r];
+                }
+            }
+    }
+}
+
 struct QgemmReduceArgs {
     const float* p0;  // [ksplit, M, N]
     const float* p1;  // second matrix (up projection) for the SwiGLU pair, or null
@@ -331,6 +515,8 @@ __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const QgemmReduceArgs
 
 namespace {
 
+uint32_t qgemm_form_lds_bytes(int mt) { return mt == 8 ? kTileLdsBytes : qgemm_lds_bytes(mt); }
+
 struct QgemmShape {
     uint32_t n_blocks, m_tiles, ksplit, k_per_split;
     int mt;  // tiles of 32 activation rows per block
@@ -339,6 +525,7 @@ struct QgemmShape {
 const void* qgemm_func(uint32_t bits, int mt) {
     const bool q4 = bits == 4;
     switch (mt) {
+        case 8: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8>);
         case 1: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 1>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 1>);
         case 2: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 2>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 2>);
         default: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 4>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 4>);
@@ -348,15 +535,16 @@ const void* qgemm_func(uint32_t bits, int mt) {
 // Blocks of this kernel form that are resident at once (registers and LDS decide).
 uint32_t qgemm_resident(const DeviceFacts* dev, uint32_t bits, int mt) {
     static std::mutex mu;
-    static int cache[2][5] = {{0, 0, 0, 0, 0}, {0, 0, 0, 0, 0}};
+    static int cache[2][9] = {};
     std::lock_guard<std::mutex> lk(mu);
     int& slot = cache[bits == 4 ? 0 : 1][mt];
     if (slot == 0) {
         const void* f = qgemm_func(bits, mt);
-        const uint32_t lds = qgemm_lds_bytes(mt);
+        const uint32_t lds = qgemm_form_lds_bytes(mt);
         if (lds > 48 * 1024) (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, f, kQgemmBlock, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, f, mt == 8 ? kTileBlock : kQgemmBlock, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+        if (mt == 8) per_cu = 1;         // the tile form: one block (two LDS buffers, 128 accumulator registers per lane) per CU
         slot = per_cu > 2 ? 2 : per_cu;  // more than two blocks per CU gain nothing here (512 rows: 66.4 us with 2, 65.9 with 4)
     }
     return (uint32_t)slot * (uint32_t)dev->cus;
@@ -370,8 +558,9 @@ fk_status qgemm_shape(const DeviceFacts* dev, uint32_t M, uint32_t N, uint32_t K
     if ((uint64_t)M * N > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "qgemm: output too large");
     QgemmShape s;
     s.n_blocks = (N + kQgemmRows - 1) / kQgemmRows;
-    s.mt = M > 64 ? 4 : (M > 32 ? 2 : 1);
+    s.mt = M >= kTileM ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));   // 8: the tile form
     s.m_tiles = (M + kQgemmMTile * s.mt - 1) / (kQgemmMTile * s.mt);
+    if (s.mt == 8) s.n_blocks = (N + kTileN - 1) / kTileN;
     // Split k until the grid fills what is resident at once, never beyond (a block that waits
     // for a slot doubles the run time), and keep at least 256 k per block.  Every split writes
     // and re-reads an fp32 copy of the output.
@@ -396,9 +585,17 @@ fk_status check_weight(const fk_weight* W, const char* who) {
     return FK_OK;
 }
 
+// `direct` (optional): where a launch that needs no second kernel -- the tile form with one k split -- writes its
+// finished outputs; *finished then says whether it does.
+struct QgemmDirect {
+    uint16_t* y;
+    const uint16_t* bias;
+    const uint16_t* res;
+};
 fk_status plan_qgemm_main(const DeviceFacts* dev, const fk_weight* W, const uint16_t* x, uint32_t M, float* partial,
-                          QgemmShape* shape, Launch* out) {
+                          QgemmShape* shape, Launch* out, const QgemmDirect* direct = nullptr, bool* finished = nullptr) {
     FK_TRY(qgemm_shape(dev, M, W->n, W->k, W->group, W->bits, shape));
+    if (finished) *finished = false;
     QgemmArgs a;
     memset(&a, 0, sizeof(a));
     a.w = reinterpret_cast<const uint4*>(W->w);
@@ -414,10 +611,16 @@ fk_status plan_qgemm_main(const DeviceFacts* dev, const fk_weight* W, const uint
     a.group = W->group;
     a.k_per_split = shape->k_per_split;
     a.n_blocks = shape->n_blocks;
+    if (direct && shape->mt == 8 && shape->ksplit == 1) {
+        a.y = direct->y;
+        a.bias = direct->bias;
+        a.res = direct->res;
+        if (finished) *finished = true;
+    }
     out->func = qgemm_func(W->bits, shape->mt);
     out->grid = dim3(shape->n_blocks * shape->ksplit, shape->m_tiles, 1);
-    out->block = dim3(kQgemmBlock, 1, 1);
-    out->shmem = qgemm_lds_bytes(shape->mt);
+    out->block = dim3(shape->mt == 8 ? kTileBlock : kQgemmBlock, 1, 1);
+    out->shmem = qgemm_form_lds_bytes(shape->mt);
     out->set_args(a);
     if (out->shmem > 48 * 1024)
         FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)out->shmem));
@@ -477,8 +680,13 @@ fk_status plan_qgemm(const fk_weight* W, const uint16_t* x, uint32_t M, const ui
         return plan_qgemm_wide(W, nullptr, x, M, bias, res, 0, y, main);
     }
     QgemmShape s;
-    FK_TRY(plan_qgemm_main(dev, W, x, M, static_cast<float*>(workspace), &s, main));
-    plan_reduce(static_cast<float*>(workspace), nullptr, bias, res, y, M, W->n, s.ksplit, 0, reduce);
+    const QgemmDirect direct{y, bias, res};
+    bool finished = false;
+    FK_TRY(plan_qgemm_main(dev, W, x, M, static_cast<float*>(workspace), &s, main, &direct, &finished));
+    if (finished)
+        *reduce = Launch();   // the tile form with one k split rounds its outputs itself
+    else
+        plan_reduce(static_cast<float*>(workspace), nullptr, bias, res, y, M, W->n, s.ksplit, 0, reduce);
     return FK_OK;
 }
 
