@@ -24,6 +24,9 @@ Prints ONE JSON line: value = generated tokens/s (wall clock around the K timed 
                   launch, three sets in rotation): the steady streaming rate of the int4 qGEMV,
   hbm_read_ceiling -- a plain read-and-XOR kernel over 1 GiB buffers: what a read-only kernel gets from
                   HBM on this device, the bound the GEMV figures are also stated against,
+  qgemm_rows   -- the multi-row matmul of the prompt path (9728 x 2560 int4 as a graph node, 512 and 2048
+                  activation rows): TFLOP/s and fraction of the dense bf16 MFMA peak,
+  moe_cfg5_decode -- configs[4]'s mixture-of-experts decoder: tokens/s of its decode loop,
   cpu_baseline -- the CPU oracle (C restatement of the reference semantics) decoding the same
                   model at the same context on the host cores, bounded to --cpu-tokens steps.
 """
@@ -336,6 +339,16 @@ def main() -> int:
         if "qgemv_steady" in out:
             out["qgemv_steady"]["median_frac_of_read_ceiling"] = round(out["qgemv_steady"]["median_GBps"] / out["hbm_read_ceiling"]["GBps"], 4)
         del bufs
+
+        # ---- the multi-row matmul on the matrix cores (the prompt path's projection: 9728 x 2560 int4 g64 as a graph
+        # node, 512 and 2048 activation rows), against the dense bf16 MFMA peak ----
+        from fusekit_amd.kernel_bench import measure_qgemm
+        out["qgemm_rows"] = {}
+        for rows in (512, 2048):
+            q_s, _, q_flops, _ = measure_qgemm(rt.d, 20, rows)
+            out["qgemm_rows"][str(rows)] = {"us_per_call": round(q_s * 1e6, 2), "TFLOPs": round(q_flops / q_s / 1e12, 1),
+                                            "frac_of_mfma_bf16_peak": round(q_flops / q_s / 2.5e15, 4)}
+        out["qgemm_rows"]["workload"] = "family fusekit_qgemm, 9728 x 2560 int4 g64, 512 / 2048 activation rows, peak 2.5 PFLOP/s"
 
         # ---- the mixture-of-experts benchmark model (BASELINE configs[4]: 27 layers, hidden 2048, 64 experts of 1408
         # top-6 + 2 shared, low-rank keys 16 heads x 192 / 128, vocab 102400, int4 g64; 9 GB of weights): 32-token

@@ -216,7 +216,9 @@ def case_moe(d, reps, bits=4, tokens=1):
         _emit(f"routed_qmv_reduce_{tag}_expert_order", _time_graph(d, o2, reps), b2, routes=routes, experts=E)
 
 
-def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
+def measure_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
+    """Seconds per call of the family fusekit_qgemm on `rows` activation rows (a serialised graph over a pool of
+    matrices larger than the last-level cache), the algorithmic bytes and flops of one call, the pool size."""
     per = bits / 8 + 4 / 64
     pool = max(2, int(600e6 // (n * k * per)) + 1)
     x = _bf16(rows * k, 1)
@@ -228,8 +230,14 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
         tasks.append(Dispatch("fusekit_qgemm_f0", [arg(x)] + _wargs(W) + [arg(y), arg(ws)],
                               {"bits": bits, "group": 64, "m": k, "n": n, "rows": rows}))
     nbytes = n * k * per + rows * k * 2 + rows * n * 2
-    _emit(f"qgemm_rows{rows}_{n}x{k}_q{bits}", _time_graph(d, tasks, reps), nbytes, flops=2.0 * rows * n * k, pool=pool,
-          note="2..10 rows: one shared-stream launch; more rows: MFMA main + split-k reduction")
+    return _time_graph(d, tasks, reps), nbytes, 2.0 * rows * n * k, pool
+
+
+def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
+    sec, nbytes, flops, pool = measure_qgemm(d, reps, rows, n, k, bits)
+    _emit(f"qgemm_rows{rows}_{n}x{k}_q{bits}", sec, nbytes, flops=flops, pool=pool,
+          note="2..10 rows: one shared-stream launch; 11..255 rows: MFMA main + split-k reduction; from 256 rows the "
+               "LDS-tiled form (finished outputs at one k split)")
 
 
 def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_bits=0, keep=False):
@@ -356,6 +364,7 @@ CASES = {
     "qgemm_32": lambda d, r: case_qgemm(d, r, 32),
     "qgemm_128": lambda d, r: case_qgemm(d, r, 128),
     "qgemm_512": lambda d, r: case_qgemm(d, r, 512),
+    "qgemm_2048": lambda d, r: case_qgemm(d, r, 2048),
     "prefill_4b_32": lambda d, r: case_prefill(d, r, 512, 32),
     "prefill_4b": lambda d, r: case_prefill(d, r),
     "prefill_4b_128": lambda d, r: case_prefill(d, r, 512, 128),
