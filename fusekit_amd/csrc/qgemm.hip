@@ -333,14 +333,20 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
     const uint32_t xr = tid >> 3, xp = tid & 7u;
     const uint32_t wr = tid >> 2, wq = tid & 3u;
     const uint32_t wrow = n0 + wr < a.N ? n0 + wr : a.N - 1;   // rows past the end read the last row; never stored
-    const unsigned char* wsrc = reinterpret_cast<const unsigned char*>(a.w + (size_t)wrow * a.cpr) + wq * (KIND == W_Q4 ? 8u : 16u);
-    const uint16_t* srow = a.sc + (size_t)wrow * a.gpr;
-    const uint16_t* brow = a.bi + (size_t)wrow * a.gpr;
-    const uint16_t* xsrc[4];
+    // Every request is a block-uniform base (scalar registers, advanced by the slab) plus a per-lane 32-bit byte offset
+    // that never changes: no vector address arithmetic per slab (the planner admits the form only while the operands
+    // stay under 4 GB).
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.w);
+    const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
+    const unsigned char* sbase = reinterpret_cast<const unsigned char*>(a.sc);
+    const unsigned char* bbase = reinterpret_cast<const unsigned char*>(a.bi);
+    const uint32_t woff = wrow * a.cpr * 16u + wq * (KIND == W_Q4 ? 8u : 16u);
+    const uint32_t soff = wrow * a.gpr * 2u;
+    uint32_t xoff[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t m = m0 + xr + 64u * (uint32_t)i;
-        xsrc[i] = a.x + (size_t)(m < a.M ? m : a.M - 1) * a.K + xp * 8u;
+        xoff[i] = (m < a.M ? m : a.M - 1) * a.K * 2u + xp * 16u;
     }
 
     f32x16_t acc[2][2];
@@ -357,19 +363,20 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
 #define FK_TILE_REQUEST(S, slab)                                                                                      \
     {                                                                                                                 \
         const uint32_t kf = k0 + ((slab) < slabs ? (slab) : 0u) * kTileK; /* past the end: the first slab (unused) */ \
-        S##x0 = *reinterpret_cast<const uint4*>(xsrc[0] + kf);                                                        \
-        S##x1 = *reinterpret_cast<const uint4*>(xsrc[1] + kf);                                                        \
-        S##x2 = *reinterpret_cast<const uint4*>(xsrc[2] + kf);                                                        \
-        S##x3 = *reinterpret_cast<const uint4*>(xsrc[3] + kf);                                                        \
+        const unsigned char* xk = xbase + (size_t)kf * 2u;                                                           \
+        S##x0 = *reinterpret_cast<const uint4*>(xk + xoff[0]);                                                        \
+        S##x1 = *reinterpret_cast<const uint4*>(xk + xoff[1]);                                                        \
+        S##x2 = *reinterpret_cast<const uint4*>(xk + xoff[2]);                                                        \
+        S##x3 = *reinterpret_cast<const uint4*>(xk + xoff[3]);                                                        \
         if constexpr (KIND == W_Q4) {                                                                                 \
-            const uint2 v = *reinterpret_cast<const uint2*>(wsrc + (kf >> 1));                                        \
+            const uint2 v = *reinterpret_cast<const uint2*>(wbase + (kf >> 1) + woff);                                \
             S##w = make_uint4(v.x, v.y, 0u, 0u);                                                                      \
         } else {                                                                                                      \
-            S##w = *reinterpret_cast<const uint4*>(wsrc + kf);                                                        \
+            S##w = *reinterpret_cast<const uint4*>(wbase + kf + woff);                                                \
         }                                                                                                             \
         const uint32_t g = kf >> gshift;                                                                              \
-        S##sc = srow[g]; /* kept apart: combining the two here would wait for both loads on the spot */              \
-        S##bi = brow[g];                                                                                              \
+        S##sc = *reinterpret_cast<const uint16_t*>(sbase + g * 2u + soff); /* kept apart: combining the two here */   \
+        S##bi = *reinterpret_cast<const uint16_t*>(bbase + g * 2u + soff); /* would wait for both loads on the spot */ \
         /* keeps the requests where they are written: left alone, the compiler moves them down to their first use */  \
         asm volatile("" ::: "memory");                                                                                \
     }
@@ -379,7 +386,11 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         uint4* xd = xs_w + xr * kTileStride + xp;                                                                     \
         xd[0 * 64 * kTileStride] = S##x0; xd[1 * 64 * kTileStride] = S##x1;                                           \
         xd[2 * 64 * kTileStride] = S##x2; xd[3 * 64 * kTileStride] = S##x3;                                           \
-        const float sf = bf16_bits_to_f32(S##sc), bf = bf16_bits_to_f32(S##bi);                                       \
+        /* pinned here: left alone, the compiler widens the two values where they are loaded, a pass earlier, and   \
+           waits there for every request in flight */                                                                 \
+        uint32_t sc_bits = S##sc, bi_bits = S##bi;                                                                    \
+        asm volatile("" : "+v"(sc_bits), "+v"(bi_bits));                                                              \
+        const float sf = bf16_bits_to_f32(sc_bits), bf = bf16_bits_to_f32(bi_bits);                                   \
         uint4* wd = xs_w + kTileM * kTileStride + wr * kTileStride + wq * 2u;                                         \
         wd[0] = tile_unpack_piece<KIND>(0, S##w, sf, bf);                                                             \
         wd[1] = tile_unpack_piece<KIND>(1, S##w, sf, bf);                                                             \
@@ -558,7 +569,9 @@ fk_status qgemm_shape(const DeviceFacts* dev, uint32_t M, uint32_t N, uint32_t K
     if ((uint64_t)M * N > 0x7fffffffull) return set_error(FK_ERR_UNSUPPORTED, "qgemm: output too large");
     QgemmShape s;
     s.n_blocks = (N + kQgemmRows - 1) / kQgemmRows;
-    s.mt = M >= kTileM ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));   // 8: the tile form
+    // 8: the tile form (its requests are 32-bit byte offsets from a uniform base: operands under 4 GB)
+    const bool tile_ok = M >= kTileM && (uint64_t)M * K * 2 < (1ull << 32) && (uint64_t)N * K < (1ull << 32);
+    s.mt = tile_ok ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));
     s.m_tiles = (M + kQgemmMTile * s.mt - 1) / (kQgemmMTile * s.mt);
     if (s.mt == 8) s.n_blocks = (N + kTileN - 1) / kTileN;
     // Split k until the grid fills what is resident at once, never beyond (a block that waits
