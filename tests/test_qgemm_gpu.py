@@ -225,6 +225,42 @@ def test_qgemm_many_rows_both_routes(fk, m, n, k, bits, group, route):
         fk.set_gemm_library_rows(256)
 
 
+@pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 128)])
+def test_qgemm_tile_form_finishes_its_outputs_at_one_k_split(fk, bits, group):
+    """From 256 rows the fused kernel stages both operands of a 256 x 128 tile in LDS; with enough tiles to fill the
+    device it takes ONE k split and adds bias and residual and rounds in the same launch (no fp32 partial sums, no
+    second kernel).  Ragged in both directions: 520 rows (a third row tile with 8 live rows), 9700 weight rows."""
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    m, n, k = 520, 9700, 256
+    W = make_qweight(80 + bits, n, k, bits, group=group)
+    x = normal_bf16(81, (m, k))
+    bias, res = normal_bf16(82, n), normal_bf16(83, (m, n))
+    dW, bx, bb, br = to_device(fk, W), _dev(fk, x), _dev(fk, bias), _dev(fk, res)
+    y, ws = fk.DeviceBuffer(2 * m * n), fk.DeviceBuffer(fk.qgemm_workspace_bytes(m, n, k, group))
+    d = Dispatcher()
+    params = {"bits": bits, "group": group, "m": k, "n": n, "rows": m}
+    plain = Dispatch("fusekit_qgemm_f0", [arg(bx), arg(dW.w), arg(dW.scales), arg(dW.biases), arg(y), arg(ws)], params)
+    geo = d.plan_geometry(plain)
+    assert geo.n_kernels == 1 and tuple(geo.threadgroup[0]) == (512, 1, 1) and tuple(geo.grid[0]) == (76, 3, 1)
+    y.upload(np.full(m * n, 0x7fc0, np.uint16))
+    d.dispatch_kernel(plain)
+    fk.sync()
+    got = y.to_numpy(np.uint16, (m, n))
+    ref, acc = _reference(W, x)
+    rows = list(range(0, m, 37)) + [255, 256, 511, 512, 519]
+    for r in rows:
+        _check(got[r], ref[r], acc[r], W, x[r])
+    full_d = Dispatch("fusekit_qgemm_f0", [arg(bx), arg(dW.w), arg(dW.scales), arg(dW.biases), arg(bb), arg(br), arg(y), arg(ws)],
+                      dict(params, has_bias=1, has_residual=1))
+    d.dispatch_kernel(full_d)
+    fk.sync()
+    got = y.to_numpy(np.uint16, (m, n))
+    full = acc + oracle.bf16_to_f32(bias)[None, :] + oracle.bf16_to_f32(res)
+    want = oracle.f32_to_bf16(full.astype(np.float32))
+    for r in rows:
+        _check(got[r], want[r], full[r], W, x[r])
+
+
 @pytest.mark.parametrize("route,m", [("kernel", 512), ("library", 512), ("library", 2048)])
 def test_qgemm_swiglu_many_rows_both_routes(fk, route, m):
     """From 2048 rows the library route lets the GEMM round gate and up to bf16 itself and runs SwiGLU over bf16."""
