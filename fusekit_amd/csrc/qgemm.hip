@@ -71,6 +71,12 @@ struct QgemmArgs {
     uint16_t* y;
     const uint16_t* bias;
     const uint16_t* res;
+    // the tile form for a gate / up pair: the second matrix (same shape), its partial sums, the SwiGLU variant
+    const uint4* w2;
+    const uint16_t* sc2;
+    const uint16_t* bi2;
+    float* partial2;
+    int variant;
 };
 
 template <WKind KIND, int MT>
@@ -290,8 +296,9 @@ __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
 constexpr int kTileBlock = 512;
 constexpr uint32_t kTileM = 256, kTileN = 128, kTileK = 64;
 constexpr uint32_t kTileStride = kTileK / 8 + 1;                            // uint4 per staged row
-constexpr uint32_t kTileBufPieces = (kTileM + kTileN) * kTileStride;        // one buffer: x rows, then weight rows
-constexpr uint32_t kTileLdsBytes = 2u * kTileBufPieces * 16u;
+// one buffer: x rows, then weight rows (a gate / up pair: the up rows behind the gate rows)
+constexpr uint32_t tile_buf_pieces(bool pair) { return (kTileM + (pair ? 2u : 1u) * kTileN) * kTileStride; }
+constexpr uint32_t tile_lds_bytes(bool pair) { return 2u * tile_buf_pieces(pair) * 16u; }
 
 // Piece p (codes 8 p .. 8 p + 7, element order) of the 16 codes one thread loaded (int4: w.x, w.y; int8: all of w) as
 // eight bf16 weights T(s q + b).
@@ -315,9 +322,13 @@ __device__ __forceinline__ uint4 tile_unpack_piece(int p, const uint4 w, float s
     return bw;
 }
 
-template <WKind KIND>
+// PAIR: a gate / up pair of the same shape in one launch -- the activations are requested and staged once for both,
+// every wave keeps a second set of accumulators, and with one k split SwiGLU is applied to the finished sums here
+// (swiglu_bits, as the second kernel applies it to the sums of one split).
+template <WKind KIND, bool PAIR>
 __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs a) {
     extern __shared__ uint4 lds_raw[];
+    constexpr uint32_t kTileBufPieces = tile_buf_pieces(PAIR);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, kb = lane >> 5, nl = lane & 31u;
     const uint32_t wm = wave >> 1, wn = wave & 1u;   // the wave's 64 x 64 part: rows 64 wm, weight rows 64 wn
@@ -340,6 +351,9 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
     const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
     const unsigned char* sbase = reinterpret_cast<const unsigned char*>(a.sc);
     const unsigned char* bbase = reinterpret_cast<const unsigned char*>(a.bi);
+    const unsigned char* w2base = reinterpret_cast<const unsigned char*>(a.w2);
+    const unsigned char* s2base = reinterpret_cast<const unsigned char*>(a.sc2);
+    const unsigned char* b2base = reinterpret_cast<const unsigned char*>(a.bi2);
     const uint32_t woff = wrow * a.cpr * 16u + wq * (KIND == W_Q4 ? 8u : 16u);
     const uint32_t soff = wrow * a.gpr * 2u;
     uint32_t xoff[4];
@@ -349,17 +363,20 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         xoff[i] = (m < a.M ? m : a.M - 1) * a.K * 2u + xp * 16u;
     }
 
-    f32x16_t acc[2][2];
+    f32x16_t acc[2][2], acc2[PAIR ? 2 : 1][PAIR ? 2 : 1];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 16; ++r) {
+                acc[i][j][r] = 0.f;
+                if constexpr (PAIR) acc2[i][j][r] = 0.f;
+            }
 
     // (Macros over named registers, not lambdas over a struct or arrays: an object whose address a closure holds, or an
     // array, stays in scratch once a fence stands between its writes and its reads.)
-#define FK_TILE_DECLARE(S) uint4 S##x0, S##x1, S##x2, S##x3, S##w; uint16_t S##sc, S##bi
+#define FK_TILE_DECLARE(S) uint4 S##x0, S##x1, S##x2, S##x3, S##w, S##v; uint16_t S##sc, S##bi, S##sc2, S##bi2
 #define FK_TILE_REQUEST(S, slab)                                                                                      \
     {                                                                                                                 \
         const uint32_t kf = k0 + ((slab) < slabs ? (slab) : 0u) * kTileK; /* past the end: the first slab (unused) */ \
@@ -377,6 +394,16 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         const uint32_t g = kf >> gshift;                                                                              \
         S##sc = *reinterpret_cast<const uint16_t*>(sbase + g * 2u + soff); /* kept apart: combining the two here */   \
         S##bi = *reinterpret_cast<const uint16_t*>(bbase + g * 2u + soff); /* would wait for both loads on the spot */ \
+        if constexpr (PAIR) {                                                                                         \
+            if constexpr (KIND == W_Q4) {                                                                             \
+                const uint2 v = *reinterpret_cast<const uint2*>(w2base + (kf >> 1) + woff);                           \
+                S##v = make_uint4(v.x, v.y, 0u, 0u);                                                                  \
+            } else {                                                                                                  \
+                S##v = *reinterpret_cast<const uint4*>(w2base + kf + woff);                                           \
+            }                                                                                                         \
+            S##sc2 = *reinterpret_cast<const uint16_t*>(s2base + g * 2u + soff);                                      \
+            S##bi2 = *reinterpret_cast<const uint16_t*>(b2base + g * 2u + soff);                                      \
+        }                                                                                                             \
         /* keeps the requests where they are written: left alone, the compiler moves them down to their first use */  \
         asm volatile("" ::: "memory");                                                                                \
     }
@@ -394,6 +421,13 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         uint4* wd = xs_w + kTileM * kTileStride + wr * kTileStride + wq * 2u;                                         \
         wd[0] = tile_unpack_piece<KIND>(0, S##w, sf, bf);                                                             \
         wd[1] = tile_unpack_piece<KIND>(1, S##w, sf, bf);                                                             \
+        if constexpr (PAIR) {                                                                                         \
+            uint32_t sc2_bits = S##sc2, bi2_bits = S##bi2;                                                            \
+            asm volatile("" : "+v"(sc2_bits), "+v"(bi2_bits));                                                        \
+            const float sf2 = bf16_bits_to_f32(sc2_bits), bf2 = bf16_bits_to_f32(bi2_bits);                           \
+            wd[kTileN * kTileStride] = tile_unpack_piece<KIND>(0, S##v, sf2, bf2);                                    \
+            wd[kTileN * kTileStride + 1] = tile_unpack_piece<KIND>(1, S##v, sf2, bf2);                                \
+        }                                                                                                             \
     }
     auto multiply = [&](uint32_t from) {
         const uint4* xs = lds_raw + from * kTileBufPieces;
@@ -412,6 +446,20 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
                                                                         __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
+            if constexpr (PAIR) {
+                uint4 bf2[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) bf2[j] = wb[((uint32_t)j * 32u + kTileN) * kTileStride + 2u * (uint32_t)st];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
+                                                                             __builtin_bit_cast(bf16x8_t, bf2[j]), acc2[i][j], 0, 0, 0);
+                // (a step's fragment reads stay behind the step before: requested all at once, the four steps' 24
+                // fragments push the pair form's 128 accumulator registers into scratch)
+                asm volatile("" ::: "memory");
+            }
         }
     };
     FK_TILE_DECLARE(e_);
@@ -437,7 +485,10 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         __syncthreads();
         buf ^= 1u;
     }
-    if (q <= slabs) multiply(buf);   // the last slab of an odd count
+    // the last slab of an odd count (the pair form is only planned for even counts: a conditional multiply behind the
+    // loop sends its 128 accumulator registers through scratch)
+    if constexpr (!PAIR)
+        if (q <= slabs) multiply(buf);
 #undef FK_TILE_DECLARE
 #undef FK_TILE_REQUEST
 #undef FK_TILE_STAGE
@@ -454,7 +505,14 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
             for (int r = 0; r < 16; ++r) {
                 const uint32_t m = m0 + wm * 64u + (uint32_t)(i * 32 + r % 4 + 8 * (r / 4)) + 4u * kb;
                 if (m >= a.M) continue;
-                if (a.y) {   // one k split: finished here, in the order of additions of the second kernel
+                if constexpr (PAIR) {
+                    if (a.y) {   // one k split: SwiGLU of the two finished sums, as the second kernel forms it
+                        a.y[(size_t)m * a.N + n] = (uint16_t)swiglu_bits(acc[i][j][r], acc2[i][j][r], a.variant, 1.0f);
+                    } else {
+                        a.partial[((size_t)ks * a.M + m) * a.N + n] = acc[i][j][r];
+                        a.partial2[((size_t)ks * a.M + m) * a.N + n] = acc2[i][j][r];
+                    }
+                } else if (a.y) {   // one k split: finished here, in the order of additions of the second kernel
                     float v = acc[i][j][r];
                     if (a.bias) v += bias;
                     if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * a.N + n]);
@@ -526,7 +584,7 @@ __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const QgemmReduceArgs
 
 namespace {
 
-uint32_t qgemm_form_lds_bytes(int mt) { return mt == 8 ? kTileLdsBytes : qgemm_lds_bytes(mt); }
+uint32_t qgemm_form_lds_bytes(int mt) { return mt >= 8 ? tile_lds_bytes(mt == 9) : qgemm_lds_bytes(mt); }
 
 struct QgemmShape {
     uint32_t n_blocks, m_tiles, ksplit, k_per_split;
@@ -536,7 +594,8 @@ struct QgemmShape {
 const void* qgemm_func(uint32_t bits, int mt) {
     const bool q4 = bits == 4;
     switch (mt) {
-        case 8: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8>);
+        case 8: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, false>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, false>);
+        case 9: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, true>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, true>);   // a gate / up pair
         case 1: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 1>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 1>);
         case 2: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 2>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 2>);
         default: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 4>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 4>);
@@ -546,7 +605,7 @@ const void* qgemm_func(uint32_t bits, int mt) {
 // Blocks of this kernel form that are resident at once (registers and LDS decide).
 uint32_t qgemm_resident(const DeviceFacts* dev, uint32_t bits, int mt) {
     static std::mutex mu;
-    static int cache[2][9] = {};
+    static int cache[2][10] = {};
     std::lock_guard<std::mutex> lk(mu);
     int& slot = cache[bits == 4 ? 0 : 1][mt];
     if (slot == 0) {
@@ -722,6 +781,29 @@ fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint
     float* p0 = static_cast<float*>(workspace);
     FK_TRY(plan_qgemm_main(dev, Wg, x, M, p0, &s, gate));
     float* p1 = p0 + (size_t)s.ksplit * M * Wg->n;
+    if (s.mt == 8 && Wg->bits == Wu->bits && Wg->k % 128u == 0 && s.k_per_split % 128u == 0) {   // (even slab counts)
+        // the tile form takes the pair in ONE launch (activations staged once, two sets of accumulators); with one k
+        // split it applies SwiGLU itself
+        QgemmArgs a;
+        memcpy(&a, gate->args, sizeof(a));
+        a.w2 = reinterpret_cast<const uint4*>(Wu->w);
+        a.sc2 = Wu->scales;
+        a.bi2 = Wu->biases;
+        a.partial2 = p1;
+        a.variant = variant;
+        a.y = s.ksplit == 1 ? out : nullptr;
+        a.bias = a.res = nullptr;
+        gate->func = qgemm_func(Wg->bits, 9);
+        gate->shmem = qgemm_form_lds_bytes(9);
+        gate->set_args(a);
+        FK_HIP(hipFuncSetAttribute(gate->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)gate->shmem));
+        *up = Launch();
+        if (s.ksplit == 1)
+            *reduce = Launch();
+        else
+            plan_reduce(p0, p1, nullptr, nullptr, out, M, Wg->n, s.ksplit, variant, reduce);
+        return FK_OK;
+    }
     FK_TRY(plan_qgemm_main(dev, Wu, x, M, p1, &s, up));
     plan_reduce(p0, p1, nullptr, nullptr, out, M, Wg->n, s.ksplit, variant, reduce);
     return FK_OK;

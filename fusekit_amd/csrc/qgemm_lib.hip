@@ -49,7 +49,9 @@ struct RocblasApi {
     std::mutex mu;  // one handle, one stream binding at a time
 };
 RocblasApi g_rb;
-uint32_t g_library_rows = 256;  // row count from which direct calls take this route (0: never)
+// row count from which direct calls take this route (0: never): below it the fused kernel's tile form is the faster
+// one on the 4B-class projections (passes of 256 / 512 / 768 rows: +16 / +3..9 / +7 % prompt rate), from 1024 rows this route
+uint32_t g_library_rows = 1024;
 
 bool rocblas_ready() {
     if (g_rb.tried) return g_rb.ok;

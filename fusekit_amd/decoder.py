@@ -435,15 +435,15 @@ class DecoderRuntime:
                      keep_bf16_weights: bool = False) -> int:
         """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
         active_m > 1 variants): the projections of up to `rows_per_pass` (<= 4096) tokens share ONE pass over each weight
-        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form, from 256 rows
-        up as a dequantisation to bf16 followed by a library GEMM), attention is
+        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form, from 256 rows in its LDS-tiled
+        form, from 1024 rows -- fk_set_gemm_library_rows -- as a dequantisation to bf16 followed by a library GEMM), attention is
         causal inside the group (fk_sdpa_prefill for the bf16 cache with head dimension 64 or 128,
         else the single-row kernel once per row).  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy
         first token.  Dense bf16 weights take the library GEMM for every row count.
         keep_bf16_weights: passes of at least 256 rows multiply with a bf16 copy of every projection that stays
         resident after its first use (2 bytes per weight: 7.3 GB for the 4B-class model) instead of
-        dequantising each matrix again in every pass; same results bit for bit."""
+        dequantising each matrix again in every pass; the results of the dequantise + library route, bit for bit."""
         c, w = self.cfg, self.w
         prompt = list(prompt)
         if start_offset + len(prompt) > c.capacity:

@@ -240,6 +240,26 @@ def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
                "LDS-tiled form (finished outputs at one k split)")
 
 
+def case_qgemm_swiglu(d, reps, rows, hidden=2560, inter=9728, bits=4):
+    """The gate / up pair with SwiGLU of the family fusekit_qgemm_swiglu on `rows` activation rows (from 256 rows one
+    launch of the tile form); flops of both products."""
+    per = bits / 8 + 4 / 64
+    pool = max(2, int(600e6 // (2 * inter * hidden * per)) + 1)
+    x = _bf16(rows * hidden, 1)
+    ws_bytes = 2 * fk.qgemm_workspace_bytes(rows, inter, hidden, 64)
+    tasks, keep = [], []
+    for i in range(pool):
+        Wg, Wu = _rand_weight(inter, hidden, bits, 700 + 5 * i), _rand_weight(inter, hidden, bits, 702 + 5 * i)
+        y, ws = fk.DeviceBuffer(rows * inter * 2), fk.DeviceBuffer(ws_bytes)
+        keep.append((Wg, Wu, y, ws))
+        tasks.append(Dispatch("fusekit_qgemm_swiglu_f0", [arg(x), arg(Wg.w), arg(Wu.w), arg(Wg.scales), arg(Wu.scales),
+                                                          arg(Wg.biases), arg(Wu.biases), arg(y), arg(ws)],
+                              {"bits": bits, "group": 64, "hidden": hidden, "inter": inter, "rows": rows, "variant": 1}))
+    nbytes = 2 * inter * hidden * per + rows * hidden * 2 + rows * inter * 2
+    _emit(f"qgemm_swiglu_rows{rows}_{inter}x{hidden}_q{bits}", _time_graph(d, tasks, reps), nbytes, flops=4.0 * rows * inter * hidden,
+          pool=pool)
+
+
 def case_prefill(d, reps, prompt_len=512, rows_per_pass=4096, capacity=1024, kv_bits=0, keep=False):
     """Chunked prefill of the 4B-class model: `rows_per_pass` prompt tokens per pass over the weights."""
     import time
@@ -365,6 +385,8 @@ CASES = {
     "qgemm_128": lambda d, r: case_qgemm(d, r, 128),
     "qgemm_512": lambda d, r: case_qgemm(d, r, 512),
     "qgemm_2048": lambda d, r: case_qgemm(d, r, 2048),
+    "qgemm_swiglu_512": lambda d, r: case_qgemm_swiglu(d, r, 512),
+    "qgemm_swiglu_2048": lambda d, r: case_qgemm_swiglu(d, r, 2048),
     "prefill_4b_32": lambda d, r: case_prefill(d, r, 512, 32),
     "prefill_4b": lambda d, r: case_prefill(d, r),
     "prefill_4b_128": lambda d, r: case_prefill(d, r, 512, 128),

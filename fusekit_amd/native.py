@@ -502,6 +502,9 @@ def dequantize_bf16(W: DeviceWeight, stream=None) -> DeviceWeight:
     return D
 
 
+GEMM_LIBRARY_ROWS_DEFAULT = 1024  # fk_set_gemm_library_rows' default
+
+
 def set_gemm_library_rows(rows: int):
     """Row count from which qgemm / qgemm_swiglu take the dequantise + library-GEMM route (0: never)."""
     check(lib.fk_set_gemm_library_rows(C.c_uint32(rows)))

@@ -795,7 +795,8 @@ fk_status fk_set_gemv_policy(uint32_t rows_per_tile, uint32_t grid_blocks);
 int fk_gemv_form(uint32_t n, uint32_t k, uint32_t bits, uint32_t group);
 fk_status fk_set_gemv_flat_only(int flat_only);
 /* Row count from which fk_qgemm / fk_qgemm_swiglu dequantise the matrix to bf16 once and hand the
- * product to rocBLAS (opened on first use; absent: the fused kernel is kept).  Default 256; 0 = never.
+ * product to rocBLAS (opened on first use; absent: the fused kernel is kept).  Default 1024 (below it the fused
+ * kernel's LDS-tiled form is the faster one on the benchmark model's projections); 0 = never.
  * Set it BEFORE sizing workspaces: fk_qgemm_workspace_bytes covers the route that will be taken. */
 fk_status fk_set_gemm_library_rows(uint32_t rows);
 /* 2..10 activation rows at group size 64 run fk_qgemm / fk_qgemm_swiglu as ONE launch that streams the weights

@@ -204,8 +204,8 @@ def test_qgemm_swiglu(fk, variant):
 @pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 128)])
 @pytest.mark.parametrize("m,n,k", [(512, 333, 2560), (700, 1152, 896), (300, 512, 4864)])
 def test_qgemm_many_rows_both_routes(fk, m, n, k, bits, group, route):
-    """From 256 rows direct calls dequantise the matrix to bf16 once and take the library GEMM; the
-    fused kernel stays reachable (and is what a graph node runs).  Same arithmetic, same oracle form,
+    """From a row threshold on (1024 by default; 256 here) direct calls dequantise the matrix to bf16 once and take
+    the library GEMM; the fused kernel stays reachable (and is what a graph node runs).  Same arithmetic, same oracle form,
     with bias and residual in the epilogue."""
     fk.set_gemm_library_rows(0 if route == "kernel" else 256)
     try:
@@ -222,7 +222,7 @@ def test_qgemm_many_rows_both_routes(fk, m, n, k, bits, group, route):
         for r in range(0, m, 7):
             _check(got[r], want[r], full[r], W, x[r])
     finally:
-        fk.set_gemm_library_rows(256)
+        fk.set_gemm_library_rows(fk.GEMM_LIBRARY_ROWS_DEFAULT)
 
 
 @pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 128)])
@@ -261,6 +261,39 @@ def test_qgemm_tile_form_finishes_its_outputs_at_one_k_split(fk, bits, group):
         _check(got[r], want[r], full[r], W, x[r])
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,hidden,inter,kernels", [(512, 256, 9700, 1), (300, 1024, 1280, 2)])
+@pytest.mark.parametrize("variant", [1, 2])
+def test_qgemm_swiglu_tile_form_takes_the_pair_in_one_launch(fk, bits, m, hidden, inter, kernels, variant):
+    """From 256 rows a gate / up pair (same shape, even count of 64-wide k slabs per split) is ONE launch of the tile
+    form: the activations staged once, two sets of accumulators; with one k split SwiGLU is applied there (1 kernel),
+    otherwise the partial sums of both go to the usual second kernel (2 kernels instead of 3)."""
+    from fusekit_amd.runtime import Dispatch, Dispatcher, arg
+    Wg, Wu = make_qweight(90 + bits, inter, hidden, bits), make_qweight(93 + bits, inter, hidden, bits)
+    x = normal_bf16(96, (m, hidden))
+    dg, du, bx = to_device(fk, Wg), to_device(fk, Wu), _dev(fk, x)
+    out = fk.DeviceBuffer(2 * m * inter)
+    ws = fk.DeviceBuffer(2 * fk.qgemm_workspace_bytes(m, inter, hidden, 64))
+    d = Dispatcher()
+    task = Dispatch("fusekit_qgemm_swiglu_f0", [arg(bx), arg(dg.w), arg(du.w), arg(dg.scales), arg(du.scales), arg(dg.biases),
+                                                arg(du.biases), arg(out), arg(ws)],
+                    {"bits": bits, "group": 64, "hidden": hidden, "inter": inter, "rows": m, "variant": variant})
+    geo = d.plan_geometry(task)
+    assert geo.n_kernels == kernels and tuple(geo.threadgroup[0]) == (512, 1, 1) and geo.lds_bytes[0] == 147456
+    out.upload(np.full(m * inter, 0x7fc0, np.uint16))
+    d.dispatch_kernel(task)
+    fk.sync()
+    got = out.to_numpy(np.uint16, (m, inter))
+    _, g = oracle.qgemm_bf16w(Wg, x, None, want_acc=True)
+    _, u = oracle.qgemm_bf16w(Wu, x, None, want_acc=True)
+    rows = list(range(0, m, 41)) + [255, 256, m - 1]
+    want = np.array([[oracle.swiglu_scalar(float(a), float(b), variant) for a, b in zip(g[r], u[r])] for r in rows], dtype=np.uint16)
+    sel = got[rows]
+    gf, wf = oracle.bf16_to_f32(sel).astype(np.float64), oracle.bf16_to_f32(want).astype(np.float64)
+    assert np.linalg.norm(gf - wf) / np.linalg.norm(wf) <= 1e-2
+    assert np.mean(sel != want) <= 0.05          # fp32 summation order may cross a bf16 rounding edge
+
+
 @pytest.mark.parametrize("route,m", [("kernel", 512), ("library", 512), ("library", 2048)])
 def test_qgemm_swiglu_many_rows_both_routes(fk, route, m):
     """From 2048 rows the library route lets the GEMM round gate and up to bf16 itself and runs SwiGLU over bf16."""
@@ -283,7 +316,7 @@ def test_qgemm_swiglu_many_rows_both_routes(fk, route, m):
         assert np.linalg.norm(gf - wf) / np.linalg.norm(wf) <= 1e-2
         assert np.mean(sel != want) <= 0.05          # fp32 summation order may cross a bf16 rounding edge
     finally:
-        fk.set_gemm_library_rows(256)
+        fk.set_gemm_library_rows(fk.GEMM_LIBRARY_ROWS_DEFAULT)
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 333, 256), (100, 1152, 896), (512, 256, 4864)])

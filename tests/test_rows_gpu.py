@@ -140,16 +140,21 @@ def test_batched_prefill_matches_token_by_token(fk, bits, prompt_len, rows_per_p
 @pytest.mark.parametrize("bits", [4, 8])
 def test_prefill_with_resident_bf16_weights_is_bit_identical(fk, bits):
     """keep_bf16_weights: passes of at least 256 rows multiply with a resident bf16 copy of every projection
-    (fk_dequantize_bf16) instead of dequantising in every pass: same caches, same logits, bit for bit; and the
-    copy itself is T(code * scale + bias) of the oracle."""
+    (fk_dequantize_bf16) instead of dequantising in every pass: the caches and logits of the dequantise + library route
+    (taken here from 256 rows, as the copy is; by default only from 1024), bit for bit; and the copy itself is
+    T(code * scale + bias) of the oracle."""
     from fusekit_amd.decoder import DecoderConfig, DecoderRuntime, DecoderWeights
     cfg = DecoderConfig(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=2000, capacity=1024,
                         bits=bits, qk_norm=True, swiglu_variant=1)
     W = DecoderWeights.random_init(cfg, seed=43)
     prompt = rng(44).integers(0, cfg.vocab, 600).tolist()
     a, b = DecoderRuntime(cfg, W), DecoderRuntime(cfg, W)
-    ta = a.prefill_rows(prompt, rows_per_pass=512)
-    tb = b.prefill_rows(prompt, rows_per_pass=512, keep_bf16_weights=True)
+    fk.set_gemm_library_rows(256)
+    try:
+        ta = a.prefill_rows(prompt, rows_per_pass=512)
+        tb = b.prefill_rows(prompt, rows_per_pass=512, keep_bf16_weights=True)
+    finally:
+        fk.set_gemm_library_rows(fk.GEMM_LIBRARY_ROWS_DEFAULT)
     assert len(b._bf16_weights) == 7 * cfg.n_layers and not a._bf16_weights
     assert ta == tb and np.array_equal(a.logits.to_numpy(np.uint16), b.logits.to_numpy(np.uint16))
     for l in range(cfg.n_layers):
