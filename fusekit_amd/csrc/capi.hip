@@ -406,6 +406,23 @@ fk_status fk_qgemm(const fk_weight* W, const uint16_t* x, uint32_t m, const uint
     return run_launch(reduce, (hipStream_t)s);
 }
 
+fk_status fk_qgemm_fanout(const fk_weight* const* W, uint32_t n_mats, const uint16_t* x, uint32_t m,
+                          const uint16_t* const* bias, uint16_t* const* y, void* workspace, fk_stream s) {
+    if (!W || !y || n_mats < 1 || n_mats > 3) return set_error(FK_ERR_INVALID, "fk_qgemm_fanout: one to three matrices");
+    bool fused = false;
+    if (n_mats > 1 && W[0] && W[0]->bits != 16 && !qgemm_takes_library(m)) {
+        Launch main, reduce;
+        FK_TRY(plan_qgemm_fanout(W, n_mats, x, m, bias, y, workspace, &main, &reduce, &fused));
+        if (fused) {
+            FK_TRY(run_launch(main, (hipStream_t)s));
+            return run_launch(reduce, (hipStream_t)s);
+        }
+    }
+    for (uint32_t i = 0; i < n_mats; ++i)   // one by one, in stream order (they share the workspace)
+        FK_TRY(fk_qgemm(W[i], x, m, bias ? bias[i] : nullptr, nullptr, y[i], workspace, s));
+    return FK_OK;
+}
+
 fk_status fk_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16_t* x, uint32_t m, int variant,
                           uint16_t* out, void* workspace, fk_stream s) {
     if (Wg && Wu && Wg->bits == 16 && Wu->bits == 16) {

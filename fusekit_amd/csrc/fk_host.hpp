@@ -160,6 +160,9 @@ fk_status plan_route_reduce(const uint16_t* parts, const uint16_t* route_weight,
 fk_status qgemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group, size_t* bytes);
 fk_status plan_qgemm(const fk_weight* W, const uint16_t* x, uint32_t M, const uint16_t* bias, const uint16_t* res,
                      uint16_t* y, void* workspace, Launch* main, Launch* reduce);
+fk_status plan_qgemm_fanout(const fk_weight* const* W, uint32_t n_mats, const uint16_t* x, uint32_t M,
+                            const uint16_t* const* bias, uint16_t* const* y, void* workspace, Launch* main, Launch* reduce,
+                            bool* fused);
 fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint16_t* x, uint32_t M, int variant,
                             uint16_t* out, void* workspace, Launch* gate, Launch* up, Launch* reduce);
 

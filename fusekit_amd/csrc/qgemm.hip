@@ -71,6 +71,18 @@ struct QgemmArgs {
     uint16_t* y;
     const uint16_t* bias;
     const uint16_t* res;
+    // the tile form over up to three matrices that share x and K (a q / k / v fan-out): n_seg > 1, the blocks along N
+    // run through the matrices in turn (seg[i].nb_end: first block behind matrix i); partial sums of all matrices lie
+    // side by side in rows of n_total columns (matrix i from column seg[i].col0)
+    uint32_t n_seg, n_total;
+    struct Seg {
+        const uint4* w;
+        const uint16_t* sc;
+        const uint16_t* bi;
+        uint16_t* y;
+        const uint16_t* bias;
+        uint32_t N, nb_end, col0, pad;
+    } seg[3];
     // the tile form for a gate / up pair: the second matrix (same shape), its partial sums, the SwiGLU variant
     const uint4* w2;
     const uint16_t* sc2;
@@ -332,7 +344,25 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, kb = lane >> 5, nl = lane & 31u;
     const uint32_t wm = wave >> 1, wn = wave & 1u;   // the wave's 64 x 64 part: rows 64 wm, weight rows 64 wn
-    const uint32_t nb = blockIdx.x % a.n_blocks, ks = blockIdx.x / a.n_blocks;
+    uint32_t nb = blockIdx.x % a.n_blocks;
+    const uint32_t ks = blockIdx.x / a.n_blocks;
+    // the matrix this block works on (one, or the fan-out's matrix whose range of blocks holds nb)
+    const uint4* w_mat = a.w;
+    const uint16_t *sc_mat = a.sc, *bi_mat = a.bi, *bias_mat = a.bias;
+    uint16_t* y_mat = a.y;
+    uint32_t N = a.N, col0 = 0, row_cols = a.N;   // row_cols: columns of a row of partial sums
+    if (!PAIR && a.n_seg > 1u) {
+        const uint32_t si = nb >= a.seg[0].nb_end ? (nb >= a.seg[1].nb_end ? 2u : 1u) : 0u;
+        nb -= si ? a.seg[si - 1u].nb_end : 0u;
+        w_mat = a.seg[si].w;
+        sc_mat = a.seg[si].sc;
+        bi_mat = a.seg[si].bi;
+        bias_mat = a.seg[si].bias;
+        y_mat = a.seg[si].y;
+        N = a.seg[si].N;
+        col0 = a.seg[si].col0;
+        row_cols = a.n_total;
+    }
     const uint32_t m0 = blockIdx.y * kTileM, n0 = nb * kTileN;
     const uint32_t k0 = ks * a.k_per_split;
     const uint32_t k1 = k0 + a.k_per_split < a.K ? k0 + a.k_per_split : a.K;
@@ -343,14 +373,14 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
     // tid % 4 of the slab (8 bytes of int4, 16 of int8)
     const uint32_t xr = tid >> 3, xp = tid & 7u;
     const uint32_t wr = tid >> 2, wq = tid & 3u;
-    const uint32_t wrow = n0 + wr < a.N ? n0 + wr : a.N - 1;   // rows past the end read the last row; never stored
+    const uint32_t wrow = n0 + wr < N ? n0 + wr : N - 1;   // rows past the end read the last row; never stored
     // Every request is a block-uniform base (scalar registers, advanced by the slab) plus a per-lane 32-bit byte offset
     // that never changes: no vector address arithmetic per slab (the planner admits the form only while the operands
     // stay under 4 GB).
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.w);
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(w_mat);
     const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
-    const unsigned char* sbase = reinterpret_cast<const unsigned char*>(a.sc);
-    const unsigned char* bbase = reinterpret_cast<const unsigned char*>(a.bi);
+    const unsigned char* sbase = reinterpret_cast<const unsigned char*>(sc_mat);
+    const unsigned char* bbase = reinterpret_cast<const unsigned char*>(bi_mat);
     const unsigned char* w2base = reinterpret_cast<const unsigned char*>(a.w2);
     const unsigned char* s2base = reinterpret_cast<const unsigned char*>(a.sc2);
     const unsigned char* b2base = reinterpret_cast<const unsigned char*>(a.bi2);
@@ -497,8 +527,8 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const uint32_t n = n0 + wn * 64u + (uint32_t)j * 32u + nl;
-        if (n >= a.N) continue;
-        const float bias = (a.y && a.bias) ? bf16_bits_to_f32(a.bias[n]) : 0.f;
+        if (n >= N) continue;
+        const float bias = (y_mat && bias_mat) ? bf16_bits_to_f32(bias_mat[n]) : 0.f;
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -512,13 +542,13 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
                         a.partial[((size_t)ks * a.M + m) * a.N + n] = acc[i][j][r];
                         a.partial2[((size_t)ks * a.M + m) * a.N + n] = acc2[i][j][r];
                     }
-                } else if (a.y) {   // one k split: finished here, in the order of additions of the second kernel
+                } else if (y_mat) {   // one k split: finished here, in the order of additions of the second kernel
                     float v = acc[i][j][r];
-                    if (a.bias) v += bias;
-                    if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * a.N + n]);
-                    a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
+                    if (bias_mat) v += bias;
+                    if (a.res) v += bf16_bits_to_f32(a.res[(size_t)m * N + n]);
+                    y_mat[(size_t)m * N + n] = (uint16_t)f32_to_bf16_bits(v);
                 } else {
-                    a.partial[((size_t)ks * a.M + m) * a.N + n] = acc[i][j][r];
+                    a.partial[((size_t)ks * a.M + m) * row_cols + col0 + n] = acc[i][j][r];
                 }
             }
     }
@@ -580,6 +610,36 @@ __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const QgemmReduceArgs
     if (a.bias) s0 += bf16_bits_to_f32(a.bias[i % a.N]);
     if (a.res) s0 += bf16_bits_to_f32(a.res[i]);
     a.y[i] = (uint16_t)f32_to_bf16_bits(s0);
+}
+
+// Split-k sums of a fan-out (rows of n_total columns, the matrices side by side) to the matrices' own outputs; four
+// consecutive columns per thread (every matrix's N is a multiple of 4), additions in split order, then the bias.
+struct QgemmFanReduceArgs {
+    const float* p;
+    uint32_t M, n_total, ksplit, n_seg;
+    uint16_t* y[3];
+    const uint16_t* bias[3];
+    uint32_t col0[3], N[3];
+};
+__global__ __launch_bounds__(256) void qgemm_fan_reduce_kernel(const QgemmFanReduceArgs a) {
+    const uint32_t total = a.M * a.n_total, i = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (i >= total) return;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t ks = 0; ks < a.ksplit; ++ks) {
+        const float4 v = *reinterpret_cast<const float4*>(a.p + (size_t)ks * total + i);
+        s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
+    }
+    const uint32_t m = i / a.n_total, c = i - m * a.n_total;
+    const uint32_t si = (a.n_seg > 2u && c >= a.col0[2]) ? 2u : ((a.n_seg > 1u && c >= a.col0[1]) ? 1u : 0u);
+    const uint32_t n = c - a.col0[si];
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v = s[e];
+        if (a.bias[si]) v += bf16_bits_to_f32(a.bias[si][n + e]);
+        o[e] = f32_to_bf16_bits(v);
+    }
+    *reinterpret_cast<uint2*>(a.y[si] + (size_t)m * a.N[si] + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
 }
 
 namespace {
@@ -759,6 +819,93 @@ fk_status plan_qgemm(const fk_weight* W, const uint16_t* x, uint32_t M, const ui
         *reduce = Launch();   // the tile form with one k split rounds its outputs itself
     else
         plan_reduce(static_cast<float*>(workspace), nullptr, bias, res, y, M, W->n, s.ksplit, 0, reduce);
+    return FK_OK;
+}
+
+// Up to three matrices over the same activation rows (same K, bits and group size; every N a multiple of 4) as ONE
+// launch of the tile form whose blocks along N run through the matrices in turn, finished by one second kernel when k
+// is split.  *fused = false (and nothing planned) when the tile form does not apply: the caller runs the matrices one
+// by one.
+fk_status plan_qgemm_fanout(const fk_weight* const* W, uint32_t n_mats, const uint16_t* x, uint32_t M,
+                            const uint16_t* const* bias, uint16_t* const* y, void* workspace, Launch* main, Launch* reduce,
+                            bool* fused) {
+    const DeviceFacts* dev;
+    FK_TRY(device_facts(&dev));
+    *fused = false;
+    if (n_mats < 2 || n_mats > 3 || !W || !y) return set_error(FK_ERR_INVALID, "qgemm fan-out: two or three matrices");
+    if (!x || !workspace) return set_error(FK_ERR_INVALID, "qgemm fan-out: null activation or workspace");
+    uint32_t n_total = 0, blocks_n = 0;
+    for (uint32_t i = 0; i < n_mats; ++i) {
+        FK_TRY(check_weight(W[i], "qgemm fan-out"));
+        if (!y[i]) return set_error(FK_ERR_INVALID, "qgemm fan-out: null output");
+        if (W[i]->k != W[0]->k || W[i]->bits != W[0]->bits || W[i]->group != W[0]->group)
+            return set_error(FK_ERR_INVALID, "qgemm fan-out: the matrices need the same K, bits and group size");
+        if (W[i]->n % 4u) return FK_OK;
+        n_total += W[i]->n;
+        blocks_n += (W[i]->n + kTileN - 1) / kTileN;
+    }
+    QgemmShape s;
+    FK_TRY(qgemm_shape(dev, M, blocks_n * kTileN, W[0]->k, W[0]->group, W[0]->bits, &s));
+    if (s.mt != 8 || (uint64_t)M * n_total > 0x7fffffffull) return FK_OK;
+    for (uint32_t i = 0; i < n_mats; ++i)
+        if ((uint64_t)W[i]->n * W[i]->k >= (1ull << 32)) return FK_OK;
+    QgemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x;
+    a.partial = static_cast<float*>(workspace);
+    a.M = M;
+    a.N = W[0]->n;
+    a.K = W[0]->k;
+    a.cpr = W[0]->k / (W[0]->bits == 4 ? 32u : 16u);
+    a.gpr = W[0]->k / W[0]->group;
+    a.group = W[0]->group;
+    a.k_per_split = s.k_per_split;
+    a.n_blocks = blocks_n;
+    a.n_seg = n_mats;
+    a.n_total = n_total;
+    QgemmFanReduceArgs r;
+    memset(&r, 0, sizeof(r));
+    uint32_t nb = 0, col = 0;
+    for (uint32_t i = 0; i < 3; ++i) {
+        const uint32_t j = i < n_mats ? i : n_mats - 1;   // unused entries repeat the last matrix (never selected)
+        if (i < n_mats) nb += (W[i]->n + kTileN - 1) / kTileN;
+        a.seg[i].w = reinterpret_cast<const uint4*>(W[j]->w);
+        a.seg[i].sc = W[j]->scales;
+        a.seg[i].bi = W[j]->biases;
+        a.seg[i].y = s.ksplit == 1 ? y[j] : nullptr;
+        a.seg[i].bias = bias ? bias[j] : nullptr;
+        a.seg[i].N = W[j]->n;
+        a.seg[i].nb_end = i < n_mats ? nb : 0xffffffffu;
+        a.seg[i].col0 = i < n_mats ? col : 0u;
+        r.y[i] = y[j];
+        r.bias[i] = bias ? bias[j] : nullptr;
+        r.col0[i] = i < n_mats ? col : 0xffffffffu;
+        r.N[i] = W[j]->n;
+        if (i < n_mats) col += W[i]->n;
+    }
+    a.w = a.seg[0].w;
+    a.sc = a.seg[0].sc;
+    a.bi = a.seg[0].bi;
+    main->func = qgemm_func(W[0]->bits, 8);
+    main->grid = dim3(blocks_n * s.ksplit, s.m_tiles, 1);
+    main->block = dim3(kTileBlock, 1, 1);
+    main->shmem = qgemm_form_lds_bytes(8);
+    main->set_args(a);
+    FK_HIP(hipFuncSetAttribute(main->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)main->shmem));
+    *reduce = Launch();
+    if (s.ksplit > 1) {
+        r.p = a.partial;
+        r.M = M;
+        r.n_total = n_total;
+        r.ksplit = s.ksplit;
+        r.n_seg = n_mats;
+        reduce->func = reinterpret_cast<const void*>(&qgemm_fan_reduce_kernel);
+        reduce->grid = dim3((M * n_total / 4u + 255u) / 256u, 1, 1);
+        reduce->block = dim3(256, 1, 1);
+        reduce->shmem = 0;
+        reduce->set_args(r);
+    }
+    *fused = true;
     return FK_OK;
 }
 

@@ -456,7 +456,8 @@ class DecoderRuntime:
             # number of 128-row tiles; the last pass of a prompt may have any row count up to R
             ws = max(native.qgemm_workspace_bytes(m, n, k, 0 if c.bits == 16 else c.group)
                      for m in {R} | {v for v in (*range(512, 4096, 128), 384, 256, 128, 64, 32) if v < R}
-                     for n, k in ((c.n_q, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
+                     for n, k in ((c.n_q, c.hidden), (c.n_q + 2 * c.n_kvd, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden),
+                                  (c.hidden, c.inter)))
             # only the single-row attention kernel (quantised cache, other head dimensions) needs a workspace
             pb, cb = (native.sdpa_workspace_bytes(c.n_heads, c.n_kv, c.head_dim, c.head_dim, c.capacity)
                       if c.head_dim not in (64, 128) else (0, 0))
@@ -492,9 +493,14 @@ class DecoderRuntime:
             for l in range(c.n_layers):
                 p = f"layers.{l}."
                 native.rmsnorm_rows(b["x"], w.vecs[p + "input_layernorm"], c.eps, m, c.hidden, b["xn"])
-                for nm, dst in (("q", b["q"]), ("k", b["k"]), ("v", b["v"])):
-                    bias = w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None
-                    native.qgemm(mat(p + f"self_attn.{nm}_proj", m), b["xn"], m, bias, None, dst, b["ws"])
+                # q, k and v over the same rows: one call (one launch of the fused kernel where its tile form applies)
+                qkv = [mat(p + f"self_attn.{nm}_proj", m) for nm in "qkv"]
+                qkv_bias = [w.vecs.get(p + f"self_attn.{nm}_proj.bias") for nm in "qkv"] if c.qkv_bias else None
+                if all(W.bits != 16 for W in qkv):
+                    native.qgemm_fanout(qkv, b["xn"], m, qkv_bias, [b["q"], b["k"], b["v"]], b["ws"])
+                else:
+                    for i, dst in enumerate((b["q"], b["k"], b["v"])):
+                        native.qgemm(qkv[i], b["xn"], m, qkv_bias[i] if qkv_bias else None, None, dst, b["ws"])
                 qn = w.vecs.get(p + "self_attn.q_norm") if c.qk_norm else None
                 kn = w.vecs.get(p + "self_attn.k_norm") if c.qk_norm else None
                 if c.kv_bits:

@@ -290,6 +290,16 @@ def qgemm(W, x, m, bias, residual, y, workspace, stream=None) -> None:
                        _ptr(stream)))
 
 
+def qgemm_fanout(Ws, x, m, biases, ys, workspace, stream=None) -> None:
+    """One to three matrices over the same activation rows (q / k / v of a prompt pass); workspace:
+    qgemm_workspace_bytes(m, sum of n, k, group)."""
+    n = len(Ws)
+    w_arr = (C.POINTER(type(Ws[0].c)) * n)(*[C.pointer(W.c) for W in Ws])
+    y_arr = (C.c_void_p * n)(*[_ptr(y).value for y in ys])
+    b_arr = None if biases is None else (C.c_void_p * n)(*[_ptr(b).value for b in biases])
+    check(lib.fk_qgemm_fanout(w_arr, C.c_uint32(n), _ptr(x), C.c_uint32(m), b_arr, y_arr, _ptr(workspace), _ptr(stream)))
+
+
 def qgemm_swiglu(Wg, Wu, x, m, variant, out, workspace, stream=None) -> None:
     check(lib.fk_qgemm_swiglu(C.byref(Wg.c), C.byref(Wu.c), _ptr(x), C.c_uint32(m), C.c_int(variant), _ptr(out),
                               _ptr(workspace), _ptr(stream)))

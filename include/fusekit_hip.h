@@ -272,6 +272,16 @@ fk_status fk_qgemm(const fk_weight *W, const uint16_t *x, uint32_t m, const uint
                    const uint16_t *residual, uint16_t *y, void *workspace, fk_stream s);
 fk_status fk_qgemm_swiglu(const fk_weight *Wg, const fk_weight *Wu, const uint16_t *x, uint32_t m, int variant,
                           uint16_t *out, void *workspace, fk_stream s);
+/*     fk_qgemm_fanout: one to three matrices over the SAME activation rows, y[i][m, N_i] = T(x @ W[i]^T (+ bias[i])) -- the
+ *     q / k / v projections of a prompt pass, which the reference dispatches one after the other (qMM per projection,
+ *     python/fusekit_runtime/dispatch.py prefill variants).  Same results as fk_qgemm per matrix (same kernel
+ *     arithmetic).  From 256 rows, below the fk_set_gemm_library_rows() threshold, with equal K, bits and group size
+ *     and every N_i a multiple of 4, the matrices run as ONE launch of the fused kernel whose blocks along N run
+ *     through them in turn (the narrow k and v projections alone leave most of the device idle); otherwise the
+ *     call is fk_qgemm per matrix.  bias: null or an array of n_mats pointers (each may be null).
+ *     workspace: fk_qgemm_workspace_bytes(m, N_0 + N_1 + N_2, k, group) bytes. */
+fk_status fk_qgemm_fanout(const fk_weight *const *W, uint32_t n_mats, const uint16_t *x, uint32_t m,
+                          const uint16_t *const *bias, uint16_t *const *y, void *workspace, fk_stream s);
 
 /* H   final RMSNorm + vocabulary GEMV, logits in T.  Replaces
  *     src/codegen/kernels/final_rmsnorm_lm_head.rs:144-629. */

@@ -294,6 +294,35 @@ def test_qgemm_swiglu_tile_form_takes_the_pair_in_one_launch(fk, bits, m, hidden
     assert np.mean(sel != want) <= 0.05          # fp32 summation order may cross a bf16 rounding edge
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,k,ns,with_bias", [(512, 256, (4096, 1024, 1024), False),   # one k split: finished in the launch
+                                              (300, 1024, (1000, 520, 260), True),     # ragged, k split, the fan-out's second kernel
+                                              (512, 512, (2048, 1024), True),          # two matrices
+                                              (100, 256, (512, 256, 256), False)])     # too few rows for the tile form: one by one
+def test_qgemm_fanout_of_the_prompt_projections(fk, bits, m, k, ns, with_bias):
+    """fk_qgemm_fanout: up to three matrices over the same rows (q / k / v of a prompt pass) as one launch of the tile
+    form whose blocks run through the matrices in turn; every output against the oracle form of its row count."""
+    Ws = [make_qweight(110 + bits + 3 * i, n, k, bits) for i, n in enumerate(ns)]
+    x = normal_bf16(120, (m, k))
+    biases = [normal_bf16(121 + i, n) if (with_bias and i != 1) else None for i, n in enumerate(ns)]
+    dWs, bx = [to_device(fk, W) for W in Ws], _dev(fk, x)
+    dbs = [_dev(fk, b) for b in biases]
+    ys = [fk.DeviceBuffer(2 * m * n) for n in ns]
+    for y, n in zip(ys, ns):
+        y.upload(np.full(m * n, 0x7fc0, np.uint16))
+    ws = fk.DeviceBuffer(max(fk.qgemm_workspace_bytes(m, sum(ns), k, 64), max(fk.qgemm_workspace_bytes(m, n, k, 64) for n in ns)))
+    fk.qgemm_fanout(dWs, bx, m, dbs if with_bias else None, ys, ws)
+    fk.sync()
+    rows = sorted(set(list(range(0, m, 53)) + [m - 1, min(255, m - 1), min(256, m - 1)]))
+    for W, b, y, n in zip(Ws, biases, ys, ns):
+        got = y.to_numpy(np.uint16, (m, n))
+        ref, acc = _reference(W, x)
+        full = acc if b is None else acc + oracle.bf16_to_f32(b)[None, :]
+        want = ref if b is None else oracle.f32_to_bf16(full.astype(np.float32))
+        for r in rows:
+            _check(got[r], want[r], full[r], W, x[r])
+
+
 @pytest.mark.parametrize("route,m", [("kernel", 512), ("library", 512), ("library", 2048)])
 def test_qgemm_swiglu_many_rows_both_routes(fk, route, m):
     """From 2048 rows the library route lets the GEMM round gate and up to bf16 itself and runs SwiGLU over bf16."""
