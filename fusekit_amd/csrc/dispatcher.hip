@@ -1388,6 +1388,57 @@ fk_status plan_qgemm_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     return FK_OK;
 }
 
+// The q / k / v projections of several token rows (fk_qgemm_fanout): x, W_q, W_k, W_v, s_q, s_k, s_v, b_q, b_k, b_v,
+// [bias_q, bias_k, bias_v], q, k, v, workspace (fk_qgemm_workspace_bytes(rows, n_q + 2 n_kv, hidden, group)).
+// Parameters: hidden (= K), n_q, n_kv, rows, bits, group, has_bias.  One launch of the fused kernel's tile form (plus the
+// fan-out's second kernel when k is split); FK_ERR_UNSUPPORTED where that form does not apply (fewer than 256 rows, an n
+// that is no multiple of 4): the caller dispatches fusekit_qgemm per matrix then.
+fk_status plan_qgemm_fanout_d(const Dispatch& d, Launch* l, SlotRW* rw) {
+    const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("hidden"), rows = d.u("rows");
+    const uint32_t ns[3] = {d.u("n_q"), d.u("n_kv"), d.u("n_kv")};
+    const bool has_bias = d.u("has_bias", 0) != 0;
+    size_t s = 10;
+    const size_t bias_slot = s;
+    if (has_bias) s += 3;
+    const size_t out_slot = s;
+    s += 3;
+    const size_t ws_slot = s++;
+    FK_TRY(need_args(d, s));
+    if (bits != 4 && bits != 8) return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": bits must be 4 or 8");
+    if (rows == 0 || K == 0 || ns[0] == 0 || ns[1] == 0) return set_error(FK_ERR_INVALID, d.kernel + ": hidden / n_q / n_kv / rows parameters missing");
+    fk_weight W[3];
+    const fk_weight* Wp[3];
+    const uint16_t* bias[3] = {nullptr, nullptr, nullptr};
+    uint16_t* y[3];
+    FK_TRY(need_bytes(d, 0, (size_t)rows * K * 2));
+    for (int m = 0; m < 3; ++m) {
+        FK_TRY(bind_weight(d, bits, group, ns[m], K, 1 + m, 4 + m, 7 + m, &W[m]));
+        Wp[m] = &W[m];
+        if (has_bias) {
+            FK_TRY(need_bytes(d, bias_slot + m, (size_t)ns[m] * 2));
+            bias[m] = arg_ptr<const uint16_t>(d, bias_slot + m);
+        }
+        FK_TRY(need_bytes(d, out_slot + m, (size_t)rows * ns[m] * 2));
+        y[m] = arg_ptr<uint16_t>(d, out_slot + m);
+    }
+    size_t ws = 0;
+    FK_TRY(qgemm_workspace_bytes(rows, ns[0] + 2 * ns[1], K, group, &ws));
+    FK_TRY(need_bytes(d, ws_slot, ws));
+    for (uint32_t i = 0; i < out_slot; ++i) rw->reads.push_back(i);
+    rw->reads.push_back((uint32_t)ws_slot);
+    rw->writes = {(uint32_t)out_slot, (uint32_t)out_slot + 1, (uint32_t)out_slot + 2, (uint32_t)ws_slot};
+    Launch reduce;
+    bool fused = false;
+    FK_TRY(plan_qgemm_fanout(Wp, 3, arg_ptr<const uint16_t>(d, 0), rows, has_bias ? bias : nullptr, y, d.args[ws_slot].ptr, l, &reduce,
+                             &fused));
+    if (fused) {
+        if (reduce.func) l->then.push_back(reduce);
+        return FK_OK;
+    }
+    return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": the fan-out needs the fused kernel's tile form (256 rows or more, every n a "
+                                         "multiple of 4); dispatch fusekit_qgemm per matrix instead");
+}
+
 // x, W_gate, W_up, s_g, s_u, b_g, b_u, out, workspace.  Parameters: hidden, inter, rows, variant.
 fk_status plan_qgemm_swiglu_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), hidden = d.u("hidden"), inter = d.u("inter");
@@ -1457,6 +1508,7 @@ const Family kFamilies[] = {
     {"fusekit_qgemv", plan_qgemv_d},
     {"fusekit_qgemm", plan_qgemm_d},
     {"fusekit_qgemm_swiglu", plan_qgemm_swiglu_d},
+    {"fusekit_qgemm_fanout", plan_qgemm_fanout_d},
     {"fusekit_routed_qmv_swiglu", plan_routed_swiglu},
     {"fusekit_routed_qmv_reduce", plan_routed_reduce},
     {"fusekit_rmsnorm_rope_q_decode",

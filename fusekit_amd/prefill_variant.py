@@ -44,7 +44,8 @@ class PrefillVariant:
         self.q, self.k, self.v = B(m * c.n_q * 2), B(m * c.n_kvd * 2), B(m * c.n_kvd * 2)
         self.att, self.mid = B(m * c.n_q * 2), B(m * c.inter * 2)
         ws = max(native.qgemm_workspace_bytes(m, n, k, c.group)
-                 for n, k in ((c.n_q, c.hidden), (c.n_kvd, c.hidden), (c.hidden, c.n_q), (c.inter, c.hidden), (c.hidden, c.inter)))
+                 for n, k in ((c.n_q, c.hidden), (c.n_q + 2 * c.n_kvd, c.hidden), (c.n_kvd, c.hidden), (c.hidden, c.n_q),
+                              (c.inter, c.hidden), (c.hidden, c.inter)))
         self.ws = B(2 * ws)
         self.tasks = self._build()
         self.graph = rt.d.build_decode_graph(self.tasks, False)
@@ -55,6 +56,16 @@ class PrefillVariant:
         return {p + "tokens": self.tokens, p + "offset": self.offset, p + "kv_len": self.kv_len, p + "x.0": self.x[0],
                 p + "x.1": self.x[1], p + "xn": self.xn, p + "q": self.q, p + "k": self.k, p + "v": self.v, p + "att": self.att,
                 p + "mid": self.mid, p + "ws": self.ws}
+
+    def _fanout_applies(self, task: Dispatch) -> bool:
+        """Whether the family fusekit_qgemm_fanout plans this dispatch (its tile form needs 256 rows or more)."""
+        if getattr(self, "_fanout", None) is None:
+            try:
+                self.rt.d.plan_geometry(task)
+                self._fanout = True
+            except native.FusekitError:
+                self._fanout = False
+        return self._fanout
 
     def _build(self) -> List[Dispatch]:
         rt, c, w, m = self.rt, self.rt.cfg, self.rt.w, self.m
@@ -93,9 +104,20 @@ class PrefillVariant:
             else:
                 t.append(Dispatch(name("rmsnorm_rows"), [arg(self.x[0]), arg(w.vecs[p + "input_layernorm"]), arg(self.xn)],
                                   dict(rows=m, hidden=c.hidden, eps=c.eps)))
-                for nm, dst in (("q", self.q), ("k", self.k), ("v", self.v)):
-                    matmul(self.xn, w.mats[p + f"self_attn.{nm}_proj"], dst,
-                           bias=w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None)
+                Wq, Wk, Wv = (w.mats[p + f"self_attn.{nm}_proj"] for nm in "qkv")
+                qkv_bias = [w.vecs.get(p + f"self_attn.{nm}_proj.bias") for nm in "qkv"] if c.qkv_bias else []
+                fan = Dispatch(name("qgemm_fanout"),
+                               [arg(self.xn), arg(Wq.w), arg(Wk.w), arg(Wv.w), arg(Wq.scales), arg(Wk.scales), arg(Wv.scales),
+                                arg(Wq.biases), arg(Wk.biases), arg(Wv.biases)] + [arg(b_) for b_ in qkv_bias] +
+                               [arg(self.q), arg(self.k), arg(self.v), arg(self.ws)],
+                               dict(quant, hidden=c.hidden, n_q=Wq.n, n_kv=Wk.n, rows=m, has_bias=int(c.qkv_bias)))
+                if self._fanout_applies(fan):      # q, k and v as one launch of the fused kernel's tile form
+                    t.append(fan)
+                else:
+                    fid[0] -= 1
+                    for nm, dst in (("q", self.q), ("k", self.k), ("v", self.v)):
+                        matmul(self.xn, w.mats[p + f"self_attn.{nm}_proj"], dst,
+                               bias=w.vecs.get(p + f"self_attn.{nm}_proj.bias") if c.qkv_bias else None)
             a = [arg(self.q), arg(self.k), arg(self.v)]
             if c.qk_norm:
                 a += [arg(w.vecs[p + "self_attn.q_norm"]), arg(w.vecs[p + "self_attn.k_norm"])]

@@ -521,6 +521,31 @@ def test_artifact_round_trip_and_launch_geometry(fk, tmp_path):
     assert t.from_device == 1 and t.wave_size == 64 and t.compute_units >= 64 and t.arch.startswith(b"gfx950")
 
 
+
+@pytest.mark.parametrize("bits,qkv_bias", [(4, False), (8, True)])
+def test_prefill_variant_of_256_rows_runs_the_fused_matmul_tile_form(fk, bits, qkv_bias):
+    """From 256 rows the variant's q / k / v projections are ONE dispatch (family fusekit_qgemm_fanout: one launch of
+    the fused matmul's tile form) and gate / up another; the graph leaves exactly the caches and the first token of the
+    direct-call prompt path, which plans the same launches."""
+    from fusekit_amd.decoder import DecoderRuntime, DecoderWeights
+    from fusekit_amd.prefill_variant import PrefillVariant
+    cfg = _small_cfg(bits=bits, qk_norm=True, qkv_bias=qkv_bias, swiglu_variant=1, capacity=512)
+    W = DecoderWeights.random_init(cfg, seed=61)
+    prompt = rng(62).integers(0, cfg.vocab, 256).tolist()
+    a, b = DecoderRuntime(cfg, W), DecoderRuntime(cfg, W)
+    first_a = a.prefill_rows(prompt, rows_per_pass=256)
+    v = PrefillVariant(b, 256)
+    kinds = [t.kernel.rsplit("_f", 1)[0] for t in v.tasks]
+    assert kinds.count("fusekit_qgemm_fanout") == cfg.n_layers and kinds.count("fusekit_qgemm") == 2 * cfg.n_layers
+    assert v.run(prompt, 0) == first_a
+    for l in range(cfg.n_layers):
+        assert np.array_equal(a.cache_k[l].to_numpy(np.uint16), b.cache_k[l].to_numpy(np.uint16))
+        assert np.array_equal(a.cache_v[l].to_numpy(np.uint16), b.cache_v[l].to_numpy(np.uint16))
+    assert np.array_equal(a.logits.to_numpy(np.uint16), b.logits.to_numpy(np.uint16))
+    small = PrefillVariant(b, 32)
+    assert not any(t.kernel.startswith("fusekit_qgemm_fanout") for t in small.tasks)   # fewer rows: one dispatch per matrix
+
+
 @pytest.mark.parametrize("bits,qk_norm,qkv_bias", [(4, True, False), (8, False, True)])
 def test_prefill_variants_as_graphs_and_in_the_artifact(fk, tmp_path, bits, qk_norm, qkv_bias):
     """`prefill_mN` variants (the reference: variants/prefill_mN, active_m = N): the whole model for N
