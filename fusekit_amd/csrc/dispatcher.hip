@@ -1391,7 +1391,7 @@ fk_status plan_qgemm_d(const Dispatch& d, Launch* l, SlotRW* rw) {
 // The q / k / v projections of several token rows (fk_qgemm_fanout): x, W_q, W_k, W_v, s_q, s_k, s_v, b_q, b_k, b_v,
 // [bias_q, bias_k, bias_v], q, k, v, workspace (fk_qgemm_workspace_bytes(rows, n_q + 2 n_kv, hidden, group)).
 // Parameters: hidden (= K), n_q, n_kv, rows, bits, group, has_bias.  One launch of the fused kernel's tile form (plus the
-// fan-out's second kernel when k is split); FK_ERR_UNSUPPORTED where that form does not apply (fewer than 256 rows, an n
+// fan-out's second kernel when k is split); FK_ERR_UNSUPPORTED where that form does not apply (fewer than 65 rows, an n
 // that is no multiple of 4): the caller dispatches fusekit_qgemm per matrix then.
 fk_status plan_qgemm_fanout_d(const Dispatch& d, Launch* l, SlotRW* rw) {
     const uint32_t bits = d.u("bits", 4), group = d.u("group", 64), K = d.u("hidden"), rows = d.u("rows");
@@ -1435,7 +1435,7 @@ fk_status plan_qgemm_fanout_d(const Dispatch& d, Launch* l, SlotRW* rw) {
         if (reduce.func) l->then.push_back(reduce);
         return FK_OK;
     }
-    return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": the fan-out needs the fused kernel's tile form (256 rows or more, every n a "
+    return set_error(FK_ERR_UNSUPPORTED, d.kernel + ": the fan-out needs the fused kernel's tile form (65 rows or more, every n a "
                                          "multiple of 4); dispatch fusekit_qgemm per matrix instead");
 }
 

@@ -435,8 +435,7 @@ class DecoderRuntime:
                      keep_bf16_weights: bool = False) -> int:
         """Prompt processing with several active rows per pass (the reference's `prefill_mN` /
         active_m > 1 variants): the projections of up to `rows_per_pass` (<= 4096) tokens share ONE pass over each weight
-        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form, from 256 rows in its LDS-tiled
-        form, from 1024 rows -- fk_set_gemm_library_rows -- as a dequantisation to bf16 followed by a library GEMM), attention is
+        matrix on the matrix cores (fk_qgemm; from 65 rows up in its bf16-weight form, which is LDS-tiled, from 1024 rows -- fk_set_gemm_library_rows -- as a dequantisation to bf16 followed by a library GEMM), attention is
         causal inside the group (fk_sdpa_prefill for the bf16 cache with head dimension 64 or 128,
         else the single-row kernel once per row).  Leaves the KV
         caches, step counter and history as token-by-token `prefill` would, and returns the greedy

@@ -236,12 +236,12 @@ def measure_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
 def case_qgemm(d, reps, rows, n=9728, k=2560, bits=4):
     sec, nbytes, flops, pool = measure_qgemm(d, reps, rows, n, k, bits)
     _emit(f"qgemm_rows{rows}_{n}x{k}_q{bits}", sec, nbytes, flops=flops, pool=pool,
-          note="2..10 rows: one shared-stream launch; 11..255 rows: MFMA main + split-k reduction; from 256 rows the "
+          note="2..10 rows: one shared-stream launch; 11..64 rows: MFMA main + split-k reduction; from 65 rows the "
                "LDS-tiled form (finished outputs at one k split)")
 
 
 def case_qgemm_swiglu(d, reps, rows, hidden=2560, inter=9728, bits=4):
-    """The gate / up pair with SwiGLU of the family fusekit_qgemm_swiglu on `rows` activation rows (from 256 rows one
+    """The gate / up pair with SwiGLU of the family fusekit_qgemm_swiglu on `rows` activation rows (from 65 rows one
     launch of the tile form); flops of both products."""
     per = bits / 8 + 4 / 64
     pool = max(2, int(600e6 // (2 * inter * hidden * per)) + 1)

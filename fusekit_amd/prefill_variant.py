@@ -58,7 +58,7 @@ class PrefillVariant:
                 p + "mid": self.mid, p + "ws": self.ws}
 
     def _fanout_applies(self, task: Dispatch) -> bool:
-        """Whether the family fusekit_qgemm_fanout plans this dispatch (its tile form needs 256 rows or more)."""
+        """Whether the family fusekit_qgemm_fanout plans this dispatch (its tile form needs 65 rows or more)."""
         if getattr(self, "_fanout", None) is None:
             try:
                 self.rt.d.plan_geometry(task)

@@ -275,7 +275,7 @@ fk_status fk_qgemm_swiglu(const fk_weight *Wg, const fk_weight *Wu, const uint16
 /*     fk_qgemm_fanout: one to three matrices over the SAME activation rows, y[i][m, N_i] = T(x @ W[i]^T (+ bias[i])) -- the
  *     q / k / v projections of a prompt pass, which the reference dispatches one after the other (qMM per projection,
  *     python/fusekit_runtime/dispatch.py prefill variants).  Same results as fk_qgemm per matrix (same kernel
- *     arithmetic).  From 256 rows, below the fk_set_gemm_library_rows() threshold, with equal K, bits and group size
+ *     arithmetic).  From 65 rows, below the fk_set_gemm_library_rows() threshold, with equal K, bits and group size
  *     and every N_i a multiple of 4, the matrices run as ONE launch of the fused kernel whose blocks along N run
  *     through them in turn (the narrow k and v projections alone leave most of the device idle); otherwise the
  *     call is fk_qgemm per matrix.  bias: null or an array of n_mats pointers (each may be null).

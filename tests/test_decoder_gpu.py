@@ -524,7 +524,7 @@ def test_artifact_round_trip_and_launch_geometry(fk, tmp_path):
 
 @pytest.mark.parametrize("bits,qkv_bias", [(4, False), (8, True)])
 def test_prefill_variant_of_256_rows_runs_the_fused_matmul_tile_form(fk, bits, qkv_bias):
-    """From 256 rows the variant's q / k / v projections are ONE dispatch (family fusekit_qgemm_fanout: one launch of
+    """From 65 rows (here 256) the variant's q / k / v projections are ONE dispatch (family fusekit_qgemm_fanout: one launch of
     the fused matmul's tile form) and gate / up another; the graph leaves exactly the caches and the first token of the
     direct-call prompt path, which plans the same launches."""
     from fusekit_amd.decoder import DecoderRuntime, DecoderWeights

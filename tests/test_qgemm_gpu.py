@@ -227,7 +227,7 @@ def test_qgemm_many_rows_both_routes(fk, m, n, k, bits, group, route):
 
 @pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 128)])
 def test_qgemm_tile_form_finishes_its_outputs_at_one_k_split(fk, bits, group):
-    """From 256 rows the fused kernel stages both operands of a 256 x 128 tile in LDS; with enough tiles to fill the
+    """From 65 rows the fused kernel stages both operands of a 256 x 128 tile in LDS; with enough tiles to fill the
     device it takes ONE k split and adds bias and residual and rounds in the same launch (no fp32 partial sums, no
     second kernel).  Ragged in both directions: 520 rows (a third row tile with 8 live rows), 9700 weight rows."""
     from fusekit_amd.runtime import Dispatch, Dispatcher, arg
@@ -265,7 +265,7 @@ def test_qgemm_tile_form_finishes_its_outputs_at_one_k_split(fk, bits, group):
 @pytest.mark.parametrize("m,hidden,inter,kernels", [(512, 256, 9700, 1), (300, 1024, 1280, 2)])
 @pytest.mark.parametrize("variant", [1, 2])
 def test_qgemm_swiglu_tile_form_takes_the_pair_in_one_launch(fk, bits, m, hidden, inter, kernels, variant):
-    """From 256 rows a gate / up pair (same shape, even count of 64-wide k slabs per split) is ONE launch of the tile
+    """From 65 rows a gate / up pair (same shape, even count of 64-wide k slabs per split) is ONE launch of the tile
     form: the activations staged once, two sets of accumulators; with one k split SwiGLU is applied there (1 kernel),
     otherwise the partial sums of both go to the usual second kernel (2 kernels instead of 3)."""
     from fusekit_amd.runtime import Dispatch, Dispatcher, arg
@@ -298,7 +298,7 @@ def test_qgemm_swiglu_tile_form_takes_the_pair_in_one_launch(fk, bits, m, hidden
 @pytest.mark.parametrize("m,k,ns,with_bias", [(512, 256, (4096, 1024, 1024), False),   # one k split: finished in the launch
                                               (300, 1024, (1000, 520, 260), True),     # ragged, k split, the fan-out's second kernel
                                               (512, 512, (2048, 1024), True),          # two matrices
-                                              (100, 256, (512, 256, 256), False)])     # too few rows for the tile form: one by one
+                                              (40, 256, (512, 256, 256), False)])      # too few rows for the tile form: one by one
 def test_qgemm_fanout_of_the_prompt_projections(fk, bits, m, k, ns, with_bias):
     """fk_qgemm_fanout: up to three matrices over the same rows (q / k / v of a prompt pass) as one launch of the tile
     form whose blocks run through the matrices in turn; every output against the oracle form of its row count."""
