@@ -523,7 +523,7 @@ def test_artifact_round_trip_and_launch_geometry(fk, tmp_path):
 
 
 @pytest.mark.parametrize("bits,qkv_bias", [(4, False), (8, True)])
-def test_prefill_variant_of_256_rows_runs_the_fused_matmul_tile_form(fk, bits, qkv_bias):
+def test_prefill_variant_of_256_rows_runs_the_fused_matmul_tile_form(fk, tmp_path, bits, qkv_bias):
     """From 65 rows (here 256) the variant's q / k / v projections are ONE dispatch (family fusekit_qgemm_fanout: one launch of
     the fused matmul's tile form) and gate / up another; the graph leaves exactly the caches and the first token of the
     direct-call prompt path, which plans the same launches."""
@@ -544,6 +544,18 @@ def test_prefill_variant_of_256_rows_runs_the_fused_matmul_tile_form(fk, bits, q
     assert np.array_equal(a.logits.to_numpy(np.uint16), b.logits.to_numpy(np.uint16))
     small = PrefillVariant(b, 32)
     assert not any(t.kernel.startswith("fusekit_qgemm_fanout") for t in small.tasks)   # fewer rows: one dispatch per matrix
+    # a consumer that knows only the artifact's files replays the same dispatches (the fan-out family among them)
+    import json
+    from fusekit_amd.artifact import ArtifactRuntime, write_artifact
+    write_artifact(b, str(tmp_path), "tiny", prefill_variants=[v])
+    vg = json.load(open(tmp_path / "variants" / "prefill_m256" / "task_graph.json"))
+    fan = next(t for t in vg["tasks"] if t["kernel"].startswith("fusekit_qgemm_fanout"))
+    assert fan["params"]["rows"] == 256.0 and len(fan["inputs"]) >= (13 if qkv_bias else 10) and len(fan["outputs"]) >= 3
+    art = ArtifactRuntime(str(tmp_path), W)
+    more = rng(63).integers(0, cfg.vocab, 4).tolist()
+    got = art.generate(prompt + more, 6)          # 256 through the variant, 4 token by token
+    want, _, _ = a.generate(prompt + more, 6)
+    assert got[0] == want[0]
 
 
 @pytest.mark.parametrize("bits,qk_norm,qkv_bias", [(4, True, False), (8, False, True)])
