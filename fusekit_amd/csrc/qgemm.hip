@@ -306,15 +306,16 @@ __global__ __launch_bounds__(kQgemmBlock) void qgemm_kernel(const QgemmArgs a) {
 // With one k split the block finishes its outputs itself (bias, residual, one rounding: the arithmetic of the second
 // kernel below for one split); otherwise partial sums go out in the layout of the form above.
 constexpr int kTileBlock = 512;
-constexpr uint32_t kTileM = 256, kTileN = 128, kTileK = 64;
+constexpr uint32_t kTileM = 256, kTileN = 128, kTileK = 64;   // (up to 128 activation rows: tiles of 128 rows, TM below)
 // activation rows from which the form is planned: every row count of the bf16-weight arithmetic (a tile of 256 rows that
 // is three quarters empty still beats the older form below, which unpacks per wave: 80-row prompt passes 14.7 k against
-// 12.8 k tok/s on the 4B-class model, 128-row passes 22.2 k against 19.5 k)
+// 12.8 k tok/s on the 4B-class model, 128-row passes 22.2 k against 19.5 k; with tiles of 128 rows for up to 128 rows
+// 18.1 k and 27.0 k)
 constexpr uint32_t kTileMinRows = 65;
 constexpr uint32_t kTileStride = kTileK / 8 + 1;                            // uint4 per staged row
 // one buffer: x rows, then weight rows (a gate / up pair: the up rows behind the gate rows)
-constexpr uint32_t tile_buf_pieces(bool pair) { return (kTileM + (pair ? 2u : 1u) * kTileN) * kTileStride; }
-constexpr uint32_t tile_lds_bytes(bool pair) { return 2u * tile_buf_pieces(pair) * 16u; }
+constexpr uint32_t tile_buf_pieces(bool pair, uint32_t tm) { return (tm + (pair ? 2u : 1u) * kTileN) * kTileStride; }
+constexpr uint32_t tile_lds_bytes(bool pair, uint32_t tm) { return 2u * tile_buf_pieces(pair, tm) * 16u; }
 
 // Piece p (codes 8 p .. 8 p + 7, element order) of the 16 codes one thread loaded (int4: w.x, w.y; int8: all of w) as
 // eight bf16 weights T(s q + b).
@@ -341,13 +342,19 @@ __device__ __forceinline__ uint4 tile_unpack_piece(int p, const uint4 w, float s
 // PAIR: a gate / up pair of the same shape in one launch -- the activations are requested and staged once for both,
 // every wave keeps a second set of accumulators, and with one k split SwiGLU is applied to the finished sums here
 // (swiglu_bits, as the second kernel applies it to the sums of one split).
-template <WKind KIND, bool PAIR>
+// TM: activation rows of a tile, 256 or 128 (row counts up to 128: four waves along the weight rows instead of two, a
+// wave's part 64 x 32).
+template <WKind KIND, bool PAIR, uint32_t TM>
 __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs a) {
     extern __shared__ uint4 lds_raw[];
-    constexpr uint32_t kTileBufPieces = tile_buf_pieces(PAIR);
+    constexpr uint32_t kTileBufPieces = tile_buf_pieces(PAIR, TM);
+    constexpr uint32_t WM = TM / 64u, WN = 8u / WM;   // waves along the activation rows / along the weight rows
+    constexpr uint32_t WCOLS = kTileN / WN;           // weight rows of a wave's part: 64 or 32
+    constexpr int NJ = (int)(WCOLS / 32u);            // 32-wide accumulator tiles along them
+    constexpr int XP = (int)(TM / 64u);               // x pieces per thread and slab
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, kb = lane >> 5, nl = lane & 31u;
-    const uint32_t wm = wave >> 1, wn = wave & 1u;   // the wave's 64 x 64 part: rows 64 wm, weight rows 64 wn
+    const uint32_t wm = wave / WN, wn = wave % WN;   // the wave's part: rows 64 wm, weight rows WCOLS wn
     uint32_t nb = blockIdx.x % a.n_blocks;
     const uint32_t ks = blockIdx.x / a.n_blocks;
     // the matrix this block works on (one, or the fan-out's matrix whose range of blocks holds nb)
@@ -367,7 +374,7 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         col0 = a.seg[si].col0;
         row_cols = a.n_total;
     }
-    const uint32_t m0 = blockIdx.y * kTileM, n0 = nb * kTileN;
+    const uint32_t m0 = blockIdx.y * TM, n0 = nb * kTileN;
     const uint32_t k0 = ks * a.k_per_split;
     const uint32_t k1 = k0 + a.k_per_split < a.K ? k0 + a.k_per_split : a.K;
     const uint32_t gshift = a.group == 128 ? 7u : 6u;
@@ -393,15 +400,15 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
     uint32_t xoff[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t m = m0 + xr + 64u * (uint32_t)i;
+        const uint32_t m = m0 + xr + 64u * (uint32_t)(i < XP ? i : 0);   // (TM = 128: two pieces per thread; 2, 3 unused)
         xoff[i] = (m < a.M ? m : a.M - 1) * a.K * 2u + xp * 16u;
     }
 
-    f32x16_t acc[2][2], acc2[PAIR ? 2 : 1][PAIR ? 2 : 1];
+    f32x16_t acc[2][NJ], acc2[PAIR ? 2 : 1][PAIR ? NJ : 1];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 acc[i][j][r] = 0.f;
@@ -417,8 +424,10 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         const unsigned char* xk = xbase + (size_t)kf * 2u;                                                           \
         S##x0 = *reinterpret_cast<const uint4*>(xk + xoff[0]);                                                        \
         S##x1 = *reinterpret_cast<const uint4*>(xk + xoff[1]);                                                        \
-        S##x2 = *reinterpret_cast<const uint4*>(xk + xoff[2]);                                                        \
-        S##x3 = *reinterpret_cast<const uint4*>(xk + xoff[3]);                                                        \
+        if constexpr (XP == 4) {                                                                                      \
+            S##x2 = *reinterpret_cast<const uint4*>(xk + xoff[2]);                                                    \
+            S##x3 = *reinterpret_cast<const uint4*>(xk + xoff[3]);                                                    \
+        }                                                                                                             \
         if constexpr (KIND == W_Q4) {                                                                                 \
             const uint2 v = *reinterpret_cast<const uint2*>(wbase + (kf >> 1) + woff);                                \
             S##w = make_uint4(v.x, v.y, 0u, 0u);                                                                      \
@@ -446,13 +455,13 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
         uint4* xs_w = lds_raw + (to) * kTileBufPieces;                                                                \
         uint4* xd = xs_w + xr * kTileStride + xp;                                                                     \
         xd[0 * 64 * kTileStride] = S##x0; xd[1 * 64 * kTileStride] = S##x1;                                           \
-        xd[2 * 64 * kTileStride] = S##x2; xd[3 * 64 * kTileStride] = S##x3;                                           \
+        if constexpr (XP == 4) { xd[2 * 64 * kTileStride] = S##x2; xd[3 * 64 * kTileStride] = S##x3; }                \
         /* pinned here: left alone, the compiler widens the two values where they are loaded, a pass earlier, and   \
            waits there for every request in flight */                                                                 \
         uint32_t sc_bits = S##sc, bi_bits = S##bi;                                                                    \
         asm volatile("" : "+v"(sc_bits), "+v"(bi_bits));                                                              \
         const float sf = bf16_bits_to_f32(sc_bits), bf = bf16_bits_to_f32(bi_bits);                                   \
-        uint4* wd = xs_w + kTileM * kTileStride + wr * kTileStride + wq * 2u;                                         \
+        uint4* wd = xs_w + TM * kTileStride + wr * kTileStride + wq * 2u;                                             \
         wd[0] = tile_unpack_piece<KIND>(0, S##w, sf, bf);                                                             \
         wd[1] = tile_unpack_piece<KIND>(1, S##w, sf, bf);                                                             \
         if constexpr (PAIR) {                                                                                         \
@@ -466,28 +475,28 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
     auto multiply = [&](uint32_t from) {
         const uint4* xs = lds_raw + from * kTileBufPieces;
         const uint4* xa = xs + (wm * 64u + nl) * kTileStride + kb;
-        const uint4* wb = xs + (kTileM + wn * 64u + nl) * kTileStride + kb;
+        const uint4* wb = xs + (TM + wn * WCOLS + nl) * kTileStride + kb;
 #pragma unroll
         for (int st = 0; st < (int)kTileK / 16; ++st) {
-            uint4 af[2], bfr[2];
+            uint4 af[2], bfr[NJ];
 #pragma unroll
             for (int i = 0; i < 2; ++i) af[i] = xa[(uint32_t)i * 32u * kTileStride + 2u * (uint32_t)st];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) bfr[j] = wb[(uint32_t)j * 32u * kTileStride + 2u * (uint32_t)st];
+            for (int j = 0; j < NJ; ++j) bfr[j] = wb[(uint32_t)j * 32u * kTileStride + 2u * (uint32_t)st];
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < NJ; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
                                                                         __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
             if constexpr (PAIR) {
-                uint4 bf2[2];
+                uint4 bf2[NJ];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) bf2[j] = wb[((uint32_t)j * 32u + kTileN) * kTileStride + 2u * (uint32_t)st];
+                for (int j = 0; j < NJ; ++j) bf2[j] = wb[((uint32_t)j * 32u + kTileN) * kTileStride + 2u * (uint32_t)st];
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < NJ; ++j)
                         acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
                                                                              __builtin_bit_cast(bf16x8_t, bf2[j]), acc2[i][j], 0, 0, 0);
                 // (a step's fragment reads stay behind the step before: requested all at once, the four steps' 24
@@ -529,8 +538,8 @@ __global__ __launch_bounds__(kTileBlock) void qgemm_tile_kernel(const QgemmArgs 
 
     // register r of a lane is activation row (r % 4) + 8 (r / 4) + 4 kb of its 32 x 32 tile, column nl
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const uint32_t n = n0 + wn * 64u + (uint32_t)j * 32u + nl;
+    for (int j = 0; j < NJ; ++j) {
+        const uint32_t n = n0 + wn * WCOLS + (uint32_t)j * 32u + nl;
         if (n >= N) continue;
         const float bias = (y_mat && bias_mat) ? bf16_bits_to_f32(bias_mat[n]) : 0.f;
 #pragma unroll
@@ -648,18 +657,23 @@ __global__ __launch_bounds__(256) void qgemm_fan_reduce_kernel(const QgemmFanRed
 
 namespace {
 
-uint32_t qgemm_form_lds_bytes(int mt) { return mt >= 8 ? tile_lds_bytes(mt == 9) : qgemm_lds_bytes(mt); }
+// forms 8 .. 11: the tile form (9, 11: a gate / up pair; 10, 11: tiles of 128 activation rows)
+uint32_t qgemm_form_lds_bytes(int mt) { return mt >= 8 ? tile_lds_bytes(mt & 1, mt >= 10 ? 128u : 256u) : qgemm_lds_bytes(mt); }
 
 struct QgemmShape {
     uint32_t n_blocks, m_tiles, ksplit, k_per_split;
-    int mt;  // tiles of 32 activation rows per block
+    int mt;           // tiles of 32 activation rows per block; 8: the tile form
+    uint32_t tile_m;  // the tile form's activation rows per tile: 256 or 128
+    int form(bool pair) const { return mt == 8 ? 8 + (pair ? 1 : 0) + (tile_m == 128u ? 2 : 0) : mt; }
 };
 
 const void* qgemm_func(uint32_t bits, int mt) {
     const bool q4 = bits == 4;
     switch (mt) {
-        case 8: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, false>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, false>);
-        case 9: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, true>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, true>);   // a gate / up pair
+        case 8: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, false, 256>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, false, 256>);
+        case 9: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, true, 256>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, true, 256>);   // a gate / up pair
+        case 10: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, false, 128>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, false, 128>);   // tiles of 128 rows
+        case 11: return q4 ? reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q4, true, 128>) : reinterpret_cast<const void*>(&qgemm_tile_kernel<W_Q8, true, 128>);
         case 1: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 1>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 1>);
         case 2: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 2>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 2>);
         default: return q4 ? reinterpret_cast<const void*>(&qgemm_kernel<W_Q4, 4>) : reinterpret_cast<const void*>(&qgemm_kernel<W_Q8, 4>);
@@ -669,7 +683,7 @@ const void* qgemm_func(uint32_t bits, int mt) {
 // Blocks of this kernel form that are resident at once (registers and LDS decide).
 uint32_t qgemm_resident(const DeviceFacts* dev, uint32_t bits, int mt) {
     static std::mutex mu;
-    static int cache[2][10] = {};
+    static int cache[2][12] = {};
     std::lock_guard<std::mutex> lk(mu);
     int& slot = cache[bits == 4 ? 0 : 1][mt];
     if (slot == 0) {
@@ -695,7 +709,8 @@ fk_status qgemm_shape(const DeviceFacts* dev, uint32_t M, uint32_t N, uint32_t K
     // 8: the tile form (its requests are 32-bit byte offsets from a uniform base: operands under 4 GB)
     const bool tile_ok = M >= kTileMinRows && (uint64_t)M * K * 2 < (1ull << 32) && (uint64_t)N * K < (1ull << 32);
     s.mt = tile_ok ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));
-    s.m_tiles = (M + kQgemmMTile * s.mt - 1) / (kQgemmMTile * s.mt);
+    s.tile_m = M <= 128u ? 128u : kTileM;   // up to 128 rows: tiles of 128 rows (a 256-row tile would be half empty)
+    s.m_tiles = s.mt == 8 ? (M + s.tile_m - 1) / s.tile_m : (M + kQgemmMTile * s.mt - 1) / (kQgemmMTile * s.mt);
     if (s.mt == 8) s.n_blocks = (N + kTileN - 1) / kTileN;
     // Split k until the grid fills what is resident at once, never beyond (a block that waits
     // for a slot doubles the run time), and keep at least 256 k per block.  Every split writes
@@ -753,10 +768,10 @@ fk_status plan_qgemm_main(const DeviceFacts* dev, const fk_weight* W, const uint
         a.res = direct->res;
         if (finished) *finished = true;
     }
-    out->func = qgemm_func(W->bits, shape->mt);
+    out->func = qgemm_func(W->bits, shape->form(false));
     out->grid = dim3(shape->n_blocks * shape->ksplit, shape->m_tiles, 1);
     out->block = dim3(shape->mt == 8 ? kTileBlock : kQgemmBlock, 1, 1);
-    out->shmem = qgemm_form_lds_bytes(shape->mt);
+    out->shmem = qgemm_form_lds_bytes(shape->form(false));
     out->set_args(a);
     if (out->shmem > 48 * 1024)
         FK_HIP(hipFuncSetAttribute(out->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)out->shmem));
@@ -890,10 +905,10 @@ fk_status plan_qgemm_fanout(const fk_weight* const* W, uint32_t n_mats, const ui
     a.w = a.seg[0].w;
     a.sc = a.seg[0].sc;
     a.bi = a.seg[0].bi;
-    main->func = qgemm_func(W[0]->bits, 8);
+    main->func = qgemm_func(W[0]->bits, s.form(false));
     main->grid = dim3(blocks_n * s.ksplit, s.m_tiles, 1);
     main->block = dim3(kTileBlock, 1, 1);
-    main->shmem = qgemm_form_lds_bytes(8);
+    main->shmem = qgemm_form_lds_bytes(s.form(false));
     main->set_args(a);
     FK_HIP(hipFuncSetAttribute(main->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)main->shmem));
     *reduce = Launch();
@@ -944,8 +959,8 @@ fk_status plan_qgemm_swiglu(const fk_weight* Wg, const fk_weight* Wu, const uint
         a.variant = variant;
         a.y = s.ksplit == 1 ? out : nullptr;
         a.bias = a.res = nullptr;
-        gate->func = qgemm_func(Wg->bits, 9);
-        gate->shmem = qgemm_form_lds_bytes(9);
+        gate->func = qgemm_func(Wg->bits, s.form(true));
+        gate->shmem = qgemm_form_lds_bytes(s.form(true));
         gate->set_args(a);
         FK_HIP(hipFuncSetAttribute(gate->func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)gate->shmem));
         *up = Launch();
